@@ -1,0 +1,467 @@
+// Network graph, device tensor management and the forward loop.
+#include "engine.h"
+
+#include <algorithm>
+#include <cstring>
+
+namespace fynhip {
+
+void fail(int code, const char* fmt, ...) {
+    char buf[1024];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof(buf), fmt, ap);
+    va_end(ap);
+    throw Error(code, buf);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Layer base
+// ---------------------------------------------------------------------------------------------
+Layer::Layer(Net* n, const fyn_layer_desc& desc) : d(desc), net(n) {}
+
+Act Layer::act() const {
+    // LayerBuilderTempl::getFlags (base/layerbuilder.h:445-493): RELU and LEAKY_RELU both set PRE_RELU,
+    // the leak value distinguishes them (gpu/gpulayerbase.cpp:775-802).
+    Act a{ACT_NONE, 0.f, 0.f, 0.f};
+    if (d.flags & FYN_FLAG_PRE_RELU) {
+        if (d.leaky_relu != 0.f) {
+            a.kind = ACT_LEAKY;
+            a.leak = d.leaky_relu;
+        } else {
+            a.kind = ACT_RELU;
+        }
+    } else if (d.flags & FYN_FLAG_PRE_CLIP) {
+        a.kind = ACT_CLIP;
+        a.lo = d.clip_low;
+        a.hi = d.clip_high;
+    }
+    return a;
+}
+
+void Layer::port_shape(int port, int& c, int& h, int& w, int& pad) const {
+    if (port == 0) {
+        c = d.in_channels;
+        h = d.height;
+        w = d.width;
+        pad = d.input_padding;
+    } else {  // residual: same net size as the output (base/layerbase.h:266-274)
+        c = oc;
+        h = oh;
+        w = ow;
+        pad = d.residual_padding;
+    }
+}
+
+const Tensor& Layer::tin(int port) const { return net->tensors[in[port]]; }
+const Tensor& Layer::tout() const { return net->tensors[out]; }
+
+// ---------------------------------------------------------------------------------------------
+// Net
+// ---------------------------------------------------------------------------------------------
+Net::Net(int dev, int stor) : device(dev), storage(stor) {
+    if (stor != FYN_STORAGE_F32 && stor != FYN_STORAGE_F16) fail(FYN_ERR_INVALID, "unknown storage type %d", stor);
+    int count = 0;
+    FYN_HIP(hipGetDeviceCount(&count));
+    if (dev < 0 || dev >= count) fail(FYN_ERR_DEVICE, "device %d not present (%d devices)", dev, count);
+    FYN_HIP(hipSetDevice(dev));
+    FYN_HIP(hipStreamCreate(&stream));
+}
+
+Net::~Net() {
+    (void)hipSetDevice(device);
+    if (stream) (void)hipStreamSynchronize(stream);
+    if (graph_exec_) (void)hipGraphExecDestroy(graph_exec_);
+    if (graph_) (void)hipGraphDestroy(graph_);
+    for (auto& kv : layers) {
+        if (kv.second->ev0) (void)hipEventDestroy(kv.second->ev0);
+        if (kv.second->ev1) (void)hipEventDestroy(kv.second->ev1);
+    }
+    layers.clear();
+    for (void* p : allocs_) (void)hipFree(p);
+    if (stream) (void)hipStreamDestroy(stream);
+}
+
+void* Net::dev_alloc(size_t bytes, bool zero) {
+    void* p = nullptr;
+    if (bytes == 0) bytes = 16;
+    FYN_HIP(hipMalloc(&p, bytes));
+    allocs_.push_back(p);
+    if (zero) {
+        launch_fill_zero(p, bytes, stream);
+        FYN_HIP(hipGetLastError());
+    }
+    return p;
+}
+
+float* Net::staging(size_t floats) {
+    if (floats > staging_floats_) {
+        FYN_HIP(hipStreamSynchronize(stream));
+        // the old area stays owned by allocs_ and is released with the net
+        staging_ = static_cast<float*>(dev_alloc(floats * sizeof(float), false));
+        staging_floats_ = floats;
+    }
+    return staging_;
+}
+
+Layer* Net::layer(int number) {
+    auto it = layers.find(number);
+    if (it == layers.end()) fail(FYN_ERR_NOTFOUND, "no layer with number %d", number);
+    return it->second.get();
+}
+
+void Net::add_layer(const fyn_layer_desc& d) {
+    if (is_setup) fail(FYN_ERR_STATE, "cannot add layers after setup");
+    // LayerFactory::pushBuilder (base/layerfactory.cpp:67-76)
+    if (d.number < 0) fail(FYN_ERR_INVALID, "Must identify each layer with a valid number (found %d in the builder)", d.number);
+    if (layers.count(d.number)) fail(FYN_ERR_DUPLICATE, "Trying to insert a layer on a position that is already taken (%d)", d.number);
+    layers[d.number].reset(create_layer(this, d));
+}
+
+void Net::connect(int out_layer, int in_layer, int port) {
+    if (is_setup) fail(FYN_ERR_STATE, "cannot connect layers after setup");
+    Layer* src = layer(out_layer);
+    Layer* dst = layer(in_layer);
+    if (port < 0 || port >= dst->num_ports())
+        fail(FYN_ERR_INVALID, "layer %s has no input port %d", dst->d.name, port);
+    if (!(in_layer > out_layer))
+        fail(FYN_ERR_INVALID, "layer %s (%d) cannot feed layer %s (%d): execution is in ascending number", src->d.name,
+             out_layer, dst->d.name, in_layer);
+    if (dst->in[port] != -1) return;  // already connected (BufferManager::checkIOMatch returns no match)
+    // I/O match (base/buffermanager.cpp:462-492): same geometry on both sides of the edge
+    int c, h, w, pad;
+    dst->port_shape(port, c, h, w, pad);
+    if (c != src->oc || h != src->oh || w != src->ow || pad != src->d.output_padding)
+        fail(FYN_ERR_INVALID,
+             "Inputs/outputs do not match (I/O) for layers %s and %s: producer %dx%dx%d pad %d, consumer port %d wants "
+             "%dx%dx%d pad %d",
+             dst->d.name, src->d.name, src->oc, src->oh, src->ow, src->d.output_padding, port, c, h, w, pad);
+    // tensors are created lazily: the producer's output tensor id
+    if (src->out == -1) {
+        if (!src->has_own_output()) {
+            fail(FYN_ERR_INVALID, "layer %s has no output that can be connected", src->d.name);
+        }
+        Tensor t;
+        t.producer = src->d.number;
+        tensors.push_back(t);
+        src->out = (int)tensors.size() - 1;
+    }
+    dst->in[port] = src->out;
+    tensors[src->out].last_reader = std::max(tensors[src->out].last_reader, in_layer);
+}
+
+void Net::setup() {
+    if (is_setup) fail(FYN_ERR_STATE, "network is already set up");
+    FYN_HIP(hipSetDevice(device));
+    // 1. tensors: external inputs for unconnected ports, outputs for every layer
+    for (auto& kv : layers) {
+        Layer* l = kv.second.get();
+        for (int p = 0; p < l->num_ports(); p++) {
+            if (l->in[p] != -1) continue;
+            Tensor t;
+            t.producer = -1;
+            t.locked = true;
+            t.last_reader = l->d.number;
+            tensors.push_back(t);
+            l->in[p] = (int)tensors.size() - 1;
+            int c, h, w, pad;
+            l->port_shape(p, c, h, w, pad);
+            TView& v = tensors.back().v;
+            v.c = c; v.h = h; v.w = w; v.pad = pad; v.cp = channel_pitch(c); v.f16 = f16();
+        }
+        if (l->has_own_output()) {
+            if (l->out == -1) {
+                Tensor t;
+                t.producer = l->d.number;
+                t.locked = true;  // nobody consumes it: it is a network output
+                tensors.push_back(t);
+                l->out = (int)tensors.size() - 1;
+            }
+            if (l->d.type == FYN_LAYER_UPLOAD) tensors[l->out].locked = true;  // filled from the host
+            TView& v = tensors[l->out].v;
+            v.c = l->oc; v.h = l->oh; v.w = l->ow; v.pad = l->d.output_padding; v.cp = channel_pitch(l->oc); v.f16 = f16();
+        } else {
+            // pass-through (download): output aliases the input, which must survive
+            l->out = l->in[0];
+            tensors[l->out].locked = true;
+        }
+    }
+    // 2. device buffers.  Liveness rule of BufferManager::findTexture (base/buffermanager.cpp:512-525)
+    //    restated for in-order stream execution: a buffer can take layer N's output when every reader of
+    //    its current tenant has a number < N; only buffers of identical geometry are shared so that the
+    //    zero halo written at allocation stays valid.
+    for (auto& kv : layers) {
+        Layer* l = kv.second.get();
+        for (int p = 0; p < l->num_ports(); p++) {
+            Tensor& t = tensors[l->in[p]];
+            if (t.buffer == -1 && t.producer == -1) {
+                DevBuffer b;
+                b.bytes = t.v.bytes();
+                b.ptr = dev_alloc(b.bytes);
+                b.locked = true;
+                buffers.push_back(b);
+                t.buffer = (int)buffers.size() - 1;
+                t.v.ptr = b.ptr;
+            }
+        }
+        if (!l->has_own_output()) continue;
+        Tensor& t = tensors[l->out];
+        int found = -1;
+        if (reuse_buffers && !t.locked) {
+            for (size_t i = 0; i < buffers.size(); i++) {
+                DevBuffer& b = buffers[i];
+                if (!b.locked && b.free_after < l->d.number && b.h == t.v.h && b.w == t.v.w && b.pad == t.v.pad &&
+                    b.cp == t.v.cp && b.f16 == t.v.f16) {
+                    found = (int)i;
+                    break;
+                }
+            }
+        }
+        if (found == -1) {
+            DevBuffer b;
+            b.bytes = t.v.bytes();
+            b.ptr = dev_alloc(b.bytes);
+            b.h = t.v.h; b.w = t.v.w; b.pad = t.v.pad; b.cp = t.v.cp; b.f16 = t.v.f16;
+            buffers.push_back(b);
+            found = (int)buffers.size() - 1;
+        }
+        DevBuffer& b = buffers[found];
+        b.locked = t.locked;
+        b.free_after = std::max(t.last_reader, l->d.number);
+        t.buffer = found;
+        t.v.ptr = b.ptr;
+    }
+    // pass-through layers were given the tensor id only; nothing else to do for them
+    // 3. per-layer setup (weight packing, kernel selection)
+    for (auto& kv : layers) {
+        kv.second->setup();
+        kv.second->set_up = true;
+    }
+    FYN_HIP(hipStreamSynchronize(stream));
+    is_setup = true;
+}
+
+void Net::dump_layer(Layer* l) {
+    // Engine::enableIntermediateOutput (base/engine.cpp:174-181,602-604): <name>_<seq>.bin, CHW fp32
+    if (!l->has_own_output()) return;
+    const TView& v = l->tout().v;
+    std::vector<float> host((size_t)v.c * v.h * v.w);
+    copy_result(l->d.number, host.data(), 0);
+    char path[1024];
+    snprintf(path, sizeof(path), "%s/%s_%llu.bin", dump_dir.c_str(), l->d.name, (unsigned long long)seq);
+    FILE* f = fopen(path, "wb");
+    if (!f) fail(FYN_ERR_INVALID, "cannot write %s", path);
+    fwrite(host.data(), sizeof(float), host.size(), f);
+    fclose(f);
+}
+
+void Net::run_layers(bool with_events) {
+    for (auto& kv : layers) {
+        Layer* l = kv.second.get();
+        if (with_events) {
+            if (!l->ev0) {
+                FYN_HIP(hipEventCreate(&l->ev0));
+                FYN_HIP(hipEventCreate(&l->ev1));
+            }
+            FYN_HIP(hipEventRecord(l->ev0, stream));
+        }
+        l->forward(stream);
+        FYN_HIP(hipGetLastError());
+        if (with_events) FYN_HIP(hipEventRecord(l->ev1, stream));
+        if (!dump_dir.empty()) dump_layer(l);
+    }
+}
+
+void Net::collect_timings() {
+    if (!events_pending_) return;
+    for (auto& kv : layers) {
+        Layer* l = kv.second.get();
+        if (!l->ev0) continue;
+        float ms = 0.f;
+        if (hipEventElapsedTime(&ms, l->ev0, l->ev1) == hipSuccess) {
+            l->ms_total += ms;
+            l->runs++;
+        }
+    }
+    events_pending_ = false;
+}
+
+void Net::forward(uint64_t* seq_out) {
+    if (!is_setup) fail(FYN_ERR_STATE, "forward() called on a network that was not set up");
+    FYN_HIP(hipSetDevice(device));
+    seq++;
+    if (seq_out) *seq_out = seq;
+    const bool plain = timings || !dump_dir.empty();
+    if (graph_enabled_ && !plain) {
+        if (!graph_exec_) {
+            FYN_HIP(hipStreamBeginCapture(stream, hipStreamCaptureModeThreadLocal));
+            try {
+                run_layers(false);
+            } catch (...) {
+                hipGraph_t g = nullptr;
+                (void)hipStreamEndCapture(stream, &g);
+                if (g) (void)hipGraphDestroy(g);
+                throw;
+            }
+            FYN_HIP(hipStreamEndCapture(stream, &graph_));
+            FYN_HIP(hipGraphInstantiate(&graph_exec_, graph_, nullptr, nullptr, 0));
+        }
+        FYN_HIP(hipGraphLaunch(graph_exec_, stream));
+        return;
+    }
+    if (timings) {
+        FYN_HIP(hipStreamSynchronize(stream));
+        collect_timings();
+    }
+    run_layers(timings);
+    events_pending_ = timings;
+}
+
+void Net::finish() {
+    FYN_HIP(hipSetDevice(device));
+    FYN_HIP(hipStreamSynchronize(stream));
+    collect_timings();
+}
+
+void Net::use_graph(bool enable) {
+    graph_enabled_ = enable;
+    if (!enable && graph_exec_) {
+        FYN_HIP(hipStreamSynchronize(stream));
+        (void)hipGraphExecDestroy(graph_exec_);
+        (void)hipGraphDestroy(graph_);
+        graph_exec_ = nullptr;
+        graph_ = nullptr;
+    }
+}
+
+void Net::set_input(int layer_no, int port, const float* data, int order) {
+    if (!is_setup) fail(FYN_ERR_STATE, "set_input() before setup()");
+    if (!data) fail(FYN_ERR_INVALID, "null input buffer");
+    FYN_HIP(hipSetDevice(device));
+    Layer* l = layer(layer_no);
+    const Tensor* t;
+    if (l->d.type == FYN_LAYER_UPLOAD) {
+        t = &l->tout();
+    } else {
+        if (port < 0 || port >= l->num_ports()) fail(FYN_ERR_INVALID, "layer %s has no input port %d", l->d.name, port);
+        t = &l->tin(port);
+        if (t->producer != -1)
+            fail(FYN_ERR_INVALID, "input port %d of layer %s is fed by layer %d", port, l->d.name, t->producer);
+    }
+    const TView& v = t->v;
+    const size_t n = (size_t)v.c * v.h * v.w;
+    float* st = staging(n);
+    FYN_HIP(hipMemcpyAsync(st, data, n * sizeof(float), hipMemcpyHostToDevice, stream));
+    if (order == FYN_ORDER_CHANNELWISE) launch_chw_to_tensor(st, v, stream);
+    else if (order == FYN_ORDER_GPU_SHALLOW) launch_hwc_to_tensor(st, v.c, v, stream);
+    else fail(FYN_ERR_UNSUPPORTED, "input order %d not supported for upload", order);
+    FYN_HIP(hipGetLastError());
+    // the host buffer is borrowed for this call only
+    FYN_HIP(hipStreamSynchronize(stream));
+}
+
+void Net::copy_result(int layer_no, float* chw, int include_padding) {
+    if (!is_setup) fail(FYN_ERR_STATE, "copy_result() before setup()");
+    FYN_HIP(hipSetDevice(device));
+    Layer* l = layer(layer_no);
+    const TView& v = l->tout().v;
+    const size_t n = include_padding ? (size_t)v.c * v.hp() * v.wp() : (size_t)v.c * v.h * v.w;
+    float* st = staging(n);
+    launch_tensor_to_chw(v, st, include_padding, stream);
+    FYN_HIP(hipGetLastError());
+    FYN_HIP(hipMemcpyAsync(chw, st, n * sizeof(float), hipMemcpyDeviceToHost, stream));
+    FYN_HIP(hipStreamSynchronize(stream));
+}
+
+static void deep_tiling(int channels, int& tx, int& ty) {
+    // CPUBufferShape::computeDeepTiling (cpu/cpubuffershape.cpp:430-448)
+    const int tiles = (channels + 3) / 4;
+    int best = 1 << 30;
+    tx = tiles;
+    ty = 1;
+    for (int y = 1; y <= tiles; y++)
+        for (int x = y; x <= tiles; x++)
+            if (x * y >= tiles) {
+                const int cost = (x - y) + (x * y - tiles);
+                if (cost < best) {
+                    best = cost;
+                    tx = x;
+                    ty = y;
+                }
+            }
+}
+
+void Net::get_output(int layer_no, float* data, int order) {
+    if (!is_setup) fail(FYN_ERR_STATE, "get_output() before setup()");
+    FYN_HIP(hipSetDevice(device));
+    Layer* l = layer(layer_no);
+    const TView& v = l->tout().v;
+    if (order == FYN_ORDER_CHANNELWISE) {
+        copy_result(layer_no, data, 0);
+    } else if (order == FYN_ORDER_GPU_SHALLOW) {
+        if (v.c > 4) fail(FYN_ERR_UNSUPPORTED, "GPU_SHALLOW download holds at most 4 channels per texel (layer has %d)", v.c);
+        const int pc = v.c == 3 ? 4 : v.c;  // rendered textures are RGBA (base/buffermanager.cpp:478-483)
+        const size_t n = (size_t)v.h * v.w * pc;
+        float* st = staging(n);
+        launch_tensor_to_hwc(v, st, pc, stream);
+        FYN_HIP(hipGetLastError());
+        FYN_HIP(hipMemcpyAsync(data, st, n * sizeof(float), hipMemcpyDeviceToHost, stream));
+        FYN_HIP(hipStreamSynchronize(stream));
+    } else if (order == FYN_ORDER_GPU_DEEP) {
+        // tiled RGBA buffer, tile t at grid (t % tx, t / tx), padding shared between tiles
+        // (gpu/deep/deeptiler.cpp:63-110)
+        std::vector<float> chw((size_t)v.c * v.h * v.w);
+        copy_result(layer_no, chw.data(), 0);
+        int tx, ty;
+        deep_tiling(v.c, tx, ty);
+        const int pad = v.pad;
+        const int dw = tx * (v.w + pad) + pad, dh = ty * (v.h + pad) + pad;
+        memset(data, 0, (size_t)dw * dh * 4 * sizeof(float));
+        for (int ch = 0; ch < v.c; ch++) {
+            const int t = ch / 4, comp = ch % 4, gx = t % tx, gy = t / tx;
+            for (int y = 0; y < v.h; y++)
+                for (int x = 0; x < v.w; x++)
+                    data[(((size_t)(pad + gy * (v.h + pad) + y)) * dw + pad + gx * (v.w + pad) + x) * 4 + comp] =
+                        chw[((size_t)ch * v.h + y) * v.w + x];
+        }
+    } else {
+        fail(FYN_ERR_INVALID, "unknown buffer order %d", order);
+    }
+}
+
+void Net::time_forward(int iters, float* ms) {
+    if (!is_setup) fail(FYN_ERR_STATE, "time_forward() before setup()");
+    FYN_HIP(hipSetDevice(device));
+    hipEvent_t a, b;
+    FYN_HIP(hipEventCreate(&a));
+    FYN_HIP(hipEventCreate(&b));
+    const bool t = timings;
+    timings = false;
+    FYN_HIP(hipEventRecord(a, stream));
+    for (int i = 0; i < iters; i++) forward(nullptr);
+    FYN_HIP(hipEventRecord(b, stream));
+    FYN_HIP(hipEventSynchronize(b));
+    timings = t;
+    FYN_HIP(hipEventElapsedTime(ms, a, b));
+    (void)hipEventDestroy(a);
+    (void)hipEventDestroy(b);
+}
+
+void Net::time_layer(int layer_no, int iters, float* ms) {
+    if (!is_setup) fail(FYN_ERR_STATE, "time_layer() before setup()");
+    FYN_HIP(hipSetDevice(device));
+    Layer* l = layer(layer_no);
+    hipEvent_t a, b;
+    FYN_HIP(hipEventCreate(&a));
+    FYN_HIP(hipEventCreate(&b));
+    FYN_HIP(hipEventRecord(a, stream));
+    for (int i = 0; i < iters; i++) l->forward(stream);
+    FYN_HIP(hipEventRecord(b, stream));
+    FYN_HIP(hipEventSynchronize(b));
+    FYN_HIP(hipGetLastError());
+    FYN_HIP(hipEventElapsedTime(ms, a, b));
+    (void)hipEventDestroy(a);
+    (void)hipEventDestroy(b);
+}
+
+}  // namespace fynhip

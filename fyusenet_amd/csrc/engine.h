@@ -1,0 +1,134 @@
+// Host-side engine: network graph, device tensors, layer objects.  This is the part of the
+// reference's base/ + gpu/ host code that survives the move from OpenGL to HIP:
+//   LayerFactory / GPULayerFactoryBackend   -> Net::add_layer          (base/layerfactory.cpp, gpu/gpulayerfactory.cpp)
+//   BufferManager                           -> Net::connect / assign_buffers (base/buffermanager.cpp)
+//   NeuralNetwork / Engine (sync branch)    -> Net::setup / forward / finish (base/neuralnetwork.cpp, base/engine.cpp)
+//   GPULayerBase subclasses                 -> Layer subclasses in layers.cpp
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdio>
+#include <map>
+#include <memory>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+#include "../../include/fynhip.h"
+#include "kernels.h"
+
+namespace fynhip {
+
+// Error carried up to the C ABI (the reference throws FynException, common/fynexception.h).
+struct Error : public std::runtime_error {
+    int code;
+    Error(int c, const std::string& m) : std::runtime_error(m), code(c) {}
+};
+[[noreturn]] void fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+
+#define FYN_HIP(call)                                                                              \
+    do {                                                                                           \
+        hipError_t e_ = (call);                                                                    \
+        if (e_ != hipSuccess) ::fynhip::fail(FYN_ERR_DEVICE, "%s failed: %s (%s:%d)", #call,       \
+                                             hipGetErrorString(e_), __FILE__, __LINE__);           \
+    } while (0)
+
+struct Tensor {
+    TView v{};
+    int producer = -1;     // layer number writing it (-1: external input)
+    int last_reader = -1;  // highest layer number reading it
+    bool locked = false;   // never reused (network outputs, external inputs)
+    int buffer = -1;       // index into Net::buffers_
+};
+
+struct DevBuffer {
+    void* ptr = nullptr;
+    size_t bytes = 0;
+    int h = 0, w = 0, pad = 0, cp = 0, f16 = 0;  // geometry key (reuse only between identical geometries)
+    int free_after = -1;                          // highest reader of the current tenant
+    bool locked = false;
+};
+
+class Net;
+
+class Layer {
+  public:
+    Layer(Net* net, const fyn_layer_desc& d);
+    virtual ~Layer() {}
+    fyn_layer_desc d;
+    Net* net;
+    std::vector<int> in;  // tensor id per input port, -1 = not connected
+    int out = -1;         // tensor id
+    int oc = 0, oh = 0, ow = 0;  // output net shape
+
+    virtual int num_ports() const { return (d.flags & FYN_FLAG_RESIDUAL_INPUT) ? 2 : 1; }
+    // shape of the tensor expected on an input port (channels, h, w, padding)
+    virtual void port_shape(int port, int& c, int& h, int& w, int& pad) const;
+    virtual bool has_own_output() const { return true; }
+    virtual size_t weight_floats() const { return 0; }
+    virtual void load_weights(const float*) { fail(FYN_ERR_INVALID, "layer %s (%d) takes no weights", d.name, d.number); }
+    virtual void setup() {}
+    virtual void forward(hipStream_t s) = 0;
+    virtual std::string info() const { return "none"; }
+    Act act() const;
+    const Tensor& tin(int port) const;
+    const Tensor& tout() const;
+    bool set_up = false;
+    // timing
+    hipEvent_t ev0 = nullptr, ev1 = nullptr;
+    float ms_total = 0.f;
+    int runs = 0;
+};
+
+class Net {
+  public:
+    Net(int device, int storage);
+    ~Net();
+    void add_layer(const fyn_layer_desc& d);
+    void connect(int out_layer, int in_layer, int port);
+    void setup();
+    void forward(uint64_t* seq);
+    void finish();
+    Layer* layer(int number);
+    void set_input(int layer, int port, const float* data, int order);
+    void copy_result(int layer, float* chw, int include_padding);
+    void get_output(int layer, float* data, int order);
+    void copy_argmax(int layer, int32_t* idx, float* val);
+    void time_forward(int iters, float* ms);
+    void time_layer(int layer, int iters, float* ms);
+    void use_graph(bool enable);
+
+    int device;
+    int storage;  // fyn_storage
+    bool f16() const { return storage == FYN_STORAGE_F16; }
+    bool is_setup = false;
+    bool timings = false;
+    bool reuse_buffers = true;
+    std::string dump_dir;
+    hipStream_t stream = nullptr;
+    std::map<int, std::unique_ptr<Layer>> layers;  // ascending number = execution order
+    std::vector<Tensor> tensors;
+    std::vector<DevBuffer> buffers;
+    uint64_t seq = 0;
+
+    // device allocations owned by the net
+    void* dev_alloc(size_t bytes, bool zero = true);
+    float* staging(size_t floats);  // fp32 staging area for layout conversion
+
+  private:
+    void run_layers(bool with_events);
+    void collect_timings();
+    void dump_layer(Layer* l);
+    std::vector<void*> allocs_;
+    float* staging_ = nullptr;
+    size_t staging_floats_ = 0;
+    hipGraph_t graph_ = nullptr;
+    hipGraphExec_t graph_exec_ = nullptr;
+    bool graph_enabled_ = false;
+    bool events_pending_ = false;
+};
+
+Layer* create_layer(Net* net, const fyn_layer_desc& d);
+
+}  // namespace fynhip

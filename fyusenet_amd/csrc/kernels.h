@@ -1,0 +1,153 @@
+// Kernel parameter blocks and host-side launchers of the gfx950 layer kernels.
+//
+// Tensor layout in HBM (all kernels): channel-packed NHWC with a physical zero halo,
+//   element (y, x, c) of a tensor with net size HxW, halo `pad`, channel pitch `cp` lives at
+//   ((y + pad) * (W + 2*pad) + (x + pad)) * cp + c
+// cp = 4 for <= 4 channels, otherwise channels rounded up to a multiple of 8; pad lanes hold 0.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace fynhip {
+
+enum ActKind : int { ACT_NONE = 0, ACT_RELU = 1, ACT_LEAKY = 2, ACT_CLIP = 3 };
+
+struct Act {
+    int kind;
+    float leak, lo, hi;
+};
+
+// View of a device tensor as kernels see it.
+struct TView {
+    void* ptr;
+    int h, w;   // net size
+    int pad;    // halo width
+    int cp;     // channel pitch (elements)
+    int c;      // real channels
+    int f16;    // element type: 1 = __half, 0 = float
+    __host__ __device__ int wp() const { return w + 2 * pad; }
+    __host__ __device__ int hp() const { return h + 2 * pad; }
+    size_t elems() const { return (size_t)hp() * wp() * cp; }
+    size_t bytes() const { return elems() * (f16 ? 2 : 4); }
+};
+
+inline int channel_pitch(int c) { return c <= 4 ? 4 : (c + 7) / 8 * 8; }
+
+// ---------------------------------------------------------------------------------------------
+// MFMA implicit-GEMM convolution (conv_mfma.hip)
+// ---------------------------------------------------------------------------------------------
+struct ConvMfmaParams {
+    const void* in;
+    void* out;
+    const void* res;     // residual tensor or nullptr
+    const void* wpack;   // packed A fragments
+    const float* scale;  // [cout padded to block tile]
+    const float* bias;   // [cout padded to block tile]
+    const int* aoff;     // [nsteps] LDS byte offsets of the k16 steps of one channel chunk
+    // input tensor (stored frame)
+    int in_hp, in_wp, in_cp;
+    int in_y0, in_x0;    // stored coordinate sampled by tile-local (0,0) for output position (0,0)
+    int in_stride;       // input step per output position
+    // output positions computed by this launch
+    int npos_y, npos_x;
+    // output tensor addressing: stored y = out_off_y + pos_y * out_step
+    int out_wp, out_cp, out_step, out_off_y, out_off_x;
+    // residual tensor addressing (same net coordinates as the output)
+    int res_wp, res_cp, res_off_y, res_off_x;
+    int res_relu, res_scale;
+    // tiling
+    int tile_w_log2;     // positions per tile row = 1 << tile_w_log2
+    int tile_h;          // rows of positions per tile
+    int tiles_x, tiles_y;
+    int halo_w, halo_h;  // staged input tile size (pixels)
+    int pitch;           // LDS bytes per staged pixel (one plane)
+    int plane;           // LDS bytes of one plane (hi); lo plane follows when split
+    int cin_chunks, nsteps;
+    int mfrags;          // cout fragments (32 each) in wpack
+    int cout_blocks;     // grid size along cout
+    float acc_mul;       // exact power of two undoing the weight pre-scaling
+    Act act;
+};
+
+// Compile-time variant of the conv kernel.
+struct ConvVariant {
+    int in_f16, out_f16; // storage types
+    int split;           // 1: hi/lo fp16 split of both operands (fp32-accurate), 3 MFMAs per pair
+    int fm, fn;          // fragments (32 cout / 32 positions) per wave
+    int wm, wn;          // waves per block along cout / positions (wm*wn == 4)
+    int kc;              // input channels staged per chunk (4 = row-run small-Cin variant, 16, 32)
+};
+
+// Returns 0 when the variant exists and was launched.
+int launch_conv_mfma(const ConvVariant& v, const ConvMfmaParams& p, size_t lds_bytes, hipStream_t s);
+bool conv_mfma_variant_exists(const ConvVariant& v);
+
+// ---------------------------------------------------------------------------------------------
+// Direct (non-MFMA) layer kernels (layers_direct.hip)
+// ---------------------------------------------------------------------------------------------
+struct ConvDirectParams {
+    TView in, out, res;  // res.ptr == nullptr: none
+    const float* w;      // [ky][kx][cin][coutp] fp32 (coutp = out.cp)
+    const float* scale;
+    const float* bias;
+    int k, dil, stride;
+    int in_y0, in_x0;    // stored coord of tap (0,0) for output (0,0)
+    int clamp;           // 1: clamp to the net area edge (shallow unpadded rule)
+    int res_relu, res_scale;
+    Act act;
+};
+void launch_conv_direct(const ConvDirectParams& p, hipStream_t s);
+
+struct DwConvParams {
+    TView in, out, res;
+    const float* w;      // [9][cp] fp32
+    const float* scale;
+    const float* bias;
+    int dil, stride;
+    int res_relu, res_scale;
+    Act act;
+};
+void launch_dwconv3x3(const DwConvParams& p, hipStream_t s);
+
+struct PoolParams {
+    TView in, out;
+    int pool, stride;
+    int off;             // window start relative to stored (y*stride, x*stride)
+    int is_max;
+    Act act;
+};
+void launch_pool(const PoolParams& p, hipStream_t s);
+void launch_global_pool(const TView& in, const TView& out, int is_max, const Act& act, hipStream_t s);
+
+struct BnParams {
+    TView in, out, res;
+    const float* scale;
+    const float* bias;
+    int res_relu, res_bn;
+    Act act;
+};
+void launch_batchnorm(const BnParams& p, hipStream_t s);
+void launch_addsub(const TView& a, const TView& b, const TView& out, int sub, const Act& act, hipStream_t s);
+// Copies channels [0, in.c) of `in` to channels [c_off, c_off + in.c) of `out` (activated).
+void launch_concat_part(const TView& in, const TView& out, int c_off, const Act& act, hipStream_t s);
+// out: 2 channels (index as float, max value); idx_out optional int32 [h*w].
+void launch_argmax(const TView& in, const TView& out, int32_t* idx_out, const Act& act, hipStream_t s);
+
+struct GemvParams {
+    TView in, out;       // 1x1 spatial
+    const void* w;       // [cout][cinp] in storage type (f16) or fp32
+    int w_f16;
+    const float* scale;
+    const float* bias;
+    Act act;
+};
+void launch_gemv(const GemvParams& p, hipStream_t s);
+
+// Layout conversion between the engine layout and CHW fp32 staging buffers.
+void launch_chw_to_tensor(const float* chw, const TView& t, hipStream_t s);               // net area only
+void launch_tensor_to_chw(const TView& t, float* chw, int include_padding, hipStream_t s);
+void launch_hwc_to_tensor(const float* hwc, int pc, const TView& t, hipStream_t s);       // GPU_SHALLOW in
+void launch_tensor_to_hwc(const TView& t, float* hwc, int pc, hipStream_t s);             // GPU_SHALLOW out
+void launch_fill_zero(void* ptr, size_t bytes, hipStream_t s);
+
+}  // namespace fynhip

@@ -1,0 +1,841 @@
+// Layer objects: validation of the builder description (the rules of
+// GPULayerFactoryBackend::createLayer, fyusenet/gpu/gpulayerfactory.cpp:112-184,358-430,490-571),
+// weight-block parsing / repacking (gpu/deep/deepconvlayerbase.cpp:293-395 and friends) and kernel
+// selection + launch.
+#include <algorithm>
+#include <cmath>
+#include <cstdlib>
+#include <cstring>
+
+#include "engine.h"
+
+namespace fynhip {
+
+static inline uint16_t f2h_bits(float f) {
+    _Float16 h = (_Float16)f;  // round to nearest even
+    uint16_t b;
+    memcpy(&b, &h, 2);
+    return b;
+}
+static inline float h2f(uint16_t b) {
+    _Float16 h;
+    memcpy(&h, &b, 2);
+    return (float)h;
+}
+
+static int pow2ceil(int x) {
+    int p = 1;
+    while (p < x) p <<= 1;
+    return p;
+}
+static int ilog2(int x) {
+    int l = 0;
+    while ((1 << l) < x) l++;
+    return l;
+}
+
+template <typename T>
+static T* upload(Net* net, const std::vector<T>& host) {
+    T* dev = static_cast<T*>(net->dev_alloc(host.size() * sizeof(T), false));
+    FYN_HIP(hipMemcpyAsync(dev, host.data(), host.size() * sizeof(T), hipMemcpyHostToDevice, net->stream));
+    FYN_HIP(hipStreamSynchronize(net->stream));
+    return dev;
+}
+template <typename T>
+static void reupload(Net* net, T* dev, const std::vector<T>& host) {
+    FYN_HIP(hipStreamSynchronize(net->stream));
+    FYN_HIP(hipMemcpyAsync(dev, host.data(), host.size() * sizeof(T), hipMemcpyHostToDevice, net->stream));
+    FYN_HIP(hipStreamSynchronize(net->stream));
+}
+
+// scale / bias' of the convolution family from a weight block:
+//   bias' = bias*bnScale + bnBias, scale = bnScale (gpu/deep/deepconvlayerbase.cpp:360-382)
+static void fold_bn(const float* bias, const float* bn, int cout, bool post_bn, int padded, std::vector<float>& scale,
+                    std::vector<float>& biasp) {
+    scale.assign(padded, 0.f);
+    biasp.assign(padded, 0.f);
+    for (int o = 0; o < cout; o++) {
+        if (post_bn) {
+            scale[o] = bn[o];
+            biasp[o] = bias[o] * bn[o] + bn[cout + o];
+        } else {
+            scale[o] = 1.f;
+            biasp[o] = bias[o];
+        }
+    }
+}
+
+// =============================================================================================
+// MFMA convolution planning (shared by convolution and transposed convolution)
+// =============================================================================================
+struct Tap {
+    int oy, ox;  // offset (input pixels) inside the staged tile of the sample used by position (0,0)
+    int ky, kx;  // weight tap
+};
+
+struct SubConv {
+    std::vector<Tap> taps;
+    int span_y = 1, span_x = 1;  // staged tile = (tile-1)*in_stride + span
+    int in_y0 = 0, in_x0 = 0, in_stride = 1;
+    int npos_y = 0, npos_x = 0;
+    int out_step = 1, out_off_y = 0, out_off_x = 0;
+    int res_off_y = 0, res_off_x = 0;
+};
+
+struct MfmaLaunch {
+    ConvVariant var{};
+    ConvMfmaParams p{};
+    size_t lds = 0;
+    // host-side description of the k16 steps of one chunk: 16 (ky,kx,ci_rel) triples, ci_rel < 0 = zero
+    struct Step {
+        int aoff;
+        int ky[16], kx[16], ci[16];
+    };
+    std::vector<Step> steps;
+    void* wpack_dev = nullptr;
+    int* aoff_dev = nullptr;
+    size_t wpack_halves = 0;
+    int cin = 0, cout = 0;
+};
+
+struct TileChoice {
+    int fm, fn, wm, wn, twl, th;
+    double score;
+};
+
+static const int kTileTable[][4] = {{2, 2, 2, 2}, {2, 2, 1, 4}, {2, 1, 2, 2}, {2, 1, 1, 4},
+                                    {1, 2, 1, 4}, {1, 1, 1, 4}, {1, 1, 4, 1}, {1, 1, 2, 2}};
+
+static TileChoice choose_tile(int cout, const SubConv& sc, int pitch, int npl, int slack) {
+    TileChoice best{0, 0, 0, 0, 0, 0, -1.0};
+    const char* force = getenv("FYNHIP_CONV_TILE");  // "fm,fn,wm,wn" for experiments
+    int ff[4] = {0, 0, 0, 0};
+    if (force) sscanf(force, "%d,%d,%d,%d", &ff[0], &ff[1], &ff[2], &ff[3]);
+    for (const auto& t : kTileTable) {
+        const int fm = t[0], fn = t[1], wm = t[2], wn = t[3];
+        if (force && (fm != ff[0] || fn != ff[1] || wm != ff[2] || wn != ff[3])) continue;
+        const int bm = wn * fn * 32;
+        int tw = std::min(bm >= 128 ? 16 : 8, pow2ceil(sc.npos_x));
+        while (bm / tw > pow2ceil(sc.npos_y) && tw < pow2ceil(sc.npos_x) && tw < bm) tw *= 2;
+        const int th = bm / tw;
+        const int tiles = ((sc.npos_x + tw - 1) / tw) * ((sc.npos_y + th - 1) / th);
+        const int cpb = wm * fm * 32;
+        const int cblocks = (cout + cpb - 1) / cpb;
+        const int halo_w = (tw - 1) * sc.in_stride + sc.span_x, halo_h = (th - 1) * sc.in_stride + sc.span_y;
+        const size_t lds = (size_t)npl * ((size_t)halo_h * halo_w * pitch + slack);
+        if (lds > 150 * 1024) continue;
+        const double util = ((double)cout * sc.npos_x * sc.npos_y) / ((double)cblocks * cpb * (double)tiles * bm);
+        const double blocks = (double)tiles * cblocks;
+        const double slots = 256.0 * (lds > 72 * 1024 ? 1 : 2);
+        const double par = blocks >= slots ? blocks / (std::ceil(blocks / slots) * slots) : blocks / slots;
+        const double bonus = (fm * fn == 4) ? 1.0 : (fm * fn == 2 ? 0.85 : 0.7);
+        const double score = util * par * bonus;
+        if (score > best.score) best = TileChoice{fm, fn, wm, wn, ilog2(tw), th, score};
+    }
+    if (best.score < 0) fail(FYN_ERR_UNSUPPORTED, "no MFMA tile configuration fits this convolution");
+    return best;
+}
+
+// Builds the launch description of one (sub-)convolution; weights are packed separately.
+static MfmaLaunch plan_mfma(Net* net, const SubConv& sc, const TView& in, const TView& out, const TView* res, int cin,
+                            int cout, const Act& act, int res_relu, int res_scale) {
+    MfmaLaunch L;
+    L.cin = cin;
+    L.cout = cout;
+    const bool split = !net->f16();
+    const int npl = split ? 2 : 1;
+    int kc;
+    if (in.cp == 4) kc = 4;
+    else if (in.cp <= 16) kc = 16;
+    else kc = 32;
+    const int pitch = (kc == 4) ? 8 : kc * 2 + 16;
+    const int slack = (kc == 4) ? 64 : 0;
+    const TileChoice tc = choose_tile(cout, sc, pitch, npl, slack);
+    const int tw = 1 << tc.twl;
+    ConvMfmaParams& p = L.p;
+    p.in = in.ptr;
+    p.out = out.ptr;
+    p.res = res ? res->ptr : nullptr;
+    p.in_hp = in.hp(); p.in_wp = in.wp(); p.in_cp = in.cp;
+    p.in_y0 = sc.in_y0; p.in_x0 = sc.in_x0; p.in_stride = sc.in_stride;
+    p.npos_y = sc.npos_y; p.npos_x = sc.npos_x;
+    p.out_wp = out.wp(); p.out_cp = out.cp; p.out_step = sc.out_step;
+    p.out_off_y = sc.out_off_y; p.out_off_x = sc.out_off_x;
+    if (res) {
+        p.res_wp = res->wp(); p.res_cp = res->cp;
+        p.res_off_y = sc.res_off_y; p.res_off_x = sc.res_off_x;
+    }
+    p.res_relu = res_relu; p.res_scale = res_scale;
+    p.tile_w_log2 = tc.twl; p.tile_h = tc.th;
+    p.tiles_x = (sc.npos_x + tw - 1) / tw;
+    p.tiles_y = (sc.npos_y + tc.th - 1) / tc.th;
+    p.halo_w = (tw - 1) * sc.in_stride + sc.span_x;
+    p.halo_h = (tc.th - 1) * sc.in_stride + sc.span_y;
+    p.pitch = pitch;
+    p.plane = p.halo_h * p.halo_w * pitch + slack;
+    p.cin_chunks = (kc == 4) ? 1 : (in.cp + kc - 1) / kc;
+    const int cpb = tc.wm * tc.fm * 32;
+    p.cout_blocks = (cout + cpb - 1) / cpb;
+    p.mfrags = p.cout_blocks * tc.wm * tc.fm;
+    p.acc_mul = 1.f;
+    p.act = act;
+    L.lds = (size_t)npl * p.plane;
+    L.var = ConvVariant{in.f16, out.f16, split ? 1 : 0, tc.fm, tc.fn, tc.wm, tc.wn, kc};
+    if (!conv_mfma_variant_exists(L.var)) fail(FYN_ERR_UNSUPPORTED, "MFMA convolution variant not compiled");
+
+    // k16 steps
+    if (kc == 4) {
+        std::vector<Tap> taps = sc.taps;
+        std::sort(taps.begin(), taps.end(), [](const Tap& a, const Tap& b) { return a.oy != b.oy ? a.oy < b.oy : a.ox < b.ox; });
+        size_t i = 0;
+        while (i < taps.size()) {
+            size_t j = i + 1;
+            while (j < taps.size() && taps[j].oy == taps[i].oy && taps[j].ox == taps[j - 1].ox + 1) j++;
+            const int len = (int)(j - i);
+            const int nst = (len * 4 + 15) / 16;
+            for (int s = 0; s < nst; s++) {
+                MfmaLaunch::Step st;
+                st.aoff = (taps[i].oy * p.halo_w + taps[i].ox) * pitch + s * 32;
+                for (int e = 0; e < 16; e++) {
+                    const int r = s * 16 + e, q = r / 4;
+                    if (q < len) {
+                        st.ky[e] = taps[i + q].ky; st.kx[e] = taps[i + q].kx; st.ci[e] = r % 4;
+                    } else {
+                        st.ky[e] = st.kx[e] = 0; st.ci[e] = -1;
+                    }
+                }
+                L.steps.push_back(st);
+            }
+            i = j;
+        }
+    } else {
+        for (const Tap& t : sc.taps)
+            for (int sub = 0; sub < kc / 16; sub++) {
+                MfmaLaunch::Step st;
+                st.aoff = (t.oy * p.halo_w + t.ox) * pitch + sub * 32;
+                for (int e = 0; e < 16; e++) {
+                    st.ky[e] = t.ky; st.kx[e] = t.kx; st.ci[e] = sub * 16 + e;
+                }
+                L.steps.push_back(st);
+            }
+    }
+    p.nsteps = (int)L.steps.size();
+    std::vector<int> aoff(L.steps.size());
+    for (size_t i = 0; i < L.steps.size(); i++) aoff[i] = L.steps[i].aoff;
+    L.aoff_dev = upload(net, aoff);
+    p.aoff = L.aoff_dev;
+    L.wpack_halves = (size_t)p.cin_chunks * p.nsteps * p.mfrags * npl * 64 * 8;
+    L.wpack_dev = net->dev_alloc(L.wpack_halves * 2, false);
+    p.wpack = L.wpack_dev;
+    return L;
+}
+
+// Packs weights W[o][ky][kx][i] (block order, base/convlayerinterface.h:71-95) into the per-lane A
+// fragment order of the kernel: [(chunk, step)][mfrag][plane][lane][8 halves].
+static void pack_mfma_weights(Net* net, MfmaLaunch& L, const float* w, int k, float wmul) {
+    const ConvMfmaParams& p = L.p;
+    const int npl = L.var.split ? 2 : 1;
+    const int kc = L.var.kc;
+    std::vector<uint16_t> pack(L.wpack_halves, 0);
+    for (int chunk = 0; chunk < p.cin_chunks; chunk++)
+        for (int t = 0; t < p.nsteps; t++) {
+            const MfmaLaunch::Step& st = L.steps[t];
+            for (int mf = 0; mf < p.mfrags; mf++) {
+                uint16_t* base = pack.data() + ((((size_t)chunk * p.nsteps + t) * p.mfrags + mf) * npl) * 64 * 8;
+                for (int lane = 0; lane < 64; lane++) {
+                    const int o = mf * 32 + (lane & 31);
+                    if (o >= L.cout) continue;
+                    for (int j = 0; j < 8; j++) {
+                        const int e = 8 * (lane >> 5) + j;
+                        if (st.ci[e] < 0) continue;
+                        const int ci = chunk * kc + st.ci[e];
+                        if (ci >= L.cin) continue;
+                        const float v = w[(((size_t)o * k + st.ky[e]) * k + st.kx[e]) * L.cin + ci] * wmul;
+                        const uint16_t hi = f2h_bits(v);
+                        base[(size_t)lane * 8 + j] = hi;
+                        if (npl == 2) base[(size_t)(64 + lane) * 8 + j] = f2h_bits(v - h2f(hi));
+                    }
+                }
+            }
+        }
+    FYN_HIP(hipStreamSynchronize(net->stream));
+    FYN_HIP(hipMemcpyAsync(L.wpack_dev, pack.data(), pack.size() * 2, hipMemcpyHostToDevice, net->stream));
+    FYN_HIP(hipStreamSynchronize(net->stream));
+}
+
+// power of two that brings the largest weight magnitude to [2^11, 2^12): keeps hi and lo parts of the
+// fp16 split in the normal range; undone exactly by acc_mul in the epilogue
+static float weight_prescale(const float* w, size_t n) {
+    float mx = 0.f;
+    for (size_t i = 0; i < n; i++) mx = std::max(mx, std::fabs(w[i]));
+    if (mx == 0.f || !std::isfinite(mx)) return 1.f;
+    int e;
+    std::frexp(mx, &e);  // mx = m * 2^e, m in [0.5,1)
+    return std::ldexp(1.f, 12 - e);
+}
+
+static std::string mfma_info(const MfmaLaunch& L) {
+    char buf[256];
+    snprintf(buf, sizeof(buf), "conv_mfma %s tile=%dx%d(cout x pos) waves=%dx%d kc=%d th=%d tw=%d blocks=%d lds=%zu steps=%d chunks=%d",
+             L.var.split ? "f16x2-split" : "f16", L.var.wm * L.var.fm * 32, L.var.wn * L.var.fn * 32, L.var.wm, L.var.wn, L.var.kc,
+             L.p.tile_h, 1 << L.p.tile_w_log2, L.p.tiles_x * L.p.tiles_y * L.p.cout_blocks, L.lds, L.p.nsteps, L.p.cin_chunks);
+    return buf;
+}
+
+// =============================================================================================
+// Convolution (CONVOLUTION2D, non-depthwise)
+// =============================================================================================
+class ConvLayer : public Layer {
+  public:
+    ConvLayer(Net* n, const fyn_layer_desc& d_) : Layer(n, d_) {
+        k = d.kernel;
+        dil = d.dilation[0] > 0 ? d.dilation[0] : 1;
+        stride = d.downsample[0] > 0 ? d.downsample[0] : 1;
+        if ((k & 1) == 0 || k < 1) fail(FYN_ERR_UNSUPPORTED, "Unsupported convolution kernel size %d (%s)", k, d.name);
+        if (d.dilation[0] != d.dilation[1] && d.dilation[1] > 0) fail(FYN_ERR_UNSUPPORTED, "anisotropic dilation not supported (%s)", d.name);
+        if (d.downsample[0] != d.downsample[1] && d.downsample[1] > 0) fail(FYN_ERR_UNSUPPORTED, "anisotropic downsampling not supported (%s)", d.name);
+        oc = d.out_channels;
+        oh = d.height / stride;  // gpu/convlayerbase.cpp:47-48
+        ow = d.width / stride;
+        const int r = (k - 1) / 2;
+        // shallow, unpadded input: the sampler clamps to the edge (gpu/gpulayerbase.h:80-90)
+        clamp = !(d.flags & FYN_FLAG_DEEP) && d.input_padding < r * dil && k > 1;
+        direct = clamp || getenv("FYNHIP_FORCE_DIRECT_CONV") != nullptr;
+    }
+    size_t weight_floats() const override {
+        return (size_t)oc + (size_t)oc * k * k * d.in_channels + ((d.flags & FYN_FLAG_POST_BATCHNORM) ? 2 * (size_t)oc : 0);
+    }
+    void load_weights(const float* blk) override {
+        block.assign(blk, blk + weight_floats());
+        if (set_up) pack();
+    }
+    void setup() override {
+        const TView& in_v = tin(0).v;
+        const TView& out_v = tout().v;
+        const TView* res_v = (d.flags & FYN_FLAG_RESIDUAL_INPUT) ? &tin(1).v : nullptr;
+        const int r = (k - 1) / 2;
+        const int res_relu = (d.flags & FYN_FLAG_RELU_ON_RESIDUAL) ? 1 : 0;
+        const int res_scale = ((d.flags & FYN_FLAG_BATCHNORM_ON_RESIDUAL) && (d.flags & FYN_FLAG_POST_BATCHNORM)) ? 1 : 0;
+        if (direct) {
+            dp.in = in_v; dp.out = out_v;
+            dp.res = res_v ? *res_v : TView{};
+            dp.k = k; dp.dil = dil; dp.stride = stride;
+            dp.in_y0 = dp.in_x0 = in_v.pad - r * dil;
+            dp.clamp = clamp ? 1 : 0;
+            dp.res_relu = res_relu; dp.res_scale = res_scale;
+            dp.act = act();
+            padded = out_v.cp;
+            wdirect_dev = static_cast<float*>(net->dev_alloc((size_t)k * k * d.in_channels * out_v.cp * sizeof(float)));
+        } else {
+            SubConv sc;
+            for (int ky = 0; ky < k; ky++)
+                for (int kx = 0; kx < k; kx++) sc.taps.push_back(Tap{ky * dil, kx * dil, ky, kx});
+            sc.span_y = sc.span_x = (k - 1) * dil + 1;
+            sc.in_y0 = sc.in_x0 = in_v.pad - r * dil;
+            sc.in_stride = stride;
+            sc.npos_y = oh; sc.npos_x = ow;
+            sc.out_step = 1;
+            sc.out_off_y = sc.out_off_x = out_v.pad;
+            if (res_v) sc.res_off_y = sc.res_off_x = res_v->pad;
+            launch = plan_mfma(net, sc, in_v, out_v, res_v, d.in_channels, oc, act(), res_relu, res_scale);
+            padded = launch.p.mfrags * 32;
+        }
+        padded = std::max(padded, out_v.cp);
+        scale_dev = static_cast<float*>(net->dev_alloc(padded * sizeof(float)));
+        bias_dev = static_cast<float*>(net->dev_alloc(padded * sizeof(float)));
+        if (direct) {
+            dp.w = wdirect_dev; dp.scale = scale_dev; dp.bias = bias_dev;
+        } else {
+            launch.p.scale = scale_dev; launch.p.bias = bias_dev;
+        }
+        set_up = true;
+        if (!block.empty()) pack();
+    }
+    void pack() {
+        const float* bias = block.data();
+        const float* w = bias + oc;
+        const float* bn = w + (size_t)oc * k * k * d.in_channels;
+        std::vector<float> sc, bi;
+        fold_bn(bias, bn, oc, (d.flags & FYN_FLAG_POST_BATCHNORM) != 0, padded, sc, bi);
+        reupload(net, scale_dev, sc);
+        reupload(net, bias_dev, bi);
+        if (direct) {
+            const int cp = tout().v.cp, cin = d.in_channels;
+            std::vector<float> wd((size_t)k * k * cin * cp, 0.f);
+            for (int o = 0; o < oc; o++)
+                for (int ky = 0; ky < k; ky++)
+                    for (int kx = 0; kx < k; kx++)
+                        for (int i = 0; i < cin; i++)
+                            wd[(((size_t)ky * k + kx) * cin + i) * cp + o] = w[(((size_t)o * k + ky) * k + kx) * cin + i];
+            reupload(net, wdirect_dev, wd);
+        } else {
+            const float wmul = weight_prescale(w, (size_t)oc * k * k * d.in_channels);
+            launch.p.acc_mul = 1.0f / wmul;
+            pack_mfma_weights(net, launch, w, k, wmul);
+        }
+        have_weights = true;
+    }
+    void forward(hipStream_t s) override {
+        if (!have_weights) fail(FYN_ERR_STATE, "layer %s (%d): forward() without weights", d.name, d.number);
+        if (direct) launch_conv_direct(dp, s);
+        else if (launch_conv_mfma(launch.var, launch.p, launch.lds, s) != 0)
+            fail(FYN_ERR_DEVICE, "layer %s: convolution launch failed", d.name);
+    }
+    std::string info() const override { return direct ? (clamp ? "conv_direct(edge-clamp)" : "conv_direct") : mfma_info(launch); }
+
+    int k, dil, stride;
+    bool clamp = false, direct = false, have_weights = false;
+    int padded = 0;
+    std::vector<float> block;
+    MfmaLaunch launch;
+    ConvDirectParams dp{};
+    float *scale_dev = nullptr, *bias_dev = nullptr, *wdirect_dev = nullptr;
+};
+
+// =============================================================================================
+// Depthwise 3x3 convolution
+// =============================================================================================
+class DwConvLayer : public Layer {
+  public:
+    DwConvLayer(Net* n, const fyn_layer_desc& d_) : Layer(n, d_) {
+        dil = d.dilation[0] > 0 ? d.dilation[0] : 1;
+        stride = d.downsample[0] > 0 ? d.downsample[0] : 1;
+        if (d.out_channels != d.in_channels)
+            fail(FYN_ERR_UNSUPPORTED, "depthwise channel multiplier %d/%d not supported (%s)", d.out_channels, d.in_channels, d.name);
+        oc = d.out_channels;
+        oh = d.height / stride;
+        ow = d.width / stride;
+    }
+    size_t weight_floats() const override {
+        return (size_t)oc + 9 * (size_t)d.in_channels + ((d.flags & FYN_FLAG_POST_BATCHNORM) ? 2 * (size_t)oc : 0);
+    }
+    void load_weights(const float* blk) override {
+        block.assign(blk, blk + weight_floats());
+        if (set_up) pack();
+    }
+    void setup() override {
+        p.in = tin(0).v; p.out = tout().v;
+        p.res = (d.flags & FYN_FLAG_RESIDUAL_INPUT) ? tin(1).v : TView{};
+        p.dil = dil; p.stride = stride;
+        p.res_relu = (d.flags & FYN_FLAG_RELU_ON_RESIDUAL) ? 1 : 0;
+        p.res_scale = ((d.flags & FYN_FLAG_BATCHNORM_ON_RESIDUAL) && (d.flags & FYN_FLAG_POST_BATCHNORM)) ? 1 : 0;
+        p.act = act();
+        const int cp = p.out.cp;
+        w_dev = static_cast<float*>(net->dev_alloc(9 * (size_t)cp * sizeof(float)));
+        scale_dev = static_cast<float*>(net->dev_alloc(cp * sizeof(float)));
+        bias_dev = static_cast<float*>(net->dev_alloc(cp * sizeof(float)));
+        p.w = w_dev; p.scale = scale_dev; p.bias = bias_dev;
+        set_up = true;
+        if (!block.empty()) pack();
+    }
+    void pack() {
+        const int cp = tout().v.cp;
+        const float* bias = block.data();
+        const float* w = bias + oc;  // [(i*9 + ky*3+kx)] (gpu/deep/deepdwconvlayerbase.cpp:242, multiplier 1)
+        const float* bn = w + 9 * (size_t)d.in_channels;
+        std::vector<float> sc, bi, wd(9 * (size_t)cp, 0.f);
+        fold_bn(bias, bn, oc, (d.flags & FYN_FLAG_POST_BATCHNORM) != 0, cp, sc, bi);
+        for (int i = 0; i < oc; i++)
+            for (int t = 0; t < 9; t++) wd[(size_t)t * cp + i] = w[(size_t)i * 9 + t];
+        reupload(net, w_dev, wd);
+        reupload(net, scale_dev, sc);
+        reupload(net, bias_dev, bi);
+        have_weights = true;
+    }
+    void forward(hipStream_t s) override {
+        if (!have_weights) fail(FYN_ERR_STATE, "layer %s (%d): forward() without weights", d.name, d.number);
+        launch_dwconv3x3(p, s);
+    }
+    std::string info() const override { return "dwconv3x3"; }
+    int dil, stride;
+    bool have_weights = false;
+    std::vector<float> block;
+    DwConvParams p{};
+    float *w_dev = nullptr, *scale_dev = nullptr, *bias_dev = nullptr;
+};
+
+// =============================================================================================
+// Transposed convolution, stride 2, K in {2,3}: one MFMA sub-convolution per output parity
+// =============================================================================================
+class TransConvLayer : public Layer {
+  public:
+    TransConvLayer(Net* n, const fyn_layer_desc& d_) : Layer(n, d_) {
+        k = d.kernel;
+        // gpu/gpulayerfactory.cpp:410-411
+        if (k != 2 && k != 3) fail(FYN_ERR_UNSUPPORTED, "Transpose convolution is currently only implemented for 2x2 and 3x3 kernels");
+        if (d.upsample[0] != 2 || d.upsample[1] != 2) fail(FYN_ERR_UNSUPPORTED, "Transpose convolution requires upsample(2) (%s)", d.name);
+        if (d.flags & FYN_FLAG_RESIDUAL_INPUT) fail(FYN_ERR_UNSUPPORTED, "Residual input is not supported on transpose convolution (%s)", d.name);
+        crop = d.transconv_crop;
+        if (crop < 0 || crop >= k) fail(FYN_ERR_INVALID, "invalid transconv_crop %d (%s)", crop, d.name);
+        oc = d.out_channels;
+        oh = 2 * d.height + k - 2 - crop;  // gpu/deep/deeptiler.cpp:71-74
+        ow = 2 * d.width + k - 2 - crop;
+    }
+    size_t weight_floats() const override {
+        return (size_t)oc + (size_t)oc * k * k * d.in_channels + ((d.flags & FYN_FLAG_POST_BATCHNORM) ? 2 * (size_t)oc : 0);
+    }
+    void load_weights(const float* blk) override {
+        block.assign(blk, blk + weight_floats());
+        if (set_up) pack();
+    }
+    void setup() override {
+        const TView& in_v = tin(0).v;
+        const TView& out_v = tout().v;
+        padded = out_v.cp;
+        for (int py = 0; py < 2; py++)
+            for (int px = 0; px < 2; px++) {
+                SubConv sc;
+                // out[2a+py, 2b+px] = sum over dy,dx of W[py+2dy, px+2dx] * in[a-dy, b-dx]
+                const int ndy = (k - py + 1) / 2, ndx = (k - px + 1) / 2;
+                for (int dy = 0; dy < ndy; dy++)
+                    for (int dx = 0; dx < ndx; dx++) sc.taps.push_back(Tap{ndy - 1 - dy, ndx - 1 - dx, py + 2 * dy, px + 2 * dx});
+                sc.span_y = ndy; sc.span_x = ndx;
+                sc.in_y0 = in_v.pad - (ndy - 1);
+                sc.in_x0 = in_v.pad - (ndx - 1);
+                sc.in_stride = 1;
+                sc.npos_y = (oh - py + 1) / 2;
+                sc.npos_x = (ow - px + 1) / 2;
+                if (sc.npos_y <= 0 || sc.npos_x <= 0) continue;
+                sc.out_step = 2;
+                sc.out_off_y = out_v.pad + py;
+                sc.out_off_x = out_v.pad + px;
+                launches.push_back(plan_mfma(net, sc, in_v, out_v, nullptr, d.in_channels, oc, act(), 0, 0));
+                padded = std::max(padded, launches.back().p.mfrags * 32);
+            }
+        scale_dev = static_cast<float*>(net->dev_alloc(padded * sizeof(float)));
+        bias_dev = static_cast<float*>(net->dev_alloc(padded * sizeof(float)));
+        for (auto& L : launches) {
+            L.p.scale = scale_dev;
+            L.p.bias = bias_dev;
+        }
+        set_up = true;
+        if (!block.empty()) pack();
+    }
+    void pack() {
+        const float* bias = block.data();
+        const float* w = bias + oc;
+        const float* bn = w + (size_t)oc * k * k * d.in_channels;
+        std::vector<float> sc, bi;
+        fold_bn(bias, bn, oc, (d.flags & FYN_FLAG_POST_BATCHNORM) != 0, padded, sc, bi);
+        reupload(net, scale_dev, sc);
+        reupload(net, bias_dev, bi);
+        const float wmul = weight_prescale(w, (size_t)oc * k * k * d.in_channels);
+        for (auto& L : launches) {
+            L.p.acc_mul = 1.0f / wmul;
+            pack_mfma_weights(net, L, w, k, wmul);
+        }
+        have_weights = true;
+    }
+    void forward(hipStream_t s) override {
+        if (!have_weights) fail(FYN_ERR_STATE, "layer %s (%d): forward() without weights", d.name, d.number);
+        for (auto& L : launches)
+            if (launch_conv_mfma(L.var, L.p, L.lds, s) != 0) fail(FYN_ERR_DEVICE, "layer %s: transposed convolution launch failed", d.name);
+    }
+    std::string info() const override { return launches.empty() ? "transconv" : "transconv 4x " + mfma_info(launches[0]); }
+    int k, crop;
+    bool have_weights = false;
+    int padded = 0;
+    std::vector<float> block;
+    std::vector<MfmaLaunch> launches;
+    float *scale_dev = nullptr, *bias_dev = nullptr;
+};
+
+// =============================================================================================
+// GEMM (fully connected; 1x1 spatial)
+// =============================================================================================
+class GemmLayer : public Layer {
+  public:
+    GemmLayer(Net* n, const fyn_layer_desc& d_) : Layer(n, d_) {
+        if (d.width != 1 || d.height != 1) fail(FYN_ERR_UNSUPPORTED, "GEMM layer expects a 1x1 spatial input (%s)", d.name);
+        oc = d.out_channels;
+        oh = ow = 1;
+    }
+    size_t weight_floats() const override {
+        return (size_t)oc + (size_t)oc * d.in_channels + ((d.flags & FYN_FLAG_POST_BATCHNORM) ? 2 * (size_t)oc : 0);
+    }
+    void load_weights(const float* blk) override {
+        block.assign(blk, blk + weight_floats());
+        if (set_up) pack();
+    }
+    void setup() override {
+        p.in = tin(0).v; p.out = tout().v;
+        p.act = act();
+        p.w_f16 = net->f16() ? 1 : 0;
+        const size_t n = (size_t)p.out.cp * p.in.cp;
+        w_dev = net->dev_alloc(n * (p.w_f16 ? 2 : 4));
+        scale_dev = static_cast<float*>(net->dev_alloc(p.out.cp * sizeof(float)));
+        bias_dev = static_cast<float*>(net->dev_alloc(p.out.cp * sizeof(float)));
+        p.w = w_dev; p.scale = scale_dev; p.bias = bias_dev;
+        set_up = true;
+        if (!block.empty()) pack();
+    }
+    void pack() {
+        const int cinp = p.in.cp, cin = d.in_channels;
+        const float* bias = block.data();
+        const float* w = bias + oc;
+        const float* bn = w + (size_t)oc * cin;
+        std::vector<float> sc, bi;
+        fold_bn(bias, bn, oc, (d.flags & FYN_FLAG_POST_BATCHNORM) != 0, p.out.cp, sc, bi);
+        reupload(net, scale_dev, sc);
+        reupload(net, bias_dev, bi);
+        if (p.w_f16) {
+            std::vector<uint16_t> wd((size_t)p.out.cp * cinp, 0);
+            for (int o = 0; o < oc; o++)
+                for (int i = 0; i < cin; i++) wd[(size_t)o * cinp + i] = f2h_bits(w[(size_t)o * cin + i]);
+            reupload(net, static_cast<uint16_t*>(w_dev), wd);
+        } else {
+            std::vector<float> wd((size_t)p.out.cp * cinp, 0.f);
+            for (int o = 0; o < oc; o++)
+                for (int i = 0; i < cin; i++) wd[(size_t)o * cinp + i] = w[(size_t)o * cin + i];
+            reupload(net, static_cast<float*>(w_dev), wd);
+        }
+        have_weights = true;
+    }
+    void forward(hipStream_t s) override {
+        if (!have_weights) fail(FYN_ERR_STATE, "layer %s (%d): forward() without weights", d.name, d.number);
+        launch_gemv(p, s);
+    }
+    std::string info() const override { return "gemv"; }
+    bool have_weights = false;
+    std::vector<float> block;
+    GemvParams p{};
+    void* w_dev = nullptr;
+    float *scale_dev = nullptr, *bias_dev = nullptr;
+};
+
+// =============================================================================================
+// Pooling
+// =============================================================================================
+class PoolLayer : public Layer {
+  public:
+    PoolLayer(Net* n, const fyn_layer_desc& d_) : Layer(n, d_) {
+        is_max = d.type == FYN_LAYER_MAXPOOL2D;
+        global = d.global_pool != 0;
+        oc = d.in_channels;
+        if (d.out_channels != 0 && d.out_channels != d.in_channels)
+            fail(FYN_ERR_INVALID, "pooling layer %s must keep the channel count", d.name);
+        if (global) {
+            oh = ow = 1;
+        } else {
+            pool = d.pool_size[0];
+            // gpu/gpulayerfactory.cpp:542-544
+            if (d.pool_size[0] == 1 && d.pool_size[1] == 1)
+                fail(FYN_ERR_INVALID, "Pooling layer with a pool size of 1 does not make sense, clean your net (%s)", d.name);
+            if (d.pool_size[0] != d.pool_size[1] || pool < 1) fail(FYN_ERR_UNSUPPORTED, "anisotropic pooling not supported (%s)", d.name);
+            stride = d.downsample[0] > 0 ? d.downsample[0] : 1;
+            oh = d.height / stride;
+            ow = d.width / stride;
+        }
+    }
+    void setup() override {
+        p.in = tin(0).v; p.out = tout().v;
+        p.pool = pool; p.stride = stride; p.is_max = is_max; p.act = act();
+        // stored-frame window start relative to (y*stride, x*stride):
+        //   max: window begins input_padding before the stride origin (deepmaxpool.frag:15-45) -> 0
+        //   avg: P=3 window [-1,1], otherwise [0,P) from the origin (deepavgpool.frag:17-44)
+        p.off = is_max ? 0 : p.in.pad + (pool == 3 ? -1 : 0);
+    }
+    void forward(hipStream_t s) override {
+        if (global) launch_global_pool(tin(0).v, tout().v, is_max, act(), s);
+        else launch_pool(p, s);
+    }
+    std::string info() const override { return global ? "global_pool" : "pool"; }
+    bool is_max, global;
+    int pool = 1, stride = 1;
+    PoolParams p{};
+};
+
+// =============================================================================================
+// Explicit batch-norm, add/sub, concat, arg-max, upload, download
+// =============================================================================================
+class BatchNormLayer : public Layer {
+  public:
+    BatchNormLayer(Net* n, const fyn_layer_desc& d_) : Layer(n, d_) {
+        oc = d.in_channels;
+        oh = d.height;
+        ow = d.width;
+    }
+    size_t weight_floats() const override { return 2 * (size_t)oc; }
+    void load_weights(const float* blk) override {
+        block.assign(blk, blk + weight_floats());
+        if (set_up) pack();
+    }
+    void setup() override {
+        p.in = tin(0).v; p.out = tout().v;
+        p.res = (d.flags & FYN_FLAG_RESIDUAL_INPUT) ? tin(1).v : TView{};
+        p.res_relu = (d.flags & FYN_FLAG_RELU_ON_RESIDUAL) ? 1 : 0;
+        p.res_bn = (d.flags & FYN_FLAG_BATCHNORM_ON_RESIDUAL) ? 1 : 0;
+        p.act = act();
+        scale_dev = static_cast<float*>(net->dev_alloc(p.out.cp * sizeof(float)));
+        bias_dev = static_cast<float*>(net->dev_alloc(p.out.cp * sizeof(float)));
+        p.scale = scale_dev; p.bias = bias_dev;
+        set_up = true;
+        if (!block.empty()) pack();
+    }
+    void pack() {
+        std::vector<float> sc(p.out.cp, 0.f), bi(p.out.cp, 0.f);
+        for (int c = 0; c < oc; c++) {
+            sc[c] = block[c];
+            bi[c] = block[oc + c];
+        }
+        reupload(net, scale_dev, sc);
+        reupload(net, bias_dev, bi);
+        have_weights = true;
+    }
+    void forward(hipStream_t s) override {
+        if (!have_weights) fail(FYN_ERR_STATE, "layer %s (%d): forward() without scale/bias", d.name, d.number);
+        launch_batchnorm(p, s);
+    }
+    std::string info() const override { return "batchnorm"; }
+    bool have_weights = false;
+    std::vector<float> block;
+    BnParams p{};
+    float *scale_dev = nullptr, *bias_dev = nullptr;
+};
+
+class AddSubLayer : public Layer {
+  public:
+    AddSubLayer(Net* n, const fyn_layer_desc& d_) : Layer(n, d_) {
+        oc = d.in_channels;
+        oh = d.height;
+        ow = d.width;
+    }
+    int num_ports() const override { return 2; }
+    void port_shape(int, int& c, int& h, int& w, int& pad) const override {
+        c = d.in_channels; h = d.height; w = d.width; pad = d.input_padding;
+    }
+    void forward(hipStream_t s) override { launch_addsub(tin(0).v, tin(1).v, tout().v, d.type == FYN_LAYER_SUB, act(), s); }
+    std::string info() const override { return "addsub"; }
+};
+
+class ConcatLayer : public Layer {
+  public:
+    ConcatLayer(Net* n, const fyn_layer_desc& d_) : Layer(n, d_) {
+        if (d.num_inputs < 1 || d.num_inputs > FYN_MAX_CONCAT_INPUTS) fail(FYN_ERR_INVALID, "concat layer %s needs 1..%d inputs", d.name, FYN_MAX_CONCAT_INPUTS);
+        int total = 0;
+        bool all_relu = true;
+        for (int i = 0; i < d.num_inputs; i++) {
+            total += d.inputs[i].channels;
+            if (!(d.inputs[i].flags & FYN_FLAG_PRE_RELU)) all_relu = false;
+        }
+        oc = total;
+        oh = d.height;
+        ow = d.width;
+        // ReLU on fetch only if every input asks for it (gpu/deep/deepconcatlayer.cpp:40-49)
+        relu = all_relu || (d.flags & FYN_FLAG_PRE_RELU);
+    }
+    int num_ports() const override { return d.num_inputs; }
+    void port_shape(int port, int& c, int& h, int& w, int& pad) const override {
+        c = d.inputs[port].channels; h = d.height; w = d.width; pad = d.inputs[port].padding;
+    }
+    void forward(hipStream_t s) override {
+        Act a = act();
+        if (relu && a.kind == ACT_NONE) a.kind = ACT_RELU;
+        int off = 0;
+        for (int i = 0; i < d.num_inputs; i++) {
+            launch_concat_part(tin(i).v, tout().v, off, a, s);
+            off += d.inputs[i].channels;
+        }
+    }
+    std::string info() const override { return "concat"; }
+    bool relu;
+};
+
+class ArgMaxLayer : public Layer {
+  public:
+    ArgMaxLayer(Net* n, const fyn_layer_desc& d_) : Layer(n, d_) {
+        oc = 2;  // index, value (shaders/deep/deepargmax2.frag:15-20)
+        oh = d.height;
+        ow = d.width;
+    }
+    void setup() override { idx_dev = static_cast<int32_t*>(net->dev_alloc((size_t)oh * ow * sizeof(int32_t))); }
+    void forward(hipStream_t s) override { launch_argmax(tin(0).v, tout().v, idx_dev, act(), s); }
+    std::string info() const override { return "argmax"; }
+    int32_t* idx_dev = nullptr;
+};
+
+class UploadLayer : public Layer {
+  public:
+    UploadLayer(Net* n, const fyn_layer_desc& d_) : Layer(n, d_) {
+        // gpu/gpulayerfactory.cpp:276-278: uploads carry at most one texel's worth of channels
+        if (d.flags & FYN_FLAG_DEEP) fail(FYN_ERR_UNSUPPORTED, "Deep upload layers are not supported (%s)", d.name);
+        oc = d.out_channels ? d.out_channels : d.in_channels;
+        oh = d.height;
+        ow = d.width;
+    }
+    int num_ports() const override { return 0; }
+    void forward(hipStream_t) override {}
+    std::string info() const override { return "upload"; }
+};
+
+class DownloadLayer : public Layer {
+  public:
+    DownloadLayer(Net* n, const fyn_layer_desc& d_) : Layer(n, d_) {
+        oc = d.in_channels;
+        oh = d.height;
+        ow = d.width;
+    }
+    bool has_own_output() const override { return false; }
+    void forward(hipStream_t) override {}
+    std::string info() const override { return "download"; }
+};
+
+Layer* create_layer(Net* net, const fyn_layer_desc& d) {
+    if (d.width <= 0 || d.height <= 0 || d.width > 65535 || d.height > 65535)
+        fail(FYN_ERR_INVALID, "layer %s: invalid spatial size %dx%d", d.name, d.width, d.height);
+    if (d.in_channels <= 0 || d.in_channels > 32767 || d.out_channels < 0 || d.out_channels > 32767)
+        fail(FYN_ERR_INVALID, "layer %s: invalid channel counts %d -> %d", d.name, d.in_channels, d.out_channels);
+    if (d.input_padding < 0 || d.output_padding < 0 || d.residual_padding < 0)
+        fail(FYN_ERR_INVALID, "layer %s: negative padding", d.name);
+    Layer* l = nullptr;
+    switch (d.type) {
+        case FYN_LAYER_CONVOLUTION2D: {
+            // gpu/gpulayerfactory.cpp:358-396
+            const bool dw = d.group_size != 1 && d.group_size != 0 && d.group_size == d.in_channels;
+            if (dw) {
+                if (d.kernel == 1) fail(FYN_ERR_UNSUPPORTED, "No 1x1 depthwise layer supported");
+                if (d.kernel != 3) fail(FYN_ERR_UNSUPPORTED, "No %dx%d depthwise layer supported", d.kernel, d.kernel);
+                l = new DwConvLayer(net, d);
+            } else {
+                if (d.group_size > 1) fail(FYN_ERR_UNSUPPORTED, "grouped convolution (group size %d) not supported (%s)", d.group_size, d.name);
+                l = new ConvLayer(net, d);
+            }
+            break;
+        }
+        case FYN_LAYER_TRANSCONVOLUTION2D: l = new TransConvLayer(net, d); break;
+        case FYN_LAYER_GEMM: l = new GemmLayer(net, d); break;
+        case FYN_LAYER_MAXPOOL2D:
+        case FYN_LAYER_AVGPOOL2D: l = new PoolLayer(net, d); break;
+        case FYN_LAYER_BATCHNORM: l = new BatchNormLayer(net, d); break;
+        case FYN_LAYER_ADD:
+        case FYN_LAYER_SUB: l = new AddSubLayer(net, d); break;
+        case FYN_LAYER_CONCAT: l = new ConcatLayer(net, d); break;
+        case FYN_LAYER_ARGMAX:
+            // gpu/gpulayerfactory.cpp:791-815: arg-max exists for deep tensors only
+            if (!(d.flags & FYN_FLAG_DEEP)) fail(FYN_ERR_UNSUPPORTED, "ArgMax layer is only supported on deep tensors (%s)", d.name);
+            l = new ArgMaxLayer(net, d);
+            break;
+        case FYN_LAYER_UPLOAD: l = new UploadLayer(net, d); break;
+        case FYN_LAYER_DOWNLOAD: l = new DownloadLayer(net, d); break;
+        default: fail(FYN_ERR_UNSUPPORTED, "Unsupported layer type %d", d.type);
+    }
+    l->in.assign(l->num_ports(), -1);
+    return l;
+}
+
+void Net::copy_argmax(int layer_no, int32_t* idx, float* val) {
+    if (!is_setup) fail(FYN_ERR_STATE, "copy_argmax() before setup()");
+    FYN_HIP(hipSetDevice(device));
+    ArgMaxLayer* l = dynamic_cast<ArgMaxLayer*>(layer(layer_no));
+    if (!l) fail(FYN_ERR_INVALID, "layer %d is not an arg-max layer", layer_no);
+    const size_t n = (size_t)l->oh * l->ow;
+    FYN_HIP(hipStreamSynchronize(stream));
+    if (idx) FYN_HIP(hipMemcpy(idx, l->idx_dev, n * sizeof(int32_t), hipMemcpyDeviceToHost));
+    if (val) {
+        std::vector<float> chw(2 * n);
+        copy_result(layer_no, chw.data(), 0);
+        memcpy(val, chw.data() + n, n * sizeof(float));
+    }
+}
+
+}  // namespace fynhip

@@ -1,0 +1,524 @@
+// Bandwidth-bound layer kernels for gfx950 (no matrix cores): depthwise 3x3 convolution, pooling,
+// global pooling, explicit batch-norm, add/sub, concat, exact arg-max, the fully connected
+// matrix-vector product, a direct (fallback) convolution and the layout converters at the
+// upload/download boundary.  All operate on the channel-packed NHWC layout described in kernels.h;
+// one thread moves 4 consecutive channels of one pixel (16 B in fp32 storage, 8 B in fp16 storage),
+// consecutive threads touch consecutive channels, so every wavefront access is one contiguous run.
+// The activation of the producing layer is applied on input fetch (shaders/activation.inc:3-18).
+#include <hip/hip_fp16.h>
+#include <hip/hip_runtime.h>
+
+#include "kernels.h"
+
+namespace fynhip {
+
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+
+__device__ __forceinline__ float act1(float x, const Act& a) {
+    switch (a.kind) {
+        case ACT_RELU: return fmaxf(x, 0.f);
+        case ACT_LEAKY: return x >= 0.f ? x : a.leak * x;
+        case ACT_CLIP: return fminf(a.hi, fmaxf(a.lo, x));
+        default: return x;
+    }
+}
+__device__ __forceinline__ float4 act4(float4 v, const Act& a) {
+    return make_float4(act1(v.x, a), act1(v.y, a), act1(v.z, a), act1(v.w, a));
+}
+
+template <typename T>
+__device__ __forceinline__ float4 ld4(const T* p);
+template <>
+__device__ __forceinline__ float4 ld4<float>(const float* p) {
+    return *reinterpret_cast<const float4*>(p);
+}
+template <>
+__device__ __forceinline__ float4 ld4<_Float16>(const _Float16* p) {
+    half4_t h = *reinterpret_cast<const half4_t*>(p);
+    return make_float4((float)h[0], (float)h[1], (float)h[2], (float)h[3]);
+}
+template <typename T>
+__device__ __forceinline__ void st4(T* p, float4 v);
+template <>
+__device__ __forceinline__ void st4<float>(float* p, float4 v) {
+    *reinterpret_cast<float4*>(p) = v;
+}
+template <>
+__device__ __forceinline__ void st4<_Float16>(_Float16* p, float4 v) {
+    half4_t h;
+    h[0] = (_Float16)v.x; h[1] = (_Float16)v.y; h[2] = (_Float16)v.z; h[3] = (_Float16)v.w;
+    *reinterpret_cast<half4_t*>(p) = h;
+}
+
+__device__ __forceinline__ size_t tv_off(const TView& t, int y, int x) {  // net coords -> element offset
+    return ((size_t)(y + t.pad) * t.wp() + (x + t.pad)) * t.cp;
+}
+
+#define FYN_DISPATCH_T(f16, KERNEL, grid, block, stream, ...)                                   \
+    do {                                                                                        \
+        if (f16) hipLaunchKernelGGL((KERNEL<_Float16>), grid, block, 0, stream, __VA_ARGS__);   \
+        else hipLaunchKernelGGL((KERNEL<float>), grid, block, 0, stream, __VA_ARGS__);          \
+    } while (0)
+
+static inline dim3 grid1d(size_t n, int block) { return dim3((unsigned)((n + block - 1) / block)); }
+
+// ---------------------------------------------------------------------------------------------
+// depthwise 3x3  (DeepDepthwiseConvLayer3x3::forward, gpu/deep/deepdwconvlayer3x3.cpp:67-102;
+//                 shaders/deep/deepconv_dw3x3_tiled.frag:36-59)
+// ---------------------------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void dwconv3x3_kernel(const DwConvParams p) {
+    const int cg = p.out.cp >> 2;
+    const size_t n = (size_t)p.out.h * p.out.w * cg;
+    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= n) return;
+    const int g = (int)(idx % cg);
+    const size_t pix = idx / cg;
+    const int x = (int)(pix % p.out.w), y = (int)(pix / p.out.w);
+    const int c = g * 4;
+    const T* in = reinterpret_cast<const T*>(p.in.ptr);
+    const int iwp = p.in.wp(), ihp = p.in.hp();
+    const int yc = y * p.stride + p.in.pad, xc = x * p.stride + p.in.pad;
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+    for (int ky = 0; ky < 3; ky++) {
+#pragma unroll
+        for (int kx = 0; kx < 3; kx++) {
+            const int sy = yc + (ky - 1) * p.dil, sx = xc + (kx - 1) * p.dil;
+            float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+            if ((unsigned)sy < (unsigned)ihp && (unsigned)sx < (unsigned)iwp)
+                v = ld4<T>(in + ((size_t)sy * iwp + sx) * p.in.cp + c);
+            v = act4(v, p.act);
+            const float4 w = *reinterpret_cast<const float4*>(p.w + (ky * 3 + kx) * p.out.cp + c);
+            acc.x = fmaf(v.x, w.x, acc.x); acc.y = fmaf(v.y, w.y, acc.y);
+            acc.z = fmaf(v.z, w.z, acc.z); acc.w = fmaf(v.w, w.w, acc.w);
+        }
+    }
+    const float4 sc = *reinterpret_cast<const float4*>(p.scale + c);
+    const float4 bi = *reinterpret_cast<const float4*>(p.bias + c);
+    float4 o = make_float4(acc.x * sc.x + bi.x, acc.y * sc.y + bi.y, acc.z * sc.z + bi.z, acc.w * sc.w + bi.w);
+    if (p.res.ptr) {
+        float4 r = ld4<T>(reinterpret_cast<const T*>(p.res.ptr) + tv_off(p.res, y, x) + c);
+        if (p.res_relu) r = make_float4(fmaxf(r.x, 0.f), fmaxf(r.y, 0.f), fmaxf(r.z, 0.f), fmaxf(r.w, 0.f));
+        if (p.res_scale) r = make_float4(r.x * sc.x, r.y * sc.y, r.z * sc.z, r.w * sc.w);
+        o = make_float4(o.x + r.x, o.y + r.y, o.z + r.z, o.w + r.w);
+    }
+    st4<T>(reinterpret_cast<T*>(p.out.ptr) + tv_off(p.out, y, x) + c, o);
+}
+void launch_dwconv3x3(const DwConvParams& p, hipStream_t s) {
+    const size_t n = (size_t)p.out.h * p.out.w * (p.out.cp >> 2);
+    FYN_DISPATCH_T(p.out.f16, dwconv3x3_kernel, grid1d(n, 256), dim3(256), s, p);
+}
+
+// ---------------------------------------------------------------------------------------------
+// max / average pooling  (DeepPoolingLayer::forward, gpu/deep/deeppoolinglayer.cpp:109-131;
+//                         shaders/deep/deepmaxpool.frag:12-59, deepavgpool.frag:15-58)
+// ---------------------------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void pool_kernel(const PoolParams p) {
+    const int cg = p.out.cp >> 2;
+    const size_t n = (size_t)p.out.h * p.out.w * cg;
+    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= n) return;
+    const int g = (int)(idx % cg);
+    const size_t pix = idx / cg;
+    const int x = (int)(pix % p.out.w), y = (int)(pix / p.out.w);
+    const int c = g * 4;
+    const T* in = reinterpret_cast<const T*>(p.in.ptr);
+    const int iwp = p.in.wp(), ihp = p.in.hp();
+    const int y0 = y * p.stride + p.off, x0 = x * p.stride + p.off;  // stored coordinates
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int py = 0; py < p.pool; py++) {
+        for (int px = 0; px < p.pool; px++) {
+            const int sy = y0 + py, sx = x0 + px;
+            float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+            if ((unsigned)sy < (unsigned)ihp && (unsigned)sx < (unsigned)iwp)
+                v = ld4<T>(in + ((size_t)sy * iwp + sx) * p.in.cp + c);
+            v = act4(v, p.act);
+            if (p.is_max) {
+                if (py == 0 && px == 0) acc = v;
+                else acc = make_float4(fmaxf(acc.x, v.x), fmaxf(acc.y, v.y), fmaxf(acc.z, v.z), fmaxf(acc.w, v.w));
+            } else {
+                acc = make_float4(acc.x + v.x, acc.y + v.y, acc.z + v.z, acc.w + v.w);
+            }
+        }
+    }
+    if (!p.is_max) {
+        const float inv = 1.0f / (float)(p.pool * p.pool);
+        acc = make_float4(acc.x * inv, acc.y * inv, acc.z * inv, acc.w * inv);
+    }
+    st4<T>(reinterpret_cast<T*>(p.out.ptr) + tv_off(p.out, y, x) + c, acc);
+}
+void launch_pool(const PoolParams& p, hipStream_t s) {
+    const size_t n = (size_t)p.out.h * p.out.w * (p.out.cp >> 2);
+    FYN_DISPATCH_T(p.out.f16, pool_kernel, grid1d(n, 256), dim3(256), s, p);
+}
+
+// ---------------------------------------------------------------------------------------------
+// global pooling  (DeepGlobalPoolLayer, gpu/deep/deepglobalpoollayer.cpp:55-135;
+//                  shaders/deep/deepglobavgpool.frag:15-24).  One block per run of up to 64
+// channel groups; the block's threads split the pixels, partial results meet in LDS.
+// ---------------------------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void global_pool_kernel(const TView in, const TView out, int is_max, const Act act,
+                                                          int cgb_log2) {
+    __shared__ float4 red[256];
+    const int cgs = in.cp >> 2;
+    const int cgb = 1 << cgb_log2;             // channel groups handled by this block
+    const int parts = 256 >> cgb_log2;         // pixel partitions
+    const int lg = threadIdx.x & (cgb - 1);
+    const int part = threadIdx.x >> cgb_log2;
+    const int g = blockIdx.x * cgb + lg;
+    const int npix = in.h * in.w;
+    const T* src = reinterpret_cast<const T*>(in.ptr);
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    bool first = true;
+    if (g < cgs) {
+        for (int pix = part; pix < npix; pix += parts) {
+            const int y = pix / in.w, x = pix - y * in.w;
+            float4 v = act4(ld4<T>(src + tv_off(in, y, x) + g * 4), act);
+            if (is_max) {
+                acc = first ? v : make_float4(fmaxf(acc.x, v.x), fmaxf(acc.y, v.y), fmaxf(acc.z, v.z), fmaxf(acc.w, v.w));
+                first = false;
+            } else {
+                acc = make_float4(acc.x + v.x, acc.y + v.y, acc.z + v.z, acc.w + v.w);
+            }
+        }
+    }
+    if (is_max && first) acc = make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
+    red[threadIdx.x] = acc;
+    __syncthreads();
+    for (int st = parts >> 1; st > 0; st >>= 1) {
+        if (part < st) {
+            float4 a = red[threadIdx.x], b = red[threadIdx.x + st * cgb];
+            red[threadIdx.x] = is_max ? make_float4(fmaxf(a.x, b.x), fmaxf(a.y, b.y), fmaxf(a.z, b.z), fmaxf(a.w, b.w))
+                                      : make_float4(a.x + b.x, a.y + b.y, a.z + b.z, a.w + b.w);
+        }
+        __syncthreads();
+    }
+    if (part == 0 && g < cgs) {
+        float4 r = red[threadIdx.x];
+        if (!is_max) {
+            const float inv = 1.0f / (float)npix;
+            r = make_float4(r.x * inv, r.y * inv, r.z * inv, r.w * inv);
+        }
+        st4<T>(reinterpret_cast<T*>(out.ptr) + tv_off(out, 0, 0) + g * 4, r);
+    }
+}
+void launch_global_pool(const TView& in, const TView& out, int is_max, const Act& act, hipStream_t s) {
+    const int cgs = in.cp >> 2;
+    int l2 = 0;
+    while ((1 << l2) < cgs && l2 < 6) l2++;
+    const int cgb = 1 << l2;
+    FYN_DISPATCH_T(in.f16, global_pool_kernel, dim3((cgs + cgb - 1) / cgb), dim3(256), s, in, out, is_max, act, l2);
+}
+
+// ---------------------------------------------------------------------------------------------
+// explicit batch-norm (DeepBatchNormLayer, shaders/deep/deepbatchnorm.frag:24-36), add/sub
+// (shaders/add.frag) and one input of a concatenation (shaders/deep/deepconcat.frag:45-76)
+// ---------------------------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void batchnorm_kernel(const BnParams p) {
+    const int cg = p.out.cp >> 2;
+    const size_t n = (size_t)p.out.h * p.out.w * cg;
+    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= n) return;
+    const int g = (int)(idx % cg);
+    const size_t pix = idx / cg;
+    const int x = (int)(pix % p.out.w), y = (int)(pix / p.out.w);
+    const int c = g * 4;
+    float4 v = act4(ld4<T>(reinterpret_cast<const T*>(p.in.ptr) + tv_off(p.in, y, x) + c), p.act);
+    const float4 sc = *reinterpret_cast<const float4*>(p.scale + c);
+    const float4 bi = *reinterpret_cast<const float4*>(p.bias + c);
+    float4 o = make_float4(v.x * sc.x + bi.x, v.y * sc.y + bi.y, v.z * sc.z + bi.z, v.w * sc.w + bi.w);
+    if (p.res.ptr) {
+        float4 r = ld4<T>(reinterpret_cast<const T*>(p.res.ptr) + tv_off(p.res, y, x) + c);
+        if (p.res_relu) r = make_float4(fmaxf(r.x, 0.f), fmaxf(r.y, 0.f), fmaxf(r.z, 0.f), fmaxf(r.w, 0.f));
+        if (p.res_bn) r = make_float4(r.x * sc.x + bi.x, r.y * sc.y + bi.y, r.z * sc.z + bi.z, r.w * sc.w + bi.w);
+        o = make_float4(o.x + r.x, o.y + r.y, o.z + r.z, o.w + r.w);
+    }
+    st4<T>(reinterpret_cast<T*>(p.out.ptr) + tv_off(p.out, y, x) + c, o);
+}
+void launch_batchnorm(const BnParams& p, hipStream_t s) {
+    const size_t n = (size_t)p.out.h * p.out.w * (p.out.cp >> 2);
+    FYN_DISPATCH_T(p.out.f16, batchnorm_kernel, grid1d(n, 256), dim3(256), s, p);
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void addsub_kernel(const TView a, const TView b, const TView out, int sub, const Act act) {
+    const int cg = out.cp >> 2;
+    const size_t n = (size_t)out.h * out.w * cg;
+    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= n) return;
+    const int g = (int)(idx % cg);
+    const size_t pix = idx / cg;
+    const int x = (int)(pix % out.w), y = (int)(pix / out.w);
+    const int c = g * 4;
+    float4 u = act4(ld4<T>(reinterpret_cast<const T*>(a.ptr) + tv_off(a, y, x) + c), act);
+    float4 v = act4(ld4<T>(reinterpret_cast<const T*>(b.ptr) + tv_off(b, y, x) + c), act);
+    float4 o = sub ? make_float4(u.x - v.x, u.y - v.y, u.z - v.z, u.w - v.w)
+                   : make_float4(u.x + v.x, u.y + v.y, u.z + v.z, u.w + v.w);
+    st4<T>(reinterpret_cast<T*>(out.ptr) + tv_off(out, y, x) + c, o);
+}
+void launch_addsub(const TView& a, const TView& b, const TView& out, int sub, const Act& act, hipStream_t s) {
+    const size_t n = (size_t)out.h * out.w * (out.cp >> 2);
+    FYN_DISPATCH_T(out.f16, addsub_kernel, grid1d(n, 256), dim3(256), s, a, b, out, sub, act);
+}
+
+// Channel offsets that are not multiples of 4 (the "component shift" case of deepconcat.frag) are
+// handled per element; aligned offsets move whole 4-channel vectors.
+template <typename T>
+__global__ __launch_bounds__(256) void concat_kernel(const TView in, const TView out, int c_off, const Act act) {
+    const int cg = (in.c + 3) >> 2;
+    const size_t n = (size_t)out.h * out.w * cg;
+    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= n) return;
+    const int g = (int)(idx % cg);
+    const size_t pix = idx / cg;
+    const int x = (int)(pix % out.w), y = (int)(pix / out.w);
+    const int c = g * 4;
+    const T* src = reinterpret_cast<const T*>(in.ptr) + tv_off(in, y, x) + c;
+    T* dst = reinterpret_cast<T*>(out.ptr) + tv_off(out, y, x) + c_off + c;
+    if ((c_off & 3) == 0 && c + 4 <= in.c) {
+        st4<T>(dst, act4(ld4<T>(src), act));
+    } else {
+        for (int i = 0; i < 4 && c + i < in.c; i++) dst[i] = (T)act1((float)src[i], act);
+    }
+}
+void launch_concat_part(const TView& in, const TView& out, int c_off, const Act& act, hipStream_t s) {
+    const size_t n = (size_t)out.h * out.w * ((in.c + 3) >> 2);
+    FYN_DISPATCH_T(out.f16, concat_kernel, grid1d(n, 256), dim3(256), s, in, out, c_off, act);
+}
+
+// ---------------------------------------------------------------------------------------------
+// exact arg-max over channels, lowest index among maxima (replaces the mantissa-bit approximation of
+// DeepArgMaxLayer::forward, gpu/deep/deepargmaxlayer.cpp:113-152).  L lanes cooperate on one pixel and
+// merge with cross-lane shuffles (DPP / ds_swizzle on gfx950).
+// ---------------------------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void argmax_kernel(const TView in, const TView out, int32_t* idx_out, const Act act,
+                                                     int l_log2) {
+    const int L = 1 << l_log2;
+    const int lane = threadIdx.x & 63;
+    const int sub = lane & (L - 1);
+    const int ppw = 64 >> l_log2;  // pixels per wave
+    const size_t wave = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const size_t pix = wave * ppw + (lane >> l_log2);
+    const size_t npix = (size_t)in.h * in.w;
+    const bool valid = pix < npix;
+    const int x = valid ? (int)(pix % in.w) : 0, y = valid ? (int)(pix / in.w) : 0;
+    const T* src = reinterpret_cast<const T*>(in.ptr) + tv_off(in, y, x);
+    float best = -INFINITY;
+    int bidx = 0x7fffffff;
+    const int cgs = (in.c + 3) >> 2;
+    if (valid) {
+        for (int g = sub; g < cgs; g += L) {
+            float4 v = act4(ld4<T>(src + g * 4), act);
+            const float vv[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int c = g * 4 + i;
+                if (c < in.c && (vv[i] > best || (vv[i] == best && c < bidx))) {
+                    best = vv[i];
+                    bidx = c;
+                }
+            }
+        }
+    }
+    for (int o = L >> 1; o > 0; o >>= 1) {
+        const float ob = __shfl_xor(best, o, 64);
+        const int oi = __shfl_xor(bidx, o, 64);
+        if (ob > best || (ob == best && oi < bidx)) {
+            best = ob;
+            bidx = oi;
+        }
+    }
+    if (valid && sub == 0) {
+        T* dst = reinterpret_cast<T*>(out.ptr) + tv_off(out, y, x);
+        st4<T>(dst, make_float4((float)bidx, best, 0.f, 0.f));
+        if (idx_out) idx_out[pix] = bidx;
+    }
+}
+void launch_argmax(const TView& in, const TView& out, int32_t* idx_out, const Act& act, hipStream_t s) {
+    const int cgs = (in.c + 3) >> 2;
+    int l2 = 0;
+    while ((1 << l2) < cgs && l2 < 6) l2++;
+    const size_t npix = (size_t)in.h * in.w;
+    const size_t ppw = 64 >> l2;
+    const size_t waves = (npix + ppw - 1) / ppw;
+    FYN_DISPATCH_T(in.f16, argmax_kernel, dim3((unsigned)((waves + 3) / 4)), dim3(256), s, in, out, idx_out, act, l2);
+}
+
+// ---------------------------------------------------------------------------------------------
+// fully connected layer as a matrix-vector product (DeepGEMMLayer::forward,
+// gpu/deep/deepgemmlayer.cpp:66-236): one wavefront per output row, the row of weights is streamed
+// once from HBM in 16-byte pieces, partial sums meet with cross-lane shuffles.
+// ---------------------------------------------------------------------------------------------
+template <typename T, typename TW>
+__global__ __launch_bounds__(256) void gemv_kernel(const GemvParams p) {
+    const int lane = threadIdx.x & 63;
+    const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= p.out.cp) return;
+    const int cinp = p.in.cp;
+    const T* x = reinterpret_cast<const T*>(p.in.ptr) + tv_off(p.in, 0, 0);
+    const TW* w = reinterpret_cast<const TW*>(p.w) + (size_t)row * cinp;
+    float acc = 0.f;
+    if (row < p.out.c) {
+        for (int c = lane * 4; c < cinp; c += 256) {
+            float4 xv = act4(ld4<T>(x + c), p.act);
+            float4 wv = ld4<TW>(w + c);
+            acc = fmaf(xv.x, wv.x, acc); acc = fmaf(xv.y, wv.y, acc);
+            acc = fmaf(xv.z, wv.z, acc); acc = fmaf(xv.w, wv.w, acc);
+        }
+    }
+    for (int o = 32; o > 0; o >>= 1) acc += __shfl_xor(acc, o, 64);
+    if (lane == 0) {
+        float r = (row < p.out.c) ? acc * p.scale[row] + p.bias[row] : 0.f;
+        reinterpret_cast<T*>(p.out.ptr)[tv_off(p.out, 0, 0) + row] = (T)r;
+    }
+}
+void launch_gemv(const GemvParams& p, hipStream_t s) {
+    dim3 grid((p.out.cp + 3) / 4), block(256);
+    if (p.out.f16) {
+        if (p.w_f16) hipLaunchKernelGGL((gemv_kernel<_Float16, _Float16>), grid, block, 0, s, p);
+        else hipLaunchKernelGGL((gemv_kernel<_Float16, float>), grid, block, 0, s, p);
+    } else {
+        if (p.w_f16) hipLaunchKernelGGL((gemv_kernel<float, _Float16>), grid, block, 0, s, p);
+        else hipLaunchKernelGGL((gemv_kernel<float, float>), grid, block, 0, s, p);
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// direct convolution (fallback for what the MFMA path does not take: edge-clamped shallow layers,
+// unusual strides).  fp32 FMA, one thread = one output pixel x 4 output channels.
+// ---------------------------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void conv_direct_kernel(const ConvDirectParams p) {
+    const int cg = p.out.cp >> 2;
+    const size_t n = (size_t)p.out.h * p.out.w * cg;
+    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= n) return;
+    const int g = (int)(idx % cg);
+    const size_t pix = idx / cg;
+    const int x = (int)(pix % p.out.w), y = (int)(pix / p.out.w);
+    const int c = g * 4;
+    const T* in = reinterpret_cast<const T*>(p.in.ptr);
+    const int iwp = p.in.wp(), ihp = p.in.hp();
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int ky = 0; ky < p.k; ky++) {
+        for (int kx = 0; kx < p.k; kx++) {
+            int sy = y * p.stride + p.in_y0 + ky * p.dil, sx = x * p.stride + p.in_x0 + kx * p.dil;
+            bool ok = true;
+            if (p.clamp) {
+                sy = min(max(sy, p.in.pad), p.in.pad + p.in.h - 1);
+                sx = min(max(sx, p.in.pad), p.in.pad + p.in.w - 1);
+            } else {
+                ok = (unsigned)sy < (unsigned)ihp && (unsigned)sx < (unsigned)iwp;
+            }
+            const T* src = in + ((size_t)sy * iwp + sx) * p.in.cp;
+            const float* w = p.w + ((size_t)(ky * p.k + kx) * p.in.c) * p.out.cp + c;
+            for (int ci = 0; ci < p.in.c; ci++) {
+                const float v = act1(ok ? (float)src[ci] : 0.f, p.act);
+                const float4 wv = *reinterpret_cast<const float4*>(w + (size_t)ci * p.out.cp);
+                acc.x = fmaf(v, wv.x, acc.x); acc.y = fmaf(v, wv.y, acc.y);
+                acc.z = fmaf(v, wv.z, acc.z); acc.w = fmaf(v, wv.w, acc.w);
+            }
+        }
+    }
+    const float4 sc = *reinterpret_cast<const float4*>(p.scale + c);
+    const float4 bi = *reinterpret_cast<const float4*>(p.bias + c);
+    float4 o = make_float4(acc.x * sc.x + bi.x, acc.y * sc.y + bi.y, acc.z * sc.z + bi.z, acc.w * sc.w + bi.w);
+    if (p.res.ptr) {
+        float4 r = ld4<T>(reinterpret_cast<const T*>(p.res.ptr) + tv_off(p.res, y, x) + c);
+        if (p.res_relu) r = make_float4(fmaxf(r.x, 0.f), fmaxf(r.y, 0.f), fmaxf(r.z, 0.f), fmaxf(r.w, 0.f));
+        if (p.res_scale) r = make_float4(r.x * sc.x, r.y * sc.y, r.z * sc.z, r.w * sc.w);
+        o = make_float4(o.x + r.x, o.y + r.y, o.z + r.z, o.w + r.w);
+    }
+    st4<T>(reinterpret_cast<T*>(p.out.ptr) + tv_off(p.out, y, x) + c, o);
+}
+void launch_conv_direct(const ConvDirectParams& p, hipStream_t s) {
+    const size_t n = (size_t)p.out.h * p.out.w * (p.out.cp >> 2);
+    FYN_DISPATCH_T(p.out.f16, conv_direct_kernel, grid1d(n, 256), dim3(256), s, p);
+}
+
+// ---------------------------------------------------------------------------------------------
+// layout converters (UploadLayer / DownloadLayer / GPULayerBase::copyResult formats)
+// ---------------------------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void chw_to_tensor_kernel(const float* chw, const TView t) {
+    const size_t n = (size_t)t.h * t.w * t.cp;
+    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= n) return;
+    const int c = (int)(idx % t.cp);
+    const size_t pix = idx / t.cp;
+    const int x = (int)(pix % t.w), y = (int)(pix / t.w);
+    const float v = c < t.c ? chw[((size_t)c * t.h + y) * t.w + x] : 0.f;
+    reinterpret_cast<T*>(t.ptr)[tv_off(t, y, x) + c] = (T)v;
+}
+void launch_chw_to_tensor(const float* chw, const TView& t, hipStream_t s) {
+    FYN_DISPATCH_T(t.f16, chw_to_tensor_kernel, grid1d((size_t)t.h * t.w * t.cp, 256), dim3(256), s, chw, t);
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void tensor_to_chw_kernel(const TView t, float* chw, int keep_pad) {
+    const int oh = keep_pad ? t.hp() : t.h, ow = keep_pad ? t.wp() : t.w;
+    const size_t n = (size_t)t.c * oh * ow;
+    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= n) return;
+    const int x = (int)(idx % ow);
+    const int y = (int)((idx / ow) % oh);
+    const int c = (int)(idx / ((size_t)ow * oh));
+    const int sy = keep_pad ? y : y + t.pad, sx = keep_pad ? x : x + t.pad;
+    chw[idx] = (float)reinterpret_cast<const T*>(t.ptr)[((size_t)sy * t.wp() + sx) * t.cp + c];
+}
+void launch_tensor_to_chw(const TView& t, float* chw, int include_padding, hipStream_t s) {
+    const int oh = include_padding ? t.hp() : t.h, ow = include_padding ? t.wp() : t.w;
+    FYN_DISPATCH_T(t.f16, tensor_to_chw_kernel, grid1d((size_t)t.c * oh * ow, 256), dim3(256), s, t, chw, include_padding);
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void hwc_to_tensor_kernel(const float* hwc, int pc, const TView t) {
+    const size_t n = (size_t)t.h * t.w * t.cp;
+    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= n) return;
+    const int c = (int)(idx % t.cp);
+    const size_t pix = idx / t.cp;
+    const int x = (int)(pix % t.w), y = (int)(pix / t.w);
+    const float v = (c < t.c && c < pc) ? hwc[pix * pc + c] : 0.f;
+    reinterpret_cast<T*>(t.ptr)[tv_off(t, y, x) + c] = (T)v;
+}
+void launch_hwc_to_tensor(const float* hwc, int pc, const TView& t, hipStream_t s) {
+    FYN_DISPATCH_T(t.f16, hwc_to_tensor_kernel, grid1d((size_t)t.h * t.w * t.cp, 256), dim3(256), s, hwc, pc, t);
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void tensor_to_hwc_kernel(const TView t, float* hwc, int pc) {
+    const size_t n = (size_t)t.h * t.w * pc;
+    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= n) return;
+    const int c = (int)(idx % pc);
+    const size_t pix = idx / pc;
+    const int x = (int)(pix % t.w), y = (int)(pix / t.w);
+    hwc[idx] = c < t.c ? (float)reinterpret_cast<const T*>(t.ptr)[tv_off(t, y, x) + c] : 0.f;
+}
+void launch_tensor_to_hwc(const TView& t, float* hwc, int pc, hipStream_t s) {
+    FYN_DISPATCH_T(t.f16, tensor_to_hwc_kernel, grid1d((size_t)t.h * t.w * pc, 256), dim3(256), s, t, hwc, pc);
+}
+
+__global__ __launch_bounds__(256) void fill_zero_kernel(uint4* p, size_t n16, unsigned char* tail, size_t ntail) {
+    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * 256;
+    for (size_t i = idx; i < n16; i += stride) p[i] = make_uint4(0, 0, 0, 0);
+    if (idx < ntail) tail[idx] = 0;
+}
+void launch_fill_zero(void* ptr, size_t bytes, hipStream_t s) {
+    const size_t n16 = bytes / 16;
+    size_t blocks = (n16 + 255) / 256;
+    if (blocks > 4096) blocks = 4096;
+    if (blocks == 0) blocks = 1;
+    hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)blocks), dim3(256), 0, s, reinterpret_cast<uint4*>(ptr), n16,
+                       reinterpret_cast<unsigned char*>(ptr) + n16 * 16, bytes - n16 * 16);
+}
+
+}  // namespace fynhip

@@ -1,0 +1,250 @@
+"""NeuralNetwork / LayerFactory / BufferManager surface on top of the C ABI.
+
+Mirrors the way the reference's networks are written (samples/samplenetworks/resnet50.cpp:200-536):
+a NeuralNetwork subclass implements buildLayers() (builders pushed into a LayerFactory),
+connectLayers(layers, bufferManager) and initializeWeights(layers); setup() runs them in the order
+of NeuralNetwork::glSetup (fyusenet/base/neuralnetwork.cpp:238-250).
+"""
+import ctypes
+
+import numpy as np
+
+from . import capi
+from .builders import LayerType
+
+
+class Layer:
+    """Handle of one compiled layer (LayerBase / GPULayerBase of the reference)."""
+
+    def __init__(self, net, builder):
+        self._net = net
+        self.builder = builder
+        self.number = builder.number_
+        self.name = builder.name_
+        self.weights = None  # host copy of the loaded block (kept for descriptions handed to checkers)
+
+    def getNumber(self):
+        return self.number
+
+    def getName(self):
+        return self.name
+
+    def loadWeightsAndBiases(self, data, offset=0):
+        """ConvLayerInterface::loadWeightsAndBiases (base/convlayerinterface.h:95)."""
+        data = np.ascontiguousarray(data, dtype=np.float32)
+        n = self.weightFloats()
+        if offset + n > data.size:
+            raise capi.FynException(capi.ERR_INVALID, "weight block of layer %s exceeds the supplied array" % self.name)
+        self.weights = data[offset:offset + n].copy()
+        capi.check(capi.lib().fyn_layer_load_weights(self._net._h, self.number, capi.fptr(data), offset))
+
+    def loadScaleAndBias(self, data, offset=0):
+        """BatchNormInterface::loadScaleAndBias (base/batchnorminterface.h:146)."""
+        data = np.ascontiguousarray(data, dtype=np.float32)
+        n = self.weightFloats()
+        if offset + n > data.size:
+            raise capi.FynException(capi.ERR_INVALID, "scale/bias block of layer %s exceeds the supplied array" % self.name)
+        self.weights = data[offset:offset + n].copy()
+        capi.check(capi.lib().fyn_layer_load_scale_bias(self._net._h, self.number, capi.fptr(data), offset))
+
+    def weightFloats(self):
+        n = ctypes.c_size_t(0)
+        capi.check(capi.lib().fyn_layer_weight_floats(self._net._h, self.number, ctypes.byref(n)))
+        return n.value
+
+    def outputShape(self):
+        c, h, w, p = ctypes.c_int(), ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+        capi.check(capi.lib().fyn_layer_output_shape(self._net._h, self.number, ctypes.byref(c), ctypes.byref(h),
+                                                     ctypes.byref(w), ctypes.byref(p)))
+        return c.value, h.value, w.value, p.value
+
+    def copyResult(self, includePadding=False):
+        """GPULayerBase::copyResult (gpu/gpulayerbase.cpp:525-564): CHW fp32."""
+        c, h, w, p = self.outputShape()
+        if includePadding:
+            h, w = h + 2 * p, w + 2 * p
+        out = np.empty((c, h, w), dtype=np.float32)
+        capi.check(capi.lib().fyn_layer_copy_result(self._net._h, self.number, capi.fptr(out), 1 if includePadding else 0))
+        return out
+
+    def setInput(self, data, port=0, order=capi.ORDER_CHANNELWISE):
+        data = np.ascontiguousarray(data, dtype=np.float32)
+        capi.check(capi.lib().fyn_net_set_input(self._net._h, self.number, port, capi.fptr(data), order))
+
+    def kernelInfo(self):
+        buf = ctypes.create_string_buffer(512)
+        capi.check(capi.lib().fyn_layer_kernel_info(self._net._h, self.number, buf, len(buf)))
+        return buf.value.decode()
+
+    def timeKernel(self, iters):
+        ms = ctypes.c_float(0)
+        capi.check(capi.lib().fyn_layer_time(self._net._h, self.number, iters, ctypes.byref(ms)))
+        return ms.value / iters
+
+
+class CompiledLayers:
+    """base/compiledlayers.h:50-291: number- and name-indexed layer store, ascending iteration."""
+
+    def __init__(self):
+        self._by_number = {}
+        self._by_name = {}
+
+    def _add(self, layer):
+        self._by_number[layer.number] = layer
+        self._by_name[layer.name] = layer
+
+    def __getitem__(self, key):
+        try:
+            return self._by_name[key] if isinstance(key, str) else self._by_number[key]
+        except KeyError:
+            raise capi.FynException(capi.ERR_NOTFOUND, "no layer %r" % (key,))
+
+    def __iter__(self):
+        return iter(self._by_number[k] for k in sorted(self._by_number))
+
+    def __len__(self):
+        return len(self._by_number)
+
+
+class LayerFactory:
+    """base/layerfactory.h:56-138."""
+
+    def __init__(self, net):
+        self._net = net
+        self._builders = {}
+
+    def pushBuilder(self, builder):
+        # base/layerfactory.cpp:67-76
+        if builder.number_ < 0:
+            raise capi.FynException(capi.ERR_INVALID, "Must identify each layer with a valid number (found %d in the builder)" % builder.number_)
+        if int(builder.type_) >= int(LayerType.LAST_SUPPORTED):
+            raise capi.FynException(capi.ERR_UNSUPPORTED, "Unsupported layer type %d" % int(builder.type_))
+        if builder.number_ in self._builders:
+            raise capi.FynException(capi.ERR_DUPLICATE, "Trying to insert a layer on a position that is already taken (%d)" % builder.number_)
+        self._builders[builder.number_] = builder
+
+    def compileLayers(self):
+        layers = CompiledLayers()
+        for no in sorted(self._builders):
+            b = self._builders[no]
+            d = b.desc()
+            capi.check(capi.lib().fyn_net_add_layer(self._net._h, ctypes.byref(d)))
+            layers._add(Layer(self._net, b))
+        return layers
+
+
+class BufferManager:
+    """base/buffermanager.cpp:160-184 (connectLayers); tensors live in the engine."""
+
+    def __init__(self, net):
+        self._net = net
+        self.connections = []
+
+    def connectLayers(self, outputLayer, inputLayer, port=0):
+        capi.check(capi.lib().fyn_net_connect(self._net._h, outputLayer.number, inputLayer.number, port))
+        self.connections.append((outputLayer.number, inputLayer.number, port))
+
+
+class NeuralNetwork:
+    """base/neuralnetwork.h:62-261.  storage: capi.STORAGE_F32 (HIGH_PRECISION) or STORAGE_F16."""
+
+    def __init__(self, storage=capi.STORAGE_F32, device=0):
+        self.storage = storage
+        self._h = ctypes.c_void_p()
+        capi.check(capi.lib().fyn_net_create(device, storage, ctypes.byref(self._h)))
+        self.layers = None
+        self.bufferManager = None
+        self._setup = False
+
+    # -- to be provided by the network description --
+    def buildLayers(self, factory):
+        raise NotImplementedError
+
+    def connectLayers(self, layers, bufferManager):
+        raise NotImplementedError
+
+    def initializeWeights(self, layers):
+        pass
+
+    # -- life cycle --
+    def setup(self, reuseBuffers=True):
+        if self._setup:
+            raise capi.FynException(capi.ERR_STATE, "network is already set up")
+        capi.check(capi.lib().fyn_net_set_buffer_reuse(self._h, 1 if reuseBuffers else 0))
+        factory = LayerFactory(self)
+        self.buildLayers(factory)
+        self.layers = factory.compileLayers()
+        self.bufferManager = BufferManager(self)
+        self.connectLayers(self.layers, self.bufferManager)
+        self.initializeWeights(self.layers)
+        capi.check(capi.lib().fyn_net_setup(self._h))
+        self._setup = True
+
+    def forward(self):
+        seq = ctypes.c_uint64(0)
+        capi.check(capi.lib().fyn_net_forward(self._h, ctypes.byref(seq)))
+        return seq.value
+
+    def finish(self):
+        capi.check(capi.lib().fyn_net_finish(self._h))
+
+    def cleanup(self):
+        if self._h:
+            capi.check(capi.lib().fyn_net_destroy(self._h))
+            self._h = ctypes.c_void_p()
+
+    def __del__(self):
+        try:
+            self.cleanup()
+        except Exception:
+            pass
+
+    # -- I/O and instrumentation --
+    def getOutput(self, layer, order=capi.ORDER_CHANNELWISE):
+        lyr = self.layers[layer] if not isinstance(layer, Layer) else layer
+        c, h, w, p = lyr.outputShape()
+        if order == capi.ORDER_CHANNELWISE:
+            out = np.empty((c, h, w), dtype=np.float32)
+        elif order == capi.ORDER_GPU_SHALLOW:
+            out = np.empty((h, w, 4 if c == 3 else c), dtype=np.float32)
+        else:
+            from .formats import deep_tiling
+            tx, ty = deep_tiling(c)
+            out = np.empty((ty * (h + p) + p, tx * (w + p) + p, 4), dtype=np.float32)
+        capi.check(capi.lib().fyn_net_get_output(self._h, lyr.number, capi.fptr(out), order))
+        return out
+
+    def getArgMax(self, layer):
+        lyr = self.layers[layer] if not isinstance(layer, Layer) else layer
+        c, h, w, p = lyr.outputShape()
+        idx = np.empty((h, w), dtype=np.int32)
+        val = np.empty((h, w), dtype=np.float32)
+        capi.check(capi.lib().fyn_layer_copy_argmax(self._h, lyr.number, idx.ctypes.data_as(ctypes.POINTER(ctypes.c_int32)), capi.fptr(val)))
+        return idx, val
+
+    def enableTimings(self, enable=True):
+        capi.check(capi.lib().fyn_net_enable_timings(self._h, 1 if enable else 0))
+
+    def getTiming(self, layer):
+        ms, runs = ctypes.c_float(0), ctypes.c_int(0)
+        capi.check(capi.lib().fyn_net_get_timing(self._h, layer, ctypes.byref(ms), ctypes.byref(runs)))
+        return ms.value, runs.value
+
+    def enableIntermediateOutput(self, directory):
+        capi.check(capi.lib().fyn_net_enable_intermediate_output(self._h, directory.encode() if directory else None))
+
+    def useGraph(self, enable=True):
+        capi.check(capi.lib().fyn_net_use_graph(self._h, 1 if enable else 0))
+
+    def timeForward(self, iters):
+        ms = ctypes.c_float(0)
+        capi.check(capi.lib().fyn_net_time_forward(self._h, iters, ctypes.byref(ms)))
+        return ms.value
+
+    def describe(self):
+        """Plain description of the graph (descs, edges, loaded weight blocks) for external checkers."""
+        out = []
+        for lyr in self.layers:
+            b = lyr.builder
+            out.append({"builder": b, "number": lyr.number, "weights": lyr.weights})
+        return {"layers": out, "connections": list(self.bufferManager.connections), "storage": self.storage}

@@ -1,0 +1,201 @@
+/*
+ * fynhip -- C ABI of the MI355X (gfx950) engine for FyuseNet's GPU layer stack.
+ *
+ * The reference exposes this path only as C++ classes; every entry point below names the reference
+ * interface it stands in for (paths relative to the reference tree).  All functions return 0 on
+ * success and a negative fyn_status on failure (exceptions never cross this boundary; the message the
+ * reference would have put into a FynException is available from fyn_last_error()).
+ *
+ * Threading: like NeuralNetwork::forward (fyusenet/base/neuralnetwork.cpp:169) a network is not
+ * re-entrant; one thread drives one network.  Different networks may be driven from different
+ * threads.  Pointers passed in are borrowed for the duration of the call only (weights are copied
+ * and repacked, as in fyusenet/gpu/deep/deepconvlayerbase.cpp:308-353).
+ */
+#ifndef FYNHIP_H
+#define FYNHIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct fyn_net fyn_net; /* opaque: NeuralNetwork + Engine + BufferManager of one network */
+
+enum fyn_status {
+    FYN_OK = 0,
+    FYN_ERR_INVALID = -1,     /* bad argument / inconsistent description (reference: FynException)   */
+    FYN_ERR_UNSUPPORTED = -2, /* layer type / kernel size not supported (gpulayerfactory.cpp:182)    */
+    FYN_ERR_STATE = -3,       /* call out of order (forward before setup, add after setup ...)       */
+    FYN_ERR_DEVICE = -4,      /* HIP runtime error                                                  */
+    FYN_ERR_NOTFOUND = -5,    /* unknown layer number                                               */
+    FYN_ERR_DUPLICATE = -6    /* layer number already in use (base/layerfactory.cpp:73)              */
+};
+
+/* Storage type of activations and weights.  FYN_STORAGE_F32 is the reference's HIGH_PRECISION build,
+ * FYN_STORAGE_F16 its default build (fyusenet/gpu/gpulayerbase.h:100-110). */
+enum fyn_storage { FYN_STORAGE_F32 = 0, FYN_STORAGE_F16 = 1 };
+
+/* Numeric values of LayerType (fyusenet/base/layerflags.h:125-160); only the types of the GPU layer
+ * stack handled here are listed, any other value yields FYN_ERR_UNSUPPORTED. */
+enum fyn_layer_type {
+    FYN_LAYER_ADD = 1,
+    FYN_LAYER_SUB = 2,
+    FYN_LAYER_ARGMAX = 3,
+    FYN_LAYER_CONCAT = 5,
+    FYN_LAYER_CONVOLUTION2D = 6,
+    FYN_LAYER_TRANSCONVOLUTION2D = 8,
+    FYN_LAYER_AVGPOOL2D = 9,
+    FYN_LAYER_MAXPOOL2D = 10,
+    FYN_LAYER_DOWNLOAD = 26,
+    FYN_LAYER_UPLOAD = 27,
+    FYN_LAYER_BATCHNORM = 30,
+    FYN_LAYER_GEMM = 31
+};
+
+/* LayerFlags bits (fyusenet/base/layerflags.h:33-50), as LayerBuilderTempl::getFlags() composes them
+ * (fyusenet/base/layerbuilder.h:445-493). */
+enum fyn_layer_flags {
+    FYN_FLAG_RESIDUAL_INPUT = 1,
+    FYN_FLAG_RELU_ON_RESIDUAL = 2,
+    FYN_FLAG_BATCHNORM_ON_RESIDUAL = 4,
+    FYN_FLAG_POST_BATCHNORM = 8,
+    FYN_FLAG_DEEP = 16,
+    FYN_FLAG_PRE_RELU = 64,
+    FYN_FLAG_PRE_CLIP = 128
+};
+
+/* ActType (fyusenet/base/layerflags.h:61-68). */
+enum fyn_act { FYN_ACT_NONE = 0, FYN_ACT_RELU = 1, FYN_ACT_LEAKY_RELU = 2, FYN_ACT_CLIP = 3 };
+
+/* Host buffer orders (CPUBufferShape::order, fyusenet/cpu/cpubuffershape.h). */
+enum fyn_order {
+    FYN_ORDER_CHANNELWISE = 0, /* [C][H][W]                                                         */
+    FYN_ORDER_GPU_SHALLOW = 1, /* [H][W][pc] interleaved, pc = channels (<= 4 channels per texel)    */
+    FYN_ORDER_GPU_DEEP = 2     /* tiled RGBA, cpu/cpubuffer.cpp:413-442, cpubuffershape.cpp:430-448  */
+};
+
+#define FYN_MAX_CONCAT_INPUTS 8
+#define FYN_NAME_LEN 64
+
+/*
+ * One layer description: the fields of LayerBuilderTempl (fyusenet/base/layerbuilder.h:497-521) plus
+ * those of ConvLayerBuilder (gpu/convlayerbuilder.h), PoolLayerBuilder (gpu/poollayerbuilder.h) and
+ * ConcatLayerBuilder (gpu/concatlayerbuilder.h).  The struct is copied by fyn_net_add_layer; no
+ * ownership is taken.  Zero-initialise it, set struct_size = sizeof(fyn_layer_desc), fill what the
+ * builder would have filled.  width/height/in_channels describe the INPUT tensor, as shape() does.
+ */
+typedef struct fyn_layer_desc {
+    uint32_t struct_size;
+    int32_t type;   /* fyn_layer_type                                                   type()            */
+    int32_t number; /* unique, layers execute in ascending number                       number()          */
+    char name[FYN_NAME_LEN];
+    uint32_t flags; /* fyn_layer_flags                                                  getFlags()        */
+    int32_t width, height, in_channels, out_channels; /*                               shape()           */
+    int32_t input_padding, output_padding, residual_padding; /*          inputPadding() ...               */
+    int32_t downsample[2]; /* x, y                                                      downsample()      */
+    int32_t upsample[2];   /* x, y                                                      upsample()        */
+    float leaky_relu;      /* != 0 with PRE_RELU: leaky ReLU                            leakyReLU()       */
+    float clip_low, clip_high; /* with PRE_CLIP                                         clip()            */
+    /* convolution family */
+    int32_t kernel;      /* isotropic kernel size                                       ConvLayerBuilder  */
+    int32_t dilation[2]; /*                                                             dilation()        */
+    int32_t group_size;  /* == in_channels and kernel 3: depthwise                      groupSize()       */
+    /* pooling */
+    int32_t pool_size[2]; /*                                                            poolSize()        */
+    int32_t global_pool;  /*                                                            global()          */
+    /* concatenation */
+    int32_t num_inputs;
+    struct {
+        int32_t channels, padding;
+        uint32_t flags;
+    } inputs[FYN_MAX_CONCAT_INPUTS]; /*                                                  input()           */
+    /* Extension without a reference counterpart: rows/columns cropped from the end of a transposed
+     * convolution's full (2H+K-2) result; 0 reproduces the reference's deep layer size
+     * (gpu/deep/deeptiler.cpp:71-74), 1 with K=3 yields the 2H size of the shallow layer
+     * (gpu/vanilla/transconvlayerbase_vanilla.cpp:61-62). */
+    int32_t transconv_crop;
+} fyn_layer_desc;
+
+/* Thread-local text of the last failure (what the reference would have thrown). */
+const char* fyn_last_error(void);
+
+/* Library / device information: writes a short text (device name, CU count, arch) into buf. */
+int fyn_device_info(int device, char* buf, size_t buflen);
+
+/* NeuralNetwork construction (fyusenet/base/neuralnetwork.h:62-261); storage = fyn_storage. */
+int fyn_net_create(int device, int storage, fyn_net** out);
+/* NeuralNetwork::cleanup + destructor (base/neuralnetwork.cpp:57-79). */
+int fyn_net_destroy(fyn_net* net);
+
+/* LayerFactory::pushBuilder + LayerFactoryBackend::createLayer (base/layerfactory.cpp:67-101,
+ * gpu/gpulayerfactory.cpp:112-184). */
+int fyn_net_add_layer(fyn_net* net, const fyn_layer_desc* desc);
+
+/* BufferManager::connectLayers(outputLayer, inputLayer, port) (base/buffermanager.cpp:160-184):
+ * port 0 = data, port 1 = residual; concat ports 0..N-1. */
+int fyn_net_connect(fyn_net* net, int out_layer, int in_layer, int port);
+
+/* ConvLayerInterface::loadWeightsAndBiases(const float*, size_t offset) (base/convlayerinterface.h:95):
+ * block at wb+offset = [bias][weights [o][ky][kx][i]][bnScale][bnBias].  May be called again after
+ * setup to swap weights (samples/samplenetworks/stylenet3x3.cpp:81-89). */
+int fyn_layer_load_weights(fyn_net* net, int layer, const float* wb, size_t offset_floats);
+/* BatchNormInterface::loadScaleAndBias (base/batchnorminterface.h:146): [scale C][bias C]. */
+int fyn_layer_load_scale_bias(fyn_net* net, int layer, const float* sb, size_t offset_floats);
+/* Number of floats the layer's block occupies (to step through a .dat stream). */
+int fyn_layer_weight_floats(fyn_net* net, int layer, size_t* count);
+
+/* NeuralNetwork::setup -> glSetup (base/neuralnetwork.cpp:88-103,238-250): allocates device tensors,
+ * packs weights, selects kernels. */
+int fyn_net_setup(fyn_net* net);
+
+/* UploadLayer::setInputBuffer + upload (gpu/uploadlayer.cpp:92-186): host fp32 buffer in `order`
+ * for the UPLOAD layer `layer`; for any other layer: writes the tensor on input port `port`
+ * directly (what LayerTestBase::generateTextures does, unit_tests/layertestbase.cpp:208-417). */
+int fyn_net_set_input(fyn_net* net, int layer, int port, const float* data, int order);
+
+/* NeuralNetwork::forward (base/neuralnetwork.cpp:173-187): runs all layers in ascending number on
+ * the network's stream; returns the sequence number used.  Asynchronous w.r.t. the host. */
+int fyn_net_forward(fyn_net* net, uint64_t* seq_out);
+/* NeuralNetwork::finish (base/neuralnetwork.cpp:196-206): waits for the stream. */
+int fyn_net_finish(fyn_net* net);
+
+/* GPULayerBase::copyResult(float*, bool) (gpu/gpulayerbase.cpp:525-564): output of `layer` as CHW
+ * fp32; include_padding != 0 keeps the output halo.  Synchronises. */
+int fyn_layer_copy_result(fyn_net* net, int layer, float* chw, int include_padding);
+/* Output geometry of a layer: channels, height, width (net size) and padding. */
+int fyn_layer_output_shape(fyn_net* net, int layer, int* channels, int* height, int* width, int* padding);
+/* DownloadLayer / CPUBuffer formats (gpu/deep/deepdownloadlayer.cpp:136-162, cpu/cpubuffer.cpp):
+ * output of `layer` (padding stripped unless GPU_DEEP, which keeps the layer's output padding) as
+ * fp32 in the requested fyn_order.  Synchronises. */
+int fyn_net_get_output(fyn_net* net, int layer, float* data, int order);
+/* ArgMax result as integers (index per pixel), the exact form of deepargmax2.frag's first channel. */
+int fyn_layer_copy_argmax(fyn_net* net, int layer, int32_t* idx, float* val);
+
+/* Engine::enableTimings / resetTimings (base/engine.cpp:208-233); here per-layer GPU time from
+ * hipEvents.  fyn_net_get_timing returns the accumulated milliseconds and run count of one layer. */
+int fyn_net_enable_timings(fyn_net* net, int enable);
+int fyn_net_get_timing(fyn_net* net, int layer, float* ms_total, int* runs);
+/* Engine::enableIntermediateOutput(dir) (base/engine.cpp:174-181): <name>_<seq>.bin CHW fp32 dumps. */
+int fyn_net_enable_intermediate_output(fyn_net* net, const char* dir);
+
+/* Output-buffer sharing between layers whose lifetimes do not overlap (the texture pool of
+ * BufferManager::findTexture, base/buffermanager.cpp:512-525).  On by default; switch off before
+ * fyn_net_setup to keep every intermediate tensor readable with fyn_layer_copy_result after forward. */
+int fyn_net_set_buffer_reuse(fyn_net* net, int enable);
+
+/* Replays forward() from a captured hipGraph (launch-latency removal; no reference counterpart). */
+int fyn_net_use_graph(fyn_net* net, int enable);
+
+/* Measurement helpers (no reference counterpart): time `iters` forwards between two hipEvents on the
+ * network's stream; per-layer variant times one layer's kernels alone.  Milliseconds total. */
+int fyn_net_time_forward(fyn_net* net, int iters, float* ms_total);
+int fyn_layer_time(fyn_net* net, int layer, int iters, float* ms_total);
+/* Text description of the kernel variant chosen for a layer (for profiles / reports). */
+int fyn_layer_kernel_info(fyn_net* net, int layer, char* buf, size_t buflen);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FYNHIP_H */

@@ -1,0 +1,119 @@
+"""Parity of the HIP convolution family against the CPU oracle, through the C ABI (ctypes).
+
+Tolerances (the north-star's): rel-L2 <= 1e-4 for fp32 storage, <= 2e-3 for fp16 storage.  For fp16
+storage the oracle emulates the storage format (inputs, weights and outputs rounded to binary16)."""
+import numpy as np
+import pytest
+
+import fyusenet_amd as fa
+from fyusenet_amd import prng
+from util import conv_block, oracle_single, rel_l2, run_single
+
+pytestmark = pytest.mark.gpu
+TOL = {fa.STORAGE_F32: 1e-4, fa.STORAGE_F16: 2e-3}
+A = fa.ActType
+
+
+def conv_builder(k, cout, h, w, cin, stride=1, dil=1, act=A.NONE, deep=True, pad_in=None, pad_out=0, bn=False, residual=None,
+                 leak=0.0, clip=None, number=1):
+    b = fa.ConvLayerBuilder(k, "conv").type(fa.LayerType.CONVOLUTION2D).number(number).shape(cout, h, w, cin)
+    b.downsample(stride).dilation(dil).prefixAct(act).outputPadding(pad_out)
+    b.inputPadding((k - 1) // 2 * dil if pad_in is None else pad_in)
+    if deep:
+        b.deep()
+    if bn:
+        b.postfixNorm(fa.NormType.BATCHNORM)
+    if residual is not None:
+        b.residual(*residual).residualPadding(pad_out)
+    if leak:
+        b.leakyReLU(leak)
+    if clip:
+        b.clip(*clip)
+    return b
+
+
+CASES = [
+    # k, cout, h, w, cin, stride, dil, act, kwargs
+    (3, 64, 64, 64, 64, 1, 1, A.RELU, {}),
+    (1, 16, 48, 40, 12, 1, 1, A.NONE, {}),
+    (1, 64, 28, 28, 256, 2, 1, A.RELU, {}),
+    (3, 8, 128, 256, 12, 2, 1, A.RELU, {}),        # unit_tests/convlayertests.cpp:380 DeepConv3x3 shape
+    (5, 16, 40, 36, 16, 1, 1, A.NONE, {}),
+    (7, 64, 64, 64, 3, 2, 1, A.NONE, {}),           # ResNet stem
+    (9, 32, 40, 56, 3, 1, 1, A.NONE, {}),           # style net first layer (row-run path)
+    (9, 3, 40, 56, 32, 1, 1, A.RELU, {"pad_out": 0}),
+    (3, 128, 39, 47, 128, 1, 1, A.RELU, {"bn": True, "residual": (A.NONE, False), "pad_out": 1}),
+    (3, 32, 20, 20, 24, 1, 2, A.RELU, {}),          # dilation
+    (3, 40, 17, 23, 40, 1, 1, A.LEAKY_RELU, {"leak": 0.1}),
+    (1, 96, 14, 14, 24, 1, 1, A.CLIP, {"clip": (0.0, 6.0)}),
+    (3, 256, 14, 14, 256, 1, 1, A.RELU, {"bn": True, "residual": (A.RELU, True)}),
+    (1, 2048, 7, 7, 512, 1, 1, A.RELU, {"bn": True}),
+    (3, 64, 30, 30, 64, 1, 1, A.RELU, {"pad_in": 2, "pad_out": 4}),   # wider halo than needed
+]
+
+
+@pytest.mark.parametrize("storage", [fa.STORAGE_F32, fa.STORAGE_F16], ids=["f32", "f16"])
+@pytest.mark.parametrize("case", CASES, ids=lambda c: "k%d_%dx%dx%d_to%d_s%d_d%d" % (c[0], c[4], c[2], c[3], c[1], c[5], c[6]))
+def test_conv_parity(case, storage):
+    k, cout, h, w, cin, stride, dil, act, kw = case
+    b = conv_builder(k, cout, h, w, cin, stride, dil, act, **kw)
+    bn = kw.get("bn", False)
+    wts = conv_block(100 + k, cout, k, cin, bn=bn)
+    x = prng.uniform(7 * k + cin, (cin, h, w), -1, 1)
+    inputs = [x]
+    if "residual" in kw:
+        inputs.append(prng.uniform(9, (cout, h // stride, w // stride), -1, 1))
+    print("case", case, "storage", storage, flush=True)
+    got, info = run_single(b, storage, inputs, wts)
+    ref = oracle_single(b, storage, inputs, wts)
+    err = rel_l2(got, ref)
+    print("  ", info, "rel_l2=%.3e" % err, flush=True)
+    assert got.shape == ref.shape
+    assert err <= TOL[storage], info
+
+
+def test_reference_known_answer_patterns_on_gpu():
+    # antisymmetric kernel on ones (convlayertests.cpp:242-261) and 1x1 ones (:165-182): exact
+    for storage in (fa.STORAGE_F32, fa.STORAGE_F16):
+        cin, cout, size = 8, 8, 32
+        w = np.zeros((cout, 3, 3, cin), np.float32)
+        w[:, 0], w[:, 2] = -1.0, 1.0
+        block = np.concatenate([np.zeros(cout, np.float32), w.ravel()])
+        got, _ = run_single(conv_builder(3, cout, size, size, cin), storage, [np.ones((cin, size, size), np.float32)], block)
+        assert np.all(got[:, 1:size - 1] == 0)
+        assert np.all(got[:, 0, 1:size - 1] == 3 * cin) and np.all(got[:, size - 1, 1:size - 1] == -3 * cin)
+        block = np.concatenate([np.zeros(16, np.float32), np.ones(16 * 12, np.float32)])
+        got, _ = run_single(conv_builder(1, 16, 20, 24, 12), storage, [np.ones((12, 20, 24), np.float32)], block)
+        assert np.all(got == 12)
+
+
+def test_shallow_unpadded_conv_edge_clamps():
+    # networktests.cpp:85-97,173-186: shallow 3x3 4->8 @32x32 without padding, zero-sum kernel on ones => 0
+    cin, cout = 4, 8
+    w = np.zeros((cout, 3, 3, cin), np.float32)
+    w[:, 0], w[:, 2] = -1.0, 1.0
+    block = np.concatenate([np.zeros(cout, np.float32), w.ravel()])
+    b = conv_builder(3, cout, 32, 32, cin, deep=False, pad_in=0)
+    got, info = run_single(b, fa.STORAGE_F32, [np.ones((cin, 32, 32), np.float32)], block)
+    assert "edge-clamp" in info
+    assert np.all(got == 0.0)
+    x = prng.uniform(3, (cin, 32, 32), -1, 1)
+    wts = conv_block(5, cout, 3, cin)
+    got, _ = run_single(b, fa.STORAGE_F32, [x], wts)
+    assert rel_l2(got, oracle_single(b, fa.STORAGE_F32, [x], wts)) < 1e-5
+
+
+@pytest.mark.parametrize("storage", [fa.STORAGE_F32, fa.STORAGE_F16], ids=["f32", "f16"])
+@pytest.mark.parametrize("k,crop,cin,cout,h,w", [(3, 0, 16, 8, 12, 10), (3, 1, 128, 64, 39, 32), (2, 0, 24, 16, 9, 17), (3, 1, 64, 32, 20, 26)])
+def test_transconv_parity(k, crop, cin, cout, h, w, storage):
+    b = fa.ConvLayerBuilder(k, "tconv").type(fa.LayerType.TRANSCONVOLUTION2D).number(1).shape(cout, h, w, cin)
+    b.upsample(2).inputPadding(1).outputPadding(1).prefixAct(A.RELU).deep().crop(crop)
+    wts = conv_block(31, cout, k, cin)
+    x = prng.uniform(32, (cin, h, w), -1, 1)
+    print("transconv", k, crop, cin, cout, h, w, storage, flush=True)
+    got, info = run_single(b, storage, [x], wts)
+    ref = oracle_single(b, storage, [x], wts)
+    err = rel_l2(got, ref)
+    print("  ", info, "rel_l2=%.3e" % err, flush=True)
+    assert got.shape == ref.shape == (cout, 2 * h + k - 2 - crop, 2 * w + k - 2 - crop)
+    assert err <= TOL[storage]

@@ -1,0 +1,198 @@
+"""Pins the CPU oracle (oracle/fyn_oracle.c) against evidence that does not come from the oracle:
+the reference tests' known-answer patterns and fp64 library routines (torch.nn.functional) /
+brute force.  Runs without a GPU."""
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from fyusenet_amd import prng
+from oracle import oracle as O
+from util import conv_block, rel_l2
+
+RELU = (O.ACT_RELU, 0.0, 0.0, 0.0)
+
+
+def _w_from_block(block, cout, k, cin):
+    """[o][ky][kx][i] -> torch [o][i][ky][kx]"""
+    w = np.asarray(block[cout:cout + cout * k * k * cin], dtype=np.float64).reshape(cout, k, k, cin)
+    return torch.from_numpy(w.transpose(0, 3, 1, 2).copy())
+
+
+# ---- reference known-answer patterns ---------------------------------------------------------
+@pytest.mark.parametrize("k,cin,cout,size", [(3, 4, 8, 32), (5, 16, 8, 24), (7, 8, 4, 20)])
+def test_pattern_antisymmetric_kernel_on_ones(k, cin, cout, size):
+    # unit_tests/convlayertests.cpp:242-261,281-304,355-376: all-ones input, kernel -1 above the centre row,
+    # 0 on it, +1 below => interior outputs 0, border rows != 0 because the halo is zero
+    r = k // 2
+    w = np.zeros((cout, k, k, cin), np.float32)
+    w[:, :r] = -1.0
+    w[:, r + 1:] = 1.0
+    block = np.concatenate([np.zeros(cout, np.float32), w.ravel()])
+    x = np.ones((cin, size, size), np.float32)
+    y = O.conv2d(O.pad_chw(x, r), r, block, cout, k)
+    assert np.all(y[:, r:size - r, :] == 0.0)
+    assert np.all(y[:, 0, r:size - r] == cin * k * r)        # top row misses the -1 rows: +k*r*cin
+    assert np.all(y[:, size - 1, r:size - r] == -cin * k * r)
+
+
+def test_pattern_1x1_ones():
+    # convlayertests.cpp:165-182,319-336: 1x1 all-ones weights on all-ones input => every output = Cin
+    cin, cout = 12, 8
+    block = np.concatenate([np.zeros(cout, np.float32), np.ones(cout * cin, np.float32)])
+    y = O.conv2d(np.ones((cin, 16, 16), np.float32), 0, block, cout, 1)
+    assert np.all(y == cin)
+
+
+def test_pattern_shallow_edge_clamp_zero_sum():
+    # unit_tests/networktests.cpp:85-97,173-186: unpadded shallow 3x3 conv 4->8 @32x32, zero-sum kernel on ones
+    # => exactly 0 everywhere including the borders (edge clamp)
+    cin, cout = 4, 8
+    w = np.zeros((cout, 3, 3, cin), np.float32)
+    w[:, 0] = -1.0
+    w[:, 2] = 1.0
+    block = np.concatenate([np.zeros(cout, np.float32), w.ravel()])
+    y = O.conv2d(np.ones((cin, 32, 32), np.float32), 0, block, cout, 3, border=1)
+    assert np.all(y == 0.0)
+    # the same with the zero-halo rule is NOT zero on the border: the rule matters
+    y0 = O.conv2d(np.ones((cin, 32, 32), np.float32), 0, block, cout, 3, border=0)
+    assert np.any(y0 != 0.0)
+
+
+def test_pattern_gemm_alternating_rows():
+    # unit_tests/misctests.cpp:238-265: 512 -> 256, rows of alternating +-1 on ones => 0
+    cin, cout = 512, 256
+    w = np.tile(np.array([1.0, -1.0], np.float32), cin // 2)
+    block = np.concatenate([np.zeros(cout, np.float32), np.tile(w, cout)])
+    assert np.all(O.gemm(np.ones(cin, np.float32), block, cout) == 0.0)
+
+
+# ---- library-routine cross checks --------------------------------------------------------------
+@pytest.mark.parametrize("k,stride,dil,cin,cout,h,w,relu", [
+    (3, 1, 1, 5, 7, 11, 13, False), (3, 2, 1, 12, 8, 16, 12, True), (5, 1, 1, 3, 4, 9, 10, True),
+    (1, 2, 1, 6, 5, 8, 8, False), (3, 1, 2, 4, 6, 12, 12, True), (7, 2, 1, 3, 8, 20, 18, False), (9, 1, 1, 3, 2, 12, 14, True)])
+def test_conv_matches_torch(k, stride, dil, cin, cout, h, w, relu):
+    r = (k - 1) // 2 * dil
+    x = prng.uniform(11, (cin, h, w), -1, 1)
+    block = conv_block(20, cout, k, cin)
+    y = O.conv2d(O.pad_chw(x, r), r, block, cout, k, dil, stride, RELU if relu else None)
+    xt = torch.from_numpy(x.astype(np.float64))[None]
+    if relu:
+        xt = xt.clamp(min=0)
+    ref = F.conv2d(xt, _w_from_block(block, cout, k, cin), torch.from_numpy(block[:cout].astype(np.float64)),
+                   stride=stride, padding=r, dilation=dil)[0].numpy()
+    ref = ref[:, :h // stride, :w // stride]
+    assert y.shape == ref.shape
+    assert rel_l2(y, ref) < 1e-6
+
+
+def test_conv_bn_residual_epilogue():
+    # order: acc*scale + (bias*scale + bnBias) + relu(res)*scale  (batchnorm.inc / residual.inc)
+    cin, cout, k, h, w = 6, 5, 3, 8, 9
+    x = prng.uniform(1, (cin, h, w), -1, 1)
+    res = prng.uniform(2, (cout, h, w), -1, 1)
+    block = conv_block(3, cout, k, cin, bn=True)
+    flags = O.POST_BATCHNORM | O.RESIDUAL_INPUT | O.RELU_ON_RESIDUAL | O.BATCHNORM_ON_RESIDUAL
+    y = O.conv2d(O.pad_chw(x, 1), 1, block, cout, k, act=RELU, flags=flags, residual=res)
+    nw = cout * k * k * cin
+    bias, scale, bnb = block[:cout].astype(np.float64), block[cout + nw:cout + nw + cout].astype(np.float64), block[cout + nw + cout:].astype(np.float64)
+    acc = F.conv2d(torch.from_numpy(x.astype(np.float64))[None].clamp(min=0), _w_from_block(block, cout, k, cin), None, padding=1)[0].numpy()
+    ref = acc * scale[:, None, None] + (bias * scale + bnb)[:, None, None] + np.maximum(res, 0) * scale[:, None, None]
+    assert rel_l2(y, ref) < 1e-6
+    # invariants: zero residual == no residual; zero weights => bias' + residual path only
+    y0 = O.conv2d(O.pad_chw(x, 1), 1, block, cout, k, act=RELU, flags=flags, residual=np.zeros_like(res))
+    y1 = O.conv2d(O.pad_chw(x, 1), 1, block, cout, k, act=RELU, flags=O.POST_BATCHNORM)
+    assert np.array_equal(y0, y1)
+
+
+@pytest.mark.parametrize("stride,dil,c,h,w", [(1, 1, 8, 10, 12), (2, 1, 24, 16, 16), (1, 2, 5, 9, 9)])
+def test_dwconv_matches_grouped_conv(stride, dil, c, h, w):
+    x = prng.uniform(5, (c, h, w), -1, 1)
+    block = conv_block(6, c, 3, c, depthwise=True)
+    clip = (O.ACT_CLIP, 0.0, 0.0, 6.0)
+    y = O.dwconv(O.pad_chw(x * 8, dil), dil, block, 1, 3, dil, stride, clip)
+    wt = torch.from_numpy(block[c:c + 9 * c].astype(np.float64).reshape(c, 1, 3, 3))
+    ref = F.conv2d(torch.from_numpy((x * 8).astype(np.float64))[None].clamp(0, 6), wt, torch.from_numpy(block[:c].astype(np.float64)),
+                   stride=stride, padding=dil, dilation=dil, groups=c)[0].numpy()[:, :h // stride, :w // stride]
+    assert rel_l2(y, ref) < 1e-6
+
+
+@pytest.mark.parametrize("k,crop,cin,cout,h,w", [(3, 0, 4, 6, 5, 7), (3, 1, 8, 3, 6, 6), (2, 0, 5, 4, 4, 9)])
+def test_transconv_matches_conv_transpose(k, crop, cin, cout, h, w):
+    x = prng.uniform(7, (cin, h, w), -1, 1)
+    block = conv_block(8, cout, k, cin)
+    y = O.transconv(x, 0, block, cout, k, crop, RELU)
+    wt = _w_from_block(block, cout, k, cin).permute(1, 0, 2, 3)  # [i][o][ky][kx]
+    ref = F.conv_transpose2d(torch.from_numpy(x.astype(np.float64))[None].clamp(min=0), wt,
+                             torch.from_numpy(block[:cout].astype(np.float64)), stride=2)[0].numpy()
+    ho, wo = 2 * h + k - 2 - crop, 2 * w + k - 2 - crop
+    assert y.shape == (cout, ho, wo)
+    assert rel_l2(y, ref[:, :ho, :wo]) < 1e-6
+
+
+def test_transconv_brute_force_tiny():
+    # out[2y+ky, 2x+kx] += w[ky,kx]*in[y,x] on a 2x2 single-channel input, by hand
+    x = np.array([[[1.0, 2.0], [3.0, 4.0]]], np.float32)
+    w = np.arange(1, 10, dtype=np.float32)  # [ky][kx]
+    block = np.concatenate([np.array([0.5], np.float32), w])
+    y = O.transconv(x, 0, block, 1, 3)[0]
+    ref = np.zeros((5, 5))
+    for yy in range(2):
+        for xx in range(2):
+            ref[2 * yy:2 * yy + 3, 2 * xx:2 * xx + 3] += x[0, yy, xx] * w.reshape(3, 3)
+    assert np.allclose(y, ref + 0.5)
+
+
+@pytest.mark.parametrize("pool", [2, 4])
+def test_pool_equals_stride_matches_torch(pool):
+    # the case PoolLayerTest::computeMaxPool/computeAvgPool cover (pool == stride, no padding)
+    x = prng.uniform(9, (12, 16, 24), -100, 100)
+    xt = torch.from_numpy(x.astype(np.float64))[None]
+    assert np.array_equal(O.maxpool(x, 0, pool, pool), F.max_pool2d(xt, pool)[0].numpy().astype(np.float32))
+    assert rel_l2(O.avgpool(x, 0, pool, pool), F.avg_pool2d(xt, pool)[0].numpy()) < 1e-6
+
+
+def test_maxpool_3x3_s2_pad1_relu_equals_neg_inf_padding():
+    # deep rule: window starts input_padding before the stride origin; with ReLU on fetch the zero halo is
+    # equivalent to -inf padding (ResNet stem pool)
+    x = prng.normal(10, (8, 14, 14))
+    y = O.maxpool(O.pad_chw(x, 1), 1, 3, 2, RELU)
+    ref = F.max_pool2d(torch.from_numpy(x.astype(np.float64))[None].clamp(min=0), 3, 2, padding=1)[0].numpy()
+    assert np.array_equal(y, ref.astype(np.float32))
+
+
+def test_avgpool_3_window_is_centred():
+    x = prng.uniform(12, (4, 9, 9), -1, 1)
+    y = O.avgpool(O.pad_chw(x, 1), 1, 3, 1)
+    ref = F.avg_pool2d(torch.from_numpy(x.astype(np.float64))[None], 3, 1, padding=1, count_include_pad=True)[0].numpy()
+    assert rel_l2(y, ref) < 1e-6
+
+
+def test_global_pool_bn_argmax_concat_closed_forms():
+    x = prng.uniform(13, (23, 7, 5), -3, 3)
+    assert rel_l2(O.global_pool(x, 0, False, RELU).ravel(), np.maximum(x, 0).astype(np.float64).mean(axis=(1, 2))) < 1e-6
+    assert np.array_equal(O.global_pool(x, 0, True).ravel(), x.max(axis=(1, 2)))
+    sb = np.concatenate([prng.uniform(14, (23,), 0.5, 1.5), prng.normal(15, (23,))])
+    assert rel_l2(O.batchnorm(x, 0, sb), x * sb[:23, None, None] + sb[23:, None, None]) < 1e-6
+    idx, val = O.argmax(x)
+    assert np.array_equal(idx, np.argmax(x, axis=0)) and np.array_equal(val, x.max(axis=0))
+    tie = np.zeros((5, 2, 2), np.float32)  # all equal: lowest index wins (strict '>' scan)
+    assert np.all(O.argmax(tie)[0] == 0)
+    a, b = x[:7], x[7:]
+    assert np.array_equal(O.concat([a, b]), x)
+
+
+def test_round_fp16_is_ieee_rn():
+    x = np.concatenate([prng.normal(16, (4096,)) * 10.0 ** prng.uniform(17, (4096,), -8, 5), [0.0, 65504.0, 65520.0, 1e-8, -5.96e-8]]).astype(np.float32)
+    with np.errstate(over="ignore"):
+        assert np.array_equal(O.round_fp16(x), x.astype(np.float16).astype(np.float32))
+
+
+def test_deep_tiling_and_layout_round_trips():
+    assert O.deep_tiling(4) == (1, 1) and O.deep_tiling(8) == (2, 1) and O.deep_tiling(16) == (2, 2)
+    assert O.deep_tiling(64) == (4, 4) and O.deep_tiling(12) == (2, 2) and O.deep_tiling(2048) == (27, 19) and O.deep_tiling(80) == (5, 4)  # by hand: 27*19=513: cost 8+1
+    x = prng.uniform(18, (23, 6, 5), -1, 1)
+    for pad in (0, 1):
+        d = O.chw_to_deep(x, pad)
+        assert np.array_equal(O.deep_to_chw(d, 23, 6, 5, pad), x)
+    assert np.array_equal(O.shallow_to_chw(O.chw_to_shallow(x[:3], 4), 3), x[:3])
