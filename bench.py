@@ -1,0 +1,208 @@
+#!/usr/bin/env python3
+"""Benchmark of the GPU layer stack on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload stylenet|resnet50|conv1|mobilenet|stylenet9x9]
+
+A step is one forward pass of the named network over one synthetic input frame that is already
+resident in HBM (uploaded before the timed region); weights are synthetic (random init).  Prints ONE
+JSON line on stdout; progress goes to stderr.  The default workload is BASELINE.json configs[1], the
+Johnson style-transfer net at 512x624 in fp32 storage; ResNet-50 imgs/s is measured in the same run and
+reported under "also".
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+import numpy as np  # noqa: E402
+
+import fyusenet_amd as fa  # noqa: E402
+from fyusenet_amd import networks  # noqa: E402
+
+PEAK_MFMA_F16_TFLOPS = 2500.0   # MI355X dense fp16/bf16 matrix peak
+PEAK_HBM_GBS = 8000.0           # MI355X HBM3E
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def make_net(workload):
+    if workload == "stylenet":
+        return networks.StyleNet(fa.STORAGE_F32, 512, 624, 3), "stylenet 512x624 ms/frame", "ms/frame", "fp32 storage, fp16x2-split MFMA, fp32 accumulate"
+    if workload == "stylenet9x9":
+        return networks.StyleNet(fa.STORAGE_F16, 1524, 1856, 9), "stylenet9x9 1524x1856 ms/frame", "ms/frame", "fp16 storage, fp16 MFMA, fp32 accumulate"
+    if workload == "resnet50":
+        return networks.ResNet50(fa.STORAGE_F32), "ResNet-50 224x224 imgs/s", "imgs/s", "fp32 storage"
+    if workload == "mobilenet":
+        return networks.MobileNetV2(fa.STORAGE_F16), "MobileNetV2 224x224 imgs/s", "imgs/s", "fp16 storage"
+    if workload == "conv1":
+        return networks.SingleConvNet(fa.STORAGE_F32), "conv3x3 64->64 256x256 us/layer", "us", "fp32 storage"
+    raise SystemExit("unknown workload %s" % workload)
+
+
+def conv_work(b):
+    """Algorithmic FLOPs and bytes of one convolution-type layer: flops = 2*Hout*Wout*Cout*Cin*K^2
+    (transposed: input pixels); bytes = s*(in + out [+ residual]) + s*(weights + 2*Cout), halo and
+    channel padding excluded."""
+    k = getattr(b, "kernel_", 1)
+    t = int(b.type_)
+    cin, cout, h, w = b.inputChannels_, b.outputChannels_, b.height_, b.width_
+    if t == int(fa.LayerType.TRANSCONVOLUTION2D):
+        ho, wo = 2 * h + k - 2 - b.transconvCrop_, 2 * w + k - 2 - b.transconvCrop_
+        flops = 2.0 * h * w * cout * cin * k * k
+    else:
+        ho, wo = h // b.downsample_[1], w // b.downsample_[0]
+        flops = 2.0 * ho * wo * cout * cin * k * k
+    return flops, (cin * h * w, cout * ho * wo, cout * cin * k * k + 2 * cout)
+
+
+def timed_forwards(net, steps, warmup, graph=True):
+    net.useGraph(graph)
+    for _ in range(warmup):
+        net.forward()
+    net.finish()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        net.forward()
+    net.finish()
+    return (time.perf_counter() - t0) * 1e3 / steps
+
+
+def dominant_conv_roofline(net, storage_bytes):
+    """Times every layer's kernel(s) alone with HIP events on the network's stream and returns the
+    roofline record of the layer class that takes the most time (identical-shape layers pooled)."""
+    groups = {}
+    for lyr in net.layers:
+        t = int(lyr.builder.type_)
+        if t in (int(fa.LayerType.UPLOAD), int(fa.LayerType.DOWNLOAD)):
+            continue
+        iters = 20
+        lyr.timeKernel(3)
+        ms = lyr.timeKernel(iters)
+        b = lyr.builder
+        key = (t, getattr(b, "kernel_", 0), b.inputChannels_, b.outputChannels_, b.height_, b.width_, tuple(b.downsample_),
+               bool(int(b.getFlags()) & 1))
+        g = groups.setdefault(key, {"ms": 0.0, "n": 0, "layer": lyr})
+        g["ms"] += ms
+        g["n"] += 1
+    key, g = max(groups.items(), key=lambda kv: kv[1]["ms"])
+    lyr, b = g["layer"], g["layer"].builder
+    avg_ms = g["ms"] / g["n"]
+    rec = {"kernel": lyr.kernelInfo(), "layer": lyr.name, "launches_per_step": g["n"], "avg_launch_us": avg_ms * 1e3}
+    if int(b.type_) in (int(fa.LayerType.CONVOLUTION2D), int(fa.LayerType.TRANSCONVOLUTION2D)) and getattr(b, "groupSize_", 1) == 1:
+        flops, (ein, eout, ew) = conv_work(b)
+        res = eout if int(b.getFlags()) & 1 else 0
+        nbytes = storage_bytes * (ein + eout + res + ew)
+        t_mfma = flops / (PEAK_MFMA_F16_TFLOPS * 1e12)
+        t_hbm = nbytes / (PEAK_HBM_GBS * 1e9)
+        if t_mfma >= t_hbm:
+            ach = flops / (avg_ms * 1e-3) / 1e12
+            rec.update({"bound": "mfma", "achieved": ach, "peak": PEAK_MFMA_F16_TFLOPS, "unit": "TFLOP/s", "frac": ach / PEAK_MFMA_F16_TFLOPS})
+        else:
+            ach = nbytes / (avg_ms * 1e-3) / 1e9
+            rec.update({"bound": "hbm", "achieved": ach, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": ach / PEAK_HBM_GBS})
+        rec["algorithmic_flops_per_launch"] = flops
+        rec["algorithmic_bytes_per_launch"] = nbytes
+    rec["traffic"] = None
+    per_layer = sorted(((v["ms"], v["n"], v["layer"].name) for v in groups.values()), reverse=True)
+    return rec, per_layer
+
+
+def cpu_baseline(net, x, total_flops):
+    """Times the CPU oracle (plain C restatement of the reference's unit-test convolution, OpenMP over
+    output channels) on the dominant convolution of the workload at full size and scales by the
+    network's algorithmic FLOPs."""
+    from oracle import oracle as O
+    threads = min(os.cpu_count() or 1, 16)
+    O.set_threads(threads)
+    conv_layers = [l for l in net.layers if int(l.builder.type_) == int(fa.LayerType.CONVOLUTION2D) and getattr(l.builder, "groupSize_", 1) == 1]
+    lyr = max(conv_layers, key=lambda l: conv_work(l.builder)[0])
+    b = lyr.builder
+    flops, _ = conv_work(b)
+    from fyusenet_amd import prng
+    xin = prng.uniform(77, (b.inputChannels_, b.height_, b.width_), -1, 1)
+    ins = [xin]
+    if int(b.getFlags()) & 1:
+        ins.append(prng.uniform(78, (b.outputChannels_, b.height_ // b.downsample_[1], b.width_ // b.downsample_[0]), -1, 1))
+    t0 = time.perf_counter()
+    O.run_layer(b, lyr.weights, ins)
+    dt = time.perf_counter() - t0
+    return dt, flops, threads, lyr.name
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="stylenet")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-also", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        raise SystemExit("bench.py: this engine is single-GPU (batch 1 inference); run with --gpus 1")
+
+    log(fa.capi.device_info(0))
+    net, metric, unit, dtype = make_net(args.workload)
+    net.setup()
+    x = net.makeInput()
+    net.setInput(x)
+    ms = timed_forwards(net, args.steps, args.warmup, graph=True)
+    ms_eager = timed_forwards(net, max(5, args.steps // 5), 2, graph=False)
+    log("%s: %.4f ms/step (hipGraph), %.4f ms/step (eager launches)" % (args.workload, ms, ms_eager))
+    net.useGraph(False)
+    storage_bytes = 4 if net.storage == fa.STORAGE_F32 else 2
+    roof, per_layer = dominant_conv_roofline(net, storage_bytes)
+    for t, n, name in per_layer[:8]:
+        log("   %-12s x%-2d %.1f us total" % (name, n, t * 1e3))
+    total_flops = sum(conv_work(l.builder)[0] for l in net.layers if int(l.builder.type_) in (6, 8) and getattr(l.builder, "groupSize_", 1) == 1)
+
+    if unit == "ms/frame":
+        value, hib = ms, False
+    elif unit == "us":
+        value, hib = ms * 1e3, False
+    else:
+        value, hib = 1e3 / ms, True
+
+    out = {"metric": metric, "value": value, "unit": unit, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+           "ms_per_step": ms, "higher_is_better": hib, "scaling": "weak", "vs_baseline": None, "dtype": dtype, "data": "synthetic",
+           "config": {"workload": args.workload, "input": list(x.shape), "batch": 1, "launch": "hipGraph replay",
+                      "algorithmic_gflop_per_step": total_flops / 1e9},
+           "ms_per_step_eager": ms_eager, "roofline": roof}
+
+    if not args.no_cpu_baseline:
+        dt, flops, threads, lname = cpu_baseline(net, x, total_flops)
+        cpu_ms = dt * 1e3 * total_flops / flops
+        if unit == "ms/frame":
+            cv = cpu_ms
+        elif unit == "us":
+            cv = cpu_ms * 1e3
+        else:
+            cv = 1e3 / cpu_ms
+        out["cpu_baseline"] = {"value": cv, "unit": unit, "cores": threads, "kind": "port",
+                               "sample": "layer %s at full size (%.2f GFLOP, %.2f s on %d threads), scaled by the step's %.1f GFLOP"
+                                         % (lname, flops / 1e9, dt, threads, total_flops / 1e9)}
+    net.cleanup()
+
+    if not args.no_also and args.workload == "stylenet":
+        also = {}
+        for wl in ("resnet50",):
+            n2, m2, u2, d2 = make_net(wl)
+            n2.setup()
+            n2.setInput(n2.makeInput())
+            ms2 = timed_forwards(n2, max(args.steps, 100), args.warmup, graph=True)
+            ms2e = timed_forwards(n2, 20, 2, graph=False)
+            also[m2] = {"value": 1e3 / ms2, "unit": u2, "ms_per_step": ms2, "ms_per_step_eager": ms2e, "dtype": d2}
+            log("%s: %.4f ms/step (hipGraph) %.4f (eager)" % (wl, ms2, ms2e))
+            n2.cleanup()
+        out["also"] = also
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -144,7 +144,8 @@ int fyn_layer_output_shape(fyn_net* net, int layer, int* channels, int* height, 
     if (channels) *channels = l->oc;
     if (height) *height = l->oh;
     if (width) *width = l->ow;
-    if (padding) *padding = l->d.output_padding;
+    // a pass-through (download) layer hands on its input tensor, halo included
+    if (padding) *padding = (N(net)->is_setup && l->out >= 0) ? l->tout().v.pad : l->d.output_padding;
     FYN_API_END
 }
 

@@ -270,12 +270,74 @@ def _round_block_fp16(layer_type, b, block):
     return block
 
 
-def run_network(desc, inputs, fp16_storage=None):
+def run_layer(b, w, ins, f16=False):
+    """One layer on the CPU.  b: builder, w: weight block, ins: unpadded CHW input per port.
+    Returns the unpadded CHW output (not yet rounded to the storage type)."""
+    t = int(b.type_)
+    flags = int(b.getFlags())
+    act = _builder_act(b, flags)
+
+    def get(port, pad):
+        return pad_chw(np.asarray(ins[port], dtype=np.float32), pad)
+
+    if t in (26, 27):  # download / upload: pass-through
+        return np.asarray(ins[0], dtype=np.float32)
+    if t == 6:
+        res = get(1, 0) if flags & RESIDUAL_INPUT else None
+        wb = _round_block_fp16(t, b, w) if f16 else w
+        dw = getattr(b, "groupSize_", 1) not in (0, 1) and b.groupSize_ == b.inputChannels_
+        if dw:
+            return dwconv(get(0, b.inputPadding_), b.inputPadding_, wb, 1, b.kernel_, b.dilation_[0], b.downsample_[0], act, flags, res)
+        r = (b.kernel_ - 1) // 2 * b.dilation_[0]
+        border = 1 if (not (flags & 16) and b.inputPadding_ < r and b.kernel_ > 1) else 0
+        return conv2d(get(0, b.inputPadding_), b.inputPadding_, wb, b.outputChannels_, b.kernel_, b.dilation_[0],
+                      b.downsample_[0], act, flags, res, border)
+    if t == 8:
+        wb = _round_block_fp16(t, b, w) if f16 else w
+        return transconv(get(0, b.inputPadding_), b.inputPadding_, wb, b.outputChannels_, b.kernel_, b.transconvCrop_, act, flags)
+    if t == 31:
+        wb = _round_block_fp16(t, b, w) if f16 else w
+        return gemm(get(0, 0), wb, b.outputChannels_, act, flags).reshape(-1, 1, 1)
+    if t in (9, 10):
+        if b.global_:
+            return global_pool(get(0, b.inputPadding_), b.inputPadding_, t == 10, act)
+        if t == 10:
+            return maxpool(get(0, b.inputPadding_), b.inputPadding_, b.poolsize_[0], b.downsample_[0], act)
+        return avgpool(get(0, b.inputPadding_), b.inputPadding_, b.poolsize_[0], b.downsample_[0], act)
+    if t == 30:
+        res = get(1, 0) if flags & RESIDUAL_INPUT else None
+        return batchnorm(get(0, 0), 0, w, act, flags, res)
+    if t in (1, 2):
+        return addsub(get(0, 0), get(1, 0), t == 2, act)
+    if t == 5:
+        all_relu = all(f & PRE_RELU for (_, _, f) in b.inputs_)
+        a = act if act is not None else ((ACT_RELU, 0.0, 0.0, 0.0) if all_relu else None)
+        return concat([get(p, 0) for p in range(len(b.inputs_))], a)
+    if t == 3:
+        idx, val = argmax(get(0, 0), act)
+        return np.stack([idx.astype(np.float32), val])
+    raise ValueError("oracle: unsupported layer type %d" % t)
+
+
+def num_ports(b):
+    t = int(b.type_)
+    if t == 27:
+        return 1  # fed from the host
+    if t == 5:
+        return len(b.inputs_)
+    if t in (1, 2):
+        return 2
+    return 2 if int(b.getFlags()) & RESIDUAL_INPUT else 1
+
+
+def run_network(desc, inputs, fp16_storage=None, forced=None):
     """Executes a network description on the CPU.
 
     desc: NeuralNetwork.describe(); inputs: {(layer_number, port): CHW array} for upload layers
     (port 0) and unconnected ports.  Returns {layer_number: CHW output (unpadded)}.
     fp16_storage: emulate fp16 tensors/weights (default: desc['storage'] == 1).
+    forced: optional {layer_number: CHW array}; when given, every layer reads these tensors instead of
+    the oracle's own upstream results (per-layer check on identical inputs).
     """
     f16 = (desc.get("storage", 0) == 1) if fp16_storage is None else fp16_storage
     rnd = round_fp16 if f16 else (lambda a: np.asarray(a, dtype=np.float32))
@@ -285,58 +347,12 @@ def run_network(desc, inputs, fp16_storage=None):
     outs = {}
     for entry in sorted(desc["layers"], key=lambda e: e["number"]):
         b, no, w = entry["builder"], entry["number"], entry["weights"]
-        t = int(b.type_)
-        flags = int(b.getFlags())
-        act = _builder_act(b, flags)
-
-        def get(port, pad):
+        ins = []
+        for port in range(num_ports(b)):
             if (no, port) in feeds:
-                x = outs[feeds[(no, port)]]
+                src = feeds[(no, port)]
+                ins.append(forced[src] if forced is not None else outs[src])
             else:
-                x = rnd(inputs[(no, port)])
-            return pad_chw(x, pad)
-
-        if t == 27:  # upload
-            y = rnd(inputs[(no, 0)])
-        elif t == 26:  # download
-            y = get(0, 0)
-        elif t == 6:
-            res = get(1, 0) if flags & RESIDUAL_INPUT else None
-            wb = _round_block_fp16(t, b, w) if f16 else w
-            dw = getattr(b, "groupSize_", 1) not in (0, 1) and b.groupSize_ == b.inputChannels_
-            if dw:
-                y = dwconv(get(0, b.inputPadding_), b.inputPadding_, wb, 1, b.kernel_, b.dilation_[0], b.downsample_[0], act, flags, res)
-            else:
-                r = (b.kernel_ - 1) // 2 * b.dilation_[0]
-                border = 1 if (not (flags & 16) and b.inputPadding_ < r and b.kernel_ > 1) else 0
-                y = conv2d(get(0, b.inputPadding_), b.inputPadding_, wb, b.outputChannels_, b.kernel_, b.dilation_[0],
-                           b.downsample_[0], act, flags, res, border)
-        elif t == 8:
-            wb = _round_block_fp16(t, b, w) if f16 else w
-            y = transconv(get(0, b.inputPadding_), b.inputPadding_, wb, b.outputChannels_, b.kernel_, b.transconvCrop_, act, flags)
-        elif t == 31:
-            wb = _round_block_fp16(t, b, w) if f16 else w
-            y = gemm(get(0, 0), wb, b.outputChannels_, act, flags).reshape(-1, 1, 1)
-        elif t in (9, 10):
-            if b.global_:
-                y = global_pool(get(0, b.inputPadding_), b.inputPadding_, t == 10, act)
-            elif t == 10:
-                y = maxpool(get(0, b.inputPadding_), b.inputPadding_, b.poolsize_[0], b.downsample_[0], act)
-            else:
-                y = avgpool(get(0, b.inputPadding_), b.inputPadding_, b.poolsize_[0], b.downsample_[0], act)
-        elif t == 30:
-            res = get(1, 0) if flags & RESIDUAL_INPUT else None
-            y = batchnorm(get(0, 0), 0, w, act, flags, res)
-        elif t in (1, 2):
-            y = addsub(get(0, 0), get(1, 0), t == 2, act)
-        elif t == 5:
-            all_relu = all(f & PRE_RELU for (_, _, f) in b.inputs_)
-            a = act if act is not None else ((ACT_RELU, 0.0, 0.0, 0.0) if all_relu else None)
-            y = concat([get(p, 0) for p in range(len(b.inputs_))], a)
-        elif t == 3:
-            idx, val = argmax(get(0, 0), act)
-            y = np.stack([idx.astype(np.float32), val])
-        else:
-            raise ValueError("oracle: unsupported layer type %d" % t)
-        outs[no] = rnd(y)
+                ins.append(rnd(inputs[(no, port)]))
+        outs[no] = rnd(run_layer(b, w, ins, f16))
     return outs

@@ -1,0 +1,152 @@
+"""Whole-network parity of the benchmark configurations against the CPU oracle, through the C ABI.
+
+Sizes: config 1 and the ResNet-50 / MobileNetV2 graphs run at BASELINE's full size (the oracle finishes
+in seconds); the style nets are checked against the oracle at reduced resolution and, at full size,
+through size-independent properties (eager == HIP-graph replay, buffer sharing on == off,
+run-to-run bit-identity).  Tolerances: rel-L2 <= 1e-4 (fp32 storage), <= 2e-3 (fp16 storage, oracle
+emulating the storage format)."""
+import numpy as np
+import pytest
+
+import fyusenet_amd as fa
+from fyusenet_amd import networks
+from oracle import oracle as O
+from util import rel_l2
+
+pytestmark = pytest.mark.gpu
+TOL = {fa.STORAGE_F32: 1e-4, fa.STORAGE_F16: 2e-3}
+STORAGES = pytest.mark.parametrize("storage", [fa.STORAGE_F32, fa.STORAGE_F16], ids=["f32", "f16"])
+
+
+# Two correct fp16-storage chains decorrelate with depth: a last-bit difference in one tensor flips binary16
+# roundings downstream until both chains differ by the storage format's own rounding noise (~3e-4 per
+# layer, accumulating).  For fp16 storage every layer is therefore checked on IDENTICAL inputs (the
+# engine's own upstream tensors fed to the oracle) at the 2e-3 bound, and the end-to-end drift against
+# the free-running oracle chain is bounded separately.
+F16_END_TO_END = 1e-2
+
+
+def run_and_compare(net, storage, reuse=False):
+    net.setup(reuseBuffers=reuse)
+    x = net.makeInput()
+    net.setInput(x)
+    net.forward()
+    net.finish()
+    desc = net.describe()
+    got = {}
+    for lyr in net.layers:
+        got[lyr.number] = lyr.copyResult()
+    ref = O.run_network(desc, {net.input_key: x})
+    forced = O.run_network(desc, {net.input_key: x}, forced=got) if storage == fa.STORAGE_F16 else ref
+    for lyr in net.layers:
+        if int(lyr.builder.type_) == int(fa.LayerType.ARGMAX):
+            continue
+        e_layer = rel_l2(got[lyr.number], forced[lyr.number])
+        e_chain = rel_l2(got[lyr.number], ref[lyr.number])
+        print("  layer %3d %-14s %-58s same-input %.2e chain %.2e" % (lyr.number, lyr.name, lyr.kernelInfo()[:58], e_layer, e_chain), flush=True)
+        assert e_layer <= TOL[storage], "layer %s (%d): rel-L2 %.3e" % (lyr.name, lyr.number, e_layer)
+        assert e_chain <= (TOL[storage] if storage == fa.STORAGE_F32 else F16_END_TO_END), "layer %s chain drift %.3e" % (lyr.name, e_chain)
+    return ref, got
+
+
+@STORAGES
+def test_config1_single_conv_full_size(storage):
+    net = networks.SingleConvNet(storage)
+    run_and_compare(net, storage)
+    net.cleanup()
+
+
+@STORAGES
+def test_config2_stylenet_reduced(storage):
+    net = networks.StyleNet(storage, width=128, height=156, res_kernel=3)
+    run_and_compare(net, storage)
+    net.cleanup()
+
+
+@STORAGES
+def test_config5_stylenet9x9_reduced(storage):
+    net = networks.StyleNet(storage, width=96, height=64, res_kernel=9)
+    run_and_compare(net, storage)
+    net.cleanup()
+
+
+@STORAGES
+def test_config3_resnet50_full_size(storage):
+    net = networks.ResNet50(storage)
+    ref, got = run_and_compare(net, storage)
+    idx, val = net.getArgMax(net.argmax_layer)
+    logits = net.layers[net.logits_layer].copyResult().ravel()
+    assert idx[0, 0] == int(np.argmax(logits))            # exact arg-max of the engine's own logits
+    assert idx[0, 0] == int(ref[net.argmax_layer][0, 0, 0])  # and the oracle's class
+    net.cleanup()
+
+
+@STORAGES
+def test_config4_mobilenetv2_full_size(storage):
+    net = networks.MobileNetV2(storage)
+    run_and_compare(net, storage)
+    net.cleanup()
+
+
+def test_config2_full_size_properties():
+    """512x624 fp32: buffer sharing, HIP-graph replay and repetition must not change a single bit."""
+    outs = []
+    for reuse in (False, True):
+        net = networks.StyleNet(fa.STORAGE_F32)
+        net.setup(reuseBuffers=reuse)
+        x = net.makeInput()
+        net.setInput(x)
+        net.forward()
+        net.finish()
+        a = net.getOutput(net.output_layer)
+        net.forward()
+        net.finish()
+        assert np.array_equal(a, net.getOutput(net.output_layer))
+        if reuse:
+            net.useGraph(True)
+            for _ in range(3):
+                net.forward()
+                net.finish()
+                assert np.array_equal(a, net.getOutput(net.output_layer))
+        assert np.all(np.isfinite(a)) and a.shape == (3, 624, 512)
+        outs.append(a)
+        net.cleanup()
+    assert np.array_equal(outs[0], outs[1])
+
+
+def test_weight_reload_swaps_style():
+    # samples/samplenetworks/stylenet3x3.cpp:81-89: weights can be loaded again after setup
+    net = networks.StyleNet(fa.STORAGE_F32, width=64, height=48)
+    net.setup()
+    x = net.makeInput()
+    net.setInput(x)
+    net.forward()
+    a = net.getOutput(net.output_layer)
+    lyr = net.layers[net.last_conv]
+    w2 = networks.conv_block(4242, 3, 9, 32)
+    lyr.loadWeightsAndBiases(w2, 0)
+    net.forward()
+    b = net.getOutput(net.output_layer)
+    assert not np.array_equal(a, b)
+    ref = O.run_network(net.describe(), {net.input_key: x})
+    assert rel_l2(b, ref[net.output_layer]) <= 1e-4
+    net.cleanup()
+
+
+def test_intermediate_output_and_timings(tmp_path):
+    net = networks.StyleNet(fa.STORAGE_F32, width=64, height=48)
+    net.setup()
+    net.setInput(net.makeInput())
+    net.enableIntermediateOutput(str(tmp_path))
+    seq = net.forward()
+    net.finish()
+    net.enableIntermediateOutput("")
+    dump = np.fromfile(str(tmp_path / ("conv1_%d.bin" % seq)), dtype=np.float32)
+    assert dump.size == 32 * 48 * 64  # CHW fp32, padding stripped (base/layerbase.h:160-203)
+    net.enableTimings(True)
+    for _ in range(3):
+        net.forward()
+    net.finish()
+    ms, runs = net.getTiming(1)
+    assert runs == 3 and ms > 0
+    net.cleanup()

