@@ -42,7 +42,32 @@ def make_net(workload):
         return networks.MobileNetV2(fa.STORAGE_F16), "MobileNetV2 224x224 imgs/s", "imgs/s", "fp16 storage"
     if workload == "conv1":
         return networks.SingleConvNet(fa.STORAGE_F32), "conv3x3 64->64 256x256 us/layer", "us", "fp32 storage"
+    if workload == "copy":
+        return CopyNet(fa.STORAGE_F32), "copy 64x1024x1024 fp32 GB/s", "GB/s", "fp32"
     raise SystemExit("unknown workload %s" % workload)
+
+
+class CopyNet(fa.NeuralNetwork):
+    """A concat layer with a single input: a plain copy kernel of known size (268 MB read, 268 MB written),
+    used to scale the FETCH_SIZE / WRITE_SIZE counters of rocprofv3."""
+    C, S = 64, 1024
+    output_layer = 1
+    input_key = (1, 0)
+
+    def buildLayers(self, f):
+        b = fa.ConcatLayerBuilder("copy").number(1).deep().input(self.C, 0)
+        b.size(self.S, self.S)
+        b.outputChannels_ = self.C
+        b.push(f)
+
+    def connectLayers(self, layers, bm):
+        pass
+
+    def makeInput(self):
+        return np.ones((self.C, self.S, self.S), np.float32)
+
+    def setInput(self, x):
+        self.layers[1].setInput(x, 0)
 
 
 def conv_work(b):
@@ -166,6 +191,8 @@ def main():
         value, hib = ms, False
     elif unit == "us":
         value, hib = ms * 1e3, False
+    elif unit == "GB/s":
+        value, hib = 2 * 4 * CopyNet.C * CopyNet.S * CopyNet.S / (ms * 1e-3) / 1e9, True
     else:
         value, hib = 1e3 / ms, True
 

@@ -18,6 +18,9 @@
 #include <hip/hip_fp16.h>
 #include <hip/hip_runtime.h>
 
+#include <map>
+#include <mutex>
+
 #include "kernels.h"
 
 namespace fynhip {
@@ -26,27 +29,22 @@ typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
 typedef float float16_t __attribute__((ext_vector_type(16)));
 
+// Branch-free activation: the host normalises every activation kind to
+//   act(x) = min(hi, max(lo, x)) + leak * min(x, 0)
+// (none: lo=-inf, hi=+inf, leak=0; ReLU: lo=0; leaky: lo=0, leak; clip: lo, hi).
 __device__ __forceinline__ float act_apply(float x, const Act& a) {
-    switch (a.kind) {
-        case ACT_RELU: return fmaxf(x, 0.f);
-        case ACT_LEAKY: return x >= 0.f ? x : a.leak * x;
-        case ACT_CLIP: return fminf(a.hi, fmaxf(a.lo, x));
-        default: return x;
-    }
+    return fminf(a.hi, fmaxf(a.lo, x)) + a.leak * fminf(x, 0.f);
 }
 
 template <typename T>
 __device__ __forceinline__ void load_vals(const T* src, float* v, int n);
 template <>
 __device__ __forceinline__ void load_vals<float>(const float* src, float* v, int n) {
+    float4 a = *reinterpret_cast<const float4*>(src);
+    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
     if (n == 8) {
-        float4 a = *reinterpret_cast<const float4*>(src);
         float4 b = *reinterpret_cast<const float4*>(src + 4);
-        v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
         v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
-    } else {
-        float4 a = *reinterpret_cast<const float4*>(src);
-        v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
     }
 }
 template <>
@@ -60,6 +58,101 @@ __device__ __forceinline__ void load_vals<_Float16>(const _Float16* src, float* 
 #pragma unroll
         for (int i = 0; i < 4; i++) v[i] = (float)a[i];
     }
+}
+
+// Raw (unconverted) staging item as it comes from HBM/L2: CPI channels of one pixel.
+template <typename T, int CPI>
+struct RawItem;
+template <>
+struct RawItem<float, 8> {
+    float4 a, b;
+    __device__ __forceinline__ void zero() { a = b = make_float4(0.f, 0.f, 0.f, 0.f); }
+    __device__ __forceinline__ void load(const float* p) {
+        a = *reinterpret_cast<const float4*>(p);
+        b = *reinterpret_cast<const float4*>(p + 4);
+    }
+    __device__ __forceinline__ void get(float* v) const {
+        v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+    }
+};
+template <>
+struct RawItem<float, 4> {
+    float4 a;
+    __device__ __forceinline__ void zero() { a = make_float4(0.f, 0.f, 0.f, 0.f); }
+    __device__ __forceinline__ void load(const float* p) { a = *reinterpret_cast<const float4*>(p); }
+    __device__ __forceinline__ void get(float* v) const { v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; }
+};
+template <>
+struct RawItem<_Float16, 8> {
+    half8_t a;
+    __device__ __forceinline__ void zero() {
+#pragma unroll
+        for (int i = 0; i < 8; i++) a[i] = (_Float16)0.f;
+    }
+    __device__ __forceinline__ void load(const _Float16* p) { a = *reinterpret_cast<const half8_t*>(p); }
+    __device__ __forceinline__ void get(float* v) const {
+#pragma unroll
+        for (int i = 0; i < 8; i++) v[i] = (float)a[i];
+    }
+};
+template <>
+struct RawItem<_Float16, 4> {
+    half4_t a;
+    __device__ __forceinline__ void zero() {
+#pragma unroll
+        for (int i = 0; i < 4; i++) a[i] = (_Float16)0.f;
+    }
+    __device__ __forceinline__ void load(const _Float16* p) { a = *reinterpret_cast<const half4_t*>(p); }
+    __device__ __forceinline__ void get(float* v) const {
+#pragma unroll
+        for (int i = 0; i < 4; i++) v[i] = (float)a[i];
+    }
+};
+
+// Activates, converts (hi / lo fp16 planes when SPLIT) and writes one staging item to LDS.
+template <bool SPLIT, int CPI>
+__device__ __forceinline__ void stage_store(unsigned char* dst, int plane, const float* raw, const Act& act) {
+    float v[8];
+#pragma unroll
+    for (int i = 0; i < CPI; i++) v[i] = act_apply(raw[i], act);
+    if (CPI == 8) {
+        half8_t hi;
+#pragma unroll
+        for (int i = 0; i < 8; i++) hi[i] = (_Float16)v[i];
+        *reinterpret_cast<half8_t*>(dst) = hi;
+        if (SPLIT) {
+            half8_t lo;
+#pragma unroll
+            for (int i = 0; i < 8; i++) lo[i] = (_Float16)(v[i] - (float)hi[i]);
+            *reinterpret_cast<half8_t*>(dst + plane) = lo;
+        }
+    } else {
+        half4_t hi;
+#pragma unroll
+        for (int i = 0; i < 4; i++) hi[i] = (_Float16)v[i];
+        *reinterpret_cast<half4_t*>(dst) = hi;
+        if (SPLIT) {
+            half4_t lo;
+#pragma unroll
+            for (int i = 0; i < 4; i++) lo[i] = (_Float16)(v[i] - (float)hi[i]);
+            *reinterpret_cast<half4_t*>(dst + plane) = lo;
+        }
+    }
+}
+
+// One B (activation) fragment of a lane: 8 consecutive halves.  The small-Cin layout is only 8-byte
+// aligned, so it is read as two 4-half pieces.
+template <int KC>
+__device__ __forceinline__ half8_t load_b_frag(const unsigned char* src) {
+    if (KC == 4) {
+        const half4_t lo4 = *reinterpret_cast<const half4_t*>(src);
+        const half4_t hi4 = *reinterpret_cast<const half4_t*>(src + 8);
+        half8_t r;
+        r[0] = lo4[0]; r[1] = lo4[1]; r[2] = lo4[2]; r[3] = lo4[3];
+        r[4] = hi4[0]; r[5] = hi4[1]; r[6] = hi4[2]; r[7] = hi4[3];
+        return r;
+    }
+    return *reinterpret_cast<const half8_t*>(src);
 }
 
 template <typename TIn, typename TOut, bool SPLIT, int FM, int FN, int WM, int WN, int KC>
@@ -99,6 +192,9 @@ __global__ __launch_bounds__(256) void conv_mfma_kernel(const ConvMfmaParams p) 
     const float inv_hw = 1.0f / (float)p.halo_w;
     const TIn* in = reinterpret_cast<const TIn*>(p.in);
 
+    // LDS holds two staging buffers (double buffering across channel chunks) when there is more
+    // than one chunk; each buffer = NPL planes.
+    const int bufsz = NPL * p.plane;
     if (KC == 4) {
         // slack behind each plane is read by the last (zero-weight) k elements of a row run
         if (tid < 16 * NPL) {
@@ -130,105 +226,169 @@ __global__ __launch_bounds__(256) void conv_mfma_kernel(const ConvMfmaParams p) 
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
 
-    half8_t a_cur[FM][NPL];
+    // Ring of weight fragments PD steps deep: the fragments of step gs+PD are requested from L2 as soon
+    // as the MFMAs of step gs have been issued, so a load has PD-1 steps of MFMA work to complete.
+    constexpr int PD = SPLIT ? 3 : 4;
+    half8_t a_ring[PD][FM][NPL];
 #pragma unroll
-    for (int fm = 0; fm < FM; fm++)
+    for (int s = 0; s < PD; s++)
 #pragma unroll
-        for (int pl = 0; pl < NPL; pl++) a_cur[fm][pl] = wfrag[(fm * NPL + pl) * 64];
+        for (int fm = 0; fm < FM; fm++)
+#pragma unroll
+            for (int pl = 0; pl < NPL; pl++)
+                a_ring[s][fm][pl] = wfrag[(size_t)(s < total_steps ? s : 0) * wstep + (fm * NPL + pl) * 64];
 
-    int gs = 0;
-    for (int chunk = 0; chunk < p.cin_chunks; chunk++) {
-        __syncthreads();
-        // ---- stage the activated input halo tile of this channel chunk into LDS ----
-        for (int idx = tid; idx < nitems; idx += 256) {
+    // ---- staging machinery: items (pixel, 8-channel group) of the halo tile; the first NB items of a
+    //      thread are described once (their addresses only shift by the chunk's channel offset) and
+    //      are fetched for chunk c+1 while the MFMAs of chunk c run ----
+    constexpr int NB = 4;
+    int g_off[NB];   // element offset of the pixel in the input tensor, -1: outside (reads as 0)
+    int l_off[NB];   // LDS byte offset inside a plane, -1: no such item
+    int c_off[NB];   // channel offset of the group inside a chunk
+#pragma unroll
+    for (int i = 0; i < NB; i++) {
+        const int idx = tid + i * 256;
+        g_off[i] = -1; l_off[i] = -1; c_off[i] = 0;
+        if (idx < nitems) {
             const int pix = (G == 1) ? idx : idx / G;
             const int g = (G == 1) ? 0 : idx - pix * G;
             const int py = (int)(((float)pix + 0.5f) * inv_hw);
             const int px = pix - py * p.halo_w;
             const int gy = gy0 + py, gx = gx0 + px;
-            const int c0 = chunk * KC + g * CPI;
-            float v[8];
+            l_off[i] = pix * p.pitch + g * 16;
+            c_off[i] = g * CPI;
+            if ((unsigned)gy < (unsigned)p.in_hp && (unsigned)gx < (unsigned)p.in_wp) g_off[i] = (gy * p.in_wp + gx) * p.in_cp;
+        }
+    }
+    RawItem<TIn, CPI> raw[NB];
+    auto fetch_first = [&](int chunk) {
 #pragma unroll
-            for (int i = 0; i < 8; i++) v[i] = 0.f;
-            if ((unsigned)gy < (unsigned)p.in_hp && (unsigned)gx < (unsigned)p.in_wp && c0 < p.in_cp)
-                load_vals<TIn>(in + ((size_t)gy * p.in_wp + gx) * p.in_cp + c0, v, CPI);
+        for (int i = 0; i < NB; i++) {
+            const int c0 = chunk * KC + c_off[i];
+            raw[i].zero();
+            if (g_off[i] >= 0 && c0 < p.in_cp) raw[i].load(in + g_off[i] + c0);
+        }
+    };
+    auto store_first = [&](unsigned char* buf) {
 #pragma unroll
-            for (int i = 0; i < CPI; i++) v[i] = act_apply(v[i], p.act);
-            unsigned char* dst = lds + pix * p.pitch + g * 16;
-            if (CPI == 8) {
-                half8_t hi;
+        for (int i = 0; i < NB; i++) {
+            if (l_off[i] >= 0) {
+                float v[8];
+                raw[i].get(v);
+                stage_store<SPLIT, CPI>(buf + l_off[i], p.plane, v, p.act);
+            }
+        }
+    };
+    // items beyond the first NB*256 (large halo tiles) are staged without prefetch, NB at a time
+    auto stage_rest = [&](int chunk, unsigned char* buf) {
+        for (int base = NB * 256; base < nitems; base += NB * 256) {
+            RawItem<TIn, CPI> r2[NB];
+            int lo2[NB];
 #pragma unroll
-                for (int i = 0; i < 8; i++) hi[i] = (_Float16)v[i];
-                *reinterpret_cast<half8_t*>(dst) = hi;
-                if (SPLIT) {
-                    half8_t lo;
-#pragma unroll
-                    for (int i = 0; i < 8; i++) lo[i] = (_Float16)(v[i] - (float)hi[i]);
-                    *reinterpret_cast<half8_t*>(dst + p.plane) = lo;
+            for (int i = 0; i < NB; i++) {
+                const int idx = base + tid + i * 256;
+                lo2[i] = -1;
+                r2[i].zero();
+                if (idx < nitems) {
+                    const int pix = (G == 1) ? idx : idx / G;
+                    const int g = (G == 1) ? 0 : idx - pix * G;
+                    const int py = (int)(((float)pix + 0.5f) * inv_hw);
+                    const int px = pix - py * p.halo_w;
+                    const int gy = gy0 + py, gx = gx0 + px;
+                    const int c0 = chunk * KC + g * CPI;
+                    lo2[i] = pix * p.pitch + g * 16;
+                    if ((unsigned)gy < (unsigned)p.in_hp && (unsigned)gx < (unsigned)p.in_wp && c0 < p.in_cp)
+                        r2[i].load(in + (gy * p.in_wp + gx) * p.in_cp + c0);
                 }
-            } else {
-                half4_t hi;
+            }
 #pragma unroll
-                for (int i = 0; i < 4; i++) hi[i] = (_Float16)v[i];
-                *reinterpret_cast<half4_t*>(dst) = hi;
-                if (SPLIT) {
-                    half4_t lo;
-#pragma unroll
-                    for (int i = 0; i < 4; i++) lo[i] = (_Float16)(v[i] - (float)hi[i]);
-                    *reinterpret_cast<half4_t*>(dst + p.plane) = lo;
+            for (int i = 0; i < NB; i++) {
+                if (lo2[i] >= 0) {
+                    float v[8];
+                    r2[i].get(v);
+                    stage_store<SPLIT, CPI>(buf + lo2[i], p.plane, v, p.act);
                 }
             }
         }
-        __syncthreads();
-        // ---- all k16 steps (taps x channel sub-blocks) of this chunk ----
-        for (int t = 0; t < p.nsteps; t++, gs++) {
-            const int ao = p.aoff[t];
-            half8_t a_nxt[FM][NPL];
-            if (gs + 1 < total_steps) {
-                const half8_t* wn_ = wfrag + (size_t)(gs + 1) * wstep;
+    };
+
+    // prologue: chunk 0 into buffer 0
+    fetch_first(0);
+    store_first(lds);
+    stage_rest(0, lds);
+    __syncthreads();
+
+    // ---- main loop over all k16 steps (chunk-major).  B fragments of step t+1 are read from LDS while
+    //      the MFMAs of step t run; at a chunk boundary the next chunk's tile (fetched from HBM during this
+    //      chunk's MFMAs) is converted into the other LDS buffer, one barrier per chunk. ----
+    int chunk = 0, t = 0;
+    unsigned char* cur = lds;
+    if (p.cin_chunks > 1) fetch_first(1);
+    half8_t b_cur[FN][NPL];
+    {
+        const int ao = p.aoff[0];
+#pragma unroll
+        for (int fn = 0; fn < FN; fn++)
+#pragma unroll
+            for (int pl = 0; pl < NPL; pl++) b_cur[fn][pl] = load_b_frag<KC>(cur + pl * p.plane + boff[fn] + ao);
+    }
+    for (int gs0 = 0; gs0 < total_steps; gs0 += PD) {
+#pragma unroll
+        for (int s = 0; s < PD; s++) {
+            const int gs = gs0 + s;
+            if (gs < total_steps) {
+                const bool last_in_chunk = (t + 1 == p.nsteps);
+                half8_t b_nxt[FN][NPL];
+                if (!last_in_chunk) {
+                    const int ao = p.aoff[t + 1];
+#pragma unroll
+                    for (int fn = 0; fn < FN; fn++)
+#pragma unroll
+                        for (int pl = 0; pl < NPL; pl++) b_nxt[fn][pl] = load_b_frag<KC>(cur + pl * p.plane + boff[fn] + ao);
+                } else {
+#pragma unroll
+                    for (int fn = 0; fn < FN; fn++)
+#pragma unroll
+                        for (int pl = 0; pl < NPL; pl++) b_nxt[fn][pl] = b_cur[fn][pl];
+                }
 #pragma unroll
                 for (int fm = 0; fm < FM; fm++)
 #pragma unroll
-                    for (int pl = 0; pl < NPL; pl++) a_nxt[fm][pl] = wn_[(fm * NPL + pl) * 64];
-            } else {
+                    for (int fn = 0; fn < FN; fn++) {
+                        acc[fm][fn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_ring[s][fm][0], b_cur[fn][0], acc[fm][fn], 0, 0, 0);
+                        if (SPLIT) {
+                            acc[fm][fn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_ring[s][fm][1], b_cur[fn][0], acc[fm][fn], 0, 0, 0);
+                            acc[fm][fn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_ring[s][fm][0], b_cur[fn][1], acc[fm][fn], 0, 0, 0);
+                        }
+                    }
+                if (gs + PD < total_steps) {
+                    const half8_t* wn_ = wfrag + (size_t)(gs + PD) * wstep;
 #pragma unroll
-                for (int fm = 0; fm < FM; fm++)
+                    for (int fm = 0; fm < FM; fm++)
 #pragma unroll
-                    for (int pl = 0; pl < NPL; pl++) a_nxt[fm][pl] = a_cur[fm][pl];
+                        for (int pl = 0; pl < NPL; pl++) a_ring[s][fm][pl] = wn_[(fm * NPL + pl) * 64];
+                }
+#pragma unroll
+                for (int fn = 0; fn < FN; fn++)
+#pragma unroll
+                    for (int pl = 0; pl < NPL; pl++) b_cur[fn][pl] = b_nxt[fn][pl];
+                t++;
+                if (last_in_chunk && chunk + 1 < p.cin_chunks) {
+                    unsigned char* nxt = lds + ((chunk + 1) & 1) * bufsz;
+                    store_first(nxt);
+                    stage_rest(chunk + 1, nxt);
+                    __syncthreads();  // everyone is done reading `cur` and writing `nxt`
+                    chunk++;
+                    t = 0;
+                    cur = nxt;
+                    if (chunk + 1 < p.cin_chunks) fetch_first(chunk + 1);
+                    const int ao = p.aoff[0];
+#pragma unroll
+                    for (int fn = 0; fn < FN; fn++)
+#pragma unroll
+                        for (int pl = 0; pl < NPL; pl++) b_cur[fn][pl] = load_b_frag<KC>(cur + pl * p.plane + boff[fn] + ao);
+                }
             }
-            half8_t b[FN][NPL];
-#pragma unroll
-            for (int fn = 0; fn < FN; fn++)
-#pragma unroll
-                for (int pl = 0; pl < NPL; pl++) {
-                    const unsigned char* src = lds + pl * p.plane + boff[fn] + ao;
-                    if (KC == 4) {
-                        half4_t lo4 = *reinterpret_cast<const half4_t*>(src);
-                        half4_t hi4 = *reinterpret_cast<const half4_t*>(src + 8);
-                        half8_t r;
-                        r[0] = lo4[0]; r[1] = lo4[1]; r[2] = lo4[2]; r[3] = lo4[3];
-                        r[4] = hi4[0]; r[5] = hi4[1]; r[6] = hi4[2]; r[7] = hi4[3];
-                        b[fn][pl] = r;
-                    } else {
-                        b[fn][pl] = *reinterpret_cast<const half8_t*>(src);
-                    }
-                }
-#pragma unroll
-            for (int fm = 0; fm < FM; fm++)
-#pragma unroll
-                for (int fn = 0; fn < FN; fn++) {
-                    acc[fm][fn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_cur[fm][0], b[fn][0], acc[fm][fn], 0, 0, 0);
-                    if (SPLIT) {
-                        acc[fm][fn] =
-                            __builtin_amdgcn_mfma_f32_32x32x16_f16(a_cur[fm][1], b[fn][0], acc[fm][fn], 0, 0, 0);
-                        acc[fm][fn] =
-                            __builtin_amdgcn_mfma_f32_32x32x16_f16(a_cur[fm][0], b[fn][1], acc[fm][fn], 0, 0, 0);
-                    }
-                }
-#pragma unroll
-            for (int fm = 0; fm < FM; fm++)
-#pragma unroll
-                for (int pl = 0; pl < NPL; pl++) a_cur[fm][pl] = a_nxt[fm][pl];
         }
     }
 
@@ -329,9 +489,17 @@ int launch_conv_mfma(const ConvVariant& v, const ConvMfmaParams& p, size_t lds_b
     conv_kernel_fn fn = pick_kernel(v);
     if (!fn) return -1;
     if (lds_bytes > 48 * 1024) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                (int)lds_bytes) != hipSuccess)
-            return -2;
+        // raise the kernel's dynamic LDS limit once per kernel and size
+        static std::mutex mu;
+        static std::map<const void*, size_t> raised;
+        std::lock_guard<std::mutex> lk(mu);
+        size_t& cur = raised[reinterpret_cast<const void*>(fn)];
+        if (cur < lds_bytes) {
+            if (hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    (int)lds_bytes) != hipSuccess)
+                return -2;
+            cur = lds_bytes;
+        }
     }
     const int blocks = p.tiles_x * p.tiles_y * p.cout_blocks;
     hipLaunchKernelGGL(fn, dim3(blocks), dim3(256), lds_bytes, s, p);

@@ -3,6 +3,7 @@
 
 #include <algorithm>
 #include <cstring>
+#include <limits>
 
 namespace fynhip {
 
@@ -23,8 +24,12 @@ Layer::Layer(Net* n, const fyn_layer_desc& desc) : d(desc), net(n) {}
 Act Layer::act() const {
     // LayerBuilderTempl::getFlags (base/layerbuilder.h:445-493): RELU and LEAKY_RELU both set PRE_RELU,
     // the leak value distinguishes them (gpu/gpulayerbase.cpp:775-802).
-    Act a{ACT_NONE, 0.f, 0.f, 0.f};
+    // Kernels may evaluate the activation branch-free as min(hi, max(lo, x)) + leak * min(x, 0); the
+    // fields are normalised for that here.
+    const float inf = std::numeric_limits<float>::infinity();
+    Act a{ACT_NONE, 0.f, -inf, inf};
     if (d.flags & FYN_FLAG_PRE_RELU) {
+        a.lo = 0.f;
         if (d.leaky_relu != 0.f) {
             a.kind = ACT_LEAKY;
             a.leak = d.leaky_relu;

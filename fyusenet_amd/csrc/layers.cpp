@@ -106,8 +106,9 @@ struct TileChoice {
 static const int kTileTable[][4] = {{2, 2, 2, 2}, {2, 2, 1, 4}, {2, 1, 2, 2}, {2, 1, 1, 4},
                                     {1, 2, 1, 4}, {1, 1, 1, 4}, {1, 1, 4, 1}, {1, 1, 2, 2}};
 
-static TileChoice choose_tile(int cout, const SubConv& sc, int pitch, int npl, int slack) {
-    TileChoice best{0, 0, 0, 0, 0, 0, -1.0};
+// All tile configurations that fit, best heuristic score first.
+static std::vector<TileChoice> enumerate_tiles(int cout, const SubConv& sc, int pitch, int npl, int slack, int nbuf) {
+    std::vector<TileChoice> all;
     const char* force = getenv("FYNHIP_CONV_TILE");  // "fm,fn,wm,wn" for experiments
     int ff[4] = {0, 0, 0, 0};
     if (force) sscanf(force, "%d,%d,%d,%d", &ff[0], &ff[1], &ff[2], &ff[3]);
@@ -122,35 +123,41 @@ static TileChoice choose_tile(int cout, const SubConv& sc, int pitch, int npl, i
         const int cpb = wm * fm * 32;
         const int cblocks = (cout + cpb - 1) / cpb;
         const int halo_w = (tw - 1) * sc.in_stride + sc.span_x, halo_h = (th - 1) * sc.in_stride + sc.span_y;
-        const size_t lds = (size_t)npl * ((size_t)halo_h * halo_w * pitch + slack);
+        const size_t lds = (size_t)nbuf * npl * ((size_t)halo_h * halo_w * pitch + slack);
         if (lds > 150 * 1024) continue;
         const double util = ((double)cout * sc.npos_x * sc.npos_y) / ((double)cblocks * cpb * (double)tiles * bm);
         const double blocks = (double)tiles * cblocks;
         const double slots = 256.0 * (lds > 72 * 1024 ? 1 : 2);
         const double par = blocks >= slots ? blocks / (std::ceil(blocks / slots) * slots) : blocks / slots;
         const double bonus = (fm * fn == 4) ? 1.0 : (fm * fn == 2 ? 0.85 : 0.7);
-        const double score = util * par * bonus;
-        if (score > best.score) best = TileChoice{fm, fn, wm, wn, ilog2(tw), th, score};
+        all.push_back(TileChoice{fm, fn, wm, wn, ilog2(tw), th, util * par * bonus});
     }
-    if (best.score < 0) fail(FYN_ERR_UNSUPPORTED, "no MFMA tile configuration fits this convolution");
-    return best;
+    if (all.empty()) fail(FYN_ERR_UNSUPPORTED, "no MFMA tile configuration fits this convolution");
+    std::sort(all.begin(), all.end(), [](const TileChoice& x, const TileChoice& y) { return x.score > y.score; });
+    return all;
 }
 
-// Builds the launch description of one (sub-)convolution; weights are packed separately.
+static void conv_geometry(const TView& in, bool split, int& kc, int& pitch, int& slack, int& npl) {
+    if (in.cp == 4) kc = 4;
+    else if (in.cp <= 16) kc = 16;
+    else kc = 32;
+    pitch = (kc == 4) ? 8 : kc * 2 + 16;
+    slack = (kc == 4) ? 64 : 0;
+    npl = split ? 2 : 1;
+}
+
+// Builds the launch description of one (sub-)convolution for one tile configuration.  The packed
+// weight layout does not depend on the tile configuration (cout fragments are padded to a multiple
+// of 4), so candidates can share one weight buffer (`share`); weights are packed separately.
 static MfmaLaunch plan_mfma(Net* net, const SubConv& sc, const TView& in, const TView& out, const TView* res, int cin,
-                            int cout, const Act& act, int res_relu, int res_scale) {
+                            int cout, const Act& act, int res_relu, int res_scale, const TileChoice& tc,
+                            const float* scale, const float* bias, const MfmaLaunch* share = nullptr) {
     MfmaLaunch L;
     L.cin = cin;
     L.cout = cout;
     const bool split = !net->f16();
-    const int npl = split ? 2 : 1;
-    int kc;
-    if (in.cp == 4) kc = 4;
-    else if (in.cp <= 16) kc = 16;
-    else kc = 32;
-    const int pitch = (kc == 4) ? 8 : kc * 2 + 16;
-    const int slack = (kc == 4) ? 64 : 0;
-    const TileChoice tc = choose_tile(cout, sc, pitch, npl, slack);
+    int kc, pitch, slack, npl;
+    conv_geometry(in, split, kc, pitch, slack, npl);
     const int tw = 1 << tc.twl;
     ConvMfmaParams& p = L.p;
     p.in = in.ptr;
@@ -176,10 +183,13 @@ static MfmaLaunch plan_mfma(Net* net, const SubConv& sc, const TView& in, const 
     p.cin_chunks = (kc == 4) ? 1 : (in.cp + kc - 1) / kc;
     const int cpb = tc.wm * tc.fm * 32;
     p.cout_blocks = (cout + cpb - 1) / cpb;
-    p.mfrags = p.cout_blocks * tc.wm * tc.fm;
+    p.mfrags = ((cout + 31) / 32 + 3) / 4 * 4;
+    p.scale = scale;
+    p.bias = bias;
     p.acc_mul = 1.f;
     p.act = act;
-    L.lds = (size_t)npl * p.plane;
+    L.lds = (size_t)npl * p.plane * (p.cin_chunks > 1 ? 2 : 1);  // double-buffered across channel chunks
+    if (in.elems() >= (size_t)1 << 31) fail(FYN_ERR_UNSUPPORTED, "input tensor too large for 32-bit element offsets");
     L.var = ConvVariant{in.f16, out.f16, split ? 1 : 0, tc.fm, tc.fn, tc.wm, tc.wn, kc};
     if (!conv_mfma_variant_exists(L.var)) fail(FYN_ERR_UNSUPPORTED, "MFMA convolution variant not compiled");
 
@@ -225,9 +235,60 @@ static MfmaLaunch plan_mfma(Net* net, const SubConv& sc, const TView& in, const 
     L.aoff_dev = upload(net, aoff);
     p.aoff = L.aoff_dev;
     L.wpack_halves = (size_t)p.cin_chunks * p.nsteps * p.mfrags * npl * 64 * 8;
-    L.wpack_dev = net->dev_alloc(L.wpack_halves * 2, false);
+    if (share) {
+        if (share->wpack_halves != L.wpack_halves) fail(FYN_ERR_INVALID, "internal: weight layouts of tile candidates differ");
+        L.wpack_dev = share->wpack_dev;
+    } else {
+        L.wpack_dev = net->dev_alloc(L.wpack_halves * 2, true);
+    }
     p.wpack = L.wpack_dev;
     return L;
+}
+
+static std::string mfma_info(const MfmaLaunch& L);
+
+static float time_launch(Net* net, const MfmaLaunch& L, int iters) {
+    hipEvent_t a, b;
+    FYN_HIP(hipEventCreate(&a));
+    FYN_HIP(hipEventCreate(&b));
+    if (launch_conv_mfma(L.var, L.p, L.lds, net->stream) != 0) fail(FYN_ERR_DEVICE, "convolution launch failed while tuning");
+    FYN_HIP(hipEventRecord(a, net->stream));
+    for (int i = 0; i < iters; i++) launch_conv_mfma(L.var, L.p, L.lds, net->stream);
+    FYN_HIP(hipEventRecord(b, net->stream));
+    FYN_HIP(hipEventSynchronize(b));
+    FYN_HIP(hipGetLastError());
+    float ms = 0.f;
+    FYN_HIP(hipEventElapsedTime(&ms, a, b));
+    (void)hipEventDestroy(a);
+    (void)hipEventDestroy(b);
+    return ms / iters;
+}
+
+// Picks the tile configuration of one (sub-)convolution: by measurement on the layer's own tensors
+// (default; timing does not depend on the data), or by the heuristic score when FYNHIP_AUTOTUNE=0.
+static MfmaLaunch tune_mfma(Net* net, const SubConv& sc, const TView& in, const TView& out, const TView* res, int cin,
+                            int cout, const Act& act, int res_relu, int res_scale, const float* scale, const float* bias) {
+    int kc, pitch, slack, npl;
+    conv_geometry(in, !net->f16(), kc, pitch, slack, npl);
+    const int chunks = (kc == 4) ? 1 : (in.cp + kc - 1) / kc;
+    std::vector<TileChoice> cands = enumerate_tiles(cout, sc, pitch, npl, slack, chunks > 1 ? 2 : 1);
+    const char* at = getenv("FYNHIP_AUTOTUNE");
+    const bool tune = !(at && at[0] == '0') && cands.size() > 1;
+    MfmaLaunch best = plan_mfma(net, sc, in, out, res, cin, cout, act, res_relu, res_scale, cands[0], scale, bias);
+    if (!tune) return best;
+    const bool verbose = getenv("FYNHIP_TUNE_VERBOSE") != nullptr;
+    float best_ms = std::min(time_launch(net, best, 4), time_launch(net, best, 4));
+    if (verbose) fprintf(stderr, "[tune] %s -> %.1f us\n", mfma_info(best).c_str(), best_ms * 1e3f);
+    for (size_t i = 1; i < cands.size(); i++) {
+        MfmaLaunch L = plan_mfma(net, sc, in, out, res, cin, cout, act, res_relu, res_scale, cands[i], scale, bias, &best);
+        const float ms = std::min(time_launch(net, L, 4), time_launch(net, L, 4));
+        if (verbose) fprintf(stderr, "[tune] %s -> %.1f us\n", mfma_info(L).c_str(), ms * 1e3f);
+        if (ms < best_ms) {
+            best_ms = ms;
+            best = L;
+        }
+    }
+    return best;
 }
 
 // Packs weights W[o][ky][kx][i] (block order, base/convlayerinterface.h:71-95) into the per-lane A
@@ -337,16 +398,15 @@ class ConvLayer : public Layer {
             sc.out_step = 1;
             sc.out_off_y = sc.out_off_x = out_v.pad;
             if (res_v) sc.res_off_y = sc.res_off_x = res_v->pad;
-            launch = plan_mfma(net, sc, in_v, out_v, res_v, d.in_channels, oc, act(), res_relu, res_scale);
-            padded = launch.p.mfrags * 32;
+            padded = std::max((oc + 127) / 128 * 128, out_v.cp);
+            scale_dev = static_cast<float*>(net->dev_alloc(padded * sizeof(float)));
+            bias_dev = static_cast<float*>(net->dev_alloc(padded * sizeof(float)));
+            launch = tune_mfma(net, sc, in_v, out_v, res_v, d.in_channels, oc, act(), res_relu, res_scale, scale_dev, bias_dev);
         }
-        padded = std::max(padded, out_v.cp);
-        scale_dev = static_cast<float*>(net->dev_alloc(padded * sizeof(float)));
-        bias_dev = static_cast<float*>(net->dev_alloc(padded * sizeof(float)));
         if (direct) {
+            scale_dev = static_cast<float*>(net->dev_alloc(padded * sizeof(float)));
+            bias_dev = static_cast<float*>(net->dev_alloc(padded * sizeof(float)));
             dp.w = wdirect_dev; dp.scale = scale_dev; dp.bias = bias_dev;
-        } else {
-            launch.p.scale = scale_dev; launch.p.bias = bias_dev;
         }
         set_up = true;
         if (!block.empty()) pack();
@@ -481,7 +541,9 @@ class TransConvLayer : public Layer {
     void setup() override {
         const TView& in_v = tin(0).v;
         const TView& out_v = tout().v;
-        padded = out_v.cp;
+        padded = std::max((oc + 127) / 128 * 128, out_v.cp);
+        scale_dev = static_cast<float*>(net->dev_alloc(padded * sizeof(float)));
+        bias_dev = static_cast<float*>(net->dev_alloc(padded * sizeof(float)));
         for (int py = 0; py < 2; py++)
             for (int px = 0; px < 2; px++) {
                 SubConv sc;
@@ -499,15 +561,8 @@ class TransConvLayer : public Layer {
                 sc.out_step = 2;
                 sc.out_off_y = out_v.pad + py;
                 sc.out_off_x = out_v.pad + px;
-                launches.push_back(plan_mfma(net, sc, in_v, out_v, nullptr, d.in_channels, oc, act(), 0, 0));
-                padded = std::max(padded, launches.back().p.mfrags * 32);
+                launches.push_back(tune_mfma(net, sc, in_v, out_v, nullptr, d.in_channels, oc, act(), 0, 0, scale_dev, bias_dev));
             }
-        scale_dev = static_cast<float*>(net->dev_alloc(padded * sizeof(float)));
-        bias_dev = static_cast<float*>(net->dev_alloc(padded * sizeof(float)));
-        for (auto& L : launches) {
-            L.p.scale = scale_dev;
-            L.p.bias = bias_dev;
-        }
         set_up = true;
         if (!block.empty()) pack();
     }
