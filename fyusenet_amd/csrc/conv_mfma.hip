@@ -226,17 +226,11 @@ __global__ __launch_bounds__(256) void conv_mfma_kernel(const ConvMfmaParams p) 
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
 
-    // Ring of weight fragments PD steps deep: the fragments of step gs+PD are requested from L2 as soon
-    // as the MFMAs of step gs have been issued, so a load has PD-1 steps of MFMA work to complete.
-    constexpr int PD = SPLIT ? 3 : 4;
-    half8_t a_ring[PD][FM][NPL];
+    half8_t a_cur[FM][NPL];
 #pragma unroll
-    for (int s = 0; s < PD; s++)
+    for (int fm = 0; fm < FM; fm++)
 #pragma unroll
-        for (int fm = 0; fm < FM; fm++)
-#pragma unroll
-            for (int pl = 0; pl < NPL; pl++)
-                a_ring[s][fm][pl] = wfrag[(size_t)(s < total_steps ? s : 0) * wstep + (fm * NPL + pl) * 64];
+        for (int pl = 0; pl < NPL; pl++) a_cur[fm][pl] = wfrag[(fm * NPL + pl) * 64];
 
     // ---- staging machinery: items (pixel, 8-channel group) of the halo tile; the first NB items of a
     //      thread are described once (their addresses only shift by the chunk's channel offset) and
@@ -332,63 +326,63 @@ __global__ __launch_bounds__(256) void conv_mfma_kernel(const ConvMfmaParams p) 
 #pragma unroll
             for (int pl = 0; pl < NPL; pl++) b_cur[fn][pl] = load_b_frag<KC>(cur + pl * p.plane + boff[fn] + ao);
     }
-    for (int gs0 = 0; gs0 < total_steps; gs0 += PD) {
+    for (int gs = 0; gs < total_steps; gs++) {
+        const bool last_in_chunk = (t + 1 == p.nsteps);
+        half8_t a_nxt[FM][NPL];
+        half8_t b_nxt[FN][NPL];
+        {
+            // fragments of step gs+1: A from L2, B from LDS, both in flight during this step's MFMAs
+            const half8_t* wn_ = wfrag + (size_t)(gs + 1 < total_steps ? gs + 1 : gs) * wstep;
 #pragma unroll
-        for (int s = 0; s < PD; s++) {
-            const int gs = gs0 + s;
-            if (gs < total_steps) {
-                const bool last_in_chunk = (t + 1 == p.nsteps);
-                half8_t b_nxt[FN][NPL];
-                if (!last_in_chunk) {
-                    const int ao = p.aoff[t + 1];
+            for (int fm = 0; fm < FM; fm++)
 #pragma unroll
-                    for (int fn = 0; fn < FN; fn++)
+                for (int pl = 0; pl < NPL; pl++) a_nxt[fm][pl] = wn_[(fm * NPL + pl) * 64];
+        }
+        if (!last_in_chunk) {
+            const int ao = p.aoff[t + 1];
 #pragma unroll
-                        for (int pl = 0; pl < NPL; pl++) b_nxt[fn][pl] = load_b_frag<KC>(cur + pl * p.plane + boff[fn] + ao);
-                } else {
+            for (int fn = 0; fn < FN; fn++)
 #pragma unroll
-                    for (int fn = 0; fn < FN; fn++)
+                for (int pl = 0; pl < NPL; pl++) b_nxt[fn][pl] = load_b_frag<KC>(cur + pl * p.plane + boff[fn] + ao);
+        } else {
 #pragma unroll
-                        for (int pl = 0; pl < NPL; pl++) b_nxt[fn][pl] = b_cur[fn][pl];
-                }
+            for (int fn = 0; fn < FN; fn++)
 #pragma unroll
-                for (int fm = 0; fm < FM; fm++)
+                for (int pl = 0; pl < NPL; pl++) b_nxt[fn][pl] = b_cur[fn][pl];
+        }
 #pragma unroll
-                    for (int fn = 0; fn < FN; fn++) {
-                        acc[fm][fn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_ring[s][fm][0], b_cur[fn][0], acc[fm][fn], 0, 0, 0);
-                        if (SPLIT) {
-                            acc[fm][fn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_ring[s][fm][1], b_cur[fn][0], acc[fm][fn], 0, 0, 0);
-                            acc[fm][fn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_ring[s][fm][0], b_cur[fn][1], acc[fm][fn], 0, 0, 0);
-                        }
-                    }
-                if (gs + PD < total_steps) {
-                    const half8_t* wn_ = wfrag + (size_t)(gs + PD) * wstep;
+        for (int fm = 0; fm < FM; fm++)
 #pragma unroll
-                    for (int fm = 0; fm < FM; fm++)
-#pragma unroll
-                        for (int pl = 0; pl < NPL; pl++) a_ring[s][fm][pl] = wn_[(fm * NPL + pl) * 64];
-                }
-#pragma unroll
-                for (int fn = 0; fn < FN; fn++)
-#pragma unroll
-                    for (int pl = 0; pl < NPL; pl++) b_cur[fn][pl] = b_nxt[fn][pl];
-                t++;
-                if (last_in_chunk && chunk + 1 < p.cin_chunks) {
-                    unsigned char* nxt = lds + ((chunk + 1) & 1) * bufsz;
-                    store_first(nxt);
-                    stage_rest(chunk + 1, nxt);
-                    __syncthreads();  // everyone is done reading `cur` and writing `nxt`
-                    chunk++;
-                    t = 0;
-                    cur = nxt;
-                    if (chunk + 1 < p.cin_chunks) fetch_first(chunk + 1);
-                    const int ao = p.aoff[0];
-#pragma unroll
-                    for (int fn = 0; fn < FN; fn++)
-#pragma unroll
-                        for (int pl = 0; pl < NPL; pl++) b_cur[fn][pl] = load_b_frag<KC>(cur + pl * p.plane + boff[fn] + ao);
+            for (int fn = 0; fn < FN; fn++) {
+                acc[fm][fn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_cur[fm][0], b_cur[fn][0], acc[fm][fn], 0, 0, 0);
+                if (SPLIT) {
+                    acc[fm][fn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_cur[fm][1], b_cur[fn][0], acc[fm][fn], 0, 0, 0);
+                    acc[fm][fn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_cur[fm][0], b_cur[fn][1], acc[fm][fn], 0, 0, 0);
                 }
             }
+#pragma unroll
+        for (int fm = 0; fm < FM; fm++)
+#pragma unroll
+            for (int pl = 0; pl < NPL; pl++) a_cur[fm][pl] = a_nxt[fm][pl];
+#pragma unroll
+        for (int fn = 0; fn < FN; fn++)
+#pragma unroll
+            for (int pl = 0; pl < NPL; pl++) b_cur[fn][pl] = b_nxt[fn][pl];
+        t++;
+        if (last_in_chunk && chunk + 1 < p.cin_chunks) {
+            unsigned char* nxt = lds + ((chunk + 1) & 1) * bufsz;
+            store_first(nxt);
+            stage_rest(chunk + 1, nxt);
+            __syncthreads();  // everyone is done reading `cur` and writing `nxt`
+            chunk++;
+            t = 0;
+            cur = nxt;
+            if (chunk + 1 < p.cin_chunks) fetch_first(chunk + 1);
+            const int ao = p.aoff[0];
+#pragma unroll
+            for (int fn = 0; fn < FN; fn++)
+#pragma unroll
+                for (int pl = 0; pl < NPL; pl++) b_cur[fn][pl] = load_b_frag<KC>(cur + pl * p.plane + boff[fn] + ao);
         }
     }
 
