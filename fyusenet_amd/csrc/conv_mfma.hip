@@ -28,6 +28,7 @@ namespace fynhip {
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
 typedef float float16_t __attribute__((ext_vector_type(16)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
 
 // Branch-free activation: the host normalises every activation kind to
 //   act(x) = min(hi, max(lo, x)) + leak * min(x, 0)
@@ -386,50 +387,69 @@ __global__ __launch_bounds__(256) void conv_mfma_kernel(const ConvMfmaParams p) 
         }
     }
 
-    // ---- epilogue: lane holds, per fragment, column (position) lane%32 and rows (channels)
-    //      8*(r/4) + 4*(lane/32) + r%4 ----
+    // ---- epilogue.  A lane holds, per fragment, column (position) lane%32 and rows (channels)
+    //      8*(r/4) + 4*(lane/32) + r%4.  The wave transposes its accumulators through a private LDS area
+    //      so that it writes, per position, one contiguous run of FM*32 channels (128-256 B) instead of
+    //      16-byte pieces; scale, bias' and the residual are applied on the way out
+    //      (shaders/deep/deepconv3x3_tiled.frag:36-45 order). ----
+    __syncthreads();  // all waves are done with the staged tiles; LDS is reused below
+    constexpr int ROWF = FM * 32 + 4;                 // floats per position row (+4: bank spread)
+    constexpr int LPP = FM * 8;                       // lanes per position on the way out
+    constexpr int PPI = 64 / LPP;                     // positions per store instruction
+    float* tr = reinterpret_cast<float*>(lds) + wave * (32 * ROWF);
     TOut* out = reinterpret_cast<TOut*>(p.out);
     const TOut* res = reinterpret_cast<const TOut*>(p.res);
+    const int c4 = (lane % LPP) * 4;                                   // channel offset inside the wave's range
+    const int c = ((cb * WM + wm) * FM) * 32 + c4;                     // absolute output channel
+    const bool c_ok = c < p.out_cp;
+    f32x4_t sc = (f32x4_t)(0.f), bi = (f32x4_t)(0.f);
+    if (c_ok) {
+        sc = *reinterpret_cast<const f32x4_t*>(p.scale + c);
+        bi = *reinterpret_cast<const f32x4_t*>(p.bias + c);
+    }
 #pragma unroll
     for (int fn = 0; fn < FN; fn++) {
-        const int m = (wn * FN + fn) * 32 + (lane & 31);
-        const int py = pos_y0 + (m >> twl), px = pos_x0 + (m & (TW - 1));
-        if (py >= p.npos_y || px >= p.npos_x) continue;
-        const size_t obase = ((size_t)(p.out_off_y + py * p.out_step) * p.out_wp + p.out_off_x + px * p.out_step) * p.out_cp;
-        const size_t rbase = res ? ((size_t)(p.res_off_y + py * p.out_step) * p.res_wp + p.res_off_x + px * p.out_step) * p.res_cp : 0;
 #pragma unroll
-        for (int fm = 0; fm < FM; fm++) {
+        for (int fm = 0; fm < FM; fm++)
 #pragma unroll
             for (int q = 0; q < 4; q++) {
-                const int c = ((cb * WM + wm) * FM + fm) * 32 + q * 8 + (lane >> 5) * 4;
-                if (c >= p.out_cp) continue;
-                const float4 sc = *reinterpret_cast<const float4*>(p.scale + c);
-                const float4 bi = *reinterpret_cast<const float4*>(p.bias + c);
-                float o[4];
-                o[0] = (acc[fm][fn][q * 4 + 0] * p.acc_mul) * sc.x + bi.x;
-                o[1] = (acc[fm][fn][q * 4 + 1] * p.acc_mul) * sc.y + bi.y;
-                o[2] = (acc[fm][fn][q * 4 + 2] * p.acc_mul) * sc.z + bi.z;
-                o[3] = (acc[fm][fn][q * 4 + 3] * p.acc_mul) * sc.w + bi.w;
-                if (res) {
-                    float r[8];
-                    load_vals<TOut>(res + rbase + c, r, 4);
-                    const float rs[4] = {sc.x, sc.y, sc.z, sc.w};
+                f32x4_t v;
+                v[0] = acc[fm][fn][q * 4 + 0]; v[1] = acc[fm][fn][q * 4 + 1];
+                v[2] = acc[fm][fn][q * 4 + 2]; v[3] = acc[fm][fn][q * 4 + 3];
+                *reinterpret_cast<f32x4_t*>(tr + (lane & 31) * ROWF + fm * 32 + q * 8 + (lane >> 5) * 4) = v;
+            }
 #pragma unroll
-                    for (int i = 0; i < 4; i++) {
-                        float rv = r[i];
-                        if (p.res_relu) rv = fmaxf(rv, 0.f);
-                        if (p.res_scale) rv *= rs[i];
-                        o[i] += rv;
-                    }
-                }
-                if (sizeof(TOut) == 4) {
-                    *reinterpret_cast<float4*>(reinterpret_cast<float*>(out) + obase + c) = make_float4(o[0], o[1], o[2], o[3]);
-                } else {
-                    half4_t hv;
+        for (int it = 0; it < 32 / PPI; it++) {
+            const int row = it * PPI + lane / LPP;
+            const f32x4_t a4 = *reinterpret_cast<const f32x4_t*>(tr + row * ROWF + c4);
+            const int m = (wn * FN + fn) * 32 + row;
+            const int py = pos_y0 + (m >> twl), px = pos_x0 + (m & (TW - 1));
+            if (!c_ok || py >= p.npos_y || px >= p.npos_x) continue;
+            float o[4];
 #pragma unroll
-                    for (int i = 0; i < 4; i++) hv[i] = (_Float16)o[i];
-                    *reinterpret_cast<half4_t*>(reinterpret_cast<_Float16*>(out) + obase + c) = hv;
+            for (int i = 0; i < 4; i++) o[i] = (a4[i] * p.acc_mul) * sc[i] + bi[i];
+            if (res) {
+                const size_t rbase = ((size_t)(p.res_off_y + py * p.out_step) * p.res_wp + p.res_off_x + px * p.out_step) * p.res_cp;
+                float r[8];
+                load_vals<TOut>(res + rbase + c, r, 4);
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    float rv = r[i];
+                    if (p.res_relu) rv = fmaxf(rv, 0.f);
+                    if (p.res_scale) rv *= sc[i];
+                    o[i] += rv;
                 }
+            }
+            const size_t obase = ((size_t)(p.out_off_y + py * p.out_step) * p.out_wp + p.out_off_x + px * p.out_step) * p.out_cp;
+            if (sizeof(TOut) == 4) {
+                f32x4_t ov;
+                ov[0] = o[0]; ov[1] = o[1]; ov[2] = o[2]; ov[3] = o[3];
+                *reinterpret_cast<f32x4_t*>(reinterpret_cast<float*>(out) + obase + c) = ov;
+            } else {
+                half4_t hv;
+#pragma unroll
+                for (int i = 0; i < 4; i++) hv[i] = (_Float16)o[i];
+                *reinterpret_cast<half4_t*>(reinterpret_cast<_Float16*>(out) + obase + c) = hv;
             }
         }
     }

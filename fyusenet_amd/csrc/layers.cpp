@@ -189,6 +189,7 @@ static MfmaLaunch plan_mfma(Net* net, const SubConv& sc, const TView& in, const 
     p.acc_mul = 1.f;
     p.act = act;
     L.lds = (size_t)npl * p.plane * (p.cin_chunks > 1 ? 2 : 1);  // double-buffered across channel chunks
+    L.lds = std::max(L.lds, (size_t)4 * 32 * (tc.fm * 32 + 4) * 4);      // epilogue transposition area
     if (in.elems() >= (size_t)1 << 31) fail(FYN_ERR_UNSUPPORTED, "input tensor too large for 32-bit element offsets");
     L.var = ConvVariant{in.f16, out.f16, split ? 1 : 0, tc.fm, tc.fn, tc.wm, tc.wn, kc};
     if (!conv_mfma_variant_exists(L.var)) fail(FYN_ERR_UNSUPPORTED, "MFMA convolution variant not compiled");
