@@ -133,6 +133,19 @@ void launch_concat_part(const TView& in, const TView& out, int c_off, const Act&
 // out: 2 channels (index as float, max value); idx_out optional int32 [h*w].
 void launch_argmax(const TView& in, const TView& out, int32_t* idx_out, const Act& act, hipStream_t s);
 
+// Second stage of a convolution with few output channels and a wide kernel (cout*K <= 32): the MFMA
+// stage produced q[y][x'][o*K+kx] = sum_{ky,ci} W[o,ky,kx,ci]*act(in[y+ky-r, x'-r, ci]) for x' in
+// [0, W+K-1); this stage forms out[y,x,o] = (sum_kx q[y][x+kx][o*K+kx]) * scale + bias' (+ residual).
+struct ShiftReduceParams {
+    TView q, out, res;
+    int k, cout;
+    float acc_mul;
+    const float* scale;
+    const float* bias;
+    int res_relu, res_scale;
+};
+void launch_shift_reduce(const ShiftReduceParams& p, hipStream_t s);
+
 struct GemvParams {
     TView in, out;       // 1x1 spatial
     const void* w;       // [cout][cinp] in storage type (f16) or fp32

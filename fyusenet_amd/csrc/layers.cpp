@@ -294,7 +294,8 @@ static MfmaLaunch tune_mfma(Net* net, const SubConv& sc, const TView& in, const 
 
 // Packs weights W[o][ky][kx][i] (block order, base/convlayerinterface.h:71-95) into the per-lane A
 // fragment order of the kernel: [(chunk, step)][mfrag][plane][lane][8 halves].
-static void pack_mfma_weights(Net* net, MfmaLaunch& L, const float* w, int k, float wmul) {
+static void pack_mfma_weights(Net* net, MfmaLaunch& L, const float* w, int k, float wmul, int kw = -1) {
+    if (kw < 0) kw = k;
     const ConvMfmaParams& p = L.p;
     const int npl = L.var.split ? 2 : 1;
     const int kc = L.var.kc;
@@ -312,7 +313,7 @@ static void pack_mfma_weights(Net* net, MfmaLaunch& L, const float* w, int k, fl
                         if (st.ci[e] < 0) continue;
                         const int ci = chunk * kc + st.ci[e];
                         if (ci >= L.cin) continue;
-                        const float v = w[(((size_t)o * k + st.ky[e]) * k + st.kx[e]) * L.cin + ci] * wmul;
+                        const float v = w[(((size_t)o * k + st.ky[e]) * kw + st.kx[e]) * L.cin + ci] * wmul;
                         const uint16_t hi = f2h_bits(v);
                         base[(size_t)lane * 8 + j] = hi;
                         if (npl == 2) base[(size_t)(64 + lane) * 8 + j] = f2h_bits(v - h2f(hi));
@@ -363,6 +364,10 @@ class ConvLayer : public Layer {
         // shallow, unpadded input: the sampler clamps to the edge (gpu/gpulayerbase.h:80-90)
         clamp = !(d.flags & FYN_FLAG_DEEP) && d.input_padding < r * dil && k > 1;
         direct = clamp || getenv("FYNHIP_FORCE_DIRECT_CONV") != nullptr;
+        // few output channels under a wide kernel: fold the kx taps into the GEMM's M dimension
+        // (cout*K virtual channels, K taps) and reduce the K shifted partial sums in a second pass
+        wide = !direct && oc <= 4 && oc * k <= 32 && k >= 3 && stride == 1 && dil == 1 && d.in_channels > 4 &&
+               getenv("FYNHIP_NO_WIDE_CONV") == nullptr;
     }
     size_t weight_floats() const override {
         return (size_t)oc + (size_t)oc * k * k * d.in_channels + ((d.flags & FYN_FLAG_POST_BATCHNORM) ? 2 * (size_t)oc : 0);
@@ -388,6 +393,30 @@ class ConvLayer : public Layer {
             dp.act = act();
             padded = out_v.cp;
             wdirect_dev = static_cast<float*>(net->dev_alloc((size_t)k * k * d.in_channels * out_v.cp * sizeof(float)));
+        } else if (wide) {
+            // stage 1: q[y][x'][o*K+kx], x' in [0, W+K-1) <-> input column x'-r
+            qv = TView{};
+            qv.h = oh; qv.w = ow + k - 1; qv.pad = 0; qv.c = oc * k; qv.cp = channel_pitch(oc * k); qv.f16 = out_v.f16;
+            qv.ptr = net->dev_alloc(qv.bytes());
+            SubConv sc;
+            for (int ky = 0; ky < k; ky++) sc.taps.push_back(Tap{ky, 0, ky, 0});
+            sc.span_y = k; sc.span_x = 1;
+            sc.in_y0 = in_v.pad - r;
+            sc.in_x0 = in_v.pad - r;
+            sc.in_stride = 1;
+            sc.npos_y = qv.h; sc.npos_x = qv.w;
+            sc.out_step = 1;
+            sc.out_off_y = sc.out_off_x = 0;
+            padded = std::max((oc * k + 127) / 128 * 128, out_v.cp);
+            scale_dev = static_cast<float*>(net->dev_alloc(padded * sizeof(float)));
+            bias_dev = static_cast<float*>(net->dev_alloc(padded * sizeof(float)));
+            q_scale_dev = static_cast<float*>(net->dev_alloc(padded * sizeof(float)));
+            q_bias_dev = static_cast<float*>(net->dev_alloc(padded * sizeof(float)));
+            launch = tune_mfma(net, sc, in_v, qv, nullptr, d.in_channels, oc * k, act(), 0, 0, q_scale_dev, q_bias_dev);
+            sr.q = qv; sr.out = out_v; sr.res = res_v ? *res_v : TView{};
+            sr.k = k; sr.cout = oc;
+            sr.scale = scale_dev; sr.bias = bias_dev;
+            sr.res_relu = res_relu; sr.res_scale = res_scale;
         } else {
             SubConv sc;
             for (int ky = 0; ky < k; ky++)
@@ -429,6 +458,22 @@ class ConvLayer : public Layer {
                         for (int i = 0; i < cin; i++)
                             wd[(((size_t)ky * k + kx) * cin + i) * cp + o] = w[(((size_t)o * k + ky) * k + kx) * cin + i];
             reupload(net, wdirect_dev, wd);
+        } else if (wide) {
+            const int cin = d.in_channels;
+            const float wmul = weight_prescale(w, (size_t)oc * k * k * cin);
+            // virtual weights Wv[o*K+kx][ky][0][ci] = W[o][ky][kx][ci]
+            std::vector<float> wv((size_t)oc * k * k * cin);
+            for (int o = 0; o < oc; o++)
+                for (int ky = 0; ky < k; ky++)
+                    for (int kx = 0; kx < k; kx++)
+                        memcpy(&wv[(((size_t)(o * k + kx)) * k + ky) * cin], &w[(((size_t)o * k + ky) * k + kx) * cin], cin * sizeof(float));
+            std::vector<float> ones(padded, 0.f), zeros(padded, 0.f);
+            for (int i = 0; i < oc * k; i++) ones[i] = 1.f;
+            reupload(net, q_scale_dev, ones);
+            reupload(net, q_bias_dev, zeros);
+            launch.p.acc_mul = 1.0f;         // the pre-scaling is undone in the second stage
+            sr.acc_mul = 1.0f / wmul;
+            pack_mfma_weights(net, launch, wv.data(), k, wmul, 1);
         } else {
             const float wmul = weight_prescale(w, (size_t)oc * k * k * d.in_channels);
             launch.p.acc_mul = 1.0f / wmul;
@@ -441,15 +486,22 @@ class ConvLayer : public Layer {
         if (direct) launch_conv_direct(dp, s);
         else if (launch_conv_mfma(launch.var, launch.p, launch.lds, s) != 0)
             fail(FYN_ERR_DEVICE, "layer %s: convolution launch failed", d.name);
+        if (wide) launch_shift_reduce(sr, s);
     }
-    std::string info() const override { return direct ? (clamp ? "conv_direct(edge-clamp)" : "conv_direct") : mfma_info(launch); }
+    std::string info() const override {
+        if (direct) return clamp ? "conv_direct(edge-clamp)" : "conv_direct";
+        return wide ? "wide-kernel(kx folded into cout)+shift_reduce " + mfma_info(launch) : mfma_info(launch);
+    }
 
     int k, dil, stride;
-    bool clamp = false, direct = false, have_weights = false;
+    bool clamp = false, direct = false, wide = false, have_weights = false;
     int padded = 0;
     std::vector<float> block;
     MfmaLaunch launch;
     ConvDirectParams dp{};
+    ShiftReduceParams sr{};
+    TView qv{};
+    float *q_scale_dev = nullptr, *q_bias_dev = nullptr;
     float *scale_dev = nullptr, *bias_dev = nullptr, *wdirect_dev = nullptr;
 };
 

@@ -443,6 +443,64 @@ void launch_conv_direct(const ConvDirectParams& p, hipStream_t s) {
 }
 
 // ---------------------------------------------------------------------------------------------
+// shift-reduce stage of the wide-kernel / few-output-channel convolution (see ShiftReduceParams):
+// one thread per output pixel, the K neighbouring q pixels it reads are shared with its neighbours
+// through L1/L2, so HBM sees q once.
+// ---------------------------------------------------------------------------------------------
+// A block takes 256 consecutive output pixels of one row: the 256+K-1 q pixels they need are one
+// contiguous run in HBM, fetched once with 16-byte loads into LDS (row pitch cp+1 floats, so that the
+// per-thread strided reads below fall into distinct banks), then every thread sums its K*cout values.
+template <typename T>
+__global__ __launch_bounds__(256) void shift_reduce_kernel(const ShiftReduceParams p) {
+    extern __shared__ float sq[];
+    const int tiles_x = (p.out.w + 255) / 256;
+    const int y = blockIdx.x / tiles_x;
+    const int x0 = (blockIdx.x - y * tiles_x) * 256;
+    const int npx = min(256, p.out.w - x0) + p.k - 1;   // q pixels needed
+    const int cp = p.q.cp, pitch = cp + 1;
+    const T* q = reinterpret_cast<const T*>(p.q.ptr) + tv_off(p.q, y, x0);
+    const int nvec = npx * (cp >> 2);
+    for (int i = threadIdx.x; i < nvec; i += 256) {
+        const float4 v = ld4<T>(q + (size_t)i * 4);
+        const int px = i / (cp >> 2), c = (i - px * (cp >> 2)) * 4;
+        float* d = sq + px * pitch + c;
+        d[0] = v.x; d[1] = v.y; d[2] = v.z; d[3] = v.w;
+    }
+    __syncthreads();
+    const int x = x0 + threadIdx.x;
+    if (x >= p.out.w) return;
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int kx = 0; kx < p.k; kx++) {
+        const float* qp = sq + (threadIdx.x + kx) * pitch + kx;
+#pragma unroll
+        for (int o = 0; o < 4; o++)
+            if (o < p.cout) acc[o] += qp[o * p.k];
+    }
+    float o4[4];
+#pragma unroll
+    for (int o = 0; o < 4; o++) o4[o] = (o < p.cout) ? (acc[o] * p.acc_mul) * p.scale[o] + p.bias[o] : 0.f;
+    if (p.res.ptr) {
+        float4 r = ld4<T>(reinterpret_cast<const T*>(p.res.ptr) + tv_off(p.res, y, x));
+        float rv[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+        for (int o = 0; o < 4; o++) {
+            if (o >= p.cout) continue;
+            float v = rv[o];
+            if (p.res_relu) v = fmaxf(v, 0.f);
+            if (p.res_scale) v *= p.scale[o];
+            o4[o] += v;
+        }
+    }
+    st4<T>(reinterpret_cast<T*>(p.out.ptr) + tv_off(p.out, y, x), make_float4(o4[0], o4[1], o4[2], o4[3]));
+}
+void launch_shift_reduce(const ShiftReduceParams& p, hipStream_t s) {
+    const int tiles_x = (p.out.w + 255) / 256;
+    const size_t lds = (size_t)(256 + p.k - 1) * (p.q.cp + 1) * sizeof(float);
+    if (p.out.f16) hipLaunchKernelGGL((shift_reduce_kernel<_Float16>), dim3(tiles_x * p.out.h), dim3(256), lds, s, p);
+    else hipLaunchKernelGGL((shift_reduce_kernel<float>), dim3(tiles_x * p.out.h), dim3(256), lds, s, p);
+}
+
+// ---------------------------------------------------------------------------------------------
 // layout converters (UploadLayer / DownloadLayer / GPULayerBase::copyResult formats)
 // ---------------------------------------------------------------------------------------------
 template <typename T>
