@@ -25,6 +25,8 @@ from fyusenet_amd import networks  # noqa: E402
 
 PEAK_MFMA_F16_TFLOPS = 2500.0   # MI355X dense fp16/bf16 matrix peak
 PEAK_HBM_GBS = 8000.0           # MI355X HBM3E
+# (layer type, kernel, cin, cout, h, w) -> measured HBM bytes per launch (fetch + write), fp32 storage
+MEASURED_TRAFFIC = {(6, 3, 128, 128, 156, 128): 18.47e6 + 10.06e6}
 
 
 def log(*a):
@@ -42,6 +44,8 @@ def make_net(workload):
         return networks.MobileNetV2(fa.STORAGE_F16), "MobileNetV2 224x224 imgs/s", "imgs/s", "fp16 storage"
     if workload == "conv1":
         return networks.SingleConvNet(fa.STORAGE_F32), "conv3x3 64->64 256x256 us/layer", "us", "fp32 storage"
+    if workload == "resconv":  # the style net's dominant layer on its own (for counter runs)
+        return networks.SingleConvNet(fa.STORAGE_F32, channels=128, width=128, height=156), "conv3x3 128->128 128x156 us/layer", "us", "fp32 storage"
     if workload == "copy":
         return CopyNet(fa.STORAGE_F32), "copy 64x1024x1024 fp32 GB/s", "GB/s", "fp32"
     raise SystemExit("unknown workload %s" % workload)
@@ -108,7 +112,7 @@ def dominant_conv_roofline(net, storage_bytes):
             continue
         iters = 20
         lyr.timeKernel(3)
-        ms = lyr.timeKernel(iters)
+        ms = lyr.timeKernel(iters)            # launches back to back in one hipGraph (dispatch gaps included)
         b = lyr.builder
         key = (t, getattr(b, "kernel_", 0), b.inputChannels_, b.outputChannels_, b.height_, b.width_, tuple(b.downsample_),
                bool(int(b.getFlags()) & 1))
@@ -128,12 +132,17 @@ def dominant_conv_roofline(net, storage_bytes):
         if t_mfma >= t_hbm:
             ach = flops / (avg_ms * 1e-3) / 1e12
             rec.update({"bound": "mfma", "achieved": ach, "peak": PEAK_MFMA_F16_TFLOPS, "unit": "TFLOP/s", "frac": ach / PEAK_MFMA_F16_TFLOPS})
+            if storage_bytes == 4:
+                # fp32 storage: every algorithmic FLOP is issued as three fp16 MFMA FLOPs (hi*hi, lo*hi, hi*lo)
+                rec.update({"mfma_passes": 3, "mfma_issue_frac": 3 * ach / PEAK_MFMA_F16_TFLOPS})
         else:
             ach = nbytes / (avg_ms * 1e-3) / 1e9
             rec.update({"bound": "hbm", "achieved": ach, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": ach / PEAK_HBM_GBS})
         rec["algorithmic_flops_per_launch"] = flops
         rec["algorithmic_bytes_per_launch"] = nbytes
-    rec["traffic"] = None
+    # HBM bytes per launch from rocprofv3 FETCH_SIZE / WRITE_SIZE, scaled by the copy-kernel factors
+    # (profiles/conv_mfma_stylenet_512x624_fp32.md); only known for the profiled workload's dominant kernel
+    rec["traffic"] = MEASURED_TRAFFIC.get((key[0], key[1], key[2], key[3], key[4], key[5]))
     per_layer = sorted(((v["ms"], v["n"], v["layer"].name) for v in groups.values()), reverse=True)
     return rec, per_layer
 

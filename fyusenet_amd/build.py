@@ -6,8 +6,10 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libfynhip.so")
-SOURCES = ["conv_mfma.hip", "layers_direct.hip", "engine.cpp", "layers.cpp", "api.cpp"]
+CONV_PARTS = 8  # conv_mfma.hip is compiled this many times, each time with a slice of the tile table
+SOURCES = ["layers_direct.hip", "engine.cpp", "layers.cpp", "api.cpp"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+EXTRA = os.environ.get("FYNHIP_EXTRA_FLAGS", "").split()  # e.g. -D switches of experimental builds
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-result",
     # packed fp32 VALU forms are kept out of the generated code
@@ -15,22 +17,25 @@ FLAGS = [
 ]
 
 
-def build(verbose=True, jobs=5):
+def build(verbose=True, jobs=8):
     objdir = os.path.join(HERE, "_obj")
     os.makedirs(objdir, exist_ok=True)
     procs = []
     objs = []
-    for src in SOURCES:
-        obj = os.path.join(objdir, src + ".o")
+    units = [("conv_mfma.hip", "conv_mfma.part%d.o" % i, ["-DFYN_CONV_PARTS=%d" % CONV_PARTS, "-DFYN_CONV_PART=%d" % i])
+             for i in range(CONV_PARTS)]
+    units += [(src, src + ".o", []) for src in SOURCES]
+    for src, objname, defs in units:
+        obj = os.path.join(objdir, objname)
         objs.append(obj)
-        cmd = [HIPCC] + FLAGS + ["-x", "hip", "-c", os.path.join(CSRC, src), "-o", obj]
+        cmd = [HIPCC] + FLAGS + EXTRA + defs + ["-x", "hip", "-c", os.path.join(CSRC, src), "-o", obj]
         if verbose:
             print(" ".join(cmd), flush=True)
-        procs.append((src, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
+        procs.append((objname, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
         if len(procs) >= jobs:
             _drain(procs)
     _drain(procs)
-    cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs
+    cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-Wl,--no-undefined", "-o", LIB] + objs
     if verbose:
         print(" ".join(cmd), flush=True)
     subprocess.check_call(cmd)

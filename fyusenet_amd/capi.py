@@ -10,7 +10,7 @@ import os
 import numpy as np
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(HERE, "libfynhip.so")
+LIB_PATH = os.environ.get("FYNHIP_LIBRARY") or os.path.join(HERE, "libfynhip.so")  # override: alternative builds
 
 FYN_MAX_CONCAT_INPUTS = 8
 FYN_NAME_LEN = 64

@@ -23,6 +23,11 @@
 
 #include "kernels.h"
 
+// prefetch distance (k16 steps) of the weight fragments, by cout fragments per wave
+#ifndef FYN_CONV_PD
+#define FYN_CONV_PD(FM) 2
+#endif
+
 namespace fynhip {
 
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
@@ -200,7 +205,7 @@ __global__ __launch_bounds__(256) void conv_mfma_kernel(const ConvMfmaParams p) 
         // slack behind each plane is read by the last (zero-weight) k elements of a row run
         if (tid < 16 * NPL) {
             int pl = tid >> 4;
-            reinterpret_cast<uint32_t*>(lds + pl * p.plane + npix * p.pitch)[tid & 15] = 0u;
+            reinterpret_cast<uint32_t*>(lds + pl * p.plane + p.halo_h * p.row_pitch)[tid & 15] = 0u;
         }
     }
 
@@ -210,7 +215,7 @@ __global__ __launch_bounds__(256) void conv_mfma_kernel(const ConvMfmaParams p) 
     for (int fn = 0; fn < FN; fn++) {
         const int m = (wn * FN + fn) * 32 + (lane & 31);
         const int ty = m >> twl, tx = m & (TW - 1);
-        boff[fn] = ((ty * p.in_stride) * p.halo_w + tx * p.in_stride) * p.pitch + (lane >> 5) * 16;
+        boff[fn] = (ty * p.in_stride) * p.row_pitch + (tx * p.in_stride) * p.pitch + (lane >> 5) * 16;
     }
 
     // A (weight) fragments: [(chunk*nsteps + step)][mfrag][plane][lane] x 8 halves
@@ -227,11 +232,33 @@ __global__ __launch_bounds__(256) void conv_mfma_kernel(const ConvMfmaParams p) 
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
 
-    half8_t a_cur[FM][NPL];
+    // A fragments are prefetched PD steps ahead into a register ring that is indexed statically (the
+    // step loop is unrolled PD-fold; the host pads nsteps to a multiple of PD with zero-weight steps):
+    // with only two or three waves per SIMD the L2 round trip of a weight fragment is several times
+    // longer than one step's MFMAs.
+    constexpr int PD = FYN_CONV_PD(FM);
+    half8_t a_q[PD][FM][NPL];
 #pragma unroll
-    for (int fm = 0; fm < FM; fm++)
+    for (int d = 0; d < PD; d++) {
+        const half8_t* w_ = wfrag + (size_t)(d < total_steps ? d : total_steps - 1) * wstep;
 #pragma unroll
-        for (int pl = 0; pl < NPL; pl++) a_cur[fm][pl] = wfrag[(fm * NPL + pl) * 64];
+        for (int fm = 0; fm < FM; fm++)
+#pragma unroll
+            for (int pl = 0; pl < NPL; pl++) a_q[d][fm][pl] = w_[(fm * NPL + pl) * 64];
+    }
+    // LDS byte offsets of the (up to 256) k16 steps, kept in four VGPRs (entry t in lane t%64 of register
+    // t/64) and read with v_readlane: no scalar memory traffic inside the step loop
+    const int tab0 = (lane < p.nsteps) ? p.aoff[lane] : 0;
+    const int tab1 = (lane + 64 < p.nsteps) ? p.aoff[lane + 64] : 0;
+    const int tab2 = (lane + 128 < p.nsteps) ? p.aoff[lane + 128] : 0;
+    const int tab3 = (lane + 192 < p.nsteps) ? p.aoff[lane + 192] : 0;
+    auto step_off = [&](int t_) -> int {
+        const int r0 = __builtin_amdgcn_readlane(tab0, t_ & 63);
+        const int r1 = __builtin_amdgcn_readlane(tab1, t_ & 63);
+        const int r2 = __builtin_amdgcn_readlane(tab2, t_ & 63);
+        const int r3 = __builtin_amdgcn_readlane(tab3, t_ & 63);
+        return t_ < 128 ? (t_ < 64 ? r0 : r1) : (t_ < 192 ? r2 : r3);
+    };
 
     // ---- staging machinery: items (pixel, 8-channel group) of the halo tile; the first NB items of a
     //      thread are described once (their addresses only shift by the chunk's channel offset) and
@@ -250,26 +277,32 @@ __global__ __launch_bounds__(256) void conv_mfma_kernel(const ConvMfmaParams p) 
             const int py = (int)(((float)pix + 0.5f) * inv_hw);
             const int px = pix - py * p.halo_w;
             const int gy = gy0 + py, gx = gx0 + px;
-            l_off[i] = pix * p.pitch + g * 16;
+            l_off[i] = py * p.row_pitch + px * p.pitch + g * 16;
             c_off[i] = g * CPI;
             if ((unsigned)gy < (unsigned)p.in_hp && (unsigned)gx < (unsigned)p.in_wp) g_off[i] = (gy * p.in_wp + gx) * p.in_cp;
         }
     }
     RawItem<TIn, CPI> raw[NB];
-    auto fetch_first = [&](int chunk) {
+    // The loads are unconditional (items outside the tensor read its first element and are zeroed when
+    // stored), so that the number of loads in flight is known at compile time.
+    auto fetch_first = [&](int chunk_) {
 #pragma unroll
         for (int i = 0; i < NB; i++) {
-            const int c0 = chunk * KC + c_off[i];
-            raw[i].zero();
-            if (g_off[i] >= 0 && c0 < p.in_cp) raw[i].load(in + g_off[i] + c0);
+            const int c0 = chunk_ * KC + c_off[i];
+            const bool ok = g_off[i] >= 0 && c0 < p.in_cp;
+            raw[i].load(in + (ok ? g_off[i] + c0 : 0));
         }
     };
-    auto store_first = [&](unsigned char* buf) {
+    auto store_first = [&](int chunk_, unsigned char* buf) {
 #pragma unroll
         for (int i = 0; i < NB; i++) {
             if (l_off[i] >= 0) {
+                const int c0 = chunk_ * KC + c_off[i];
+                const bool ok = g_off[i] >= 0 && c0 < p.in_cp;
                 float v[8];
                 raw[i].get(v);
+#pragma unroll
+                for (int e = 0; e < CPI; e++) v[e] = ok ? v[e] : 0.f;
                 stage_store<SPLIT, CPI>(buf + l_off[i], p.plane, v, p.act);
             }
         }
@@ -291,7 +324,7 @@ __global__ __launch_bounds__(256) void conv_mfma_kernel(const ConvMfmaParams p) 
                     const int px = pix - py * p.halo_w;
                     const int gy = gy0 + py, gx = gx0 + px;
                     const int c0 = chunk * KC + g * CPI;
-                    lo2[i] = pix * p.pitch + g * 16;
+                    lo2[i] = py * p.row_pitch + px * p.pitch + g * 16;
                     if ((unsigned)gy < (unsigned)p.in_hp && (unsigned)gx < (unsigned)p.in_wp && c0 < p.in_cp)
                         r2[i].load(in + (gy * p.in_wp + gx) * p.in_cp + c0);
                 }
@@ -309,81 +342,76 @@ __global__ __launch_bounds__(256) void conv_mfma_kernel(const ConvMfmaParams p) 
 
     // prologue: chunk 0 into buffer 0
     fetch_first(0);
-    store_first(lds);
+    store_first(0, lds);
     stage_rest(0, lds);
     __syncthreads();
 
-    // ---- main loop over all k16 steps (chunk-major).  B fragments of step t+1 are read from LDS while
-    //      the MFMAs of step t run; at a chunk boundary the next chunk's tile (fetched from HBM during this
-    //      chunk's MFMAs) is converted into the other LDS buffer, one barrier per chunk. ----
-    int chunk = 0, t = 0;
-    unsigned char* cur = lds;
-    if (p.cin_chunks > 1) fetch_first(1);
+    // ---- main loop: channel chunks, each nsteps k16 steps in groups of PD.  B fragments of step t+1 are
+    //      read from LDS while the MFMAs of step t run; the next chunk's tile is fetched from HBM/L2 at the
+    //      start of a chunk and converted into the other LDS buffer at its end, one barrier per chunk. ----
+    int gs = 0;  // global step = chunk * nsteps + t
     half8_t b_cur[FN][NPL];
-    {
-        const int ao = p.aoff[0];
+    unsigned char* cur = lds;
+    // PD steps starting at step t0 of the current chunk; `more`: another group follows in this chunk
+    auto run_group = [&](int t0, bool more) {
 #pragma unroll
-        for (int fn = 0; fn < FN; fn++)
+        for (int d = 0; d < PD; d++) {
+            const bool has_next = (d + 1 < PD) || more;
+            half8_t b_nxt[FN][NPL];
+            if (has_next) {
+                const int ao = step_off(t0 + d + 1);
 #pragma unroll
-            for (int pl = 0; pl < NPL; pl++) b_cur[fn][pl] = load_b_frag<KC>(cur + pl * p.plane + boff[fn] + ao);
-    }
-    for (int gs = 0; gs < total_steps; gs++) {
-        const bool last_in_chunk = (t + 1 == p.nsteps);
-        half8_t a_nxt[FM][NPL];
-        half8_t b_nxt[FN][NPL];
-        {
-            // fragments of step gs+1: A from L2, B from LDS, both in flight during this step's MFMAs
-            const half8_t* wn_ = wfrag + (size_t)(gs + 1 < total_steps ? gs + 1 : gs) * wstep;
+                for (int fn = 0; fn < FN; fn++)
+#pragma unroll
+                    for (int pl = 0; pl < NPL; pl++) b_nxt[fn][pl] = load_b_frag<KC>(cur + pl * p.plane + boff[fn] + ao);
+            }
 #pragma unroll
             for (int fm = 0; fm < FM; fm++)
 #pragma unroll
-                for (int pl = 0; pl < NPL; pl++) a_nxt[fm][pl] = wn_[(fm * NPL + pl) * 64];
-        }
-        if (!last_in_chunk) {
-            const int ao = p.aoff[t + 1];
-#pragma unroll
-            for (int fn = 0; fn < FN; fn++)
-#pragma unroll
-                for (int pl = 0; pl < NPL; pl++) b_nxt[fn][pl] = load_b_frag<KC>(cur + pl * p.plane + boff[fn] + ao);
-        } else {
-#pragma unroll
-            for (int fn = 0; fn < FN; fn++)
-#pragma unroll
-                for (int pl = 0; pl < NPL; pl++) b_nxt[fn][pl] = b_cur[fn][pl];
-        }
-#pragma unroll
-        for (int fm = 0; fm < FM; fm++)
-#pragma unroll
-            for (int fn = 0; fn < FN; fn++) {
-                acc[fm][fn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_cur[fm][0], b_cur[fn][0], acc[fm][fn], 0, 0, 0);
-                if (SPLIT) {
-                    acc[fm][fn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_cur[fm][1], b_cur[fn][0], acc[fm][fn], 0, 0, 0);
-                    acc[fm][fn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_cur[fm][0], b_cur[fn][1], acc[fm][fn], 0, 0, 0);
+                for (int fn = 0; fn < FN; fn++) {
+                    acc[fm][fn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_q[d][fm][0], b_cur[fn][0], acc[fm][fn], 0, 0, 0);
+                    if (SPLIT) {
+                        acc[fm][fn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_q[d][fm][1], b_cur[fn][0], acc[fm][fn], 0, 0, 0);
+                        acc[fm][fn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_q[d][fm][0], b_cur[fn][1], acc[fm][fn], 0, 0, 0);
+                    }
                 }
+            {
+                // refill this ring slot with the fragments of step gs+PD (past the end: the last step again)
+                const int nx = gs + PD < total_steps ? gs + PD : total_steps - 1;
+                const half8_t* w_ = wfrag + (size_t)nx * wstep;
+#pragma unroll
+                for (int fm = 0; fm < FM; fm++)
+#pragma unroll
+                    for (int pl = 0; pl < NPL; pl++) a_q[d][fm][pl] = w_[(fm * NPL + pl) * 64];
             }
+            if (has_next) {
 #pragma unroll
-        for (int fm = 0; fm < FM; fm++)
+                for (int fn = 0; fn < FN; fn++)
 #pragma unroll
-            for (int pl = 0; pl < NPL; pl++) a_cur[fm][pl] = a_nxt[fm][pl];
-#pragma unroll
-        for (int fn = 0; fn < FN; fn++)
-#pragma unroll
-            for (int pl = 0; pl < NPL; pl++) b_cur[fn][pl] = b_nxt[fn][pl];
-        t++;
-        if (last_in_chunk && chunk + 1 < p.cin_chunks) {
-            unsigned char* nxt = lds + ((chunk + 1) & 1) * bufsz;
-            store_first(nxt);
-            stage_rest(chunk + 1, nxt);
-            __syncthreads();  // everyone is done reading `cur` and writing `nxt`
-            chunk++;
-            t = 0;
-            cur = nxt;
-            if (chunk + 1 < p.cin_chunks) fetch_first(chunk + 1);
-            const int ao = p.aoff[0];
+                    for (int pl = 0; pl < NPL; pl++) b_cur[fn][pl] = b_nxt[fn][pl];
+            }
+            gs++;
+        }
+    };
+    for (int chunk = 0; chunk < p.cin_chunks; chunk++) {
+        const bool more_chunks = chunk + 1 < p.cin_chunks;
+        fetch_first(more_chunks ? chunk + 1 : chunk);  // (unused after the last chunk; keeps the load count static)
+        {
+            const int ao = step_off(0);
 #pragma unroll
             for (int fn = 0; fn < FN; fn++)
 #pragma unroll
                 for (int pl = 0; pl < NPL; pl++) b_cur[fn][pl] = load_b_frag<KC>(cur + pl * p.plane + boff[fn] + ao);
+        }
+        // first group peeled: the tile loads issued above are younger than the ring's loads only here
+        run_group(0, p.nsteps > PD);
+        for (int t0 = PD; t0 < p.nsteps; t0 += PD) run_group(t0, t0 + PD < p.nsteps);
+        if (more_chunks) {
+            unsigned char* nxt = lds + ((chunk + 1) & 1) * bufsz;
+            store_first(chunk + 1, nxt);
+            stage_rest(chunk + 1, nxt);
+            __syncthreads();  // everyone is done reading `cur` and writing `nxt`
+            cur = nxt;
         }
     }
 
@@ -456,9 +484,35 @@ __global__ __launch_bounds__(256) void conv_mfma_kernel(const ConvMfmaParams p) 
 }
 
 // ---------------------------------------------------------------------------------------------
-// variant table
+// variant table.  This file is compiled FYN_CONV_PARTS times with -DFYN_CONV_PART=0..N-1 (in parallel);
+// every part instantiates the kernels of the tiles whose table index is congruent to it, and part 0
+// also holds the dispatcher.
 // ---------------------------------------------------------------------------------------------
 typedef void (*conv_kernel_fn)(const ConvMfmaParams);
+
+#ifndef FYN_CONV_PARTS
+#define FYN_CONV_PARTS 1
+#endif
+#ifndef FYN_CONV_PART
+#define FYN_CONV_PART 0
+#endif
+
+// (index, fm, fn, wm, wn): cout tile = wm*fm*32, position tile = wn*fn*32
+#define FYN_CONV_TILES(X) \
+    X(0, 2, 2, 2, 2)      \
+    X(1, 2, 2, 1, 4)      \
+    X(2, 2, 1, 2, 2)      \
+    X(3, 2, 1, 1, 4)      \
+    X(4, 1, 2, 1, 4)      \
+    X(5, 1, 1, 1, 4)      \
+    X(6, 1, 1, 4, 1)      \
+    X(7, 1, 1, 2, 2)      \
+    X(8, 1, 2, 4, 1)      \
+    X(9, 1, 3, 4, 1)      \
+    X(10, 1, 4, 4, 1)     \
+    X(11, 1, 2, 2, 2)     \
+    X(12, 1, 4, 2, 2)     \
+    X(13, 1, 3, 2, 2)
 
 template <typename TIn, typename TOut, bool SPLIT, int FM, int FN, int WM, int WN>
 static conv_kernel_fn pick_kc(int kc) {
@@ -470,38 +524,94 @@ static conv_kernel_fn pick_kc(int kc) {
     }
 }
 
-template <typename TIn, typename TOut, bool SPLIT>
-static conv_kernel_fn pick_tile(const ConvVariant& v) {
-#define FYN_TILE(fm_, fn_, wm_, wn_) \
-    if (v.fm == fm_ && v.fn == fn_ && v.wm == wm_ && v.wn == wn_) return pick_kc<TIn, TOut, SPLIT, fm_, fn_, wm_, wn_>(v.kc);
-    FYN_TILE(2, 2, 2, 2)  // 128 cout x 128 positions
-    FYN_TILE(2, 2, 1, 4)  //  64 cout x 256 positions
-    FYN_TILE(2, 1, 2, 2)  // 128 cout x  64 positions
-    FYN_TILE(2, 1, 1, 4)  //  64 cout x 128 positions
-    FYN_TILE(1, 2, 1, 4)  //  32 cout x 256 positions
-    FYN_TILE(1, 1, 1, 4)  //  32 cout x 128 positions
-    FYN_TILE(1, 1, 4, 1)  // 128 cout x  32 positions
-    FYN_TILE(1, 1, 2, 2)  //  64 cout x  64 positions
+#define FYN_CAT2(a, b) a##b
+#define FYN_CAT(a, b) FYN_CAT2(a, b)
+
+// lookup among the tiles of one part (a template so that the tiles of other parts are not instantiated)
+template <int PART>
+static conv_kernel_fn lookup_part(const ConvVariant& v) {
+    const bool f16 = v.in_f16 && v.out_f16 && !v.split;
+    const bool f32 = !v.in_f16 && !v.out_f16 && v.split;  // split arithmetic is the fp32-storage path
+    if (!f16 && !f32) return nullptr;
+#define FYN_TILE(idx_, fm_, fn_, wm_, wn_)                                                \
+    if constexpr ((idx_) % FYN_CONV_PARTS == PART) {                                       \
+        if (v.fm == fm_ && v.fn == fn_ && v.wm == wm_ && v.wn == wn_)                      \
+            return f32 ? pick_kc<float, float, true, fm_, fn_, wm_, wn_>(v.kc)             \
+                       : pick_kc<_Float16, _Float16, false, fm_, fn_, wm_, wn_>(v.kc);     \
+    }
+    FYN_CONV_TILES(FYN_TILE)
 #undef FYN_TILE
     return nullptr;
 }
 
+conv_kernel_fn FYN_CAT(conv_mfma_lookup_part, FYN_CONV_PART)(const ConvVariant& v) { return lookup_part<FYN_CONV_PART>(v); }
+
+#if FYN_CONV_PART == 0
+#define FYN_DECL(i_) conv_kernel_fn conv_mfma_lookup_part##i_(const ConvVariant& v);
+#if FYN_CONV_PARTS > 1
+FYN_DECL(1)
+#endif
+#if FYN_CONV_PARTS > 2
+FYN_DECL(2)
+#endif
+#if FYN_CONV_PARTS > 3
+FYN_DECL(3)
+#endif
+#if FYN_CONV_PARTS > 4
+FYN_DECL(4)
+FYN_DECL(5)
+#endif
+#if FYN_CONV_PARTS > 6
+FYN_DECL(6)
+FYN_DECL(7)
+#endif
+#undef FYN_DECL
+
 static conv_kernel_fn pick_kernel(const ConvVariant& v) {
-    if (v.split) {
-        if (v.in_f16 || v.out_f16) return nullptr;  // split arithmetic is the fp32-storage path
-        return pick_tile<float, float, true>(v);
-    }
-    if (v.in_f16 && v.out_f16) return pick_tile<_Float16, _Float16, false>(v);
-    if (!v.in_f16 && v.out_f16) return pick_tile<float, _Float16, false>(v);
-    if (!v.in_f16 && !v.out_f16) return pick_tile<float, float, false>(v);
-    return nullptr;
+    conv_kernel_fn fn = conv_mfma_lookup_part0(v);
+#if FYN_CONV_PARTS > 1
+    if (!fn) fn = conv_mfma_lookup_part1(v);
+#endif
+#if FYN_CONV_PARTS > 2
+    if (!fn) fn = conv_mfma_lookup_part2(v);
+#endif
+#if FYN_CONV_PARTS > 3
+    if (!fn) fn = conv_mfma_lookup_part3(v);
+#endif
+#if FYN_CONV_PARTS > 4
+    if (!fn) fn = conv_mfma_lookup_part4(v);
+    if (!fn) fn = conv_mfma_lookup_part5(v);
+#endif
+#if FYN_CONV_PARTS > 6
+    if (!fn) fn = conv_mfma_lookup_part6(v);
+    if (!fn) fn = conv_mfma_lookup_part7(v);
+#endif
+    return fn;
 }
 
 bool conv_mfma_variant_exists(const ConvVariant& v) { return pick_kernel(v) != nullptr; }
 
+int conv_mfma_step_multiple(const ConvVariant& v) { return FYN_CONV_PD(v.fm); }
+
+int conv_mfma_tile_count() {
+    int n = 0;
+#define FYN_TILE(idx_, fm_, fn_, wm_, wn_) n++;
+    FYN_CONV_TILES(FYN_TILE)
+#undef FYN_TILE
+    return n;
+}
+
+void conv_mfma_tile(int index, int* fm, int* fn, int* wm, int* wn) {
+#define FYN_TILE(idx_, fm_, fn_, wm_, wn_) \
+    if (index == idx_) { *fm = fm_; *fn = fn_; *wm = wm_; *wn = wn_; }
+    FYN_CONV_TILES(FYN_TILE)
+#undef FYN_TILE
+}
+
 int launch_conv_mfma(const ConvVariant& v, const ConvMfmaParams& p, size_t lds_bytes, hipStream_t s) {
     conv_kernel_fn fn = pick_kernel(v);
     if (!fn) return -1;
+    if (p.nsteps < 1 || p.nsteps > 256 || p.nsteps % FYN_CONV_PD(v.fm) != 0) return -5;
     if (lds_bytes > 48 * 1024) {
         // raise the kernel's dynamic LDS limit once per kernel and size
         static std::mutex mu;
@@ -519,5 +629,6 @@ int launch_conv_mfma(const ConvVariant& v, const ConvMfmaParams& p, size_t lds_b
     hipLaunchKernelGGL(fn, dim3(blocks), dim3(256), lds_bytes, s, p);
     return hipGetLastError() == hipSuccess ? 0 : -3;
 }
+#endif  // FYN_CONV_PART == 0
 
 }  // namespace fynhip

@@ -456,17 +456,34 @@ void Net::time_layer(int layer_no, int iters, float* ms) {
     if (!is_setup) fail(FYN_ERR_STATE, "time_layer() before setup()");
     FYN_HIP(hipSetDevice(device));
     Layer* l = layer(layer_no);
+    // The launches are captured into one hipGraph so that host-side dispatch gaps do not enter the
+    // measurement; the events bracket the graph on the network's stream.
+    hipGraph_t g = nullptr;
+    hipGraphExec_t ge = nullptr;
+    FYN_HIP(hipStreamBeginCapture(stream, hipStreamCaptureModeThreadLocal));
+    try {
+        for (int i = 0; i < iters; i++) l->forward(stream);
+    } catch (...) {
+        (void)hipStreamEndCapture(stream, &g);
+        if (g) (void)hipGraphDestroy(g);
+        throw;
+    }
+    FYN_HIP(hipStreamEndCapture(stream, &g));
+    FYN_HIP(hipGraphInstantiate(&ge, g, nullptr, nullptr, 0));
     hipEvent_t a, b;
     FYN_HIP(hipEventCreate(&a));
     FYN_HIP(hipEventCreate(&b));
+    FYN_HIP(hipGraphLaunch(ge, stream));  // warm-up
     FYN_HIP(hipEventRecord(a, stream));
-    for (int i = 0; i < iters; i++) l->forward(stream);
+    FYN_HIP(hipGraphLaunch(ge, stream));
     FYN_HIP(hipEventRecord(b, stream));
     FYN_HIP(hipEventSynchronize(b));
     FYN_HIP(hipGetLastError());
     FYN_HIP(hipEventElapsedTime(ms, a, b));
     (void)hipEventDestroy(a);
     (void)hipEventDestroy(b);
+    (void)hipGraphExecDestroy(ge);
+    (void)hipGraphDestroy(g);
 }
 
 }  // namespace fynhip

@@ -61,6 +61,7 @@ struct ConvMfmaParams {
     int tiles_x, tiles_y;
     int halo_w, halo_h;  // staged input tile size (pixels)
     int pitch;           // LDS bytes per staged pixel (one plane)
+    int row_pitch;       // LDS bytes per staged pixel row (>= halo_w * pitch; padded against bank conflicts)
     int plane;           // LDS bytes of one plane (hi); lo plane follows when split
     int cin_chunks, nsteps;
     int mfrags;          // cout fragments (32 each) in wpack
@@ -81,6 +82,11 @@ struct ConvVariant {
 // Returns 0 when the variant exists and was launched.
 int launch_conv_mfma(const ConvVariant& v, const ConvMfmaParams& p, size_t lds_bytes, hipStream_t s);
 bool conv_mfma_variant_exists(const ConvVariant& v);
+// The kernel runs its k16 steps in groups of this size: nsteps must be a multiple (pad with zero-weight steps).
+int conv_mfma_step_multiple(const ConvVariant& v);
+// The compiled tile configurations (fragments per wave fm x fn, waves per block wm x wn).
+int conv_mfma_tile_count();
+void conv_mfma_tile(int index, int* fm, int* fn, int* wm, int* wn);
 
 // ---------------------------------------------------------------------------------------------
 // Direct (non-MFMA) layer kernels (layers_direct.hip)

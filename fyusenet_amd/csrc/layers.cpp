@@ -3,6 +3,7 @@
 // weight-block parsing / repacking (gpu/deep/deepconvlayerbase.cpp:293-395 and friends) and kernel
 // selection + launch.
 #include <algorithm>
+#include <array>
 #include <cmath>
 #include <cstdlib>
 #include <cstring>
@@ -94,17 +95,16 @@ struct MfmaLaunch {
     std::vector<Step> steps;
     void* wpack_dev = nullptr;
     int* aoff_dev = nullptr;
-    size_t wpack_halves = 0;
+    size_t wpack_halves = 0;  // halves used by this launch's layout
+    size_t wpack_alloc = 0;   // halves allocated
     int cin = 0, cout = 0;
 };
 
 struct TileChoice {
     int fm, fn, wm, wn, twl, th;
     double score;
+    int rowpad;  // bytes added to each staged pixel row in LDS
 };
-
-static const int kTileTable[][4] = {{2, 2, 2, 2}, {2, 2, 1, 4}, {2, 1, 2, 2}, {2, 1, 1, 4},
-                                    {1, 2, 1, 4}, {1, 1, 1, 4}, {1, 1, 4, 1}, {1, 1, 2, 2}};
 
 // All tile configurations that fit, best heuristic score first.
 static std::vector<TileChoice> enumerate_tiles(int cout, const SubConv& sc, int pitch, int npl, int slack, int nbuf) {
@@ -112,8 +112,9 @@ static std::vector<TileChoice> enumerate_tiles(int cout, const SubConv& sc, int 
     const char* force = getenv("FYNHIP_CONV_TILE");  // "fm,fn,wm,wn" for experiments
     int ff[4] = {0, 0, 0, 0};
     if (force) sscanf(force, "%d,%d,%d,%d", &ff[0], &ff[1], &ff[2], &ff[3]);
-    for (const auto& t : kTileTable) {
-        const int fm = t[0], fn = t[1], wm = t[2], wn = t[3];
+    for (int ti = 0; ti < conv_mfma_tile_count(); ti++) {
+        int fm, fn, wm, wn;
+        conv_mfma_tile(ti, &fm, &fn, &wm, &wn);
         if (force && (fm != ff[0] || fn != ff[1] || wm != ff[2] || wn != ff[3])) continue;
         const int bm = wn * fn * 32;
         int tw = std::min(bm >= 128 ? 16 : 8, pow2ceil(sc.npos_x));
@@ -123,14 +124,15 @@ static std::vector<TileChoice> enumerate_tiles(int cout, const SubConv& sc, int 
         const int cpb = wm * fm * 32;
         const int cblocks = (cout + cpb - 1) / cpb;
         const int halo_w = (tw - 1) * sc.in_stride + sc.span_x, halo_h = (th - 1) * sc.in_stride + sc.span_y;
-        const size_t lds = (size_t)nbuf * npl * ((size_t)halo_h * halo_w * pitch + slack);
+        const int rowpad = 0;
+        const size_t lds = (size_t)nbuf * npl * ((size_t)halo_h * (halo_w * pitch + rowpad) + slack);
         if (lds > 150 * 1024) continue;
         const double util = ((double)cout * sc.npos_x * sc.npos_y) / ((double)cblocks * cpb * (double)tiles * bm);
         const double blocks = (double)tiles * cblocks;
         const double slots = 256.0 * (lds > 72 * 1024 ? 1 : 2);
         const double par = blocks >= slots ? blocks / (std::ceil(blocks / slots) * slots) : blocks / slots;
         const double bonus = (fm * fn == 4) ? 1.0 : (fm * fn == 2 ? 0.85 : 0.7);
-        all.push_back(TileChoice{fm, fn, wm, wn, ilog2(tw), th, util * par * bonus});
+        all.push_back(TileChoice{fm, fn, wm, wn, ilog2(tw), th, util * par * bonus, rowpad});
     }
     if (all.empty()) fail(FYN_ERR_UNSUPPORTED, "no MFMA tile configuration fits this convolution");
     std::sort(all.begin(), all.end(), [](const TileChoice& x, const TileChoice& y) { return x.score > y.score; });
@@ -179,7 +181,8 @@ static MfmaLaunch plan_mfma(Net* net, const SubConv& sc, const TView& in, const 
     p.halo_w = (tw - 1) * sc.in_stride + sc.span_x;
     p.halo_h = (tc.th - 1) * sc.in_stride + sc.span_y;
     p.pitch = pitch;
-    p.plane = p.halo_h * p.halo_w * pitch + slack;
+    p.row_pitch = p.halo_w * pitch + ((kc == 4) ? 0 : tc.rowpad);
+    p.plane = p.halo_h * p.row_pitch + slack;
     p.cin_chunks = (kc == 4) ? 1 : (in.cp + kc - 1) / kc;
     const int cpb = tc.wm * tc.fm * 32;
     p.cout_blocks = (cout + cpb - 1) / cpb;
@@ -206,7 +209,7 @@ static MfmaLaunch plan_mfma(Net* net, const SubConv& sc, const TView& in, const 
             const int nst = (len * 4 + 15) / 16;
             for (int s = 0; s < nst; s++) {
                 MfmaLaunch::Step st;
-                st.aoff = (taps[i].oy * p.halo_w + taps[i].ox) * pitch + s * 32;
+                st.aoff = taps[i].oy * p.row_pitch + taps[i].ox * pitch + s * 32;
                 for (int e = 0; e < 16; e++) {
                     const int r = s * 16 + e, q = r / 4;
                     if (q < len) {
@@ -223,24 +226,35 @@ static MfmaLaunch plan_mfma(Net* net, const SubConv& sc, const TView& in, const 
         for (const Tap& t : sc.taps)
             for (int sub = 0; sub < kc / 16; sub++) {
                 MfmaLaunch::Step st;
-                st.aoff = (t.oy * p.halo_w + t.ox) * pitch + sub * 32;
+                st.aoff = t.oy * p.row_pitch + t.ox * pitch + sub * 32;
                 for (int e = 0; e < 16; e++) {
                     st.ky[e] = t.ky; st.kx[e] = t.kx; st.ci[e] = sub * 16 + e;
                 }
                 L.steps.push_back(st);
             }
     }
+    // pad to the kernel's step group size with steps whose weights are all zero
+    while (L.steps.size() % conv_mfma_step_multiple(L.var) != 0) {
+        MfmaLaunch::Step st;
+        st.aoff = 0;
+        for (int e = 0; e < 16; e++) { st.ky[e] = st.kx[e] = 0; st.ci[e] = -1; }
+        L.steps.push_back(st);
+    }
+    if (L.steps.size() > 256) fail(FYN_ERR_UNSUPPORTED, "too many kernel taps for the MFMA convolution (%zu steps per chunk)", L.steps.size());
     p.nsteps = (int)L.steps.size();
     std::vector<int> aoff(L.steps.size());
     for (size_t i = 0; i < L.steps.size(); i++) aoff[i] = L.steps[i].aoff;
     L.aoff_dev = upload(net, aoff);
     p.aoff = L.aoff_dev;
     L.wpack_halves = (size_t)p.cin_chunks * p.nsteps * p.mfrags * npl * 64 * 8;
+    // the buffer is sized for any step padding (groups of up to 12), so that tile candidates can share it
+    L.wpack_alloc = (size_t)p.cin_chunks * ((p.nsteps + 11) / 12 * 12 + 12) * p.mfrags * npl * 64 * 8;
     if (share) {
-        if (share->wpack_halves != L.wpack_halves) fail(FYN_ERR_INVALID, "internal: weight layouts of tile candidates differ");
+        if (share->wpack_alloc < L.wpack_halves) fail(FYN_ERR_INVALID, "internal: weight layouts of tile candidates differ");
         L.wpack_dev = share->wpack_dev;
+        L.wpack_alloc = share->wpack_alloc;
     } else {
-        L.wpack_dev = net->dev_alloc(L.wpack_halves * 2, true);
+        L.wpack_dev = net->dev_alloc(L.wpack_alloc * 2, true);
     }
     p.wpack = L.wpack_dev;
     return L;
@@ -265,6 +279,43 @@ static float time_launch(Net* net, const MfmaLaunch& L, int iters) {
     return ms / iters;
 }
 
+// ---- optional on-disk memory of tuning results (text: "<key> fm fn wm wn" per line) ----
+static std::map<std::string, std::array<int, 4>>& tune_cache() {
+    static std::map<std::string, std::array<int, 4>> cache;
+    static bool loaded = false;
+    if (!loaded) {
+        loaded = true;
+        const char* path = getenv("FYNHIP_TUNE_CACHE");
+        FILE* f = path ? fopen(path, "r") : nullptr;
+        if (f) {
+            char k[160];
+            int a, b, c, d;
+            while (fscanf(f, "%159s %d %d %d %d", k, &a, &b, &c, &d) == 5) cache[k] = {a, b, c, d};
+            fclose(f);
+        }
+    }
+    return cache;
+}
+
+static const TileChoice* tune_cache_lookup(const char* key, const std::vector<TileChoice>& cands) {
+    if (!getenv("FYNHIP_TUNE_CACHE")) return nullptr;
+    auto it = tune_cache().find(key);
+    if (it == tune_cache().end()) return nullptr;
+    for (const TileChoice& c : cands)
+        if (c.fm == it->second[0] && c.fn == it->second[1] && c.wm == it->second[2] && c.wn == it->second[3]) return &c;
+    return nullptr;
+}
+
+static void tune_cache_store(const char* key, const ConvVariant& v) {
+    const char* path = getenv("FYNHIP_TUNE_CACHE");
+    if (!path) return;
+    tune_cache()[key] = {v.fm, v.fn, v.wm, v.wn};
+    FILE* f = fopen(path, "a");
+    if (!f) return;
+    fprintf(f, "%s %d %d %d %d\n", key, v.fm, v.fn, v.wm, v.wn);
+    fclose(f);
+}
+
 // Picks the tile configuration of one (sub-)convolution: by measurement on the layer's own tensors
 // (default; timing does not depend on the data), or by the heuristic score when FYNHIP_AUTOTUNE=0.
 static MfmaLaunch tune_mfma(Net* net, const SubConv& sc, const TView& in, const TView& out, const TView* res, int cin,
@@ -275,6 +326,15 @@ static MfmaLaunch tune_mfma(Net* net, const SubConv& sc, const TView& in, const 
     std::vector<TileChoice> cands = enumerate_tiles(cout, sc, pitch, npl, slack, chunks > 1 ? 2 : 1);
     const char* at = getenv("FYNHIP_AUTOTUNE");
     const bool tune = !(at && at[0] == '0') && cands.size() > 1;
+    // FYNHIP_TUNE_CACHE=<file>: measured choices are remembered per problem geometry, so that later
+    // processes (e.g. under a profiler, where timing is distorted) pick the same kernels
+    char key[160];
+    snprintf(key, sizeof(key), "%d%d:%dx%d:%dx%d:s%d:t%zu:%dx%d:o%d:r%d:cp%d", in.f16, out.f16, cin, cout, sc.npos_y, sc.npos_x,
+             sc.in_stride, sc.taps.size(), sc.span_y, sc.span_x, sc.out_step, res ? 1 : 0, in.cp);
+    if (tune) {
+        const TileChoice* hit = tune_cache_lookup(key, cands);
+        if (hit) return plan_mfma(net, sc, in, out, res, cin, cout, act, res_relu, res_scale, *hit, scale, bias);
+    }
     MfmaLaunch best = plan_mfma(net, sc, in, out, res, cin, cout, act, res_relu, res_scale, cands[0], scale, bias);
     if (!tune) return best;
     const bool verbose = getenv("FYNHIP_TUNE_VERBOSE") != nullptr;
@@ -289,6 +349,7 @@ static MfmaLaunch tune_mfma(Net* net, const SubConv& sc, const TView& in, const 
             best = L;
         }
     }
+    tune_cache_store(key, best.var);
     return best;
 }
 

@@ -106,15 +106,15 @@ class SingleConvNet(_StreamNet):
     (ConvLayerBuilder(3).shape(64,256,256,64).deep().inputPadding(1).prefixAct(RELU))."""
     config_id = 1
 
-    def __init__(self, storage=STORAGE_F32, size=256, channels=64, device=0):
+    def __init__(self, storage=STORAGE_F32, size=256, channels=64, device=0, width=None, height=None):
         super().__init__(storage, device)
-        self.size, self.ch = size, channels
+        self.width, self.height, self.ch = width or size, height or size, channels
 
     def define(self):
-        self.conv(1, "conv3x3", 3, self.ch, self.ch, self.size, self.size, None, act=ActType.RELU, bn=False)
+        self.conv(1, "conv3x3", 3, self.ch, self.ch, self.width, self.height, None, act=ActType.RELU, bn=False)
 
     def makeInput(self):
-        return prng.uniform(SEED_BASE + 256 + 200, (self.ch, self.size, self.size), -1.0, 1.0)
+        return prng.uniform(SEED_BASE + 256 + 200, (self.ch, self.height, self.width), -1.0, 1.0)
 
     def setInput(self, x):
         self.layers[1].setInput(x, 0)
