@@ -111,7 +111,7 @@ class SingleConvNet(_StreamNet):
         self.width, self.height, self.ch = width or size, height or size, channels
 
     def define(self):
-        self.conv(1, "conv3x3", 3, self.ch, self.ch, self.width, self.height, None, act=ActType.RELU, bn=False)
+        self.conv(1, "conv3x3", 3, self.ch, self.ch, self.height, self.width, None, act=ActType.RELU, bn=False)
 
     def makeInput(self):
         return prng.uniform(SEED_BASE + 256 + 200, (self.ch, self.height, self.width), -1.0, 1.0)

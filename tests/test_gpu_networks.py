@@ -117,6 +117,76 @@ def test_config2_full_size_properties():
     assert np.array_equal(outs[0], outs[1])
 
 
+def _window_check(net, storage, windows_per_layer=2, win=40):
+    """Full-size check of every (transposed) convolution on windows: the engine's own input tensor is
+    cropped around a window, the oracle evaluates the layer on the crop, and the part of the result that
+    does not depend on what lies outside the crop is compared with the engine's output there.  One window
+    sits in the image corner (so the zero halo at the real border takes part), one in the interior."""
+    desc = net.describe()
+    src = {(i, port): o for (o, i, port) in desc["connections"]}
+    checked = 0
+    for lyr in net.layers:
+        b = lyr.builder
+        t = int(b.type_)
+        if t not in (int(fa.LayerType.CONVOLUTION2D), int(fa.LayerType.TRANSCONVOLUTION2D)):
+            continue
+        if (lyr.number, 0) not in src:
+            continue
+        x = net.layers[src[(lyr.number, 0)]].copyResult()
+        y = lyr.copyResult()
+        res = net.layers[src[(lyr.number, 1)]].copyResult() if (lyr.number, 1) in src else None
+        k = b.kernel_
+        up = t == int(fa.LayerType.TRANSCONVOLUTION2D)
+        s = 1 if up else b.downsample_[0]
+        r = (k - 1) // 2 * (1 if up else b.dilation_[0])
+        H, W = x.shape[1:]
+        for wi in range(windows_per_layer):
+            hh, ww = min(win * s, H), min(win * s, W)
+            y0 = 0 if wi == 0 else ((H - hh) // 2) // s * s
+            x0 = 0 if wi == 0 else ((W - ww) // 2) // s * s
+            crop = x[:, y0:y0 + hh, x0:x0 + ww]
+            if up:
+                oy0, ox0, oh, ow = 2 * y0, 2 * x0, 2 * hh, 2 * ww
+            else:
+                oy0, ox0, oh, ow = y0 // s, x0 // s, hh // s, ww // s
+            ins = [crop] + ([res[:, oy0:oy0 + oh, ox0:ox0 + ow]] if res is not None else [])
+            ref = O.run_layer(b, lyr.weights, ins, f16=(storage == fa.STORAGE_F16))
+            ref = ref[:, :oh, :ow]
+            m = (r + s - 1) // s + (2 if up else 0)  # outputs near a cut edge depend on pixels outside the crop
+            ty0 = 0 if y0 == 0 else m
+            tx0 = 0 if x0 == 0 else m
+            ty1 = oh if y0 + hh >= H else oh - m
+            tx1 = ow if x0 + ww >= W else ow - m
+            a = y[:, oy0 + ty0:oy0 + ty1, ox0 + tx0:ox0 + tx1]
+            e = rel_l2(a, ref[:, ty0:ty1, tx0:tx1])
+            print("  layer %3d %-10s window %d (%d,%d)+%dx%d rel-L2 %.2e" % (lyr.number, lyr.name, wi, oy0, ox0, oh, ow, e), flush=True)
+            assert e <= TOL[storage], "layer %s window %d: rel-L2 %.3e" % (lyr.name, wi, e)
+            checked += 1
+    return checked
+
+
+def test_config2_full_size_windows_against_oracle():
+    """512x624 fp32: every convolution of the full-size style net against the oracle on image windows."""
+    net = networks.StyleNet(fa.STORAGE_F32)
+    net.setup(reuseBuffers=False)
+    net.setInput(net.makeInput())
+    net.forward()
+    net.finish()
+    assert _window_check(net, fa.STORAGE_F32) >= 30
+    net.cleanup()
+
+
+def test_config5_full_size_windows_against_oracle():
+    """1524x1856 fp16 storage, 9x9 residual convolutions: full size, windows against the oracle."""
+    net = networks.StyleNet(fa.STORAGE_F16, 1524, 1856, 9)
+    net.setup(reuseBuffers=False)
+    net.setInput(net.makeInput())
+    net.forward()
+    net.finish()
+    assert _window_check(net, fa.STORAGE_F16, win=24) >= 30
+    net.cleanup()
+
+
 def test_weight_reload_swaps_style():
     # samples/samplenetworks/stylenet3x3.cpp:81-89: weights can be loaded again after setup
     net = networks.StyleNet(fa.STORAGE_F32, width=64, height=48)
