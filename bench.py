@@ -127,14 +127,15 @@ def dominant_conv_roofline(net, storage_bytes):
         flops, (ein, eout, ew) = conv_work(b)
         res = eout if int(b.getFlags()) & 1 else 0
         nbytes = storage_bytes * (ein + eout + res + ew)
-        t_mfma = flops / (PEAK_MFMA_F16_TFLOPS * 1e12)
+        # fp32 storage: every algorithmic FLOP is issued as three fp16 MFMA FLOPs (hi*hi, lo*hi, hi*lo),
+        # which decides the bound; `achieved` stays the ALGORITHMIC rate against the fp16 matrix peak
+        passes = 3 if storage_bytes == 4 else 1
+        t_mfma = passes * flops / (PEAK_MFMA_F16_TFLOPS * 1e12)
         t_hbm = nbytes / (PEAK_HBM_GBS * 1e9)
         if t_mfma >= t_hbm:
             ach = flops / (avg_ms * 1e-3) / 1e12
-            rec.update({"bound": "mfma", "achieved": ach, "peak": PEAK_MFMA_F16_TFLOPS, "unit": "TFLOP/s", "frac": ach / PEAK_MFMA_F16_TFLOPS})
-            if storage_bytes == 4:
-                # fp32 storage: every algorithmic FLOP is issued as three fp16 MFMA FLOPs (hi*hi, lo*hi, hi*lo)
-                rec.update({"mfma_passes": 3, "mfma_issue_frac": 3 * ach / PEAK_MFMA_F16_TFLOPS})
+            rec.update({"bound": "mfma", "achieved": ach, "peak": PEAK_MFMA_F16_TFLOPS, "unit": "TFLOP/s", "frac": ach / PEAK_MFMA_F16_TFLOPS,
+                        "mfma_passes": passes, "mfma_issue_frac": passes * ach / PEAK_MFMA_F16_TFLOPS})
         else:
             ach = nbytes / (avg_ms * 1e-3) / 1e9
             rec.update({"bound": "hbm", "achieved": ach, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": ach / PEAK_HBM_GBS})
@@ -186,9 +187,12 @@ def main():
     net.setup()
     x = net.makeInput()
     net.setInput(x)
-    ms = timed_forwards(net, args.steps, args.warmup, graph=True)
-    ms_eager = timed_forwards(net, max(5, args.steps // 5), 2, graph=False)
-    log("%s: %.4f ms/step (hipGraph), %.4f ms/step (eager launches)" % (args.workload, ms, ms_eager))
+    # both launch modes of the engine are timed over exactly K steps; the faster one is reported as `value`
+    ms_graph = timed_forwards(net, args.steps, args.warmup, graph=True)
+    ms_eager = timed_forwards(net, args.steps, args.warmup, graph=False)
+    log("%s: %.4f ms/step (hipGraph), %.4f ms/step (eager launches)" % (args.workload, ms_graph, ms_eager))
+    ms = min(ms_graph, ms_eager)
+    launch = "hipGraph replay" if ms_graph <= ms_eager else "eager launches on one stream"
     net.useGraph(False)
     storage_bytes = 4 if net.storage == fa.STORAGE_F32 else 2
     roof, per_layer = dominant_conv_roofline(net, storage_bytes)
@@ -207,9 +211,9 @@ def main():
 
     out = {"metric": metric, "value": value, "unit": unit, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
            "ms_per_step": ms, "higher_is_better": hib, "scaling": "weak", "vs_baseline": None, "dtype": dtype, "data": "synthetic",
-           "config": {"workload": args.workload, "input": list(x.shape), "batch": 1, "launch": "hipGraph replay",
+           "config": {"workload": args.workload, "input": list(x.shape), "batch": 1, "launch": launch,
                       "algorithmic_gflop_per_step": total_flops / 1e9},
-           "ms_per_step_eager": ms_eager, "roofline": roof}
+           "ms_per_step_graph": ms_graph, "ms_per_step_eager": ms_eager, "roofline": roof}
 
     if not args.no_cpu_baseline:
         dt, flops, threads, lname = cpu_baseline(net, x, total_flops)
@@ -231,10 +235,11 @@ def main():
             n2, m2, u2, d2 = make_net(wl)
             n2.setup()
             n2.setInput(n2.makeInput())
-            ms2 = timed_forwards(n2, max(args.steps, 100), args.warmup, graph=True)
-            ms2e = timed_forwards(n2, 20, 2, graph=False)
-            also[m2] = {"value": 1e3 / ms2, "unit": u2, "ms_per_step": ms2, "ms_per_step_eager": ms2e, "dtype": d2}
-            log("%s: %.4f ms/step (hipGraph) %.4f (eager)" % (wl, ms2, ms2e))
+            ms2g = timed_forwards(n2, max(args.steps, 100), args.warmup, graph=True)
+            ms2e = timed_forwards(n2, max(args.steps, 100), args.warmup, graph=False)
+            ms2 = min(ms2g, ms2e)
+            also[m2] = {"value": 1e3 / ms2, "unit": u2, "ms_per_step": ms2, "ms_per_step_graph": ms2g, "ms_per_step_eager": ms2e, "dtype": d2}
+            log("%s: %.4f ms/step (hipGraph) %.4f (eager)" % (wl, ms2g, ms2e))
             n2.cleanup()
         out["also"] = also
     print(json.dumps(out), flush=True)

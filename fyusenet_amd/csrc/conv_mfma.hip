@@ -18,16 +18,25 @@
 #include <hip/hip_fp16.h>
 #include <hip/hip_runtime.h>
 
+#include <cstdio>
+#include <cstdlib>
 #include <map>
 #include <mutex>
+#include <vector>
 
 #include "kernels.h"
 
 // prefetch distance (k16 steps) of the weight fragments, by cout fragments per wave
-#ifndef FYN_CONV_PD
-#define FYN_CONV_PD(FM) 2
+// Timing-study builds (-DFYN_CONV_TRACE): wave 0 of every workgroup records the shader clock at phase boundaries.
+#ifdef FYN_CONV_TRACE
+#define FYN_TRACE(slot) do { if (tid == 0 && (slot) < 16) p.trace[(size_t)blockIdx.x * 16 + (slot)] = clock64(); } while (0)
+#else
+#define FYN_TRACE(slot) do { } while (0)
 #endif
 
+#ifndef FYN_ABL
+#define FYN_ABL 0
+#endif
 namespace fynhip {
 
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
@@ -161,7 +170,7 @@ __device__ __forceinline__ half8_t load_b_frag(const unsigned char* src) {
     return *reinterpret_cast<const half8_t*>(src);
 }
 
-template <typename TIn, typename TOut, bool SPLIT, int FM, int FN, int WM, int WN, int KC>
+template <typename TIn, typename TOut, bool SPLIT, int FM, int FN, int WM, int WN, int KC, int PD>
 __global__ __launch_bounds__(256) void conv_mfma_kernel(const ConvMfmaParams p) {
     extern __shared__ __align__(16) unsigned char lds[];
     constexpr int NPL = SPLIT ? 2 : 1;         // operand planes (hi, lo)
@@ -170,8 +179,9 @@ __global__ __launch_bounds__(256) void conv_mfma_kernel(const ConvMfmaParams p) 
     static_assert(WM * WN == 4, "4 waves per block");
 
     const int tid = threadIdx.x;
+    FYN_TRACE(0);
     const int lane = tid & 63;
-    const int wave = tid >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: keeps tile/fragment index math scalar
     const int wm = wave % WM;
     const int wn = wave / WM;
 
@@ -205,7 +215,7 @@ __global__ __launch_bounds__(256) void conv_mfma_kernel(const ConvMfmaParams p) 
         // slack behind each plane is read by the last (zero-weight) k elements of a row run
         if (tid < 16 * NPL) {
             int pl = tid >> 4;
-            reinterpret_cast<uint32_t*>(lds + pl * p.plane + p.halo_h * p.row_pitch)[tid & 15] = 0u;
+            reinterpret_cast<uint32_t*>(lds + 1024 + pl * p.plane + p.halo_h * p.row_pitch)[tid & 15] = 0u;
         }
     }
 
@@ -232,11 +242,9 @@ __global__ __launch_bounds__(256) void conv_mfma_kernel(const ConvMfmaParams p) 
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
 
-    // A fragments are prefetched PD steps ahead into a register ring that is indexed statically (the
-    // step loop is unrolled PD-fold; the host pads nsteps to a multiple of PD with zero-weight steps):
-    // with only two or three waves per SIMD the L2 round trip of a weight fragment is several times
-    // longer than one step's MFMAs.
-    constexpr int PD = FYN_CONV_PD(FM);
+    // A fragments are prefetched PD-1 steps ahead into a register ring that is indexed statically (the
+    // step loop is unrolled PD-fold; nsteps is a multiple of PD): with one to three waves per SIMD the L2
+    // round trip of a weight fragment is several times longer than one step's MFMAs.
     half8_t a_q[PD][FM][NPL];
 #pragma unroll
     for (int d = 0; d < PD; d++) {
@@ -246,19 +254,12 @@ __global__ __launch_bounds__(256) void conv_mfma_kernel(const ConvMfmaParams p) 
 #pragma unroll
             for (int pl = 0; pl < NPL; pl++) a_q[d][fm][pl] = w_[(fm * NPL + pl) * 64];
     }
-    // LDS byte offsets of the (up to 256) k16 steps, kept in four VGPRs (entry t in lane t%64 of register
-    // t/64) and read with v_readlane: no scalar memory traffic inside the step loop
-    const int tab0 = (lane < p.nsteps) ? p.aoff[lane] : 0;
-    const int tab1 = (lane + 64 < p.nsteps) ? p.aoff[lane + 64] : 0;
-    const int tab2 = (lane + 128 < p.nsteps) ? p.aoff[lane + 128] : 0;
-    const int tab3 = (lane + 192 < p.nsteps) ? p.aoff[lane + 192] : 0;
-    auto step_off = [&](int t_) -> int {
-        const int r0 = __builtin_amdgcn_readlane(tab0, t_ & 63);
-        const int r1 = __builtin_amdgcn_readlane(tab1, t_ & 63);
-        const int r2 = __builtin_amdgcn_readlane(tab2, t_ & 63);
-        const int r3 = __builtin_amdgcn_readlane(tab3, t_ & 63);
-        return t_ < 128 ? (t_ < 64 ? r0 : r1) : (t_ < 192 ? r2 : r3);
-    };
+    // LDS byte offsets of the (up to 256) k16 steps of a chunk: a 1 KB table at the start of LDS.  A step
+    // reads the entry of step t+2 with an ordinary (asynchronous) LDS load into a VGPR; the value is only
+    // consumed one step later, so the lookup never stalls the instruction stream.
+    int* steptab = reinterpret_cast<int*>(lds);
+    if (tid < p.nsteps) steptab[tid] = p.aoff[tid];
+    unsigned char* const sbase = lds + 1024;   // staging buffers follow the table
 
     // ---- staging machinery: items (pixel, 8-channel group) of the halo tile; the first NB items of a
     //      thread are described once (their addresses only shift by the chunk's channel offset) and
@@ -342,53 +343,57 @@ __global__ __launch_bounds__(256) void conv_mfma_kernel(const ConvMfmaParams p) 
 
     // prologue: chunk 0 into buffer 0
     fetch_first(0);
-    store_first(0, lds);
-    stage_rest(0, lds);
+    store_first(0, sbase);
+    stage_rest(0, sbase);
     __syncthreads();
+    FYN_TRACE(1);
 
     // ---- main loop: channel chunks, each nsteps k16 steps in groups of PD.  B fragments of step t+1 are
     //      read from LDS while the MFMAs of step t run; the next chunk's tile is fetched from HBM/L2 at the
     //      start of a chunk and converted into the other LDS buffer at its end, one barrier per chunk. ----
     int gs = 0;  // global step = chunk * nsteps + t
-    half8_t b_cur[FN][NPL];
-    unsigned char* cur = lds;
-    // PD steps starting at step t0 of the current chunk; `more`: another group follows in this chunk
-    auto run_group = [&](int t0, bool more) {
+    // B fragments ping-pong between two statically indexed register sets (PD is even, so the set of a
+    // step is the parity of its position in the group): the LDS reads of step t+1 are issued before the
+    // MFMAs of step t and nothing is copied.
+    static_assert(PD % 2 == 0, "the B fragment ping-pong needs an even step group");
+    half8_t b_buf[2][FN][NPL];
+    unsigned char* cur = sbase;
+    // step offsets of the next two steps (ping-pong like the B fragments)
+    int ao_reg[2];
+    ao_reg[0] = steptab[0];
+    ao_reg[1] = steptab[p.nsteps > 1 ? 1 : 0];
+    // PD steps starting at step t0 of the current chunk.  The body is branch-free (after the chunk's last
+    // step the B prefetch re-reads step 0, unused) and written as one slot per MFMA: the MFMA, then a share
+    // of the step's memory instructions -- LDS reads of the B fragments of step t+1, and the refill of the
+    // ring slot used by step t-1 with the A fragments of step t+PD-1 -- fenced so that the compiler keeps
+    // this order.  A memory instruction issued right after an MFMA runs in that MFMA's shadow; a block of
+    // memory instructions between two MFMAs leaves the matrix pipe idle (one wave cannot queue MFMAs).
+    constexpr int NMF = FM * FN * (SPLIT ? 3 : 1);     // MFMAs per step
+    constexpr int NDS = FN * NPL;                      // B fragment reads per step
+    constexpr int NVM = FM * NPL;                      // A fragment loads per step
+    auto run_group = [&](int t0) {
 #pragma unroll
         for (int d = 0; d < PD; d++) {
-            const bool has_next = (d + 1 < PD) || more;
-            half8_t b_nxt[FN][NPL];
-            if (has_next) {
-                const int ao = step_off(t0 + d + 1);
+            const int ao = ao_reg[(d + 1) & 1];               // offset of step t+1 (loaded one step ago)
+            const int t2 = t0 + d + 2;                        // the table wraps: the next chunk starts at step 0 again
+            const int* tab2 = steptab + (t2 < p.nsteps ? t2 : t2 - p.nsteps);
+            const int dprev = (d + PD - 1) % PD;       // ring slot of the previous step: free for refill
+            const int nx = gs + PD - 1 < total_steps ? gs + PD - 1 : total_steps - 1;
+            const half8_t* w_ = wfrag + (size_t)nx * wstep;
 #pragma unroll
-                for (int fn = 0; fn < FN; fn++)
+            for (int i = 0; i < NMF; i++) {
+                const int kind = i / (FM * FN), rem = i % (FM * FN);
+                const int fm = rem / FN, fn = rem % FN;
+                const int apl = (kind == 1) ? 1 : 0, bpl = (kind == 2) ? 1 : 0;
+                acc[fm][fn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_q[d][fm][apl], b_buf[d & 1][fn][bpl], acc[fm][fn], 0, 0, 0);
+                if (i == NMF - 1) ao_reg[d & 1] = *tab2;    // after the step's last use of the other parity's consumers
 #pragma unroll
-                    for (int pl = 0; pl < NPL; pl++) b_nxt[fn][pl] = load_b_frag<KC>(cur + pl * p.plane + boff[fn] + ao);
-            }
+                for (int j = i * NDS / NMF; j < ((FYN_ABL & 2) ? 0 : (i + 1) * NDS / NMF); j++)   // plane 0 of all fragments first
+                    b_buf[(d + 1) & 1][j % FN][j / FN] = load_b_frag<KC>(cur + (j / FN) * p.plane + (boff[j % FN] + ao));
 #pragma unroll
-            for (int fm = 0; fm < FM; fm++)
-#pragma unroll
-                for (int fn = 0; fn < FN; fn++) {
-                    acc[fm][fn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_q[d][fm][0], b_cur[fn][0], acc[fm][fn], 0, 0, 0);
-                    if (SPLIT) {
-                        acc[fm][fn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_q[d][fm][1], b_cur[fn][0], acc[fm][fn], 0, 0, 0);
-                        acc[fm][fn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_q[d][fm][0], b_cur[fn][1], acc[fm][fn], 0, 0, 0);
-                    }
-                }
-            {
-                // refill this ring slot with the fragments of step gs+PD (past the end: the last step again)
-                const int nx = gs + PD < total_steps ? gs + PD : total_steps - 1;
-                const half8_t* w_ = wfrag + (size_t)nx * wstep;
-#pragma unroll
-                for (int fm = 0; fm < FM; fm++)
-#pragma unroll
-                    for (int pl = 0; pl < NPL; pl++) a_q[d][fm][pl] = w_[(fm * NPL + pl) * 64];
-            }
-            if (has_next) {
-#pragma unroll
-                for (int fn = 0; fn < FN; fn++)
-#pragma unroll
-                    for (int pl = 0; pl < NPL; pl++) b_cur[fn][pl] = b_nxt[fn][pl];
+                for (int j = i * NVM / NMF; j < ((FYN_ABL & 1) ? 0 : (i + 1) * NVM / NMF); j++)
+                    a_q[dprev][j % FM][j / FM] = w_[((j % FM) * NPL + j / FM) * 64];
+                __builtin_amdgcn_sched_barrier(0);
             }
             gs++;
         }
@@ -397,21 +402,21 @@ __global__ __launch_bounds__(256) void conv_mfma_kernel(const ConvMfmaParams p) 
         const bool more_chunks = chunk + 1 < p.cin_chunks;
         fetch_first(more_chunks ? chunk + 1 : chunk);  // (unused after the last chunk; keeps the load count static)
         {
-            const int ao = step_off(0);
+            const int ao = ao_reg[0];
 #pragma unroll
             for (int fn = 0; fn < FN; fn++)
 #pragma unroll
-                for (int pl = 0; pl < NPL; pl++) b_cur[fn][pl] = load_b_frag<KC>(cur + pl * p.plane + boff[fn] + ao);
+                for (int pl = 0; pl < NPL; pl++) b_buf[0][fn][pl] = load_b_frag<KC>(cur + pl * p.plane + (boff[fn] + ao));
         }
-        // first group peeled: the tile loads issued above are younger than the ring's loads only here
-        run_group(0, p.nsteps > PD);
-        for (int t0 = PD; t0 < p.nsteps; t0 += PD) run_group(t0, t0 + PD < p.nsteps);
+        for (int t0 = 0; t0 < p.nsteps; t0 += PD) run_group(t0);
+        FYN_TRACE(2 + 2 * chunk);
         if (more_chunks) {
-            unsigned char* nxt = lds + ((chunk + 1) & 1) * bufsz;
+            unsigned char* nxt = sbase + ((chunk + 1) & 1) * bufsz;
             store_first(chunk + 1, nxt);
             stage_rest(chunk + 1, nxt);
             __syncthreads();  // everyone is done reading `cur` and writing `nxt`
             cur = nxt;
+            FYN_TRACE(3 + 2 * chunk);
         }
     }
 
@@ -421,10 +426,11 @@ __global__ __launch_bounds__(256) void conv_mfma_kernel(const ConvMfmaParams p) 
     //      16-byte pieces; scale, bias' and the residual are applied on the way out
     //      (shaders/deep/deepconv3x3_tiled.frag:36-45 order). ----
     __syncthreads();  // all waves are done with the staged tiles; LDS is reused below
+    FYN_TRACE(14);
     constexpr int ROWF = FM * 32 + 4;                 // floats per position row (+4: bank spread)
     constexpr int LPP = FM * 8;                       // lanes per position on the way out
     constexpr int PPI = 64 / LPP;                     // positions per store instruction
-    float* tr = reinterpret_cast<float*>(lds) + wave * (32 * ROWF);
+    float* tr = reinterpret_cast<float*>(lds) + wave * (FN * 32 * ROWF);   // FN fragments of 32 rows per wave
     TOut* out = reinterpret_cast<TOut*>(p.out);
     const TOut* res = reinterpret_cast<const TOut*>(p.res);
     const int c4 = (lane % LPP) * 4;                                   // channel offset inside the wave's range
@@ -435,8 +441,40 @@ __global__ __launch_bounds__(256) void conv_mfma_kernel(const ConvMfmaParams p) 
         sc = *reinterpret_cast<const f32x4_t*>(p.scale + c);
         bi = *reinterpret_cast<const f32x4_t*>(p.bias + c);
     }
+    // Phases instead of a per-fragment round trip (one wave per SIMD cannot hide latencies behind other
+    // waves): (1) all residual loads, (2) all accumulators into LDS, (3) all rows back, (4) arithmetic and
+    // stores.
+    // Row r of a fragment is position m = frag*32 + it*PPI + lane/LPP; PPI divides the tile width, so the
+    // tile row (and with it the image row) of an (fn, it) pair is wave-uniform and only the column carries a
+    // per-lane part: base addresses are scalar, the per-lane offset is computed once.
+    constexpr int ITS = 32 / PPI;
+    const int lrow = lane / LPP;
+    const int out_lane = lrow * p.out_step * p.out_cp + c;
+    const int res_lane = lrow * p.out_step * p.res_cp + c;
+    bool ok[FN][ITS];
+    size_t obase[FN][ITS];
+    float rres[FN][ITS][4];
 #pragma unroll
-    for (int fn = 0; fn < FN; fn++) {
+    for (int fn = 0; fn < FN; fn++)
+#pragma unroll
+        for (int it = 0; it < ITS; it++) {
+            const int m0 = (wn * FN + fn) * 32 + it * PPI;
+            const int py = pos_y0 + (m0 >> twl), px0 = pos_x0 + (m0 & (TW - 1));
+            ok[fn][it] = c_ok && py < p.npos_y && px0 + lrow < p.npos_x;
+            obase[fn][it] = ((size_t)(p.out_off_y + py * p.out_step) * p.out_wp + p.out_off_x + px0 * p.out_step) * p.out_cp + out_lane;
+#pragma unroll
+            for (int i = 0; i < 4; i++) rres[fn][it][i] = 0.f;
+            if (res && ok[fn][it]) {
+                const size_t rbase = ((size_t)(p.res_off_y + py * p.out_step) * p.res_wp + p.res_off_x + px0 * p.out_step) * p.res_cp + res_lane;
+                float r[8];
+                load_vals<TOut>(res + rbase, r, 4);
+#pragma unroll
+                for (int i = 0; i < 4; i++) rres[fn][it][i] = r[i];
+            }
+        }
+    FYN_TRACE(9);
+#pragma unroll
+    for (int fn = 0; fn < FN; fn++)
 #pragma unroll
         for (int fm = 0; fm < FM; fm++)
 #pragma unroll
@@ -444,43 +482,50 @@ __global__ __launch_bounds__(256) void conv_mfma_kernel(const ConvMfmaParams p) 
                 f32x4_t v;
                 v[0] = acc[fm][fn][q * 4 + 0]; v[1] = acc[fm][fn][q * 4 + 1];
                 v[2] = acc[fm][fn][q * 4 + 2]; v[3] = acc[fm][fn][q * 4 + 3];
-                *reinterpret_cast<f32x4_t*>(tr + (lane & 31) * ROWF + fm * 32 + q * 8 + (lane >> 5) * 4) = v;
+                *reinterpret_cast<f32x4_t*>(tr + (fn * 32 + (lane & 31)) * ROWF + fm * 32 + q * 8 + (lane >> 5) * 4) = v;
             }
+    FYN_TRACE(10);
+    f32x4_t a4[FN][ITS];
 #pragma unroll
-        for (int it = 0; it < 32 / PPI; it++) {
-            const int row = it * PPI + lane / LPP;
-            const f32x4_t a4 = *reinterpret_cast<const f32x4_t*>(tr + row * ROWF + c4);
-            const int m = (wn * FN + fn) * 32 + row;
-            const int py = pos_y0 + (m >> twl), px = pos_x0 + (m & (TW - 1));
-            if (!c_ok || py >= p.npos_y || px >= p.npos_x) continue;
-            float o[4];
+    for (int fn = 0; fn < FN; fn++)
 #pragma unroll
-            for (int i = 0; i < 4; i++) o[i] = (a4[i] * p.acc_mul) * sc[i] + bi[i];
-            if (res) {
-                const size_t rbase = ((size_t)(p.res_off_y + py * p.out_step) * p.res_wp + p.res_off_x + px * p.out_step) * p.res_cp;
-                float r[8];
-                load_vals<TOut>(res + rbase + c, r, 4);
+        for (int it = 0; it < ITS; it++)
+            a4[fn][it] = *reinterpret_cast<const f32x4_t*>(tr + (fn * 32 + it * PPI + lane / LPP) * ROWF + c4);
+    // arithmetic for every row unconditionally (one wait for the loads above), then predicated stores only:
+    // a wait inside a predicated region would also wait for the stores issued before it
 #pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    float rv = r[i];
-                    if (p.res_relu) rv = fmaxf(rv, 0.f);
-                    if (p.res_scale) rv *= sc[i];
-                    o[i] += rv;
-                }
+    for (int fn = 0; fn < FN; fn++)
+#pragma unroll
+        for (int it = 0; it < ITS; it++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                float rv = rres[fn][it][i];   // zero without a residual input
+                if (p.res_relu) rv = fmaxf(rv, 0.f);
+                if (p.res_scale) rv *= sc[i];
+                a4[fn][it][i] = ((a4[fn][it][i] * p.acc_mul) * sc[i] + bi[i]) + rv;
             }
-            const size_t obase = ((size_t)(p.out_off_y + py * p.out_step) * p.out_wp + p.out_off_x + px * p.out_step) * p.out_cp;
+    // pin the results in registers here: the compiler would otherwise sink the arithmetic (and the waits for
+    // its inputs) into the predicated store regions below
+#pragma unroll
+    for (int fn = 0; fn < FN; fn++)
+#pragma unroll
+        for (int it = 0; it < ITS; it++) asm volatile("" : "+v"(a4[fn][it]));
+    FYN_TRACE(11);
+#pragma unroll
+    for (int fn = 0; fn < FN; fn++)
+#pragma unroll
+        for (int it = 0; it < ITS; it++) {
+            if (!ok[fn][it]) continue;
             if (sizeof(TOut) == 4) {
-                f32x4_t ov;
-                ov[0] = o[0]; ov[1] = o[1]; ov[2] = o[2]; ov[3] = o[3];
-                *reinterpret_cast<f32x4_t*>(reinterpret_cast<float*>(out) + obase + c) = ov;
+                *reinterpret_cast<f32x4_t*>(reinterpret_cast<float*>(out) + obase[fn][it]) = a4[fn][it];
             } else {
                 half4_t hv;
 #pragma unroll
-                for (int i = 0; i < 4; i++) hv[i] = (_Float16)o[i];
-                *reinterpret_cast<half4_t*>(reinterpret_cast<_Float16*>(out) + obase + c) = hv;
+                for (int i = 0; i < 4; i++) hv[i] = (_Float16)a4[fn][it][i];
+                *reinterpret_cast<half4_t*>(reinterpret_cast<_Float16*>(out) + obase[fn][it]) = hv;
             }
         }
-    }
+    FYN_TRACE(15);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -514,14 +559,15 @@ typedef void (*conv_kernel_fn)(const ConvMfmaParams);
     X(12, 1, 4, 2, 2)     \
     X(13, 1, 3, 2, 2)
 
+// Step group sizes (prefetch ring depths): 2 for every chunk width, 4 and 6 for 32-channel chunks only.
 template <typename TIn, typename TOut, bool SPLIT, int FM, int FN, int WM, int WN>
-static conv_kernel_fn pick_kc(int kc) {
-    switch (kc) {
-        case 4: return conv_mfma_kernel<TIn, TOut, SPLIT, FM, FN, WM, WN, 4>;
-        case 16: return conv_mfma_kernel<TIn, TOut, SPLIT, FM, FN, WM, WN, 16>;
-        case 32: return conv_mfma_kernel<TIn, TOut, SPLIT, FM, FN, WM, WN, 32>;
-        default: return nullptr;
-    }
+static conv_kernel_fn pick_kc(int kc, int pd) {
+    if (kc == 4 && pd == 2) return conv_mfma_kernel<TIn, TOut, SPLIT, FM, FN, WM, WN, 4, 2>;
+    if (kc == 16 && pd == 2) return conv_mfma_kernel<TIn, TOut, SPLIT, FM, FN, WM, WN, 16, 2>;
+    if (kc == 32 && pd == 2) return conv_mfma_kernel<TIn, TOut, SPLIT, FM, FN, WM, WN, 32, 2>;
+    if (kc == 32 && pd == 4) return conv_mfma_kernel<TIn, TOut, SPLIT, FM, FN, WM, WN, 32, 4>;
+    if (kc == 32 && pd == 6) return conv_mfma_kernel<TIn, TOut, SPLIT, FM, FN, WM, WN, 32, 6>;
+    return nullptr;
 }
 
 #define FYN_CAT2(a, b) a##b
@@ -536,8 +582,8 @@ static conv_kernel_fn lookup_part(const ConvVariant& v) {
 #define FYN_TILE(idx_, fm_, fn_, wm_, wn_)                                                \
     if constexpr ((idx_) % FYN_CONV_PARTS == PART) {                                       \
         if (v.fm == fm_ && v.fn == fn_ && v.wm == wm_ && v.wn == wn_)                      \
-            return f32 ? pick_kc<float, float, true, fm_, fn_, wm_, wn_>(v.kc)             \
-                       : pick_kc<_Float16, _Float16, false, fm_, fn_, wm_, wn_>(v.kc);     \
+            return f32 ? pick_kc<float, float, true, fm_, fn_, wm_, wn_>(v.kc, v.pd)             \
+                       : pick_kc<_Float16, _Float16, false, fm_, fn_, wm_, wn_>(v.kc, v.pd);     \
     }
     FYN_CONV_TILES(FYN_TILE)
 #undef FYN_TILE
@@ -591,7 +637,7 @@ static conv_kernel_fn pick_kernel(const ConvVariant& v) {
 
 bool conv_mfma_variant_exists(const ConvVariant& v) { return pick_kernel(v) != nullptr; }
 
-int conv_mfma_step_multiple(const ConvVariant& v) { return FYN_CONV_PD(v.fm); }
+int conv_mfma_step_multiple(const ConvVariant& v) { return v.pd; }
 
 int conv_mfma_tile_count() {
     int n = 0;
@@ -611,7 +657,7 @@ void conv_mfma_tile(int index, int* fm, int* fn, int* wm, int* wn) {
 int launch_conv_mfma(const ConvVariant& v, const ConvMfmaParams& p, size_t lds_bytes, hipStream_t s) {
     conv_kernel_fn fn = pick_kernel(v);
     if (!fn) return -1;
-    if (p.nsteps < 1 || p.nsteps > 256 || p.nsteps % FYN_CONV_PD(v.fm) != 0) return -5;
+    if (p.nsteps < 1 || p.nsteps > 256 || v.pd < 2 || p.nsteps % v.pd != 0) return -5;
     if (lds_bytes > 48 * 1024) {
         // raise the kernel's dynamic LDS limit once per kernel and size
         static std::mutex mu;
@@ -626,7 +672,25 @@ int launch_conv_mfma(const ConvVariant& v, const ConvMfmaParams& p, size_t lds_b
         }
     }
     const int blocks = p.tiles_x * p.tiles_y * p.cout_blocks;
+#ifdef FYN_CONV_TRACE
+    static long long* trace_dev = nullptr;
+    if (!trace_dev && hipMalloc(&trace_dev, sizeof(long long) * 16 * 65536) != hipSuccess) return -6;
+    if (blocks > 65536) return -6;
+    ConvMfmaParams pt = p;
+    pt.trace = trace_dev;
+    hipLaunchKernelGGL(fn, dim3(blocks), dim3(256), lds_bytes, s, pt);
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    (void)hipStreamIsCapturing(s, &cap);
+    const char* path = cap == hipStreamCaptureStatusNone ? getenv("FYNHIP_TRACE_DUMP") : nullptr;
+    if (path) {
+        std::vector<long long> h((size_t)blocks * 16);
+        if (hipStreamSynchronize(s) == hipSuccess && hipMemcpy(h.data(), trace_dev, h.size() * 8, hipMemcpyDeviceToHost) == hipSuccess) {
+            if (FILE* f = fopen(path, "wb")) { fwrite(h.data(), 8, h.size(), f); fclose(f); }
+        }
+    }
+#else
     hipLaunchKernelGGL(fn, dim3(blocks), dim3(256), lds_bytes, s, p);
+#endif
     return hipGetLastError() == hipSuccess ? 0 : -3;
 }
 #endif  // FYN_CONV_PART == 0

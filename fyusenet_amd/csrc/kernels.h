@@ -67,6 +67,9 @@ struct ConvMfmaParams {
     int mfrags;          // cout fragments (32 each) in wpack
     int cout_blocks;     // grid size along cout
     float acc_mul;       // exact power of two undoing the weight pre-scaling
+#ifdef FYN_CONV_TRACE
+    long long* trace;    // timing-study builds only: 16 timestamps per workgroup
+#endif
     Act act;
 };
 
@@ -77,6 +80,7 @@ struct ConvVariant {
     int fm, fn;          // fragments (32 cout / 32 positions) per wave
     int wm, wn;          // waves per block along cout / positions (wm*wn == 4)
     int kc;              // input channels staged per chunk (4 = row-run small-Cin variant, 16, 32)
+    int pd;              // k16 steps per unrolled group = depth of the weight-fragment prefetch ring (2, 4, 6)
 };
 
 // Returns 0 when the variant exists and was launched.

@@ -124,8 +124,9 @@ static std::vector<TileChoice> enumerate_tiles(int cout, const SubConv& sc, int 
         const int cpb = wm * fm * 32;
         const int cblocks = (cout + cpb - 1) / cpb;
         const int halo_w = (tw - 1) * sc.in_stride + sc.span_x, halo_h = (th - 1) * sc.in_stride + sc.span_y;
-        const int rowpad = 0;
-        const size_t lds = (size_t)nbuf * npl * ((size_t)halo_h * (halo_w * pitch + rowpad) + slack);
+        const char* rp = getenv("FYNHIP_ROWPAD");
+        const int rowpad = rp ? atoi(rp) : 0;
+        const size_t lds = 1024 + (size_t)nbuf * npl * ((size_t)halo_h * (halo_w * pitch + rowpad) + slack);
         if (lds > 150 * 1024) continue;
         const double util = ((double)cout * sc.npos_x * sc.npos_y) / ((double)cblocks * cpb * (double)tiles * bm);
         const double blocks = (double)tiles * cblocks;
@@ -191,11 +192,10 @@ static MfmaLaunch plan_mfma(Net* net, const SubConv& sc, const TView& in, const 
     p.bias = bias;
     p.acc_mul = 1.f;
     p.act = act;
-    L.lds = (size_t)npl * p.plane * (p.cin_chunks > 1 ? 2 : 1);  // double-buffered across channel chunks
-    L.lds = std::max(L.lds, (size_t)4 * 32 * (tc.fm * 32 + 4) * 4);      // epilogue transposition area
+    L.lds = 1024 + (size_t)npl * p.plane * (p.cin_chunks > 1 ? 2 : 1);  // step table + tiles (double-buffered across chunks)
+    L.lds = std::max(L.lds, (size_t)4 * tc.fn * 32 * (tc.fm * 32 + 4) * 4);  // epilogue transposition area (all waves, all fragments)
     if (in.elems() >= (size_t)1 << 31) fail(FYN_ERR_UNSUPPORTED, "input tensor too large for 32-bit element offsets");
-    L.var = ConvVariant{in.f16, out.f16, split ? 1 : 0, tc.fm, tc.fn, tc.wm, tc.wn, kc};
-    if (!conv_mfma_variant_exists(L.var)) fail(FYN_ERR_UNSUPPORTED, "MFMA convolution variant not compiled");
+    L.var = ConvVariant{in.f16, out.f16, split ? 1 : 0, tc.fm, tc.fn, tc.wm, tc.wn, kc, 2};
 
     // k16 steps
     if (kc == 4) {
@@ -233,7 +233,16 @@ static MfmaLaunch plan_mfma(Net* net, const SubConv& sc, const TView& in, const 
                 L.steps.push_back(st);
             }
     }
-    // pad to the kernel's step group size with steps whose weights are all zero
+    // step group size = depth of the kernel's weight prefetch ring: the largest compiled one that divides
+    // the step count (32-channel chunks: 6, 4, 2; otherwise 2); an odd count is padded with a zero-weight step
+    {
+        const int raw = (int)L.steps.size();
+        int pd = 2;
+        if (kc == 32) pd = (raw % 6 == 0) ? 6 : ((raw % 4 == 0) ? 4 : 2);
+        if (const char* e = getenv("FYNHIP_CONV_PD")) pd = atoi(e);
+        L.var.pd = pd;
+        if (!conv_mfma_variant_exists(L.var)) fail(FYN_ERR_UNSUPPORTED, "MFMA convolution variant not compiled");
+    }
     while (L.steps.size() % conv_mfma_step_multiple(L.var) != 0) {
         MfmaLaunch::Step st;
         st.aoff = 0;
