@@ -170,9 +170,15 @@ __device__ __forceinline__ half8_t load_b_frag(const unsigned char* src) {
     return *reinterpret_cast<const half8_t*>(src);
 }
 
-template <typename TIn, typename TOut, bool SPLIT, int FM, int FN, int WM, int WN, int KC, int PD>
-__global__ __launch_bounds__(256) void conv_mfma_kernel(const ConvMfmaParams p) {
+template <typename TIn, typename TOut, bool SPLIT, int FM, int FN, int WM, int WN, int KC, int PD, int UNR>
+__global__ __launch_bounds__((FM * FN >= 2) ? 512 : 256) void conv_mfma_kernel(const ConvMfmaParams p) {
     extern __shared__ __align__(16) unsigned char lds[];
+    // Tiles with two or more fragments per wave run one MFMA wave per SIMD; such workgroups get four more
+    // waves (threads 256..511) that do nothing but stage the next input chunk (global loads, activation,
+    // fp32 -> fp16 hi/lo conversion, LDS writes), so that this work shares the SIMDs with the MFMA waves
+    // instead of interrupting them.  Single-fragment tiles (two to three workgroups per CU) stage with the
+    // MFMA waves themselves.
+    constexpr bool SPEC = FM * FN >= 2;
     constexpr int NPL = SPLIT ? 2 : 1;         // operand planes (hi, lo)
     constexpr int CPI = (KC == 4) ? 4 : 8;     // channels per staging item
     constexpr int G = (KC == 4) ? 1 : KC / 8;  // staging items per pixel
@@ -182,8 +188,11 @@ __global__ __launch_bounds__(256) void conv_mfma_kernel(const ConvMfmaParams p) 
     FYN_TRACE(0);
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: keeps tile/fragment index math scalar
-    const int wm = wave % WM;
-    const int wn = wave / WM;
+    const bool consumer = !SPEC || wave < 4;   // issues MFMAs, owns accumulators, writes the output
+    const bool stager = !SPEC || wave >= 4;    // stages input tiles
+    const int stid = SPEC ? (tid & 255) : tid; // thread index among the staging threads
+    const int wm = (wave & 3) % WM;
+    const int wn = (wave & 3) / WM;
 
     // Workgroups are dealt round-robin to the 8 XCDs; remap so that neighbouring tiles (shared
     // halos, same input tile for all cout blocks) meet in one XCD's L2.
@@ -229,10 +238,12 @@ __global__ __launch_bounds__(256) void conv_mfma_kernel(const ConvMfmaParams p) 
     }
 
     // A (weight) fragments: [(chunk*nsteps + step)][mfrag][plane][lane] x 8 halves
-    const half8_t* wfrag = reinterpret_cast<const half8_t*>(p.wpack) +
-                           (size_t)((cb * WM + wm) * FM) * NPL * 64 + lane;
-    const size_t wstep = (size_t)p.mfrags * NPL * 64;
-    const int total_steps = p.cin_chunks * p.nsteps;
+    // (uniform base + per-lane 32-bit offset: the loads use the scalar-base addressing form and stepping
+    // through K costs two scalar adds; the buffer has PD steps of zero slack behind the last step, so the
+    // prefetch needs no clamp)
+    const unsigned char* wbase = reinterpret_cast<const unsigned char*>(p.wpack) + (size_t)((cb * WM + wm) * FM) * NPL * 1024;
+    const unsigned wlane = lane * 16;
+    const unsigned wstep = (unsigned)p.mfrags * NPL * 1024;   // bytes per k16 step
 
     float16_t acc[FM][FN];
 #pragma unroll
@@ -246,13 +257,14 @@ __global__ __launch_bounds__(256) void conv_mfma_kernel(const ConvMfmaParams p) 
     // step loop is unrolled PD-fold; nsteps is a multiple of PD): with one to three waves per SIMD the L2
     // round trip of a weight fragment is several times longer than one step's MFMAs.
     half8_t a_q[PD][FM][NPL];
+    if (consumer)
 #pragma unroll
     for (int d = 0; d < PD; d++) {
-        const half8_t* w_ = wfrag + (size_t)(d < total_steps ? d : total_steps - 1) * wstep;
+        const unsigned char* w_ = wbase + (size_t)d * wstep;
 #pragma unroll
         for (int fm = 0; fm < FM; fm++)
 #pragma unroll
-            for (int pl = 0; pl < NPL; pl++) a_q[d][fm][pl] = w_[(fm * NPL + pl) * 64];
+            for (int pl = 0; pl < NPL; pl++) a_q[d][fm][pl] = *reinterpret_cast<const half8_t*>(w_ + (fm * NPL + pl) * 1024 + wlane);
     }
     // LDS byte offsets of the (up to 256) k16 steps of a chunk: a 1 KB table at the start of LDS.  A step
     // reads the entry of step t+2 with an ordinary (asynchronous) LDS load into a VGPR; the value is only
@@ -270,7 +282,7 @@ __global__ __launch_bounds__(256) void conv_mfma_kernel(const ConvMfmaParams p) 
     int c_off[NB];   // channel offset of the group inside a chunk
 #pragma unroll
     for (int i = 0; i < NB; i++) {
-        const int idx = tid + i * 256;
+        const int idx = stid + i * 256;
         g_off[i] = -1; l_off[i] = -1; c_off[i] = 0;
         if (idx < nitems) {
             const int pix = (G == 1) ? idx : idx / G;
@@ -315,7 +327,7 @@ __global__ __launch_bounds__(256) void conv_mfma_kernel(const ConvMfmaParams p) 
             int lo2[NB];
 #pragma unroll
             for (int i = 0; i < NB; i++) {
-                const int idx = base + tid + i * 256;
+                const int idx = base + stid + i * 256;
                 lo2[i] = -1;
                 r2[i].zero();
                 if (idx < nitems) {
@@ -342,20 +354,22 @@ __global__ __launch_bounds__(256) void conv_mfma_kernel(const ConvMfmaParams p) 
     };
 
     // prologue: chunk 0 into buffer 0
-    fetch_first(0);
-    store_first(0, sbase);
-    stage_rest(0, sbase);
+    if (stager) {
+        fetch_first(0);
+        store_first(0, sbase);
+        stage_rest(0, sbase);
+    }
     __syncthreads();
     FYN_TRACE(1);
 
     // ---- main loop: channel chunks, each nsteps k16 steps in groups of PD.  B fragments of step t+1 are
     //      read from LDS while the MFMAs of step t run; the next chunk's tile is fetched from HBM/L2 at the
     //      start of a chunk and converted into the other LDS buffer at its end, one barrier per chunk. ----
-    int gs = 0;  // global step = chunk * nsteps + t
+    const unsigned char* wnext = wbase + (size_t)(PD - 1) * wstep;   // next ring refill: step PD-1 (again), PD, ...
     // B fragments ping-pong between two statically indexed register sets (PD is even, so the set of a
     // step is the parity of its position in the group): the LDS reads of step t+1 are issued before the
     // MFMAs of step t and nothing is copied.
-    static_assert(PD % 2 == 0, "the B fragment ping-pong needs an even step group");
+    static_assert(PD % 2 == 0 && UNR % PD == 0, "the B fragment ping-pong needs an even step group; the unrolled group covers whole ring turns");
     half8_t b_buf[2][FN][NPL];
     unsigned char* cur = sbase;
     // step offsets of the next two steps (ping-pong like the B fragments)
@@ -373,47 +387,50 @@ __global__ __launch_bounds__(256) void conv_mfma_kernel(const ConvMfmaParams p) 
     constexpr int NVM = FM * NPL;                      // A fragment loads per step
     auto run_group = [&](int t0) {
 #pragma unroll
-        for (int d = 0; d < PD; d++) {
-            const int ao = ao_reg[(d + 1) & 1];               // offset of step t+1 (loaded one step ago)
-            const int t2 = t0 + d + 2;                        // the table wraps: the next chunk starts at step 0 again
+        for (int dd = 0; dd < UNR; dd++) {
+            const int d = dd % PD;                            // ring slot of this step
+            const int ao = ao_reg[(dd + 1) & 1];              // offset of step t+1 (loaded one step ago)
+            const int t2 = t0 + dd + 2;                       // the table wraps: the next chunk starts at step 0 again
             const int* tab2 = steptab + (t2 < p.nsteps ? t2 : t2 - p.nsteps);
             const int dprev = (d + PD - 1) % PD;       // ring slot of the previous step: free for refill
-            const int nx = gs + PD - 1 < total_steps ? gs + PD - 1 : total_steps - 1;
-            const half8_t* w_ = wfrag + (size_t)nx * wstep;
+            const unsigned char* w_ = wnext;                  // fragments of step gs+PD-1
+            wnext += wstep;
 #pragma unroll
             for (int i = 0; i < NMF; i++) {
                 const int kind = i / (FM * FN), rem = i % (FM * FN);
                 const int fm = rem / FN, fn = rem % FN;
                 const int apl = (kind == 1) ? 1 : 0, bpl = (kind == 2) ? 1 : 0;
-                acc[fm][fn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_q[d][fm][apl], b_buf[d & 1][fn][bpl], acc[fm][fn], 0, 0, 0);
-                if (i == NMF - 1) ao_reg[d & 1] = *tab2;    // after the step's last use of the other parity's consumers
+                acc[fm][fn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_q[d][fm][apl], b_buf[dd & 1][fn][bpl], acc[fm][fn], 0, 0, 0);
+                if (i == 0) ao_reg[dd & 1] = *tab2;          // this parity's old value (step t) was consumed during step t-1
 #pragma unroll
                 for (int j = i * NDS / NMF; j < ((FYN_ABL & 2) ? 0 : (i + 1) * NDS / NMF); j++)   // plane 0 of all fragments first
-                    b_buf[(d + 1) & 1][j % FN][j / FN] = load_b_frag<KC>(cur + (j / FN) * p.plane + (boff[j % FN] + ao));
+                    b_buf[(dd + 1) & 1][j % FN][j / FN] = load_b_frag<KC>(cur + (j / FN) * p.plane + (boff[j % FN] + ao));
 #pragma unroll
                 for (int j = i * NVM / NMF; j < ((FYN_ABL & 1) ? 0 : (i + 1) * NVM / NMF); j++)
-                    a_q[dprev][j % FM][j / FM] = w_[((j % FM) * NPL + j / FM) * 64];
+                    a_q[dprev][j % FM][j / FM] = *reinterpret_cast<const half8_t*>(w_ + ((j % FM) * NPL + j / FM) * 1024 + wlane);
                 __builtin_amdgcn_sched_barrier(0);
             }
-            gs++;
         }
     };
     for (int chunk = 0; chunk < p.cin_chunks; chunk++) {
         const bool more_chunks = chunk + 1 < p.cin_chunks;
-        fetch_first(more_chunks ? chunk + 1 : chunk);  // (unused after the last chunk; keeps the load count static)
-        {
+        // (after the last chunk the fetch is unused; it keeps the number of loads in flight static)
+        if (stager) fetch_first(more_chunks ? chunk + 1 : chunk);
+        if (consumer) {
             const int ao = ao_reg[0];
 #pragma unroll
             for (int fn = 0; fn < FN; fn++)
 #pragma unroll
                 for (int pl = 0; pl < NPL; pl++) b_buf[0][fn][pl] = load_b_frag<KC>(cur + pl * p.plane + (boff[fn] + ao));
+            for (int t0 = 0; t0 < p.nsteps; t0 += UNR) run_group(t0);
         }
-        for (int t0 = 0; t0 < p.nsteps; t0 += PD) run_group(t0);
         FYN_TRACE(2 + 2 * chunk);
         if (more_chunks) {
             unsigned char* nxt = sbase + ((chunk + 1) & 1) * bufsz;
-            store_first(chunk + 1, nxt);
-            stage_rest(chunk + 1, nxt);
+            if (stager) {
+                store_first(chunk + 1, nxt);
+                stage_rest(chunk + 1, nxt);
+            }
             __syncthreads();  // everyone is done reading `cur` and writing `nxt`
             cur = nxt;
             FYN_TRACE(3 + 2 * chunk);
@@ -426,11 +443,12 @@ __global__ __launch_bounds__(256) void conv_mfma_kernel(const ConvMfmaParams p) 
     //      16-byte pieces; scale, bias' and the residual are applied on the way out
     //      (shaders/deep/deepconv3x3_tiled.frag:36-45 order). ----
     __syncthreads();  // all waves are done with the staged tiles; LDS is reused below
+    if (!consumer) return;
     FYN_TRACE(14);
     constexpr int ROWF = FM * 32 + 4;                 // floats per position row (+4: bank spread)
     constexpr int LPP = FM * 8;                       // lanes per position on the way out
     constexpr int PPI = 64 / LPP;                     // positions per store instruction
-    float* tr = reinterpret_cast<float*>(lds) + wave * (FN * 32 * ROWF);   // FN fragments of 32 rows per wave
+    float* tr = reinterpret_cast<float*>(lds) + (wave & 3) * (FN * 32 * ROWF);   // FN fragments of 32 rows per wave
     TOut* out = reinterpret_cast<TOut*>(p.out);
     const TOut* res = reinterpret_cast<const TOut*>(p.res);
     const int c4 = (lane % LPP) * 4;                                   // channel offset inside the wave's range
@@ -559,14 +577,16 @@ typedef void (*conv_kernel_fn)(const ConvMfmaParams);
     X(12, 1, 4, 2, 2)     \
     X(13, 1, 3, 2, 2)
 
-// Step group sizes (prefetch ring depths): 2 for every chunk width, 4 and 6 for 32-channel chunks only.
+// (ring depth, unroll) pairs: 2/2 for every chunk width; for 32-channel chunks also 4/4, 6/6 and 6/18 (a whole
+// 3x3 chunk unrolled: no loop back-edge, hence no conservative wait, inside a chunk).
 template <typename TIn, typename TOut, bool SPLIT, int FM, int FN, int WM, int WN>
-static conv_kernel_fn pick_kc(int kc, int pd) {
-    if (kc == 4 && pd == 2) return conv_mfma_kernel<TIn, TOut, SPLIT, FM, FN, WM, WN, 4, 2>;
-    if (kc == 16 && pd == 2) return conv_mfma_kernel<TIn, TOut, SPLIT, FM, FN, WM, WN, 16, 2>;
-    if (kc == 32 && pd == 2) return conv_mfma_kernel<TIn, TOut, SPLIT, FM, FN, WM, WN, 32, 2>;
-    if (kc == 32 && pd == 4) return conv_mfma_kernel<TIn, TOut, SPLIT, FM, FN, WM, WN, 32, 4>;
-    if (kc == 32 && pd == 6) return conv_mfma_kernel<TIn, TOut, SPLIT, FM, FN, WM, WN, 32, 6>;
+static conv_kernel_fn pick_kc(int kc, int pd, int unr) {
+    if (kc == 4 && pd == 2 && unr == 2) return conv_mfma_kernel<TIn, TOut, SPLIT, FM, FN, WM, WN, 4, 2, 2>;
+    if (kc == 16 && pd == 2 && unr == 2) return conv_mfma_kernel<TIn, TOut, SPLIT, FM, FN, WM, WN, 16, 2, 2>;
+    if (kc == 32 && pd == 2 && unr == 2) return conv_mfma_kernel<TIn, TOut, SPLIT, FM, FN, WM, WN, 32, 2, 2>;
+    if (kc == 32 && pd == 4 && unr == 4) return conv_mfma_kernel<TIn, TOut, SPLIT, FM, FN, WM, WN, 32, 4, 4>;
+    if (kc == 32 && pd == 6 && unr == 6) return conv_mfma_kernel<TIn, TOut, SPLIT, FM, FN, WM, WN, 32, 6, 6>;
+    if (kc == 32 && pd == 6 && unr == 18) return conv_mfma_kernel<TIn, TOut, SPLIT, FM, FN, WM, WN, 32, 6, 18>;
     return nullptr;
 }
 
@@ -582,8 +602,8 @@ static conv_kernel_fn lookup_part(const ConvVariant& v) {
 #define FYN_TILE(idx_, fm_, fn_, wm_, wn_)                                                \
     if constexpr ((idx_) % FYN_CONV_PARTS == PART) {                                       \
         if (v.fm == fm_ && v.fn == fn_ && v.wm == wm_ && v.wn == wn_)                      \
-            return f32 ? pick_kc<float, float, true, fm_, fn_, wm_, wn_>(v.kc, v.pd)             \
-                       : pick_kc<_Float16, _Float16, false, fm_, fn_, wm_, wn_>(v.kc, v.pd);     \
+            return f32 ? pick_kc<float, float, true, fm_, fn_, wm_, wn_>(v.kc, v.pd, v.unr)             \
+                       : pick_kc<_Float16, _Float16, false, fm_, fn_, wm_, wn_>(v.kc, v.pd, v.unr);     \
     }
     FYN_CONV_TILES(FYN_TILE)
 #undef FYN_TILE
@@ -637,7 +657,7 @@ static conv_kernel_fn pick_kernel(const ConvVariant& v) {
 
 bool conv_mfma_variant_exists(const ConvVariant& v) { return pick_kernel(v) != nullptr; }
 
-int conv_mfma_step_multiple(const ConvVariant& v) { return v.pd; }
+int conv_mfma_step_multiple(const ConvVariant& v) { return v.unr; }
 
 int conv_mfma_tile_count() {
     int n = 0;
@@ -657,7 +677,7 @@ void conv_mfma_tile(int index, int* fm, int* fn, int* wm, int* wn) {
 int launch_conv_mfma(const ConvVariant& v, const ConvMfmaParams& p, size_t lds_bytes, hipStream_t s) {
     conv_kernel_fn fn = pick_kernel(v);
     if (!fn) return -1;
-    if (p.nsteps < 1 || p.nsteps > 256 || v.pd < 2 || p.nsteps % v.pd != 0) return -5;
+    if (p.nsteps < 1 || p.nsteps > 256 || v.unr < 2 || p.nsteps % v.unr != 0) return -5;
     if (lds_bytes > 48 * 1024) {
         // raise the kernel's dynamic LDS limit once per kernel and size
         static std::mutex mu;
@@ -678,7 +698,7 @@ int launch_conv_mfma(const ConvVariant& v, const ConvMfmaParams& p, size_t lds_b
     if (blocks > 65536) return -6;
     ConvMfmaParams pt = p;
     pt.trace = trace_dev;
-    hipLaunchKernelGGL(fn, dim3(blocks), dim3(256), lds_bytes, s, pt);
+    hipLaunchKernelGGL(fn, dim3(blocks), dim3(v.fm * v.fn >= 2 ? 512 : 256), lds_bytes, s, pt);
     hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
     (void)hipStreamIsCapturing(s, &cap);
     const char* path = cap == hipStreamCaptureStatusNone ? getenv("FYNHIP_TRACE_DUMP") : nullptr;
@@ -689,7 +709,7 @@ int launch_conv_mfma(const ConvVariant& v, const ConvMfmaParams& p, size_t lds_b
         }
     }
 #else
-    hipLaunchKernelGGL(fn, dim3(blocks), dim3(256), lds_bytes, s, p);
+    hipLaunchKernelGGL(fn, dim3(blocks), dim3(v.fm * v.fn >= 2 ? 512 : 256), lds_bytes, s, p);
 #endif
     return hipGetLastError() == hipSuccess ? 0 : -3;
 }

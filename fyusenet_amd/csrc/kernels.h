@@ -80,7 +80,8 @@ struct ConvVariant {
     int fm, fn;          // fragments (32 cout / 32 positions) per wave
     int wm, wn;          // waves per block along cout / positions (wm*wn == 4)
     int kc;              // input channels staged per chunk (4 = row-run small-Cin variant, 16, 32)
-    int pd;              // k16 steps per unrolled group = depth of the weight-fragment prefetch ring (2, 4, 6)
+    int pd;              // depth of the weight-fragment prefetch ring in k16 steps (2, 4, 6)
+    int unr;             // k16 steps per unrolled group (a multiple of pd; nsteps is a multiple of it)
 };
 
 // Returns 0 when the variant exists and was launched.

@@ -195,7 +195,7 @@ static MfmaLaunch plan_mfma(Net* net, const SubConv& sc, const TView& in, const 
     L.lds = 1024 + (size_t)npl * p.plane * (p.cin_chunks > 1 ? 2 : 1);  // step table + tiles (double-buffered across chunks)
     L.lds = std::max(L.lds, (size_t)4 * tc.fn * 32 * (tc.fm * 32 + 4) * 4);  // epilogue transposition area (all waves, all fragments)
     if (in.elems() >= (size_t)1 << 31) fail(FYN_ERR_UNSUPPORTED, "input tensor too large for 32-bit element offsets");
-    L.var = ConvVariant{in.f16, out.f16, split ? 1 : 0, tc.fm, tc.fn, tc.wm, tc.wn, kc, 2};
+    L.var = ConvVariant{in.f16, out.f16, split ? 1 : 0, tc.fm, tc.fn, tc.wm, tc.wn, kc, 2, 2};
 
     // k16 steps
     if (kc == 4) {
@@ -241,6 +241,7 @@ static MfmaLaunch plan_mfma(Net* net, const SubConv& sc, const TView& in, const 
         if (kc == 32) pd = (raw % 6 == 0) ? 6 : ((raw % 4 == 0) ? 4 : 2);
         if (const char* e = getenv("FYNHIP_CONV_PD")) pd = atoi(e);
         L.var.pd = pd;
+        L.var.unr = (pd == 6 && raw == 18 && !getenv("FYNHIP_CONV_NO_FULL_UNROLL")) ? 18 : pd;
         if (!conv_mfma_variant_exists(L.var)) fail(FYN_ERR_UNSUPPORTED, "MFMA convolution variant not compiled");
     }
     while (L.steps.size() % conv_mfma_step_multiple(L.var) != 0) {
