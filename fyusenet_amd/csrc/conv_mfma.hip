@@ -276,7 +276,7 @@ __global__ __launch_bounds__((FM * FN >= 2) ? 512 : 256) void conv_mfma_kernel(c
     // ---- staging machinery: items (pixel, 8-channel group) of the halo tile; the first NB items of a
     //      thread are described once (their addresses only shift by the chunk's channel offset) and
     //      are fetched for chunk c+1 while the MFMAs of chunk c run ----
-    constexpr int NB = 4;
+    constexpr int NB = (KC >= 64) ? 8 : 4;
     int g_off[NB];   // element offset of the pixel in the input tensor, -1: outside (reads as 0)
     int l_off[NB];   // LDS byte offset inside a plane, -1: no such item
     int c_off[NB];   // channel offset of the group inside a chunk
@@ -577,8 +577,9 @@ typedef void (*conv_kernel_fn)(const ConvMfmaParams);
     X(12, 1, 4, 2, 2)     \
     X(13, 1, 3, 2, 2)
 
-// (ring depth, unroll) pairs: 2/2 for every chunk width; for 32-channel chunks also 4/4, 6/6 and 6/18 (a whole
-// 3x3 chunk unrolled: no loop back-edge, hence no conservative wait, inside a chunk).
+// (ring depth, unroll) pairs: 2/2 for chunks of 4, 16 and 32 channels; for 32-channel chunks also 4/4, 6/6 and
+// 6/18 (a whole 3x3 chunk unrolled: no loop back-edge, hence no conservative wait, inside a chunk); 64- and
+// 128-channel chunks (kernels of one to four taps: fewer chunk barriers) use 4/4 and 4/8.
 template <typename TIn, typename TOut, bool SPLIT, int FM, int FN, int WM, int WN>
 static conv_kernel_fn pick_kc(int kc, int pd, int unr) {
     if (kc == 4 && pd == 2 && unr == 2) return conv_mfma_kernel<TIn, TOut, SPLIT, FM, FN, WM, WN, 4, 2, 2>;
@@ -587,6 +588,8 @@ static conv_kernel_fn pick_kc(int kc, int pd, int unr) {
     if (kc == 32 && pd == 4 && unr == 4) return conv_mfma_kernel<TIn, TOut, SPLIT, FM, FN, WM, WN, 32, 4, 4>;
     if (kc == 32 && pd == 6 && unr == 6) return conv_mfma_kernel<TIn, TOut, SPLIT, FM, FN, WM, WN, 32, 6, 6>;
     if (kc == 32 && pd == 6 && unr == 18) return conv_mfma_kernel<TIn, TOut, SPLIT, FM, FN, WM, WN, 32, 6, 18>;
+    if (kc == 64 && pd == 4 && unr == 4) return conv_mfma_kernel<TIn, TOut, SPLIT, FM, FN, WM, WN, 64, 4, 4>;
+    if (kc == 128 && pd == 4 && unr == 8) return conv_mfma_kernel<TIn, TOut, SPLIT, FM, FN, WM, WN, 128, 4, 8>;
     return nullptr;
 }
 

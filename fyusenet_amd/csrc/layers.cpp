@@ -104,6 +104,7 @@ struct TileChoice {
     int fm, fn, wm, wn, twl, th;
     double score;
     int rowpad;  // bytes added to each staged pixel row in LDS
+    int kc;      // input channels per staged chunk
 };
 
 // All tile configurations that fit, best heuristic score first.
@@ -133,17 +134,24 @@ static std::vector<TileChoice> enumerate_tiles(int cout, const SubConv& sc, int 
         const double slots = 256.0 * (lds > 72 * 1024 ? 1 : 2);
         const double par = blocks >= slots ? blocks / (std::ceil(blocks / slots) * slots) : blocks / slots;
         const double bonus = (fm * fn == 4) ? 1.0 : (fm * fn == 2 ? 0.85 : 0.7);
-        all.push_back(TileChoice{fm, fn, wm, wn, ilog2(tw), th, util * par * bonus, rowpad});
+        all.push_back(TileChoice{fm, fn, wm, wn, ilog2(tw), th, util * par * bonus, rowpad, 0});
     }
     if (all.empty()) fail(FYN_ERR_UNSUPPORTED, "no MFMA tile configuration fits this convolution");
     std::sort(all.begin(), all.end(), [](const TileChoice& x, const TileChoice& y) { return x.score > y.score; });
     return all;
 }
 
-static void conv_geometry(const TView& in, bool split, int& kc, int& pitch, int& slack, int& npl) {
+// kc_force > 0 selects the chunk width, 0 the default for the geometry.
+static void conv_geometry(const TView& in, bool split, int ntaps, int kc_force, int& kc, int& pitch, int& slack, int& npl) {
+    // input channels staged per chunk: kernels with few taps take wide chunks (fewer barriers per output)
+    const char* kmax = getenv("FYNHIP_CONV_KC_MAX");
+    const int cap = kmax ? atoi(kmax) : 128;
     if (in.cp == 4) kc = 4;
     else if (in.cp <= 16) kc = 16;
+    else if (ntaps <= 2 && in.cp >= 128 && cap >= 128) kc = 128;
+    else if (ntaps <= 4 && in.cp >= 64 && cap >= 64) kc = 64;
     else kc = 32;
+    if (kc_force > 0) kc = kc_force;
     pitch = (kc == 4) ? 8 : kc * 2 + 16;
     slack = (kc == 4) ? 64 : 0;
     npl = split ? 2 : 1;
@@ -160,7 +168,7 @@ static MfmaLaunch plan_mfma(Net* net, const SubConv& sc, const TView& in, const 
     L.cout = cout;
     const bool split = !net->f16();
     int kc, pitch, slack, npl;
-    conv_geometry(in, split, kc, pitch, slack, npl);
+    conv_geometry(in, split, (int)sc.taps.size(), tc.kc, kc, pitch, slack, npl);
     const int tw = 1 << tc.twl;
     ConvMfmaParams& p = L.p;
     p.in = in.ptr;
@@ -239,9 +247,11 @@ static MfmaLaunch plan_mfma(Net* net, const SubConv& sc, const TView& in, const 
         const int raw = (int)L.steps.size();
         int pd = 2;
         if (kc == 32) pd = (raw % 6 == 0) ? 6 : ((raw % 4 == 0) ? 4 : 2);
+        if (kc >= 64) pd = 4;
         if (const char* e = getenv("FYNHIP_CONV_PD")) pd = atoi(e);
         L.var.pd = pd;
         L.var.unr = (pd == 6 && raw == 18 && !getenv("FYNHIP_CONV_NO_FULL_UNROLL")) ? 18 : pd;
+        if (kc == 128) L.var.unr = 8;
         if (!conv_mfma_variant_exists(L.var)) fail(FYN_ERR_UNSUPPORTED, "MFMA convolution variant not compiled");
     }
     while (L.steps.size() % conv_mfma_step_multiple(L.var) != 0) {
@@ -257,13 +267,14 @@ static MfmaLaunch plan_mfma(Net* net, const SubConv& sc, const TView& in, const 
     L.aoff_dev = upload(net, aoff);
     p.aoff = L.aoff_dev;
     L.wpack_halves = (size_t)p.cin_chunks * p.nsteps * p.mfrags * npl * 64 * 8;
-    // the buffer is sized for any step padding (groups of up to 12), so that tile candidates can share it
-    L.wpack_alloc = (size_t)p.cin_chunks * ((p.nsteps + 11) / 12 * 12 + 12) * p.mfrags * npl * 64 * 8;
-    if (share) {
-        if (share->wpack_alloc < L.wpack_halves) fail(FYN_ERR_INVALID, "internal: weight layouts of tile candidates differ");
+    // the buffer is sized generously (any step padding, any chunk width, the prefetch slack behind the last
+    // step), so that tuning candidates can share it
+    const size_t slack_halves = (size_t)16 * p.mfrags * npl * 64 * 8;
+    if (share && share->wpack_alloc >= L.wpack_halves + slack_halves) {
         L.wpack_dev = share->wpack_dev;
         L.wpack_alloc = share->wpack_alloc;
     } else {
+        L.wpack_alloc = 2 * L.wpack_halves + 4 * slack_halves;
         L.wpack_dev = net->dev_alloc(L.wpack_alloc * 2, true);
     }
     p.wpack = L.wpack_dev;
@@ -289,9 +300,9 @@ static float time_launch(Net* net, const MfmaLaunch& L, int iters) {
     return ms / iters;
 }
 
-// ---- optional on-disk memory of tuning results (text: "<key> fm fn wm wn" per line) ----
-static std::map<std::string, std::array<int, 4>>& tune_cache() {
-    static std::map<std::string, std::array<int, 4>> cache;
+// ---- optional on-disk memory of tuning results (text: "<key> fm fn wm wn kc" per line) ----
+static std::map<std::string, std::array<int, 5>>& tune_cache() {
+    static std::map<std::string, std::array<int, 5>> cache;
     static bool loaded = false;
     if (!loaded) {
         loaded = true;
@@ -299,8 +310,8 @@ static std::map<std::string, std::array<int, 4>>& tune_cache() {
         FILE* f = path ? fopen(path, "r") : nullptr;
         if (f) {
             char k[160];
-            int a, b, c, d;
-            while (fscanf(f, "%159s %d %d %d %d", k, &a, &b, &c, &d) == 5) cache[k] = {a, b, c, d};
+            int a, b, c, d, e;
+            while (fscanf(f, "%159s %d %d %d %d %d", k, &a, &b, &c, &d, &e) == 6) cache[k] = {a, b, c, d, e};
             fclose(f);
         }
     }
@@ -312,17 +323,17 @@ static const TileChoice* tune_cache_lookup(const char* key, const std::vector<Ti
     auto it = tune_cache().find(key);
     if (it == tune_cache().end()) return nullptr;
     for (const TileChoice& c : cands)
-        if (c.fm == it->second[0] && c.fn == it->second[1] && c.wm == it->second[2] && c.wn == it->second[3]) return &c;
+        if (c.fm == it->second[0] && c.fn == it->second[1] && c.wm == it->second[2] && c.wn == it->second[3] && c.kc == it->second[4]) return &c;
     return nullptr;
 }
 
 static void tune_cache_store(const char* key, const ConvVariant& v) {
     const char* path = getenv("FYNHIP_TUNE_CACHE");
     if (!path) return;
-    tune_cache()[key] = {v.fm, v.fn, v.wm, v.wn};
+    tune_cache()[key] = {v.fm, v.fn, v.wm, v.wn, v.kc};
     FILE* f = fopen(path, "a");
     if (!f) return;
-    fprintf(f, "%s %d %d %d %d\n", key, v.fm, v.fn, v.wm, v.wn);
+    fprintf(f, "%s %d %d %d %d %d\n", key, v.fm, v.fn, v.wm, v.wn, v.kc);
     fclose(f);
 }
 
@@ -330,10 +341,27 @@ static void tune_cache_store(const char* key, const ConvVariant& v) {
 // (default; timing does not depend on the data), or by the heuristic score when FYNHIP_AUTOTUNE=0.
 static MfmaLaunch tune_mfma(Net* net, const SubConv& sc, const TView& in, const TView& out, const TView* res, int cin,
                             int cout, const Act& act, int res_relu, int res_scale, const float* scale, const float* bias) {
-    int kc, pitch, slack, npl;
-    conv_geometry(in, !net->f16(), kc, pitch, slack, npl);
-    const int chunks = (kc == 4) ? 1 : (in.cp + kc - 1) / kc;
-    std::vector<TileChoice> cands = enumerate_tiles(cout, sc, pitch, npl, slack, chunks > 1 ? 2 : 1);
+    // candidates: every tile that fits, for the geometry's default chunk width and, where that is wider
+    // than 32 channels, for 32-channel chunks too
+    std::vector<TileChoice> cands;
+    {
+        int kc0, pitch, slack, npl;
+        conv_geometry(in, !net->f16(), (int)sc.taps.size(), 0, kc0, pitch, slack, npl);
+        std::vector<int> kcs{kc0};
+        if (kc0 > 32) kcs.push_back(32);
+        for (int kco : kcs) {
+            int kc;
+            conv_geometry(in, !net->f16(), (int)sc.taps.size(), kco, kc, pitch, slack, npl);
+            const int chunks = (kc == 4) ? 1 : (in.cp + kc - 1) / kc;
+            std::vector<TileChoice> c = enumerate_tiles(cout, sc, pitch, npl, slack, chunks > 1 ? 2 : 1);
+            for (TileChoice& tc : c) {
+                tc.kc = kc;
+                if (kco != kc0) tc.score *= 0.9;
+                cands.push_back(tc);
+            }
+        }
+        std::stable_sort(cands.begin(), cands.end(), [](const TileChoice& x, const TileChoice& y) { return x.score > y.score; });
+    }
     const char* at = getenv("FYNHIP_AUTOTUNE");
     const bool tune = !(at && at[0] == '0') && cands.size() > 1;
     // FYNHIP_TUNE_CACHE=<file>: measured choices are remembered per problem geometry, so that later
