@@ -201,6 +201,9 @@ __global__ __launch_bounds__((FM * FN >= 2) ? 512 : 256) void conv_mfma_kernel(c
         const int per = gridDim.x >> 3;
         if (bid < (per << 3)) bid = (bid & 7) * per + (bid >> 3);
     }
+    const int ntile_blocks = p.tiles_x * p.tiles_y * p.cout_blocks;
+    const int ks = bid / ntile_blocks;           // split-K slice (0 without split-K)
+    bid -= ks * ntile_blocks;
     const int cb = bid % p.cout_blocks;
     const int tile = bid / p.cout_blocks;
     const int tyi = tile / p.tiles_x;
@@ -241,9 +244,12 @@ __global__ __launch_bounds__((FM * FN >= 2) ? 512 : 256) void conv_mfma_kernel(c
     // (uniform base + per-lane 32-bit offset: the loads use the scalar-base addressing form and stepping
     // through K costs two scalar adds; the buffer has PD steps of zero slack behind the last step, so the
     // prefetch needs no clamp)
-    const unsigned char* wbase = reinterpret_cast<const unsigned char*>(p.wpack) + (size_t)((cb * WM + wm) * FM) * NPL * 1024;
-    const unsigned wlane = lane * 16;
     const unsigned wstep = (unsigned)p.mfrags * NPL * 1024;   // bytes per k16 step
+    const int chunk0 = ks * p.chunks_per_split;                // this workgroup's channel chunks: [chunk0, chunk1)
+    const int chunk1 = (chunk0 + p.chunks_per_split < p.cin_chunks) ? chunk0 + p.chunks_per_split : p.cin_chunks;
+    const unsigned char* wbase = reinterpret_cast<const unsigned char*>(p.wpack) + (size_t)((cb * WM + wm) * FM) * NPL * 1024 +
+                                 (size_t)chunk0 * p.nsteps * wstep;
+    const unsigned wlane = lane * 16;
 
     float16_t acc[FM][FN];
 #pragma unroll
@@ -355,9 +361,9 @@ __global__ __launch_bounds__((FM * FN >= 2) ? 512 : 256) void conv_mfma_kernel(c
 
     // prologue: chunk 0 into buffer 0
     if (stager) {
-        fetch_first(0);
-        store_first(0, sbase);
-        stage_rest(0, sbase);
+        fetch_first(chunk0);
+        store_first(chunk0, sbase);
+        stage_rest(chunk0, sbase);
     }
     __syncthreads();
     FYN_TRACE(1);
@@ -412,8 +418,8 @@ __global__ __launch_bounds__((FM * FN >= 2) ? 512 : 256) void conv_mfma_kernel(c
             }
         }
     };
-    for (int chunk = 0; chunk < p.cin_chunks; chunk++) {
-        const bool more_chunks = chunk + 1 < p.cin_chunks;
+    for (int chunk = chunk0; chunk < chunk1; chunk++) {
+        const bool more_chunks = chunk + 1 < chunk1;
         // (after the last chunk the fetch is unused; it keeps the number of loads in flight static)
         if (stager) fetch_first(more_chunks ? chunk + 1 : chunk);
         if (consumer) {
@@ -424,16 +430,16 @@ __global__ __launch_bounds__((FM * FN >= 2) ? 512 : 256) void conv_mfma_kernel(c
                 for (int pl = 0; pl < NPL; pl++) b_buf[0][fn][pl] = load_b_frag<KC>(cur + pl * p.plane + (boff[fn] + ao));
             for (int t0 = 0; t0 < p.nsteps; t0 += UNR) run_group(t0);
         }
-        FYN_TRACE(2 + 2 * chunk);
+        FYN_TRACE(2 + 2 * (chunk - chunk0));
         if (more_chunks) {
-            unsigned char* nxt = sbase + ((chunk + 1) & 1) * bufsz;
+            unsigned char* nxt = sbase + ((chunk - chunk0 + 1) & 1) * bufsz;
             if (stager) {
                 store_first(chunk + 1, nxt);
                 stage_rest(chunk + 1, nxt);
             }
             __syncthreads();  // everyone is done reading `cur` and writing `nxt`
             cur = nxt;
-            FYN_TRACE(3 + 2 * chunk);
+            FYN_TRACE(3 + 2 * (chunk - chunk0));
         }
     }
 
@@ -462,6 +468,33 @@ __global__ __launch_bounds__((FM * FN >= 2) ? 512 : 256) void conv_mfma_kernel(c
     // Phases instead of a per-fragment round trip (one wave per SIMD cannot hide latencies behind other
     // waves): (1) all residual loads, (2) all accumulators into LDS, (3) all rows back, (4) arithmetic and
     // stores.
+    if (p.ksplit > 1) {
+        // split-K: raw partial sums, [ks][position][cout_pad] fp32; the reduce pass finishes the layer
+        float* part = p.partial + (size_t)ks * p.npos_y * p.npos_x * p.cout_pad;
+        const bool cp_ok = c < p.cout_pad;
+#pragma unroll
+        for (int fn = 0; fn < FN; fn++) {
+#pragma unroll
+            for (int fm = 0; fm < FM; fm++)
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    f32x4_t v;
+                    v[0] = acc[fm][fn][q * 4 + 0]; v[1] = acc[fm][fn][q * 4 + 1];
+                    v[2] = acc[fm][fn][q * 4 + 2]; v[3] = acc[fm][fn][q * 4 + 3];
+                    *reinterpret_cast<f32x4_t*>(tr + (fn * 32 + (lane & 31)) * ROWF + fm * 32 + q * 8 + (lane >> 5) * 4) = v;
+                }
+#pragma unroll
+            for (int it = 0; it < 32 / PPI; it++) {
+                const int row = it * PPI + lane / LPP;
+                const f32x4_t v = *reinterpret_cast<const f32x4_t*>(tr + (fn * 32 + row) * ROWF + c4);
+                const int m = (wn * FN + fn) * 32 + row;
+                const int py = pos_y0 + (m >> twl), px = pos_x0 + (m & (TW - 1));
+                if (cp_ok && py < p.npos_y && px < p.npos_x)
+                    *reinterpret_cast<f32x4_t*>(part + ((size_t)py * p.npos_x + px) * p.cout_pad + c) = v;
+            }
+        }
+        return;
+    }
     // Row r of a fragment is position m = frag*32 + it*PPI + lane/LPP; PPI divides the tile width, so the
     // tile row (and with it the image row) of an (fn, it) pair is wave-uniform and only the column carries a
     // per-lane part: base addresses are scalar, the per-lane offset is computed once.
@@ -694,7 +727,9 @@ int launch_conv_mfma(const ConvVariant& v, const ConvMfmaParams& p, size_t lds_b
             cur = lds_bytes;
         }
     }
-    const int blocks = p.tiles_x * p.tiles_y * p.cout_blocks;
+    const int blocks = p.tiles_x * p.tiles_y * p.cout_blocks * (p.ksplit > 1 ? p.ksplit : 1);
+    if (p.ksplit > 1 && (!p.partial || p.chunks_per_split < 1 || (p.ksplit - 1) * p.chunks_per_split >= p.cin_chunks)) return -7;
+    if (p.ksplit <= 1 && p.chunks_per_split < p.cin_chunks) return -7;
 #ifdef FYN_CONV_TRACE
     static long long* trace_dev = nullptr;
     if (!trace_dev && hipMalloc(&trace_dev, sizeof(long long) * 16 * 65536) != hipSuccess) return -6;

@@ -67,6 +67,12 @@ struct ConvMfmaParams {
     int mfrags;          // cout fragments (32 each) in wpack
     int cout_blocks;     // grid size along cout
     float acc_mul;       // exact power of two undoing the weight pre-scaling
+    // split-K: the grid holds ksplit copies of the (tile, cout block) set; copy ks reduces the channel chunks
+    // [ks*chunks_per_split, (ks+1)*chunks_per_split) and writes raw fp32 partial sums, [ks][position][cout_pad],
+    // which splitk_reduce sums and finishes (scale, bias, residual).  ksplit == 1: no partials.
+    int ksplit, chunks_per_split;
+    float* partial;
+    int cout_pad;
 #ifdef FYN_CONV_TRACE
     long long* trace;    // timing-study builds only: 16 timestamps per workgroup
 #endif
@@ -156,6 +162,22 @@ struct ShiftReduceParams {
     int res_relu, res_scale;
 };
 void launch_shift_reduce(const ShiftReduceParams& p, hipStream_t s);
+
+// Second pass of a split-K convolution: out = (sum_ks partial[ks]) * acc_mul * scale + bias (+ residual).
+struct SplitKReduceParams {
+    const float* partial;      // [ksplit][npos_y * npos_x][cout_pad]
+    int ksplit, npos_y, npos_x, cout_pad;
+    void* out;                 // engine tensor; same addressing fields as ConvMfmaParams
+    const void* res;
+    int out_f16;
+    int out_wp, out_cp, out_step, out_off_y, out_off_x;
+    int res_wp, res_cp, res_off_y, res_off_x;
+    int res_relu, res_scale;
+    float acc_mul;
+    const float* scale;
+    const float* bias;
+};
+void launch_splitk_reduce(const SplitKReduceParams& p, hipStream_t s);
 
 struct GemvParams {
     TView in, out;       // 1x1 spatial

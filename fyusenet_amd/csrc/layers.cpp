@@ -97,6 +97,7 @@ struct MfmaLaunch {
     int* aoff_dev = nullptr;
     size_t wpack_halves = 0;  // halves used by this launch's layout
     size_t wpack_alloc = 0;   // halves allocated
+    SplitKReduceParams red{};  // second pass when p.ksplit > 1
     int cin = 0, cout = 0;
 };
 
@@ -200,6 +201,9 @@ static MfmaLaunch plan_mfma(Net* net, const SubConv& sc, const TView& in, const 
     p.bias = bias;
     p.acc_mul = 1.f;
     p.act = act;
+    p.ksplit = 1;
+    p.partial = nullptr;
+    p.cout_pad = out.cp;
     L.lds = 1024 + (size_t)npl * p.plane * (p.cin_chunks > 1 ? 2 : 1);  // step table + tiles (double-buffered across chunks)
     L.lds = std::max(L.lds, (size_t)4 * tc.fn * 32 * (tc.fm * 32 + 4) * 4);  // epilogue transposition area (all waves, all fragments)
     if (in.elems() >= (size_t)1 << 31) fail(FYN_ERR_UNSUPPORTED, "input tensor too large for 32-bit element offsets");
@@ -278,18 +282,49 @@ static MfmaLaunch plan_mfma(Net* net, const SubConv& sc, const TView& in, const 
         L.wpack_dev = net->dev_alloc(L.wpack_alloc * 2, true);
     }
     p.wpack = L.wpack_dev;
+    p.chunks_per_split = p.cin_chunks;
     return L;
 }
 
 static std::string mfma_info(const MfmaLaunch& L);
 
+// Launches a planned (sub-)convolution: the MFMA kernel and, with split-K, the reduce pass.
+static int run_mfma(const MfmaLaunch& L, hipStream_t s) {
+    const int rc = launch_conv_mfma(L.var, L.p, L.lds, s);
+    if (rc != 0) return rc;
+    if (L.p.ksplit > 1) launch_splitk_reduce(L.red, s);
+    return 0;
+}
+
+// Turns a planned launch into its split-K form (ksplit slices over the input-channel chunks).
+static void set_ksplit(Net* net, MfmaLaunch& L, int ksplit) {
+    ConvMfmaParams& p = L.p;
+    if (ksplit <= 1) {
+        p.ksplit = 1;
+        p.chunks_per_split = p.cin_chunks;
+        p.partial = nullptr;
+        return;
+    }
+    p.ksplit = ksplit;
+    p.chunks_per_split = (p.cin_chunks + ksplit - 1) / ksplit;
+    const size_t floats = (size_t)ksplit * p.npos_y * p.npos_x * p.cout_pad;
+    p.partial = reinterpret_cast<float*>(net->dev_alloc(floats * sizeof(float), true));
+    SplitKReduceParams& r = L.red;
+    r.partial = p.partial; r.ksplit = ksplit; r.npos_y = p.npos_y; r.npos_x = p.npos_x; r.cout_pad = p.cout_pad;
+    r.out = p.out; r.res = p.res; r.out_f16 = L.var.out_f16;
+    r.out_wp = p.out_wp; r.out_cp = p.out_cp; r.out_step = p.out_step; r.out_off_y = p.out_off_y; r.out_off_x = p.out_off_x;
+    r.res_wp = p.res_wp; r.res_cp = p.res_cp; r.res_off_y = p.res_off_y; r.res_off_x = p.res_off_x;
+    r.res_relu = p.res_relu; r.res_scale = p.res_scale;
+    r.acc_mul = p.acc_mul; r.scale = p.scale; r.bias = p.bias;
+}
+
 static float time_launch(Net* net, const MfmaLaunch& L, int iters) {
     hipEvent_t a, b;
     FYN_HIP(hipEventCreate(&a));
     FYN_HIP(hipEventCreate(&b));
-    if (launch_conv_mfma(L.var, L.p, L.lds, net->stream) != 0) fail(FYN_ERR_DEVICE, "convolution launch failed while tuning");
+    if (run_mfma(L, net->stream) != 0) fail(FYN_ERR_DEVICE, "convolution launch failed while tuning");
     FYN_HIP(hipEventRecord(a, net->stream));
-    for (int i = 0; i < iters; i++) launch_conv_mfma(L.var, L.p, L.lds, net->stream);
+    for (int i = 0; i < iters; i++) run_mfma(L, net->stream);
     FYN_HIP(hipEventRecord(b, net->stream));
     FYN_HIP(hipEventSynchronize(b));
     FYN_HIP(hipGetLastError());
@@ -300,9 +335,9 @@ static float time_launch(Net* net, const MfmaLaunch& L, int iters) {
     return ms / iters;
 }
 
-// ---- optional on-disk memory of tuning results (text: "<key> fm fn wm wn kc" per line) ----
-static std::map<std::string, std::array<int, 5>>& tune_cache() {
-    static std::map<std::string, std::array<int, 5>> cache;
+// ---- optional on-disk memory of tuning results (text: "<key> fm fn wm wn kc ksplit" per line) ----
+static std::map<std::string, std::array<int, 6>>& tune_cache() {
+    static std::map<std::string, std::array<int, 6>> cache;
     static bool loaded = false;
     if (!loaded) {
         loaded = true;
@@ -310,30 +345,33 @@ static std::map<std::string, std::array<int, 5>>& tune_cache() {
         FILE* f = path ? fopen(path, "r") : nullptr;
         if (f) {
             char k[160];
-            int a, b, c, d, e;
-            while (fscanf(f, "%159s %d %d %d %d %d", k, &a, &b, &c, &d, &e) == 6) cache[k] = {a, b, c, d, e};
+            int a, b, c, d, e, g;
+            while (fscanf(f, "%159s %d %d %d %d %d %d", k, &a, &b, &c, &d, &e, &g) == 7) cache[k] = {a, b, c, d, e, g};
             fclose(f);
         }
     }
     return cache;
 }
 
-static const TileChoice* tune_cache_lookup(const char* key, const std::vector<TileChoice>& cands) {
+static const TileChoice* tune_cache_lookup(const char* key, const std::vector<TileChoice>& cands, int* ksplit) {
     if (!getenv("FYNHIP_TUNE_CACHE")) return nullptr;
     auto it = tune_cache().find(key);
     if (it == tune_cache().end()) return nullptr;
     for (const TileChoice& c : cands)
-        if (c.fm == it->second[0] && c.fn == it->second[1] && c.wm == it->second[2] && c.wn == it->second[3] && c.kc == it->second[4]) return &c;
+        if (c.fm == it->second[0] && c.fn == it->second[1] && c.wm == it->second[2] && c.wn == it->second[3] && c.kc == it->second[4]) {
+            *ksplit = it->second[5];
+            return &c;
+        }
     return nullptr;
 }
 
-static void tune_cache_store(const char* key, const ConvVariant& v) {
+static void tune_cache_store(const char* key, const ConvVariant& v, int ksplit) {
     const char* path = getenv("FYNHIP_TUNE_CACHE");
     if (!path) return;
-    tune_cache()[key] = {v.fm, v.fn, v.wm, v.wn, v.kc};
+    tune_cache()[key] = {v.fm, v.fn, v.wm, v.wn, v.kc, ksplit};
     FILE* f = fopen(path, "a");
     if (!f) return;
-    fprintf(f, "%s %d %d %d %d %d\n", key, v.fm, v.fn, v.wm, v.wn, v.kc);
+    fprintf(f, "%s %d %d %d %d %d %d\n", key, v.fm, v.fn, v.wm, v.wn, v.kc, ksplit);
     fclose(f);
 }
 
@@ -370,8 +408,13 @@ static MfmaLaunch tune_mfma(Net* net, const SubConv& sc, const TView& in, const 
     snprintf(key, sizeof(key), "%d%d:%dx%d:%dx%d:s%d:t%zu:%dx%d:o%d:r%d:cp%d", in.f16, out.f16, cin, cout, sc.npos_y, sc.npos_x,
              sc.in_stride, sc.taps.size(), sc.span_y, sc.span_x, sc.out_step, res ? 1 : 0, in.cp);
     if (tune) {
-        const TileChoice* hit = tune_cache_lookup(key, cands);
-        if (hit) return plan_mfma(net, sc, in, out, res, cin, cout, act, res_relu, res_scale, *hit, scale, bias);
+        int ks = 1;
+        const TileChoice* hit = tune_cache_lookup(key, cands, &ks);
+        if (hit) {
+            MfmaLaunch L = plan_mfma(net, sc, in, out, res, cin, cout, act, res_relu, res_scale, *hit, scale, bias);
+            set_ksplit(net, L, ks);
+            return L;
+        }
     }
     MfmaLaunch best = plan_mfma(net, sc, in, out, res, cin, cout, act, res_relu, res_scale, cands[0], scale, bias);
     if (!tune) return best;
@@ -387,7 +430,23 @@ static MfmaLaunch tune_mfma(Net* net, const SubConv& sc, const TView& in, const 
             best = L;
         }
     }
-    tune_cache_store(key, best.var);
+    // few workgroups and several channel chunks: try splitting the reduction over more workgroups
+    {
+        const int blocks = best.p.tiles_x * best.p.tiles_y * best.p.cout_blocks;
+        for (int ks = 2; ks <= 16 && blocks < 192; ks *= 2) {
+            const int cps = (best.p.cin_chunks + ks - 1) / ks;
+            if (best.p.cin_chunks < 2 || (ks - 1) * cps >= best.p.cin_chunks || blocks * ks > 1024) break;
+            MfmaLaunch L = best;
+            set_ksplit(net, L, ks);
+            const float ms = std::min(time_launch(net, L, 4), time_launch(net, L, 4));
+            if (verbose) fprintf(stderr, "[tune] %s -> %.1f us\n", mfma_info(L).c_str(), ms * 1e3f);
+            if (ms < best_ms) {
+                best_ms = ms;
+                best = L;
+            }
+        }
+    }
+    tune_cache_store(key, best.var, best.p.ksplit);
     return best;
 }
 
@@ -438,9 +497,9 @@ static float weight_prescale(const float* w, size_t n) {
 
 static std::string mfma_info(const MfmaLaunch& L) {
     char buf[256];
-    snprintf(buf, sizeof(buf), "conv_mfma %s tile=%dx%d(cout x pos) waves=%dx%d kc=%d th=%d tw=%d blocks=%d lds=%zu steps=%d chunks=%d",
+    snprintf(buf, sizeof(buf), "conv_mfma %s tile=%dx%d(cout x pos) waves=%dx%d kc=%d th=%d tw=%d blocks=%d lds=%zu steps=%d chunks=%d ksplit=%d",
              L.var.split ? "f16x2-split" : "f16", L.var.wm * L.var.fm * 32, L.var.wn * L.var.fn * 32, L.var.wm, L.var.wn, L.var.kc,
-             L.p.tile_h, 1 << L.p.tile_w_log2, L.p.tiles_x * L.p.tiles_y * L.p.cout_blocks, L.lds, L.p.nsteps, L.p.cin_chunks);
+             L.p.tile_h, 1 << L.p.tile_w_log2, L.p.tiles_x * L.p.tiles_y * L.p.cout_blocks, L.lds, L.p.nsteps, L.p.cin_chunks, L.p.ksplit);
     return buf;
 }
 
@@ -571,11 +630,13 @@ class ConvLayer : public Layer {
             reupload(net, q_scale_dev, ones);
             reupload(net, q_bias_dev, zeros);
             launch.p.acc_mul = 1.0f;         // the pre-scaling is undone in the second stage
+            launch.red.acc_mul = 1.0f;
             sr.acc_mul = 1.0f / wmul;
             pack_mfma_weights(net, launch, wv.data(), k, wmul, 1);
         } else {
             const float wmul = weight_prescale(w, (size_t)oc * k * k * d.in_channels);
             launch.p.acc_mul = 1.0f / wmul;
+            launch.red.acc_mul = 1.0f / wmul;
             pack_mfma_weights(net, launch, w, k, wmul);
         }
         have_weights = true;
@@ -583,7 +644,7 @@ class ConvLayer : public Layer {
     void forward(hipStream_t s) override {
         if (!have_weights) fail(FYN_ERR_STATE, "layer %s (%d): forward() without weights", d.name, d.number);
         if (direct) launch_conv_direct(dp, s);
-        else if (launch_conv_mfma(launch.var, launch.p, launch.lds, s) != 0)
+        else if (run_mfma(launch, s) != 0)
             fail(FYN_ERR_DEVICE, "layer %s: convolution launch failed", d.name);
         if (wide) launch_shift_reduce(sr, s);
     }
@@ -729,6 +790,7 @@ class TransConvLayer : public Layer {
         const float wmul = weight_prescale(w, (size_t)oc * k * k * d.in_channels);
         for (auto& L : launches) {
             L.p.acc_mul = 1.0f / wmul;
+            L.red.acc_mul = 1.0f / wmul;
             pack_mfma_weights(net, L, w, k, wmul);
         }
         have_weights = true;
@@ -736,7 +798,7 @@ class TransConvLayer : public Layer {
     void forward(hipStream_t s) override {
         if (!have_weights) fail(FYN_ERR_STATE, "layer %s (%d): forward() without weights", d.name, d.number);
         for (auto& L : launches)
-            if (launch_conv_mfma(L.var, L.p, L.lds, s) != 0) fail(FYN_ERR_DEVICE, "layer %s: transposed convolution launch failed", d.name);
+            if (run_mfma(L, s) != 0) fail(FYN_ERR_DEVICE, "layer %s: transposed convolution launch failed", d.name);
     }
     std::string info() const override { return launches.empty() ? "transconv" : "transconv 4x " + mfma_info(launches[0]); }
     int k, crop;

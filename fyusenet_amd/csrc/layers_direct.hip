@@ -13,6 +13,7 @@
 namespace fynhip {
 
 typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 
 __device__ __forceinline__ float act1(float x, const Act& a) {
@@ -577,6 +578,48 @@ void launch_fill_zero(void* ptr, size_t bytes, hipStream_t s) {
     if (blocks == 0) blocks = 1;
     hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)blocks), dim3(256), 0, s, reinterpret_cast<uint4*>(ptr), n16,
                        reinterpret_cast<unsigned char*>(ptr) + n16 * 16, bytes - n16 * 16);
+}
+
+// Second pass of a split-K convolution (see ConvMfmaParams::ksplit): one thread per (position, 4 channels).
+template <typename TOut>
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const SplitKReduceParams p) {
+    const int cq = p.cout_pad >> 2;
+    const size_t n = (size_t)p.npos_y * p.npos_x * cq;
+    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= n) return;
+    const int c = (int)(idx % cq) * 4;
+    const size_t pos = idx / cq;
+    const int py = (int)(pos / p.npos_x), px = (int)(pos - (size_t)py * p.npos_x);
+    const size_t slice = (size_t)p.npos_y * p.npos_x * p.cout_pad;
+    f32x4 a = (f32x4)(0.f);
+    for (int ks = 0; ks < p.ksplit; ks++) a += *reinterpret_cast<const f32x4*>(p.partial + ks * slice + pos * p.cout_pad + c);
+    if (c >= p.out_cp) return;
+    const f32x4 sc = *reinterpret_cast<const f32x4*>(p.scale + c), bi = *reinterpret_cast<const f32x4*>(p.bias + c);
+    float o[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) o[i] = (a[i] * p.acc_mul) * sc[i] + bi[i];
+    if (p.res) {
+        const TOut* res = reinterpret_cast<const TOut*>(p.res);
+        const size_t rbase = ((size_t)(p.res_off_y + py * p.out_step) * p.res_wp + p.res_off_x + px * p.out_step) * p.res_cp + c;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            float rv = (float)res[rbase + i];
+            if (p.res_relu) rv = fmaxf(rv, 0.f);
+            if (p.res_scale) rv *= sc[i];
+            o[i] += rv;
+        }
+    }
+    TOut* out = reinterpret_cast<TOut*>(p.out);
+    const size_t obase = ((size_t)(p.out_off_y + py * p.out_step) * p.out_wp + p.out_off_x + px * p.out_step) * p.out_cp + c;
+#pragma unroll
+    for (int i = 0; i < 4; i++) out[obase + i] = (TOut)o[i];
+}
+
+void launch_splitk_reduce(const SplitKReduceParams& p, hipStream_t s) {
+    const size_t n = (size_t)p.npos_y * p.npos_x * (p.cout_pad >> 2);
+    const unsigned blocks = (unsigned)((n + 255) / 256);
+    if (p.out_f16) hipLaunchKernelGGL(splitk_reduce_kernel<_Float16>, dim3(blocks), dim3(256), 0, s, p);
+    else hipLaunchKernelGGL(splitk_reduce_kernel<float>, dim3(blocks), dim3(256), 0, s, p);
 }
 
 }  // namespace fynhip
