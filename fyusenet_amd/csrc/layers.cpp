@@ -417,6 +417,12 @@ static MfmaLaunch tune_mfma(Net* net, const SubConv& sc, const TView& in, const 
         }
     }
     MfmaLaunch best = plan_mfma(net, sc, in, out, res, cin, cout, act, res_relu, res_scale, cands[0], scale, bias);
+    if (const char* fk = getenv("FYNHIP_FORCE_KSPLIT")) {   // testing: fixed split-K factor (clamped to what the layer allows)
+        int ks = atoi(fk);
+        while (ks > 1 && (ks - 1) * ((best.p.cin_chunks + ks - 1) / ks) >= best.p.cin_chunks) ks--;
+        set_ksplit(net, best, ks);
+        return best;
+    }
     if (!tune) return best;
     const bool verbose = getenv("FYNHIP_TUNE_VERBOSE") != nullptr;
     float best_ms = std::min(time_launch(net, best, 4), time_launch(net, best, 4));

@@ -72,6 +72,34 @@ def test_conv_parity(case, storage):
     assert err <= TOL[storage], info
 
 
+@pytest.mark.parametrize("storage", [fa.STORAGE_F32, fa.STORAGE_F16], ids=["f32", "f16"])
+@pytest.mark.parametrize("k,cin,cout,size,ksplit,kcmax,kw", [
+    (1, 512, 128, 14, 4, 128, {"bn": True}),                                   # 128-channel chunks, 4 slices
+    (1, 192, 64, 9, 2, 128, {}),                                               # ragged last chunk (192 = 128 + 64)
+    (3, 256, 256, 7, 8, 32, {"bn": True, "residual": (A.RELU, True)}),         # residual applied by the reduce pass
+    (3, 96, 40, 13, 3, 32, {}),                                                # uneven slices (3 chunks over 3), cout not a tile multiple
+    (1, 320, 100, 7, 1, 128, {}),                                              # wide chunks without split-K
+])
+def test_split_k_and_wide_chunks(k, cin, cout, size, ksplit, kcmax, kw, storage, monkeypatch):
+    """The split-K path (partial sums + reduce pass) and the 64/128-channel chunk variants, forced through the
+    engine's test switches instead of left to the tuner."""
+    monkeypatch.setenv("FYNHIP_FORCE_KSPLIT", str(ksplit))
+    monkeypatch.setenv("FYNHIP_CONV_KC_MAX", str(kcmax))
+    b = conv_builder(k, cout, size, size, cin, 1, 1, A.RELU, **kw)
+    wts = conv_block(300 + k + cin, cout, k, cin, bn=kw.get("bn", False))
+    x = prng.uniform(11 * k + cin, (cin, size, size), -1, 1)
+    inputs = [x]
+    if "residual" in kw:
+        inputs.append(prng.uniform(19, (cout, size, size), -1, 1))
+    got, info = run_single(b, storage, inputs, wts)
+    ref = oracle_single(b, storage, inputs, wts)
+    err = rel_l2(got, ref)
+    print("  ", info, "rel_l2=%.3e" % err, flush=True)
+    if ksplit > 1:
+        assert "ksplit=%d" % ksplit in info
+    assert err <= TOL[storage], info
+
+
 def test_reference_known_answer_patterns_on_gpu():
     # antisymmetric kernel on ones (convlayertests.cpp:242-261) and 1x1 ones (:165-182): exact
     for storage in (fa.STORAGE_F32, fa.STORAGE_F16):
