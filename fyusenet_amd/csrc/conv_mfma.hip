@@ -29,7 +29,7 @@
 // prefetch distance (k16 steps) of the weight fragments, by cout fragments per wave
 // Timing-study builds (-DFYN_CONV_TRACE): wave 0 of every workgroup records the shader clock at phase boundaries.
 #ifdef FYN_CONV_TRACE
-#define FYN_TRACE(slot) do { if (tid == 0 && (slot) < 16) p.trace[(size_t)blockIdx.x * 16 + (slot)] = clock64(); } while (0)
+#define FYN_TRACE(slot) do { if (tid == 0 && (slot) < 16) p.trace[((size_t)blockIdx.y * gridDim.x + blockIdx.x) * 16 + (slot)] = clock64(); } while (0)
 #else
 #define FYN_TRACE(slot) do { } while (0)
 #endif
@@ -171,8 +171,7 @@ __device__ __forceinline__ half8_t load_b_frag(const unsigned char* src) {
 }
 
 template <typename TIn, typename TOut, bool SPLIT, int FM, int FN, int WM, int WN, int KC, int PD, int UNR>
-__global__ __launch_bounds__((FM * FN >= 2) ? 512 : 256) void conv_mfma_kernel(const ConvMfmaParams p) {
-    extern __shared__ __align__(16) unsigned char lds[];
+__device__ __forceinline__ void conv_mfma_body(const ConvMfmaParams& p, unsigned char* lds) {
     // Tiles with two or more fragments per wave run one MFMA wave per SIMD; such workgroups get four more
     // waves (threads 256..511) that do nothing but stage the next input chunk (global loads, activation,
     // fp32 -> fp16 hi/lo conversion, LDS writes), so that this work shares the SIMDs with the MFMA waves
@@ -185,7 +184,6 @@ __global__ __launch_bounds__((FM * FN >= 2) ? 512 : 256) void conv_mfma_kernel(c
     static_assert(WM * WN == 4, "4 waves per block");
 
     const int tid = threadIdx.x;
-    FYN_TRACE(0);
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: keeps tile/fragment index math scalar
     const bool consumer = !SPEC || wave < 4;   // issues MFMAs, owns accumulators, writes the output
@@ -198,9 +196,12 @@ __global__ __launch_bounds__((FM * FN >= 2) ? 512 : 256) void conv_mfma_kernel(c
     // halos, same input tile for all cout blocks) meet in one XCD's L2.
     int bid = blockIdx.x;
     {
-        const int per = gridDim.x >> 3;
+        const int nblk = p.tiles_x * p.tiles_y * p.cout_blocks * (p.ksplit > 1 ? p.ksplit : 1);
+        if (bid >= nblk) return;   // rows are as long as the largest member
+        const int per = nblk >> 3;
         if (bid < (per << 3)) bid = (bid & 7) * per + (bid >> 3);
     }
+    FYN_TRACE(0);
     const int ntile_blocks = p.tiles_x * p.tiles_y * p.cout_blocks;
     const int ks = bid / ntile_blocks;           // split-K slice (0 without split-K)
     bid -= ks * ntile_blocks;
@@ -579,12 +580,31 @@ __global__ __launch_bounds__((FM * FN >= 2) ? 512 : 256) void conv_mfma_kernel(c
     FYN_TRACE(15);
 }
 
+// Entry points: one convolution per launch (parameters by value), or up to four sub-convolutions of one layer
+// per launch (grid row blockIdx.y works on sub[blockIdx.y]; rows are as long as the largest member).
+template <typename TIn, typename TOut, bool SPLIT, int FM, int FN, int WM, int WN, int KC, int PD, int UNR>
+__global__ __launch_bounds__((FM * FN >= 2) ? 512 : 256) void conv_mfma_kernel(const ConvMfmaParams p) {
+    extern __shared__ __align__(16) unsigned char lds[];
+    conv_mfma_body<TIn, TOut, SPLIT, FM, FN, WM, WN, KC, PD, UNR>(p, lds);
+}
+
+template <typename TIn, typename TOut, bool SPLIT, int FM, int FN, int WM, int WN, int KC, int PD, int UNR>
+__global__ __launch_bounds__((FM * FN >= 2) ? 512 : 256) void conv_mfma_multi_kernel(const ConvMfmaMulti P) {
+    extern __shared__ __align__(16) unsigned char lds[];
+    conv_mfma_body<TIn, TOut, SPLIT, FM, FN, WM, WN, KC, PD, UNR>(P.sub[blockIdx.y], lds);
+}
+
 // ---------------------------------------------------------------------------------------------
 // variant table.  This file is compiled FYN_CONV_PARTS times with -DFYN_CONV_PART=0..N-1 (in parallel);
 // every part instantiates the kernels of the tiles whose table index is congruent to it, and part 0
 // also holds the dispatcher.
 // ---------------------------------------------------------------------------------------------
 typedef void (*conv_kernel_fn)(const ConvMfmaParams);
+typedef void (*conv_multi_fn)(const ConvMfmaMulti);
+struct ConvEntry {
+    conv_kernel_fn single = nullptr;
+    conv_multi_fn multi = nullptr;   // may be absent for a variant
+};
 
 #ifndef FYN_CONV_PARTS
 #define FYN_CONV_PARTS 1
@@ -626,30 +646,47 @@ static conv_kernel_fn pick_kc(int kc, int pd, int unr) {
     return nullptr;
 }
 
+// multi-launch entry points exist for 32-, 64- and 128-channel chunks at their smallest step group
+template <typename TIn, typename TOut, bool SPLIT, int FM, int FN, int WM, int WN>
+static conv_multi_fn pick_kc_multi(int kc, int pd, int unr) {
+    if (kc == 32 && pd == 2 && unr == 2) return conv_mfma_multi_kernel<TIn, TOut, SPLIT, FM, FN, WM, WN, 32, 2, 2>;
+    if (kc == 64 && pd == 4 && unr == 4) return conv_mfma_multi_kernel<TIn, TOut, SPLIT, FM, FN, WM, WN, 64, 4, 4>;
+    if (kc == 128 && pd == 4 && unr == 8) return conv_mfma_multi_kernel<TIn, TOut, SPLIT, FM, FN, WM, WN, 128, 4, 8>;
+    return nullptr;
+}
+
 #define FYN_CAT2(a, b) a##b
 #define FYN_CAT(a, b) FYN_CAT2(a, b)
 
 // lookup among the tiles of one part (a template so that the tiles of other parts are not instantiated)
 template <int PART>
-static conv_kernel_fn lookup_part(const ConvVariant& v) {
+static ConvEntry lookup_part(const ConvVariant& v) {
     const bool f16 = v.in_f16 && v.out_f16 && !v.split;
     const bool f32 = !v.in_f16 && !v.out_f16 && v.split;  // split arithmetic is the fp32-storage path
-    if (!f16 && !f32) return nullptr;
-#define FYN_TILE(idx_, fm_, fn_, wm_, wn_)                                                \
-    if constexpr ((idx_) % FYN_CONV_PARTS == PART) {                                       \
-        if (v.fm == fm_ && v.fn == fn_ && v.wm == wm_ && v.wn == wn_)                      \
-            return f32 ? pick_kc<float, float, true, fm_, fn_, wm_, wn_>(v.kc, v.pd, v.unr)             \
-                       : pick_kc<_Float16, _Float16, false, fm_, fn_, wm_, wn_>(v.kc, v.pd, v.unr);     \
+    ConvEntry e;
+    if (!f16 && !f32) return e;
+#define FYN_TILE(idx_, fm_, fn_, wm_, wn_)                                                                    \
+    if constexpr ((idx_) % FYN_CONV_PARTS == PART) {                                                           \
+        if (v.fm == fm_ && v.fn == fn_ && v.wm == wm_ && v.wn == wn_) {                                        \
+            if (f32) {                                                                                         \
+                e.single = pick_kc<float, float, true, fm_, fn_, wm_, wn_>(v.kc, v.pd, v.unr);                 \
+                e.multi = pick_kc_multi<float, float, true, fm_, fn_, wm_, wn_>(v.kc, v.pd, v.unr);            \
+            } else {                                                                                           \
+                e.single = pick_kc<_Float16, _Float16, false, fm_, fn_, wm_, wn_>(v.kc, v.pd, v.unr);          \
+                e.multi = pick_kc_multi<_Float16, _Float16, false, fm_, fn_, wm_, wn_>(v.kc, v.pd, v.unr);     \
+            }                                                                                                  \
+            return e;                                                                                          \
+        }                                                                                                      \
     }
     FYN_CONV_TILES(FYN_TILE)
 #undef FYN_TILE
-    return nullptr;
+    return e;
 }
 
-conv_kernel_fn FYN_CAT(conv_mfma_lookup_part, FYN_CONV_PART)(const ConvVariant& v) { return lookup_part<FYN_CONV_PART>(v); }
+ConvEntry FYN_CAT(conv_mfma_lookup_part, FYN_CONV_PART)(const ConvVariant& v) { return lookup_part<FYN_CONV_PART>(v); }
 
 #if FYN_CONV_PART == 0
-#define FYN_DECL(i_) conv_kernel_fn conv_mfma_lookup_part##i_(const ConvVariant& v);
+#define FYN_DECL(i_) ConvEntry conv_mfma_lookup_part##i_(const ConvVariant& v);
 #if FYN_CONV_PARTS > 1
 FYN_DECL(1)
 #endif
@@ -669,29 +706,30 @@ FYN_DECL(7)
 #endif
 #undef FYN_DECL
 
-static conv_kernel_fn pick_kernel(const ConvVariant& v) {
-    conv_kernel_fn fn = conv_mfma_lookup_part0(v);
+static ConvEntry pick_kernel(const ConvVariant& v) {
+    ConvEntry e = conv_mfma_lookup_part0(v);
 #if FYN_CONV_PARTS > 1
-    if (!fn) fn = conv_mfma_lookup_part1(v);
+    if (!e.single) e = conv_mfma_lookup_part1(v);
 #endif
 #if FYN_CONV_PARTS > 2
-    if (!fn) fn = conv_mfma_lookup_part2(v);
+    if (!e.single) e = conv_mfma_lookup_part2(v);
 #endif
 #if FYN_CONV_PARTS > 3
-    if (!fn) fn = conv_mfma_lookup_part3(v);
+    if (!e.single) e = conv_mfma_lookup_part3(v);
 #endif
 #if FYN_CONV_PARTS > 4
-    if (!fn) fn = conv_mfma_lookup_part4(v);
-    if (!fn) fn = conv_mfma_lookup_part5(v);
+    if (!e.single) e = conv_mfma_lookup_part4(v);
+    if (!e.single) e = conv_mfma_lookup_part5(v);
 #endif
 #if FYN_CONV_PARTS > 6
-    if (!fn) fn = conv_mfma_lookup_part6(v);
-    if (!fn) fn = conv_mfma_lookup_part7(v);
+    if (!e.single) e = conv_mfma_lookup_part6(v);
+    if (!e.single) e = conv_mfma_lookup_part7(v);
 #endif
-    return fn;
+    return e;
 }
 
-bool conv_mfma_variant_exists(const ConvVariant& v) { return pick_kernel(v) != nullptr; }
+bool conv_mfma_variant_exists(const ConvVariant& v) { return pick_kernel(v).single != nullptr; }
+bool conv_mfma_multi_exists(const ConvVariant& v) { return pick_kernel(v).multi != nullptr; }
 
 int conv_mfma_step_multiple(const ConvVariant& v) { return v.unr; }
 
@@ -710,44 +748,87 @@ void conv_mfma_tile(int index, int* fm, int* fn, int* wm, int* wn) {
 #undef FYN_TILE
 }
 
-int launch_conv_mfma(const ConvVariant& v, const ConvMfmaParams& p, size_t lds_bytes, hipStream_t s) {
-    conv_kernel_fn fn = pick_kernel(v);
-    if (!fn) return -1;
+static int blocks_of(const ConvMfmaParams& p) { return p.tiles_x * p.tiles_y * p.cout_blocks * (p.ksplit > 1 ? p.ksplit : 1); }
+
+static int check_params(const ConvVariant& v, const ConvMfmaParams& p) {
     if (p.nsteps < 1 || p.nsteps > 256 || v.unr < 2 || p.nsteps % v.unr != 0) return -5;
-    if (lds_bytes > 48 * 1024) {
-        // raise the kernel's dynamic LDS limit once per kernel and size
-        static std::mutex mu;
-        static std::map<const void*, size_t> raised;
-        std::lock_guard<std::mutex> lk(mu);
-        size_t& cur = raised[reinterpret_cast<const void*>(fn)];
-        if (cur < lds_bytes) {
-            if (hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                    (int)lds_bytes) != hipSuccess)
-                return -2;
-            cur = lds_bytes;
-        }
-    }
-    const int blocks = p.tiles_x * p.tiles_y * p.cout_blocks * (p.ksplit > 1 ? p.ksplit : 1);
     if (p.ksplit > 1 && (!p.partial || p.chunks_per_split < 1 || (p.ksplit - 1) * p.chunks_per_split >= p.cin_chunks)) return -7;
     if (p.ksplit <= 1 && p.chunks_per_split < p.cin_chunks) return -7;
+    return 0;
+}
+
+// raises a kernel's dynamic LDS limit once per kernel and size
+static int ensure_lds(const void* fn, size_t lds_bytes) {
+    if (lds_bytes <= 48 * 1024) return 0;
+    static std::mutex mu;
+    static std::map<const void*, size_t> raised;
+    std::lock_guard<std::mutex> lk(mu);
+    size_t& cur = raised[fn];
+    if (cur < lds_bytes) {
+        if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes) != hipSuccess) return -2;
+        cur = lds_bytes;
+    }
+    return 0;
+}
+
 #ifdef FYN_CONV_TRACE
-    static long long* trace_dev = nullptr;
-    if (!trace_dev && hipMalloc(&trace_dev, sizeof(long long) * 16 * 65536) != hipSuccess) return -6;
-    if (blocks > 65536) return -6;
-    ConvMfmaParams pt = p;
-    pt.trace = trace_dev;
-    hipLaunchKernelGGL(fn, dim3(blocks), dim3(v.fm * v.fn >= 2 ? 512 : 256), lds_bytes, s, pt);
+static long long* trace_buffer() {
+    static long long* dev = nullptr;
+    if (!dev && hipMalloc(&dev, sizeof(long long) * 16 * 65536) != hipSuccess) return nullptr;
+    return dev;
+}
+static void trace_dump(hipStream_t s, long long* dev, size_t blocks) {
     hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
     (void)hipStreamIsCapturing(s, &cap);
     const char* path = cap == hipStreamCaptureStatusNone ? getenv("FYNHIP_TRACE_DUMP") : nullptr;
-    if (path) {
-        std::vector<long long> h((size_t)blocks * 16);
-        if (hipStreamSynchronize(s) == hipSuccess && hipMemcpy(h.data(), trace_dev, h.size() * 8, hipMemcpyDeviceToHost) == hipSuccess) {
-            if (FILE* f = fopen(path, "wb")) { fwrite(h.data(), 8, h.size(), f); fclose(f); }
-        }
+    if (!path) return;
+    std::vector<long long> h(blocks * 16);
+    if (hipStreamSynchronize(s) == hipSuccess && hipMemcpy(h.data(), dev, h.size() * 8, hipMemcpyDeviceToHost) == hipSuccess) {
+        if (FILE* f = fopen(path, "wb")) { fwrite(h.data(), 8, h.size(), f); fclose(f); }
     }
+}
+#endif
+
+int launch_conv_mfma(const ConvVariant& v, const ConvMfmaParams& p_in, size_t lds_bytes, hipStream_t s) {
+    conv_kernel_fn fn = pick_kernel(v).single;
+    if (!fn) return -1;
+    if (int rc = check_params(v, p_in)) return rc;
+    if (int rc = ensure_lds(reinterpret_cast<const void*>(fn), lds_bytes)) return rc;
+    const int blocks = blocks_of(p_in);
+    const dim3 threads(v.fm * v.fn >= 2 ? 512 : 256);
+#ifdef FYN_CONV_TRACE
+    ConvMfmaParams p = p_in;
+    p.trace = trace_buffer();
+    if (!p.trace || blocks > 65536) return -6;
+    hipLaunchKernelGGL(fn, dim3(blocks), threads, lds_bytes, s, p);
+    trace_dump(s, p.trace, blocks);
 #else
-    hipLaunchKernelGGL(fn, dim3(blocks), dim3(v.fm * v.fn >= 2 ? 512 : 256), lds_bytes, s, p);
+    hipLaunchKernelGGL(fn, dim3(blocks), threads, lds_bytes, s, p_in);
+#endif
+    return hipGetLastError() == hipSuccess ? 0 : -3;
+}
+
+int launch_conv_mfma_multi(const ConvVariant& v, const ConvMfmaMulti& m_in, size_t lds_bytes, hipStream_t s) {
+    if (m_in.nsub == 1) return launch_conv_mfma(v, m_in.sub[0], lds_bytes, s);
+    conv_multi_fn fn = pick_kernel(v).multi;
+    if (!fn) return -1;
+    if (m_in.nsub < 1 || m_in.nsub > FYN_CONV_MAX_SUB) return -8;
+    int blocks = 0;
+    for (int i = 0; i < m_in.nsub; i++) {
+        if (int rc = check_params(v, m_in.sub[i])) return rc;
+        blocks = blocks_of(m_in.sub[i]) > blocks ? blocks_of(m_in.sub[i]) : blocks;
+    }
+    if (int rc = ensure_lds(reinterpret_cast<const void*>(fn), lds_bytes)) return rc;
+    const dim3 threads(v.fm * v.fn >= 2 ? 512 : 256);
+#ifdef FYN_CONV_TRACE
+    ConvMfmaMulti m = m_in;
+    long long* tb = trace_buffer();
+    if (!tb || (size_t)blocks * m.nsub > 65536) return -6;
+    for (int i = 0; i < m.nsub; i++) m.sub[i].trace = tb;
+    hipLaunchKernelGGL(fn, dim3(blocks, m.nsub), threads, lds_bytes, s, m);
+    trace_dump(s, tb, (size_t)blocks * m.nsub);
+#else
+    hipLaunchKernelGGL(fn, dim3(blocks, m_in.nsub), threads, lds_bytes, s, m_in);
 #endif
     return hipGetLastError() == hipSuccess ? 0 : -3;
 }

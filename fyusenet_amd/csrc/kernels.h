@@ -90,9 +90,19 @@ struct ConvVariant {
     int unr;             // k16 steps per unrolled group (a multiple of pd; nsteps is a multiple of it)
 };
 
+// Up to four (sub-)convolutions that share one kernel variant run as ONE launch (the four output parities
+// of a transposed convolution): grid row blockIdx.y works on sub[blockIdx.y].
+#define FYN_CONV_MAX_SUB 4
+struct ConvMfmaMulti {
+    ConvMfmaParams sub[FYN_CONV_MAX_SUB];
+    int nsub;
+};
+
 // Returns 0 when the variant exists and was launched.
 int launch_conv_mfma(const ConvVariant& v, const ConvMfmaParams& p, size_t lds_bytes, hipStream_t s);
+int launch_conv_mfma_multi(const ConvVariant& v, const ConvMfmaMulti& m, size_t lds_bytes, hipStream_t s);
 bool conv_mfma_variant_exists(const ConvVariant& v);
+bool conv_mfma_multi_exists(const ConvVariant& v);   // a multi-launch entry point is compiled for the variant
 // The kernel runs its k16 steps in groups of this size: nsteps must be a multiple (pad with zero-weight steps).
 int conv_mfma_step_multiple(const ConvVariant& v);
 // The compiled tile configurations (fragments per wave fm x fn, waves per block wm x wn).

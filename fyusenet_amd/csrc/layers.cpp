@@ -163,7 +163,7 @@ static void conv_geometry(const TView& in, bool split, int ntaps, int kc_force, 
 // of 4), so candidates can share one weight buffer (`share`); weights are packed separately.
 static MfmaLaunch plan_mfma(Net* net, const SubConv& sc, const TView& in, const TView& out, const TView* res, int cin,
                             int cout, const Act& act, int res_relu, int res_scale, const TileChoice& tc,
-                            const float* scale, const float* bias, const MfmaLaunch* share = nullptr) {
+                            const float* scale, const float* bias, const MfmaLaunch* share = nullptr, int force_pd = 0) {
     MfmaLaunch L;
     L.cin = cin;
     L.cout = cout;
@@ -253,8 +253,9 @@ static MfmaLaunch plan_mfma(Net* net, const SubConv& sc, const TView& in, const 
         if (kc == 32) pd = (raw % 6 == 0) ? 6 : ((raw % 4 == 0) ? 4 : 2);
         if (kc >= 64) pd = 4;
         if (const char* e = getenv("FYNHIP_CONV_PD")) pd = atoi(e);
+        if (force_pd > 0 && kc <= 32) pd = force_pd;
         L.var.pd = pd;
-        L.var.unr = (pd == 6 && raw == 18 && !getenv("FYNHIP_CONV_NO_FULL_UNROLL")) ? 18 : pd;
+        L.var.unr = (pd == 6 && raw == 18 && force_pd == 0 && !getenv("FYNHIP_CONV_NO_FULL_UNROLL")) ? 18 : pd;
         if (kc == 128) L.var.unr = 8;
         if (!conv_mfma_variant_exists(L.var)) fail(FYN_ERR_UNSUPPORTED, "MFMA convolution variant not compiled");
     }
@@ -453,6 +454,100 @@ static MfmaLaunch tune_mfma(Net* net, const SubConv& sc, const TView& in, const 
         }
     }
     tune_cache_store(key, best.var, best.p.ksplit);
+    return best;
+}
+
+// Several sub-convolutions of one layer (the output parities of a transposed convolution) that run as one launch.
+struct MfmaGroup {
+    std::vector<MfmaLaunch> subs;
+    ConvMfmaMulti multi{};
+    size_t lds = 0;
+    ConvVariant var{};
+    void sync() {
+        multi.nsub = (int)subs.size();
+        lds = 0;
+        for (size_t i = 0; i < subs.size(); i++) {
+            multi.sub[i] = subs[i].p;
+            lds = std::max(lds, subs[i].lds);
+        }
+        if (!subs.empty()) var = subs[0].var;
+    }
+};
+
+static int run_group(const MfmaGroup& g, hipStream_t s) {
+    if (conv_mfma_multi_exists(g.var)) return launch_conv_mfma_multi(g.var, g.multi, g.lds, s);
+    for (const MfmaLaunch& L : g.subs)   // no merged entry point for this variant (narrow channel chunks): one launch each
+        if (int rc = launch_conv_mfma(L.var, L.p, L.lds, s)) return rc;
+    return 0;
+}
+
+static float time_group(Net* net, const MfmaGroup& g, int iters) {
+    hipEvent_t a, b;
+    FYN_HIP(hipEventCreate(&a));
+    FYN_HIP(hipEventCreate(&b));
+    if (run_group(g, net->stream) != 0) fail(FYN_ERR_DEVICE, "convolution launch failed while tuning");
+    FYN_HIP(hipEventRecord(a, net->stream));
+    for (int i = 0; i < iters; i++) run_group(g, net->stream);
+    FYN_HIP(hipEventRecord(b, net->stream));
+    FYN_HIP(hipEventSynchronize(b));
+    FYN_HIP(hipGetLastError());
+    float ms = 0.f;
+    FYN_HIP(hipEventElapsedTime(&ms, a, b));
+    (void)hipEventDestroy(a);
+    (void)hipEventDestroy(b);
+    return ms / iters;
+}
+
+// Picks ONE tile configuration and chunk width for a group of sub-convolutions (same tensors, different taps
+// and output offsets) by timing the merged launch; the step group size is fixed so that all members fit it.
+static MfmaGroup tune_mfma_group(Net* net, const std::vector<SubConv>& scs, const TView& in, const TView& out, int cin, int cout,
+                                 const Act& act, const float* scale, const float* bias) {
+    if (scs.empty() || scs.size() > FYN_CONV_MAX_SUB) fail(FYN_ERR_INVALID, "internal: bad sub-convolution group");
+    // candidates from the member with the most taps (largest staged tile)
+    size_t big = 0;
+    for (size_t i = 1; i < scs.size(); i++)
+        if (scs[i].taps.size() > scs[big].taps.size()) big = i;
+    std::vector<TileChoice> cands;
+    {
+        int kc0, pitch, slack, npl;
+        conv_geometry(in, !net->f16(), (int)scs[big].taps.size(), 0, kc0, pitch, slack, npl);
+        std::vector<int> kcs{kc0};
+        if (kc0 > 32) kcs.push_back(32);
+        for (int kco : kcs) {
+            int kc;
+            conv_geometry(in, !net->f16(), (int)scs[big].taps.size(), kco, kc, pitch, slack, npl);
+            const int chunks = (kc == 4) ? 1 : (in.cp + kc - 1) / kc;
+            std::vector<TileChoice> c = enumerate_tiles(cout, scs[big], pitch, npl, slack, chunks > 1 ? 2 : 1);
+            for (TileChoice& tc : c) {
+                tc.kc = kc;
+                cands.push_back(tc);
+            }
+        }
+        std::stable_sort(cands.begin(), cands.end(), [](const TileChoice& x, const TileChoice& y) { return x.score > y.score; });
+    }
+    auto plan_all = [&](const TileChoice& tc, const MfmaGroup* share) {
+        MfmaGroup g;
+        for (size_t i = 0; i < scs.size(); i++)
+            g.subs.push_back(plan_mfma(net, scs[i], in, out, nullptr, cin, cout, act, 0, 0, tc, scale, bias, share ? &share->subs[i] : nullptr, 2));
+        g.sync();
+        return g;
+    };
+    const char* at = getenv("FYNHIP_AUTOTUNE");
+    const bool tune = !(at && at[0] == '0') && cands.size() > 1;
+    MfmaGroup best = plan_all(cands[0], nullptr);
+    if (!tune) return best;
+    const bool verbose = getenv("FYNHIP_TUNE_VERBOSE") != nullptr;
+    float best_ms = std::min(time_group(net, best, 4), time_group(net, best, 4));
+    if (verbose) fprintf(stderr, "[tune] group of %zu: %s -> %.1f us\n", scs.size(), mfma_info(best.subs[0]).c_str(), best_ms * 1e3f);
+    for (size_t i = 1; i < cands.size(); i++) {
+        MfmaGroup g = plan_all(cands[i], &best);
+        const float ms = std::min(time_group(net, g, 4), time_group(net, g, 4));
+        if (verbose) fprintf(stderr, "[tune] group of %zu: %s -> %.1f us\n", scs.size(), mfma_info(g.subs[0]).c_str(), ms * 1e3f);
+        if (ms < best_ms) {
+            best_ms = ms;
+            best = g;
+        }
+    }
     return best;
 }
 
@@ -780,8 +875,9 @@ class TransConvLayer : public Layer {
                 sc.out_step = 2;
                 sc.out_off_y = out_v.pad + py;
                 sc.out_off_x = out_v.pad + px;
-                launches.push_back(tune_mfma(net, sc, in_v, out_v, nullptr, d.in_channels, oc, act(), 0, 0, scale_dev, bias_dev));
+                subconvs.push_back(sc);
             }
+        group = tune_mfma_group(net, subconvs, in_v, out_v, d.in_channels, oc, act(), scale_dev, bias_dev);
         set_up = true;
         if (!block.empty()) pack();
     }
@@ -794,24 +890,26 @@ class TransConvLayer : public Layer {
         reupload(net, scale_dev, sc);
         reupload(net, bias_dev, bi);
         const float wmul = weight_prescale(w, (size_t)oc * k * k * d.in_channels);
-        for (auto& L : launches) {
+        for (auto& L : group.subs) {
             L.p.acc_mul = 1.0f / wmul;
-            L.red.acc_mul = 1.0f / wmul;
             pack_mfma_weights(net, L, w, k, wmul);
         }
+        group.sync();
         have_weights = true;
     }
     void forward(hipStream_t s) override {
         if (!have_weights) fail(FYN_ERR_STATE, "layer %s (%d): forward() without weights", d.name, d.number);
-        for (auto& L : launches)
-            if (run_mfma(L, s) != 0) fail(FYN_ERR_DEVICE, "layer %s: transposed convolution launch failed", d.name);
+        if (run_group(group, s) != 0) fail(FYN_ERR_DEVICE, "layer %s: transposed convolution launch failed", d.name);
     }
-    std::string info() const override { return launches.empty() ? "transconv" : "transconv 4x " + mfma_info(launches[0]); }
+    std::string info() const override {
+        return group.subs.empty() ? "transconv" : "transconv, " + std::to_string(group.subs.size()) + " parities in one launch: " + mfma_info(group.subs[0]);
+    }
     int k, crop;
     bool have_weights = false;
     int padded = 0;
     std::vector<float> block;
-    std::vector<MfmaLaunch> launches;
+    std::vector<SubConv> subconvs;
+    MfmaGroup group;
     float *scale_dev = nullptr, *bias_dev = nullptr;
 };
 
