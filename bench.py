@@ -26,7 +26,7 @@ from fyusenet_amd import networks  # noqa: E402
 PEAK_MFMA_F16_TFLOPS = 2500.0   # MI355X dense fp16/bf16 matrix peak
 PEAK_HBM_GBS = 8000.0           # MI355X HBM3E
 # (layer type, kernel, cin, cout, h, w) -> measured HBM bytes per launch (fetch + write), fp32 storage
-MEASURED_TRAFFIC = {(6, 3, 128, 128, 156, 128): 26.58e6 + 10.22e6}  # launches with the fused residual read
+MEASURED_TRAFFIC = {(6, 3, 128, 128, 156, 128): 27.13e6 + 10.22e6}  # launches with the fused residual read
 
 
 def log(*a):

@@ -534,6 +534,14 @@ static MfmaGroup tune_mfma_group(Net* net, const std::vector<SubConv>& scs, cons
     };
     const char* at = getenv("FYNHIP_AUTOTUNE");
     const bool tune = !(at && at[0] == '0') && cands.size() > 1;
+    char key[160];
+    snprintf(key, sizeof(key), "g%zu:%d%d:%dx%d:%dx%d:t%zu:o%d:cp%d", scs.size(), in.f16, out.f16, cin, cout, scs[big].npos_y, scs[big].npos_x,
+             scs[big].taps.size(), scs[big].out_step, in.cp);
+    if (tune) {
+        int ks = 1;
+        const TileChoice* hit = tune_cache_lookup(key, cands, &ks);
+        if (hit) return plan_all(*hit, nullptr);
+    }
     MfmaGroup best = plan_all(cands[0], nullptr);
     if (!tune) return best;
     const bool verbose = getenv("FYNHIP_TUNE_VERBOSE") != nullptr;
@@ -548,6 +556,7 @@ static MfmaGroup tune_mfma_group(Net* net, const std::vector<SubConv>& scs, cons
             best = g;
         }
     }
+    tune_cache_store(key, best.var, 1);
     return best;
 }
 
