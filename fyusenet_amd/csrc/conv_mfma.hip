@@ -628,7 +628,9 @@ struct ConvEntry {
     X(10, 1, 4, 4, 1)     \
     X(11, 1, 2, 2, 2)     \
     X(12, 1, 4, 2, 2)     \
-    X(13, 1, 3, 2, 2)
+    X(13, 1, 3, 2, 2)     \
+    X(14, 1, 4, 1, 4)     \
+    X(15, 1, 3, 1, 4)
 
 // (ring depth, unroll) pairs: 2/2 for chunks of 4, 16 and 32 channels; for 32-channel chunks also 4/4, 6/6 and
 // 6/18 (a whole 3x3 chunk unrolled: no loop back-edge, hence no conservative wait, inside a chunk); 64- and
