@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the GPU layer stack on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload stylenet|resnet50|conv1|mobilenet|stylenet9x9]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload stylenet|resnet50|resnet50ref|conv1|mobilenet|stylenet9x9]
 
 A step is one forward pass of the named network over one synthetic input frame that is already
 resident in HBM (uploaded before the timed region); weights are synthetic (random init).  Prints ONE
@@ -40,6 +40,9 @@ def make_net(workload):
         return networks.StyleNet(fa.STORAGE_F16, 1524, 1856, 9), "stylenet9x9 1524x1856 ms/frame", "ms/frame", "fp16 storage, fp16 MFMA, fp32 accumulate"
     if workload == "resnet50":
         return networks.ResNet50(fa.STORAGE_F32), "ResNet-50 224x224 imgs/s", "imgs/s", "fp32 storage"
+    if workload == "resnet50ref":   # the reference's own sample graph (explicit batch-norm layers), .dat-compatible
+        from fyusenet_amd import samples
+        return samples.ResNet50Sample(fa.STORAGE_F32), "ResNet-50 (reference sample graph) 224x224 imgs/s", "imgs/s", "fp32 storage"
     if workload == "mobilenet":
         return networks.MobileNetV2(fa.STORAGE_F16), "MobileNetV2 224x224 imgs/s", "imgs/s", "fp16 storage"
     if workload == "conv1":
@@ -231,7 +234,7 @@ def main():
 
     if not args.no_also and args.workload == "stylenet":
         also = {}
-        for wl in ("resnet50",):
+        for wl in ("resnet50", "resnet50ref"):
             n2, m2, u2, d2 = make_net(wl)
             n2.setup()
             n2.setInput(n2.makeInput())

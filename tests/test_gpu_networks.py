@@ -223,3 +223,20 @@ def test_intermediate_output_and_timings(tmp_path):
     ms, runs = net.getTiming(1)
     assert runs == 3 and ms > 0
     net.cleanup()
+
+
+def test_reference_resnet50_sample_graph():
+    """The reference's own ResNet-50 sample graph (explicit batch-norm layers, batch-norm on the residual, a 7x7
+    stem on a halo of 1) with a synthetic weight stream of the .dat file's exact size and layout."""
+    from fyusenet_amd import samples
+    net = samples.ResNet50Sample(fa.STORAGE_F32)
+    assert net.total_weight_bytes() == 102304184
+    ref, got = run_and_compare(net, fa.STORAGE_F32)
+    logits = got[net.GEMM]
+    assert logits.shape == (1000, 1, 1) and np.all(np.isfinite(logits)) and float(np.std(logits)) > 0
+    net.cleanup()
+    # a wrong-sized weight stream is refused
+    bad = samples.ResNet50Sample(fa.STORAGE_F32, weights=np.zeros(1000, np.float32))
+    with pytest.raises(fa.FynException):
+        bad.setup()
+    bad.cleanup()

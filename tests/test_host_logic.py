@@ -83,3 +83,34 @@ def test_prng_is_stable():
     assert list(map(float, prng.uniform(1234, (4,), -1, 1))) == list(map(float, u))
     assert abs(float(prng.normal(5, (200000,)).std()) - 1.0) < 0.01
     assert abs(float(prng.uniform(6, (200000,), 0, 1).mean()) - 0.5) < 0.01
+
+
+def test_resnet50_sample_weight_layout_matches_the_reference_file_layout():
+    """Byte offsets derived from the layer descriptions against the values the reference hard-codes
+    (samples/samplenetworks/resnet50.cpp:539-677); none of this needs the library."""
+    from fyusenet_amd import samples
+
+    class _Dry(samples.ResNet50Sample):
+        def __init__(self):   # graph description only, no engine handle
+            self._weights, self._specs, self._edges, self._file_order = None, [], [], []
+            self._define()
+
+        def __del__(self):
+            pass
+
+    net = _Dry()
+    lay = net.weight_layout()
+    assert net.total_weight_bytes() == samples.RESNET50_TOTAL_WEIGHT_BYTES == 102304184
+    anchors = {2: (0, 24), 3: (24, 38400), 5: (38424, 512), 6: (38936, 17152), 8: (56088, 148224), 9: (204312, 66560),
+               7: (270872, 66560), 10: (337432, 2048), 17: (837144, 68608), 19: (1893912, 526336), 20: (1038360, 591360),
+               35: (9736728, 2101248), 36: (6321688, 2362368), 57: (33159704, 1060864), 59: (49969688, 8396800),
+               62: (58366488, 16384), 69: (89889304, 4218880), 72: (94108184, 8196000)}
+    for no, v in anchors.items():
+        assert lay[no] == v, (no, lay[no], v)
+    assert len(lay) == 68 and len(net._specs) == 72 and len(net._edges) == 87
+    # every edge joins layers whose shapes agree
+    spec = {no: b for no, b, _ in net._specs}
+    for src, dst, port in net._edges:
+        s, d = spec[src], spec[dst]
+        if port == 0:
+            assert s.outputChannels_ == d.inputChannels_, (src, dst)

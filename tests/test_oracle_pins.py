@@ -86,6 +86,21 @@ def test_conv_matches_torch(k, stride, dil, cin, cout, h, w, relu):
     assert rel_l2(y, ref) < 1e-6
 
 
+def test_conv_with_halo_narrower_than_the_kernel_radius_reads_zero():
+    # the reference's ResNet-50 stem: 7x7 stride 2 on a tensor stored with a halo of 1
+    # (samples/samplenetworks/resnet50.cpp:211-212); what lies beyond the stored frame is zero, so the result
+    # equals an ordinary padding-3 convolution
+    k, cin, cout, h, w, stride, pad = 7, 3, 8, 20, 18, 2, 1
+    x = prng.uniform(12, (cin, h, w), -1, 1)
+    block = conv_block(21, cout, k, cin)
+    y = O.conv2d(O.pad_chw(x, pad), pad, block, cout, k, 1, stride, None)
+    ref = F.conv2d(torch.from_numpy(x.astype(np.float64))[None], _w_from_block(block, cout, k, cin),
+                   torch.from_numpy(block[:cout].astype(np.float64)), stride=stride, padding=3)[0].numpy()
+    ref = ref[:, :h // stride, :w // stride]
+    assert y.shape == ref.shape
+    assert rel_l2(y, ref) < 1e-6
+
+
 def test_conv_bn_residual_epilogue():
     # order: acc*scale + (bias*scale + bnBias) + relu(res)*scale  (batchnorm.inc / residual.inc)
     cin, cout, k, h, w = 6, 5, 3, 8, 9
