@@ -151,6 +151,36 @@ def dominant_conv_roofline(net, storage_bytes):
     return rec, per_layer
 
 
+def host_io_rates(net, x, frames):
+    """Frame rate with the frame handed over and returned in host memory (PCIe in both directions inside the timed
+    region): the synchronous call sequence, then the frame pipeline at depth 2 and 3.  Reported beside `value`,
+    never as `value`."""
+    in_layer, in_port = net.input_key
+    net.useGraph(False)
+    rec = {}
+    for _ in range(3):
+        net.setInput(x); net.forward(); net.finish(); y = net.getOutput(net.output_layer)
+    t0 = time.perf_counter()
+    for _ in range(frames):
+        net.setInput(x); net.forward(); net.finish(); net.getOutput(net.output_layer)
+    rec["ms_per_frame_synchronous"] = (time.perf_counter() - t0) * 1e3 / frames
+    for depth in (2, 3):
+        outs = [np.empty_like(y) for _ in range(depth + 1)]
+        net.asyncBegin(in_layer, net.output_layer, depth=depth, inPort=in_port)
+        for i in range(depth + 2):
+            t = net.asyncSubmit(x, outs[i % len(outs)])
+        net.asyncWait(t)
+        t0 = time.perf_counter()
+        for i in range(frames):
+            t = net.asyncSubmit(x, outs[i % len(outs)])
+        net.asyncWait(t)
+        rec["ms_per_frame_pipeline_depth%d" % depth] = (time.perf_counter() - t0) * 1e3 / frames
+        net.asyncEnd()
+        assert np.array_equal(outs[(frames - 1) % len(outs)], y)
+    rec["bytes_in"], rec["bytes_out"] = int(x.nbytes), int(y.nbytes)
+    return rec
+
+
 def cpu_baseline(net, x, total_flops):
     """Times the CPU oracle (plain C restatement of the reference's unit-test convolution, OpenMP over
     output channels) on the dominant convolution of the workload at full size and scales by the
@@ -217,6 +247,10 @@ def main():
            "config": {"workload": args.workload, "input": list(x.shape), "batch": 1, "launch": launch,
                       "algorithmic_gflop_per_step": total_flops / 1e9},
            "ms_per_step_graph": ms_graph, "ms_per_step_eager": ms_eager, "roofline": roof}
+
+    if hasattr(net, "input_key") and args.workload != "copy":
+        out["host_io"] = host_io_rates(net, x, max(args.steps, 50))
+        log("host I/O inclusive: %s" % out["host_io"])
 
     if not args.no_cpu_baseline:
         dt, flops, threads, lname = cpu_baseline(net, x, total_flops)

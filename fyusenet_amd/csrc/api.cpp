@@ -219,6 +219,30 @@ int fyn_layer_time(fyn_net* net, int layer, int iters, float* ms_total) {
     FYN_API_END
 }
 
+int fyn_net_async_begin(fyn_net* net, int in_layer, int in_port, int in_order, int out_layer, int out_order, int depth) {
+    FYN_API_BEGIN
+    N(net)->async_begin(in_layer, in_port, in_order, out_layer, out_order, depth);
+    FYN_API_END
+}
+
+int fyn_net_async_submit(fyn_net* net, const float* in, float* out, uint64_t* ticket) {
+    FYN_API_BEGIN
+    N(net)->async_submit(in, out, ticket);
+    FYN_API_END
+}
+
+int fyn_net_async_wait(fyn_net* net, uint64_t ticket) {
+    FYN_API_BEGIN
+    N(net)->async_wait(ticket);
+    FYN_API_END
+}
+
+int fyn_net_async_end(fyn_net* net) {
+    FYN_API_BEGIN
+    N(net)->async_end();
+    FYN_API_END
+}
+
 int fyn_layer_kernel_info(fyn_net* net, int layer, char* buf, size_t buflen) {
     FYN_API_BEGIN
     if (!buf || buflen == 0) fynhip::fail(FYN_ERR_INVALID, "null buffer");

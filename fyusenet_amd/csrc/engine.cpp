@@ -75,6 +75,10 @@ Net::Net(int dev, int stor) : device(dev), storage(stor) {
 
 Net::~Net() {
     (void)hipSetDevice(device);
+    try {
+        async_end();
+    } catch (...) {
+    }
     if (stream) (void)hipStreamSynchronize(stream);
     if (graph_exec_) (void)hipGraphExecDestroy(graph_exec_);
     if (graph_) (void)hipGraphDestroy(graph_);
@@ -484,6 +488,125 @@ void Net::time_layer(int layer_no, int iters, float* ms) {
     (void)hipEventDestroy(b);
     (void)hipGraphExecDestroy(ge);
     (void)hipGraphDestroy(g);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Frame pipeline (the counterpart of the reference engine's asynchronous mode, base/engine.cpp:386-683, with
+// its two upload/download buffer sets, gpu/uploadlayer.h:74): three streams of equal priority joined by events.
+// Frame i:   up stream    pinned host slot -> device staging slot
+//            main stream  staging -> input tensor, all layers, output tensor -> device staging slot
+//            down stream  device staging slot -> pinned host slot
+// A slot is reused only after its download has completed, which also orders the staging buffers.
+// ---------------------------------------------------------------------------------------------
+void Net::async_begin(int in_layer, int in_port, int in_order, int out_layer, int out_order, int depth) {
+    if (!is_setup) fail(FYN_ERR_STATE, "async_begin() before setup()");
+    if (!slots_.empty()) fail(FYN_ERR_STATE, "frame pipeline is already active");
+    if (depth < 1 || depth > 8) fail(FYN_ERR_INVALID, "pipeline depth %d out of range (1..8)", depth);
+    FYN_HIP(hipSetDevice(device));
+    Layer* li = layer(in_layer);
+    if (li->d.type == FYN_LAYER_UPLOAD) {
+        async_in_ = &li->tout();
+    } else {
+        if (in_port < 0 || in_port >= li->num_ports()) fail(FYN_ERR_INVALID, "layer %s has no input port %d", li->d.name, in_port);
+        async_in_ = &li->tin(in_port);
+        if (async_in_->producer != -1) fail(FYN_ERR_INVALID, "input port %d of layer %s is fed by layer %d", in_port, li->d.name, async_in_->producer);
+    }
+    async_out_ = &layer(out_layer)->tout();
+    const TView& vi = async_in_->v;
+    const TView& vo = async_out_->v;
+    if (in_order != FYN_ORDER_CHANNELWISE && in_order != FYN_ORDER_GPU_SHALLOW) fail(FYN_ERR_UNSUPPORTED, "input order %d not supported for upload", in_order);
+    if (out_order == FYN_ORDER_GPU_SHALLOW) {
+        if (vo.c > 4) fail(FYN_ERR_UNSUPPORTED, "GPU_SHALLOW download holds at most 4 channels per texel (layer has %d)", vo.c);
+        async_out_floats_ = (size_t)vo.h * vo.w * (vo.c == 3 ? 4 : vo.c);
+    } else if (out_order == FYN_ORDER_CHANNELWISE) {
+        async_out_floats_ = (size_t)vo.c * vo.h * vo.w;
+    } else {
+        fail(FYN_ERR_UNSUPPORTED, "output order %d not supported by the frame pipeline", out_order);
+    }
+    async_in_floats_ = (size_t)vi.c * vi.h * vi.w;
+    async_in_order_ = in_order;
+    async_out_order_ = out_order;
+    FYN_HIP(hipStreamCreateWithFlags(&up_stream_, hipStreamNonBlocking));
+    FYN_HIP(hipStreamCreateWithFlags(&down_stream_, hipStreamNonBlocking));
+    slots_.resize(depth);
+    for (AsyncSlot& s : slots_) {
+        FYN_HIP(hipHostMalloc(reinterpret_cast<void**>(&s.pin_in), async_in_floats_ * sizeof(float), hipHostMallocDefault));
+        FYN_HIP(hipHostMalloc(reinterpret_cast<void**>(&s.pin_out), async_out_floats_ * sizeof(float), hipHostMallocDefault));
+        FYN_HIP(hipMalloc(reinterpret_cast<void**>(&s.dev_in), async_in_floats_ * sizeof(float)));
+        FYN_HIP(hipMalloc(reinterpret_cast<void**>(&s.dev_out), async_out_floats_ * sizeof(float)));
+        FYN_HIP(hipEventCreateWithFlags(&s.up, hipEventDisableTiming));
+        FYN_HIP(hipEventCreateWithFlags(&s.comp, hipEventDisableTiming));
+        FYN_HIP(hipEventCreateWithFlags(&s.down, hipEventDisableTiming));
+    }
+}
+
+void Net::async_complete(AsyncSlot& s) {
+    if (!s.busy) return;
+    FYN_HIP(hipEventSynchronize(s.down));
+    if (s.user_out) memcpy(s.user_out, s.pin_out, async_out_floats_ * sizeof(float));
+    s.busy = false;
+}
+
+void Net::async_submit(const float* in, float* out, uint64_t* ticket) {
+    if (slots_.empty()) fail(FYN_ERR_STATE, "async_submit() without async_begin()");
+    if (!in || !out) fail(FYN_ERR_INVALID, "null frame buffer");
+    FYN_HIP(hipSetDevice(device));
+    AsyncSlot& s = slots_[async_seq_ % slots_.size()];
+    async_complete(s);  // oldest frame: its output is delivered before the slot is reused
+    memcpy(s.pin_in, in, async_in_floats_ * sizeof(float));
+    FYN_HIP(hipMemcpyAsync(s.dev_in, s.pin_in, async_in_floats_ * sizeof(float), hipMemcpyHostToDevice, up_stream_));
+    FYN_HIP(hipEventRecord(s.up, up_stream_));
+    FYN_HIP(hipStreamWaitEvent(stream, s.up, 0));
+    if (async_in_order_ == FYN_ORDER_CHANNELWISE) launch_chw_to_tensor(s.dev_in, async_in_->v, stream);
+    else launch_hwc_to_tensor(s.dev_in, async_in_->v.c, async_in_->v, stream);
+    forward(nullptr);
+    const TView& vo = async_out_->v;
+    if (async_out_order_ == FYN_ORDER_CHANNELWISE) launch_tensor_to_chw(vo, s.dev_out, 0, stream);
+    else launch_tensor_to_hwc(vo, s.dev_out, vo.c == 3 ? 4 : vo.c, stream);
+    FYN_HIP(hipGetLastError());
+    FYN_HIP(hipEventRecord(s.comp, stream));
+    FYN_HIP(hipStreamWaitEvent(down_stream_, s.comp, 0));
+    FYN_HIP(hipMemcpyAsync(s.pin_out, s.dev_out, async_out_floats_ * sizeof(float), hipMemcpyDeviceToHost, down_stream_));
+    FYN_HIP(hipEventRecord(s.down, down_stream_));
+    s.user_out = out;
+    s.busy = true;
+    s.ticket = ++async_seq_;
+    if (ticket) *ticket = s.ticket;
+}
+
+void Net::async_wait(uint64_t ticket) {
+    if (slots_.empty()) fail(FYN_ERR_STATE, "async_wait() without async_begin()");
+    FYN_HIP(hipSetDevice(device));
+    if (ticket == 0 || ticket > async_seq_) fail(FYN_ERR_INVALID, "unknown frame ticket %llu", (unsigned long long)ticket);
+    // frames complete in submission order: deliver everything up to the requested one
+    for (uint64_t t = (async_seq_ > slots_.size() ? async_seq_ - slots_.size() + 1 : 1); t <= ticket; t++) {
+        AsyncSlot& s = slots_[(t - 1) % slots_.size()];
+        if (s.busy && s.ticket == t) async_complete(s);
+    }
+}
+
+void Net::async_end() {
+    if (slots_.empty()) return;
+    (void)hipSetDevice(device);
+    for (uint64_t t = (async_seq_ > slots_.size() ? async_seq_ - slots_.size() + 1 : 1); t <= async_seq_; t++) {
+        AsyncSlot& s = slots_[(t - 1) % slots_.size()];
+        if (s.busy && s.ticket == t) async_complete(s);
+    }
+    if (stream) (void)hipStreamSynchronize(stream);
+    for (AsyncSlot& s : slots_) {
+        if (s.pin_in) (void)hipHostFree(s.pin_in);
+        if (s.pin_out) (void)hipHostFree(s.pin_out);
+        if (s.dev_in) (void)hipFree(s.dev_in);
+        if (s.dev_out) (void)hipFree(s.dev_out);
+        if (s.up) (void)hipEventDestroy(s.up);
+        if (s.comp) (void)hipEventDestroy(s.comp);
+        if (s.down) (void)hipEventDestroy(s.down);
+    }
+    slots_.clear();
+    if (up_stream_) (void)hipStreamDestroy(up_stream_);
+    if (down_stream_) (void)hipStreamDestroy(down_stream_);
+    up_stream_ = down_stream_ = nullptr;
+    async_seq_ = 0;
 }
 
 }  // namespace fynhip

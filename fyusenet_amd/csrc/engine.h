@@ -98,6 +98,11 @@ class Net {
     void time_forward(int iters, float* ms);
     void time_layer(int layer, int iters, float* ms);
     void use_graph(bool enable);
+    // frame pipeline: upload of frame i+1 and download of frame i-1 overlap the layers of frame i
+    void async_begin(int in_layer, int in_port, int in_order, int out_layer, int out_order, int depth);
+    void async_submit(const float* in, float* out, uint64_t* ticket);
+    void async_wait(uint64_t ticket);
+    void async_end();
 
     int device;
     int storage;  // fyn_storage
@@ -117,6 +122,21 @@ class Net {
     float* staging(size_t floats);  // fp32 staging area for layout conversion
 
   private:
+    struct AsyncSlot {
+        float *pin_in = nullptr, *pin_out = nullptr, *dev_in = nullptr, *dev_out = nullptr;
+        hipEvent_t up = nullptr, comp = nullptr, down = nullptr;
+        float* user_out = nullptr;
+        uint64_t ticket = 0;
+        bool busy = false;
+    };
+    std::vector<AsyncSlot> slots_;
+    hipStream_t up_stream_ = nullptr, down_stream_ = nullptr;
+    const Tensor* async_in_ = nullptr;
+    const Tensor* async_out_ = nullptr;
+    int async_in_order_ = 0, async_out_order_ = 0;
+    size_t async_in_floats_ = 0, async_out_floats_ = 0;
+    uint64_t async_seq_ = 0;
+    void async_complete(AsyncSlot& s);
     void run_layers(bool with_events);
     void collect_timings();
     void dump_layer(Layer* l);

@@ -241,6 +241,24 @@ class NeuralNetwork:
         capi.check(capi.lib().fyn_net_time_forward(self._h, iters, ctypes.byref(ms)))
         return ms.value
 
+    # -- frame pipeline (asynchronous engine mode of the reference, base/engine.cpp:386-683) --
+    def asyncBegin(self, inLayer, outLayer, inOrder=capi.ORDER_CHANNELWISE, outOrder=capi.ORDER_CHANNELWISE, depth=2, inPort=0):
+        capi.check(capi.lib().fyn_net_async_begin(self._h, inLayer, inPort, inOrder, outLayer, outOrder, depth))
+
+    def asyncSubmit(self, frame, out):
+        """Queues one frame; `out` (a C-contiguous float32 array) is filled once asyncWait(ticket) has returned."""
+        frame = np.ascontiguousarray(frame, dtype=np.float32)
+        assert out.dtype == np.float32 and out.flags["C_CONTIGUOUS"]
+        t = ctypes.c_uint64(0)
+        capi.check(capi.lib().fyn_net_async_submit(self._h, capi.fptr(frame), capi.fptr(out), ctypes.byref(t)))
+        return t.value
+
+    def asyncWait(self, ticket):
+        capi.check(capi.lib().fyn_net_async_wait(self._h, ticket))
+
+    def asyncEnd(self):
+        capi.check(capi.lib().fyn_net_async_end(self._h))
+
     def describe(self):
         """Plain description of the graph (descs, edges, loaded weight blocks) for external checkers."""
         out = []

@@ -192,6 +192,18 @@ int fyn_net_use_graph(fyn_net* net, int enable);
  * network's stream; per-layer variant times one layer's kernels alone.  Milliseconds total. */
 int fyn_net_time_forward(fyn_net* net, int iters, float* ms_total);
 int fyn_layer_time(fyn_net* net, int layer, int iters, float* ms_total);
+/* Frame pipeline for streams of frames handed over in host memory -- the reference engine's asynchronous mode
+ * (fyusenet/base/engine.cpp:386-683, two upload/download buffer sets: gpu/uploadlayer.h:74).  The upload of frame
+ * i+1 and the download of frame i-1 overlap the layers of frame i (pinned staging buffers, three streams).
+ *   begin : input = an upload layer (or an unconnected input port), output = any layer; `depth` frames in flight.
+ *   submit: copies `in` (borrowed for the call) and queues the frame; `out` must stay valid until the frame's
+ *           ticket has been waited for (it is filled then, or when its slot is reused `depth` submits later).
+ *   wait  : blocks until the frame (and all earlier ones) has been delivered.   end: drains and frees the pipeline.
+ * Orders: input CHANNELWISE or GPU_SHALLOW, output CHANNELWISE or GPU_SHALLOW. */
+int fyn_net_async_begin(fyn_net* net, int in_layer, int in_port, int in_order, int out_layer, int out_order, int depth);
+int fyn_net_async_submit(fyn_net* net, const float* in, float* out, uint64_t* ticket);
+int fyn_net_async_wait(fyn_net* net, uint64_t ticket);
+int fyn_net_async_end(fyn_net* net);
 /* Text description of the kernel variant chosen for a layer (for profiles / reports). */
 int fyn_layer_kernel_info(fyn_net* net, int layer, char* buf, size_t buflen);
 

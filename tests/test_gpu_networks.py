@@ -240,3 +240,46 @@ def test_reference_resnet50_sample_graph():
     with pytest.raises(fa.FynException):
         bad.setup()
     bad.cleanup()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("depth", [1, 2, 3])
+def test_frame_pipeline_matches_synchronous_path(depth):
+    """Asynchronous frame pipeline (upload / layers / download on three streams) against
+    setInput -> forward -> getOutput for a stream of different frames: bit-identical outputs, in order."""
+    from fyusenet_amd import prng
+    net = networks.StyleNet(fa.STORAGE_F32, width=96, height=80)
+    net.setup()
+    frames = [prng.uniform(900 + i, (3, 80, 96), -1.0, 1.0) for i in range(7)]
+    want = []
+    for f in frames:
+        net.setInput(f)
+        net.forward()
+        net.finish()
+        want.append(net.getOutput(net.output_layer).copy())
+    assert not np.array_equal(want[0], want[1])
+    in_layer, in_port = net.input_key
+    net.asyncBegin(in_layer, net.output_layer, depth=depth, inPort=in_port)
+    outs = [np.full_like(want[0], np.nan) for _ in frames]
+    tickets = [net.asyncSubmit(f, o) for f, o in zip(frames, outs)]
+    assert tickets == list(range(1, len(frames) + 1))
+    # frames older than `depth` submissions have been delivered already when their slot was reused
+    for i in range(len(frames) - depth):
+        assert np.array_equal(outs[i], want[i]), i
+    net.asyncWait(tickets[-1])
+    for i in range(len(frames)):
+        assert np.array_equal(outs[i], want[i]), i
+    with pytest.raises(fa.FynException):
+        net.asyncWait(len(frames) + 5)
+    # the synchronous path still works while the pipeline is open, and the pipeline can be reopened
+    net.setInput(frames[2]); net.forward(); net.finish()
+    assert np.array_equal(net.getOutput(net.output_layer), want[2])
+    net.asyncEnd()
+    with pytest.raises(fa.FynException):
+        net.asyncSubmit(frames[0], outs[0])
+    net.asyncBegin(in_layer, net.output_layer, outOrder=fa.capi.ORDER_GPU_SHALLOW, depth=2, inPort=in_port)
+    hwc = np.zeros((80, 96, 4), np.float32)
+    net.asyncWait(net.asyncSubmit(frames[3], hwc))
+    assert np.array_equal(hwc[..., :3].transpose(2, 0, 1), want[3])
+    net.asyncEnd()
+    net.cleanup()
