@@ -6,7 +6,9 @@ LayerBuilder / LayerFactory / NeuralNetwork description surface.  There is no CP
 package without the built library raises ImportError at the first call.
 """
 from . import capi  # noqa: F401
-from .builders import (ActType, ArgMaxLayerBuilder, ConcatLayerBuilder, ConvLayerBuilder, GPULayerBuilder,  # noqa: F401
-                       LayerBuilder, LayerFlags, LayerType, NormType, PoolLayerBuilder, UpDownLayerBuilder)
+from .builders import (ActType, ArgMaxLayerBuilder, ArithType, BlurKernelType, BlurLayerBuilder, CastLayerBuilder,  # noqa: F401
+                       CastTarget, ConcatLayerBuilder, ConvLayerBuilder, GPULayerBuilder, ImgExtractLayerBuilder,
+                       LayerBuilder, LayerFlags, LayerType, NormType, PoolLayerBuilder, ScaleLayerBuilder, ScalingType,
+                       SingletonArithLayerBuilder, TransposeLayerBuilder, UpDownLayerBuilder)
 from .capi import FynException, ORDER_CHANNELWISE, ORDER_GPU_DEEP, ORDER_GPU_SHALLOW, STORAGE_F16, STORAGE_F32  # noqa: F401
 from .network import BufferManager, CompiledLayers, Layer, LayerFactory, NeuralNetwork  # noqa: F401

@@ -7,6 +7,12 @@ PoolLayerBuilder    -> fyusenet/gpu/poollayerbuilder.h
 ConcatLayerBuilder  -> fyusenet/gpu/concatlayerbuilder.h
 ArgMaxLayerBuilder  -> fyusenet/gpu/argmaxlayerbuilder.h
 UpDownLayerBuilder  -> fyusenet/gpu/updownlayerbuilder.h
+ScaleLayerBuilder   -> fyusenet/gpu/scalelayerbuilder.h
+SingletonArithLayerBuilder -> fyusenet/gpu/singleton_arithlayerbuilder.h
+CastLayerBuilder    -> fyusenet/gpu/castlayerbuilder.h
+TransposeLayerBuilder -> fyusenet/gpu/transposelayerbuilder.h
+ImgExtractLayerBuilder -> fyusenet/gpu/imgextractlayerbuilder.h
+BlurLayerBuilder    -> fyusenet/gpu/blurlayerbuilder.h
 
 Method names keep the reference's spelling (inputPadding, prefixAct, ...) so that a network
 description reads like samples/samplenetworks/resnet50.cpp.  A builder only collects fields; the
@@ -38,6 +44,38 @@ class ActType(enum.IntEnum):
     CLIP = 3
     SIGMOID = 4
     TANH = 5
+
+
+class ScalingType(enum.IntEnum):
+    """fyusenet/base/layerflags.h:89-92."""
+    NEAREST = 0
+    LINEAR = 1
+
+
+class BlurKernelType(enum.IntEnum):
+    """fyusenet/base/layerflags.h:99-102."""
+    AVERAGE = 0
+    GAUSSIAN = 1
+
+
+class ArithType(enum.IntEnum):
+    """fyusenet/base/layerflags.h:109-114."""
+    ADD = 0
+    SUB = 1
+    MUL = 2
+    DIV = 3
+
+
+class CastTarget(enum.IntEnum):
+    """fyusenet/base/layerflags.h:121-130."""
+    CT_INT32 = 0
+    CT_INT16 = 1
+    CT_INT8 = 2
+    CT_UINT32 = 3
+    CT_UINT16 = 4
+    CT_UINT8 = 5
+    CT_FLOAT16 = 6
+    CT_FLOAT32 = 7
 
 
 class NormType(enum.IntEnum):
@@ -371,3 +409,114 @@ class UpDownLayerBuilder(GPULayerBuilder):
         super().__init__(name)
         self.direction_ = direction
         self.type_ = LayerType.UPLOAD if direction == self.UPLOAD else LayerType.DOWNLOAD
+
+
+class ScaleLayerBuilder(GPULayerBuilder):
+    """gpu/scalelayerbuilder.h:38-135: integer up-/down-scaling, nearest or linear; also the builder of RELU,
+    CLIP and PADDING2D layers, which the factory maps to a scale layer (gpu/gpulayerfactory.cpp:125-140)."""
+
+    def __init__(self, name):
+        super().__init__(name)
+        self.type_ = LayerType.SCALE2D
+        self.scaleType_ = ScalingType.NEAREST
+        self.rotation_ = 0
+
+    def scaleType(self, typ):
+        self.scaleType_ = ScalingType(typ)
+        return self
+
+    def rotate(self, angle):
+        self.rotation_ = angle
+        return self
+
+    def scale(self, scaleX, scaleY=None):
+        scaleY = scaleX if scaleY is None else scaleY
+        for axis, sc in ((0, scaleX), (1, scaleY)):
+            if sc > 1.0:
+                self.upsample_[axis] = int(sc)
+                if abs(self.upsample_[axis] - sc) > 1e-4:
+                    raise capi.FynException(capi.ERR_INVALID, "Only supporting integer upscales for now")
+            elif sc < 1.0:
+                dn = 1.0 / sc
+                self.downsample_[axis] = int(dn + 1e-6)
+                if abs(self.downsample_[axis] - dn) > 1e-4:
+                    raise capi.FynException(capi.ERR_INVALID, "Only supporting integer downscales for now")
+        return self
+
+    def equal(self):
+        return self.upsample_[0] == self.upsample_[1] and self.downsample_[0] == self.downsample_[1]
+
+    def _fill(self, d):
+        if self.rotation_ % 360 != 0:
+            raise capi.FynException(capi.ERR_UNSUPPORTED, "rotation in scale layers is not supported")
+        d.scale_type = int(self.scaleType_)
+
+
+class SingletonArithLayerBuilder(GPULayerBuilder):
+    def __init__(self, name, optype):
+        super().__init__(name)
+        self.type_ = LayerType.SINGLETON_ARITH
+        self.opType_ = ArithType(optype)
+        self.operand_ = 0.0
+
+    def operand(self, opd):
+        self.operand_ = float(opd)
+        return self
+
+    def _fill(self, d):
+        d.arith_op = int(self.opType_)
+        d.operand = self.operand_
+
+
+class CastLayerBuilder(GPULayerBuilder):
+    def __init__(self, name, target):
+        super().__init__(name)
+        self.type_ = LayerType.CAST
+        self.target_ = CastTarget(target)
+
+    def target(self, tgt):
+        self.target_ = CastTarget(tgt)
+        return self
+
+    def _fill(self, d):
+        d.cast_target = int(self.target_)
+
+
+class TransposeLayerBuilder(GPULayerBuilder):
+    def __init__(self, name):
+        super().__init__(name)
+        self.type_ = LayerType.TRANSPOSE
+
+    def equal(self):
+        return True
+
+
+class ImgExtractLayerBuilder(GPULayerBuilder):
+    def __init__(self, window, name):
+        super().__init__(name)
+        self.type_ = LayerType.IMGEXTRACT
+        self.window_ = window
+        self.downsample_ = [window, window]
+
+    def _fill(self, d):
+        d.window = self.window_
+
+
+class BlurLayerBuilder(GPULayerBuilder):
+    def __init__(self, name):
+        super().__init__(name)
+        self.type_ = LayerType.BLUR2D
+        self.kernel_ = 3
+        self.blurType_ = BlurKernelType.AVERAGE
+
+    def kernel(self, sz):
+        self.kernel_ = sz
+        return self
+
+    def blurType(self, typ):
+        self.blurType_ = BlurKernelType(typ)
+        return self
+
+    def _fill(self, d):
+        d.kernel = self.kernel_
+        d.blur_type = int(self.blurType_)

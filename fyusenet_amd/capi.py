@@ -63,6 +63,12 @@ class LayerDesc(ctypes.Structure):
         ("num_inputs", ctypes.c_int32),
         ("inputs", _ConcatInput * FYN_MAX_CONCAT_INPUTS),
         ("transconv_crop", ctypes.c_int32),
+        ("scale_type", ctypes.c_int32),
+        ("arith_op", ctypes.c_int32),
+        ("operand", ctypes.c_float),
+        ("cast_target", ctypes.c_int32),
+        ("window", ctypes.c_int32),
+        ("blur_type", ctypes.c_int32),
     ]
 
 

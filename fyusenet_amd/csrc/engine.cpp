@@ -124,7 +124,8 @@ void Net::add_layer(const fyn_layer_desc& d) {
     // LayerFactory::pushBuilder (base/layerfactory.cpp:67-76)
     if (d.number < 0) fail(FYN_ERR_INVALID, "Must identify each layer with a valid number (found %d in the builder)", d.number);
     if (layers.count(d.number)) fail(FYN_ERR_DUPLICATE, "Trying to insert a layer on a position that is already taken (%d)", d.number);
-    layers[d.number].reset(create_layer(this, d));
+    std::unique_ptr<Layer> l(create_layer(this, d));   // may throw: nothing is registered then
+    layers[d.number] = std::move(l);
 }
 
 void Net::connect(int out_layer, int in_layer, int port) {

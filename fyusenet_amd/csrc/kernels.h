@@ -155,6 +155,27 @@ struct BnParams {
 };
 void launch_batchnorm(const BnParams& p, hipStream_t s);
 void launch_addsub(const TView& a, const TView& b, const TView& out, int sub, const Act& act, hipStream_t s);
+
+// Function-type layers with one input and no weights.  Every output texel (4 channels) is produced from ONE source
+// texel picked by `map` and passed through `fn`; the stencil modes (linear scaling, non-maximum suppression,
+// blur) have kernels of their own.  Source coordinates beyond the stored input repeat its edge.
+enum FuncMap { FMAP_SCALE = 0, FMAP_TRANSPOSE = 1, FMAP_IMGEXTRACT = 2 };
+enum FuncFn { FFN_COPY = 0, FFN_SIGMOID = 1, FFN_TANH = 2, FFN_ARITH = 3, FFN_CAST = 4, FFN_BGR = 5 };
+struct FuncParams {
+    TView in, out;
+    Act act;
+    int map, fn;
+    int op;          // FFN_ARITH: 0 add, 1 sub, 2 mul, 3 div; FFN_CAST: cast target 0..7
+    float operand;
+    // FMAP_SCALE: source position of output x = ((2x+1)*dx - ox) / (2*ux) texels (floor = nearest)
+    int ux, uy, dx, dy, ox, oy;
+    int window, in_groups;   // FMAP_IMGEXTRACT
+};
+void launch_func(const FuncParams& p, hipStream_t s);
+void launch_scale_linear(const FuncParams& p, hipStream_t s);
+void launch_nonmax(const TView& in, const TView& out, hipStream_t s);
+// coef: device array [k*k] floats, taps (-r..last)^2 with coefficients in running order
+void launch_blur(const TView& in, const TView& out, const float* coef, int r, int last, hipStream_t s);
 // Copies channels [0, in.c) of `in` to channels [c_off, c_off + in.c) of `out` (activated).
 void launch_concat_part(const TView& in, const TView& out, int c_off, const Act& act, hipStream_t s);
 // out: 2 channels (index as float, max value); idx_out optional int32 [h*w].

@@ -1110,6 +1110,136 @@ class AddSubLayer : public Layer {
     std::string info() const override { return "addsub"; }
 };
 
+// Function-type layers with one input and no weights: scale / padding / relu / clip / deep<->shallow conversion
+// (all a scale layer in the reference, gpu/gpulayerfactory.cpp:125-140,471-476), sigmoid, tanh, singleton
+// arithmetic, cast, transpose, image-patch extraction, RGB<->BGR, non-maximum suppression and blur.
+class FuncLayer : public Layer {
+  public:
+    FuncLayer(Net* n, const fyn_layer_desc& d_) : Layer(n, d_) {
+        const bool deep = (d.flags & FYN_FLAG_DEEP) != 0;
+        if (d.flags & FYN_FLAG_RESIDUAL_INPUT) fail(FYN_ERR_UNSUPPORTED, "layer %s: this layer does not support residual input", d.name);
+        oc = d.out_channels > 0 ? d.out_channels : d.in_channels;
+        oh = d.height;
+        ow = d.width;
+        p.map = FMAP_SCALE;
+        p.fn = FFN_COPY;
+        p.ux = p.uy = p.dx = p.dy = 1;
+        switch (d.type) {
+            case FYN_LAYER_SCALE2D:
+            case FYN_LAYER_PADDING2D:
+            case FYN_LAYER_RELU:
+            case FYN_LAYER_CLIP:
+            case FYN_LAYER_DEEP2SHALLOW:
+            case FYN_LAYER_SHALLOW2DEEP: {
+                p.ux = std::max(1, d.upsample[0]); p.uy = std::max(1, d.upsample[1]);
+                p.dx = std::max(1, d.downsample[0]); p.dy = std::max(1, d.downsample[1]);
+                if (d.type != FYN_LAYER_SCALE2D && (p.ux != 1 || p.uy != 1 || p.dx != 1 || p.dy != 1))
+                    fail(FYN_ERR_INVALID, "layer %s: only SCALE2D layers change the spatial size", d.name);
+                if (oc != d.in_channels) fail(FYN_ERR_INVALID, "layer %s: input and output channels differ", d.name);
+                // output size as the tiler / viewport computes it (gpu/deep/deeptiler.cpp:47-48, gpu/scalelayer.cpp:41-44)
+                ow = (int)((float)d.width * ((float)p.ux / (float)p.dx));
+                oh = (int)((float)d.height * ((float)p.uy / (float)p.dy));
+                if (ow < 1 || oh < 1) fail(FYN_ERR_INVALID, "layer %s: scaled size is empty", d.name);
+                // deep tensors: the input quad starts (d-1)/2 texels early (gpu/deep/deeptiler.cpp:97-110)
+                p.ox = deep ? p.ux * (p.dx - 1) : 0;
+                p.oy = deep ? p.uy * (p.dy - 1) : 0;
+                linear = d.type == FYN_LAYER_SCALE2D && d.scale_type == 1;
+                if (d.scale_type != 0 && d.scale_type != 1) fail(FYN_ERR_INVALID, "layer %s: unknown scaling type %d", d.name, d.scale_type);
+                if (deep && (d.width == 1 || d.height == 1)) linear = false;   // gpu/deep/deepscalelayer.cpp:44
+                kind = linear ? "scale-linear" : "scale-nearest";
+                break;
+            }
+            case FYN_LAYER_SIGMOID: p.fn = FFN_SIGMOID; kind = "sigmoid"; break;
+            case FYN_LAYER_TANH: p.fn = FFN_TANH; kind = "tanh"; break;
+            case FYN_LAYER_SINGLETON_ARITH:
+                if (d.arith_op < 0 || d.arith_op > 3) fail(FYN_ERR_INVALID, "layer %s: unknown arithmetic operation %d", d.name, d.arith_op);
+                p.fn = FFN_ARITH; p.op = d.arith_op; p.operand = d.operand; kind = "singleton-arith";
+                break;
+            case FYN_LAYER_CAST:
+                if (d.cast_target < 0 || d.cast_target > 7) fail(FYN_ERR_INVALID, "layer %s: unknown cast target %d", d.name, d.cast_target);
+                p.fn = FFN_CAST; p.op = d.cast_target; kind = "cast";
+                break;
+            case FYN_LAYER_TRANSPOSE:
+                // gpu/gpulayerfactory.cpp (createTransposeLayer): deep tensors only
+                if (!deep) fail(FYN_ERR_UNSUPPORTED, "No shallow transpose layer support (yet)");
+                p.map = FMAP_TRANSPOSE; oh = d.width; ow = d.height; kind = "transpose";
+                break;
+            case FYN_LAYER_IMGEXTRACT:
+                // createImgExtractLayer rejects builders flagged deep (the layer itself works on deep-format tensors)
+                if (deep) fail(FYN_ERR_UNSUPPORTED, "Shallow imgextract currently not supported");
+                if (d.window < 1) fail(FYN_ERR_INVALID, "layer %s: invalid window %d", d.name, d.window);
+                if (d.width % d.window || d.height % d.window)
+                    fail(FYN_ERR_INVALID, "layer %s: size %dx%d is not divisible by window size %d", d.name, d.width, d.height, d.window);
+                p.map = FMAP_IMGEXTRACT; p.window = d.window; p.in_groups = (d.in_channels + 3) / 4;
+                if ((oc + 3) / 4 > p.in_groups * d.window * d.window)
+                    fail(FYN_ERR_INVALID, "layer %s: %d output channels exceed what a %dx%d window of %d channels yields", d.name, oc, d.window, d.window, d.in_channels);
+                oh = d.height / d.window; ow = d.width / d.window; kind = "imgextract";
+                break;
+            case FYN_LAYER_RGB2BGR:
+                if (deep) fail(FYN_ERR_UNSUPPORTED, "Deep rgb->bgr currently not supported");
+                p.fn = FFN_BGR; kind = "rgb2bgr";
+                break;
+            case FYN_LAYER_NONMAX2D:
+                if (deep) fail(FYN_ERR_UNSUPPORTED, "Deep nonmax suppression currently not supported");
+                kind = "nonmax2d";
+                break;
+            case FYN_LAYER_BLUR2D:
+                if (deep) fail(FYN_ERR_UNSUPPORTED, "Deep blurring currently not supported");
+                if ((d.kernel & 1) == 0) fail(FYN_ERR_INVALID, "This layer only supports odd kernel sizes");
+                if (d.kernel < 3 || d.kernel > 15) fail(FYN_ERR_UNSUPPORTED, "layer %s: blur kernel size %d outside 3..15", d.name, d.kernel);
+                if (d.blur_type != 0 && d.blur_type != 1) fail(FYN_ERR_INVALID, "layer %s: unknown blur kernel type %d", d.name, d.blur_type);
+                kind = "blur2d";
+                break;
+            default: fail(FYN_ERR_UNSUPPORTED, "Unsupported layer type %d", d.type);
+        }
+        if (d.type != FYN_LAYER_IMGEXTRACT && oc != d.in_channels) fail(FYN_ERR_INVALID, "layer %s: input and output channels differ", d.name);
+    }
+    void setup() override {
+        p.in = tin(0).v;
+        p.out = tout().v;
+        p.act = act();
+        if (d.type == FYN_LAYER_BLUR2D) {
+            // gpu/blurlayer.cpp:86-113 in its own float arithmetic
+            const int k = d.kernel;
+            std::vector<float> coef((size_t)k * k);
+            if (d.blur_type == 0) {
+                const float c = 1.0f / (float)(k * k);
+                for (float& v : coef) v = c;
+            } else {
+                std::vector<float> g(k);
+                const float fac = (float)(1.0 / std::sqrt(2.0 * 3.14159265358979323846));
+                for (int i = 0; i < k; i++) {
+                    const float x = (float)(i - (k - 1) / 2);
+                    g[i] = fac * expf(-(x * x));
+                }
+                float denom = 0.f;
+                for (int y = 0; y < k; y++)
+                    for (int x = 0; x < k; x++) {
+                        coef[(size_t)y * k + x] = g[y] * g[x];
+                        denom += coef[(size_t)y * k + x];
+                    }
+                for (float& v : coef) v /= denom;
+            }
+            coef_dev = upload(net, coef);
+        }
+    }
+    void forward(hipStream_t s) override {
+        if (d.type == FYN_LAYER_NONMAX2D) launch_nonmax(p.in, p.out, s);
+        else if (d.type == FYN_LAYER_BLUR2D) {
+            // shaders/generickernel.frag:83-107: 3x3 visits (-1..1)^2; larger kernels stop one short of the last
+            // row and column and take the coefficients in running order
+            const int r = (d.kernel - 1) / 2;
+            launch_blur(p.in, p.out, coef_dev, r, d.kernel == 3 ? r : r - 1, s);
+        } else if (linear) launch_scale_linear(p, s);
+        else launch_func(p, s);
+    }
+    std::string info() const override { return kind; }
+    FuncParams p{};
+    bool linear = false;
+    const char* kind = "function";
+    float* coef_dev = nullptr;
+};
+
 class ConcatLayer : public Layer {
   public:
     ConcatLayer(Net* n, const fyn_layer_desc& d_) : Layer(n, d_) {
@@ -1217,6 +1347,23 @@ Layer* create_layer(Net* net, const fyn_layer_desc& d) {
             if (!(d.flags & FYN_FLAG_DEEP)) fail(FYN_ERR_UNSUPPORTED, "ArgMax layer is only supported on deep tensors (%s)", d.name);
             l = new ArgMaxLayer(net, d);
             break;
+        case FYN_LAYER_SCALE2D:
+        case FYN_LAYER_PADDING2D:
+        case FYN_LAYER_RELU:
+        case FYN_LAYER_CLIP:
+        case FYN_LAYER_DEEP2SHALLOW:
+        case FYN_LAYER_SHALLOW2DEEP:
+        case FYN_LAYER_SIGMOID:
+        case FYN_LAYER_TANH:
+        case FYN_LAYER_SINGLETON_ARITH:
+        case FYN_LAYER_CAST:
+        case FYN_LAYER_TRANSPOSE:
+        case FYN_LAYER_IMGEXTRACT:
+        case FYN_LAYER_RGB2BGR:
+        case FYN_LAYER_NONMAX2D:
+        case FYN_LAYER_BLUR2D: l = new FuncLayer(net, d); break;
+        case FYN_LAYER_FRACCONVOLUTION2D:
+            fail(FYN_ERR_UNSUPPORTED, "fractional convolution (%s) is not supported: its sampling positions fall on texel boundaries of the nearest-neighbour filter", d.name);
         case FYN_LAYER_UPLOAD: l = new UploadLayer(net, d); break;
         case FYN_LAYER_DOWNLOAD: l = new DownloadLayer(net, d); break;
         default: fail(FYN_ERR_UNSUPPORTED, "Unsupported layer type %d", d.type);

@@ -246,6 +246,180 @@ void launch_batchnorm(const BnParams& p, hipStream_t s) {
     FYN_DISPATCH_T(p.out.f16, batchnorm_kernel, grid1d(n, 256), dim3(256), s, p);
 }
 
+// ---------------------------------------------------------------------------------------------
+// function-type layers: scale / padding / relu / clip / deep<->shallow (shaders/deep/deepdefault.frag, scaling.frag),
+// sigmoid (deepsigmoid.frag), tanh (deeptanh.frag), singleton arithmetic (deep_singleton_arith.frag), cast
+// (typecast.inc), transpose (deeptransposelayer.cpp:141-156), image-patch extraction (deepimgpatch.frag),
+// RGB<->BGR (rgb2bgr.frag), non-maximum suppression (nonmax2d.frag), blur (generickernel.frag)
+// ---------------------------------------------------------------------------------------------
+__device__ __forceinline__ int floordiv_pos(int a, int b) { return a >= 0 ? a / b : -((-a + b - 1) / b); }
+
+// Texel at stored coordinates, edge repeated beyond the stored tensor; channels >= in.c read as zero.
+template <typename T>
+__device__ __forceinline__ float4 fetch_clamped(const TView& t, int sy, int sx, int c) {
+    sy = min(max(sy, 0), t.hp() - 1);
+    sx = min(max(sx, 0), t.wp() - 1);
+    float4 v = ld4<T>(reinterpret_cast<const T*>(t.ptr) + ((size_t)sy * t.wp() + sx) * t.cp + c);
+    if (c + 3 >= t.c) {
+        if (c + 0 >= t.c) v.x = 0.f;
+        if (c + 1 >= t.c) v.y = 0.f;
+        if (c + 2 >= t.c) v.z = 0.f;
+        if (c + 3 >= t.c) v.w = 0.f;
+    }
+    return v;
+}
+
+__device__ __forceinline__ float4 mask_channels(float4 v, int c, int nc) {
+    if (c + 3 >= nc) {
+        if (c + 0 >= nc) v.x = 0.f;
+        if (c + 1 >= nc) v.y = 0.f;
+        if (c + 2 >= nc) v.z = 0.f;
+        if (c + 3 >= nc) v.w = 0.f;
+    }
+    return v;
+}
+
+__device__ __forceinline__ float func1(float x, int fn, int op, float operand) {
+    switch (fn) {
+        case FFN_SIGMOID: return 1.0f / (1.0f + expf(-x));
+        case FFN_TANH: return tanhf(x);
+        case FFN_ARITH: return op == 0 ? x + operand : op == 1 ? x - operand : op == 2 ? x * operand : x / operand;
+        case FFN_CAST: {
+            if (op == 7) return x;
+            if (op == 6) return (float)(_Float16)x;
+            const float r = rintf(x);   // ties to even
+            switch (op) {
+                case 0: return fminf(fmaxf(r, -2147483648.0f), 2147483647.0f);
+                case 1: return fminf(fmaxf(r, -32768.0f), 32767.0f);
+                case 2: return fminf(fmaxf(r, -128.0f), 127.0f);
+                case 3: return fminf(fmaxf(r, 0.0f), 4294967295.0f);
+                case 4: return fminf(fmaxf(r, 0.0f), 65535.0f);
+                default: return fminf(fmaxf(r, 0.0f), 255.0f);
+            }
+        }
+        default: return x;
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void func_kernel(const FuncParams p) {
+    const int cg = p.out.cp >> 2;
+    const size_t n = (size_t)p.out.h * p.out.w * cg;
+    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= n) return;
+    const int g = (int)(idx % cg);
+    const size_t pix = idx / cg;
+    const int x = (int)(pix % p.out.w), y = (int)(pix / p.out.w);
+    int sy, sx, sg = g;
+    if (p.map == FMAP_TRANSPOSE) {
+        sy = x;
+        sx = y;
+    } else if (p.map == FMAP_IMGEXTRACT) {
+        const int b = g / p.in_groups;
+        sg = g - b * p.in_groups;
+        sy = y * p.window + b / p.window;
+        sx = x * p.window + b % p.window;
+    } else {
+        sy = floordiv_pos((2 * y + 1) * p.dy - p.oy, 2 * p.uy);
+        sx = floordiv_pos((2 * x + 1) * p.dx - p.ox, 2 * p.ux);
+    }
+    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (sg * 4 < p.in.cp) v = fetch_clamped<T>(p.in, sy + p.in.pad, sx + p.in.pad, sg * 4);
+    if (p.fn == FFN_BGR) {
+        const float t = v.x;
+        v.x = v.z;
+        v.z = t;
+    } else {
+        v = act4(v, p.act);
+        if (p.fn != FFN_COPY)
+            v = make_float4(func1(v.x, p.fn, p.op, p.operand), func1(v.y, p.fn, p.op, p.operand),
+                            func1(v.z, p.fn, p.op, p.operand), func1(v.w, p.fn, p.op, p.operand));
+    }
+    st4<T>(reinterpret_cast<T*>(p.out.ptr) + tv_off(p.out, y, x) + g * 4, mask_channels(v, g * 4, p.out.c));
+}
+void launch_func(const FuncParams& p, hipStream_t s) {
+    const size_t n = (size_t)p.out.h * p.out.w * (p.out.cp >> 2);
+    FYN_DISPATCH_T(p.out.f16, func_kernel, grid1d(n, 256), dim3(256), s, p);
+}
+
+// Bilinear scaling: the raw texels around position ((2x+1)*dx - ox)/(2*ux) - 1/2 are blended, then activated.
+template <typename T>
+__global__ __launch_bounds__(256) void scale_linear_kernel(const FuncParams p) {
+    const int cg = p.out.cp >> 2;
+    const size_t n = (size_t)p.out.h * p.out.w * cg;
+    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= n) return;
+    const int g = (int)(idx % cg);
+    const size_t pix = idx / cg;
+    const int x = (int)(pix % p.out.w), y = (int)(pix / p.out.w);
+    const int ny = (2 * y + 1) * p.dy - p.oy - p.uy, nx = (2 * x + 1) * p.dx - p.ox - p.ux;
+    const int y0 = floordiv_pos(ny, 2 * p.uy), x0 = floordiv_pos(nx, 2 * p.ux);
+    const float fy = (float)(ny - y0 * 2 * p.uy) / (float)(2 * p.uy), fx = (float)(nx - x0 * 2 * p.ux) / (float)(2 * p.ux);
+    const int c = g * 4, sy = y0 + p.in.pad, sx = x0 + p.in.pad;
+    const float4 a = fetch_clamped<T>(p.in, sy, sx, c), b = fetch_clamped<T>(p.in, sy, sx + 1, c);
+    const float4 cc = fetch_clamped<T>(p.in, sy + 1, sx, c), d = fetch_clamped<T>(p.in, sy + 1, sx + 1, c);
+    const float w00 = (1.f - fy) * (1.f - fx), w01 = (1.f - fy) * fx, w10 = fy * (1.f - fx), w11 = fy * fx;
+    float4 v = make_float4(w00 * a.x + w01 * b.x + w10 * cc.x + w11 * d.x, w00 * a.y + w01 * b.y + w10 * cc.y + w11 * d.y,
+                           w00 * a.z + w01 * b.z + w10 * cc.z + w11 * d.z, w00 * a.w + w01 * b.w + w10 * cc.w + w11 * d.w);
+    v = act4(v, p.act);
+    st4<T>(reinterpret_cast<T*>(p.out.ptr) + tv_off(p.out, y, x) + c, mask_channels(v, c, p.out.c));
+}
+void launch_scale_linear(const FuncParams& p, hipStream_t s) {
+    const size_t n = (size_t)p.out.h * p.out.w * (p.out.cp >> 2);
+    FYN_DISPATCH_T(p.out.f16, scale_linear_kernel, grid1d(n, 256), dim3(256), s, p);
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void nonmax_kernel(const TView in, const TView out) {
+    const int cg = out.cp >> 2;
+    const size_t n = (size_t)out.h * out.w * cg;
+    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= n) return;
+    const int g = (int)(idx % cg);
+    const size_t pix = idx / cg;
+    const int x = (int)(pix % out.w), y = (int)(pix / out.w);
+    const int c = g * 4, sy = y + in.pad, sx = x + in.pad;
+    const float4 m = fetch_clamped<T>(in, sy, sx, c);
+    const float4 r = fetch_clamped<T>(in, sy, sx + 1, c), l = fetch_clamped<T>(in, sy, sx - 1, c);
+    const float4 t = fetch_clamped<T>(in, sy - 1, sx, c), b = fetch_clamped<T>(in, sy + 1, sx, c);
+    float4 v;
+    v.x = (m.x >= r.x && m.x >= l.x && m.x >= t.x && m.x >= b.x && m.x > 0.1f) ? m.x : 0.f;
+    v.y = (m.y >= r.y && m.y >= l.y && m.y >= t.y && m.y >= b.y && m.y > 0.1f) ? m.y : 0.f;
+    v.z = (m.z >= r.z && m.z >= l.z && m.z >= t.z && m.z >= b.z && m.z > 0.1f) ? m.z : 0.f;
+    v.w = (m.w >= r.w && m.w >= l.w && m.w >= t.w && m.w >= b.w && m.w > 0.1f) ? m.w : 0.f;
+    st4<T>(reinterpret_cast<T*>(out.ptr) + tv_off(out, y, x) + c, v);
+}
+void launch_nonmax(const TView& in, const TView& out, hipStream_t s) {
+    const size_t n = (size_t)out.h * out.w * (out.cp >> 2);
+    FYN_DISPATCH_T(out.f16, nonmax_kernel, grid1d(n, 256), dim3(256), s, in, out);
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void blur_kernel(const TView in, const TView out, const float* __restrict__ coef, int r, int last) {
+    const int cg = out.cp >> 2;
+    const size_t n = (size_t)out.h * out.w * cg;
+    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= n) return;
+    const int g = (int)(idx % cg);
+    const size_t pix = idx / cg;
+    const int x = (int)(pix % out.w), y = (int)(pix / out.w);
+    const int c = g * 4;
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    int kidx = 0;
+    for (int oy = -r; oy <= last; oy++)
+        for (int ox = -r; ox <= last; ox++) {
+            const float w = coef[kidx++];
+            const float4 v = fetch_clamped<T>(in, y + in.pad + oy, x + in.pad + ox, c);
+            acc.x = fmaf(w, v.x, acc.x); acc.y = fmaf(w, v.y, acc.y);
+            acc.z = fmaf(w, v.z, acc.z); acc.w = fmaf(w, v.w, acc.w);
+        }
+    st4<T>(reinterpret_cast<T*>(out.ptr) + tv_off(out, y, x) + c, acc);
+}
+void launch_blur(const TView& in, const TView& out, const float* coef, int r, int last, hipStream_t s) {
+    const size_t n = (size_t)out.h * out.w * (out.cp >> 2);
+    FYN_DISPATCH_T(out.f16, blur_kernel, grid1d(n, 256), dim3(256), s, in, out, coef, r, last);
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void addsub_kernel(const TView a, const TView b, const TView out, int sub, const Act act) {
     const int cg = out.cp >> 2;

@@ -43,11 +43,27 @@ enum fyn_layer_type {
     FYN_LAYER_ADD = 1,
     FYN_LAYER_SUB = 2,
     FYN_LAYER_ARGMAX = 3,
+    FYN_LAYER_CAST = 4,
     FYN_LAYER_CONCAT = 5,
     FYN_LAYER_CONVOLUTION2D = 6,
+    FYN_LAYER_FRACCONVOLUTION2D = 7, /* known, always rejected with FYN_ERR_UNSUPPORTED */
     FYN_LAYER_TRANSCONVOLUTION2D = 8,
     FYN_LAYER_AVGPOOL2D = 9,
     FYN_LAYER_MAXPOOL2D = 10,
+    FYN_LAYER_PADDING2D = 11,
+    FYN_LAYER_SCALE2D = 12,
+    FYN_LAYER_SINGLETON_ARITH = 13,
+    FYN_LAYER_RELU = 14,
+    FYN_LAYER_CLIP = 15,
+    FYN_LAYER_TANH = 16,
+    FYN_LAYER_SIGMOID = 17,
+    FYN_LAYER_TRANSPOSE = 19,
+    FYN_LAYER_IMGEXTRACT = 20,
+    FYN_LAYER_BLUR2D = 21,
+    FYN_LAYER_NONMAX2D = 22,
+    FYN_LAYER_RGB2BGR = 23,
+    FYN_LAYER_DEEP2SHALLOW = 24,
+    FYN_LAYER_SHALLOW2DEEP = 25,
     FYN_LAYER_DOWNLOAD = 26,
     FYN_LAYER_UPLOAD = 27,
     FYN_LAYER_BATCHNORM = 30,
@@ -81,8 +97,8 @@ enum fyn_order {
 
 /*
  * One layer description: the fields of LayerBuilderTempl (fyusenet/base/layerbuilder.h:497-521) plus
- * those of ConvLayerBuilder (gpu/convlayerbuilder.h), PoolLayerBuilder (gpu/poollayerbuilder.h) and
- * ConcatLayerBuilder (gpu/concatlayerbuilder.h).  The struct is copied by fyn_net_add_layer; no
+ * those of ConvLayerBuilder (gpu/convlayerbuilder.h), PoolLayerBuilder (gpu/poollayerbuilder.h),
+ * ConcatLayerBuilder (gpu/concatlayerbuilder.h) and the builders of the function-type layers.  The struct is copied by fyn_net_add_layer; no
  * ownership is taken.  Zero-initialise it, set struct_size = sizeof(fyn_layer_desc), fill what the
  * builder would have filled.  width/height/in_channels describe the INPUT tensor, as shape() does.
  */
@@ -116,6 +132,13 @@ typedef struct fyn_layer_desc {
      * (gpu/deep/deeptiler.cpp:71-74), 1 with K=3 yields the 2H size of the shallow layer
      * (gpu/vanilla/transconvlayerbase_vanilla.cpp:61-62). */
     int32_t transconv_crop;
+    /* function-type layers */
+    int32_t scale_type;  /* SCALE2D: ScalingType 0 nearest, 1 linear      ScaleLayerBuilder::scaleType() (gpu/scalelayerbuilder.h) */
+    int32_t arith_op;    /* SINGLETON_ARITH: ArithType 0 add 1 sub 2 mul 3 div  (gpu/singleton_arithlayerbuilder.h)             */
+    float operand;       /*                                                SingletonArithLayerBuilder::operand()                */
+    int32_t cast_target; /* CAST: CastTarget 0..7 (base/layerflags.h:121-130)  CastLayerBuilder::target()                       */
+    int32_t window;      /* IMGEXTRACT: window size                        ImgExtractLayerBuilder (gpu/imgextractlayerbuilder.h) */
+    int32_t blur_type;   /* BLUR2D: BlurKernelType 0 average, 1 Gaussian; size in `kernel`  (gpu/blurlayerbuilder.h)            */
 } fyn_layer_desc;
 
 /* Thread-local text of the last failure (what the reference would have thrown). */

@@ -25,6 +25,17 @@
  *   fyo_concat        memcpy identity
  *   fyo_deep_*        round trip + hand-computed tilings           (parity unpinned against the
  *                     reference binary: cpubuffershape.cpp needs the GL wrapper to link)
+ *   fyo_unary         arithmetic: reference patterns arithtests.cpp:205-234; sigmoid/tanh: scipy expit /
+ *                     numpy tanh fp64; cast: numpy rint + clip (exact halves: parity unpinned, GLSL
+ *                     leaves the tie direction open)
+ *   fyo_scale         nearest: numpy repeat / strided slices; linear: torch interpolate(bilinear,
+ *                     align_corners=False) fp64 on the stored array, avg_pool2d for the shallow halving
+ *                     (no reference test exists; GL's fixed-point filter weights: parity unpinned)
+ *   fyo_transpose     numpy transpose, involution
+ *   fyo_imgextract    numpy reshape/transpose space-to-depth + brute force for partial groups
+ *   fyo_nonmax        scipy maximum_filter with the cross footprint
+ *   fyo_blur          scipy correlate for 3x3; literal loop restatement for larger kernels
+ *   fyo_rgb2bgr       index permutation
  */
 #include <math.h>
 #include <stdint.h>
@@ -480,5 +491,213 @@ int fyo_chw_to_shallow(const float* chw, int c, int h, int w, int pc, float* hwc
     memset(hwc, 0, (size_t)h * w * pc * sizeof(float));
     for (int ch = 0; ch < c; ch++)
         for (size_t p = 0; p < (size_t)h * w; p++) hwc[p * pc + ch] = chw[(size_t)ch * h * w + p];
+    return 0;
+}
+
+/* ---------------------------------------------------------------------------------------------
+ * Function-type layers (one input, no weights).
+ * ------------------------------------------------------------------------------------------- */
+
+/* Floor division for a positive divisor. */
+static inline long fyo_floordiv(long a, long b) { return a >= 0 ? a / b : -((-a + b - 1) / b); }
+
+/* Element-wise functions of the activated input; n elements.
+ *   fn 0  copy                    shaders/deep/deepdefault.frag:20-22 (also RELU/CLIP/PADDING2D layers, which the
+ *                                 factory maps to a scale layer of factor 1, gpu/gpulayerfactory.cpp:125-140)
+ *   fn 1  sigmoid 1/(1+exp(-x))   shaders/deep/deepsigmoid.frag:19-22
+ *   fn 2  tanh, written there as 2*(e^{2x}/(1+e^{2x}))-1   shaders/deep/deeptanh.frag:19-22
+ *   fn 3  x (op) operand, op = ArithType 0 add, 1 sub, 2 mul, 3 div   shaders/deep/deep_singleton_arith.frag:21-39
+ *   fn 4  cast: op = CastTarget 0..5 (int32, int16, int8, uint32, uint16, uint8): round, then clamp to the
+ *         type's range, result kept as float; 6 (float16): value rounded to fp16; 7 (float32): unchanged
+ *         (shaders/typecast.inc:10-35, shaders/deep/deepcast.frag:20-27).  GLSL leaves the direction of
+ *         round() at exact halves to the implementation; ties go to even here. */
+int fyo_unary(const float* in, size_t n, int fn, int op, float operand, int act, float leak, float lo, float hi,
+              float* out) {
+    static const double cast_lo[6] = {-2147483648.0, -32768.0, -128.0, 0.0, 0.0, 0.0};
+    static const double cast_hi[6] = {2147483647.0, 32767.0, 127.0, 4294967295.0, 65535.0, 255.0};
+    for (size_t i = 0; i < n; i++) {
+        const double x = (double)fyo_activate(in[i], act, leak, lo, hi);
+        double r = x;
+        switch (fn) {
+            case 0: break;
+            case 1: r = 1.0 / (1.0 + exp(-x)); break;
+            case 2: r = tanh(x); break;
+            case 3:
+                if (op == 0) r = x + (double)operand;
+                else if (op == 1) r = x - (double)operand;
+                else if (op == 2) r = x * (double)operand;
+                else if (op == 3) r = x / (double)operand;
+                else return -1;
+                break;
+            case 4:
+                if (op >= 0 && op < 6) {
+                    r = nearbyint(x);
+                    if (r < cast_lo[op]) r = cast_lo[op];
+                    if (r > cast_hi[op]) r = cast_hi[op];
+                } else if (op == 6) {
+                    float xf = (float)x, hf;
+                    fyo_round_fp16(&xf, 1, &hf);
+                    r = (double)hf;
+                } else if (op != 7) {
+                    return -1;
+                }
+                break;
+            default: return -1;
+        }
+        out[i] = (float)r;
+    }
+    return 0;
+}
+
+/* Scale layer: integer up- or down-scaling with nearest or bilinear sampling
+ * (gpu/deep/deepscalelayer.cpp:41-96, gpu/scalelayer.cpp:38-108, shaders/deep/deepdefault.frag, shaders/scaling.frag).
+ * The sampling position of output column x in input texel units, relative to the first net texel, is what the
+ * proxy polygon's texture coordinates interpolate to:
+ *   deep    (x + 1/2) * d/u - (d - 1)/2     (gpu/deep/deeptiler.cpp:97-110: the quad starts (d-1)/2 texels early)
+ *   shallow (x + 1/2) * d/u                 (gpu/functionlayer.cpp:194-219)
+ * Nearest takes the texel containing that position, linear blends the two texels around it (per axis) with
+ * GL_LINEAR weights; the RAW texels are blended and the activation is applied to the result.  Texels outside the
+ * net area are the stored halo (zero) where the input has padding, beyond the stored texture the edge is repeated
+ * (GL_CLAMP_TO_EDGE).  in_stored [c][hs][ws] with halo pad; out [c][H*uy/dy][W*ux/dx]. */
+int fyo_scale(const float* in_stored, int c, int hs, int ws, int pad, int ux, int uy, int dx, int dy, int linear,
+              int deep, int act, float leak, float lo, float hi, float* out) {
+    if (ux < 1 || uy < 1 || dx < 1 || dy < 1) return -1;
+    const int h = hs - 2 * pad, w = ws - 2 * pad;
+    const int ho = h * uy / dy, wo = w * ux / dx;
+    for (int ch = 0; ch < c; ch++) {
+        const float* plane = in_stored + (size_t)ch * hs * ws;
+        for (int y = 0; y < ho; y++) {
+            const long ny = (long)(2 * y + 1) * dy - (deep ? (long)uy * (dy - 1) : 0);   /* position = ny / (2 uy) */
+            for (int x = 0; x < wo; x++) {
+                const long nx = (long)(2 * x + 1) * dx - (deep ? (long)ux * (dx - 1) : 0);
+                double v;
+                if (!linear) {
+                    const int sy = (int)fyo_floordiv(ny, 2L * uy), sx = (int)fyo_floordiv(nx, 2L * ux);
+                    v = fyo_fetch(plane, hs, ws, sy + pad, sx + pad, 1);
+                } else {
+                    const long y0 = fyo_floordiv(ny - uy, 2L * uy), x0 = fyo_floordiv(nx - ux, 2L * ux);
+                    const double fy = (double)((ny - uy) - y0 * 2L * uy) / (double)(2L * uy);
+                    const double fx = (double)((nx - ux) - x0 * 2L * ux) / (double)(2L * ux);
+                    const double a = fyo_fetch(plane, hs, ws, (int)y0 + pad, (int)x0 + pad, 1);
+                    const double b = fyo_fetch(plane, hs, ws, (int)y0 + pad, (int)x0 + 1 + pad, 1);
+                    const double cc = fyo_fetch(plane, hs, ws, (int)y0 + 1 + pad, (int)x0 + pad, 1);
+                    const double d = fyo_fetch(plane, hs, ws, (int)y0 + 1 + pad, (int)x0 + 1 + pad, 1);
+                    v = (1.0 - fy) * ((1.0 - fx) * a + fx * b) + fy * ((1.0 - fx) * cc + fx * d);
+                }
+                out[((size_t)ch * ho + y) * wo + x] = fyo_activate((float)v, act, leak, lo, hi);
+            }
+        }
+    }
+    return 0;
+}
+
+/* Spatial transposition out[c][x][y] = act(in[c][y][x]) (gpu/deep/deeptransposelayer.cpp:141-156: the input quad's
+ * texture coordinates are attached to the output quad in transposed vertex order). */
+int fyo_transpose(const float* in, int c, int h, int w, int act, float leak, float lo, float hi, float* out) {
+    for (int ch = 0; ch < c; ch++)
+        for (int y = 0; y < h; y++)
+            for (int x = 0; x < w; x++)
+                out[((size_t)ch * w + x) * h + y] = fyo_activate(in[((size_t)ch * h + y) * w + x], act, leak, lo, hi);
+    return 0;
+}
+
+/* Image-patch extraction (space to depth) with window n (gpu/deep/deepextractimgpatches.cpp:150-186,
+ * shaders/deep/deepimgpatch.frag:28-33): output 4-channel group g takes input group g mod G (G = groups of the
+ * input) at in-window offset (xpix, ypix) = (b mod n, b / n), b = g / G; out(y, x) = act(in(y*n + ypix, x*n + xpix)).
+ * Channels of an input group beyond cin read as zero.  in [cin][h][w], out [cout][h/n][w/n]. */
+int fyo_imgextract(const float* in, int cin, int h, int w, int window, int cout, int act, float leak, float lo,
+                   float hi, float* out) {
+    const int groups = (cin + 3) / 4, ho = h / window, wo = w / window;
+    if (window < 1 || (cout + 3) / 4 > groups * window * window) return -1;
+    for (int o = 0; o < cout; o++) {
+        const int g = o / 4, j = o % 4, b = g / groups, src = (g % groups) * 4 + j;
+        const int xpix = b % window, ypix = b / window;
+        for (int y = 0; y < ho; y++)
+            for (int x = 0; x < wo; x++) {
+                const float v = src < cin ? in[((size_t)src * h + y * window + ypix) * w + x * window + xpix] : 0.f;
+                out[((size_t)o * ho + y) * wo + x] = fyo_activate(v, act, leak, lo, hi);
+            }
+    }
+    return 0;
+}
+
+/* 2D non-maximum suppression over the 4-neighbourhood (shaders/nonmax2d.frag:88-101): a value survives if it is
+ * >= its left, right, upper and lower neighbour and > 0.1, everything else becomes 0.  No activation.  Neighbours
+ * outside the net area are the stored halo, beyond the stored texture the edge is repeated. */
+int fyo_nonmax(const float* in_stored, int c, int hs, int ws, int pad, float* out) {
+    const int h = hs - 2 * pad, w = ws - 2 * pad;
+    for (int ch = 0; ch < c; ch++) {
+        const float* p = in_stored + (size_t)ch * hs * ws;
+        for (int y = 0; y < h; y++)
+            for (int x = 0; x < w; x++) {
+                const int sy = y + pad, sx = x + pad;
+                const float m = p[(size_t)sy * ws + sx];
+                const int keep = m >= fyo_fetch(p, hs, ws, sy, sx + 1, 1) && m >= fyo_fetch(p, hs, ws, sy, sx - 1, 1) &&
+                                 m >= fyo_fetch(p, hs, ws, sy - 1, sx, 1) && m >= fyo_fetch(p, hs, ws, sy + 1, sx, 1) &&
+                                 m > 0.1f;
+                out[((size_t)ch * h + y) * w + x] = keep ? m : 0.f;
+            }
+    }
+    return 0;
+}
+
+/* Blur layer coefficients (gpu/blurlayer.cpp:86-113): box = 1/k^2; Gaussian = outer product of
+ * exp(-x^2)/sqrt(2 pi), x = i - (k-1)/2, normalised to sum 1.  coef [k*k] row-major. */
+int fyo_blur_coeffs(int k, int gaussian, float* coef) {
+    if (k < 1 || !(k & 1)) return -1;
+    if (!gaussian) {
+        for (int i = 0; i < k * k; i++) coef[i] = 1.0f / (float)(k * k);
+        return 0;
+    }
+    float g[64];
+    if (k > 63) return -1;
+    const float fac = (float)(1.0 / sqrt(2.0 * 3.14159265358979323846));
+    for (int i = 0; i < k; i++) {
+        const float x = (float)(i - (k - 1) / 2);
+        g[i] = fac * expf(-(x * x));
+    }
+    float denom = 0.f;
+    for (int y = 0; y < k; y++)
+        for (int x = 0; x < k; x++) {
+            coef[y * k + x] = g[y] * g[x];
+            denom += coef[y * k + x];
+        }
+    for (int i = 0; i < k * k; i++) coef[i] /= denom;
+    return 0;
+}
+
+/* Blur layer (shaders/generickernel.frag:83-107), no activation.  k == 3: the nine taps (-1..1)^2 with
+ * coefficients in row-major order.  k > 3: the shader's loops run over offsets -(k-1)/2 .. (k-1)/2 - 1 in both
+ * directions (the last row and column of the window are never visited) and take the coefficients in running
+ * order from the start of the k*k array; that is restated literally.  Borders as in fyo_nonmax. */
+int fyo_blur(const float* in_stored, int c, int hs, int ws, int pad, int k, int gaussian, float* out) {
+    float coef[64 * 64];
+    if (k > 15 || fyo_blur_coeffs(k, gaussian, coef) != 0) return -1;   /* MAX_KERNEL_SIZE 15, generickernel.frag:18 */
+    const int h = hs - 2 * pad, w = ws - 2 * pad, r = (k - 1) / 2;
+    const int last = (k == 3) ? r : r - 1;
+    for (int ch = 0; ch < c; ch++) {
+        const float* p = in_stored + (size_t)ch * hs * ws;
+        for (int y = 0; y < h; y++)
+            for (int x = 0; x < w; x++) {
+                double acc = 0.0;
+                int kidx = 0;
+                for (int oy = -r; oy <= last; oy++)
+                    for (int ox = -r; ox <= last; ox++)
+                        acc += (double)coef[kidx++] * (double)fyo_fetch(p, hs, ws, y + pad + oy, x + pad + ox, 1);
+                out[((size_t)ch * h + y) * w + x] = (float)acc;
+            }
+    }
+    return 0;
+}
+
+/* RGB <-> BGR: within every group of four channels the first and third swap (val.bgra, shaders/rgb2bgr.frag:88-92).
+ * No activation.  in/out [c][h][w]; a partner channel beyond c reads as zero. */
+int fyo_rgb2bgr(const float* in, int c, int h, int w, float* out) {
+    const size_t plane = (size_t)h * w;
+    for (int ch = 0; ch < c; ch++) {
+        const int j = ch % 4, src = (j == 0) ? ch + 2 : (j == 2) ? ch - 2 : ch;
+        if (src < c) memcpy(out + ch * plane, in + src * plane, plane * sizeof(float));
+        else memset(out + ch * plane, 0, plane * sizeof(float));
+    }
     return 0;
 }

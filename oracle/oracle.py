@@ -33,7 +33,9 @@ def lib():
         _lib = ctypes.CDLL(LIB_PATH)
         for name in ("fyo_conv2d", "fyo_dwconv", "fyo_transconv", "fyo_gemm", "fyo_maxpool", "fyo_avgpool",
                      "fyo_global_pool", "fyo_batchnorm", "fyo_addsub", "fyo_concat", "fyo_argmax",
-                     "fyo_chw_to_deep", "fyo_deep_to_chw", "fyo_shallow_to_chw", "fyo_chw_to_shallow"):
+                     "fyo_chw_to_deep", "fyo_deep_to_chw", "fyo_shallow_to_chw", "fyo_chw_to_shallow",
+                     "fyo_unary", "fyo_scale", "fyo_transpose", "fyo_imgextract", "fyo_nonmax", "fyo_blur",
+                     "fyo_blur_coeffs", "fyo_rgb2bgr"):
             getattr(_lib, name).restype = ctypes.c_int
     return _lib
 
@@ -197,6 +199,85 @@ def argmax(x, act=None):
     return idx, val
 
 
+FN_COPY, FN_SIGMOID, FN_TANH, FN_ARITH, FN_CAST = 0, 1, 2, 3, 4
+
+
+def unary(x, fn, op=0, operand=0.0, act=None):
+    """Element-wise function layer on an unpadded tensor: copy / sigmoid / tanh / singleton arithmetic / cast."""
+    xv, xp = _f(x)
+    out = np.empty_like(xv)
+    a = _act(act)
+    rc = lib().fyo_unary(xp, ctypes.c_size_t(xv.size), fn, op, ctypes.c_float(operand), a[0], ctypes.c_float(a[1]),
+                         ctypes.c_float(a[2]), ctypes.c_float(a[3]), out.ctypes.data_as(_F))
+    assert rc == 0
+    return out
+
+
+def scale(x_stored, pad_in, up=(1, 1), down=(1, 1), linear=False, deep=True, act=None):
+    """Scale layer; up/down = (x, y) integer factors.  x_stored [c][H+2pad][W+2pad]."""
+    x, xp = _f(x_stored)
+    c, hs, ws = x.shape
+    h, w = hs - 2 * pad_in, ws - 2 * pad_in
+    out = np.empty((c, h * up[1] // down[1], w * up[0] // down[0]), dtype=np.float32)
+    a = _act(act)
+    rc = lib().fyo_scale(xp, c, hs, ws, pad_in, up[0], up[1], down[0], down[1], 1 if linear else 0, 1 if deep else 0,
+                         a[0], ctypes.c_float(a[1]), ctypes.c_float(a[2]), ctypes.c_float(a[3]), out.ctypes.data_as(_F))
+    assert rc == 0
+    return out
+
+
+def transpose(x, act=None):
+    xv, xp = _f(x)
+    c, h, w = xv.shape
+    out = np.empty((c, w, h), dtype=np.float32)
+    a = _act(act)
+    rc = lib().fyo_transpose(xp, c, h, w, a[0], ctypes.c_float(a[1]), ctypes.c_float(a[2]), ctypes.c_float(a[3]),
+                             out.ctypes.data_as(_F))
+    assert rc == 0
+    return out
+
+
+def imgextract(x, window, cout, act=None):
+    xv, xp = _f(x)
+    c, h, w = xv.shape
+    out = np.empty((cout, h // window, w // window), dtype=np.float32)
+    a = _act(act)
+    rc = lib().fyo_imgextract(xp, c, h, w, window, cout, a[0], ctypes.c_float(a[1]), ctypes.c_float(a[2]),
+                              ctypes.c_float(a[3]), out.ctypes.data_as(_F))
+    assert rc == 0
+    return out
+
+
+def nonmax(x_stored, pad_in):
+    x, xp = _f(x_stored)
+    c, hs, ws = x.shape
+    out = np.empty((c, hs - 2 * pad_in, ws - 2 * pad_in), dtype=np.float32)
+    assert lib().fyo_nonmax(xp, c, hs, ws, pad_in, out.ctypes.data_as(_F)) == 0
+    return out
+
+
+def blur_coeffs(k, gaussian):
+    out = np.empty((k, k), dtype=np.float32)
+    assert lib().fyo_blur_coeffs(k, 1 if gaussian else 0, out.ctypes.data_as(_F)) == 0
+    return out
+
+
+def blur(x_stored, pad_in, k, gaussian=False):
+    x, xp = _f(x_stored)
+    c, hs, ws = x.shape
+    out = np.empty((c, hs - 2 * pad_in, ws - 2 * pad_in), dtype=np.float32)
+    assert lib().fyo_blur(xp, c, hs, ws, pad_in, k, 1 if gaussian else 0, out.ctypes.data_as(_F)) == 0
+    return out
+
+
+def rgb2bgr(x):
+    xv, xp = _f(x)
+    c, h, w = xv.shape
+    out = np.empty_like(xv)
+    assert lib().fyo_rgb2bgr(xp, c, h, w, out.ctypes.data_as(_F)) == 0
+    return out
+
+
 def round_fp16(x):
     xv, xp = _f(x)
     out = np.empty_like(xv)
@@ -316,6 +397,30 @@ def run_layer(b, w, ins, f16=False):
     if t == 3:
         idx, val = argmax(get(0, 0), act)
         return np.stack([idx.astype(np.float32), val])
+    if t in (11, 12, 14, 15, 24, 25):   # padding / scale / relu / clip / deep<->shallow: all a scale layer
+        deep = bool(flags & 16)
+        linear = int(getattr(b, "scaleType_", 0)) == 1
+        if deep and (b.width_ == 1 or b.height_ == 1):
+            linear = False                  # gpu/deep/deepscalelayer.cpp:44
+        return scale(get(0, b.inputPadding_), b.inputPadding_, tuple(b.upsample_), tuple(b.downsample_), linear, deep, act)
+    if t == 17:
+        return unary(get(0, 0), FN_SIGMOID, act=act)
+    if t == 16:
+        return unary(get(0, 0), FN_TANH, act=act)
+    if t == 13:
+        return unary(get(0, 0), FN_ARITH, int(b.opType_), float(b.operand_), act)
+    if t == 4:
+        return unary(get(0, 0), FN_CAST, int(b.target_), act=act)
+    if t == 19:
+        return transpose(get(0, 0), act)
+    if t == 20:
+        return imgextract(get(0, 0), b.window_, b.outputChannels_, act)
+    if t == 22:
+        return nonmax(get(0, b.inputPadding_), b.inputPadding_)
+    if t == 21:
+        return blur(get(0, b.inputPadding_), b.inputPadding_, b.kernel_, int(b.blurType_) == 1)
+    if t == 23:
+        return rgb2bgr(get(0, 0))
     raise ValueError("oracle: unsupported layer type %d" % t)
 
 

@@ -25,7 +25,21 @@ def test_library_exports_every_declared_symbol():
 def test_desc_struct_layout_matches_header():
     # 4-byte fields only, no padding: size must equal the sum of the members
     d = capi.LayerDesc()
-    assert ctypes.sizeof(d) == 4 * 3 + 64 + 4 * (1 + 4 + 3 + 2 + 2 + 3 + 1 + 2 + 1 + 2 + 1 + 1) + 12 * 8 + 4
+    assert ctypes.sizeof(d) == 4 * 3 + 64 + 4 * (1 + 4 + 3 + 2 + 2 + 3 + 1 + 2 + 1 + 2 + 1 + 1) + 12 * 8 + 4 + 4 * 6
+    # member names and order as the header declares them
+    import re
+    text = open(os.path.join(ROOT, "include", "fynhip.h")).read()
+    body = text[text.index("typedef struct fyn_layer_desc {"):text.index("} fyn_layer_desc;")]
+    body = re.sub(r"/\*.*?\*/", "", body, flags=re.S).split("{", 1)[1]
+    body = re.sub(r"struct\s*\{[^}]*\}", "struct_t", body)
+    names = []
+    for decl in body.split(";"):
+        decl = decl.strip()
+        if not decl:
+            continue
+        for part in decl.split(None, 1)[1].split(","):
+            names.append(re.sub(r"\[.*", "", part).strip())
+    assert names == [f[0] for f in capi.LayerDesc._fields_]
 
 
 def test_flags_follow_getflags():
