@@ -354,7 +354,15 @@ static std::map<std::string, std::array<int, 6>>& tune_cache() {
     return cache;
 }
 
+// switches that pin part of the choice are for experiments: choices are neither remembered nor recalled then
+static bool tune_cache_bypassed() {
+    for (const char* e : {"FYNHIP_FORCE_KSPLIT", "FYNHIP_CONV_TILE", "FYNHIP_CONV_KC_MAX", "FYNHIP_CONV_PD"})
+        if (getenv(e)) return true;
+    return false;
+}
+
 static const TileChoice* tune_cache_lookup(const char* key, const std::vector<TileChoice>& cands, int* ksplit) {
+    if (tune_cache_bypassed()) return nullptr;
     auto it = tune_cache().find(key);
     if (it == tune_cache().end()) return nullptr;
     for (const TileChoice& c : cands)
@@ -366,6 +374,7 @@ static const TileChoice* tune_cache_lookup(const char* key, const std::vector<Ti
 }
 
 static void tune_cache_store(const char* key, const ConvVariant& v, int ksplit) {
+    if (tune_cache_bypassed()) return;
     tune_cache()[key] = {v.fm, v.fn, v.wm, v.wn, v.kc, ksplit};   // same geometry later in this process: same choice
     const char* path = getenv("FYNHIP_TUNE_CACHE");
     if (!path) return;
