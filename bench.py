@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the GPU layer stack on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload stylenet|resnet50|resnet50ref|conv1|mobilenet|stylenet9x9]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload stylenet|resnet50|resnet50ref|conv1|mobilenet|stylenet9x9|copy|bw-<layer>]
 
 A step is one forward pass of the named network over one synthetic input frame that is already
 resident in HBM (uploaded before the timed region); weights are synthetic (random init).  Prints ONE
@@ -51,7 +51,80 @@ def make_net(workload):
         return networks.SingleConvNet(fa.STORAGE_F32, channels=128, width=128, height=156), "conv3x3 128->128 128x156 us/layer", "us", "fp32 storage"
     if workload == "copy":
         return CopyNet(fa.STORAGE_F32), "copy 64x1024x1024 fp32 GB/s", "GB/s", "fp32"
+    if workload.startswith("bw-"):   # one bandwidth-bound layer at a size far beyond the caches
+        kind = workload[3:]
+        if kind not in BandwidthNet.KINDS:
+            raise SystemExit("unknown workload %s (bw-%s)" % (workload, "|bw-".join(BandwidthNet.KINDS)))
+        return BandwidthNet(kind), "%s 128x1024x1024 fp16 GB/s" % kind, "GB/s", "fp16 storage"
     raise SystemExit("unknown workload %s" % workload)
+
+
+class BandwidthNet(fa.NeuralNetwork):
+    """One layer of a bandwidth-bound class on a 128 x 1024 x 1024 fp16 tensor (268 MB), inputs fed from the host."""
+    KINDS = ("dwconv", "maxpool", "avgpool", "batchnorm", "add", "concat", "scale", "sigmoid")
+    C, S = 128, 1024
+    output_layer = 1
+
+    def __init__(self, kind):
+        super().__init__(fa.STORAGE_F16)
+        self.kind = kind
+        self.input_key = (1, 0)
+
+    def buildLayers(self, f):
+        C, S, k = self.C, self.S, self.kind
+        if k == "dwconv":
+            b = fa.ConvLayerBuilder(3, k).type(fa.LayerType.CONVOLUTION2D).shape(C, S, S, C).groupSize(C).inputPadding(1).prefixAct(fa.ActType.RELU)
+        elif k in ("maxpool", "avgpool"):
+            op = fa.PoolLayerBuilder.POOL_MAX if k == "maxpool" else fa.PoolLayerBuilder.POOL_AVG
+            b = fa.PoolLayerBuilder(op, k).shape(C, S, S, C).poolSize(2).downsample(2)
+        elif k == "batchnorm":
+            b = fa.GPULayerBuilder(k).type(fa.LayerType.BATCHNORM).shape(C, S, S, C).prefixAct(fa.ActType.RELU)
+        elif k == "add":
+            b = fa.GPULayerBuilder(k).type(fa.LayerType.ADD).shape(C, S, S, C)
+        elif k == "concat":
+            b = fa.ConcatLayerBuilder(k).input(C // 2, 0).input(C // 2, 0)
+            b.size(S, S)
+            b.outputChannels_ = C
+        elif k == "scale":
+            b = fa.ScaleLayerBuilder(k).shape(C, S // 2, S // 2, C).scale(2.0)
+        else:
+            b = fa.GPULayerBuilder(k).type(fa.LayerType.SIGMOID).shape(C, S, S, C)
+        if k != "add":
+            b.deep()
+        b.number(1).push(f)
+
+    def connectLayers(self, layers, bm):
+        pass
+
+    def initializeWeights(self, layers):
+        C = self.C
+        if self.kind == "dwconv":
+            layers[1].loadWeightsAndBiases(np.concatenate([np.zeros(C, np.float32), np.full(9 * C, 1.0 / 9.0, np.float32)]), 0)
+        elif self.kind == "batchnorm":
+            layers[1].loadScaleAndBias(np.concatenate([np.full(C, 0.5, np.float32), np.zeros(C, np.float32)]), 0)
+
+    def ports(self):
+        C, S = self.C, self.S
+        if self.kind == "add":
+            return [(C, S, S)] * 2
+        if self.kind == "concat":
+            return [(C // 2, S, S)] * 2
+        if self.kind == "scale":
+            return [(C, S // 2, S // 2)]
+        return [(C, S, S)]
+
+    def makeInput(self):
+        return np.ones(self.ports()[0], np.float32)
+
+    def setInput(self, x):
+        for port, shape in enumerate(self.ports()):
+            self.layers[1].setInput(x if port == 0 else np.ones(shape, np.float32), port)
+
+    def algorithmic_bytes(self):
+        """Bytes one launch has to move: every input element once, every output element once (fp16)."""
+        n_in = sum(c * h * w for c, h, w in self.ports())
+        oc, oh, ow = self.layers[1].outputShape()[:3]
+        return 2 * (n_in + oc * oh * ow)
 
 
 class CopyNet(fa.NeuralNetwork):
@@ -238,7 +311,8 @@ def main():
     elif unit == "us":
         value, hib = ms * 1e3, False
     elif unit == "GB/s":
-        value, hib = 2 * 4 * CopyNet.C * CopyNet.S * CopyNet.S / (ms * 1e-3) / 1e9, True
+        nbytes = net.algorithmic_bytes() if isinstance(net, BandwidthNet) else 2 * 4 * CopyNet.C * CopyNet.S * CopyNet.S
+        value, hib = nbytes / (ms * 1e-3) / 1e9, True
     else:
         value, hib = 1e3 / ms, True
 
@@ -247,12 +321,17 @@ def main():
            "config": {"workload": args.workload, "input": list(x.shape), "batch": 1, "launch": launch,
                       "algorithmic_gflop_per_step": total_flops / 1e9},
            "ms_per_step_graph": ms_graph, "ms_per_step_eager": ms_eager, "roofline": roof}
+    if isinstance(net, BandwidthNet):   # a single bandwidth-bound kernel: the roofline record is the step itself
+        nbytes = net.algorithmic_bytes()
+        ach = nbytes / (roof["avg_launch_us"] * 1e-6) / 1e9
+        roof.update({"bound": "hbm", "achieved": ach, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": ach / PEAK_HBM_GBS,
+                     "algorithmic_bytes_per_launch": nbytes})
 
-    if hasattr(net, "input_key") and args.workload != "copy":
+    if hasattr(net, "input_key") and args.workload != "copy" and not isinstance(net, BandwidthNet):
         out["host_io"] = host_io_rates(net, x, max(args.steps, 50))
         log("host I/O inclusive: %s" % out["host_io"])
 
-    if not args.no_cpu_baseline:
+    if not args.no_cpu_baseline and total_flops > 0:
         dt, flops, threads, lname = cpu_baseline(net, x, total_flops)
         cpu_ms = dt * 1e3 * total_flops / flops
         if unit == "ms/frame":

@@ -1271,7 +1271,10 @@ class ConcatLayer : public Layer {
     }
     void forward(hipStream_t s) override {
         Act a = act();
-        if (relu && a.kind == ACT_NONE) a.kind = ACT_RELU;
+        if (relu && a.kind == ACT_NONE) {
+            a.kind = ACT_RELU;
+            a.lo = 0.f;
+        }
         int off = 0;
         for (int i = 0; i < d.num_inputs; i++) {
             launch_concat_part(tin(i).v, tout().v, off, a, s);

@@ -8,6 +8,8 @@
 #include <hip/hip_fp16.h>
 #include <hip/hip_runtime.h>
 
+#include <cstdlib>
+
 #include "kernels.h"
 
 namespace fynhip {
@@ -16,16 +18,16 @@ typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 
+// Activation on fetch.  The host normalises every kind to act(x) = min(hi, max(lo, x)) + leak * min(x, 0)
+// (none: lo = -inf, hi = +inf, leak = 0; ReLU: lo = 0; leaky: lo = 0, leak; clip: lo, hi), which is evaluated without
+// branches; "none" skips the arithmetic altogether (one uniform branch per vector).
 __device__ __forceinline__ float act1(float x, const Act& a) {
-    switch (a.kind) {
-        case ACT_RELU: return fmaxf(x, 0.f);
-        case ACT_LEAKY: return x >= 0.f ? x : a.leak * x;
-        case ACT_CLIP: return fminf(a.hi, fmaxf(a.lo, x));
-        default: return x;
-    }
+    return (a.kind == ACT_NONE) ? x : fminf(a.hi, fmaxf(a.lo, x)) + a.leak * fminf(x, 0.f);
 }
 __device__ __forceinline__ float4 act4(float4 v, const Act& a) {
-    return make_float4(act1(v.x, a), act1(v.y, a), act1(v.z, a), act1(v.w, a));
+    if (a.kind == ACT_NONE) return v;
+    return make_float4(fminf(a.hi, fmaxf(a.lo, v.x)) + a.leak * fminf(v.x, 0.f), fminf(a.hi, fmaxf(a.lo, v.y)) + a.leak * fminf(v.y, 0.f),
+                       fminf(a.hi, fmaxf(a.lo, v.z)) + a.leak * fminf(v.z, 0.f), fminf(a.hi, fmaxf(a.lo, v.w)) + a.leak * fminf(v.w, 0.f));
 }
 
 template <typename T>
@@ -55,6 +57,63 @@ __device__ __forceinline__ void st4<_Float16>(_Float16* p, float4 v) {
 __device__ __forceinline__ size_t tv_off(const TView& t, int y, int x) {  // net coords -> element offset
     return ((size_t)(y + t.pad) * t.wp() + (x + t.pad)) * t.cp;
 }
+
+// V consecutive channels of one pixel as floats.  fp16 tensors whose channel pitch allows it are moved 8 channels
+// (16 bytes) per thread, everything else 4 channels per thread.
+template <int V>
+struct FV {
+    float v[V];
+};
+template <typename T, int V>
+__device__ __forceinline__ FV<V> ldv(const T* p) {
+    FV<V> r;
+    if constexpr (V == 8 && sizeof(T) == 2) {
+        const half8_t h = *reinterpret_cast<const half8_t*>(p);
+#pragma unroll
+        for (int i = 0; i < 8; i++) r.v[i] = (float)h[i];
+    } else {
+#pragma unroll
+        for (int q = 0; q < V / 4; q++) {
+            const float4 a = ld4<T>(p + 4 * q);
+            r.v[4 * q + 0] = a.x; r.v[4 * q + 1] = a.y; r.v[4 * q + 2] = a.z; r.v[4 * q + 3] = a.w;
+        }
+    }
+    return r;
+}
+template <typename T, int V>
+__device__ __forceinline__ void stv(T* p, const FV<V>& r) {
+    if constexpr (V == 8 && sizeof(T) == 2) {
+        half8_t h;
+#pragma unroll
+        for (int i = 0; i < 8; i++) h[i] = (_Float16)r.v[i];
+        *reinterpret_cast<half8_t*>(p) = h;
+    } else {
+#pragma unroll
+        for (int q = 0; q < V / 4; q++) st4<T>(p + 4 * q, make_float4(r.v[4 * q + 0], r.v[4 * q + 1], r.v[4 * q + 2], r.v[4 * q + 3]));
+    }
+}
+template <int V>
+__device__ __forceinline__ FV<V> zerov() {
+    FV<V> r;
+#pragma unroll
+    for (int i = 0; i < V; i++) r.v[i] = 0.f;
+    return r;
+}
+template <int V>
+__device__ __forceinline__ FV<V> actv(FV<V> r, const Act& a) {
+    if (a.kind == ACT_NONE) return r;
+#pragma unroll
+    for (int i = 0; i < V; i++) r.v[i] = fminf(a.hi, fmaxf(a.lo, r.v[i])) + a.leak * fminf(r.v[i], 0.f);
+    return r;
+}
+
+// wide: every tensor of the launch has a channel pitch that is a multiple of 8
+#define FYN_DISPATCH_TV(f16, wide, KERNEL, grid, block, stream, ...)                                       \
+    do {                                                                                                   \
+        if ((f16) && (wide)) hipLaunchKernelGGL((KERNEL<_Float16, 8>), grid, block, 0, stream, __VA_ARGS__); \
+        else if (f16) hipLaunchKernelGGL((KERNEL<_Float16, 4>), grid, block, 0, stream, __VA_ARGS__);       \
+        else hipLaunchKernelGGL((KERNEL<float, 4>), grid, block, 0, stream, __VA_ARGS__);                  \
+    } while (0)
 
 #define FYN_DISPATCH_T(f16, KERNEL, grid, block, stream, ...)                                   \
     do {                                                                                        \
@@ -107,7 +166,117 @@ __global__ __launch_bounds__(256) void dwconv3x3_kernel(const DwConvParams p) {
     }
     st4<T>(reinterpret_cast<T*>(p.out.ptr) + tv_off(p.out, y, x) + c, o);
 }
+// V stored elements as they come from memory (one 8- or 16-byte load).
+template <typename T, int V>
+struct alignas(sizeof(T) * V) RawV {
+    T v[V];
+};
+
+// Undilated depthwise 3x3, stride S: one thread produces four neighbouring output pixels of V channels from a
+// 3 x ((4-1)*S+3) input window, so that an input texel is fetched once per thread instead of up to three times and
+// the nine weight vectors are loaded once per four outputs.  All loads of the window are issued before the first
+// use (one memory round trip per thread); the texels stay in their stored type until they are consumed.  Same
+// accumulation order per output (ky outer, kx inner, fused multiply-add) as dwconv3x3_kernel.
+template <typename T, int V, int S>
+__global__ __launch_bounds__(256) void dwconv3x3_row_kernel(const DwConvParams p) {
+    constexpr int PX = 4, WIN = (PX - 1) * S + 3;
+    const int cg = p.out.cp / V;
+    const int xb = (p.out.w + PX - 1) / PX;
+    const size_t n = (size_t)p.out.h * xb * cg;
+    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= n) return;
+    const int g = (int)(idx % cg);
+    const size_t t = idx / cg;
+    const int bx = (int)(t % xb), y = (int)(t / xb);
+    const int c = g * V, x0 = bx * PX;
+    const T* in = reinterpret_cast<const T*>(p.in.ptr);
+    const int iwp = p.in.wp(), ihp = p.in.hp();
+    const int sx0 = x0 * S + p.in.pad - 1;
+    RawV<T, V> raw[3][WIN];
+#pragma unroll
+    for (int ky = 0; ky < 3; ky++) {
+        const int sy = y * S + p.in.pad + (ky - 1);
+        const bool row_ok = (unsigned)sy < (unsigned)ihp;
+#pragma unroll
+        for (int j = 0; j < WIN; j++) {
+            const int sx = sx0 + j;
+#pragma unroll
+            for (int i = 0; i < V; i++) raw[ky][j].v[i] = (T)0.f;
+            if (row_ok && (unsigned)sx < (unsigned)iwp) raw[ky][j] = *reinterpret_cast<const RawV<T, V>*>(in + ((size_t)sy * iwp + sx) * p.in.cp + c);
+        }
+    }
+    // min(hi, max(lo, x)) in fp16 equals the fp32 evaluation when there is no leak and both bounds are fp16 values:
+    // then it is applied to the packed halves, two elements per instruction, before the conversion
+    const _Float16 hlo = (_Float16)p.act.lo, hhi = (_Float16)p.act.hi;
+    const bool packed_act = sizeof(T) == 2 && V == 8 && p.act.leak == 0.f && (float)hlo == p.act.lo && (float)hhi == p.act.hi;
+    FV<V> acc[PX];
+#pragma unroll
+    for (int px = 0; px < PX; px++) acc[px] = zerov<V>();
+#pragma unroll
+    for (int ky = 0; ky < 3; ky++) {
+        FV<V> row[WIN];
+#pragma unroll
+        for (int j = 0; j < WIN; j++) {
+            if constexpr (V == 8 && sizeof(T) == 2) {
+                if (packed_act) {
+                    half8_t h = __builtin_bit_cast(half8_t, raw[ky][j]);
+                    h = __builtin_elementwise_min(__builtin_elementwise_max(h, (half8_t)hlo), (half8_t)hhi);
+#pragma unroll
+                    for (int i = 0; i < 8; i++) row[j].v[i] = (float)h[i];
+                    continue;
+                }
+            }
+            FV<V> v;
+#pragma unroll
+            for (int i = 0; i < V; i++) v.v[i] = (float)raw[ky][j].v[i];
+            row[j] = actv<V>(v, p.act);
+        }
+#pragma unroll
+        for (int kx = 0; kx < 3; kx++) {
+            const FV<V> w = ldv<float, V>(p.w + (ky * 3 + kx) * p.out.cp + c);
+#pragma unroll
+            for (int px = 0; px < PX; px++)
+#pragma unroll
+                for (int i = 0; i < V; i++) acc[px].v[i] = fmaf(row[px * S + kx].v[i], w.v[i], acc[px].v[i]);
+        }
+    }
+    const FV<V> sc = ldv<float, V>(p.scale + c), bi = ldv<float, V>(p.bias + c);
+#pragma unroll
+    for (int px = 0; px < PX; px++) {
+        const int x = x0 + px;
+        if (x >= p.out.w) break;
+        FV<V> o;
+#pragma unroll
+        for (int i = 0; i < V; i++) o.v[i] = acc[px].v[i] * sc.v[i] + bi.v[i];
+        if (p.res.ptr) {
+            const FV<V> r = ldv<T, V>(reinterpret_cast<const T*>(p.res.ptr) + tv_off(p.res, y, x) + c);
+#pragma unroll
+            for (int i = 0; i < V; i++) {
+                float rv = r.v[i];
+                if (p.res_relu) rv = fmaxf(rv, 0.f);
+                if (p.res_scale) rv *= sc.v[i];
+                o.v[i] += rv;
+            }
+        }
+        stv<T, V>(reinterpret_cast<T*>(p.out.ptr) + tv_off(p.out, y, x) + c, o);
+    }
+}
+
+template <typename T, int V>
+static void launch_dw_row(const DwConvParams& p, hipStream_t s) {
+    const size_t n = (size_t)p.out.h * ((p.out.w + 3) / 4) * (p.out.cp / V);
+    if (p.stride == 1) hipLaunchKernelGGL((dwconv3x3_row_kernel<T, V, 1>), grid1d(n, 256), dim3(256), 0, s, p);
+    else hipLaunchKernelGGL((dwconv3x3_row_kernel<T, V, 2>), grid1d(n, 256), dim3(256), 0, s, p);
+}
+
 void launch_dwconv3x3(const DwConvParams& p, hipStream_t s) {
+    if (p.dil == 1 && (p.stride == 1 || p.stride == 2) && p.out.w >= 4) {
+        const bool wide = (p.in.cp % 8 == 0) && (p.out.cp % 8 == 0) && (!p.res.ptr || p.res.cp % 8 == 0);
+        if (p.out.f16 && wide) launch_dw_row<_Float16, 8>(p, s);
+        else if (p.out.f16) launch_dw_row<_Float16, 4>(p, s);
+        else launch_dw_row<float, 4>(p, s);
+        return;
+    }
     const size_t n = (size_t)p.out.h * p.out.w * (p.out.cp >> 2);
     FYN_DISPATCH_T(p.out.f16, dwconv3x3_kernel, grid1d(n, 256), dim3(256), s, p);
 }
@@ -116,44 +285,45 @@ void launch_dwconv3x3(const DwConvParams& p, hipStream_t s) {
 // max / average pooling  (DeepPoolingLayer::forward, gpu/deep/deeppoolinglayer.cpp:109-131;
 //                         shaders/deep/deepmaxpool.frag:12-59, deepavgpool.frag:15-58)
 // ---------------------------------------------------------------------------------------------
-template <typename T>
+template <typename T, int V>
 __global__ __launch_bounds__(256) void pool_kernel(const PoolParams p) {
-    const int cg = p.out.cp >> 2;
+    const int cg = p.out.cp / V;
     const size_t n = (size_t)p.out.h * p.out.w * cg;
     const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
     if (idx >= n) return;
     const int g = (int)(idx % cg);
     const size_t pix = idx / cg;
     const int x = (int)(pix % p.out.w), y = (int)(pix / p.out.w);
-    const int c = g * 4;
+    const int c = g * V;
     const T* in = reinterpret_cast<const T*>(p.in.ptr);
     const int iwp = p.in.wp(), ihp = p.in.hp();
     const int y0 = y * p.stride + p.off, x0 = x * p.stride + p.off;  // stored coordinates
-    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    FV<V> acc = zerov<V>();
     for (int py = 0; py < p.pool; py++) {
         for (int px = 0; px < p.pool; px++) {
             const int sy = y0 + py, sx = x0 + px;
-            float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+            FV<V> v = zerov<V>();
             if ((unsigned)sy < (unsigned)ihp && (unsigned)sx < (unsigned)iwp)
-                v = ld4<T>(in + ((size_t)sy * iwp + sx) * p.in.cp + c);
-            v = act4(v, p.act);
-            if (p.is_max) {
-                if (py == 0 && px == 0) acc = v;
-                else acc = make_float4(fmaxf(acc.x, v.x), fmaxf(acc.y, v.y), fmaxf(acc.z, v.z), fmaxf(acc.w, v.w));
-            } else {
-                acc = make_float4(acc.x + v.x, acc.y + v.y, acc.z + v.z, acc.w + v.w);
+                v = ldv<T, V>(in + ((size_t)sy * iwp + sx) * p.in.cp + c);
+            v = actv<V>(v, p.act);
+#pragma unroll
+            for (int i = 0; i < V; i++) {
+                if (p.is_max) acc.v[i] = (py == 0 && px == 0) ? v.v[i] : fmaxf(acc.v[i], v.v[i]);
+                else acc.v[i] += v.v[i];
             }
         }
     }
     if (!p.is_max) {
         const float inv = 1.0f / (float)(p.pool * p.pool);
-        acc = make_float4(acc.x * inv, acc.y * inv, acc.z * inv, acc.w * inv);
+#pragma unroll
+        for (int i = 0; i < V; i++) acc.v[i] *= inv;
     }
-    st4<T>(reinterpret_cast<T*>(p.out.ptr) + tv_off(p.out, y, x) + c, acc);
+    stv<T, V>(reinterpret_cast<T*>(p.out.ptr) + tv_off(p.out, y, x) + c, acc);
 }
 void launch_pool(const PoolParams& p, hipStream_t s) {
-    const size_t n = (size_t)p.out.h * p.out.w * (p.out.cp >> 2);
-    FYN_DISPATCH_T(p.out.f16, pool_kernel, grid1d(n, 256), dim3(256), s, p);
+    const bool wide = (p.in.cp % 8 == 0) && (p.out.cp % 8 == 0);
+    const size_t n = (size_t)p.out.h * p.out.w * (p.out.cp / ((p.out.f16 && wide) ? 8 : 4));
+    FYN_DISPATCH_TV(p.out.f16, wide, pool_kernel, grid1d(n, 256), dim3(256), s, p);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -219,31 +389,37 @@ void launch_global_pool(const TView& in, const TView& out, int is_max, const Act
 // explicit batch-norm (DeepBatchNormLayer, shaders/deep/deepbatchnorm.frag:24-36), add/sub
 // (shaders/add.frag) and one input of a concatenation (shaders/deep/deepconcat.frag:45-76)
 // ---------------------------------------------------------------------------------------------
-template <typename T>
+template <typename T, int V>
 __global__ __launch_bounds__(256) void batchnorm_kernel(const BnParams p) {
-    const int cg = p.out.cp >> 2;
+    const int cg = p.out.cp / V;
     const size_t n = (size_t)p.out.h * p.out.w * cg;
     const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
     if (idx >= n) return;
     const int g = (int)(idx % cg);
     const size_t pix = idx / cg;
     const int x = (int)(pix % p.out.w), y = (int)(pix / p.out.w);
-    const int c = g * 4;
-    float4 v = act4(ld4<T>(reinterpret_cast<const T*>(p.in.ptr) + tv_off(p.in, y, x) + c), p.act);
-    const float4 sc = *reinterpret_cast<const float4*>(p.scale + c);
-    const float4 bi = *reinterpret_cast<const float4*>(p.bias + c);
-    float4 o = make_float4(v.x * sc.x + bi.x, v.y * sc.y + bi.y, v.z * sc.z + bi.z, v.w * sc.w + bi.w);
+    const int c = g * V;
+    FV<V> v = actv<V>(ldv<T, V>(reinterpret_cast<const T*>(p.in.ptr) + tv_off(p.in, y, x) + c), p.act);
+    const FV<V> sc = ldv<float, V>(p.scale + c), bi = ldv<float, V>(p.bias + c);
+    FV<V> o;
+#pragma unroll
+    for (int i = 0; i < V; i++) o.v[i] = v.v[i] * sc.v[i] + bi.v[i];
     if (p.res.ptr) {
-        float4 r = ld4<T>(reinterpret_cast<const T*>(p.res.ptr) + tv_off(p.res, y, x) + c);
-        if (p.res_relu) r = make_float4(fmaxf(r.x, 0.f), fmaxf(r.y, 0.f), fmaxf(r.z, 0.f), fmaxf(r.w, 0.f));
-        if (p.res_bn) r = make_float4(r.x * sc.x + bi.x, r.y * sc.y + bi.y, r.z * sc.z + bi.z, r.w * sc.w + bi.w);
-        o = make_float4(o.x + r.x, o.y + r.y, o.z + r.z, o.w + r.w);
+        FV<V> r = ldv<T, V>(reinterpret_cast<const T*>(p.res.ptr) + tv_off(p.res, y, x) + c);
+#pragma unroll
+        for (int i = 0; i < V; i++) {
+            float rv = r.v[i];
+            if (p.res_relu) rv = fmaxf(rv, 0.f);
+            if (p.res_bn) rv = rv * sc.v[i] + bi.v[i];
+            o.v[i] += rv;
+        }
     }
-    st4<T>(reinterpret_cast<T*>(p.out.ptr) + tv_off(p.out, y, x) + c, o);
+    stv<T, V>(reinterpret_cast<T*>(p.out.ptr) + tv_off(p.out, y, x) + c, o);
 }
 void launch_batchnorm(const BnParams& p, hipStream_t s) {
-    const size_t n = (size_t)p.out.h * p.out.w * (p.out.cp >> 2);
-    FYN_DISPATCH_T(p.out.f16, batchnorm_kernel, grid1d(n, 256), dim3(256), s, p);
+    const bool wide = (p.in.cp % 8 == 0) && (p.out.cp % 8 == 0) && (!p.res.ptr || p.res.cp % 8 == 0);
+    const size_t n = (size_t)p.out.h * p.out.w * (p.out.cp / ((p.out.f16 && wide) ? 8 : 4));
+    FYN_DISPATCH_TV(p.out.f16, wide, batchnorm_kernel, grid1d(n, 256), dim3(256), s, p);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -281,8 +457,8 @@ __device__ __forceinline__ float4 mask_channels(float4 v, int c, int nc) {
 
 __device__ __forceinline__ float func1(float x, int fn, int op, float operand) {
     switch (fn) {
-        case FFN_SIGMOID: return 1.0f / (1.0f + expf(-x));
-        case FFN_TANH: return tanhf(x);
+        case FFN_SIGMOID: return __frcp_rn(1.0f + __expf(-x));
+        case FFN_TANH: return 1.0f - 2.0f * __frcp_rn(1.0f + __expf(2.0f * x));   // = 2 e^{2x}/(1+e^{2x}) - 1 without the inf/inf of large x
         case FFN_ARITH: return op == 0 ? x + operand : op == 1 ? x - operand : op == 2 ? x * operand : x / operand;
         case FFN_CAST: {
             if (op == 7) return x;
@@ -301,45 +477,70 @@ __device__ __forceinline__ float func1(float x, int fn, int op, float operand) {
     }
 }
 
-template <typename T>
+// Texel of V channels at stored coordinates, edge repeated beyond the stored tensor; channels >= in.c read as zero.
+template <typename T, int V>
+__device__ __forceinline__ FV<V> fetch_clamped_v(const TView& t, int sy, int sx, int c) {
+    sy = min(max(sy, 0), t.hp() - 1);
+    sx = min(max(sx, 0), t.wp() - 1);
+    FV<V> v = ldv<T, V>(reinterpret_cast<const T*>(t.ptr) + ((size_t)sy * t.wp() + sx) * t.cp + c);
+    if (c + V > t.c) {
+#pragma unroll
+        for (int i = 0; i < V; i++)
+            if (c + i >= t.c) v.v[i] = 0.f;
+    }
+    return v;
+}
+
+template <typename T, int V>
 __global__ __launch_bounds__(256) void func_kernel(const FuncParams p) {
-    const int cg = p.out.cp >> 2;
+    const int cg = p.out.cp / V;
     const size_t n = (size_t)p.out.h * p.out.w * cg;
     const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
     if (idx >= n) return;
     const int g = (int)(idx % cg);
     const size_t pix = idx / cg;
     const int x = (int)(pix % p.out.w), y = (int)(pix / p.out.w);
-    int sy, sx, sg = g;
+    int sy, sx, sc = g * V;   // source texel and first source channel
     if (p.map == FMAP_TRANSPOSE) {
         sy = x;
         sx = y;
-    } else if (p.map == FMAP_IMGEXTRACT) {
+    } else if (p.map == FMAP_IMGEXTRACT) {   // (always launched 4 channels wide: the groups of the reference are texels)
         const int b = g / p.in_groups;
-        sg = g - b * p.in_groups;
+        sc = (g - b * p.in_groups) * 4;
         sy = y * p.window + b / p.window;
         sx = x * p.window + b % p.window;
     } else {
         sy = floordiv_pos((2 * y + 1) * p.dy - p.oy, 2 * p.uy);
         sx = floordiv_pos((2 * x + 1) * p.dx - p.ox, 2 * p.ux);
     }
-    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (sg * 4 < p.in.cp) v = fetch_clamped<T>(p.in, sy + p.in.pad, sx + p.in.pad, sg * 4);
+    FV<V> v = zerov<V>();
+    if (sc < p.in.cp) v = fetch_clamped_v<T, V>(p.in, sy + p.in.pad, sx + p.in.pad, sc);
     if (p.fn == FFN_BGR) {
-        const float t = v.x;
-        v.x = v.z;
-        v.z = t;
+#pragma unroll
+        for (int q = 0; q < V / 4; q++) {
+            const float t = v.v[4 * q];
+            v.v[4 * q] = v.v[4 * q + 2];
+            v.v[4 * q + 2] = t;
+        }
     } else {
-        v = act4(v, p.act);
-        if (p.fn != FFN_COPY)
-            v = make_float4(func1(v.x, p.fn, p.op, p.operand), func1(v.y, p.fn, p.op, p.operand),
-                            func1(v.z, p.fn, p.op, p.operand), func1(v.w, p.fn, p.op, p.operand));
+        v = actv<V>(v, p.act);
+        if (p.fn != FFN_COPY) {
+#pragma unroll
+            for (int i = 0; i < V; i++) v.v[i] = func1(v.v[i], p.fn, p.op, p.operand);
+        }
     }
-    st4<T>(reinterpret_cast<T*>(p.out.ptr) + tv_off(p.out, y, x) + g * 4, mask_channels(v, g * 4, p.out.c));
+    const int c = g * V;
+    if (c + V > p.out.c) {
+#pragma unroll
+        for (int i = 0; i < V; i++)
+            if (c + i >= p.out.c) v.v[i] = 0.f;
+    }
+    stv<T, V>(reinterpret_cast<T*>(p.out.ptr) + tv_off(p.out, y, x) + c, v);
 }
 void launch_func(const FuncParams& p, hipStream_t s) {
-    const size_t n = (size_t)p.out.h * p.out.w * (p.out.cp >> 2);
-    FYN_DISPATCH_T(p.out.f16, func_kernel, grid1d(n, 256), dim3(256), s, p);
+    const bool wide = p.map != FMAP_IMGEXTRACT && (p.in.cp % 8 == 0) && (p.out.cp % 8 == 0);
+    const size_t n = (size_t)p.out.h * p.out.w * (p.out.cp / ((p.out.f16 && wide) ? 8 : 4));
+    FYN_DISPATCH_TV(p.out.f16, wide, func_kernel, grid1d(n, 256), dim3(256), s, p);
 }
 
 // Bilinear scaling: the raw texels around position ((2x+1)*dx - ox)/(2*ux) - 1/2 are blended, then activated.
@@ -420,50 +621,54 @@ void launch_blur(const TView& in, const TView& out, const float* coef, int r, in
     FYN_DISPATCH_T(out.f16, blur_kernel, grid1d(n, 256), dim3(256), s, in, out, coef, r, last);
 }
 
-template <typename T>
+template <typename T, int V>
 __global__ __launch_bounds__(256) void addsub_kernel(const TView a, const TView b, const TView out, int sub, const Act act) {
-    const int cg = out.cp >> 2;
+    const int cg = out.cp / V;
     const size_t n = (size_t)out.h * out.w * cg;
     const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
     if (idx >= n) return;
     const int g = (int)(idx % cg);
     const size_t pix = idx / cg;
     const int x = (int)(pix % out.w), y = (int)(pix / out.w);
-    const int c = g * 4;
-    float4 u = act4(ld4<T>(reinterpret_cast<const T*>(a.ptr) + tv_off(a, y, x) + c), act);
-    float4 v = act4(ld4<T>(reinterpret_cast<const T*>(b.ptr) + tv_off(b, y, x) + c), act);
-    float4 o = sub ? make_float4(u.x - v.x, u.y - v.y, u.z - v.z, u.w - v.w)
-                   : make_float4(u.x + v.x, u.y + v.y, u.z + v.z, u.w + v.w);
-    st4<T>(reinterpret_cast<T*>(out.ptr) + tv_off(out, y, x) + c, o);
+    const int c = g * V;
+    const FV<V> u = actv<V>(ldv<T, V>(reinterpret_cast<const T*>(a.ptr) + tv_off(a, y, x) + c), act);
+    const FV<V> v = actv<V>(ldv<T, V>(reinterpret_cast<const T*>(b.ptr) + tv_off(b, y, x) + c), act);
+    FV<V> o;
+#pragma unroll
+    for (int i = 0; i < V; i++) o.v[i] = sub ? u.v[i] - v.v[i] : u.v[i] + v.v[i];
+    stv<T, V>(reinterpret_cast<T*>(out.ptr) + tv_off(out, y, x) + c, o);
 }
 void launch_addsub(const TView& a, const TView& b, const TView& out, int sub, const Act& act, hipStream_t s) {
-    const size_t n = (size_t)out.h * out.w * (out.cp >> 2);
-    FYN_DISPATCH_T(out.f16, addsub_kernel, grid1d(n, 256), dim3(256), s, a, b, out, sub, act);
+    const bool wide = (a.cp % 8 == 0) && (b.cp % 8 == 0) && (out.cp % 8 == 0);
+    const size_t n = (size_t)out.h * out.w * (out.cp / ((out.f16 && wide) ? 8 : 4));
+    FYN_DISPATCH_TV(out.f16, wide, addsub_kernel, grid1d(n, 256), dim3(256), s, a, b, out, sub, act);
 }
 
-// Channel offsets that are not multiples of 4 (the "component shift" case of deepconcat.frag) are
-// handled per element; aligned offsets move whole 4-channel vectors.
-template <typename T>
+// Channel offsets that are not multiples of the vector width (the "component shift" case of deepconcat.frag) are
+// handled per element; aligned offsets move whole vectors.
+template <typename T, int V>
 __global__ __launch_bounds__(256) void concat_kernel(const TView in, const TView out, int c_off, const Act act) {
-    const int cg = (in.c + 3) >> 2;
+    const int cg = (in.c + V - 1) / V;
     const size_t n = (size_t)out.h * out.w * cg;
     const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
     if (idx >= n) return;
     const int g = (int)(idx % cg);
     const size_t pix = idx / cg;
     const int x = (int)(pix % out.w), y = (int)(pix / out.w);
-    const int c = g * 4;
+    const int c = g * V;
     const T* src = reinterpret_cast<const T*>(in.ptr) + tv_off(in, y, x) + c;
     T* dst = reinterpret_cast<T*>(out.ptr) + tv_off(out, y, x) + c_off + c;
-    if ((c_off & 3) == 0 && c + 4 <= in.c) {
-        st4<T>(dst, act4(ld4<T>(src), act));
+    if ((c_off % V) == 0 && c + V <= in.c) {
+        stv<T, V>(dst, actv<V>(ldv<T, V>(src), act));
     } else {
-        for (int i = 0; i < 4 && c + i < in.c; i++) dst[i] = (T)act1((float)src[i], act);
+        for (int i = 0; i < V && c + i < in.c; i++) dst[i] = (T)act1((float)src[i], act);
     }
 }
 void launch_concat_part(const TView& in, const TView& out, int c_off, const Act& act, hipStream_t s) {
-    const size_t n = (size_t)out.h * out.w * ((in.c + 3) >> 2);
-    FYN_DISPATCH_T(out.f16, concat_kernel, grid1d(n, 256), dim3(256), s, in, out, c_off, act);
+    const bool wide = (in.cp % 8 == 0) && (out.cp % 8 == 0);
+    const int v = (out.f16 && wide) ? 8 : 4;
+    const size_t n = (size_t)out.h * out.w * ((in.c + v - 1) / v);
+    FYN_DISPATCH_TV(out.f16, wide, concat_kernel, grid1d(n, 256), dim3(256), s, in, out, c_off, act);
 }
 
 // ---------------------------------------------------------------------------------------------
