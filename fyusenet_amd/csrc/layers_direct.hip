@@ -967,31 +967,45 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const SplitKReducePa
     const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
     if (idx >= n) return;
     const int c = (int)(idx % cq) * 4;
+    if (c >= p.out_cp) return;
     const size_t pos = idx / cq;
     const int py = (int)(pos / p.npos_x), px = (int)(pos - (size_t)py * p.npos_x);
     const size_t slice = (size_t)p.npos_y * p.npos_x * p.cout_pad;
-    f32x4 a = (f32x4)(0.f);
-    for (int ks = 0; ks < p.ksplit; ks++) a += *reinterpret_cast<const f32x4*>(p.partial + ks * slice + pos * p.cout_pad + c);
-    if (c >= p.out_cp) return;
-    const f32x4 sc = *reinterpret_cast<const f32x4*>(p.scale + c), bi = *reinterpret_cast<const f32x4*>(p.bias + c);
-    float o[4];
-#pragma unroll
-    for (int i = 0; i < 4; i++) o[i] = (a[i] * p.acc_mul) * sc[i] + bi[i];
+    // everything this thread reads is requested up front: residual, scale, bias and the first eight slices share
+    // one memory round trip
+    float rv[4] = {0.f, 0.f, 0.f, 0.f};
     if (p.res) {
         const TOut* res = reinterpret_cast<const TOut*>(p.res);
         const size_t rbase = ((size_t)(p.res_off_y + py * p.out_step) * p.res_wp + p.res_off_x + px * p.out_step) * p.res_cp + c;
+        const float4 r = ld4<TOut>(res + rbase);
+        rv[0] = r.x; rv[1] = r.y; rv[2] = r.z; rv[3] = r.w;
+    }
+    const f32x4 sc = *reinterpret_cast<const f32x4*>(p.scale + c), bi = *reinterpret_cast<const f32x4*>(p.bias + c);
+    // slices are summed in slice order; their loads are issued eight at a time (one round trip per eight slices)
+    f32x4 a = (f32x4)(0.f);
+    const float* src = p.partial + pos * p.cout_pad + c;
+    for (int k0 = 0; k0 < p.ksplit; k0 += 8) {
+        f32x4 v[8];
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            float rv = (float)res[rbase + i];
-            if (p.res_relu) rv = fmaxf(rv, 0.f);
-            if (p.res_scale) rv *= sc[i];
-            o[i] += rv;
+        for (int j = 0; j < 8; j++) v[j] = *reinterpret_cast<const f32x4*>(src + (size_t)(k0 + j < p.ksplit ? k0 + j : k0) * slice);
+#pragma unroll
+        for (int j = 0; j < 8; j++)
+            if (k0 + j < p.ksplit) a += v[j];
+    }
+    float o[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        o[i] = (a[i] * p.acc_mul) * sc[i] + bi[i];
+        if (p.res) {
+            float r = rv[i];
+            if (p.res_relu) r = fmaxf(r, 0.f);
+            if (p.res_scale) r *= sc[i];
+            o[i] += r;
         }
     }
     TOut* out = reinterpret_cast<TOut*>(p.out);
     const size_t obase = ((size_t)(p.out_off_y + py * p.out_step) * p.out_wp + p.out_off_x + px * p.out_step) * p.out_cp + c;
-#pragma unroll
-    for (int i = 0; i < 4; i++) out[obase + i] = (TOut)o[i];
+    st4<TOut>(out + obase, make_float4(o[0], o[1], o[2], o[3]));
 }
 
 void launch_splitk_reduce(const SplitKReduceParams& p, hipStream_t s) {
