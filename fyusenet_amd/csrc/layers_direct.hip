@@ -285,7 +285,8 @@ void launch_dwconv3x3(const DwConvParams& p, hipStream_t s) {
 // max / average pooling  (DeepPoolingLayer::forward, gpu/deep/deeppoolinglayer.cpp:109-131;
 //                         shaders/deep/deepmaxpool.frag:12-59, deepavgpool.frag:15-58)
 // ---------------------------------------------------------------------------------------------
-template <typename T, int V>
+// P: window size known at compile time (2, 3: all loads of a window are issued before the first use), 0: any size
+template <typename T, int V, int P>
 __global__ __launch_bounds__(256) void pool_kernel(const PoolParams p) {
     const int cg = p.out.cp / V;
     const size_t n = (size_t)p.out.h * p.out.w * cg;
@@ -299,19 +300,31 @@ __global__ __launch_bounds__(256) void pool_kernel(const PoolParams p) {
     const int iwp = p.in.wp(), ihp = p.in.hp();
     const int y0 = y * p.stride + p.off, x0 = x * p.stride + p.off;  // stored coordinates
     FV<V> acc = zerov<V>();
-    for (int py = 0; py < p.pool; py++) {
-        for (int px = 0; px < p.pool; px++) {
-            const int sy = y0 + py, sx = x0 + px;
-            FV<V> v = zerov<V>();
-            if ((unsigned)sy < (unsigned)ihp && (unsigned)sx < (unsigned)iwp)
-                v = ldv<T, V>(in + ((size_t)sy * iwp + sx) * p.in.cp + c);
-            v = actv<V>(v, p.act);
+    auto fold = [&](const FV<V>& v, bool first_tap) {
 #pragma unroll
-            for (int i = 0; i < V; i++) {
-                if (p.is_max) acc.v[i] = (py == 0 && px == 0) ? v.v[i] : fmaxf(acc.v[i], v.v[i]);
-                else acc.v[i] += v.v[i];
-            }
+        for (int i = 0; i < V; i++) {
+            if (p.is_max) acc.v[i] = first_tap ? v.v[i] : fmaxf(acc.v[i], v.v[i]);
+            else acc.v[i] += v.v[i];
         }
+    };
+    auto fetch = [&](int sy, int sx) {
+        FV<V> v = zerov<V>();
+        if ((unsigned)sy < (unsigned)ihp && (unsigned)sx < (unsigned)iwp) v = ldv<T, V>(in + ((size_t)sy * iwp + sx) * p.in.cp + c);
+        return v;
+    };
+    if constexpr (P > 0) {
+        FV<V> win[P][P];
+#pragma unroll
+        for (int py = 0; py < P; py++)
+#pragma unroll
+            for (int px = 0; px < P; px++) win[py][px] = fetch(y0 + py, x0 + px);
+#pragma unroll
+        for (int py = 0; py < P; py++)
+#pragma unroll
+            for (int px = 0; px < P; px++) fold(actv<V>(win[py][px], p.act), py == 0 && px == 0);
+    } else {
+        for (int py = 0; py < p.pool; py++)
+            for (int px = 0; px < p.pool; px++) fold(actv<V>(fetch(y0 + py, x0 + px), p.act), py == 0 && px == 0);
     }
     if (!p.is_max) {
         const float inv = 1.0f / (float)(p.pool * p.pool);
@@ -320,10 +333,18 @@ __global__ __launch_bounds__(256) void pool_kernel(const PoolParams p) {
     }
     stv<T, V>(reinterpret_cast<T*>(p.out.ptr) + tv_off(p.out, y, x) + c, acc);
 }
-void launch_pool(const PoolParams& p, hipStream_t s) {
+template <int P>
+static void launch_pool_p(const PoolParams& p, hipStream_t s) {
     const bool wide = (p.in.cp % 8 == 0) && (p.out.cp % 8 == 0);
     const size_t n = (size_t)p.out.h * p.out.w * (p.out.cp / ((p.out.f16 && wide) ? 8 : 4));
-    FYN_DISPATCH_TV(p.out.f16, wide, pool_kernel, grid1d(n, 256), dim3(256), s, p);
+    if (p.out.f16 && wide) hipLaunchKernelGGL((pool_kernel<_Float16, 8, P>), grid1d(n, 256), dim3(256), 0, s, p);
+    else if (p.out.f16) hipLaunchKernelGGL((pool_kernel<_Float16, 4, P>), grid1d(n, 256), dim3(256), 0, s, p);
+    else hipLaunchKernelGGL((pool_kernel<float, 4, P>), grid1d(n, 256), dim3(256), 0, s, p);
+}
+void launch_pool(const PoolParams& p, hipStream_t s) {
+    if (p.pool == 2) launch_pool_p<2>(p, s);
+    else if (p.pool == 3) launch_pool_p<3>(p, s);
+    else launch_pool_p<0>(p, s);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -346,14 +367,26 @@ __global__ __launch_bounds__(256) void global_pool_kernel(const TView in, const 
     float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
     bool first = true;
     if (g < cgs) {
-        for (int pix = part; pix < npix; pix += parts) {
-            const int y = pix / in.w, x = pix - y * in.w;
-            float4 v = act4(ld4<T>(src + tv_off(in, y, x) + g * 4), act);
-            if (is_max) {
-                acc = first ? v : make_float4(fmaxf(acc.x, v.x), fmaxf(acc.y, v.y), fmaxf(acc.z, v.z), fmaxf(acc.w, v.w));
-                first = false;
-            } else {
-                acc = make_float4(acc.x + v.x, acc.y + v.y, acc.z + v.z, acc.w + v.w);
+        // four pixels per trip: their loads are issued together, then folded in pixel order
+        for (int pix0 = part; pix0 < npix; pix0 += 4 * parts) {
+            float4 v4[4];
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const int pix = pix0 + j * parts;
+                const int pc = pix < npix ? pix : pix0;
+                const int y = pc / in.w, x = pc - y * in.w;
+                v4[j] = ld4<T>(src + tv_off(in, y, x) + g * 4);
+            }
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                if (pix0 + j * parts >= npix) break;
+                const float4 v = act4(v4[j], act);
+                if (is_max) {
+                    acc = first ? v : make_float4(fmaxf(acc.x, v.x), fmaxf(acc.y, v.y), fmaxf(acc.z, v.z), fmaxf(acc.w, v.w));
+                    first = false;
+                } else {
+                    acc = make_float4(acc.x + v.x, acc.y + v.y, acc.z + v.z, acc.w + v.w);
+                }
             }
         }
     }
@@ -379,8 +412,9 @@ __global__ __launch_bounds__(256) void global_pool_kernel(const TView in, const 
 }
 void launch_global_pool(const TView& in, const TView& out, int is_max, const Act& act, hipStream_t s) {
     const int cgs = in.cp >> 2;
+    // few channel groups per workgroup: more workgroups, and more threads sharing the pixels of a group
     int l2 = 0;
-    while ((1 << l2) < cgs && l2 < 6) l2++;
+    while ((1 << l2) < cgs && l2 < 4) l2++;
     const int cgb = 1 << l2;
     FYN_DISPATCH_T(in.f16, global_pool_kernel, dim3((cgs + cgb - 1) / cgb), dim3(256), s, in, out, is_max, act, l2);
 }
