@@ -727,15 +727,24 @@ __global__ __launch_bounds__(256) void argmax_kernel(const TView in, const TView
     int bidx = 0x7fffffff;
     const int cgs = (in.c + 3) >> 2;
     if (valid) {
-        for (int g = sub; g < cgs; g += L) {
-            float4 v = act4(ld4<T>(src + g * 4), act);
-            const float vv[4] = {v.x, v.y, v.z, v.w};
+        // four channel groups per trip: loads first, then the scan in channel order
+        for (int g0 = sub; g0 < cgs; g0 += 4 * L) {
+            float4 v4[4];
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const int c = g * 4 + i;
-                if (c < in.c && (vv[i] > best || (vv[i] == best && c < bidx))) {
-                    best = vv[i];
-                    bidx = c;
+            for (int j = 0; j < 4; j++) v4[j] = ld4<T>(src + (g0 + j * L < cgs ? g0 + j * L : g0) * 4);
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const int g = g0 + j * L;
+                if (g >= cgs) break;
+                const float4 v = act4(v4[j], act);
+                const float vv[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const int c = g * 4 + i;
+                    if (c < in.c && (vv[i] > best || (vv[i] == best && c < bidx))) {
+                        best = vv[i];
+                        bidx = c;
+                    }
                 }
             }
         }
@@ -779,11 +788,22 @@ __global__ __launch_bounds__(256) void gemv_kernel(const GemvParams p) {
     const TW* w = reinterpret_cast<const TW*>(p.w) + (size_t)row * cinp;
     float acc = 0.f;
     if (row < p.out.c) {
-        for (int c = lane * 4; c < cinp; c += 256) {
-            float4 xv = act4(ld4<T>(x + c), p.act);
-            float4 wv = ld4<TW>(w + c);
-            acc = fmaf(xv.x, wv.x, acc); acc = fmaf(xv.y, wv.y, acc);
-            acc = fmaf(xv.z, wv.z, acc); acc = fmaf(xv.w, wv.w, acc);
+        // four 16-byte pieces of the row per trip: loads first, multiply-adds in column order
+        for (int c0 = lane * 4; c0 < cinp; c0 += 4 * 256) {
+            float4 xv[4], wv[4];
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const int c = c0 + j * 256 < cinp ? c0 + j * 256 : c0;
+                xv[j] = ld4<T>(x + c);
+                wv[j] = ld4<TW>(w + c);
+            }
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                if (c0 + j * 256 >= cinp) break;
+                const float4 a = act4(xv[j], p.act);
+                acc = fmaf(a.x, wv[j].x, acc); acc = fmaf(a.y, wv[j].y, acc);
+                acc = fmaf(a.z, wv[j].z, acc); acc = fmaf(a.w, wv[j].w, acc);
+            }
         }
     }
     for (int o = 32; o > 0; o >>= 1) acc += __shfl_xor(acc, o, 64);
