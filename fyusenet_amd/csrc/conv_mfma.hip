@@ -26,7 +26,6 @@
 
 #include "kernels.h"
 
-// prefetch distance (k16 steps) of the weight fragments, by cout fragments per wave
 // Timing-study builds (-DFYN_CONV_TRACE): wave 0 of every workgroup records the shader clock at phase boundaries.
 #ifdef FYN_CONV_TRACE
 #define FYN_TRACE(slot) do { if (tid == 0 && (slot) < 16) p.trace[((size_t)blockIdx.y * gridDim.x + blockIdx.x) * 16 + (slot)] = clock64(); } while (0)
@@ -34,9 +33,6 @@
 #define FYN_TRACE(slot) do { } while (0)
 #endif
 
-#ifndef FYN_ABL
-#define FYN_ABL 0
-#endif
 namespace fynhip {
 
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
@@ -410,10 +406,10 @@ __device__ __forceinline__ void conv_mfma_body(const ConvMfmaParams& p, unsigned
                 acc[fm][fn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_q[d][fm][apl], b_buf[dd & 1][fn][bpl], acc[fm][fn], 0, 0, 0);
                 if (i == 0) ao_reg[dd & 1] = *tab2;          // this parity's old value (step t) was consumed during step t-1
 #pragma unroll
-                for (int j = i * NDS / NMF; j < ((FYN_ABL & 2) ? 0 : (i + 1) * NDS / NMF); j++)   // plane 0 of all fragments first
+                for (int j = i * NDS / NMF; j < (i + 1) * NDS / NMF; j++)   // plane 0 of all fragments first
                     b_buf[(dd + 1) & 1][j % FN][j / FN] = load_b_frag<KC>(cur + (j / FN) * p.plane + (boff[j % FN] + ao));
 #pragma unroll
-                for (int j = i * NVM / NMF; j < ((FYN_ABL & 1) ? 0 : (i + 1) * NVM / NMF); j++)
+                for (int j = i * NVM / NMF; j < (i + 1) * NVM / NMF; j++)
                     a_q[dprev][j % FM][j / FM] = *reinterpret_cast<const half8_t*>(w_ + ((j % FM) * NPL + j / FM) * 1024 + wlane);
                 __builtin_amdgcn_sched_barrier(0);
             }
