@@ -7,7 +7,7 @@ package without the built library raises ImportError at the first call.
 """
 from . import capi  # noqa: F401
 from .builders import (ActType, ArgMaxLayerBuilder, ArithType, BlurKernelType, BlurLayerBuilder, CastLayerBuilder,  # noqa: F401
-                       CastTarget, ConcatLayerBuilder, ConvLayerBuilder, GPULayerBuilder, ImgExtractLayerBuilder,
+                       CastTarget, ConcatLayerBuilder, ConvLayerBuilder, CustomLayerBuilder, GPULayerBuilder, ImgExtractLayerBuilder,
                        LayerBuilder, LayerFlags, LayerType, NormType, PoolLayerBuilder, ScaleLayerBuilder, ScalingType,
                        SingletonArithLayerBuilder, TransposeLayerBuilder, UpDownLayerBuilder)
 from .capi import FynException, ORDER_CHANNELWISE, ORDER_GPU_DEEP, ORDER_GPU_SHALLOW, STORAGE_F16, STORAGE_F32  # noqa: F401

@@ -520,3 +520,27 @@ class BlurLayerBuilder(GPULayerBuilder):
     def _fill(self, d):
         d.kernel = self.kernel_
         d.blur_type = int(self.blurType_)
+
+
+class CustomLayerBuilder(GPULayerBuilder):
+    """gpu/customlayerbuilder.h:53-90: `initCallback(builder)` returns the layer object.  Here that object provides
+    forward(inputs, output, stream, sequence) and optionally setup(inputs, output) and cleanup(); inputs/output are
+    capi.TensorView structures of device tensors, `stream` the hipStream_t (as an integer) to enqueue work on."""
+
+    def __init__(self, name, initCallback):
+        super().__init__(name)
+        self.type_ = LayerType.CUSTOM
+        self.initCallback_ = initCallback
+        self.inputs_ = []
+
+    def input(self, channels, padding):
+        self.inputs_.append((channels, padding))
+        return self
+
+    def init(self):
+        return self.initCallback_(self)
+
+    def _fill(self, d):
+        d.num_inputs = len(self.inputs_)
+        for i, (c, p) in enumerate(self.inputs_):
+            d.inputs[i].channels, d.inputs[i].padding, d.inputs[i].flags = c, p, 0

@@ -72,6 +72,23 @@ class LayerDesc(ctypes.Structure):
     ]
 
 
+class TensorView(ctypes.Structure):
+    """struct fyn_tensor_view."""
+    _fields_ = [("data", ctypes.c_void_p), ("channels", ctypes.c_int32), ("height", ctypes.c_int32), ("width", ctypes.c_int32),
+                ("padding", ctypes.c_int32), ("channel_pitch", ctypes.c_int32), ("storage", ctypes.c_int32)]
+
+
+CUSTOM_SETUP_FN = ctypes.CFUNCTYPE(ctypes.c_int, ctypes.c_void_p, ctypes.POINTER(TensorView), ctypes.c_int, ctypes.POINTER(TensorView))
+CUSTOM_FORWARD_FN = ctypes.CFUNCTYPE(ctypes.c_int, ctypes.c_void_p, ctypes.POINTER(TensorView), ctypes.c_int, ctypes.POINTER(TensorView),
+                                     ctypes.c_void_p, ctypes.c_uint64)
+CUSTOM_CLEANUP_FN = ctypes.CFUNCTYPE(None, ctypes.c_void_p)
+
+
+class CustomLayer(ctypes.Structure):
+    """struct fyn_custom_layer."""
+    _fields_ = [("user", ctypes.c_void_p), ("setup", CUSTOM_SETUP_FN), ("forward", CUSTOM_FORWARD_FN), ("cleanup", CUSTOM_CLEANUP_FN)]
+
+
 # every symbol include/fynhip.h declares: name -> (restype, argtypes)
 _P = ctypes.c_void_p
 _F = ctypes.POINTER(ctypes.c_float)
@@ -81,6 +98,7 @@ SYMBOLS = {
     "fyn_net_create": (ctypes.c_int, [ctypes.c_int, ctypes.c_int, ctypes.POINTER(_P)]),
     "fyn_net_destroy": (ctypes.c_int, [_P]),
     "fyn_net_add_layer": (ctypes.c_int, [_P, ctypes.POINTER(LayerDesc)]),
+    "fyn_net_add_custom_layer": (ctypes.c_int, [_P, ctypes.POINTER(LayerDesc), ctypes.POINTER(CustomLayer)]),
     "fyn_net_connect": (ctypes.c_int, [_P, ctypes.c_int, ctypes.c_int, ctypes.c_int]),
     "fyn_layer_load_weights": (ctypes.c_int, [_P, ctypes.c_int, _F, ctypes.c_size_t]),
     "fyn_layer_load_scale_bias": (ctypes.c_int, [_P, ctypes.c_int, _F, ctypes.c_size_t]),

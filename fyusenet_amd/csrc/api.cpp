@@ -76,6 +76,17 @@ int fyn_net_add_layer(fyn_net* net, const fyn_layer_desc* desc) {
     FYN_API_END
 }
 
+int fyn_net_add_custom_layer(fyn_net* net, const fyn_layer_desc* desc, const fyn_custom_layer* impl) {
+    FYN_API_BEGIN
+    if (!desc || !impl) fynhip::fail(FYN_ERR_INVALID, "No builder supplied to layer factory line");
+    if (desc->struct_size != sizeof(fyn_layer_desc))
+        fynhip::fail(FYN_ERR_INVALID, "fyn_layer_desc size mismatch (%u, library expects %zu)", desc->struct_size, sizeof(fyn_layer_desc));
+    fyn_layer_desc d = *desc;
+    d.name[FYN_NAME_LEN - 1] = 0;
+    N(net)->add_custom_layer(d, *impl);
+    FYN_API_END
+}
+
 int fyn_net_connect(fyn_net* net, int out_layer, int in_layer, int port) {
     FYN_API_BEGIN
     N(net)->connect(out_layer, in_layer, port);

@@ -128,6 +128,14 @@ void Net::add_layer(const fyn_layer_desc& d) {
     layers[d.number] = std::move(l);
 }
 
+void Net::add_custom_layer(const fyn_layer_desc& d, const fyn_custom_layer& impl) {
+    if (is_setup) fail(FYN_ERR_STATE, "cannot add layers after setup");
+    if (d.number < 0) fail(FYN_ERR_INVALID, "Must identify each layer with a valid number (found %d in the builder)", d.number);
+    if (layers.count(d.number)) fail(FYN_ERR_DUPLICATE, "Trying to insert a layer on a position that is already taken (%d)", d.number);
+    std::unique_ptr<Layer> l(create_custom_layer(this, d, impl));
+    layers[d.number] = std::move(l);
+}
+
 void Net::connect(int out_layer, int in_layer, int port) {
     if (is_setup) fail(FYN_ERR_STATE, "cannot connect layers after setup");
     Layer* src = layer(out_layer);

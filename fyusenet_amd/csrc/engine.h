@@ -86,6 +86,7 @@ class Net {
     Net(int device, int storage);
     ~Net();
     void add_layer(const fyn_layer_desc& d);
+    void add_custom_layer(const fyn_layer_desc& d, const fyn_custom_layer& impl);
     void connect(int out_layer, int in_layer, int port);
     void setup();
     void forward(uint64_t* seq);
@@ -150,5 +151,6 @@ class Net {
 };
 
 Layer* create_layer(Net* net, const fyn_layer_desc& d);
+Layer* create_custom_layer(Net* net, const fyn_layer_desc& d, const fyn_custom_layer& impl);
 
 }  // namespace fynhip

@@ -1324,6 +1324,63 @@ class DownloadLayer : public Layer {
     std::string info() const override { return "download"; }
 };
 
+// User-supplied layer behind C callbacks (the reference's CustomLayerBuilder hook, gpu/customlayerbuilder.h:53-90).
+class CustomLayer : public Layer {
+  public:
+    CustomLayer(Net* n, const fyn_layer_desc& d_, const fyn_custom_layer& impl) : Layer(n, d_), cb(impl) {
+        if (!cb.forward) fail(FYN_ERR_INVALID, "custom layer %s has no forward function", d.name);
+        if (d.num_inputs < 0 || d.num_inputs > FYN_MAX_CONCAT_INPUTS) fail(FYN_ERR_INVALID, "custom layer %s: bad number of inputs %d", d.name, d.num_inputs);
+        const int ux = std::max(1, d.upsample[0]), uy = std::max(1, d.upsample[1]);
+        const int dx = std::max(1, d.downsample[0]), dy = std::max(1, d.downsample[1]);
+        oc = d.out_channels > 0 ? d.out_channels : d.in_channels;
+        ow = d.width * ux / dx;
+        oh = d.height * uy / dy;
+        if (ow < 1 || oh < 1) fail(FYN_ERR_INVALID, "custom layer %s: empty output", d.name);
+    }
+    ~CustomLayer() override {
+        if (cb.cleanup) cb.cleanup(cb.user);
+    }
+    int num_ports() const override { return d.num_inputs > 0 ? d.num_inputs : ((d.flags & FYN_FLAG_RESIDUAL_INPUT) ? 2 : 1); }
+    void port_shape(int port, int& c, int& h, int& w, int& pad) const override {
+        if (d.num_inputs > 0) {
+            c = d.inputs[port].channels; h = d.height; w = d.width; pad = d.inputs[port].padding;
+        } else {
+            Layer::port_shape(port, c, h, w, pad);
+        }
+    }
+    static fyn_tensor_view view_of(const TView& v) {
+        return fyn_tensor_view{v.ptr, v.c, v.h, v.w, v.pad, v.cp, v.f16 ? FYN_STORAGE_F16 : FYN_STORAGE_F32};
+    }
+    void setup() override {
+        ins.clear();
+        for (int i = 0; i < num_ports(); i++) ins.push_back(view_of(tin(i).v));
+        outv = view_of(tout().v);
+        if (cb.setup) {
+            const int rc = cb.setup(cb.user, ins.data(), (int)ins.size(), &outv);
+            if (rc != 0) fail(FYN_ERR_INVALID, "custom layer %s: setup callback failed (%d)", d.name, rc);
+        }
+    }
+    void forward(hipStream_t s) override {
+        const int rc = cb.forward(cb.user, ins.data(), (int)ins.size(), &outv, s, net->seq);
+        if (rc != 0) fail(FYN_ERR_DEVICE, "custom layer %s: forward callback failed (%d)", d.name, rc);
+    }
+    std::string info() const override { return "custom"; }
+    fyn_custom_layer cb;
+    std::vector<fyn_tensor_view> ins;
+    fyn_tensor_view outv{};
+};
+
+Layer* create_custom_layer(Net* net, const fyn_layer_desc& d, const fyn_custom_layer& impl) {
+    if (d.type != FYN_LAYER_CUSTOM) fail(FYN_ERR_INVALID, "layer %s: a custom layer needs type FYN_LAYER_CUSTOM", d.name);
+    if (d.width <= 0 || d.height <= 0 || d.width > 65535 || d.height > 65535)
+        fail(FYN_ERR_INVALID, "layer %s: invalid spatial size %dx%d", d.name, d.width, d.height);
+    if (d.in_channels < 0 || d.in_channels > 32767 || d.out_channels < 0 || d.out_channels > 32767 || (d.in_channels == 0 && d.num_inputs == 0))
+        fail(FYN_ERR_INVALID, "layer %s: invalid channel counts %d -> %d", d.name, d.in_channels, d.out_channels);
+    Layer* l = new CustomLayer(net, d, impl);
+    l->in.assign(l->num_ports(), -1);
+    return l;
+}
+
 Layer* create_layer(Net* net, const fyn_layer_desc& d) {
     if (d.width <= 0 || d.height <= 0 || d.width > 65535 || d.height > 65535)
         fail(FYN_ERR_INVALID, "layer %s: invalid spatial size %dx%d", d.name, d.width, d.height);
@@ -1376,6 +1433,7 @@ Layer* create_layer(Net* net, const fyn_layer_desc& d) {
         case FYN_LAYER_BLUR2D: l = new FuncLayer(net, d); break;
         case FYN_LAYER_FRACCONVOLUTION2D:
             fail(FYN_ERR_UNSUPPORTED, "fractional convolution (%s) is not supported: its sampling positions fall on texel boundaries of the nearest-neighbour filter", d.name);
+        case FYN_LAYER_CUSTOM: fail(FYN_ERR_INVALID, "layer %s: custom layers are added with fyn_net_add_custom_layer", d.name);
         case FYN_LAYER_UPLOAD: l = new UploadLayer(net, d); break;
         case FYN_LAYER_DOWNLOAD: l = new DownloadLayer(net, d); break;
         default: fail(FYN_ERR_UNSUPPORTED, "Unsupported layer type %d", d.type);

@@ -123,14 +123,57 @@ class LayerFactory:
             raise capi.FynException(capi.ERR_DUPLICATE, "Trying to insert a layer on a position that is already taken (%d)" % builder.number_)
         self._builders[builder.number_] = builder
 
+    def _add_custom(self, b, d):
+        # gpu/gpulayerfactory.cpp:586-589: the builder's callback creates the layer
+        if not hasattr(b, "init"):
+            raise capi.FynException(capi.ERR_INVALID, "layer %s: a CUSTOM layer needs a CustomLayerBuilder with its init callback" % b.name_)
+        impl = b.init()
+        thunks = _custom_thunks(impl)
+        self._net._keepalive.append((impl, thunks))     # the engine calls them until the network is destroyed
+        c = capi.CustomLayer(None, *thunks)
+        capi.check(capi.lib().fyn_net_add_custom_layer(self._net._h, ctypes.byref(d), ctypes.byref(c)))
+
     def compileLayers(self):
         layers = CompiledLayers()
         for no in sorted(self._builders):
             b = self._builders[no]
             d = b.desc()
-            capi.check(capi.lib().fyn_net_add_layer(self._net._h, ctypes.byref(d)))
+            if int(b.type_) == int(LayerType.CUSTOM):
+                self._add_custom(b, d)
+            else:
+                capi.check(capi.lib().fyn_net_add_layer(self._net._h, ctypes.byref(d)))
             layers._add(Layer(self._net, b))
         return layers
+
+
+def _custom_thunks(impl):
+    """C callbacks around a Python custom-layer object; exceptions become a non-zero status."""
+    def views(ptr, n):
+        return [ptr[i] for i in range(n)]
+
+    def setup(_user, ins, n, out):
+        try:
+            if hasattr(impl, "setup"):
+                impl.setup(views(ins, n), out[0])
+            return 0
+        except Exception:   # noqa: BLE001 -- must not propagate through the C frame
+            return 1
+
+    def forward(_user, ins, n, out, stream, seq):
+        try:
+            impl.forward(views(ins, n), out[0], stream or 0, seq)
+            return 0
+        except Exception:   # noqa: BLE001
+            return 1
+
+    def cleanup(_user):
+        try:
+            if hasattr(impl, "cleanup"):
+                impl.cleanup()
+        except Exception:   # noqa: BLE001
+            pass
+
+    return capi.CUSTOM_SETUP_FN(setup), capi.CUSTOM_FORWARD_FN(forward), capi.CUSTOM_CLEANUP_FN(cleanup)
 
 
 class BufferManager:
@@ -150,6 +193,7 @@ class NeuralNetwork:
 
     def __init__(self, storage=capi.STORAGE_F32, device=0):
         self.storage = storage
+        self._keepalive = []   # custom-layer objects and their C thunks
         self._h = ctypes.c_void_p()
         capi.check(capi.lib().fyn_net_create(device, storage, ctypes.byref(self._h)))
         self.layers = None

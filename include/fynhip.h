@@ -67,7 +67,8 @@ enum fyn_layer_type {
     FYN_LAYER_DOWNLOAD = 26,
     FYN_LAYER_UPLOAD = 27,
     FYN_LAYER_BATCHNORM = 30,
-    FYN_LAYER_GEMM = 31
+    FYN_LAYER_GEMM = 31,
+    FYN_LAYER_CUSTOM = 32 /* only through fyn_net_add_custom_layer */
 };
 
 /* LayerFlags bits (fyusenet/base/layerflags.h:33-50), as LayerBuilderTempl::getFlags() composes them
@@ -155,6 +156,32 @@ int fyn_net_destroy(fyn_net* net);
 /* LayerFactory::pushBuilder + LayerFactoryBackend::createLayer (base/layerfactory.cpp:67-101,
  * gpu/gpulayerfactory.cpp:112-184). */
 int fyn_net_add_layer(fyn_net* net, const fyn_layer_desc* desc);
+
+/* A device tensor as a custom layer sees it: channel-packed NHWC with a zero halo.  Element (y, x, c) of the net
+ * area lives at data[((y + padding) * (width + 2*padding) + (x + padding)) * channel_pitch + c]; the element type is
+ * float (storage FYN_STORAGE_F32) or IEEE half (FYN_STORAGE_F16).  Channels [channels, channel_pitch) and the halo
+ * of an output must stay zero. */
+typedef struct fyn_tensor_view {
+    void* data;
+    int32_t channels, height, width, padding, channel_pitch, storage;
+} fyn_tensor_view;
+
+/* User-supplied layer: the C form of CustomLayerBuilder's init callback returning a GPULayerBase subclass
+ * (fyusenet/gpu/customlayerbuilder.h:53-90, gpu/gpulayerfactory.cpp:586-589).  `forward` must only ENQUEUE work on
+ * the given hipStream_t (it is called once while a forward pass is being captured when fyn_net_use_graph is on, and
+ * the enqueued work is what later passes replay); a non-zero return fails the pass.  `setup` (after the tensors
+ * exist) and `cleanup` (when the network is destroyed) may be NULL.  The struct is copied. */
+typedef struct fyn_custom_layer {
+    void* user;
+    int (*setup)(void* user, const fyn_tensor_view* inputs, int num_inputs, const fyn_tensor_view* output);
+    int (*forward)(void* user, const fyn_tensor_view* inputs, int num_inputs, const fyn_tensor_view* output, void* hip_stream,
+                   uint64_t sequence);
+    void (*cleanup)(void* user);
+} fyn_custom_layer;
+/* desc->type must be FYN_LAYER_CUSTOM.  Input ports: desc->num_inputs ports of desc->inputs[i].channels/.padding (all
+ * width x height), or, with num_inputs == 0, one port of in_channels/input_padding (plus a residual port with
+ * FYN_FLAG_RESIDUAL_INPUT).  Output: out_channels x (height*upsample/downsample) x (width*...), output_padding. */
+int fyn_net_add_custom_layer(fyn_net* net, const fyn_layer_desc* desc, const fyn_custom_layer* impl);
 
 /* BufferManager::connectLayers(outputLayer, inputLayer, port) (base/buffermanager.cpp:160-184):
  * port 0 = data, port 1 = residual; concat ports 0..N-1. */

@@ -225,3 +225,95 @@ def test_style_net_tail_with_sigmoid(storage):
     assert got.shape == (3, 48, 64) and rel_l2(got, ref) <= TOL[storage]
     assert got.min() > 0.0 and got.max() < 1.0
     net.cleanup()
+
+
+def _hip():
+    import ctypes
+    lib = ctypes.CDLL("libamdhip64.so")
+    lib.hipMemcpyAsync.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int, ctypes.c_void_p]
+    lib.hipMemcpyAsync.restype = ctypes.c_int
+    return lib
+
+
+class _CopyLayer:
+    """A user layer: device-to-device copy of its input (same geometry on both sides), enqueued on the given stream."""
+    calls = 0
+
+    def __init__(self, fail_forward=False):
+        self.hip = _hip()
+        self.fail_forward = fail_forward
+        self.was_set_up = self.cleaned = False
+
+    def setup(self, inputs, output):
+        i = inputs[0]
+        assert (i.channels, i.height, i.width, i.padding, i.channel_pitch, i.storage) == \
+               (output.channels, output.height, output.width, output.padding, output.channel_pitch, output.storage)
+        self.nbytes = (i.height + 2 * i.padding) * (i.width + 2 * i.padding) * i.channel_pitch * (2 if i.storage else 4)
+        self.was_set_up = True
+
+    def forward(self, inputs, output, stream, sequence):
+        if self.fail_forward:
+            raise RuntimeError("told to fail")
+        type(self).calls += 1
+        assert self.hip.hipMemcpyAsync(output.data, inputs[0].data, self.nbytes, 3, stream) == 0   # hipMemcpyDeviceToDevice
+
+    def cleanup(self):
+        self.cleaned = True
+
+
+@STORAGES
+def test_custom_layer_hook(storage):
+    """CustomLayerBuilder (gpu/customlayerbuilder.h:53-90): a layer supplied by the application sits between two engine
+    layers, receives device views of its tensors and the stream, and its work is ordered with theirs."""
+    from util import conv_block
+    made = []
+
+    def init(builder):
+        made.append(_CopyLayer())
+        return made[-1]
+
+    class Net(fa.NeuralNetwork):
+        def buildLayers(self, f):
+            fa.ConvLayerBuilder(3, "conv").type(T.CONVOLUTION2D).number(1).shape(16, 20, 24, 8).inputPadding(1).outputPadding(1).deep().push(f)
+            fa.CustomLayerBuilder("mine", init).number(2).shape(16, 20, 24, 16).inputPadding(1).outputPadding(1).deep().push(f)
+            fa.GPULayerBuilder("sig").type(T.SIGMOID).number(3).shape(16, 20, 24, 16).inputPadding(1).prefixAct(A.RELU).deep().push(f)
+
+        def connectLayers(self, layers, bm):
+            bm.connectLayers(layers[1], layers[2], 0)
+            bm.connectLayers(layers[2], layers[3], 0)
+
+        def initializeWeights(self, layers):
+            layers[1].loadWeightsAndBiases(conv_block(120, 16, 3, 8), 0)
+
+    net = Net(storage)
+    net.setup()
+    assert made[0].was_set_up and net.layers[2].kernelInfo() == "custom"
+    x = prng.normal(121, (8, 20, 24))
+    net.layers[1].setInput(x, 0)
+    for graph in (False, True):
+        net.useGraph(graph)
+        for _ in range(3):
+            net.forward()
+            net.finish()
+            conv = net.layers[1].copyResult()
+            assert np.array_equal(net.layers[2].copyResult(), conv)
+            want = 1.0 / (1.0 + np.exp(-np.maximum(conv.astype(np.float64), 0)))
+            assert rel_l2(net.getOutput(3), want) <= TOL[storage]
+    assert _CopyLayer.calls >= 4          # every eager pass plus the captured one
+    net.cleanup()
+    assert made[0].cleaned
+
+    class Failing(Net):
+        def buildLayers(self, f):
+            fa.ConvLayerBuilder(3, "conv").type(T.CONVOLUTION2D).number(1).shape(16, 20, 24, 8).inputPadding(1).outputPadding(1).deep().push(f)
+            fa.CustomLayerBuilder("mine", lambda b: _CopyLayer(fail_forward=True)).number(2).shape(16, 20, 24, 16).inputPadding(1).outputPadding(1).deep().push(f)
+            fa.GPULayerBuilder("sig").type(T.SIGMOID).number(3).shape(16, 20, 24, 16).inputPadding(1).deep().push(f)
+
+    bad = Failing(storage)
+    bad.setup()
+    bad.layers[1].setInput(x, 0)
+    with pytest.raises(fa.FynException, match="forward callback failed"):
+        bad.forward()
+    bad.cleanup()
+    with pytest.raises(fa.FynException):     # a custom type without its implementation
+        run_single(fa.GPULayerBuilder("x").type(T.CUSTOM).number(1).shape(4, 8, 8, 4), storage, [np.zeros((4, 8, 8), np.float32)])
