@@ -937,36 +937,46 @@ void launch_shift_reduce(const ShiftReduceParams& p, hipStream_t s) {
 // ---------------------------------------------------------------------------------------------
 // layout converters (UploadLayer / DownloadLayer / GPULayerBase::copyResult formats)
 // ---------------------------------------------------------------------------------------------
+// One thread converts four channels of one pixel; pixels are the fastest index, so that plane accesses are
+// contiguous across a wavefront (image-like tensors of up to 4 channels are contiguous on the packed side too).
 template <typename T>
 __global__ __launch_bounds__(256) void chw_to_tensor_kernel(const float* chw, const TView t) {
-    const size_t n = (size_t)t.h * t.w * t.cp;
+    const size_t npix = (size_t)t.h * t.w;
+    const size_t n = npix * (t.cp >> 2);
     const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
     if (idx >= n) return;
-    const int c = (int)(idx % t.cp);
-    const size_t pix = idx / t.cp;
+    const size_t pix = idx % npix;
+    const int c = (int)(idx / npix) * 4;
     const int x = (int)(pix % t.w), y = (int)(pix / t.w);
-    const float v = c < t.c ? chw[((size_t)c * t.h + y) * t.w + x] : 0.f;
-    reinterpret_cast<T*>(t.ptr)[tv_off(t, y, x) + c] = (T)v;
+    float v[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) v[i] = c + i < t.c ? chw[(size_t)(c + i) * npix + pix] : 0.f;
+    st4<T>(reinterpret_cast<T*>(t.ptr) + tv_off(t, y, x) + c, make_float4(v[0], v[1], v[2], v[3]));
 }
 void launch_chw_to_tensor(const float* chw, const TView& t, hipStream_t s) {
-    FYN_DISPATCH_T(t.f16, chw_to_tensor_kernel, grid1d((size_t)t.h * t.w * t.cp, 256), dim3(256), s, chw, t);
+    FYN_DISPATCH_T(t.f16, chw_to_tensor_kernel, grid1d((size_t)t.h * t.w * (t.cp >> 2), 256), dim3(256), s, chw, t);
 }
 
 template <typename T>
 __global__ __launch_bounds__(256) void tensor_to_chw_kernel(const TView t, float* chw, int keep_pad) {
     const int oh = keep_pad ? t.hp() : t.h, ow = keep_pad ? t.wp() : t.w;
-    const size_t n = (size_t)t.c * oh * ow;
+    const size_t npix = (size_t)oh * ow;
+    const size_t n = npix * ((t.c + 3) >> 2);
     const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
     if (idx >= n) return;
-    const int x = (int)(idx % ow);
-    const int y = (int)((idx / ow) % oh);
-    const int c = (int)(idx / ((size_t)ow * oh));
+    const size_t pix = idx % npix;
+    const int c = (int)(idx / npix) * 4;
+    const int x = (int)(pix % ow), y = (int)(pix / ow);
     const int sy = keep_pad ? y : y + t.pad, sx = keep_pad ? x : x + t.pad;
-    chw[idx] = (float)reinterpret_cast<const T*>(t.ptr)[((size_t)sy * t.wp() + sx) * t.cp + c];
+    const float4 v = ld4<T>(reinterpret_cast<const T*>(t.ptr) + ((size_t)sy * t.wp() + sx) * t.cp + c);
+    const float vv[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+        if (c + i < t.c) chw[(size_t)(c + i) * npix + pix] = vv[i];
 }
 void launch_tensor_to_chw(const TView& t, float* chw, int include_padding, hipStream_t s) {
     const int oh = include_padding ? t.hp() : t.h, ow = include_padding ? t.wp() : t.w;
-    FYN_DISPATCH_T(t.f16, tensor_to_chw_kernel, grid1d((size_t)t.c * oh * ow, 256), dim3(256), s, t, chw, include_padding);
+    FYN_DISPATCH_T(t.f16, tensor_to_chw_kernel, grid1d((size_t)oh * ow * ((t.c + 3) >> 2), 256), dim3(256), s, t, chw, include_padding);
 }
 
 template <typename T>
