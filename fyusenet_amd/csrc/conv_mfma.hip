@@ -752,6 +752,7 @@ static int check_params(const ConvVariant& v, const ConvMfmaParams& p) {
     if (p.nsteps < 1 || p.nsteps > 256 || v.unr < 2 || p.nsteps % v.unr != 0) return -5;
     if (p.ksplit > 1 && (!p.partial || p.chunks_per_split < 1 || (p.ksplit - 1) * p.chunks_per_split >= p.cin_chunks)) return -7;
     if (p.ksplit <= 1 && p.chunks_per_split < p.cin_chunks) return -7;
+    if ((1 << p.tile_w_log2) * v.fm < 8) return -10;   // the epilogue's row mapping needs 8 / FM positions of one tile row
     return 0;
 }
 

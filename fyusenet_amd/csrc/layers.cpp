@@ -119,7 +119,8 @@ static std::vector<TileChoice> enumerate_tiles(int cout, const SubConv& sc, int 
         conv_mfma_tile(ti, &fm, &fn, &wm, &wn);
         if (force && (fm != ff[0] || fn != ff[1] || wm != ff[2] || wn != ff[3])) continue;
         const int bm = wn * fn * 32;
-        int tw = std::min(bm >= 128 ? 16 : 8, pow2ceil(sc.npos_x));
+        // (at least 8 columns: the epilogue writes 8 / FM consecutive positions of one tile row per instruction)
+        int tw = std::max(8, std::min(bm >= 128 ? 16 : 8, pow2ceil(sc.npos_x)));
         while (bm / tw > pow2ceil(sc.npos_y) && tw < pow2ceil(sc.npos_x) && tw < bm) tw *= 2;
         const int th = bm / tw;
         const int tiles = ((sc.npos_x + tw - 1) / tw) * ((sc.npos_y + th - 1) / th);

@@ -49,6 +49,18 @@ CASES = [
     (3, 256, 14, 14, 256, 1, 1, A.RELU, {"bn": True, "residual": (A.RELU, True)}),
     (1, 2048, 7, 7, 512, 1, 1, A.RELU, {"bn": True}),
     (3, 64, 30, 30, 64, 1, 1, A.RELU, {"pad_in": 2, "pad_out": 4}),   # wider halo than needed
+    # degenerate and ragged shapes
+    (3, 1, 1, 1, 1, 1, 1, A.NONE, {}),              # one pixel, one channel
+    (1, 1, 5, 7, 1, 1, 1, A.RELU, {}),
+    (3, 5, 2, 3, 7, 1, 1, A.RELU, {"bn": True}),
+    (3, 33, 9, 11, 33, 1, 1, A.RELU, {"residual": (A.NONE, False)}),   # channel counts one past a multiple of 32
+    (5, 1000, 3, 3, 17, 1, 1, A.NONE, {}),
+    (11, 8, 24, 24, 8, 1, 1, A.NONE, {}),           # largest kernel of the reference's shader set is 9x9; 11x11 still fits the step table
+    (3, 16, 31, 29, 16, 2, 1, A.RELU, {}),          # odd size with stride 2 (output = floor(size / 2))
+    (9, 3, 5, 6, 32, 1, 1, A.RELU, {}),             # wide-kernel path on images narrower than the kernel
+    (9, 3, 12, 3, 32, 1, 1, A.NONE, {}),
+    (7, 2, 3, 40, 16, 1, 1, A.RELU, {"bn": True}),
+    (5, 64, 9, 9, 3, 2, 2, A.NONE, {}),             # stride and dilation together on a 3-channel input
 ]
 
 
@@ -100,6 +112,15 @@ def test_split_k_and_wide_chunks(k, cin, cout, size, ksplit, kcmax, kw, storage,
     assert err <= TOL[storage], info
 
 
+def test_kernel_too_large_for_the_step_table_is_rejected():
+    # 13x13 on 32 channels = 338 k16 steps per chunk, more than the 256-entry step table
+    b = conv_builder(13, 8, 32, 32, 32)
+    with pytest.raises(fa.FynException, match="too many kernel taps"):
+        run_single(b, fa.STORAGE_F32, [np.zeros((32, 32, 32), np.float32)], conv_block(1, 8, 13, 32))
+    with pytest.raises(fa.FynException):          # even kernel sizes do not exist in the reference either
+        run_single(conv_builder(4, 8, 16, 16, 8), fa.STORAGE_F32, [np.zeros((8, 16, 16), np.float32)], conv_block(1, 8, 4, 8))
+
+
 def test_reference_known_answer_patterns_on_gpu():
     # antisymmetric kernel on ones (convlayertests.cpp:242-261) and 1x1 ones (:165-182): exact
     for storage in (fa.STORAGE_F32, fa.STORAGE_F16):
@@ -132,7 +153,8 @@ def test_shallow_unpadded_conv_edge_clamps():
 
 
 @pytest.mark.parametrize("storage", [fa.STORAGE_F32, fa.STORAGE_F16], ids=["f32", "f16"])
-@pytest.mark.parametrize("k,crop,cin,cout,h,w", [(3, 0, 16, 8, 12, 10), (3, 1, 128, 64, 39, 32), (2, 0, 24, 16, 9, 17), (3, 1, 64, 32, 20, 26)])
+@pytest.mark.parametrize("k,crop,cin,cout,h,w", [(3, 0, 16, 8, 12, 10), (3, 1, 128, 64, 39, 32), (2, 0, 24, 16, 9, 17), (3, 1, 64, 32, 20, 26),
+                                                 (3, 0, 1, 1, 1, 1), (2, 0, 3, 5, 1, 2), (3, 1, 7, 33, 2, 3), (3, 0, 40, 3, 5, 1)])
 def test_transconv_parity(k, crop, cin, cout, h, w, storage):
     b = fa.ConvLayerBuilder(k, "tconv").type(fa.LayerType.TRANSCONVOLUTION2D).number(1).shape(cout, h, w, cin)
     b.upsample(2).inputPadding(1).outputPadding(1).prefixAct(A.RELU).deep().crop(crop)

@@ -17,7 +17,9 @@ STORAGES = pytest.mark.parametrize("storage", [fa.STORAGE_F32, fa.STORAGE_F16], 
 
 
 @STORAGES
-@pytest.mark.parametrize("c,h,w,stride,dil,res,bn", [(32, 112, 112, 1, 1, False, True), (96, 56, 56, 2, 1, False, False),
+@pytest.mark.parametrize("c,h,w,stride,dil,res,bn", [(2, 1, 1, 1, 1, False, False), (5, 3, 2, 1, 1, True, True), (8, 2, 9, 2, 1, False, False),
+                                                      (16, 5, 4, 1, 1, False, False), (24, 7, 6, 2, 1, False, True), (40, 4, 33, 1, 1, True, False),
+                                                      (32, 112, 112, 1, 1, False, True), (96, 56, 56, 2, 1, False, False),
                                                       (144, 28, 28, 1, 1, True, True), (24, 17, 19, 1, 2, False, False),
                                                       (960, 7, 7, 1, 1, False, True), (12, 9, 9, 1, 1, True, False)])
 def test_depthwise_parity(c, h, w, stride, dil, res, bn, storage):
@@ -39,7 +41,8 @@ def test_depthwise_parity(c, h, w, stride, dil, res, bn, storage):
 
 @STORAGES
 @pytest.mark.parametrize("op,pool,stride,pad,c,h,w,act", [
-    ("max", 2, 2, 0, 4, 8, 8, A.NONE), ("max", 2, 2, 0, 23, 200, 200, A.NONE), ("max", 3, 2, 1, 64, 112, 112, A.RELU),
+    ("max", 2, 2, 0, 1, 2, 2, A.NONE), ("avg", 2, 2, 0, 3, 2, 6, A.RELU), ("max", 3, 2, 1, 9, 5, 3, A.RELU), ("avg", 3, 1, 1, 2, 1, 1, A.NONE),
+    ("max", 4, 4, 0, 8, 8, 4, A.NONE), ("max", 2, 2, 0, 4, 8, 8, A.NONE), ("max", 2, 2, 0, 23, 200, 200, A.NONE), ("max", 3, 2, 1, 64, 112, 112, A.RELU),
     ("max", 2, 2, 0, 80, 40, 30, A.RELU), ("avg", 2, 2, 0, 12, 32, 32, A.NONE), ("avg", 3, 1, 1, 16, 20, 20, A.RELU),
     ("avg", 4, 4, 0, 80, 64, 48, A.NONE), ("avg", 2, 2, 0, 23, 200, 200, A.NONE)])  # shapes of pooltests.cpp:323-354
 def test_pool_parity(op, pool, stride, pad, c, h, w, act, storage):
@@ -56,7 +59,7 @@ def test_pool_parity(op, pool, stride, pad, c, h, w, act, storage):
 
 
 @STORAGES
-@pytest.mark.parametrize("op,c,h,w", [("avg", 2048, 7, 7), ("max", 4, 200, 200), ("avg", 4, 200, 200), ("avg", 23, 13, 9), ("max", 80, 16, 16)])
+@pytest.mark.parametrize("op,c,h,w", [("avg", 1, 1, 1), ("max", 3, 1, 5), ("avg", 9, 2, 2), ("avg", 2048, 7, 7), ("max", 4, 200, 200), ("avg", 4, 200, 200), ("avg", 23, 13, 9), ("max", 80, 16, 16)])
 def test_global_pool_parity(op, c, h, w, storage):
     kind = fa.PoolLayerBuilder.POOL_MAX if op == "max" else fa.PoolLayerBuilder.POOL_AVG
     b = fa.PoolLayerBuilder(kind, "gpool").number(1).shape(c, h, w, c).prefixAct(A.RELU).deep().global_pool()
@@ -119,7 +122,7 @@ def test_concat_bit_exact(chans, relu, storage):
 
 
 @STORAGES
-@pytest.mark.parametrize("c,h,w", [(1000, 1, 1), (64, 128, 256), (128, 40, 40), (21, 33, 17), (2048, 3, 5)])  # misctests.cpp:269-275 shapes
+@pytest.mark.parametrize("c,h,w", [(1, 1, 1), (2, 3, 1), (5, 1, 7), (1000, 1, 1), (64, 128, 256), (128, 40, 40), (21, 33, 17), (2048, 3, 5)])  # misctests.cpp:269-275 shapes
 def test_argmax_indices_exact(c, h, w, storage):
     b = fa.ArgMaxLayerBuilder("argmax").number(1).shape(2, h, w, c).deep()
     x = prng.normal(90, (c, h, w))
@@ -139,7 +142,7 @@ def test_argmax_indices_exact(c, h, w, storage):
 
 
 @STORAGES
-@pytest.mark.parametrize("cin,cout,bn", [(2048, 1000, False), (512, 256, False), (100, 10, True)])
+@pytest.mark.parametrize("cin,cout,bn", [(1, 1, False), (3, 7, True), (1025, 2, False), (2048, 1000, False), (512, 256, False), (100, 10, True)])
 def test_gemm_parity(cin, cout, bn, storage):
     b = fa.GPULayerBuilder("fc").type(fa.LayerType.GEMM).number(1).shape(cout, 1, 1, cin).prefixAct(A.RELU).deep()
     if bn:
