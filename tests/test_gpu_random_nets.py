@@ -1,4 +1,4 @@
-"""Randomly composed layer chains against the CPU oracle, through the C ABI: shapes, strides, paddings, activations
+"""Randomly composed layer graphs (chains with residual and concatenation edges) against the CPU oracle, through the C ABI: shapes, strides, paddings, activations
 and layer types are drawn from a seeded generator, so that halo handling, tile selection at odd sizes, buffer reuse
 between unrelated layers and the hand-over of activations are exercised in combinations no hand-written case lists.
 Every layer is compared on identical inputs (fp16 storage) or along the free-running chain (fp32 storage)."""
@@ -29,6 +29,10 @@ def _random_chain(seed):
             kinds.append("tconv")
         if c <= 64:
             kinds.append("transpose")
+        if specs:
+            kinds += ["resconv", "resconv"]
+            if len(specs) >= 2 and specs[-2]["out"][1:] == (h, w) and c + specs[-2]["out"][0] <= 128:
+                kinds += ["cat", "cat"]
         kind = str(rng.choice(kinds))
         act = [A.NONE, A.RELU, A.CLIP, A.LEAKY_RELU][int(rng.randint(0, 4))]
         s = {"kind": kind, "act": act, "cin": c, "h": h, "w": w}
@@ -40,6 +44,14 @@ def _random_chain(seed):
             s["bn"] = bool(rng.randint(0, 2))
             s["pad_in"] = (s["k"] - 1) // 2 * s["dil"]
             c, h, w = s["cout"], h // s["stride"], w // s["stride"]
+        elif kind == "resconv":       # y = conv3x3(x) (+BN) + [ReLU](x): both ports read the previous layer
+            s["bn"] = bool(rng.randint(0, 2))
+            s["res_relu"] = bool(rng.randint(0, 2))
+            s["pad_in"] = 1
+        elif kind == "cat":           # concat(previous layer, the layer before it)
+            s["other"] = len(specs) - 2
+            s["pad_in"] = int(rng.randint(0, 2))
+            c = c + specs[-2]["out"][0]
         elif kind == "dw":
             s["stride"] = int(rng.choice([1, 2])) if min(h, w) >= 4 else 1
             s["bn"] = bool(rng.randint(0, 2))
@@ -87,11 +99,23 @@ def _random_chain(seed):
     return shape0, specs, int(rng.randint(0, 2))
 
 
-def _builder(i, s, pad_out):
+def _builder(i, s, pad_out, specs=None, pads=None):
     no, name = i + 1, "%s%d" % (s["kind"], i + 1)
     cin, h, w = s["cin"], s["h"], s["w"]
     k = s["kind"]
-    if k in ("conv", "dw", "tconv"):
+    if k == "resconv":
+        b = fa.ConvLayerBuilder(3, name).type(T.CONVOLUTION2D).shape(cin, h, w, cin)
+        if s["bn"]:
+            b.postfixNorm(fa.NormType.BATCHNORM)
+        b.residual(A.RELU if s["res_relu"] else A.NONE, s["bn"]).residualPadding(s["pad_in"])
+        weights = conv_block(1000 + 17 * no, cin, 3, cin, bn=s["bn"])
+    elif k == "cat":
+        o = s["other"]
+        b = fa.ConcatLayerBuilder(name).input(cin, s["pad_in"]).input(specs[o]["out"][0], pads[o])
+        b.size(w, h)
+        b.outputChannels_ = s["out"][0]
+        weights = None
+    elif k in ("conv", "dw", "tconv"):
         kk = 3 if k == "dw" else s["k"]
         cout = cin if k == "dw" else s["cout"]
         b = fa.ConvLayerBuilder(kk, name).type(T.TRANSCONVOLUTION2D if k == "tconv" else T.CONVOLUTION2D).shape(cout, h, w, cin)
@@ -126,6 +150,8 @@ def _builder(i, s, pad_out):
         weights = None
     b.number(no).inputPadding(s["pad_in"]).outputPadding(pad_out).deep()
     act = s["act"]
+    if k == "cat" and act == A.LEAKY_RELU:
+        act = A.RELU
     if k in ("pool",) and s["op"] == "max" and act in (A.CLIP, A.LEAKY_RELU):
         act = A.RELU      # the zero halo of a max-pool only equals -inf padding under a non-negative activation
     b.prefixAct(act)
@@ -143,9 +169,9 @@ def test_random_chain(seed, storage):
     if not specs:
         pytest.skip("empty chain")
     built = []
+    pads = [specs[i + 1]["pad_in"] if i + 1 < len(specs) else last_pad for i in range(len(specs))]   # output padding per layer
     for i, s in enumerate(specs):
-        pad_out = specs[i + 1]["pad_in"] if i + 1 < len(specs) else last_pad
-        built.append(_builder(i, s, pad_out))
+        built.append(_builder(i, s, pads[i], specs, pads))
     print("seed", seed, "input", shape0, [(s["kind"], s["out"]) for s in specs], flush=True)
 
     class Net(fa.NeuralNetwork):
@@ -156,6 +182,10 @@ def test_random_chain(seed, storage):
         def connectLayers(self, layers, bm):
             for i in range(1, len(built)):
                 bm.connectLayers(layers[i], layers[i + 1], 0)
+                if specs[i]["kind"] == "resconv":
+                    bm.connectLayers(layers[i], layers[i + 1], 1)
+                if specs[i]["kind"] == "cat":
+                    bm.connectLayers(layers[specs[i]["other"] + 1], layers[i + 1], 1)
 
         def initializeWeights(self, layers):
             for b, w in built:
