@@ -151,19 +151,39 @@ __device__ __forceinline__ void stage_store(unsigned char* dst, int plane, const
     }
 }
 
-// One B (activation) fragment of a lane: 8 consecutive halves.  The small-Cin layout is only 8-byte
-// aligned, so it is read as two 4-half pieces.
+// Per-step LDS offset(s) of the B fragments.  Chunks of 8 or more channels: one offset per step, a lane's 8 halves
+// are consecutive channels of one tap.  Small-Cin layout (KC == 4, pixels of 4 channels = 8 bytes): a lane's 8 halves
+// are two taps, each with an offset of its own (taps are packed densely, four per k16 step, whatever their
+// positions), selected by the lane's half of the wavefront.
 template <int KC>
-__device__ __forceinline__ half8_t load_b_frag(const unsigned char* src) {
-    if (KC == 4) {
-        const half4_t lo4 = *reinterpret_cast<const half4_t*>(src);
-        const half4_t hi4 = *reinterpret_cast<const half4_t*>(src + 8);
+struct StepOff {
+    int v;
+};
+template <>
+struct StepOff<4> {
+    int2 v;
+};
+template <int KC>
+__device__ __forceinline__ StepOff<KC> load_step_off(const int* steptab, int step, int lane) {
+    StepOff<KC> r;
+    if constexpr (KC == 4) r.v = reinterpret_cast<const int2*>(steptab)[2 * step + (lane >> 5)];
+    else r.v = steptab[step];
+    return r;
+}
+
+// One B (activation) fragment of a lane: 8 halves.
+template <int KC>
+__device__ __forceinline__ half8_t load_b_frag(const unsigned char* base, const StepOff<KC>& ao) {
+    if constexpr (KC == 4) {
+        const half4_t lo4 = *reinterpret_cast<const half4_t*>(base + ao.v.x);
+        const half4_t hi4 = *reinterpret_cast<const half4_t*>(base + ao.v.y);
         half8_t r;
         r[0] = lo4[0]; r[1] = lo4[1]; r[2] = lo4[2]; r[3] = lo4[3];
         r[4] = hi4[0]; r[5] = hi4[1]; r[6] = hi4[2]; r[7] = hi4[3];
         return r;
+    } else {
+        return *reinterpret_cast<const half8_t*>(base + ao.v);
     }
-    return *reinterpret_cast<const half8_t*>(src);
 }
 
 template <typename TIn, typename TOut, bool SPLIT, int FM, int FN, int WM, int WN, int KC, int PD, int UNR>
@@ -234,7 +254,7 @@ __device__ __forceinline__ void conv_mfma_body(const ConvMfmaParams& p, unsigned
     for (int fn = 0; fn < FN; fn++) {
         const int m = (wn * FN + fn) * 32 + (lane & 31);
         const int ty = m >> twl, tx = m & (TW - 1);
-        boff[fn] = (ty * p.in_stride) * p.row_pitch + (tx * p.in_stride) * p.pitch + (lane >> 5) * 16;
+        boff[fn] = (ty * p.in_stride) * p.row_pitch + (tx * p.in_stride) * p.pitch + ((KC == 4) ? 0 : (lane >> 5) * 16);
     }
 
     // A (weight) fragments: [(chunk*nsteps + step)][mfrag][plane][lane] x 8 halves
@@ -273,7 +293,7 @@ __device__ __forceinline__ void conv_mfma_body(const ConvMfmaParams& p, unsigned
     // reads the entry of step t+2 with an ordinary (asynchronous) LDS load into a VGPR; the value is only
     // consumed one step later, so the lookup never stalls the instruction stream.
     int* steptab = reinterpret_cast<int*>(lds);
-    if (tid < p.nsteps) steptab[tid] = p.aoff[tid];
+    if (tid < p.nsteps * ((KC == 4) ? 4 : 1)) steptab[tid] = p.aoff[tid];   // (KC == 4: four tap offsets per step)
     unsigned char* const sbase = lds + 1024;   // staging buffers follow the table
 
     // ---- staging machinery: items (pixel, 8-channel group) of the halo tile; the first NB items of a
@@ -376,9 +396,9 @@ __device__ __forceinline__ void conv_mfma_body(const ConvMfmaParams& p, unsigned
     half8_t b_buf[2][FN][NPL];
     unsigned char* cur = sbase;
     // step offsets of the next two steps (ping-pong like the B fragments)
-    int ao_reg[2];
-    ao_reg[0] = steptab[0];
-    ao_reg[1] = steptab[p.nsteps > 1 ? 1 : 0];
+    StepOff<KC> ao_reg[2];
+    ao_reg[0] = load_step_off<KC>(steptab, 0, lane);
+    ao_reg[1] = load_step_off<KC>(steptab, p.nsteps > 1 ? 1 : 0, lane);
     // PD steps starting at step t0 of the current chunk.  The body is branch-free (after the chunk's last
     // step the B prefetch re-reads step 0, unused) and written as one slot per MFMA: the MFMA, then a share
     // of the step's memory instructions -- LDS reads of the B fragments of step t+1, and the refill of the
@@ -392,9 +412,9 @@ __device__ __forceinline__ void conv_mfma_body(const ConvMfmaParams& p, unsigned
 #pragma unroll
         for (int dd = 0; dd < UNR; dd++) {
             const int d = dd % PD;                            // ring slot of this step
-            const int ao = ao_reg[(dd + 1) & 1];              // offset of step t+1 (loaded one step ago)
+            const StepOff<KC> ao = ao_reg[(dd + 1) & 1];      // offset of step t+1 (loaded one step ago)
             const int t2 = t0 + dd + 2;                       // the table wraps: the next chunk starts at step 0 again
-            const int* tab2 = steptab + (t2 < p.nsteps ? t2 : t2 - p.nsteps);
+            const int step2 = t2 < p.nsteps ? t2 : t2 - p.nsteps;
             const int dprev = (d + PD - 1) % PD;       // ring slot of the previous step: free for refill
             const unsigned char* w_ = wnext;                  // fragments of step gs+PD-1
             wnext += wstep;
@@ -404,10 +424,10 @@ __device__ __forceinline__ void conv_mfma_body(const ConvMfmaParams& p, unsigned
                 const int fm = rem / FN, fn = rem % FN;
                 const int apl = (kind == 1) ? 1 : 0, bpl = (kind == 2) ? 1 : 0;
                 acc[fm][fn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_q[d][fm][apl], b_buf[dd & 1][fn][bpl], acc[fm][fn], 0, 0, 0);
-                if (i == 0) ao_reg[dd & 1] = *tab2;          // this parity's old value (step t) was consumed during step t-1
+                if (i == 0) ao_reg[dd & 1] = load_step_off<KC>(steptab, step2, lane);   // this parity's old value (step t) was consumed during step t-1
 #pragma unroll
                 for (int j = i * NDS / NMF; j < (i + 1) * NDS / NMF; j++)   // plane 0 of all fragments first
-                    b_buf[(dd + 1) & 1][j % FN][j / FN] = load_b_frag<KC>(cur + (j / FN) * p.plane + (boff[j % FN] + ao));
+                    b_buf[(dd + 1) & 1][j % FN][j / FN] = load_b_frag<KC>(cur + (j / FN) * p.plane + boff[j % FN], ao);
 #pragma unroll
                 for (int j = i * NVM / NMF; j < (i + 1) * NVM / NMF; j++)
                     a_q[dprev][j % FM][j / FM] = *reinterpret_cast<const half8_t*>(w_ + ((j % FM) * NPL + j / FM) * 1024 + wlane);
@@ -420,11 +440,11 @@ __device__ __forceinline__ void conv_mfma_body(const ConvMfmaParams& p, unsigned
         // (after the last chunk the fetch is unused; it keeps the number of loads in flight static)
         if (stager) fetch_first(more_chunks ? chunk + 1 : chunk);
         if (consumer) {
-            const int ao = ao_reg[0];
+            const StepOff<KC> ao = ao_reg[0];
 #pragma unroll
             for (int fn = 0; fn < FN; fn++)
 #pragma unroll
-                for (int pl = 0; pl < NPL; pl++) b_buf[0][fn][pl] = load_b_frag<KC>(cur + pl * p.plane + (boff[fn] + ao));
+                for (int pl = 0; pl < NPL; pl++) b_buf[0][fn][pl] = load_b_frag<KC>(cur + pl * p.plane + boff[fn], ao);
             for (int t0 = 0; t0 < p.nsteps; t0 += UNR) run_group(t0);
         }
         FYN_TRACE(2 + 2 * (chunk - chunk0));
@@ -752,7 +772,8 @@ static int check_params(const ConvVariant& v, const ConvMfmaParams& p) {
     if (p.nsteps < 1 || p.nsteps > 256 || v.unr < 2 || p.nsteps % v.unr != 0) return -5;
     if (p.ksplit > 1 && (!p.partial || p.chunks_per_split < 1 || (p.ksplit - 1) * p.chunks_per_split >= p.cin_chunks)) return -7;
     if (p.ksplit <= 1 && p.chunks_per_split < p.cin_chunks) return -7;
-    if ((1 << p.tile_w_log2) * v.fm < 8) return -10;   // the epilogue's row mapping needs 8 / FM positions of one tile row
+    if ((1 << p.tile_w_log2) * v.fm < 8) return -10;
+    if (v.kc == 4 && p.nsteps > 64) return -5;   // four table entries per step in the 1 KB table   // the epilogue's row mapping needs 8 / FM positions of one tile row
     return 0;
 }
 

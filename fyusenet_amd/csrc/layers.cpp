@@ -90,6 +90,7 @@ struct MfmaLaunch {
     // host-side description of the k16 steps of one chunk: 16 (ky,kx,ci_rel) triples, ci_rel < 0 = zero
     struct Step {
         int aoff;
+        int off4[4] = {0, 0, 0, 0};   // chunks of 4 channels: one LDS offset per tap of the step
         int ky[16], kx[16], ci[16];
     };
     std::vector<Step> steps;
@@ -212,28 +213,22 @@ static MfmaLaunch plan_mfma(Net* net, const SubConv& sc, const TView& in, const 
 
     // k16 steps
     if (kc == 4) {
+        // small-Cin layout: a pixel is 4 channels (8 bytes); a k16 step holds four taps wherever they are, each
+        // with its own LDS offset (table entry = 4 offsets per step), so K is padded only at the very end
         std::vector<Tap> taps = sc.taps;
         std::sort(taps.begin(), taps.end(), [](const Tap& a, const Tap& b) { return a.oy != b.oy ? a.oy < b.oy : a.ox < b.ox; });
-        size_t i = 0;
-        while (i < taps.size()) {
-            size_t j = i + 1;
-            while (j < taps.size() && taps[j].oy == taps[i].oy && taps[j].ox == taps[j - 1].ox + 1) j++;
-            const int len = (int)(j - i);
-            const int nst = (len * 4 + 15) / 16;
-            for (int s = 0; s < nst; s++) {
-                MfmaLaunch::Step st;
-                st.aoff = taps[i].oy * p.row_pitch + taps[i].ox * pitch + s * 32;
-                for (int e = 0; e < 16; e++) {
-                    const int r = s * 16 + e, q = r / 4;
-                    if (q < len) {
-                        st.ky[e] = taps[i + q].ky; st.kx[e] = taps[i + q].kx; st.ci[e] = r % 4;
-                    } else {
-                        st.ky[e] = st.kx[e] = 0; st.ci[e] = -1;
-                    }
+        for (size_t i = 0; i < taps.size(); i += 4) {
+            MfmaLaunch::Step st;
+            st.aoff = 0;
+            for (int q = 0; q < 4; q++) {
+                const bool have = i + q < taps.size();
+                const Tap& t = taps[have ? i + q : i];      // an absent tap reads the step's first tap with zero weights
+                st.off4[q] = t.oy * p.row_pitch + t.ox * pitch;
+                for (int e = 0; e < 4; e++) {
+                    st.ky[4 * q + e] = t.ky; st.kx[4 * q + e] = t.kx; st.ci[4 * q + e] = have ? e : -1;
                 }
-                L.steps.push_back(st);
             }
-            i = j;
+            L.steps.push_back(st);
         }
     } else {
         for (const Tap& t : sc.taps)
@@ -266,10 +261,14 @@ static MfmaLaunch plan_mfma(Net* net, const SubConv& sc, const TView& in, const 
         for (int e = 0; e < 16; e++) { st.ky[e] = st.kx[e] = 0; st.ci[e] = -1; }
         L.steps.push_back(st);
     }
+    if (kc == 4 && L.steps.size() > 64) fail(FYN_ERR_UNSUPPORTED, "too many kernel taps for the MFMA convolution (%zu steps)", L.steps.size());
     if (L.steps.size() > 256) fail(FYN_ERR_UNSUPPORTED, "too many kernel taps for the MFMA convolution (%zu steps per chunk)", L.steps.size());
     p.nsteps = (int)L.steps.size();
-    std::vector<int> aoff(L.steps.size());
-    for (size_t i = 0; i < L.steps.size(); i++) aoff[i] = L.steps[i].aoff;
+    std::vector<int> aoff;
+    for (const MfmaLaunch::Step& st : L.steps) {
+        if (kc == 4) aoff.insert(aoff.end(), st.off4, st.off4 + 4);
+        else aoff.push_back(st.aoff);
+    }
     L.aoff_dev = upload(net, aoff);
     p.aoff = L.aoff_dev;
     L.wpack_halves = (size_t)p.cin_chunks * p.nsteps * p.mfrags * npl * 64 * 8;
