@@ -240,13 +240,6 @@ __device__ __forceinline__ void conv_mfma_body(const ConvMfmaParams& p, unsigned
     // LDS holds two staging buffers (double buffering across channel chunks) when there is more
     // than one chunk; each buffer = NPL planes.
     const int bufsz = NPL * p.plane;
-    if (KC == 4) {
-        // slack behind each plane is read by the last (zero-weight) k elements of a row run
-        if (tid < 16 * NPL) {
-            int pl = tid >> 4;
-            reinterpret_cast<uint32_t*>(lds + 1024 + pl * p.plane + p.halo_h * p.row_pitch)[tid & 15] = 0u;
-        }
-    }
 
     // per-lane LDS byte offsets of the B (activation) fragments
     int boff[FN];

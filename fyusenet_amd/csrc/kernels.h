@@ -85,7 +85,7 @@ struct ConvVariant {
     int split;           // 1: hi/lo fp16 split of both operands (fp32-accurate), 3 MFMAs per pair
     int fm, fn;          // fragments (32 cout / 32 positions) per wave
     int wm, wn;          // waves per block along cout / positions (wm*wn == 4)
-    int kc;              // input channels staged per chunk (4 = row-run small-Cin variant, 16, 32)
+    int kc;              // input channels staged per chunk (4 = small-Cin layout with per-tap offsets, 16, 32, 64, 128)
     int pd;              // depth of the weight-fragment prefetch ring in k16 steps (2, 4, 6)
     int unr;             // k16 steps per unrolled group (a multiple of pd; nsteps is a multiple of it)
 };

@@ -156,7 +156,7 @@ static void conv_geometry(const TView& in, bool split, int ntaps, int kc_force, 
     else kc = 32;
     if (kc_force > 0) kc = kc_force;
     pitch = (kc == 4) ? 8 : kc * 2 + 16;
-    slack = (kc == 4) ? 64 : 0;
+    slack = 0;
     npl = split ? 2 : 1;
 }
 
