@@ -197,7 +197,12 @@ __device__ __forceinline__ void conv_mfma_body(const ConvMfmaParams& p, unsigned
     constexpr int NPL = SPLIT ? 2 : 1;         // operand planes (hi, lo)
     constexpr int CPI = (KC == 4) ? 4 : 8;     // channels per staging item
     constexpr int G = (KC == 4) ? 1 : KC / 8;  // staging items per pixel
-    static_assert(WM * WN == 4, "4 waves per block");
+    // The four MFMA waves are arranged WM x WN over the tile; when WM*WN < 4 the remaining factor WK splits the
+    // k16 steps of every chunk among waves that share an output sub-tile (their accumulators meet in LDS in the
+    // epilogue): small tiles keep four waves busy and the reduction of a layer with few positions is spread
+    // over more workgroups without a second pass.
+    static_assert(WM * WN == 1 || WM * WN == 2 || WM * WN == 4, "1, 2 or 4 sub-tiles per block");
+    constexpr int WK = 4 / (WM * WN);
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -206,7 +211,8 @@ __device__ __forceinline__ void conv_mfma_body(const ConvMfmaParams& p, unsigned
     const bool stager = !SPEC || wave >= 4;    // stages input tiles
     const int stid = SPEC ? (tid & 255) : tid; // thread index among the staging threads
     const int wm = (wave & 3) % WM;
-    const int wn = (wave & 3) / WM;
+    const int wn = ((wave & 3) / WM) % WN;
+    const int wk = (wave & 3) / (WM * WN);      // 0 when WK == 1
 
     // Workgroups are dealt round-robin to the 8 XCDs; remap so that neighbouring tiles (shared
     // halos, same input tile for all cout blocks) meet in one XCD's L2.
@@ -257,8 +263,10 @@ __device__ __forceinline__ void conv_mfma_body(const ConvMfmaParams& p, unsigned
     const unsigned wstep = (unsigned)p.mfrags * NPL * 1024;   // bytes per k16 step
     const int chunk0 = ks * p.chunks_per_split;                // this workgroup's channel chunks: [chunk0, chunk1)
     const int chunk1 = (chunk0 + p.chunks_per_split < p.cin_chunks) ? chunk0 + p.chunks_per_split : p.cin_chunks;
+    // (WK > 1: the steps of wave group wk are stored as a contiguous run over all chunks, [wk][chunk][step of the group])
+    const int nsub = p.nsteps / WK;                            // steps per chunk of this wave
     const unsigned char* wbase = reinterpret_cast<const unsigned char*>(p.wpack) + (size_t)((cb * WM + wm) * FM) * NPL * 1024 +
-                                 (size_t)chunk0 * p.nsteps * wstep;
+                                 ((size_t)wk * p.cin_chunks + chunk0) * nsub * wstep;
     const unsigned wlane = lane * 16;
 
     float16_t acc[FM][FN];
@@ -390,8 +398,9 @@ __device__ __forceinline__ void conv_mfma_body(const ConvMfmaParams& p, unsigned
     unsigned char* cur = sbase;
     // step offsets of the next two steps (ping-pong like the B fragments)
     StepOff<KC> ao_reg[2];
-    ao_reg[0] = load_step_off<KC>(steptab, 0, lane);
-    ao_reg[1] = load_step_off<KC>(steptab, p.nsteps > 1 ? 1 : 0, lane);
+    const int tab0 = wk * nsub;                                // this wave's first step in the table
+    ao_reg[0] = load_step_off<KC>(steptab, tab0, lane);
+    ao_reg[1] = load_step_off<KC>(steptab, tab0 + (nsub > 1 ? 1 : 0), lane);
     // PD steps starting at step t0 of the current chunk.  The body is branch-free (after the chunk's last
     // step the B prefetch re-reads step 0, unused) and written as one slot per MFMA: the MFMA, then a share
     // of the step's memory instructions -- LDS reads of the B fragments of step t+1, and the refill of the
@@ -407,7 +416,7 @@ __device__ __forceinline__ void conv_mfma_body(const ConvMfmaParams& p, unsigned
             const int d = dd % PD;                            // ring slot of this step
             const StepOff<KC> ao = ao_reg[(dd + 1) & 1];      // offset of step t+1 (loaded one step ago)
             const int t2 = t0 + dd + 2;                       // the table wraps: the next chunk starts at step 0 again
-            const int step2 = t2 < p.nsteps ? t2 : t2 - p.nsteps;
+            const int step2 = tab0 + (t2 < nsub ? t2 : t2 - nsub);
             const int dprev = (d + PD - 1) % PD;       // ring slot of the previous step: free for refill
             const unsigned char* w_ = wnext;                  // fragments of step gs+PD-1
             wnext += wstep;
@@ -438,7 +447,7 @@ __device__ __forceinline__ void conv_mfma_body(const ConvMfmaParams& p, unsigned
             for (int fn = 0; fn < FN; fn++)
 #pragma unroll
                 for (int pl = 0; pl < NPL; pl++) b_buf[0][fn][pl] = load_b_frag<KC>(cur + pl * p.plane + boff[fn], ao);
-            for (int t0 = 0; t0 < p.nsteps; t0 += UNR) run_group(t0);
+            for (int t0 = 0; t0 < nsub; t0 += UNR) run_group(t0);
         }
         FYN_TRACE(2 + 2 * (chunk - chunk0));
         if (more_chunks) {
@@ -459,12 +468,42 @@ __device__ __forceinline__ void conv_mfma_body(const ConvMfmaParams& p, unsigned
     //      16-byte pieces; scale, bias' and the residual are applied on the way out
     //      (shaders/deep/deepconv3x3_tiled.frag:36-45 order). ----
     __syncthreads();  // all waves are done with the staged tiles; LDS is reused below
-    if (!consumer) return;
-    FYN_TRACE(14);
     constexpr int ROWF = FM * 32 + 4;                 // floats per position row (+4: bank spread)
     constexpr int LPP = FM * 8;                       // lanes per position on the way out
     constexpr int PPI = 64 / LPP;                     // positions per store instruction
+    constexpr int ITS = 32 / PPI;                     // store instructions per fragment ...
+    constexpr int ITW = ITS / WK;                     // ... of which a wave issues this many (K groups share the rows out)
+    static_assert(ITS % WK == 0, "rows of a fragment divide among the K groups");
     float* tr = reinterpret_cast<float*>(lds) + (wave & 3) * (FN * 32 * ROWF);   // FN fragments of 32 rows per wave
+    auto acc_to_lds = [&]() {
+#pragma unroll
+        for (int fn = 0; fn < FN; fn++)
+#pragma unroll
+            for (int fm = 0; fm < FM; fm++)
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    f32x4_t v;
+                    v[0] = acc[fm][fn][q * 4 + 0]; v[1] = acc[fm][fn][q * 4 + 1];
+                    v[2] = acc[fm][fn][q * 4 + 2]; v[3] = acc[fm][fn][q * 4 + 3];
+                    *reinterpret_cast<f32x4_t*>(tr + (fn * 32 + (lane & 31)) * ROWF + fm * 32 + q * 8 + (lane >> 5) * 4) = v;
+                }
+    };
+    // With K groups, every wave first publishes its partial accumulators; a wave then finishes the rows
+    // it = i*WK + wk of its sub-tile, adding the groups' partial sums in group order.
+    if constexpr (WK > 1) {
+        if (consumer) acc_to_lds();
+        __syncthreads();
+    }
+    if (!consumer) return;
+    FYN_TRACE(14);
+    const float* tr0 = reinterpret_cast<const float*>(lds) + ((wave & 3) % (WM * WN)) * (FN * 32 * ROWF);   // K group 0's area of this sub-tile
+    constexpr int TRK = WM * WN * FN * 32 * ROWF;     // floats between the areas of consecutive K groups
+    auto row_from_lds = [&](int fn, int it) {
+        f32x4_t v = *reinterpret_cast<const f32x4_t*>(tr0 + (fn * 32 + it * PPI + lane / LPP) * ROWF + (lane % LPP) * 4);
+#pragma unroll
+        for (int k = 1; k < WK; k++) v += *reinterpret_cast<const f32x4_t*>(tr0 + k * TRK + (fn * 32 + it * PPI + lane / LPP) * ROWF + (lane % LPP) * 4);
+        return v;
+    };
     TOut* out = reinterpret_cast<TOut*>(p.out);
     const TOut* res = reinterpret_cast<const TOut*>(p.res);
     const int c4 = (lane % LPP) * 4;                                   // channel offset inside the wave's range
@@ -482,21 +521,14 @@ __device__ __forceinline__ void conv_mfma_body(const ConvMfmaParams& p, unsigned
         // split-K: raw partial sums, [ks][position][cout_pad] fp32; the reduce pass finishes the layer
         float* part = p.partial + (size_t)ks * p.npos_y * p.npos_x * p.cout_pad;
         const bool cp_ok = c < p.cout_pad;
+        if constexpr (WK == 1) acc_to_lds();
 #pragma unroll
         for (int fn = 0; fn < FN; fn++) {
 #pragma unroll
-            for (int fm = 0; fm < FM; fm++)
-#pragma unroll
-                for (int q = 0; q < 4; q++) {
-                    f32x4_t v;
-                    v[0] = acc[fm][fn][q * 4 + 0]; v[1] = acc[fm][fn][q * 4 + 1];
-                    v[2] = acc[fm][fn][q * 4 + 2]; v[3] = acc[fm][fn][q * 4 + 3];
-                    *reinterpret_cast<f32x4_t*>(tr + (fn * 32 + (lane & 31)) * ROWF + fm * 32 + q * 8 + (lane >> 5) * 4) = v;
-                }
-#pragma unroll
-            for (int it = 0; it < 32 / PPI; it++) {
+            for (int i = 0; i < ITW; i++) {
+                const int it = (WK == 1) ? i : i * WK + wk;
                 const int row = it * PPI + lane / LPP;
-                const f32x4_t v = *reinterpret_cast<const f32x4_t*>(tr + (fn * 32 + row) * ROWF + c4);
+                const f32x4_t v = row_from_lds(fn, it);
                 const int m = (wn * FN + fn) * 32 + row;
                 const int py = pos_y0 + (m >> twl), px = pos_x0 + (m & (TW - 1));
                 if (cp_ok && py < p.npos_y && px < p.npos_x)
@@ -508,18 +540,17 @@ __device__ __forceinline__ void conv_mfma_body(const ConvMfmaParams& p, unsigned
     // Row r of a fragment is position m = frag*32 + it*PPI + lane/LPP; PPI divides the tile width, so the
     // tile row (and with it the image row) of an (fn, it) pair is wave-uniform and only the column carries a
     // per-lane part: base addresses are scalar, the per-lane offset is computed once.
-    constexpr int ITS = 32 / PPI;
     const int lrow = lane / LPP;
     const int out_lane = lrow * p.out_step * p.out_cp + c;
     const int res_lane = lrow * p.out_step * p.res_cp + c;
-    bool ok[FN][ITS];
-    size_t obase[FN][ITS];
-    float rres[FN][ITS][4];
+    bool ok[FN][ITW];
+    size_t obase[FN][ITW];
+    float rres[FN][ITW][4];
 #pragma unroll
     for (int fn = 0; fn < FN; fn++)
 #pragma unroll
-        for (int it = 0; it < ITS; it++) {
-            const int m0 = (wn * FN + fn) * 32 + it * PPI;
+        for (int it = 0; it < ITW; it++) {
+            const int m0 = (wn * FN + fn) * 32 + ((WK == 1) ? it : it * WK + wk) * PPI;
             const int py = pos_y0 + (m0 >> twl), px0 = pos_x0 + (m0 & (TW - 1));
             ok[fn][it] = c_ok && py < p.npos_y && px0 + lrow < p.npos_x;
             obase[fn][it] = ((size_t)(p.out_off_y + py * p.out_step) * p.out_wp + p.out_off_x + px0 * p.out_step) * p.out_cp + out_lane;
@@ -534,30 +565,19 @@ __device__ __forceinline__ void conv_mfma_body(const ConvMfmaParams& p, unsigned
             }
         }
     FYN_TRACE(9);
-#pragma unroll
-    for (int fn = 0; fn < FN; fn++)
-#pragma unroll
-        for (int fm = 0; fm < FM; fm++)
-#pragma unroll
-            for (int q = 0; q < 4; q++) {
-                f32x4_t v;
-                v[0] = acc[fm][fn][q * 4 + 0]; v[1] = acc[fm][fn][q * 4 + 1];
-                v[2] = acc[fm][fn][q * 4 + 2]; v[3] = acc[fm][fn][q * 4 + 3];
-                *reinterpret_cast<f32x4_t*>(tr + (fn * 32 + (lane & 31)) * ROWF + fm * 32 + q * 8 + (lane >> 5) * 4) = v;
-            }
+    if constexpr (WK == 1) acc_to_lds();
     FYN_TRACE(10);
-    f32x4_t a4[FN][ITS];
+    f32x4_t a4[FN][ITW];
 #pragma unroll
     for (int fn = 0; fn < FN; fn++)
 #pragma unroll
-        for (int it = 0; it < ITS; it++)
-            a4[fn][it] = *reinterpret_cast<const f32x4_t*>(tr + (fn * 32 + it * PPI + lane / LPP) * ROWF + c4);
+        for (int it = 0; it < ITW; it++) a4[fn][it] = row_from_lds(fn, (WK == 1) ? it : it * WK + wk);
     // arithmetic for every row unconditionally (one wait for the loads above), then predicated stores only:
     // a wait inside a predicated region would also wait for the stores issued before it
 #pragma unroll
     for (int fn = 0; fn < FN; fn++)
 #pragma unroll
-        for (int it = 0; it < ITS; it++)
+        for (int it = 0; it < ITW; it++)
 #pragma unroll
             for (int i = 0; i < 4; i++) {
                 float rv = rres[fn][it][i];   // zero without a residual input
@@ -570,12 +590,12 @@ __device__ __forceinline__ void conv_mfma_body(const ConvMfmaParams& p, unsigned
 #pragma unroll
     for (int fn = 0; fn < FN; fn++)
 #pragma unroll
-        for (int it = 0; it < ITS; it++) asm volatile("" : "+v"(a4[fn][it]));
+        for (int it = 0; it < ITW; it++) asm volatile("" : "+v"(a4[fn][it]));
     FYN_TRACE(11);
 #pragma unroll
     for (int fn = 0; fn < FN; fn++)
 #pragma unroll
-        for (int it = 0; it < ITS; it++) {
+        for (int it = 0; it < ITW; it++) {
             if (!ok[fn][it]) continue;
             if (sizeof(TOut) == 4) {
                 *reinterpret_cast<f32x4_t*>(reinterpret_cast<float*>(out) + obase[fn][it]) = a4[fn][it];
@@ -622,7 +642,7 @@ struct ConvEntry {
 #define FYN_CONV_PART 0
 #endif
 
-// (index, fm, fn, wm, wn): cout tile = wm*fm*32, position tile = wn*fn*32
+// (index, fm, fn, wm, wn): cout tile = wm*fm*32, position tile = wn*fn*32; wm*wn < 4: the other waves split K
 #define FYN_CONV_TILES(X) \
     X(0, 2, 2, 2, 2)      \
     X(1, 2, 2, 1, 4)      \
@@ -639,13 +659,22 @@ struct ConvEntry {
     X(12, 1, 4, 2, 2)     \
     X(13, 1, 3, 2, 2)     \
     X(14, 1, 4, 1, 4)     \
-    X(15, 1, 3, 1, 4)
+    X(15, 1, 3, 1, 4)     \
+    X(16, 1, 1, 1, 1)     \
+    X(17, 1, 1, 2, 1)     \
+    X(18, 1, 1, 1, 2)
 
 // (ring depth, unroll) pairs: 2/2 for chunks of 4, 16 and 32 channels; for 32-channel chunks also 4/4, 6/6 and
 // 6/18 (a whole 3x3 chunk unrolled: no loop back-edge, hence no conservative wait, inside a chunk); 64- and
 // 128-channel chunks (kernels of one to four taps: fewer chunk barriers) use 4/4 and 4/8.
 template <typename TIn, typename TOut, bool SPLIT, int FM, int FN, int WM, int WN>
 static conv_kernel_fn pick_kc(int kc, int pd, int unr) {
+    if constexpr (WM * WN < 4) {   // K-split tiles: layers with few positions and many channels; smallest step group only
+        if (kc == 32 && pd == 2 && unr == 2) return conv_mfma_kernel<TIn, TOut, SPLIT, FM, FN, WM, WN, 32, 2, 2>;
+        if (kc == 64 && pd == 2 && unr == 2) return conv_mfma_kernel<TIn, TOut, SPLIT, FM, FN, WM, WN, 64, 2, 2>;
+        if (kc == 128 && pd == 2 && unr == 2) return conv_mfma_kernel<TIn, TOut, SPLIT, FM, FN, WM, WN, 128, 2, 2>;
+        return nullptr;
+    } else {
     if (kc == 4 && pd == 2 && unr == 2) return conv_mfma_kernel<TIn, TOut, SPLIT, FM, FN, WM, WN, 4, 2, 2>;
     if (kc == 16 && pd == 2 && unr == 2) return conv_mfma_kernel<TIn, TOut, SPLIT, FM, FN, WM, WN, 16, 2, 2>;
     if (kc == 32 && pd == 2 && unr == 2) return conv_mfma_kernel<TIn, TOut, SPLIT, FM, FN, WM, WN, 32, 2, 2>;
@@ -655,15 +684,19 @@ static conv_kernel_fn pick_kc(int kc, int pd, int unr) {
     if (kc == 64 && pd == 4 && unr == 4) return conv_mfma_kernel<TIn, TOut, SPLIT, FM, FN, WM, WN, 64, 4, 4>;
     if (kc == 128 && pd == 4 && unr == 8) return conv_mfma_kernel<TIn, TOut, SPLIT, FM, FN, WM, WN, 128, 4, 8>;
     return nullptr;
+    }
 }
 
 // multi-launch entry points exist for 32-, 64- and 128-channel chunks at their smallest step group
 template <typename TIn, typename TOut, bool SPLIT, int FM, int FN, int WM, int WN>
 static conv_multi_fn pick_kc_multi(int kc, int pd, int unr) {
+    if constexpr (WM * WN < 4) return nullptr;
+    else {
     if (kc == 32 && pd == 2 && unr == 2) return conv_mfma_multi_kernel<TIn, TOut, SPLIT, FM, FN, WM, WN, 32, 2, 2>;
     if (kc == 64 && pd == 4 && unr == 4) return conv_mfma_multi_kernel<TIn, TOut, SPLIT, FM, FN, WM, WN, 64, 4, 4>;
     if (kc == 128 && pd == 4 && unr == 8) return conv_mfma_multi_kernel<TIn, TOut, SPLIT, FM, FN, WM, WN, 128, 4, 8>;
     return nullptr;
+    }
 }
 
 #define FYN_CAT2(a, b) a##b
@@ -742,7 +775,8 @@ static ConvEntry pick_kernel(const ConvVariant& v) {
 bool conv_mfma_variant_exists(const ConvVariant& v) { return pick_kernel(v).single != nullptr; }
 bool conv_mfma_multi_exists(const ConvVariant& v) { return pick_kernel(v).multi != nullptr; }
 
-int conv_mfma_step_multiple(const ConvVariant& v) { return v.unr; }
+// the steps of a chunk divide evenly among the K groups of waves, each taking whole unrolled groups
+int conv_mfma_step_multiple(const ConvVariant& v) { return v.unr * (4 / (v.wm * v.wn)); }
 
 int conv_mfma_tile_count() {
     int n = 0;
@@ -762,11 +796,11 @@ void conv_mfma_tile(int index, int* fm, int* fn, int* wm, int* wn) {
 static int blocks_of(const ConvMfmaParams& p) { return p.tiles_x * p.tiles_y * p.cout_blocks * (p.ksplit > 1 ? p.ksplit : 1); }
 
 static int check_params(const ConvVariant& v, const ConvMfmaParams& p) {
-    if (p.nsteps < 1 || p.nsteps > 256 || v.unr < 2 || p.nsteps % v.unr != 0) return -5;
+    if (p.nsteps < 1 || p.nsteps > 256 || v.unr < 2 || p.nsteps % conv_mfma_step_multiple(v) != 0) return -5;
     if (p.ksplit > 1 && (!p.partial || p.chunks_per_split < 1 || (p.ksplit - 1) * p.chunks_per_split >= p.cin_chunks)) return -7;
     if (p.ksplit <= 1 && p.chunks_per_split < p.cin_chunks) return -7;
-    if ((1 << p.tile_w_log2) * v.fm < 8) return -10;
-    if (v.kc == 4 && p.nsteps > 64) return -5;   // four table entries per step in the 1 KB table   // the epilogue's row mapping needs 8 / FM positions of one tile row
+    if ((1 << p.tile_w_log2) * v.fm < 8) return -10;   // the epilogue's row mapping needs 8 / FM positions of one tile row
+    if (v.kc == 4 && p.nsteps > 64) return -5;         // four table entries per step in the 1 KB table
     return 0;
 }
 

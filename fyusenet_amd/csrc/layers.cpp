@@ -109,7 +109,7 @@ struct TileChoice {
     int kc;      // input channels per staged chunk
 };
 
-// All tile configurations that fit, best heuristic score first.
+// All tile configurations that fit (possibly none), best heuristic score first.
 static std::vector<TileChoice> enumerate_tiles(int cout, const SubConv& sc, int pitch, int npl, int slack, int nbuf) {
     std::vector<TileChoice> all;
     const char* force = getenv("FYNHIP_CONV_TILE");  // "fm,fn,wm,wn" for experiments
@@ -139,7 +139,6 @@ static std::vector<TileChoice> enumerate_tiles(int cout, const SubConv& sc, int 
         const double bonus = (fm * fn == 4) ? 1.0 : (fm * fn == 2 ? 0.85 : 0.7);
         all.push_back(TileChoice{fm, fn, wm, wn, ilog2(tw), th, util * par * bonus, rowpad, 0});
     }
-    if (all.empty()) fail(FYN_ERR_UNSUPPORTED, "no MFMA tile configuration fits this convolution");
     std::sort(all.begin(), all.end(), [](const TileChoice& x, const TileChoice& y) { return x.score > y.score; });
     return all;
 }
@@ -250,9 +249,11 @@ static MfmaLaunch plan_mfma(Net* net, const SubConv& sc, const TView& in, const 
         if (kc >= 64) pd = 4;
         if (const char* e = getenv("FYNHIP_CONV_PD")) pd = atoi(e);
         if (force_pd > 0 && kc <= 32) pd = force_pd;
+        const bool ksplit_tile = tc.wm * tc.wn < 4;      // waves split the steps of a chunk: smallest step group
+        if (ksplit_tile) pd = 2;
         L.var.pd = pd;
         L.var.unr = (pd == 6 && raw == 18 && force_pd == 0 && !getenv("FYNHIP_CONV_NO_FULL_UNROLL")) ? 18 : pd;
-        if (kc == 128) L.var.unr = 8;
+        if (kc == 128 && !ksplit_tile) L.var.unr = 8;
         if (!conv_mfma_variant_exists(L.var)) fail(FYN_ERR_UNSUPPORTED, "MFMA convolution variant not compiled");
     }
     while (L.steps.size() % conv_mfma_step_multiple(L.var) != 0) {
@@ -404,11 +405,17 @@ static MfmaLaunch tune_mfma(Net* net, const SubConv& sc, const TView& in, const 
             for (TileChoice& tc : c) {
                 tc.kc = kc;
                 if (kco != kc0) tc.score *= 0.9;
+                if (tc.wm * tc.wn < 4) {   // tiles whose waves split K exist for chunks of 32 and more channels
+                    const int wk = 4 / (tc.wm * tc.wn);
+                    const int raw = (int)sc.taps.size() * (kc / 16);
+                    if (kc < 32 || (raw + 2 * wk - 1) / (2 * wk) * (2 * wk) > 256) continue;
+                }
                 cands.push_back(tc);
             }
         }
         std::stable_sort(cands.begin(), cands.end(), [](const TileChoice& x, const TileChoice& y) { return x.score > y.score; });
     }
+    if (cands.empty()) fail(FYN_ERR_UNSUPPORTED, "no MFMA tile configuration fits this convolution");
     const char* at = getenv("FYNHIP_AUTOTUNE");
     const bool tune = !(at && at[0] == '0') && cands.size() > 1;
     // FYNHIP_TUNE_CACHE=<file>: measured choices are remembered per problem geometry, so that later
@@ -466,13 +473,21 @@ static MfmaLaunch tune_mfma(Net* net, const SubConv& sc, const TView& in, const 
             }
         }
     }
-    // few workgroups and several channel chunks: try splitting the reduction over more workgroups
-    {
-        const int blocks = best.p.tiles_x * best.p.tiles_y * best.p.cout_blocks;
+    // few workgroups and several channel chunks: try splitting the reduction over more workgroups (for the
+    // winner and, if its waves already split K inside the workgroup, also for the best tile that does not)
+    std::vector<MfmaLaunch> bases{best};
+    if (best.var.wm * best.var.wn < 4)
+        for (const auto& t : timed)
+            if (t.second.var.wm * t.second.var.wn == 4) {
+                bases.push_back(t.second);
+                break;
+            }
+    for (const MfmaLaunch& base : bases) {
+        const int blocks = base.p.tiles_x * base.p.tiles_y * base.p.cout_blocks;
         for (int ks = 2; ks <= 16 && blocks < 192; ks *= 2) {
-            const int cps = (best.p.cin_chunks + ks - 1) / ks;
-            if (best.p.cin_chunks < 2 || (ks - 1) * cps >= best.p.cin_chunks || blocks * ks > 1024) break;
-            MfmaLaunch L = best;
+            const int cps = (base.p.cin_chunks + ks - 1) / ks;
+            if (base.p.cin_chunks < 2 || (ks - 1) * cps >= base.p.cin_chunks || blocks * ks > 1024) break;
+            MfmaLaunch L = base;
             set_ksplit(net, L, ks);
             const float ms = std::min(time_launch(net, L, 4), time_launch(net, L, 4));
             if (verbose) fprintf(stderr, "[tune] %s -> %.1f us\n", mfma_info(L).c_str(), ms * 1e3f);
@@ -549,11 +564,13 @@ static MfmaGroup tune_mfma_group(Net* net, const std::vector<SubConv>& scs, cons
             std::vector<TileChoice> c = enumerate_tiles(cout, scs[big], pitch, npl, slack, chunks > 1 ? 2 : 1);
             for (TileChoice& tc : c) {
                 tc.kc = kc;
+                if (tc.wm * tc.wn < 4) continue;   // no merged entry point for tiles whose waves split K
                 cands.push_back(tc);
             }
         }
         std::stable_sort(cands.begin(), cands.end(), [](const TileChoice& x, const TileChoice& y) { return x.score > y.score; });
     }
+    if (cands.empty()) fail(FYN_ERR_UNSUPPORTED, "no MFMA tile configuration fits this convolution");
     auto plan_all = [&](const TileChoice& tc, const MfmaGroup* share) {
         MfmaGroup g;
         for (size_t i = 0; i < scs.size(); i++)
@@ -590,18 +607,21 @@ static MfmaGroup tune_mfma_group(Net* net, const std::vector<SubConv>& scs, cons
 }
 
 // Packs weights W[o][ky][kx][i] (block order, base/convlayerinterface.h:71-95) into the per-lane A
-// fragment order of the kernel: [(chunk, step)][mfrag][plane][lane][8 halves].
+// fragment order of the kernel: [(chunk, step)][mfrag][plane][lane][8 halves]; for tiles whose waves split the
+// steps of a chunk into WK groups, [group][chunk][step of the group]... (a wave walks its steps over all chunks
+// with one stride).
 static void pack_mfma_weights(Net* net, MfmaLaunch& L, const float* w, int k, float wmul, int kw = -1) {
     if (kw < 0) kw = k;
     const ConvMfmaParams& p = L.p;
     const int npl = L.var.split ? 2 : 1;
     const int kc = L.var.kc;
     std::vector<uint16_t> pack(L.wpack_halves, 0);
+    const int nsub = p.nsteps / (4 / (L.var.wm * L.var.wn));   // steps per chunk and K group of waves
     for (int chunk = 0; chunk < p.cin_chunks; chunk++)
         for (int t = 0; t < p.nsteps; t++) {
             const MfmaLaunch::Step& st = L.steps[t];
             for (int mf = 0; mf < p.mfrags; mf++) {
-                uint16_t* base = pack.data() + ((((size_t)chunk * p.nsteps + t) * p.mfrags + mf) * npl) * 64 * 8;
+                uint16_t* base = pack.data() + (((((size_t)(t / nsub) * p.cin_chunks + chunk) * nsub + t % nsub) * p.mfrags + mf) * npl) * 64 * 8;
                 for (int lane = 0; lane < 64; lane++) {
                     const int o = mf * 32 + (lane & 31);
                     if (o >= L.cout) continue;

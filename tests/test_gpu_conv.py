@@ -112,6 +112,37 @@ def test_split_k_and_wide_chunks(k, cin, cout, size, ksplit, kcmax, kw, storage,
     assert err <= TOL[storage], info
 
 
+@pytest.mark.parametrize("storage", [fa.STORAGE_F32, fa.STORAGE_F16], ids=["f32", "f16"])
+@pytest.mark.parametrize("tile", ["1,1,1,1", "1,1,2,1", "1,1,1,2"], ids=["32x32", "64x32", "32x64"])
+@pytest.mark.parametrize("k,cin,cout,h,w,ksplit,kw", [
+    (1, 512, 96, 7, 7, 0, {"bn": True}),                                        # 128-channel chunks, two steps per wave group
+    (3, 64, 40, 14, 14, 0, {"bn": True, "residual": (A.RELU, True)}),           # 18 steps padded to a multiple of 8 (or 4)
+    (1, 160, 33, 9, 5, 0, {}),                                                  # ragged last chunk, ragged channels and tile
+    (3, 256, 64, 7, 7, 4, {"residual": (A.NONE, False)}),                       # together with split-K over workgroups
+    (5, 32, 8, 20, 12, 0, {}),
+])
+def test_tiles_whose_waves_split_k(k, cin, cout, h, w, ksplit, kw, tile, storage, monkeypatch):
+    """Small tiles (one or two 32x32 sub-tiles) whose remaining waves split the k16 steps of each chunk and add
+    their partial sums in LDS; forced through the engine's tile switch."""
+    monkeypatch.setenv("FYNHIP_CONV_TILE", tile)
+    if ksplit:
+        monkeypatch.setenv("FYNHIP_FORCE_KSPLIT", str(ksplit))
+    b = conv_builder(k, cout, h, w, cin, 1, 1, A.RELU, **kw)
+    wts = conv_block(500 + k + cin, cout, k, cin, bn=kw.get("bn", False))
+    inputs = [prng.uniform(13 * k + cin, (cin, h, w), -1, 1)]
+    if "residual" in kw:
+        inputs.append(prng.uniform(23, (cout, h, w), -1, 1))
+    got, info = run_single(b, storage, inputs, wts)
+    ref = oracle_single(b, storage, inputs, wts)
+    err = rel_l2(got, ref)
+    print("  ", info, "rel_l2=%.3e" % err, flush=True)
+    fm, fn, wm, wn = (int(v) for v in tile.split(","))
+    assert "tile=%dx%d" % (32 * fm * wm, 32 * fn * wn) in info and "waves=%dx%d" % (wm, wn) in info
+    if ksplit:
+        assert "ksplit=%d" % ksplit in info
+    assert err <= TOL[storage], info
+
+
 def test_kernel_too_large_for_the_step_table_is_rejected():
     # 13x13 on 32 channels = 338 k16 steps per chunk, more than the 256-entry step table
     b = conv_builder(13, 8, 32, 32, 32)
