@@ -345,6 +345,7 @@ class ConvLayerBuilder(GPULayerBuilder):
         d.dilation[0], d.dilation[1] = self.dilation_
         d.group_size = self.groupSize_
         d.transconv_crop = self.transconvCrop_
+        d.source_step = self.sourceStep_
 
 
 class PoolLayerBuilder(GPULayerBuilder):

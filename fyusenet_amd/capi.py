@@ -69,6 +69,7 @@ class LayerDesc(ctypes.Structure):
         ("cast_target", ctypes.c_int32),
         ("window", ctypes.c_int32),
         ("blur_type", ctypes.c_int32),
+        ("source_step", ctypes.c_float),
     ]
 
 

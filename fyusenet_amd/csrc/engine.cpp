@@ -146,10 +146,13 @@ void Net::connect(int out_layer, int in_layer, int port) {
         fail(FYN_ERR_INVALID, "layer %s (%d) cannot feed layer %s (%d): execution is in ascending number", src->d.name,
              out_layer, dst->d.name, in_layer);
     if (dst->in[port] != -1) return;  // already connected (BufferManager::checkIOMatch returns no match)
-    // I/O match (base/buffermanager.cpp:462-492): same geometry on both sides of the edge
+    // I/O match (base/buffermanager.cpp:462-492): same geometry on both sides of the edge.  The reference compares
+    // textures, four channels each, not channel counts: a consumer may name up to three channels more or fewer
+    // than were produced (the style-transfer samples download 4 channels of a 3-channel result,
+    // samples/samplenetworks/stylenet3x3.cpp:175,180).  Channels beyond the produced ones read as zero.
     int c, h, w, pad;
     dst->port_shape(port, c, h, w, pad);
-    if (c != src->oc || h != src->oh || w != src->ow || pad != src->d.output_padding)
+    if ((c + 3) / 4 != (src->oc + 3) / 4 || h != src->oh || w != src->ow || pad != src->d.output_padding)
         fail(FYN_ERR_INVALID,
              "Inputs/outputs do not match (I/O) for layers %s and %s: producer %dx%dx%d pad %d, consumer port %d wants "
              "%dx%dx%d pad %d",
@@ -378,11 +381,19 @@ void Net::set_input(int layer_no, int port, const float* data, int order) {
     FYN_HIP(hipStreamSynchronize(stream));
 }
 
+// What a layer hands out: its output tensor; a layer that only passes its input on (download) may name up to three
+// channels more or fewer than were produced, inside the same group of four (the extra ones are zero).
+static TView result_view(Layer* l) {
+    TView v = l->tout().v;
+    if (!l->has_own_output()) v.c = std::min(l->oc, v.cp);
+    return v;
+}
+
 void Net::copy_result(int layer_no, float* chw, int include_padding) {
     if (!is_setup) fail(FYN_ERR_STATE, "copy_result() before setup()");
     FYN_HIP(hipSetDevice(device));
     Layer* l = layer(layer_no);
-    const TView& v = l->tout().v;
+    const TView v = result_view(l);
     const size_t n = include_padding ? (size_t)v.c * v.hp() * v.wp() : (size_t)v.c * v.h * v.w;
     float* st = staging(n);
     launch_tensor_to_chw(v, st, include_padding, stream);
@@ -413,7 +424,7 @@ void Net::get_output(int layer_no, float* data, int order) {
     if (!is_setup) fail(FYN_ERR_STATE, "get_output() before setup()");
     FYN_HIP(hipSetDevice(device));
     Layer* l = layer(layer_no);
-    const TView& v = l->tout().v;
+    const TView v = result_view(l);
     if (order == FYN_ORDER_CHANNELWISE) {
         copy_result(layer_no, data, 0);
     } else if (order == FYN_ORDER_GPU_SHALLOW) {
@@ -521,8 +532,9 @@ void Net::async_begin(int in_layer, int in_port, int in_order, int out_layer, in
         if (async_in_->producer != -1) fail(FYN_ERR_INVALID, "input port %d of layer %s is fed by layer %d", in_port, li->d.name, async_in_->producer);
     }
     async_out_ = &layer(out_layer)->tout();
+    async_out_view_ = result_view(layer(out_layer));
     const TView& vi = async_in_->v;
-    const TView& vo = async_out_->v;
+    const TView& vo = async_out_view_;
     if (in_order != FYN_ORDER_CHANNELWISE && in_order != FYN_ORDER_GPU_SHALLOW) fail(FYN_ERR_UNSUPPORTED, "input order %d not supported for upload", in_order);
     if (out_order == FYN_ORDER_GPU_SHALLOW) {
         if (vo.c > 4) fail(FYN_ERR_UNSUPPORTED, "GPU_SHALLOW download holds at most 4 channels per texel (layer has %d)", vo.c);
@@ -569,7 +581,7 @@ void Net::async_submit(const float* in, float* out, uint64_t* ticket) {
     if (async_in_order_ == FYN_ORDER_CHANNELWISE) launch_chw_to_tensor(s.dev_in, async_in_->v, stream);
     else launch_hwc_to_tensor(s.dev_in, async_in_->v.c, async_in_->v, stream);
     forward(nullptr);
-    const TView& vo = async_out_->v;
+    const TView& vo = async_out_view_;
     if (async_out_order_ == FYN_ORDER_CHANNELWISE) launch_tensor_to_chw(vo, s.dev_out, 0, stream);
     else launch_tensor_to_hwc(vo, s.dev_out, vo.c == 3 ? 4 : vo.c, stream);
     FYN_HIP(hipGetLastError());

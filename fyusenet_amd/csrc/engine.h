@@ -134,6 +134,7 @@ class Net {
     hipStream_t up_stream_ = nullptr, down_stream_ = nullptr;
     const Tensor* async_in_ = nullptr;
     const Tensor* async_out_ = nullptr;
+    TView async_out_view_{};   // what the output layer hands out (a download layer may name other channel counts)
     int async_in_order_ = 0, async_out_order_ = 0;
     size_t async_in_floats_ = 0, async_out_floats_ = 0;
     uint64_t async_seq_ = 0;

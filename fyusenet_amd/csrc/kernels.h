@@ -119,7 +119,11 @@ struct ConvDirectParams {
     const float* bias;
     int k, dil, stride;
     int in_y0, in_x0;    // stored coord of tap (0,0) for output (0,0)
-    int clamp;           // 1: clamp to the net area edge (shallow unpadded rule)
+    int clamp;           // 1: coordinates clamp to the stored tensor's edge (the sampler's rule for shallow layers: an
+                         //    unpadded input repeats its edge, a padded one reads its zero halo)
+    int frac_shift;      // 0: ordinary taps.  s > 0 (fractional-step convolution, sourceStep = 2^(1-s)): tap t of output
+                         //    x reads stored column pad + floor((2*(stride*x + t) + 1) / 2^s), t = kx + tap_x0 (ky + tap_y0)
+    int tap_x0, tap_y0;
     int res_relu, res_scale;
     Act act;
 };

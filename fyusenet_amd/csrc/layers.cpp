@@ -678,6 +678,28 @@ class ConvLayer : public Layer {
         oh = d.height / stride;  // gpu/convlayerbase.cpp:47-48
         ow = d.width / stride;
         const int r = (k - 1) / 2;
+        if (d.type == FYN_LAYER_FRACCONVOLUTION2D) {
+            // gpu/gpulayerfactory.cpp:447-456, gpu/vanilla/fractionalconvlayerNxN_vanilla.cpp:43-50
+            if (d.flags & FYN_FLAG_DEEP) fail(FYN_ERR_UNSUPPORTED, "Fractional convolution is not supported for deep layers");
+            if (k == 1) fail(FYN_ERR_UNSUPPORTED, "Kernel size 1 not supported for fractional convolution (%s)", d.name);
+            if (k > 9) fail(FYN_ERR_UNSUPPORTED, "Unsupported fractional convolution kernel size %d (%s)", k, d.name);   // shaders exist for 3, 5, 7, 9
+            if (dil > 1 || d.dilation[1] > 1) fail(FYN_ERR_UNSUPPORTED, "Dilations not supported for fractional convolution");
+            const float step = d.source_step > 0.f ? d.source_step : 1.f;
+            int inv = 0;
+            for (int s = 1; s <= 16; s *= 2)
+                if (step * (float)s == 1.f) inv = s;
+            // other steps put sample positions on texel boundaries, where the nearest filter's choice is the
+            // GL implementation's; sizes must divide so that the positions stay dyadic
+            if (!inv) fail(FYN_ERR_UNSUPPORTED, "fractional convolution (%s): sourceStep %g is not 1, 1/2, 1/4, 1/8 or 1/16", d.name, step);
+            if ((d.width * inv) % stride || (d.height * inv) % stride)
+                fail(FYN_ERR_UNSUPPORTED, "fractional convolution (%s): %dx%d is not a multiple of sourceStep*downsample", d.name, d.width, d.height);
+            frac_shift = 1;
+            while ((1 << (frac_shift - 1)) < inv) frac_shift++;
+            oh = d.height * inv / stride;
+            ow = d.width * inv / stride;
+            clamp = direct = true;
+            return;
+        }
         // shallow, unpadded input: the sampler clamps to the edge (gpu/gpulayerbase.h:80-90)
         clamp = !(d.flags & FYN_FLAG_DEEP) && d.input_padding < r * dil && k > 1;
         direct = clamp || getenv("FYNHIP_FORCE_DIRECT_CONV") != nullptr;
@@ -702,10 +724,17 @@ class ConvLayer : public Layer {
         const int res_scale = ((d.flags & FYN_FLAG_BATCHNORM_ON_RESIDUAL) && (d.flags & FYN_FLAG_POST_BATCHNORM)) ? 1 : 0;
         if (direct) {
             dp.in = in_v; dp.out = out_v;
+            dp.in.c = std::min(d.in_channels, in_v.cp);   // the weights' channel count (the producer may name up to 3 more or fewer)
             dp.res = res_v ? *res_v : TView{};
             dp.k = k; dp.dil = dil; dp.stride = stride;
             dp.in_y0 = dp.in_x0 = in_v.pad - r * dil;
             dp.clamp = clamp ? 1 : 0;
+            dp.frac_shift = frac_shift;
+            // taps sit at kx - r steps, except under the 3x3 kernel, whose shader samples at -2, -1 and 0 steps
+            // (shaders/vanilla/fraconv3x3.frag:14-19 against fraconv5x5.frag:14-22); rows are offset through the
+            // proxy polygons, symmetrically for every size (gpu/vanilla/convlayerbase_vanilla.cpp:365)
+            dp.tap_x0 = (k == 3) ? -2 : -r;
+            dp.tap_y0 = -r;
             dp.res_relu = res_relu; dp.res_scale = res_scale;
             dp.act = act();
             padded = out_v.cp;
@@ -808,11 +837,13 @@ class ConvLayer : public Layer {
         if (wide) launch_shift_reduce(sr, s);
     }
     std::string info() const override {
+        if (frac_shift) return "conv_direct(fractional step 1/" + std::to_string(1 << (frac_shift - 1)) + ")";
         if (direct) return clamp ? "conv_direct(edge-clamp)" : "conv_direct";
         return wide ? "wide-kernel(kx folded into cout)+shift_reduce " + mfma_info(launch) : mfma_info(launch);
     }
 
     int k, dil, stride;
+    int frac_shift = 0;   // fractional-step convolution: log2(1/sourceStep) + 1
     bool clamp = false, direct = false, wide = false, have_weights = false;
     int padded = 0;
     std::vector<float> block;
@@ -1452,7 +1483,9 @@ Layer* create_layer(Net* net, const fyn_layer_desc& d) {
         case FYN_LAYER_NONMAX2D:
         case FYN_LAYER_BLUR2D: l = new FuncLayer(net, d); break;
         case FYN_LAYER_FRACCONVOLUTION2D:
-            fail(FYN_ERR_UNSUPPORTED, "fractional convolution (%s) is not supported: its sampling positions fall on texel boundaries of the nearest-neighbour filter", d.name);
+            if (d.group_size > 1) fail(FYN_ERR_UNSUPPORTED, "grouped convolution (group size %d) not supported (%s)", d.group_size, d.name);
+            l = new ConvLayer(net, d);
+            break;
         case FYN_LAYER_CUSTOM: fail(FYN_ERR_INVALID, "layer %s: custom layers are added with fyn_net_add_custom_layer", d.name);
         case FYN_LAYER_UPLOAD: l = new UploadLayer(net, d); break;
         case FYN_LAYER_DOWNLOAD: l = new DownloadLayer(net, d); break;

@@ -843,10 +843,14 @@ __global__ __launch_bounds__(256) void conv_direct_kernel(const ConvDirectParams
     for (int ky = 0; ky < p.k; ky++) {
         for (int kx = 0; kx < p.k; kx++) {
             int sy = y * p.stride + p.in_y0 + ky * p.dil, sx = x * p.stride + p.in_x0 + kx * p.dil;
+            if (p.frac_shift) {   // (an arithmetic shift: floor for negative numerators too)
+                sy = p.in.pad + ((2 * (y * p.stride + ky + p.tap_y0) + 1) >> p.frac_shift);
+                sx = p.in.pad + ((2 * (x * p.stride + kx + p.tap_x0) + 1) >> p.frac_shift);
+            }
             bool ok = true;
             if (p.clamp) {
-                sy = min(max(sy, p.in.pad), p.in.pad + p.in.h - 1);
-                sx = min(max(sx, p.in.pad), p.in.pad + p.in.w - 1);
+                sy = min(max(sy, 0), ihp - 1);
+                sx = min(max(sx, 0), iwp - 1);
             } else {
                 ok = (unsigned)sy < (unsigned)ihp && (unsigned)sx < (unsigned)iwp;
             }

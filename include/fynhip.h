@@ -46,7 +46,7 @@ enum fyn_layer_type {
     FYN_LAYER_CAST = 4,
     FYN_LAYER_CONCAT = 5,
     FYN_LAYER_CONVOLUTION2D = 6,
-    FYN_LAYER_FRACCONVOLUTION2D = 7, /* known, always rejected with FYN_ERR_UNSUPPORTED */
+    FYN_LAYER_FRACCONVOLUTION2D = 7, /* shallow only, like the reference (gpu/gpulayerfactory.cpp:447-456) */
     FYN_LAYER_TRANSCONVOLUTION2D = 8,
     FYN_LAYER_AVGPOOL2D = 9,
     FYN_LAYER_MAXPOOL2D = 10,
@@ -140,6 +140,7 @@ typedef struct fyn_layer_desc {
     int32_t cast_target; /* CAST: CastTarget 0..7 (base/layerflags.h:121-130)  CastLayerBuilder::target()                       */
     int32_t window;      /* IMGEXTRACT: window size                        ImgExtractLayerBuilder (gpu/imgextractlayerbuilder.h) */
     int32_t blur_type;   /* BLUR2D: BlurKernelType 0 average, 1 Gaussian; size in `kernel`  (gpu/blurlayerbuilder.h)            */
+    float source_step;   /* FRACCONVOLUTION2D: step on the input per tap, 1/2, 1/4 ...; 0 reads as 1  ConvLayerBuilder::sourceStep() (gpu/convlayerbuilder.h:80) */
 } fyn_layer_desc;
 
 /* Thread-local text of the last failure (what the reference would have thrown). */

@@ -14,6 +14,9 @@
  * Pinning status (what independent evidence fixes each function; see tests/test_oracle_*.py):
  *   fyo_conv2d        reference known-answer patterns (convlayertests.cpp:165-182,242-261,
  *                     networktests.cpp:85-97) + torch.nn.functional.conv2d in fp64
+ *   fyo_fracconv      fyo_conv2d (pinned above) on a numpy.repeat up-sampled input, the exact identity of its
+ *                     sampling rule, + a float restatement of the proxy polygon's texture coordinates on
+ *                     tiny inputs (no reference test exists)
  *   fyo_dwconv        conv2d(groups=C) fp64 + brute force          (no reference test exists)
  *   fyo_transconv     conv_transpose2d(stride=2) fp64 + brute force (no reference test exists)
  *   fyo_gemm          reference pattern misctests.cpp:238-265 + torch linear fp64
@@ -129,6 +132,59 @@ int fyo_conv2d(const float* in, int cin, int hs, int ws, int pad_in, const float
                     for (int ky = 0; ky < k; ky++) {
                         for (int kx = 0; kx < k; kx++) {
                             float v = fyo_fetch(plane, hs, ws, yc + (ky - r) * dil, xc + (kx - r) * dil, border);
+                            v = fyo_activate(v, act, leak, lo, hi);
+                            acc += (double)v * (double)wts[(((size_t)o * k + ky) * k + kx) * cin + i];
+                        }
+                    }
+                }
+                size_t oidx = ((size_t)o * ho + yo) * wo + xo;
+                out[oidx] = fyo_epilogue(acc, block[o], flags, bn, cout, o, residual, oidx);
+            }
+        }
+    }
+    return 0;
+}
+
+/*
+ * Fractional-step ("up-sampling") convolution of the shallow path, FRACCONVOLUTION2D.
+ * gpu/vanilla/fractionalconvlayerNxN_vanilla.cpp:43-50: output size = int(size / (sourceStep * downsample));
+ * :91: the shader's horizontal tap distance is sourceStep texels.  The proxy polygons
+ * (gpu/vanilla/convlayerbase_vanilla.cpp:361-371) map the output's net area onto the input's, shift row
+ * pass `ky` by sourceStep*(ky - r) texels and both axes by -sourceStep*(downsample-1)/2; the texture is read
+ * with nearest filtering, so with sourceStep = 1/inv_step the stored texel of tap t at output x is
+ *      pad + floor((downsample*x + t + 1/2) / inv_step)
+ * (never on a texel boundary for an integer inv_step).  Vertical taps are t = ky - r.  Horizontal taps are
+ * t = kx - r for 5x5, 7x7 and 9x9 (shaders/vanilla/fraconv5x5.frag:14-22, fraconv9x9.frag:14-30) but
+ * t = kx - 2 for 3x3 (shaders/vanilla/fraconv3x3.frag:14-19 samples at -2, -1 and 0 steps): reproduced as is.
+ * Activation on fetch, bias / BN / residual epilogue and the weight block are those of fyo_conv2d.
+ * Sizes that sourceStep*downsample does not divide are refused (their sample positions are not dyadic).
+ *   in        [cin][hs][ws], hs = H + 2*pad_in;  out / residual [cout][H*inv_step/stride][W*inv_step/stride]
+ */
+int fyo_fracconv(const float* in, int cin, int hs, int ws, int pad_in, const float* block, int cout, int k,
+                 int stride, int inv_step, int act, float leak, float lo, float hi, unsigned flags,
+                 const float* residual, int border, float* out) {
+    if ((k & 1) == 0 || k < 3 || k > 9 || stride < 1 || inv_step < 1) return -1;
+    const int H = hs - 2 * pad_in, W = ws - 2 * pad_in;
+    if ((H * inv_step) % stride || (W * inv_step) % stride) return -2;
+    const int ho = H * inv_step / stride, wo = W * inv_step / stride, r = (k - 1) / 2;
+    const int tx0 = (k == 3) ? -2 : -r;
+    const float* wts = block + cout;
+    const float* bn = wts + (size_t)cout * k * k * cin;
+#pragma omp parallel for schedule(static)
+    for (int o = 0; o < cout; o++) {
+        for (int yo = 0; yo < ho; yo++) {
+            for (int xo = 0; xo < wo; xo++) {
+                double acc = 0.0;
+                for (int i = 0; i < cin; i++) {
+                    const float* plane = in + (size_t)i * hs * ws;
+                    for (int ky = 0; ky < k; ky++) {
+                        /* floor((2n + 1) / (2*inv_step)) for any sign of n */
+                        const int ny = 2 * (stride * yo + ky - r) + 1;
+                        const int sy = pad_in + (ny >= 0 ? ny / (2 * inv_step) : -((-ny + 2 * inv_step - 1) / (2 * inv_step)));
+                        for (int kx = 0; kx < k; kx++) {
+                            const int nx = 2 * (stride * xo + kx + tx0) + 1;
+                            const int sx = pad_in + (nx >= 0 ? nx / (2 * inv_step) : -((-nx + 2 * inv_step - 1) / (2 * inv_step)));
+                            float v = fyo_fetch(plane, hs, ws, sy, sx, border);
                             v = fyo_activate(v, act, leak, lo, hi);
                             acc += (double)v * (double)wts[(((size_t)o * k + ky) * k + kx) * cin + i];
                         }

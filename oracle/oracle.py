@@ -31,7 +31,7 @@ def lib():
         if not os.path.exists(LIB_PATH):
             build()
         _lib = ctypes.CDLL(LIB_PATH)
-        for name in ("fyo_conv2d", "fyo_dwconv", "fyo_transconv", "fyo_gemm", "fyo_maxpool", "fyo_avgpool",
+        for name in ("fyo_conv2d", "fyo_fracconv", "fyo_dwconv", "fyo_transconv", "fyo_gemm", "fyo_maxpool", "fyo_avgpool",
                      "fyo_global_pool", "fyo_batchnorm", "fyo_addsub", "fyo_concat", "fyo_argmax",
                      "fyo_chw_to_deep", "fyo_deep_to_chw", "fyo_shallow_to_chw", "fyo_chw_to_shallow",
                      "fyo_unary", "fyo_scale", "fyo_transpose", "fyo_imgextract", "fyo_nonmax", "fyo_blur",
@@ -79,6 +79,22 @@ def conv2d(x_stored, pad_in, block, cout, k, dil=1, stride=1, act=None, flags=0,
                           ctypes.c_float(a[2]), ctypes.c_float(a[3]), ctypes.c_uint(flags), rp, border,
                           out.ctypes.data_as(_F))
     assert rc == 0
+    return out
+
+
+def fracconv(x_stored, pad_in, block, cout, k, stride=1, inv_step=2, act=None, flags=0, residual=None, border=1):
+    """x_stored [cin][H+2pad][W+2pad]; returns [cout][H*inv_step/stride][W*inv_step/stride]."""
+    x, xp = _f(x_stored)
+    b, bp = _f(block)
+    cin, hs, ws = x.shape
+    ho, wo = (hs - 2 * pad_in) * inv_step // stride, (ws - 2 * pad_in) * inv_step // stride
+    out = np.empty((cout, ho, wo), dtype=np.float32)
+    r, rp = (None, None) if residual is None else _f(residual)
+    a = _act(act)
+    rc = lib().fyo_fracconv(xp, cin, hs, ws, pad_in, bp, cout, k, stride, inv_step, a[0], ctypes.c_float(a[1]),
+                            ctypes.c_float(a[2]), ctypes.c_float(a[3]), ctypes.c_uint(flags), rp, border,
+                            out.ctypes.data_as(_F))
+    assert rc == 0, rc
     return out
 
 
@@ -341,7 +357,7 @@ def _round_block_fp16(layer_type, b, block):
     """fp16 storage rounds the weights (not bias / BN terms, which the engine keeps in fp32)."""
     block = np.array(block, dtype=np.float32, copy=True)
     cout = b.outputChannels_
-    if layer_type in (6, 8, 31):  # conv, transconv, gemm
+    if layer_type in (6, 7, 8, 31):  # conv, fractional conv, transconv, gemm
         dw = layer_type == 6 and getattr(b, "groupSize_", 1) not in (0, 1) and b.groupSize_ == b.inputChannels_
         if dw:
             return block  # depthwise weights stay fp32 in the engine
@@ -373,6 +389,11 @@ def run_layer(b, w, ins, f16=False):
         border = 1 if (not (flags & 16) and b.inputPadding_ < r and b.kernel_ > 1) else 0
         return conv2d(get(0, b.inputPadding_), b.inputPadding_, wb, b.outputChannels_, b.kernel_, b.dilation_[0],
                       b.downsample_[0], act, flags, res, border)
+    if t == 7:
+        res = get(1, 0) if flags & RESIDUAL_INPUT else None
+        wb = _round_block_fp16(t, b, w) if f16 else w
+        inv = int(round(1.0 / b.sourceStep_))
+        return fracconv(get(0, b.inputPadding_), b.inputPadding_, wb, b.outputChannels_, b.kernel_, b.downsample_[0], inv, act, flags, res)
     if t == 8:
         wb = _round_block_fp16(t, b, w) if f16 else w
         return transconv(get(0, b.inputPadding_), b.inputPadding_, wb, b.outputChannels_, b.kernel_, b.transconvCrop_, act, flags)
@@ -435,6 +456,16 @@ def num_ports(b):
     return 2 if int(b.getFlags()) & RESIDUAL_INPUT else 1
 
 
+def port_channels(b, port):
+    """Channels a layer expects on an input port, None when the builder does not say."""
+    if int(b.type_) == 5:                                  # concatenation: per-input channel counts
+        ins = getattr(b, "inputs_", None)
+        return ins[port][0] if ins and port < len(ins) else None
+    if port == 0:
+        return b.inputChannels_
+    return b.outputChannels_ if port == 1 else None       # residual input
+
+
 def run_network(desc, inputs, fp16_storage=None, forced=None):
     """Executes a network description on the CPU.
 
@@ -456,7 +487,13 @@ def run_network(desc, inputs, fp16_storage=None, forced=None):
         for port in range(num_ports(b)):
             if (no, port) in feeds:
                 src = feeds[(no, port)]
-                ins.append(forced[src] if forced is not None else outs[src])
+                x = forced[src] if forced is not None else outs[src]
+                want = port_channels(b, port)
+                if want is not None and want != x.shape[0] and (want + 3) // 4 == (x.shape[0] + 3) // 4:
+                    # the consumer names another channel count inside the same group of four (buffers are matched
+                    # texture by texture, base/buffermanager.cpp:476): missing channels read as zero
+                    x = np.concatenate([x, np.zeros((want - x.shape[0],) + x.shape[1:], x.dtype)]) if want > x.shape[0] else x[:want]
+                ins.append(x)
             else:
                 ins.append(rnd(inputs[(no, port)]))
         outs[no] = rnd(run_layer(b, w, ins, f16))

@@ -198,3 +198,68 @@ def test_transconv_parity(k, crop, cin, cout, h, w, storage):
     print("  ", info, "rel_l2=%.3e" % err, flush=True)
     assert got.shape == ref.shape == (cout, 2 * h + k - 2 - crop, 2 * w + k - 2 - crop)
     assert err <= TOL[storage]
+
+
+FRAC_CASES = [
+    # k, cin, cout, h, w, step, stride, pad_in, act, kwargs
+    (3, 40, 20, 12, 16, 0.5, 2, 0, A.NONE, {}),                   # deconv1 of the reference's style nets (stylenet3x3.cpp:163)
+    (3, 20, 12, 12, 16, 0.25, 2, 0, A.RELU, {}),                  # deconv2 (:167): twice the size
+    (3, 12, 3, 24, 32, 0.5, 1, 0, A.RELU, {}),                    # deconv3 (:171)
+    (9, 12, 3, 10, 14, 0.5, 1, 0, A.RELU, {}),                    # deconv3 of stylenet9x9.cpp:201
+    (5, 7, 9, 6, 5, 0.5, 1, 2, A.LEAKY_RELU, {"bn": True, "leak": 0.2}),
+    (7, 4, 8, 5, 9, 0.25, 1, 1, A.CLIP, {"clip": (-0.5, 0.5)}),
+    (5, 16, 33, 8, 8, 0.5, 2, 1, A.RELU, {"bn": True, "residual": (A.RELU, True), "pad_out": 2}),
+    (3, 5, 4, 3, 2, 0.125, 2, 1, A.NONE, {"residual": (A.NONE, False)}),
+    (9, 3, 2, 4, 4, 1.0, 1, 4, A.NONE, {}),                       # step 1: the ordinary convolution
+    (3, 1, 1, 1, 1, 0.5, 1, 0, A.NONE, {}),
+]
+
+
+@pytest.mark.parametrize("storage", [fa.STORAGE_F32, fa.STORAGE_F16], ids=["f32", "f16"])
+@pytest.mark.parametrize("case", FRAC_CASES, ids=lambda c: "k%d_%dx%dx%d_to%d_step%g_s%d_p%d" % (c[0], c[1], c[3], c[4], c[2], c[5], c[6], c[7]))
+def test_fractional_convolution_parity(case, storage):
+    k, cin, cout, h, w, step, stride, pad_in, act, kw = case
+    b = fa.ConvLayerBuilder(k, "fracconv").type(fa.LayerType.FRACCONVOLUTION2D).number(1).shape(cout, h, w, cin)
+    b.downsample(stride).sourceStep(step).prefixAct(act).inputPadding(pad_in).outputPadding(kw.get("pad_out", 0))
+    bn = kw.get("bn", False)
+    if bn:
+        b.postfixNorm(fa.NormType.BATCHNORM)
+    if "residual" in kw:
+        b.residual(*kw["residual"]).residualPadding(kw.get("pad_out", 0))
+    if "leak" in kw:
+        b.leakyReLU(kw["leak"])
+    if "clip" in kw:
+        b.clip(*kw["clip"])
+    inv = int(round(1 / step))
+    oh, ow = h * inv // stride, w * inv // stride
+    wts = conv_block(700 + k, cout, k, cin, bn=bn)
+    inputs = [prng.uniform(17 * k + cin, (cin, h, w), -1, 1)]
+    if "residual" in kw:
+        inputs.append(prng.uniform(29, (cout, oh, ow), -1, 1))
+    print("case", case, "storage", storage, flush=True)
+    got, info = run_single(b, storage, inputs, wts)
+    ref = oracle_single(b, storage, inputs, wts)
+    err = rel_l2(got, ref)
+    print("  ", info, "rel_l2=%.3e" % err, flush=True)
+    assert "fractional step 1/%d" % inv in info
+    assert got.shape == ref.shape == (cout, oh, ow)
+    assert err <= TOL[storage], info
+
+
+def test_fractional_convolution_rejections():
+    """gpu/gpulayerfactory.cpp:447-456 and gpu/vanilla/fractionalconvlayerNxN_vanilla.cpp:44: deep tensors, 1x1
+    kernels and dilation are refused; so are steps and sizes whose sample positions would not be dyadic."""
+    def builder(k=3, step=0.5, h=8, w=8, stride=1):
+        return fa.ConvLayerBuilder(k, "fracconv").type(fa.LayerType.FRACCONVOLUTION2D).number(1).shape(4, h, w, 4).sourceStep(step).downsample(stride)
+
+    x = np.zeros((4, 8, 8), np.float32)
+    with pytest.raises(fa.FynException, match="not supported for deep layers"):
+        run_single(builder().deep(), fa.STORAGE_F32, [x], conv_block(1, 4, 3, 4))
+    with pytest.raises(fa.FynException, match="Kernel size 1 not supported"):
+        run_single(builder(k=1), fa.STORAGE_F32, [x], conv_block(1, 4, 1, 4))
+    with pytest.raises(fa.FynException, match="Dilations not supported"):
+        run_single(builder().dilation(2), fa.STORAGE_F32, [x], conv_block(1, 4, 3, 4))
+    with pytest.raises(fa.FynException, match="sourceStep"):
+        run_single(builder(step=0.3), fa.STORAGE_F32, [x], conv_block(1, 4, 3, 4))
+    with pytest.raises(fa.FynException, match="not a multiple"):
+        run_single(builder(step=1.0, h=7, w=7, stride=2), fa.STORAGE_F32, [np.zeros((4, 7, 7), np.float32)], conv_block(1, 4, 3, 4))

@@ -188,12 +188,6 @@ def test_rgb2bgr_nonmax_blur_parity(c, h, w, pad, storage):
         run_single(fa.BlurLayerBuilder("x").number(1).shape(c, h, w, c).kernel(4), storage, [x])
 
 
-def test_fractional_convolution_is_rejected():
-    b = fa.ConvLayerBuilder(3, "frac").type(T.FRACCONVOLUTION2D).number(1).shape(8, 16, 16, 8).sourceStep(0.5)
-    with pytest.raises(fa.FynException, match="fractional convolution"):
-        run_single(b, fa.STORAGE_F32, [np.zeros((8, 16, 16), np.float32)])
-
-
 @STORAGES
 def test_style_net_tail_with_sigmoid(storage):
     """Transposed convolution -> sigmoid -> download, the tail of the reference's style-transfer samples

@@ -242,6 +242,23 @@ def test_reference_resnet50_sample_graph():
     bad.cleanup()
 
 
+@pytest.mark.parametrize("storage", [fa.STORAGE_F32, fa.STORAGE_F16], ids=["f32", "f16"])
+@pytest.mark.parametrize("kernel,width,height", [(3, 64, 48), (9, 40, 56)])
+def test_reference_style_net_sample_graphs(kernel, width, height, storage):
+    """The reference's own style-transfer graphs (shallow unpadded convolutions, residual blocks, three fractional-step
+    convolutions, sigmoid, a download layer that names 4 channels of the 3-channel result) with a synthetic weight
+    stream of the reference's size and layout, layer by layer."""
+    from fyusenet_amd import samples
+    net = samples.StyleNetSample(kernel, width, height, storage)
+    assert net.total_weight_bytes() == 4 * (77235 if kernel == 3 else 169059)
+    ref, got = run_and_compare(net, storage)
+    out = got[net.SIGMOID]
+    assert out.shape == (3, height, width) and np.all(out > 0) and np.all(out < 1) and float(np.std(out)) > 0
+    rgba = got[net.DOWNLOAD]
+    assert rgba.shape == (4, height, width) and np.array_equal(rgba[:3], out) and not np.any(rgba[3])
+    net.cleanup()
+
+
 @pytest.mark.gpu
 @pytest.mark.parametrize("depth", [1, 2, 3])
 def test_frame_pipeline_matches_synchronous_path(depth):

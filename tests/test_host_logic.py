@@ -25,7 +25,7 @@ def test_library_exports_every_declared_symbol():
 def test_desc_struct_layout_matches_header():
     # 4-byte fields only, no padding: size must equal the sum of the members
     d = capi.LayerDesc()
-    assert ctypes.sizeof(d) == 4 * 3 + 64 + 4 * (1 + 4 + 3 + 2 + 2 + 3 + 1 + 2 + 1 + 2 + 1 + 1) + 12 * 8 + 4 + 4 * 6
+    assert ctypes.sizeof(d) == 4 * 3 + 64 + 4 * (1 + 4 + 3 + 2 + 2 + 3 + 1 + 2 + 1 + 2 + 1 + 1) + 12 * 8 + 4 + 4 * 7
     # member names and order as the header declares them
     import re
     text = open(os.path.join(ROOT, "include", "fynhip.h")).read()
@@ -128,3 +128,34 @@ def test_resnet50_sample_weight_layout_matches_the_reference_file_layout():
         s, d = spec[src], spec[dst]
         if port == 0:
             assert s.outputChannels_ == d.inputChannels_, (src, dst)
+
+
+def test_style_net_sample_weight_offsets_match_the_reference_tables():
+    """Float offsets derived from the layer descriptions against the tables the reference hard-codes
+    (samples/samplenetworks/stylenet3x3.cpp:41-50, stylenet9x9.cpp:41-56) and its stream sizes (stylenet3x3.h:53,
+    stylenet9x9.h:59); none of this needs the library."""
+    from fyusenet_amd import samples
+
+    class _Dry(samples.StyleNetSample):
+        def __init__(self, kernel):   # graph description only, no engine handle
+            self.kernel, self.width, self.height, self.blocks = kernel, 64, 48, 2 if kernel == 3 else 5
+            self.DECONV1 = self.FIRST_RES + 2 * self.blocks
+            self.DECONV2, self.DECONV3, self.SIGMOID, self.DOWNLOAD = (self.DECONV1 + i for i in (1, 2, 3, 4))
+            self._weights, self._specs, self._edges, self._file_order = None, [], [], []
+            self._define()
+
+        def __del__(self):
+            pass
+
+    n3 = _Dry(3)
+    # enum of stylenet3x3.h:39-51: CONV1 1, CONV2 2, CONV3 3, RES1_1..RES2_2 4..7, DECONV1..3 8..10, SIGMOID 11, DOWNLOAD 12
+    assert n3.weight_offsets() == {1: 0, 2: 336, 3: 2516, 4: 19475, 5: 33915, 6: 48355, 7: 62795, 8: 9756, 9: 16976, 10: 19148}
+    assert n3.total_weight_bytes() == 4 * samples.STYLENET3X3_WEIGHT_FLOATS == 4 * 77235
+    assert (n3.SIGMOID, n3.DOWNLOAD) == (11, 12) and len(n3._edges) == 14
+    n9 = _Dry(9)
+    assert n9.weight_offsets() == {1: 0, 2: 2928, 3: 5108, 4: 24659, 5: 39099, 6: 53539, 7: 67979, 8: 82419, 9: 96859, 10: 111299,
+                                   11: 125739, 12: 140179, 13: 154619, 14: 12348, 15: 19568, 16: 21740}
+    assert n9.total_weight_bytes() == 4 * samples.STYLENET9X9_WEIGHT_FLOATS == 4 * 169059
+    assert (n9.SIGMOID, n9.DOWNLOAD) == (17, 18) and len(n9._edges) == 23
+    spec = {no: b for no, b, _ in n9._specs}
+    assert spec[n9.DECONV2].sourceStep_ == 0.25 and spec[n9.DECONV2].downsample_[0] == 2 and spec[n9.DECONV3].kernel_ == 9

@@ -218,3 +218,75 @@ def test_scale_factor_one_is_a_copy_with_activation():
     x = prng.normal(75, (5, 6, 7))
     assert np.array_equal(O.scale(O.pad_chw(x, 2), 2, (1, 1), (1, 1), False, True), x)
     assert np.array_equal(O.scale(x, 0, (1, 1), (1, 1), True, False, (O.ACT_CLIP, 0.0, -0.5, 0.5)), np.clip(x, -0.5, 0.5))
+
+
+# ---- fractional-step convolution ---------------------------------------------------------------
+def _conv_block(seed, cout, k, cin, bn=False):
+    parts = [prng.normal(seed, (cout,), 0, 0.3), prng.normal(seed + 1, (cout, k, k, cin), 0, 0.5).ravel()]
+    if bn:
+        parts += [prng.uniform(seed + 2, (cout,), 0.5, 1.5), prng.normal(seed + 3, (cout,), 0, 0.2)]
+    return np.concatenate(parts).astype(np.float32)
+
+
+@pytest.mark.parametrize("border", [0, 1])
+@pytest.mark.parametrize("k,inv,stride,pad", [(5, 2, 1, 2), (9, 2, 1, 3), (7, 4, 2, 2), (5, 2, 2, 1), (9, 4, 1, 2), (5, 1, 1, 2), (7, 2, 1, 0),
+                                              (5, 4, 2, 0), (3, 2, 1, 1), (3, 2, 2, 1), (3, 4, 2, 1), (3, 2, 1, 0), (3, 4, 2, 0)])
+def test_fracconv_is_a_convolution_of_the_repeated_input(k, inv, stride, pad, border):
+    """Sampling at floor((stride*x + t + 1/2) / inv) reads, from the input whose every stored pixel is repeated
+    inv x inv times (numpy.repeat), the pixel stride*x + t: the layer equals the ordinary strided convolution (pinned
+    elsewhere against torch and the reference's patterns) of that image.  The 3x3 shader's taps sit one step to the
+    left (fraconv3x3.frag:14-19): there the comparison image is shifted right by one column."""
+    cin, cout, h, w = 3, 4, 6, 8
+    x = prng.uniform(71 + k, (cin, h, w), -1, 1)
+    xs = np.pad(x, ((0, 0), (pad, pad), (pad, pad)))
+    blk = _conv_block(900 + k, cout, k, cin, bn=True)
+    res = prng.uniform(5, (cout, h * inv // stride, w * inv // stride), -1, 1)
+    flags = O.POST_BATCHNORM | O.RESIDUAL_INPUT | O.RELU_ON_RESIDUAL
+    got = O.fracconv(xs, pad, blk, cout, k, stride, inv, RELU, flags, res, border)
+    up = np.repeat(np.repeat(xs, inv, axis=1), inv, axis=2)
+    if k == 3:
+        first = up[:, :, :1] if border else np.zeros_like(up[:, :, :1])     # what lies left of the stored image
+        up = np.concatenate([first, up[:, :, :-1]], axis=2)
+    want = O.conv2d(up, pad * inv, blk, cout, k, 1, stride, RELU, flags, res, border)
+    assert got.shape == want.shape == (cout, h * inv // stride, w * inv // stride)
+    if k == 3:      # the shifted comparison image has lost its last column, which the last output column reads
+        got, want = got[:, :, :-1], want[:, :, :-1]
+    assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("k,step,stride,pad", [(3, 0.5, 1, 0), (3, 0.5, 2, 0), (3, 0.25, 2, 0), (5, 0.5, 1, 1), (9, 0.5, 1, 0), (7, 0.25, 2, 2)])
+def test_fracconv_against_the_proxy_polygon_arithmetic(k, step, stride, pad):
+    """Brute force from the geometry the reference renders with (gpu/vanilla/convlayerbase_vanilla.cpp:361-371,
+    fractionalconvlayerNxN_vanilla.cpp:47-48,91): normalised texture coordinates of the polygon of row pass ky,
+    interpolated at the fragment centre, the shader's horizontal offsets in units of texStep, nearest filtering
+    (floor of coordinate x texture size) with clamping to the texture's edge.  Floats as in the reference."""
+    f = np.float32
+    cin, cout, h, w = 2, 3, 4, 8
+    x = prng.uniform(31 + k, (cin, h, w), -1, 1)
+    xs = np.pad(x, ((0, 0), (pad, pad), (pad, pad)))
+    blk = _conv_block(700 + k, cout, k, cin)
+    bias, wts = blk[:cout], blk[cout:].reshape(cout, k, k, cin)
+    tw, th = int(f(w) / (f(step) * f(stride))), int(f(h) / (f(step) * f(stride)))
+    texstep = f(step) / f(w + 2 * pad)
+    hoffs = {3: [-2, -1, 0]}.get(k, list(range(-(k // 2), k // 2 + 1)))
+    want = np.zeros((cout, th, tw))
+    for ky in range(k):
+        thspan, tvspan = f(w) / f(w + 2 * pad), f(h) / f(h + 2 * pad)
+        tleft = f(pad) / f(w + 2 * pad)
+        ttop = (f(pad) + f(step) * f(ky - (k - 1) // 2)) / f(h + 2 * pad)
+        if stride > 1:
+            tleft = tleft - f(step) * f(0.5) * f(stride - 1) / f(w + 2 * pad)
+            ttop = ttop - f(step) * f(0.5) * f(stride - 1) / f(h + 2 * pad)
+        for yo in range(th):
+            v = float(ttop) + (yo + 0.5) / th * float(tvspan)
+            sy = min(max(int(np.floor(v * (h + 2 * pad))), 0), h + 2 * pad - 1)
+            for xo in range(tw):
+                u0 = float(tleft) + (xo + 0.5) / tw * float(thspan)
+                for kx in range(k):
+                    u = u0 + hoffs[kx] * float(texstep)
+                    sx = min(max(int(np.floor(u * (w + 2 * pad))), 0), w + 2 * pad - 1)
+                    want[:, yo, xo] += wts[:, ky, kx, :].astype(np.float64) @ xs[:, sy, sx].astype(np.float64)
+    want += bias[:, None, None]
+    got = O.fracconv(xs, pad, blk, cout, k, stride, int(round(1 / step)), None, 0, None, 1)
+    assert got.shape == want.shape
+    assert np.allclose(got, want, rtol=1e-6, atol=1e-6)
