@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the GPU layer stack on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload stylenet|resnet50|resnet50ref|conv1|mobilenet|stylenet9x9|copy|bw-<layer>]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload stylenet|resnet50|resnet50ref|stylenet3x3ref|stylenet9x9ref|conv1|mobilenet|stylenet9x9|copy|bw-<layer>]
 
 A step is one forward pass of the named network over one synthetic input frame that is already
 resident in HBM (uploaded before the timed region); weights are synthetic (random init).  Prints ONE
@@ -43,6 +43,10 @@ def make_net(workload):
     if workload == "resnet50ref":   # the reference's own sample graph (explicit batch-norm layers), .dat-compatible
         from fyusenet_amd import samples
         return samples.ResNet50Sample(fa.STORAGE_F32), "ResNet-50 (reference sample graph) 224x224 imgs/s", "imgs/s", "fp32 storage"
+    if workload in ("stylenet3x3ref", "stylenet9x9ref"):   # the reference's own sample graphs (shallow, fractional-step convolutions)
+        from fyusenet_amd import samples
+        k = 3 if workload == "stylenet3x3ref" else 9
+        return samples.StyleNetSample(k, 512, 624, fa.STORAGE_F32), "stylenet%dx%d (reference sample graph) 512x624 ms/frame" % (k, k), "ms/frame", "fp32 storage"
     if workload == "mobilenet":
         return networks.MobileNetV2(fa.STORAGE_F16), "MobileNetV2 224x224 imgs/s", "imgs/s", "fp16 storage"
     if workload == "conv1":

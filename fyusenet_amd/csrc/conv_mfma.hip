@@ -241,6 +241,7 @@ __device__ __forceinline__ void conv_mfma_body(const ConvMfmaParams& p, unsigned
     const int gy0 = pos_y0 * p.in_stride + p.in_y0;
     const int gx0 = pos_x0 * p.in_stride + p.in_x0;
     const float inv_hw = 1.0f / (float)p.halo_w;
+    const int vhp = p.in_hp << p.in_shift, vwp = p.in_wp << p.in_shift;   // frame that gy0/gx0 and the taps count in
     const TIn* in = reinterpret_cast<const TIn*>(p.in);
 
     // LDS holds two staging buffers (double buffering across channel chunks) when there is more
@@ -313,10 +314,14 @@ __device__ __forceinline__ void conv_mfma_body(const ConvMfmaParams& p, unsigned
             const int g = (G == 1) ? 0 : idx - pix * G;
             const int py = (int)(((float)pix + 0.5f) * inv_hw);
             const int px = pix - py * p.halo_w;
-            const int gy = gy0 + py, gx = gx0 + px;
+            int gy = gy0 + py, gx = gx0 + px;
             l_off[i] = py * p.row_pitch + px * p.pitch + g * 16;
             c_off[i] = g * CPI;
-            if ((unsigned)gy < (unsigned)p.in_hp && (unsigned)gx < (unsigned)p.in_wp) g_off[i] = (gy * p.in_wp + gx) * p.in_cp;
+            if (p.in_clamp) {
+                gy = min(max(gy, 0), vhp - 1);
+                gx = min(max(gx, 0), vwp - 1);
+            }
+            if ((unsigned)gy < (unsigned)vhp && (unsigned)gx < (unsigned)vwp) g_off[i] = ((gy >> p.in_shift) * p.in_wp + (gx >> p.in_shift)) * p.in_cp;
         }
     }
     RawItem<TIn, CPI> raw[NB];
@@ -359,11 +364,15 @@ __device__ __forceinline__ void conv_mfma_body(const ConvMfmaParams& p, unsigned
                     const int g = (G == 1) ? 0 : idx - pix * G;
                     const int py = (int)(((float)pix + 0.5f) * inv_hw);
                     const int px = pix - py * p.halo_w;
-                    const int gy = gy0 + py, gx = gx0 + px;
+                    int gy = gy0 + py, gx = gx0 + px;
                     const int c0 = chunk * KC + g * CPI;
                     lo2[i] = py * p.row_pitch + px * p.pitch + g * 16;
-                    if ((unsigned)gy < (unsigned)p.in_hp && (unsigned)gx < (unsigned)p.in_wp && c0 < p.in_cp)
-                        r2[i].load(in + (gy * p.in_wp + gx) * p.in_cp + c0);
+                    if (p.in_clamp) {
+                        gy = min(max(gy, 0), vhp - 1);
+                        gx = min(max(gx, 0), vwp - 1);
+                    }
+                    if ((unsigned)gy < (unsigned)vhp && (unsigned)gx < (unsigned)vwp && c0 < p.in_cp)
+                        r2[i].load(in + ((gy >> p.in_shift) * p.in_wp + (gx >> p.in_shift)) * p.in_cp + c0);
                 }
             }
 #pragma unroll

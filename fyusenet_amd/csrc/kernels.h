@@ -48,6 +48,10 @@ struct ConvMfmaParams {
     int in_hp, in_wp, in_cp;
     int in_y0, in_x0;    // stored coordinate sampled by tile-local (0,0) for output position (0,0)
     int in_stride;       // input step per output position
+    // Sampling rule of shallow layers.  in_clamp: coordinates outside the frame repeat its edge instead of reading 0.
+    // in_shift = s > 0 (fractional-step convolution): in_y0/in_x0 and the taps count in a virtual frame in which
+    // every stored pixel is repeated 2^s times in both directions; virtual coordinate v reads stored pixel v >> s.
+    int in_clamp, in_shift;
     // output positions computed by this launch
     int npos_y, npos_x;
     // output tensor addressing: stored y = out_off_y + pos_y * out_step

@@ -81,6 +81,8 @@ struct SubConv {
     int npos_y = 0, npos_x = 0;
     int out_step = 1, out_off_y = 0, out_off_x = 0;
     int res_off_y = 0, res_off_x = 0;
+    int clamp = 0;     // shallow sampling rule: repeat the frame's edge
+    int in_shift = 0;  // fractional-step convolution: coordinates count in the frame repeated 2^in_shift times
 };
 
 struct MfmaLaunch {
@@ -178,6 +180,7 @@ static MfmaLaunch plan_mfma(Net* net, const SubConv& sc, const TView& in, const 
     p.res = res ? res->ptr : nullptr;
     p.in_hp = in.hp(); p.in_wp = in.wp(); p.in_cp = in.cp;
     p.in_y0 = sc.in_y0; p.in_x0 = sc.in_x0; p.in_stride = sc.in_stride;
+    p.in_clamp = sc.clamp; p.in_shift = sc.in_shift;
     p.npos_y = sc.npos_y; p.npos_x = sc.npos_x;
     p.out_wp = out.wp(); p.out_cp = out.cp; p.out_step = sc.out_step;
     p.out_off_y = sc.out_off_y; p.out_off_x = sc.out_off_x;
@@ -421,8 +424,8 @@ static MfmaLaunch tune_mfma(Net* net, const SubConv& sc, const TView& in, const 
     // FYNHIP_TUNE_CACHE=<file>: measured choices are remembered per problem geometry, so that later
     // processes (e.g. under a profiler, where timing is distorted) pick the same kernels
     char key[160];
-    snprintf(key, sizeof(key), "%d%d:%dx%d:%dx%d:s%d:t%zu:%dx%d:o%d:r%d:cp%d", in.f16, out.f16, cin, cout, sc.npos_y, sc.npos_x,
-             sc.in_stride, sc.taps.size(), sc.span_y, sc.span_x, sc.out_step, res ? 1 : 0, in.cp);
+    snprintf(key, sizeof(key), "%d%d:%dx%d:%dx%d:s%d:t%zu:%dx%d:o%d:r%d:cp%d:e%d%d", in.f16, out.f16, cin, cout, sc.npos_y, sc.npos_x,
+             sc.in_stride, sc.taps.size(), sc.span_y, sc.span_x, sc.out_step, res ? 1 : 0, in.cp, sc.clamp, sc.in_shift);
     if (tune) {
         int ks = 1;
         const TileChoice* hit = tune_cache_lookup(key, cands, &ks);
@@ -697,12 +700,14 @@ class ConvLayer : public Layer {
             while ((1 << (frac_shift - 1)) < inv) frac_shift++;
             oh = d.height * inv / stride;
             ow = d.width * inv / stride;
-            clamp = direct = true;
+            clamp = true;
+            direct = getenv("FYNHIP_FORCE_DIRECT_CONV") != nullptr;
+            wide = !direct && oc <= 4 && oc * k <= 32 && stride == 1 && d.in_channels > 4 && getenv("FYNHIP_NO_WIDE_CONV") == nullptr;
             return;
         }
         // shallow, unpadded input: the sampler clamps to the edge (gpu/gpulayerbase.h:80-90)
         clamp = !(d.flags & FYN_FLAG_DEEP) && d.input_padding < r * dil && k > 1;
-        direct = clamp || getenv("FYNHIP_FORCE_DIRECT_CONV") != nullptr;
+        direct = getenv("FYNHIP_FORCE_DIRECT_CONV") != nullptr;   // (testing: the plain fp32 kernel instead of the MFMA path)
         // few output channels under a wide kernel: fold the kx taps into the GEMM's M dimension
         // (cout*K virtual channels, K taps) and reduce the K shifted partial sums in a second pass
         wide = !direct && oc <= 4 && oc * k <= 32 && k >= 3 && stride == 1 && dil == 1 && d.in_channels > 4 &&
@@ -746,9 +751,15 @@ class ConvLayer : public Layer {
             qv.ptr = net->dev_alloc(qv.bytes());
             SubConv sc;
             for (int ky = 0; ky < k; ky++) sc.taps.push_back(Tap{ky, 0, ky, 0});
+            sc.clamp = clamp ? 1 : 0;
             sc.span_y = k; sc.span_x = 1;
             sc.in_y0 = in_v.pad - r;
             sc.in_x0 = in_v.pad - r;
+            if (frac_shift) {   // (the frame of repeated pixels, as in the one-stage form below)
+                sc.in_shift = frac_shift - 1;
+                sc.in_y0 = (in_v.pad << sc.in_shift) - r;
+                sc.in_x0 = (in_v.pad << sc.in_shift) + ((k == 3) ? -2 : -r);
+            }
             sc.in_stride = 1;
             sc.npos_y = qv.h; sc.npos_x = qv.w;
             sc.out_step = 1;
@@ -769,6 +780,15 @@ class ConvLayer : public Layer {
                 for (int kx = 0; kx < k; kx++) sc.taps.push_back(Tap{ky * dil, kx * dil, ky, kx});
             sc.span_y = sc.span_x = (k - 1) * dil + 1;
             sc.in_y0 = sc.in_x0 = in_v.pad - r * dil;
+            sc.clamp = clamp ? 1 : 0;
+            if (frac_shift) {
+                // an ordinary strided convolution in the frame whose pixels are repeated 1/sourceStep times: taps one
+                // virtual pixel apart, rows centred, columns centred except under the 3x3 kernel, whose shader samples
+                // at -2, -1 and 0 steps (shaders/vanilla/fraconv3x3.frag:14-19 against fraconv5x5.frag:14-22)
+                sc.in_shift = frac_shift - 1;
+                sc.in_y0 = (in_v.pad << sc.in_shift) - r;
+                sc.in_x0 = (in_v.pad << sc.in_shift) + ((k == 3) ? -2 : -r);
+            }
             sc.in_stride = stride;
             sc.npos_y = oh; sc.npos_x = ow;
             sc.out_step = 1;
@@ -817,9 +837,11 @@ class ConvLayer : public Layer {
             for (int i = 0; i < oc * k; i++) ones[i] = 1.f;
             reupload(net, q_scale_dev, ones);
             reupload(net, q_bias_dev, zeros);
-            launch.p.acc_mul = 1.0f;         // the pre-scaling is undone in the second stage
-            launch.red.acc_mul = 1.0f;
-            sr.acc_mul = 1.0f / wmul;
+            // the pre-scaling is undone on the way into the intermediate tensor (a power of two: no rounding), so that
+            // fp16 storage holds the partial sums at their own magnitude
+            launch.p.acc_mul = 1.0f / wmul;
+            launch.red.acc_mul = 1.0f / wmul;
+            sr.acc_mul = 1.0f;
             pack_mfma_weights(net, launch, wv.data(), k, wmul, 1);
         } else {
             const float wmul = weight_prescale(w, (size_t)oc * k * k * d.in_channels);
@@ -837,9 +859,9 @@ class ConvLayer : public Layer {
         if (wide) launch_shift_reduce(sr, s);
     }
     std::string info() const override {
-        if (frac_shift) return "conv_direct(fractional step 1/" + std::to_string(1 << (frac_shift - 1)) + ")";
-        if (direct) return clamp ? "conv_direct(edge-clamp)" : "conv_direct";
-        return wide ? "wide-kernel(kx folded into cout)+shift_reduce " + mfma_info(launch) : mfma_info(launch);
+        const std::string mode = frac_shift ? "(fractional step 1/" + std::to_string(1 << (frac_shift - 1)) + ") " : (clamp ? "(edge-clamp) " : "");
+        if (direct) return "conv_direct" + mode;
+        return mode + (wide ? "wide-kernel(kx folded into cout)+shift_reduce " + mfma_info(launch) : mfma_info(launch));
     }
 
     int k, dil, stride;

@@ -824,8 +824,9 @@ void launch_gemv(const GemvParams& p, hipStream_t s) {
 }
 
 // ---------------------------------------------------------------------------------------------
-// direct convolution (fallback for what the MFMA path does not take: edge-clamped shallow layers,
-// unusual strides).  fp32 FMA, one thread = one output pixel x 4 output channels.
+// direct convolution: the engine's second, plain implementation of the convolution family's sampling rules (zero halo,
+// edge clamp of shallow layers, fractional steps), selected by FYNHIP_FORCE_DIRECT_CONV for cross-checks.
+// fp32 FMA, one thread = one output pixel x 4 output channels.
 // ---------------------------------------------------------------------------------------------
 template <typename T>
 __global__ __launch_bounds__(256) void conv_direct_kernel(const ConvDirectParams p) {

@@ -217,7 +217,7 @@ FRAC_CASES = [
 
 @pytest.mark.parametrize("storage", [fa.STORAGE_F32, fa.STORAGE_F16], ids=["f32", "f16"])
 @pytest.mark.parametrize("case", FRAC_CASES, ids=lambda c: "k%d_%dx%dx%d_to%d_step%g_s%d_p%d" % (c[0], c[1], c[3], c[4], c[2], c[5], c[6], c[7]))
-def test_fractional_convolution_parity(case, storage):
+def test_fractional_convolution_parity(case, storage, expect="conv_mfma"):
     k, cin, cout, h, w, step, stride, pad_in, act, kw = case
     b = fa.ConvLayerBuilder(k, "fracconv").type(fa.LayerType.FRACCONVOLUTION2D).number(1).shape(cout, h, w, cin)
     b.downsample(stride).sourceStep(step).prefixAct(act).inputPadding(pad_in).outputPadding(kw.get("pad_out", 0))
@@ -241,9 +241,17 @@ def test_fractional_convolution_parity(case, storage):
     ref = oracle_single(b, storage, inputs, wts)
     err = rel_l2(got, ref)
     print("  ", info, "rel_l2=%.3e" % err, flush=True)
-    assert "fractional step 1/%d" % inv in info
+    assert "fractional step 1/%d" % inv in info and expect in info
     assert got.shape == ref.shape == (cout, oh, ow)
     assert err <= TOL[storage], info
+
+
+@pytest.mark.parametrize("case", [FRAC_CASES[1], FRAC_CASES[3], FRAC_CASES[6]], ids=["deconv2", "deconv3_9x9", "k5_bn_residual"])
+def test_fractional_convolution_on_the_plain_kernel(case, monkeypatch):
+    """The fp32 FMA kernel (one thread per output pixel), kept as the engine's second implementation of the shallow
+    sampling rules, selected by the engine's test switch."""
+    monkeypatch.setenv("FYNHIP_FORCE_DIRECT_CONV", "1")
+    test_fractional_convolution_parity(case, fa.STORAGE_F32, expect="conv_direct")
 
 
 def test_fractional_convolution_rejections():
