@@ -220,3 +220,124 @@ def test_random_chain(seed, storage):
             assert e <= TOL[storage], (seed, lyr.name, e)
         assert np.array_equal(outs["reuse"], got[len(built)])       # buffer sharing does not change a bit
         net.cleanup()
+
+
+def _random_shallow_chain(seed):
+    """Shallow layers only: convolutions whose halo may be narrower than the kernel reaches (edge repeat or zero halo),
+    residual convolutions, fractional-step convolutions, batch norm and function layers."""
+    rng = np.random.RandomState(10_000 + seed)
+    c, h, w = int(rng.choice([3, 4, 12, 20])), int(rng.randint(4, 20)), int(rng.randint(4, 20))
+    shape0, specs = (c, h, w), []
+    for _ in range(int(rng.randint(3, 7))):
+        kinds = ["conv", "conv", "frac", "bn", "func"] + (["resconv"] if specs else [])
+        if h * w > 1600:
+            kinds = [k for k in kinds if k != "frac"] or ["conv"]
+        kind = str(rng.choice(kinds))
+        act = [A.NONE, A.RELU, A.CLIP, A.LEAKY_RELU][int(rng.randint(0, 4))]
+        s = {"kind": kind, "act": act, "cin": c, "h": h, "w": w}
+        if kind == "conv":
+            s["k"] = int(rng.choice([1, 3, 3, 5, 9]))
+            s["stride"] = 2 if (min(h, w) >= 4 and h % 2 == 0 and w % 2 == 0 and rng.randint(0, 3) == 0) else 1
+            s["cout"] = int(rng.choice([3, 12, 20, 40]))
+            s["bn"] = bool(rng.randint(0, 2))
+            s["pad_in"] = int(rng.randint(0, (s["k"] - 1) // 2 + 1))     # 0 .. r: anything short of r repeats or pads
+            c, h, w = s["cout"], h // s["stride"], w // s["stride"]
+        elif kind == "resconv":
+            s["bn"] = bool(rng.randint(0, 2))
+            s["res_relu"] = bool(rng.randint(0, 2))
+            s["pad_in"] = int(rng.randint(0, 2))
+        elif kind == "frac":
+            s["k"] = int(rng.choice([3, 3, 5, 7, 9]))
+            s["inv"] = int(rng.choice([2, 2, 4]))
+            s["stride"] = int(rng.choice([1, 2]))
+            s["cout"] = int(rng.choice([3, 12, 20]))
+            s["bn"] = bool(rng.randint(0, 2))
+            s["pad_in"] = int(rng.randint(0, 3))
+            c, h, w = s["cout"], h * s["inv"] // s["stride"], w * s["inv"] // s["stride"]
+        elif kind == "func":
+            s["fn"] = str(rng.choice(["sigmoid", "tanh", "arith", "relu"]))
+            s["pad_in"] = int(rng.randint(0, 2))
+        else:
+            s["pad_in"] = int(rng.randint(0, 2))
+        s["out"] = (c, h, w)
+        specs.append(s)
+    return shape0, specs, int(rng.randint(0, 2))
+
+
+def _shallow_builder(i, s, pad_out):
+    no, name = i + 1, "%s%d" % (s["kind"], i + 1)
+    cin, h, w, k = s["cin"], s["h"], s["w"], s["kind"]
+    weights = None
+    if k == "resconv":
+        b = fa.ConvLayerBuilder(3, name).type(T.CONVOLUTION2D).shape(cin, h, w, cin)
+        if s["bn"]:
+            b.postfixNorm(fa.NormType.BATCHNORM)
+        b.residual(A.RELU if s["res_relu"] else A.NONE, s["bn"]).residualPadding(s["pad_in"])
+        weights = conv_block(4000 + 17 * no, cin, 3, cin, bn=s["bn"])
+    elif k in ("conv", "frac"):
+        b = fa.ConvLayerBuilder(s["k"], name).type(T.CONVOLUTION2D if k == "conv" else T.FRACCONVOLUTION2D).shape(s["cout"], h, w, cin)
+        b.downsample(s["stride"])
+        if k == "frac":
+            b.sourceStep(1.0 / s["inv"])
+        if s["bn"]:
+            b.postfixNorm(fa.NormType.BATCHNORM)
+        weights = conv_block(4000 + 17 * no, s["cout"], s["k"], cin, bn=s["bn"])
+    elif k == "bn":
+        b = fa.GPULayerBuilder(name).type(T.BATCHNORM).shape(cin, h, w, cin)
+        weights = np.concatenate([prng.uniform(6000 + no, (cin,), 0.5, 1.5), prng.normal(7000 + no, (cin,), 0, 0.2)]).astype(np.float32)
+    elif s["fn"] == "arith":
+        b = fa.SingletonArithLayerBuilder(name, fa.ArithType.MUL).operand(0.75).shape(cin, h, w, cin)
+    else:
+        b = fa.GPULayerBuilder(name).type({"sigmoid": T.SIGMOID, "tanh": T.TANH, "relu": T.RELU}[s["fn"]]).shape(cin, h, w, cin)
+    b.number(no).inputPadding(s["pad_in"]).outputPadding(pad_out).prefixAct(s["act"])
+    if s["act"] == A.CLIP:
+        b.clip(-0.5, 1.5)
+    if s["act"] == A.LEAKY_RELU:
+        b.leakyReLU(0.2)
+    return b, weights
+
+
+@pytest.mark.parametrize("storage", [fa.STORAGE_F32, fa.STORAGE_F16], ids=["f32", "f16"])
+@pytest.mark.parametrize("seed", range(24))
+def test_random_shallow_chain(seed, storage):
+    shape0, specs, last_pad = _random_shallow_chain(seed)
+    pads = [specs[i + 1]["pad_in"] if i + 1 < len(specs) else last_pad for i in range(len(specs))]
+    built = [_shallow_builder(i, s, pads[i]) for i, s in enumerate(specs)]
+    print("seed", seed, "input", shape0, [(s["kind"], s.get("k"), s["pad_in"], s["out"]) for s in specs], flush=True)
+
+    class Net(fa.NeuralNetwork):
+        def buildLayers(self, f):
+            for b, _ in built:
+                b.push(f)
+
+        def connectLayers(self, layers, bm):
+            for i in range(1, len(built)):
+                bm.connectLayers(layers[i], layers[i + 1], 0)
+                if specs[i]["kind"] == "resconv":
+                    bm.connectLayers(layers[i], layers[i + 1], 1)
+
+        def initializeWeights(self, layers):
+            for b, w in built:
+                if w is None:
+                    continue
+                if int(b.type_) == int(T.BATCHNORM):
+                    layers[b.number_].loadScaleAndBias(w, 0)
+                else:
+                    layers[b.number_].loadWeightsAndBiases(w, 0)
+
+    x = prng.uniform(8000 + seed, shape0, -1.5, 1.5)
+    net = Net(storage)
+    net.setup(reuseBuffers=False)
+    net.layers[1].setInput(x, 0)
+    net.forward()
+    net.finish()
+    got = {lyr.number: lyr.copyResult() for lyr in net.layers}
+    desc = net.describe()
+    ref = O.run_network(desc, {(1, 0): x})
+    forced = O.run_network(desc, {(1, 0): x}, forced=got) if storage == fa.STORAGE_F16 else ref
+    for lyr in net.layers:
+        e = rel_l2(got[lyr.number], forced[lyr.number])
+        print("   %2d %-12s %-70s %.2e" % (lyr.number, lyr.name, lyr.kernelInfo()[:70], e), flush=True)
+        assert got[lyr.number].shape == tuple(specs[lyr.number - 1]["out"])
+        assert e <= TOL[storage], (seed, lyr.name, e)
+    net.cleanup()
