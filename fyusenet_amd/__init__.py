@@ -11,4 +11,4 @@ from .builders import (ActType, ArgMaxLayerBuilder, ArithType, BlurKernelType, B
                        LayerBuilder, LayerFlags, LayerType, NormType, PoolLayerBuilder, ScaleLayerBuilder, ScalingType,
                        SingletonArithLayerBuilder, TransposeLayerBuilder, UpDownLayerBuilder)
 from .capi import FynException, ORDER_CHANNELWISE, ORDER_GPU_DEEP, ORDER_GPU_SHALLOW, STORAGE_F16, STORAGE_F32  # noqa: F401
-from .network import BufferManager, CompiledLayers, Layer, LayerFactory, NeuralNetwork  # noqa: F401
+from .network import BufferManager, CompiledLayers, FramePool, Layer, LayerFactory, NeuralNetwork  # noqa: F401

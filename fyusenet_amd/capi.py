@@ -119,7 +119,7 @@ SYMBOLS = {
     "fyn_net_use_graph": (ctypes.c_int, [_P, ctypes.c_int]),
     "fyn_net_time_forward": (ctypes.c_int, [_P, ctypes.c_int, _F]),
     "fyn_layer_time": (ctypes.c_int, [_P, ctypes.c_int, ctypes.c_int, _F]),
-    "fyn_net_async_begin": (ctypes.c_int, [_P, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int]),
+    "fyn_net_async_begin": (ctypes.c_int, [_P, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int]),
     "fyn_net_async_submit": (ctypes.c_int, [_P, _F, _F, ctypes.POINTER(ctypes.c_uint64)]),
     "fyn_net_async_wait": (ctypes.c_int, [_P, ctypes.c_uint64]),
     "fyn_net_async_end": (ctypes.c_int, [_P]),

@@ -230,9 +230,9 @@ int fyn_layer_time(fyn_net* net, int layer, int iters, float* ms_total) {
     FYN_API_END
 }
 
-int fyn_net_async_begin(fyn_net* net, int in_layer, int in_port, int in_order, int out_layer, int out_order, int depth) {
+int fyn_net_async_begin(fyn_net* net, int in_layer, int in_port, int in_order, int out_layer, int out_order, int depth, int copy_streams) {
     FYN_API_BEGIN
-    N(net)->async_begin(in_layer, in_port, in_order, out_layer, out_order, depth);
+    N(net)->async_begin(in_layer, in_port, in_order, out_layer, out_order, depth, copy_streams != 0);
     FYN_API_END
 }
 

@@ -518,7 +518,7 @@ void Net::time_layer(int layer_no, int iters, float* ms) {
 //            down stream  device staging slot -> pinned host slot
 // A slot is reused only after its download has completed, which also orders the staging buffers.
 // ---------------------------------------------------------------------------------------------
-void Net::async_begin(int in_layer, int in_port, int in_order, int out_layer, int out_order, int depth) {
+void Net::async_begin(int in_layer, int in_port, int in_order, int out_layer, int out_order, int depth, bool copy_streams) {
     if (!is_setup) fail(FYN_ERR_STATE, "async_begin() before setup()");
     if (!slots_.empty()) fail(FYN_ERR_STATE, "frame pipeline is already active");
     if (depth < 1 || depth > 8) fail(FYN_ERR_INVALID, "pipeline depth %d out of range (1..8)", depth);
@@ -547,8 +547,13 @@ void Net::async_begin(int in_layer, int in_port, int in_order, int out_layer, in
     async_in_floats_ = (size_t)vi.c * vi.h * vi.w;
     async_in_order_ = in_order;
     async_out_order_ = out_order;
-    FYN_HIP(hipStreamCreateWithFlags(&up_stream_, hipStreamNonBlocking));
-    FYN_HIP(hipStreamCreateWithFlags(&down_stream_, hipStreamNonBlocking));
+    async_own_streams_ = copy_streams;
+    if (async_own_streams_) {
+        FYN_HIP(hipStreamCreateWithFlags(&up_stream_, hipStreamNonBlocking));
+        FYN_HIP(hipStreamCreateWithFlags(&down_stream_, hipStreamNonBlocking));
+    } else {
+        up_stream_ = down_stream_ = stream;
+    }
     slots_.resize(depth);
     for (AsyncSlot& s : slots_) {
         FYN_HIP(hipHostMalloc(reinterpret_cast<void**>(&s.pin_in), async_in_floats_ * sizeof(float), hipHostMallocDefault));
@@ -624,8 +629,8 @@ void Net::async_end() {
         if (s.down) (void)hipEventDestroy(s.down);
     }
     slots_.clear();
-    if (up_stream_) (void)hipStreamDestroy(up_stream_);
-    if (down_stream_) (void)hipStreamDestroy(down_stream_);
+    if (async_own_streams_ && up_stream_) (void)hipStreamDestroy(up_stream_);
+    if (async_own_streams_ && down_stream_) (void)hipStreamDestroy(down_stream_);
     up_stream_ = down_stream_ = nullptr;
     async_seq_ = 0;
 }

@@ -100,7 +100,7 @@ class Net {
     void time_layer(int layer, int iters, float* ms);
     void use_graph(bool enable);
     // frame pipeline: upload of frame i+1 and download of frame i-1 overlap the layers of frame i
-    void async_begin(int in_layer, int in_port, int in_order, int out_layer, int out_order, int depth);
+    void async_begin(int in_layer, int in_port, int in_order, int out_layer, int out_order, int depth, bool copy_streams);
     void async_submit(const float* in, float* out, uint64_t* ticket);
     void async_wait(uint64_t ticket);
     void async_end();
@@ -134,6 +134,7 @@ class Net {
     hipStream_t up_stream_ = nullptr, down_stream_ = nullptr;
     const Tensor* async_in_ = nullptr;
     const Tensor* async_out_ = nullptr;
+    bool async_own_streams_ = true;
     TView async_out_view_{};   // what the output layer hands out (a download layer may name other channel counts)
     int async_in_order_ = 0, async_out_order_ = 0;
     size_t async_in_floats_ = 0, async_out_floats_ = 0;

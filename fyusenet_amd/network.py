@@ -6,6 +6,7 @@ connectLayers(layers, bufferManager) and initializeWeights(layers); setup() runs
 of NeuralNetwork::glSetup (fyusenet/base/neuralnetwork.cpp:238-250).
 """
 import ctypes
+import os
 
 import numpy as np
 
@@ -286,8 +287,10 @@ class NeuralNetwork:
         return ms.value
 
     # -- frame pipeline (asynchronous engine mode of the reference, base/engine.cpp:386-683) --
-    def asyncBegin(self, inLayer, outLayer, inOrder=capi.ORDER_CHANNELWISE, outOrder=capi.ORDER_CHANNELWISE, depth=2, inPort=0):
-        capi.check(capi.lib().fyn_net_async_begin(self._h, inLayer, inPort, inOrder, outLayer, outOrder, depth))
+    def asyncBegin(self, inLayer, outLayer, inOrder=capi.ORDER_CHANNELWISE, outOrder=capi.ORDER_CHANNELWISE, depth=2, inPort=0, copyStreams=True):
+        """copyStreams=False queues uploads and downloads on the network's own stream (for networks that run side by
+        side, see FramePool)."""
+        capi.check(capi.lib().fyn_net_async_begin(self._h, inLayer, inPort, inOrder, outLayer, outOrder, depth, 1 if copyStreams else 0))
 
     def asyncSubmit(self, frame, out):
         """Queues one frame; `out` (a C-contiguous float32 array) is filled once asyncWait(ticket) has returned."""
@@ -310,3 +313,60 @@ class NeuralNetwork:
             b = lyr.builder
             out.append({"builder": b, "number": lyr.number, "weights": lyr.weights})
         return {"layers": out, "connections": list(self.bufferManager.connections), "storage": self.storage}
+
+
+class FramePool:
+    """Several instances of one network, each with its own streams and frame pipeline.  Frames are dealt to the
+    instances in turn, so that the kernels of up to `instances` frames share the GPU: small networks at batch 1 are
+    bound by launch latency and leave most of the chip idle, and frames of different instances do not depend on each
+    other.  Results are delivered in submission order through tickets, like NeuralNetwork.asyncSubmit / asyncWait
+    (the reference runs one frame pipeline per network, base/engine.cpp:386-683; several of them side by side are
+    several NeuralNetwork objects there as well).  More instances than hardware queues per process (4 by default)
+    do not add throughput.
+
+    make_net: callable returning a NeuralNetwork (not yet set up) with `input_key` and `output_layer` attributes.
+    graph: replay each instance's forward pass as one captured graph, which cuts the host thread's share per frame from
+    one launch per layer to one per frame (with 70-90 launches per frame the host thread is the limit otherwise)."""
+
+    def __init__(self, make_net, instances=4, depth=2, inOrder=capi.ORDER_CHANNELWISE, outOrder=capi.ORDER_CHANNELWISE, graph=True):
+        if instances < 1:
+            raise capi.FynException(capi.ERR_INVALID, "a frame pool needs at least one network instance")
+        self.nets, self._open, self._submitted = [], {}, 0
+        try:
+            for _ in range(instances):
+                net = make_net()
+                self.nets.append(net)
+                net.setup()
+                if graph:
+                    net.useGraph(True)
+                in_layer, in_port = net.input_key
+                # one stream per instance: the instances overlap each other, and more streams than hardware queues
+                # (4 per process by default) would wait for each other's events
+                net.asyncBegin(in_layer, net.output_layer, inOrder, outOrder, depth, in_port, copyStreams=(instances == 1))
+        except Exception:
+            self.close()
+            raise
+
+    def submit(self, frame, out):
+        """Queues one frame on the next instance; `out` is filled once wait(ticket) has returned.  Blocks while that
+        instance's pipeline is full."""
+        net = self.nets[self._submitted % len(self.nets)]
+        self._submitted += 1
+        self._open[self._submitted] = (net, net.asyncSubmit(frame, out))
+        return self._submitted
+
+    def wait(self, ticket):
+        """Returns when the frame of `ticket` and every frame submitted before it have been delivered."""
+        if ticket < 1 or ticket > self._submitted:
+            raise capi.FynException(capi.ERR_INVALID, "unknown frame ticket %d" % ticket)
+        for t in sorted(k for k in self._open if k <= ticket):
+            net, local = self._open.pop(t)
+            net.asyncWait(local)
+
+    def close(self):
+        for net in self.nets:
+            try:
+                net.asyncEnd()
+            finally:
+                net.cleanup()
+        self.nets, self._open = [], {}

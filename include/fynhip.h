@@ -250,8 +250,12 @@ int fyn_layer_time(fyn_net* net, int layer, int iters, float* ms_total);
  *   submit: copies `in` (borrowed for the call) and queues the frame; `out` must stay valid until the frame's
  *           ticket has been waited for (it is filled then, or when its slot is reused `depth` submits later).
  *   wait  : blocks until the frame (and all earlier ones) has been delivered.   end: drains and frees the pipeline.
- * Orders: input CHANNELWISE or GPU_SHALLOW, output CHANNELWISE or GPU_SHALLOW. */
-int fyn_net_async_begin(fyn_net* net, int in_layer, int in_port, int in_order, int out_layer, int out_order, int depth);
+ * Orders: input CHANNELWISE or GPU_SHALLOW, output CHANNELWISE or GPU_SHALLOW.
+ * copy_streams != 0: uploads and downloads run on two streams of the pipeline's own (overlap inside this network).
+ * copy_streams == 0: they are queued on the network's stream, between the frames' layers; for several networks that
+ * run side by side, whose frames overlap each other, and whose streams would otherwise outnumber the hardware queues
+ * of the process (streams that share a queue wait for each other's events). */
+int fyn_net_async_begin(fyn_net* net, int in_layer, int in_port, int in_order, int out_layer, int out_order, int depth, int copy_streams);
 int fyn_net_async_submit(fyn_net* net, const float* in, float* out, uint64_t* ticket);
 int fyn_net_async_wait(fyn_net* net, uint64_t ticket);
 int fyn_net_async_end(fyn_net* net);

@@ -260,8 +260,9 @@ def test_reference_style_net_sample_graphs(kernel, width, height, storage):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("copy_streams", [True, False], ids=["three_streams", "one_stream"])
 @pytest.mark.parametrize("depth", [1, 2, 3])
-def test_frame_pipeline_matches_synchronous_path(depth):
+def test_frame_pipeline_matches_synchronous_path(depth, copy_streams):
     """Asynchronous frame pipeline (upload / layers / download on three streams) against
     setInput -> forward -> getOutput for a stream of different frames: bit-identical outputs, in order."""
     from fyusenet_amd import prng
@@ -276,7 +277,7 @@ def test_frame_pipeline_matches_synchronous_path(depth):
         want.append(net.getOutput(net.output_layer).copy())
     assert not np.array_equal(want[0], want[1])
     in_layer, in_port = net.input_key
-    net.asyncBegin(in_layer, net.output_layer, depth=depth, inPort=in_port)
+    net.asyncBegin(in_layer, net.output_layer, depth=depth, inPort=in_port, copyStreams=copy_streams)
     outs = [np.full_like(want[0], np.nan) for _ in frames]
     tickets = [net.asyncSubmit(f, o) for f, o in zip(frames, outs)]
     assert tickets == list(range(1, len(frames) + 1))
@@ -300,3 +301,35 @@ def test_frame_pipeline_matches_synchronous_path(depth):
     assert np.array_equal(hwc[..., :3].transpose(2, 0, 1), want[3])
     net.asyncEnd()
     net.cleanup()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("instances,depth", [(1, 2), (3, 1), (4, 2)])
+def test_frame_pool_delivers_in_order_and_bit_identical(instances, depth):
+    """Several network instances with a frame pipeline each, frames dealt round-robin: every frame's result equals
+    the synchronous path's, bit for bit, and arrives under its own ticket."""
+    from fyusenet_amd import prng
+    make = lambda: networks.StyleNet(fa.STORAGE_F32, width=64, height=48)   # noqa: E731
+    ref = make()
+    ref.setup()
+    frames = [prng.uniform(1200 + i, (3, 48, 64), -1.0, 1.0) for i in range(11)]
+    want = []
+    for f in frames:
+        ref.setInput(f)
+        ref.forward()
+        ref.finish()
+        want.append(ref.getOutput(ref.output_layer).copy())
+    ref.cleanup()
+    pool = fa.FramePool(make, instances=instances, depth=depth)
+    outs = [np.full_like(want[0], np.nan) for _ in frames]
+    tickets = [pool.submit(f, o) for f, o in zip(frames[:6], outs[:6])]
+    pool.wait(tickets[2])
+    for i in range(3):
+        assert np.array_equal(outs[i], want[i]), i
+    tickets += [pool.submit(f, o) for f, o in zip(frames[6:], outs[6:])]
+    pool.wait(tickets[-1])
+    for i in range(len(frames)):
+        assert np.array_equal(outs[i], want[i]), i
+    with pytest.raises(fa.FynException):
+        pool.wait(len(frames) + 1)
+    pool.close()
