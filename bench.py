@@ -352,7 +352,7 @@ def main():
     if hasattr(net, "input_key") and args.workload != "copy" and not isinstance(net, BandwidthNet):
         out["host_io"] = host_io_rates(net, x, max(args.steps, 50))
         log("host I/O inclusive: %s" % out["host_io"])
-        pool_shape = net.getOutput(net.output_layer).shape if unit == "imgs/s" else None
+        pool_shape = net.getOutput(net.output_layer).shape if unit in ("imgs/s", "ms/frame") else None
 
     if not args.no_cpu_baseline and total_flops > 0:
         dt, flops, threads, lname = cpu_baseline(net, x, total_flops)
@@ -367,10 +367,11 @@ def main():
                                "sample": "layer %s at full size (%.2f GFLOP, %.2f s on %d threads), scaled by the step's %.1f GFLOP"
                                          % (lname, flops / 1e9, dt, threads, total_flops / 1e9)}
     net.cleanup()
-    if hasattr(net, "input_key") and unit == "imgs/s":
-        # latency-bound batch-1 networks: several instances side by side (after this network's stream is gone: the
-        # pool's streams should have the process's hardware queues to themselves)
-        out["frame_pool"] = frame_pool_rate(args.workload, x, pool_shape, max(8 * args.steps, 800))
+    if hasattr(net, "input_key") and unit in ("imgs/s", "ms/frame"):
+        # several instances side by side: batch-1 networks of small layers are latency-bound, and even the style net's
+        # launches leave a fifth of the chip idle (after this network is gone: the pool's streams should have the
+        # process's hardware queues to themselves)
+        out["frame_pool"] = frame_pool_rate(args.workload, x, pool_shape, max(8 * args.steps, 400))
         log("frame pool: %s" % out["frame_pool"])
 
     if not args.no_also and args.workload == "stylenet":

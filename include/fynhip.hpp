@@ -734,6 +734,57 @@ class NeuralNetwork {
     std::unique_ptr<BufferManager> buffers_;
 };
 
+/*
+ * Several instances of one network, each with its own stream, frame pipeline and captured graph; frames are dealt to the
+ * instances in turn, so that the kernels of up to `instances` frames share the GPU (batch-1 networks of small layers are
+ * bound by launch latency and leave most of the chip idle).  Results are delivered in submission order through
+ * tickets.  The reference runs one frame pipeline per network (base/engine.cpp:386-683); several side by side are several
+ * NeuralNetwork objects there as well.  More instances than hardware queues per process (4 by default) add nothing.
+ *   Net: a NeuralNetwork subclass; make(): returns a new, not yet set up instance.
+ */
+template <typename Net>
+class FramePool {
+  public:
+    FramePool(const std::function<std::unique_ptr<Net>()>& make, int inLayer, int outLayer, int instances = 4, int depth = 2,
+              int inOrder = FYN_ORDER_CHANNELWISE, int outOrder = FYN_ORDER_CHANNELWISE, bool graph = true) {
+        if (instances < 1) detail::raise(FYN_ERR_INVALID, "a frame pool needs at least one network instance");
+        for (int i = 0; i < instances; i++) {
+            nets_.push_back(make());
+            Net& n = *nets_.back();
+            n.setup();
+            if (graph) n.useGraph(true);
+            // one stream per instance: the instances overlap each other, and more streams than hardware queues would
+            // wait for each other's events
+            n.asyncBegin(inLayer, outLayer, inOrder, outOrder, depth, 0, instances == 1);
+        }
+    }
+    ~FramePool() {
+        for (auto& n : nets_) {
+            try { n->asyncEnd(); } catch (...) {}
+        }
+    }
+    /* Queues one frame on the next instance; `out` is filled once wait(ticket) has returned. */
+    uint64_t submit(const float* frame, float* out) {
+        Net& n = *nets_[submitted_ % nets_.size()];
+        open_[++submitted_] = std::make_pair(&n, n.asyncSubmit(frame, out));
+        return submitted_;
+    }
+    /* Returns when the frame of `ticket` and every frame submitted before it have been delivered. */
+    void wait(uint64_t ticket) {
+        if (ticket < 1 || ticket > submitted_) detail::raise(FYN_ERR_INVALID, "unknown frame ticket %llu", (unsigned long long)ticket);
+        while (!open_.empty() && open_.begin()->first <= ticket) {
+            open_.begin()->second.first->asyncWait(open_.begin()->second.second);
+            open_.erase(open_.begin());
+        }
+    }
+    size_t instances() const { return nets_.size(); }
+
+  private:
+    std::vector<std::unique_ptr<Net>> nets_;
+    std::map<uint64_t, std::pair<Net*, uint64_t>> open_;
+    uint64_t submitted_ = 0;
+};
+
 }  // namespace fynhip
 
 #ifdef FYNHIP_REFERENCE_NAMESPACE

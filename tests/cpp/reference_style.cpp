@@ -280,6 +280,24 @@ int main(int argc, char** argv) {
         net.finish();
         net.getOutput(StyleNet3x3::DOWNLOAD, again.data(), FYN_ORDER_GPU_SHALLOW);
         EXPECT(again == rgba);
+        {   // three instances side by side: every frame's result under its own ticket, equal to the single network's
+            std::vector<float> w = weights;
+            FramePool<StyleNet3x3> pool(
+                [&]() {
+                    std::unique_ptr<StyleNet3x3> n(new StyleNet3x3(width, height));
+                    n->loadWeightsAndBiases(w.data(), w.size());
+                    return n;
+                },
+                StyleNet3x3::UPLOAD, StyleNet3x3::DOWNLOAD, 3, 2, FYN_ORDER_GPU_SHALLOW, FYN_ORDER_GPU_SHALLOW);
+            std::vector<std::vector<float>> outs(7, std::vector<float>(rgba.size(), -1.f));
+            uint64_t last = 0;
+            for (auto& o : outs) last = pool.submit(rgb.data(), o.data());
+            pool.wait(last);
+            bool same = true;
+            for (auto& o : outs) same = same && o == rgba;
+            EXPECT(same);
+            EXPECT(pool.instances() == 3);
+        }
         FILE* f = std::fopen(argv[3], "wb");
         if (!f || std::fwrite(rgba.data(), sizeof(float), rgba.size(), f) != rgba.size()) {
             std::fprintf(stderr, "cannot write %s\n", argv[3]);
