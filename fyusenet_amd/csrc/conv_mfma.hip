@@ -446,28 +446,43 @@ __device__ __forceinline__ void conv_mfma_body(const ConvMfmaParams& p, unsigned
             }
         }
     };
-    for (int chunk = chunk0; chunk < chunk1; chunk++) {
-        const bool more_chunks = chunk + 1 < chunk1;
-        // (after the last chunk the fetch is unused; it keeps the number of loads in flight static)
-        if (stager) fetch_first(more_chunks ? chunk + 1 : chunk);
-        if (consumer) {
-            const StepOff<KC> ao = ao_reg[0];
-#pragma unroll
-            for (int fn = 0; fn < FN; fn++)
-#pragma unroll
-                for (int pl = 0; pl < NPL; pl++) b_buf[0][fn][pl] = load_b_frag<KC>(cur + pl * p.plane + boff[fn], ao);
-            for (int t0 = 0; t0 < nsub; t0 += UNR) run_group(t0);
-        }
-        FYN_TRACE(2 + 2 * (chunk - chunk0));
-        if (more_chunks) {
-            unsigned char* nxt = sbase + ((chunk - chunk0 + 1) & 1) * bufsz;
-            if (stager) {
+    // One loop per role where the roles are separate waves: a wave's registers then hold either the staging items or
+    // the fragments and accumulators, not both (the two kinds of waves execute the same barriers, one per chunk).
+    if (SPEC && !consumer) {
+        for (int chunk = chunk0; chunk < chunk1; chunk++) {
+            const bool more_chunks = chunk + 1 < chunk1;
+            if (more_chunks) {
+                fetch_first(chunk + 1);
+                unsigned char* nxt = sbase + ((chunk - chunk0 + 1) & 1) * bufsz;
                 store_first(chunk + 1, nxt);
                 stage_rest(chunk + 1, nxt);
+                __syncthreads();  // everyone is done reading the current buffer and writing `nxt`
             }
-            __syncthreads();  // everyone is done reading `cur` and writing `nxt`
-            cur = nxt;
-            FYN_TRACE(3 + 2 * (chunk - chunk0));
+        }
+    } else {
+        for (int chunk = chunk0; chunk < chunk1; chunk++) {
+            const bool more_chunks = chunk + 1 < chunk1;
+            // (after the last chunk the fetch is unused; it keeps the number of loads in flight static)
+            if (!SPEC) fetch_first(more_chunks ? chunk + 1 : chunk);
+            {
+                const StepOff<KC> ao = ao_reg[0];
+#pragma unroll
+                for (int fn = 0; fn < FN; fn++)
+#pragma unroll
+                    for (int pl = 0; pl < NPL; pl++) b_buf[0][fn][pl] = load_b_frag<KC>(cur + pl * p.plane + boff[fn], ao);
+                for (int t0 = 0; t0 < nsub; t0 += UNR) run_group(t0);
+            }
+            FYN_TRACE(2 + 2 * (chunk - chunk0));
+            if (more_chunks) {
+                unsigned char* nxt = sbase + ((chunk - chunk0 + 1) & 1) * bufsz;
+                if (!SPEC) {
+                    store_first(chunk + 1, nxt);
+                    stage_rest(chunk + 1, nxt);
+                }
+                __syncthreads();  // everyone is done reading `cur` and writing `nxt`
+                cur = nxt;
+                FYN_TRACE(3 + 2 * (chunk - chunk0));
+            }
         }
     }
 
