@@ -276,6 +276,21 @@ def frame_pool_rate(workload, x, y_shape, frames, instances=4):
     return {"instances": instances, "frames_per_s": frames / dt, "ms_per_frame": dt * 1e3 / frames}
 
 
+def frame_pool_rate_in_child(workload, frames, instances=4):
+    """frame_pool_rate in a process of its own (started as a child, never exec'ed into): the side measurement gets a
+    fresh HIP runtime with the hardware queues to itself, and a failure in it cannot take the main record with it."""
+    import subprocess
+    cmd = [sys.executable, os.path.abspath(__file__), "--frame-pool-only", "--workload", workload, "--steps", str(frames),
+           "--instances", str(instances)]
+    try:
+        r = subprocess.run(cmd, capture_output=True, text=True, timeout=240)
+        if r.returncode != 0:
+            return {"error": "child exited with %d: %s" % (r.returncode, r.stderr.strip()[-300:])}
+        return json.loads(r.stdout.strip().splitlines()[-1])
+    except Exception as e:   # noqa: BLE001 -- a side measurement must not fail the benchmark
+        return {"error": repr(e)}
+
+
 def cpu_baseline(net, x, total_flops):
     """Times the CPU oracle (plain C restatement of the reference's unit-test convolution, OpenMP over
     output channels) on the dominant convolution of the workload at full size and scales by the
@@ -306,9 +321,24 @@ def main():
     ap.add_argument("--workload", default="stylenet")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-also", action="store_true")
+    ap.add_argument("--no-pool", action="store_true", help="skip the side measurement of several instances side by side")
+    ap.add_argument("--frame-pool-only", action="store_true", help="(internal) print the frame pool's record for --workload; --steps = frames")
+    ap.add_argument("--instances", type=int, default=4)
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py: this engine is single-GPU (batch 1 inference); run with --gpus 1")
+
+    if args.frame_pool_only:
+        probe = make_net(args.workload)[0]
+        probe.setup()
+        x = probe.makeInput()
+        probe.setInput(x)
+        probe.forward()
+        probe.finish()
+        y_shape = probe.getOutput(probe.output_layer).shape
+        probe.cleanup()
+        print(json.dumps(frame_pool_rate(args.workload, x, y_shape, args.steps, args.instances)), flush=True)
+        return
 
     log(fa.capi.device_info(0))
     net, metric, unit, dtype = make_net(args.workload)
@@ -352,7 +382,6 @@ def main():
     if hasattr(net, "input_key") and args.workload != "copy" and not isinstance(net, BandwidthNet):
         out["host_io"] = host_io_rates(net, x, max(args.steps, 50))
         log("host I/O inclusive: %s" % out["host_io"])
-        pool_shape = net.getOutput(net.output_layer).shape if unit in ("imgs/s", "ms/frame") else None
 
     if not args.no_cpu_baseline and total_flops > 0:
         dt, flops, threads, lname = cpu_baseline(net, x, total_flops)
@@ -371,8 +400,9 @@ def main():
         # several instances side by side: batch-1 networks of small layers are latency-bound, and even the style net's
         # launches leave a fifth of the chip idle (after this network is gone: the pool's streams should have the
         # process's hardware queues to themselves)
-        out["frame_pool"] = frame_pool_rate(args.workload, x, pool_shape, max(8 * args.steps, 400))
-        log("frame pool: %s" % out["frame_pool"])
+        if not args.no_pool:
+            out["frame_pool"] = frame_pool_rate_in_child(args.workload, max(8 * args.steps, 400))
+            log("frame pool: %s" % out["frame_pool"])
 
     if not args.no_also and args.workload == "stylenet":
         also = {}
@@ -385,10 +415,9 @@ def main():
             ms2 = min(ms2g, ms2e)
             also[m2] = {"value": 1e3 / ms2 if u2 == "imgs/s" else ms2, "unit": u2, "ms_per_step": ms2, "ms_per_step_graph": ms2g, "ms_per_step_eager": ms2e, "dtype": d2}
             log("%s: %.4f ms/step (hipGraph) %.4f (eager)" % (wl, ms2g, ms2e))
-            x2, y2_shape = n2.makeInput(), n2.getOutput(n2.output_layer).shape
             n2.cleanup()
-            if wl == "resnet50":
-                also[m2]["frame_pool"] = frame_pool_rate(wl, x2, y2_shape, 800)
+            if wl == "resnet50" and not args.no_pool:
+                also[m2]["frame_pool"] = frame_pool_rate_in_child(wl, 800)
         out["also"] = also
     print(json.dumps(out), flush=True)
 
