@@ -255,7 +255,7 @@ static MfmaLaunch plan_mfma(Net* net, const SubConv& sc, const TView& in, const 
         const bool ksplit_tile = tc.wm * tc.wn < 4;      // waves split the steps of a chunk: smallest step group
         if (ksplit_tile) pd = 2;
         L.var.pd = pd;
-        L.var.unr = (pd == 6 && raw == 18 && force_pd == 0 && !getenv("FYNHIP_CONV_NO_FULL_UNROLL")) ? 18 : pd;
+        L.var.unr = (pd == 6 && raw % 18 == 0 && force_pd == 0 && !getenv("FYNHIP_CONV_NO_FULL_UNROLL")) ? 18 : pd;
         if (kc == 128 && !ksplit_tile) L.var.unr = 8;
         if (!conv_mfma_variant_exists(L.var)) fail(FYN_ERR_UNSUPPORTED, "MFMA convolution variant not compiled");
     }
