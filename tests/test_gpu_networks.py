@@ -333,3 +333,41 @@ def test_frame_pool_delivers_in_order_and_bit_identical(instances, depth):
     with pytest.raises(fa.FynException):
         pool.wait(len(frames) + 1)
     pool.close()
+
+
+@pytest.mark.gpu
+def test_many_networks_at_once_and_in_sequence():
+    """Networks lease their streams from a per-device set created at first use: more networks alive at once than that
+    set holds (the overflow gets streams of its own), and many created and destroyed in sequence, all give the single
+    network's result."""
+    from fyusenet_amd import prng
+    x = prng.uniform(77, (3, 32, 40), -1.0, 1.0)
+
+    def run(net):
+        net.setInput(x)
+        net.forward()
+        net.finish()
+        return net.getOutput(net.output_layer).copy()
+
+    first = networks.StyleNet(fa.STORAGE_F32, width=40, height=32)
+    first.setup()
+    want = run(first)
+    crowd = [networks.StyleNet(fa.STORAGE_F32, width=40, height=32) for _ in range(11)]
+    for n in crowd:
+        n.setup()
+    for n in crowd:            # all launched before any is waited for
+        n.setInput(x)
+        n.forward()
+    for n in crowd:
+        n.finish()
+        assert np.array_equal(n.getOutput(n.output_layer), want)
+    for n in crowd:
+        n.cleanup()
+    for _ in range(12):
+        n = networks.StyleNet(fa.STORAGE_F32, width=40, height=32)
+        n.setup()
+        n.useGraph(True)
+        assert np.array_equal(run(n), want)
+        n.cleanup()
+    assert np.array_equal(run(first), want)
+    first.cleanup()
