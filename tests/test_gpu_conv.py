@@ -143,6 +143,38 @@ def test_tiles_whose_waves_split_k(k, cin, cout, h, w, ksplit, kw, tile, storage
     assert err <= TOL[storage], info
 
 
+ALL_TILES = ["2,2,2,2", "2,2,1,4", "2,1,2,2", "2,1,1,4", "1,2,1,4", "1,1,1,4", "1,1,4,1", "1,1,2,2", "1,2,4,1", "1,3,4,1", "1,4,4,1",
+             "1,2,2,2", "1,4,2,2", "1,3,2,2", "1,4,1,4", "1,3,1,4", "1,1,1,1", "1,1,2,1", "1,1,1,2"]
+
+
+@pytest.mark.parametrize("storage", [fa.STORAGE_F32, fa.STORAGE_F16], ids=["f32", "f16"])
+@pytest.mark.parametrize("tile", ALL_TILES)
+@pytest.mark.parametrize("k,cin,cout,h,w,stride,kw", [
+    (3, 64, 40, 20, 24, 1, {"bn": True, "residual": (A.RELU, True)}),
+    (1, 160, 24, 9, 13, 1, {}),
+    (5, 16, 130, 12, 10, 2, {"bn": True}),
+], ids=["k3_res", "k1_wide_chunks", "k5_s2_16ch"])
+def test_every_tile_shape(k, cin, cout, h, w, stride, kw, tile, storage, monkeypatch):
+    """Every workgroup shape of the convolution kernel (fragments per wave x wave arrangement), forced through the
+    engine's tile switch: the tuner only ever picks a few of them for a given layer."""
+    monkeypatch.setenv("FYNHIP_CONV_TILE", tile)
+    b = conv_builder(k, cout, h, w, cin, stride, 1, A.RELU, **kw)
+    wts = conv_block(600 + k + cin, cout, k, cin, bn=kw.get("bn", False))
+    inputs = [prng.uniform(15 * k + cin, (cin, h, w), -1, 1)]
+    if "residual" in kw:
+        inputs.append(prng.uniform(27, (cout, h // stride, w // stride), -1, 1))
+    try:
+        got, info = run_single(b, storage, inputs, wts)
+    except fa.FynException as e:
+        if "no MFMA tile configuration fits" in str(e):     # e.g. the K-split tiles exist for chunks of 32+ channels only
+            pytest.skip("tile %s does not exist for this layer" % tile)
+        raise
+    fm, fn, wm, wn = (int(v) for v in tile.split(","))
+    assert "tile=%dx%d" % (32 * fm * wm, 32 * fn * wn) in info and "waves=%dx%d" % (wm, wn) in info
+    err = rel_l2(got, oracle_single(b, storage, inputs, wts))
+    assert err <= TOL[storage], info
+
+
 def test_kernel_too_large_for_the_step_table_is_rejected():
     # 13x13 on 32 channels = 338 k16 steps per chunk, more than the 256-entry step table
     b = conv_builder(13, 8, 32, 32, 32)
