@@ -3,7 +3,9 @@
 // Replaces the additive-blend render passes of DeepConvLayerNxN::forward
 // (fyusenet/gpu/deep/deepconvlayerNxN.cpp:129-211), DeepConvLayer1x1::forward
 // (deepconvlayer1x1.cpp:67-117), the shallow ConvLayerNxN::forward
-// (gpu/vanilla/convlayerNxN_vanilla.cpp:72-141) and, launched once per output parity, the stencil
+// (gpu/vanilla/convlayerNxN_vanilla.cpp:72-141) with its sampler's edge clamp, the fractional-step
+// FractionalConvLayerNxN (gpu/vanilla/fractionalconvlayerNxN_vanilla.cpp:43-91; both applied while a
+// halo tile is staged: in_clamp, in_shift) and, launched once per output parity, the stencil
 // passes of DeepTransConvLayerBase::forward (gpu/deep/deeptransconvlayerbase.cpp:83-130).
 //
 // GEMM view: M = output channels (A operand = weights, pre-packed per lane in HBM, streamed
