@@ -258,11 +258,11 @@ def host_io_rates(net, x, frames):
     return rec
 
 
-def frame_pool_rate(workload, x, y_shape, frames, instances=4):
+def frame_pool_rate(workload, x, y_shape, frames, instances=4, graph=True):
     """Frames per second through a pool of `instances` networks of this workload, each with its own streams and frame
     pipeline; frames come from host memory and results return there (PCIe inside the timed region).  Reported beside
     `value`, never as `value`."""
-    pool = fa.FramePool(lambda: make_net(workload)[0], instances=instances, depth=2)
+    pool = fa.FramePool(lambda: make_net(workload)[0], instances=instances, depth=2, graph=graph)
     outs = [np.empty(y_shape, np.float32) for _ in range(3 * instances)]
     for i in range(2 * instances):
         t = pool.submit(x, outs[i % len(outs)])
@@ -273,15 +273,16 @@ def frame_pool_rate(workload, x, y_shape, frames, instances=4):
     pool.wait(t)
     dt = time.perf_counter() - t0
     pool.close()
-    return {"instances": instances, "frames_per_s": frames / dt, "ms_per_frame": dt * 1e3 / frames}
+    return {"instances": instances, "launch": "hipGraph replay" if graph else "eager launches", "frames_per_s": frames / dt,
+            "ms_per_frame": dt * 1e3 / frames}
 
 
-def frame_pool_rate_in_child(workload, frames, instances=4):
+def frame_pool_rate_in_child(workload, frames, instances=4, graph=True):
     """frame_pool_rate in a process of its own (started as a child, never exec'ed into): the side measurement gets a
     fresh HIP runtime with the hardware queues to itself, and a failure in it cannot take the main record with it."""
     import subprocess
     cmd = [sys.executable, os.path.abspath(__file__), "--frame-pool-only", "--workload", workload, "--steps", str(frames),
-           "--instances", str(instances)]
+           "--instances", str(instances)] + ([] if graph else ["--pool-eager"])
     try:
         r = subprocess.run(cmd, capture_output=True, text=True, timeout=240)
         if r.returncode != 0:
@@ -324,6 +325,7 @@ def main():
     ap.add_argument("--no-pool", action="store_true", help="skip the side measurement of several instances side by side")
     ap.add_argument("--frame-pool-only", action="store_true", help="(internal) print the frame pool's record for --workload; --steps = frames")
     ap.add_argument("--instances", type=int, default=4)
+    ap.add_argument("--pool-eager", action="store_true", help="(internal) the pool's instances launch eagerly instead of replaying graphs")
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py: this engine is single-GPU (batch 1 inference); run with --gpus 1")
@@ -337,7 +339,7 @@ def main():
         probe.finish()
         y_shape = probe.getOutput(probe.output_layer).shape
         probe.cleanup()
-        print(json.dumps(frame_pool_rate(args.workload, x, y_shape, args.steps, args.instances)), flush=True)
+        print(json.dumps(frame_pool_rate(args.workload, x, y_shape, args.steps, args.instances, not args.pool_eager)), flush=True)
         return
 
     log(fa.capi.device_info(0))
@@ -396,10 +398,9 @@ def main():
                                "sample": "layer %s at full size (%.2f GFLOP, %.2f s on %d threads), scaled by the step's %.1f GFLOP"
                                          % (lname, flops / 1e9, dt, threads, total_flops / 1e9)}
     net.cleanup()
-    if hasattr(net, "input_key") and unit in ("imgs/s", "ms/frame"):
-        # several instances side by side: batch-1 networks of small layers are latency-bound, and even the style net's
-        # launches leave a fifth of the chip idle (after this network is gone: the pool's streams should have the
-        # process's hardware queues to themselves)
+    if hasattr(net, "input_key") and unit == "imgs/s":
+        # several instances side by side: batch-1 networks of small layers are latency-bound.  (The style nets' launches
+        # fill most of the chip: 2 to 4 instances of them run at the single frame pipeline's rate, 0.43-0.50 ms/frame.)
         if not args.no_pool:
             out["frame_pool"] = frame_pool_rate_in_child(args.workload, max(8 * args.steps, 400))
             log("frame pool: %s" % out["frame_pool"])
