@@ -699,6 +699,11 @@ static conv_kernel_fn pick_kc(int kc, int pd, int unr) {
         if (kc == 32 && pd == 2 && unr == 2) return conv_mfma_kernel<TIn, TOut, SPLIT, FM, FN, WM, WN, 32, 2, 2>;
         if (kc == 64 && pd == 2 && unr == 2) return conv_mfma_kernel<TIn, TOut, SPLIT, FM, FN, WM, WN, 64, 2, 2>;
         if (kc == 128 && pd == 2 && unr == 2) return conv_mfma_kernel<TIn, TOut, SPLIT, FM, FN, WM, WN, 128, 2, 2>;
+        // pointwise layers with many input channels: chunks of 256 to 1024 channels, so that a workgroup fetches its
+        // whole reduction in one or two memory round trips instead of one per 128 channels
+        if (kc == 256 && pd == 4 && unr == 4) return conv_mfma_kernel<TIn, TOut, SPLIT, FM, FN, WM, WN, 256, 4, 4>;
+        if (kc == 512 && pd == 4 && unr == 4) return conv_mfma_kernel<TIn, TOut, SPLIT, FM, FN, WM, WN, 512, 4, 4>;
+        if (kc == 1024 && pd == 4 && unr == 4) return conv_mfma_kernel<TIn, TOut, SPLIT, FM, FN, WM, WN, 1024, 4, 4>;
         return nullptr;
     } else {
     if (kc == 4 && pd == 2 && unr == 2) return conv_mfma_kernel<TIn, TOut, SPLIT, FM, FN, WM, WN, 4, 2, 2>;

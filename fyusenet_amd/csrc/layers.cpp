@@ -253,7 +253,7 @@ static MfmaLaunch plan_mfma(Net* net, const SubConv& sc, const TView& in, const 
         if (const char* e = getenv("FYNHIP_CONV_PD")) pd = atoi(e);
         if (force_pd > 0 && kc <= 32) pd = force_pd;
         const bool ksplit_tile = tc.wm * tc.wn < 4;      // waves split the steps of a chunk: smallest step group
-        if (ksplit_tile) pd = 2;
+        if (ksplit_tile) pd = kc > 128 ? 4 : 2;
         L.var.pd = pd;
         L.var.unr = (pd == 6 && raw % 18 == 0 && force_pd == 0 && !getenv("FYNHIP_CONV_NO_FULL_UNROLL")) ? 18 : pd;
         if (kc == 128 && !ksplit_tile) L.var.unr = 8;
@@ -392,15 +392,26 @@ static void tune_cache_store(const char* key, const ConvVariant& v, int ksplit) 
 // (default; timing does not depend on the data), or by the heuristic score when FYNHIP_AUTOTUNE=0.
 static MfmaLaunch tune_mfma(Net* net, const SubConv& sc, const TView& in, const TView& out, const TView* res, int cin,
                             int cout, const Act& act, int res_relu, int res_scale, const float* scale, const float* bias) {
-    // candidates: every tile that fits, for the geometry's default chunk width and, where that is wider
-    // than 32 channels, for 32-channel chunks too
+    // candidates: every tile that fits, for the geometry's default chunk width, where that is wider than 32
+    // channels for 32-channel chunks too, and for one-tap layers with 256 and more input channels chunks of
+    // 256 to 1024 channels (a workgroup then fetches its whole reduction in one to three memory round trips)
     std::vector<TileChoice> cands;
     {
         int kc0, pitch, slack, npl;
         conv_geometry(in, !net->f16(), (int)sc.taps.size(), 0, kc0, pitch, slack, npl);
         std::vector<int> kcs{kc0};
         if (kc0 > 32) kcs.push_back(32);
+        // one-tap layers with many input channels: also chunks of 256 to 1024 channels (K-split tiles only)
+        if (sc.taps.size() == 1 && !getenv("FYNHIP_CONV_KC_MAX"))
+            for (int big : {256, 512, 1024})
+                if (in.cp >= big) kcs.push_back(big);
+        if (const char* fk = getenv("FYNHIP_CONV_KC")) {   // testing: this chunk width first, the others only if it fits no tile
+            const int f = atoi(fk);
+            const bool known = f == 32 || f == 64 || f == 128 || ((f == 256 || f == 512 || f == 1024) && sc.taps.size() == 1);
+            if (known && in.cp >= 32) kcs.insert(kcs.begin(), f);
+        }
         for (int kco : kcs) {
+            if (getenv("FYNHIP_CONV_KC") && kco != kcs[0] && !cands.empty()) break;
             int kc;
             conv_geometry(in, !net->f16(), (int)sc.taps.size(), kco, kc, pitch, slack, npl);
             const int chunks = (kc == 4) ? 1 : (in.cp + kc - 1) / kc;
@@ -408,10 +419,12 @@ static MfmaLaunch tune_mfma(Net* net, const SubConv& sc, const TView& in, const 
             for (TileChoice& tc : c) {
                 tc.kc = kc;
                 if (kco != kc0) tc.score *= 0.9;
+                if (kc > 128 && tc.wm * tc.wn == 4) continue;
                 if (tc.wm * tc.wn < 4) {   // tiles whose waves split K exist for chunks of 32 and more channels
                     const int wk = 4 / (tc.wm * tc.wn);
+                    const int unr = kc > 128 ? 4 : 2;
                     const int raw = (int)sc.taps.size() * (kc / 16);
-                    if (kc < 32 || (raw + 2 * wk - 1) / (2 * wk) * (2 * wk) > 256) continue;
+                    if (kc < 32 || (raw + unr * wk - 1) / (unr * wk) * (unr * wk) > 256) continue;
                 }
                 cands.push_back(tc);
             }

@@ -143,6 +143,38 @@ def test_tiles_whose_waves_split_k(k, cin, cout, h, w, ksplit, kw, tile, storage
     assert err <= TOL[storage], info
 
 
+@pytest.mark.parametrize("storage", [fa.STORAGE_F32, fa.STORAGE_F16], ids=["f32", "f16"])
+@pytest.mark.parametrize("tile", ["1,1,1,1", "1,1,2,1", "1,1,1,2"], ids=["32x32", "64x32", "32x64"])
+@pytest.mark.parametrize("kc", [256, 512, 1024])
+@pytest.mark.parametrize("cin,cout,h,w,stride,ksplit,kw", [
+    (1024, 96, 7, 7, 1, 0, {"bn": True}),                                   # whole chunks
+    (600, 33, 9, 5, 1, 0, {"residual": (A.RELU, True)}),                    # ragged last chunk, ragged channels and tile
+    (1100, 40, 14, 14, 2, 0, {"bn": True}),                                 # stride 2, more than one chunk at every width
+    (2048, 64, 7, 7, 1, 2, {"residual": (A.NONE, False)}),                  # together with split-K over workgroups
+], ids=["1024ch", "600ch_ragged", "1100ch_s2", "2048ch_ksplit"])
+def test_wide_chunks_on_pointwise_layers(cin, cout, h, w, stride, ksplit, kw, kc, tile, storage, monkeypatch):
+    """1x1 convolutions over many input channels staged 256 to 1024 channels at a time (the tiles whose waves split
+    K), forced through the engine's tile and chunk-width switches."""
+    monkeypatch.setenv("FYNHIP_CONV_TILE", tile)
+    monkeypatch.setenv("FYNHIP_CONV_KC", str(kc))
+    if ksplit:
+        monkeypatch.setenv("FYNHIP_FORCE_KSPLIT", str(ksplit))
+    b = conv_builder(1, cout, h, w, cin, stride, 1, A.RELU, **kw)
+    wts = conv_block(700 + cin, cout, 1, cin, bn=kw.get("bn", False))
+    inputs = [prng.uniform(17 + cin, (cin, h, w), -1, 1)]
+    if "residual" in kw:
+        inputs.append(prng.uniform(29, (cout, (h + stride - 1) // stride, (w + stride - 1) // stride), -1, 1))
+    got, info = run_single(b, storage, inputs, wts)
+    ref = oracle_single(b, storage, inputs, wts)
+    err = rel_l2(got, ref)
+    print("  ", info, "rel_l2=%.3e" % err, flush=True)
+    fm, fn, wm, wn = (int(v) for v in tile.split(","))
+    planes, buffers = (2 if storage == fa.STORAGE_F32 else 1), (2 if cin > kc else 1)
+    if stride == 1 and 1024 + buffers * planes * 32 * fn * wn * (2 * kc + 16) <= 150 * 1024:   # the chunk fits in LDS
+        assert "kc=%d" % kc in info and "waves=%dx%d" % (wm, wn) in info
+    assert err <= TOL[storage], info
+
+
 ALL_TILES = ["2,2,2,2", "2,2,1,4", "2,1,2,2", "2,1,1,4", "1,2,1,4", "1,1,1,4", "1,1,4,1", "1,1,2,2", "1,2,4,1", "1,3,4,1", "1,4,4,1",
              "1,2,2,2", "1,4,2,2", "1,3,2,2", "1,4,1,4", "1,3,1,4", "1,1,1,1", "1,1,2,1", "1,1,1,2"]
 
