@@ -243,7 +243,9 @@ __device__ __forceinline__ void conv_mfma_body(const ConvMfmaParams& p, unsigned
     const int gy0 = pos_y0 * p.in_stride + p.in_y0;
     const int gx0 = pos_x0 * p.in_stride + p.in_x0;
     const float inv_hw = 1.0f / (float)p.halo_w;
-    const int vhp = p.in_hp << p.in_shift, vwp = p.in_wp << p.in_shift;   // frame that gy0/gx0 and the taps count in
+    // frame that gy0/gx0 and the taps count in, and its step and origin in the stored frame
+    const int vhp = p.in_sub ? p.npos_y : p.in_hp << p.in_shift, vwp = p.in_sub ? p.npos_x : p.in_wp << p.in_shift;
+    const int gstep = p.in_sub ? p.in_sub : 1;
     const TIn* in = reinterpret_cast<const TIn*>(p.in);
 
     // LDS holds two staging buffers (double buffering across channel chunks) when there is more
@@ -323,7 +325,7 @@ __device__ __forceinline__ void conv_mfma_body(const ConvMfmaParams& p, unsigned
                 gy = min(max(gy, 0), vhp - 1);
                 gx = min(max(gx, 0), vwp - 1);
             }
-            if ((unsigned)gy < (unsigned)vhp && (unsigned)gx < (unsigned)vwp) g_off[i] = ((gy >> p.in_shift) * p.in_wp + (gx >> p.in_shift)) * p.in_cp;
+            if ((unsigned)gy < (unsigned)vhp && (unsigned)gx < (unsigned)vwp) g_off[i] = (((gy >> p.in_shift) * gstep + p.in_oy) * p.in_wp + (gx >> p.in_shift) * gstep + p.in_ox) * p.in_cp;
         }
     }
     RawItem<TIn, CPI> raw[NB];
@@ -374,7 +376,7 @@ __device__ __forceinline__ void conv_mfma_body(const ConvMfmaParams& p, unsigned
                         gx = min(max(gx, 0), vwp - 1);
                     }
                     if ((unsigned)gy < (unsigned)vhp && (unsigned)gx < (unsigned)vwp && c0 < p.in_cp)
-                        r2[i].load(in + ((gy >> p.in_shift) * p.in_wp + (gx >> p.in_shift)) * p.in_cp + c0);
+                        r2[i].load(in + (((gy >> p.in_shift) * gstep + p.in_oy) * p.in_wp + (gx >> p.in_shift) * gstep + p.in_ox) * p.in_cp + c0);
                 }
             }
 #pragma unroll
@@ -832,6 +834,10 @@ static int check_params(const ConvVariant& v, const ConvMfmaParams& p) {
     if (p.ksplit <= 1 && p.chunks_per_split < p.cin_chunks) return -7;
     if ((1 << p.tile_w_log2) * v.fm < 8) return -10;   // the epilogue's row mapping needs 8 / FM positions of one tile row
     if (v.kc == 4 && p.nsteps > 64) return -5;         // four table entries per step in the 1 KB table
+    // sub-sampled frame: every one of its pixels must be a pixel of the stored frame
+    if (p.in_sub && (p.in_sub < 2 || p.in_stride != 1 || p.in_shift != 0 || p.in_y0 != 0 || p.in_x0 != 0 || p.in_oy < 0 || p.in_ox < 0 ||
+                     (p.npos_y - 1) * p.in_sub + p.in_oy >= p.in_hp || (p.npos_x - 1) * p.in_sub + p.in_ox >= p.in_wp))
+        return -11;
     return 0;
 }
 

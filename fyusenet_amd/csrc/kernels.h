@@ -52,6 +52,10 @@ struct ConvMfmaParams {
     // in_shift = s > 0 (fractional-step convolution): in_y0/in_x0 and the taps count in a virtual frame in which
     // every stored pixel is repeated 2^s times in both directions; virtual coordinate v reads stored pixel v >> s.
     int in_clamp, in_shift;
+    // in_sub = s > 1 (one-tap layers with stride s): the frame the kernel works in is the sub-sampled grid of the
+    // npos_y x npos_x pixels that the layer reads, frame pixel (y, x) being stored pixel (in_oy + y*s, in_ox + x*s);
+    // in_stride is 1 then, so a tile stages only the pixels it uses.  0: the stored frame itself.
+    int in_sub, in_oy, in_ox;
     // output positions computed by this launch
     int npos_y, npos_x;
     // output tensor addressing: stored y = out_off_y + pos_y * out_step

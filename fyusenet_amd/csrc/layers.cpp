@@ -83,6 +83,8 @@ struct SubConv {
     int res_off_y = 0, res_off_x = 0;
     int clamp = 0;     // shallow sampling rule: repeat the frame's edge
     int in_shift = 0;  // fractional-step convolution: coordinates count in the frame repeated 2^in_shift times
+    int in_sub = 0;    // one-tap layer with stride in_sub > 1: the kernel works in the sub-sampled frame (in_stride is 1,
+                       // in_y0/in_x0 are the stored coordinates of its pixel (0,0))
 };
 
 struct MfmaLaunch {
@@ -180,6 +182,10 @@ static MfmaLaunch plan_mfma(Net* net, const SubConv& sc, const TView& in, const 
     p.res = res ? res->ptr : nullptr;
     p.in_hp = in.hp(); p.in_wp = in.wp(); p.in_cp = in.cp;
     p.in_y0 = sc.in_y0; p.in_x0 = sc.in_x0; p.in_stride = sc.in_stride;
+    if (sc.in_sub > 1) {
+        p.in_sub = sc.in_sub; p.in_oy = sc.in_y0; p.in_ox = sc.in_x0;
+        p.in_y0 = p.in_x0 = 0;
+    }
     p.in_clamp = sc.clamp; p.in_shift = sc.in_shift;
     p.npos_y = sc.npos_y; p.npos_x = sc.npos_x;
     p.out_wp = out.wp(); p.out_cp = out.cp; p.out_step = sc.out_step;
@@ -437,8 +443,8 @@ static MfmaLaunch tune_mfma(Net* net, const SubConv& sc, const TView& in, const 
     // FYNHIP_TUNE_CACHE=<file>: measured choices are remembered per problem geometry, so that later
     // processes (e.g. under a profiler, where timing is distorted) pick the same kernels
     char key[160];
-    snprintf(key, sizeof(key), "%d%d:%dx%d:%dx%d:s%d:t%zu:%dx%d:o%d:r%d:cp%d:e%d%d", in.f16, out.f16, cin, cout, sc.npos_y, sc.npos_x,
-             sc.in_stride, sc.taps.size(), sc.span_y, sc.span_x, sc.out_step, res ? 1 : 0, in.cp, sc.clamp, sc.in_shift);
+    snprintf(key, sizeof(key), "%d%d:%dx%d:%dx%d:s%d:t%zu:%dx%d:o%d:r%d:cp%d:e%d%d%d", in.f16, out.f16, cin, cout, sc.npos_y, sc.npos_x,
+             sc.in_stride, sc.taps.size(), sc.span_y, sc.span_x, sc.out_step, res ? 1 : 0, in.cp, sc.clamp, sc.in_shift, sc.in_sub);
     if (tune) {
         int ks = 1;
         const TileChoice* hit = tune_cache_lookup(key, cands, &ks);
@@ -803,6 +809,12 @@ class ConvLayer : public Layer {
                 sc.in_x0 = (in_v.pad << sc.in_shift) + ((k == 3) ? -2 : -r);
             }
             sc.in_stride = stride;
+            if (k == 1 && stride > 1 && !frac_shift && !getenv("FYNHIP_NO_SUBSAMPLED_STAGING")) {
+                // strided pointwise layer: stage the pixels it reads and nothing between them
+                sc.in_sub = stride;
+                sc.in_stride = 1;
+                sc.clamp = 0;   // (every position reads a pixel of the frame)
+            }
             sc.npos_y = oh; sc.npos_x = ow;
             sc.out_step = 1;
             sc.out_off_y = sc.out_off_x = out_v.pad;

@@ -61,6 +61,12 @@ CASES = [
     (9, 3, 12, 3, 32, 1, 1, A.NONE, {}),
     (7, 2, 3, 40, 16, 1, 1, A.RELU, {"bn": True}),
     (5, 64, 9, 9, 3, 2, 2, A.NONE, {}),             # stride and dilation together on a 3-channel input
+    # strided pointwise layers (staged from the sub-sampled frame): odd sizes, stride 3, few channels, padded input, shallow
+    (1, 24, 31, 29, 16, 2, 1, A.RELU, {}),
+    (1, 8, 17, 23, 3, 2, 1, A.NONE, {}),
+    (1, 40, 20, 21, 64, 3, 1, A.RELU, {"bn": True}),
+    (1, 128, 28, 28, 96, 2, 1, A.RELU, {"pad_in": 1, "pad_out": 1, "residual": (A.RELU, True)}),
+    (1, 16, 15, 18, 8, 2, 1, A.RELU, {"deep": False}),
 ]
 
 
