@@ -477,12 +477,12 @@ static MfmaLaunch tune_mfma(Net* net, const SubConv& sc, const TView& in, const 
             best = L;
         }
     }
-    // candidates within a few percent of the winner are measured again over more launches
+    // the winner and the candidates within a few percent of it are measured again over more launches
     {
         std::sort(timed.begin(), timed.end(), [](const std::pair<float, MfmaLaunch>& a, const std::pair<float, MfmaLaunch>& b) { return a.first < b.first; });
         size_t finalists = 1;
         while (finalists < timed.size() && finalists < 4 && timed[finalists].first <= 1.06f * timed[0].first) finalists++;
-        if (finalists > 1) {
+        {
             best_ms = 1e30f;
             for (size_t i = 0; i < finalists; i++) {
                 float ms = 1e30f;
@@ -511,7 +511,9 @@ static MfmaLaunch tune_mfma(Net* net, const SubConv& sc, const TView& in, const 
             if (base.p.cin_chunks < 2 || (ks - 1) * cps >= base.p.cin_chunks || blocks * ks > 1024) break;
             MfmaLaunch L = base;
             set_ksplit(net, L, ks);
-            const float ms = std::min(time_launch(net, L, 4), time_launch(net, L, 4));
+            // (timed like the finalists above: the event pair's share of a short measurement would count against it)
+            float ms = 1e30f;
+            for (int r = 0; r < 3; r++) ms = std::min(ms, time_launch(net, L, 10));
             if (verbose) fprintf(stderr, "[tune] %s -> %.1f us\n", mfma_info(L).c_str(), ms * 1e3f);
             if (ms < best_ms) {
                 best_ms = ms;
