@@ -236,7 +236,7 @@ __device__ __forceinline__ void conv_mfma_body(const ConvMfmaParams& p, unsigned
     const int twl = p.tile_w_log2;
     const int TW = 1 << twl;
     const int pos_y0 = tyi * p.tile_h;
-    const int pos_x0 = txi * TW;
+    const int pos_x0 = txi * (TW - (p.fuse_k ? p.fuse_k - 1 : 0));
 
     const int npix = p.halo_h * p.halo_w;
     const int nitems = npix * G;
@@ -521,6 +521,59 @@ __device__ __forceinline__ void conv_mfma_body(const ConvMfmaParams& p, unsigned
     if constexpr (WK > 1) {
         if (consumer) acc_to_lds();
         __syncthreads();
+    }
+    if constexpr (FM == 1 && WM == 1 && WN == 4) {
+        if (p.fuse_k) {
+            // Folded kx taps: position m of the tile is row m of the transposed accumulators (the four waves' areas
+            // are consecutive), its virtual channels are consecutive floats.  Every thread sums whole outputs.
+            if (consumer) acc_to_lds();
+            __syncthreads();
+            if (!consumer) return;
+            const int K = p.fuse_k, nox = TW - K + 1, ow = p.npos_x - (K - 1);
+            const float* q = reinterpret_cast<const float*>(lds);
+            TOut* outp = reinterpret_cast<TOut*>(p.out);
+            const TOut* resp = reinterpret_cast<const TOut*>(p.res);
+            float sc4[4], bi4[4];
+#pragma unroll
+            for (int o = 0; o < 4; o++) {
+                sc4[o] = o < p.fuse_cout ? p.scale[o] : 0.f;
+                bi4[o] = o < p.fuse_cout ? p.bias[o] : 0.f;
+            }
+            const float inv_nox = 1.0f / (float)nox;
+            for (int idx = tid & 255; idx < p.tile_h * nox; idx += 256) {
+                const int ty = (int)(((float)idx + 0.5f) * inv_nox);
+                const int tx = idx - ty * nox;
+                const int py = pos_y0 + ty, px = pos_x0 + tx;
+                if (py >= p.npos_y || px >= ow) continue;
+                float a[4] = {0.f, 0.f, 0.f, 0.f};
+                const float* row = q + ((ty << twl) + tx) * ROWF;
+                for (int kx = 0; kx < K; kx++) {
+#pragma unroll
+                    for (int o = 0; o < 4; o++)
+                        if (o < p.fuse_cout) a[o] += row[kx * ROWF + o * K + kx];
+                }
+                float rv[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+                if (resp) load_vals<TOut>(resp + ((size_t)(p.res_off_y + py) * p.res_wp + p.res_off_x + px) * p.res_cp, rv, 4);
+                f32x4_t v;
+#pragma unroll
+                for (int o = 0; o < 4; o++) {
+                    float r = rv[o];
+                    if (p.res_relu) r = fmaxf(r, 0.f);
+                    if (p.res_scale) r *= sc4[o];
+                    v[o] = o < p.fuse_cout ? ((a[o] * p.acc_mul) * sc4[o] + bi4[o]) + r : 0.f;
+                }
+                const size_t oidx = ((size_t)(p.out_off_y + py) * p.out_wp + p.out_off_x + px) * p.out_cp;
+                if (sizeof(TOut) == 4) {
+                    *reinterpret_cast<f32x4_t*>(reinterpret_cast<float*>(outp) + oidx) = v;
+                } else {
+                    half4_t hv;
+#pragma unroll
+                    for (int o = 0; o < 4; o++) hv[o] = (_Float16)v[o];
+                    *reinterpret_cast<half4_t*>(reinterpret_cast<_Float16*>(outp) + oidx) = hv;
+                }
+            }
+            return;
+        }
     }
     if (!consumer) return;
     FYN_TRACE(14);
@@ -834,6 +887,11 @@ static int check_params(const ConvVariant& v, const ConvMfmaParams& p) {
     if (p.ksplit <= 1 && p.chunks_per_split < p.cin_chunks) return -7;
     if ((1 << p.tile_w_log2) * v.fm < 8) return -10;   // the epilogue's row mapping needs 8 / FM positions of one tile row
     if (v.kc == 4 && p.nsteps > 64) return -5;         // four table entries per step in the 1 KB table
+    // folded kx taps: one cout block of a 32 x (32*FN*4) tile, no split-K, tile wider than the kernel
+    if (p.fuse_k && (v.fm != 1 || v.wm != 1 || v.wn != 4 || p.cout_blocks != 1 || p.ksplit > 1 || p.fuse_cout < 1 || p.fuse_cout > 4 ||
+                     p.fuse_k * p.fuse_cout > 32 || (1 << p.tile_w_log2) < p.fuse_k || p.out_step != 1 || p.out_cp < 4 ||
+                     p.tiles_x * ((1 << p.tile_w_log2) - p.fuse_k + 1) < p.npos_x - (p.fuse_k - 1)))
+        return -12;
     // sub-sampled frame: every one of its pixels must be a pixel of the stored frame
     if (p.in_sub && (p.in_sub < 2 || p.in_stride != 1 || p.in_shift != 0 || p.in_y0 != 0 || p.in_x0 != 0 || p.in_oy < 0 || p.in_ox < 0 ||
                      (p.npos_y - 1) * p.in_sub + p.in_oy >= p.in_hp || (p.npos_x - 1) * p.in_sub + p.in_ox >= p.in_wp))

@@ -161,6 +161,14 @@ void* Net::dev_alloc(size_t bytes, bool zero) {
     return p;
 }
 
+void Net::dev_free(void* p) {
+    auto it = std::find(allocs_.begin(), allocs_.end(), p);
+    if (it == allocs_.end()) return;
+    FYN_HIP(hipStreamSynchronize(stream));
+    allocs_.erase(it);
+    (void)hipFree(p);
+}
+
 float* Net::staging(size_t floats) {
     if (floats > staging_floats_) {
         FYN_HIP(hipStreamSynchronize(stream));

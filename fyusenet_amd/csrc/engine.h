@@ -120,6 +120,7 @@ class Net {
 
     // device allocations owned by the net
     void* dev_alloc(size_t bytes, bool zero = true);
+    void dev_free(void* p);   // setup-time only (waits for the stream)
     float* staging(size_t floats);  // fp32 staging area for layout conversion
 
   private:

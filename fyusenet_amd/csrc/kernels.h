@@ -81,6 +81,12 @@ struct ConvMfmaParams {
     int ksplit, chunks_per_split;
     float* partial;
     int cout_pad;
+    // fuse_k = K > 0: a K x K convolution with fuse_cout <= 4 output channels whose kx taps are folded into the GEMM's
+    // M dimension (virtual channel o*K + kx, K vertical taps).  Positions are columns of the intermediate
+    // q[y][x'][o*K + kx], x' in [0, W + K - 1); the epilogue sums out[y][x][o] = sum_kx q[y][x + kx][o*K + kx] inside
+    // the tile, so tiles overlap by K - 1 columns (tile column step tile_w - K + 1) and q never leaves LDS.  scale
+    // and bias are indexed by o then; out/res describe the real output.  Tiles with FM = WM = 1, WN = 4 only.
+    int fuse_k, fuse_cout;
 #ifdef FYN_CONV_TRACE
     long long* trace;    // timing-study builds only: 16 timestamps per workgroup
 #endif

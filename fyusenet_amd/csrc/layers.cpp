@@ -83,6 +83,7 @@ struct SubConv {
     int res_off_y = 0, res_off_x = 0;
     int clamp = 0;     // shallow sampling rule: repeat the frame's edge
     int in_shift = 0;  // fractional-step convolution: coordinates count in the frame repeated 2^in_shift times
+    int fuse_k = 0, fuse_cout = 0;   // kx taps folded into the output channels and summed in the epilogue (ConvMfmaParams::fuse_k)
     int in_sub = 0;    // one-tap layer with stride in_sub > 1: the kernel works in the sub-sampled frame (in_stride is 1,
                        // in_y0/in_x0 are the stored coordinates of its pixel (0,0))
 };
@@ -124,6 +125,22 @@ static std::vector<TileChoice> enumerate_tiles(int cout, const SubConv& sc, int 
         conv_mfma_tile(ti, &fm, &fn, &wm, &wn);
         if (force && (fm != ff[0] || fn != ff[1] || wm != ff[2] || wn != ff[3])) continue;
         const int bm = wn * fn * 32;
+        if (sc.fuse_k) {
+            // folded kx taps: one row of 32 virtual channels, four waves along the positions; tiles overlap by K-1
+            // columns, so they are made wide (32 and 64 columns where the image has them)
+            if (fm != 1 || wm != 1 || wn != 4 || cout > 32) continue;
+            for (int tw = 16; tw <= 64; tw *= 2) {
+                if (tw < 2 * sc.fuse_k || tw > bm || (tw > 16 && tw / 2 >= sc.npos_x)) continue;
+                const int th = bm / tw, step = tw - sc.fuse_k + 1;
+                const int tiles = ((sc.npos_x - (sc.fuse_k - 1) + step - 1) / step) * ((sc.npos_y + th - 1) / th);
+                const int halo_w = (tw - 1) * sc.in_stride + sc.span_x, halo_h = (th - 1) * sc.in_stride + sc.span_y;
+                const size_t lds = 1024 + (size_t)nbuf * npl * ((size_t)halo_h * (halo_w * pitch) + slack);
+                if (lds > 150 * 1024) continue;
+                const double util = ((double)sc.npos_x * sc.npos_y) / ((double)tiles * bm);
+                all.push_back(TileChoice{fm, fn, wm, wn, ilog2(tw), th, util, 0, 0});
+            }
+            continue;
+        }
         // (at least 8 columns: the epilogue writes 8 / FM consecutive positions of one tile row per instruction)
         int tw = std::max(8, std::min(bm >= 128 ? 16 : 8, pow2ceil(sc.npos_x)));
         while (bm / tw > pow2ceil(sc.npos_y) && tw < pow2ceil(sc.npos_x) && tw < bm) tw *= 2;
@@ -197,6 +214,11 @@ static MfmaLaunch plan_mfma(Net* net, const SubConv& sc, const TView& in, const 
     p.res_relu = res_relu; p.res_scale = res_scale;
     p.tile_w_log2 = tc.twl; p.tile_h = tc.th;
     p.tiles_x = (sc.npos_x + tw - 1) / tw;
+    if (sc.fuse_k) {
+        p.fuse_k = sc.fuse_k; p.fuse_cout = sc.fuse_cout;
+        const int step = tw - sc.fuse_k + 1;
+        p.tiles_x = (sc.npos_x - (sc.fuse_k - 1) + step - 1) / step;
+    }
     p.tiles_y = (sc.npos_y + tc.th - 1) / tc.th;
     p.halo_w = (tw - 1) * sc.in_stride + sc.span_x;
     p.halo_h = (tc.th - 1) * sc.in_stride + sc.span_y;
@@ -329,13 +351,14 @@ static void set_ksplit(Net* net, MfmaLaunch& L, int ksplit) {
     r.acc_mul = p.acc_mul; r.scale = p.scale; r.bias = p.bias;
 }
 
-static float time_launch(Net* net, const MfmaLaunch& L, int iters) {
+template <typename F>
+static float time_calls(Net* net, F&& call, int iters) {
     hipEvent_t a, b;
     FYN_HIP(hipEventCreate(&a));
     FYN_HIP(hipEventCreate(&b));
-    if (run_mfma(L, net->stream) != 0) fail(FYN_ERR_DEVICE, "convolution launch failed while tuning");
+    call();
     FYN_HIP(hipEventRecord(a, net->stream));
-    for (int i = 0; i < iters; i++) run_mfma(L, net->stream);
+    for (int i = 0; i < iters; i++) call();
     FYN_HIP(hipEventRecord(b, net->stream));
     FYN_HIP(hipEventSynchronize(b));
     FYN_HIP(hipGetLastError());
@@ -344,6 +367,11 @@ static float time_launch(Net* net, const MfmaLaunch& L, int iters) {
     (void)hipEventDestroy(a);
     (void)hipEventDestroy(b);
     return ms / iters;
+}
+static float time_launch(Net* net, const MfmaLaunch& L, int iters) {
+    return time_calls(net, [&]() {
+        if (run_mfma(L, net->stream) != 0) fail(FYN_ERR_DEVICE, "convolution launch failed while tuning");
+    }, iters);
 }
 
 // ---- optional on-disk memory of tuning results (text: "<key> fm fn wm wn kc ksplit" per line) ----
@@ -443,8 +471,8 @@ static MfmaLaunch tune_mfma(Net* net, const SubConv& sc, const TView& in, const 
     // FYNHIP_TUNE_CACHE=<file>: measured choices are remembered per problem geometry, so that later
     // processes (e.g. under a profiler, where timing is distorted) pick the same kernels
     char key[160];
-    snprintf(key, sizeof(key), "%d%d:%dx%d:%dx%d:s%d:t%zu:%dx%d:o%d:r%d:cp%d:e%d%d%d", in.f16, out.f16, cin, cout, sc.npos_y, sc.npos_x,
-             sc.in_stride, sc.taps.size(), sc.span_y, sc.span_x, sc.out_step, res ? 1 : 0, in.cp, sc.clamp, sc.in_shift, sc.in_sub);
+    snprintf(key, sizeof(key), "%d%d:%dx%d:%dx%d:s%d:t%zu:%dx%d:o%d:r%d:cp%d:e%d%d%d:f%d", in.f16, out.f16, cin, cout, sc.npos_y, sc.npos_x,
+             sc.in_stride, sc.taps.size(), sc.span_y, sc.span_x, sc.out_step, res ? 1 : 0, in.cp, sc.clamp, sc.in_shift, sc.in_sub, sc.fuse_k);
     if (tune) {
         int ks = 1;
         const TileChoice* hit = tune_cache_lookup(key, cands, &ks);
@@ -456,7 +484,7 @@ static MfmaLaunch tune_mfma(Net* net, const SubConv& sc, const TView& in, const 
     }
     MfmaLaunch best = plan_mfma(net, sc, in, out, res, cin, cout, act, res_relu, res_scale, cands[0], scale, bias);
     if (const char* fk = getenv("FYNHIP_FORCE_KSPLIT")) {   // testing: fixed split-K factor (clamped to what the layer allows)
-        int ks = atoi(fk);
+        int ks = sc.fuse_k ? 1 : atoi(fk);   // (the fused shift-sum needs the whole reduction in one workgroup)
         while (ks > 1 && (ks - 1) * ((best.p.cin_chunks + ks - 1) / ks) >= best.p.cin_chunks) ks--;
         set_ksplit(net, best, ks);
         return best;
@@ -506,7 +534,7 @@ static MfmaLaunch tune_mfma(Net* net, const SubConv& sc, const TView& in, const 
             }
     for (const MfmaLaunch& base : bases) {
         const int blocks = base.p.tiles_x * base.p.tiles_y * base.p.cout_blocks;
-        for (int ks = 2; ks <= 16 && blocks < 192; ks *= 2) {
+        for (int ks = 2; ks <= 16 && blocks < 192 && !sc.fuse_k; ks *= 2) {
             const int cps = (base.p.cin_chunks + ks - 1) / ks;
             if (base.p.cin_chunks < 2 || (ks - 1) * cps >= base.p.cin_chunks || blocks * ks > 1024) break;
             MfmaLaunch L = base;
@@ -734,6 +762,46 @@ class ConvLayer : public Layer {
         wide = !direct && oc <= 4 && oc * k <= 32 && k >= 3 && stride == 1 && dil == 1 && d.in_channels > 4 &&
                getenv("FYNHIP_NO_WIDE_CONV") == nullptr;
     }
+    // the sub-convolution of the folded form: K vertical taps over the columns of q
+    SubConv wide_subconv() {
+        const TView& in_v = tin(0).v;
+        const int r = (k - 1) / 2;
+        SubConv sc;
+        for (int ky = 0; ky < k; ky++) sc.taps.push_back(Tap{ky, 0, ky, 0});
+        sc.clamp = clamp ? 1 : 0;
+        sc.span_y = k; sc.span_x = 1;
+        sc.in_y0 = in_v.pad - r;
+        sc.in_x0 = in_v.pad - r;
+        if (frac_shift) {   // (the frame of repeated pixels, as in the one-stage form)
+            sc.in_shift = frac_shift - 1;
+            sc.in_y0 = (in_v.pad << sc.in_shift) - r;
+            sc.in_x0 = (in_v.pad << sc.in_shift) + ((k == 3) ? -2 : -r);
+        }
+        sc.in_stride = 1;
+        sc.npos_y = oh; sc.npos_x = ow + k - 1;
+        sc.out_step = 1;
+        sc.out_off_y = sc.out_off_x = 0;
+        return sc;
+    }
+    // q through memory: stage 1 writes it, shift_reduce sums it
+    void setup_two_pass_wide(const TView& in_v, const TView& out_v, const TView* res_v, int res_relu, int res_scale) {
+        qv = TView{};
+        qv.h = oh; qv.w = ow + k - 1; qv.pad = 0; qv.c = oc * k; qv.cp = channel_pitch(oc * k); qv.f16 = out_v.f16;
+        qv.ptr = net->dev_alloc(qv.bytes());
+        SubConv sc = wide_subconv();
+        if (!scale_dev) padded = std::max((oc * k + 127) / 128 * 128, out_v.cp);
+        if (!scale_dev) {
+            scale_dev = static_cast<float*>(net->dev_alloc(padded * sizeof(float)));
+            bias_dev = static_cast<float*>(net->dev_alloc(padded * sizeof(float)));
+        }
+        q_scale_dev = static_cast<float*>(net->dev_alloc(padded * sizeof(float)));
+        q_bias_dev = static_cast<float*>(net->dev_alloc(padded * sizeof(float)));
+        launch = tune_mfma(net, sc, in_v, qv, nullptr, d.in_channels, oc * k, act(), 0, 0, q_scale_dev, q_bias_dev);
+        sr.q = qv; sr.out = out_v; sr.res = res_v ? *res_v : TView{};
+        sr.k = k; sr.cout = oc;
+        sr.scale = scale_dev; sr.bias = bias_dev;
+        sr.res_relu = res_relu; sr.res_scale = res_scale;
+    }
     size_t weight_floats() const override {
         return (size_t)oc + (size_t)oc * k * k * d.in_channels + ((d.flags & FYN_FLAG_POST_BATCHNORM) ? 2 * (size_t)oc : 0);
     }
@@ -766,35 +834,57 @@ class ConvLayer : public Layer {
             padded = out_v.cp;
             wdirect_dev = static_cast<float*>(net->dev_alloc((size_t)k * k * d.in_channels * out_v.cp * sizeof(float)));
         } else if (wide) {
-            // stage 1: q[y][x'][o*K+kx], x' in [0, W+K-1) <-> input column x'-r
-            qv = TView{};
-            qv.h = oh; qv.w = ow + k - 1; qv.pad = 0; qv.c = oc * k; qv.cp = channel_pitch(oc * k); qv.f16 = out_v.f16;
-            qv.ptr = net->dev_alloc(qv.bytes());
-            SubConv sc;
-            for (int ky = 0; ky < k; ky++) sc.taps.push_back(Tap{ky, 0, ky, 0});
-            sc.clamp = clamp ? 1 : 0;
-            sc.span_y = k; sc.span_x = 1;
-            sc.in_y0 = in_v.pad - r;
-            sc.in_x0 = in_v.pad - r;
-            if (frac_shift) {   // (the frame of repeated pixels, as in the one-stage form below)
-                sc.in_shift = frac_shift - 1;
-                sc.in_y0 = (in_v.pad << sc.in_shift) - r;
-                sc.in_x0 = (in_v.pad << sc.in_shift) + ((k == 3) ? -2 : -r);
+            // q[y][x'][o*K+kx], x' in [0, W+K-1) <-> input column x'-r; out[y][x][o] = sum_kx q[y][x+kx][o*K+kx].
+            // One launch when a tile as wide as two kernels fits (q stays in the workgroup's LDS), else q goes through
+            // memory and a second pass sums it.
+            const bool never = getenv("FYNHIP_NO_FUSED_WIDE_CONV") != nullptr, always = getenv("FYNHIP_FORCE_FUSED_WIDE_CONV") != nullptr;
+            MfmaLaunch one;
+            bool have_one = false;
+            if (!never) {
+                SubConv sc = wide_subconv();
+                sc.fuse_k = k; sc.fuse_cout = oc;
+                sc.out_off_y = sc.out_off_x = out_v.pad;
+                if (res_v) sc.res_off_y = sc.res_off_x = res_v->pad;
+                padded = std::max((oc * k + 127) / 128 * 128, out_v.cp);
+                scale_dev = static_cast<float*>(net->dev_alloc(padded * sizeof(float)));
+                bias_dev = static_cast<float*>(net->dev_alloc(padded * sizeof(float)));
+                try {
+                    one = tune_mfma(net, sc, in_v, out_v, res_v, d.in_channels, oc * k, act(), res_relu, res_scale, scale_dev, bias_dev);
+                    have_one = true;
+                } catch (const Error& e) {
+                    if (e.code != FYN_ERR_UNSUPPORTED) throw;   // (no tile fits)
+                }
             }
-            sc.in_stride = 1;
-            sc.npos_y = qv.h; sc.npos_x = qv.w;
-            sc.out_step = 1;
-            sc.out_off_y = sc.out_off_x = 0;
-            padded = std::max((oc * k + 127) / 128 * 128, out_v.cp);
-            scale_dev = static_cast<float*>(net->dev_alloc(padded * sizeof(float)));
-            bias_dev = static_cast<float*>(net->dev_alloc(padded * sizeof(float)));
-            q_scale_dev = static_cast<float*>(net->dev_alloc(padded * sizeof(float)));
-            q_bias_dev = static_cast<float*>(net->dev_alloc(padded * sizeof(float)));
-            launch = tune_mfma(net, sc, in_v, qv, nullptr, d.in_channels, oc * k, act(), 0, 0, q_scale_dev, q_bias_dev);
-            sr.q = qv; sr.out = out_v; sr.res = res_v ? *res_v : TView{};
-            sr.k = k; sr.cout = oc;
-            sr.scale = scale_dev; sr.bias = bias_dev;
-            sr.res_relu = res_relu; sr.res_scale = res_scale;
+            if (have_one && always) {
+                fused = true;
+                launch = one;
+            } else {
+                setup_two_pass_wide(in_v, out_v, res_v, res_relu, res_scale);
+                if (have_one) {
+                    // The one-launch form needs halo rows and columns, i.e. large tiles and few workgroups per CU; which
+                    // form is faster depends on the image size and the storage type, so both are timed.
+                    const char* at = getenv("FYNHIP_AUTOTUNE");
+                    bool pick = out_v.f16 != 0;
+                    if (!(at && at[0] == '0')) {
+                        float t1 = 1e30f, t2 = 1e30f;
+                        for (int rep = 0; rep < 3; rep++) {
+                            t1 = std::min(t1, time_launch(net, one, 10));
+                            t2 = std::min(t2, time_calls(net, [&]() {
+                                run_mfma(launch, net->stream);
+                                launch_shift_reduce(sr, net->stream);
+                            }, 10));
+                        }
+                        if (getenv("FYNHIP_TUNE_VERBOSE")) fprintf(stderr, "[tune] folded kx taps: one launch %.1f us, two passes %.1f us\n", t1 * 1e3f, t2 * 1e3f);
+                        pick = t1 < t2;
+                    }
+                    if (pick) {
+                        fused = true;
+                        launch = one;
+                        net->dev_free(qv.ptr);
+                        qv.ptr = nullptr;
+                    }
+                }
+            }
         } else {
             SubConv sc;
             for (int ky = 0; ky < k; ky++)
@@ -862,8 +952,10 @@ class ConvLayer : public Layer {
                         memcpy(&wv[(((size_t)(o * k + kx)) * k + ky) * cin], &w[(((size_t)o * k + ky) * k + kx) * cin], cin * sizeof(float));
             std::vector<float> ones(padded, 0.f), zeros(padded, 0.f);
             for (int i = 0; i < oc * k; i++) ones[i] = 1.f;
-            reupload(net, q_scale_dev, ones);
-            reupload(net, q_bias_dev, zeros);
+            if (!fused) {
+                reupload(net, q_scale_dev, ones);
+                reupload(net, q_bias_dev, zeros);
+            }
             // the pre-scaling is undone on the way into the intermediate tensor (a power of two: no rounding), so that
             // fp16 storage holds the partial sums at their own magnitude
             launch.p.acc_mul = 1.0f / wmul;
@@ -883,17 +975,18 @@ class ConvLayer : public Layer {
         if (direct) launch_conv_direct(dp, s);
         else if (run_mfma(launch, s) != 0)
             fail(FYN_ERR_DEVICE, "layer %s: convolution launch failed", d.name);
-        if (wide) launch_shift_reduce(sr, s);
+        if (wide && !fused) launch_shift_reduce(sr, s);
     }
     std::string info() const override {
         const std::string mode = frac_shift ? "(fractional step 1/" + std::to_string(1 << (frac_shift - 1)) + ") " : (clamp ? "(edge-clamp) " : "");
         if (direct) return "conv_direct" + mode;
-        return mode + (wide ? "wide-kernel(kx folded into cout)+shift_reduce " + mfma_info(launch) : mfma_info(launch));
+        if (wide) return mode + (fused ? "wide-kernel(kx folded into cout, summed in the epilogue) " : "wide-kernel(kx folded into cout)+shift_reduce ") + mfma_info(launch);
+        return mode + mfma_info(launch);
     }
 
     int k, dil, stride;
     int frac_shift = 0;   // fractional-step convolution: log2(1/sourceStep) + 1
-    bool clamp = false, direct = false, wide = false, have_weights = false;
+    bool clamp = false, direct = false, wide = false, fused = false, have_weights = false;
     int padded = 0;
     std::vector<float> block;
     MfmaLaunch launch;

@@ -181,6 +181,40 @@ def test_wide_chunks_on_pointwise_layers(cin, cout, h, w, stride, ksplit, kw, kc
     assert err <= TOL[storage], info
 
 
+WIDE_CASES = [
+    # k, cout, h, w, cin, kwargs: few output channels under a wide kernel (the kx taps become output channels)
+    (9, 3, 40, 56, 32, {}),
+    (9, 3, 70, 200, 32, {"residual": (A.NONE, False), "pad_out": 1}),      # 64-column tiles, residual, padded output
+    (7, 4, 33, 47, 24, {"bn": True, "residual": (A.RELU, True)}),
+    (5, 2, 19, 90, 40, {"bn": True}),
+    (3, 1, 25, 31, 64, {}),                                                 # two channel chunks
+    (9, 3, 12, 3, 32, {}),                                                  # narrower than the kernel: no tile is wide enough
+]
+
+
+@pytest.mark.parametrize("storage", [fa.STORAGE_F32, fa.STORAGE_F16], ids=["f32", "f16"])
+@pytest.mark.parametrize("two_pass", [False, True], ids=["one_launch", "two_pass"])
+@pytest.mark.parametrize("case", WIDE_CASES, ids=lambda c: "k%d_%dx%dx%d_to%d" % (c[0], c[4], c[2], c[3], c[1]))
+def test_wide_kernel_few_output_channels(case, two_pass, storage, monkeypatch):
+    """Both forms of the folded-kx convolution: partial sums summed inside the workgroup (one launch) and written out
+    and summed by a second pass."""
+    k, cout, h, w, cin, kw = case
+    monkeypatch.setenv("FYNHIP_NO_FUSED_WIDE_CONV" if two_pass else "FYNHIP_FORCE_FUSED_WIDE_CONV", "1")   # (else: whichever is faster)
+    b = conv_builder(k, cout, h, w, cin, 1, 1, A.RELU, **kw)
+    wts = conv_block(800 + k, cout, k, cin, bn=kw.get("bn", False))
+    inputs = [prng.uniform(31 * k + cin, (cin, h, w), -1, 1)]
+    if "residual" in kw:
+        inputs.append(prng.uniform(37, (cout, h, w), -1, 1))
+    got, info = run_single(b, storage, inputs, wts)
+    ref = oracle_single(b, storage, inputs, wts)
+    err = rel_l2(got, ref)
+    print("  ", info, "rel_l2=%.3e" % err, flush=True)
+    assert "wide-kernel" in info
+    one_launch = "summed in the epilogue" in info
+    assert one_launch == (not two_pass and w + k - 1 > 16)
+    assert err <= TOL[storage], info
+
+
 ALL_TILES = ["2,2,2,2", "2,2,1,4", "2,1,2,2", "2,1,1,4", "1,2,1,4", "1,1,1,4", "1,1,4,1", "1,1,2,2", "1,2,4,1", "1,3,4,1", "1,4,4,1",
              "1,2,2,2", "1,4,2,2", "1,3,2,2", "1,4,1,4", "1,3,1,4", "1,1,1,1", "1,1,2,1", "1,1,1,2"]
 
