@@ -374,9 +374,9 @@ static float time_launch(Net* net, const MfmaLaunch& L, int iters) {
     }, iters);
 }
 
-// ---- optional on-disk memory of tuning results (text: "<key> fm fn wm wn kc ksplit" per line) ----
-static std::map<std::string, std::array<int, 6>>& tune_cache() {
-    static std::map<std::string, std::array<int, 6>> cache;
+// ---- optional on-disk memory of tuning results (text: "<key> fm fn wm wn kc ksplit tile_w_log2" per line) ----
+static std::map<std::string, std::array<int, 7>>& tune_cache() {
+    static std::map<std::string, std::array<int, 7>> cache;
     static bool loaded = false;
     if (!loaded) {
         loaded = true;
@@ -384,8 +384,8 @@ static std::map<std::string, std::array<int, 6>>& tune_cache() {
         FILE* f = path ? fopen(path, "r") : nullptr;
         if (f) {
             char k[160];
-            int a, b, c, d, e, g;
-            while (fscanf(f, "%159s %d %d %d %d %d %d", k, &a, &b, &c, &d, &e, &g) == 7) cache[k] = {a, b, c, d, e, g};
+            int a, b, c, d, e, g, h;
+            while (fscanf(f, "%159s %d %d %d %d %d %d %d", k, &a, &b, &c, &d, &e, &g, &h) == 8) cache[k] = {a, b, c, d, e, g, h};
             fclose(f);
         }
     }
@@ -394,7 +394,7 @@ static std::map<std::string, std::array<int, 6>>& tune_cache() {
 
 // switches that pin part of the choice are for experiments: choices are neither remembered nor recalled then
 static bool tune_cache_bypassed() {
-    for (const char* e : {"FYNHIP_FORCE_KSPLIT", "FYNHIP_CONV_TILE", "FYNHIP_CONV_KC_MAX", "FYNHIP_CONV_PD"})
+    for (const char* e : {"FYNHIP_FORCE_KSPLIT", "FYNHIP_CONV_TILE", "FYNHIP_CONV_KC_MAX", "FYNHIP_CONV_KC", "FYNHIP_CONV_PD"})
         if (getenv(e)) return true;
     return false;
 }
@@ -404,22 +404,37 @@ static const TileChoice* tune_cache_lookup(const char* key, const std::vector<Ti
     auto it = tune_cache().find(key);
     if (it == tune_cache().end()) return nullptr;
     for (const TileChoice& c : cands)
-        if (c.fm == it->second[0] && c.fn == it->second[1] && c.wm == it->second[2] && c.wn == it->second[3] && c.kc == it->second[4]) {
+        if (c.fm == it->second[0] && c.fn == it->second[1] && c.wm == it->second[2] && c.wn == it->second[3] && c.kc == it->second[4] &&
+            c.twl == it->second[6]) {
             *ksplit = it->second[5];
             return &c;
         }
     return nullptr;
 }
 
-static void tune_cache_store(const char* key, const ConvVariant& v, int ksplit) {
+static void tune_cache_store(const char* key, const ConvVariant& v, int ksplit, int twl) {
     if (tune_cache_bypassed()) return;
-    tune_cache()[key] = {v.fm, v.fn, v.wm, v.wn, v.kc, ksplit};   // same geometry later in this process: same choice
+    tune_cache()[key] = {v.fm, v.fn, v.wm, v.wn, v.kc, ksplit, twl};   // same geometry later in this process: same choice
     const char* path = getenv("FYNHIP_TUNE_CACHE");
     if (!path) return;
     FILE* f = fopen(path, "a");
     if (!f) return;
-    fprintf(f, "%s %d %d %d %d %d %d\n", key, v.fm, v.fn, v.wm, v.wn, v.kc, ksplit);
+    fprintf(f, "%s %d %d %d %d %d %d %d\n", key, v.fm, v.fn, v.wm, v.wn, v.kc, ksplit, twl);
     fclose(f);
+}
+
+// a measured yes/no choice under a key of its own (same file, the first number is the flag)
+static bool tune_cache_flag(const char* key, bool* flag) {
+    if (tune_cache_bypassed()) return false;
+    auto it = tune_cache().find(key);
+    if (it == tune_cache().end()) return false;
+    *flag = it->second[0] != 0;
+    return true;
+}
+static void tune_cache_store_flag(const char* key, bool flag) {
+    ConvVariant v{};
+    v.fm = flag ? 1 : 0;
+    tune_cache_store(key, v, 0, 0);
 }
 
 // Picks the tile configuration of one (sub-)convolution: by measurement on the layer's own tensors
@@ -549,7 +564,7 @@ static MfmaLaunch tune_mfma(Net* net, const SubConv& sc, const TView& in, const 
             }
         }
     }
-    tune_cache_store(key, best.var, best.p.ksplit);
+    tune_cache_store(key, best.var, best.p.ksplit, best.p.tile_w_log2);
     return best;
 }
 
@@ -654,7 +669,7 @@ static MfmaGroup tune_mfma_group(Net* net, const std::vector<SubConv>& scs, cons
             best = g;
         }
     }
-    tune_cache_store(key, best.var, 1);
+    tune_cache_store(key, best.var, 1, best.subs[0].p.tile_w_log2);
     return best;
 }
 
@@ -865,7 +880,11 @@ class ConvLayer : public Layer {
                     // form is faster depends on the image size and the storage type, so both are timed.
                     const char* at = getenv("FYNHIP_AUTOTUNE");
                     bool pick = out_v.f16 != 0;
-                    if (!(at && at[0] == '0')) {
+                    char key[160];
+                    snprintf(key, sizeof(key), "folded:%d:%dx%d:%dx%d:k%d:cp%d:r%d:e%d%d", out_v.f16, d.in_channels, oc, oh, ow, k, in_v.cp,
+                             res_v ? 1 : 0, clamp ? 1 : 0, frac_shift);
+                    if (tune_cache_flag(key, &pick)) {
+                    } else if (!(at && at[0] == '0')) {
                         float t1 = 1e30f, t2 = 1e30f;
                         for (int rep = 0; rep < 3; rep++) {
                             t1 = std::min(t1, time_launch(net, one, 10));
@@ -876,6 +895,7 @@ class ConvLayer : public Layer {
                         }
                         if (getenv("FYNHIP_TUNE_VERBOSE")) fprintf(stderr, "[tune] folded kx taps: one launch %.1f us, two passes %.1f us\n", t1 * 1e3f, t2 * 1e3f);
                         pick = t1 < t2;
+                        tune_cache_store_flag(key, pick);
                     }
                     if (pick) {
                         fused = true;

@@ -375,3 +375,38 @@ def test_fractional_convolution_rejections():
         run_single(builder(step=0.3), fa.STORAGE_F32, [x], conv_block(1, 4, 3, 4))
     with pytest.raises(fa.FynException, match="not a multiple"):
         run_single(builder(step=1.0, h=7, w=7, stride=2), fa.STORAGE_F32, [np.zeros((4, 7, 7), np.float32)], conv_block(1, 4, 3, 4))
+
+
+_CACHE_CHILD = r"""
+import sys
+sys.path.insert(0, sys.argv[1]); sys.path.insert(0, sys.argv[1] + "/tests")
+import fyusenet_amd as fa
+from fyusenet_amd import prng
+from util import conv_block, run_single
+from test_gpu_conv import conv_builder
+A = fa.ActType
+for k, cout, h, w, cin, stride in ((9, 3, 70, 200, 32, 1), (1, 64, 14, 14, 512, 1), (3, 48, 30, 30, 48, 1), (1, 96, 28, 28, 64, 2)):
+    b = conv_builder(k, cout, h, w, cin, stride, 1, A.RELU)
+    out, info = run_single(b, fa.STORAGE_F16, [prng.uniform(5, (cin, h, w), -1, 1)], conv_block(900 + k, cout, k, cin))
+    print(info, "%.6e" % float(abs(out).sum()))
+"""
+
+
+def test_tuning_choices_are_remembered_across_processes(tmp_path):
+    """FYNHIP_TUNE_CACHE: a second process finds the first one's measured choices (tile, tile width, chunk width, split-K
+    factor) in the file, sets up the same kernels without measuring and adds nothing to the file."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    cache = tmp_path / "tune.txt"
+    env = dict(os.environ, FYNHIP_TUNE_CACHE=str(cache))
+    runs = []
+    for _ in range(2):
+        r = subprocess.run([sys.executable, "-c", _CACHE_CHILD, root], env=env, capture_output=True, text=True, timeout=300)
+        assert r.returncode == 0, r.stderr[-2000:]
+        runs.append((r.stdout, cache.read_text()))
+    assert runs[0][0] == runs[1][0]                      # same kernels, same results
+    assert runs[0][1] == runs[1][1]                      # nothing measured again
+    lines = runs[0][1].splitlines()
+    assert len(lines) >= 4 and all(len(ln.split()) == 8 for ln in lines)
