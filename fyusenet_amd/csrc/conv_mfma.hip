@@ -15,6 +15,10 @@
 // (shaders/activation.inc:3-18 semantics: activation on input fetch).  Epilogue: acc*scale + bias
 // (+ residual), the order of shaders/deep/deepconv3x3_tiled.frag:36-45.
 //
+// Two more sampling and output rules, described at their fields in ConvMfmaParams: strided one-tap layers work in the
+// sub-sampled frame (in_sub), and a K x K convolution with at most four output channels can run with its kx taps
+// folded into the output channels, the epilogue summing them inside the workgroup (fuse_k).
+//
 // fp32 storage: both operands are split into fp16 hi + lo parts (x = hi + lo, 22 significant
 // bits) and three MFMAs (hi*hi, lo*hi, hi*lo) are issued per fragment pair; fp16 storage: one.
 #include <hip/hip_fp16.h>
