@@ -55,14 +55,14 @@ def _drain(procs):
 
 
 def build_cpp_example(verbose=True):
-    """Compiles tests/cpp/reference_style.cpp, a program written against the C++ description surface of
+    """Compiles tests/cpp/surface_example.cpp, a program written against the C++ description surface of
     include/fynhip.hpp, and links it with libfynhip.so (host compiler only; the GPU tests run it)."""
     root = os.path.dirname(HERE)
     outdir = os.path.join(root, "tests", "cpp", "_build")
     os.makedirs(outdir, exist_ok=True)
-    exe = os.path.join(outdir, "reference_style")
+    exe = os.path.join(outdir, "surface_example")
     cmd = [os.environ.get("CXX", "g++"), "-std=c++17", "-O1", "-Wall", "-Wextra", "-I", os.path.join(root, "include"),
-           os.path.join(root, "tests", "cpp", "reference_style.cpp"), "-o", exe, "-L", HERE, "-lfynhip",
+           os.path.join(root, "tests", "cpp", "surface_example.cpp"), "-o", exe, "-L", HERE, "-lfynhip",
            "-Wl,-rpath,$ORIGIN/../../../fyusenet_amd", "-Wl,--allow-shlib-undefined"]
     if verbose:
         print(" ".join(cmd), flush=True)

@@ -211,3 +211,129 @@ def test_deep_tiling_and_layout_round_trips():
         d = O.chw_to_deep(x, pad)
         assert np.array_equal(O.deep_to_chw(d, 23, 6, 5, pad), x)
     assert np.array_equal(O.shallow_to_chw(O.chw_to_shallow(x[:3], 4), 3), x[:3])
+
+
+# ---- leaky ReLU, batch-norm layer with residual, GPU_DEEP layout ----------------------------------
+@pytest.mark.parametrize("leak", [0.1, 0.25, 1.5])
+def test_leaky_relu_on_fetch(leak):
+    # shaders/activation.inc:6-8: sg = step(0, x); out = (sg + leak*(1 - sg)) * x, i.e. x for x >= 0 (step(0,0) = 1)
+    # and leak*x below.  Checked through three oracle entry points that apply the activation while reading.
+    cin, cout, k, h, w = 5, 4, 3, 7, 6
+    x = prng.uniform(40, (cin, h, w), -2, 2)
+    x[0, 0, :3] = (0.0, -0.0, 1e-30)
+    act = (O.ACT_LEAKY, leak, 0.0, 0.0)
+    x64 = x.astype(np.float64)
+    sg = (x64 >= 0).astype(np.float64)
+    shader = (sg + leak * (1.0 - sg)) * x64
+    lib = F.leaky_relu(torch.from_numpy(x64), leak).numpy()
+    assert np.allclose(shader, lib, rtol=0, atol=0)
+    # (1) identity function layer: act(x) itself, to fp32 rounding of leak*x
+    y = O.unary(x, O.FN_COPY, act=act)
+    # (2) batch-norm layer with scale 1, bias 0 is act(x)
+    sb = np.concatenate([np.ones(cin, np.float32), np.zeros(cin, np.float32)])
+    yb = O.batchnorm(x, 0, sb, act=act)
+    assert rel_l2(yb, shader) < 1e-7
+    assert np.array_equal(yb[x >= 0], x[x >= 0])          # the positive side passes unchanged, -0.0 and 0.0 included
+    assert np.all(yb[x < 0] == (np.float32(leak) * x[x < 0]))
+    assert np.array_equal(y, yb)
+    # (3) convolution reading a leaky input == library convolution of the library's leaky_relu
+    block = conv_block(41, cout, k, cin)
+    yc = O.conv2d(O.pad_chw(x, 1), 1, block, cout, k, act=act)
+    ref = F.conv2d(torch.from_numpy(lib)[None], _w_from_block(block, cout, k, cin),
+                   torch.from_numpy(block[:cout].astype(np.float64)), padding=1)[0].numpy()
+    assert rel_l2(yc, ref) < 1e-6
+    # a sign error or a swapped branch would give relu or leak*x everywhere: both differ
+    assert rel_l2(yb, np.maximum(x64, 0)) > 1e-2 and rel_l2(yb, leak * x64) > 1e-2
+
+
+@pytest.mark.parametrize("flags_names", [("RESIDUAL_INPUT",), ("RESIDUAL_INPUT", "RELU_ON_RESIDUAL"),
+                                         ("RESIDUAL_INPUT", "BATCHNORM_ON_RESIDUAL"),
+                                         ("RESIDUAL_INPUT", "RELU_ON_RESIDUAL", "BATCHNORM_ON_RESIDUAL")])
+def test_batchnorm_layer_residual_variants(flags_names):
+    # shaders/deep/deepbatchnorm.frag:26-35: out = act(in)*s + b; r = res; RELU_ON_RESIDUAL: r = max(0, r);
+    # BATCHNORM_ON_RESIDUAL: r = r*s + b (scale AND bias, unlike the convolution's applyBNNB); out += r
+    c, h, w = 7, 5, 6
+    x = prng.uniform(42, (c, h, w), -2, 2)
+    res = prng.uniform(43, (c, h, w), -2, 2)
+    sb = np.concatenate([prng.uniform(44, (c,), 0.5, 1.5), prng.normal(45, (c,))]).astype(np.float32)
+    s, b = sb[:c].astype(np.float64)[:, None, None], sb[c:].astype(np.float64)[:, None, None]
+    flags = 0
+    for n in flags_names:
+        flags |= getattr(O, n)
+    y = O.batchnorm(O.pad_chw(x, 1), 1, sb, act=RELU, flags=flags, residual=res)
+    r = res.astype(np.float64)
+    if "RELU_ON_RESIDUAL" in flags_names:
+        r = np.maximum(r, 0.0)
+    if "BATCHNORM_ON_RESIDUAL" in flags_names:
+        r = r * s + b
+    ref = np.maximum(x.astype(np.float64), 0.0) * s + b + r
+    assert rel_l2(y, ref) < 1e-6
+    # each flag changes the result (a dropped term would pass one of the other parametrisations unchanged)
+    plain = np.maximum(x.astype(np.float64), 0.0) * s + b
+    assert rel_l2(y, plain) > 1e-2
+    if "BATCHNORM_ON_RESIDUAL" in flags_names:
+        assert rel_l2(y, plain + (np.maximum(res, 0) if "RELU_ON_RESIDUAL" in flags_names else res) * s) > 1e-2  # bias is included
+    # the residual flag without a residual tensor and a zero residual without BN-on-residual are the plain layer
+    assert np.array_equal(O.batchnorm(O.pad_chw(x, 1), 1, sb, act=RELU, flags=O.RESIDUAL_INPUT, residual=np.zeros_like(res)),
+                          O.batchnorm(O.pad_chw(x, 1), 1, sb, act=RELU))
+
+
+def _deep_by_tiler(x, pad):
+    """GPU_DEEP buffer written pixel by pixel from the output-tile arithmetic of DeepTiler
+    (gpu/deep/deeptiler.cpp:73-76 viewport, :97-110: tiles in y-outer / x-inner order, tile (x, y) at image
+    coordinates x*(w+pad)+pad, y*(h+pad)+pad), four channels per pixel."""
+    c, h, w = x.shape
+    tiles = (c + 3) // 4
+    tx, ty = O.deep_tiling(c)
+    vw, vh = tx * (w + pad) + pad, ty * (h + pad) + pad
+    buf = np.zeros((vh, vw, 4), np.float32)
+    tilenum = 0
+    for y in range(ty):
+        for xx in range(tx):
+            if tilenum >= tiles:
+                break
+            ox, oy = xx * (w + pad) + pad, y * (h + pad) + pad
+            for l in range(min(4, c - 4 * tilenum)):
+                buf[oy:oy + h, ox:ox + w, l] = x[4 * tilenum + l]
+            tilenum += 1
+    return buf
+
+
+def _chw_by_cpubuffer(src, c, th, tw, tx, ty):
+    """CPUBuffer::deepToChannelWise at padding 0 (cpu/cpubuffer.cpp:424-437) restated index by index: tile
+    (tx, ty) starts at row ty*tileHeight, column tx*tileWidth of a buffer that is shape.width_ = tx_count*tileWidth
+    pixels wide; channels count up over ty-outer / tx-inner tiles.  (The reference multiplies the row index by
+    PIXEL_PACKING twice, `(y*srcstride+x)*PIXEL_PACKING` with srcstride already in elements; the row stride used
+    here is the buffer's actual one, width_*PIXEL_PACKING elements.)"""
+    width = tx * tw
+    flat = src.reshape(-1)
+    out = np.zeros((c, th, tw), np.float32)
+    ch = 0
+    for tyi in range(ty):
+        for txi in range(tx):
+            rem = min(4, c - ch)
+            base = (tyi * th) * width * 4 + (txi * tw) * 4
+            for l in range(max(rem, 0)):
+                for y in range(th):
+                    for xx in range(tw):
+                        out[ch, y, xx] = flat[base + (y * width + xx) * 4 + l]
+                ch += 1
+    return out
+
+
+@pytest.mark.parametrize("c,h,w", [(23, 6, 5), (8, 3, 7), (36, 4, 4), (80, 2, 3), (5, 5, 2)])
+def test_deep_layout_against_tiler_and_cpubuffer_arithmetic(c, h, w):
+    x = prng.uniform(46, (c, h, w), -1, 1)
+    x += np.arange(c, dtype=np.float32)[:, None, None]  # every channel distinct: a swapped tile row/column cannot pass
+    tx, ty = O.deep_tiling(c)
+    for pad in (0, 1):
+        d = O.chw_to_deep(x, pad)
+        ref = _deep_by_tiler(x, pad)
+        assert d.shape == ref.shape == (ty * (h + pad) + pad, tx * (w + pad) + pad, 4)
+        assert np.array_equal(d, ref)
+    # padding 0: the reference's CPU-side reader gives back the tensor from the oracle's buffer, and the oracle's
+    # own reader agrees with it
+    d0 = O.chw_to_deep(x, 0)
+    assert np.array_equal(_chw_by_cpubuffer(d0, c, h, w, tx, ty), x)
+    assert np.array_equal(O.deep_to_chw(d0, c, h, w, 0), x)
+    assert np.array_equal(O.deep_to_chw(_deep_by_tiler(x, 1), c, h, w, 1), x)
