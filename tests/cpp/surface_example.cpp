@@ -83,7 +83,8 @@ class Hourglass : public fn::NeuralNetwork {
             const int h = height_ / r.shrink, w = width_ / r.shrink;
             if (r.kind == UP || r.kind == DOWN) {
                 auto* b = new fn::gpu::UpDownLayerBuilder(r.kind == UP ? fn::gpu::UpDownLayerBuilder::UPLOAD : fn::gpu::UpDownLayerBuilder::DOWNLOAD, r.name);
-                b->shape(r.cout, h, w, r.cin).outputPadding((short)r.padOut).deep().context(context()).number(r.no);
+                b->shape(r.cout, h, w, r.cin).outputPadding((short)r.padOut).context(context()).number(r.no);
+                if (r.kind == DOWN) b->deep();   // uploads are shallow (three channels), the download reads a deep tensor
                 b->push(factory);
                 continue;
             }

@@ -47,7 +47,9 @@ def _python_twin(width, height, stream):
                 h, w = height // shrink, width // shrink
                 if kind in ("up", "down"):
                     b = UpDownLayerBuilder(UpDownLayerBuilder.UPLOAD if kind == "up" else UpDownLayerBuilder.DOWNLOAD, name)
-                    b.shape(cout, h, w, cin).outputPadding(pad_out).deep().number(no)
+                    b.shape(cout, h, w, cin).outputPadding(pad_out).number(no)
+                    if kind == "down":
+                        b.deep()
                 else:
                     b = ConvLayerBuilder(k, name).shape(cout, h, w, cin).deep().inputPadding((k - 1) // 2).outputPadding(pad_out)
                     b.prefixAct(acts[act]).number(no)
