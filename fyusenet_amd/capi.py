@@ -109,6 +109,7 @@ SYMBOLS = {
     "fyn_net_forward": (ctypes.c_int, [_P, ctypes.POINTER(ctypes.c_uint64)]),
     "fyn_net_finish": (ctypes.c_int, [_P]),
     "fyn_layer_copy_result": (ctypes.c_int, [_P, ctypes.c_int, _F, ctypes.c_int]),
+    "fyn_layer_copy_result_noalloc": (ctypes.c_int, [_P, ctypes.c_int, _F, ctypes.c_int]),
     "fyn_layer_output_shape": (ctypes.c_int, [_P, ctypes.c_int] + [ctypes.POINTER(ctypes.c_int)] * 4),
     "fyn_net_get_output": (ctypes.c_int, [_P, ctypes.c_int, _F, ctypes.c_int]),
     "fyn_layer_copy_argmax": (ctypes.c_int, [_P, ctypes.c_int, ctypes.POINTER(ctypes.c_int32), _F]),

@@ -149,6 +149,13 @@ int fyn_layer_copy_result(fyn_net* net, int layer, float* chw, int include_paddi
     FYN_API_END
 }
 
+int fyn_layer_copy_result_noalloc(fyn_net* net, int layer, float* chw, int include_padding) {
+    FYN_API_BEGIN
+    if (!chw) fynhip::fail(FYN_ERR_INVALID, "null output pointer");
+    N(net)->copy_result_static(layer, chw, include_padding);
+    FYN_API_END
+}
+
 int fyn_layer_output_shape(fyn_net* net, int layer, int* channels, int* height, int* width, int* padding) {
     FYN_API_BEGIN
     fynhip::Layer* l = N(net)->layer(layer);

@@ -120,6 +120,31 @@ void return_stream(int device, hipStream_t st) {
 }  // namespace
 
 // ---------------------------------------------------------------------------------------------
+// Fixed staging area for read-backs that must not allocate (Net::copy_result_static).  One array per GPU, part of the
+// loaded code object and held until the process ends.  In host code the array's name is only a handle for
+// hipGetSymbolAddress; the address it yields on each device is what kernels and copies receive.
+// ---------------------------------------------------------------------------------------------
+static __device__ __align__(256) __attribute__((used)) float scratch[FYN_STATIC_SCRATCH_FLOATS];
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mu;
+float* g_scratch_ptr[kMaxDevices] = {};
+
+// The calling thread's current device must be `device`.
+float* static_scratch(int device) {
+    if (device < 0 || device >= kMaxDevices) fail(FYN_ERR_DEVICE, "device %d beyond the %d devices the fixed staging area covers", device, kMaxDevices);
+    std::lock_guard<std::mutex> lk(g_scratch_mu);
+    if (!g_scratch_ptr[device]) {
+        float* p = nullptr;
+        FYN_HIP(hipGetSymbolAddress(reinterpret_cast<void**>(&p), HIP_SYMBOL(scratch)));
+        if (!p) fail(FYN_ERR_DEVICE, "no device address for the fixed staging area on device %d", device);
+        g_scratch_ptr[device] = p;
+    }
+    return g_scratch_ptr[device];
+}
+}  // namespace
+
+// ---------------------------------------------------------------------------------------------
 // Net
 // ---------------------------------------------------------------------------------------------
 Net::Net(int dev, int stor) : device(dev), storage(stor) {
@@ -129,6 +154,8 @@ Net::Net(int dev, int stor) : device(dev), storage(stor) {
     if (dev < 0 || dev >= count) fail(FYN_ERR_DEVICE, "device %d not present (%d devices)", dev, count);
     FYN_HIP(hipSetDevice(dev));
     stream = lease_stream(dev, false);
+    // resolved here, where the caller may still allocate: looking the symbol up loads the code object on this device
+    static_scratch_ = static_scratch(dev);
 }
 
 Net::~Net() {
@@ -465,6 +492,23 @@ void Net::copy_result(int layer_no, float* chw, int include_padding) {
     launch_tensor_to_chw(v, st, include_padding, stream);
     FYN_HIP(hipGetLastError());
     FYN_HIP(hipMemcpyAsync(chw, st, n * sizeof(float), hipMemcpyDeviceToHost, stream));
+    FYN_HIP(hipStreamSynchronize(stream));
+}
+
+void Net::copy_result_static(int layer_no, float* chw, int include_padding) {
+    if (!is_setup) fail(FYN_ERR_STATE, "copy_result() before setup()");
+    if (!chw) fail(FYN_ERR_INVALID, "null result buffer");
+    FYN_HIP(hipSetDevice(device));
+    Layer* l = layer(layer_no);
+    const TView v = result_view(l);
+    const size_t n = include_padding ? (size_t)v.c * v.hp() * v.wp() : (size_t)v.c * v.h * v.w;
+    if (n > (size_t)FYN_STATIC_SCRATCH_FLOATS)
+        fail(FYN_ERR_INVALID, "result of layer %s (%d) has %zu floats, the fixed staging area holds %zu: use fyn_layer_copy_result",
+             l->d.name, l->d.number, n, (size_t)FYN_STATIC_SCRATCH_FLOATS);
+    // every element of [0, n) is written by the conversion kernel: nothing of an earlier call is read
+    launch_tensor_to_chw(v, static_scratch_, include_padding, stream);
+    FYN_HIP(hipGetLastError());
+    FYN_HIP(hipMemcpyAsync(chw, static_scratch_, n * sizeof(float), hipMemcpyDefault, stream));
     FYN_HIP(hipStreamSynchronize(stream));
 }
 

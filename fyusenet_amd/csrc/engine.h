@@ -94,6 +94,7 @@ class Net {
     Layer* layer(int number);
     void set_input(int layer, int port, const float* data, int order);
     void copy_result(int layer, float* chw, int include_padding);
+    void copy_result_static(int layer, float* chw, int include_padding);   // through the fixed staging area, no allocation
     void get_output(int layer, float* data, int order);
     void copy_argmax(int layer, int32_t* idx, float* val);
     void time_forward(int iters, float* ms);
@@ -147,6 +148,7 @@ class Net {
     std::vector<void*> allocs_;
     float* staging_ = nullptr;
     size_t staging_floats_ = 0;
+    float* static_scratch_ = nullptr;   // this device's address of the fixed staging area
     hipGraph_t graph_ = nullptr;
     hipGraphExec_t graph_exec_ = nullptr;
     bool graph_enabled_ = false;

@@ -215,6 +215,16 @@ int fyn_net_finish(fyn_net* net);
 /* GPULayerBase::copyResult(float*, bool) (gpu/gpulayerbase.cpp:525-564): output of `layer` as CHW
  * fp32; include_padding != 0 keeps the output halo.  Synchronises. */
 int fyn_layer_copy_result(fyn_net* net, int layer, float* chw, int include_padding);
+/* fyn_layer_copy_result for callers that cannot allocate (code under HIP graph capture on another stream, tight serving
+ * loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  The layout conversion goes through
+ * a fixed device array of FYN_STATIC_SCRATCH_FLOATS floats that is part of the library's code object (one per GPU, held
+ * until the process ends; its device address is looked up when the network is created) instead of the growable staging
+ * area of fyn_layer_copy_result; no hipMalloc/hipFree is called.  A result with more floats is refused with
+ * FYN_ERR_INVALID.  `chw` may be host memory (pinned memory keeps the HIP runtime from staging the copy itself) or
+ * device memory.  All networks on one GPU share the array: calls that overlap on one GPU (from different threads) race;
+ * every call overwrites all of the part it uses, so nothing of an earlier call is ever read.  Synchronises. */
+#define FYN_STATIC_SCRATCH_FLOATS (8u << 20) /* 32 MiB */
+int fyn_layer_copy_result_noalloc(fyn_net* net, int layer, float* chw, int include_padding);
 /* Output geometry of a layer: channels, height, width (net size) and padding. */
 int fyn_layer_output_shape(fyn_net* net, int layer, int* channels, int* height, int* width, int* padding);
 /* DownloadLayer / CPUBuffer formats (gpu/deep/deepdownloadlayer.cpp:136-162, cpu/cpubuffer.cpp):
