@@ -119,6 +119,9 @@ SYMBOLS = {
     "fyn_net_set_buffer_reuse": (ctypes.c_int, [_P, ctypes.c_int]),
     "fyn_net_use_graph": (ctypes.c_int, [_P, ctypes.c_int]),
     "fyn_net_time_forward": (ctypes.c_int, [_P, ctypes.c_int, _F]),
+    "fyn_net_time_steps": (ctypes.c_int, [_P, ctypes.c_int, _F]),
+    "fyn_net_input_floats": (ctypes.c_int, [_P, ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_size_t)]),
+    "fyn_net_async_sizes": (ctypes.c_int, [_P, ctypes.POINTER(ctypes.c_size_t), ctypes.POINTER(ctypes.c_size_t)]),
     "fyn_layer_time": (ctypes.c_int, [_P, ctypes.c_int, ctypes.c_int, _F]),
     "fyn_net_async_begin": (ctypes.c_int, [_P, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int]),
     "fyn_net_async_submit": (ctypes.c_int, [_P, _F, _F, ctypes.POINTER(ctypes.c_uint64)]),

@@ -99,6 +99,7 @@ int fyn_layer_load_weights(fyn_net* net, int layer, const float* wb, size_t offs
     fynhip::Layer* l = N(net)->layer(layer);
     if (l->d.type == FYN_LAYER_BATCHNORM) fynhip::fail(FYN_ERR_INVALID, "layer %s takes scale/bias, not weights", l->d.name);
     l->load_weights(wb + offset_floats);
+    N(net)->weights_changed();
     FYN_API_END
 }
 
@@ -108,6 +109,7 @@ int fyn_layer_load_scale_bias(fyn_net* net, int layer, const float* sb, size_t o
     fynhip::Layer* l = N(net)->layer(layer);
     if (l->d.type != FYN_LAYER_BATCHNORM) fynhip::fail(FYN_ERR_INVALID, "layer %s is not a batchnorm layer", l->d.name);
     l->load_weights(sb + offset_floats);
+    N(net)->weights_changed();
     FYN_API_END
 }
 
@@ -127,6 +129,13 @@ int fyn_net_setup(fyn_net* net) {
 int fyn_net_set_input(fyn_net* net, int layer, int port, const float* data, int order) {
     FYN_API_BEGIN
     N(net)->set_input(layer, port, data, order);
+    FYN_API_END
+}
+
+int fyn_net_input_floats(fyn_net* net, int layer, int port, size_t* count) {
+    FYN_API_BEGIN
+    if (!count) fynhip::fail(FYN_ERR_INVALID, "null output pointer");
+    *count = N(net)->input_floats(layer, port);
     FYN_API_END
 }
 
@@ -230,6 +239,13 @@ int fyn_net_time_forward(fyn_net* net, int iters, float* ms_total) {
     FYN_API_END
 }
 
+int fyn_net_time_steps(fyn_net* net, int iters, float* ms_each) {
+    FYN_API_BEGIN
+    if (!ms_each || iters < 1) fynhip::fail(FYN_ERR_INVALID, "need an output array and at least one step");
+    N(net)->time_steps(iters, ms_each);
+    FYN_API_END
+}
+
 int fyn_layer_time(fyn_net* net, int layer, int iters, float* ms_total) {
     FYN_API_BEGIN
     if (!ms_total || iters < 1) fynhip::fail(FYN_ERR_INVALID, "invalid arguments");
@@ -246,6 +262,13 @@ int fyn_net_async_begin(fyn_net* net, int in_layer, int in_port, int in_order, i
 int fyn_net_async_submit(fyn_net* net, const float* in, float* out, uint64_t* ticket) {
     FYN_API_BEGIN
     N(net)->async_submit(in, out, ticket);
+    FYN_API_END
+}
+
+int fyn_net_async_sizes(fyn_net* net, size_t* in_floats, size_t* out_floats) {
+    FYN_API_BEGIN
+    if (!in_floats || !out_floats) fynhip::fail(FYN_ERR_INVALID, "null output pointer");
+    N(net)->async_sizes(in_floats, out_floats);
     FYN_API_END
 }
 

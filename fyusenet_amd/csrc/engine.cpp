@@ -196,6 +196,20 @@ void Net::dev_free(void* p) {
     (void)hipFree(p);
 }
 
+void Net::dev_free_many(const std::vector<void*>& ptrs) {
+    bool synced = false;
+    for (void* p : ptrs) {
+        auto it = std::find(allocs_.begin(), allocs_.end(), p);
+        if (it == allocs_.end()) continue;
+        if (!synced) {
+            FYN_HIP(hipStreamSynchronize(stream));
+            synced = true;
+        }
+        allocs_.erase(it);
+        (void)hipFree(p);
+    }
+}
+
 float* Net::staging(size_t floats) {
     if (floats > staging_floats_) {
         FYN_HIP(hipStreamSynchronize(stream));
@@ -448,21 +462,32 @@ void Net::use_graph(bool enable) {
     }
 }
 
+const Tensor& Net::input_tensor(int layer_no, int port) {
+    if (!is_setup) fail(FYN_ERR_STATE, "set_input() before setup()");
+    Layer* l = layer(layer_no);
+    if (l->d.type == FYN_LAYER_UPLOAD) return l->tout();
+    if (port < 0 || port >= l->num_ports()) fail(FYN_ERR_INVALID, "layer %s has no input port %d", l->d.name, port);
+    const Tensor& t = l->tin(port);
+    if (t.producer != -1) fail(FYN_ERR_INVALID, "input port %d of layer %s is fed by layer %d", port, l->d.name, t.producer);
+    return t;
+}
+
+size_t Net::input_floats(int layer_no, int port) {
+    const TView& v = input_tensor(layer_no, port).v;
+    return (size_t)v.c * v.h * v.w;
+}
+
+void Net::async_sizes(size_t* in_floats, size_t* out_floats) const {
+    if (slots_.empty()) fail(FYN_ERR_STATE, "no frame pipeline is active");
+    *in_floats = async_in_floats_;
+    *out_floats = async_out_floats_;
+}
+
 void Net::set_input(int layer_no, int port, const float* data, int order) {
     if (!is_setup) fail(FYN_ERR_STATE, "set_input() before setup()");
     if (!data) fail(FYN_ERR_INVALID, "null input buffer");
     FYN_HIP(hipSetDevice(device));
-    Layer* l = layer(layer_no);
-    const Tensor* t;
-    if (l->d.type == FYN_LAYER_UPLOAD) {
-        t = &l->tout();
-    } else {
-        if (port < 0 || port >= l->num_ports()) fail(FYN_ERR_INVALID, "layer %s has no input port %d", l->d.name, port);
-        t = &l->tin(port);
-        if (t->producer != -1)
-            fail(FYN_ERR_INVALID, "input port %d of layer %s is fed by layer %d", port, l->d.name, t->producer);
-    }
-    const TView& v = t->v;
+    const TView& v = input_tensor(layer_no, port).v;
     const size_t n = (size_t)v.c * v.h * v.w;
     float* st = staging(n);
     FYN_HIP(hipMemcpyAsync(st, data, n * sizeof(float), hipMemcpyHostToDevice, stream));
@@ -584,6 +609,43 @@ void Net::time_forward(int iters, float* ms) {
     FYN_HIP(hipEventElapsedTime(ms, a, b));
     (void)hipEventDestroy(a);
     (void)hipEventDestroy(b);
+}
+
+void Net::time_steps(int iters, float* ms_each) {
+    if (!is_setup) fail(FYN_ERR_STATE, "time_steps() before setup()");
+    if (iters > 65536) fail(FYN_ERR_INVALID, "at most 65536 steps per call");
+    FYN_HIP(hipSetDevice(device));
+    // one event after every forward pass, all queued without waiting; differences of consecutive events are the steps
+    std::vector<hipEvent_t> ev((size_t)iters + 1, nullptr);
+    const bool t = timings;
+    timings = false;
+    try {
+        for (auto& e : ev) FYN_HIP(hipEventCreate(&e));
+        FYN_HIP(hipEventRecord(ev[0], stream));
+        for (int i = 0; i < iters; i++) {
+            forward(nullptr);
+            FYN_HIP(hipEventRecord(ev[(size_t)i + 1], stream));
+        }
+        FYN_HIP(hipEventSynchronize(ev[(size_t)iters]));
+        for (int i = 0; i < iters; i++) FYN_HIP(hipEventElapsedTime(&ms_each[i], ev[(size_t)i], ev[(size_t)i + 1]));
+    } catch (...) {
+        timings = t;
+        (void)hipStreamSynchronize(stream);
+        for (auto e : ev) if (e) (void)hipEventDestroy(e);
+        throw;
+    }
+    timings = t;
+    for (auto e : ev) (void)hipEventDestroy(e);
+}
+
+void Net::weights_changed() {
+    if (!graph_exec_) return;
+    FYN_HIP(hipSetDevice(device));
+    FYN_HIP(hipStreamSynchronize(stream));
+    (void)hipGraphExecDestroy(graph_exec_);
+    (void)hipGraphDestroy(graph_);
+    graph_exec_ = nullptr;
+    graph_ = nullptr;
 }
 
 void Net::time_layer(int layer_no, int iters, float* ms) {

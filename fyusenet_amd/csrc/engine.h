@@ -93,11 +93,18 @@ class Net {
     void finish();
     Layer* layer(int number);
     void set_input(int layer, int port, const float* data, int order);
+    const Tensor& input_tensor(int layer, int port);     // what set_input writes: an upload layer's output or an unconnected port
+    size_t input_floats(int layer, int port);            // floats that set_input reads from the host buffer
+    void async_sizes(size_t* in_floats, size_t* out_floats) const;   // per frame, of the active frame pipeline
     void copy_result(int layer, float* chw, int include_padding);
     void copy_result_static(int layer, float* chw, int include_padding);   // through the fixed staging area, no allocation
     void get_output(int layer, float* data, int order);
     void copy_argmax(int layer, int32_t* idx, float* val);
     void time_forward(int iters, float* ms);
+    void time_steps(int iters, float* ms_each);
+    // A captured forward pass holds kernel arguments by value (among them the power of two that undoes a layer's weight
+    // pre-scaling): after a weight load on a set-up network the next forward() captures again.
+    void weights_changed();
     void time_layer(int layer, int iters, float* ms);
     void use_graph(bool enable);
     // frame pipeline: upload of frame i+1 and download of frame i-1 overlap the layers of frame i
@@ -122,6 +129,7 @@ class Net {
     // device allocations owned by the net
     void* dev_alloc(size_t bytes, bool zero = true);
     void dev_free(void* p);   // setup-time only (waits for the stream)
+    void dev_free_many(const std::vector<void*>& ptrs);   // the same for several areas, one wait
     float* staging(size_t floats);  // fp32 staging area for layout conversion
 
   private:

@@ -194,8 +194,9 @@ void launch_scale_linear(const FuncParams& p, hipStream_t s);
 void launch_nonmax(const TView& in, const TView& out, hipStream_t s);
 // coef: device array [k*k] floats, taps (-r..last)^2 with coefficients in running order
 void launch_blur(const TView& in, const TView& out, const float* coef, int r, int last, hipStream_t s);
-// Copies channels [0, in.c) of `in` to channels [c_off, c_off + in.c) of `out` (activated).
-void launch_concat_part(const TView& in, const TView& out, int c_off, const Act& act, hipStream_t s);
+// Copies channels [0, in.c) of `in` to channels [c_off, c_off + in.c) of `out` (activated); last: also zeroes the pad
+// lanes [c_off + in.c, out.cp).
+void launch_concat_part(const TView& in, const TView& out, int c_off, const Act& act, hipStream_t s, bool last);
 // out: 2 channels (index as float, max value); idx_out optional int32 [h*w].
 void launch_argmax(const TView& in, const TView& out, int32_t* idx_out, const Act& act, hipStream_t s);
 

@@ -7,6 +7,7 @@
 #include <cmath>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 
 #include "engine.h"
 
@@ -375,6 +376,7 @@ static float time_launch(Net* net, const MfmaLaunch& L, int iters) {
 }
 
 // ---- optional on-disk memory of tuning results (text: "<key> fm fn wm wn kc ksplit tile_w_log2" per line) ----
+static std::mutex g_tune_mu;   // guards the map and the file: networks may be set up from several threads
 static std::map<std::string, std::array<int, 7>>& tune_cache() {
     static std::map<std::string, std::array<int, 7>> cache;
     static bool loaded = false;
@@ -401,6 +403,7 @@ static bool tune_cache_bypassed() {
 
 static const TileChoice* tune_cache_lookup(const char* key, const std::vector<TileChoice>& cands, int* ksplit) {
     if (tune_cache_bypassed()) return nullptr;
+    std::lock_guard<std::mutex> lk(g_tune_mu);
     auto it = tune_cache().find(key);
     if (it == tune_cache().end()) return nullptr;
     for (const TileChoice& c : cands)
@@ -414,6 +417,7 @@ static const TileChoice* tune_cache_lookup(const char* key, const std::vector<Ti
 
 static void tune_cache_store(const char* key, const ConvVariant& v, int ksplit, int twl) {
     if (tune_cache_bypassed()) return;
+    std::lock_guard<std::mutex> lk(g_tune_mu);
     tune_cache()[key] = {v.fm, v.fn, v.wm, v.wn, v.kc, ksplit, twl};   // same geometry later in this process: same choice
     const char* path = getenv("FYNHIP_TUNE_CACHE");
     if (!path) return;
@@ -426,6 +430,7 @@ static void tune_cache_store(const char* key, const ConvVariant& v, int ksplit, 
 // a measured yes/no choice under a key of its own (same file, the first number is the flag)
 static bool tune_cache_flag(const char* key, bool* flag) {
     if (tune_cache_bypassed()) return false;
+    std::lock_guard<std::mutex> lk(g_tune_mu);
     auto it = tune_cache().find(key);
     if (it == tune_cache().end()) return false;
     *flag = it->second[0] != 0;
@@ -437,8 +442,10 @@ static void tune_cache_store_flag(const char* key, bool flag) {
     tune_cache_store(key, v, 0, 0);
 }
 
-// Picks the tile configuration of one (sub-)convolution: by measurement on the layer's own tensors
-// (default; timing does not depend on the data), or by the heuristic score when FYNHIP_AUTOTUNE=0.
+// Picks the tile configuration of one (sub-)convolution: by measurement on the layer's own tensors (default), or by
+// the heuristic score when FYNHIP_AUTOTUNE=0.  Candidates are timed before the weights are packed, i.e. on zero
+// operands; the matrix pipes run about a tenth faster on those than on real data (the part holds a higher clock when
+// fewer operand bits toggle), for all candidates alike, so the ranking carries over while the figures do not.
 static MfmaLaunch tune_mfma(Net* net, const SubConv& sc, const TView& in, const TView& out, const TView* res, int cin,
                             int cout, const Act& act, int res_relu, int res_scale, const float* scale, const float* bias) {
     // candidates: every tile that fits, for the geometry's default chunk width, where that is wider than 32
@@ -493,6 +500,9 @@ static MfmaLaunch tune_mfma(Net* net, const SubConv& sc, const TView& in, const 
         const TileChoice* hit = tune_cache_lookup(key, cands, &ks);
         if (hit) {
             MfmaLaunch L = plan_mfma(net, sc, in, out, res, cin, cout, act, res_relu, res_scale, *hit, scale, bias);
+            // a remembered split factor is held to what this layer allows, like a forced one
+            if (sc.fuse_k || ks < 1) ks = 1;
+            while (ks > 1 && ((ks - 1) * ((L.p.cin_chunks + ks - 1) / ks) >= L.p.cin_chunks || ks > 16)) ks--;
             set_ksplit(net, L, ks);
             return L;
         }
@@ -540,6 +550,7 @@ static MfmaLaunch tune_mfma(Net* net, const SubConv& sc, const TView& in, const 
     }
     // few workgroups and several channel chunks: try splitting the reduction over more workgroups (for the
     // winner and, if its waves already split K inside the workgroup, also for the best tile that does not)
+    std::vector<MfmaLaunch> trials;   // split-K variants that were timed
     std::vector<MfmaLaunch> bases{best};
     if (best.var.wm * best.var.wn < 4)
         for (const auto& t : timed)
@@ -554,6 +565,7 @@ static MfmaLaunch tune_mfma(Net* net, const SubConv& sc, const TView& in, const 
             if (base.p.cin_chunks < 2 || (ks - 1) * cps >= base.p.cin_chunks || blocks * ks > 1024) break;
             MfmaLaunch L = base;
             set_ksplit(net, L, ks);
+            trials.push_back(L);
             // (timed like the finalists above: the event pair's share of a short measurement would count against it)
             float ms = 1e30f;
             for (int r = 0; r < 3; r++) ms = std::min(ms, time_launch(net, L, 10));
@@ -565,6 +577,18 @@ static MfmaLaunch tune_mfma(Net* net, const SubConv& sc, const TView& in, const 
         }
     }
     tune_cache_store(key, best.var, best.p.ksplit, best.p.tile_w_log2);
+    // the losing candidates' device buffers (step tables, weight buffers of their own, split-K partial sums) go back
+    {
+        std::vector<void*> drop;
+        auto consider = [&](const MfmaLaunch& L) {
+            for (void* q : {static_cast<void*>(L.aoff_dev), L.wpack_dev, static_cast<void*>(L.p.partial)})
+                if (q && q != best.aoff_dev && q != best.wpack_dev && q != best.p.partial && std::find(drop.begin(), drop.end(), q) == drop.end())
+                    drop.push_back(q);
+        };
+        for (const auto& t : timed) consider(t.second);
+        for (const MfmaLaunch& L : trials) consider(L);
+        net->dev_free_many(drop);
+    }
     return best;
 }
 
@@ -1490,7 +1514,7 @@ class ConcatLayer : public Layer {
         }
         int off = 0;
         for (int i = 0; i < d.num_inputs; i++) {
-            launch_concat_part(tin(i).v, tout().v, off, a, s);
+            launch_concat_part(tin(i).v, tout().v, off, a, s, i == d.num_inputs - 1);
             off += d.inputs[i].channels;
         }
     }

@@ -681,7 +681,7 @@ void launch_addsub(const TView& a, const TView& b, const TView& out, int sub, co
 // Channel offsets that are not multiples of the vector width (the "component shift" case of deepconcat.frag) are
 // handled per element; aligned offsets move whole vectors.
 template <typename T, int V>
-__global__ __launch_bounds__(256) void concat_kernel(const TView in, const TView out, int c_off, const Act act) {
+__global__ __launch_bounds__(256) void concat_kernel(const TView in, const TView out, int c_off, const Act act, int zero_to) {
     const int cg = (in.c + V - 1) / V;
     const size_t n = (size_t)out.h * out.w * cg;
     const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
@@ -697,12 +697,17 @@ __global__ __launch_bounds__(256) void concat_kernel(const TView in, const TView
     } else {
         for (int i = 0; i < V && c + i < in.c; i++) dst[i] = (T)act1((float)src[i], act);
     }
+    // last part: the pad lanes behind the last real channel are written as zero (the buffer may have held another tensor)
+    if (g == cg - 1) {
+        T* px = reinterpret_cast<T*>(out.ptr) + tv_off(out, y, x);
+        for (int i = c_off + in.c; i < zero_to; i++) px[i] = (T)0.f;
+    }
 }
-void launch_concat_part(const TView& in, const TView& out, int c_off, const Act& act, hipStream_t s) {
+void launch_concat_part(const TView& in, const TView& out, int c_off, const Act& act, hipStream_t s, bool last) {
     const bool wide = (in.cp % 8 == 0) && (out.cp % 8 == 0);
     const int v = (out.f16 && wide) ? 8 : 4;
     const size_t n = (size_t)out.h * out.w * ((in.c + v - 1) / v);
-    FYN_DISPATCH_TV(out.f16, wide, concat_kernel, grid1d(n, 256), dim3(256), s, in, out, c_off, act);
+    FYN_DISPATCH_TV(out.f16, wide, concat_kernel, grid1d(n, 256), dim3(256), s, in, out, c_off, act, last ? out.cp : 0);
 }
 
 // ---------------------------------------------------------------------------------------------

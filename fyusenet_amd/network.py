@@ -70,6 +70,10 @@ class Layer:
 
     def setInput(self, data, port=0, order=capi.ORDER_CHANNELWISE):
         data = np.ascontiguousarray(data, dtype=np.float32)
+        want = ctypes.c_size_t(0)
+        capi.check(capi.lib().fyn_net_input_floats(self._net._h, self.number, port, ctypes.byref(want)))
+        if data.size != want.value:
+            raise capi.FynException(capi.ERR_INVALID, "input of layer %s, port %d, takes %d floats, the buffer holds %d" % (self.name, port, want.value, data.size))
         capi.check(capi.lib().fyn_net_set_input(self._net._h, self.number, port, capi.fptr(data), order))
 
     def kernelInfo(self):
@@ -281,6 +285,12 @@ class NeuralNetwork:
     def useGraph(self, enable=True):
         capi.check(capi.lib().fyn_net_use_graph(self._h, 1 if enable else 0))
 
+    def timeSteps(self, iters):
+        """GPU time of each of `iters` forward passes queued back to back (events on the network's stream), ms."""
+        ms = np.zeros(iters, np.float32)
+        capi.check(capi.lib().fyn_net_time_steps(self._h, iters, capi.fptr(ms)))
+        return ms
+
     def timeForward(self, iters):
         ms = ctypes.c_float(0)
         capi.check(capi.lib().fyn_net_time_forward(self._h, iters, ctypes.byref(ms)))
@@ -291,20 +301,37 @@ class NeuralNetwork:
         """copyStreams=False queues uploads and downloads on the network's own stream (for networks that run side by
         side, see FramePool)."""
         capi.check(capi.lib().fyn_net_async_begin(self._h, inLayer, inPort, inOrder, outLayer, outOrder, depth, 1 if copyStreams else 0))
+        a, b = ctypes.c_size_t(0), ctypes.c_size_t(0)
+        capi.check(capi.lib().fyn_net_async_sizes(self._h, ctypes.byref(a), ctypes.byref(b)))
+        self._async_sizes = (a.value, b.value)
+        self._async_outs = {}   # ticket -> output array, kept alive until the engine has written it
 
     def asyncSubmit(self, frame, out):
         """Queues one frame; `out` (a C-contiguous float32 array) is filled once asyncWait(ticket) has returned."""
         frame = np.ascontiguousarray(frame, dtype=np.float32)
-        assert out.dtype == np.float32 and out.flags["C_CONTIGUOUS"]
+        if not (isinstance(out, np.ndarray) and out.dtype == np.float32 and out.flags["C_CONTIGUOUS"] and out.flags["WRITEABLE"]):
+            raise capi.FynException(capi.ERR_INVALID, "the output buffer must be a writable C-contiguous float32 array")
+        n_in, n_out = getattr(self, "_async_sizes", (None, None))
+        if n_in is None:
+            raise capi.FynException(capi.ERR_STATE, "no frame pipeline is active")
+        if frame.size != n_in or out.size != n_out:
+            raise capi.FynException(capi.ERR_INVALID, "a frame takes %d floats in and %d out, the buffers hold %d and %d" % (n_in, n_out, frame.size, out.size))
         t = ctypes.c_uint64(0)
         capi.check(capi.lib().fyn_net_async_submit(self._h, capi.fptr(frame), capi.fptr(out), ctypes.byref(t)))
+        self._async_outs[t.value] = out
+        for old in [k for k in self._async_outs if k + 8 < t.value]:   # delivered when their slot was reused (depth <= 8)
+            del self._async_outs[old]
         return t.value
 
     def asyncWait(self, ticket):
         capi.check(capi.lib().fyn_net_async_wait(self._h, ticket))
+        for t in [k for k in self._async_outs if k <= ticket]:
+            del self._async_outs[t]
 
     def asyncEnd(self):
         capi.check(capi.lib().fyn_net_async_end(self._h))
+        self._async_outs = {}
+        self._async_sizes = (None, None)
 
     def describe(self):
         """Plain description of the graph (descs, edges, loaded weight blocks) for external checkers."""

@@ -190,7 +190,8 @@ int fyn_net_connect(fyn_net* net, int out_layer, int in_layer, int port);
 
 /* ConvLayerInterface::loadWeightsAndBiases(const float*, size_t offset) (base/convlayerinterface.h:95):
  * block at wb+offset = [bias][weights [o][ky][kx][i]][bnScale][bnBias].  May be called again after
- * setup to swap weights (samples/samplenetworks/stylenet3x3.cpp:81-89). */
+ * setup to swap weights (samples/samplenetworks/stylenet3x3.cpp:81-89); a captured forward pass (fyn_net_use_graph) is
+ * captured again on the next fyn_net_forward. */
 int fyn_layer_load_weights(fyn_net* net, int layer, const float* wb, size_t offset_floats);
 /* BatchNormInterface::loadScaleAndBias (base/batchnorminterface.h:146): [scale C][bias C]. */
 int fyn_layer_load_scale_bias(fyn_net* net, int layer, const float* sb, size_t offset_floats);
@@ -205,6 +206,9 @@ int fyn_net_setup(fyn_net* net);
  * for the UPLOAD layer `layer`; for any other layer: writes the tensor on input port `port`
  * directly (what LayerTestBase::generateTextures does, unit_tests/layertestbase.cpp:208-417). */
 int fyn_net_set_input(fyn_net* net, int layer, int port, const float* data, int order);
+/* Number of floats fyn_net_set_input reads from `data` for that layer and port (channels x height x width; the size
+ * the CPUBuffer handed to UploadLayer::setInputBuffer must have). */
+int fyn_net_input_floats(fyn_net* net, int layer, int port, size_t* count);
 
 /* NeuralNetwork::forward (base/neuralnetwork.cpp:173-187): runs all layers in ascending number on
  * the network's stream; returns the sequence number used.  Asynchronous w.r.t. the host. */
@@ -253,6 +257,9 @@ int fyn_net_use_graph(fyn_net* net, int enable);
  * network's stream; per-layer variant times one layer's kernels alone.  Milliseconds total. */
 int fyn_net_time_forward(fyn_net* net, int iters, float* ms_total);
 int fyn_layer_time(fyn_net* net, int layer, int iters, float* ms_total);
+/* `iters` forward passes queued back to back with an event after each; ms_each[i] receives the GPU time between the
+ * events around pass i (for medians and percentiles). */
+int fyn_net_time_steps(fyn_net* net, int iters, float* ms_each);
 /* Frame pipeline for streams of frames handed over in host memory -- the reference engine's asynchronous mode
  * (fyusenet/base/engine.cpp:386-683, two upload/download buffer sets: gpu/uploadlayer.h:74).  The upload of frame
  * i+1 and the download of frame i-1 overlap the layers of frame i (pinned staging buffers, three streams).
@@ -268,6 +275,8 @@ int fyn_layer_time(fyn_net* net, int layer, int iters, float* ms_total);
 int fyn_net_async_begin(fyn_net* net, int in_layer, int in_port, int in_order, int out_layer, int out_order, int depth, int copy_streams);
 int fyn_net_async_submit(fyn_net* net, const float* in, float* out, uint64_t* ticket);
 int fyn_net_async_wait(fyn_net* net, uint64_t ticket);
+/* Floats per frame that submit reads from `in` and writes to `out` (between begin and end). */
+int fyn_net_async_sizes(fyn_net* net, size_t* in_floats, size_t* out_floats);
 int fyn_net_async_end(fyn_net* net);
 /* Text description of the kernel variant chosen for a layer (for profiles / reports). */
 int fyn_layer_kernel_info(fyn_net* net, int layer, char* buf, size_t buflen);
