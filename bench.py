@@ -1,13 +1,15 @@
 #!/usr/bin/env python3
 """Benchmark of the GPU layer stack on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload stylenet|resnet50|resnet50ref|stylenet3x3ref|stylenet9x9ref|conv1|mobilenet|stylenet9x9|copy|bw-<layer>]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload stylenet|resnet50|resnet50ref|stylenet3x3ref|stylenet9x9ref|conv1|mobilenet|stylenet9x9|resconv|resconv-res|copy|bw-<layer>]
 
 A step is one forward pass of the named network over one synthetic input frame that is already
-resident in HBM (uploaded before the timed region); weights are synthetic (random init).  Prints ONE
-JSON line on stdout; progress goes to stderr.  The default workload is BASELINE.json configs[1], the
-Johnson style-transfer net at 512x624 in fp32 storage; ResNet-50 imgs/s is measured in the same run and
-reported under "also".
+resident in HBM (uploaded before the timed region); weights are synthetic (random init).  Steps are
+timed with HIP events on the network's stream (one after every pass; mean, median, p10, p90), between
+two host synchronisations.  Prints ONE JSON line on stdout; progress goes to stderr.  The default
+workload is BASELINE.json configs[1], the Johnson style-transfer net at 512x624 in fp32 storage; the
+other BASELINE configurations (ResNet-50 imgs/s first) are measured in the same run and reported under
+"also", each with a roofline record of its own.
 """
 import argparse
 import json
@@ -25,8 +27,6 @@ from fyusenet_amd import networks  # noqa: E402
 
 PEAK_MFMA_F16_TFLOPS = 2500.0   # MI355X dense fp16/bf16 matrix peak
 PEAK_HBM_GBS = 8000.0           # MI355X HBM3E
-# (layer type, kernel, cin, cout, h, w) -> measured HBM bytes per launch (fetch + write), fp32 storage
-MEASURED_TRAFFIC = {(6, 3, 128, 128, 156, 128): 27.13e6 + 10.22e6}  # launches with the fused residual read
 
 
 def log(*a):
@@ -51,8 +51,9 @@ def make_net(workload):
         return networks.MobileNetV2(fa.STORAGE_F16), "MobileNetV2 224x224 imgs/s", "imgs/s", "fp16 storage"
     if workload == "conv1":
         return networks.SingleConvNet(fa.STORAGE_F32), "conv3x3 64->64 256x256 us/layer", "us", "fp32 storage"
-    if workload == "resconv":  # the style net's dominant layer on its own (for counter runs)
-        return networks.SingleConvNet(fa.STORAGE_F32, channels=128, width=128, height=156), "conv3x3 128->128 128x156 us/layer", "us", "fp32 storage"
+    if workload in ("resconv", "resconv-res"):  # the style net's dominant layer on its own (for counter runs), without / with the fused residual add
+        return (networks.SingleConvNet(fa.STORAGE_F32, channels=128, width=128, height=156, residual=workload.endswith("-res")),
+                "conv3x3 128->128 128x156 us/layer", "us", "fp32 storage")
     if workload == "copy":
         return CopyNet(fa.STORAGE_F32), "copy 64x1024x1024 fp32 GB/s", "GB/s", "fp32"
     if workload.startswith("bw-"):   # one bandwidth-bound layer at a size far beyond the caches
@@ -154,78 +155,156 @@ class CopyNet(fa.NeuralNetwork):
         self.layers[1].setInput(x, 0)
 
 
-def conv_work(b):
-    """Algorithmic FLOPs and bytes of one convolution-type layer: flops = 2*Hout*Wout*Cout*Cin*K^2
-    (transposed: input pixels); bytes = s*(in + out [+ residual]) + s*(weights + 2*Cout), halo and
-    channel padding excluded."""
-    k = getattr(b, "kernel_", 1)
+def layer_work(b, storage_bytes):
+    """Algorithmic work of one layer: (flops, bytes, matrix passes).  Convolutions: flops = 2*Hout*Wout*Cout*Cin*K^2
+    (depthwise: 2*Hout*Wout*C*K^2; transposed: input pixels; fully connected: 2*Cin*Cout), bytes = s*(in + out
+    [+ residual]) + s*(weights + 2*Cout); every other layer moves s*(in + out) and its flops are ignored.  Halo and
+    channel padding are excluded.  passes: fp16 MFMAs issued per algorithmic multiply-add pair (3 with fp32 storage, the
+    hi/lo operand split; 1 with fp16 storage; 0 for layers that do not use the matrix pipes)."""
     t = int(b.type_)
+    k = getattr(b, "kernel_", 1)
     cin, cout, h, w = b.inputChannels_, b.outputChannels_, b.height_, b.width_
-    if t == int(fa.LayerType.TRANSCONVOLUTION2D):
+    res = 1 if int(b.getFlags()) & 1 else 0
+    s = storage_bytes
+    LT = fa.LayerType
+    if t == int(LT.TRANSCONVOLUTION2D):
         ho, wo = 2 * h + k - 2 - b.transconvCrop_, 2 * w + k - 2 - b.transconvCrop_
-        flops = 2.0 * h * w * cout * cin * k * k
-    else:
+        return 2.0 * h * w * cout * cin * k * k, s * (cin * h * w + cout * ho * wo + cout * cin * k * k + 2 * cout), (3 if s == 4 else 1)
+    if t in (int(LT.CONVOLUTION2D), int(LT.FRACCONVOLUTION2D)):
         ho, wo = h // b.downsample_[1], w // b.downsample_[0]
-        flops = 2.0 * ho * wo * cout * cin * k * k
-    return flops, (cin * h * w, cout * ho * wo, cout * cin * k * k + 2 * cout)
+        if t == int(LT.FRACCONVOLUTION2D):
+            step = b.sourceStep_ if getattr(b, "sourceStep_", 0) else 1.0
+            ho, wo = int(h / (step * b.downsample_[1])), int(w / (step * b.downsample_[0]))
+        if getattr(b, "groupSize_", 1) != 1:   # depthwise: vector ALUs, bandwidth-bound
+            return 2.0 * ho * wo * cout * k * k, s * (cin * h * w + (1 + res) * cout * ho * wo) + 4 * (cout * k * k + 2 * cout), 0
+        return 2.0 * ho * wo * cout * cin * k * k, s * (cin * h * w + (1 + res) * cout * ho * wo + cout * cin * k * k + 2 * cout), (3 if s == 4 else 1)
+    if t == int(LT.GEMM):
+        return 2.0 * cin * cout, s * (cin + cout + cin * cout + cout), 0
+    # pooling, batch-norm, add/sub, concat, arg-max and the function layers: elements in + elements out
+    n_in = cin * h * w
+    if t in (int(LT.ADD), int(LT.SUB)):
+        n_in *= 2
+    if t == int(LT.CONCAT):
+        n_in = sum(c for c, _p, _f in getattr(b, "inputs_", [])) * h * w or n_in
+    ho, wo = h, w
+    if t in (int(LT.MAXPOOL2D), int(LT.AVGPOOL2D)):
+        ho, wo = (1, 1) if getattr(b, "global_", False) else (h // b.downsample_[1], w // b.downsample_[0])
+    if t == int(LT.SCALE2D):
+        ho, wo = h * b.upsample_[1] // b.downsample_[1], w * b.upsample_[0] // b.downsample_[0]
+    if t == int(LT.ARGMAX):
+        cout = 2
+    return 0.0, s * (n_in + (1 + res) * cout * ho * wo), 0
+
+
+def conv_work(b):
+    """(flops, bytes) of a convolution-type layer at fp32 storage (for totals)."""
+    f, by, _ = layer_work(b, 4)
+    return f, by
+
+
+def launches_of(info):
+    """Kernel launches a layer's forward() makes, from its kernel description."""
+    n = 1
+    if "+shift_reduce" in info:
+        n += 1
+    if "ksplit=" in info and int(info.split("ksplit=")[1].split()[0]) > 1:
+        n += 1
+    return n
+
+
+def step_stats(ms_each):
+    a = np.sort(np.asarray(ms_each, dtype=np.float64))
+    return {"mean": float(a.mean()), "median": float(np.median(a)), "p10": float(np.percentile(a, 10)), "p90": float(np.percentile(a, 90))}
 
 
 def timed_forwards(net, steps, warmup, graph=True):
+    """W untimed and K timed forward passes, queued back to back on the network's stream with a HIP event after each
+    (fyn_net_time_steps), between two host synchronisations.  Returns the per-step statistics in ms; `mean` is the
+    K steps' total GPU time / K, `wall` the host clock over the same region / K."""
     net.useGraph(graph)
-    for _ in range(warmup):
-        net.forward()
+    if warmup > 0:
+        net.timeSteps(warmup)
     net.finish()
     t0 = time.perf_counter()
-    for _ in range(steps):
-        net.forward()
+    ms_each = net.timeSteps(steps)
     net.finish()
-    return (time.perf_counter() - t0) * 1e3 / steps
+    wall = (time.perf_counter() - t0) * 1e3 / steps
+    st = step_stats(ms_each)
+    st["wall"] = wall
+    return st
 
 
-def dominant_conv_roofline(net, storage_bytes):
-    """Times every layer's kernel(s) alone with HIP events on the network's stream and returns the
-    roofline record of the layer class that takes the most time (identical-shape layers pooled)."""
+def load_traffic():
+    """HBM bytes per launch measured with rocprofv3 (FETCH_SIZE / WRITE_SIZE scaled by a copy kernel), keyed by the
+    kernel description: the lines of profiles/hbm_traffic.txt, written by `python -m fyusenet_amd.rocprof_summary`."""
+    path = os.path.join(ROOT, "profiles", "hbm_traffic.txt")
+    table = {}
+    if os.path.exists(path):
+        for line in open(path):
+            if line.startswith("#") or not line.strip():
+                continue
+            parts = line.rstrip("\n").split("\t")
+            if len(parts) >= 4:
+                table[(parts[3], parts[0])] = float(parts[1]) + float(parts[2])
+    return table
+
+
+def roofline_records(net, storage_bytes, iters=20):
+    """Times every layer's kernel(s) alone (HIP events on the network's stream, `iters` launches captured in one graph)
+    and prices each against max(t_mem, t_flop) at MI355X's published peaks.  Returns (record of the layer class that
+    takes the most time, network-wide record, per-class table)."""
+    traffic = load_traffic()
     groups = {}
+    LT = fa.LayerType
     for lyr in net.layers:
-        t = int(lyr.builder.type_)
-        if t in (int(fa.LayerType.UPLOAD), int(fa.LayerType.DOWNLOAD)):
-            continue
-        iters = 20
-        lyr.timeKernel(3)
-        ms = lyr.timeKernel(iters)            # launches back to back in one hipGraph (dispatch gaps included)
         b = lyr.builder
-        key = (t, getattr(b, "kernel_", 0), b.inputChannels_, b.outputChannels_, b.height_, b.width_, tuple(b.downsample_),
-               bool(int(b.getFlags()) & 1))
-        g = groups.setdefault(key, {"ms": 0.0, "n": 0, "layer": lyr})
+        t = int(b.type_)
+        if t in (int(LT.UPLOAD), int(LT.DOWNLOAD)):
+            continue
+        lyr.timeKernel(3)
+        ms = lyr.timeKernel(iters)                # launches back to back in one hipGraph (dispatch gaps included)
+        flops, nbytes, passes = layer_work(b, storage_bytes)
+        info = lyr.kernelInfo()
+        res = bool(int(b.getFlags()) & 1)
+        key = (t, getattr(b, "kernel_", 0), b.inputChannels_, b.outputChannels_, b.height_, b.width_, tuple(b.downsample_), res)
+        g = groups.setdefault(key, {"ms": 0.0, "n": 0, "layer": lyr, "flops": flops, "bytes": nbytes, "passes": passes, "info": info,
+                                    "launches": launches_of(info), "res": res})
         g["ms"] += ms
         g["n"] += 1
+    table = []
+    sum_ms = sum_bound = 0.0
+    launches = 0
+    for key, g in groups.items():
+        avg = g["ms"] / g["n"]
+        t_flop = g["passes"] * g["flops"] / (PEAK_MFMA_F16_TFLOPS * 1e12)
+        t_mem = g["bytes"] / (PEAK_HBM_GBS * 1e9)
+        bound = max(t_flop, t_mem)
+        table.append({"layer": g["layer"].name, "count": g["n"], "avg_us": avg * 1e3, "bound": "mfma" if t_flop >= t_mem else "hbm",
+                      "bound_us": bound * 1e6, "frac": bound / (avg * 1e-3) if avg > 0 else 0.0})
+        sum_ms += g["ms"]
+        sum_bound += bound * g["n"]
+        launches += g["launches"] * g["n"]
+    table.sort(key=lambda r: -r["avg_us"] * r["count"])
     key, g = max(groups.items(), key=lambda kv: kv[1]["ms"])
-    lyr, b = g["layer"], g["layer"].builder
     avg_ms = g["ms"] / g["n"]
-    rec = {"kernel": lyr.kernelInfo(), "layer": lyr.name, "launches_per_step": g["n"], "avg_launch_us": avg_ms * 1e3}
-    if int(b.type_) in (int(fa.LayerType.CONVOLUTION2D), int(fa.LayerType.TRANSCONVOLUTION2D)) and getattr(b, "groupSize_", 1) == 1:
-        flops, (ein, eout, ew) = conv_work(b)
-        res = eout if int(b.getFlags()) & 1 else 0
-        nbytes = storage_bytes * (ein + eout + res + ew)
-        # fp32 storage: every algorithmic FLOP is issued as three fp16 MFMA FLOPs (hi*hi, lo*hi, hi*lo),
-        # which decides the bound; `achieved` stays the ALGORITHMIC rate against the fp16 matrix peak
-        passes = 3 if storage_bytes == 4 else 1
-        t_mfma = passes * flops / (PEAK_MFMA_F16_TFLOPS * 1e12)
-        t_hbm = nbytes / (PEAK_HBM_GBS * 1e9)
-        if t_mfma >= t_hbm:
-            ach = flops / (avg_ms * 1e-3) / 1e12
-            rec.update({"bound": "mfma", "achieved": ach, "peak": PEAK_MFMA_F16_TFLOPS, "unit": "TFLOP/s", "frac": ach / PEAK_MFMA_F16_TFLOPS,
-                        "mfma_passes": passes, "mfma_issue_frac": passes * ach / PEAK_MFMA_F16_TFLOPS})
-        else:
-            ach = nbytes / (avg_ms * 1e-3) / 1e9
-            rec.update({"bound": "hbm", "achieved": ach, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": ach / PEAK_HBM_GBS})
-        rec["algorithmic_flops_per_launch"] = flops
-        rec["algorithmic_bytes_per_launch"] = nbytes
-    # HBM bytes per launch from rocprofv3 FETCH_SIZE / WRITE_SIZE, scaled by the copy-kernel factors
-    # (profiles/conv_mfma_stylenet_512x624_fp32.md); only known for the profiled workload's dominant kernel
-    rec["traffic"] = MEASURED_TRAFFIC.get((key[0], key[1], key[2], key[3], key[4], key[5]))
-    per_layer = sorted(((v["ms"], v["n"], v["layer"].name) for v in groups.values()), reverse=True)
-    return rec, per_layer
+    rec = {"kernel": g["info"], "layer": g["layer"].name, "launches_per_step": g["n"], "avg_launch_us": avg_ms * 1e3}
+    t_flop = g["passes"] * g["flops"] / (PEAK_MFMA_F16_TFLOPS * 1e12)
+    t_mem = g["bytes"] / (PEAK_HBM_GBS * 1e9)
+    if g["passes"] and t_flop >= t_mem:
+        # fp32 storage: every algorithmic FLOP is issued as three fp16 MFMA FLOPs (hi*hi, lo*hi, hi*lo), which decides
+        # the bound; `achieved` stays the ALGORITHMIC rate against the fp16 matrix peak
+        ach = g["flops"] / (avg_ms * 1e-3) / 1e12
+        rec.update({"bound": "mfma", "achieved": ach, "peak": PEAK_MFMA_F16_TFLOPS, "unit": "TFLOP/s", "frac": ach / PEAK_MFMA_F16_TFLOPS,
+                    "mfma_passes": g["passes"], "mfma_issue_frac": g["passes"] * ach / PEAK_MFMA_F16_TFLOPS})
+    else:
+        ach = g["bytes"] / (avg_ms * 1e-3) / 1e9
+        rec.update({"bound": "hbm", "achieved": ach, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": ach / PEAK_HBM_GBS})
+    rec["algorithmic_flops_per_launch"] = g["flops"]
+    rec["algorithmic_bytes_per_launch"] = g["bytes"]
+    rec["traffic"] = traffic.get((g["info"], "residual" if g["res"] else "plain"))
+    whole = {"sum_kernel_us": sum_ms * 1e3, "launches_per_step": launches, "sum_bound_us": sum_bound * 1e6,
+             "frac_of_bound": sum_bound / (sum_ms * 1e-3) if sum_ms > 0 else 0.0}
+    return rec, whole, table
 
 
 def host_io_rates(net, x, frames):
@@ -292,43 +371,111 @@ def frame_pool_rate_in_child(workload, frames, instances=4, graph=True):
         return {"error": repr(e)}
 
 
-def cpu_baseline(net, x, total_flops):
-    """Times the CPU oracle (plain C restatement of the reference's unit-test convolution, OpenMP over
-    output channels) on the dominant convolution of the workload at full size and scales by the
-    network's algorithmic FLOPs."""
+def cpu_baseline(net, x, unit, total_flops):
+    """The CPU oracle (plain C restatement of the reference's unit-test convolution and layer arithmetic, OpenMP over
+    output channels) on the host's cores: one whole step of the workload when that is at most ~100 GFLOP, otherwise
+    its largest convolution scaled by the step's FLOPs.  Plus the one-core figure of BASELINE config 1 in full."""
     from oracle import oracle as O
+    from fyusenet_amd import prng
     threads = min(os.cpu_count() or 1, 16)
     O.set_threads(threads)
-    conv_layers = [l for l in net.layers if int(l.builder.type_) == int(fa.LayerType.CONVOLUTION2D) and getattr(l.builder, "groupSize_", 1) == 1]
-    lyr = max(conv_layers, key=lambda l: conv_work(l.builder)[0])
-    b = lyr.builder
-    flops, _ = conv_work(b)
-    from fyusenet_amd import prng
-    xin = prng.uniform(77, (b.inputChannels_, b.height_, b.width_), -1, 1)
-    ins = [xin]
-    if int(b.getFlags()) & 1:
-        ins.append(prng.uniform(78, (b.outputChannels_, b.height_ // b.downsample_[1], b.width_ // b.downsample_[0]), -1, 1))
+    rec = {"unit": unit, "cores": threads, "kind": "port"}
+    if total_flops <= 100e9:
+        t0 = time.perf_counter()
+        O.run_network(net.describe(), {net.input_key: x})
+        dt = time.perf_counter() - t0
+        cpu_ms = dt * 1e3
+        rec["sample"] = "one whole step (%.1f GFLOP) through the oracle, %.1f s on %d threads" % (total_flops / 1e9, dt, threads)
+    else:
+        convs = [l for l in net.layers if int(l.builder.type_) == int(fa.LayerType.CONVOLUTION2D) and getattr(l.builder, "groupSize_", 1) == 1]
+        lyr = min(convs, key=lambda l: abs(conv_work(l.builder)[0] - 20e9))   # a layer of about 20 GFLOP: 10-30 s of CPU work
+        b = lyr.builder
+        flops = conv_work(b)[0]
+        ins = [prng.uniform(77, (b.inputChannels_, b.height_, b.width_), -1, 1)]
+        if int(b.getFlags()) & 1:
+            ins.append(prng.uniform(78, (b.outputChannels_, b.height_ // b.downsample_[1], b.width_ // b.downsample_[0]), -1, 1))
+        t0 = time.perf_counter()
+        O.run_layer(b, lyr.weights, ins)
+        dt = time.perf_counter() - t0
+        cpu_ms = dt * 1e3 * total_flops / flops
+        rec["sample"] = "layer %s at full size (%.2f GFLOP, %.2f s on %d threads), scaled by the step's %.1f GFLOP" % (lyr.name, flops / 1e9, dt, threads, total_flops / 1e9)
+    rec["value"] = cpu_ms if unit == "ms/frame" else (cpu_ms * 1e3 if unit == "us" else 1e3 / cpu_ms)
+    # BASELINE config 1 on ONE core, in full: 3x3 64->64 at 256x256, ReLU on fetch (4.83 GFLOP)
+    O.set_threads(1)
+    c1 = networks.SingleConvNet(fa.STORAGE_F32)
+    c1.define()
+    b1 = c1._builders[0]
+    blk = c1._blocks[0][1]()
     t0 = time.perf_counter()
-    O.run_layer(b, lyr.weights, ins)
-    dt = time.perf_counter() - t0
-    return dt, flops, threads, lyr.name
+    O.run_layer(b1, blk, [c1.makeInput()])
+    dt1 = time.perf_counter() - t0
+    O.set_threads(threads)
+    rec["one_core_config1"] = {"value": dt1 * 1e6, "unit": "us/layer", "cores": 1, "kind": "port",
+                               "sample": "BASELINE config 1 in full (4.83 GFLOP) through the oracle's convolution on one thread"}
+    rec["b1_llvmpipe"] = ("unavailable: the reference's GL path needs its sources, a cmake build with generated shader resources and a "
+                          "software-GL context (EGL/OSMesa or an X server); neither the sources nor such a context exist on the GPU box")
+    return rec
+
+
+def measure(workload, steps, warmup, want_roofline=True):
+    """Sets the workload's network up, times K steps in both launch modes and prices its layers.  Returns (net, x, record)."""
+    net, metric, unit, dtype = make_net(workload)
+    net.setup()
+    x = net.makeInput()
+    net.setInput(x)
+    st_graph = timed_forwards(net, steps, warmup, graph=True)
+    st_eager = timed_forwards(net, steps, warmup, graph=False)
+    log("%s: hipGraph %.4f ms/step (median %.4f, p10 %.4f, p90 %.4f); eager %.4f (median %.4f)" %
+        (workload, st_graph["mean"], st_graph["median"], st_graph["p10"], st_graph["p90"], st_eager["mean"], st_eager["median"]))
+    best, launch = (st_graph, "hipGraph replay") if st_graph["mean"] <= st_eager["mean"] else (st_eager, "eager launches on one stream")
+    ms = best["mean"]
+    net.useGraph(False)
+    storage_bytes = 4 if net.storage == fa.STORAGE_F32 else 2
+    if unit == "ms/frame":
+        value, hib = ms, False
+    elif unit == "us":
+        value, hib = ms * 1e3, False
+    elif unit == "GB/s":
+        nbytes = net.algorithmic_bytes() if isinstance(net, BandwidthNet) else 2 * 4 * CopyNet.C * CopyNet.S * CopyNet.S
+        value, hib = nbytes / (ms * 1e-3) / 1e9, True
+    else:
+        value, hib = 1e3 / ms, True
+    total_flops = sum(layer_work(l.builder, storage_bytes)[0] for l in net.layers if int(l.builder.type_) not in (int(fa.LayerType.UPLOAD), int(fa.LayerType.DOWNLOAD)))
+    rec = {"metric": metric, "value": value, "unit": unit, "ms_per_step": ms, "higher_is_better": hib, "dtype": dtype,
+           "config": {"workload": workload, "input": list(x.shape), "batch": 1, "launch": launch, "algorithmic_gflop_per_step": total_flops / 1e9},
+           "step_ms": {"median": best["median"], "p10": best["p10"], "p90": best["p90"], "host_clock": best["wall"]},
+           "ms_per_step_graph": st_graph["mean"], "ms_per_step_eager": st_eager["mean"]}
+    if want_roofline:
+        roof, whole, table = roofline_records(net, storage_bytes)
+        if isinstance(net, BandwidthNet):   # a single bandwidth-bound kernel: the algorithmic bytes are the net's own count
+            nbytes = net.algorithmic_bytes()
+            ach = nbytes / (roof["avg_launch_us"] * 1e-6) / 1e9
+            roof.update({"bound": "hbm", "achieved": ach, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": ach / PEAK_HBM_GBS, "algorithmic_bytes_per_launch": nbytes})
+        rec["roofline"] = roof
+        rec["network_roofline"] = whole
+        rec["layers"] = table[:10]
+        for r in table[:8]:
+            log("   %-12s x%-2d %7.1f us each  bound %-4s %6.1f us  (%.0f %% of bound)" % (r["layer"], r["count"], r["avg_us"], r["bound"], r["bound_us"], 100 * r["frac"]))
+        log("   sum of kernels %.1f us in %d launches, sum of bounds %.1f us (%.0f %%)" % (whole["sum_kernel_us"], whole["launches_per_step"], whole["sum_bound_us"], 100 * whole["frac_of_bound"]))
+    return net, x, rec, total_flops
 
 
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="stylenet")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-also", action="store_true")
+    ap.add_argument("--no-host-io", action="store_true")
     ap.add_argument("--no-pool", action="store_true", help="skip the side measurement of several instances side by side")
     ap.add_argument("--frame-pool-only", action="store_true", help="(internal) print the frame pool's record for --workload; --steps = frames")
     ap.add_argument("--instances", type=int, default=4)
     ap.add_argument("--pool-eager", action="store_true", help="(internal) the pool's instances launch eagerly instead of replaying graphs")
     args = ap.parse_args()
     if args.gpus != 1:
-        raise SystemExit("bench.py: this engine is single-GPU (batch 1 inference); run with --gpus 1")
+        raise SystemExit("bench.py: this engine runs on one GPU (batch 1 inference, nothing is exchanged between GPUs); run with --gpus 1")
 
     if args.frame_pool_only:
         probe = make_net(args.workload)[0]
@@ -343,82 +490,41 @@ def main():
         return
 
     log(fa.capi.device_info(0))
-    net, metric, unit, dtype = make_net(args.workload)
-    net.setup()
-    x = net.makeInput()
-    net.setInput(x)
-    # both launch modes of the engine are timed over exactly K steps; the faster one is reported as `value`
-    ms_graph = timed_forwards(net, args.steps, args.warmup, graph=True)
-    ms_eager = timed_forwards(net, args.steps, args.warmup, graph=False)
-    log("%s: %.4f ms/step (hipGraph), %.4f ms/step (eager launches)" % (args.workload, ms_graph, ms_eager))
-    ms = min(ms_graph, ms_eager)
-    launch = "hipGraph replay" if ms_graph <= ms_eager else "eager launches on one stream"
-    net.useGraph(False)
-    storage_bytes = 4 if net.storage == fa.STORAGE_F32 else 2
-    roof, per_layer = dominant_conv_roofline(net, storage_bytes)
-    for t, n, name in per_layer[:8]:
-        log("   %-12s x%-2d %.1f us total" % (name, n, t * 1e3))
-    total_flops = sum(conv_work(l.builder)[0] for l in net.layers if int(l.builder.type_) in (6, 8) and getattr(l.builder, "groupSize_", 1) == 1)
-
-    if unit == "ms/frame":
-        value, hib = ms, False
-    elif unit == "us":
-        value, hib = ms * 1e3, False
-    elif unit == "GB/s":
-        nbytes = net.algorithmic_bytes() if isinstance(net, BandwidthNet) else 2 * 4 * CopyNet.C * CopyNet.S * CopyNet.S
-        value, hib = nbytes / (ms * 1e-3) / 1e9, True
-    else:
-        value, hib = 1e3 / ms, True
-
-    out = {"metric": metric, "value": value, "unit": unit, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-           "ms_per_step": ms, "higher_is_better": hib, "scaling": "weak", "vs_baseline": None, "dtype": dtype, "data": "synthetic",
-           "config": {"workload": args.workload, "input": list(x.shape), "batch": 1, "launch": launch,
-                      "algorithmic_gflop_per_step": total_flops / 1e9},
-           "ms_per_step_graph": ms_graph, "ms_per_step_eager": ms_eager, "roofline": roof}
-    if isinstance(net, BandwidthNet):   # a single bandwidth-bound kernel: the roofline record is the step itself
-        nbytes = net.algorithmic_bytes()
-        ach = nbytes / (roof["avg_launch_us"] * 1e-6) / 1e9
-        roof.update({"bound": "hbm", "achieved": ach, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": ach / PEAK_HBM_GBS,
-                     "algorithmic_bytes_per_launch": nbytes})
-
-    if hasattr(net, "input_key") and args.workload != "copy" and not isinstance(net, BandwidthNet):
-        out["host_io"] = host_io_rates(net, x, max(args.steps, 50))
+    net, x, rec, total_flops = measure(args.workload, args.steps, args.warmup)
+    out = {"metric": rec["metric"], "value": rec["value"], "unit": rec["unit"], "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+           "ms_per_step": rec["ms_per_step"], "higher_is_better": rec["higher_is_better"], "scaling": "weak", "vs_baseline": None,
+           "dtype": rec["dtype"], "data": "synthetic"}
+    for k in ("config", "step_ms", "ms_per_step_graph", "ms_per_step_eager", "roofline", "network_roofline", "layers"):
+        if k in rec:
+            out[k] = rec[k]
+    plain = hasattr(net, "input_key") and args.workload != "copy" and not isinstance(net, BandwidthNet)
+    if plain and not args.no_host_io:
+        out["host_io"] = host_io_rates(net, x, max(min(args.steps, 100), 50))
         log("host I/O inclusive: %s" % out["host_io"])
-
-    if not args.no_cpu_baseline and total_flops > 0:
-        dt, flops, threads, lname = cpu_baseline(net, x, total_flops)
-        cpu_ms = dt * 1e3 * total_flops / flops
-        if unit == "ms/frame":
-            cv = cpu_ms
-        elif unit == "us":
-            cv = cpu_ms * 1e3
-        else:
-            cv = 1e3 / cpu_ms
-        out["cpu_baseline"] = {"value": cv, "unit": unit, "cores": threads, "kind": "port",
-                               "sample": "layer %s at full size (%.2f GFLOP, %.2f s on %d threads), scaled by the step's %.1f GFLOP"
-                                         % (lname, flops / 1e9, dt, threads, total_flops / 1e9)}
+    if not args.no_cpu_baseline and total_flops > 0 and plain:
+        out["cpu_baseline"] = cpu_baseline(net, x, rec["unit"], total_flops)
+        log("cpu baseline: %s" % out["cpu_baseline"])
     net.cleanup()
-    if hasattr(net, "input_key") and unit == "imgs/s":
+    if plain and rec["unit"] == "imgs/s" and not args.no_pool:
         # several instances side by side: batch-1 networks of small layers are latency-bound.  (The style nets' launches
-        # fill most of the chip: 2 to 4 instances of them run at the single frame pipeline's rate, 0.43-0.50 ms/frame.)
-        if not args.no_pool:
-            out["frame_pool"] = frame_pool_rate_in_child(args.workload, max(8 * args.steps, 400))
-            log("frame pool: %s" % out["frame_pool"])
+        # fill most of the chip: 2 to 4 instances of them run at the single frame pipeline's rate.)
+        out["frame_pool"] = frame_pool_rate_in_child(args.workload, max(8 * args.steps, 400))
+        log("frame pool: %s" % out["frame_pool"])
 
     if not args.no_also and args.workload == "stylenet":
+        # the other BASELINE configurations and the reference's own sample graphs, each with its own roofline record
         also = {}
-        for wl in ("resnet50", "resnet50ref", "stylenet3x3ref", "stylenet9x9ref"):
-            n2, m2, u2, d2 = make_net(wl)
-            n2.setup()
-            n2.setInput(n2.makeInput())
-            ms2g = timed_forwards(n2, max(args.steps, 100), args.warmup, graph=True)
-            ms2e = timed_forwards(n2, max(args.steps, 100), args.warmup, graph=False)
-            ms2 = min(ms2g, ms2e)
-            also[m2] = {"value": 1e3 / ms2 if u2 == "imgs/s" else ms2, "unit": u2, "ms_per_step": ms2, "ms_per_step_graph": ms2g, "ms_per_step_eager": ms2e, "dtype": d2}
-            log("%s: %.4f ms/step (hipGraph) %.4f (eager)" % (wl, ms2g, ms2e))
+        for wl, steps in (("resnet50", max(args.steps, 100)), ("conv1", max(args.steps, 100)), ("mobilenet", max(args.steps, 100)),
+                          ("stylenet9x9", min(max(args.steps // 4, 10), 25)), ("resnet50ref", max(args.steps, 100)),
+                          ("stylenet3x3ref", max(args.steps, 100)), ("stylenet9x9ref", max(args.steps, 100))):
+            n2, _x2, r2, _f2 = measure(wl, steps, args.warmup)
             n2.cleanup()
+            entry = {k: r2[k] for k in ("value", "unit", "ms_per_step", "step_ms", "ms_per_step_graph", "ms_per_step_eager", "dtype", "roofline", "network_roofline")}
+            entry["steps"] = steps
+            entry["layers"] = r2["layers"][:5]
             if wl == "resnet50" and not args.no_pool:
-                also[m2]["frame_pool"] = frame_pool_rate_in_child(wl, 800)
+                entry["frame_pool"] = frame_pool_rate_in_child(wl, 800)
+            also[r2["metric"]] = entry
         out["also"] = also
     print(json.dumps(out), flush=True)
 

@@ -106,18 +106,22 @@ class SingleConvNet(_StreamNet):
     (ConvLayerBuilder(3).shape(64,256,256,64).deep().inputPadding(1).prefixAct(RELU))."""
     config_id = 1
 
-    def __init__(self, storage=STORAGE_F32, size=256, channels=64, device=0, width=None, height=None):
+    def __init__(self, storage=STORAGE_F32, size=256, channels=64, device=0, width=None, height=None, residual=False):
         super().__init__(storage, device)
-        self.width, self.height, self.ch = width or size, height or size, channels
+        self.width, self.height, self.ch, self.residual = width or size, height or size, channels, residual
 
     def define(self):
         self.conv(1, "conv3x3", 3, self.ch, self.ch, self.height, self.width, None, act=ActType.RELU, bn=False)
+        if self.residual:   # residual tensor on port 1, fed from the host like the input (ReLU applied on its fetch)
+            self._builders[-1].residual(ActType.RELU)
 
     def makeInput(self):
         return prng.uniform(SEED_BASE + 256 + 200, (self.ch, self.height, self.width), -1.0, 1.0)
 
     def setInput(self, x):
         self.layers[1].setInput(x, 0)
+        if self.residual:
+            self.layers[1].setInput(prng.uniform(SEED_BASE + 256 + 201, (self.ch, self.height, self.width), -1.0, 1.0), 1)
 
     output_layer = 1
     input_key = (1, 0)
