@@ -1,0 +1,383 @@
+// Wide-kernel convolution with at most four output channels (the 9x9 32->3 output layer of a style-transfer net) as
+// a row-rolling implicit GEMM on gfx950 matrix cores.
+//
+// Replaces, for such layers, the render passes of DeepConvLayerNxN::forward (fyusenet/gpu/deep/deepconvlayerNxN.cpp:
+// 129-211) and of the shallow ConvLayerNxN::forward (gpu/vanilla/convlayerNxN_vanilla.cpp:72-141).
+//
+// GEMM view: M = virtual output channels (o, kx), cout*K <= 32 of them: one 32-row fragment; K = (ky, input channel);
+// N = the columns x' of one image row of q[y][x'][o*K+kx] = sum_{ky,ci} W[o,ky,kx,ci] * act(in[y+ky-r, x'-r, ci]).
+// The output is out[y][x][o] = sum_kx q[y][x+kx][o*K+kx], summed from the accumulators inside the wave.
+//
+// A workgroup owns a strip of 32*FN columns of q (32*FN - K + 1 output columns) and walks down a block of rows.  The
+// input rows of the strip live in an LDS ring of 16 rows (fp16, hi and lo planes with fp32 storage); every input row
+// is fetched from memory once per strip, by four staging waves, four rows ahead of the four MFMA waves, each of which
+// computes one output row per round (K input rows, K*CS k16-steps).  The weights -- one fragment per step and plane --
+// stay in registers for the whole kernel, so the step loop reads nothing but the ring.
+#include <hip/hip_fp16.h>
+#include <hip/hip_runtime.h>
+
+#include "kernels.h"
+
+// Timing-study builds (-DFYN_ROWS_TRACE): wave 0 and wave 4 of every workgroup record the shader clock at phase boundaries.
+#ifdef FYN_ROWS_TRACE
+#include <cstdio>
+#include <cstdlib>
+#include <vector>
+#define FYN_RTRACE(slot) do { if (lane == 0 && (wave & 3) == 0 && (slot) < 32) p.trace[((size_t)blockIdx.x * 2 + (wave >> 2)) * 32 + (slot)] = clock64(); } while (0)
+#else
+#define FYN_RTRACE(slot) do { } while (0)
+#endif
+
+namespace fynhip {
+
+namespace {
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef float float16_t __attribute__((ext_vector_type(16)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+
+constexpr int RING = 16;   // input rows resident per strip: K + 3 in use by a round, 4 being staged (K <= 9)
+// Floats per column of a wave's epilogue area [column][virtual channel]: odd, so that the lanes of a wave (one column
+// each) fall into distinct banks; cout*K <= 28 virtual channels are kept.
+constexpr int ROWS_SCRATCH_PITCH = 29;
+
+// Workgroup barrier that orders LDS traffic only: outstanding global loads (rows fetched two rounds ahead) and global
+// stores (finished output rows) stay in flight across it.  __syncthreads() would wait for them as well.
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+__device__ __forceinline__ float act1r(float x, const Act& a) { return fminf(a.hi, fmaxf(a.lo, x)) + a.leak * fminf(x, 0.f); }
+
+template <typename T>
+__device__ __forceinline__ void load8(const T* src, float* v);
+template <>
+__device__ __forceinline__ void load8<float>(const float* src, float* v) {
+    const float4 a = *reinterpret_cast<const float4*>(src), b = *reinterpret_cast<const float4*>(src + 4);
+    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+}
+template <>
+__device__ __forceinline__ void load8<_Float16>(const _Float16* src, float* v) {
+    const half8_t a = *reinterpret_cast<const half8_t*>(src);
+#pragma unroll
+    for (int i = 0; i < 8; i++) v[i] = (float)a[i];
+}
+
+// CS: k16 steps per input row (input channels padded to 16*CS); a column of the ring holds 2*CS chunks of 8 halves.
+// The chunk order inside a column is permuted with the column index so that the 16-byte reads of 8 neighbouring lanes
+// cover all 32 banks.
+template <int CS>
+__device__ __forceinline__ int ring_off(int col, int chunk) {
+    constexpr int NCH = 2 * CS, CPB = 8 / NCH;   // chunks per column, columns per 128 bytes
+    return col * (NCH * 16) + ((chunk ^ ((col / CPB) & (NCH - 1))) * 16);
+}
+
+template <typename TIn, typename TOut, bool SPLIT, int K, int CS, int FN>
+__global__ __launch_bounds__(512) void conv_rows_kernel(const ConvRowsParams p) {
+    extern __shared__ __align__(16) unsigned char lds[];
+    constexpr int NPL = SPLIT ? 2 : 1;
+    constexpr int WC = 32 * FN;               // q columns per strip
+    constexpr int OW = WC - (K - 1);          // output columns per strip
+    constexpr int NCH = 2 * CS;
+    constexpr int PLANE = WC * NCH * 16;      // bytes of one plane of one ring row
+    constexpr int ROWB = NPL * PLANE;
+    constexpr int NSTEPS = K * CS;
+    constexpr int ITEMS = WC * NCH;           // staging items (8 channels of one column) per row
+    static_assert(K >= 3 && K <= 9 && (K & 1), "kernel sizes 3, 5, 7, 9");
+    static_assert(4 * ((K + 2) / 4 + 2) <= RING, "ring too small");
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const bool mfma_wave = wave < 4;
+    const int strip = blockIdx.x % p.strips;
+    const int rblk = blockIdx.x / p.strips;
+    const int y_begin = rblk * p.rows_per_block;
+    const int y_end = min(y_begin + p.rows_per_block, p.out_h);
+    const int x0 = strip * OW;                // first q column (= first output column) of the strip
+    constexpr int sp = ROWS_SCRATCH_PITCH;    // floats per column of the epilogue area
+    unsigned char* ring = lds;
+    float* scratch = reinterpret_cast<float*>(lds + RING * ROWB) + (wave & 3) * (WC * sp);
+
+    // ---- staging: q row j (relative to y_begin) is stored input row in_y0 + y_begin + j ----
+    const TIn* in = reinterpret_cast<const TIn*>(p.in);
+    const int stid = tid & 255;
+    // Four rows at a time: ITEMS items per row dealt to the 256 staging threads.  fetch() issues the loads of a batch
+    // into registers, store() converts and writes them into the ring; a batch is fetched one round before it is stored.
+    constexpr int PER = (4 * ITEMS + 255) / 256;   // items per thread and batch
+    struct Batch {
+        float v[PER][8];
+        int dst[PER];
+    };
+    auto fetch = [&](Batch& bt, int j_first, int nrows) {
+#pragma unroll
+        for (int i = 0; i < PER; i++) {
+            const int idx = i * 256 + stid;
+            bt.dst[i] = -1;
+#pragma unroll
+            for (int e = 0; e < 8; e++) bt.v[i][e] = 0.f;
+            if (idx < nrows * ITEMS) {
+                const int jr = idx / ITEMS, it = idx - jr * ITEMS;
+                const int col = it / NCH, chunk = it - col * NCH;
+                const int j = j_first + jr;
+                int gy = p.in_y0 + y_begin + j, gx = p.in_x0 + x0 + col;
+                if (p.in_clamp) {
+                    gy = min(max(gy, 0), p.in_hp - 1);
+                    gx = min(max(gx, 0), p.in_wp - 1);
+                }
+                bt.dst[i] = (j & (RING - 1)) * ROWB + ring_off<CS>(col, chunk);
+                if ((unsigned)gy < (unsigned)p.in_hp && (unsigned)gx < (unsigned)p.in_wp && chunk * 8 < p.in_cp)
+                    load8<TIn>(in + ((size_t)gy * p.in_wp + gx) * p.in_cp + chunk * 8, bt.v[i]);
+            }
+        }
+    };
+    auto store = [&](const Batch& bt) {
+#pragma unroll
+        for (int i = 0; i < PER; i++) {
+            if (bt.dst[i] < 0) continue;
+            half8_t hi, lo;
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                const float a = act1r(bt.v[i][e], p.act);
+                hi[e] = (_Float16)a;
+                lo[e] = (_Float16)(a - (float)hi[e]);
+            }
+            *reinterpret_cast<half8_t*>(ring + bt.dst[i]) = hi;
+            if (SPLIT) *reinterpret_cast<half8_t*>(ring + bt.dst[i] + PLANE) = lo;
+        }
+    };
+
+    const int rows_total = y_end - y_begin + (K - 1);   // q rows this block needs
+    // batch b holds q rows [4b, 4b + 4); round g reads batches g .. g + (K + 2) / 4, batch g + 3 is written during round g
+    constexpr int NB0 = (K + 2) / 4 + 1;      // batches in the ring before the first round
+    const int nbatches = (rows_total + 3) >> 2;
+    auto rows_of = [&](int b) { return min(4, rows_total - 4 * b); };
+    Batch nxt;   // the batch in flight (staging waves)
+    FYN_RTRACE(0);
+    if (!mfma_wave) {
+        // all loads of the first rounds' rows are issued before the first conversion
+        Batch first[NB0];
+#pragma unroll
+        for (int b = 0; b < NB0; b++) fetch(first[b], 4 * b, b < nbatches ? rows_of(b) : 0);
+#pragma unroll
+        for (int b = 0; b < NB0; b++) store(first[b]);
+        // (the batch of the second round is requested once the first round's rows are in: every workgroup of the
+        // launch is in this phase at the same time, and it is bound by memory bandwidth)
+        fetch(nxt, 4 * NB0, NB0 < nbatches ? rows_of(NB0) : 0);
+    }
+    // ---- weights: one fragment per step and plane, in registers from here on (loaded while the staging waves fill
+    //      the ring; placed behind their code so that the two never hold registers at the same point) ----
+    half8_t a_reg[NSTEPS][NPL];
+    if (mfma_wave) {
+        const half8_t* w = reinterpret_cast<const half8_t*>(p.wpack);
+#pragma unroll
+        for (int t = 0; t < NSTEPS; t++)
+#pragma unroll
+            for (int pl = 0; pl < NPL; pl++) a_reg[t][pl] = w[(t * NPL + pl) * 64 + lane];
+    }
+    FYN_RTRACE(1);
+    lds_barrier();
+    FYN_RTRACE(2);
+
+    // per-lane byte offsets of the B fragments inside a ring row: column fn*32 + lane%32, chunk 2*sub + lane/32
+    int boff[CS][FN];
+#pragma unroll
+    for (int sub = 0; sub < CS; sub++)
+#pragma unroll
+        for (int fn = 0; fn < FN; fn++) boff[sub][fn] = ring_off<CS>(fn * 32 + (lane & 31), 2 * sub + (lane >> 5));
+
+    float sc4[4], bi4[4];
+#pragma unroll
+    for (int o = 0; o < 4; o++) {
+        sc4[o] = o < p.cout ? p.scale[o] : 0.f;
+        bi4[o] = o < p.cout ? p.bias[o] : 0.f;
+    }
+    TOut* out = reinterpret_cast<TOut*>(p.out);
+    const TOut* res = reinterpret_cast<const TOut*>(p.res);
+
+    const int nrounds = (y_end - y_begin + 3) >> 2;
+    // One loop per role (the same barriers in both), so that a wave's registers hold either the staged items or the
+    // weights, fragments and accumulators.
+    if (!mfma_wave) {
+        for (int g = 0; g < nrounds; g++) {
+            // write batch NB0 + g (fetched a round ago; no round up to g reads its ring slots), fetch the next one
+            store(nxt);
+            FYN_RTRACE(3 + 3 * g);
+            const int b = NB0 + g + 1;
+            fetch(nxt, 4 * b, b < nbatches ? rows_of(b) : 0);
+            FYN_RTRACE(4 + 3 * g);
+            lds_barrier();
+            FYN_RTRACE(5 + 3 * g);
+        }
+        return;
+    }
+    for (int g = 0; g < nrounds; g++) {
+        {
+            const int yl = 4 * g + wave;          // output row relative to y_begin
+            const int y = y_begin + yl;
+            if (y < y_end) {
+                float16_t acc[FN];
+#pragma unroll
+                for (int fn = 0; fn < FN; fn++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++) acc[fn][r] = 0.f;
+                half8_t b[2][FN][NPL];
+                auto load_b = [&](int t, half8_t (&dst)[FN][NPL]) {
+                    const int ky = t / CS, sub = t % CS;
+                    const unsigned char* row = ring + ((yl + ky) & (RING - 1)) * ROWB;
+#pragma unroll
+                    for (int pl = 0; pl < NPL; pl++)
+#pragma unroll
+                        for (int fn = 0; fn < FN; fn++) dst[fn][pl] = *reinterpret_cast<const half8_t*>(row + pl * PLANE + boff[sub][fn]);
+                };
+                load_b(0, b[0]);
+                // one slot per MFMA: the MFMA, then a share of the next step's LDS reads, in this order (a memory
+                // instruction issued right behind an MFMA runs in its shadow; one wave cannot queue MFMAs)
+                constexpr int NMF = FN * (SPLIT ? 3 : 1), NDS = FN * NPL;
+#pragma unroll
+                for (int t = 0; t < NSTEPS; t++) {
+                    const int kyn = (t + 1) / CS, subn = (t + 1) % CS;
+                    const unsigned char* rown = ring + ((yl + kyn) & (RING - 1)) * ROWB;
+#pragma unroll
+                    for (int i = 0; i < NMF; i++) {
+                        const int kind = i / FN, fn = i % FN;
+                        const int apl = (kind == 1) ? 1 : 0, bpl = (kind == 2) ? 1 : 0;
+                        acc[fn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_reg[t][apl], b[t & 1][fn][bpl], acc[fn], 0, 0, 0);
+                        if (t + 1 < NSTEPS) {
+#pragma unroll
+                            for (int j = i * NDS / NMF; j < (i + 1) * NDS / NMF; j++)
+                                b[(t + 1) & 1][j % FN][j / FN] = *reinterpret_cast<const half8_t*>(rown + (j / FN) * PLANE + boff[subn][j % FN]);
+                        }
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                }
+                FYN_RTRACE(3 + 3 * g);
+                // accumulators -> this wave's area [column][virtual channel]: a lane holds column lane%32 of each
+                // fragment and rows 8*(r/4) + 4*(lane/32) + r%4
+#pragma unroll
+                for (int fn = 0; fn < FN; fn++)
+#pragma unroll
+                    for (int q = 0; q < 4; q++) {
+                        const int rowb = q * 8 + (lane >> 5) * 4;
+                        if (rowb < 28) {
+                            float* dstp = scratch + (fn * 32 + (lane & 31)) * sp + rowb;
+#pragma unroll
+                            for (int e = 0; e < 4; e++) dstp[e] = acc[fn][q * 4 + e];
+                        }
+                    }
+                // out[y][x][o] = sum_kx q[x + kx][o*K + kx]: one output column per lane
+                for (int x = lane; x < OW; x += 64) {
+                    const int gx = x0 + x;
+                    if (gx >= p.out_w) break;
+                    // all K*4 reads are issued before the first sum (a read under a condition would cost one LDS round
+                    // trip each); channels beyond cout read some row of the column and are discarded below
+                    float qv[K][4];
+#pragma unroll
+                    for (int kx = 0; kx < K; kx++) {
+                        const float* qp = scratch + (x + kx) * sp;
+#pragma unroll
+                        for (int o = 0; o < 4; o++) qv[kx][o] = qp[(o * K + kx < 28) ? o * K + kx : 27];
+                    }
+                    float a[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int kx = 0; kx < K; kx++)
+#pragma unroll
+                        for (int o = 0; o < 4; o++) a[o] += qv[kx][o];
+                    float rv[4] = {0.f, 0.f, 0.f, 0.f};
+                    if (res) {
+                        const TOut* rp = res + ((size_t)(p.res_off_y + y) * p.res_wp + p.res_off_x + gx) * p.res_cp;
+                        if (sizeof(TOut) == 4) {
+                            const float4 r4 = *reinterpret_cast<const float4*>(rp);
+                            rv[0] = r4.x; rv[1] = r4.y; rv[2] = r4.z; rv[3] = r4.w;
+                        } else {
+                            const half4_t r4 = *reinterpret_cast<const half4_t*>(rp);
+#pragma unroll
+                            for (int o = 0; o < 4; o++) rv[o] = (float)r4[o];
+                        }
+                    }
+                    f32x4_t v;
+#pragma unroll
+                    for (int o = 0; o < 4; o++) {
+                        float r = rv[o];
+                        if (p.res_relu) r = fmaxf(r, 0.f);
+                        if (p.res_scale) r *= sc4[o];
+                        v[o] = o < p.cout ? ((a[o] * p.acc_mul) * sc4[o] + bi4[o]) + r : 0.f;
+                    }
+                    const size_t oidx = ((size_t)(p.out_off_y + y) * p.out_wp + p.out_off_x + gx) * p.out_cp;
+                    if (sizeof(TOut) == 4) {
+                        *reinterpret_cast<f32x4_t*>(reinterpret_cast<float*>(out) + oidx) = v;
+                    } else {
+                        half4_t hv;
+#pragma unroll
+                        for (int o = 0; o < 4; o++) hv[o] = (_Float16)v[o];
+                        *reinterpret_cast<half4_t*>(reinterpret_cast<_Float16*>(out) + oidx) = hv;
+                    }
+                }
+            }
+        }
+        FYN_RTRACE(4 + 3 * g);
+        lds_barrier();   // the round's rows are consumed, the next round's rows are in the ring
+        FYN_RTRACE(5 + 3 * g);
+    }
+}
+
+typedef void (*rows_fn)(const ConvRowsParams);
+
+template <typename TIn, typename TOut, bool SPLIT, int FN>
+rows_fn pick_rows(int k, int cs) {
+#define FYN_ROWS(K_, CS_) \
+    if (k == K_ && cs == CS_) return conv_rows_kernel<TIn, TOut, SPLIT, K_, CS_, FN>;
+    FYN_ROWS(3, 1) FYN_ROWS(3, 2) FYN_ROWS(5, 1) FYN_ROWS(5, 2) FYN_ROWS(7, 1) FYN_ROWS(7, 2) FYN_ROWS(9, 1) FYN_ROWS(9, 2)
+#undef FYN_ROWS
+    return nullptr;
+}
+}  // namespace
+
+bool conv_rows_supported(int k, int cin_pitch, int cout, bool f16) {
+    (void)f16;
+    return (k == 3 || k == 5 || k == 7 || k == 9) && cout >= 1 && cout <= 4 && cout * k <= 28 && cin_pitch >= 8 && cin_pitch <= 32 &&
+           cin_pitch % 8 == 0;
+}
+
+size_t conv_rows_lds_bytes(const ConvRowsParams& p, bool f16) {
+    const int wc = 32 * p.fn, nch = 2 * p.cs;
+    return (size_t)RING * (f16 ? 1 : 2) * wc * nch * 16 + (size_t)4 * wc * ROWS_SCRATCH_PITCH * sizeof(float);
+}
+
+int launch_conv_rows(const ConvRowsParams& p, bool f16, hipStream_t s) {
+    if (p.fn != 2) return -1;
+    rows_fn fn = f16 ? pick_rows<_Float16, _Float16, false, 2>(p.k, p.cs) : pick_rows<float, float, true, 2>(p.k, p.cs);
+    if (!fn) return -1;
+    // what the kernel's indexing assumes
+    if (p.cout * p.k > 28 || p.out_cp != 4 || p.strips < 1 || p.row_blocks < 1 ||
+        p.rows_per_block < 1 || p.rows_per_block % 4 || p.in_cp > 16 * p.cs || p.in_cp % 8 || p.cout * p.k > 32 ||
+        (long long)p.strips * (32 * p.fn - (p.k - 1)) < p.out_w || (long long)p.row_blocks * p.rows_per_block < p.out_h)
+        return -5;
+    const size_t lds_bytes = conv_rows_lds_bytes(p, f16);
+    if (lds_bytes > 160 * 1024) return -2;
+    if (lds_bytes > 48 * 1024) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes) != hipSuccess) return -2;
+    }
+#ifdef FYN_ROWS_TRACE
+    {
+        static long long* dev = nullptr;
+        const size_t n = (size_t)p.strips * p.row_blocks * 64;
+        if (!dev && hipMalloc(&dev, sizeof(long long) * 65536 * 64) != hipSuccess) return -6;
+        ConvRowsParams q = p;
+        q.trace = dev;
+        hipLaunchKernelGGL(fn, dim3(p.strips * p.row_blocks), dim3(512), lds_bytes, s, q);
+        hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+        (void)hipStreamIsCapturing(s, &cap);
+        const char* path = cap == hipStreamCaptureStatusNone ? getenv("FYNHIP_TRACE_DUMP") : nullptr;
+        if (path) {
+            std::vector<long long> h(n);
+            if (hipStreamSynchronize(s) == hipSuccess && hipMemcpy(h.data(), dev, n * 8, hipMemcpyDeviceToHost) == hipSuccess) {
+                if (FILE* f = fopen(path, "wb")) { fwrite(h.data(), 8, n, f); fclose(f); }
+            }
+        }
+        return hipGetLastError() == hipSuccess ? 0 : -3;
+    }
+#endif
+    hipLaunchKernelGGL(fn, dim3(p.strips * p.row_blocks), dim3(512), lds_bytes, s, p);
+    return hipGetLastError() == hipSuccess ? 0 : -3;
+}
+
+}  // namespace fynhip

@@ -124,6 +124,35 @@ int conv_mfma_tile_count();
 void conv_mfma_tile(int index, int* fm, int* fn, int* wm, int* wn);
 
 // ---------------------------------------------------------------------------------------------
+// Row-rolling MFMA convolution for wide kernels with at most four output channels (conv_rows.hip)
+// ---------------------------------------------------------------------------------------------
+struct ConvRowsParams {
+    const void* in;
+    void* out;
+    const void* res;      // residual tensor or nullptr
+    const void* wpack;    // [k*cs steps][plane][lane 0..63][8 halves]: virtual channel o*k+kx = lane%32, input channel 16*sub + 8*(lane/32) + j
+    const float* scale;   // [cout]
+    const float* bias;    // [cout]
+    int k, cs, fn;        // kernel size; k16 steps per input row (input channel pitch <= 16*cs); 32-column fragments per strip
+    int in_hp, in_wp, in_cp;   // stored input frame
+    int in_y0, in_x0;     // stored row of (output row 0, tap ky 0) and stored column of q column 0 (input padding - radius)
+    int in_clamp;         // coordinates outside the stored frame repeat its edge instead of reading 0
+    int out_h, out_w;
+    int out_wp, out_cp, out_off_y, out_off_x;
+    int res_wp, res_cp, res_off_y, res_off_x, res_relu, res_scale;
+    int strips, row_blocks, rows_per_block;   // grid = strips * row_blocks workgroups; rows_per_block is a multiple of 4
+    int cout;
+    float acc_mul;
+#ifdef FYN_ROWS_TRACE
+    long long* trace;     // timing-study builds only: 32 timestamps per workgroup and role
+#endif
+    Act act;
+};
+bool conv_rows_supported(int k, int cin_pitch, int cout, bool f16);
+size_t conv_rows_lds_bytes(const ConvRowsParams& p, bool f16);
+int launch_conv_rows(const ConvRowsParams& p, bool f16, hipStream_t s);
+
+// ---------------------------------------------------------------------------------------------
 // Direct (non-MFMA) layer kernels (layers_direct.hip)
 // ---------------------------------------------------------------------------------------------
 struct ConvDirectParams {

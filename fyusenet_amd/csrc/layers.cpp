@@ -841,6 +841,85 @@ class ConvLayer : public Layer {
         sr.scale = scale_dev; sr.bias = bias_dev;
         sr.res_relu = res_relu; sr.res_scale = res_scale;
     }
+    void setup_rows_wide(const TView& in_v, const TView& out_v, const TView* res_v, int res_relu, int res_scale) {
+        const int r = (k - 1) / 2;
+        ConvRowsParams q{};
+        q.in = in_v.ptr; q.out = out_v.ptr; q.res = res_v ? res_v->ptr : nullptr;
+        q.k = k; q.cs = (in_v.cp + 15) / 16; q.fn = 2;
+        q.in_hp = in_v.hp(); q.in_wp = in_v.wp(); q.in_cp = in_v.cp;
+        q.in_y0 = in_v.pad - r; q.in_x0 = in_v.pad - r;
+        q.in_clamp = clamp ? 1 : 0;
+        q.out_h = oh; q.out_w = ow;
+        q.out_wp = out_v.wp(); q.out_cp = out_v.cp; q.out_off_y = q.out_off_x = out_v.pad;
+        if (res_v) { q.res_wp = res_v->wp(); q.res_cp = res_v->cp; q.res_off_y = q.res_off_x = res_v->pad; }
+        q.res_relu = res_relu; q.res_scale = res_scale;
+        const int strip_w = 32 * q.fn - (k - 1);
+        q.strips = (ow + strip_w - 1) / strip_w;
+        // one workgroup per CU (the ring takes most of the LDS): as many row blocks as fill the chip in one round
+        int blocks = std::max(1, 256 / q.strips);
+        q.rows_per_block = ((oh + blocks - 1) / blocks + 3) / 4 * 4;
+        q.row_blocks = (oh + q.rows_per_block - 1) / q.rows_per_block;
+        q.cout = oc;
+        q.scale = scale_dev; q.bias = bias_dev;
+        q.acc_mul = 1.f;
+        q.act = act();
+        if (conv_rows_lds_bytes(q, out_v.f16 != 0) > 160 * 1024) return;
+        const size_t halves = (size_t)k * q.cs * (out_v.f16 ? 1 : 2) * 64 * 8;
+        q.wpack = rows_wpack_dev = net->dev_alloc(halves * 2, true);
+        const bool always = getenv("FYNHIP_FORCE_ROWS_WIDE_CONV") != nullptr;
+        const char* at = getenv("FYNHIP_AUTOTUNE");
+        bool pick = true;
+        char key[160];
+        snprintf(key, sizeof(key), "rows:%d:%dx%d:%dx%d:k%d:cp%d:r%d:e%d", out_v.f16, d.in_channels, oc, oh, ow, k, in_v.cp, res_v ? 1 : 0, clamp ? 1 : 0);
+        if (always) {
+        } else if (tune_cache_flag(key, &pick)) {
+        } else if (!(at && at[0] == '0')) {
+            float t_rows = 1e30f, t_other = 1e30f;
+            for (int rep = 0; rep < 3; rep++) {
+                t_rows = std::min(t_rows, time_calls(net, [&]() {
+                    if (launch_conv_rows(q, out_v.f16 != 0, net->stream) != 0) fail(FYN_ERR_DEVICE, "row-rolling convolution launch failed while tuning");
+                }, 10));
+                t_other = std::min(t_other, time_calls(net, [&]() {
+                    run_mfma(launch, net->stream);
+                    if (!fused) launch_shift_reduce(sr, net->stream);
+                }, 10));
+            }
+            if (getenv("FYNHIP_TUNE_VERBOSE")) fprintf(stderr, "[tune] folded kx taps: row-rolling %.1f us, %s %.1f us\n", t_rows * 1e3f, fused ? "one launch" : "two passes", t_other * 1e3f);
+            pick = t_rows < t_other;
+            tune_cache_store_flag(key, pick);
+        }
+        if (pick) {
+            rows = true;
+            rp = q;
+            if (qv.ptr) { net->dev_free(qv.ptr); qv.ptr = nullptr; }
+        } else {
+            net->dev_free(rows_wpack_dev);
+            rows_wpack_dev = nullptr;
+        }
+    }
+    // weights of the row-rolling form: [step = ky*cs + sub][plane][lane][8 halves]
+    void pack_rows(const float* w, float wmul) {
+        const int cin = d.in_channels, npl = tout().v.f16 ? 1 : 2;
+        std::vector<uint16_t> pack((size_t)k * rp.cs * npl * 64 * 8, 0);
+        for (int ky = 0; ky < k; ky++)
+            for (int sub = 0; sub < rp.cs; sub++)
+                for (int lane = 0; lane < 64; lane++) {
+                    const int vch = lane & 31, o = vch / k, kx = vch % k;
+                    if (o >= oc) continue;
+                    for (int j = 0; j < 8; j++) {
+                        const int ci = sub * 16 + 8 * (lane >> 5) + j;
+                        if (ci >= cin) continue;
+                        const float v = w[(((size_t)o * k + ky) * k + kx) * cin + ci] * wmul;
+                        const uint16_t hi = f2h_bits(v);
+                        const size_t base = ((size_t)(ky * rp.cs + sub) * npl) * 64 * 8;
+                        pack[base + (size_t)lane * 8 + j] = hi;
+                        if (npl == 2) pack[base + (size_t)(64 + lane) * 8 + j] = f2h_bits(v - h2f(hi));
+                    }
+                }
+        FYN_HIP(hipStreamSynchronize(net->stream));
+        FYN_HIP(hipMemcpyAsync(rows_wpack_dev, pack.data(), pack.size() * 2, hipMemcpyHostToDevice, net->stream));
+        FYN_HIP(hipStreamSynchronize(net->stream));
+    }
     size_t weight_floats() const override {
         return (size_t)oc + (size_t)oc * k * k * d.in_channels + ((d.flags & FYN_FLAG_POST_BATCHNORM) ? 2 * (size_t)oc : 0);
     }
@@ -929,6 +1008,10 @@ class ConvLayer : public Layer {
                     }
                 }
             }
+            // Third form: a workgroup walks down a strip of the image with the input rows in an LDS ring and the weights
+            // in registers (conv_rows.hip); every input row is fetched once per strip and q never leaves the wave.
+            if (!frac_shift && conv_rows_supported(k, in_v.cp, oc, out_v.f16 != 0) && out_v.cp == 4 && !getenv("FYNHIP_NO_ROWS_WIDE_CONV"))
+                setup_rows_wide(in_v, out_v, res_v, res_relu, res_scale);
         } else {
             SubConv sc;
             for (int ky = 0; ky < k; ky++)
@@ -985,6 +1068,10 @@ class ConvLayer : public Layer {
                         for (int i = 0; i < cin; i++)
                             wd[(((size_t)ky * k + kx) * cin + i) * cp + o] = w[(((size_t)o * k + ky) * k + kx) * cin + i];
             reupload(net, wdirect_dev, wd);
+        } else if (wide && rows) {
+            const float wmul = weight_prescale(w, (size_t)oc * k * k * d.in_channels);
+            rp.acc_mul = 1.0f / wmul;
+            pack_rows(w, wmul);
         } else if (wide) {
             const int cin = d.in_channels;
             const float wmul = weight_prescale(w, (size_t)oc * k * k * cin);
@@ -1016,6 +1103,10 @@ class ConvLayer : public Layer {
     }
     void forward(hipStream_t s) override {
         if (!have_weights) fail(FYN_ERR_STATE, "layer %s (%d): forward() without weights", d.name, d.number);
+        if (rows) {
+            if (launch_conv_rows(rp, tout().v.f16 != 0, s) != 0) fail(FYN_ERR_DEVICE, "layer %s: convolution launch failed", d.name);
+            return;
+        }
         if (direct) launch_conv_direct(dp, s);
         else if (run_mfma(launch, s) != 0)
             fail(FYN_ERR_DEVICE, "layer %s: convolution launch failed", d.name);
@@ -1024,16 +1115,24 @@ class ConvLayer : public Layer {
     std::string info() const override {
         const std::string mode = frac_shift ? "(fractional step 1/" + std::to_string(1 << (frac_shift - 1)) + ") " : (clamp ? "(edge-clamp) " : "");
         if (direct) return "conv_direct" + mode;
+        if (rows) {
+            char buf[200];
+            snprintf(buf, sizeof(buf), "conv_rows %s(kx folded into cout, rows rolled through an LDS ring) strips=%d x %d row blocks of %d rows, lds=%zu",
+                     tout().v.f16 ? "f16 " : "f16x2-split ", rp.strips, rp.row_blocks, rp.rows_per_block, conv_rows_lds_bytes(rp, tout().v.f16 != 0));
+            return mode + buf;
+        }
         if (wide) return mode + (fused ? "wide-kernel(kx folded into cout, summed in the epilogue) " : "wide-kernel(kx folded into cout)+shift_reduce ") + mfma_info(launch);
         return mode + mfma_info(launch);
     }
 
     int k, dil, stride;
     int frac_shift = 0;   // fractional-step convolution: log2(1/sourceStep) + 1
-    bool clamp = false, direct = false, wide = false, fused = false, have_weights = false;
+    bool clamp = false, direct = false, wide = false, fused = false, rows = false, have_weights = false;
     int padded = 0;
     std::vector<float> block;
     MfmaLaunch launch;
+    ConvRowsParams rp{};          // row-rolling form of the folded convolution (conv_rows.hip)
+    void* rows_wpack_dev = nullptr;
     ConvDirectParams dp{};
     ShiftReduceParams sr{};
     TView qv{};

@@ -200,6 +200,7 @@ def test_wide_kernel_few_output_channels(case, two_pass, storage, monkeypatch):
     and summed by a second pass."""
     k, cout, h, w, cin, kw = case
     monkeypatch.setenv("FYNHIP_NO_FUSED_WIDE_CONV" if two_pass else "FYNHIP_FORCE_FUSED_WIDE_CONV", "1")   # (else: whichever is faster)
+    monkeypatch.setenv("FYNHIP_NO_ROWS_WIDE_CONV", "1")   # (the third form has a test of its own)
     b = conv_builder(k, cout, h, w, cin, 1, 1, A.RELU, **kw)
     wts = conv_block(800 + k, cout, k, cin, bn=kw.get("bn", False))
     inputs = [prng.uniform(31 * k + cin, (cin, h, w), -1, 1)]
@@ -212,6 +213,39 @@ def test_wide_kernel_few_output_channels(case, two_pass, storage, monkeypatch):
     assert "wide-kernel" in info
     one_launch = "summed in the epilogue" in info
     assert one_launch == (not two_pass and w + k - 1 > 16)
+    assert err <= TOL[storage], info
+
+
+ROWS_CASES = WIDE_CASES[:3] + [
+    (9, 3, 37, 113, 16, {"bn": True}),                                       # one k16 step per input row, ragged strips and rounds
+    (9, 3, 5, 60, 32, {"residual": (A.RELU, False)}),                        # fewer rows than one round of a full block
+    (9, 3, 300, 130, 32, {}),                                                # several row blocks per strip
+    (3, 4, 21, 64, 8, {}),
+    (5, 3, 44, 71, 24, {"pad_out": 2}),
+]
+
+
+@pytest.mark.parametrize("storage", [fa.STORAGE_F32, fa.STORAGE_F16], ids=["f32", "f16"])
+@pytest.mark.parametrize("shallow", [False, True], ids=["deep", "shallow_edge_clamp"])
+@pytest.mark.parametrize("case", ROWS_CASES, ids=lambda c: "k%d_%dx%dx%d_to%d" % (c[0], c[4], c[2], c[3], c[1]))
+def test_wide_kernel_row_rolling_form(case, shallow, storage, monkeypatch):
+    """The folded-kx convolution with the input rows rolled through an LDS ring and the weights held in registers."""
+    k, cout, h, w, cin, kw = case
+    if shallow and ("residual" in kw or "pad_out" in kw):
+        pytest.skip("the shallow variant is run on the plain cases")
+    monkeypatch.setenv("FYNHIP_FORCE_ROWS_WIDE_CONV", "1")
+    if shallow:   # unpadded shallow input: the sampler repeats the edge
+        kw = dict(kw, deep=False, pad_in=0)
+    b = conv_builder(k, cout, h, w, cin, 1, 1, A.RELU, **kw)
+    wts = conv_block(900 + k, cout, k, cin, bn=kw.get("bn", False))
+    inputs = [prng.uniform(41 * k + cin, (cin, h, w), -1, 1)]
+    if "residual" in kw:
+        inputs.append(prng.uniform(43, (cout, h, w), -1, 1))
+    got, info = run_single(b, storage, inputs, wts)
+    ref = oracle_single(b, storage, inputs, wts)
+    err = rel_l2(got, ref)
+    print("  ", info, "rel_l2=%.3e" % err, flush=True)
+    assert "conv_rows" in info
     assert err <= TOL[storage], info
 
 
