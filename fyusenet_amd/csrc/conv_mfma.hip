@@ -31,6 +31,7 @@
 #include <vector>
 
 #include "kernels.h"
+#include "range.h"
 
 // Timing-study builds (-DFYN_CONV_TRACE): wave 0 of every workgroup records the shader clock at phase boundaries.
 #ifdef FYN_CONV_TRACE
@@ -49,8 +50,9 @@ typedef float f32x4_t __attribute__((ext_vector_type(4)));
 // Branch-free activation: the host normalises every activation kind to
 //   act(x) = min(hi, max(lo, x)) + leak * min(x, 0)
 // (none: lo=-inf, hi=+inf, leak=0; ReLU: lo=0; leaky: lo=0, leak; clip: lo, hi).
+// (the clamp is one median-of-three instruction: lo <= hi always)
 __device__ __forceinline__ float act_apply(float x, const Act& a) {
-    return fminf(a.hi, fmaxf(a.lo, x)) + a.leak * fminf(x, 0.f);
+    return __builtin_amdgcn_fmed3f(x, a.lo, a.hi) + a.leak * fminf(x, 0.f);
 }
 
 template <typename T>
@@ -127,11 +129,12 @@ struct RawItem<_Float16, 4> {
 };
 
 // Activates, converts (hi / lo fp16 planes when SPLIT) and writes one staging item to LDS.
+// (SPLIT: `scale` is the power of two that moves the tensor's magnitudes into the window where hi + lo is exact)
 template <bool SPLIT, int CPI>
-__device__ __forceinline__ void stage_store(unsigned char* dst, int plane, const float* raw, const Act& act) {
+__device__ __forceinline__ void stage_store(unsigned char* dst, int plane, const float* raw, const Act& act, float scale) {
     float v[8];
 #pragma unroll
-    for (int i = 0; i < CPI; i++) v[i] = act_apply(raw[i], act);
+    for (int i = 0; i < CPI; i++) v[i] = SPLIT ? act_apply(raw[i], act) * scale : act_apply(raw[i], act);
     if (CPI == 8) {
         half8_t hi;
 #pragma unroll
@@ -230,6 +233,10 @@ __device__ __forceinline__ void conv_mfma_body(const ConvMfmaParams& p, unsigned
         if (bid < (per << 3)) bid = (bid & 7) * per + (bid >> 3);
     }
     FYN_TRACE(0);
+    // value ranges (range.h): read the input tensor's record (the records in this launch's care are cleared by the
+    // kernel entry points)
+    float in_scale = 1.f, inv_in_scale = 1.f;   // (set once the first tile's loads are on their way)
+    const unsigned range_bits = (SPLIT && p.in_amax) ? range_load(p.in_amax) : 0u;
     const int ntile_blocks = p.tiles_x * p.tiles_y * p.cout_blocks;
     const int ks = bid / ntile_blocks;           // split-K slice (0 without split-K)
     bid -= ks * ntile_blocks;
@@ -304,6 +311,8 @@ __device__ __forceinline__ void conv_mfma_body(const ConvMfmaParams& p, unsigned
     // consumed one step later, so the lookup never stalls the instruction stream.
     int* steptab = reinterpret_cast<int*>(lds);
     if (tid < p.nsteps * ((KC == 4) ? 4 : 1)) steptab[tid] = p.aoff[tid];   // (KC == 4: four tap offsets per step)
+    __shared__ unsigned range_box[2];   // meeting point of the waves' output maxima (range.h); zero before the first barrier
+    if (tid < 2) range_box[tid] = 0u;
     unsigned char* const sbase = lds + 1024;   // staging buffers follow the table
 
     // ---- staging machinery: items (pixel, 8-channel group) of the halo tile; the first NB items of a
@@ -353,7 +362,7 @@ __device__ __forceinline__ void conv_mfma_body(const ConvMfmaParams& p, unsigned
                 raw[i].get(v);
 #pragma unroll
                 for (int e = 0; e < CPI; e++) v[e] = ok ? v[e] : 0.f;
-                stage_store<SPLIT, CPI>(buf + l_off[i], p.plane, v, p.act);
+                stage_store<SPLIT, CPI>(buf + l_off[i], p.plane, v, p.act, in_scale);
             }
         }
     };
@@ -388,15 +397,17 @@ __device__ __forceinline__ void conv_mfma_body(const ConvMfmaParams& p, unsigned
                 if (lo2[i] >= 0) {
                     float v[8];
                     r2[i].get(v);
-                    stage_store<SPLIT, CPI>(buf + lo2[i], p.plane, v, p.act);
+                    stage_store<SPLIT, CPI>(buf + lo2[i], p.plane, v, p.act, in_scale);
                 }
             }
         }
     };
 
     // prologue: chunk 0 into buffer 0
+    if (stager) fetch_first(chunk0);
+    if (SPLIT && p.in_amax) in_scale = range_scale(range_after_act(range_reduce(range_bits), p.act), &inv_in_scale);
+    const float acc_mul = p.acc_mul * inv_in_scale;
     if (stager) {
-        fetch_first(chunk0);
         store_first(chunk0, sbase);
         stage_rest(chunk0, sbase);
     }
@@ -544,6 +555,7 @@ __device__ __forceinline__ void conv_mfma_body(const ConvMfmaParams& p, unsigned
                 bi4[o] = o < p.fuse_cout ? p.bias[o] : 0.f;
             }
             const float inv_nox = 1.0f / (float)nox;
+            float vmax = 0.f;
             for (int idx = tid & 255; idx < p.tile_h * nox; idx += 256) {
                 const int ty = (int)(((float)idx + 0.5f) * inv_nox);
                 const int tx = idx - ty * nox;
@@ -564,7 +576,8 @@ __device__ __forceinline__ void conv_mfma_body(const ConvMfmaParams& p, unsigned
                     float r = rv[o];
                     if (p.res_relu) r = fmaxf(r, 0.f);
                     if (p.res_scale) r *= sc4[o];
-                    v[o] = o < p.fuse_cout ? ((a[o] * p.acc_mul) * sc4[o] + bi4[o]) + r : 0.f;
+                    v[o] = o < p.fuse_cout ? ((a[o] * acc_mul) * sc4[o] + bi4[o]) + r : 0.f;
+                    vmax = fmaxf(vmax, fabsf(v[o]));
                 }
                 const size_t oidx = ((size_t)(p.out_off_y + py) * p.out_wp + p.out_off_x + px) * p.out_cp;
                 if (sizeof(TOut) == 4) {
@@ -576,6 +589,7 @@ __device__ __forceinline__ void conv_mfma_body(const ConvMfmaParams& p, unsigned
                     *reinterpret_cast<half4_t*>(reinterpret_cast<_Float16*>(outp) + oidx) = hv;
                 }
             }
+            if (SPLIT && p.out_amax) range_publish_waves(p.out_amax, vmax, range_box, 4);
             return;
         }
     }
@@ -613,7 +627,8 @@ __device__ __forceinline__ void conv_mfma_body(const ConvMfmaParams& p, unsigned
             for (int i = 0; i < ITW; i++) {
                 const int it = (WK == 1) ? i : i * WK + wk;
                 const int row = it * PPI + lane / LPP;
-                const f32x4_t v = row_from_lds(fn, it);
+                f32x4_t v = row_from_lds(fn, it);
+                if (SPLIT) v *= inv_in_scale;   // partial sums in the units the reduce pass expects (a power of two)
                 const int m = (wn * FN + fn) * 32 + row;
                 const int py = pos_y0 + (m >> twl), px = pos_x0 + (m & (TW - 1));
                 if (cp_ok && py < p.npos_y && px < p.npos_x)
@@ -668,7 +683,7 @@ __device__ __forceinline__ void conv_mfma_body(const ConvMfmaParams& p, unsigned
                 float rv = rres[fn][it][i];   // zero without a residual input
                 if (p.res_relu) rv = fmaxf(rv, 0.f);
                 if (p.res_scale) rv *= sc[i];
-                a4[fn][it][i] = ((a4[fn][it][i] * p.acc_mul) * sc[i] + bi[i]) + rv;
+                a4[fn][it][i] = ((a4[fn][it][i] * acc_mul) * sc[i] + bi[i]) + rv;
             }
     // pin the results in registers here: the compiler would otherwise sink the arithmetic (and the waits for
     // its inputs) into the predicated store regions below
@@ -677,6 +692,16 @@ __device__ __forceinline__ void conv_mfma_body(const ConvMfmaParams& p, unsigned
 #pragma unroll
         for (int it = 0; it < ITW; it++) asm volatile("" : "+v"(a4[fn][it]));
     FYN_TRACE(11);
+    if (SPLIT && p.out_amax) {
+        float vmax = 0.f;
+#pragma unroll
+        for (int fn = 0; fn < FN; fn++)
+#pragma unroll
+            for (int it = 0; it < ITW; it++)
+#pragma unroll
+                for (int i = 0; i < 4; i++) vmax = fmaxf(vmax, ok[fn][it] ? fabsf(a4[fn][it][i]) : 0.f);
+        range_publish_waves(p.out_amax, vmax, range_box, 4);
+    }
 #pragma unroll
     for (int fn = 0; fn < FN; fn++)
 #pragma unroll
@@ -699,12 +724,14 @@ __device__ __forceinline__ void conv_mfma_body(const ConvMfmaParams& p, unsigned
 template <typename TIn, typename TOut, bool SPLIT, int FM, int FN, int WM, int WN, int KC, int PD, int UNR>
 __global__ __launch_bounds__((FM * FN >= 2) ? 512 : 256) void conv_mfma_kernel(const ConvMfmaParams p) {
     extern __shared__ __align__(16) unsigned char lds[];
+    if (blockIdx.x == 0) range_clear(p.reset[0], p.reset[1], p.reset[2], p.reset[3], p.nreset);
     conv_mfma_body<TIn, TOut, SPLIT, FM, FN, WM, WN, KC, PD, UNR>(p, lds);
 }
 
 template <typename TIn, typename TOut, bool SPLIT, int FM, int FN, int WM, int WN, int KC, int PD, int UNR>
 __global__ __launch_bounds__((FM * FN >= 2) ? 512 : 256) void conv_mfma_multi_kernel(const ConvMfmaMulti P) {
     extern __shared__ __align__(16) unsigned char lds[];
+    if (blockIdx.x == 0 && blockIdx.y == 0) range_clear(P.sub[0].reset[0], P.sub[0].reset[1], P.sub[0].reset[2], P.sub[0].reset[3], P.sub[0].nreset);
     conv_mfma_body<TIn, TOut, SPLIT, FM, FN, WM, WN, KC, PD, UNR>(P.sub[blockIdx.y], lds);
 }
 

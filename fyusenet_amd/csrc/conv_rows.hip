@@ -17,6 +17,7 @@
 #include <hip/hip_runtime.h>
 
 #include "kernels.h"
+#include "range.h"
 
 // Timing-study builds (-DFYN_ROWS_TRACE): wave 0 and wave 4 of every workgroup record the shader clock at phase boundaries.
 #ifdef FYN_ROWS_TRACE
@@ -45,7 +46,7 @@ constexpr int ROWS_SCRATCH_PITCH = 29;
 // stores (finished output rows) stay in flight across it.  __syncthreads() would wait for them as well.
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
-__device__ __forceinline__ float act1r(float x, const Act& a) { return fminf(a.hi, fmaxf(a.lo, x)) + a.leak * fminf(x, 0.f); }
+__device__ __forceinline__ float act1r(float x, const Act& a) { return __builtin_amdgcn_fmed3f(x, a.lo, a.hi) + a.leak * fminf(x, 0.f); }
 
 template <typename T>
 __device__ __forceinline__ void load8(const T* src, float* v);
@@ -97,6 +98,14 @@ __global__ __launch_bounds__(512) void conv_rows_kernel(const ConvRowsParams p) 
     unsigned char* ring = lds;
     float* scratch = reinterpret_cast<float*>(lds + RING * ROWB) + (wave & 3) * (WC * sp);
 
+    // value ranges (range.h): clear the words assigned to this launch, read the input tensor's
+    __shared__ unsigned range_box[2];   // meeting point of the MFMA waves' output maxima; zero before the first barrier
+    if (tid < 2) range_box[tid] = 0u;
+    if (blockIdx.x == 0) range_clear(p.reset[0], p.reset[1], p.reset[2], p.reset[3], p.nreset);
+    float in_scale = 1.f, inv_in_scale = 1.f;
+    if (SPLIT && p.in_amax) in_scale = range_scale(range_after_act(range_reduce(range_load(p.in_amax)), p.act), &inv_in_scale);
+    const float acc_mul = p.acc_mul * inv_in_scale;
+
     // ---- staging: q row j (relative to y_begin) is stored input row in_y0 + y_begin + j ----
     const TIn* in = reinterpret_cast<const TIn*>(p.in);
     const int stid = tid & 255;
@@ -136,7 +145,7 @@ __global__ __launch_bounds__(512) void conv_rows_kernel(const ConvRowsParams p) 
             half8_t hi, lo;
 #pragma unroll
             for (int e = 0; e < 8; e++) {
-                const float a = act1r(bt.v[i][e], p.act);
+                const float a = SPLIT ? act1r(bt.v[i][e], p.act) * in_scale : act1r(bt.v[i][e], p.act);
                 hi[e] = (_Float16)a;
                 lo[e] = (_Float16)(a - (float)hi[e]);
             }
@@ -209,6 +218,7 @@ __global__ __launch_bounds__(512) void conv_rows_kernel(const ConvRowsParams p) 
         }
         return;
     }
+    float vmax = 0.f;   // largest magnitude this lane wrote
     for (int g = 0; g < nrounds; g++) {
         {
             const int yl = 4 * g + wave;          // output row relative to y_begin
@@ -299,7 +309,8 @@ __global__ __launch_bounds__(512) void conv_rows_kernel(const ConvRowsParams p) 
                         float r = rv[o];
                         if (p.res_relu) r = fmaxf(r, 0.f);
                         if (p.res_scale) r *= sc4[o];
-                        v[o] = o < p.cout ? ((a[o] * p.acc_mul) * sc4[o] + bi4[o]) + r : 0.f;
+                        v[o] = o < p.cout ? ((a[o] * acc_mul) * sc4[o] + bi4[o]) + r : 0.f;
+                        vmax = fmaxf(vmax, fabsf(v[o]));
                     }
                     const size_t oidx = ((size_t)(p.out_off_y + y) * p.out_wp + p.out_off_x + gx) * p.out_cp;
                     if (sizeof(TOut) == 4) {
@@ -317,6 +328,7 @@ __global__ __launch_bounds__(512) void conv_rows_kernel(const ConvRowsParams p) 
         lds_barrier();   // the round's rows are consumed, the next round's rows are in the ring
         FYN_RTRACE(5 + 3 * g);
     }
+    if (SPLIT && p.out_amax) range_publish_waves(p.out_amax, vmax, range_box, 4);
 }
 
 typedef void (*rows_fn)(const ConvRowsParams);

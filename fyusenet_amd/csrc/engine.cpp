@@ -1,5 +1,6 @@
 // Network graph, device tensor management and the forward loop.
 #include "engine.h"
+#include "range.h"
 
 #include <algorithm>
 #include <cstring>
@@ -360,13 +361,65 @@ void Net::setup() {
         t.v.ptr = b.ptr;
     }
     // pass-through layers were given the tensor id only; nothing else to do for them
+    assign_range_words();
     // 3. per-layer setup (weight packing, kernel selection)
     for (auto& kv : layers) {
         kv.second->setup();
         kv.second->set_up = true;
     }
+    assign_range_resets();
     FYN_HIP(hipStreamSynchronize(stream));
     is_setup = true;
+}
+
+// Value ranges (range.h), fp32 storage only.  A tensor gets a word when whoever writes it keeps the word up to date:
+// tensors fed from the host (set_input and the frame pipeline clear and raise the word themselves) and the outputs of
+// layers whose kernels do (tracks_range()).
+void Net::assign_range_words() {
+    if (f16() || getenv("FYNHIP_NO_RANGE_TRACKING") || getenv("FYNHIP_FORCE_DIRECT_CONV") || tensors.empty()) return;
+    amax_dev_ = static_cast<unsigned*>(dev_alloc(tensors.size() * RANGE_WORDS * sizeof(unsigned), true));
+    for (size_t i = 0; i < tensors.size(); i++) {
+        Tensor& t = tensors[i];
+        bool tracked = t.producer == -1;
+        if (t.producer >= 0) {
+            Layer* pl = layer(t.producer);
+            tracked = pl->d.type == FYN_LAYER_UPLOAD || pl->tracks_range();
+        }
+        if (tracked) t.amax = amax_dev_ + i * RANGE_WORDS;
+    }
+}
+
+// A word raised during a forward pass must read 0 again before the tensor's producer runs in the next pass.  The
+// clearing is given to a convolution kernel that runs after the tensor's last reader (kernels of one stream run one
+// after the other, so nothing else touches the word at that time): the first such layer behind the last reader,
+// wrapping around to the layers in front of the producer.  A tensor for which no layer is found loses its word.
+void Net::assign_range_resets() {
+    if (!amax_dev_) return;
+    std::vector<int> order;
+    for (auto& kv : layers) order.push_back(kv.first);
+    bool lost = false;
+    for (Tensor& t : tensors) {
+        if (!t.amax || t.producer < 0) continue;
+        Layer* pl = layer(t.producer);
+        if (pl->d.type == FYN_LAYER_UPLOAD) continue;   // cleared where it is written from the host
+        const int last = std::max(t.last_reader, t.producer);
+        bool done = false;
+        // layers behind the last reader, in execution order ...
+        for (int no : order)
+            if (no > last && layer(no)->add_range_reset(t.amax)) { done = true; break; }
+        // ... then the layers in front of the producer (they run in the next pass, before it)
+        if (!done)
+            for (int no : order)
+                if (no < t.producer && layer(no)->add_range_reset(t.amax)) { done = true; break; }
+        if (!done) {
+            t.amax = nullptr;
+            lost = true;
+        }
+    }
+    if (lost) {
+        // layers copied the word addresses into their kernel arguments during setup: let them look again
+        for (auto& kv : layers) kv.second->setup_ranges();
+    }
 }
 
 void Net::dump_layer(Layer* l) {
@@ -491,8 +544,10 @@ void Net::set_input(int layer_no, int port, const float* data, int order) {
     const size_t n = (size_t)v.c * v.h * v.w;
     float* st = staging(n);
     FYN_HIP(hipMemcpyAsync(st, data, n * sizeof(float), hipMemcpyHostToDevice, stream));
-    if (order == FYN_ORDER_CHANNELWISE) launch_chw_to_tensor(st, v, stream);
-    else if (order == FYN_ORDER_GPU_SHALLOW) launch_hwc_to_tensor(st, v.c, v, stream);
+    unsigned* amax = input_tensor(layer_no, port).amax;
+    if (amax) launch_fill_zero(amax, RANGE_WORDS * sizeof(unsigned), stream);   // the tensor's value-range record starts over
+    if (order == FYN_ORDER_CHANNELWISE) launch_chw_to_tensor(st, v, stream, amax);
+    else if (order == FYN_ORDER_GPU_SHALLOW) launch_hwc_to_tensor(st, v.c, v, stream, amax);
     else fail(FYN_ERR_UNSUPPORTED, "input order %d not supported for upload", order);
     FYN_HIP(hipGetLastError());
     // the host buffer is borrowed for this call only
@@ -755,8 +810,9 @@ void Net::async_submit(const float* in, float* out, uint64_t* ticket) {
     FYN_HIP(hipMemcpyAsync(s.dev_in, s.pin_in, async_in_floats_ * sizeof(float), hipMemcpyHostToDevice, up_stream_));
     FYN_HIP(hipEventRecord(s.up, up_stream_));
     FYN_HIP(hipStreamWaitEvent(stream, s.up, 0));
-    if (async_in_order_ == FYN_ORDER_CHANNELWISE) launch_chw_to_tensor(s.dev_in, async_in_->v, stream);
-    else launch_hwc_to_tensor(s.dev_in, async_in_->v.c, async_in_->v, stream);
+    if (async_in_->amax) launch_fill_zero(async_in_->amax, RANGE_WORDS * sizeof(unsigned), stream);   // the tensor's value-range record starts over
+    if (async_in_order_ == FYN_ORDER_CHANNELWISE) launch_chw_to_tensor(s.dev_in, async_in_->v, stream, async_in_->amax);
+    else launch_hwc_to_tensor(s.dev_in, async_in_->v.c, async_in_->v, stream, async_in_->amax);
     forward(nullptr);
     const TView& vo = async_out_view_;
     if (async_out_order_ == FYN_ORDER_CHANNELWISE) launch_tensor_to_chw(vo, s.dev_out, 0, stream);

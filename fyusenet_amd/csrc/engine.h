@@ -40,6 +40,7 @@ struct Tensor {
     int last_reader = -1;  // highest layer number reading it
     bool locked = false;   // never reused (network outputs, external inputs)
     int buffer = -1;       // index into Net::buffers_
+    unsigned* amax = nullptr;   // value-range word (range.h) when a producer keeps it, else null
 };
 
 struct DevBuffer {
@@ -71,6 +72,11 @@ class Layer {
     virtual void setup() {}
     virtual void forward(hipStream_t s) = 0;
     virtual std::string info() const { return "none"; }
+    // value ranges (range.h): whether this layer's kernels raise the word of their output tensor, and whether they can
+    // take on clearing another tensor's word (true: taken)
+    virtual bool tracks_range() const { return false; }
+    virtual bool add_range_reset(unsigned*) { return false; }
+    virtual void setup_ranges() {}   // (re)reads the words of the layer's tensors into its kernel arguments
     Act act() const;
     const Tensor& tin(int port) const;
     const Tensor& tout() const;
@@ -157,6 +163,9 @@ class Net {
     float* staging_ = nullptr;
     size_t staging_floats_ = 0;
     float* static_scratch_ = nullptr;   // this device's address of the fixed staging area
+    unsigned* amax_dev_ = nullptr;      // one value-range word per tensor
+    void assign_range_words();
+    void assign_range_resets();
     hipGraph_t graph_ = nullptr;
     hipGraphExec_t graph_exec_ = nullptr;
     bool graph_enabled_ = false;

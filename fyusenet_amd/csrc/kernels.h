@@ -87,6 +87,13 @@ struct ConvMfmaParams {
     // the tile, so tiles overlap by K - 1 columns (tile column step tile_w - K + 1) and q never leaves LDS.  scale
     // and bias are indexed by o then; out/res describe the real output.  Tiles with FM = WM = 1, WN = 4 only.
     int fuse_k, fuse_cout;
+    // Value ranges (range.h; fp32 storage only, any of them may be null): the word of the input tensor, read at kernel
+    // start; the word of the output tensor, raised by the epilogue; up to four words that workgroup 0 clears (tensors
+    // that are dead while this kernel runs).
+    const unsigned* in_amax;
+    unsigned* out_amax;
+    unsigned* reset[4];
+    int nreset;
 #ifdef FYN_CONV_TRACE
     long long* trace;    // timing-study builds only: 16 timestamps per workgroup
 #endif
@@ -143,6 +150,10 @@ struct ConvRowsParams {
     int strips, row_blocks, rows_per_block;   // grid = strips * row_blocks workgroups; rows_per_block is a multiple of 4
     int cout;
     float acc_mul;
+    const unsigned* in_amax;   // value-range words as in ConvMfmaParams
+    unsigned* out_amax;
+    unsigned* reset[4];
+    int nreset;
 #ifdef FYN_ROWS_TRACE
     long long* trace;     // timing-study builds only: 32 timestamps per workgroup and role
 #endif
@@ -239,6 +250,7 @@ struct ShiftReduceParams {
     const float* scale;
     const float* bias;
     int res_relu, res_scale;
+    unsigned* out_amax;        // value-range word of the output tensor or null (range.h)
 };
 void launch_shift_reduce(const ShiftReduceParams& p, hipStream_t s);
 
@@ -255,6 +267,7 @@ struct SplitKReduceParams {
     float acc_mul;
     const float* scale;
     const float* bias;
+    unsigned* out_amax;        // value-range word of the output tensor or null (range.h)
 };
 void launch_splitk_reduce(const SplitKReduceParams& p, hipStream_t s);
 
@@ -269,9 +282,10 @@ struct GemvParams {
 void launch_gemv(const GemvParams& p, hipStream_t s);
 
 // Layout conversion between the engine layout and CHW fp32 staging buffers.
-void launch_chw_to_tensor(const float* chw, const TView& t, hipStream_t s);               // net area only
+// (amax: value-range word of the tensor, raised by what is written, or null; range.h)
+void launch_chw_to_tensor(const float* chw, const TView& t, hipStream_t s, unsigned* amax = nullptr);   // net area only
 void launch_tensor_to_chw(const TView& t, float* chw, int include_padding, hipStream_t s);
-void launch_hwc_to_tensor(const float* hwc, int pc, const TView& t, hipStream_t s);       // GPU_SHALLOW in
+void launch_hwc_to_tensor(const float* hwc, int pc, const TView& t, hipStream_t s, unsigned* amax = nullptr);   // GPU_SHALLOW in
 void launch_tensor_to_hwc(const TView& t, float* hwc, int pc, hipStream_t s);             // GPU_SHALLOW out
 void launch_fill_zero(void* ptr, size_t bytes, hipStream_t s);
 

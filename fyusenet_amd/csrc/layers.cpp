@@ -841,6 +841,25 @@ class ConvLayer : public Layer {
         sr.scale = scale_dev; sr.bias = bias_dev;
         sr.res_relu = res_relu; sr.res_scale = res_scale;
     }
+    // value ranges (range.h)
+    bool tracks_range() const override { return !direct; }
+    void setup_ranges() override {
+        const unsigned* in_w = tin(0).amax;
+        unsigned* out_w = tout().amax;
+        launch.p.in_amax = in_w;
+        launch.p.out_amax = (launch.p.ksplit > 1 || (wide && !fused)) ? nullptr : out_w;   // the pass that writes the tensor raises its word
+        launch.red.out_amax = out_w;
+        sr.out_amax = out_w;
+        rp.in_amax = in_w;
+        rp.out_amax = out_w;
+    }
+    bool add_range_reset(unsigned* w) override {
+        if (direct || !set_up) return false;
+        int& n = rows ? rp.nreset : launch.p.nreset;
+        if (n >= 4) return false;
+        (rows ? rp.reset : launch.p.reset)[n++] = w;
+        return true;
+    }
     void setup_rows_wide(const TView& in_v, const TView& out_v, const TView* res_v, int res_relu, int res_scale) {
         const int r = (k - 1) / 2;
         ConvRowsParams q{};
@@ -1049,6 +1068,7 @@ class ConvLayer : public Layer {
             dp.w = wdirect_dev; dp.scale = scale_dev; dp.bias = bias_dev;
         }
         set_up = true;
+        setup_ranges();
         if (!block.empty()) pack();
     }
     void pack() {
@@ -1253,7 +1273,23 @@ class TransConvLayer : public Layer {
             }
         group = tune_mfma_group(net, subconvs, in_v, out_v, d.in_channels, oc, act(), scale_dev, bias_dev);
         set_up = true;
+        setup_ranges();
         if (!block.empty()) pack();
+    }
+    // value ranges (range.h): every parity reads the input's word and raises the output's; the first one clears
+    bool tracks_range() const override { return true; }
+    void setup_ranges() override {
+        for (auto& L : group.subs) {
+            L.p.in_amax = tin(0).amax;
+            L.p.out_amax = tout().amax;
+        }
+        group.sync();
+    }
+    bool add_range_reset(unsigned* w) override {
+        if (!set_up || group.subs.empty() || group.subs[0].p.nreset >= 4) return false;
+        group.subs[0].p.reset[group.subs[0].p.nreset++] = w;
+        group.sync();
+        return true;
     }
     void pack() {
         const float* bias = block.data();

@@ -11,6 +11,7 @@
 #include <cstdlib>
 
 #include "kernels.h"
+#include "range.h"
 
 namespace fynhip {
 
@@ -912,30 +913,34 @@ __global__ __launch_bounds__(256) void shift_reduce_kernel(const ShiftReducePara
     }
     __syncthreads();
     const int x = x0 + threadIdx.x;
-    if (x >= p.out.w) return;
-    float acc[4] = {0.f, 0.f, 0.f, 0.f};
-    for (int kx = 0; kx < p.k; kx++) {
-        const float* qp = sq + (threadIdx.x + kx) * pitch + kx;
+    float vmax = 0.f;
+    if (x < p.out.w) {
+        float acc[4] = {0.f, 0.f, 0.f, 0.f};
+        for (int kx = 0; kx < p.k; kx++) {
+            const float* qp = sq + (threadIdx.x + kx) * pitch + kx;
 #pragma unroll
-        for (int o = 0; o < 4; o++)
-            if (o < p.cout) acc[o] += qp[o * p.k];
-    }
-    float o4[4];
-#pragma unroll
-    for (int o = 0; o < 4; o++) o4[o] = (o < p.cout) ? (acc[o] * p.acc_mul) * p.scale[o] + p.bias[o] : 0.f;
-    if (p.res.ptr) {
-        float4 r = ld4<T>(reinterpret_cast<const T*>(p.res.ptr) + tv_off(p.res, y, x));
-        float rv[4] = {r.x, r.y, r.z, r.w};
-#pragma unroll
-        for (int o = 0; o < 4; o++) {
-            if (o >= p.cout) continue;
-            float v = rv[o];
-            if (p.res_relu) v = fmaxf(v, 0.f);
-            if (p.res_scale) v *= p.scale[o];
-            o4[o] += v;
+            for (int o = 0; o < 4; o++)
+                if (o < p.cout) acc[o] += qp[o * p.k];
         }
+        float o4[4];
+#pragma unroll
+        for (int o = 0; o < 4; o++) o4[o] = (o < p.cout) ? (acc[o] * p.acc_mul) * p.scale[o] + p.bias[o] : 0.f;
+        if (p.res.ptr) {
+            float4 r = ld4<T>(reinterpret_cast<const T*>(p.res.ptr) + tv_off(p.res, y, x));
+            float rv[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+            for (int o = 0; o < 4; o++) {
+                if (o >= p.cout) continue;
+                float v = rv[o];
+                if (p.res_relu) v = fmaxf(v, 0.f);
+                if (p.res_scale) v *= p.scale[o];
+                o4[o] += v;
+            }
+        }
+        st4<T>(reinterpret_cast<T*>(p.out.ptr) + tv_off(p.out, y, x), make_float4(o4[0], o4[1], o4[2], o4[3]));
+        vmax = fmaxf(fmaxf(fabsf(o4[0]), fabsf(o4[1])), fmaxf(fabsf(o4[2]), fabsf(o4[3])));
     }
-    st4<T>(reinterpret_cast<T*>(p.out.ptr) + tv_off(p.out, y, x), make_float4(o4[0], o4[1], o4[2], o4[3]));
+    if (p.out_amax) range_publish_block256(p.out_amax, vmax);   // (every thread takes part)
 }
 void launch_shift_reduce(const ShiftReduceParams& p, hipStream_t s) {
     const int tiles_x = (p.out.w + 255) / 256;
@@ -950,21 +955,27 @@ void launch_shift_reduce(const ShiftReduceParams& p, hipStream_t s) {
 // One thread converts four channels of one pixel; pixels are the fastest index, so that plane accesses are
 // contiguous across a wavefront (image-like tensors of up to 4 channels are contiguous on the packed side too).
 template <typename T>
-__global__ __launch_bounds__(256) void chw_to_tensor_kernel(const float* chw, const TView t) {
+__global__ __launch_bounds__(256) void chw_to_tensor_kernel(const float* chw, const TView t, unsigned* amax) {
     const size_t npix = (size_t)t.h * t.w;
     const size_t n = npix * (t.cp >> 2);
     const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
-    if (idx >= n) return;
-    const size_t pix = idx % npix;
-    const int c = (int)(idx / npix) * 4;
-    const int x = (int)(pix % t.w), y = (int)(pix / t.w);
-    float v[4];
+    float vmax = 0.f;
+    if (idx < n) {
+        const size_t pix = idx % npix;
+        const int c = (int)(idx / npix) * 4;
+        const int x = (int)(pix % t.w), y = (int)(pix / t.w);
+        float v[4];
 #pragma unroll
-    for (int i = 0; i < 4; i++) v[i] = c + i < t.c ? chw[(size_t)(c + i) * npix + pix] : 0.f;
-    st4<T>(reinterpret_cast<T*>(t.ptr) + tv_off(t, y, x) + c, make_float4(v[0], v[1], v[2], v[3]));
+        for (int i = 0; i < 4; i++) {
+            v[i] = c + i < t.c ? chw[(size_t)(c + i) * npix + pix] : 0.f;
+            vmax = fmaxf(vmax, fabsf(v[i]));
+        }
+        st4<T>(reinterpret_cast<T*>(t.ptr) + tv_off(t, y, x) + c, make_float4(v[0], v[1], v[2], v[3]));
+    }
+    if (amax) range_publish_block256(amax, vmax);   // (every thread takes part)
 }
-void launch_chw_to_tensor(const float* chw, const TView& t, hipStream_t s) {
-    FYN_DISPATCH_T(t.f16, chw_to_tensor_kernel, grid1d((size_t)t.h * t.w * (t.cp >> 2), 256), dim3(256), s, chw, t);
+void launch_chw_to_tensor(const float* chw, const TView& t, hipStream_t s, unsigned* amax) {
+    FYN_DISPATCH_T(t.f16, chw_to_tensor_kernel, grid1d((size_t)t.h * t.w * (t.cp >> 2), 256), dim3(256), s, chw, t, amax);
 }
 
 template <typename T>
@@ -990,18 +1001,22 @@ void launch_tensor_to_chw(const TView& t, float* chw, int include_padding, hipSt
 }
 
 template <typename T>
-__global__ __launch_bounds__(256) void hwc_to_tensor_kernel(const float* hwc, int pc, const TView t) {
+__global__ __launch_bounds__(256) void hwc_to_tensor_kernel(const float* hwc, int pc, const TView t, unsigned* amax) {
     const size_t n = (size_t)t.h * t.w * t.cp;
     const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
-    if (idx >= n) return;
-    const int c = (int)(idx % t.cp);
-    const size_t pix = idx / t.cp;
-    const int x = (int)(pix % t.w), y = (int)(pix / t.w);
-    const float v = (c < t.c && c < pc) ? hwc[pix * pc + c] : 0.f;
-    reinterpret_cast<T*>(t.ptr)[tv_off(t, y, x) + c] = (T)v;
+    float vmax = 0.f;
+    if (idx < n) {
+        const int c = (int)(idx % t.cp);
+        const size_t pix = idx / t.cp;
+        const int x = (int)(pix % t.w), y = (int)(pix / t.w);
+        const float v = (c < t.c && c < pc) ? hwc[pix * pc + c] : 0.f;
+        reinterpret_cast<T*>(t.ptr)[tv_off(t, y, x) + c] = (T)v;
+        vmax = fabsf(v);
+    }
+    if (amax) range_publish_block256(amax, vmax);   // (every thread takes part)
 }
-void launch_hwc_to_tensor(const float* hwc, int pc, const TView& t, hipStream_t s) {
-    FYN_DISPATCH_T(t.f16, hwc_to_tensor_kernel, grid1d((size_t)t.h * t.w * t.cp, 256), dim3(256), s, hwc, pc, t);
+void launch_hwc_to_tensor(const float* hwc, int pc, const TView& t, hipStream_t s, unsigned* amax) {
+    FYN_DISPATCH_T(t.f16, hwc_to_tensor_kernel, grid1d((size_t)t.h * t.w * t.cp, 256), dim3(256), s, hwc, pc, t, amax);
 }
 
 template <typename T>
@@ -1039,47 +1054,50 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const SplitKReducePa
     const int cq = p.cout_pad >> 2;
     const size_t n = (size_t)p.npos_y * p.npos_x * cq;
     const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
-    if (idx >= n) return;
     const int c = (int)(idx % cq) * 4;
-    if (c >= p.out_cp) return;
-    const size_t pos = idx / cq;
-    const int py = (int)(pos / p.npos_x), px = (int)(pos - (size_t)py * p.npos_x);
-    const size_t slice = (size_t)p.npos_y * p.npos_x * p.cout_pad;
-    // everything this thread reads is requested up front: residual, scale, bias and the first eight slices share
-    // one memory round trip
-    float rv[4] = {0.f, 0.f, 0.f, 0.f};
-    if (p.res) {
-        const TOut* res = reinterpret_cast<const TOut*>(p.res);
-        const size_t rbase = ((size_t)(p.res_off_y + py * p.out_step) * p.res_wp + p.res_off_x + px * p.out_step) * p.res_cp + c;
-        const float4 r = ld4<TOut>(res + rbase);
-        rv[0] = r.x; rv[1] = r.y; rv[2] = r.z; rv[3] = r.w;
-    }
-    const f32x4 sc = *reinterpret_cast<const f32x4*>(p.scale + c), bi = *reinterpret_cast<const f32x4*>(p.bias + c);
-    // slices are summed in slice order; their loads are issued eight at a time (one round trip per eight slices)
-    f32x4 a = (f32x4)(0.f);
-    const float* src = p.partial + pos * p.cout_pad + c;
-    for (int k0 = 0; k0 < p.ksplit; k0 += 8) {
-        f32x4 v[8];
-#pragma unroll
-        for (int j = 0; j < 8; j++) v[j] = *reinterpret_cast<const f32x4*>(src + (size_t)(k0 + j < p.ksplit ? k0 + j : k0) * slice);
-#pragma unroll
-        for (int j = 0; j < 8; j++)
-            if (k0 + j < p.ksplit) a += v[j];
-    }
-    float o[4];
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-        o[i] = (a[i] * p.acc_mul) * sc[i] + bi[i];
+    float vmax = 0.f;
+    if (idx < n && c < p.out_cp) {
+        const size_t pos = idx / cq;
+        const int py = (int)(pos / p.npos_x), px = (int)(pos - (size_t)py * p.npos_x);
+        const size_t slice = (size_t)p.npos_y * p.npos_x * p.cout_pad;
+        // everything this thread reads is requested up front: residual, scale, bias and the first eight slices share
+        // one memory round trip
+        float rv[4] = {0.f, 0.f, 0.f, 0.f};
         if (p.res) {
-            float r = rv[i];
-            if (p.res_relu) r = fmaxf(r, 0.f);
-            if (p.res_scale) r *= sc[i];
-            o[i] += r;
+            const TOut* res = reinterpret_cast<const TOut*>(p.res);
+            const size_t rbase = ((size_t)(p.res_off_y + py * p.out_step) * p.res_wp + p.res_off_x + px * p.out_step) * p.res_cp + c;
+            const float4 r = ld4<TOut>(res + rbase);
+            rv[0] = r.x; rv[1] = r.y; rv[2] = r.z; rv[3] = r.w;
         }
+        const f32x4 sc = *reinterpret_cast<const f32x4*>(p.scale + c), bi = *reinterpret_cast<const f32x4*>(p.bias + c);
+        // slices are summed in slice order; their loads are issued eight at a time (one round trip per eight slices)
+        f32x4 a = (f32x4)(0.f);
+        const float* src = p.partial + pos * p.cout_pad + c;
+        for (int k0 = 0; k0 < p.ksplit; k0 += 8) {
+            f32x4 v[8];
+#pragma unroll
+            for (int j = 0; j < 8; j++) v[j] = *reinterpret_cast<const f32x4*>(src + (size_t)(k0 + j < p.ksplit ? k0 + j : k0) * slice);
+#pragma unroll
+            for (int j = 0; j < 8; j++)
+                if (k0 + j < p.ksplit) a += v[j];
+        }
+        float o[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            o[i] = (a[i] * p.acc_mul) * sc[i] + bi[i];
+            if (p.res) {
+                float r = rv[i];
+                if (p.res_relu) r = fmaxf(r, 0.f);
+                if (p.res_scale) r *= sc[i];
+                o[i] += r;
+            }
+        }
+        TOut* out = reinterpret_cast<TOut*>(p.out);
+        const size_t obase = ((size_t)(p.out_off_y + py * p.out_step) * p.out_wp + p.out_off_x + px * p.out_step) * p.out_cp + c;
+        st4<TOut>(out + obase, make_float4(o[0], o[1], o[2], o[3]));
+        vmax = fmaxf(fmaxf(fabsf(o[0]), fabsf(o[1])), fmaxf(fabsf(o[2]), fabsf(o[3])));
     }
-    TOut* out = reinterpret_cast<TOut*>(p.out);
-    const size_t obase = ((size_t)(p.out_off_y + py * p.out_step) * p.out_wp + p.out_off_x + px * p.out_step) * p.out_cp + c;
-    st4<TOut>(out + obase, make_float4(o[0], o[1], o[2], o[3]));
+    if (p.out_amax) range_publish_block256(p.out_amax, vmax);   // (every thread takes part)
 }
 
 void launch_splitk_reduce(const SplitKReduceParams& p, hipStream_t s) {

@@ -117,3 +117,86 @@ def test_python_wrappers_check_buffer_sizes():
     net.asyncEnd()
     assert np.array_equal(out, y)
     net.cleanup()
+
+
+@pytest.mark.parametrize("magnitude", [1e5, 3e2, 1.0, 1e-5, 1e-9], ids=lambda m: "x%g" % m)
+@pytest.mark.parametrize("k,cin,cout", [(3, 64, 64), (1, 256, 32), (9, 32, 3), (9, 3, 32)])
+def test_fp32_storage_keeps_its_accuracy_over_the_value_range(magnitude, k, cin, cout):
+    """With fp32 storage the matrix path splits operands into fp16 pairs; the engine moves a tensor's magnitudes into
+    the window where the split is exact (a power of two taken from the largest magnitude written), so inputs far from
+    1 -- beyond fp16's largest number or deep in its subnormal range -- keep the 1e-4 bound against the oracle."""
+    from util import oracle_single, run_single
+    h, w = 24, 40
+    b = fa.ConvLayerBuilder(k, "conv").type(fa.LayerType.CONVOLUTION2D).number(1).shape(cout, h, w, cin).deep()
+    b.inputPadding((k - 1) // 2).prefixAct(A.RELU)
+    wts = conv_block(500 + k, cout, k, cin)
+    x = (prng.uniform(501, (cin, h, w), -1, 1) * magnitude).astype(np.float32)
+    got, info = run_single(b, fa.STORAGE_F32, [x], wts)
+    ref = oracle_single(b, fa.STORAGE_F32, [x], wts)
+    assert np.isfinite(got).all(), info
+    # (the bias of about 0.01 dominates the tiny cases; compare what the convolution adds to it as well)
+    bias = wts[:cout].astype(np.float64)[:, None, None]
+    assert rel_l2(got, ref) <= 1e-4, info
+    if magnitude >= 1e-5:
+        assert rel_l2(got.astype(np.float64) - bias, ref.astype(np.float64) - bias) <= 1e-4, info
+
+
+class _RangeChain(fa.NeuralNetwork):
+    """Three convolutions whose weights make the intermediate tensors huge (first layer x 3e5) and small again."""
+    H, W = 20, 24
+
+    def buildLayers(self, f):
+        H, W = self.H, self.W
+        fa.UpDownLayerBuilder(fa.UpDownLayerBuilder.UPLOAD, "in").number(0).shape(8, H, W, 8).outputPadding(1).push(f)
+        for no, (ci, co) in enumerate([(8, 32), (32, 32), (32, 16)], start=1):
+            b = fa.ConvLayerBuilder(3, "c%d" % no).type(fa.LayerType.CONVOLUTION2D).number(no).shape(co, H, W, ci).deep()
+            b.inputPadding(1).outputPadding(1 if no < 3 else 0).prefixAct(A.RELU if no > 1 else A.NONE)
+            if no == 3:
+                b.residual(A.RELU).residualPadding(0)
+            b.push(f)
+
+    def connectLayers(self, layers, bm):
+        bm.connectLayers(layers[0], layers[1], 0)
+        bm.connectLayers(layers[1], layers[2], 0)
+        bm.connectLayers(layers[2], layers[3], 0)
+
+    def initializeWeights(self, layers):
+        self.blocks = []
+        for no, (ci, co, gain) in enumerate([(8, 32, 3e5), (32, 32, 1.0), (32, 16, 1e-7)], start=1):
+            blk = conv_block(520 + 4 * no, co, 3, ci)
+            blk[co:] *= np.float32(gain)
+            layers[no].loadWeightsAndBiases(blk, 0)
+
+
+def test_value_range_words_start_over_every_frame():
+    """A frame's result does not depend on the frames before it: the per-tensor magnitude words are cleared between
+    passes (bit-identical outputs for a frame run after a frame of 1e6 times its magnitude and on a fresh network),
+    and the chain stays within the fp32-storage bound although its middle tensors reach 1e6."""
+    from oracle import oracle as O
+    small = prng.uniform(540, (8, _RangeChain.H, _RangeChain.W), -1, 1)
+    res = prng.uniform(541, (16, _RangeChain.H, _RangeChain.W), -1, 1)
+    huge = (small * 1e6).astype(np.float32)
+
+    def run(net, x, graph):
+        net.useGraph(graph)
+        net.layers[0].setInput(x, 0)
+        net.layers[3].setInput(res, 1)
+        net.forward()
+        net.finish()
+        return net.getOutput(3)
+
+    fresh = _RangeChain(fa.STORAGE_F32)
+    fresh.setup()
+    want = run(fresh, small, False)
+    ref = O.run_network(fresh.describe(), {(0, 0): small, (3, 1): res})[3]
+    assert rel_l2(want, ref) <= 1e-4
+    assert np.abs(fresh.layers[2].copyResult()).max() > 1e5     # the middle tensors are far beyond fp16's range
+    fresh.cleanup()
+    for graph in (False, True):
+        net = _RangeChain(fa.STORAGE_F32)
+        net.setup()
+        first = run(net, huge, graph)
+        assert np.isfinite(first).all()
+        again = run(net, small, graph)
+        net.cleanup()
+        assert np.array_equal(again, want), "graph=%s" % graph
