@@ -263,6 +263,118 @@ __global__ __launch_bounds__(256) void dwconv3x3_row_kernel(const DwConvParams p
     }
 }
 
+// The same convolution with a thread walking DOWN a strip of four output columns: the three input rows of a window
+// stay in registers (in their stored type, already activated) and every step fetches only the row(s) that enter the
+// window, one step ahead of their use, so an input texel is fetched 1.5 times (the strips' horizontal overlap) instead
+// of 4.5 times, and the nine weight vectors are loaded once per strip.  Same accumulation order per output as the
+// kernels above.  fp16 tensors: the activation must be a clamp that is exact on halves (no leak, bounds representable;
+// the caller checks), it is applied to the packed halves; products are formed from the halves with fp32 accumulation.
+template <typename T, int V, int S>
+__global__ __launch_bounds__(256) void dwconv3x3_col_kernel(const DwConvParams p, int rows_per_thread) {
+    constexpr int PX = 4, WIN = (PX - 1) * S + 3;
+    typedef RawV<T, V> Raw;
+    const int cg = p.out.cp / V;
+    const int xb = (p.out.w + PX - 1) / PX;
+    const int yb = (p.out.h + rows_per_thread - 1) / rows_per_thread;
+    const size_t n = (size_t)yb * xb * cg;
+    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= n) return;
+    const int g = (int)(idx % cg);
+    const size_t t = idx / cg;
+    const int bx = (int)(t % xb), by = (int)(t / xb);
+    const int c = g * V, x0 = bx * PX;
+    const int y_begin = by * rows_per_thread, y_end = min(y_begin + rows_per_thread, p.out.h);
+    const T* in = reinterpret_cast<const T*>(p.in.ptr);
+    const int iwp = p.in.wp(), ihp = p.in.hp();
+    const int sx0 = x0 * S + p.in.pad - 1;
+    const _Float16 hlo = (_Float16)p.act.lo, hhi = (_Float16)p.act.hi;
+    auto load_row = [&](Raw (&dst)[WIN], int sy) {
+        const bool row_ok = (unsigned)sy < (unsigned)ihp;
+#pragma unroll
+        for (int j = 0; j < WIN; j++) {
+            const int sx = sx0 + j;
+#pragma unroll
+            for (int i = 0; i < V; i++) dst[j].v[i] = (T)0.f;
+            if (row_ok && (unsigned)sx < (unsigned)iwp) dst[j] = *reinterpret_cast<const Raw*>(in + ((size_t)sy * iwp + sx) * p.in.cp + c);
+        }
+    };
+    auto activate = [&](Raw (&r)[WIN]) {
+#pragma unroll
+        for (int j = 0; j < WIN; j++) {
+            if constexpr (sizeof(T) == 2) {
+                typedef _Float16 halfv_t __attribute__((ext_vector_type(V)));
+                halfv_t h = __builtin_bit_cast(halfv_t, r[j]);
+                h = __builtin_elementwise_min(__builtin_elementwise_max(h, (halfv_t)hlo), (halfv_t)hhi);
+                r[j] = __builtin_bit_cast(Raw, h);
+            } else {
+#pragma unroll
+                for (int i = 0; i < V; i++) r[j].v[i] = (T)act1((float)r[j].v[i], p.act);
+            }
+        }
+    };
+    FV<V> w[9];
+#pragma unroll
+    for (int k = 0; k < 9; k++) w[k] = ldv<float, V>(p.w + k * p.out.cp + c);
+    const FV<V> sc = ldv<float, V>(p.scale + c), bi = ldv<float, V>(p.bias + c);
+    // window rows of output row y: stored rows y*S + pad - 1 + {0, 1, 2}
+    Raw win[3][WIN], nxt[S][WIN];
+    const int sy0 = y_begin * S + p.in.pad - 1;
+#pragma unroll
+    for (int ky = 0; ky < 3; ky++) load_row(win[ky], sy0 + ky);
+#pragma unroll
+    for (int ky = 0; ky < 3; ky++) activate(win[ky]);
+    for (int y = y_begin; y < y_end; y++) {
+        // the S rows that enter the window of the next output row are requested before this row is computed
+        if (y + 1 < y_end) {
+#pragma unroll
+            for (int q = 0; q < S; q++) load_row(nxt[q], (y + 1) * S + p.in.pad - 1 + (3 - S) + q);
+        }
+        FV<V> acc[PX];
+#pragma unroll
+        for (int px = 0; px < PX; px++) acc[px] = zerov<V>();
+#pragma unroll
+        for (int ky = 0; ky < 3; ky++)
+#pragma unroll
+            for (int kx = 0; kx < 3; kx++)
+#pragma unroll
+                for (int px = 0; px < PX; px++)
+#pragma unroll
+                    for (int i = 0; i < V; i++) acc[px].v[i] = fmaf((float)win[ky][px * S + kx].v[i], w[ky * 3 + kx].v[i], acc[px].v[i]);
+#pragma unroll
+        for (int px = 0; px < PX; px++) {
+            const int x = x0 + px;
+            if (x >= p.out.w) break;
+            FV<V> o;
+#pragma unroll
+            for (int i = 0; i < V; i++) o.v[i] = acc[px].v[i] * sc.v[i] + bi.v[i];
+            if (p.res.ptr) {
+                const FV<V> r = ldv<T, V>(reinterpret_cast<const T*>(p.res.ptr) + tv_off(p.res, y, x) + c);
+#pragma unroll
+                for (int i = 0; i < V; i++) {
+                    float rv = r.v[i];
+                    if (p.res_relu) rv = fmaxf(rv, 0.f);
+                    if (p.res_scale) rv *= sc.v[i];
+                    o.v[i] += rv;
+                }
+            }
+            stv<T, V>(reinterpret_cast<T*>(p.out.ptr) + tv_off(p.out, y, x) + c, o);
+        }
+        if (y + 1 < y_end) {
+            // slide the window down by S rows
+#pragma unroll
+            for (int q = 0; q < S; q++) activate(nxt[q]);
+#pragma unroll
+            for (int ky = 0; ky + S < 3; ky++)
+#pragma unroll
+                for (int j = 0; j < WIN; j++) win[ky][j] = win[ky + S][j];
+#pragma unroll
+            for (int q = 0; q < S; q++)
+#pragma unroll
+                for (int j = 0; j < WIN; j++) win[3 - S + q][j] = nxt[q][j];
+        }
+    }
+}
+
 template <typename T, int V>
 static void launch_dw_row(const DwConvParams& p, hipStream_t s) {
     const size_t n = (size_t)p.out.h * ((p.out.w + 3) / 4) * (p.out.cp / V);
@@ -270,9 +382,29 @@ static void launch_dw_row(const DwConvParams& p, hipStream_t s) {
     else hipLaunchKernelGGL((dwconv3x3_row_kernel<T, V, 2>), grid1d(n, 256), dim3(256), 0, s, p);
 }
 
+// strips of `rows` output rows per thread, when the image is tall enough to leave the chip enough threads
+template <typename T, int V>
+static bool launch_dw_col(const DwConvParams& p, hipStream_t s) {
+    if (getenv("FYNHIP_NO_DW_STRIPS")) return false;
+    const size_t per_row = (size_t)((p.out.w + 3) / 4) * (p.out.cp / V);
+    int rows = 16;
+    if (const char* e = getenv("FYNHIP_DW_ROWS")) rows = atoi(e);   // (experiments)
+    while (rows > 2 && per_row * ((p.out.h + rows - 1) / rows) < 256 * 256 * 2) rows /= 2;   // at least two waves per SIMD of work
+    if (rows < 4 || p.out.h < rows) return false;
+    const size_t n = per_row * ((p.out.h + rows - 1) / rows);
+    if (p.stride == 1) hipLaunchKernelGGL((dwconv3x3_col_kernel<T, V, 1>), grid1d(n, 256), dim3(256), 0, s, p, rows);
+    else hipLaunchKernelGGL((dwconv3x3_col_kernel<T, V, 2>), grid1d(n, 256), dim3(256), 0, s, p, rows);
+    return true;
+}
+
 void launch_dwconv3x3(const DwConvParams& p, hipStream_t s) {
     if (p.dil == 1 && (p.stride == 1 || p.stride == 2) && p.out.w >= 4) {
         const bool wide = (p.in.cp % 8 == 0) && (p.out.cp % 8 == 0) && (!p.res.ptr || p.res.cp % 8 == 0);
+        // a clamp that is exact on halves (the strip kernel applies it to the packed halves)
+        const _Float16 hlo = (_Float16)p.act.lo, hhi = (_Float16)p.act.hi;
+        const bool half_act = p.act.leak == 0.f && (float)hlo == p.act.lo && (float)hhi == p.act.hi;
+        if (p.out.f16 && half_act && launch_dw_col<_Float16, 4>(p, s)) return;
+        if (!p.out.f16 && launch_dw_col<float, 4>(p, s)) return;
         if (p.out.f16 && wide) launch_dw_row<_Float16, 8>(p, s);
         else if (p.out.f16) launch_dw_row<_Float16, 4>(p, s);
         else launch_dw_row<float, 4>(p, s);
