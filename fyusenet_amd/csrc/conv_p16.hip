@@ -1,0 +1,373 @@
+// 3x3 convolution between wide layers with fp32 storage (the residual blocks of a style-transfer net) as an
+// implicit GEMM on gfx950 matrix cores with 16-position fragments (v_mfma_f32_16x16x32_f16, fp32 accumulate).
+//
+// Replaces, for such layers, the render passes of DeepConvLayerNxN::forward (fyusenet/gpu/deep/deepconvlayerNxN.cpp:
+// 129-211); epilogue order of shaders/deep/deepconv3x3_tiled.frag:36-45 (acc*scale + bias, then the residual).
+//
+// Why a second MFMA kernel: with 32x32 fragments a workgroup's tile is a multiple of 32 positions, and a layer of
+// 128x156 positions then fills 208 of the 256 CUs for three fragment rounds.  16-position fragments allow tiles of
+// 8x10 positions: 16x16 = 256 workgroups, one per CU, five fragments each (the work of 2.5 of the larger ones).
+//
+// GEMM view as in conv_mfma.hip: M = output channels (A = weights, packed per lane, streamed through L2 into a register
+// ring), N = positions (B = activations, staged per 32-channel chunk as a halo tile in LDS, fp16 hi and lo planes),
+// K = taps x input channels, one tap of one chunk (32 channels) per step.  Three MFMAs per fragment pair (hi*hi,
+// lo*hi, hi*lo).  Tile size, halo pitch and the tap offsets are compile-time constants, so a B fragment read is one
+// LDS instruction with an immediate offset and the step loop has no address arithmetic.
+//
+// Workgroup = 4 staging waves (next chunk: global loads, activation, hi/lo conversion, LDS writes; scale and bias at
+// the start and, during the last chunk, the residual tile into LDS) + 4 MFMA waves (32 output channels each: 2 channel
+// fragments x FN position fragments).  A lane's accumulators of one fragment are 4 consecutive output channels of one
+// position, so the epilogue needs no transposition: residual and scale/bias from LDS, one 16-byte store per fragment.
+#include <hip/hip_fp16.h>
+#include <hip/hip_runtime.h>
+
+#include "kernels.h"
+#include "range.h"
+
+// Timing-study builds (-DFYN_P16_TRACE): wave 0 and wave 4 of every workgroup record the shader clock at phase boundaries.
+#ifdef FYN_P16_TRACE
+#include <cstdio>
+#include <cstdlib>
+#include <vector>
+#define FYN_PTRACE(slot) do { if (lane == 0 && (wave & 3) == 0 && (slot) < 32) p.trace[((size_t)blockIdx.x * 2 + 1 - (wave >> 2)) * 32 + (slot)] = clock64(); } while (0)
+#else
+#define FYN_PTRACE(slot) do { } while (0)
+#endif
+
+namespace fynhip {
+
+namespace {
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+
+// Workgroup barrier that orders LDS traffic only (global loads and stores stay in flight across it).
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+__device__ __forceinline__ float act_p16(float x, const Act& a) { return __builtin_amdgcn_fmed3f(x, a.lo, a.hi) + a.leak * fminf(x, 0.f); }
+
+constexpr int KC = 32;        // input channels per chunk
+constexpr int NT = 9;         // taps
+constexpr int PD = 6;         // depth of the weight-fragment ring (steps)
+constexpr int UNR = 2 * NT;   // steps per unrolled group: two chunks (one per staging buffer)
+constexpr int CPB = 128;      // output channels per workgroup
+
+template <int TH, int TW>
+struct Geo {
+    static constexpr int HW = TW + 2, HH = TH + 2;
+    static constexpr int PITCH = KC * 2 + 16;            // bytes per staged pixel and plane: 8 neighbouring lanes' 16-byte reads cover all banks
+    static constexpr int ROW_PITCH = HW * PITCH + 96;    // (+96: the 16 positions of a fragment span up to four tile rows; with this pad their reads fall into distinct banks)
+    static constexpr int PLANE = HH * ROW_PITCH;
+    static constexpr int BUF = 2 * PLANE;                // hi, lo
+    static constexpr int NPOS = TH * TW, FN = NPOS / 16;
+    static constexpr int NITEMS = HH * HW * (KC / 8);    // staging items: (pixel, 8 channels)
+    static constexpr int NB = (NITEMS + 255) / 256;      // ... per staging thread
+    static constexpr int SB_OFF = 2 * BUF;               // scale[128], bias[128]
+    static constexpr int RES_OFF = SB_OFF + 2 * CPB * 4;
+    static constexpr int RES_PITCH = CPB * 4 + 16;       // bytes per position of the residual tile
+    static constexpr int RNB = NPOS * (CPB / 4) / 256;   // residual 16-byte pieces per staging thread
+    static constexpr int LDS = RES_OFF + NPOS * RES_PITCH;
+    static_assert(NPOS % 16 == 0, "whole position fragments");
+    static_assert((NPOS * (CPB / 4)) % 256 == 0, "residual pieces divide among the staging threads");
+    static_assert(2 * BUF + 2 * ROW_PITCH + 2 * PITCH + 64 < 65536, "B fragment offsets fit the LDS instructions' immediate field");
+};
+
+template <int TH, int TW>
+__global__ __launch_bounds__(512) void conv_p16_kernel(const ConvP16Params p) {
+    using G = Geo<TH, TW>;
+    constexpr int FN = G::FN;
+    extern __shared__ __align__(16) unsigned char lds[];
+    __shared__ unsigned range_box[2];   // meeting point of the MFMA waves' output maxima (range.h)
+    if (blockIdx.x == 0) range_clear(p.reset[0], p.reset[1], p.reset[2], p.reset[3], p.nreset);
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    // Workgroups are dealt round-robin to the 8 XCDs; remap so that neighbouring tiles (shared halos) meet in one L2.
+    int bid = blockIdx.x;
+    {
+        const int nblk = p.tiles_x * p.tiles_y * p.cout_blocks;
+        const int per = nblk >> 3;
+        if (bid < (per << 3)) bid = (bid & 7) * per + (bid >> 3);
+    }
+    const int cb = bid % p.cout_blocks;
+    const int tile = bid / p.cout_blocks;
+    const int tyi = tile / p.tiles_x, txi = tile - tyi * p.tiles_x;
+    const int pos_y0 = tyi * TH, pos_x0 = txi * TW;
+    if (tid < 2) range_box[tid] = 0u;
+    const unsigned range_bits = p.in_amax ? range_load(p.in_amax) : 0u;
+    const int nchunks = p.cin_chunks;   // even (checked at launch)
+
+    if (wave < 4) {
+        // ------------------------------------------------------------------ staging waves (the first four: they start first)
+        const int stid = tid & 255;
+        const float* in = reinterpret_cast<const float*>(p.in);
+        int g_off[G::NB], l_off[G::NB];
+#pragma unroll
+        for (int i = 0; i < G::NB; i++) {
+            const int idx = stid + i * 256;
+            g_off[i] = -1; l_off[i] = -1;
+            if (idx < G::NITEMS) {
+                const int pix = idx >> 2, g = idx & 3;
+                const int py = pix / G::HW, px = pix - py * G::HW;
+                int gy = pos_y0 + p.in_y0 + py, gx = pos_x0 + p.in_x0 + px;
+                l_off[i] = py * G::ROW_PITCH + px * G::PITCH + g * 16;
+                if (p.in_clamp) {
+                    gy = min(max(gy, 0), p.in_hp - 1);
+                    gx = min(max(gx, 0), p.in_wp - 1);
+                }
+                if ((unsigned)gy < (unsigned)p.in_hp && (unsigned)gx < (unsigned)p.in_wp) g_off[i] = (gy * p.in_wp + gx) * p.in_cp + g * 8;
+            }
+        }
+        float4 raw[G::NB][2];
+        // (unconditional loads: items outside the tensor read its first element and are zeroed when stored)
+        auto fetch = [&](int chunk) {
+#pragma unroll
+            for (int i = 0; i < G::NB; i++) {
+                const float* src = in + (g_off[i] >= 0 ? g_off[i] + chunk * KC : 0);
+                raw[i][0] = *reinterpret_cast<const float4*>(src);
+                raw[i][1] = *reinterpret_cast<const float4*>(src + 4);
+            }
+        };
+        float in_scale = 1.f, inv_unused;
+        auto store = [&](unsigned char* buf) {
+#pragma unroll
+            for (int i = 0; i < G::NB; i++) {
+                if (l_off[i] < 0) continue;
+                const bool ok = g_off[i] >= 0;
+                const float r[8] = {raw[i][0].x, raw[i][0].y, raw[i][0].z, raw[i][0].w, raw[i][1].x, raw[i][1].y, raw[i][1].z, raw[i][1].w};
+                half8_t hi, lo;
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    const float v = ok ? act_p16(r[e], p.act) * in_scale : 0.f;
+                    hi[e] = (_Float16)v;
+                    lo[e] = (_Float16)(v - (float)hi[e]);
+                }
+                *reinterpret_cast<half8_t*>(buf + l_off[i]) = hi;
+                *reinterpret_cast<half8_t*>(buf + G::PLANE + l_off[i]) = lo;
+            }
+        };
+        FYN_PTRACE(0);
+        fetch(0);
+        if (p.in_amax) in_scale = range_scale(range_after_act(range_reduce(range_bits), p.act), &inv_unused);
+        if (stid < CPB) {
+            reinterpret_cast<float*>(lds + G::SB_OFF)[stid] = p.scale[cb * CPB + stid];
+            reinterpret_cast<float*>(lds + G::SB_OFF)[CPB + stid] = p.bias[cb * CPB + stid];
+        }
+        store(lds);
+        FYN_PTRACE(1);
+        lds_barrier();
+        for (int c = 0; c < nchunks; c++) {
+            FYN_PTRACE(2 + 2 * c);
+            if (c + 1 < nchunks) {
+                fetch(c + 1);
+                store(lds + ((c + 1) & 1) * G::BUF);
+                FYN_PTRACE(3 + 2 * c);
+            } else if (p.res) {
+                // the residual tile: [position][128 channels] fp32
+                const float* res = reinterpret_cast<const float*>(p.res);
+                f32x4_t rv[G::RNB];
+#pragma unroll
+                for (int i = 0; i < G::RNB; i++) {
+                    const int idx = stid + i * 256;
+                    const int m = idx >> 5, c4 = idx & 31;
+                    const int ty = m / TW, tx = m - ty * TW;
+                    const int py = pos_y0 + ty, px = pos_x0 + tx;
+                    const bool ok = py < p.npos_y && px < p.npos_x;
+                    rv[i] = *reinterpret_cast<const f32x4_t*>(res + (ok ? ((size_t)(p.res_off_y + py) * p.res_wp + p.res_off_x + px) * p.res_cp + cb * CPB + c4 * 4 : 0));
+                }
+#pragma unroll
+                for (int i = 0; i < G::RNB; i++) {
+                    const int idx = stid + i * 256;
+                    *reinterpret_cast<f32x4_t*>(lds + G::RES_OFF + (idx >> 5) * G::RES_PITCH + (idx & 31) * 16) = rv[i];
+                }
+            }
+            lds_barrier();
+        }
+        return;
+    }
+
+    // ---------------------------------------------------------------------- MFMA waves
+    FYN_PTRACE(0);
+    const int mq = lane & 15, kq = lane >> 4;
+    const int mw = wave - 4;   // this wave's 32 output channels of the workgroup's 128
+    int bbase[FN];   // per-lane LDS offset of the B fragments: position, then the lane's 8 channels of the chunk
+#pragma unroll
+    for (int fn = 0; fn < FN; fn++) {
+        const int m = fn * 16 + mq;
+        const int ty = m / TW, tx = m - ty * TW;
+        bbase[fn] = ty * G::ROW_PITCH + tx * G::PITCH + kq * 16;
+    }
+    // A fragments: [(chunk*9 + tap)][cout fragment of 16][plane][lane] x 8 halves; the buffer has PD steps of zero
+    // slack behind the last step, so the prefetch needs no clamp.
+    const unsigned wstep = (unsigned)p.mfrags * 2 * 1024;
+    const unsigned char* wbase = reinterpret_cast<const unsigned char*>(p.wpack) + (size_t)((cb * 8 + mw * 2) * 2) * 1024 + lane * 16;
+    half8_t a_q[PD][2][2];
+#pragma unroll
+    for (int d = 0; d < PD; d++)
+#pragma unroll
+        for (int fm = 0; fm < 2; fm++)
+#pragma unroll
+            for (int pl = 0; pl < 2; pl++) a_q[d][fm][pl] = *reinterpret_cast<const half8_t*>(wbase + (size_t)d * wstep + (fm * 2 + pl) * 1024);
+    f32x4_t acc[2][FN];
+#pragma unroll
+    for (int fm = 0; fm < 2; fm++)
+#pragma unroll
+        for (int fn = 0; fn < FN; fn++) acc[fm][fn] = (f32x4_t)(0.f);
+    float inv_in_scale = 1.f;
+    if (p.in_amax) (void)range_scale(range_after_act(range_reduce(range_bits), p.act), &inv_in_scale);
+    const float acc_mul = p.acc_mul * inv_in_scale;
+
+    FYN_PTRACE(1);
+    lds_barrier();   // chunk 0 is staged
+    FYN_PTRACE(2);
+    half8_t b[FN][2];
+#pragma unroll
+    for (int fn = 0; fn < FN; fn++)
+#pragma unroll
+        for (int pl = 0; pl < 2; pl++) b[fn][pl] = *reinterpret_cast<const half8_t*>(lds + bbase[fn] + pl * G::PLANE);
+
+    // One slot per MFMA: the MFMA, then a share of the step's memory instructions, fenced so that the compiler keeps
+    // the order (a memory instruction issued right after an MFMA runs in its shadow).  Position fragment fn is used
+    // by six consecutive MFMAs; its registers are then refilled with the fragment of the next step, so one register
+    // set per fragment is enough.  The ring slot of the previous step is refilled with the weights of step t+PD-1.
+    // The barrier of a chunk sits in its last step, before the first read of the next chunk's buffer: the staging
+    // waves have filled that buffer by then, and all reads of the current buffer were issued a step earlier.
+    const unsigned char* wnext = wbase + (size_t)(PD - 1) * wstep;
+    for (int g = 0; g < nchunks; g += 2) {
+#pragma unroll
+        for (int dd = 0; dd < UNR; dd++) {
+            const int d = dd % PD, dprev = (d + PD - 1) % PD;
+            const int nd = (dd + 1) % UNR;                       // the next step: buffer and tap
+            const int ntap = nd % NT;
+            const int noff = (nd / NT) * G::BUF + (ntap / 3) * G::ROW_PITCH + (ntap % 3) * G::PITCH;
+            const unsigned char* w_ = wnext;
+            wnext += wstep;
+#pragma unroll
+            for (int i = 0; i < 6 * FN; i++) {
+                const int fn = i / 6, r = i % 6, kind = r / 2, fm = r % 2;
+                const int apl = (kind == 1) ? 1 : 0, bpl = (kind == 2) ? 1 : 0;
+                acc[fm][fn] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_q[d][fm][apl], b[fn][bpl], acc[fm][fn], 0, 0, 0);
+                if (dd % NT == NT - 1 && i == 3) lds_barrier();
+                if (r == 5) {
+                    b[fn][0] = *reinterpret_cast<const half8_t*>(lds + bbase[fn] + noff);
+                    b[fn][1] = *reinterpret_cast<const half8_t*>(lds + bbase[fn] + noff + G::PLANE);
+                }
+#pragma unroll
+                for (int j = 0; j < 4; j++)   // the four weight fragments of a step, spread over its slots
+                    if (i == (j * 6 * FN) / 4 + 1) a_q[dprev][j % 2][j / 2] = *reinterpret_cast<const half8_t*>(w_ + ((j % 2) * 2 + j / 2) * 1024);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            if (dd % NT == NT - 1) FYN_PTRACE(3 + g + dd / NT);
+        }
+    }
+
+    // ---- epilogue: a lane holds, per fragment, output channels 4*kq .. 4*kq+3 of position fn*16 + mq.  One wave per
+    //      SIMD pays four cycles per vector instruction, so the arithmetic is kept short (acc_mul is a power of two:
+    //      folding it into the scale changes no bit) and every fragment is stored as soon as it is finished. ----
+    const float* sb = reinterpret_cast<const float*>(lds + G::SB_OFF);
+    f32x4_t sc[2], bi[2], scm[2];
+#pragma unroll
+    for (int fm = 0; fm < 2; fm++) {
+        sc[fm] = *reinterpret_cast<const f32x4_t*>(sb + mw * 32 + fm * 16 + kq * 4);
+        bi[fm] = *reinterpret_cast<const f32x4_t*>(sb + CPB + mw * 32 + fm * 16 + kq * 4);
+        scm[fm] = sc[fm] * acc_mul;
+    }
+    float* out = reinterpret_cast<float*>(p.out);
+    const bool have_res = p.res != nullptr;
+    const bool res_relu = p.res_relu != 0, res_scale = p.res_scale != 0;
+    float vmax = 0.f;
+    FYN_PTRACE(29);
+#pragma unroll
+    for (int fn = 0; fn < FN; fn++) {
+        const int m = fn * 16 + mq;
+        const int ty = m / TW, tx = m - ty * TW;
+        const int py = pos_y0 + ty, px = pos_x0 + tx;
+        const bool ok = py < p.npos_y && px < p.npos_x;
+        const size_t obase = ((size_t)(p.out_off_y + py) * p.out_wp + p.out_off_x + px) * p.out_cp + cb * CPB + mw * 32 + kq * 4;
+        float fmax_ = 0.f;
+#pragma unroll
+        for (int fm = 0; fm < 2; fm++) {
+            f32x4_t v;
+#pragma unroll
+            for (int e = 0; e < 4; e++) v[e] = acc[fm][fn][e] * scm[fm][e] + bi[fm][e];
+            if (have_res) {
+                f32x4_t rv = *reinterpret_cast<const f32x4_t*>(lds + G::RES_OFF + m * G::RES_PITCH + (mw * 32 + fm * 16 + kq * 4) * 4);
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    float r = rv[e];
+                    if (res_relu) r = fmaxf(r, 0.f);
+                    if (res_scale) r *= sc[fm][e];
+                    v[e] += r;
+                }
+            }
+#pragma unroll
+            for (int e = 0; e < 4; e++) fmax_ = fmaxf(fmax_, fabsf(v[e]));
+            if (ok) *reinterpret_cast<f32x4_t*>(out + obase + fm * 16) = v;
+        }
+        vmax = fmaxf(vmax, ok ? fmax_ : 0.f);
+    }
+    FYN_PTRACE(30);
+    if (p.out_amax) range_publish_waves(p.out_amax, vmax, range_box, 4);
+    FYN_PTRACE(31);
+}
+
+typedef void (*p16_fn)(const ConvP16Params);
+struct P16Entry {
+    int th, tw;
+    p16_fn fn;
+    size_t lds;
+};
+template <int TH, int TW>
+constexpr P16Entry entry() { return P16Entry{TH, TW, conv_p16_kernel<TH, TW>, (size_t)Geo<TH, TW>::LDS}; }
+const P16Entry kEntries[] = {entry<8, 10>(), entry<10, 8>(), entry<8, 8>(), entry<8, 6>(), entry<4, 8>(), entry<4, 4>()};
+}  // namespace
+
+int conv_p16_tile_count() { return (int)(sizeof(kEntries) / sizeof(kEntries[0])); }
+void conv_p16_tile(int index, int* th, int* tw, size_t* lds) {
+    *th = kEntries[index].th; *tw = kEntries[index].tw; *lds = kEntries[index].lds;
+}
+
+bool conv_p16_supported(int k, int stride, int dil, int in_cp, int cout, int out_cp, bool f16) {
+    return k == 3 && stride == 1 && dil == 1 && !f16 && in_cp % (2 * KC) == 0 && cout % CPB == 0 && out_cp % 4 == 0 && out_cp >= cout;
+}
+
+int launch_conv_p16(const ConvP16Params& p, hipStream_t s) {
+    const P16Entry* e = nullptr;
+    for (const P16Entry& c : kEntries)
+        if (c.th == p.tile_h && c.tw == p.tile_w) e = &c;
+    if (!e) return -1;
+    // what the kernel's indexing assumes
+    if (p.cin_chunks < 2 || p.cin_chunks % 2 || p.in_cp != p.cin_chunks * KC || p.cout_blocks < 1 || p.mfrags < p.cout_blocks * 8 ||
+        p.tiles_x * p.tile_w < p.npos_x || p.tiles_y * p.tile_h < p.npos_y || p.out_cp < p.cout_blocks * CPB ||
+        (p.res && p.res_cp < p.cout_blocks * CPB) || p.nreset < 0 || p.nreset > 4)
+        return -5;
+    if (e->lds > 160 * 1024) return -2;
+    if (e->lds > 48 * 1024) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(e->fn), hipFuncAttributeMaxDynamicSharedMemorySize, (int)e->lds) != hipSuccess) return -2;
+    }
+#ifdef FYN_P16_TRACE
+    {
+        static long long* dev = nullptr;
+        const size_t n = (size_t)p.tiles_x * p.tiles_y * p.cout_blocks * 64;
+        if (!dev && hipMalloc(&dev, sizeof(long long) * 65536 * 64) != hipSuccess) return -6;
+        ConvP16Params q = p;
+        q.trace = dev;
+        if (const char* e = getenv("FYNHIP_P16_CHUNKS")) q.cin_chunks = atoi(e);   // (timing study: fewer chunks, wrong results)
+        hipLaunchKernelGGL(e->fn, dim3(p.tiles_x * p.tiles_y * p.cout_blocks), dim3(512), e->lds, s, q);
+        hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+        (void)hipStreamIsCapturing(s, &cap);
+        const char* path = cap == hipStreamCaptureStatusNone ? getenv("FYNHIP_TRACE_DUMP") : nullptr;
+        if (path) {
+            std::vector<long long> h(n);
+            if (hipStreamSynchronize(s) == hipSuccess && hipMemcpy(h.data(), dev, n * 8, hipMemcpyDeviceToHost) == hipSuccess) {
+                if (FILE* f = fopen(path, "wb")) { fwrite(h.data(), 8, n, f); fclose(f); }
+            }
+        }
+        return hipGetLastError() == hipSuccess ? 0 : -3;
+    }
+#endif
+    hipLaunchKernelGGL(e->fn, dim3(p.tiles_x * p.tiles_y * p.cout_blocks), dim3(512), e->lds, s, p);
+    return hipGetLastError() == hipSuccess ? 0 : -3;
+}
+
+}  // namespace fynhip

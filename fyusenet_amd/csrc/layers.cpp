@@ -852,13 +852,104 @@ class ConvLayer : public Layer {
         sr.out_amax = out_w;
         rp.in_amax = in_w;
         rp.out_amax = out_w;
+        pp.in_amax = in_w;
+        pp.out_amax = out_w;
     }
     bool add_range_reset(unsigned* w) override {
         if (direct || !set_up) return false;
-        int& n = rows ? rp.nreset : launch.p.nreset;
+        int& n = rows ? rp.nreset : (p16 ? pp.nreset : launch.p.nreset);
         if (n >= 4) return false;
-        (rows ? rp.reset : launch.p.reset)[n++] = w;
+        (rows ? rp.reset : (p16 ? pp.reset : launch.p.reset))[n++] = w;
         return true;
+    }
+    // 16-position-fragment form of a 3x3 convolution (conv_p16.hip): the compiled tile that needs the fewest fragment
+    // rounds on 256 CUs, kept when it is faster than the tuned launch of the general kernel.
+    void setup_p16(const TView& in_v, const TView& out_v, const TView* res_v, int res_relu, int res_scale) {
+        ConvP16Params q{};
+        q.in = in_v.ptr; q.out = out_v.ptr; q.res = res_v ? res_v->ptr : nullptr;
+        q.in_hp = in_v.hp(); q.in_wp = in_v.wp(); q.in_cp = in_v.cp;
+        q.in_y0 = q.in_x0 = in_v.pad - 1;
+        q.in_clamp = clamp ? 1 : 0;
+        q.npos_y = oh; q.npos_x = ow;
+        q.out_wp = out_v.wp(); q.out_cp = out_v.cp; q.out_off_y = q.out_off_x = out_v.pad;
+        if (res_v) { q.res_wp = res_v->wp(); q.res_cp = res_v->cp; q.res_off_y = q.res_off_x = res_v->pad; }
+        q.res_relu = res_relu; q.res_scale = res_scale;
+        q.cin_chunks = in_v.cp / 32;
+        q.cout_blocks = oc / 128;
+        q.mfrags = q.cout_blocks * 8;
+        q.scale = scale_dev; q.bias = bias_dev;
+        q.acc_mul = 1.f;
+        q.act = act();
+        double best = 1e30;
+        int want_h = 0, want_w = 0;   // FYNHIP_P16_TILE=h,w (tests): that tile
+        if (const char* e = getenv("FYNHIP_P16_TILE")) sscanf(e, "%d,%d", &want_h, &want_w);
+        for (int i = 0; i < conv_p16_tile_count(); i++) {
+            int th, tw;
+            size_t lds;
+            conv_p16_tile(i, &th, &tw, &lds);
+            if (lds > 160 * 1024 || (want_h && (th != want_h || tw != want_w))) continue;
+            const int tx = (ow + tw - 1) / tw, ty = (oh + th - 1) / th;
+            const int rounds = (tx * ty * q.cout_blocks + 255) / 256;
+            const double cost = (double)rounds * (th * tw + 24);   // (+24: a round's fixed part, in positions)
+            if (cost < best) {
+                best = cost;
+                q.tile_h = th; q.tile_w = tw; q.tiles_x = tx; q.tiles_y = ty;
+            }
+        }
+        if (best >= 1e30) return;
+        const size_t halves = ((size_t)q.cin_chunks * 9 + 8) * q.mfrags * 2 * 64 * 8;
+        q.wpack = p16_wpack_dev = net->dev_alloc(halves * 2, true);
+        const bool always = getenv("FYNHIP_FORCE_P16_CONV") != nullptr;
+        const char* at = getenv("FYNHIP_AUTOTUNE");
+        bool pick = true;
+        char key[160];
+        snprintf(key, sizeof(key), "p16:%dx%d:%dx%d:cp%d:r%d:e%d", d.in_channels, oc, oh, ow, in_v.cp, res_v ? 1 : 0, clamp ? 1 : 0);
+        if (always) {
+        } else if (tune_cache_flag(key, &pick)) {
+        } else if (!(at && at[0] == '0')) {
+            float t_p16 = 1e30f, t_other = 1e30f;
+            for (int rep = 0; rep < 3; rep++) {
+                t_p16 = std::min(t_p16, time_calls(net, [&]() {
+                    if (launch_conv_p16(q, net->stream) != 0) fail(FYN_ERR_DEVICE, "16-position convolution launch failed while tuning");
+                }, 10));
+                t_other = std::min(t_other, time_launch(net, launch, 10));
+            }
+            if (getenv("FYNHIP_TUNE_VERBOSE")) fprintf(stderr, "[tune] 3x3: 16-position fragments (%dx%d tiles) %.1f us, general kernel %.1f us\n", q.tile_h, q.tile_w, t_p16 * 1e3f, t_other * 1e3f);
+            pick = t_p16 < t_other;
+            tune_cache_store_flag(key, pick);
+        }
+        if (pick) {
+            p16 = true;
+            pp = q;
+        } else {
+            net->dev_free(p16_wpack_dev);
+            p16_wpack_dev = nullptr;
+        }
+    }
+    // weights of that form: [(chunk*9 + tap)][cout fragment of 16][plane][lane][8 halves], zero steps behind the last
+    void pack_p16(const float* w, float wmul) {
+        const int cin = d.in_channels;
+        std::vector<uint16_t> pack(((size_t)pp.cin_chunks * 9 + 8) * pp.mfrags * 2 * 64 * 8, 0);
+        for (int chunk = 0; chunk < pp.cin_chunks; chunk++)
+            for (int tap = 0; tap < 9; tap++)
+                for (int mf = 0; mf < pp.mfrags; mf++) {
+                    uint16_t* base = pack.data() + (((size_t)(chunk * 9 + tap) * pp.mfrags + mf) * 2) * 64 * 8;
+                    for (int lane = 0; lane < 64; lane++) {
+                        const int o = mf * 16 + (lane & 15);
+                        if (o >= oc) continue;
+                        for (int j = 0; j < 8; j++) {
+                            const int ci = chunk * 32 + 8 * (lane >> 4) + j;
+                            if (ci >= cin) continue;
+                            const float v = w[(((size_t)o * 3 + tap / 3) * 3 + tap % 3) * cin + ci] * wmul;
+                            const uint16_t hi = f2h_bits(v);
+                            base[(size_t)lane * 8 + j] = hi;
+                            base[(size_t)(64 + lane) * 8 + j] = f2h_bits(v - h2f(hi));
+                        }
+                    }
+                }
+        FYN_HIP(hipStreamSynchronize(net->stream));
+        FYN_HIP(hipMemcpyAsync(p16_wpack_dev, pack.data(), pack.size() * 2, hipMemcpyHostToDevice, net->stream));
+        FYN_HIP(hipStreamSynchronize(net->stream));
     }
     void setup_rows_wide(const TView& in_v, const TView& out_v, const TView* res_v, int res_relu, int res_scale) {
         const int r = (k - 1) / 2;
@@ -1061,6 +1152,9 @@ class ConvLayer : public Layer {
             scale_dev = static_cast<float*>(net->dev_alloc(padded * sizeof(float)));
             bias_dev = static_cast<float*>(net->dev_alloc(padded * sizeof(float)));
             launch = tune_mfma(net, sc, in_v, out_v, res_v, d.in_channels, oc, act(), res_relu, res_scale, scale_dev, bias_dev);
+            if (!frac_shift && conv_p16_supported(k, stride, dil, in_v.cp, oc, out_v.cp, out_v.f16 != 0) && d.in_channels == in_v.cp &&
+                (!res_v || res_v->cp >= oc) && !getenv("FYNHIP_NO_P16_CONV"))
+                setup_p16(in_v, out_v, res_v, res_relu, res_scale);
         }
         if (direct) {
             scale_dev = static_cast<float*>(net->dev_alloc(padded * sizeof(float)));
@@ -1088,6 +1182,10 @@ class ConvLayer : public Layer {
                         for (int i = 0; i < cin; i++)
                             wd[(((size_t)ky * k + kx) * cin + i) * cp + o] = w[(((size_t)o * k + ky) * k + kx) * cin + i];
             reupload(net, wdirect_dev, wd);
+        } else if (p16) {
+            const float wmul = weight_prescale(w, (size_t)oc * k * k * d.in_channels);
+            pp.acc_mul = 1.0f / wmul;
+            pack_p16(w, wmul);
         } else if (wide && rows) {
             const float wmul = weight_prescale(w, (size_t)oc * k * k * d.in_channels);
             rp.acc_mul = 1.0f / wmul;
@@ -1127,6 +1225,10 @@ class ConvLayer : public Layer {
             if (launch_conv_rows(rp, tout().v.f16 != 0, s) != 0) fail(FYN_ERR_DEVICE, "layer %s: convolution launch failed", d.name);
             return;
         }
+        if (p16) {
+            if (launch_conv_p16(pp, s) != 0) fail(FYN_ERR_DEVICE, "layer %s: convolution launch failed", d.name);
+            return;
+        }
         if (direct) launch_conv_direct(dp, s);
         else if (run_mfma(launch, s) != 0)
             fail(FYN_ERR_DEVICE, "layer %s: convolution launch failed", d.name);
@@ -1141,6 +1243,19 @@ class ConvLayer : public Layer {
                      tout().v.f16 ? "f16 " : "f16x2-split ", rp.strips, rp.row_blocks, rp.rows_per_block, conv_rows_lds_bytes(rp, tout().v.f16 != 0));
             return mode + buf;
         }
+        if (p16) {
+            char buf[200];
+            size_t lds = 0;
+            for (int i = 0; i < conv_p16_tile_count(); i++) {
+                int th, tw;
+                size_t l;
+                conv_p16_tile(i, &th, &tw, &l);
+                if (th == pp.tile_h && tw == pp.tile_w) lds = l;
+            }
+            snprintf(buf, sizeof(buf), "conv_p16 f16x2-split tile=128x%d(cout x pos) th=%d tw=%d blocks=%d lds=%zu steps=9 chunks=%d",
+                     pp.tile_h * pp.tile_w, pp.tile_h, pp.tile_w, pp.tiles_x * pp.tiles_y * pp.cout_blocks, lds, pp.cin_chunks);
+            return mode + buf;
+        }
         if (wide) return mode + (fused ? "wide-kernel(kx folded into cout, summed in the epilogue) " : "wide-kernel(kx folded into cout)+shift_reduce ") + mfma_info(launch);
         return mode + mfma_info(launch);
     }
@@ -1153,6 +1268,9 @@ class ConvLayer : public Layer {
     MfmaLaunch launch;
     ConvRowsParams rp{};          // row-rolling form of the folded convolution (conv_rows.hip)
     void* rows_wpack_dev = nullptr;
+    bool p16 = false;             // 16-position-fragment form of a 3x3 convolution (conv_p16.hip)
+    ConvP16Params pp{};
+    void* p16_wpack_dev = nullptr;
     ConvDirectParams dp{};
     ShiftReduceParams sr{};
     TView qv{};
