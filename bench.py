@@ -360,6 +360,11 @@ def frame_pool_rate_in_child(workload, frames, instances=4, graph=True):
     """frame_pool_rate in a process of its own (started as a child, never exec'ed into): the side measurement gets a
     fresh HIP runtime with the hardware queues to itself, and a failure in it cannot take the main record with it."""
     import subprocess
+    # Under rocprofv3 the child would inherit the profiler's preload environment and start a second tool instance that
+    # writes to the parent's output files; the one profiled pool run on record died in that child with a host-side
+    # segmentation fault inside the tool's interception.  The side measurement is therefore left out of profiled runs.
+    if any(k.startswith(("ROCPROF", "ROCP_", "ROCPROFILER")) for k in os.environ):
+        return {"skipped": "a profiler's environment is present; the pool is measured in unprofiled runs only"}
     cmd = [sys.executable, os.path.abspath(__file__), "--frame-pool-only", "--workload", workload, "--steps", str(frames),
            "--instances", str(instances)] + ([] if graph else ["--pool-eager"])
     try:

@@ -930,8 +930,9 @@ static int check_params(const ConvVariant& v, const ConvMfmaParams& p) {
     return 0;
 }
 
-// raises a kernel's dynamic LDS limit once per kernel and size
-static int ensure_lds(const void* fn, size_t lds_bytes) {
+// raises a kernel's dynamic LDS limit once per kernel and size (also for the other convolution files: a launch that
+// is being captured into a graph then makes no attribute call)
+int ensure_lds(const void* fn, size_t lds_bytes) {
     if (lds_bytes <= 48 * 1024) return 0;
     static std::mutex mu;
     static std::map<const void*, size_t> raised;

@@ -342,9 +342,7 @@ int launch_conv_p16(const ConvP16Params& p, hipStream_t s) {
         (p.res && p.res_cp < p.cout_blocks * CPB) || p.nreset < 0 || p.nreset > 4)
         return -5;
     if (e->lds > 160 * 1024) return -2;
-    if (e->lds > 48 * 1024) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void*>(e->fn), hipFuncAttributeMaxDynamicSharedMemorySize, (int)e->lds) != hipSuccess) return -2;
-    }
+    if (ensure_lds(reinterpret_cast<const void*>(e->fn), e->lds) != 0) return -2;
 #ifdef FYN_P16_TRACE
     {
         static long long* dev = nullptr;

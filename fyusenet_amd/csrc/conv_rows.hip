@@ -365,9 +365,7 @@ int launch_conv_rows(const ConvRowsParams& p, bool f16, hipStream_t s) {
         return -5;
     const size_t lds_bytes = conv_rows_lds_bytes(p, f16);
     if (lds_bytes > 160 * 1024) return -2;
-    if (lds_bytes > 48 * 1024) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes) != hipSuccess) return -2;
-    }
+    if (ensure_lds(reinterpret_cast<const void*>(fn), lds_bytes) != 0) return -2;
 #ifdef FYN_ROWS_TRACE
     {
         static long long* dev = nullptr;

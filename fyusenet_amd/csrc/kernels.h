@@ -159,6 +159,7 @@ struct ConvRowsParams {
 #endif
     Act act;
 };
+int ensure_lds(const void* fn, size_t lds_bytes);   // 0, or -2 when the device refuses the size (conv_mfma.hip)
 bool conv_rows_supported(int k, int cin_pitch, int cout, bool f16);
 size_t conv_rows_lds_bytes(const ConvRowsParams& p, bool f16);
 int launch_conv_rows(const ConvRowsParams& p, bool f16, hipStream_t s);

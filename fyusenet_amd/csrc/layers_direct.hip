@@ -914,8 +914,20 @@ void launch_argmax(const TView& in, const TView& out, int32_t* idx_out, const Ac
 // ---------------------------------------------------------------------------------------------
 // fully connected layer as a matrix-vector product (DeepGEMMLayer::forward,
 // gpu/deep/deepgemmlayer.cpp:66-236): one wavefront per output row, the row of weights is streamed
-// once from HBM in 16-byte pieces, partial sums meet with cross-lane shuffles.
+// once from HBM in 16-byte pieces, partial sums meet on the DPP paths.
 // ---------------------------------------------------------------------------------------------
+// Sum of a wave's 64 values on the vector ALUs' data-parallel paths (prefix sums inside rows of 16 lanes, then the row
+// sums carried into the following rows); every lane gets the total.
+__device__ __forceinline__ float wave_sum_dpp(float v) {
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x111, 0xf, 0xf, false));   // row_shr:1
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x112, 0xf, 0xf, false));   // row_shr:2
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x114, 0xf, 0xf, false));   // row_shr:4
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x118, 0xf, 0xf, false));   // row_shr:8
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x142, 0xa, 0xf, false));   // row_bcast:15 into rows 1, 3
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x143, 0xc, 0xf, false));   // row_bcast:31 into rows 2, 3
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
+}
+
 template <typename T, typename TW>
 __global__ __launch_bounds__(256) void gemv_kernel(const GemvParams p) {
     const int lane = threadIdx.x & 63;
@@ -926,17 +938,23 @@ __global__ __launch_bounds__(256) void gemv_kernel(const GemvParams p) {
     const TW* w = reinterpret_cast<const TW*>(p.w) + (size_t)row * cinp;
     float acc = 0.f;
     if (row < p.out.c) {
-        // four 16-byte pieces of the row per trip: loads first, multiply-adds in column order
-        for (int c0 = lane * 4; c0 < cinp; c0 += 4 * 256) {
-            float4 xv[4], wv[4];
+        // eight 16-byte pieces of the row per trip (a row of 2048 fp32 weights in one): every load of a trip is on its
+        // way before the first multiply-add, so the wave pays the memory latency once per trip
+        constexpr int NP = 8;
+        for (int c0 = lane * 4; c0 < cinp; c0 += NP * 256) {
+            float4 xv[NP], wv[NP];
 #pragma unroll
-            for (int j = 0; j < 4; j++) {
+            for (int j = 0; j < NP; j++) {
                 const int c = c0 + j * 256 < cinp ? c0 + j * 256 : c0;
-                xv[j] = ld4<T>(x + c);
                 wv[j] = ld4<TW>(w + c);
             }
 #pragma unroll
-            for (int j = 0; j < 4; j++) {
+            for (int j = 0; j < NP; j++) {
+                const int c = c0 + j * 256 < cinp ? c0 + j * 256 : c0;
+                xv[j] = ld4<T>(x + c);
+            }
+#pragma unroll
+            for (int j = 0; j < NP; j++) {
                 if (c0 + j * 256 >= cinp) break;
                 const float4 a = act4(xv[j], p.act);
                 acc = fmaf(a.x, wv[j].x, acc); acc = fmaf(a.y, wv[j].y, acc);
@@ -944,7 +962,7 @@ __global__ __launch_bounds__(256) void gemv_kernel(const GemvParams p) {
             }
         }
     }
-    for (int o = 32; o > 0; o >>= 1) acc += __shfl_xor(acc, o, 64);
+    acc = wave_sum_dpp(acc);
     if (lane == 0) {
         float r = (row < p.out.c) ? acc * p.scale[row] + p.bias[row] : 0.f;
         reinterpret_cast<T*>(p.out.ptr)[tv_off(p.out, 0, 0) + row] = (T)r;
