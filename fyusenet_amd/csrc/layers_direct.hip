@@ -388,7 +388,6 @@ static bool launch_dw_col(const DwConvParams& p, hipStream_t s) {
     if (getenv("FYNHIP_NO_DW_STRIPS")) return false;
     const size_t per_row = (size_t)((p.out.w + 3) / 4) * (p.out.cp / V);
     int rows = 16;
-    if (const char* e = getenv("FYNHIP_DW_ROWS")) rows = atoi(e);   // (experiments)
     while (rows > 2 && per_row * ((p.out.h + rows - 1) / rows) < 256 * 256 * 2) rows /= 2;   // at least two waves per SIMD of work
     if (rows < 4 || p.out.h < rows) return false;
     const size_t n = per_row * ((p.out.h + rows - 1) / rows);
