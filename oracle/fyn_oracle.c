@@ -26,8 +26,13 @@
  *   fyo_batchnorm     closed form x*s+b (misctests.cpp:118-126)
  *   fyo_argmax        numpy argmax (first maximum) (misctests.cpp:84-102)
  *   fyo_concat        memcpy identity
- *   fyo_deep_*        round trip + hand-computed tilings           (parity unpinned against the
- *                     reference binary: cpubuffershape.cpp needs the GL wrapper to link)
+ *   fyo_deep_*        round trip + hand-computed tilings + DeepTiler's arithmetic (gpu/deep/deeptiler.cpp:73-76,
+ *                     97-110: tile origin and channel order) + the copy loop of cpu/cpubuffer.cpp:424-437 at padding 0
+ *                     with its row stride corrected (the reference multiplies the row index by the pixel packing twice)
+ *   activations       leaky ReLU on fetch: shaders/activation.inc's form against the library's leaky_relu in fp64,
+ *                     through unary copy, batch-norm and convolution; clip: numpy clip
+ *   fyo_batchnorm     residual variants (residual / ReLU on it / batch-norm on it / both): closed form of
+ *                     shaders/deep/deepbatchnorm.frag:26-35 per flag
  *   fyo_unary         arithmetic: reference patterns arithtests.cpp:205-234; sigmoid/tanh: scipy expit /
  *                     numpy tanh fp64; cast: numpy rint + clip (exact halves: parity unpinned, GLSL
  *                     leaves the tie direction open)
