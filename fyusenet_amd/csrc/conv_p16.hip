@@ -48,33 +48,103 @@ __device__ __forceinline__ float act_p16(float x, const Act& a) { return __built
 constexpr int KC = 32;        // input channels per chunk
 constexpr int NT = 9;         // taps
 constexpr int PD = 6;         // depth of the weight-fragment ring (steps)
-constexpr int UNR = 2 * NT;   // steps per unrolled group: two chunks (one per staging buffer)
-constexpr int CPB = 128;      // output channels per workgroup
+constexpr int PITCH = KC * 2 + 16;   // bytes per staged pixel and plane: 8 neighbouring lanes' 16-byte reads cover all banks
 
-template <int TH, int TW>
+// Row padding (bytes, a multiple of 16) with which the sixteen positions of every fragment of every wave read distinct
+// LDS banks, for both ways the hardware may group the lanes of a 16-byte read (8 lanes over 32 banks, 16 over 64).
+constexpr bool p16_pad_ok(int TH, int TW, int S, int WN, int row_pitch) {
+    for (int model = 0; model < 2; model++) {
+        const int banks = model ? 64 : 32, group = model ? 16 : 8;
+        for (int wn = 0; wn < WN; wn++)
+            for (int fn = 0; fn < TH * TW / 16; fn++)
+                for (int g0 = 0; g0 < 64; g0 += group)
+                    for (int i = g0; i < g0 + group; i++)
+                        for (int j = i + 1; j < g0 + group; j++) {
+                            const int mi = fn * 16 + (i & 15), mj = fn * 16 + (j & 15);
+                            const int ai = (S * (mi / TW) * row_pitch + (wn * TW + mi % TW) * PITCH + (i >> 4) * 16) / 4;
+                            const int aj = (S * (mj / TW) * row_pitch + (wn * TW + mj % TW) * PITCH + (j >> 4) * 16) / 4;
+                            for (int di = 0; di < 4; di++)
+                                for (int dj = 0; dj < 4; dj++)
+                                    if ((ai + di) % banks == (aj + dj) % banks && ai + di != aj + dj) return false;
+                        }
+    }
+    return true;
+}
+constexpr int p16_row_pad(int TH, int TW, int S, int WN, int slots) {
+    for (int pad = 0; pad < 256; pad += 16)
+        if (p16_pad_ok(TH, TW, S, WN, slots * PITCH + pad)) return pad;
+    return 96;
+}
+
+// Geometry of one instantiation.  A workgroup's four MFMA waves are WM groups of 32 output channels x WN = 4 / WM tiles
+// of TH x TW positions side by side; S is the input step per position (1 or 2).  With S = 2 the staged tile keeps even
+// and odd columns in separate halves of a row, so that the positions of a fragment are neighbours in LDS whatever the
+// tap: column c lives in slot (c & 1) * HWH + (c >> 1).
+template <int TH, int TW, int S, int WM>
 struct Geo {
-    static constexpr int HW = TW + 2, HH = TH + 2;
-    static constexpr int PITCH = KC * 2 + 16;            // bytes per staged pixel and plane: 8 neighbouring lanes' 16-byte reads cover all banks
-    static constexpr int ROW_PITCH = HW * PITCH + 96;    // (+96: the 16 positions of a fragment span up to four tile rows; with this pad their reads fall into distinct banks)
+    static constexpr int WN = 4 / WM;
+    static constexpr int TWG = WN * TW;                  // positions per row of the workgroup's tile
+    static constexpr int HW = S * (TWG - 1) + 3, HH = S * (TH - 1) + 3;
+    static constexpr int HWH = (HW + 1) / 2;
+    static constexpr int SLOTS = (S == 1) ? HW : 2 * HWH;
+    static constexpr int ROW_PITCH = SLOTS * PITCH + p16_row_pad(TH, TW, S, WN, SLOTS);
     static constexpr int PLANE = HH * ROW_PITCH;
     static constexpr int BUF = 2 * PLANE;                // hi, lo
-    static constexpr int NPOS = TH * TW, FN = NPOS / 16;
+    static constexpr int NPOS = TH * TW, FN = NPOS / 16;  // per wave
     static constexpr int NITEMS = HH * HW * (KC / 8);    // staging items: (pixel, 8 channels)
     static constexpr int NB = (NITEMS + 255) / 256;      // ... per staging thread
-    static constexpr int SB_OFF = 2 * BUF;               // scale[128], bias[128]
-    static constexpr int RES_OFF = SB_OFF + 2 * CPB * 4;
+    static constexpr int CPB = 32 * WM;                  // output channels per workgroup
     static constexpr int RES_PITCH = CPB * 4 + 16;       // bytes per position of the residual tile
-    static constexpr int RNB = NPOS * (CPB / 4) / 256;   // residual 16-byte pieces per staging thread
-    static constexpr int LDS = RES_OFF + NPOS * RES_PITCH;
+    static constexpr int RPIECES = TH * TWG * (CPB / 4);  // residual 16-byte pieces
+    static constexpr int RNB = (RPIECES + 255) / 256;    // ... per staging thread
+    static constexpr int slot_off(int c) { return (S == 1) ? c * PITCH : ((c & 1) * HWH + (c >> 1)) * PITCH; }
+    static constexpr int tap_off(int t) { return (t / 3) * ROW_PITCH + slot_off(t % 3); }
+    static_assert(S == 1 || S == 2, "input step 1 or 2");
     static_assert(NPOS % 16 == 0, "whole position fragments");
-    static_assert((NPOS * (CPB / 4)) % 256 == 0, "residual pieces divide among the staging threads");
-    static_assert(2 * BUF + 2 * ROW_PITCH + 2 * PITCH + 64 < 65536, "B fragment offsets fit the LDS instructions' immediate field");
+    static_assert(PLANE + 2 * ROW_PITCH + 2 * PITCH + HWH * PITCH + 64 < 65536, "B fragment offsets inside a staging buffer fit the LDS instructions' immediate field");
 };
-
-template <int TH, int TW>
-__global__ __launch_bounds__(512) void conv_p16_kernel(const ConvP16Params p) {
-    using G = Geo<TH, TW>;
+// NCH chunks of nine steps, starting in staging buffer 0 (the B fragments of its first step are in `b`); two chunks end
+// with the fragments of the first step of buffer 0 again.  One slot per MFMA: the MFMA, then a share of the
+// step's memory instructions, fenced so that the compiler keeps the order (a memory instruction issued right after an
+// MFMA runs in its shadow).  Position fragment fn is used by six consecutive MFMAs; its registers are then refilled
+// with the fragment of the next step, so one register set per fragment is enough.  The ring slot of the previous
+// step is refilled with the weights of step t+PD-1.  The barrier of a chunk sits in its last step, before the first
+// read of the next chunk's buffer: the staging waves have filled that buffer by then, and all reads of the current
+// buffer were issued a step earlier.
+template <class G, int NCH>
+__device__ __forceinline__ void p16_steps(f32x4_t (&acc)[2][G::FN], half8_t (&a_q)[PD][2][2], half8_t (&b)[G::FN][2],
+                                          const int (&bbase)[2][G::FN], const unsigned char* lds, const unsigned char*& wnext,
+                                          unsigned wstep) {
     constexpr int FN = G::FN;
+#pragma unroll
+    for (int dd = 0; dd < NCH * NT; dd++) {
+        const int d = dd % PD, dprev = (d + PD - 1) % PD;
+        const int nd = dd + 1;                                   // the next step: buffer and tap
+        const int nbuf = (nd / NT) & 1, noff = G::tap_off(nd % NT);
+        const unsigned char* w_ = wnext;
+        wnext += wstep;
+#pragma unroll
+        for (int i = 0; i < 6 * FN; i++) {
+            const int fn = i / 6, r = i % 6, kind = r / 2, fm = r % 2;
+            const int apl = (kind == 1) ? 1 : 0, bpl = (kind == 2) ? 1 : 0;
+            acc[fm][fn] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_q[d][fm][apl], b[fn][bpl], acc[fm][fn], 0, 0, 0);
+            if (dd % NT == NT - 1 && i == 3) lds_barrier();
+            if (r == 5 && !(NCH == 1 && dd == NT - 1)) {   // (a single chunk is the launch's last: nothing follows its last step)
+                b[fn][0] = *reinterpret_cast<const half8_t*>(lds + bbase[nbuf][fn] + noff);
+                b[fn][1] = *reinterpret_cast<const half8_t*>(lds + bbase[nbuf][fn] + noff + G::PLANE);
+            }
+#pragma unroll
+            for (int j = 0; j < 4; j++)   // the four weight fragments of a step, spread over its slots
+                if (i == (j * 6 * FN) / 4 + 1) a_q[dprev][j % 2][j / 2] = *reinterpret_cast<const half8_t*>(w_ + ((j % 2) * 2 + j / 2) * 1024);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+}
+
+template <int TH, int TW, int S, int WM>
+__global__ __launch_bounds__(512) void conv_p16_kernel(const ConvP16Params p) {
+    using G = Geo<TH, TW, S, WM>;
+    constexpr int FN = G::FN, CPB = G::CPB;
     extern __shared__ __align__(16) unsigned char lds[];
     __shared__ unsigned range_box[2];   // meeting point of the MFMA waves' output maxima (range.h)
     if (blockIdx.x == 0) range_clear(p.reset[0], p.reset[1], p.reset[2], p.reset[3], p.nreset);
@@ -92,10 +162,13 @@ __global__ __launch_bounds__(512) void conv_p16_kernel(const ConvP16Params p) {
     const int cb = bid % p.cout_blocks;
     const int tile = bid / p.cout_blocks;
     const int tyi = tile / p.tiles_x, txi = tile - tyi * p.tiles_x;
-    const int pos_y0 = tyi * TH, pos_x0 = txi * TW;
+    const int pos_y0 = tyi * TH, pos_x0 = txi * G::TWG;
     if (tid < 2) range_box[tid] = 0u;
     const unsigned range_bits = p.in_amax ? range_load(p.in_amax) : 0u;
-    const int nchunks = p.cin_chunks;   // even (checked at launch)
+    const int nchunks = p.cin_chunks;
+    // LDS: one staging buffer (two when there is more than one chunk), scale and bias, the residual tile
+    const int sb_off = (nchunks > 1 ? 2 : 1) * G::BUF;
+    const int res_off = sb_off + 2 * CPB * 4;
 
     if (wave < 4) {
         // ------------------------------------------------------------------ staging waves (the first four: they start first)
@@ -109,8 +182,8 @@ __global__ __launch_bounds__(512) void conv_p16_kernel(const ConvP16Params p) {
             if (idx < G::NITEMS) {
                 const int pix = idx >> 2, g = idx & 3;
                 const int py = pix / G::HW, px = pix - py * G::HW;
-                int gy = pos_y0 + p.in_y0 + py, gx = pos_x0 + p.in_x0 + px;
-                l_off[i] = py * G::ROW_PITCH + px * G::PITCH + g * 16;
+                int gy = pos_y0 * S + p.in_y0 + py, gx = pos_x0 * S + p.in_x0 + px;
+                l_off[i] = py * G::ROW_PITCH + ((S == 1) ? px * PITCH : ((px & 1) * G::HWH + (px >> 1)) * PITCH) + g * 16;
                 if (p.in_clamp) {
                     gy = min(max(gy, 0), p.in_hp - 1);
                     gx = min(max(gx, 0), p.in_wp - 1);
@@ -150,8 +223,8 @@ __global__ __launch_bounds__(512) void conv_p16_kernel(const ConvP16Params p) {
         fetch(0);
         if (p.in_amax) in_scale = range_scale(range_after_act(range_reduce(range_bits), p.act), &inv_unused);
         if (stid < CPB) {
-            reinterpret_cast<float*>(lds + G::SB_OFF)[stid] = p.scale[cb * CPB + stid];
-            reinterpret_cast<float*>(lds + G::SB_OFF)[CPB + stid] = p.bias[cb * CPB + stid];
+            reinterpret_cast<float*>(lds + sb_off)[stid] = p.scale[cb * CPB + stid];
+            reinterpret_cast<float*>(lds + sb_off)[CPB + stid] = p.bias[cb * CPB + stid];
         }
         store(lds);
         FYN_PTRACE(1);
@@ -163,22 +236,22 @@ __global__ __launch_bounds__(512) void conv_p16_kernel(const ConvP16Params p) {
                 store(lds + ((c + 1) & 1) * G::BUF);
                 FYN_PTRACE(3 + 2 * c);
             } else if (p.res) {
-                // the residual tile: [position][128 channels] fp32
+                // the residual tile: [position][CPB channels] fp32
                 const float* res = reinterpret_cast<const float*>(p.res);
                 f32x4_t rv[G::RNB];
 #pragma unroll
                 for (int i = 0; i < G::RNB; i++) {
                     const int idx = stid + i * 256;
-                    const int m = idx >> 5, c4 = idx & 31;
-                    const int ty = m / TW, tx = m - ty * TW;
+                    const int m = idx / (CPB / 4), c4 = idx % (CPB / 4);
+                    const int ty = m / G::TWG, tx = m - ty * G::TWG;
                     const int py = pos_y0 + ty, px = pos_x0 + tx;
-                    const bool ok = py < p.npos_y && px < p.npos_x;
+                    const bool ok = idx < G::RPIECES && py < p.npos_y && px < p.npos_x;
                     rv[i] = *reinterpret_cast<const f32x4_t*>(res + (ok ? ((size_t)(p.res_off_y + py) * p.res_wp + p.res_off_x + px) * p.res_cp + cb * CPB + c4 * 4 : 0));
                 }
 #pragma unroll
                 for (int i = 0; i < G::RNB; i++) {
                     const int idx = stid + i * 256;
-                    *reinterpret_cast<f32x4_t*>(lds + G::RES_OFF + (idx >> 5) * G::RES_PITCH + (idx & 31) * 16) = rv[i];
+                    if (idx < G::RPIECES) *reinterpret_cast<f32x4_t*>(lds + res_off + (idx / (CPB / 4)) * G::RES_PITCH + (idx % (CPB / 4)) * 16) = rv[i];
                 }
             }
             lds_barrier();
@@ -189,18 +262,20 @@ __global__ __launch_bounds__(512) void conv_p16_kernel(const ConvP16Params p) {
     // ---------------------------------------------------------------------- MFMA waves
     FYN_PTRACE(0);
     const int mq = lane & 15, kq = lane >> 4;
-    const int mw = wave - 4;   // this wave's 32 output channels of the workgroup's 128
-    int bbase[FN];   // per-lane LDS offset of the B fragments: position, then the lane's 8 channels of the chunk
+    const int mw = (wave - 4) % WM;   // this wave's 32 output channels of the workgroup's CPB
+    const int wn = (wave - 4) / WM;   // ... and its tile of positions
+    int bbase[2][FN];   // per-lane LDS offset of the B fragments in either staging buffer: position, then the lane's 8 channels of the chunk
 #pragma unroll
     for (int fn = 0; fn < FN; fn++) {
         const int m = fn * 16 + mq;
         const int ty = m / TW, tx = m - ty * TW;
-        bbase[fn] = ty * G::ROW_PITCH + tx * G::PITCH + kq * 16;
+        bbase[0][fn] = S * ty * G::ROW_PITCH + (wn * TW + tx) * PITCH + kq * 16;
+        bbase[1][fn] = bbase[0][fn] + G::BUF;
     }
     // A fragments: [(chunk*9 + tap)][cout fragment of 16][plane][lane] x 8 halves; the buffer has PD steps of zero
     // slack behind the last step, so the prefetch needs no clamp.
     const unsigned wstep = (unsigned)p.mfrags * 2 * 1024;
-    const unsigned char* wbase = reinterpret_cast<const unsigned char*>(p.wpack) + (size_t)((cb * 8 + mw * 2) * 2) * 1024 + lane * 16;
+    const unsigned char* wbase = reinterpret_cast<const unsigned char*>(p.wpack) + (size_t)((cb * 2 * WM + mw * 2) * 2) * 1024 + lane * 16;
     half8_t a_q[PD][2][2];
 #pragma unroll
     for (int d = 0; d < PD; d++)
@@ -224,47 +299,21 @@ __global__ __launch_bounds__(512) void conv_p16_kernel(const ConvP16Params p) {
 #pragma unroll
     for (int fn = 0; fn < FN; fn++)
 #pragma unroll
-        for (int pl = 0; pl < 2; pl++) b[fn][pl] = *reinterpret_cast<const half8_t*>(lds + bbase[fn] + pl * G::PLANE);
+        for (int pl = 0; pl < 2; pl++) b[fn][pl] = *reinterpret_cast<const half8_t*>(lds + bbase[0][fn] + pl * G::PLANE);
 
-    // One slot per MFMA: the MFMA, then a share of the step's memory instructions, fenced so that the compiler keeps
-    // the order (a memory instruction issued right after an MFMA runs in its shadow).  Position fragment fn is used
-    // by six consecutive MFMAs; its registers are then refilled with the fragment of the next step, so one register
-    // set per fragment is enough.  The ring slot of the previous step is refilled with the weights of step t+PD-1.
-    // The barrier of a chunk sits in its last step, before the first read of the next chunk's buffer: the staging
-    // waves have filled that buffer by then, and all reads of the current buffer were issued a step earlier.
+    // pairs of chunks (one per staging buffer), then the odd one
     const unsigned char* wnext = wbase + (size_t)(PD - 1) * wstep;
-    for (int g = 0; g < nchunks; g += 2) {
-#pragma unroll
-        for (int dd = 0; dd < UNR; dd++) {
-            const int d = dd % PD, dprev = (d + PD - 1) % PD;
-            const int nd = (dd + 1) % UNR;                       // the next step: buffer and tap
-            const int ntap = nd % NT;
-            const int noff = (nd / NT) * G::BUF + (ntap / 3) * G::ROW_PITCH + (ntap % 3) * G::PITCH;
-            const unsigned char* w_ = wnext;
-            wnext += wstep;
-#pragma unroll
-            for (int i = 0; i < 6 * FN; i++) {
-                const int fn = i / 6, r = i % 6, kind = r / 2, fm = r % 2;
-                const int apl = (kind == 1) ? 1 : 0, bpl = (kind == 2) ? 1 : 0;
-                acc[fm][fn] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_q[d][fm][apl], b[fn][bpl], acc[fm][fn], 0, 0, 0);
-                if (dd % NT == NT - 1 && i == 3) lds_barrier();
-                if (r == 5) {
-                    b[fn][0] = *reinterpret_cast<const half8_t*>(lds + bbase[fn] + noff);
-                    b[fn][1] = *reinterpret_cast<const half8_t*>(lds + bbase[fn] + noff + G::PLANE);
-                }
-#pragma unroll
-                for (int j = 0; j < 4; j++)   // the four weight fragments of a step, spread over its slots
-                    if (i == (j * 6 * FN) / 4 + 1) a_q[dprev][j % 2][j / 2] = *reinterpret_cast<const half8_t*>(w_ + ((j % 2) * 2 + j / 2) * 1024);
-                __builtin_amdgcn_sched_barrier(0);
-            }
-            if (dd % NT == NT - 1) FYN_PTRACE(3 + g + dd / NT);
-        }
+    int g = 0;
+    for (; g + 2 <= nchunks; g += 2) {
+        p16_steps<G, 2>(acc, a_q, b, bbase, lds, wnext, wstep);
+        FYN_PTRACE(3 + g);
     }
+    if (g < nchunks) p16_steps<G, 1>(acc, a_q, b, bbase, lds, wnext, wstep);
 
     // ---- epilogue: a lane holds, per fragment, output channels 4*kq .. 4*kq+3 of position fn*16 + mq.  One wave per
     //      SIMD pays four cycles per vector instruction, so the arithmetic is kept short (acc_mul is a power of two:
     //      folding it into the scale changes no bit) and every fragment is stored as soon as it is finished. ----
-    const float* sb = reinterpret_cast<const float*>(lds + G::SB_OFF);
+    const float* sb = reinterpret_cast<const float*>(lds + sb_off);
     f32x4_t sc[2], bi[2], scm[2];
 #pragma unroll
     for (int fm = 0; fm < 2; fm++) {
@@ -280,7 +329,7 @@ __global__ __launch_bounds__(512) void conv_p16_kernel(const ConvP16Params p) {
 #pragma unroll
     for (int fn = 0; fn < FN; fn++) {
         const int m = fn * 16 + mq;
-        const int ty = m / TW, tx = m - ty * TW;
+        const int ty = m / TW, tx = wn * TW + (m - ty * TW);
         const int py = pos_y0 + ty, px = pos_x0 + tx;
         const bool ok = py < p.npos_y && px < p.npos_x;
         const size_t obase = ((size_t)(p.out_off_y + py) * p.out_wp + p.out_off_x + px) * p.out_cp + cb * CPB + mw * 32 + kq * 4;
@@ -291,7 +340,7 @@ __global__ __launch_bounds__(512) void conv_p16_kernel(const ConvP16Params p) {
 #pragma unroll
             for (int e = 0; e < 4; e++) v[e] = acc[fm][fn][e] * scm[fm][e] + bi[fm][e];
             if (have_res) {
-                f32x4_t rv = *reinterpret_cast<const f32x4_t*>(lds + G::RES_OFF + m * G::RES_PITCH + (mw * 32 + fm * 16 + kq * 4) * 4);
+                f32x4_t rv = *reinterpret_cast<const f32x4_t*>(lds + res_off + (ty * G::TWG + tx) * G::RES_PITCH + (mw * 32 + fm * 16 + kq * 4) * 4);
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
                     float r = rv[e];
@@ -313,36 +362,55 @@ __global__ __launch_bounds__(512) void conv_p16_kernel(const ConvP16Params p) {
 
 typedef void (*p16_fn)(const ConvP16Params);
 struct P16Entry {
-    int th, tw;
+    int th, tw, stride, wm;
     p16_fn fn;
-    size_t lds;
+    size_t buf, res_bytes;   // one staging buffer; the residual tile
 };
-template <int TH, int TW>
-constexpr P16Entry entry() { return P16Entry{TH, TW, conv_p16_kernel<TH, TW>, (size_t)Geo<TH, TW>::LDS}; }
-const P16Entry kEntries[] = {entry<8, 10>(), entry<10, 8>(), entry<8, 8>(), entry<8, 6>(), entry<4, 8>(), entry<4, 4>()};
+template <int TH, int TW, int S, int WM>
+constexpr P16Entry entry() {
+    using G = Geo<TH, TW, S, WM>;
+    return P16Entry{TH, TW, S, WM, conv_p16_kernel<TH, TW, S, WM>, (size_t)G::BUF, (size_t)TH * G::TWG * G::RES_PITCH};
+}
+const P16Entry kEntries[] = {
+    entry<8, 10, 1, 4>(), entry<10, 8, 1, 4>(), entry<8, 8, 1, 4>(), entry<8, 6, 1, 4>(), entry<4, 8, 1, 4>(), entry<4, 4, 1, 4>(),
+    entry<10, 8, 2, 4>(), entry<8, 10, 2, 4>(), entry<8, 8, 2, 4>(),
+    entry<8, 6, 2, 2>(), entry<4, 8, 2, 2>(), entry<8, 4, 2, 2>(),
+};
+size_t entry_lds(const P16Entry& e, int cin_chunks, bool residual) {
+    return (size_t)(cin_chunks > 1 ? 2 : 1) * e.buf + 2 * (size_t)(32 * e.wm) * 4 + (residual ? e.res_bytes : 0);
+}
 }  // namespace
 
 int conv_p16_tile_count() { return (int)(sizeof(kEntries) / sizeof(kEntries[0])); }
-void conv_p16_tile(int index, int* th, int* tw, size_t* lds) {
-    *th = kEntries[index].th; *tw = kEntries[index].tw; *lds = kEntries[index].lds;
+void conv_p16_tile(int index, int* th, int* tw, int* stride, int* wm) {
+    *th = kEntries[index].th; *tw = kEntries[index].tw; *stride = kEntries[index].stride; *wm = kEntries[index].wm;
+}
+static const P16Entry* find_entry(const ConvP16Params& p) {
+    for (const P16Entry& c : kEntries)
+        if (c.th == p.tile_h && c.tw == p.tile_w && c.stride == p.stride && c.wm == p.wm) return &c;
+    return nullptr;
+}
+size_t conv_p16_lds_bytes(const ConvP16Params& p) {
+    const P16Entry* e = find_entry(p);
+    return e ? entry_lds(*e, p.cin_chunks, p.res != nullptr) : 0;
 }
 
 bool conv_p16_supported(int k, int stride, int dil, int in_cp, int cout, int out_cp, bool f16) {
-    return k == 3 && stride == 1 && dil == 1 && !f16 && in_cp % (2 * KC) == 0 && cout % CPB == 0 && out_cp % 4 == 0 && out_cp >= cout;
+    return k == 3 && (stride == 1 || stride == 2) && dil == 1 && !f16 && in_cp % KC == 0 && cout % 64 == 0 && out_cp % 4 == 0 && out_cp >= cout;
 }
 
 int launch_conv_p16(const ConvP16Params& p, hipStream_t s) {
-    const P16Entry* e = nullptr;
-    for (const P16Entry& c : kEntries)
-        if (c.th == p.tile_h && c.tw == p.tile_w) e = &c;
+    const P16Entry* e = find_entry(p);
     if (!e) return -1;
+    const int cpb = 32 * e->wm, twg = (4 / e->wm) * e->tw;
     // what the kernel's indexing assumes
-    if (p.cin_chunks < 2 || p.cin_chunks % 2 || p.in_cp != p.cin_chunks * KC || p.cout_blocks < 1 || p.mfrags < p.cout_blocks * 8 ||
-        p.tiles_x * p.tile_w < p.npos_x || p.tiles_y * p.tile_h < p.npos_y || p.out_cp < p.cout_blocks * CPB ||
-        (p.res && p.res_cp < p.cout_blocks * CPB) || p.nreset < 0 || p.nreset > 4)
+    if (p.cin_chunks < 1 || p.in_cp != p.cin_chunks * KC || p.cout_blocks < 1 || p.mfrags < p.cout_blocks * 2 * e->wm ||
+        p.tiles_x * twg < p.npos_x || p.tiles_y * p.tile_h < p.npos_y || p.out_cp < p.cout_blocks * cpb ||
+        (p.res && p.res_cp < p.cout_blocks * cpb) || p.nreset < 0 || p.nreset > 4)
         return -5;
-    if (e->lds > 160 * 1024) return -2;
-    if (ensure_lds(reinterpret_cast<const void*>(e->fn), e->lds) != 0) return -2;
+    const size_t lds_bytes = entry_lds(*e, p.cin_chunks, p.res != nullptr);
+    if (lds_bytes > 160 * 1024) return -2;
+    if (ensure_lds(reinterpret_cast<const void*>(e->fn), lds_bytes) != 0) return -2;
 #ifdef FYN_P16_TRACE
     {
         static long long* dev = nullptr;
@@ -351,7 +419,7 @@ int launch_conv_p16(const ConvP16Params& p, hipStream_t s) {
         ConvP16Params q = p;
         q.trace = dev;
         if (const char* e = getenv("FYNHIP_P16_CHUNKS")) q.cin_chunks = atoi(e);   // (timing study: fewer chunks, wrong results)
-        hipLaunchKernelGGL(e->fn, dim3(p.tiles_x * p.tiles_y * p.cout_blocks), dim3(512), e->lds, s, q);
+        hipLaunchKernelGGL(e->fn, dim3(p.tiles_x * p.tiles_y * p.cout_blocks), dim3(512), lds_bytes, s, q);
         hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
         (void)hipStreamIsCapturing(s, &cap);
         const char* path = cap == hipStreamCaptureStatusNone ? getenv("FYNHIP_TRACE_DUMP") : nullptr;
@@ -364,7 +432,7 @@ int launch_conv_p16(const ConvP16Params& p, hipStream_t s) {
         return hipGetLastError() == hipSuccess ? 0 : -3;
     }
 #endif
-    hipLaunchKernelGGL(e->fn, dim3(p.tiles_x * p.tiles_y * p.cout_blocks), dim3(512), e->lds, s, p);
+    hipLaunchKernelGGL(e->fn, dim3(p.tiles_x * p.tiles_y * p.cout_blocks), dim3(512), lds_bytes, s, p);
     return hipGetLastError() == hipSuccess ? 0 : -3;
 }
 

@@ -164,26 +164,29 @@ bool conv_rows_supported(int k, int cin_pitch, int cout, bool f16);
 size_t conv_rows_lds_bytes(const ConvRowsParams& p, bool f16);
 int launch_conv_rows(const ConvRowsParams& p, bool f16, hipStream_t s);
 
-// 3x3 stride-1 convolution with fp32 storage on 16-position fragments (conv_p16.hip): tiles of tile_h x tile_w
-// positions (compiled pairs only, see conv_p16_tile), 128 output channels per workgroup.
+// 3x3 convolution (stride 1 or 2) with fp32 storage on 16-position fragments (conv_p16.hip).  A workgroup's four MFMA
+// waves are wm groups of 32 output channels x 4/wm tiles of tile_h x tile_w positions side by side (compiled
+// combinations only, see conv_p16_tile).
 struct ConvP16Params {
     const void* in;
     void* out;
     const void* res;      // residual tensor or nullptr
     const void* wpack;    // [(chunk*9 + ky*3 + kx)][cout fragment of 16][plane hi, lo][lane 0..63][8 halves]: output channel
                           // 16*fragment + lane%16, input channel 32*chunk + 8*(lane/16) + j; 6 steps of zeros behind the last
-    const float* scale;   // [cout_blocks*128]
-    const float* bias;    // [cout_blocks*128]
+    const float* scale;   // [cout_blocks*32*wm]
+    const float* bias;    // [cout_blocks*32*wm]
     int in_hp, in_wp, in_cp;   // stored input frame; in_cp = 32*cin_chunks
+    int stride;           // input step per output position
     int in_y0, in_x0;     // stored coordinate of tap (0,0) of output position (0,0) (input padding - 1)
     int in_clamp;         // coordinates outside the stored frame repeat its edge instead of reading 0
     int npos_y, npos_x;
     int out_wp, out_cp, out_off_y, out_off_x;
     int res_wp, res_cp, res_off_y, res_off_x, res_relu, res_scale;
-    int tile_h, tile_w, tiles_x, tiles_y;
-    int cin_chunks;       // even
+    int tile_h, tile_w, wm;    // tiles_x counts workgroup tiles of (4/wm)*tile_w columns
+    int tiles_x, tiles_y;
+    int cin_chunks;
     int mfrags;           // cout fragments (16 each) in wpack
-    int cout_blocks;
+    int cout_blocks;      // workgroups along cout (32*wm channels each)
     float acc_mul;
     const unsigned* in_amax;   // value-range words as in ConvMfmaParams
     unsigned* out_amax;
@@ -196,7 +199,8 @@ struct ConvP16Params {
 };
 bool conv_p16_supported(int k, int stride, int dil, int in_cp, int cout, int out_cp, bool f16);
 int conv_p16_tile_count();
-void conv_p16_tile(int index, int* th, int* tw, size_t* lds_bytes);
+void conv_p16_tile(int index, int* th, int* tw, int* stride, int* wm);
+size_t conv_p16_lds_bytes(const ConvP16Params& p);   // 0: no such compiled combination
 int launch_conv_p16(const ConvP16Params& p, hipStream_t s);
 
 // ---------------------------------------------------------------------------------------------

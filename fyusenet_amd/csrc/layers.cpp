@@ -441,6 +441,20 @@ static void tune_cache_store_flag(const char* key, bool flag) {
     v.fm = flag ? 1 : 0;
     tune_cache_store(key, v, 0, 0);
 }
+// three numbers under a key of their own (same file)
+static bool tune_cache_triple(const char* key, int (&out)[3]) {
+    if (tune_cache_bypassed()) return false;
+    std::lock_guard<std::mutex> lk(g_tune_mu);
+    auto it = tune_cache().find(key);
+    if (it == tune_cache().end()) return false;
+    out[0] = it->second[0]; out[1] = it->second[1]; out[2] = it->second[2];
+    return true;
+}
+static void tune_cache_store_triple(const char* key, int a, int b, int c) {
+    ConvVariant v{};
+    v.fm = a; v.fn = b; v.wm = c;
+    tune_cache_store(key, v, 0, 0);
+}
 
 // Picks the tile configuration of one (sub-)convolution: by measurement on the layer's own tensors (default), or by
 // the heuristic score when FYNHIP_AUTOTUNE=0.  Candidates are timed before the weights are packed, i.e. on zero
@@ -862,12 +876,14 @@ class ConvLayer : public Layer {
         (rows ? rp.reset : (p16 ? pp.reset : launch.p.reset))[n++] = w;
         return true;
     }
-    // 16-position-fragment form of a 3x3 convolution (conv_p16.hip): the compiled tile that needs the fewest fragment
-    // rounds on 256 CUs, kept when it is faster than the tuned launch of the general kernel.
+    // 16-position-fragment form of a 3x3 convolution (conv_p16.hip): the compiled combinations that fit the layer are
+    // timed (the three with the fewest fragment rounds on 256 CUs), and the best is kept if it beats the tuned launch of
+    // the general kernel.
     void setup_p16(const TView& in_v, const TView& out_v, const TView* res_v, int res_relu, int res_scale) {
         ConvP16Params q{};
         q.in = in_v.ptr; q.out = out_v.ptr; q.res = res_v ? res_v->ptr : nullptr;
         q.in_hp = in_v.hp(); q.in_wp = in_v.wp(); q.in_cp = in_v.cp;
+        q.stride = stride;
         q.in_y0 = q.in_x0 = in_v.pad - 1;
         q.in_clamp = clamp ? 1 : 0;
         q.npos_y = oh; q.npos_x = ow;
@@ -875,52 +891,72 @@ class ConvLayer : public Layer {
         if (res_v) { q.res_wp = res_v->wp(); q.res_cp = res_v->cp; q.res_off_y = q.res_off_x = res_v->pad; }
         q.res_relu = res_relu; q.res_scale = res_scale;
         q.cin_chunks = in_v.cp / 32;
-        q.cout_blocks = oc / 128;
-        q.mfrags = q.cout_blocks * 8;
+        q.mfrags = oc / 16;
         q.scale = scale_dev; q.bias = bias_dev;
         q.acc_mul = 1.f;
         q.act = act();
-        double best = 1e30;
-        int want_h = 0, want_w = 0;   // FYNHIP_P16_TILE=h,w (tests): that tile
-        if (const char* e = getenv("FYNHIP_P16_TILE")) sscanf(e, "%d,%d", &want_h, &want_w);
+        int want_h = 0, want_w = 0, want_wm = 0;   // FYNHIP_P16_TILE=h,w[,wm] (tests): that combination
+        if (const char* e = getenv("FYNHIP_P16_TILE")) sscanf(e, "%d,%d,%d", &want_h, &want_w, &want_wm);
+        struct Cand { double cost; ConvP16Params q; };
+        std::vector<Cand> cands;
         for (int i = 0; i < conv_p16_tile_count(); i++) {
-            int th, tw;
-            size_t lds;
-            conv_p16_tile(i, &th, &tw, &lds);
-            if (lds > 160 * 1024 || (want_h && (th != want_h || tw != want_w))) continue;
-            const int tx = (ow + tw - 1) / tw, ty = (oh + th - 1) / th;
-            const int rounds = (tx * ty * q.cout_blocks + 255) / 256;
-            const double cost = (double)rounds * (th * tw + 24);   // (+24: a round's fixed part, in positions)
-            if (cost < best) {
-                best = cost;
-                q.tile_h = th; q.tile_w = tw; q.tiles_x = tx; q.tiles_y = ty;
-            }
+            int th, tw, st, wm;
+            conv_p16_tile(i, &th, &tw, &st, &wm);
+            if (st != stride || oc % (32 * wm) != 0) continue;
+            if (want_h && (th != want_h || tw != want_w || (want_wm && wm != want_wm))) continue;
+            ConvP16Params c = q;
+            c.tile_h = th; c.tile_w = tw; c.wm = wm;
+            const int twg = (4 / wm) * tw;
+            c.tiles_x = (ow + twg - 1) / twg; c.tiles_y = (oh + th - 1) / th;
+            c.cout_blocks = oc / (32 * wm);
+            const size_t lds = conv_p16_lds_bytes(c);
+            if (lds == 0 || lds > 160 * 1024) continue;
+            // (a workgroup's eight waves take 140-240 registers each: one workgroup per CU whatever its LDS share)
+            const int rounds = (c.tiles_x * c.tiles_y * c.cout_blocks + 255) / 256;
+            cands.push_back(Cand{(double)rounds * (th * tw + 24), c});   // (+24: a round's fixed part, in positions)
         }
-        if (best >= 1e30) return;
+        if (cands.empty()) return;
+        std::sort(cands.begin(), cands.end(), [](const Cand& a, const Cand& b) { return a.cost < b.cost; });
+        if (cands.size() > 3) cands.resize(3);
         const size_t halves = ((size_t)q.cin_chunks * 9 + 8) * q.mfrags * 2 * 64 * 8;
-        q.wpack = p16_wpack_dev = net->dev_alloc(halves * 2, true);
+        p16_wpack_dev = net->dev_alloc(halves * 2, true);
+        for (Cand& c : cands) c.q.wpack = p16_wpack_dev;
         const bool always = getenv("FYNHIP_FORCE_P16_CONV") != nullptr;
         const char* at = getenv("FYNHIP_AUTOTUNE");
-        bool pick = true;
+        const bool timing = !(at && at[0] == '0');
+        int pick = 0;   // index into cands, -1: the general kernel
         char key[160];
-        snprintf(key, sizeof(key), "p16:%dx%d:%dx%d:cp%d:r%d:e%d", d.in_channels, oc, oh, ow, in_v.cp, res_v ? 1 : 0, clamp ? 1 : 0);
-        if (always) {
-        } else if (tune_cache_flag(key, &pick)) {
-        } else if (!(at && at[0] == '0')) {
-            float t_p16 = 1e30f, t_other = 1e30f;
+        snprintf(key, sizeof(key), "p16:%dx%d:%dx%d:s%d:cp%d:r%d:e%d", d.in_channels, oc, oh, ow, stride, in_v.cp, res_v ? 1 : 0, clamp ? 1 : 0);
+        int cached[3] = {0, 0, 0};
+        bool have_cached = false;
+        if (!want_h) have_cached = tune_cache_triple(key, cached);   // (the cache keeps: chosen?, tile_h*1000 + tile_w, wm)
+        if (have_cached) {
+            pick = -1;
+            if (cached[0] || always)
+                for (size_t i = 0; i < cands.size(); i++)
+                    if (cands[i].q.tile_h * 1000 + cands[i].q.tile_w == cached[1] && cands[i].q.wm == cached[2]) pick = (int)i;
+            if (always && pick < 0) pick = 0;
+        } else if (timing) {
+            float best = 1e30f, t_other = 1e30f;
             for (int rep = 0; rep < 3; rep++) {
-                t_p16 = std::min(t_p16, time_calls(net, [&]() {
-                    if (launch_conv_p16(q, net->stream) != 0) fail(FYN_ERR_DEVICE, "16-position convolution launch failed while tuning");
-                }, 10));
+                for (size_t i = 0; i < cands.size(); i++) {
+                    const float t = time_calls(net, [&]() {
+                        if (launch_conv_p16(cands[i].q, net->stream) != 0) fail(FYN_ERR_DEVICE, "16-position convolution launch failed while tuning");
+                    }, 10);
+                    if (t < best) { best = t; pick = (int)i; }
+                }
                 t_other = std::min(t_other, time_launch(net, launch, 10));
             }
-            if (getenv("FYNHIP_TUNE_VERBOSE")) fprintf(stderr, "[tune] 3x3: 16-position fragments (%dx%d tiles) %.1f us, general kernel %.1f us\n", q.tile_h, q.tile_w, t_p16 * 1e3f, t_other * 1e3f);
-            pick = t_p16 < t_other;
-            tune_cache_store_flag(key, pick);
+            if (getenv("FYNHIP_TUNE_VERBOSE"))
+                fprintf(stderr, "[tune] 3x3: 16-position fragments (%dx%d tiles, %d channel groups) %.1f us, general kernel %.1f us\n",
+                        cands[pick].q.tile_h, cands[pick].q.tile_w, cands[pick].q.wm, best * 1e3f, t_other * 1e3f);
+            const bool win = best < t_other;
+            if (!want_h) tune_cache_store_triple(key, win ? 1 : 0, cands[pick].q.tile_h * 1000 + cands[pick].q.tile_w, cands[pick].q.wm);
+            if (!win && !always) pick = -1;
         }
-        if (pick) {
+        if (pick >= 0) {
             p16 = true;
-            pp = q;
+            pp = cands[pick].q;
         } else {
             net->dev_free(p16_wpack_dev);
             p16_wpack_dev = nullptr;
@@ -1152,7 +1188,7 @@ class ConvLayer : public Layer {
             scale_dev = static_cast<float*>(net->dev_alloc(padded * sizeof(float)));
             bias_dev = static_cast<float*>(net->dev_alloc(padded * sizeof(float)));
             launch = tune_mfma(net, sc, in_v, out_v, res_v, d.in_channels, oc, act(), res_relu, res_scale, scale_dev, bias_dev);
-            if (!frac_shift && conv_p16_supported(k, stride, dil, in_v.cp, oc, out_v.cp, out_v.f16 != 0) && d.in_channels == in_v.cp &&
+            if (!frac_shift && !sc.in_sub && conv_p16_supported(k, stride, dil, in_v.cp, oc, out_v.cp, out_v.f16 != 0) && d.in_channels == in_v.cp &&
                 (!res_v || res_v->cp >= oc) && !getenv("FYNHIP_NO_P16_CONV"))
                 setup_p16(in_v, out_v, res_v, res_relu, res_scale);
         }
@@ -1245,15 +1281,9 @@ class ConvLayer : public Layer {
         }
         if (p16) {
             char buf[200];
-            size_t lds = 0;
-            for (int i = 0; i < conv_p16_tile_count(); i++) {
-                int th, tw;
-                size_t l;
-                conv_p16_tile(i, &th, &tw, &l);
-                if (th == pp.tile_h && tw == pp.tile_w) lds = l;
-            }
-            snprintf(buf, sizeof(buf), "conv_p16 f16x2-split tile=128x%d(cout x pos) th=%d tw=%d blocks=%d lds=%zu steps=9 chunks=%d",
-                     pp.tile_h * pp.tile_w, pp.tile_h, pp.tile_w, pp.tiles_x * pp.tiles_y * pp.cout_blocks, lds, pp.cin_chunks);
+            snprintf(buf, sizeof(buf), "conv_p16 f16x2-split tile=%dx%d(cout x pos) waves=%dx%d th=%d tw=%d blocks=%d lds=%zu steps=9 chunks=%d",
+                     32 * pp.wm, pp.tile_h * pp.tile_w * (4 / pp.wm), pp.wm, 4 / pp.wm, pp.tile_h, pp.tile_w, pp.tiles_x * pp.tiles_y * pp.cout_blocks,
+                     conv_p16_lds_bytes(pp), pp.cin_chunks);
             return mode + buf;
         }
         if (wide) return mode + (fused ? "wide-kernel(kx folded into cout, summed in the epilogue) " : "wide-kernel(kx folded into cout)+shift_reduce ") + mfma_info(launch);

@@ -250,28 +250,36 @@ def test_wide_kernel_row_rolling_form(case, shallow, storage, monkeypatch):
 
 
 P16_CASES = [
-    # (cin, cout, h, w, tile, kw)
-    (128, 128, 16, 20, "8,10", {}),                                           # whole tiles
-    (128, 128, 19, 23, "8,10", {"bn": True, "residual": (A.RELU, True)}),     # ragged in both directions
-    (64, 128, 9, 7, "8,8", {"residual": (A.NONE, False)}),                    # two chunks, one partial tile
-    (192, 256, 13, 30, "8,6", {"bn": True}),                                  # six chunks, two blocks of output channels
-    (128, 128, 11, 17, "4,8", {"pad_out": 2}),
-    (64, 128, 6, 5, "4,4", {"residual": (A.RELU, False)}),
-    (128, 128, 30, 41, None, {"residual": (A.NONE, False)}),                    # the engine's own choice of tile
+    # (cin, cout, h, w, stride, tile "h,w,channel groups", kw)  -- h, w: input size
+    (128, 128, 16, 20, 1, "8,10,4", {}),                                           # whole tiles
+    (128, 128, 19, 23, 1, "8,10,4", {"bn": True, "residual": (A.RELU, True)}),     # ragged in both directions
+    (64, 128, 9, 7, 1, "8,8,4", {"residual": (A.NONE, False)}),                    # two chunks, one partial tile
+    (192, 256, 13, 30, 1, "8,6,4", {"bn": True}),                                  # six chunks, two blocks of output channels
+    (128, 128, 11, 17, 1, "4,8,4", {"pad_out": 2}),
+    (64, 128, 6, 5, 1, "4,4,4", {"residual": (A.RELU, False)}),
+    (128, 128, 30, 41, 1, None, {"residual": (A.NONE, False)}),                    # the engine's own choice of tile
+    (96, 128, 21, 18, 1, "10,8,4", {"bn": True}),                                  # three chunks: a pair and an odd one
+    (32, 128, 12, 9, 1, "8,8,4", {"residual": (A.RELU, True), "bn": True}),        # a single chunk (one staging buffer)
+    (64, 128, 40, 34, 2, "10,8,4", {"bn": True}),                                  # stride 2: even/odd column halves
+    (64, 128, 26, 44, 2, "8,10,4", {"pad_out": 1}),
+    (96, 256, 18, 30, 2, "8,8,4", {}),
+    (32, 64, 50, 46, 2, "8,6,2", {"bn": True}),                                    # two channel groups x two tiles side by side
+    (32, 64, 22, 70, 2, "4,8,2", {"pad_out": 1}),
+    (64, 192, 34, 20, 2, "8,4,2", {}),
 ]
 
 
 @pytest.mark.parametrize("shallow", [False, True], ids=["deep", "shallow_edge_clamp"])
 @pytest.mark.parametrize("act", [A.RELU, A.LEAKY_RELU, A.NONE], ids=["relu", "leaky", "none"])
-@pytest.mark.parametrize("case", P16_CASES, ids=lambda c: "%dx%dx%d_to%d_%s" % (c[0], c[2], c[3], c[1], (c[4] or "auto").replace(",", "x")))
+@pytest.mark.parametrize("case", P16_CASES, ids=lambda c: "%dx%dx%d_to%d_s%d_%s" % (c[0], c[2], c[3], c[1], c[4], (c[5] or "auto").replace(",", "x")))
 def test_sixteen_position_fragment_form(case, act, shallow, monkeypatch):
     """The 3x3 convolution on 16-position fragments (fp32 storage only): every compiled tile, ragged edges, the
     residual tile through LDS, value ranges on both sides."""
-    cin, cout, h, w, tile, kw = case
+    cin, cout, h, w, stride, tile, kw = case
     if shallow and ("residual" in kw or "pad_out" in kw):
         pytest.skip("the shallow variant is run on the plain cases")
-    if act is not A.RELU and ("pad_out" in kw or tile in ("4,4", "8,6")):
-        pytest.skip("activations are varied on three of the cases")
+    if act is not A.RELU and ("pad_out" in kw or tile in ("4,4,4", "8,6,4", "8,8,4", "8,4,2", "4,8,2")):
+        pytest.skip("activations are varied on some of the cases")
     monkeypatch.setenv("FYNHIP_FORCE_P16_CONV", "1")
     if tile:
         monkeypatch.setenv("FYNHIP_P16_TILE", tile)
@@ -279,18 +287,19 @@ def test_sixteen_position_fragment_form(case, act, shallow, monkeypatch):
         kw = dict(kw, deep=False, pad_in=0)
     if act is A.LEAKY_RELU:
         kw = dict(kw, leak=0.1)
-    b = conv_builder(3, cout, h, w, cin, 1, 1, act, **kw)
+    b = conv_builder(3, cout, h, w, cin, stride, 1, act, **kw)
     wts = conv_block(1000 + cin, cout, 3, cin, bn=kw.get("bn", False))
     inputs = [prng.uniform(47 * cin + h, (cin, h, w), -1, 1)]
     if "residual" in kw:
-        inputs.append(prng.uniform(53, (cout, h, w), -1, 1))
+        inputs.append(prng.uniform(53, (cout, h // stride, w // stride), -1, 1))
     got, info = run_single(b, fa.STORAGE_F32, inputs, wts)
     ref = oracle_single(b, fa.STORAGE_F32, inputs, wts)
     err = rel_l2(got, ref)
     print("  ", info, "rel_l2=%.3e" % err, flush=True)
     assert "conv_p16" in info
     if tile:
-        assert "th=%s tw=%s" % tuple(tile.split(",")) in info
+        th, tw, wm = tile.split(",")
+        assert "waves=%sx" % wm in info and "th=%s tw=%s" % (th, tw) in info
     assert err <= TOL[fa.STORAGE_F32], info
 
 
