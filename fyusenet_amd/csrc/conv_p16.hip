@@ -21,6 +21,9 @@
 #include <hip/hip_fp16.h>
 #include <hip/hip_runtime.h>
 
+#include <cstdlib>
+#include <type_traits>
+
 #include "kernels.h"
 #include "range.h"
 
@@ -103,33 +106,34 @@ struct Geo {
     static_assert(NPOS % 16 == 0, "whole position fragments");
     static_assert(PLANE + 2 * ROW_PITCH + 2 * PITCH + HWH * PITCH + 64 < 65536, "B fragment offsets inside a staging buffer fit the LDS instructions' immediate field");
 };
-// NCH chunks of nine steps, starting in staging buffer 0 (the B fragments of its first step are in `b`); two chunks end
-// with the fragments of the first step of buffer 0 again.  One slot per MFMA: the MFMA, then a share of the
-// step's memory instructions, fenced so that the compiler keeps the order (a memory instruction issued right after an
-// MFMA runs in its shadow).  Position fragment fn is used by six consecutive MFMAs; its registers are then refilled
-// with the fragment of the next step, so one register set per fragment is enough.  The ring slot of the previous
-// step is refilled with the weights of step t+PD-1.  The barrier of a chunk sits in its last step, before the first
-// read of the next chunk's buffer: the staging waves have filled that buffer by then, and all reads of the current
-// buffer were issued a step earlier.
-template <class G, int NCH>
-__device__ __forceinline__ void p16_steps(f32x4_t (&acc)[2][G::FN], half8_t (&a_q)[PD][2][2], half8_t (&b)[G::FN][2],
+// One stage = the nine steps of one 32-channel chunk of one tile, read from staging buffer BUFI (stages alternate between
+// the two buffers; the B fragments of the stage's first step are in `b`, and the stage ends with those of the first step
+// of the other buffer, i.e. of the stage that follows).  One slot per MFMA: the MFMA, then a share of the step's memory
+// instructions, fenced so that the compiler keeps the order (a memory instruction issued right after an MFMA runs in
+// its shadow).  Position fragment fn is used by six consecutive MFMAs; its registers are then refilled with the
+// fragment of the next step, so one register set per fragment is enough.  The ring slot of the previous step is
+// refilled with the weights of step t+PD-1 (the weight stream wraps from the last step of a tile to the first of the
+// next).  The barrier of a stage sits in its last step, before the first read of the other buffer: the staging waves
+// have filled that buffer by then, and all reads of this stage's buffer were issued a step earlier.
+template <class G, int BUFI>
+__device__ __forceinline__ void p16_stage(f32x4_t (&acc)[2][G::FN], half8_t (&a_q)[PD][2][2], half8_t (&b)[G::FN][2],
                                           const int (&bbase)[2][G::FN], const unsigned char* lds, const unsigned char*& wnext,
-                                          unsigned wstep) {
+                                          const unsigned char* wbase, const unsigned char* wend, unsigned wstep) {
     constexpr int FN = G::FN;
 #pragma unroll
-    for (int dd = 0; dd < NCH * NT; dd++) {
-        const int d = dd % PD, dprev = (d + PD - 1) % PD;
-        const int nd = dd + 1;                                   // the next step: buffer and tap
-        const int nbuf = (nd / NT) & 1, noff = G::tap_off(nd % NT);
+    for (int dd = 0; dd < NT; dd++) {
+        const int d = (BUFI * NT + dd) % PD, dprev = (d + PD - 1) % PD;   // (two stages = 18 steps = three turns of the ring)
+        const int nbuf = (dd + 1 == NT) ? 1 - BUFI : BUFI, noff = G::tap_off((dd + 1) % NT);
         const unsigned char* w_ = wnext;
         wnext += wstep;
+        if (wnext == wend) wnext = wbase;
 #pragma unroll
         for (int i = 0; i < 6 * FN; i++) {
             const int fn = i / 6, r = i % 6, kind = r / 2, fm = r % 2;
             const int apl = (kind == 1) ? 1 : 0, bpl = (kind == 2) ? 1 : 0;
             acc[fm][fn] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_q[d][fm][apl], b[fn][bpl], acc[fm][fn], 0, 0, 0);
-            if (dd % NT == NT - 1 && i == 3) lds_barrier();
-            if (r == 5 && !(NCH == 1 && dd == NT - 1)) {   // (a single chunk is the launch's last: nothing follows its last step)
+            if (dd == NT - 1 && i == 3) lds_barrier();
+            if (r == 5) {
                 b[fn][0] = *reinterpret_cast<const half8_t*>(lds + bbase[nbuf][fn] + noff);
                 b[fn][1] = *reinterpret_cast<const half8_t*>(lds + bbase[nbuf][fn] + noff + G::PLANE);
             }
@@ -141,6 +145,10 @@ __device__ __forceinline__ void p16_steps(f32x4_t (&acc)[2][G::FN], half8_t (&a_
     }
 }
 
+// Grid: cout_blocks x pos_groups workgroups; a workgroup keeps its block of output channels and walks the tiles
+// group, group + pos_groups, ... (one tile each when the layer has no more tiles than the chip has CUs).  The staging
+// waves run one stage ahead of the MFMA waves, across tile boundaries, so that from the second tile on a tile's fetch
+// and the previous tile's stores overlap with MFMA work.
 template <int TH, int TW, int S, int WM>
 __global__ __launch_bounds__(512) void conv_p16_kernel(const ConvP16Params p) {
     using G = Geo<TH, TW, S, WM>;
@@ -155,59 +163,69 @@ __global__ __launch_bounds__(512) void conv_p16_kernel(const ConvP16Params p) {
     // Workgroups are dealt round-robin to the 8 XCDs; remap so that neighbouring tiles (shared halos) meet in one L2.
     int bid = blockIdx.x;
     {
-        const int nblk = p.tiles_x * p.tiles_y * p.cout_blocks;
+        const int nblk = p.pos_groups * p.cout_blocks;
         const int per = nblk >> 3;
         if (bid < (per << 3)) bid = (bid & 7) * per + (bid >> 3);
     }
     const int cb = bid % p.cout_blocks;
-    const int tile = bid / p.cout_blocks;
-    const int tyi = tile / p.tiles_x, txi = tile - tyi * p.tiles_x;
-    const int pos_y0 = tyi * TH, pos_x0 = txi * G::TWG;
+    const int group = bid / p.cout_blocks;
+    const int ntiles = p.tiles_x * p.tiles_y;
     if (tid < 2) range_box[tid] = 0u;
     const unsigned range_bits = p.in_amax ? range_load(p.in_amax) : 0u;
     const int nchunks = p.cin_chunks;
-    // LDS: one staging buffer (two when there is more than one chunk), scale and bias, the residual tile
-    const int sb_off = (nchunks > 1 ? 2 : 1) * G::BUF;
-    const int res_off = sb_off + 2 * CPB * 4;
+    // LDS: two staging buffers, scale and bias, the residual tile
+    constexpr int sb_off = 2 * G::BUF;
+    constexpr int res_off = sb_off + 2 * CPB * 4;
 
     if (wave < 4) {
         // ------------------------------------------------------------------ staging waves (the first four: they start first)
         const int stid = tid & 255;
         const float* in = reinterpret_cast<const float*>(p.in);
-        int g_off[G::NB], l_off[G::NB];
+        int i_y[G::NB], i_x[G::NB];   // an item's pixel inside the halo tile (rows above 2^15: no such item)
+        int l_off[G::NB];
 #pragma unroll
         for (int i = 0; i < G::NB; i++) {
             const int idx = stid + i * 256;
-            g_off[i] = -1; l_off[i] = -1;
+            l_off[i] = -1; i_y[i] = 1 << 20; i_x[i] = 0;
             if (idx < G::NITEMS) {
                 const int pix = idx >> 2, g = idx & 3;
                 const int py = pix / G::HW, px = pix - py * G::HW;
-                int gy = pos_y0 * S + p.in_y0 + py, gx = pos_x0 * S + p.in_x0 + px;
+                i_y[i] = py; i_x[i] = px;
                 l_off[i] = py * G::ROW_PITCH + ((S == 1) ? px * PITCH : ((px & 1) * G::HWH + (px >> 1)) * PITCH) + g * 16;
-                if (p.in_clamp) {
+            }
+        }
+        const int g8 = (stid & 3) * 8;
+        // Two sets of staging registers: the loads of stage n+2 are issued before stage n+1 is converted, so a stage's
+        // memory latency passes while the stage before it is written to LDS.
+        int g_off[2][G::NB];       // element offsets of a set's items, -1: outside the frame (reads as 0)
+        float4 raw[2][G::NB][2];
+        float in_scale = 1.f, inv_unused;
+        // (unconditional loads: items outside the tensor read its first element and are zeroed when stored)
+        auto fetch = [&](auto set_, int tile, int chunk) {
+            constexpr int SET = decltype(set_)::value;
+            const int tyi = (int)(((float)tile + 0.5f) * p.rcp_tiles_x), txi = tile - tyi * p.tiles_x;
+            const int y0 = tyi * TH * S + p.in_y0, x0 = txi * G::TWG * S + p.in_x0;
+#pragma unroll
+            for (int i = 0; i < G::NB; i++) {
+                int gy = y0 + i_y[i], gx = x0 + i_x[i];
+                if (p.in_clamp && l_off[i] >= 0) {
                     gy = min(max(gy, 0), p.in_hp - 1);
                     gx = min(max(gx, 0), p.in_wp - 1);
                 }
-                if ((unsigned)gy < (unsigned)p.in_hp && (unsigned)gx < (unsigned)p.in_wp) g_off[i] = (gy * p.in_wp + gx) * p.in_cp + g * 8;
-            }
-        }
-        float4 raw[G::NB][2];
-        // (unconditional loads: items outside the tensor read its first element and are zeroed when stored)
-        auto fetch = [&](int chunk) {
-#pragma unroll
-            for (int i = 0; i < G::NB; i++) {
-                const float* src = in + (g_off[i] >= 0 ? g_off[i] + chunk * KC : 0);
-                raw[i][0] = *reinterpret_cast<const float4*>(src);
-                raw[i][1] = *reinterpret_cast<const float4*>(src + 4);
+                g_off[SET][i] = ((unsigned)gy < (unsigned)p.in_hp && (unsigned)gx < (unsigned)p.in_wp) ? (gy * p.in_wp + gx) * p.in_cp + g8 + chunk * KC : -1;
+                const float* src = in + (g_off[SET][i] >= 0 ? g_off[SET][i] : 0);
+                raw[SET][i][0] = *reinterpret_cast<const float4*>(src);
+                raw[SET][i][1] = *reinterpret_cast<const float4*>(src + 4);
             }
         };
-        float in_scale = 1.f, inv_unused;
-        auto store = [&](unsigned char* buf) {
+        auto store = [&](auto set_, unsigned char* buf) {
+            constexpr int SET = decltype(set_)::value;
 #pragma unroll
             for (int i = 0; i < G::NB; i++) {
                 if (l_off[i] < 0) continue;
-                const bool ok = g_off[i] >= 0;
-                const float r[8] = {raw[i][0].x, raw[i][0].y, raw[i][0].z, raw[i][0].w, raw[i][1].x, raw[i][1].y, raw[i][1].z, raw[i][1].w};
+                const bool ok = g_off[SET][i] >= 0;
+                const float4 r0 = raw[SET][i][0], r1 = raw[SET][i][1];
+                const float r[8] = {r0.x, r0.y, r0.z, r0.w, r1.x, r1.y, r1.z, r1.w};
                 half8_t hi, lo;
 #pragma unroll
                 for (int e = 0; e < 8; e++) {
@@ -219,42 +237,63 @@ __global__ __launch_bounds__(512) void conv_p16_kernel(const ConvP16Params p) {
                 *reinterpret_cast<half8_t*>(buf + G::PLANE + l_off[i]) = lo;
             }
         };
+        auto residual_in = [&](int tile) {   // the residual tile of a tile: [position][CPB channels] fp32
+            const float* res = reinterpret_cast<const float*>(p.res);
+            const int tyi = (int)(((float)tile + 0.5f) * p.rcp_tiles_x), txi = tile - tyi * p.tiles_x;
+            f32x4_t rv[G::RNB];
+#pragma unroll
+            for (int i = 0; i < G::RNB; i++) {
+                const int idx = stid + i * 256;
+                const int m = idx / (CPB / 4), c4 = idx % (CPB / 4);
+                const int ty = m / G::TWG, tx = m - ty * G::TWG;
+                const int py = tyi * TH + ty, px = txi * G::TWG + tx;
+                const bool ok = idx < G::RPIECES && py < p.npos_y && px < p.npos_x;
+                rv[i] = *reinterpret_cast<const f32x4_t*>(res + (ok ? ((size_t)(p.res_off_y + py) * p.res_wp + p.res_off_x + px) * p.res_cp + cb * CPB + c4 * 4 : 0));
+            }
+#pragma unroll
+            for (int i = 0; i < G::RNB; i++) {
+                const int idx = stid + i * 256;
+                if (idx < G::RPIECES) *reinterpret_cast<f32x4_t*>(lds + res_off + (idx / (CPB / 4)) * G::RES_PITCH + (idx % (CPB / 4)) * 16) = rv[i];
+            }
+        };
+        // the stage after (tile, c); false: there is none
+        auto advance = [&](int& tile, int& c) {
+            if (++c == nchunks) { c = 0; tile += p.pos_groups; }
+            return tile < ntiles;
+        };
+        typedef std::integral_constant<int, 0> Set0;
+        typedef std::integral_constant<int, 1> Set1;
         FYN_PTRACE(0);
-        fetch(0);
+        int tile = group, c = 0;          // the stage the MFMA waves are on (stage n)
+        int t1 = group, c1 = 0;           // stage n+1
+        fetch(Set0(), tile, 0);
+        bool have1 = advance(t1, c1);
+        int t2 = t1, c2 = c1;             // stage n+2
+        bool have2 = have1 && advance(t2, c2);
         if (p.in_amax) in_scale = range_scale(range_after_act(range_reduce(range_bits), p.act), &inv_unused);
         if (stid < CPB) {
             reinterpret_cast<float*>(lds + sb_off)[stid] = p.scale[cb * CPB + stid];
             reinterpret_cast<float*>(lds + sb_off)[CPB + stid] = p.bias[cb * CPB + stid];
         }
-        store(lds);
+        store(Set0(), lds);
         FYN_PTRACE(1);
         lds_barrier();
-        for (int c = 0; c < nchunks; c++) {
-            FYN_PTRACE(2 + 2 * c);
-            if (c + 1 < nchunks) {
-                fetch(c + 1);
-                store(lds + ((c + 1) & 1) * G::BUF);
-                FYN_PTRACE(3 + 2 * c);
-            } else if (p.res) {
-                // the residual tile: [position][CPB channels] fp32
-                const float* res = reinterpret_cast<const float*>(p.res);
-                f32x4_t rv[G::RNB];
-#pragma unroll
-                for (int i = 0; i < G::RNB; i++) {
-                    const int idx = stid + i * 256;
-                    const int m = idx / (CPB / 4), c4 = idx % (CPB / 4);
-                    const int ty = m / G::TWG, tx = m - ty * G::TWG;
-                    const int py = pos_y0 + ty, px = pos_x0 + tx;
-                    const bool ok = idx < G::RPIECES && py < p.npos_y && px < p.npos_x;
-                    rv[i] = *reinterpret_cast<const f32x4_t*>(res + (ok ? ((size_t)(p.res_off_y + py) * p.res_wp + p.res_off_x + px) * p.res_cp + cb * CPB + c4 * 4 : 0));
-                }
-#pragma unroll
-                for (int i = 0; i < G::RNB; i++) {
-                    const int idx = stid + i * 256;
-                    if (idx < G::RPIECES) *reinterpret_cast<f32x4_t*>(lds + res_off + (idx / (CPB / 4)) * G::RES_PITCH + (idx % (CPB / 4)) * 16) = rv[i];
-                }
-            }
+        if (have1) fetch(Set1(), t1, c1);   // (not before the first stage is handed over: every workgroup of the launch is fetching at that moment)
+        // One iteration per stage n of the MFMA waves: stage n+1 (fetched an iteration ago) is written to the other
+        // buffer, then stage n+2 is fetched into the registers that stage n left.  Unrolled by two: set = parity of the stage.
+        auto iteration = [&](auto next_set, auto free_set, unsigned char* next_buf) {
+            if (c + 1 == nchunks && p.res) residual_in(tile);
+            if (have1) store(next_set, next_buf);
+            if (have2) fetch(free_set, t2, c2);
             lds_barrier();
+            const bool go_on = have1;
+            tile = t1; c = c1; t1 = t2; c1 = c2; have1 = have2;
+            if (have2) have2 = advance(t2, c2);
+            return go_on;
+        };
+        for (;;) {
+            if (!iteration(Set1(), Set0(), lds + G::BUF)) break;   // stage n even: n+1 is in set 1, goes into buffer 1
+            if (!iteration(Set0(), Set1(), lds)) break;
         }
         return;
     }
@@ -272,10 +311,10 @@ __global__ __launch_bounds__(512) void conv_p16_kernel(const ConvP16Params p) {
         bbase[0][fn] = S * ty * G::ROW_PITCH + (wn * TW + tx) * PITCH + kq * 16;
         bbase[1][fn] = bbase[0][fn] + G::BUF;
     }
-    // A fragments: [(chunk*9 + tap)][cout fragment of 16][plane][lane] x 8 halves; the buffer has PD steps of zero
-    // slack behind the last step, so the prefetch needs no clamp.
+    // A fragments: [(chunk*9 + tap)][cout fragment of 16][plane][lane] x 8 halves
     const unsigned wstep = (unsigned)p.mfrags * 2 * 1024;
     const unsigned char* wbase = reinterpret_cast<const unsigned char*>(p.wpack) + (size_t)((cb * 2 * WM + mw * 2) * 2) * 1024 + lane * 16;
+    const unsigned char* wend = wbase + (size_t)nchunks * NT * wstep;
     half8_t a_q[PD][2][2];
 #pragma unroll
     for (int d = 0; d < PD; d++)
@@ -284,16 +323,67 @@ __global__ __launch_bounds__(512) void conv_p16_kernel(const ConvP16Params p) {
 #pragma unroll
             for (int pl = 0; pl < 2; pl++) a_q[d][fm][pl] = *reinterpret_cast<const half8_t*>(wbase + (size_t)d * wstep + (fm * 2 + pl) * 1024);
     f32x4_t acc[2][FN];
+    auto zero_acc = [&]() {
 #pragma unroll
-    for (int fm = 0; fm < 2; fm++)
+        for (int fm = 0; fm < 2; fm++)
 #pragma unroll
-        for (int fn = 0; fn < FN; fn++) acc[fm][fn] = (f32x4_t)(0.f);
+            for (int fn = 0; fn < FN; fn++) acc[fm][fn] = (f32x4_t)(0.f);
+    };
+    zero_acc();
     float inv_in_scale = 1.f;
     if (p.in_amax) (void)range_scale(range_after_act(range_reduce(range_bits), p.act), &inv_in_scale);
     const float acc_mul = p.acc_mul * inv_in_scale;
+    float* out = reinterpret_cast<float*>(p.out);
+    const bool have_res = p.res != nullptr;
+    const bool res_relu = p.res_relu != 0, res_scale = p.res_scale != 0;
+    float vmax = 0.f;
+
+    // Epilogue of a tile.  A lane holds, per fragment, output channels 4*kq .. 4*kq+3 of position fn*16 + mq.  One
+    // wave per SIMD pays four cycles per vector instruction, so the arithmetic is kept short (acc_mul is a power of two:
+    // folding it into the scale changes no bit) and every fragment is stored as soon as it is finished.
+    auto finish_tile = [&](int tile) {
+        const int tyi = (int)(((float)tile + 0.5f) * p.rcp_tiles_x), txi = tile - tyi * p.tiles_x;
+        const float* sb = reinterpret_cast<const float*>(lds + sb_off);
+        f32x4_t sc[2], bi[2], scm[2];
+#pragma unroll
+        for (int fm = 0; fm < 2; fm++) {
+            sc[fm] = *reinterpret_cast<const f32x4_t*>(sb + mw * 32 + fm * 16 + kq * 4);
+            bi[fm] = *reinterpret_cast<const f32x4_t*>(sb + CPB + mw * 32 + fm * 16 + kq * 4);
+            scm[fm] = sc[fm] * acc_mul;
+        }
+#pragma unroll
+        for (int fn = 0; fn < FN; fn++) {
+            const int m = fn * 16 + mq;
+            const int ty = m / TW, tx = wn * TW + (m - ty * TW);
+            const int py = tyi * TH + ty, px = txi * G::TWG + tx;
+            const bool ok = py < p.npos_y && px < p.npos_x;
+            const size_t obase = ((size_t)(p.out_off_y + py) * p.out_wp + p.out_off_x + px) * p.out_cp + cb * CPB + mw * 32 + kq * 4;
+            float fmax_ = 0.f;
+#pragma unroll
+            for (int fm = 0; fm < 2; fm++) {
+                f32x4_t v;
+#pragma unroll
+                for (int e = 0; e < 4; e++) v[e] = acc[fm][fn][e] * scm[fm][e] + bi[fm][e];
+                if (have_res) {
+                    f32x4_t rv = *reinterpret_cast<const f32x4_t*>(lds + res_off + (ty * G::TWG + tx) * G::RES_PITCH + (mw * 32 + fm * 16 + kq * 4) * 4);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        float r = rv[e];
+                        if (res_relu) r = fmaxf(r, 0.f);
+                        if (res_scale) r *= sc[fm][e];
+                        v[e] += r;
+                    }
+                }
+#pragma unroll
+                for (int e = 0; e < 4; e++) fmax_ = fmaxf(fmax_, fabsf(v[e]));
+                if (ok) *reinterpret_cast<f32x4_t*>(out + obase + fm * 16) = v;
+            }
+            vmax = fmaxf(vmax, ok ? fmax_ : 0.f);
+        }
+    };
 
     FYN_PTRACE(1);
-    lds_barrier();   // chunk 0 is staged
+    lds_barrier();   // the first stage is staged
     FYN_PTRACE(2);
     half8_t b[FN][2];
 #pragma unroll
@@ -301,61 +391,26 @@ __global__ __launch_bounds__(512) void conv_p16_kernel(const ConvP16Params p) {
 #pragma unroll
         for (int pl = 0; pl < 2; pl++) b[fn][pl] = *reinterpret_cast<const half8_t*>(lds + bbase[0][fn] + pl * G::PLANE);
 
-    // pairs of chunks (one per staging buffer), then the odd one
-    const unsigned char* wnext = wbase + (size_t)(PD - 1) * wstep;
-    int g = 0;
-    for (; g + 2 <= nchunks; g += 2) {
-        p16_steps<G, 2>(acc, a_q, b, bbase, lds, wnext, wstep);
-        FYN_PTRACE(3 + g);
-    }
-    if (g < nchunks) p16_steps<G, 1>(acc, a_q, b, bbase, lds, wnext, wstep);
-
-    // ---- epilogue: a lane holds, per fragment, output channels 4*kq .. 4*kq+3 of position fn*16 + mq.  One wave per
-    //      SIMD pays four cycles per vector instruction, so the arithmetic is kept short (acc_mul is a power of two:
-    //      folding it into the scale changes no bit) and every fragment is stored as soon as it is finished. ----
-    const float* sb = reinterpret_cast<const float*>(lds + sb_off);
-    f32x4_t sc[2], bi[2], scm[2];
-#pragma unroll
-    for (int fm = 0; fm < 2; fm++) {
-        sc[fm] = *reinterpret_cast<const f32x4_t*>(sb + mw * 32 + fm * 16 + kq * 4);
-        bi[fm] = *reinterpret_cast<const f32x4_t*>(sb + CPB + mw * 32 + fm * 16 + kq * 4);
-        scm[fm] = sc[fm] * acc_mul;
-    }
-    float* out = reinterpret_cast<float*>(p.out);
-    const bool have_res = p.res != nullptr;
-    const bool res_relu = p.res_relu != 0, res_scale = p.res_scale != 0;
-    float vmax = 0.f;
-    FYN_PTRACE(29);
-#pragma unroll
-    for (int fn = 0; fn < FN; fn++) {
-        const int m = fn * 16 + mq;
-        const int ty = m / TW, tx = wn * TW + (m - ty * TW);
-        const int py = pos_y0 + ty, px = pos_x0 + tx;
-        const bool ok = py < p.npos_y && px < p.npos_x;
-        const size_t obase = ((size_t)(p.out_off_y + py) * p.out_wp + p.out_off_x + px) * p.out_cp + cb * CPB + mw * 32 + kq * 4;
-        float fmax_ = 0.f;
-#pragma unroll
-        for (int fm = 0; fm < 2; fm++) {
-            f32x4_t v;
-#pragma unroll
-            for (int e = 0; e < 4; e++) v[e] = acc[fm][fn][e] * scm[fm][e] + bi[fm][e];
-            if (have_res) {
-                f32x4_t rv = *reinterpret_cast<const f32x4_t*>(lds + res_off + (ty * G::TWG + tx) * G::RES_PITCH + (mw * 32 + fm * 16 + kq * 4) * 4);
-#pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    float r = rv[e];
-                    if (res_relu) r = fmaxf(r, 0.f);
-                    if (res_scale) r *= sc[fm][e];
-                    v[e] += r;
-                }
-            }
-#pragma unroll
-            for (int e = 0; e < 4; e++) fmax_ = fmaxf(fmax_, fabsf(v[e]));
-            if (ok) *reinterpret_cast<f32x4_t*>(out + obase + fm * 16) = v;
+    const unsigned char* wnext = wbase + (size_t)((PD - 1) % (nchunks * NT)) * wstep;
+    int tile = group, c = 0;
+    for (;;) {
+        p16_stage<G, 0>(acc, a_q, b, bbase, lds, wnext, wbase, wend, wstep);
+        if (++c == nchunks) {
+            FYN_PTRACE(29);
+            finish_tile(tile);
+            FYN_PTRACE(30);
+            c = 0; tile += p.pos_groups;
+            if (tile >= ntiles) break;
+            zero_acc();
         }
-        vmax = fmaxf(vmax, ok ? fmax_ : 0.f);
+        p16_stage<G, 1>(acc, a_q, b, bbase, lds, wnext, wbase, wend, wstep);
+        if (++c == nchunks) {
+            finish_tile(tile);
+            c = 0; tile += p.pos_groups;
+            if (tile >= ntiles) break;
+            zero_acc();
+        }
     }
-    FYN_PTRACE(30);
     if (p.out_amax) range_publish_waves(p.out_amax, vmax, range_box, 4);
     FYN_PTRACE(31);
 }
@@ -376,8 +431,8 @@ const P16Entry kEntries[] = {
     entry<10, 8, 2, 4>(), entry<8, 10, 2, 4>(), entry<8, 8, 2, 4>(),
     entry<8, 6, 2, 2>(), entry<4, 8, 2, 2>(), entry<8, 4, 2, 2>(),
 };
-size_t entry_lds(const P16Entry& e, int cin_chunks, bool residual) {
-    return (size_t)(cin_chunks > 1 ? 2 : 1) * e.buf + 2 * (size_t)(32 * e.wm) * 4 + (residual ? e.res_bytes : 0);
+size_t entry_lds(const P16Entry& e, bool residual) {
+    return 2 * e.buf + 2 * (size_t)(32 * e.wm) * 4 + (residual ? e.res_bytes : 0);
 }
 }  // namespace
 
@@ -392,7 +447,7 @@ static const P16Entry* find_entry(const ConvP16Params& p) {
 }
 size_t conv_p16_lds_bytes(const ConvP16Params& p) {
     const P16Entry* e = find_entry(p);
-    return e ? entry_lds(*e, p.cin_chunks, p.res != nullptr) : 0;
+    return e ? entry_lds(*e, p.res != nullptr) : 0;
 }
 
 bool conv_p16_supported(int k, int stride, int dil, int in_cp, int cout, int out_cp, bool f16) {
@@ -406,20 +461,23 @@ int launch_conv_p16(const ConvP16Params& p, hipStream_t s) {
     // what the kernel's indexing assumes
     if (p.cin_chunks < 1 || p.in_cp != p.cin_chunks * KC || p.cout_blocks < 1 || p.mfrags < p.cout_blocks * 2 * e->wm ||
         p.tiles_x * twg < p.npos_x || p.tiles_y * p.tile_h < p.npos_y || p.out_cp < p.cout_blocks * cpb ||
-        (p.res && p.res_cp < p.cout_blocks * cpb) || p.nreset < 0 || p.nreset > 4)
+        (p.res && p.res_cp < p.cout_blocks * cpb) || p.nreset < 0 || p.nreset > 4 || p.pos_groups < 1 || p.pos_groups > p.tiles_x * p.tiles_y ||
+        // (a tile's residual tile may not be overwritten while its epilogue reads it: the next one comes a stage later)
+        (p.res && p.cin_chunks < 2 && p.pos_groups < p.tiles_x * p.tiles_y) || p.rcp_tiles_x != 1.0f / (float)p.tiles_x ||
+        p.tiles_x * p.tiles_y > 4000000)   // (tile index -> row and column through the reciprocal: exact below four million tiles)
         return -5;
-    const size_t lds_bytes = entry_lds(*e, p.cin_chunks, p.res != nullptr);
+    const size_t lds_bytes = entry_lds(*e, p.res != nullptr);
     if (lds_bytes > 160 * 1024) return -2;
     if (ensure_lds(reinterpret_cast<const void*>(e->fn), lds_bytes) != 0) return -2;
 #ifdef FYN_P16_TRACE
     {
         static long long* dev = nullptr;
-        const size_t n = (size_t)p.tiles_x * p.tiles_y * p.cout_blocks * 64;
+        const size_t n = (size_t)p.pos_groups * p.cout_blocks * 64;
         if (!dev && hipMalloc(&dev, sizeof(long long) * 65536 * 64) != hipSuccess) return -6;
         ConvP16Params q = p;
         q.trace = dev;
         if (const char* e = getenv("FYNHIP_P16_CHUNKS")) q.cin_chunks = atoi(e);   // (timing study: fewer chunks, wrong results)
-        hipLaunchKernelGGL(e->fn, dim3(p.tiles_x * p.tiles_y * p.cout_blocks), dim3(512), lds_bytes, s, q);
+        hipLaunchKernelGGL(e->fn, dim3(p.pos_groups * p.cout_blocks), dim3(512), lds_bytes, s, q);
         hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
         (void)hipStreamIsCapturing(s, &cap);
         const char* path = cap == hipStreamCaptureStatusNone ? getenv("FYNHIP_TRACE_DUMP") : nullptr;
@@ -432,7 +490,7 @@ int launch_conv_p16(const ConvP16Params& p, hipStream_t s) {
         return hipGetLastError() == hipSuccess ? 0 : -3;
     }
 #endif
-    hipLaunchKernelGGL(e->fn, dim3(p.tiles_x * p.tiles_y * p.cout_blocks), dim3(512), lds_bytes, s, p);
+    hipLaunchKernelGGL(e->fn, dim3(p.pos_groups * p.cout_blocks), dim3(512), lds_bytes, s, p);
     return hipGetLastError() == hipSuccess ? 0 : -3;
 }
 

@@ -184,6 +184,8 @@ struct ConvP16Params {
     int res_wp, res_cp, res_off_y, res_off_x, res_relu, res_scale;
     int tile_h, tile_w, wm;    // tiles_x counts workgroup tiles of (4/wm)*tile_w columns
     int tiles_x, tiles_y;
+    float rcp_tiles_x;    // 1.0f / tiles_x
+    int pos_groups;       // workgroups per block of output channels; workgroup g walks tiles g, g + pos_groups, ...
     int cin_chunks;
     int mfrags;           // cout fragments (16 each) in wpack
     int cout_blocks;      // workgroups along cout (32*wm channels each)

@@ -908,12 +908,16 @@ class ConvLayer : public Layer {
             c.tile_h = th; c.tile_w = tw; c.wm = wm;
             const int twg = (4 / wm) * tw;
             c.tiles_x = (ow + twg - 1) / twg; c.tiles_y = (oh + th - 1) / th;
+            c.rcp_tiles_x = 1.0f / (float)c.tiles_x;
             c.cout_blocks = oc / (32 * wm);
+            // one workgroup per CU: as many tile walkers per block of output channels as the chip has room for
+            c.pos_groups = std::max(1, std::min(c.tiles_x * c.tiles_y, 256 / c.cout_blocks));
+            if (res_v && c.cin_chunks < 2) c.pos_groups = c.tiles_x * c.tiles_y;   // (residual tile: one stage per tile is too few to walk)
             const size_t lds = conv_p16_lds_bytes(c);
             if (lds == 0 || lds > 160 * 1024) continue;
             // (a workgroup's eight waves take 140-240 registers each: one workgroup per CU whatever its LDS share)
             const int rounds = (c.tiles_x * c.tiles_y * c.cout_blocks + 255) / 256;
-            cands.push_back(Cand{(double)rounds * (th * tw + 24), c});   // (+24: a round's fixed part, in positions)
+            cands.push_back(Cand{(double)rounds * (th * tw + 8) + 16, c});   // (+8: a tile's fixed part, +16: the launch's, in positions)
         }
         if (cands.empty()) return;
         std::sort(cands.begin(), cands.end(), [](const Cand& a, const Cand& b) { return a.cost < b.cost; });
@@ -1281,9 +1285,9 @@ class ConvLayer : public Layer {
         }
         if (p16) {
             char buf[200];
-            snprintf(buf, sizeof(buf), "conv_p16 f16x2-split tile=%dx%d(cout x pos) waves=%dx%d th=%d tw=%d blocks=%d lds=%zu steps=9 chunks=%d",
-                     32 * pp.wm, pp.tile_h * pp.tile_w * (4 / pp.wm), pp.wm, 4 / pp.wm, pp.tile_h, pp.tile_w, pp.tiles_x * pp.tiles_y * pp.cout_blocks,
-                     conv_p16_lds_bytes(pp), pp.cin_chunks);
+            snprintf(buf, sizeof(buf), "conv_p16 f16x2-split tile=%dx%d(cout x pos) waves=%dx%d th=%d tw=%d blocks=%d tiles=%d lds=%zu steps=9 chunks=%d",
+                     32 * pp.wm, pp.tile_h * pp.tile_w * (4 / pp.wm), pp.wm, 4 / pp.wm, pp.tile_h, pp.tile_w, pp.pos_groups * pp.cout_blocks,
+                     pp.tiles_x * pp.tiles_y * pp.cout_blocks, conv_p16_lds_bytes(pp), pp.cin_chunks);
             return mode + buf;
         }
         if (wide) return mode + (fused ? "wide-kernel(kx folded into cout, summed in the epilogue) " : "wide-kernel(kx folded into cout)+shift_reduce ") + mfma_info(launch);
