@@ -83,11 +83,12 @@ constexpr int p16_row_pad(int TH, int TW, int S, int WN, int slots) {
 // of TH x TW positions side by side; S is the input step per position (1 or 2).  With S = 2 the staged tile keeps even
 // and odd columns in separate halves of a row, so that the positions of a fragment are neighbours in LDS whatever the
 // tap: column c lives in slot (c & 1) * HWH + (c >> 1).
-template <int TH, int TW, int S, int WM>
+template <int TH_, int TW, int S, int WM, int KH = 2>
 struct Geo {
+    static constexpr int TH = TH_, STEP = S;
     static constexpr int WN = 4 / WM;
     static constexpr int TWG = WN * TW;                  // positions per row of the workgroup's tile
-    static constexpr int HW = S * (TWG - 1) + 3, HH = S * (TH - 1) + 3;
+    static constexpr int HW = S * (TWG - 1) + 1 + KH, HH = S * (TH - 1) + 1 + KH;   // (KH: 2 for 3x3 taps, 1 for the transposed layer's)
     static constexpr int HWH = (HW + 1) / 2;
     static constexpr int SLOTS = (S == 1) ? HW : 2 * HWH;
     static constexpr int ROW_PITCH = SLOTS * PITCH + p16_row_pad(TH, TW, S, WN, SLOTS);
@@ -145,6 +146,133 @@ __device__ __forceinline__ void p16_stage(f32x4_t (&acc)[2][G::FN], half8_t (&a_
     }
 }
 
+// The staging waves of a workgroup (threads 0..255): stage after stage -- a 32-channel chunk of a tile's halo: global
+// loads, activation, hi/lo conversion, LDS writes -- one stage ahead of the MFMA waves, across tile boundaries; scale and
+// bias at the start and, during a tile's last chunk, its residual tile.  One barrier per stage, after the one that hands
+// over the first.
+template <class G>
+__device__ __forceinline__ void p16_stager(const ConvP16Params& p, unsigned char* lds, int stid, int cb, int group, int ntiles,
+                                           int nchunks, unsigned range_bits) {
+    constexpr int CPB = G::CPB;
+    constexpr int sb_off = 2 * G::BUF;
+    constexpr int res_off = sb_off + 2 * CPB * 4;
+    const float* in = reinterpret_cast<const float*>(p.in);
+    int i_y[G::NB], i_x[G::NB];   // an item's pixel inside the halo tile (rows above 2^15: no such item)
+    int l_off[G::NB];
+#pragma unroll
+    for (int i = 0; i < G::NB; i++) {
+        const int idx = stid + i * 256;
+        l_off[i] = -1; i_y[i] = 1 << 20; i_x[i] = 0;
+        if (idx < G::NITEMS) {
+            const int pix = idx >> 2, g = idx & 3;
+            const int py = pix / G::HW, px = pix - py * G::HW;
+            i_y[i] = py; i_x[i] = px;
+            l_off[i] = py * G::ROW_PITCH + ((G::STEP == 1) ? px * PITCH : ((px & 1) * G::HWH + (px >> 1)) * PITCH) + g * 16;
+        }
+    }
+    const int g8 = (stid & 3) * 8;
+    // Two sets of staging registers: the loads of stage n+2 are issued before stage n+1 is converted, so a stage's
+    // memory latency passes while the stage before it is written to LDS.
+    int g_off[2][G::NB];       // element offsets of a set's items, -1: outside the frame (reads as 0)
+    float4 raw[2][G::NB][2];
+    float in_scale = 1.f, inv_unused;
+    // (unconditional loads: items outside the tensor read its first element and are zeroed when stored)
+    auto fetch = [&](auto set_, int tile, int chunk) {
+        constexpr int SET = decltype(set_)::value;
+        const int tyi = (int)(((float)tile + 0.5f) * p.rcp_tiles_x), txi = tile - tyi * p.tiles_x;
+        const int y0 = tyi * G::TH * G::STEP + p.in_y0, x0 = txi * G::TWG * G::STEP + p.in_x0;
+#pragma unroll
+        for (int i = 0; i < G::NB; i++) {
+            int gy = y0 + i_y[i], gx = x0 + i_x[i];
+            if (p.in_clamp && l_off[i] >= 0) {
+                gy = min(max(gy, 0), p.in_hp - 1);
+                gx = min(max(gx, 0), p.in_wp - 1);
+            }
+            g_off[SET][i] = ((unsigned)gy < (unsigned)p.in_hp && (unsigned)gx < (unsigned)p.in_wp) ? (gy * p.in_wp + gx) * p.in_cp + g8 + chunk * KC : -1;
+            const float* src = in + (g_off[SET][i] >= 0 ? g_off[SET][i] : 0);
+            raw[SET][i][0] = *reinterpret_cast<const float4*>(src);
+            raw[SET][i][1] = *reinterpret_cast<const float4*>(src + 4);
+        }
+    };
+    auto store = [&](auto set_, unsigned char* buf) {
+        constexpr int SET = decltype(set_)::value;
+#pragma unroll
+        for (int i = 0; i < G::NB; i++) {
+            if (l_off[i] < 0) continue;
+            const bool ok = g_off[SET][i] >= 0;
+            const float4 r0 = raw[SET][i][0], r1 = raw[SET][i][1];
+            const float r[8] = {r0.x, r0.y, r0.z, r0.w, r1.x, r1.y, r1.z, r1.w};
+            half8_t hi, lo;
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                const float v = ok ? act_p16(r[e], p.act) * in_scale : 0.f;
+                hi[e] = (_Float16)v;
+                lo[e] = (_Float16)(v - (float)hi[e]);
+            }
+            *reinterpret_cast<half8_t*>(buf + l_off[i]) = hi;
+            *reinterpret_cast<half8_t*>(buf + G::PLANE + l_off[i]) = lo;
+        }
+    };
+    auto residual_in = [&](int tile) {   // the residual tile of a tile: [position][CPB channels] fp32
+        const float* res = reinterpret_cast<const float*>(p.res);
+        const int tyi = (int)(((float)tile + 0.5f) * p.rcp_tiles_x), txi = tile - tyi * p.tiles_x;
+        f32x4_t rv[G::RNB];
+#pragma unroll
+        for (int i = 0; i < G::RNB; i++) {
+            const int idx = stid + i * 256;
+            const int m = idx / (CPB / 4), c4 = idx % (CPB / 4);
+            const int ty = m / G::TWG, tx = m - ty * G::TWG;
+            const int py = tyi * G::TH + ty, px = txi * G::TWG + tx;
+            const bool ok = idx < G::RPIECES && py < p.npos_y && px < p.npos_x;
+            rv[i] = *reinterpret_cast<const f32x4_t*>(res + (ok ? ((size_t)(p.res_off_y + py) * p.res_wp + p.res_off_x + px) * p.res_cp + cb * CPB + c4 * 4 : 0));
+        }
+#pragma unroll
+        for (int i = 0; i < G::RNB; i++) {
+            const int idx = stid + i * 256;
+            if (idx < G::RPIECES) *reinterpret_cast<f32x4_t*>(lds + res_off + (idx / (CPB / 4)) * G::RES_PITCH + (idx % (CPB / 4)) * 16) = rv[i];
+        }
+    };
+    // the stage after (tile, c); false: there is none
+    auto advance = [&](int& tile, int& c) {
+        if (++c == nchunks) { c = 0; tile += p.pos_groups; }
+        return tile < ntiles;
+    };
+    typedef std::integral_constant<int, 0> Set0;
+    typedef std::integral_constant<int, 1> Set1;
+    
+    int tile = group, c = 0;          // the stage the MFMA waves are on (stage n)
+    int t1 = group, c1 = 0;           // stage n+1
+    fetch(Set0(), tile, 0);
+    bool have1 = advance(t1, c1);
+    int t2 = t1, c2 = c1;             // stage n+2
+    bool have2 = have1 && advance(t2, c2);
+    if (p.in_amax) in_scale = range_scale(range_after_act(range_reduce(range_bits), p.act), &inv_unused);
+    if (stid < CPB) {
+        reinterpret_cast<float*>(lds + sb_off)[stid] = p.scale[cb * CPB + stid];
+        reinterpret_cast<float*>(lds + sb_off)[CPB + stid] = p.bias[cb * CPB + stid];
+    }
+    store(Set0(), lds);
+    
+    lds_barrier();
+    if (have1) fetch(Set1(), t1, c1);   // (not before the first stage is handed over: every workgroup of the launch is fetching at that moment)
+    // One iteration per stage n of the MFMA waves: stage n+1 (fetched an iteration ago) is written to the other
+    // buffer, then stage n+2 is fetched into the registers that stage n left.  Unrolled by two: set = parity of the stage.
+    auto iteration = [&](auto next_set, auto free_set, unsigned char* next_buf) {
+        if (c + 1 == nchunks && p.res) residual_in(tile);
+        if (have1) store(next_set, next_buf);
+        if (have2) fetch(free_set, t2, c2);
+        lds_barrier();
+        const bool go_on = have1;
+        tile = t1; c = c1; t1 = t2; c1 = c2; have1 = have2;
+        if (have2) have2 = advance(t2, c2);
+        return go_on;
+    };
+    for (;;) {
+        if (!iteration(Set1(), Set0(), lds + G::BUF)) break;   // stage n even: n+1 is in set 1, goes into buffer 1
+        if (!iteration(Set0(), Set1(), lds)) break;
+    }
+}
+
 // Grid: cout_blocks x pos_groups workgroups; a workgroup keeps its block of output channels and walks the tiles
 // group, group + pos_groups, ... (one tile each when the layer has no more tiles than the chip has CUs).  The staging
 // waves run one stage ahead of the MFMA waves, across tile boundaries, so that from the second tile on a tile's fetch
@@ -177,124 +305,8 @@ __global__ __launch_bounds__(512) void conv_p16_kernel(const ConvP16Params p) {
     constexpr int sb_off = 2 * G::BUF;
     constexpr int res_off = sb_off + 2 * CPB * 4;
 
-    if (wave < 4) {
-        // ------------------------------------------------------------------ staging waves (the first four: they start first)
-        const int stid = tid & 255;
-        const float* in = reinterpret_cast<const float*>(p.in);
-        int i_y[G::NB], i_x[G::NB];   // an item's pixel inside the halo tile (rows above 2^15: no such item)
-        int l_off[G::NB];
-#pragma unroll
-        for (int i = 0; i < G::NB; i++) {
-            const int idx = stid + i * 256;
-            l_off[i] = -1; i_y[i] = 1 << 20; i_x[i] = 0;
-            if (idx < G::NITEMS) {
-                const int pix = idx >> 2, g = idx & 3;
-                const int py = pix / G::HW, px = pix - py * G::HW;
-                i_y[i] = py; i_x[i] = px;
-                l_off[i] = py * G::ROW_PITCH + ((S == 1) ? px * PITCH : ((px & 1) * G::HWH + (px >> 1)) * PITCH) + g * 16;
-            }
-        }
-        const int g8 = (stid & 3) * 8;
-        // Two sets of staging registers: the loads of stage n+2 are issued before stage n+1 is converted, so a stage's
-        // memory latency passes while the stage before it is written to LDS.
-        int g_off[2][G::NB];       // element offsets of a set's items, -1: outside the frame (reads as 0)
-        float4 raw[2][G::NB][2];
-        float in_scale = 1.f, inv_unused;
-        // (unconditional loads: items outside the tensor read its first element and are zeroed when stored)
-        auto fetch = [&](auto set_, int tile, int chunk) {
-            constexpr int SET = decltype(set_)::value;
-            const int tyi = (int)(((float)tile + 0.5f) * p.rcp_tiles_x), txi = tile - tyi * p.tiles_x;
-            const int y0 = tyi * TH * S + p.in_y0, x0 = txi * G::TWG * S + p.in_x0;
-#pragma unroll
-            for (int i = 0; i < G::NB; i++) {
-                int gy = y0 + i_y[i], gx = x0 + i_x[i];
-                if (p.in_clamp && l_off[i] >= 0) {
-                    gy = min(max(gy, 0), p.in_hp - 1);
-                    gx = min(max(gx, 0), p.in_wp - 1);
-                }
-                g_off[SET][i] = ((unsigned)gy < (unsigned)p.in_hp && (unsigned)gx < (unsigned)p.in_wp) ? (gy * p.in_wp + gx) * p.in_cp + g8 + chunk * KC : -1;
-                const float* src = in + (g_off[SET][i] >= 0 ? g_off[SET][i] : 0);
-                raw[SET][i][0] = *reinterpret_cast<const float4*>(src);
-                raw[SET][i][1] = *reinterpret_cast<const float4*>(src + 4);
-            }
-        };
-        auto store = [&](auto set_, unsigned char* buf) {
-            constexpr int SET = decltype(set_)::value;
-#pragma unroll
-            for (int i = 0; i < G::NB; i++) {
-                if (l_off[i] < 0) continue;
-                const bool ok = g_off[SET][i] >= 0;
-                const float4 r0 = raw[SET][i][0], r1 = raw[SET][i][1];
-                const float r[8] = {r0.x, r0.y, r0.z, r0.w, r1.x, r1.y, r1.z, r1.w};
-                half8_t hi, lo;
-#pragma unroll
-                for (int e = 0; e < 8; e++) {
-                    const float v = ok ? act_p16(r[e], p.act) * in_scale : 0.f;
-                    hi[e] = (_Float16)v;
-                    lo[e] = (_Float16)(v - (float)hi[e]);
-                }
-                *reinterpret_cast<half8_t*>(buf + l_off[i]) = hi;
-                *reinterpret_cast<half8_t*>(buf + G::PLANE + l_off[i]) = lo;
-            }
-        };
-        auto residual_in = [&](int tile) {   // the residual tile of a tile: [position][CPB channels] fp32
-            const float* res = reinterpret_cast<const float*>(p.res);
-            const int tyi = (int)(((float)tile + 0.5f) * p.rcp_tiles_x), txi = tile - tyi * p.tiles_x;
-            f32x4_t rv[G::RNB];
-#pragma unroll
-            for (int i = 0; i < G::RNB; i++) {
-                const int idx = stid + i * 256;
-                const int m = idx / (CPB / 4), c4 = idx % (CPB / 4);
-                const int ty = m / G::TWG, tx = m - ty * G::TWG;
-                const int py = tyi * TH + ty, px = txi * G::TWG + tx;
-                const bool ok = idx < G::RPIECES && py < p.npos_y && px < p.npos_x;
-                rv[i] = *reinterpret_cast<const f32x4_t*>(res + (ok ? ((size_t)(p.res_off_y + py) * p.res_wp + p.res_off_x + px) * p.res_cp + cb * CPB + c4 * 4 : 0));
-            }
-#pragma unroll
-            for (int i = 0; i < G::RNB; i++) {
-                const int idx = stid + i * 256;
-                if (idx < G::RPIECES) *reinterpret_cast<f32x4_t*>(lds + res_off + (idx / (CPB / 4)) * G::RES_PITCH + (idx % (CPB / 4)) * 16) = rv[i];
-            }
-        };
-        // the stage after (tile, c); false: there is none
-        auto advance = [&](int& tile, int& c) {
-            if (++c == nchunks) { c = 0; tile += p.pos_groups; }
-            return tile < ntiles;
-        };
-        typedef std::integral_constant<int, 0> Set0;
-        typedef std::integral_constant<int, 1> Set1;
-        FYN_PTRACE(0);
-        int tile = group, c = 0;          // the stage the MFMA waves are on (stage n)
-        int t1 = group, c1 = 0;           // stage n+1
-        fetch(Set0(), tile, 0);
-        bool have1 = advance(t1, c1);
-        int t2 = t1, c2 = c1;             // stage n+2
-        bool have2 = have1 && advance(t2, c2);
-        if (p.in_amax) in_scale = range_scale(range_after_act(range_reduce(range_bits), p.act), &inv_unused);
-        if (stid < CPB) {
-            reinterpret_cast<float*>(lds + sb_off)[stid] = p.scale[cb * CPB + stid];
-            reinterpret_cast<float*>(lds + sb_off)[CPB + stid] = p.bias[cb * CPB + stid];
-        }
-        store(Set0(), lds);
-        FYN_PTRACE(1);
-        lds_barrier();
-        if (have1) fetch(Set1(), t1, c1);   // (not before the first stage is handed over: every workgroup of the launch is fetching at that moment)
-        // One iteration per stage n of the MFMA waves: stage n+1 (fetched an iteration ago) is written to the other
-        // buffer, then stage n+2 is fetched into the registers that stage n left.  Unrolled by two: set = parity of the stage.
-        auto iteration = [&](auto next_set, auto free_set, unsigned char* next_buf) {
-            if (c + 1 == nchunks && p.res) residual_in(tile);
-            if (have1) store(next_set, next_buf);
-            if (have2) fetch(free_set, t2, c2);
-            lds_barrier();
-            const bool go_on = have1;
-            tile = t1; c = c1; t1 = t2; c1 = c2; have1 = have2;
-            if (have2) have2 = advance(t2, c2);
-            return go_on;
-        };
-        for (;;) {
-            if (!iteration(Set1(), Set0(), lds + G::BUF)) break;   // stage n even: n+1 is in set 1, goes into buffer 1
-            if (!iteration(Set0(), Set1(), lds)) break;
-        }
+    if (wave < 4) {   // the first four waves stage: they start first
+        p16_stager<G>(p, lds, tid & 255, cb, group, ntiles, nchunks, range_bits);
         return;
     }
 
@@ -415,6 +427,178 @@ __global__ __launch_bounds__(512) void conv_p16_kernel(const ConvP16Params p) {
     FYN_PTRACE(31);
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// Transposed 3x3 convolution that up-samples by two, cropped to exactly twice the input size (replaces the stencil
+// passes of DeepTransConvLayerBase::forward, gpu/deep/deeptransconvlayerbase.cpp:83-130, for such layers):
+//     out[2a+py, 2b+px] = sum over dy, dx of W[py+2dy, px+2dx] * in[a-dy, b-dx],   py+2dy <= 2, px+2dx <= 2.
+// Positions are input pixels; every tap (ky, kx) feeds the accumulators of exactly one output parity (ky&1, kx&1) and
+// reads the input shifted by (ky>>1, kx>>1), so a chunk is nine steps as in a 3x3 convolution, with four accumulator
+// sets and four distinct B fragments per position fragment (two register sets: the next shift's fragments are read
+// while the current shift's taps run).  Taps in the order of their shift:
+constexpr int TT_KY[NT] = {0, 0, 1, 1, 0, 1, 2, 2, 2};
+constexpr int TT_KX[NT] = {0, 1, 0, 1, 2, 2, 0, 1, 2};
+constexpr int tt_shift(int t) { return (TT_KY[t] >> 1) * 2 + (TT_KX[t] >> 1); }
+constexpr int tt_parity(int t) { return (TT_KY[t] & 1) * 2 + (TT_KX[t] & 1); }
+constexpr bool tt_last_of_shift(int t) { return t == NT - 1 || tt_shift(t + 1) != tt_shift(t); }
+
+template <class G, int BUFI>
+__device__ __forceinline__ void tp16_stage(f32x4_t (&acc)[4][2][G::FN], half8_t (&a_q)[PD][2][2], half8_t (&b)[2][G::FN][2],
+                                           const int (&bbase)[2][G::FN], const unsigned char* lds, const unsigned char*& wnext,
+                                           const unsigned char* wbase, const unsigned char* wend, unsigned wstep) {
+    constexpr int FN = G::FN;
+#pragma unroll
+    for (int t = 0; t < NT; t++) {
+        const int d = (BUFI * NT + t) % PD, dprev = (d + PD - 1) % PD;
+        const int sh = tt_shift(t), set = sh & 1, par = tt_parity(t);
+        const int nsh = (sh + 1) & 3, nbuf = (t == NT - 1) ? 1 - BUFI : BUFI;
+        // the tile is staged with one pixel of halo above and to the left: shift (dy, dx) reads pixel (1-dy, 1-dx) + position
+        const int noff = (1 - (nsh >> 1)) * G::ROW_PITCH + (1 - (nsh & 1)) * PITCH;
+        const int first_read = (t == NT - 1) ? 4 : 0;   // (the stage's barrier sits in slot 3 of its last step)
+        const unsigned char* w_ = wnext;
+        wnext += wstep;
+        if (wnext == wend) wnext = wbase;
+#pragma unroll
+        for (int i = 0; i < 6 * FN; i++) {
+            const int fn = i / 6, r = i % 6, kind = r / 2, fm = r % 2;
+            const int apl = (kind == 1) ? 1 : 0, bpl = (kind == 2) ? 1 : 0;
+            acc[par][fm][fn] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_q[d][fm][apl], b[set][fn][bpl], acc[par][fm][fn], 0, 0, 0);
+            if (t == NT - 1 && i == 3) lds_barrier();
+            if (tt_last_of_shift(t) && i >= first_read && i < first_read + 2 * FN) {
+                const int j = i - first_read;
+                b[1 - set][j / 2][j % 2] = *reinterpret_cast<const half8_t*>(lds + bbase[nbuf][j / 2] + noff + (j % 2) * G::PLANE);
+            }
+#pragma unroll
+            for (int j = 0; j < 4; j++)   // the four weight fragments of a step, spread over its slots
+                if (i == (j * 6 * FN) / 4 + 1) a_q[dprev][j % 2][j / 2] = *reinterpret_cast<const half8_t*>(w_ + ((j % 2) * 2 + j / 2) * 1024);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+}
+
+template <int TH, int TW, int WM>
+__global__ __launch_bounds__(512) void tconv_p16_kernel(const ConvP16Params p) {
+    using G = Geo<TH, TW, 1, WM, 1>;
+    constexpr int FN = G::FN, CPB = G::CPB;
+    static_assert(6 * FN >= 4 + 2 * FN, "the last step of a stage has room for the next stage's first fragments");
+    extern __shared__ __align__(16) unsigned char lds[];
+    __shared__ unsigned range_box[2];
+    if (blockIdx.x == 0) range_clear(p.reset[0], p.reset[1], p.reset[2], p.reset[3], p.nreset);
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    int bid = blockIdx.x;
+    {
+        const int nblk = p.pos_groups * p.cout_blocks;
+        const int per = nblk >> 3;
+        if (bid < (per << 3)) bid = (bid & 7) * per + (bid >> 3);
+    }
+    const int cb = bid % p.cout_blocks;
+    const int group = bid / p.cout_blocks;
+    const int ntiles = p.tiles_x * p.tiles_y;
+    if (tid < 2) range_box[tid] = 0u;
+    const unsigned range_bits = p.in_amax ? range_load(p.in_amax) : 0u;
+    const int nchunks = p.cin_chunks;
+    constexpr int sb_off = 2 * G::BUF;
+    if (wave < 4) {
+        p16_stager<G>(p, lds, tid & 255, cb, group, ntiles, nchunks, range_bits);
+        return;
+    }
+    const int mq = lane & 15, kq = lane >> 4;
+    const int mw = (wave - 4) % WM, wn = (wave - 4) / WM;
+    int bbase[2][FN];
+#pragma unroll
+    for (int fn = 0; fn < FN; fn++) {
+        const int m = fn * 16 + mq;
+        const int ty = m / TW, tx = m - ty * TW;
+        bbase[0][fn] = ty * G::ROW_PITCH + (wn * TW + tx) * PITCH + kq * 16;
+        bbase[1][fn] = bbase[0][fn] + G::BUF;
+    }
+    const unsigned wstep = (unsigned)p.mfrags * 2 * 1024;
+    const unsigned char* wbase = reinterpret_cast<const unsigned char*>(p.wpack) + (size_t)((cb * 2 * WM + mw * 2) * 2) * 1024 + lane * 16;
+    const unsigned char* wend = wbase + (size_t)nchunks * NT * wstep;
+    half8_t a_q[PD][2][2];
+#pragma unroll
+    for (int d = 0; d < PD; d++)
+#pragma unroll
+        for (int fm = 0; fm < 2; fm++)
+#pragma unroll
+            for (int pl = 0; pl < 2; pl++) a_q[d][fm][pl] = *reinterpret_cast<const half8_t*>(wbase + (size_t)d * wstep + (fm * 2 + pl) * 1024);
+    f32x4_t acc[4][2][FN];
+    auto zero_acc = [&]() {
+#pragma unroll
+        for (int par = 0; par < 4; par++)
+#pragma unroll
+            for (int fm = 0; fm < 2; fm++)
+#pragma unroll
+                for (int fn = 0; fn < FN; fn++) acc[par][fm][fn] = (f32x4_t)(0.f);
+    };
+    zero_acc();
+    float inv_in_scale = 1.f;
+    if (p.in_amax) (void)range_scale(range_after_act(range_reduce(range_bits), p.act), &inv_in_scale);
+    const float acc_mul = p.acc_mul * inv_in_scale;
+    float* out = reinterpret_cast<float*>(p.out);
+    float vmax = 0.f;
+    auto finish_tile = [&](int tile) {
+        const int tyi = (int)(((float)tile + 0.5f) * p.rcp_tiles_x), txi = tile - tyi * p.tiles_x;
+        const float* sb = reinterpret_cast<const float*>(lds + sb_off);
+        f32x4_t bi[2], scm[2];
+#pragma unroll
+        for (int fm = 0; fm < 2; fm++) {
+            scm[fm] = *reinterpret_cast<const f32x4_t*>(sb + mw * 32 + fm * 16 + kq * 4) * acc_mul;
+            bi[fm] = *reinterpret_cast<const f32x4_t*>(sb + CPB + mw * 32 + fm * 16 + kq * 4);
+        }
+#pragma unroll
+        for (int fn = 0; fn < FN; fn++) {
+            const int m = fn * 16 + mq;
+            const int ty = m / TW, tx = wn * TW + (m - ty * TW);
+            const int a = tyi * TH + ty, bx = txi * G::TWG + tx;
+            const bool ok = a < p.npos_y && bx < p.npos_x;
+            const size_t obase = ((size_t)(p.out_off_y + 2 * a) * p.out_wp + p.out_off_x + 2 * bx) * p.out_cp + cb * CPB + mw * 32 + kq * 4;
+            float fmax_ = 0.f;
+#pragma unroll
+            for (int par = 0; par < 4; par++) {
+                const size_t o = obase + ((size_t)(par >> 1) * p.out_wp + (par & 1)) * p.out_cp;
+#pragma unroll
+                for (int fm = 0; fm < 2; fm++) {
+                    f32x4_t v;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        v[e] = acc[par][fm][fn][e] * scm[fm][e] + bi[fm][e];
+                        fmax_ = fmaxf(fmax_, fabsf(v[e]));
+                    }
+                    if (ok) *reinterpret_cast<f32x4_t*>(out + o + fm * 16) = v;
+                }
+            }
+            vmax = fmaxf(vmax, ok ? fmax_ : 0.f);
+        }
+    };
+    lds_barrier();   // the first stage is staged
+    half8_t b[2][FN][2];
+#pragma unroll
+    for (int fn = 0; fn < FN; fn++)
+#pragma unroll
+        for (int pl = 0; pl < 2; pl++) b[0][fn][pl] = *reinterpret_cast<const half8_t*>(lds + bbase[0][fn] + G::ROW_PITCH + PITCH + pl * G::PLANE);
+    const unsigned char* wnext = wbase + (size_t)((PD - 1) % (nchunks * NT)) * wstep;
+    int tile = group, c = 0;
+    for (;;) {
+        tp16_stage<G, 0>(acc, a_q, b, bbase, lds, wnext, wbase, wend, wstep);
+        if (++c == nchunks) {
+            finish_tile(tile);
+            c = 0; tile += p.pos_groups;
+            if (tile >= ntiles) break;
+            zero_acc();
+        }
+        tp16_stage<G, 1>(acc, a_q, b, bbase, lds, wnext, wbase, wend, wstep);
+        if (++c == nchunks) {
+            finish_tile(tile);
+            c = 0; tile += p.pos_groups;
+            if (tile >= ntiles) break;
+            zero_acc();
+        }
+    }
+    if (p.out_amax) range_publish_waves(p.out_amax, vmax, range_box, 4);
+}
+
 typedef void (*p16_fn)(const ConvP16Params);
 struct P16Entry {
     int th, tw, stride, wm;
@@ -434,6 +618,19 @@ const P16Entry kEntries[] = {
 size_t entry_lds(const P16Entry& e, bool residual) {
     return 2 * e.buf + 2 * (size_t)(32 * e.wm) * 4 + (residual ? e.res_bytes : 0);
 }
+struct TP16Entry {
+    int th, tw, wm;
+    p16_fn fn;
+    size_t buf;
+};
+template <int TH, int TW, int WM>
+constexpr TP16Entry tentry() {
+    return TP16Entry{TH, TW, WM, tconv_p16_kernel<TH, TW, WM>, (size_t)Geo<TH, TW, 1, WM, 1>::BUF};
+}
+const TP16Entry kTEntries[] = {
+    tentry<4, 8, 1>(), tentry<8, 4, 1>(), tentry<2, 8, 1>(),
+    tentry<4, 8, 2>(), tentry<8, 4, 2>(), tentry<2, 8, 2>(),
+};
 }  // namespace
 
 int conv_p16_tile_count() { return (int)(sizeof(kEntries) / sizeof(kEntries[0])); }
@@ -490,6 +687,41 @@ int launch_conv_p16(const ConvP16Params& p, hipStream_t s) {
         return hipGetLastError() == hipSuccess ? 0 : -3;
     }
 #endif
+    hipLaunchKernelGGL(e->fn, dim3(p.pos_groups * p.cout_blocks), dim3(512), lds_bytes, s, p);
+    return hipGetLastError() == hipSuccess ? 0 : -3;
+}
+
+int tconv_p16_tile_count() { return (int)(sizeof(kTEntries) / sizeof(kTEntries[0])); }
+void tconv_p16_tile(int index, int* th, int* tw, int* wm) {
+    *th = kTEntries[index].th; *tw = kTEntries[index].tw; *wm = kTEntries[index].wm;
+}
+static const TP16Entry* find_tentry(const ConvP16Params& p) {
+    for (const TP16Entry& c : kTEntries)
+        if (c.th == p.tile_h && c.tw == p.tile_w && c.wm == p.wm) return &c;
+    return nullptr;
+}
+void tconv_p16_tap(int t, int* ky, int* kx) { *ky = TT_KY[t]; *kx = TT_KX[t]; }
+size_t tconv_p16_lds_bytes(const ConvP16Params& p) {
+    const TP16Entry* e = find_tentry(p);
+    return e ? 2 * e->buf + 2 * (size_t)(32 * e->wm) * 4 : 0;
+}
+bool tconv_p16_supported(int k, int crop, int in_cp, int in_pad, int cout, int out_cp, bool f16) {
+    return k == 3 && crop == 1 && !f16 && in_cp % KC == 0 && in_pad >= 1 && cout % 32 == 0 && out_cp % 4 == 0 && out_cp >= cout;
+}
+
+// npos_y x npos_x: the input size (positions are input pixels); out_off_*: stored coordinate of output pixel (0, 0)
+int launch_tconv_p16(const ConvP16Params& p, hipStream_t s) {
+    const TP16Entry* e = find_tentry(p);
+    if (!e) return -1;
+    const int cpb = 32 * e->wm, twg = (4 / e->wm) * e->tw;
+    if (p.cin_chunks < 1 || p.in_cp != p.cin_chunks * KC || p.cout_blocks < 1 || p.mfrags < p.cout_blocks * 2 * e->wm ||
+        p.tiles_x * twg < p.npos_x || p.tiles_y * p.tile_h < p.npos_y || p.out_cp < p.cout_blocks * cpb || p.res || p.stride != 1 ||
+        p.nreset < 0 || p.nreset > 4 || p.pos_groups < 1 || p.pos_groups > p.tiles_x * p.tiles_y ||
+        p.rcp_tiles_x != 1.0f / (float)p.tiles_x || p.tiles_x * p.tiles_y > 4000000)
+        return -5;
+    const size_t lds_bytes = tconv_p16_lds_bytes(p);
+    if (lds_bytes > 160 * 1024) return -2;
+    if (ensure_lds(reinterpret_cast<const void*>(e->fn), lds_bytes) != 0) return -2;
     hipLaunchKernelGGL(e->fn, dim3(p.pos_groups * p.cout_blocks), dim3(512), lds_bytes, s, p);
     return hipGetLastError() == hipSuccess ? 0 : -3;
 }

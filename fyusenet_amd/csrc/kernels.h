@@ -204,6 +204,15 @@ int conv_p16_tile_count();
 void conv_p16_tile(int index, int* th, int* tw, int* stride, int* wm);
 size_t conv_p16_lds_bytes(const ConvP16Params& p);   // 0: no such compiled combination
 int launch_conv_p16(const ConvP16Params& p, hipStream_t s);
+// the transposed 3x3 convolution that doubles the image size, on the same parameters: positions (npos_y x npos_x,
+// tiles) are input pixels, out_off_* the stored coordinate of output pixel (0, 0), wpack holds the nine taps of a chunk
+// in the order of their input shift (conv_p16.hip: TT_KY / TT_KX)
+bool tconv_p16_supported(int k, int crop, int in_cp, int in_pad, int cout, int out_cp, bool f16);
+int tconv_p16_tile_count();
+void tconv_p16_tile(int index, int* th, int* tw, int* wm);
+void tconv_p16_tap(int t, int* ky, int* kx);   // kernel tap of step t of a chunk
+size_t tconv_p16_lds_bytes(const ConvP16Params& p);
+int launch_tconv_p16(const ConvP16Params& p, hipStream_t s);
 
 // ---------------------------------------------------------------------------------------------
 // Direct (non-MFMA) layer kernels (layers_direct.hip)

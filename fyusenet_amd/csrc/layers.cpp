@@ -1424,9 +1424,115 @@ class TransConvLayer : public Layer {
                 subconvs.push_back(sc);
             }
         group = tune_mfma_group(net, subconvs, in_v, out_v, d.in_channels, oc, act(), scale_dev, bias_dev);
+        if (tconv_p16_supported(k, crop, in_v.cp, in_v.pad, oc, out_v.cp, out_v.f16 != 0) && d.in_channels == in_v.cp && !getenv("FYNHIP_NO_P16_CONV"))
+            setup_p16(in_v, out_v);
         set_up = true;
         setup_ranges();
         if (!block.empty()) pack();
+    }
+    // 16-position-fragment form (conv_p16.hip): all four output parities from one staged input tile; the compiled
+    // combinations that fit are timed and the best is kept if it beats the grouped launch of the general kernel
+    void setup_p16(const TView& in_v, const TView& out_v) {
+        ConvP16Params q{};
+        q.in = in_v.ptr; q.out = out_v.ptr; q.res = nullptr;
+        q.in_hp = in_v.hp(); q.in_wp = in_v.wp(); q.in_cp = in_v.cp;
+        q.stride = 1;
+        q.in_y0 = q.in_x0 = in_v.pad - 1;
+        q.npos_y = d.height; q.npos_x = d.width;
+        q.out_wp = out_v.wp(); q.out_cp = out_v.cp; q.out_off_y = q.out_off_x = out_v.pad;
+        q.cin_chunks = in_v.cp / 32;
+        q.mfrags = oc / 16;
+        q.scale = scale_dev; q.bias = bias_dev;
+        q.acc_mul = 1.f;
+        q.act = act();
+        int want_h = 0, want_w = 0, want_wm = 0;   // FYNHIP_P16_TILE=h,w[,wm] (tests): that combination
+        if (const char* e = getenv("FYNHIP_P16_TILE")) sscanf(e, "%d,%d,%d", &want_h, &want_w, &want_wm);
+        std::vector<ConvP16Params> cands;
+        for (int i = 0; i < tconv_p16_tile_count(); i++) {
+            int th, tw, wm;
+            tconv_p16_tile(i, &th, &tw, &wm);
+            if (oc % (32 * wm) != 0) continue;
+            if (want_h && (th != want_h || tw != want_w || (want_wm && wm != want_wm))) continue;
+            ConvP16Params c = q;
+            c.tile_h = th; c.tile_w = tw; c.wm = wm;
+            const int twg = (4 / wm) * tw;
+            c.tiles_x = (d.width + twg - 1) / twg; c.tiles_y = (d.height + th - 1) / th;
+            c.rcp_tiles_x = 1.0f / (float)c.tiles_x;
+            c.cout_blocks = oc / (32 * wm);
+            c.pos_groups = std::max(1, std::min(c.tiles_x * c.tiles_y, 256 / c.cout_blocks));
+            const size_t lds = tconv_p16_lds_bytes(c);
+            if (lds == 0 || lds > 160 * 1024) continue;
+            cands.push_back(c);
+        }
+        if (cands.empty()) return;
+        const size_t halves = ((size_t)q.cin_chunks * 9 + 8) * q.mfrags * 2 * 64 * 8;
+        p16_wpack_dev = net->dev_alloc(halves * 2, true);
+        for (ConvP16Params& c : cands) c.wpack = p16_wpack_dev;
+        const bool always = getenv("FYNHIP_FORCE_P16_CONV") != nullptr;
+        const char* at = getenv("FYNHIP_AUTOTUNE");
+        int pick = 0;
+        char key[160];
+        snprintf(key, sizeof(key), "tp16:%dx%d:%dx%d:cp%d", d.in_channels, oc, d.height, d.width, in_v.cp);
+        int cached[3] = {0, 0, 0};
+        if (!want_h && tune_cache_triple(key, cached)) {
+            pick = -1;
+            if (cached[0] || always)
+                for (size_t i = 0; i < cands.size(); i++)
+                    if (cands[i].tile_h * 1000 + cands[i].tile_w == cached[1] && cands[i].wm == cached[2]) pick = (int)i;
+            if (always && pick < 0) pick = 0;
+        } else if (!(at && at[0] == '0')) {
+            float best = 1e30f, t_other = 1e30f;
+            for (int rep = 0; rep < 3; rep++) {
+                for (size_t i = 0; i < cands.size(); i++) {
+                    const float t = time_calls(net, [&]() {
+                        if (launch_tconv_p16(cands[i], net->stream) != 0) fail(FYN_ERR_DEVICE, "16-position transposed convolution launch failed while tuning");
+                    }, 10);
+                    if (t < best) { best = t; pick = (int)i; }
+                }
+                t_other = std::min(t_other, time_group(net, group, 10));
+            }
+            if (getenv("FYNHIP_TUNE_VERBOSE"))
+                fprintf(stderr, "[tune] transposed 3x3: 16-position fragments (%dx%d tiles, %d channel groups) %.1f us, general kernel %.1f us\n",
+                        cands[pick].tile_h, cands[pick].tile_w, cands[pick].wm, best * 1e3f, t_other * 1e3f);
+            const bool win = best < t_other;
+            if (!want_h) tune_cache_store_triple(key, win ? 1 : 0, cands[pick].tile_h * 1000 + cands[pick].tile_w, cands[pick].wm);
+            if (!win && !always) pick = -1;
+        }
+        if (pick >= 0) {
+            p16 = true;
+            pp = cands[pick];
+        } else {
+            net->dev_free(p16_wpack_dev);
+            p16_wpack_dev = nullptr;
+        }
+    }
+    // weights of that form: [(chunk*9 + step)][cout fragment of 16][plane][lane][8 halves], steps in the kernel's tap order
+    void pack_p16(const float* w, float wmul) {
+        const int cin = d.in_channels;
+        std::vector<uint16_t> pack(((size_t)pp.cin_chunks * 9 + 8) * pp.mfrags * 2 * 64 * 8, 0);
+        for (int chunk = 0; chunk < pp.cin_chunks; chunk++)
+            for (int t = 0; t < 9; t++) {
+                int ky, kx;
+                tconv_p16_tap(t, &ky, &kx);
+                for (int mf = 0; mf < pp.mfrags; mf++) {
+                    uint16_t* base = pack.data() + (((size_t)(chunk * 9 + t) * pp.mfrags + mf) * 2) * 64 * 8;
+                    for (int lane = 0; lane < 64; lane++) {
+                        const int o = mf * 16 + (lane & 15);
+                        if (o >= oc) continue;
+                        for (int j = 0; j < 8; j++) {
+                            const int ci = chunk * 32 + 8 * (lane >> 4) + j;
+                            if (ci >= cin) continue;
+                            const float v = w[(((size_t)o * 3 + ky) * 3 + kx) * cin + ci] * wmul;
+                            const uint16_t hi = f2h_bits(v);
+                            base[(size_t)lane * 8 + j] = hi;
+                            base[(size_t)(64 + lane) * 8 + j] = f2h_bits(v - h2f(hi));
+                        }
+                    }
+                }
+            }
+        FYN_HIP(hipStreamSynchronize(net->stream));
+        FYN_HIP(hipMemcpyAsync(p16_wpack_dev, pack.data(), pack.size() * 2, hipMemcpyHostToDevice, net->stream));
+        FYN_HIP(hipStreamSynchronize(net->stream));
     }
     // value ranges (range.h): every parity reads the input's word and raises the output's; the first one clears
     bool tracks_range() const override { return true; }
@@ -1436,8 +1542,15 @@ class TransConvLayer : public Layer {
             L.p.out_amax = tout().amax;
         }
         group.sync();
+        pp.in_amax = tin(0).amax;
+        pp.out_amax = tout().amax;
     }
     bool add_range_reset(unsigned* w) override {
+        if (p16) {
+            if (!set_up || pp.nreset >= 4) return false;
+            pp.reset[pp.nreset++] = w;
+            return true;
+        }
         if (!set_up || group.subs.empty() || group.subs[0].p.nreset >= 4) return false;
         group.subs[0].p.reset[group.subs[0].p.nreset++] = w;
         group.sync();
@@ -1452,6 +1565,12 @@ class TransConvLayer : public Layer {
         reupload(net, scale_dev, sc);
         reupload(net, bias_dev, bi);
         const float wmul = weight_prescale(w, (size_t)oc * k * k * d.in_channels);
+        if (p16) {
+            pp.acc_mul = 1.0f / wmul;
+            pack_p16(w, wmul);
+            have_weights = true;
+            return;
+        }
         for (auto& L : group.subs) {
             L.p.acc_mul = 1.0f / wmul;
             pack_mfma_weights(net, L, w, k, wmul);
@@ -1461,9 +1580,20 @@ class TransConvLayer : public Layer {
     }
     void forward(hipStream_t s) override {
         if (!have_weights) fail(FYN_ERR_STATE, "layer %s (%d): forward() without weights", d.name, d.number);
+        if (p16) {
+            if (launch_tconv_p16(pp, s) != 0) fail(FYN_ERR_DEVICE, "layer %s: transposed convolution launch failed", d.name);
+            return;
+        }
         if (run_group(group, s) != 0) fail(FYN_ERR_DEVICE, "layer %s: transposed convolution launch failed", d.name);
     }
     std::string info() const override {
+        if (p16) {
+            char buf[220];
+            snprintf(buf, sizeof(buf), "transconv, tconv_p16 f16x2-split 4 parities per tile, tile=%dx%d(cout x input pos) waves=%dx%d th=%d tw=%d blocks=%d tiles=%d lds=%zu steps=9 chunks=%d",
+                     32 * pp.wm, pp.tile_h * pp.tile_w * (4 / pp.wm), pp.wm, 4 / pp.wm, pp.tile_h, pp.tile_w, pp.pos_groups * pp.cout_blocks,
+                     pp.tiles_x * pp.tiles_y * pp.cout_blocks, tconv_p16_lds_bytes(pp), pp.cin_chunks);
+            return buf;
+        }
         return group.subs.empty() ? "transconv" : "transconv, " + std::to_string(group.subs.size()) + " parities in one launch: " + mfma_info(group.subs[0]);
     }
     int k, crop;
@@ -1472,6 +1602,9 @@ class TransConvLayer : public Layer {
     std::vector<float> block;
     std::vector<SubConv> subconvs;
     MfmaGroup group;
+    bool p16 = false;             // 16-position-fragment form (conv_p16.hip)
+    ConvP16Params pp{};
+    void* p16_wpack_dev = nullptr;
     float *scale_dev = nullptr, *bias_dev = nullptr;
 };
 

@@ -396,6 +396,48 @@ def test_transconv_parity(k, crop, cin, cout, h, w, storage):
     assert err <= TOL[storage]
 
 
+TP16_CASES = [
+    # cin, cout, h, w, tile "h,w,channel groups", batch-norm
+    (64, 32, 20, 26, "4,8,1", True),        # four tiles of positions side by side, ragged on both sides
+    (128, 64, 39, 32, "4,8,2", False),      # the style net's first up-sampling layer, reduced
+    (32, 32, 9, 70, "8,4,1", True),         # a single chunk
+    (96, 64, 33, 17, "8,4,2", False),       # three chunks
+    (64, 96, 7, 11, "2,8,1", True),         # three blocks of output channels
+    (64, 128, 21, 40, "2,8,2", False),
+    (64, 32, 80, 150, "4,8,1", True),       # 375 tiles: workgroups walk
+    (64, 32, 31, 45, None, False),          # the engine's own choice
+]
+
+
+@pytest.mark.parametrize("act", [A.RELU, A.NONE], ids=["relu", "none"])
+@pytest.mark.parametrize("case", TP16_CASES, ids=lambda c: "%dx%dx%d_to%d_%s" % (c[0], c[2], c[3], c[1], (c[4] or "auto").replace(",", "x")))
+def test_transconv_sixteen_position_fragment_form(case, act, monkeypatch):
+    """The doubling transposed 3x3 convolution on 16-position fragments (fp32 storage): all four output parities from
+    one staged input tile."""
+    cin, cout, h, w, tile, bn = case
+    if act is A.NONE and (tile is None or h > 60):
+        pytest.skip("the activation is varied on the small cases")
+    monkeypatch.setenv("FYNHIP_FORCE_P16_CONV", "1")
+    if tile:
+        monkeypatch.setenv("FYNHIP_P16_TILE", tile)
+    b = fa.ConvLayerBuilder(3, "tconv").type(fa.LayerType.TRANSCONVOLUTION2D).number(1).shape(cout, h, w, cin)
+    b.upsample(2).inputPadding(1).outputPadding(2).prefixAct(act).deep().crop(1)
+    if bn:
+        b.postfixNorm(fa.NormType.BATCHNORM)
+    wts = conv_block(1100 + cin, cout, 3, cin, bn=bn)
+    x = prng.uniform(57 * cin + w, (cin, h, w), -1, 1)
+    got, info = run_single(b, fa.STORAGE_F32, [x], wts)
+    ref = oracle_single(b, fa.STORAGE_F32, [x], wts)
+    err = rel_l2(got, ref)
+    print("  ", info, "rel_l2=%.3e" % err, flush=True)
+    assert "tconv_p16" in info
+    if tile:
+        th, tw, wm = tile.split(",")
+        assert "waves=%sx" % wm in info and "th=%s tw=%s" % (th, tw) in info
+    assert got.shape == ref.shape == (cout, 2 * h, 2 * w)
+    assert err <= TOL[fa.STORAGE_F32], info
+
+
 FRAC_CASES = [
     # k, cin, cout, h, w, step, stride, pad_in, act, kwargs
     (3, 40, 20, 12, 16, 0.5, 2, 0, A.NONE, {}),                   # deconv1 of the reference's style nets (stylenet3x3.cpp:163)
