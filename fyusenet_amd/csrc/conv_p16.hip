@@ -441,14 +441,16 @@ constexpr int tt_shift(int t) { return (TT_KY[t] >> 1) * 2 + (TT_KX[t] >> 1); }
 constexpr int tt_parity(int t) { return (TT_KY[t] & 1) * 2 + (TT_KX[t] & 1); }
 constexpr bool tt_last_of_shift(int t) { return t == NT - 1 || tt_shift(t + 1) != tt_shift(t); }
 
-template <class G, int BUFI>
-__device__ __forceinline__ void tp16_stage(f32x4_t (&acc)[4][2][G::FN], half8_t (&a_q)[PD][2][2], half8_t (&b)[2][G::FN][2],
+// (PDT: depth of the weight ring; three position fragments per wave leave room for three steps only, which at 288 cycles
+// per step still covers an L2 round trip)
+template <class G, int BUFI, int PDT>
+__device__ __forceinline__ void tp16_stage(f32x4_t (&acc)[4][2][G::FN], half8_t (&a_q)[PDT][2][2], half8_t (&b)[2][G::FN][2],
                                            const int (&bbase)[2][G::FN], const unsigned char* lds, const unsigned char*& wnext,
                                            const unsigned char* wbase, const unsigned char* wend, unsigned wstep) {
     constexpr int FN = G::FN;
 #pragma unroll
     for (int t = 0; t < NT; t++) {
-        const int d = (BUFI * NT + t) % PD, dprev = (d + PD - 1) % PD;
+        const int d = (BUFI * NT + t) % PDT, dprev = (d + PDT - 1) % PDT;
         const int sh = tt_shift(t), set = sh & 1, par = tt_parity(t);
         const int nsh = (sh + 1) & 3, nbuf = (t == NT - 1) ? 1 - BUFI : BUFI;
         // the tile is staged with one pixel of halo above and to the left: shift (dy, dx) reads pixel (1-dy, 1-dx) + position
@@ -479,6 +481,8 @@ template <int TH, int TW, int WM>
 __global__ __launch_bounds__(512) void tconv_p16_kernel(const ConvP16Params p) {
     using G = Geo<TH, TW, 1, WM, 1>;
     constexpr int FN = G::FN, CPB = G::CPB;
+    constexpr int PDT = (FN >= 3) ? 3 : 6;
+    static_assert((2 * NT) % PDT == 0, "two stages are whole turns of the weight ring");
     static_assert(6 * FN >= 4 + 2 * FN, "the last step of a stage has room for the next stage's first fragments");
     extern __shared__ __align__(16) unsigned char lds[];
     __shared__ unsigned range_box[2];
@@ -516,9 +520,9 @@ __global__ __launch_bounds__(512) void tconv_p16_kernel(const ConvP16Params p) {
     const unsigned wstep = (unsigned)p.mfrags * 2 * 1024;
     const unsigned char* wbase = reinterpret_cast<const unsigned char*>(p.wpack) + (size_t)((cb * 2 * WM + mw * 2) * 2) * 1024 + lane * 16;
     const unsigned char* wend = wbase + (size_t)nchunks * NT * wstep;
-    half8_t a_q[PD][2][2];
+    half8_t a_q[PDT][2][2];
 #pragma unroll
-    for (int d = 0; d < PD; d++)
+    for (int d = 0; d < PDT; d++)
 #pragma unroll
         for (int fm = 0; fm < 2; fm++)
 #pragma unroll
@@ -578,17 +582,17 @@ __global__ __launch_bounds__(512) void tconv_p16_kernel(const ConvP16Params p) {
     for (int fn = 0; fn < FN; fn++)
 #pragma unroll
         for (int pl = 0; pl < 2; pl++) b[0][fn][pl] = *reinterpret_cast<const half8_t*>(lds + bbase[0][fn] + G::ROW_PITCH + PITCH + pl * G::PLANE);
-    const unsigned char* wnext = wbase + (size_t)((PD - 1) % (nchunks * NT)) * wstep;
+    const unsigned char* wnext = wbase + (size_t)((PDT - 1) % (nchunks * NT)) * wstep;
     int tile = group, c = 0;
     for (;;) {
-        tp16_stage<G, 0>(acc, a_q, b, bbase, lds, wnext, wbase, wend, wstep);
+        tp16_stage<G, 0, PDT>(acc, a_q, b, bbase, lds, wnext, wbase, wend, wstep);
         if (++c == nchunks) {
             finish_tile(tile);
             c = 0; tile += p.pos_groups;
             if (tile >= ntiles) break;
             zero_acc();
         }
-        tp16_stage<G, 1>(acc, a_q, b, bbase, lds, wnext, wbase, wend, wstep);
+        tp16_stage<G, 1, PDT>(acc, a_q, b, bbase, lds, wnext, wbase, wend, wstep);
         if (++c == nchunks) {
             finish_tile(tile);
             c = 0; tile += p.pos_groups;
@@ -628,8 +632,8 @@ constexpr TP16Entry tentry() {
     return TP16Entry{TH, TW, WM, tconv_p16_kernel<TH, TW, WM>, (size_t)Geo<TH, TW, 1, WM, 1>::BUF};
 }
 const TP16Entry kTEntries[] = {
-    tentry<4, 8, 1>(), tentry<8, 4, 1>(), tentry<2, 8, 1>(),
-    tentry<4, 8, 2>(), tentry<8, 4, 2>(), tentry<2, 8, 2>(),
+    tentry<4, 8, 1>(), tentry<8, 4, 1>(), tentry<2, 8, 1>(), tentry<6, 8, 1>(),
+    tentry<4, 8, 2>(), tentry<8, 4, 2>(), tentry<2, 8, 2>(), tentry<6, 8, 2>(), tentry<8, 6, 2>(),
 };
 }  // namespace
 

@@ -404,6 +404,9 @@ TP16_CASES = [
     (96, 64, 33, 17, "8,4,2", False),       # three chunks
     (64, 96, 7, 11, "2,8,1", True),         # three blocks of output channels
     (64, 128, 21, 40, "2,8,2", False),
+    (128, 64, 29, 37, "6,8,2", True),       # three position fragments per wave: weight ring of three steps
+    (64, 32, 15, 70, "6,8,1", False),
+    (96, 64, 20, 26, "8,6,2", True),
     (64, 32, 80, 150, "4,8,1", True),       # 375 tiles: workgroups walk
     (64, 32, 31, 45, None, False),          # the engine's own choice
 ]
