@@ -603,6 +603,270 @@ __global__ __launch_bounds__(512) void tconv_p16_kernel(const ConvP16Params p) {
     if (p.out_amax) range_publish_waves(p.out_amax, vmax, range_box, 4);
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// K x K convolution (K = 9) on an input of at most four channels (the first layer of a style-transfer net; replaces the
+// render passes of DeepConvLayerNxN::forward, gpu/deep/deepconvlayerNxN.cpp:129-211, for such layers).  A staged pixel
+// is four fp16 channels = 8 bytes per plane, so a lane's eight halves of a k32 step are two horizontally neighbouring
+// taps: a kernel row is padded to (K+1)/2 tap pairs, a step takes four pairs in row-major order (45 pairs = 12 steps for
+// 9x9, the last three pairs empty), and every lane keeps the LDS offset of its pair for each step in a register.  One
+// group of 32 output channels, four tiles of positions side by side; a tile is one stage, walked as above.
+template <int K, int TH_, int TW>
+struct GeoC4 {
+    static constexpr int TH = TH_, STEP = 1, WN = 4, TWG = 4 * TW;
+    static constexpr int HW = TWG + K - 1, HH = TH + K - 1;
+    static constexpr int PPR = (K + 1) / 2, NPAIR = K * PPR;          // tap pairs per kernel row, in all
+    static constexpr int NS = ((NPAIR + 3) / 4 + 2) / 3 * 3;          // steps per stage (two stages are whole turns of the weight ring)
+    static constexpr int PIX = 8;                                     // bytes per staged pixel and plane
+    static constexpr int ROW_PITCH = (HW * PIX + 15) / 16 * 16 + 16;
+    static constexpr int PLANE = HH * ROW_PITCH;
+    static constexpr int BUF = 2 * PLANE;
+    static constexpr int NPOS = TH * TW, FN = NPOS / 16;
+    static constexpr int NITEMS = HH * HW;                            // staging items: pixels
+    static constexpr int NB = (NITEMS + 255) / 256;
+    static constexpr int CPB = 32;
+    static_assert(NPOS % 16 == 0 && (2 * NS) % PD == 0, "whole position fragments; whole ring turns");
+    static_assert(2 * BUF + PLANE < 65536, "offsets fit the LDS instructions' immediate field");
+};
+
+template <class G>
+__device__ __forceinline__ void c4_stager(const ConvP16Params& p, unsigned char* lds, int stid, int cb, int group, int ntiles, unsigned range_bits) {
+    constexpr int sb_off = 2 * G::BUF;
+    const float* in = reinterpret_cast<const float*>(p.in);
+    int i_y[G::NB], i_x[G::NB], l_off[G::NB];
+#pragma unroll
+    for (int i = 0; i < G::NB; i++) {
+        const int idx = stid + i * 256;
+        l_off[i] = -1; i_y[i] = 1 << 20; i_x[i] = 0;
+        if (idx < G::NITEMS) {
+            const int py = idx / G::HW, px = idx - py * G::HW;
+            i_y[i] = py; i_x[i] = px;
+            l_off[i] = py * G::ROW_PITCH + px * G::PIX;
+        }
+    }
+    int g_off[2][G::NB];
+    float4 raw[2][G::NB];
+    float in_scale = 1.f, inv_unused;
+    auto fetch = [&](auto set_, int tile) {
+        constexpr int SET = decltype(set_)::value;
+        const int tyi = (int)(((float)tile + 0.5f) * p.rcp_tiles_x), txi = tile - tyi * p.tiles_x;
+        const int y0 = tyi * G::TH + p.in_y0, x0 = txi * G::TWG + p.in_x0;
+#pragma unroll
+        for (int i = 0; i < G::NB; i++) {
+            int gy = y0 + i_y[i], gx = x0 + i_x[i];
+            if (p.in_clamp && l_off[i] >= 0) {
+                gy = min(max(gy, 0), p.in_hp - 1);
+                gx = min(max(gx, 0), p.in_wp - 1);
+            }
+            g_off[SET][i] = ((unsigned)gy < (unsigned)p.in_hp && (unsigned)gx < (unsigned)p.in_wp) ? (gy * p.in_wp + gx) * 4 : -1;
+            raw[SET][i] = *reinterpret_cast<const float4*>(in + (g_off[SET][i] >= 0 ? g_off[SET][i] : 0));
+        }
+    };
+    auto store = [&](auto set_, unsigned char* buf) {
+        constexpr int SET = decltype(set_)::value;
+        typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+#pragma unroll
+        for (int i = 0; i < G::NB; i++) {
+            if (l_off[i] < 0) continue;
+            const bool ok = g_off[SET][i] >= 0;
+            const float r[4] = {raw[SET][i].x, raw[SET][i].y, raw[SET][i].z, raw[SET][i].w};
+            half4_t hi, lo;
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const float v = ok ? act_p16(r[e], p.act) * in_scale : 0.f;
+                hi[e] = (_Float16)v;
+                lo[e] = (_Float16)(v - (float)hi[e]);
+            }
+            *reinterpret_cast<half4_t*>(buf + l_off[i]) = hi;
+            *reinterpret_cast<half4_t*>(buf + G::PLANE + l_off[i]) = lo;
+        }
+    };
+    typedef std::integral_constant<int, 0> Set0;
+    typedef std::integral_constant<int, 1> Set1;
+    int tile = group;                       // the stage the MFMA waves are on
+    int t1 = tile + p.pos_groups, t2 = t1 + p.pos_groups;
+    fetch(Set0(), tile);
+    if (p.in_amax) in_scale = range_scale(range_after_act(range_reduce(range_bits), p.act), &inv_unused);
+    if (stid < 32) {
+        reinterpret_cast<float*>(lds + sb_off)[stid] = p.scale[cb * 32 + stid];
+        reinterpret_cast<float*>(lds + sb_off)[32 + stid] = p.bias[cb * 32 + stid];
+    }
+    store(Set0(), lds);
+    lds_barrier();
+    if (t1 < ntiles) fetch(Set1(), t1);
+    auto iteration = [&](auto next_set, auto free_set, unsigned char* next_buf) {
+        if (t1 < ntiles) store(next_set, next_buf);
+        if (t2 < ntiles) fetch(free_set, t2);
+        lds_barrier();
+        const bool go_on = t1 < ntiles;
+        tile = t1; t1 = t2; t2 += p.pos_groups;
+        return go_on;
+    };
+    for (;;) {
+        if (!iteration(Set1(), Set0(), lds + G::BUF)) break;
+        if (!iteration(Set0(), Set1(), lds)) break;
+    }
+}
+
+template <class G, int BUFI>
+__device__ __forceinline__ void c4_stage(f32x4_t (&acc)[2][G::FN], half8_t (&a_q)[PD][2][2], half8_t (&b)[G::FN][2], const int (&bbase)[G::FN],
+                                         const int (&off)[G::NS], const unsigned char* lds, const unsigned char*& wnext,
+                                         const unsigned char* wbase, const unsigned char* wend, unsigned wstep) {
+    constexpr int FN = G::FN, NS = G::NS;
+    typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+#pragma unroll
+    for (int dd = 0; dd < NS; dd++) {
+        const int d = (BUFI * NS + dd) % PD, dprev = (d + PD - 1) % PD;
+        const int nbuf = (dd + 1 == NS) ? 1 - BUFI : BUFI, ns = (dd + 1) % NS;
+        const unsigned char* w_ = wnext;
+        wnext += wstep;
+        if (wnext == wend) wnext = wbase;
+#pragma unroll
+        for (int i = 0; i < 6 * FN; i++) {
+            const int fn = i / 6, r = i % 6, kind = r / 2, fm = r % 2;
+            const int apl = (kind == 1) ? 1 : 0, bpl = (kind == 2) ? 1 : 0;
+            acc[fm][fn] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_q[d][fm][apl], b[fn][bpl], acc[fm][fn], 0, 0, 0);
+            if (dd == NS - 1 && i == 3) lds_barrier();
+            if (r == 5) {
+                const unsigned char* src = lds + nbuf * G::BUF + bbase[fn] + off[ns];
+#pragma unroll
+                for (int pl = 0; pl < 2; pl++) {
+                    const half4_t t0 = *reinterpret_cast<const half4_t*>(src + pl * G::PLANE);
+                    const half4_t t1 = *reinterpret_cast<const half4_t*>(src + pl * G::PLANE + G::PIX);
+                    b[fn][pl] = half8_t{t0[0], t0[1], t0[2], t0[3], t1[0], t1[1], t1[2], t1[3]};
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+                if (i == (j * 6 * FN) / 4 + 1) a_q[dprev][j % 2][j / 2] = *reinterpret_cast<const half8_t*>(w_ + ((j % 2) * 2 + j / 2) * 1024);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+}
+
+template <int K, int TH, int TW>
+__global__ __launch_bounds__(512) void conv_p16c4_kernel(const ConvP16Params p) {
+    using G = GeoC4<K, TH, TW>;
+    constexpr int FN = G::FN, NS = G::NS;
+    typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+    extern __shared__ __align__(16) unsigned char lds[];
+    __shared__ unsigned range_box[2];
+    if (blockIdx.x == 0) range_clear(p.reset[0], p.reset[1], p.reset[2], p.reset[3], p.nreset);
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    int bid = blockIdx.x;
+    {
+        const int nblk = p.pos_groups * p.cout_blocks;
+        const int per = nblk >> 3;
+        if (bid < (per << 3)) bid = (bid & 7) * per + (bid >> 3);
+    }
+    const int cb = bid % p.cout_blocks;
+    const int group = bid / p.cout_blocks;
+    const int ntiles = p.tiles_x * p.tiles_y;
+    if (tid < 2) range_box[tid] = 0u;
+    const unsigned range_bits = p.in_amax ? range_load(p.in_amax) : 0u;
+    constexpr int sb_off = 2 * G::BUF;
+    if (wave < 4) {
+        c4_stager<G>(p, lds, tid & 255, cb, group, ntiles, range_bits);
+        return;
+    }
+    const int mq = lane & 15, kq = lane >> 4;
+    const int wn = wave - 4;
+    int bbase[FN];
+#pragma unroll
+    for (int fn = 0; fn < FN; fn++) {
+        const int m = fn * 16 + mq;
+        const int ty = m / TW, tx = m - ty * TW;
+        bbase[fn] = ty * G::ROW_PITCH + (wn * TW + tx) * G::PIX;
+    }
+    int off[NS];   // LDS offset of this lane's tap pair in each step (pairs beyond the kernel: pair 0, their weights are zero)
+#pragma unroll
+    for (int st = 0; st < NS; st++) {
+        const int pi = 4 * st + kq;
+        const int row = pi / G::PPR, col = 2 * (pi - row * G::PPR);
+        off[st] = pi < G::NPAIR ? row * G::ROW_PITCH + col * G::PIX : 0;
+    }
+    const unsigned wstep = (unsigned)p.mfrags * 2 * 1024;
+    const unsigned char* wbase = reinterpret_cast<const unsigned char*>(p.wpack) + (size_t)(cb * 2 * 2) * 1024 + lane * 16;
+    const unsigned char* wend = wbase + (size_t)NS * wstep;
+    half8_t a_q[PD][2][2];
+#pragma unroll
+    for (int d = 0; d < PD; d++)
+#pragma unroll
+        for (int fm = 0; fm < 2; fm++)
+#pragma unroll
+            for (int pl = 0; pl < 2; pl++) a_q[d][fm][pl] = *reinterpret_cast<const half8_t*>(wbase + (size_t)d * wstep + (fm * 2 + pl) * 1024);
+    f32x4_t acc[2][FN];
+    auto zero_acc = [&]() {
+#pragma unroll
+        for (int fm = 0; fm < 2; fm++)
+#pragma unroll
+            for (int fn = 0; fn < FN; fn++) acc[fm][fn] = (f32x4_t)(0.f);
+    };
+    zero_acc();
+    float inv_in_scale = 1.f;
+    if (p.in_amax) (void)range_scale(range_after_act(range_reduce(range_bits), p.act), &inv_in_scale);
+    const float acc_mul = p.acc_mul * inv_in_scale;
+    float* out = reinterpret_cast<float*>(p.out);
+    float vmax = 0.f;
+    auto finish_tile = [&](int tile) {
+        const int tyi = (int)(((float)tile + 0.5f) * p.rcp_tiles_x), txi = tile - tyi * p.tiles_x;
+        const float* sb = reinterpret_cast<const float*>(lds + sb_off);
+        f32x4_t bi[2], scm[2];
+#pragma unroll
+        for (int fm = 0; fm < 2; fm++) {
+            scm[fm] = *reinterpret_cast<const f32x4_t*>(sb + fm * 16 + kq * 4) * acc_mul;
+            bi[fm] = *reinterpret_cast<const f32x4_t*>(sb + 32 + fm * 16 + kq * 4);
+        }
+#pragma unroll
+        for (int fn = 0; fn < FN; fn++) {
+            const int m = fn * 16 + mq;
+            const int ty = m / TW, tx = wn * TW + (m - ty * TW);
+            const int py = tyi * TH + ty, px = txi * G::TWG + tx;
+            const bool ok = py < p.npos_y && px < p.npos_x;
+            const size_t obase = ((size_t)(p.out_off_y + py) * p.out_wp + p.out_off_x + px) * p.out_cp + cb * 32 + kq * 4;
+            float fmax_ = 0.f;
+#pragma unroll
+            for (int fm = 0; fm < 2; fm++) {
+                f32x4_t v;
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    v[e] = acc[fm][fn][e] * scm[fm][e] + bi[fm][e];
+                    fmax_ = fmaxf(fmax_, fabsf(v[e]));
+                }
+                if (ok) *reinterpret_cast<f32x4_t*>(out + obase + fm * 16) = v;
+            }
+            vmax = fmaxf(vmax, ok ? fmax_ : 0.f);
+        }
+    };
+    lds_barrier();   // the first stage is staged
+    half8_t b[FN][2];
+#pragma unroll
+    for (int fn = 0; fn < FN; fn++)
+#pragma unroll
+        for (int pl = 0; pl < 2; pl++) {
+            const unsigned char* src = lds + bbase[fn] + off[0] + pl * G::PLANE;
+            const half4_t t0 = *reinterpret_cast<const half4_t*>(src);
+            const half4_t t1 = *reinterpret_cast<const half4_t*>(src + G::PIX);
+            b[fn][pl] = half8_t{t0[0], t0[1], t0[2], t0[3], t1[0], t1[1], t1[2], t1[3]};
+        }
+    const unsigned char* wnext = wbase + (size_t)(PD - 1) * wstep;
+    int tile = group;
+    for (;;) {
+        c4_stage<G, 0>(acc, a_q, b, bbase, off, lds, wnext, wbase, wend, wstep);
+        finish_tile(tile);
+        tile += p.pos_groups;
+        if (tile >= ntiles) break;
+        zero_acc();
+        c4_stage<G, 1>(acc, a_q, b, bbase, off, lds, wnext, wbase, wend, wstep);
+        finish_tile(tile);
+        tile += p.pos_groups;
+        if (tile >= ntiles) break;
+        zero_acc();
+    }
+    if (p.out_amax) range_publish_waves(p.out_amax, vmax, range_box, 4);
+}
+
 typedef void (*p16_fn)(const ConvP16Params);
 struct P16Entry {
     int th, tw, stride, wm;
@@ -635,6 +899,15 @@ const TP16Entry kTEntries[] = {
     tentry<4, 8, 1>(), tentry<8, 4, 1>(), tentry<2, 8, 1>(), tentry<6, 8, 1>(),
     tentry<4, 8, 2>(), tentry<8, 4, 2>(), tentry<2, 8, 2>(), tentry<6, 8, 2>(), tentry<8, 6, 2>(),
 };
+struct C4Entry {
+    int k, th, tw;
+    p16_fn fn;
+    size_t buf;
+    int steps;
+};
+template <int K, int TH, int TW>
+constexpr C4Entry c4entry() { return C4Entry{K, TH, TW, conv_p16c4_kernel<K, TH, TW>, (size_t)GeoC4<K, TH, TW>::BUF, GeoC4<K, TH, TW>::NS}; }
+const C4Entry kC4Entries[] = {c4entry<9, 8, 8>(), c4entry<9, 4, 8>(), c4entry<9, 8, 4>()};
 }  // namespace
 
 int conv_p16_tile_count() { return (int)(sizeof(kEntries) / sizeof(kEntries[0])); }
@@ -724,6 +997,41 @@ int launch_tconv_p16(const ConvP16Params& p, hipStream_t s) {
         p.rcp_tiles_x != 1.0f / (float)p.tiles_x || p.tiles_x * p.tiles_y > 4000000)
         return -5;
     const size_t lds_bytes = tconv_p16_lds_bytes(p);
+    if (lds_bytes > 160 * 1024) return -2;
+    if (ensure_lds(reinterpret_cast<const void*>(e->fn), lds_bytes) != 0) return -2;
+    hipLaunchKernelGGL(e->fn, dim3(p.pos_groups * p.cout_blocks), dim3(512), lds_bytes, s, p);
+    return hipGetLastError() == hipSuccess ? 0 : -3;
+}
+
+int conv_p16c4_tile_count() { return (int)(sizeof(kC4Entries) / sizeof(kC4Entries[0])); }
+void conv_p16c4_tile(int index, int* k, int* th, int* tw, int* steps) {
+    *k = kC4Entries[index].k; *th = kC4Entries[index].th; *tw = kC4Entries[index].tw; *steps = kC4Entries[index].steps;
+}
+static const C4Entry* find_c4entry(const ConvP16Params& p, int k) {
+    for (const C4Entry& c : kC4Entries)
+        if (c.k == k && c.th == p.tile_h && c.tw == p.tile_w) return &c;
+    return nullptr;
+}
+size_t conv_p16c4_lds_bytes(const ConvP16Params& p, int k) {
+    const C4Entry* e = find_c4entry(p, k);
+    return e ? 2 * e->buf + 2 * 32 * 4 : 0;
+}
+bool conv_p16c4_supported(int k, int stride, int dil, int in_cp, int cout, int out_cp, bool f16) {
+    return k == 9 && stride == 1 && dil == 1 && !f16 && in_cp == 4 && cout % 32 == 0 && out_cp % 4 == 0 && out_cp >= cout;
+}
+
+// k x k convolution on a four-channel input: wpack = [step][cout fragment of 16][plane][lane][8 halves], lane = (output
+// channel lane%16, tap pair 4*step + lane/16 = kernel row pair/((k+1)/2), columns 2*(pair%((k+1)/2)) and +1), four input
+// channels per tap; in_y0/in_x0 = input padding - (k-1)/2
+int launch_conv_p16c4(const ConvP16Params& p, int k, hipStream_t s) {
+    const C4Entry* e = find_c4entry(p, k);
+    if (!e) return -1;
+    if (p.in_cp != 4 || p.cin_chunks != 1 || p.cout_blocks < 1 || p.mfrags < p.cout_blocks * 2 || p.wm != 1 || p.stride != 1 || p.res ||
+        p.tiles_x * 4 * e->tw < p.npos_x || p.tiles_y * e->th < p.npos_y || p.out_cp < p.cout_blocks * 32 ||
+        p.nreset < 0 || p.nreset > 4 || p.pos_groups < 1 || p.pos_groups > p.tiles_x * p.tiles_y ||
+        p.rcp_tiles_x != 1.0f / (float)p.tiles_x || p.tiles_x * p.tiles_y > 4000000)
+        return -5;
+    const size_t lds_bytes = conv_p16c4_lds_bytes(p, k);
     if (lds_bytes > 160 * 1024) return -2;
     if (ensure_lds(reinterpret_cast<const void*>(e->fn), lds_bytes) != 0) return -2;
     hipLaunchKernelGGL(e->fn, dim3(p.pos_groups * p.cout_blocks), dim3(512), lds_bytes, s, p);

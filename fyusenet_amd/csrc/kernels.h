@@ -213,6 +213,12 @@ void tconv_p16_tile(int index, int* th, int* tw, int* wm);
 void tconv_p16_tap(int t, int* ky, int* kx);   // kernel tap of step t of a chunk
 size_t tconv_p16_lds_bytes(const ConvP16Params& p);
 int launch_tconv_p16(const ConvP16Params& p, hipStream_t s);
+// the 9x9 convolution on an input of at most four channels, on the same parameters (one chunk, one channel group)
+bool conv_p16c4_supported(int k, int stride, int dil, int in_cp, int cout, int out_cp, bool f16);
+int conv_p16c4_tile_count();
+void conv_p16c4_tile(int index, int* k, int* th, int* tw, int* steps);
+size_t conv_p16c4_lds_bytes(const ConvP16Params& p, int k);
+int launch_conv_p16c4(const ConvP16Params& p, int k, hipStream_t s);
 
 // ---------------------------------------------------------------------------------------------
 // Direct (non-MFMA) layer kernels (layers_direct.hip)

@@ -966,6 +966,108 @@ class ConvLayer : public Layer {
             p16_wpack_dev = nullptr;
         }
     }
+    // the small-input form (conv_p16.hip, conv_p16c4_kernel): 9x9 on at most four input channels
+    void setup_c4(const TView& in_v, const TView& out_v) {
+        ConvP16Params q{};
+        q.in = in_v.ptr; q.out = out_v.ptr; q.res = nullptr;
+        q.in_hp = in_v.hp(); q.in_wp = in_v.wp(); q.in_cp = in_v.cp;
+        q.stride = 1; q.wm = 1;
+        q.in_y0 = q.in_x0 = in_v.pad - (k - 1) / 2;
+        q.in_clamp = clamp ? 1 : 0;
+        q.npos_y = oh; q.npos_x = ow;
+        q.out_wp = out_v.wp(); q.out_cp = out_v.cp; q.out_off_y = q.out_off_x = out_v.pad;
+        q.cin_chunks = 1;
+        q.mfrags = oc / 16;
+        q.cout_blocks = oc / 32;
+        q.scale = scale_dev; q.bias = bias_dev;
+        q.acc_mul = 1.f;
+        q.act = act();
+        int want_h = 0, want_w = 0;
+        if (const char* e = getenv("FYNHIP_P16_TILE")) sscanf(e, "%d,%d", &want_h, &want_w);
+        std::vector<ConvP16Params> cands;
+        int steps = 0;
+        for (int i = 0; i < conv_p16c4_tile_count(); i++) {
+            int kk, th, tw, ns;
+            conv_p16c4_tile(i, &kk, &th, &tw, &ns);
+            if (kk != k || (want_h && (th != want_h || tw != want_w))) continue;
+            ConvP16Params c = q;
+            c.tile_h = th; c.tile_w = tw;
+            c.tiles_x = (ow + 4 * tw - 1) / (4 * tw); c.tiles_y = (oh + th - 1) / th;
+            c.rcp_tiles_x = 1.0f / (float)c.tiles_x;
+            c.pos_groups = std::max(1, std::min(c.tiles_x * c.tiles_y, 256 / c.cout_blocks));
+            const size_t lds = conv_p16c4_lds_bytes(c, k);
+            if (lds == 0 || lds > 160 * 1024) continue;
+            steps = ns;
+            cands.push_back(c);
+        }
+        if (cands.empty()) return;
+        c4_steps = steps;
+        const size_t halves = ((size_t)steps + 8) * q.mfrags * 2 * 64 * 8;
+        p16_wpack_dev = net->dev_alloc(halves * 2, true);
+        for (ConvP16Params& c : cands) c.wpack = p16_wpack_dev;
+        const bool always = getenv("FYNHIP_FORCE_P16_CONV") != nullptr;
+        const char* at = getenv("FYNHIP_AUTOTUNE");
+        int pick = 0;
+        char key[160];
+        snprintf(key, sizeof(key), "c4p16:k%d:%dx%d:%dx%d:e%d", k, d.in_channels, oc, oh, ow, clamp ? 1 : 0);
+        int cached[3] = {0, 0, 0};
+        if (!want_h && tune_cache_triple(key, cached)) {
+            pick = -1;
+            if (cached[0] || always)
+                for (size_t i = 0; i < cands.size(); i++)
+                    if (cands[i].tile_h * 1000 + cands[i].tile_w == cached[1]) pick = (int)i;
+            if (always && pick < 0) pick = 0;
+        } else if (!(at && at[0] == '0')) {
+            float best = 1e30f, t_other = 1e30f;
+            for (int rep = 0; rep < 3; rep++) {
+                for (size_t i = 0; i < cands.size(); i++) {
+                    const float t = time_calls(net, [&]() {
+                        if (launch_conv_p16c4(cands[i], k, net->stream) != 0) fail(FYN_ERR_DEVICE, "small-input 16-position convolution launch failed while tuning");
+                    }, 10);
+                    if (t < best) { best = t; pick = (int)i; }
+                }
+                t_other = std::min(t_other, time_launch(net, launch, 10));
+            }
+            if (getenv("FYNHIP_TUNE_VERBOSE"))
+                fprintf(stderr, "[tune] %dx%d on %d channels: 16-position fragments (%dx%d tiles) %.1f us, general kernel %.1f us\n", k, k, d.in_channels,
+                        cands[pick].tile_h, cands[pick].tile_w, best * 1e3f, t_other * 1e3f);
+            const bool win = best < t_other;
+            if (!want_h) tune_cache_store_triple(key, win ? 1 : 0, cands[pick].tile_h * 1000 + cands[pick].tile_w, 1);
+            if (!win && !always) pick = -1;
+        }
+        if (pick >= 0) {
+            p16 = true; c4 = true;
+            pp = cands[pick];
+        } else {
+            net->dev_free(p16_wpack_dev);
+            p16_wpack_dev = nullptr;
+        }
+    }
+    // weights of that form: [step][cout fragment of 16][plane][lane][8 halves]; lane = (channel lane%16, tap pair 4*step + lane/16)
+    void pack_c4(const float* w, float wmul) {
+        const int cin = d.in_channels, ppr = (k + 1) / 2;
+        std::vector<uint16_t> pack(((size_t)c4_steps + 8) * pp.mfrags * 2 * 64 * 8, 0);
+        for (int st = 0; st < c4_steps; st++)
+            for (int mf = 0; mf < pp.mfrags; mf++) {
+                uint16_t* base = pack.data() + (((size_t)st * pp.mfrags + mf) * 2) * 64 * 8;
+                for (int lane = 0; lane < 64; lane++) {
+                    const int o = mf * 16 + (lane & 15), pi = 4 * st + (lane >> 4);
+                    const int ky = pi / ppr, kx0 = 2 * (pi % ppr);
+                    if (o >= oc || ky >= k) continue;
+                    for (int j = 0; j < 8; j++) {
+                        const int kx = kx0 + j / 4, ci = j % 4;
+                        if (kx >= k || ci >= cin) continue;
+                        const float v = w[(((size_t)o * k + ky) * k + kx) * cin + ci] * wmul;
+                        const uint16_t hi = f2h_bits(v);
+                        base[(size_t)lane * 8 + j] = hi;
+                        base[(size_t)(64 + lane) * 8 + j] = f2h_bits(v - h2f(hi));
+                    }
+                }
+            }
+        FYN_HIP(hipStreamSynchronize(net->stream));
+        FYN_HIP(hipMemcpyAsync(p16_wpack_dev, pack.data(), pack.size() * 2, hipMemcpyHostToDevice, net->stream));
+        FYN_HIP(hipStreamSynchronize(net->stream));
+    }
     // weights of that form: [(chunk*9 + tap)][cout fragment of 16][plane][lane][8 halves], zero steps behind the last
     void pack_p16(const float* w, float wmul) {
         const int cin = d.in_channels;
@@ -1195,6 +1297,9 @@ class ConvLayer : public Layer {
             if (!frac_shift && !sc.in_sub && conv_p16_supported(k, stride, dil, in_v.cp, oc, out_v.cp, out_v.f16 != 0) && d.in_channels == in_v.cp &&
                 (!res_v || res_v->cp >= oc) && !getenv("FYNHIP_NO_P16_CONV"))
                 setup_p16(in_v, out_v, res_v, res_relu, res_scale);
+            if (!frac_shift && !res_v && conv_p16c4_supported(k, stride, dil, in_v.cp, oc, out_v.cp, out_v.f16 != 0) &&
+                !getenv("FYNHIP_NO_P16_CONV"))
+                setup_c4(in_v, out_v);
         }
         if (direct) {
             scale_dev = static_cast<float*>(net->dev_alloc(padded * sizeof(float)));
@@ -1225,7 +1330,8 @@ class ConvLayer : public Layer {
         } else if (p16) {
             const float wmul = weight_prescale(w, (size_t)oc * k * k * d.in_channels);
             pp.acc_mul = 1.0f / wmul;
-            pack_p16(w, wmul);
+            if (c4) pack_c4(w, wmul);
+            else pack_p16(w, wmul);
         } else if (wide && rows) {
             const float wmul = weight_prescale(w, (size_t)oc * k * k * d.in_channels);
             rp.acc_mul = 1.0f / wmul;
@@ -1266,7 +1372,7 @@ class ConvLayer : public Layer {
             return;
         }
         if (p16) {
-            if (launch_conv_p16(pp, s) != 0) fail(FYN_ERR_DEVICE, "layer %s: convolution launch failed", d.name);
+            if ((c4 ? launch_conv_p16c4(pp, k, s) : launch_conv_p16(pp, s)) != 0) fail(FYN_ERR_DEVICE, "layer %s: convolution launch failed", d.name);
             return;
         }
         if (direct) launch_conv_direct(dp, s);
@@ -1281,6 +1387,13 @@ class ConvLayer : public Layer {
             char buf[200];
             snprintf(buf, sizeof(buf), "conv_rows %s(kx folded into cout, rows rolled through an LDS ring) strips=%d x %d row blocks of %d rows, lds=%zu",
                      tout().v.f16 ? "f16 " : "f16x2-split ", rp.strips, rp.row_blocks, rp.rows_per_block, conv_rows_lds_bytes(rp, tout().v.f16 != 0));
+            return mode + buf;
+        }
+        if (p16 && c4) {
+            char buf[220];
+            snprintf(buf, sizeof(buf), "conv_p16c4 f16x2-split (tap pairs of a 4-channel pixel) tile=32x%d(cout x pos) th=%d tw=%d blocks=%d tiles=%d lds=%zu steps=%d",
+                     pp.tile_h * pp.tile_w * 4, pp.tile_h, pp.tile_w, pp.pos_groups * pp.cout_blocks, pp.tiles_x * pp.tiles_y * pp.cout_blocks,
+                     conv_p16c4_lds_bytes(pp, k), c4_steps);
             return mode + buf;
         }
         if (p16) {
@@ -1303,6 +1416,8 @@ class ConvLayer : public Layer {
     ConvRowsParams rp{};          // row-rolling form of the folded convolution (conv_rows.hip)
     void* rows_wpack_dev = nullptr;
     bool p16 = false;             // 16-position-fragment form of a 3x3 convolution (conv_p16.hip)
+    bool c4 = false;              // ... its variant for inputs of at most four channels
+    int c4_steps = 0;
     ConvP16Params pp{};
     void* p16_wpack_dev = nullptr;
     ConvDirectParams dp{};

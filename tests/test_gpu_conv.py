@@ -396,6 +396,43 @@ def test_transconv_parity(k, crop, cin, cout, h, w, storage):
     assert err <= TOL[storage]
 
 
+C4_CASES = [
+    # cin, cout, h, w, tile "h,w", kw
+    (3, 32, 40, 56, "8,8", {"bn": True}),            # the style net's first layer, reduced
+    (3, 32, 19, 37, "4,8", {}),                      # ragged
+    (4, 64, 23, 30, "8,4", {"pad_out": 1}),          # four channels, two blocks of output channels
+    (1, 32, 12, 70, "4,8", {"bn": True}),
+    (3, 32, 90, 300, "8,8", {}),                     # 360 tiles: workgroups walk
+    (3, 32, 33, 50, None, {"pad_out": 2}),
+]
+
+
+@pytest.mark.parametrize("shallow", [False, True], ids=["deep", "shallow_edge_clamp"])
+@pytest.mark.parametrize("case", C4_CASES, ids=lambda c: "%dx%dx%d_to%d_%s" % (c[0], c[2], c[3], c[1], (c[4] or "auto").replace(",", "x")))
+def test_small_input_sixteen_position_fragment_form(case, shallow, monkeypatch):
+    """The 9x9 convolution on at most four input channels with two taps of a 4-channel pixel per lane and step (fp32
+    storage)."""
+    cin, cout, h, w, tile, kw = case
+    if shallow and ("pad_out" in kw or h > 60):
+        pytest.skip("the shallow variant is run on the plain cases")
+    monkeypatch.setenv("FYNHIP_FORCE_P16_CONV", "1")
+    if tile:
+        monkeypatch.setenv("FYNHIP_P16_TILE", tile)
+    if shallow:
+        kw = dict(kw, deep=False, pad_in=0)
+    b = conv_builder(9, cout, h, w, cin, 1, 1, A.NONE, **kw)
+    wts = conv_block(1200 + cin, cout, 9, cin, bn=kw.get("bn", False))
+    x = prng.uniform(61 * cin + w, (cin, h, w), 0, 1)
+    got, info = run_single(b, fa.STORAGE_F32, [x], wts)
+    ref = oracle_single(b, fa.STORAGE_F32, [x], wts)
+    err = rel_l2(got, ref)
+    print("  ", info, "rel_l2=%.3e" % err, flush=True)
+    assert "conv_p16c4" in info
+    if tile:
+        assert "th=%s tw=%s" % tuple(tile.split(",")) in info
+    assert err <= TOL[fa.STORAGE_F32], info
+
+
 TP16_CASES = [
     # cin, cout, h, w, tile "h,w,channel groups", batch-norm
     (64, 32, 20, 26, "4,8,1", True),        # four tiles of positions side by side, ragged on both sides
