@@ -119,7 +119,7 @@ struct Geo {
 template <class G, int BUFI>
 __device__ __forceinline__ void p16_stage(f32x4_t (&acc)[2][G::FN], half8_t (&a_q)[PD][2][2], half8_t (&b)[G::FN][2],
                                           const int (&bbase)[2][G::FN], const unsigned char* lds, const unsigned char*& wnext,
-                                          const unsigned char* wbase, const unsigned char* wend, unsigned wstep) {
+                                          const unsigned char* wbase, const unsigned char* wend, unsigned wstep, unsigned wlane) {
     constexpr int FN = G::FN;
 #pragma unroll
     for (int dd = 0; dd < NT; dd++) {
@@ -140,7 +140,7 @@ __device__ __forceinline__ void p16_stage(f32x4_t (&acc)[2][G::FN], half8_t (&a_
             }
 #pragma unroll
             for (int j = 0; j < 4; j++)   // the four weight fragments of a step, spread over its slots
-                if (i == (j * 6 * FN) / 4 + 1) a_q[dprev][j % 2][j / 2] = *reinterpret_cast<const half8_t*>(w_ + ((j % 2) * 2 + j / 2) * 1024);
+                if (i == (j * 6 * FN) / 4 + 1) a_q[dprev][j % 2][j / 2] = *reinterpret_cast<const half8_t*>(w_ + ((j % 2) * 2 + j / 2) * 1024 + wlane);
             __builtin_amdgcn_sched_barrier(0);
         }
     }
@@ -325,7 +325,8 @@ __global__ __launch_bounds__(512) void conv_p16_kernel(const ConvP16Params p) {
     }
     // A fragments: [(chunk*9 + tap)][cout fragment of 16][plane][lane] x 8 halves
     const unsigned wstep = (unsigned)p.mfrags * 2 * 1024;
-    const unsigned char* wbase = reinterpret_cast<const unsigned char*>(p.wpack) + (size_t)((cb * 2 * WM + mw * 2) * 2) * 1024 + lane * 16;
+    const unsigned char* wbase = reinterpret_cast<const unsigned char*>(p.wpack) + (size_t)((cb * 2 * WM + mw * 2) * 2) * 1024;   // (uniform: the loads take it as their scalar base)
+    const unsigned wlane = lane * 16;
     const unsigned char* wend = wbase + (size_t)nchunks * NT * wstep;
     half8_t a_q[PD][2][2];
 #pragma unroll
@@ -333,7 +334,7 @@ __global__ __launch_bounds__(512) void conv_p16_kernel(const ConvP16Params p) {
 #pragma unroll
         for (int fm = 0; fm < 2; fm++)
 #pragma unroll
-            for (int pl = 0; pl < 2; pl++) a_q[d][fm][pl] = *reinterpret_cast<const half8_t*>(wbase + (size_t)d * wstep + (fm * 2 + pl) * 1024);
+            for (int pl = 0; pl < 2; pl++) a_q[d][fm][pl] = *reinterpret_cast<const half8_t*>(wbase + (size_t)d * wstep + (fm * 2 + pl) * 1024 + wlane);
     f32x4_t acc[2][FN];
     auto zero_acc = [&]() {
 #pragma unroll
@@ -406,7 +407,8 @@ __global__ __launch_bounds__(512) void conv_p16_kernel(const ConvP16Params p) {
     const unsigned char* wnext = wbase + (size_t)((PD - 1) % (nchunks * NT)) * wstep;
     int tile = group, c = 0;
     for (;;) {
-        p16_stage<G, 0>(acc, a_q, b, bbase, lds, wnext, wbase, wend, wstep);
+        p16_stage<G, 0>(acc, a_q, b, bbase, lds, wnext, wbase, wend, wstep, wlane);
+        FYN_PTRACE(3 + (c < 12 ? c : 12));
         if (++c == nchunks) {
             FYN_PTRACE(29);
             finish_tile(tile);
@@ -415,9 +417,12 @@ __global__ __launch_bounds__(512) void conv_p16_kernel(const ConvP16Params p) {
             if (tile >= ntiles) break;
             zero_acc();
         }
-        p16_stage<G, 1>(acc, a_q, b, bbase, lds, wnext, wbase, wend, wstep);
+        p16_stage<G, 1>(acc, a_q, b, bbase, lds, wnext, wbase, wend, wstep, wlane);
+        FYN_PTRACE(3 + (c < 12 ? c : 12));
         if (++c == nchunks) {
+            FYN_PTRACE(29);
             finish_tile(tile);
+            FYN_PTRACE(30);
             c = 0; tile += p.pos_groups;
             if (tile >= ntiles) break;
             zero_acc();
@@ -446,7 +451,7 @@ constexpr bool tt_last_of_shift(int t) { return t == NT - 1 || tt_shift(t + 1) !
 template <class G, int BUFI, int PDT>
 __device__ __forceinline__ void tp16_stage(f32x4_t (&acc)[4][2][G::FN], half8_t (&a_q)[PDT][2][2], half8_t (&b)[2][G::FN][2],
                                            const int (&bbase)[2][G::FN], const unsigned char* lds, const unsigned char*& wnext,
-                                           const unsigned char* wbase, const unsigned char* wend, unsigned wstep) {
+                                           const unsigned char* wbase, const unsigned char* wend, unsigned wstep, unsigned wlane) {
     constexpr int FN = G::FN;
 #pragma unroll
     for (int t = 0; t < NT; t++) {
@@ -471,7 +476,7 @@ __device__ __forceinline__ void tp16_stage(f32x4_t (&acc)[4][2][G::FN], half8_t 
             }
 #pragma unroll
             for (int j = 0; j < 4; j++)   // the four weight fragments of a step, spread over its slots
-                if (i == (j * 6 * FN) / 4 + 1) a_q[dprev][j % 2][j / 2] = *reinterpret_cast<const half8_t*>(w_ + ((j % 2) * 2 + j / 2) * 1024);
+                if (i == (j * 6 * FN) / 4 + 1) a_q[dprev][j % 2][j / 2] = *reinterpret_cast<const half8_t*>(w_ + ((j % 2) * 2 + j / 2) * 1024 + wlane);
             __builtin_amdgcn_sched_barrier(0);
         }
     }
@@ -518,7 +523,8 @@ __global__ __launch_bounds__(512) void tconv_p16_kernel(const ConvP16Params p) {
         bbase[1][fn] = bbase[0][fn] + G::BUF;
     }
     const unsigned wstep = (unsigned)p.mfrags * 2 * 1024;
-    const unsigned char* wbase = reinterpret_cast<const unsigned char*>(p.wpack) + (size_t)((cb * 2 * WM + mw * 2) * 2) * 1024 + lane * 16;
+    const unsigned char* wbase = reinterpret_cast<const unsigned char*>(p.wpack) + (size_t)((cb * 2 * WM + mw * 2) * 2) * 1024;   // (uniform: the loads take it as their scalar base)
+    const unsigned wlane = lane * 16;
     const unsigned char* wend = wbase + (size_t)nchunks * NT * wstep;
     half8_t a_q[PDT][2][2];
 #pragma unroll
@@ -526,7 +532,7 @@ __global__ __launch_bounds__(512) void tconv_p16_kernel(const ConvP16Params p) {
 #pragma unroll
         for (int fm = 0; fm < 2; fm++)
 #pragma unroll
-            for (int pl = 0; pl < 2; pl++) a_q[d][fm][pl] = *reinterpret_cast<const half8_t*>(wbase + (size_t)d * wstep + (fm * 2 + pl) * 1024);
+            for (int pl = 0; pl < 2; pl++) a_q[d][fm][pl] = *reinterpret_cast<const half8_t*>(wbase + (size_t)d * wstep + (fm * 2 + pl) * 1024 + wlane);
     f32x4_t acc[4][2][FN];
     auto zero_acc = [&]() {
 #pragma unroll
@@ -585,14 +591,14 @@ __global__ __launch_bounds__(512) void tconv_p16_kernel(const ConvP16Params p) {
     const unsigned char* wnext = wbase + (size_t)((PDT - 1) % (nchunks * NT)) * wstep;
     int tile = group, c = 0;
     for (;;) {
-        tp16_stage<G, 0, PDT>(acc, a_q, b, bbase, lds, wnext, wbase, wend, wstep);
+        tp16_stage<G, 0, PDT>(acc, a_q, b, bbase, lds, wnext, wbase, wend, wstep, wlane);
         if (++c == nchunks) {
             finish_tile(tile);
             c = 0; tile += p.pos_groups;
             if (tile >= ntiles) break;
             zero_acc();
         }
-        tp16_stage<G, 1, PDT>(acc, a_q, b, bbase, lds, wnext, wbase, wend, wstep);
+        tp16_stage<G, 1, PDT>(acc, a_q, b, bbase, lds, wnext, wbase, wend, wstep, wlane);
         if (++c == nchunks) {
             finish_tile(tile);
             c = 0; tile += p.pos_groups;
@@ -710,7 +716,7 @@ __device__ __forceinline__ void c4_stager(const ConvP16Params& p, unsigned char*
 template <class G, int BUFI>
 __device__ __forceinline__ void c4_stage(f32x4_t (&acc)[2][G::FN], half8_t (&a_q)[PD][2][2], half8_t (&b)[G::FN][2], const int (&bbase)[G::FN],
                                          const int (&off)[G::NS], const unsigned char* lds, const unsigned char*& wnext,
-                                         const unsigned char* wbase, const unsigned char* wend, unsigned wstep) {
+                                         const unsigned char* wbase, const unsigned char* wend, unsigned wstep, unsigned wlane) {
     constexpr int FN = G::FN, NS = G::NS;
     typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
 #pragma unroll
@@ -737,7 +743,7 @@ __device__ __forceinline__ void c4_stage(f32x4_t (&acc)[2][G::FN], half8_t (&a_q
             }
 #pragma unroll
             for (int j = 0; j < 4; j++)
-                if (i == (j * 6 * FN) / 4 + 1) a_q[dprev][j % 2][j / 2] = *reinterpret_cast<const half8_t*>(w_ + ((j % 2) * 2 + j / 2) * 1024);
+                if (i == (j * 6 * FN) / 4 + 1) a_q[dprev][j % 2][j / 2] = *reinterpret_cast<const half8_t*>(w_ + ((j % 2) * 2 + j / 2) * 1024 + wlane);
             __builtin_amdgcn_sched_barrier(0);
         }
     }
@@ -787,7 +793,8 @@ __global__ __launch_bounds__(512) void conv_p16c4_kernel(const ConvP16Params p) 
         off[st] = pi < G::NPAIR ? row * G::ROW_PITCH + col * G::PIX : 0;
     }
     const unsigned wstep = (unsigned)p.mfrags * 2 * 1024;
-    const unsigned char* wbase = reinterpret_cast<const unsigned char*>(p.wpack) + (size_t)(cb * 2 * 2) * 1024 + lane * 16;
+    const unsigned char* wbase = reinterpret_cast<const unsigned char*>(p.wpack) + (size_t)(cb * 2 * 2) * 1024;   // (uniform: the loads take it as their scalar base)
+    const unsigned wlane = lane * 16;
     const unsigned char* wend = wbase + (size_t)NS * wstep;
     half8_t a_q[PD][2][2];
 #pragma unroll
@@ -795,7 +802,7 @@ __global__ __launch_bounds__(512) void conv_p16c4_kernel(const ConvP16Params p) 
 #pragma unroll
         for (int fm = 0; fm < 2; fm++)
 #pragma unroll
-            for (int pl = 0; pl < 2; pl++) a_q[d][fm][pl] = *reinterpret_cast<const half8_t*>(wbase + (size_t)d * wstep + (fm * 2 + pl) * 1024);
+            for (int pl = 0; pl < 2; pl++) a_q[d][fm][pl] = *reinterpret_cast<const half8_t*>(wbase + (size_t)d * wstep + (fm * 2 + pl) * 1024 + wlane);
     f32x4_t acc[2][FN];
     auto zero_acc = [&]() {
 #pragma unroll
@@ -853,12 +860,12 @@ __global__ __launch_bounds__(512) void conv_p16c4_kernel(const ConvP16Params p) 
     const unsigned char* wnext = wbase + (size_t)(PD - 1) * wstep;
     int tile = group;
     for (;;) {
-        c4_stage<G, 0>(acc, a_q, b, bbase, off, lds, wnext, wbase, wend, wstep);
+        c4_stage<G, 0>(acc, a_q, b, bbase, off, lds, wnext, wbase, wend, wstep, wlane);
         finish_tile(tile);
         tile += p.pos_groups;
         if (tile >= ntiles) break;
         zero_acc();
-        c4_stage<G, 1>(acc, a_q, b, bbase, off, lds, wnext, wbase, wend, wstep);
+        c4_stage<G, 1>(acc, a_q, b, bbase, off, lds, wnext, wbase, wend, wstep, wlane);
         finish_tile(tile);
         tile += p.pos_groups;
         if (tile >= ntiles) break;
