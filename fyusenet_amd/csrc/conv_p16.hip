@@ -348,7 +348,8 @@ __global__ __launch_bounds__(512) void conv_p16_kernel(const ConvP16Params p) {
     const float acc_mul = p.acc_mul * inv_in_scale;
     float* out = reinterpret_cast<float*>(p.out);
     const bool have_res = p.res != nullptr;
-    const bool res_relu = p.res_relu != 0, res_scale = p.res_scale != 0;
+    const bool res_scale = p.res_scale != 0;
+    const float res_floor = p.res_relu ? 0.f : -__builtin_inff();
     float vmax = 0.f;
 
     // Epilogue of a tile.  A lane holds, per fragment, output channels 4*kq .. 4*kq+3 of position fn*16 + mq.  One
@@ -357,12 +358,13 @@ __global__ __launch_bounds__(512) void conv_p16_kernel(const ConvP16Params p) {
     auto finish_tile = [&](int tile) {
         const int tyi = (int)(((float)tile + 0.5f) * p.rcp_tiles_x), txi = tile - tyi * p.tiles_x;
         const float* sb = reinterpret_cast<const float*>(lds + sb_off);
-        f32x4_t sc[2], bi[2], scm[2];
+        f32x4_t rs[2], bi[2], scm[2];
 #pragma unroll
         for (int fm = 0; fm < 2; fm++) {
-            sc[fm] = *reinterpret_cast<const f32x4_t*>(sb + mw * 32 + fm * 16 + kq * 4);
+            const f32x4_t sc = *reinterpret_cast<const f32x4_t*>(sb + mw * 32 + fm * 16 + kq * 4);
             bi[fm] = *reinterpret_cast<const f32x4_t*>(sb + CPB + mw * 32 + fm * 16 + kq * 4);
-            scm[fm] = sc[fm] * acc_mul;
+            scm[fm] = sc * acc_mul;
+            rs[fm] = res_scale ? sc : (f32x4_t)(1.f);
         }
 #pragma unroll
         for (int fn = 0; fn < FN; fn++) {
@@ -378,14 +380,10 @@ __global__ __launch_bounds__(512) void conv_p16_kernel(const ConvP16Params p) {
 #pragma unroll
                 for (int e = 0; e < 4; e++) v[e] = acc[fm][fn][e] * scm[fm][e] + bi[fm][e];
                 if (have_res) {
-                    f32x4_t rv = *reinterpret_cast<const f32x4_t*>(lds + res_off + (ty * G::TWG + tx) * G::RES_PITCH + (mw * 32 + fm * 16 + kq * 4) * 4);
+                    // (the two options as operands instead of selects: max(r, 0 or -inf), times scale or 1)
+                    const f32x4_t rv = *reinterpret_cast<const f32x4_t*>(lds + res_off + (ty * G::TWG + tx) * G::RES_PITCH + (mw * 32 + fm * 16 + kq * 4) * 4);
 #pragma unroll
-                    for (int e = 0; e < 4; e++) {
-                        float r = rv[e];
-                        if (res_relu) r = fmaxf(r, 0.f);
-                        if (res_scale) r *= sc[fm][e];
-                        v[e] += r;
-                    }
+                    for (int e = 0; e < 4; e++) v[e] = fmaf(fmaxf(rv[e], res_floor), rs[fm][e], v[e]);
                 }
 #pragma unroll
                 for (int e = 0; e < 4; e++) fmax_ = fmaxf(fmax_, fabsf(v[e]));
