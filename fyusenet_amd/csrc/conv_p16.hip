@@ -617,8 +617,10 @@ __global__ __launch_bounds__(512) void tconv_p16_kernel(const ConvP16Params p) {
 template <int K, int TH_, int TW>
 struct GeoC4 {
     static constexpr int TH = TH_, STEP = 1, WN = 4, TWG = 4 * TW;
-    static constexpr int HW = TWG + K - 1, HH = TH + K - 1;
     static constexpr int PPR = (K + 1) / 2, NPAIR = K * PPR;          // tap pairs per kernel row, in all
+    // (the staged width covers the empty tap that pads an odd kernel row to whole pairs: its weight is zero, but the
+    // pixel it is multiplied with must be a number)
+    static constexpr int HW = TWG + 2 * PPR - 1, HH = TH + K - 1;
     static constexpr int NS = ((NPAIR + 3) / 4 + 2) / 3 * 3;          // steps per stage (two stages are whole turns of the weight ring)
     static constexpr int PIX = 8;                                     // bytes per staged pixel and plane
     static constexpr int ROW_PITCH = (HW * PIX + 15) / 16 * 16 + 16;

@@ -368,6 +368,7 @@ void Net::setup() {
         kv.second->set_up = true;
     }
     assign_range_resets();
+    poison_lds_ = getenv("FYNHIP_POISON_LDS") != nullptr;
     FYN_HIP(hipStreamSynchronize(stream));
     is_setup = true;
 }
@@ -446,6 +447,7 @@ void Net::run_layers(bool with_events) {
             }
             FYN_HIP(hipEventRecord(l->ev0, stream));
         }
+        if (poison_lds_ && launch_poison_lds(stream) != 0) fail(FYN_ERR_DEVICE, "LDS fill failed");
         l->forward(stream);
         FYN_HIP(hipGetLastError());
         if (with_events) FYN_HIP(hipEventRecord(l->ev1, stream));

@@ -170,6 +170,7 @@ class Net {
     hipGraphExec_t graph_exec_ = nullptr;
     bool graph_enabled_ = false;
     bool events_pending_ = false;
+    bool poison_lds_ = false;           // FYNHIP_POISON_LDS: fill the LDS with NaN patterns in front of every layer
 };
 
 Layer* create_layer(Net* net, const fyn_layer_desc& d);

@@ -345,5 +345,6 @@ void launch_tensor_to_chw(const TView& t, float* chw, int include_padding, hipSt
 void launch_hwc_to_tensor(const float* hwc, int pc, const TView& t, hipStream_t s, unsigned* amax = nullptr);   // GPU_SHALLOW in
 void launch_tensor_to_hwc(const TView& t, float* hwc, int pc, hipStream_t s);             // GPU_SHALLOW out
 void launch_fill_zero(void* ptr, size_t bytes, hipStream_t s);
+int launch_poison_lds(hipStream_t s);   // debugging aid: all-ones words into every CU's LDS
 
 }  // namespace fynhip

@@ -1197,6 +1197,22 @@ void launch_fill_zero(void* ptr, size_t bytes, hipStream_t s) {
                        reinterpret_cast<unsigned char*>(ptr) + n16 * 16, bytes - n16 * 16);
 }
 
+// Debugging aid: fills the LDS of every CU with all-ones words (a NaN as fp16 and as fp32, -1 as an integer).  The LDS
+// keeps its contents from one kernel to the next, so a kernel that reads a location it never wrote shows it in its
+// results when this ran just before it.  One workgroup takes a CU's whole LDS; there are several per CU, each busy long
+// enough for the others to land elsewhere.
+__global__ __launch_bounds__(256) void poison_lds_kernel(unsigned words) {
+    extern __shared__ unsigned poison_words[];
+    volatile unsigned* w = poison_words;
+    for (unsigned i = threadIdx.x; i < words; i += 256) w[i] = 0xffffffffu;
+}
+int launch_poison_lds(hipStream_t s) {
+    constexpr size_t bytes = 160 * 1024;
+    if (ensure_lds(reinterpret_cast<const void*>(poison_lds_kernel), bytes) != 0) return -1;
+    hipLaunchKernelGGL(poison_lds_kernel, dim3(1024), dim3(256), bytes, s, (unsigned)(bytes / 4));
+    return hipGetLastError() == hipSuccess ? 0 : -1;
+}
+
 // Second pass of a split-K convolution (see ConvMfmaParams::ksplit): one thread per (position, 4 channels).
 template <typename TOut>
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(const SplitKReduceParams p) {

@@ -8,6 +8,12 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 
+# Every network of the test session fills the LDS of all CUs with NaN patterns in front of each layer (a debugging aid
+# of the library): the LDS keeps its contents between kernels, so a kernel that multiplies a location it never staged
+# with a zero weight passes or fails by what ran before it unless the leftovers are made poisonous.
+os.environ.setdefault("FYNHIP_POISON_LDS", "1")
+
+
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs an MI355X (run with -m gpu on the GPU box)")
 
