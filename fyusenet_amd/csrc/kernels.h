@@ -219,6 +219,14 @@ int conv_p16c4_tile_count();
 void conv_p16c4_tile(int index, int* k, int* th, int* tw, int* steps);
 size_t conv_p16c4_lds_bytes(const ConvP16Params& p, int k);
 int launch_conv_p16c4(const ConvP16Params& p, int k, hipStream_t s);
+// the K x K convolution (K = 3 or 9, stride 1) between fp16 tensors on the same parameters (conv_h16.hip): 128 output
+// channels per workgroup, two tiles of tile_h x tile_w positions side by side; wpack: [(chunk*K + ky)*K + kx][cout
+// fragment of 16][lane][8 halves], one plane
+bool conv_h16_supported(int k, int stride, int dil, int in_cp, int cout, int out_cp, bool f16);
+int conv_h16_tile_count();
+void conv_h16_tile(int index, int* k, int* th, int* tw);
+size_t conv_h16_lds_bytes(const ConvP16Params& p, int k);
+int launch_conv_h16(const ConvP16Params& p, int k, hipStream_t s);
 
 // ---------------------------------------------------------------------------------------------
 // Direct (non-MFMA) layer kernels (layers_direct.hip)

@@ -1043,6 +1043,108 @@ class ConvLayer : public Layer {
             p16_wpack_dev = nullptr;
         }
     }
+    // the fp16-storage form for wide layers (conv_h16.hip): K = 3 or 9, stride 1, blocks of 128 output channels
+    void setup_h16(const TView& in_v, const TView& out_v, const TView* res_v, int res_relu, int res_scale) {
+        ConvP16Params q{};
+        q.in = in_v.ptr; q.out = out_v.ptr; q.res = res_v ? res_v->ptr : nullptr;
+        q.in_hp = in_v.hp(); q.in_wp = in_v.wp(); q.in_cp = in_v.cp;
+        q.stride = 1; q.wm = 2;
+        q.in_y0 = q.in_x0 = in_v.pad - (k - 1) / 2;
+        q.in_clamp = clamp ? 1 : 0;
+        q.npos_y = oh; q.npos_x = ow;
+        q.out_wp = out_v.wp(); q.out_cp = out_v.cp; q.out_off_y = q.out_off_x = out_v.pad;
+        if (res_v) { q.res_wp = res_v->wp(); q.res_cp = res_v->cp; q.res_off_y = q.res_off_x = res_v->pad; }
+        q.res_relu = res_relu; q.res_scale = res_scale;
+        q.cin_chunks = in_v.cp / 32;
+        q.mfrags = oc / 16;
+        q.cout_blocks = oc / 128;
+        q.scale = scale_dev; q.bias = bias_dev;
+        q.acc_mul = 1.f;
+        q.act = act();
+        int want_h = 0, want_w = 0;
+        if (const char* e = getenv("FYNHIP_P16_TILE")) sscanf(e, "%d,%d", &want_h, &want_w);
+        struct Cand { double cost; ConvP16Params q; };
+        std::vector<Cand> cands;
+        for (int i = 0; i < conv_h16_tile_count(); i++) {
+            int kk, th, tw;
+            conv_h16_tile(i, &kk, &th, &tw);
+            if (kk != k || (want_h && (th != want_h || tw != want_w))) continue;
+            ConvP16Params c = q;
+            c.tile_h = th; c.tile_w = tw;
+            c.tiles_x = (ow + 2 * tw - 1) / (2 * tw); c.tiles_y = (oh + th - 1) / th;
+            c.rcp_tiles_x = 1.0f / (float)c.tiles_x;
+            c.pos_groups = std::max(1, std::min(c.tiles_x * c.tiles_y, 256 / c.cout_blocks));
+            if (res_v && c.cin_chunks < 2) c.pos_groups = c.tiles_x * c.tiles_y;   // (residual tile: one stage per tile is too few to walk)
+            const size_t lds = conv_h16_lds_bytes(c, k);
+            if (lds == 0 || lds > 160 * 1024) continue;
+            const int rounds = (c.tiles_x * c.tiles_y * c.cout_blocks + 255) / 256;
+            cands.push_back(Cand{(double)rounds * (th * tw + 4) + 8, c});
+        }
+        if (cands.empty()) return;
+        std::sort(cands.begin(), cands.end(), [](const Cand& a, const Cand& b) { return a.cost < b.cost; });
+        const size_t halves = ((size_t)q.cin_chunks * k * k + 8) * q.mfrags * 64 * 8;
+        p16_wpack_dev = net->dev_alloc(halves * 2, true);
+        for (Cand& c : cands) c.q.wpack = p16_wpack_dev;
+        const bool always = getenv("FYNHIP_FORCE_P16_CONV") != nullptr;
+        const char* at = getenv("FYNHIP_AUTOTUNE");
+        int pick = 0;
+        char key[160];
+        snprintf(key, sizeof(key), "h16:k%d:%dx%d:%dx%d:cp%d:r%d:e%d", k, d.in_channels, oc, oh, ow, in_v.cp, res_v ? 1 : 0, clamp ? 1 : 0);
+        int cached[3] = {0, 0, 0};
+        if (!want_h && tune_cache_triple(key, cached)) {
+            pick = -1;
+            if (cached[0] || always)
+                for (size_t i = 0; i < cands.size(); i++)
+                    if (cands[i].q.tile_h * 1000 + cands[i].q.tile_w == cached[1]) pick = (int)i;
+            if (always && pick < 0) pick = 0;
+        } else if (!(at && at[0] == '0')) {
+            float best = 1e30f, t_other = 1e30f;
+            for (int rep = 0; rep < 2; rep++) {
+                for (size_t i = 0; i < cands.size(); i++) {
+                    const float t = time_calls(net, [&]() {
+                        if (launch_conv_h16(cands[i].q, k, net->stream) != 0) fail(FYN_ERR_DEVICE, "fp16 16-position convolution launch failed while tuning");
+                    }, 5);
+                    if (t < best) { best = t; pick = (int)i; }
+                }
+                t_other = std::min(t_other, time_launch(net, launch, 5));
+            }
+            if (getenv("FYNHIP_TUNE_VERBOSE"))
+                fprintf(stderr, "[tune] %dx%d fp16: 16-position fragments (%dx%d tiles) %.1f us, general kernel %.1f us\n", k, k,
+                        cands[pick].q.tile_h, cands[pick].q.tile_w, best * 1e3f, t_other * 1e3f);
+            const bool win = best < t_other;
+            if (!want_h) tune_cache_store_triple(key, win ? 1 : 0, cands[pick].q.tile_h * 1000 + cands[pick].q.tile_w, 2);
+            if (!win && !always) pick = -1;
+        }
+        if (pick >= 0) {
+            p16 = true; h16 = true;
+            pp = cands[pick].q;
+        } else {
+            net->dev_free(p16_wpack_dev);
+            p16_wpack_dev = nullptr;
+        }
+    }
+    // weights of that form: [(chunk*K + ky)*K + kx][cout fragment of 16][lane][8 halves], zero steps behind the last
+    void pack_h16(const float* w, float wmul) {
+        const int cin = d.in_channels;
+        std::vector<uint16_t> pack(((size_t)pp.cin_chunks * k * k + 8) * pp.mfrags * 64 * 8, 0);
+        for (int chunk = 0; chunk < pp.cin_chunks; chunk++)
+            for (int tap = 0; tap < k * k; tap++)
+                for (int mf = 0; mf < pp.mfrags; mf++) {
+                    uint16_t* base = pack.data() + ((size_t)(chunk * k * k + tap) * pp.mfrags + mf) * 64 * 8;
+                    for (int lane = 0; lane < 64; lane++) {
+                        const int o = mf * 16 + (lane & 15);
+                        if (o >= oc) continue;
+                        for (int j = 0; j < 8; j++) {
+                            const int ci = chunk * 32 + 8 * (lane >> 4) + j;
+                            if (ci >= cin) continue;
+                            base[(size_t)lane * 8 + j] = f2h_bits(w[((size_t)o * k * k + tap) * cin + ci] * wmul);
+                        }
+                    }
+                }
+        FYN_HIP(hipStreamSynchronize(net->stream));
+        FYN_HIP(hipMemcpyAsync(p16_wpack_dev, pack.data(), pack.size() * 2, hipMemcpyHostToDevice, net->stream));
+        FYN_HIP(hipStreamSynchronize(net->stream));
+    }
     // weights of that form: [step][cout fragment of 16][plane][lane][8 halves]; lane = (channel lane%16, tap pair 4*step + lane/16)
     void pack_c4(const float* w, float wmul) {
         const int cin = d.in_channels, ppr = (k + 1) / 2;
@@ -1300,6 +1402,9 @@ class ConvLayer : public Layer {
             if (!frac_shift && !res_v && conv_p16c4_supported(k, stride, dil, in_v.cp, oc, out_v.cp, out_v.f16 != 0) &&
                 !getenv("FYNHIP_NO_P16_CONV"))
                 setup_c4(in_v, out_v);
+            if (!frac_shift && conv_h16_supported(k, stride, dil, in_v.cp, oc, out_v.cp, out_v.f16 != 0) && in_v.f16 && d.in_channels == in_v.cp &&
+                (!res_v || (res_v->cp >= oc && res_v->f16)) && !getenv("FYNHIP_NO_P16_CONV"))
+                setup_h16(in_v, out_v, res_v, res_relu, res_scale);
         }
         if (direct) {
             scale_dev = static_cast<float*>(net->dev_alloc(padded * sizeof(float)));
@@ -1331,6 +1436,7 @@ class ConvLayer : public Layer {
             const float wmul = weight_prescale(w, (size_t)oc * k * k * d.in_channels);
             pp.acc_mul = 1.0f / wmul;
             if (c4) pack_c4(w, wmul);
+            else if (h16) pack_h16(w, wmul);
             else pack_p16(w, wmul);
         } else if (wide && rows) {
             const float wmul = weight_prescale(w, (size_t)oc * k * k * d.in_channels);
@@ -1372,7 +1478,8 @@ class ConvLayer : public Layer {
             return;
         }
         if (p16) {
-            if ((c4 ? launch_conv_p16c4(pp, k, s) : launch_conv_p16(pp, s)) != 0) fail(FYN_ERR_DEVICE, "layer %s: convolution launch failed", d.name);
+            if ((c4 ? launch_conv_p16c4(pp, k, s) : (h16 ? launch_conv_h16(pp, k, s) : launch_conv_p16(pp, s))) != 0)
+                fail(FYN_ERR_DEVICE, "layer %s: convolution launch failed", d.name);
             return;
         }
         if (direct) launch_conv_direct(dp, s);
@@ -1394,6 +1501,13 @@ class ConvLayer : public Layer {
             snprintf(buf, sizeof(buf), "conv_p16c4 f16x2-split (tap pairs of a 4-channel pixel) tile=32x%d(cout x pos) th=%d tw=%d blocks=%d tiles=%d lds=%zu steps=%d",
                      pp.tile_h * pp.tile_w * 4, pp.tile_h, pp.tile_w, pp.pos_groups * pp.cout_blocks, pp.tiles_x * pp.tiles_y * pp.cout_blocks,
                      conv_p16c4_lds_bytes(pp, k), c4_steps);
+            return mode + buf;
+        }
+        if (p16 && h16) {
+            char buf[220];
+            snprintf(buf, sizeof(buf), "conv_h16 f16 tile=128x%d(cout x pos) waves=2x2 th=%d tw=%d blocks=%d tiles=%d lds=%zu steps=%d chunks=%d",
+                     pp.tile_h * pp.tile_w * 2, pp.tile_h, pp.tile_w, pp.pos_groups * pp.cout_blocks, pp.tiles_x * pp.tiles_y * pp.cout_blocks,
+                     conv_h16_lds_bytes(pp, k), k * k, pp.cin_chunks);
             return mode + buf;
         }
         if (p16) {
@@ -1418,6 +1532,7 @@ class ConvLayer : public Layer {
     bool p16 = false;             // 16-position-fragment form of a 3x3 convolution (conv_p16.hip)
     bool c4 = false;              // ... its variant for inputs of at most four channels
     int c4_steps = 0;
+    bool h16 = false;             // ... its fp16-storage form for wide layers (conv_h16.hip)
     ConvP16Params pp{};
     void* p16_wpack_dev = nullptr;
     ConvDirectParams dp{};

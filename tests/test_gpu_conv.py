@@ -307,6 +307,56 @@ def test_sixteen_position_fragment_form(case, act, shallow, monkeypatch):
     assert err <= TOL[fa.STORAGE_F32], info
 
 
+H16_CASES = [
+    # (k, cin, cout, h, w, tile "h,w", kw)
+    (9, 64, 128, 30, 40, "12,8", {}),                                              # two chunks, ragged in both directions
+    (9, 128, 128, 25, 33, "8,8", {"bn": True, "residual": (A.RELU, True)}),
+    (9, 64, 256, 14, 20, "4,8", {"residual": (A.NONE, False)}),                    # two blocks of output channels
+    (9, 96, 128, 24, 32, "12,8", {"bn": True, "pad_out": 2}),                      # whole tiles, three chunks
+    (9, 64, 128, 130, 150, "4,8", {"bn": True, "residual": (A.RELU, False)}),      # 330 tiles: workgroups walk two tiles
+    (9, 128, 128, 60, 70, None, {"residual": (A.NONE, False)}),                    # the engine's own choice of tile
+    (3, 128, 128, 40, 50, "12,8", {"bn": True, "residual": (A.NONE, True)}),
+    (3, 64, 128, 150, 130, "4,8", {"pad_out": 1}),                                 # 342 tiles
+    (3, 32, 128, 66, 68, "4,8", {"residual": (A.RELU, True), "bn": True}),         # one chunk and a residual input: one workgroup per tile
+    (3, 32, 128, 150, 140, "4,8", {"bn": True}),                                   # one chunk, tiles walked: a stage per tile
+    (3, 96, 384, 19, 23, "8,8", {}),                                               # three blocks of output channels
+]
+
+
+@pytest.mark.parametrize("shallow", [False, True], ids=["deep", "shallow_edge_clamp"])
+@pytest.mark.parametrize("act", [A.RELU, A.LEAKY_RELU, A.NONE], ids=["relu", "leaky", "none"])
+@pytest.mark.parametrize("case", H16_CASES, ids=lambda c: "k%d_%dx%dx%d_to%d_%s" % (c[0], c[1], c[3], c[4], c[2], (c[5] or "auto").replace(",", "x")))
+def test_fp16_sixteen_position_fragment_form(case, act, shallow, monkeypatch):
+    """The 3x3 / 9x9 convolution between wide fp16 tensors on 16-position fragments: every compiled tile, ragged edges,
+    tile walking, the residual tile through LDS."""
+    k, cin, cout, h, w, tile, kw = case
+    if shallow and ("residual" in kw or "pad_out" in kw or h > 100):
+        pytest.skip("the shallow variant is run on the plain cases")
+    if act is not A.RELU and ("pad_out" in kw or h > 100 or cout > 128):
+        pytest.skip("activations are varied on some of the cases")
+    monkeypatch.setenv("FYNHIP_FORCE_P16_CONV", "1")
+    if tile:
+        monkeypatch.setenv("FYNHIP_P16_TILE", tile)
+    if shallow:
+        kw = dict(kw, deep=False, pad_in=0)
+    if act is A.LEAKY_RELU:
+        kw = dict(kw, leak=0.1)
+    b = conv_builder(k, cout, h, w, cin, 1, 1, act, **kw)
+    wts = conv_block(2000 + cin + k, cout, k, cin, bn=kw.get("bn", False))
+    inputs = [prng.uniform(43 * cin + h, (cin, h, w), -1, 1)]
+    if "residual" in kw:
+        inputs.append(prng.uniform(59, (cout, h, w), -1, 1))
+    got, info = run_single(b, fa.STORAGE_F16, inputs, wts)
+    ref = oracle_single(b, fa.STORAGE_F16, inputs, wts)
+    err = rel_l2(got, ref)
+    print("  ", info, "rel_l2=%.3e" % err, flush=True)
+    assert "conv_h16" in info
+    if tile:
+        th, tw = tile.split(",")
+        assert "th=%s tw=%s" % (th, tw) in info
+    assert err <= TOL[fa.STORAGE_F16], info
+
+
 ALL_TILES = ["2,2,2,2", "2,2,1,4", "2,1,2,2", "2,1,1,4", "1,2,1,4", "1,1,1,4", "1,1,4,1", "1,1,2,2", "1,2,4,1", "1,3,4,1", "1,4,4,1",
              "1,2,2,2", "1,4,2,2", "1,3,2,2", "1,4,1,4", "1,3,1,4", "1,1,1,1", "1,1,2,1", "1,1,1,2"]
 
