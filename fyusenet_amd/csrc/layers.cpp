@@ -1043,7 +1043,10 @@ class ConvLayer : public Layer {
             p16_wpack_dev = nullptr;
         }
     }
-    // the fp16-storage form for wide layers (conv_h16.hip): K = 3 or 9, stride 1, blocks of 128 output channels
+    // the fp16-storage form for wide layers (conv_h16.hip): K = 3 or 9, stride 1, blocks of 128 output channels.  A
+    // launch takes a whole number of rounds of tiles over the chip's 256 CUs; when the last round of the best single
+    // tile size would be far from full, the image is cut into two bands of rows with different tile heights (two
+    // launches: e.g. 384 rows as three full rounds of 12-row tiles, the remaining 80 as one round of 8-row tiles).
     void setup_h16(const TView& in_v, const TView& out_v, const TView* res_v, int res_relu, int res_scale) {
         ConvP16Params q{};
         q.in = in_v.ptr; q.out = out_v.ptr; q.res = res_v ? res_v->ptr : nullptr;
@@ -1061,63 +1064,105 @@ class ConvLayer : public Layer {
         q.scale = scale_dev; q.bias = bias_dev;
         q.acc_mul = 1.f;
         q.act = act();
-        int want_h = 0, want_w = 0;
+        int want_h = 0, want_w = 0, want_rows1 = 0, want_h2 = 0;   // FYNHIP_P16_TILE=h,w and FYNHIP_H16_SPLIT=rows of the first band,h of the second (tests)
         if (const char* e = getenv("FYNHIP_P16_TILE")) sscanf(e, "%d,%d", &want_h, &want_w);
-        struct Cand { double cost; ConvP16Params q; };
+        if (const char* e = getenv("FYNHIP_H16_SPLIT")) sscanf(e, "%d,%d", &want_rows1, &want_h2);
+        // a band of `rows` output rows from row `row0` on, in tiles of th x tw; cost in MFMA cycles per wave (0: cannot be built)
+        auto band = [&](int th, int tw, int row0, int rows, ConvP16Params* c, double* cost) {
+            *c = q;
+            c->tile_h = th; c->tile_w = tw;
+            c->npos_y = rows;
+            c->in_y0 = q.in_y0 + row0; c->out_off_y = q.out_off_y + row0; c->res_off_y = q.res_off_y + row0;
+            c->tiles_x = (ow + 2 * tw - 1) / (2 * tw); c->tiles_y = (rows + th - 1) / th;
+            c->rcp_tiles_x = 1.0f / (float)c->tiles_x;
+            c->pos_groups = std::max(1, std::min(c->tiles_x * c->tiles_y, 256 / c->cout_blocks));
+            if (res_v && c->cin_chunks < 2) c->pos_groups = c->tiles_x * c->tiles_y;   // (residual tile: one stage per tile is too few to walk)
+            const size_t lds = conv_h16_lds_bytes(*c, k);
+            if (lds == 0 || lds > 160 * 1024) return false;
+            const int rounds = (c->tiles_x * c->tiles_y * c->cout_blocks + 255) / 256;
+            *cost = (double)rounds * ((double)c->cin_chunks * k * k * (th * tw / 16) * 64 + 5000) + 10000;
+            return true;
+        };
+        struct Cand { double cost; ConvP16Params a, b; bool two; };
         std::vector<Cand> cands;
+        std::vector<std::pair<int, int>> tiles;
         for (int i = 0; i < conv_h16_tile_count(); i++) {
             int kk, th, tw;
             conv_h16_tile(i, &kk, &th, &tw);
-            if (kk != k || (want_h && (th != want_h || tw != want_w))) continue;
-            ConvP16Params c = q;
-            c.tile_h = th; c.tile_w = tw;
-            c.tiles_x = (ow + 2 * tw - 1) / (2 * tw); c.tiles_y = (oh + th - 1) / th;
-            c.rcp_tiles_x = 1.0f / (float)c.tiles_x;
-            c.pos_groups = std::max(1, std::min(c.tiles_x * c.tiles_y, 256 / c.cout_blocks));
-            if (res_v && c.cin_chunks < 2) c.pos_groups = c.tiles_x * c.tiles_y;   // (residual tile: one stage per tile is too few to walk)
-            const size_t lds = conv_h16_lds_bytes(c, k);
-            if (lds == 0 || lds > 160 * 1024) continue;
-            const int rounds = (c.tiles_x * c.tiles_y * c.cout_blocks + 255) / 256;
-            cands.push_back(Cand{(double)rounds * (th * tw + 4) + 8, c});
+            if (kk == k) tiles.push_back({th, tw});
+        }
+        for (auto& t : tiles) {
+            if (want_h && (t.first != want_h || t.second != want_w)) continue;
+            Cand c{};
+            if (!want_rows1 && band(t.first, t.second, 0, oh, &c.a, &c.cost)) cands.push_back(c);
+        }
+        // the best cut into two bands (whole tiles of the first band's height above the cut)
+        {
+            Cand best{};
+            best.cost = 1e300;
+            for (auto& t1 : tiles)
+                for (auto& t2 : tiles) {
+                    if (want_h && (t1.first != want_h || t1.second != want_w)) continue;
+                    if (want_h2 && t2.first != want_h2) continue;
+                    for (int rows1 = t1.first; rows1 < oh; rows1 += t1.first) {
+                        if (want_rows1 && rows1 != want_rows1) continue;
+                        Cand c{};
+                        double c1, c2;
+                        if (!band(t1.first, t1.second, 0, rows1, &c.a, &c1) || !band(t2.first, t2.second, rows1, oh - rows1, &c.b, &c2)) continue;
+                        c.cost = c1 + c2;
+                        c.two = true;
+                        if (c.cost < best.cost) best = c;
+                    }
+                }
+            if (best.cost < 1e299) cands.push_back(best);
         }
         if (cands.empty()) return;
         std::sort(cands.begin(), cands.end(), [](const Cand& a, const Cand& b) { return a.cost < b.cost; });
+        if (cands.size() > 3) cands.resize(3);
         const size_t halves = ((size_t)q.cin_chunks * k * k + 8) * q.mfrags * 64 * 8;
         p16_wpack_dev = net->dev_alloc(halves * 2, true);
-        for (Cand& c : cands) c.q.wpack = p16_wpack_dev;
+        for (Cand& c : cands) c.a.wpack = c.b.wpack = p16_wpack_dev;
+        auto run = [&](const Cand& c) {
+            if (launch_conv_h16(c.a, k, net->stream) != 0 || (c.two && launch_conv_h16(c.b, k, net->stream) != 0))
+                fail(FYN_ERR_DEVICE, "fp16 16-position convolution launch failed while tuning");
+        };
+        const bool forced = want_h || want_rows1;
         const bool always = getenv("FYNHIP_FORCE_P16_CONV") != nullptr;
         const char* at = getenv("FYNHIP_AUTOTUNE");
         int pick = 0;
         char key[160];
         snprintf(key, sizeof(key), "h16:k%d:%dx%d:%dx%d:cp%d:r%d:e%d", k, d.in_channels, oc, oh, ow, in_v.cp, res_v ? 1 : 0, clamp ? 1 : 0);
+        // (the cache keeps: chosen?, tile_h*1000 + tile_w of the first band, rows*1000 + tile_h of the second or 0)
+        auto code1 = [](const Cand& c) { return c.a.tile_h * 1000 + c.a.tile_w; };
+        auto code2 = [](const Cand& c) { return c.two ? c.a.npos_y * 1000 + c.b.tile_h : 0; };
         int cached[3] = {0, 0, 0};
-        if (!want_h && tune_cache_triple(key, cached)) {
+        if (!forced && tune_cache_triple(key, cached)) {
             pick = -1;
             if (cached[0] || always)
                 for (size_t i = 0; i < cands.size(); i++)
-                    if (cands[i].q.tile_h * 1000 + cands[i].q.tile_w == cached[1]) pick = (int)i;
+                    if (code1(cands[i]) == cached[1] && code2(cands[i]) == cached[2]) pick = (int)i;
             if (always && pick < 0) pick = 0;
         } else if (!(at && at[0] == '0')) {
             float best = 1e30f, t_other = 1e30f;
             for (int rep = 0; rep < 2; rep++) {
                 for (size_t i = 0; i < cands.size(); i++) {
-                    const float t = time_calls(net, [&]() {
-                        if (launch_conv_h16(cands[i].q, k, net->stream) != 0) fail(FYN_ERR_DEVICE, "fp16 16-position convolution launch failed while tuning");
-                    }, 5);
+                    const float t = time_calls(net, [&]() { run(cands[i]); }, 5);
                     if (t < best) { best = t; pick = (int)i; }
                 }
                 t_other = std::min(t_other, time_launch(net, launch, 5));
             }
             if (getenv("FYNHIP_TUNE_VERBOSE"))
-                fprintf(stderr, "[tune] %dx%d fp16: 16-position fragments (%dx%d tiles) %.1f us, general kernel %.1f us\n", k, k,
-                        cands[pick].q.tile_h, cands[pick].q.tile_w, best * 1e3f, t_other * 1e3f);
+                fprintf(stderr, "[tune] %dx%d fp16: 16-position fragments (%dx%d tiles%s) %.1f us, general kernel %.1f us\n", k, k,
+                        cands[pick].a.tile_h, cands[pick].a.tile_w, cands[pick].two ? ", two bands" : "", best * 1e3f, t_other * 1e3f);
             const bool win = best < t_other;
-            if (!want_h) tune_cache_store_triple(key, win ? 1 : 0, cands[pick].q.tile_h * 1000 + cands[pick].q.tile_w, 2);
+            if (!forced) tune_cache_store_triple(key, win ? 1 : 0, code1(cands[pick]), code2(cands[pick]));
             if (!win && !always) pick = -1;
         }
         if (pick >= 0) {
             p16 = true; h16 = true;
-            pp = cands[pick].q;
+            pp = cands[pick].a;
+            h16_two = cands[pick].two;
+            pp2 = cands[pick].b;
         } else {
             net->dev_free(p16_wpack_dev);
             p16_wpack_dev = nullptr;
@@ -1434,7 +1479,7 @@ class ConvLayer : public Layer {
             reupload(net, wdirect_dev, wd);
         } else if (p16) {
             const float wmul = weight_prescale(w, (size_t)oc * k * k * d.in_channels);
-            pp.acc_mul = 1.0f / wmul;
+            pp.acc_mul = pp2.acc_mul = 1.0f / wmul;
             if (c4) pack_c4(w, wmul);
             else if (h16) pack_h16(w, wmul);
             else pack_p16(w, wmul);
@@ -1478,7 +1523,8 @@ class ConvLayer : public Layer {
             return;
         }
         if (p16) {
-            if ((c4 ? launch_conv_p16c4(pp, k, s) : (h16 ? launch_conv_h16(pp, k, s) : launch_conv_p16(pp, s))) != 0)
+            if ((c4 ? launch_conv_p16c4(pp, k, s) : (h16 ? launch_conv_h16(pp, k, s) : launch_conv_p16(pp, s))) != 0 ||
+                (h16 && h16_two && launch_conv_h16(pp2, k, s) != 0))
                 fail(FYN_ERR_DEVICE, "layer %s: convolution launch failed", d.name);
             return;
         }
@@ -1508,7 +1554,13 @@ class ConvLayer : public Layer {
             snprintf(buf, sizeof(buf), "conv_h16 f16 tile=128x%d(cout x pos) waves=2x2 th=%d tw=%d blocks=%d tiles=%d lds=%zu steps=%d chunks=%d",
                      pp.tile_h * pp.tile_w * 2, pp.tile_h, pp.tile_w, pp.pos_groups * pp.cout_blocks, pp.tiles_x * pp.tiles_y * pp.cout_blocks,
                      conv_h16_lds_bytes(pp, k), k * k, pp.cin_chunks);
-            return mode + buf;
+            std::string info = mode + buf;
+            if (h16_two) {
+                snprintf(buf, sizeof(buf), "; second launch from row %d: th=%d tw=%d blocks=%d tiles=%d lds=%zu", pp.npos_y, pp2.tile_h, pp2.tile_w,
+                         pp2.pos_groups * pp2.cout_blocks, pp2.tiles_x * pp2.tiles_y * pp2.cout_blocks, conv_h16_lds_bytes(pp2, k));
+                info += buf;
+            }
+            return info;
         }
         if (p16) {
             char buf[200];
@@ -1533,7 +1585,8 @@ class ConvLayer : public Layer {
     bool c4 = false;              // ... its variant for inputs of at most four channels
     int c4_steps = 0;
     bool h16 = false;             // ... its fp16-storage form for wide layers (conv_h16.hip)
-    ConvP16Params pp{};
+    bool h16_two = false;         // ...... as two launches on two bands of rows (pp, pp2)
+    ConvP16Params pp{}, pp2{};
     void* p16_wpack_dev = nullptr;
     ConvDirectParams dp{};
     ShiftReduceParams sr{};

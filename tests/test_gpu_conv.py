@@ -320,12 +320,16 @@ H16_CASES = [
     (3, 32, 128, 66, 68, "4,8", {"residual": (A.RELU, True), "bn": True}),         # one chunk and a residual input: one workgroup per tile
     (3, 32, 128, 150, 140, "4,8", {"bn": True}),                                   # one chunk, tiles walked: a stage per tile
     (3, 96, 384, 19, 23, "8,8", {}),                                               # three blocks of output channels
+    # two bands of rows with different tile heights (two launches): "h,w;rows of the first band,h of the second"
+    (9, 64, 128, 44, 30, "12,8;24,8", {"bn": True, "residual": (A.RELU, True)}),
+    (3, 128, 128, 37, 50, "8,8;32,4", {"residual": (A.NONE, False), "pad_out": 1}),
+    (9, 64, 128, 21, 18, "4,8;12,12", {}),
 ]
 
 
 @pytest.mark.parametrize("shallow", [False, True], ids=["deep", "shallow_edge_clamp"])
 @pytest.mark.parametrize("act", [A.RELU, A.LEAKY_RELU, A.NONE], ids=["relu", "leaky", "none"])
-@pytest.mark.parametrize("case", H16_CASES, ids=lambda c: "k%d_%dx%dx%d_to%d_%s" % (c[0], c[1], c[3], c[4], c[2], (c[5] or "auto").replace(",", "x")))
+@pytest.mark.parametrize("case", H16_CASES, ids=lambda c: "k%d_%dx%dx%d_to%d_%s" % (c[0], c[1], c[3], c[4], c[2], (c[5] or "auto").replace(",", "x").replace(";", "_")))
 def test_fp16_sixteen_position_fragment_form(case, act, shallow, monkeypatch):
     """The 3x3 / 9x9 convolution between wide fp16 tensors on 16-position fragments: every compiled tile, ragged edges,
     tile walking, the residual tile through LDS."""
@@ -335,6 +339,10 @@ def test_fp16_sixteen_position_fragment_form(case, act, shallow, monkeypatch):
     if act is not A.RELU and ("pad_out" in kw or h > 100 or cout > 128):
         pytest.skip("activations are varied on some of the cases")
     monkeypatch.setenv("FYNHIP_FORCE_P16_CONV", "1")
+    split = None
+    if tile and ";" in tile:
+        tile, split = tile.split(";")
+        monkeypatch.setenv("FYNHIP_H16_SPLIT", split)
     if tile:
         monkeypatch.setenv("FYNHIP_P16_TILE", tile)
     if shallow:
@@ -354,6 +362,9 @@ def test_fp16_sixteen_position_fragment_form(case, act, shallow, monkeypatch):
     if tile:
         th, tw = tile.split(",")
         assert "th=%s tw=%s" % (th, tw) in info
+    if split:
+        rows1, th2 = split.split(",")
+        assert "second launch from row %s: th=%s" % (rows1, th2) in info
     assert err <= TOL[fa.STORAGE_F16], info
 
 
