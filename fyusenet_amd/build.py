@@ -7,7 +7,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.environ.get("FYNHIP_BUILD_LIB", os.path.join(HERE, "libfynhip.so"))  # experimental builds go elsewhere
 CONV_PARTS = 8  # conv_mfma.hip is compiled this many times, each time with a slice of the tile table
-SOURCES = ["layers_direct.hip", "conv_rows.hip", "conv_p16.hip", "conv_h16.hip", "engine.cpp", "layers.cpp", "api.cpp"]
+SOURCES = ["layers_direct.hip", "conv_rows.hip", "conv_h16.hip", "engine.cpp", "layers.cpp", "api.cpp"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 EXTRA = os.environ.get("FYNHIP_EXTRA_FLAGS", "").split()  # e.g. -D switches of experimental builds
 FLAGS = [
@@ -24,6 +24,8 @@ def build(verbose=True, jobs=8):
     objs = []
     units = [("conv_mfma.hip", "conv_mfma.part%d.o" % i, ["-DFYN_CONV_PARTS=%d" % CONV_PARTS, "-DFYN_CONV_PART=%d" % i])
              for i in range(CONV_PARTS)]
+    # conv_p16.hip once per storage type (fp32 tensors with the host entry points, fp16 tensors)
+    units += [("conv_p16.hip", "conv_p16.f32.o", ["-DFYN_P16_HALF=0"]), ("conv_p16.hip", "conv_p16.f16.o", ["-DFYN_P16_HALF=1"])]
     units += [(src, src + ".o", []) for src in SOURCES]
     for src, objname, defs in units:
         obj = os.path.join(objdir, objname)

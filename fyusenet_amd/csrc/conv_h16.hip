@@ -363,7 +363,8 @@ int launch_conv_h16(const ConvP16Params& p, int k, hipStream_t s) {
     // what the kernel and its grid assume
     if (p.cin_chunks < 1 || p.in_cp < p.cin_chunks * KC || p.mfrags % 8 != 0 || p.cout_blocks * 8 != p.mfrags || p.out_cp < p.cout_blocks * 128 ||
         (p.res && p.res_cp < p.cout_blocks * 128) || (p.res && p.cin_chunks < 2 && p.pos_groups != p.tiles_x * p.tiles_y) ||
-        p.pos_groups < 1 || p.pos_groups > p.tiles_x * p.tiles_y || p.tiles_x < 1 || p.tiles_y < 1 ||
+        p.pos_groups < 1 || p.pos_groups > p.tiles_x * p.tiles_y || p.tiles_x < 1 || p.tiles_y < 1 || !p.f16 ||
+        p.rcp_tiles_x != 1.0f / (float)p.tiles_x || p.tiles_x * p.tiles_y > 4000000 || p.in_cp % 8 != 0 || p.out_cp % 4 != 0 || (p.res && p.res_cp % 8 != 0) ||
         p.tiles_x * 2 * e->tw < p.npos_x || p.tiles_y * e->th < p.npos_y || !p.in || !p.out || !p.wpack || !p.scale || !p.bias)
         return -1;
     const size_t lds = conv_h16_lds_bytes(p, k);

@@ -40,9 +40,21 @@
 
 namespace fynhip {
 
+// The file is compiled twice: for fp32 tensors (operands split into fp16 hi and lo planes, three MFMA passes; this
+// translation unit also holds the host entry points) and, with -DFYN_P16_HALF=1, for fp16 tensors (one plane, one pass).
+#ifndef FYN_P16_HALF
+#define FYN_P16_HALF 0
+#endif
+
 namespace {
 constexpr int NT = 9;         // taps
 constexpr int PD = 6;         // depth of the weight-fragment ring (steps)
+constexpr bool HSTORE = FYN_P16_HALF != 0;   // fp16 tensors
+constexpr int NPL = HSTORE ? 1 : 2;          // staged planes (hi, lo)
+constexpr int NPASS = HSTORE ? 1 : 3;        // MFMAs per fragment pair (hi*hi, lo*hi, hi*lo)
+constexpr int ESZ = HSTORE ? 2 : 4;          // bytes per stored element
+typedef std::conditional<HSTORE, _Float16, float>::type store_t;
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
 
 // Geometry of one instantiation.  A workgroup's four MFMA waves are WM groups of 32 output channels x WN = 4 / WM tiles
 // of TH x TW positions side by side; S is the input step per position (1 or 2).  With S = 2 the staged tile keeps even
@@ -58,13 +70,14 @@ struct Geo {
     static constexpr int SLOTS = (S == 1) ? HW : 2 * HWH;
     static constexpr int ROW_PITCH = SLOTS * PITCH + p16_row_pad(TH, TW, S, WN, SLOTS);
     static constexpr int PLANE = HH * ROW_PITCH;
-    static constexpr int BUF = 2 * PLANE;                // hi, lo
+    static constexpr int BUF = NPL * PLANE;              // hi, lo
     static constexpr int NPOS = TH * TW, FN = NPOS / 16;  // per wave
     static constexpr int NITEMS = HH * HW * (KC / 8);    // staging items: (pixel, 8 channels)
     static constexpr int NB = (NITEMS + 255) / 256;      // ... per staging thread
     static constexpr int CPB = 32 * WM;                  // output channels per workgroup
-    static constexpr int RES_PITCH = CPB * 4 + 16;       // bytes per position of the residual tile
-    static constexpr int RPIECES = TH * TWG * (CPB / 4);  // residual 16-byte pieces
+    static constexpr int RES_PITCH = CPB * ESZ + 16;     // bytes per position of the residual tile
+    static constexpr int RPP = CPB * ESZ / 16;           // 16-byte pieces per position
+    static constexpr int RPIECES = TH * TWG * RPP;       // residual 16-byte pieces
     static constexpr int RNB = (RPIECES + 255) / 256;    // ... per staging thread
     static constexpr int slot_off(int c) { return (S == 1) ? c * PITCH : ((c & 1) * HWH + (c >> 1)) * PITCH; }
     static constexpr int tap_off(int t) { return (t / 3) * ROW_PITCH + slot_off(t % 3); }
@@ -82,7 +95,7 @@ struct Geo {
 // next).  The barrier of a stage sits in its last step, before the first read of the other buffer: the staging waves
 // have filled that buffer by then, and all reads of this stage's buffer were issued a step earlier.
 template <class G, int BUFI>
-__device__ __forceinline__ void p16_stage(f32x4_t (&acc)[2][G::FN], half8_t (&a_q)[PD][2][2], half8_t (&b)[G::FN][2],
+__device__ __forceinline__ void p16_stage(f32x4_t (&acc)[2][G::FN], half8_t (&a_q)[PD][2][NPL], half8_t (&b)[G::FN][NPL],
                                           const int (&bbase)[2][G::FN], const unsigned char* lds, const unsigned char*& wnext,
                                           const unsigned char* wbase, const unsigned char* wend, unsigned wstep, unsigned wlane) {
     constexpr int FN = G::FN;
@@ -93,19 +106,21 @@ __device__ __forceinline__ void p16_stage(f32x4_t (&acc)[2][G::FN], half8_t (&a_
         const unsigned char* w_ = wnext;
         wnext += wstep;
         if (wnext == wend) wnext = wbase;
+        constexpr int SL = 2 * NPASS, NS = SL * FN, NW = 2 * NPL;   // slots per position fragment and per step; weight fragments per step
 #pragma unroll
-        for (int i = 0; i < 6 * FN; i++) {
-            const int fn = i / 6, r = i % 6, kind = r / 2, fm = r % 2;
+        for (int i = 0; i < NS; i++) {
+            const int fn = i / SL, r = i % SL, kind = r / 2, fm = r % 2;
             const int apl = (kind == 1) ? 1 : 0, bpl = (kind == 2) ? 1 : 0;
             acc[fm][fn] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_q[d][fm][apl], b[fn][bpl], acc[fm][fn], 0, 0, 0);
-            if (dd == NT - 1 && i == 3) lds_barrier();
-            if (r == 5) {
-                b[fn][0] = *reinterpret_cast<const half8_t*>(lds + bbase[nbuf][fn] + noff);
-                b[fn][1] = *reinterpret_cast<const half8_t*>(lds + bbase[nbuf][fn] + noff + G::PLANE);
+            if (dd == NT - 1 && i == (SL - 1 < 3 ? SL - 1 : 3)) lds_barrier();   // (ahead of the slot's own fragment read)
+            if (r == SL - 1) {
+#pragma unroll
+                for (int pl = 0; pl < NPL; pl++) b[fn][pl] = *reinterpret_cast<const half8_t*>(lds + bbase[nbuf][fn] + noff + pl * G::PLANE);
             }
 #pragma unroll
-            for (int j = 0; j < 4; j++)   // the four weight fragments of a step, spread over its slots
-                if (i == (j * 6 * FN) / 4 + 1) a_q[dprev][j % 2][j / 2] = *reinterpret_cast<const half8_t*>(w_ + ((j % 2) * 2 + j / 2) * 1024 + wlane);
+            for (int j = 0; j < NW; j++)   // the weight fragments of a step, spread over its slots
+                if (i == ((j * NS) / NW + 1 < NS ? (j * NS) / NW + 1 : NS - 1))
+                    a_q[dprev][j % 2][j / 2] = *reinterpret_cast<const half8_t*>(w_ + ((j % 2) * NPL + j / 2) * 1024 + wlane);
             __builtin_amdgcn_sched_barrier(0);
         }
     }
@@ -121,7 +136,7 @@ __device__ __forceinline__ void p16_stager(const ConvP16Params& p, unsigned char
     constexpr int CPB = G::CPB;
     constexpr int sb_off = 2 * G::BUF;
     constexpr int res_off = sb_off + 2 * CPB * 4;
-    const float* in = reinterpret_cast<const float*>(p.in);
+    const store_t* in = reinterpret_cast<const store_t*>(p.in);
     int i_y[G::NB], i_x[G::NB];   // an item's pixel inside the halo tile (rows above 2^15: no such item)
     int l_off[G::NB];
 #pragma unroll
@@ -139,7 +154,9 @@ __device__ __forceinline__ void p16_stager(const ConvP16Params& p, unsigned char
     // Two sets of staging registers: the loads of stage n+2 are issued before stage n+1 is converted, so a stage's
     // memory latency passes while the stage before it is written to LDS.
     int g_off[2][G::NB];       // element offsets of a set's items, -1: outside the frame (reads as 0)
-    float4 raw[2][G::NB][2];
+    struct RawF { float4 a, b; };
+    typedef typename std::conditional<HSTORE, half8_t, RawF>::type raw_t;   // an item as it comes from memory: 8 channels
+    raw_t raw[2][G::NB];
     float in_scale = 1.f, inv_unused;
     // (unconditional loads: items outside the tensor read its first element and are zeroed when stored)
     auto fetch = [&](auto set_, int tile, int chunk) {
@@ -154,9 +171,13 @@ __device__ __forceinline__ void p16_stager(const ConvP16Params& p, unsigned char
                 gx = min(max(gx, 0), p.in_wp - 1);
             }
             g_off[SET][i] = ((unsigned)gy < (unsigned)p.in_hp && (unsigned)gx < (unsigned)p.in_wp) ? (gy * p.in_wp + gx) * p.in_cp + g8 + chunk * KC : -1;
-            const float* src = in + (g_off[SET][i] >= 0 ? g_off[SET][i] : 0);
-            raw[SET][i][0] = *reinterpret_cast<const float4*>(src);
-            raw[SET][i][1] = *reinterpret_cast<const float4*>(src + 4);
+            const store_t* src = in + (g_off[SET][i] >= 0 ? g_off[SET][i] : 0);
+            if constexpr (HSTORE) {
+                raw[SET][i] = *reinterpret_cast<const half8_t*>(src);
+            } else {
+                raw[SET][i].a = *reinterpret_cast<const float4*>(src);
+                raw[SET][i].b = *reinterpret_cast<const float4*>(src + 4);
+            }
         }
     };
     auto store = [&](auto set_, unsigned char* buf) {
@@ -165,36 +186,43 @@ __device__ __forceinline__ void p16_stager(const ConvP16Params& p, unsigned char
         for (int i = 0; i < G::NB; i++) {
             if (l_off[i] < 0) continue;
             const bool ok = g_off[SET][i] >= 0;
-            const float4 r0 = raw[SET][i][0], r1 = raw[SET][i][1];
-            const float r[8] = {r0.x, r0.y, r0.z, r0.w, r1.x, r1.y, r1.z, r1.w};
-            half8_t hi, lo;
+            if constexpr (HSTORE) {
+                half8_t v;
 #pragma unroll
-            for (int e = 0; e < 8; e++) {
-                const float v = ok ? act_p16(r[e], p.act) * in_scale : 0.f;
-                hi[e] = (_Float16)v;
-                lo[e] = (_Float16)(v - (float)hi[e]);
+                for (int e = 0; e < 8; e++) v[e] = ok ? (_Float16)act_p16((float)raw[SET][i][e], p.act) : (_Float16)0.f;
+                *reinterpret_cast<half8_t*>(buf + l_off[i]) = v;
+            } else {
+                const float4 r0 = raw[SET][i].a, r1 = raw[SET][i].b;
+                const float r[8] = {r0.x, r0.y, r0.z, r0.w, r1.x, r1.y, r1.z, r1.w};
+                half8_t hi, lo;
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    const float v = ok ? act_p16(r[e], p.act) * in_scale : 0.f;
+                    hi[e] = (_Float16)v;
+                    lo[e] = (_Float16)(v - (float)hi[e]);
+                }
+                *reinterpret_cast<half8_t*>(buf + l_off[i]) = hi;
+                *reinterpret_cast<half8_t*>(buf + G::PLANE + l_off[i]) = lo;
             }
-            *reinterpret_cast<half8_t*>(buf + l_off[i]) = hi;
-            *reinterpret_cast<half8_t*>(buf + G::PLANE + l_off[i]) = lo;
         }
     };
-    auto residual_in = [&](int tile) {   // the residual tile of a tile: [position][CPB channels] fp32
-        const float* res = reinterpret_cast<const float*>(p.res);
+    auto residual_in = [&](int tile) {   // the residual tile of a tile: [position][CPB channels] as stored, in 16-byte pieces
+        const store_t* res = reinterpret_cast<const store_t*>(p.res);
         const int tyi = (int)(((float)tile + 0.5f) * p.rcp_tiles_x), txi = tile - tyi * p.tiles_x;
         f32x4_t rv[G::RNB];
 #pragma unroll
         for (int i = 0; i < G::RNB; i++) {
             const int idx = stid + i * 256;
-            const int m = idx / (CPB / 4), c4 = idx % (CPB / 4);
+            const int m = idx / G::RPP, piece = idx % G::RPP;
             const int ty = m / G::TWG, tx = m - ty * G::TWG;
             const int py = tyi * G::TH + ty, px = txi * G::TWG + tx;
             const bool ok = idx < G::RPIECES && py < p.npos_y && px < p.npos_x;
-            rv[i] = *reinterpret_cast<const f32x4_t*>(res + (ok ? ((size_t)(p.res_off_y + py) * p.res_wp + p.res_off_x + px) * p.res_cp + cb * CPB + c4 * 4 : 0));
+            rv[i] = *reinterpret_cast<const f32x4_t*>(res + (ok ? ((size_t)(p.res_off_y + py) * p.res_wp + p.res_off_x + px) * p.res_cp + cb * CPB + piece * (16 / ESZ) : 0));
         }
 #pragma unroll
         for (int i = 0; i < G::RNB; i++) {
             const int idx = stid + i * 256;
-            if (idx < G::RPIECES) *reinterpret_cast<f32x4_t*>(lds + res_off + (idx / (CPB / 4)) * G::RES_PITCH + (idx % (CPB / 4)) * 16) = rv[i];
+            if (idx < G::RPIECES) *reinterpret_cast<f32x4_t*>(lds + res_off + (idx / G::RPP) * G::RES_PITCH + (idx % G::RPP) * 16) = rv[i];
         }
     };
     // the stage after (tile, c); false: there is none
@@ -289,17 +317,17 @@ __global__ __launch_bounds__(512) void conv_p16_kernel(const ConvP16Params p) {
         bbase[1][fn] = bbase[0][fn] + G::BUF;
     }
     // A fragments: [(chunk*9 + tap)][cout fragment of 16][plane][lane] x 8 halves
-    const unsigned wstep = (unsigned)p.mfrags * 2 * 1024;
-    const unsigned char* wbase = reinterpret_cast<const unsigned char*>(p.wpack) + (size_t)((cb * 2 * WM + mw * 2) * 2) * 1024;   // (uniform: the loads take it as their scalar base)
+    const unsigned wstep = (unsigned)p.mfrags * NPL * 1024;
+    const unsigned char* wbase = reinterpret_cast<const unsigned char*>(p.wpack) + (size_t)((cb * 2 * WM + mw * 2) * NPL) * 1024;   // (uniform: the loads take it as their scalar base)
     const unsigned wlane = lane * 16;
     const unsigned char* wend = wbase + (size_t)nchunks * NT * wstep;
-    half8_t a_q[PD][2][2];
+    half8_t a_q[PD][2][NPL];
 #pragma unroll
     for (int d = 0; d < PD; d++)
 #pragma unroll
         for (int fm = 0; fm < 2; fm++)
 #pragma unroll
-            for (int pl = 0; pl < 2; pl++) a_q[d][fm][pl] = *reinterpret_cast<const half8_t*>(wbase + (size_t)d * wstep + (fm * 2 + pl) * 1024 + wlane);
+            for (int pl = 0; pl < NPL; pl++) a_q[d][fm][pl] = *reinterpret_cast<const half8_t*>(wbase + (size_t)d * wstep + (fm * NPL + pl) * 1024 + wlane);
     f32x4_t acc[2][FN];
     auto zero_acc = [&]() {
 #pragma unroll
@@ -311,7 +339,7 @@ __global__ __launch_bounds__(512) void conv_p16_kernel(const ConvP16Params p) {
     float inv_in_scale = 1.f;
     if (p.in_amax) (void)range_scale(range_after_act(range_reduce(range_bits), p.act), &inv_in_scale);
     const float acc_mul = p.acc_mul * inv_in_scale;
-    float* out = reinterpret_cast<float*>(p.out);
+    store_t* out = reinterpret_cast<store_t*>(p.out);
     const bool have_res = p.res != nullptr;
     const bool res_scale = p.res_scale != 0;
     const float res_floor = p.res_relu ? 0.f : -__builtin_inff();
@@ -346,13 +374,28 @@ __global__ __launch_bounds__(512) void conv_p16_kernel(const ConvP16Params p) {
                 for (int e = 0; e < 4; e++) v[e] = acc[fm][fn][e] * scm[fm][e] + bi[fm][e];
                 if (have_res) {
                     // (the two options as operands instead of selects: max(r, 0 or -inf), times scale or 1)
-                    const f32x4_t rv = *reinterpret_cast<const f32x4_t*>(lds + res_off + (ty * G::TWG + tx) * G::RES_PITCH + (mw * 32 + fm * 16 + kq * 4) * 4);
+                    const unsigned char* rsrc = lds + res_off + (ty * G::TWG + tx) * G::RES_PITCH + (mw * 32 + fm * 16 + kq * 4) * ESZ;
+                    f32x4_t rv;
+                    if constexpr (HSTORE) {
+                        const half4_t rh = *reinterpret_cast<const half4_t*>(rsrc);
+#pragma unroll
+                        for (int e = 0; e < 4; e++) rv[e] = (float)rh[e];
+                    } else {
+                        rv = *reinterpret_cast<const f32x4_t*>(rsrc);
+                    }
 #pragma unroll
                     for (int e = 0; e < 4; e++) v[e] = fmaf(fmaxf(rv[e], res_floor), rs[fm][e], v[e]);
                 }
+                if constexpr (HSTORE) {
+                    half4_t hv;
 #pragma unroll
-                for (int e = 0; e < 4; e++) fmax_ = fmaxf(fmax_, fabsf(v[e]));
-                if (ok) *reinterpret_cast<f32x4_t*>(out + obase + fm * 16) = v;
+                    for (int e = 0; e < 4; e++) hv[e] = (_Float16)v[e];
+                    if (ok) *reinterpret_cast<half4_t*>(out + obase + fm * 16) = hv;
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; e++) fmax_ = fmaxf(fmax_, fabsf(v[e]));
+                    if (ok) *reinterpret_cast<f32x4_t*>(out + obase + fm * 16) = v;
+                }
             }
             vmax = fmaxf(vmax, ok ? fmax_ : 0.f);
         }
@@ -361,11 +404,11 @@ __global__ __launch_bounds__(512) void conv_p16_kernel(const ConvP16Params p) {
     FYN_PTRACE(1);
     lds_barrier();   // the first stage is staged
     FYN_PTRACE(2);
-    half8_t b[FN][2];
+    half8_t b[FN][NPL];
 #pragma unroll
     for (int fn = 0; fn < FN; fn++)
 #pragma unroll
-        for (int pl = 0; pl < 2; pl++) b[fn][pl] = *reinterpret_cast<const half8_t*>(lds + bbase[0][fn] + pl * G::PLANE);
+        for (int pl = 0; pl < NPL; pl++) b[fn][pl] = *reinterpret_cast<const half8_t*>(lds + bbase[0][fn] + pl * G::PLANE);
 
     const unsigned char* wnext = wbase + (size_t)((PD - 1) % (nchunks * NT)) * wstep;
     int tile = group, c = 0;
@@ -412,7 +455,7 @@ constexpr bool tt_last_of_shift(int t) { return t == NT - 1 || tt_shift(t + 1) !
 // (PDT: depth of the weight ring; three position fragments per wave leave room for three steps only, which at 288 cycles
 // per step still covers an L2 round trip)
 template <class G, int BUFI, int PDT>
-__device__ __forceinline__ void tp16_stage(f32x4_t (&acc)[4][2][G::FN], half8_t (&a_q)[PDT][2][2], half8_t (&b)[2][G::FN][2],
+__device__ __forceinline__ void tp16_stage(f32x4_t (&acc)[4][2][G::FN], half8_t (&a_q)[PDT][2][NPL], half8_t (&b)[2][G::FN][NPL],
                                            const int (&bbase)[2][G::FN], const unsigned char* lds, const unsigned char*& wnext,
                                            const unsigned char* wbase, const unsigned char* wend, unsigned wstep, unsigned wlane) {
     constexpr int FN = G::FN;
@@ -423,23 +466,26 @@ __device__ __forceinline__ void tp16_stage(f32x4_t (&acc)[4][2][G::FN], half8_t 
         const int nsh = (sh + 1) & 3, nbuf = (t == NT - 1) ? 1 - BUFI : BUFI;
         // the tile is staged with one pixel of halo above and to the left: shift (dy, dx) reads pixel (1-dy, 1-dx) + position
         const int noff = (1 - (nsh >> 1)) * G::ROW_PITCH + (1 - (nsh & 1)) * PITCH;
-        const int first_read = (t == NT - 1) ? 4 : 0;   // (the stage's barrier sits in slot 3 of its last step)
+        constexpr int SL = 2 * NPASS, NS = SL * FN, NW = 2 * NPL;
+        constexpr int BAR = HSTORE ? 0 : 3;             // the slot of the stage's barrier in its last step
+        const int first_read = (t == NT - 1) ? BAR + 1 : 0;
         const unsigned char* w_ = wnext;
         wnext += wstep;
         if (wnext == wend) wnext = wbase;
 #pragma unroll
-        for (int i = 0; i < 6 * FN; i++) {
-            const int fn = i / 6, r = i % 6, kind = r / 2, fm = r % 2;
+        for (int i = 0; i < NS; i++) {
+            const int fn = i / SL, r = i % SL, kind = r / 2, fm = r % 2;
             const int apl = (kind == 1) ? 1 : 0, bpl = (kind == 2) ? 1 : 0;
             acc[par][fm][fn] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_q[d][fm][apl], b[set][fn][bpl], acc[par][fm][fn], 0, 0, 0);
-            if (t == NT - 1 && i == 3) lds_barrier();
-            if (tt_last_of_shift(t) && i >= first_read && i < first_read + 2 * FN) {
+            if (t == NT - 1 && i == BAR) lds_barrier();
+            if (tt_last_of_shift(t) && i >= first_read && i < first_read + NPL * FN) {
                 const int j = i - first_read;
-                b[1 - set][j / 2][j % 2] = *reinterpret_cast<const half8_t*>(lds + bbase[nbuf][j / 2] + noff + (j % 2) * G::PLANE);
+                b[1 - set][j / NPL][j % NPL] = *reinterpret_cast<const half8_t*>(lds + bbase[nbuf][j / NPL] + noff + (j % NPL) * G::PLANE);
             }
 #pragma unroll
-            for (int j = 0; j < 4; j++)   // the four weight fragments of a step, spread over its slots
-                if (i == (j * 6 * FN) / 4 + 1) a_q[dprev][j % 2][j / 2] = *reinterpret_cast<const half8_t*>(w_ + ((j % 2) * 2 + j / 2) * 1024 + wlane);
+            for (int j = 0; j < NW; j++)   // the weight fragments of a step, spread over its slots
+                if (i == ((j * NS) / NW + 1 < NS ? (j * NS) / NW + 1 : NS - 1))
+                    a_q[dprev][j % 2][j / 2] = *reinterpret_cast<const half8_t*>(w_ + ((j % 2) * NPL + j / 2) * 1024 + wlane);
             __builtin_amdgcn_sched_barrier(0);
         }
     }
@@ -451,7 +497,7 @@ __global__ __launch_bounds__(512) void tconv_p16_kernel(const ConvP16Params p) {
     constexpr int FN = G::FN, CPB = G::CPB;
     constexpr int PDT = (FN >= 3) ? 3 : 6;
     static_assert((2 * NT) % PDT == 0, "two stages are whole turns of the weight ring");
-    static_assert(6 * FN >= 4 + 2 * FN, "the last step of a stage has room for the next stage's first fragments");
+    static_assert(2 * NPASS * FN >= (HSTORE ? 1 : 4) + NPL * FN, "the last step of a stage has room for the next stage's first fragments");
     extern __shared__ __align__(16) unsigned char lds[];
     __shared__ unsigned range_box[2];
     if (blockIdx.x == 0) range_clear(p.reset[0], p.reset[1], p.reset[2], p.reset[3], p.nreset);
@@ -485,17 +531,17 @@ __global__ __launch_bounds__(512) void tconv_p16_kernel(const ConvP16Params p) {
         bbase[0][fn] = ty * G::ROW_PITCH + (wn * TW + tx) * PITCH + kq * 16;
         bbase[1][fn] = bbase[0][fn] + G::BUF;
     }
-    const unsigned wstep = (unsigned)p.mfrags * 2 * 1024;
-    const unsigned char* wbase = reinterpret_cast<const unsigned char*>(p.wpack) + (size_t)((cb * 2 * WM + mw * 2) * 2) * 1024;   // (uniform: the loads take it as their scalar base)
+    const unsigned wstep = (unsigned)p.mfrags * NPL * 1024;
+    const unsigned char* wbase = reinterpret_cast<const unsigned char*>(p.wpack) + (size_t)((cb * 2 * WM + mw * 2) * NPL) * 1024;   // (uniform: the loads take it as their scalar base)
     const unsigned wlane = lane * 16;
     const unsigned char* wend = wbase + (size_t)nchunks * NT * wstep;
-    half8_t a_q[PDT][2][2];
+    half8_t a_q[PDT][2][NPL];
 #pragma unroll
     for (int d = 0; d < PDT; d++)
 #pragma unroll
         for (int fm = 0; fm < 2; fm++)
 #pragma unroll
-            for (int pl = 0; pl < 2; pl++) a_q[d][fm][pl] = *reinterpret_cast<const half8_t*>(wbase + (size_t)d * wstep + (fm * 2 + pl) * 1024 + wlane);
+            for (int pl = 0; pl < NPL; pl++) a_q[d][fm][pl] = *reinterpret_cast<const half8_t*>(wbase + (size_t)d * wstep + (fm * NPL + pl) * 1024 + wlane);
     f32x4_t acc[4][2][FN];
     auto zero_acc = [&]() {
 #pragma unroll
@@ -509,7 +555,7 @@ __global__ __launch_bounds__(512) void tconv_p16_kernel(const ConvP16Params p) {
     float inv_in_scale = 1.f;
     if (p.in_amax) (void)range_scale(range_after_act(range_reduce(range_bits), p.act), &inv_in_scale);
     const float acc_mul = p.acc_mul * inv_in_scale;
-    float* out = reinterpret_cast<float*>(p.out);
+    store_t* out = reinterpret_cast<store_t*>(p.out);
     float vmax = 0.f;
     auto finish_tile = [&](int tile) {
         const int tyi = (int)(((float)tile + 0.5f) * p.rcp_tiles_x), txi = tile - tyi * p.tiles_x;
@@ -537,20 +583,27 @@ __global__ __launch_bounds__(512) void tconv_p16_kernel(const ConvP16Params p) {
 #pragma unroll
                     for (int e = 0; e < 4; e++) {
                         v[e] = acc[par][fm][fn][e] * scm[fm][e] + bi[fm][e];
-                        fmax_ = fmaxf(fmax_, fabsf(v[e]));
+                        if constexpr (!HSTORE) fmax_ = fmaxf(fmax_, fabsf(v[e]));
                     }
-                    if (ok) *reinterpret_cast<f32x4_t*>(out + o + fm * 16) = v;
+                    if constexpr (HSTORE) {
+                        half4_t hv;
+#pragma unroll
+                        for (int e = 0; e < 4; e++) hv[e] = (_Float16)v[e];
+                        if (ok) *reinterpret_cast<half4_t*>(out + o + fm * 16) = hv;
+                    } else {
+                        if (ok) *reinterpret_cast<f32x4_t*>(out + o + fm * 16) = v;
+                    }
                 }
             }
             vmax = fmaxf(vmax, ok ? fmax_ : 0.f);
         }
     };
     lds_barrier();   // the first stage is staged
-    half8_t b[2][FN][2];
+    half8_t b[2][FN][NPL];
 #pragma unroll
     for (int fn = 0; fn < FN; fn++)
 #pragma unroll
-        for (int pl = 0; pl < 2; pl++) b[0][fn][pl] = *reinterpret_cast<const half8_t*>(lds + bbase[0][fn] + G::ROW_PITCH + PITCH + pl * G::PLANE);
+        for (int pl = 0; pl < NPL; pl++) b[0][fn][pl] = *reinterpret_cast<const half8_t*>(lds + bbase[0][fn] + G::ROW_PITCH + PITCH + pl * G::PLANE);
     const unsigned char* wnext = wbase + (size_t)((PDT - 1) % (nchunks * NT)) * wstep;
     int tile = group, c = 0;
     for (;;) {
@@ -590,7 +643,7 @@ struct GeoC4 {
     static constexpr int PIX = 8;                                     // bytes per staged pixel and plane
     static constexpr int ROW_PITCH = (HW * PIX + 15) / 16 * 16 + 16;
     static constexpr int PLANE = HH * ROW_PITCH;
-    static constexpr int BUF = 2 * PLANE;
+    static constexpr int BUF = NPL * PLANE;
     static constexpr int NPOS = TH * TW, FN = NPOS / 16;
     static constexpr int NITEMS = HH * HW;                            // staging items: pixels
     static constexpr int NB = (NITEMS + 255) / 256;
@@ -602,7 +655,7 @@ struct GeoC4 {
 template <class G>
 __device__ __forceinline__ void c4_stager(const ConvP16Params& p, unsigned char* lds, int stid, int cb, int group, int ntiles, unsigned range_bits) {
     constexpr int sb_off = 2 * G::BUF;
-    const float* in = reinterpret_cast<const float*>(p.in);
+    const store_t* in = reinterpret_cast<const store_t*>(p.in);
     int i_y[G::NB], i_x[G::NB], l_off[G::NB];
 #pragma unroll
     for (int i = 0; i < G::NB; i++) {
@@ -615,7 +668,8 @@ __device__ __forceinline__ void c4_stager(const ConvP16Params& p, unsigned char*
         }
     }
     int g_off[2][G::NB];
-    float4 raw[2][G::NB];
+    typedef typename std::conditional<HSTORE, half4_t, float4>::type raw_t;   // a pixel as it comes from memory
+    raw_t raw[2][G::NB];
     float in_scale = 1.f, inv_unused;
     auto fetch = [&](auto set_, int tile) {
         constexpr int SET = decltype(set_)::value;
@@ -629,26 +683,32 @@ __device__ __forceinline__ void c4_stager(const ConvP16Params& p, unsigned char*
                 gx = min(max(gx, 0), p.in_wp - 1);
             }
             g_off[SET][i] = ((unsigned)gy < (unsigned)p.in_hp && (unsigned)gx < (unsigned)p.in_wp) ? (gy * p.in_wp + gx) * 4 : -1;
-            raw[SET][i] = *reinterpret_cast<const float4*>(in + (g_off[SET][i] >= 0 ? g_off[SET][i] : 0));
+            raw[SET][i] = *reinterpret_cast<const raw_t*>(in + (g_off[SET][i] >= 0 ? g_off[SET][i] : 0));
         }
     };
     auto store = [&](auto set_, unsigned char* buf) {
         constexpr int SET = decltype(set_)::value;
-        typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
 #pragma unroll
         for (int i = 0; i < G::NB; i++) {
             if (l_off[i] < 0) continue;
             const bool ok = g_off[SET][i] >= 0;
-            const float r[4] = {raw[SET][i].x, raw[SET][i].y, raw[SET][i].z, raw[SET][i].w};
-            half4_t hi, lo;
+            if constexpr (HSTORE) {
+                half4_t v;
 #pragma unroll
-            for (int e = 0; e < 4; e++) {
-                const float v = ok ? act_p16(r[e], p.act) * in_scale : 0.f;
-                hi[e] = (_Float16)v;
-                lo[e] = (_Float16)(v - (float)hi[e]);
+                for (int e = 0; e < 4; e++) v[e] = ok ? (_Float16)act_p16((float)raw[SET][i][e], p.act) : (_Float16)0.f;
+                *reinterpret_cast<half4_t*>(buf + l_off[i]) = v;
+            } else {
+                const float r[4] = {raw[SET][i].x, raw[SET][i].y, raw[SET][i].z, raw[SET][i].w};
+                half4_t hi, lo;
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    const float v = ok ? act_p16(r[e], p.act) * in_scale : 0.f;
+                    hi[e] = (_Float16)v;
+                    lo[e] = (_Float16)(v - (float)hi[e]);
+                }
+                *reinterpret_cast<half4_t*>(buf + l_off[i]) = hi;
+                *reinterpret_cast<half4_t*>(buf + G::PLANE + l_off[i]) = lo;
             }
-            *reinterpret_cast<half4_t*>(buf + l_off[i]) = hi;
-            *reinterpret_cast<half4_t*>(buf + G::PLANE + l_off[i]) = lo;
         }
     };
     typedef std::integral_constant<int, 0> Set0;
@@ -679,11 +739,10 @@ __device__ __forceinline__ void c4_stager(const ConvP16Params& p, unsigned char*
 }
 
 template <class G, int BUFI>
-__device__ __forceinline__ void c4_stage(f32x4_t (&acc)[2][G::FN], half8_t (&a_q)[PD][2][2], half8_t (&b)[G::FN][2], const int (&bbase)[G::FN],
+__device__ __forceinline__ void c4_stage(f32x4_t (&acc)[2][G::FN], half8_t (&a_q)[PD][2][NPL], half8_t (&b)[G::FN][NPL], const int (&bbase)[G::FN],
                                          const int (&off)[G::NS], const unsigned char* lds, const unsigned char*& wnext,
                                          const unsigned char* wbase, const unsigned char* wend, unsigned wstep, unsigned wlane) {
     constexpr int FN = G::FN, NS = G::NS;
-    typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
 #pragma unroll
     for (int dd = 0; dd < NS; dd++) {
         const int d = (BUFI * NS + dd) % PD, dprev = (d + PD - 1) % PD;
@@ -691,24 +750,26 @@ __device__ __forceinline__ void c4_stage(f32x4_t (&acc)[2][G::FN], half8_t (&a_q
         const unsigned char* w_ = wnext;
         wnext += wstep;
         if (wnext == wend) wnext = wbase;
+        constexpr int SL = 2 * NPASS, NSL = SL * FN, NW = 2 * NPL;
 #pragma unroll
-        for (int i = 0; i < 6 * FN; i++) {
-            const int fn = i / 6, r = i % 6, kind = r / 2, fm = r % 2;
+        for (int i = 0; i < NSL; i++) {
+            const int fn = i / SL, r = i % SL, kind = r / 2, fm = r % 2;
             const int apl = (kind == 1) ? 1 : 0, bpl = (kind == 2) ? 1 : 0;
             acc[fm][fn] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_q[d][fm][apl], b[fn][bpl], acc[fm][fn], 0, 0, 0);
-            if (dd == NS - 1 && i == 3) lds_barrier();
-            if (r == 5) {
+            if (dd == NS - 1 && i == (SL - 1 < 3 ? SL - 1 : 3)) lds_barrier();
+            if (r == SL - 1) {
                 const unsigned char* src = lds + nbuf * G::BUF + bbase[fn] + off[ns];
 #pragma unroll
-                for (int pl = 0; pl < 2; pl++) {
+                for (int pl = 0; pl < NPL; pl++) {
                     const half4_t t0 = *reinterpret_cast<const half4_t*>(src + pl * G::PLANE);
                     const half4_t t1 = *reinterpret_cast<const half4_t*>(src + pl * G::PLANE + G::PIX);
                     b[fn][pl] = half8_t{t0[0], t0[1], t0[2], t0[3], t1[0], t1[1], t1[2], t1[3]};
                 }
             }
 #pragma unroll
-            for (int j = 0; j < 4; j++)
-                if (i == (j * 6 * FN) / 4 + 1) a_q[dprev][j % 2][j / 2] = *reinterpret_cast<const half8_t*>(w_ + ((j % 2) * 2 + j / 2) * 1024 + wlane);
+            for (int j = 0; j < NW; j++)
+                if (i == ((j * NSL) / NW + 1 < NSL ? (j * NSL) / NW + 1 : NSL - 1))
+                    a_q[dprev][j % 2][j / 2] = *reinterpret_cast<const half8_t*>(w_ + ((j % 2) * NPL + j / 2) * 1024 + wlane);
             __builtin_amdgcn_sched_barrier(0);
         }
     }
@@ -718,7 +779,6 @@ template <int K, int TH, int TW>
 __global__ __launch_bounds__(512) void conv_p16c4_kernel(const ConvP16Params p) {
     using G = GeoC4<K, TH, TW>;
     constexpr int FN = G::FN, NS = G::NS;
-    typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
     extern __shared__ __align__(16) unsigned char lds[];
     __shared__ unsigned range_box[2];
     if (blockIdx.x == 0) range_clear(p.reset[0], p.reset[1], p.reset[2], p.reset[3], p.nreset);
@@ -757,17 +817,17 @@ __global__ __launch_bounds__(512) void conv_p16c4_kernel(const ConvP16Params p) 
         const int row = pi / G::PPR, col = 2 * (pi - row * G::PPR);
         off[st] = pi < G::NPAIR ? row * G::ROW_PITCH + col * G::PIX : 0;
     }
-    const unsigned wstep = (unsigned)p.mfrags * 2 * 1024;
-    const unsigned char* wbase = reinterpret_cast<const unsigned char*>(p.wpack) + (size_t)(cb * 2 * 2) * 1024;   // (uniform: the loads take it as their scalar base)
+    const unsigned wstep = (unsigned)p.mfrags * NPL * 1024;
+    const unsigned char* wbase = reinterpret_cast<const unsigned char*>(p.wpack) + (size_t)(cb * 2 * NPL) * 1024;   // (uniform: the loads take it as their scalar base)
     const unsigned wlane = lane * 16;
     const unsigned char* wend = wbase + (size_t)NS * wstep;
-    half8_t a_q[PD][2][2];
+    half8_t a_q[PD][2][NPL];
 #pragma unroll
     for (int d = 0; d < PD; d++)
 #pragma unroll
         for (int fm = 0; fm < 2; fm++)
 #pragma unroll
-            for (int pl = 0; pl < 2; pl++) a_q[d][fm][pl] = *reinterpret_cast<const half8_t*>(wbase + (size_t)d * wstep + (fm * 2 + pl) * 1024 + wlane);
+            for (int pl = 0; pl < NPL; pl++) a_q[d][fm][pl] = *reinterpret_cast<const half8_t*>(wbase + (size_t)d * wstep + (fm * NPL + pl) * 1024 + wlane);
     f32x4_t acc[2][FN];
     auto zero_acc = [&]() {
 #pragma unroll
@@ -779,7 +839,7 @@ __global__ __launch_bounds__(512) void conv_p16c4_kernel(const ConvP16Params p) 
     float inv_in_scale = 1.f;
     if (p.in_amax) (void)range_scale(range_after_act(range_reduce(range_bits), p.act), &inv_in_scale);
     const float acc_mul = p.acc_mul * inv_in_scale;
-    float* out = reinterpret_cast<float*>(p.out);
+    store_t* out = reinterpret_cast<store_t*>(p.out);
     float vmax = 0.f;
     auto finish_tile = [&](int tile) {
         const int tyi = (int)(((float)tile + 0.5f) * p.rcp_tiles_x), txi = tile - tyi * p.tiles_x;
@@ -804,19 +864,26 @@ __global__ __launch_bounds__(512) void conv_p16c4_kernel(const ConvP16Params p) 
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
                     v[e] = acc[fm][fn][e] * scm[fm][e] + bi[fm][e];
-                    fmax_ = fmaxf(fmax_, fabsf(v[e]));
+                    if constexpr (!HSTORE) fmax_ = fmaxf(fmax_, fabsf(v[e]));
                 }
-                if (ok) *reinterpret_cast<f32x4_t*>(out + obase + fm * 16) = v;
+                if constexpr (HSTORE) {
+                    half4_t hv;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) hv[e] = (_Float16)v[e];
+                    if (ok) *reinterpret_cast<half4_t*>(out + obase + fm * 16) = hv;
+                } else {
+                    if (ok) *reinterpret_cast<f32x4_t*>(out + obase + fm * 16) = v;
+                }
             }
             vmax = fmaxf(vmax, ok ? fmax_ : 0.f);
         }
     };
     lds_barrier();   // the first stage is staged
-    half8_t b[FN][2];
+    half8_t b[FN][NPL];
 #pragma unroll
     for (int fn = 0; fn < FN; fn++)
 #pragma unroll
-        for (int pl = 0; pl < 2; pl++) {
+        for (int pl = 0; pl < NPL; pl++) {
             const unsigned char* src = lds + bbase[fn] + off[0] + pl * G::PLANE;
             const half4_t t0 = *reinterpret_cast<const half4_t*>(src);
             const half4_t t1 = *reinterpret_cast<const half4_t*>(src + G::PIX);
@@ -855,7 +922,7 @@ const P16Entry kEntries[] = {
     entry<10, 8, 2, 4>(), entry<8, 10, 2, 4>(), entry<8, 8, 2, 4>(),
     entry<8, 6, 2, 2>(), entry<4, 8, 2, 2>(), entry<8, 4, 2, 2>(),
 };
-size_t entry_lds(const P16Entry& e, bool residual) {
+size_t entry_lds(const P16Entry& e, bool residual) {   // (e.buf and e.res_bytes are this translation unit's: they depend on the storage type)
     return 2 * e.buf + 2 * (size_t)(32 * e.wm) * 4 + (residual ? e.res_bytes : 0);
 }
 struct TP16Entry {
@@ -882,32 +949,71 @@ constexpr C4Entry c4entry() { return C4Entry{K, TH, TW, conv_p16c4_kernel<K, TH,
 const C4Entry kC4Entries[] = {c4entry<9, 8, 8>(), c4entry<9, 4, 8>(), c4entry<9, 8, 4>()};
 }  // namespace
 
+// Host entry points.  The fp32 unit holds the public ones and hands launches on fp16 tensors (p.f16) to the other
+// unit's, which carry the suffix _half; tile tables are the same in both.
+#if FYN_P16_HALF
+#define P16_NAME(n) n##_half
+#else
+#define P16_NAME(n) n
+size_t conv_p16_lds_bytes_half(const ConvP16Params& p);
+int launch_conv_p16_half(const ConvP16Params& p, hipStream_t s);
+size_t tconv_p16_lds_bytes_half(const ConvP16Params& p);
+int launch_tconv_p16_half(const ConvP16Params& p, hipStream_t s);
+size_t conv_p16c4_lds_bytes_half(const ConvP16Params& p, int k);
+int launch_conv_p16c4_half(const ConvP16Params& p, int k, hipStream_t s);
+
 int conv_p16_tile_count() { return (int)(sizeof(kEntries) / sizeof(kEntries[0])); }
 void conv_p16_tile(int index, int* th, int* tw, int* stride, int* wm) {
     *th = kEntries[index].th; *tw = kEntries[index].tw; *stride = kEntries[index].stride; *wm = kEntries[index].wm;
 }
+bool conv_p16_supported(int k, int stride, int dil, int in_cp, int cout, int out_cp, bool f16) {
+    (void)f16;   // (both storage types; 16-byte loads and 8- or 16-byte stores hold for any pitch that is a multiple of 32 / 4)
+    return k == 3 && (stride == 1 || stride == 2) && dil == 1 && in_cp % KC == 0 && cout % 64 == 0 && out_cp % 4 == 0 && out_cp >= cout;
+}
+int tconv_p16_tile_count() { return (int)(sizeof(kTEntries) / sizeof(kTEntries[0])); }
+void tconv_p16_tile(int index, int* th, int* tw, int* wm) {
+    *th = kTEntries[index].th; *tw = kTEntries[index].tw; *wm = kTEntries[index].wm;
+}
+void tconv_p16_tap(int t, int* ky, int* kx) { *ky = TT_KY[t]; *kx = TT_KX[t]; }
+bool tconv_p16_supported(int k, int crop, int in_cp, int in_pad, int cout, int out_cp, bool f16) {
+    (void)f16;
+    return k == 3 && crop == 1 && in_cp % KC == 0 && in_pad >= 1 && cout % 32 == 0 && out_cp % 4 == 0 && out_cp >= cout;
+}
+int conv_p16c4_tile_count() { return (int)(sizeof(kC4Entries) / sizeof(kC4Entries[0])); }
+void conv_p16c4_tile(int index, int* k, int* th, int* tw, int* steps) {
+    *k = kC4Entries[index].k; *th = kC4Entries[index].th; *tw = kC4Entries[index].tw; *steps = kC4Entries[index].steps;
+}
+bool conv_p16c4_supported(int k, int stride, int dil, int in_cp, int cout, int out_cp, bool f16) {
+    (void)f16;
+    return k == 9 && stride == 1 && dil == 1 && in_cp == 4 && cout % 32 == 0 && out_cp % 4 == 0 && out_cp >= cout;
+}
+#endif
+
 static const P16Entry* find_entry(const ConvP16Params& p) {
     for (const P16Entry& c : kEntries)
         if (c.th == p.tile_h && c.tw == p.tile_w && c.stride == p.stride && c.wm == p.wm) return &c;
     return nullptr;
 }
-size_t conv_p16_lds_bytes(const ConvP16Params& p) {
+size_t P16_NAME(conv_p16_lds_bytes)(const ConvP16Params& p) {
+#if !FYN_P16_HALF
+    if (p.f16) return conv_p16_lds_bytes_half(p);
+#endif
     const P16Entry* e = find_entry(p);
     return e ? entry_lds(*e, p.res != nullptr) : 0;
 }
 
-bool conv_p16_supported(int k, int stride, int dil, int in_cp, int cout, int out_cp, bool f16) {
-    return k == 3 && (stride == 1 || stride == 2) && dil == 1 && !f16 && in_cp % KC == 0 && cout % 64 == 0 && out_cp % 4 == 0 && out_cp >= cout;
-}
-
-int launch_conv_p16(const ConvP16Params& p, hipStream_t s) {
+int P16_NAME(launch_conv_p16)(const ConvP16Params& p, hipStream_t s) {
+#if !FYN_P16_HALF
+    if (p.f16) return launch_conv_p16_half(p, s);
+#endif
     const P16Entry* e = find_entry(p);
     if (!e) return -1;
     const int cpb = 32 * e->wm, twg = (4 / e->wm) * e->tw;
     // what the kernel's indexing assumes
     if (p.cin_chunks < 1 || p.in_cp != p.cin_chunks * KC || p.cout_blocks < 1 || p.mfrags < p.cout_blocks * 2 * e->wm ||
-        p.tiles_x * twg < p.npos_x || p.tiles_y * p.tile_h < p.npos_y || p.out_cp < p.cout_blocks * cpb ||
-        (p.res && p.res_cp < p.cout_blocks * cpb) || p.nreset < 0 || p.nreset > 4 || p.pos_groups < 1 || p.pos_groups > p.tiles_x * p.tiles_y ||
+        p.tiles_x * twg < p.npos_x || p.tiles_y * p.tile_h < p.npos_y || p.out_cp < p.cout_blocks * cpb || p.out_cp % 4 != 0 ||
+        (p.res && (p.res_cp < p.cout_blocks * cpb || (p.res_cp * ESZ) % 16 != 0)) || p.nreset < 0 || p.nreset > 4 || p.pos_groups < 1 ||
+        p.pos_groups > p.tiles_x * p.tiles_y || (p.f16 != 0) != HSTORE ||
         // (a tile's residual tile may not be overwritten while its epilogue reads it: the next one comes a stage later)
         (p.res && p.cin_chunks < 2 && p.pos_groups < p.tiles_x * p.tiles_y) || p.rcp_tiles_x != 1.0f / (float)p.tiles_x ||
         p.tiles_x * p.tiles_y > 4000000)   // (tile index -> row and column through the reciprocal: exact below four million tiles)
@@ -940,70 +1046,67 @@ int launch_conv_p16(const ConvP16Params& p, hipStream_t s) {
     return hipGetLastError() == hipSuccess ? 0 : -3;
 }
 
-int tconv_p16_tile_count() { return (int)(sizeof(kTEntries) / sizeof(kTEntries[0])); }
-void tconv_p16_tile(int index, int* th, int* tw, int* wm) {
-    *th = kTEntries[index].th; *tw = kTEntries[index].tw; *wm = kTEntries[index].wm;
-}
 static const TP16Entry* find_tentry(const ConvP16Params& p) {
     for (const TP16Entry& c : kTEntries)
         if (c.th == p.tile_h && c.tw == p.tile_w && c.wm == p.wm) return &c;
     return nullptr;
 }
-void tconv_p16_tap(int t, int* ky, int* kx) { *ky = TT_KY[t]; *kx = TT_KX[t]; }
-size_t tconv_p16_lds_bytes(const ConvP16Params& p) {
+size_t P16_NAME(tconv_p16_lds_bytes)(const ConvP16Params& p) {
+#if !FYN_P16_HALF
+    if (p.f16) return tconv_p16_lds_bytes_half(p);
+#endif
     const TP16Entry* e = find_tentry(p);
     return e ? 2 * e->buf + 2 * (size_t)(32 * e->wm) * 4 : 0;
 }
-bool tconv_p16_supported(int k, int crop, int in_cp, int in_pad, int cout, int out_cp, bool f16) {
-    return k == 3 && crop == 1 && !f16 && in_cp % KC == 0 && in_pad >= 1 && cout % 32 == 0 && out_cp % 4 == 0 && out_cp >= cout;
-}
 
 // npos_y x npos_x: the input size (positions are input pixels); out_off_*: stored coordinate of output pixel (0, 0)
-int launch_tconv_p16(const ConvP16Params& p, hipStream_t s) {
+int P16_NAME(launch_tconv_p16)(const ConvP16Params& p, hipStream_t s) {
+#if !FYN_P16_HALF
+    if (p.f16) return launch_tconv_p16_half(p, s);
+#endif
     const TP16Entry* e = find_tentry(p);
     if (!e) return -1;
     const int cpb = 32 * e->wm, twg = (4 / e->wm) * e->tw;
     if (p.cin_chunks < 1 || p.in_cp != p.cin_chunks * KC || p.cout_blocks < 1 || p.mfrags < p.cout_blocks * 2 * e->wm ||
-        p.tiles_x * twg < p.npos_x || p.tiles_y * p.tile_h < p.npos_y || p.out_cp < p.cout_blocks * cpb || p.res || p.stride != 1 ||
-        p.nreset < 0 || p.nreset > 4 || p.pos_groups < 1 || p.pos_groups > p.tiles_x * p.tiles_y ||
+        p.tiles_x * twg < p.npos_x || p.tiles_y * p.tile_h < p.npos_y || p.out_cp < p.cout_blocks * cpb || p.out_cp % 4 != 0 || p.res || p.stride != 1 ||
+        p.nreset < 0 || p.nreset > 4 || p.pos_groups < 1 || p.pos_groups > p.tiles_x * p.tiles_y || (p.f16 != 0) != HSTORE ||
         p.rcp_tiles_x != 1.0f / (float)p.tiles_x || p.tiles_x * p.tiles_y > 4000000)
         return -5;
-    const size_t lds_bytes = tconv_p16_lds_bytes(p);
+    const size_t lds_bytes = P16_NAME(tconv_p16_lds_bytes)(p);
     if (lds_bytes > 160 * 1024) return -2;
     if (ensure_lds(reinterpret_cast<const void*>(e->fn), lds_bytes) != 0) return -2;
     hipLaunchKernelGGL(e->fn, dim3(p.pos_groups * p.cout_blocks), dim3(512), lds_bytes, s, p);
     return hipGetLastError() == hipSuccess ? 0 : -3;
 }
 
-int conv_p16c4_tile_count() { return (int)(sizeof(kC4Entries) / sizeof(kC4Entries[0])); }
-void conv_p16c4_tile(int index, int* k, int* th, int* tw, int* steps) {
-    *k = kC4Entries[index].k; *th = kC4Entries[index].th; *tw = kC4Entries[index].tw; *steps = kC4Entries[index].steps;
-}
 static const C4Entry* find_c4entry(const ConvP16Params& p, int k) {
     for (const C4Entry& c : kC4Entries)
         if (c.k == k && c.th == p.tile_h && c.tw == p.tile_w) return &c;
     return nullptr;
 }
-size_t conv_p16c4_lds_bytes(const ConvP16Params& p, int k) {
+size_t P16_NAME(conv_p16c4_lds_bytes)(const ConvP16Params& p, int k) {
+#if !FYN_P16_HALF
+    if (p.f16) return conv_p16c4_lds_bytes_half(p, k);
+#endif
     const C4Entry* e = find_c4entry(p, k);
     return e ? 2 * e->buf + 2 * 32 * 4 : 0;
-}
-bool conv_p16c4_supported(int k, int stride, int dil, int in_cp, int cout, int out_cp, bool f16) {
-    return k == 9 && stride == 1 && dil == 1 && !f16 && in_cp == 4 && cout % 32 == 0 && out_cp % 4 == 0 && out_cp >= cout;
 }
 
 // k x k convolution on a four-channel input: wpack = [step][cout fragment of 16][plane][lane][8 halves], lane = (output
 // channel lane%16, tap pair 4*step + lane/16 = kernel row pair/((k+1)/2), columns 2*(pair%((k+1)/2)) and +1), four input
 // channels per tap; in_y0/in_x0 = input padding - (k-1)/2
-int launch_conv_p16c4(const ConvP16Params& p, int k, hipStream_t s) {
+int P16_NAME(launch_conv_p16c4)(const ConvP16Params& p, int k, hipStream_t s) {
+#if !FYN_P16_HALF
+    if (p.f16) return launch_conv_p16c4_half(p, k, s);
+#endif
     const C4Entry* e = find_c4entry(p, k);
     if (!e) return -1;
     if (p.in_cp != 4 || p.cin_chunks != 1 || p.cout_blocks < 1 || p.mfrags < p.cout_blocks * 2 || p.wm != 1 || p.stride != 1 || p.res ||
-        p.tiles_x * 4 * e->tw < p.npos_x || p.tiles_y * e->th < p.npos_y || p.out_cp < p.cout_blocks * 32 ||
-        p.nreset < 0 || p.nreset > 4 || p.pos_groups < 1 || p.pos_groups > p.tiles_x * p.tiles_y ||
+        p.tiles_x * 4 * e->tw < p.npos_x || p.tiles_y * e->th < p.npos_y || p.out_cp < p.cout_blocks * 32 || p.out_cp % 4 != 0 ||
+        p.nreset < 0 || p.nreset > 4 || p.pos_groups < 1 || p.pos_groups > p.tiles_x * p.tiles_y || (p.f16 != 0) != HSTORE ||
         p.rcp_tiles_x != 1.0f / (float)p.tiles_x || p.tiles_x * p.tiles_y > 4000000)
         return -5;
-    const size_t lds_bytes = conv_p16c4_lds_bytes(p, k);
+    const size_t lds_bytes = P16_NAME(conv_p16c4_lds_bytes)(p, k);
     if (lds_bytes > 160 * 1024) return -2;
     if (ensure_lds(reinterpret_cast<const void*>(e->fn), lds_bytes) != 0) return -2;
     hipLaunchKernelGGL(e->fn, dim3(p.pos_groups * p.cout_blocks), dim3(512), lds_bytes, s, p);

@@ -189,6 +189,7 @@ struct ConvP16Params {
     int cin_chunks;
     int mfrags;           // cout fragments (16 each) in wpack
     int cout_blocks;      // workgroups along cout (32*wm channels each)
+    int f16;              // tensors hold fp16 (wpack then has one plane, and there are no value-range words)
     float acc_mul;
     const unsigned* in_amax;   // value-range words as in ConvMfmaParams
     unsigned* out_amax;

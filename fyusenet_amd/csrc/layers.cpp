@@ -892,6 +892,7 @@ class ConvLayer : public Layer {
         q.res_relu = res_relu; q.res_scale = res_scale;
         q.cin_chunks = in_v.cp / 32;
         q.mfrags = oc / 16;
+        q.f16 = out_v.f16 ? 1 : 0;
         q.scale = scale_dev; q.bias = bias_dev;
         q.acc_mul = 1.f;
         q.act = act();
@@ -922,7 +923,7 @@ class ConvLayer : public Layer {
         if (cands.empty()) return;
         std::sort(cands.begin(), cands.end(), [](const Cand& a, const Cand& b) { return a.cost < b.cost; });
         if (cands.size() > 3) cands.resize(3);
-        const size_t halves = ((size_t)q.cin_chunks * 9 + 8) * q.mfrags * 2 * 64 * 8;
+        const size_t halves = ((size_t)q.cin_chunks * 9 + 8) * q.mfrags * (q.f16 ? 1 : 2) * 64 * 8;
         p16_wpack_dev = net->dev_alloc(halves * 2, true);
         for (Cand& c : cands) c.q.wpack = p16_wpack_dev;
         const bool always = getenv("FYNHIP_FORCE_P16_CONV") != nullptr;
@@ -930,7 +931,7 @@ class ConvLayer : public Layer {
         const bool timing = !(at && at[0] == '0');
         int pick = 0;   // index into cands, -1: the general kernel
         char key[160];
-        snprintf(key, sizeof(key), "p16:%dx%d:%dx%d:s%d:cp%d:r%d:e%d", d.in_channels, oc, oh, ow, stride, in_v.cp, res_v ? 1 : 0, clamp ? 1 : 0);
+        snprintf(key, sizeof(key), "p16:%dx%d:%dx%d:s%d:cp%d:r%d:e%d:h%d", d.in_channels, oc, oh, ow, stride, in_v.cp, res_v ? 1 : 0, clamp ? 1 : 0, q.f16);
         int cached[3] = {0, 0, 0};
         bool have_cached = false;
         if (!want_h) have_cached = tune_cache_triple(key, cached);   // (the cache keeps: chosen?, tile_h*1000 + tile_w, wm)
@@ -979,6 +980,7 @@ class ConvLayer : public Layer {
         q.cin_chunks = 1;
         q.mfrags = oc / 16;
         q.cout_blocks = oc / 32;
+        q.f16 = out_v.f16 ? 1 : 0;
         q.scale = scale_dev; q.bias = bias_dev;
         q.acc_mul = 1.f;
         q.act = act();
@@ -1002,14 +1004,14 @@ class ConvLayer : public Layer {
         }
         if (cands.empty()) return;
         c4_steps = steps;
-        const size_t halves = ((size_t)steps + 8) * q.mfrags * 2 * 64 * 8;
+        const size_t halves = ((size_t)steps + 8) * q.mfrags * (q.f16 ? 1 : 2) * 64 * 8;
         p16_wpack_dev = net->dev_alloc(halves * 2, true);
         for (ConvP16Params& c : cands) c.wpack = p16_wpack_dev;
         const bool always = getenv("FYNHIP_FORCE_P16_CONV") != nullptr;
         const char* at = getenv("FYNHIP_AUTOTUNE");
         int pick = 0;
         char key[160];
-        snprintf(key, sizeof(key), "c4p16:k%d:%dx%d:%dx%d:e%d", k, d.in_channels, oc, oh, ow, clamp ? 1 : 0);
+        snprintf(key, sizeof(key), "c4p16:k%d:%dx%d:%dx%d:e%d:h%d", k, d.in_channels, oc, oh, ow, clamp ? 1 : 0, q.f16);
         int cached[3] = {0, 0, 0};
         if (!want_h && tune_cache_triple(key, cached)) {
             pick = -1;
@@ -1061,6 +1063,7 @@ class ConvLayer : public Layer {
         q.cin_chunks = in_v.cp / 32;
         q.mfrags = oc / 16;
         q.cout_blocks = oc / 128;
+        q.f16 = 1;
         q.scale = scale_dev; q.bias = bias_dev;
         q.acc_mul = 1.f;
         q.act = act();
@@ -1193,10 +1196,11 @@ class ConvLayer : public Layer {
     // weights of that form: [step][cout fragment of 16][plane][lane][8 halves]; lane = (channel lane%16, tap pair 4*step + lane/16)
     void pack_c4(const float* w, float wmul) {
         const int cin = d.in_channels, ppr = (k + 1) / 2;
-        std::vector<uint16_t> pack(((size_t)c4_steps + 8) * pp.mfrags * 2 * 64 * 8, 0);
+        const int npl = pp.f16 ? 1 : 2;   // (fp16 tensors: the hi plane only)
+        std::vector<uint16_t> pack(((size_t)c4_steps + 8) * pp.mfrags * npl * 64 * 8, 0);
         for (int st = 0; st < c4_steps; st++)
             for (int mf = 0; mf < pp.mfrags; mf++) {
-                uint16_t* base = pack.data() + (((size_t)st * pp.mfrags + mf) * 2) * 64 * 8;
+                uint16_t* base = pack.data() + (((size_t)st * pp.mfrags + mf) * npl) * 64 * 8;
                 for (int lane = 0; lane < 64; lane++) {
                     const int o = mf * 16 + (lane & 15), pi = 4 * st + (lane >> 4);
                     const int ky = pi / ppr, kx0 = 2 * (pi % ppr);
@@ -1207,7 +1211,7 @@ class ConvLayer : public Layer {
                         const float v = w[(((size_t)o * k + ky) * k + kx) * cin + ci] * wmul;
                         const uint16_t hi = f2h_bits(v);
                         base[(size_t)lane * 8 + j] = hi;
-                        base[(size_t)(64 + lane) * 8 + j] = f2h_bits(v - h2f(hi));
+                        if (npl == 2) base[(size_t)(64 + lane) * 8 + j] = f2h_bits(v - h2f(hi));
                     }
                 }
             }
@@ -1218,11 +1222,12 @@ class ConvLayer : public Layer {
     // weights of that form: [(chunk*9 + tap)][cout fragment of 16][plane][lane][8 halves], zero steps behind the last
     void pack_p16(const float* w, float wmul) {
         const int cin = d.in_channels;
-        std::vector<uint16_t> pack(((size_t)pp.cin_chunks * 9 + 8) * pp.mfrags * 2 * 64 * 8, 0);
+        const int npl = pp.f16 ? 1 : 2;
+        std::vector<uint16_t> pack(((size_t)pp.cin_chunks * 9 + 8) * pp.mfrags * npl * 64 * 8, 0);
         for (int chunk = 0; chunk < pp.cin_chunks; chunk++)
             for (int tap = 0; tap < 9; tap++)
                 for (int mf = 0; mf < pp.mfrags; mf++) {
-                    uint16_t* base = pack.data() + (((size_t)(chunk * 9 + tap) * pp.mfrags + mf) * 2) * 64 * 8;
+                    uint16_t* base = pack.data() + (((size_t)(chunk * 9 + tap) * pp.mfrags + mf) * npl) * 64 * 8;
                     for (int lane = 0; lane < 64; lane++) {
                         const int o = mf * 16 + (lane & 15);
                         if (o >= oc) continue;
@@ -1232,7 +1237,7 @@ class ConvLayer : public Layer {
                             const float v = w[(((size_t)o * 3 + tap / 3) * 3 + tap % 3) * cin + ci] * wmul;
                             const uint16_t hi = f2h_bits(v);
                             base[(size_t)lane * 8 + j] = hi;
-                            base[(size_t)(64 + lane) * 8 + j] = f2h_bits(v - h2f(hi));
+                            if (npl == 2) base[(size_t)(64 + lane) * 8 + j] = f2h_bits(v - h2f(hi));
                         }
                     }
                 }
@@ -1441,15 +1446,18 @@ class ConvLayer : public Layer {
             scale_dev = static_cast<float*>(net->dev_alloc(padded * sizeof(float)));
             bias_dev = static_cast<float*>(net->dev_alloc(padded * sizeof(float)));
             launch = tune_mfma(net, sc, in_v, out_v, res_v, d.in_channels, oc, act(), res_relu, res_scale, scale_dev, bias_dev);
-            if (!frac_shift && !sc.in_sub && conv_p16_supported(k, stride, dil, in_v.cp, oc, out_v.cp, out_v.f16 != 0) && d.in_channels == in_v.cp &&
-                (!res_v || res_v->cp >= oc) && !getenv("FYNHIP_NO_P16_CONV"))
+            // the 16-position-fragment forms, each against the tuned launch of the general kernel: for wide fp16 layers the
+            // one with 64-channel wave tiles first, then the 3x3 form, then the small-input form
+            const bool same_storage = in_v.f16 == out_v.f16 && (!res_v || res_v->f16 == out_v.f16);
+            if (!frac_shift && same_storage && conv_h16_supported(k, stride, dil, in_v.cp, oc, out_v.cp, out_v.f16 != 0) && d.in_channels == in_v.cp &&
+                (!res_v || res_v->cp >= oc) && !getenv("FYNHIP_NO_P16_CONV") && !getenv("FYNHIP_NO_H16_CONV"))
+                setup_h16(in_v, out_v, res_v, res_relu, res_scale);
+            if (!p16 && !frac_shift && same_storage && !sc.in_sub && conv_p16_supported(k, stride, dil, in_v.cp, oc, out_v.cp, out_v.f16 != 0) &&
+                d.in_channels == in_v.cp && (!res_v || (res_v->cp >= oc && res_v->cp % 8 == 0)) && !getenv("FYNHIP_NO_P16_CONV"))
                 setup_p16(in_v, out_v, res_v, res_relu, res_scale);
-            if (!frac_shift && !res_v && conv_p16c4_supported(k, stride, dil, in_v.cp, oc, out_v.cp, out_v.f16 != 0) &&
+            if (!p16 && !frac_shift && same_storage && !res_v && conv_p16c4_supported(k, stride, dil, in_v.cp, oc, out_v.cp, out_v.f16 != 0) &&
                 !getenv("FYNHIP_NO_P16_CONV"))
                 setup_c4(in_v, out_v);
-            if (!frac_shift && conv_h16_supported(k, stride, dil, in_v.cp, oc, out_v.cp, out_v.f16 != 0) && in_v.f16 && d.in_channels == in_v.cp &&
-                (!res_v || (res_v->cp >= oc && res_v->f16)) && !getenv("FYNHIP_NO_P16_CONV"))
-                setup_h16(in_v, out_v, res_v, res_relu, res_scale);
         }
         if (direct) {
             scale_dev = static_cast<float*>(net->dev_alloc(padded * sizeof(float)));
@@ -1544,8 +1552,8 @@ class ConvLayer : public Layer {
         }
         if (p16 && c4) {
             char buf[220];
-            snprintf(buf, sizeof(buf), "conv_p16c4 f16x2-split (tap pairs of a 4-channel pixel) tile=32x%d(cout x pos) th=%d tw=%d blocks=%d tiles=%d lds=%zu steps=%d",
-                     pp.tile_h * pp.tile_w * 4, pp.tile_h, pp.tile_w, pp.pos_groups * pp.cout_blocks, pp.tiles_x * pp.tiles_y * pp.cout_blocks,
+            snprintf(buf, sizeof(buf), "conv_p16c4 %s (tap pairs of a 4-channel pixel) tile=32x%d(cout x pos) th=%d tw=%d blocks=%d tiles=%d lds=%zu steps=%d",
+                     pp.f16 ? "f16" : "f16x2-split", pp.tile_h * pp.tile_w * 4, pp.tile_h, pp.tile_w, pp.pos_groups * pp.cout_blocks, pp.tiles_x * pp.tiles_y * pp.cout_blocks,
                      conv_p16c4_lds_bytes(pp, k), c4_steps);
             return mode + buf;
         }
@@ -1564,8 +1572,8 @@ class ConvLayer : public Layer {
         }
         if (p16) {
             char buf[200];
-            snprintf(buf, sizeof(buf), "conv_p16 f16x2-split tile=%dx%d(cout x pos) waves=%dx%d th=%d tw=%d blocks=%d tiles=%d lds=%zu steps=9 chunks=%d",
-                     32 * pp.wm, pp.tile_h * pp.tile_w * (4 / pp.wm), pp.wm, 4 / pp.wm, pp.tile_h, pp.tile_w, pp.pos_groups * pp.cout_blocks,
+            snprintf(buf, sizeof(buf), "conv_p16 %s tile=%dx%d(cout x pos) waves=%dx%d th=%d tw=%d blocks=%d tiles=%d lds=%zu steps=9 chunks=%d",
+                     pp.f16 ? "f16" : "f16x2-split", 32 * pp.wm, pp.tile_h * pp.tile_w * (4 / pp.wm), pp.wm, 4 / pp.wm, pp.tile_h, pp.tile_w, pp.pos_groups * pp.cout_blocks,
                      pp.tiles_x * pp.tiles_y * pp.cout_blocks, conv_p16_lds_bytes(pp), pp.cin_chunks);
             return mode + buf;
         }
@@ -1707,7 +1715,8 @@ class TransConvLayer : public Layer {
                 subconvs.push_back(sc);
             }
         group = tune_mfma_group(net, subconvs, in_v, out_v, d.in_channels, oc, act(), scale_dev, bias_dev);
-        if (tconv_p16_supported(k, crop, in_v.cp, in_v.pad, oc, out_v.cp, out_v.f16 != 0) && d.in_channels == in_v.cp && !getenv("FYNHIP_NO_P16_CONV"))
+        if (tconv_p16_supported(k, crop, in_v.cp, in_v.pad, oc, out_v.cp, out_v.f16 != 0) && in_v.f16 == out_v.f16 && d.in_channels == in_v.cp &&
+            !getenv("FYNHIP_NO_P16_CONV"))
             setup_p16(in_v, out_v);
         set_up = true;
         setup_ranges();
@@ -1725,6 +1734,7 @@ class TransConvLayer : public Layer {
         q.out_wp = out_v.wp(); q.out_cp = out_v.cp; q.out_off_y = q.out_off_x = out_v.pad;
         q.cin_chunks = in_v.cp / 32;
         q.mfrags = oc / 16;
+        q.f16 = out_v.f16 ? 1 : 0;
         q.scale = scale_dev; q.bias = bias_dev;
         q.acc_mul = 1.f;
         q.act = act();
@@ -1748,14 +1758,14 @@ class TransConvLayer : public Layer {
             cands.push_back(c);
         }
         if (cands.empty()) return;
-        const size_t halves = ((size_t)q.cin_chunks * 9 + 8) * q.mfrags * 2 * 64 * 8;
+        const size_t halves = ((size_t)q.cin_chunks * 9 + 8) * q.mfrags * (q.f16 ? 1 : 2) * 64 * 8;
         p16_wpack_dev = net->dev_alloc(halves * 2, true);
         for (ConvP16Params& c : cands) c.wpack = p16_wpack_dev;
         const bool always = getenv("FYNHIP_FORCE_P16_CONV") != nullptr;
         const char* at = getenv("FYNHIP_AUTOTUNE");
         int pick = 0;
         char key[160];
-        snprintf(key, sizeof(key), "tp16:%dx%d:%dx%d:cp%d", d.in_channels, oc, d.height, d.width, in_v.cp);
+        snprintf(key, sizeof(key), "tp16:%dx%d:%dx%d:cp%d:h%d", d.in_channels, oc, d.height, d.width, in_v.cp, q.f16);
         int cached[3] = {0, 0, 0};
         if (!want_h && tune_cache_triple(key, cached)) {
             pick = -1;
@@ -1792,13 +1802,14 @@ class TransConvLayer : public Layer {
     // weights of that form: [(chunk*9 + step)][cout fragment of 16][plane][lane][8 halves], steps in the kernel's tap order
     void pack_p16(const float* w, float wmul) {
         const int cin = d.in_channels;
-        std::vector<uint16_t> pack(((size_t)pp.cin_chunks * 9 + 8) * pp.mfrags * 2 * 64 * 8, 0);
+        const int npl = pp.f16 ? 1 : 2;
+        std::vector<uint16_t> pack(((size_t)pp.cin_chunks * 9 + 8) * pp.mfrags * npl * 64 * 8, 0);
         for (int chunk = 0; chunk < pp.cin_chunks; chunk++)
             for (int t = 0; t < 9; t++) {
                 int ky, kx;
                 tconv_p16_tap(t, &ky, &kx);
                 for (int mf = 0; mf < pp.mfrags; mf++) {
-                    uint16_t* base = pack.data() + (((size_t)(chunk * 9 + t) * pp.mfrags + mf) * 2) * 64 * 8;
+                    uint16_t* base = pack.data() + (((size_t)(chunk * 9 + t) * pp.mfrags + mf) * npl) * 64 * 8;
                     for (int lane = 0; lane < 64; lane++) {
                         const int o = mf * 16 + (lane & 15);
                         if (o >= oc) continue;
@@ -1808,7 +1819,7 @@ class TransConvLayer : public Layer {
                             const float v = w[(((size_t)o * 3 + ky) * 3 + kx) * cin + ci] * wmul;
                             const uint16_t hi = f2h_bits(v);
                             base[(size_t)lane * 8 + j] = hi;
-                            base[(size_t)(64 + lane) * 8 + j] = f2h_bits(v - h2f(hi));
+                            if (npl == 2) base[(size_t)(64 + lane) * 8 + j] = f2h_bits(v - h2f(hi));
                         }
                     }
                 }
@@ -1872,7 +1883,7 @@ class TransConvLayer : public Layer {
     std::string info() const override {
         if (p16) {
             char buf[220];
-            snprintf(buf, sizeof(buf), "transconv, tconv_p16 f16x2-split 4 parities per tile, tile=%dx%d(cout x input pos) waves=%dx%d th=%d tw=%d blocks=%d tiles=%d lds=%zu steps=9 chunks=%d",
+            snprintf(buf, sizeof(buf), "transconv, tconv_p16 %s 4 parities per tile, tile=%dx%d(cout x input pos) waves=%dx%d th=%d tw=%d blocks=%d tiles=%d lds=%zu steps=9 chunks=%d", pp.f16 ? "f16" : "f16x2-split",
                      32 * pp.wm, pp.tile_h * pp.tile_w * (4 / pp.wm), pp.wm, 4 / pp.wm, pp.tile_h, pp.tile_w, pp.pos_groups * pp.cout_blocks,
                      pp.tiles_x * pp.tiles_y * pp.cout_blocks, tconv_p16_lds_bytes(pp), pp.cin_chunks);
             return buf;

@@ -273,17 +273,22 @@ P16_CASES = [
 ]
 
 
+@pytest.mark.parametrize("storage", [fa.STORAGE_F32, fa.STORAGE_F16], ids=["f32", "f16"])
 @pytest.mark.parametrize("shallow", [False, True], ids=["deep", "shallow_edge_clamp"])
 @pytest.mark.parametrize("act", [A.RELU, A.LEAKY_RELU, A.NONE], ids=["relu", "leaky", "none"])
 @pytest.mark.parametrize("case", P16_CASES, ids=lambda c: "%dx%dx%d_to%d_s%d_%s" % (c[0], c[2], c[3], c[1], c[4], (c[5] or "auto").replace(",", "x")))
-def test_sixteen_position_fragment_form(case, act, shallow, monkeypatch):
-    """The 3x3 convolution on 16-position fragments (fp32 storage only): every compiled tile, ragged edges, the
-    residual tile through LDS, value ranges on both sides."""
+def test_sixteen_position_fragment_form(case, act, shallow, storage, monkeypatch):
+    """The 3x3 convolution on 16-position fragments: every compiled tile, ragged edges, the residual tile through LDS;
+    fp32 storage (operand split, value ranges on both sides) and fp16 storage (one plane, one pass)."""
     cin, cout, h, w, stride, tile, kw = case
     if shallow and ("residual" in kw or "pad_out" in kw):
         pytest.skip("the shallow variant is run on the plain cases")
     if act is not A.RELU and ("pad_out" in kw or tile in ("4,4,4", "8,6,4", "8,8,4", "8,4,2", "4,8,2") or h > 60):
         pytest.skip("activations are varied on some of the cases")
+    if storage == fa.STORAGE_F16 and (act is A.NONE or (shallow and h > 30)):
+        pytest.skip("fp16 storage is run on some of the combinations")
+    if storage == fa.STORAGE_F16:
+        monkeypatch.setenv("FYNHIP_NO_H16_CONV", "1")   # (the form with 64-channel wave tiles has its own test)
     monkeypatch.setenv("FYNHIP_FORCE_P16_CONV", "1")
     if tile:
         monkeypatch.setenv("FYNHIP_P16_TILE", tile)
@@ -296,15 +301,15 @@ def test_sixteen_position_fragment_form(case, act, shallow, monkeypatch):
     inputs = [prng.uniform(47 * cin + h, (cin, h, w), -1, 1)]
     if "residual" in kw:
         inputs.append(prng.uniform(53, (cout, h // stride, w // stride), -1, 1))
-    got, info = run_single(b, fa.STORAGE_F32, inputs, wts)
-    ref = oracle_single(b, fa.STORAGE_F32, inputs, wts)
+    got, info = run_single(b, storage, inputs, wts)
+    ref = oracle_single(b, storage, inputs, wts)
     err = rel_l2(got, ref)
     print("  ", info, "rel_l2=%.3e" % err, flush=True)
-    assert "conv_p16" in info
+    assert "conv_p16 f16x2-split" in info if storage == fa.STORAGE_F32 else "conv_p16 f16 " in info
     if tile:
         th, tw, wm = tile.split(",")
         assert "waves=%sx" % wm in info and "th=%s tw=%s" % (th, tw) in info
-    assert err <= TOL[fa.STORAGE_F32], info
+    assert err <= TOL[storage], info
 
 
 H16_CASES = [
@@ -468,11 +473,11 @@ C4_CASES = [
 ]
 
 
+@pytest.mark.parametrize("storage", [fa.STORAGE_F32, fa.STORAGE_F16], ids=["f32", "f16"])
 @pytest.mark.parametrize("shallow", [False, True], ids=["deep", "shallow_edge_clamp"])
 @pytest.mark.parametrize("case", C4_CASES, ids=lambda c: "%dx%dx%d_to%d_%s" % (c[0], c[2], c[3], c[1], (c[4] or "auto").replace(",", "x")))
-def test_small_input_sixteen_position_fragment_form(case, shallow, monkeypatch):
-    """The 9x9 convolution on at most four input channels with two taps of a 4-channel pixel per lane and step (fp32
-    storage)."""
+def test_small_input_sixteen_position_fragment_form(case, shallow, storage, monkeypatch):
+    """The 9x9 convolution on at most four input channels with two taps of a 4-channel pixel per lane and step."""
     cin, cout, h, w, tile, kw = case
     if shallow and ("pad_out" in kw or h > 60):
         pytest.skip("the shallow variant is run on the plain cases")
@@ -484,14 +489,14 @@ def test_small_input_sixteen_position_fragment_form(case, shallow, monkeypatch):
     b = conv_builder(9, cout, h, w, cin, 1, 1, A.NONE, **kw)
     wts = conv_block(1200 + cin, cout, 9, cin, bn=kw.get("bn", False))
     x = prng.uniform(61 * cin + w, (cin, h, w), 0, 1)
-    got, info = run_single(b, fa.STORAGE_F32, [x], wts)
-    ref = oracle_single(b, fa.STORAGE_F32, [x], wts)
+    got, info = run_single(b, storage, [x], wts)
+    ref = oracle_single(b, storage, [x], wts)
     err = rel_l2(got, ref)
     print("  ", info, "rel_l2=%.3e" % err, flush=True)
-    assert "conv_p16c4" in info
+    assert "conv_p16c4 f16x2-split" in info if storage == fa.STORAGE_F32 else "conv_p16c4 f16 " in info
     if tile:
         assert "th=%s tw=%s" % tuple(tile.split(",")) in info
-    assert err <= TOL[fa.STORAGE_F32], info
+    assert err <= TOL[storage], info
 
 
 TP16_CASES = [
@@ -510,13 +515,14 @@ TP16_CASES = [
 ]
 
 
+@pytest.mark.parametrize("storage", [fa.STORAGE_F32, fa.STORAGE_F16], ids=["f32", "f16"])
 @pytest.mark.parametrize("act", [A.RELU, A.NONE], ids=["relu", "none"])
 @pytest.mark.parametrize("case", TP16_CASES, ids=lambda c: "%dx%dx%d_to%d_%s" % (c[0], c[2], c[3], c[1], (c[4] or "auto").replace(",", "x")))
-def test_transconv_sixteen_position_fragment_form(case, act, monkeypatch):
-    """The doubling transposed 3x3 convolution on 16-position fragments (fp32 storage): all four output parities from
-    one staged input tile."""
+def test_transconv_sixteen_position_fragment_form(case, act, storage, monkeypatch):
+    """The doubling transposed 3x3 convolution on 16-position fragments: all four output parities from one staged input
+    tile; fp32 and fp16 storage."""
     cin, cout, h, w, tile, bn = case
-    if act is A.NONE and (tile is None or h > 60):
+    if act is A.NONE and (tile is None or h > 60 or storage == fa.STORAGE_F16):
         pytest.skip("the activation is varied on the small cases")
     monkeypatch.setenv("FYNHIP_FORCE_P16_CONV", "1")
     if tile:
@@ -527,16 +533,16 @@ def test_transconv_sixteen_position_fragment_form(case, act, monkeypatch):
         b.postfixNorm(fa.NormType.BATCHNORM)
     wts = conv_block(1100 + cin, cout, 3, cin, bn=bn)
     x = prng.uniform(57 * cin + w, (cin, h, w), -1, 1)
-    got, info = run_single(b, fa.STORAGE_F32, [x], wts)
-    ref = oracle_single(b, fa.STORAGE_F32, [x], wts)
+    got, info = run_single(b, storage, [x], wts)
+    ref = oracle_single(b, storage, [x], wts)
     err = rel_l2(got, ref)
     print("  ", info, "rel_l2=%.3e" % err, flush=True)
-    assert "tconv_p16" in info
+    assert "tconv_p16 f16x2-split" in info if storage == fa.STORAGE_F32 else "tconv_p16 f16 " in info
     if tile:
         th, tw, wm = tile.split(",")
         assert "waves=%sx" % wm in info and "th=%s tw=%s" % (th, tw) in info
     assert got.shape == ref.shape == (cout, 2 * h, 2 * w)
-    assert err <= TOL[fa.STORAGE_F32], info
+    assert err <= TOL[storage], info
 
 
 FRAC_CASES = [
