@@ -16,8 +16,10 @@
 //
 // Workgroup = 4 staging waves (next chunk: global loads, activation, hi/lo conversion, LDS writes; scale and bias at
 // the start and, during the last chunk, the residual tile into LDS) + 4 MFMA waves (32 output channels each: 2 channel
-// fragments x FN position fragments).  A lane's accumulators of one fragment are 4 consecutive output channels of one
-// position, so the epilogue needs no transposition: residual and scale/bias from LDS, one 16-byte store per fragment.
+// fragments x FN position fragments).  A lane's accumulators of one fragment are 4 consecutive fragment rows of one
+// position, so the epilogue needs no transposition: residual and scale/bias from LDS, one 16-byte store per fragment
+// (fp16 tensors: the weights are packed so that row r of fragment fm of a wave's pair is output channel
+// 8*(r/4) + 4*fm + r%4 of the wave's 32, a lane's eight values are eight consecutive channels and go out in one store).
 #include <hip/hip_fp16.h>
 #include <hip/hip_runtime.h>
 
@@ -54,6 +56,12 @@ constexpr int NPL = HSTORE ? 1 : 2;          // staged planes (hi, lo)
 constexpr int NPASS = HSTORE ? 1 : 3;        // MFMAs per fragment pair (hi*hi, lo*hi, hi*lo)
 constexpr int ESZ = HSTORE ? 2 : 4;          // bytes per stored element
 typedef std::conditional<HSTORE, _Float16, float>::type store_t;
+// Output channel, inside a wave's 32, of accumulator element e of channel fragment fm in the lanes kq = lane / 16:
+// kq * CHK + fm * CHF + e.  fp32 tensors: fragment rows are channels in order (a fragment's store is 64 contiguous bytes
+// from the four lanes of a position).  fp16 tensors: the weights are packed so that a lane's eight values are eight
+// consecutive channels (one 16-byte store per lane and position instead of two of 8 bytes; with fp32 tensors the same
+// layout -- two 16-byte stores per lane, interleaved between lanes -- measured slower).
+constexpr int CHK = HSTORE ? 8 : 4, CHF = HSTORE ? 4 : 16;
 typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
 
 // Geometry of one instantiation.  A workgroup's four MFMA waves are WM groups of 32 output channels x WN = 4 / WM tiles
@@ -354,8 +362,8 @@ __global__ __launch_bounds__(512) void conv_p16_kernel(const ConvP16Params p) {
         f32x4_t rs[2], bi[2], scm[2];
 #pragma unroll
         for (int fm = 0; fm < 2; fm++) {
-            const f32x4_t sc = *reinterpret_cast<const f32x4_t*>(sb + mw * 32 + fm * 16 + kq * 4);
-            bi[fm] = *reinterpret_cast<const f32x4_t*>(sb + CPB + mw * 32 + fm * 16 + kq * 4);
+            const f32x4_t sc = *reinterpret_cast<const f32x4_t*>(sb + mw * 32 + kq * CHK + fm * CHF);
+            bi[fm] = *reinterpret_cast<const f32x4_t*>(sb + CPB + mw * 32 + kq * CHK + fm * CHF);
             scm[fm] = sc * acc_mul;
             rs[fm] = res_scale ? sc : (f32x4_t)(1.f);
         }
@@ -365,8 +373,9 @@ __global__ __launch_bounds__(512) void conv_p16_kernel(const ConvP16Params p) {
             const int ty = m / TW, tx = wn * TW + (m - ty * TW);
             const int py = tyi * TH + ty, px = txi * G::TWG + tx;
             const bool ok = py < p.npos_y && px < p.npos_x;
-            const size_t obase = ((size_t)(p.out_off_y + py) * p.out_wp + p.out_off_x + px) * p.out_cp + cb * CPB + mw * 32 + kq * 4;
+            const size_t obase = ((size_t)(p.out_off_y + py) * p.out_wp + p.out_off_x + px) * p.out_cp + cb * CPB + mw * 32 + kq * CHK;
             float fmax_ = 0.f;
+            half8_t hv;
 #pragma unroll
             for (int fm = 0; fm < 2; fm++) {
                 f32x4_t v;
@@ -374,7 +383,7 @@ __global__ __launch_bounds__(512) void conv_p16_kernel(const ConvP16Params p) {
                 for (int e = 0; e < 4; e++) v[e] = acc[fm][fn][e] * scm[fm][e] + bi[fm][e];
                 if (have_res) {
                     // (the two options as operands instead of selects: max(r, 0 or -inf), times scale or 1)
-                    const unsigned char* rsrc = lds + res_off + (ty * G::TWG + tx) * G::RES_PITCH + (mw * 32 + fm * 16 + kq * 4) * ESZ;
+                    const unsigned char* rsrc = lds + res_off + (ty * G::TWG + tx) * G::RES_PITCH + (mw * 32 + kq * CHK + fm * CHF) * ESZ;
                     f32x4_t rv;
                     if constexpr (HSTORE) {
                         const half4_t rh = *reinterpret_cast<const half4_t*>(rsrc);
@@ -387,14 +396,13 @@ __global__ __launch_bounds__(512) void conv_p16_kernel(const ConvP16Params p) {
                     for (int e = 0; e < 4; e++) v[e] = fmaf(fmaxf(rv[e], res_floor), rs[fm][e], v[e]);
                 }
                 if constexpr (HSTORE) {
-                    half4_t hv;
 #pragma unroll
-                    for (int e = 0; e < 4; e++) hv[e] = (_Float16)v[e];
-                    if (ok) *reinterpret_cast<half4_t*>(out + obase + fm * 16) = hv;
+                    for (int e = 0; e < 4; e++) hv[fm * 4 + e] = (_Float16)v[e];
+                    if (fm == 1 && ok) *reinterpret_cast<half8_t*>(out + obase) = hv;   // the lane's eight channels in one store
                 } else {
 #pragma unroll
                     for (int e = 0; e < 4; e++) fmax_ = fmaxf(fmax_, fabsf(v[e]));
-                    if (ok) *reinterpret_cast<f32x4_t*>(out + obase + fm * 16) = v;
+                    if (ok) *reinterpret_cast<f32x4_t*>(out + obase + fm * CHF) = v;
                 }
             }
             vmax = fmaxf(vmax, ok ? fmax_ : 0.f);
@@ -563,8 +571,8 @@ __global__ __launch_bounds__(512) void tconv_p16_kernel(const ConvP16Params p) {
         f32x4_t bi[2], scm[2];
 #pragma unroll
         for (int fm = 0; fm < 2; fm++) {
-            scm[fm] = *reinterpret_cast<const f32x4_t*>(sb + mw * 32 + fm * 16 + kq * 4) * acc_mul;
-            bi[fm] = *reinterpret_cast<const f32x4_t*>(sb + CPB + mw * 32 + fm * 16 + kq * 4);
+            scm[fm] = *reinterpret_cast<const f32x4_t*>(sb + mw * 32 + kq * CHK + fm * CHF) * acc_mul;
+            bi[fm] = *reinterpret_cast<const f32x4_t*>(sb + CPB + mw * 32 + kq * CHK + fm * CHF);
         }
 #pragma unroll
         for (int fn = 0; fn < FN; fn++) {
@@ -572,11 +580,12 @@ __global__ __launch_bounds__(512) void tconv_p16_kernel(const ConvP16Params p) {
             const int ty = m / TW, tx = wn * TW + (m - ty * TW);
             const int a = tyi * TH + ty, bx = txi * G::TWG + tx;
             const bool ok = a < p.npos_y && bx < p.npos_x;
-            const size_t obase = ((size_t)(p.out_off_y + 2 * a) * p.out_wp + p.out_off_x + 2 * bx) * p.out_cp + cb * CPB + mw * 32 + kq * 4;
+            const size_t obase = ((size_t)(p.out_off_y + 2 * a) * p.out_wp + p.out_off_x + 2 * bx) * p.out_cp + cb * CPB + mw * 32 + kq * CHK;
             float fmax_ = 0.f;
 #pragma unroll
             for (int par = 0; par < 4; par++) {
                 const size_t o = obase + ((size_t)(par >> 1) * p.out_wp + (par & 1)) * p.out_cp;
+                half8_t hv;
 #pragma unroll
                 for (int fm = 0; fm < 2; fm++) {
                     f32x4_t v;
@@ -586,12 +595,11 @@ __global__ __launch_bounds__(512) void tconv_p16_kernel(const ConvP16Params p) {
                         if constexpr (!HSTORE) fmax_ = fmaxf(fmax_, fabsf(v[e]));
                     }
                     if constexpr (HSTORE) {
-                        half4_t hv;
 #pragma unroll
-                        for (int e = 0; e < 4; e++) hv[e] = (_Float16)v[e];
-                        if (ok) *reinterpret_cast<half4_t*>(out + o + fm * 16) = hv;
+                        for (int e = 0; e < 4; e++) hv[fm * 4 + e] = (_Float16)v[e];
+                        if (fm == 1 && ok) *reinterpret_cast<half8_t*>(out + o) = hv;
                     } else {
-                        if (ok) *reinterpret_cast<f32x4_t*>(out + o + fm * 16) = v;
+                        if (ok) *reinterpret_cast<f32x4_t*>(out + o + fm * CHF) = v;
                     }
                 }
             }
@@ -847,8 +855,8 @@ __global__ __launch_bounds__(512) void conv_p16c4_kernel(const ConvP16Params p) 
         f32x4_t bi[2], scm[2];
 #pragma unroll
         for (int fm = 0; fm < 2; fm++) {
-            scm[fm] = *reinterpret_cast<const f32x4_t*>(sb + fm * 16 + kq * 4) * acc_mul;
-            bi[fm] = *reinterpret_cast<const f32x4_t*>(sb + 32 + fm * 16 + kq * 4);
+            scm[fm] = *reinterpret_cast<const f32x4_t*>(sb + kq * CHK + fm * CHF) * acc_mul;
+            bi[fm] = *reinterpret_cast<const f32x4_t*>(sb + 32 + kq * CHK + fm * CHF);
         }
 #pragma unroll
         for (int fn = 0; fn < FN; fn++) {
@@ -856,8 +864,9 @@ __global__ __launch_bounds__(512) void conv_p16c4_kernel(const ConvP16Params p) 
             const int ty = m / TW, tx = wn * TW + (m - ty * TW);
             const int py = tyi * TH + ty, px = txi * G::TWG + tx;
             const bool ok = py < p.npos_y && px < p.npos_x;
-            const size_t obase = ((size_t)(p.out_off_y + py) * p.out_wp + p.out_off_x + px) * p.out_cp + cb * 32 + kq * 4;
+            const size_t obase = ((size_t)(p.out_off_y + py) * p.out_wp + p.out_off_x + px) * p.out_cp + cb * 32 + kq * CHK;
             float fmax_ = 0.f;
+            half8_t hv;
 #pragma unroll
             for (int fm = 0; fm < 2; fm++) {
                 f32x4_t v;
@@ -867,12 +876,11 @@ __global__ __launch_bounds__(512) void conv_p16c4_kernel(const ConvP16Params p) 
                     if constexpr (!HSTORE) fmax_ = fmaxf(fmax_, fabsf(v[e]));
                 }
                 if constexpr (HSTORE) {
-                    half4_t hv;
 #pragma unroll
-                    for (int e = 0; e < 4; e++) hv[e] = (_Float16)v[e];
-                    if (ok) *reinterpret_cast<half4_t*>(out + obase + fm * 16) = hv;
+                    for (int e = 0; e < 4; e++) hv[fm * 4 + e] = (_Float16)v[e];
+                    if (fm == 1 && ok) *reinterpret_cast<half8_t*>(out + obase) = hv;
                 } else {
-                    if (ok) *reinterpret_cast<f32x4_t*>(out + obase + fm * 16) = v;
+                    if (ok) *reinterpret_cast<f32x4_t*>(out + obase + fm * CHF) = v;
                 }
             }
             vmax = fmaxf(vmax, ok ? fmax_ : 0.f);
@@ -1011,7 +1019,7 @@ int P16_NAME(launch_conv_p16)(const ConvP16Params& p, hipStream_t s) {
     const int cpb = 32 * e->wm, twg = (4 / e->wm) * e->tw;
     // what the kernel's indexing assumes
     if (p.cin_chunks < 1 || p.in_cp != p.cin_chunks * KC || p.cout_blocks < 1 || p.mfrags < p.cout_blocks * 2 * e->wm ||
-        p.tiles_x * twg < p.npos_x || p.tiles_y * p.tile_h < p.npos_y || p.out_cp < p.cout_blocks * cpb || p.out_cp % 4 != 0 ||
+        p.tiles_x * twg < p.npos_x || p.tiles_y * p.tile_h < p.npos_y || p.out_cp < p.cout_blocks * cpb || (p.out_cp * ESZ) % 16 != 0 ||
         (p.res && (p.res_cp < p.cout_blocks * cpb || (p.res_cp * ESZ) % 16 != 0)) || p.nreset < 0 || p.nreset > 4 || p.pos_groups < 1 ||
         p.pos_groups > p.tiles_x * p.tiles_y || (p.f16 != 0) != HSTORE ||
         // (a tile's residual tile may not be overwritten while its epilogue reads it: the next one comes a stage later)
@@ -1068,7 +1076,7 @@ int P16_NAME(launch_tconv_p16)(const ConvP16Params& p, hipStream_t s) {
     if (!e) return -1;
     const int cpb = 32 * e->wm, twg = (4 / e->wm) * e->tw;
     if (p.cin_chunks < 1 || p.in_cp != p.cin_chunks * KC || p.cout_blocks < 1 || p.mfrags < p.cout_blocks * 2 * e->wm ||
-        p.tiles_x * twg < p.npos_x || p.tiles_y * p.tile_h < p.npos_y || p.out_cp < p.cout_blocks * cpb || p.out_cp % 4 != 0 || p.res || p.stride != 1 ||
+        p.tiles_x * twg < p.npos_x || p.tiles_y * p.tile_h < p.npos_y || p.out_cp < p.cout_blocks * cpb || (p.out_cp * ESZ) % 16 != 0 || p.res || p.stride != 1 ||
         p.nreset < 0 || p.nreset > 4 || p.pos_groups < 1 || p.pos_groups > p.tiles_x * p.tiles_y || (p.f16 != 0) != HSTORE ||
         p.rcp_tiles_x != 1.0f / (float)p.tiles_x || p.tiles_x * p.tiles_y > 4000000)
         return -5;
@@ -1102,7 +1110,7 @@ int P16_NAME(launch_conv_p16c4)(const ConvP16Params& p, int k, hipStream_t s) {
     const C4Entry* e = find_c4entry(p, k);
     if (!e) return -1;
     if (p.in_cp != 4 || p.cin_chunks != 1 || p.cout_blocks < 1 || p.mfrags < p.cout_blocks * 2 || p.wm != 1 || p.stride != 1 || p.res ||
-        p.tiles_x * 4 * e->tw < p.npos_x || p.tiles_y * e->th < p.npos_y || p.out_cp < p.cout_blocks * 32 || p.out_cp % 4 != 0 ||
+        p.tiles_x * 4 * e->tw < p.npos_x || p.tiles_y * e->th < p.npos_y || p.out_cp < p.cout_blocks * 32 || (p.out_cp * ESZ) % 16 != 0 ||
         p.nreset < 0 || p.nreset > 4 || p.pos_groups < 1 || p.pos_groups > p.tiles_x * p.tiles_y || (p.f16 != 0) != HSTORE ||
         p.rcp_tiles_x != 1.0f / (float)p.tiles_x || p.tiles_x * p.tiles_y > 4000000)
         return -5;

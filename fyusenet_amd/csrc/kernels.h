@@ -200,6 +200,9 @@ struct ConvP16Params {
 #endif
     Act act;
 };
+// Output channel held by row `row` (0..15) of packed weight fragment `mf` when a wave holds groups of `fm` fragments: the
+// rows a lane ends up with (four consecutive ones of every fragment) are 4*fm consecutive channels.
+inline int p16_row_channel(int mf, int row, int fm) { return (mf / fm) * 16 * fm + 4 * fm * (row / 4) + 4 * (mf % fm) + (row % 4); }
 bool conv_p16_supported(int k, int stride, int dil, int in_cp, int cout, int out_cp, bool f16);
 int conv_p16_tile_count();
 void conv_p16_tile(int index, int* th, int* tw, int* stride, int* wm);

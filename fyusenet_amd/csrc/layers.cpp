@@ -1202,7 +1202,7 @@ class ConvLayer : public Layer {
             for (int mf = 0; mf < pp.mfrags; mf++) {
                 uint16_t* base = pack.data() + (((size_t)st * pp.mfrags + mf) * npl) * 64 * 8;
                 for (int lane = 0; lane < 64; lane++) {
-                    const int o = mf * 16 + (lane & 15), pi = 4 * st + (lane >> 4);
+                    const int o = p16_row_channel(mf, lane & 15, pp.f16 ? 2 : 1), pi = 4 * st + (lane >> 4);
                     const int ky = pi / ppr, kx0 = 2 * (pi % ppr);
                     if (o >= oc || ky >= k) continue;
                     for (int j = 0; j < 8; j++) {
@@ -1229,7 +1229,7 @@ class ConvLayer : public Layer {
                 for (int mf = 0; mf < pp.mfrags; mf++) {
                     uint16_t* base = pack.data() + (((size_t)(chunk * 9 + tap) * pp.mfrags + mf) * npl) * 64 * 8;
                     for (int lane = 0; lane < 64; lane++) {
-                        const int o = mf * 16 + (lane & 15);
+                        const int o = p16_row_channel(mf, lane & 15, pp.f16 ? 2 : 1);
                         if (o >= oc) continue;
                         for (int j = 0; j < 8; j++) {
                             const int ci = chunk * 32 + 8 * (lane >> 4) + j;
@@ -1811,7 +1811,7 @@ class TransConvLayer : public Layer {
                 for (int mf = 0; mf < pp.mfrags; mf++) {
                     uint16_t* base = pack.data() + (((size_t)(chunk * 9 + t) * pp.mfrags + mf) * npl) * 64 * 8;
                     for (int lane = 0; lane < 64; lane++) {
-                        const int o = mf * 16 + (lane & 15);
+                        const int o = p16_row_channel(mf, lane & 15, pp.f16 ? 2 : 1);
                         if (o >= oc) continue;
                         for (int j = 0; j < 8; j++) {
                             const int ci = chunk * 32 + 8 * (lane >> 4) + j;
