@@ -927,6 +927,7 @@ constexpr P16Entry entry() {
 }
 const P16Entry kEntries[] = {
     entry<8, 10, 1, 4>(), entry<10, 8, 1, 4>(), entry<8, 8, 1, 4>(), entry<8, 6, 1, 4>(), entry<4, 8, 1, 4>(), entry<4, 4, 1, 4>(),
+    entry<8, 8, 1, 2>(), entry<8, 6, 1, 2>(), entry<4, 8, 1, 2>(),
     entry<10, 8, 2, 4>(), entry<8, 10, 2, 4>(), entry<8, 8, 2, 4>(),
     entry<8, 6, 2, 2>(), entry<4, 8, 2, 2>(), entry<8, 4, 2, 2>(),
 };

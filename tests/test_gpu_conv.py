@@ -270,6 +270,10 @@ P16_CASES = [
     (32, 128, 66, 68, 1, "4,4,4", {"residual": (A.NONE, True), "bn": True}),       # one chunk and a residual input: one workgroup per tile
     (32, 64, 150, 130, 2, "4,8,2", {"bn": True}),                                  # one chunk, 380 tiles: a stage per tile, weight ring wraps
     (96, 128, 82, 66, 2, "8,8,4", {"pad_out": 1}),                                 # three chunks per tile, odd stage count per tile
+    (64, 64, 40, 37, 1, "8,8,2", {"bn": True, "residual": (A.RELU, True)}),        # stride 1, 64-channel blocks: two tiles side by side
+    (32, 192, 21, 50, 1, "8,6,2", {}),
+    (64, 64, 90, 100, 1, "4,8,2", {"residual": (A.NONE, False)}),                  # 161 tiles x 1 block
+    (64, 64, 256, 256, 1, None, {}),                                               # BASELINE's single-layer case
 ]
 
 
