@@ -914,6 +914,226 @@ __global__ __launch_bounds__(512) void conv_p16c4_kernel(const ConvP16Params p) 
     if (p.out_amax) range_publish_waves(p.out_amax, vmax, range_box, 4);
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// 1x1 and 3x3 convolutions (stride 1) on layers with few positions and many input channels (the last stages of a
+// classification net at batch 1: 14x14 or 7x7 positions, 256 to 1024 input channels).  There the general kernel cuts
+// the reduction into slices for separate workgroups and sums them in a second launch.  Here a workgroup owns a tile of
+// 4x4 positions and 16*FM output channels and keeps the tile's whole reduction resident in LDS: the staging waves fetch
+// all 4*CPW chunks of 32 channels at once (one memory round trip), the four MFMA waves take every fourth chunk each --
+// a stream of CPW*NTAPS steps, fully unrolled, weights through a register ring, B fragments read three steps ahead --
+// and add their accumulators through LDS; wave 0 runs the epilogue.  Small tiles make many workgroups (13 tiles x 16
+// blocks of 16 channels for 1024 -> 256 at 14x14), so the layer's activations and weights are pulled through many CUs.
+// Weights: [cout block][wave][step][fragment][plane][lane][8 halves], the wave's steps being (chunk wave + 4*i, tap).
+template <int NTAPS, int CPW>
+struct GeoR {
+    static constexpr int TH = 4, TW = 4, KH = (NTAPS == 9) ? 2 : 0;
+    static constexpr int HW = TW + KH, HH = TH + KH;
+    static constexpr int ROW_PITCH = HW * PITCH + p16_row_pad(TH, TW, 1, 1, HW);
+    static constexpr int PLANE = HH * ROW_PITCH;
+    static constexpr int BUFC = NPL * PLANE;            // one chunk of the tile
+    static constexpr int NCH = 4 * CPW;                 // chunks of the layer
+    static constexpr int NITEMS = HH * HW * (KC / 8);   // staging items per chunk
+    static constexpr int TOTAL = NITEMS * NCH, NB = (TOTAL + 255) / 256;
+    static constexpr int STEPS = CPW * NTAPS;           // per MFMA wave
+    static constexpr int RPD = STEPS < 8 ? STEPS : 8;   // weight ring depth (steps; the step loop is unrolled, so any depth fits)
+    static constexpr int BD = STEPS < 4 ? STEPS : 4;    // B fragment ring depth (steps)
+    static constexpr int RED_OFF = NCH * BUFC;          // [wave 1..3][fragment][lane] x 16 bytes, then scale and bias
+    static constexpr int tap_off(int t) { return NTAPS == 9 ? (t / 3) * ROW_PITCH + (t % 3) * PITCH : 0; }
+    static_assert(NTAPS == 1 || NTAPS == 9, "1x1 or 3x3");
+};
+
+template <int NTAPS, int CPW, int FM>
+__global__ __launch_bounds__(512) void conv_kr16_kernel(const ConvP16Params p) {
+    using G = GeoR<NTAPS, CPW>;
+    constexpr int RPD = G::RPD, BD = G::BD, STEPS = G::STEPS;
+    extern __shared__ __align__(16) unsigned char lds[];
+    __shared__ unsigned range_box[2];
+    if (blockIdx.x == 0) range_clear(p.reset[0], p.reset[1], p.reset[2], p.reset[3], p.nreset);
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int cb = blockIdx.x % p.cout_blocks;
+    const int tile = blockIdx.x / p.cout_blocks;
+    const int tyi = tile / p.tiles_x, txi = tile - tyi * p.tiles_x;
+    if (tid < 2) range_box[tid] = 0u;
+    const unsigned range_bits = p.in_amax ? range_load(p.in_amax) : 0u;
+    constexpr int red_off = G::RED_OFF;
+    constexpr int sb_off = red_off + 3 * FM * 1024;
+
+    if (wave < 4) {   // ------------------------------------------------------------ staging waves
+        const int stid = tid & 255;
+        const store_t* in = reinterpret_cast<const store_t*>(p.in);
+        struct RawF { float4 a, b; };
+        typedef typename std::conditional<HSTORE, half8_t, RawF>::type raw_t;
+        raw_t raw[G::NB];
+        int l_off[G::NB];
+        bool ok[G::NB];
+        const int y0 = tyi * G::TH + p.in_y0, x0 = txi * G::TW + p.in_x0;
+#pragma unroll
+        for (int i = 0; i < G::NB; i++) {
+            const int idx = stid + i * 256;
+            const int chunk = idx / G::NITEMS, rem = idx - chunk * G::NITEMS;
+            const int pix = rem >> 2, g = rem & 3;
+            const int py = pix / G::HW, px = pix - py * G::HW;
+            l_off[i] = idx < G::TOTAL ? chunk * G::BUFC + py * G::ROW_PITCH + px * PITCH + g * 16 : -1;
+            int gy = y0 + py, gx = x0 + px;
+            if (p.in_clamp) {
+                gy = min(max(gy, 0), p.in_hp - 1);
+                gx = min(max(gx, 0), p.in_wp - 1);
+            }
+            ok[i] = idx < G::TOTAL && (unsigned)gy < (unsigned)p.in_hp && (unsigned)gx < (unsigned)p.in_wp;
+            const store_t* src = in + (ok[i] ? (gy * p.in_wp + gx) * p.in_cp + chunk * KC + g * 8 : 0);
+            if constexpr (HSTORE) {
+                raw[i] = *reinterpret_cast<const half8_t*>(src);
+            } else {
+                raw[i].a = *reinterpret_cast<const float4*>(src);
+                raw[i].b = *reinterpret_cast<const float4*>(src + 4);
+            }
+        }
+        float in_scale = 1.f, inv_unused;
+        if (p.in_amax) in_scale = range_scale(range_after_act(range_reduce(range_bits), p.act), &inv_unused);
+        if (stid < 16 * FM) {
+            reinterpret_cast<float*>(lds + sb_off)[stid] = p.scale[cb * 16 * FM + stid];
+            reinterpret_cast<float*>(lds + sb_off)[16 * FM + stid] = p.bias[cb * 16 * FM + stid];
+        }
+#pragma unroll
+        for (int i = 0; i < G::NB; i++) {
+            if (l_off[i] < 0) continue;
+            if constexpr (HSTORE) {
+                half8_t v;
+#pragma unroll
+                for (int e = 0; e < 8; e++) v[e] = ok[i] ? (_Float16)act_p16((float)raw[i][e], p.act) : (_Float16)0.f;
+                *reinterpret_cast<half8_t*>(lds + l_off[i]) = v;
+            } else {
+                const float r[8] = {raw[i].a.x, raw[i].a.y, raw[i].a.z, raw[i].a.w, raw[i].b.x, raw[i].b.y, raw[i].b.z, raw[i].b.w};
+                half8_t hi, lo;
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    const float v = ok[i] ? act_p16(r[e], p.act) * in_scale : 0.f;
+                    hi[e] = (_Float16)v;
+                    lo[e] = (_Float16)(v - (float)hi[e]);
+                }
+                *reinterpret_cast<half8_t*>(lds + l_off[i]) = hi;
+                *reinterpret_cast<half8_t*>(lds + G::PLANE + l_off[i]) = lo;
+            }
+        }
+        lds_barrier();   // the tile is staged
+        lds_barrier();   // the MFMA waves have left their accumulators for wave 0
+        return;
+    }
+
+    // ---------------------------------------------------------------------- MFMA waves
+    const int w = wave - 4;
+    const int mq = lane & 15, kq = lane >> 4;
+    const int bbase = (mq / G::TW) * G::ROW_PITCH + (mq % G::TW) * PITCH + kq * 16 + w * G::BUFC;   // chunk `w` of the tile
+    constexpr unsigned wstep = FM * NPL * 1024;
+    const unsigned char* wbase = reinterpret_cast<const unsigned char*>(p.wpack) + (size_t)((cb * 4 + w) * STEPS) * wstep + lane * 16;
+    half8_t a_q[RPD][FM][NPL];
+#pragma unroll
+    for (int d = 0; d < RPD - 1; d++)
+#pragma unroll
+        for (int fm = 0; fm < FM; fm++)
+#pragma unroll
+            for (int pl = 0; pl < NPL; pl++) a_q[d][fm][pl] = *reinterpret_cast<const half8_t*>(wbase + (size_t)d * wstep + (fm * NPL + pl) * 1024);
+#pragma unroll
+    for (int fm = 0; fm < FM; fm++)
+#pragma unroll
+        for (int pl = 0; pl < NPL; pl++) a_q[RPD - 1][fm][pl] = a_q[0][fm][pl];   // (defined; replaced during the first step)
+    f32x4_t acc[FM];
+#pragma unroll
+    for (int fm = 0; fm < FM; fm++) acc[fm] = (f32x4_t)(0.f);
+    float inv_in_scale = 1.f;
+    if (p.in_amax) (void)range_scale(range_after_act(range_reduce(range_bits), p.act), &inv_in_scale);
+    const float acc_mul = p.acc_mul * inv_in_scale;
+
+    lds_barrier();   // the tile is staged
+    // B fragment of step s: chunk w + 4*(s / NTAPS), tap s % NTAPS
+    auto b_off = [&](int s) { return (s / NTAPS) * 4 * G::BUFC + G::tap_off(s % NTAPS); };
+    half8_t b[BD][NPL];
+#pragma unroll
+    for (int s = 0; s < BD - 1; s++)
+#pragma unroll
+        for (int pl = 0; pl < NPL; pl++) b[s][pl] = *reinterpret_cast<const half8_t*>(lds + bbase + b_off(s) + pl * G::PLANE);
+#pragma unroll
+    for (int s = 0; s < STEPS; s++) {
+        const int d = s % RPD, dload = (s + RPD - 1) % RPD, bs = s % BD, bload = (s + BD - 1) % BD;
+        // the weights of step s + RPD - 1 and the fragment of step s + BD - 1 go into the slots the previous step left
+        if (s + RPD - 1 < STEPS) {
+#pragma unroll
+            for (int fm = 0; fm < FM; fm++)
+#pragma unroll
+                for (int pl = 0; pl < NPL; pl++)
+                    a_q[dload][fm][pl] = *reinterpret_cast<const half8_t*>(wbase + (size_t)(s + RPD - 1) * wstep + (fm * NPL + pl) * 1024);
+        }
+        if (s + BD - 1 < STEPS) {
+#pragma unroll
+            for (int pl = 0; pl < NPL; pl++) b[bload][pl] = *reinterpret_cast<const half8_t*>(lds + bbase + b_off(s + BD - 1) + pl * G::PLANE);
+        }
+#pragma unroll
+        for (int i = 0; i < NPASS * FM; i++) {
+            const int kind = i / FM, fm = i % FM;
+            const int apl = (kind == 1) ? 1 : 0, bpl = (kind == 2) ? 1 : 0;
+            acc[fm] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_q[d][fm][apl], b[bs][bpl], acc[fm], 0, 0, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    // the four partial sums meet in wave 0
+    if (w > 0) {
+#pragma unroll
+        for (int fm = 0; fm < FM; fm++) *reinterpret_cast<f32x4_t*>(lds + red_off + ((w - 1) * FM + fm) * 1024 + lane * 16) = acc[fm];
+    }
+    lds_barrier();
+    if (w > 0) return;
+    float vmax = 0.f;
+    {
+        const float* sb = reinterpret_cast<const float*>(lds + sb_off);
+        store_t* out = reinterpret_cast<store_t*>(p.out);
+        const store_t* res = reinterpret_cast<const store_t*>(p.res);
+        const int py = tyi * G::TH + mq / G::TW, px = txi * G::TW + mq % G::TW;
+        const bool okp = py < p.npos_y && px < p.npos_x;
+#pragma unroll
+        for (int fm = 0; fm < FM; fm++) {
+            f32x4_t v = acc[fm];
+#pragma unroll
+            for (int o = 0; o < 3; o++) v += *reinterpret_cast<const f32x4_t*>(lds + red_off + (o * FM + fm) * 1024 + lane * 16);
+            const f32x4_t sc = *reinterpret_cast<const f32x4_t*>(sb + fm * 16 + kq * 4);
+            const f32x4_t bi = *reinterpret_cast<const f32x4_t*>(sb + 16 * FM + fm * 16 + kq * 4);
+            const int ch = cb * 16 * FM + fm * 16 + kq * 4;
+#pragma unroll
+            for (int e = 0; e < 4; e++) v[e] = v[e] * (sc[e] * acc_mul) + bi[e];
+            if (res && okp) {
+                const store_t* rp = res + ((size_t)(p.res_off_y + py) * p.res_wp + p.res_off_x + px) * p.res_cp + ch;
+                f32x4_t rv;
+                if constexpr (HSTORE) {
+                    const half4_t rh = *reinterpret_cast<const half4_t*>(rp);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) rv[e] = (float)rh[e];
+                } else {
+                    rv = *reinterpret_cast<const f32x4_t*>(rp);
+                }
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    float r = p.res_relu ? fmaxf(rv[e], 0.f) : rv[e];
+                    if (p.res_scale) r *= sc[e];
+                    v[e] += r;
+                }
+            }
+            store_t* op = out + ((size_t)(p.out_off_y + py) * p.out_wp + p.out_off_x + px) * p.out_cp + ch;
+            if constexpr (HSTORE) {
+                half4_t hv;
+#pragma unroll
+                for (int e = 0; e < 4; e++) hv[e] = (_Float16)v[e];
+                if (okp) *reinterpret_cast<half4_t*>(op) = hv;
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; e++) vmax = fmaxf(vmax, okp ? fabsf(v[e]) : 0.f);
+                if (okp) *reinterpret_cast<f32x4_t*>(op) = v;
+            }
+        }
+    }
+    if (p.out_amax) range_publish_waves(p.out_amax, vmax, range_box, 1);
+}
+
 typedef void (*p16_fn)(const ConvP16Params);
 struct P16Entry {
     int th, tw, stride, wm;
@@ -956,6 +1176,20 @@ struct C4Entry {
 template <int K, int TH, int TW>
 constexpr C4Entry c4entry() { return C4Entry{K, TH, TW, conv_p16c4_kernel<K, TH, TW>, (size_t)GeoC4<K, TH, TW>::BUF, GeoC4<K, TH, TW>::NS}; }
 const C4Entry kC4Entries[] = {c4entry<9, 8, 8>(), c4entry<9, 4, 8>(), c4entry<9, 8, 4>()};
+struct KREntry {
+    int taps, cpw, fm;
+    p16_fn fn;
+    size_t lds;
+};
+template <int NTAPS, int CPW, int FM>
+constexpr KREntry krentry() {
+    using G = GeoR<NTAPS, CPW>;
+    return KREntry{NTAPS, CPW, FM, conv_kr16_kernel<NTAPS, CPW, FM>, (size_t)(G::RED_OFF + 3 * FM * 1024 + 2 * 16 * FM * 4)};
+}
+const KREntry kKREntries[] = {
+    krentry<1, 2, 1>(), krentry<1, 4, 1>(), krentry<1, 8, 1>(), krentry<1, 2, 2>(), krentry<1, 4, 2>(), krentry<1, 8, 2>(),
+    krentry<9, 2, 1>(), krentry<9, 4, 1>(), krentry<9, 2, 2>(), krentry<9, 4, 2>(),
+};
 }  // namespace
 
 // Host entry points.  The fp32 unit holds the public ones and hands launches on fp16 tensors (p.f16) to the other
@@ -970,6 +1204,8 @@ size_t tconv_p16_lds_bytes_half(const ConvP16Params& p);
 int launch_tconv_p16_half(const ConvP16Params& p, hipStream_t s);
 size_t conv_p16c4_lds_bytes_half(const ConvP16Params& p, int k);
 int launch_conv_p16c4_half(const ConvP16Params& p, int k, hipStream_t s);
+size_t conv_kr16_lds_bytes_half(const ConvP16Params& p, int k);
+int launch_conv_kr16_half(const ConvP16Params& p, int k, hipStream_t s);
 
 int conv_p16_tile_count() { return (int)(sizeof(kEntries) / sizeof(kEntries[0])); }
 void conv_p16_tile(int index, int* th, int* tw, int* stride, int* wm) {
@@ -992,11 +1228,46 @@ int conv_p16c4_tile_count() { return (int)(sizeof(kC4Entries) / sizeof(kC4Entrie
 void conv_p16c4_tile(int index, int* k, int* th, int* tw, int* steps) {
     *k = kC4Entries[index].k; *th = kC4Entries[index].th; *tw = kC4Entries[index].tw; *steps = kC4Entries[index].steps;
 }
+int conv_kr16_variant_count() { return (int)(sizeof(kKREntries) / sizeof(kKREntries[0])); }
+void conv_kr16_variant(int index, int* taps, int* chunks, int* fm) {
+    *taps = kKREntries[index].taps; *chunks = 4 * kKREntries[index].cpw; *fm = kKREntries[index].fm;
+}
 bool conv_p16c4_supported(int k, int stride, int dil, int in_cp, int cout, int out_cp, bool f16) {
     (void)f16;
     return k == 9 && stride == 1 && dil == 1 && in_cp == 4 && cout % 32 == 0 && out_cp % 4 == 0 && out_cp >= cout;
 }
 #endif
+
+static const KREntry* find_krentry(const ConvP16Params& p, int k) {
+    for (const KREntry& c : kKREntries)
+        if (c.taps == k * k && c.cpw * 4 == p.cin_chunks && c.fm == p.wm) return &c;
+    return nullptr;
+}
+size_t P16_NAME(conv_kr16_lds_bytes)(const ConvP16Params& p, int k) {
+#if !FYN_P16_HALF
+    if (p.f16) return conv_kr16_lds_bytes_half(p, k);
+#endif
+    const KREntry* e = find_krentry(p, k);
+    return e ? e->lds : 0;
+}
+// The K-resident form: k = 1 or 3, stride 1; tiles of 4x4 positions, blocks of 16*p.wm output channels (p.wm = 1 or 2),
+// p.cin_chunks = 8, 16 or 32 (3x3: 8 or 16); in_y0/in_x0 = input padding - (k-1)/2; one workgroup per tile and block
+int P16_NAME(launch_conv_kr16)(const ConvP16Params& p, int k, hipStream_t s) {
+#if !FYN_P16_HALF
+    if (p.f16) return launch_conv_kr16_half(p, k, s);
+#endif
+    const KREntry* e = find_krentry(p, k);
+    if (!e) return -1;
+    if (p.in_cp != p.cin_chunks * KC || p.cout_blocks < 1 || p.mfrags != p.cout_blocks * e->fm || p.stride != 1 || p.tile_h != 4 || p.tile_w != 4 ||
+        p.tiles_x * 4 < p.npos_x || p.tiles_y * 4 < p.npos_y || p.out_cp < p.cout_blocks * 16 * e->fm || (p.out_cp * ESZ) % 16 != 0 ||
+        (p.res && (p.res_cp < p.cout_blocks * 16 * e->fm || (p.res_cp * ESZ) % 16 != 0)) || p.nreset < 0 || p.nreset > 4 || (p.f16 != 0) != HSTORE ||
+        p.tiles_x < 1 || p.tiles_y < 1 || (long long)p.tiles_x * p.tiles_y * p.cout_blocks > 65535)
+        return -5;
+    if (e->lds > 160 * 1024) return -2;
+    if (ensure_lds(reinterpret_cast<const void*>(e->fn), e->lds) != 0) return -2;
+    hipLaunchKernelGGL(e->fn, dim3(p.tiles_x * p.tiles_y * p.cout_blocks), dim3(512), e->lds, s, p);
+    return hipGetLastError() == hipSuccess ? 0 : -3;
+}
 
 static const P16Entry* find_entry(const ConvP16Params& p) {
     for (const P16Entry& c : kEntries)

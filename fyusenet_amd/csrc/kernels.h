@@ -223,6 +223,13 @@ int conv_p16c4_tile_count();
 void conv_p16c4_tile(int index, int* k, int* th, int* tw, int* steps);
 size_t conv_p16c4_lds_bytes(const ConvP16Params& p, int k);
 int launch_conv_p16c4(const ConvP16Params& p, int k, hipStream_t s);
+// the K-resident form for layers with few positions (k = 1 or 3, stride 1) on the same parameters: tiles of 4x4
+// positions, blocks of 16*wm output channels, the whole reduction of a tile in LDS; wpack: [cout block][wave 0..3][step]
+// [fragment][plane][lane][8 halves], a wave's steps being (chunk wave + 4*i, tap)
+int conv_kr16_variant_count();
+void conv_kr16_variant(int index, int* taps, int* chunks, int* fm);   // compiled combinations: kernel taps, 32-channel chunks, fragments per block
+size_t conv_kr16_lds_bytes(const ConvP16Params& p, int k);
+int launch_conv_kr16(const ConvP16Params& p, int k, hipStream_t s);
 // the K x K convolution (K = 3 or 9, stride 1) between fp16 tensors on the same parameters (conv_h16.hip): 128 output
 // channels per workgroup, two tiles of tile_h x tile_w positions side by side; wpack: [(chunk*K + ky)*K + kx][cout
 // fragment of 16][lane][8 halves], one plane

@@ -1193,6 +1193,114 @@ class ConvLayer : public Layer {
         FYN_HIP(hipMemcpyAsync(p16_wpack_dev, pack.data(), pack.size() * 2, hipMemcpyHostToDevice, net->stream));
         FYN_HIP(hipStreamSynchronize(net->stream));
     }
+    // the K-resident form for layers with few positions and many input channels (conv_p16.hip, conv_kr16_kernel)
+    void setup_kr16(const TView& in_v, const TView& out_v, const TView* res_v, int res_relu, int res_scale) {
+        ConvP16Params q{};
+        q.in = in_v.ptr; q.out = out_v.ptr; q.res = res_v ? res_v->ptr : nullptr;
+        q.in_hp = in_v.hp(); q.in_wp = in_v.wp(); q.in_cp = in_v.cp;
+        q.stride = 1;
+        q.in_y0 = q.in_x0 = in_v.pad - (k - 1) / 2;
+        q.in_clamp = clamp ? 1 : 0;
+        q.npos_y = oh; q.npos_x = ow;
+        q.out_wp = out_v.wp(); q.out_cp = out_v.cp; q.out_off_y = q.out_off_x = out_v.pad;
+        if (res_v) { q.res_wp = res_v->wp(); q.res_cp = res_v->cp; q.res_off_y = q.res_off_x = res_v->pad; }
+        q.res_relu = res_relu; q.res_scale = res_scale;
+        q.cin_chunks = in_v.cp / 32;
+        q.f16 = out_v.f16 ? 1 : 0;
+        q.tile_h = q.tile_w = 4;
+        q.tiles_x = (ow + 3) / 4; q.tiles_y = (oh + 3) / 4;
+        q.rcp_tiles_x = 1.0f / (float)q.tiles_x;
+        q.pos_groups = q.tiles_x * q.tiles_y;
+        q.scale = scale_dev; q.bias = bias_dev;
+        q.acc_mul = 1.f;
+        q.act = act();
+        int want_fm = 0;   // FYNHIP_KR16_FM (tests): fragments per block of output channels
+        if (const char* e = getenv("FYNHIP_KR16_FM")) want_fm = atoi(e);
+        std::vector<ConvP16Params> cands;
+        for (int i = 0; i < conv_kr16_variant_count(); i++) {
+            int taps, chunks, fm;
+            conv_kr16_variant(i, &taps, &chunks, &fm);
+            if (taps != k * k || chunks != q.cin_chunks || oc % (16 * fm) != 0 || (want_fm && fm != want_fm)) continue;
+            ConvP16Params c = q;
+            c.wm = fm;
+            c.cout_blocks = oc / (16 * fm);
+            c.mfrags = oc / 16;
+            const size_t lds = conv_kr16_lds_bytes(c, k);
+            if (lds == 0 || lds > 160 * 1024 || (long long)c.pos_groups * c.cout_blocks > 65535) continue;
+            cands.push_back(c);
+        }
+        if (cands.empty()) return;
+        // (the same size for every candidate: cout blocks x 4 waves x steps x fragments x planes)
+        const size_t halves = (size_t)(oc / 16) * 4 * (q.cin_chunks / 4) * k * k * (q.f16 ? 1 : 2) * 64 * 8;
+        p16_wpack_dev = net->dev_alloc(halves * 2, true);
+        for (ConvP16Params& c : cands) c.wpack = p16_wpack_dev;
+        const bool always = getenv("FYNHIP_FORCE_KR16_CONV") != nullptr;
+        const char* at = getenv("FYNHIP_AUTOTUNE");
+        int pick = 0;
+        char key[160];
+        snprintf(key, sizeof(key), "kr16:k%d:%dx%d:%dx%d:r%d:e%d:h%d", k, d.in_channels, oc, oh, ow, res_v ? 1 : 0, clamp ? 1 : 0, q.f16);
+        int cached[3] = {0, 0, 0};
+        if (!want_fm && tune_cache_triple(key, cached)) {
+            pick = -1;
+            if (cached[0] || always)
+                for (size_t i = 0; i < cands.size(); i++)
+                    if (cands[i].wm == cached[1]) pick = (int)i;
+            if (always && pick < 0) pick = 0;
+        } else if (!(at && at[0] == '0')) {
+            float best = 1e30f, t_other = 1e30f;
+            for (int rep = 0; rep < 3; rep++) {
+                for (size_t i = 0; i < cands.size(); i++) {
+                    const float t = time_calls(net, [&]() {
+                        if (launch_conv_kr16(cands[i], k, net->stream) != 0) fail(FYN_ERR_DEVICE, "K-resident convolution launch failed while tuning");
+                    }, 10);
+                    if (t < best) { best = t; pick = (int)i; }
+                }
+                t_other = std::min(t_other, time_launch(net, launch, 10));
+            }
+            if (getenv("FYNHIP_TUNE_VERBOSE"))
+                fprintf(stderr, "[tune] %dx%d on %d channels, %dx%d positions: K-resident form (%d-channel blocks) %.1f us, general kernel %.1f us\n", k, k,
+                        d.in_channels, oh, ow, 16 * cands[pick].wm, best * 1e3f, t_other * 1e3f);
+            const bool win = best < t_other;
+            if (!want_fm) tune_cache_store_triple(key, win ? 1 : 0, cands[pick].wm, 0);
+            if (!win && !always) pick = -1;
+        }
+        if (pick >= 0) {
+            p16 = true; kr16 = true;
+            pp = cands[pick];
+        } else {
+            net->dev_free(p16_wpack_dev);
+            p16_wpack_dev = nullptr;
+        }
+    }
+    // weights of that form: [cout block][wave][step][fragment][plane][lane][8 halves]; step s of wave w = (chunk w + 4*(s / taps), tap s % taps)
+    void pack_kr16(const float* w, float wmul) {
+        const int cin = d.in_channels, taps = k * k, fm_n = pp.wm, npl = pp.f16 ? 1 : 2;
+        const int steps = pp.cin_chunks / 4 * taps;
+        std::vector<uint16_t> pack((size_t)pp.cout_blocks * 4 * steps * fm_n * npl * 64 * 8, 0);
+        for (int cb = 0; cb < pp.cout_blocks; cb++)
+            for (int wv = 0; wv < 4; wv++)
+                for (int st = 0; st < steps; st++) {
+                    const int chunk = wv + 4 * (st / taps), tap = st % taps;
+                    for (int fm = 0; fm < fm_n; fm++) {
+                        uint16_t* base = pack.data() + ((((size_t)(cb * 4 + wv) * steps + st) * fm_n + fm) * npl) * 64 * 8;
+                        for (int lane = 0; lane < 64; lane++) {
+                            const int o = (cb * fm_n + fm) * 16 + (lane & 15);
+                            if (o >= oc) continue;
+                            for (int j = 0; j < 8; j++) {
+                                const int ci = chunk * 32 + 8 * (lane >> 4) + j;
+                                if (ci >= cin) continue;
+                                const float v = w[((size_t)o * taps + tap) * cin + ci] * wmul;
+                                const uint16_t hi = f2h_bits(v);
+                                base[(size_t)lane * 8 + j] = hi;
+                                if (npl == 2) base[(size_t)(64 + lane) * 8 + j] = f2h_bits(v - h2f(hi));
+                            }
+                        }
+                    }
+                }
+        FYN_HIP(hipStreamSynchronize(net->stream));
+        FYN_HIP(hipMemcpyAsync(p16_wpack_dev, pack.data(), pack.size() * 2, hipMemcpyHostToDevice, net->stream));
+        FYN_HIP(hipStreamSynchronize(net->stream));
+    }
     // weights of that form: [step][cout fragment of 16][plane][lane][8 halves]; lane = (channel lane%16, tap pair 4*step + lane/16)
     void pack_c4(const float* w, float wmul) {
         const int cin = d.in_channels, ppr = (k + 1) / 2;
@@ -1449,15 +1557,23 @@ class ConvLayer : public Layer {
             // the 16-position-fragment forms, each against the tuned launch of the general kernel: for wide fp16 layers the
             // one with 64-channel wave tiles first, then the 3x3 form, then the small-input form
             const bool same_storage = in_v.f16 == out_v.f16 && (!res_v || res_v->f16 == out_v.f16);
-            if (!frac_shift && same_storage && conv_h16_supported(k, stride, dil, in_v.cp, oc, out_v.cp, out_v.f16 != 0) && d.in_channels == in_v.cp &&
+            const bool only_kr = getenv("FYNHIP_FORCE_KR16_CONV") != nullptr;   // (tests: the K-resident form or nothing)
+            if (!only_kr && !frac_shift && same_storage && conv_h16_supported(k, stride, dil, in_v.cp, oc, out_v.cp, out_v.f16 != 0) && d.in_channels == in_v.cp &&
                 (!res_v || res_v->cp >= oc) && !getenv("FYNHIP_NO_P16_CONV") && !getenv("FYNHIP_NO_H16_CONV"))
                 setup_h16(in_v, out_v, res_v, res_relu, res_scale);
-            if (!p16 && !frac_shift && same_storage && !sc.in_sub && conv_p16_supported(k, stride, dil, in_v.cp, oc, out_v.cp, out_v.f16 != 0) &&
+            if (!only_kr && !p16 && !frac_shift && same_storage && !sc.in_sub && conv_p16_supported(k, stride, dil, in_v.cp, oc, out_v.cp, out_v.f16 != 0) &&
                 d.in_channels == in_v.cp && (!res_v || (res_v->cp >= oc && res_v->cp % 8 == 0)) && !getenv("FYNHIP_NO_P16_CONV"))
                 setup_p16(in_v, out_v, res_v, res_relu, res_scale);
-            if (!p16 && !frac_shift && same_storage && !res_v && conv_p16c4_supported(k, stride, dil, in_v.cp, oc, out_v.cp, out_v.f16 != 0) &&
+            if (!only_kr && !p16 && !frac_shift && same_storage && !res_v && conv_p16c4_supported(k, stride, dil, in_v.cp, oc, out_v.cp, out_v.f16 != 0) &&
                 !getenv("FYNHIP_NO_P16_CONV"))
                 setup_c4(in_v, out_v);
+            // few positions, many input channels: the whole reduction of a 4x4 tile resident in LDS instead of K-split launches
+            if (!p16 && !frac_shift && same_storage && !sc.in_sub && (k == 1 || k == 3) && stride == 1 && dil == 1 && d.in_channels == in_v.cp &&
+                in_v.cp % 128 == 0 && oc % 16 == 0 && out_v.cp >= oc && oh * ow <= 1024 && (!res_v || (res_v->cp >= oc && res_v->cp % 8 == 0)) &&
+                !getenv("FYNHIP_NO_P16_CONV") && !getenv("FYNHIP_NO_KR16_CONV") &&
+                // (a test that forces a variant of the general kernel wants the general kernel)
+                !getenv("FYNHIP_FORCE_KSPLIT") && !getenv("FYNHIP_CONV_TILE") && !getenv("FYNHIP_CONV_KC") && !getenv("FYNHIP_CONV_KC_MAX") && !getenv("FYNHIP_CONV_PD"))
+                setup_kr16(in_v, out_v, res_v, res_relu, res_scale);
         }
         if (direct) {
             scale_dev = static_cast<float*>(net->dev_alloc(padded * sizeof(float)));
@@ -1489,6 +1605,7 @@ class ConvLayer : public Layer {
             const float wmul = weight_prescale(w, (size_t)oc * k * k * d.in_channels);
             pp.acc_mul = pp2.acc_mul = 1.0f / wmul;
             if (c4) pack_c4(w, wmul);
+            else if (kr16) pack_kr16(w, wmul);
             else if (h16) pack_h16(w, wmul);
             else pack_p16(w, wmul);
         } else if (wide && rows) {
@@ -1531,7 +1648,7 @@ class ConvLayer : public Layer {
             return;
         }
         if (p16) {
-            if ((c4 ? launch_conv_p16c4(pp, k, s) : (h16 ? launch_conv_h16(pp, k, s) : launch_conv_p16(pp, s))) != 0 ||
+            if ((c4 ? launch_conv_p16c4(pp, k, s) : (kr16 ? launch_conv_kr16(pp, k, s) : (h16 ? launch_conv_h16(pp, k, s) : launch_conv_p16(pp, s)))) != 0 ||
                 (h16 && h16_two && launch_conv_h16(pp2, k, s) != 0))
                 fail(FYN_ERR_DEVICE, "layer %s: convolution launch failed", d.name);
             return;
@@ -1555,6 +1672,12 @@ class ConvLayer : public Layer {
             snprintf(buf, sizeof(buf), "conv_p16c4 %s (tap pairs of a 4-channel pixel) tile=32x%d(cout x pos) th=%d tw=%d blocks=%d tiles=%d lds=%zu steps=%d",
                      pp.f16 ? "f16" : "f16x2-split", pp.tile_h * pp.tile_w * 4, pp.tile_h, pp.tile_w, pp.pos_groups * pp.cout_blocks, pp.tiles_x * pp.tiles_y * pp.cout_blocks,
                      conv_p16c4_lds_bytes(pp, k), c4_steps);
+            return mode + buf;
+        }
+        if (p16 && kr16) {
+            char buf[220];
+            snprintf(buf, sizeof(buf), "conv_kr16 %s tile=%dx16(cout x pos) K-resident, 4 waves split %d chunks, blocks=%d lds=%zu steps=%d", pp.f16 ? "f16" : "f16x2-split",
+                     16 * pp.wm, pp.cin_chunks, pp.pos_groups * pp.cout_blocks, conv_kr16_lds_bytes(pp, k), pp.cin_chunks / 4 * k * k);
             return mode + buf;
         }
         if (p16 && h16) {
@@ -1593,6 +1716,7 @@ class ConvLayer : public Layer {
     bool c4 = false;              // ... its variant for inputs of at most four channels
     int c4_steps = 0;
     bool h16 = false;             // ... its fp16-storage form for wide layers (conv_h16.hip)
+    bool kr16 = false;            // ... the K-resident form for layers with few positions (conv_p16.hip, conv_kr16_kernel)
     bool h16_two = false;         // ...... as two launches on two bands of rows (pp, pp2)
     ConvP16Params pp{}, pp2{};
     void* p16_wpack_dev = nullptr;

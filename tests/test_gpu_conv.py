@@ -377,6 +377,50 @@ def test_fp16_sixteen_position_fragment_form(case, act, shallow, monkeypatch):
     assert err <= TOL[fa.STORAGE_F16], info
 
 
+KR16_CASES = [
+    # (k, cin, cout, h, w, fragments per block, kw)
+    (1, 1024, 256, 14, 14, 1, {}),                                              # a ResNet stage-3 reduction layer
+    (1, 1024, 64, 7, 9, 2, {"bn": True, "residual": (A.RELU, True)}),           # ragged tiles, residual read in the epilogue
+    (1, 256, 48, 5, 6, 1, {"pad_out": 1}),                                      # two chunks per wave
+    (1, 512, 32, 13, 3, 2, {"bn": True}),
+    (3, 256, 256, 14, 14, 2, {"bn": True}),                                     # a ResNet stage-3 3x3 layer
+    (3, 512, 32, 7, 7, 1, {"residual": (A.NONE, False)}),
+    (3, 256, 48, 9, 6, 1, {"pad_out": 2, "bn": True}),
+    (3, 512, 64, 18, 30, 2, {}),                                                # 40 tiles x 2 blocks
+]
+
+
+@pytest.mark.parametrize("storage", [fa.STORAGE_F32, fa.STORAGE_F16], ids=["f32", "f16"])
+@pytest.mark.parametrize("shallow", [False, True], ids=["deep", "shallow_edge_clamp"])
+@pytest.mark.parametrize("act", [A.RELU, A.LEAKY_RELU], ids=["relu", "leaky"])
+@pytest.mark.parametrize("case", KR16_CASES, ids=lambda c: "k%d_%dx%dx%d_to%d_fm%d" % (c[0], c[1], c[3], c[4], c[2], c[5]))
+def test_reduction_resident_form(case, act, shallow, storage, monkeypatch):
+    """1x1 / 3x3 convolutions on few positions and many input channels with a tile's whole reduction resident in LDS and
+    the four MFMA waves of a workgroup splitting the chunks."""
+    k, cin, cout, h, w, fm, kw = case
+    if shallow and (k == 1 or "residual" in kw or "pad_out" in kw):
+        pytest.skip("the shallow variant is run on the plain 3x3 cases")
+    if act is A.LEAKY_RELU and (cin > 512 or "pad_out" in kw):
+        pytest.skip("activations are varied on some of the cases")
+    monkeypatch.setenv("FYNHIP_FORCE_KR16_CONV", "1")
+    monkeypatch.setenv("FYNHIP_KR16_FM", str(fm))
+    if shallow:
+        kw = dict(kw, deep=False, pad_in=0)
+    if act is A.LEAKY_RELU:
+        kw = dict(kw, leak=0.1)
+    b = conv_builder(k, cout, h, w, cin, 1, 1, act, **kw)
+    wts = conv_block(3000 + cin + k, cout, k, cin, bn=kw.get("bn", False))
+    inputs = [prng.uniform(41 * cin + h, (cin, h, w), -1, 1)]
+    if "residual" in kw:
+        inputs.append(prng.uniform(67, (cout, h, w), -1, 1))
+    got, info = run_single(b, storage, inputs, wts)
+    ref = oracle_single(b, storage, inputs, wts)
+    err = rel_l2(got, ref)
+    print("  ", info, "rel_l2=%.3e" % err, flush=True)
+    assert "conv_kr16" in info and "tile=%dx16" % (16 * fm) in info
+    assert err <= TOL[storage], info
+
+
 ALL_TILES = ["2,2,2,2", "2,2,1,4", "2,1,2,2", "2,1,1,4", "1,2,1,4", "1,1,1,4", "1,1,4,1", "1,1,2,2", "1,2,4,1", "1,3,4,1", "1,4,4,1",
              "1,2,2,2", "1,4,2,2", "1,3,2,2", "1,4,1,4", "1,3,1,4", "1,1,1,1", "1,1,2,1", "1,1,1,2"]
 
