@@ -968,7 +968,9 @@ __global__ __launch_bounds__(512) void conv_kr16_kernel(const ConvP16Params p) {
         raw_t raw[G::NB];
         int l_off[G::NB];
         bool ok[G::NB];
-        const int y0 = tyi * G::TH + p.in_y0, x0 = txi * G::TW + p.in_x0;
+        // (a 1x1 layer may step over the input: position (y, x) reads pixel (y, x) * stride)
+        const int st = NTAPS == 1 ? p.stride : 1;
+        const int y0 = tyi * G::TH * st + p.in_y0, x0 = txi * G::TW * st + p.in_x0;
 #pragma unroll
         for (int i = 0; i < G::NB; i++) {
             const int idx = stid + i * 256;
@@ -976,12 +978,13 @@ __global__ __launch_bounds__(512) void conv_kr16_kernel(const ConvP16Params p) {
             const int pix = rem >> 2, g = rem & 3;
             const int py = pix / G::HW, px = pix - py * G::HW;
             l_off[i] = idx < G::TOTAL ? chunk * G::BUFC + py * G::ROW_PITCH + px * PITCH + g * 16 : -1;
-            int gy = y0 + py, gx = x0 + px;
+            int gy = y0 + py * st, gx = x0 + px * st;
             if (p.in_clamp) {
                 gy = min(max(gy, 0), p.in_hp - 1);
                 gx = min(max(gx, 0), p.in_wp - 1);
             }
-            ok[i] = idx < G::TOTAL && (unsigned)gy < (unsigned)p.in_hp && (unsigned)gx < (unsigned)p.in_wp;
+            // (channels behind the tensor's pitch -- the chunk count is rounded up to four per wave -- read as zero)
+            ok[i] = idx < G::TOTAL && (unsigned)gy < (unsigned)p.in_hp && (unsigned)gx < (unsigned)p.in_wp && chunk * KC + g * 8 < p.in_cp;
             const store_t* src = in + (ok[i] ? (gy * p.in_wp + gx) * p.in_cp + chunk * KC + g * 8 : 0);
             if constexpr (HSTORE) {
                 raw[i] = *reinterpret_cast<const half8_t*>(src);
@@ -1187,8 +1190,9 @@ constexpr KREntry krentry() {
     return KREntry{NTAPS, CPW, FM, conv_kr16_kernel<NTAPS, CPW, FM>, (size_t)(G::RED_OFF + 3 * FM * 1024 + 2 * 16 * FM * 4)};
 }
 const KREntry kKREntries[] = {
-    krentry<1, 2, 1>(), krentry<1, 4, 1>(), krentry<1, 8, 1>(), krentry<1, 2, 2>(), krentry<1, 4, 2>(), krentry<1, 8, 2>(),
-    krentry<9, 2, 1>(), krentry<9, 4, 1>(), krentry<9, 2, 2>(), krentry<9, 4, 2>(),
+    krentry<1, 1, 1>(), krentry<1, 2, 1>(), krentry<1, 3, 1>(), krentry<1, 4, 1>(), krentry<1, 5, 1>(), krentry<1, 8, 1>(),
+    krentry<1, 1, 2>(), krentry<1, 2, 2>(), krentry<1, 3, 2>(), krentry<1, 4, 2>(), krentry<1, 5, 2>(), krentry<1, 8, 2>(),
+    krentry<9, 1, 1>(), krentry<9, 2, 1>(), krentry<9, 4, 1>(), krentry<9, 1, 2>(), krentry<9, 2, 2>(), krentry<9, 4, 2>(),
 };
 }  // namespace
 
@@ -1250,15 +1254,16 @@ size_t P16_NAME(conv_kr16_lds_bytes)(const ConvP16Params& p, int k) {
     const KREntry* e = find_krentry(p, k);
     return e ? e->lds : 0;
 }
-// The K-resident form: k = 1 or 3, stride 1; tiles of 4x4 positions, blocks of 16*p.wm output channels (p.wm = 1 or 2),
-// p.cin_chunks = 8, 16 or 32 (3x3: 8 or 16); in_y0/in_x0 = input padding - (k-1)/2; one workgroup per tile and block
+// The K-resident form: k = 1 (any stride) or 3 (stride 1); tiles of 4x4 positions, blocks of 16*p.wm output channels (p.wm = 1 or 2),
+// p.cin_chunks = 4, 8, 12, 16, 20 or 32 (3x3: 4, 8 or 16), channels behind in_cp reading as zero; in_y0/in_x0 = input padding - (k-1)/2; one workgroup per tile and block
 int P16_NAME(launch_conv_kr16)(const ConvP16Params& p, int k, hipStream_t s) {
 #if !FYN_P16_HALF
     if (p.f16) return launch_conv_kr16_half(p, k, s);
 #endif
     const KREntry* e = find_krentry(p, k);
     if (!e) return -1;
-    if (p.in_cp != p.cin_chunks * KC || p.cout_blocks < 1 || p.mfrags != p.cout_blocks * e->fm || p.stride != 1 || p.tile_h != 4 || p.tile_w != 4 ||
+    if (p.in_cp > p.cin_chunks * KC || p.in_cp % 8 != 0 || p.in_cp < 8 || p.cout_blocks < 1 || p.mfrags != p.cout_blocks * e->fm || p.stride < 1 || (k != 1 && p.stride != 1) ||
+        p.tile_h != 4 || p.tile_w != 4 ||
         p.tiles_x * 4 < p.npos_x || p.tiles_y * 4 < p.npos_y || p.out_cp < p.cout_blocks * 16 * e->fm || (p.out_cp * ESZ) % 16 != 0 ||
         (p.res && (p.res_cp < p.cout_blocks * 16 * e->fm || (p.res_cp * ESZ) % 16 != 0)) || p.nreset < 0 || p.nreset > 4 || (p.f16 != 0) != HSTORE ||
         p.tiles_x < 1 || p.tiles_y < 1 || (long long)p.tiles_x * p.tiles_y * p.cout_blocks > 65535)

@@ -1198,14 +1198,14 @@ class ConvLayer : public Layer {
         ConvP16Params q{};
         q.in = in_v.ptr; q.out = out_v.ptr; q.res = res_v ? res_v->ptr : nullptr;
         q.in_hp = in_v.hp(); q.in_wp = in_v.wp(); q.in_cp = in_v.cp;
-        q.stride = 1;
+        q.stride = stride;   // (k = 1 only: position (y, x) reads pixel (y, x) * stride)
         q.in_y0 = q.in_x0 = in_v.pad - (k - 1) / 2;
         q.in_clamp = clamp ? 1 : 0;
         q.npos_y = oh; q.npos_x = ow;
         q.out_wp = out_v.wp(); q.out_cp = out_v.cp; q.out_off_y = q.out_off_x = out_v.pad;
         if (res_v) { q.res_wp = res_v->wp(); q.res_cp = res_v->cp; q.res_off_y = q.res_off_x = res_v->pad; }
         q.res_relu = res_relu; q.res_scale = res_scale;
-        q.cin_chunks = in_v.cp / 32;
+        q.cin_chunks = (in_v.cp + 127) / 128 * 4;   // (four waves share the chunks: rounded up, the channels behind the pitch read as zero)
         q.f16 = out_v.f16 ? 1 : 0;
         q.tile_h = q.tile_w = 4;
         q.tiles_x = (ow + 3) / 4; q.tiles_y = (oh + 3) / 4;
@@ -1232,13 +1232,14 @@ class ConvLayer : public Layer {
         if (cands.empty()) return;
         // (the same size for every candidate: cout blocks x 4 waves x steps x fragments x planes)
         const size_t halves = (size_t)(oc / 16) * 4 * (q.cin_chunks / 4) * k * k * (q.f16 ? 1 : 2) * 64 * 8;
-        p16_wpack_dev = net->dev_alloc(halves * 2, true);
-        for (ConvP16Params& c : cands) c.wpack = p16_wpack_dev;
+        void* const kr_wpack = net->dev_alloc(halves * 2, true);
+        for (ConvP16Params& c : cands) c.wpack = kr_wpack;
+        const bool had_p16 = p16;   // the 3x3 16-position form was chosen over the general kernel: this form has to beat it instead
         const bool always = getenv("FYNHIP_FORCE_KR16_CONV") != nullptr;
         const char* at = getenv("FYNHIP_AUTOTUNE");
         int pick = 0;
         char key[160];
-        snprintf(key, sizeof(key), "kr16:k%d:%dx%d:%dx%d:r%d:e%d:h%d", k, d.in_channels, oc, oh, ow, res_v ? 1 : 0, clamp ? 1 : 0, q.f16);
+        snprintf(key, sizeof(key), "kr16:k%d:%dx%d:%dx%d:s%d:r%d:e%d:h%d:p%d", k, d.in_channels, oc, oh, ow, stride, res_v ? 1 : 0, clamp ? 1 : 0, q.f16, had_p16 ? 1 : 0);
         int cached[3] = {0, 0, 0};
         if (!want_fm && tune_cache_triple(key, cached)) {
             pick = -1;
@@ -1255,21 +1256,27 @@ class ConvLayer : public Layer {
                     }, 10);
                     if (t < best) { best = t; pick = (int)i; }
                 }
-                t_other = std::min(t_other, time_launch(net, launch, 10));
+                if (had_p16)
+                    t_other = std::min(t_other, time_calls(net, [&]() {
+                        if (launch_conv_p16(pp, net->stream) != 0) fail(FYN_ERR_DEVICE, "16-position convolution launch failed while tuning");
+                    }, 10));
+                else
+                    t_other = std::min(t_other, time_launch(net, launch, 10));
             }
             if (getenv("FYNHIP_TUNE_VERBOSE"))
-                fprintf(stderr, "[tune] %dx%d on %d channels, %dx%d positions: K-resident form (%d-channel blocks) %.1f us, general kernel %.1f us\n", k, k,
-                        d.in_channels, oh, ow, 16 * cands[pick].wm, best * 1e3f, t_other * 1e3f);
+                fprintf(stderr, "[tune] %dx%d on %d channels, %dx%d positions: K-resident form (%d-channel blocks) %.1f us, %s %.1f us\n", k, k,
+                        d.in_channels, oh, ow, 16 * cands[pick].wm, best * 1e3f, had_p16 ? "16-position 3x3 form" : "general kernel", t_other * 1e3f);
             const bool win = best < t_other;
             if (!want_fm) tune_cache_store_triple(key, win ? 1 : 0, cands[pick].wm, 0);
             if (!win && !always) pick = -1;
         }
         if (pick >= 0) {
+            if (had_p16) net->dev_free(p16_wpack_dev);
+            p16_wpack_dev = kr_wpack;
             p16 = true; kr16 = true;
             pp = cands[pick];
         } else {
-            net->dev_free(p16_wpack_dev);
-            p16_wpack_dev = nullptr;
+            net->dev_free(kr_wpack);
         }
     }
     // weights of that form: [cout block][wave][step][fragment][plane][lane][8 halves]; step s of wave w = (chunk w + 4*(s / taps), tap s % taps)
@@ -1568,9 +1575,9 @@ class ConvLayer : public Layer {
                 !getenv("FYNHIP_NO_P16_CONV"))
                 setup_c4(in_v, out_v);
             // few positions, many input channels: the whole reduction of a 4x4 tile resident in LDS instead of K-split launches
-            if (!p16 && !frac_shift && same_storage && !sc.in_sub && (k == 1 || k == 3) && stride == 1 && dil == 1 && d.in_channels == in_v.cp &&
-                in_v.cp % 128 == 0 && oc % 16 == 0 && out_v.cp >= oc && oh * ow <= 1024 && (!res_v || (res_v->cp >= oc && res_v->cp % 8 == 0)) &&
-                !getenv("FYNHIP_NO_P16_CONV") && !getenv("FYNHIP_NO_KR16_CONV") &&
+            if ((!p16 || (!h16 && !c4)) && !frac_shift && same_storage && (k == 1 || (k == 3 && stride == 1)) && dil == 1 && in_v.cp % 8 == 0 &&
+                d.in_channels == in_v.cp && in_v.cp >= 16 && oc % 16 == 0 && out_v.cp >= oc && oh * ow <= 4096 && (!res_v || (res_v->cp >= oc && res_v->cp % 8 == 0)) &&
+                !getenv("FYNHIP_NO_P16_CONV") && !getenv("FYNHIP_NO_KR16_CONV") && !getenv("FYNHIP_FORCE_P16_CONV") &&
                 // (a test that forces a variant of the general kernel wants the general kernel)
                 !getenv("FYNHIP_FORCE_KSPLIT") && !getenv("FYNHIP_CONV_TILE") && !getenv("FYNHIP_CONV_KC") && !getenv("FYNHIP_CONV_KC_MAX") && !getenv("FYNHIP_CONV_PD"))
                 setup_kr16(in_v, out_v, res_v, res_relu, res_scale);

@@ -387,6 +387,18 @@ KR16_CASES = [
     (3, 512, 32, 7, 7, 1, {"residual": (A.NONE, False)}),
     (3, 256, 48, 9, 6, 1, {"pad_out": 2, "bn": True}),
     (3, 512, 64, 18, 30, 2, {}),                                                # 40 tiles x 2 blocks
+    (1, 128, 96, 11, 10, 2, {"bn": True, "residual": (A.NONE, False)}),         # one chunk per wave: a single step
+    (3, 128, 128, 28, 28, 1, {"bn": True}),                                     # one chunk per wave, nine steps
+    (1, 256, 64, 22, 30, 1, {"stride": 2, "bn": True}),                         # stride 2: positions read every other pixel
+    (1, 512, 128, 13, 15, 2, {"stride": 2, "residual": (A.RELU, True)}),        # odd input size with stride 2
+    # channel counts that are no multiple of 128: the chunk count is rounded up to four per wave, the rest reads as zero
+    (1, 64, 256, 20, 20, 2, {"bn": True}),
+    (1, 96, 48, 9, 9, 1, {}),
+    (1, 160, 32, 7, 7, 2, {"residual": (A.NONE, False)}),
+    (1, 320, 64, 7, 7, 1, {"bn": True}),                                        # 10 -> 12 chunks
+    (1, 576, 96, 14, 14, 2, {}),                                                # 18 -> 20 chunks
+    (1, 24, 144, 10, 12, 1, {"bn": True}),                                      # less than one chunk
+    (3, 64, 64, 12, 12, 1, {"bn": True, "residual": (A.RELU, True)}),
 ]
 
 
@@ -408,11 +420,13 @@ def test_reduction_resident_form(case, act, shallow, storage, monkeypatch):
         kw = dict(kw, deep=False, pad_in=0)
     if act is A.LEAKY_RELU:
         kw = dict(kw, leak=0.1)
-    b = conv_builder(k, cout, h, w, cin, 1, 1, act, **kw)
+    kw = dict(kw)
+    stride = kw.pop("stride", 1)
+    b = conv_builder(k, cout, h, w, cin, stride, 1, act, **kw)
     wts = conv_block(3000 + cin + k, cout, k, cin, bn=kw.get("bn", False))
     inputs = [prng.uniform(41 * cin + h, (cin, h, w), -1, 1)]
     if "residual" in kw:
-        inputs.append(prng.uniform(67, (cout, h, w), -1, 1))
+        inputs.append(prng.uniform(67, (cout, h // stride, w // stride), -1, 1))
     got, info = run_single(b, storage, inputs, wts)
     ref = oracle_single(b, storage, inputs, wts)
     err = rel_l2(got, ref)
