@@ -173,14 +173,14 @@ struct alignas(sizeof(T) * V) RawV {
     T v[V];
 };
 
-// Undilated depthwise 3x3, stride S: one thread produces four neighbouring output pixels of V channels from a
-// 3 x ((4-1)*S+3) input window, so that an input texel is fetched once per thread instead of up to three times and
-// the nine weight vectors are loaded once per four outputs.  All loads of the window are issued before the first
+// Undilated depthwise 3x3, stride S: one thread produces PX (four, on small layers two or one: more threads, each
+// done sooner) neighbouring output pixels of V channels from a 3 x ((PX-1)*S+3) input window, so that an input texel is
+// fetched once per thread instead of up to three times and the nine weight vectors are loaded once per PX outputs.  All loads of the window are issued before the first
 // use (one memory round trip per thread); the texels stay in their stored type until they are consumed.  Same
 // accumulation order per output (ky outer, kx inner, fused multiply-add) as dwconv3x3_kernel.
-template <typename T, int V, int S>
+template <typename T, int V, int S, int PX>
 __global__ __launch_bounds__(256) void dwconv3x3_row_kernel(const DwConvParams p) {
-    constexpr int PX = 4, WIN = (PX - 1) * S + 3;
+    constexpr int WIN = (PX - 1) * S + 3;
     const int cg = p.out.cp / V;
     const int xb = (p.out.w + PX - 1) / PX;
     const size_t n = (size_t)p.out.h * xb * cg;
@@ -375,11 +375,20 @@ __global__ __launch_bounds__(256) void dwconv3x3_col_kernel(const DwConvParams p
     }
 }
 
+template <typename T, int V, int PX>
+static void launch_dw_row_px(const DwConvParams& p, hipStream_t s) {
+    const size_t n = (size_t)p.out.h * ((p.out.w + PX - 1) / PX) * (p.out.cp / V);
+    if (p.stride == 1) hipLaunchKernelGGL((dwconv3x3_row_kernel<T, V, 1, PX>), grid1d(n, 256), dim3(256), 0, s, p);
+    else hipLaunchKernelGGL((dwconv3x3_row_kernel<T, V, 2, PX>), grid1d(n, 256), dim3(256), 0, s, p);
+}
+// (pixels per thread: four when that still gives every SIMD of the chip a wave, else two, else one)
 template <typename T, int V>
 static void launch_dw_row(const DwConvParams& p, hipStream_t s) {
-    const size_t n = (size_t)p.out.h * ((p.out.w + 3) / 4) * (p.out.cp / V);
-    if (p.stride == 1) hipLaunchKernelGGL((dwconv3x3_row_kernel<T, V, 1>), grid1d(n, 256), dim3(256), 0, s, p);
-    else hipLaunchKernelGGL((dwconv3x3_row_kernel<T, V, 2>), grid1d(n, 256), dim3(256), 0, s, p);
+    const size_t per_px = (size_t)p.out.h * (p.out.cp / V);
+    const size_t want = 256 * 4 * 64;
+    if (per_px * ((p.out.w + 3) / 4) >= want) launch_dw_row_px<T, V, 4>(p, s);
+    else if (per_px * ((p.out.w + 1) / 2) >= want) launch_dw_row_px<T, V, 2>(p, s);
+    else launch_dw_row_px<T, V, 1>(p, s);
 }
 
 // strips of `rows` output rows per thread, when the image is tall enough to leave the chip enough threads
