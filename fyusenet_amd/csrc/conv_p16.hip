@@ -928,17 +928,20 @@ template <int NTAPS, int CPW>
 struct GeoR {
     static constexpr int TH = 4, TW = 4, KH = (NTAPS == 9) ? 2 : 0;
     static constexpr int HW = TW + KH, HH = TH + KH;
-    static constexpr int ROW_PITCH = HW * PITCH + p16_row_pad(TH, TW, 1, 1, HW);
+    static constexpr int NCH = 4 * CPW;                 // chunks of the layer
+    // (64 chunks -- 2048 input channels -- fit the LDS only without the padding that keeps the fragment reads free of
+    // bank conflicts; the reads are a small part of this kernel)
+    static constexpr int PIT = (NCH > 32) ? KC * 2 : PITCH;
+    static constexpr int ROW_PITCH = HW * PIT + ((NCH > 32) ? 0 : p16_row_pad(TH, TW, 1, 1, HW));
     static constexpr int PLANE = HH * ROW_PITCH;
     static constexpr int BUFC = NPL * PLANE;            // one chunk of the tile
-    static constexpr int NCH = 4 * CPW;                 // chunks of the layer
     static constexpr int NITEMS = HH * HW * (KC / 8);   // staging items per chunk
     static constexpr int TOTAL = NITEMS * NCH, NB = (TOTAL + 255) / 256;
     static constexpr int STEPS = CPW * NTAPS;           // per MFMA wave
     static constexpr int RPD = STEPS < 8 ? STEPS : 8;   // weight ring depth (steps; the step loop is unrolled, so any depth fits)
     static constexpr int BD = STEPS < 4 ? STEPS : 4;    // B fragment ring depth (steps)
     static constexpr int RED_OFF = NCH * BUFC;          // [wave 1..3][fragment][lane] x 16 bytes, then scale and bias
-    static constexpr int tap_off(int t) { return NTAPS == 9 ? (t / 3) * ROW_PITCH + (t % 3) * PITCH : 0; }
+    static constexpr int tap_off(int t) { return NTAPS == 9 ? (t / 3) * ROW_PITCH + (t % 3) * PIT : 0; }
     static_assert(NTAPS == 1 || NTAPS == 9, "1x1 or 3x3");
 };
 
@@ -977,7 +980,7 @@ __global__ __launch_bounds__(512) void conv_kr16_kernel(const ConvP16Params p) {
             const int chunk = idx / G::NITEMS, rem = idx - chunk * G::NITEMS;
             const int pix = rem >> 2, g = rem & 3;
             const int py = pix / G::HW, px = pix - py * G::HW;
-            l_off[i] = idx < G::TOTAL ? chunk * G::BUFC + py * G::ROW_PITCH + px * PITCH + g * 16 : -1;
+            l_off[i] = idx < G::TOTAL ? chunk * G::BUFC + py * G::ROW_PITCH + px * G::PIT + g * 16 : -1;
             int gy = y0 + py * st, gx = x0 + px * st;
             if (p.in_clamp) {
                 gy = min(max(gy, 0), p.in_hp - 1);
@@ -1028,7 +1031,7 @@ __global__ __launch_bounds__(512) void conv_kr16_kernel(const ConvP16Params p) {
     // ---------------------------------------------------------------------- MFMA waves
     const int w = wave - 4;
     const int mq = lane & 15, kq = lane >> 4;
-    const int bbase = (mq / G::TW) * G::ROW_PITCH + (mq % G::TW) * PITCH + kq * 16 + w * G::BUFC;   // chunk `w` of the tile
+    const int bbase = (mq / G::TW) * G::ROW_PITCH + (mq % G::TW) * G::PIT + kq * 16 + w * G::BUFC;   // chunk `w` of the tile
     constexpr unsigned wstep = FM * NPL * 1024;
     const unsigned char* wbase = reinterpret_cast<const unsigned char*>(p.wpack) + (size_t)((cb * 4 + w) * STEPS) * wstep + lane * 16;
     half8_t a_q[RPD][FM][NPL];
@@ -1190,8 +1193,8 @@ constexpr KREntry krentry() {
     return KREntry{NTAPS, CPW, FM, conv_kr16_kernel<NTAPS, CPW, FM>, (size_t)(G::RED_OFF + 3 * FM * 1024 + 2 * 16 * FM * 4)};
 }
 const KREntry kKREntries[] = {
-    krentry<1, 1, 1>(), krentry<1, 2, 1>(), krentry<1, 3, 1>(), krentry<1, 4, 1>(), krentry<1, 5, 1>(), krentry<1, 8, 1>(),
-    krentry<1, 1, 2>(), krentry<1, 2, 2>(), krentry<1, 3, 2>(), krentry<1, 4, 2>(), krentry<1, 5, 2>(), krentry<1, 8, 2>(),
+    krentry<1, 1, 1>(), krentry<1, 2, 1>(), krentry<1, 3, 1>(), krentry<1, 4, 1>(), krentry<1, 5, 1>(), krentry<1, 8, 1>(), krentry<1, 16, 1>(),
+    krentry<1, 1, 2>(), krentry<1, 2, 2>(), krentry<1, 3, 2>(), krentry<1, 4, 2>(), krentry<1, 5, 2>(), krentry<1, 8, 2>(), krentry<1, 16, 2>(),
     krentry<9, 1, 1>(), krentry<9, 2, 1>(), krentry<9, 4, 1>(), krentry<9, 1, 2>(), krentry<9, 2, 2>(), krentry<9, 4, 2>(),
 };
 }  // namespace
@@ -1255,7 +1258,7 @@ size_t P16_NAME(conv_kr16_lds_bytes)(const ConvP16Params& p, int k) {
     return e ? e->lds : 0;
 }
 // The K-resident form: k = 1 (any stride) or 3 (stride 1); tiles of 4x4 positions, blocks of 16*p.wm output channels (p.wm = 1 or 2),
-// p.cin_chunks = 4, 8, 12, 16, 20 or 32 (3x3: 4, 8 or 16), channels behind in_cp reading as zero; in_y0/in_x0 = input padding - (k-1)/2; one workgroup per tile and block
+// p.cin_chunks = 4, 8, 12, 16, 20, 32 or 64 (3x3: 4, 8 or 16), channels behind in_cp reading as zero; in_y0/in_x0 = input padding - (k-1)/2; one workgroup per tile and block
 int P16_NAME(launch_conv_kr16)(const ConvP16Params& p, int k, hipStream_t s) {
 #if !FYN_P16_HALF
     if (p.f16) return launch_conv_kr16_half(p, k, s);

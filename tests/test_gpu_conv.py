@@ -399,6 +399,8 @@ KR16_CASES = [
     (1, 576, 96, 14, 14, 2, {}),                                                # 18 -> 20 chunks
     (1, 24, 144, 10, 12, 1, {"bn": True}),                                      # less than one chunk
     (3, 64, 64, 12, 12, 1, {"bn": True, "residual": (A.RELU, True)}),
+    (1, 2048, 64, 7, 7, 1, {"bn": True}),                                       # 64 chunks: unpadded pixel pitch in LDS
+    (1, 2048, 32, 5, 9, 2, {}),
 ]
 
 
