@@ -924,9 +924,11 @@ __global__ __launch_bounds__(512) void conv_p16c4_kernel(const ConvP16Params p) 
 // and add their accumulators through LDS; wave 0 runs the epilogue.  Small tiles make many workgroups (13 tiles x 16
 // blocks of 16 channels for 1024 -> 256 at 14x14), so the layer's activations and weights are pulled through many CUs.
 // Weights: [cout block][wave][step][fragment][plane][lane][8 halves], the wave's steps being (chunk wave + 4*i, tap).
-template <int NTAPS, int CPW>
+template <int NTAPS, int CPW, int FN_ = 1>
 struct GeoR {
-    static constexpr int TH = 4, TW = 4, KH = (NTAPS == 9) ? 2 : 0;
+    static constexpr int FN = FN_;                      // position fragments per tile: 4x4, 4x8 or 8x8 positions
+    static constexpr int TH = (FN == 4) ? 8 : 4, TW = (FN == 1) ? 4 : 8, KH = (NTAPS == 9) ? 2 : 0;
+    static_assert(FN == 1 || FN == 2 || FN == 4, "tiles of 16, 32 or 64 positions");
     static constexpr int HW = TW + KH, HH = TH + KH;
     static constexpr int NCH = 4 * CPW;                 // chunks of the layer
     // (64 chunks -- 2048 input channels -- fit the LDS only without the padding that keeps the fragment reads free of
@@ -939,15 +941,15 @@ struct GeoR {
     static constexpr int TOTAL = NITEMS * NCH, NB = (TOTAL + 255) / 256;
     static constexpr int STEPS = CPW * NTAPS;           // per MFMA wave
     static constexpr int RPD = STEPS < 8 ? STEPS : 8;   // weight ring depth (steps; the step loop is unrolled, so any depth fits)
-    static constexpr int BD = STEPS < 4 ? STEPS : 4;    // B fragment ring depth (steps)
+    static constexpr int BD = FN > 1 ? (STEPS < 2 ? STEPS : 2) : (STEPS < 4 ? STEPS : 4);    // B fragment ring depth (steps)
     static constexpr int RED_OFF = NCH * BUFC;          // [wave 1..3][fragment][lane] x 16 bytes, then scale and bias
     static constexpr int tap_off(int t) { return NTAPS == 9 ? (t / 3) * ROW_PITCH + (t % 3) * PIT : 0; }
     static_assert(NTAPS == 1 || NTAPS == 9, "1x1 or 3x3");
 };
 
-template <int NTAPS, int CPW, int FM>
+template <int NTAPS, int CPW, int FM, int FN>
 __global__ __launch_bounds__(512) void conv_kr16_kernel(const ConvP16Params p) {
-    using G = GeoR<NTAPS, CPW>;
+    using G = GeoR<NTAPS, CPW, FN>;
     constexpr int RPD = G::RPD, BD = G::BD, STEPS = G::STEPS;
     extern __shared__ __align__(16) unsigned char lds[];
     __shared__ unsigned range_box[2];
@@ -961,7 +963,7 @@ __global__ __launch_bounds__(512) void conv_kr16_kernel(const ConvP16Params p) {
     if (tid < 2) range_box[tid] = 0u;
     const unsigned range_bits = p.in_amax ? range_load(p.in_amax) : 0u;
     constexpr int red_off = G::RED_OFF;
-    constexpr int sb_off = red_off + 3 * FM * 1024;
+    constexpr int sb_off = red_off + 3 * FM * FN * 1024;
 
     if (wave < 4) {   // ------------------------------------------------------------ staging waves
         const int stid = tid & 255;
@@ -1031,7 +1033,12 @@ __global__ __launch_bounds__(512) void conv_kr16_kernel(const ConvP16Params p) {
     // ---------------------------------------------------------------------- MFMA waves
     const int w = wave - 4;
     const int mq = lane & 15, kq = lane >> 4;
-    const int bbase = (mq / G::TW) * G::ROW_PITCH + (mq % G::TW) * G::PIT + kq * 16 + w * G::BUFC;   // chunk `w` of the tile
+    int bbase[FN];   // chunk `w` of the tile, the lane's position of each fragment
+#pragma unroll
+    for (int fn = 0; fn < FN; fn++) {
+        const int m = fn * 16 + mq;
+        bbase[fn] = (m / G::TW) * G::ROW_PITCH + (m % G::TW) * G::PIT + kq * 16 + w * G::BUFC;
+    }
     constexpr unsigned wstep = FM * NPL * 1024;
     const unsigned char* wbase = reinterpret_cast<const unsigned char*>(p.wpack) + (size_t)((cb * 4 + w) * STEPS) * wstep + lane * 16;
     half8_t a_q[RPD][FM][NPL];
@@ -1045,9 +1052,11 @@ __global__ __launch_bounds__(512) void conv_kr16_kernel(const ConvP16Params p) {
     for (int fm = 0; fm < FM; fm++)
 #pragma unroll
         for (int pl = 0; pl < NPL; pl++) a_q[RPD - 1][fm][pl] = a_q[0][fm][pl];   // (defined; replaced during the first step)
-    f32x4_t acc[FM];
+    f32x4_t acc[FM][FN];
 #pragma unroll
-    for (int fm = 0; fm < FM; fm++) acc[fm] = (f32x4_t)(0.f);
+    for (int fm = 0; fm < FM; fm++)
+#pragma unroll
+        for (int fn = 0; fn < FN; fn++) acc[fm][fn] = (f32x4_t)(0.f);
     float inv_in_scale = 1.f;
     if (p.in_amax) (void)range_scale(range_after_act(range_reduce(range_bits), p.act), &inv_in_scale);
     const float acc_mul = p.acc_mul * inv_in_scale;
@@ -1055,11 +1064,13 @@ __global__ __launch_bounds__(512) void conv_kr16_kernel(const ConvP16Params p) {
     lds_barrier();   // the tile is staged
     // B fragment of step s: chunk w + 4*(s / NTAPS), tap s % NTAPS
     auto b_off = [&](int s) { return (s / NTAPS) * 4 * G::BUFC + G::tap_off(s % NTAPS); };
-    half8_t b[BD][NPL];
+    half8_t b[BD][FN][NPL];
 #pragma unroll
     for (int s = 0; s < BD - 1; s++)
 #pragma unroll
-        for (int pl = 0; pl < NPL; pl++) b[s][pl] = *reinterpret_cast<const half8_t*>(lds + bbase + b_off(s) + pl * G::PLANE);
+        for (int fn = 0; fn < FN; fn++)
+#pragma unroll
+            for (int pl = 0; pl < NPL; pl++) b[s][fn][pl] = *reinterpret_cast<const half8_t*>(lds + bbase[fn] + b_off(s) + pl * G::PLANE);
 #pragma unroll
     for (int s = 0; s < STEPS; s++) {
         const int d = s % RPD, dload = (s + RPD - 1) % RPD, bs = s % BD, bload = (s + BD - 1) % BD;
@@ -1073,20 +1084,28 @@ __global__ __launch_bounds__(512) void conv_kr16_kernel(const ConvP16Params p) {
         }
         if (s + BD - 1 < STEPS) {
 #pragma unroll
-            for (int pl = 0; pl < NPL; pl++) b[bload][pl] = *reinterpret_cast<const half8_t*>(lds + bbase + b_off(s + BD - 1) + pl * G::PLANE);
+            for (int fn = 0; fn < FN; fn++)
+#pragma unroll
+                for (int pl = 0; pl < NPL; pl++)
+                    b[bload][fn][pl] = *reinterpret_cast<const half8_t*>(lds + bbase[fn] + b_off(s + BD - 1) + pl * G::PLANE);
         }
 #pragma unroll
-        for (int i = 0; i < NPASS * FM; i++) {
-            const int kind = i / FM, fm = i % FM;
-            const int apl = (kind == 1) ? 1 : 0, bpl = (kind == 2) ? 1 : 0;
-            acc[fm] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_q[d][fm][apl], b[bs][bpl], acc[fm], 0, 0, 0);
-        }
+        for (int fn = 0; fn < FN; fn++)
+#pragma unroll
+            for (int i = 0; i < NPASS * FM; i++) {
+                const int kind = i / FM, fm = i % FM;
+                const int apl = (kind == 1) ? 1 : 0, bpl = (kind == 2) ? 1 : 0;
+                acc[fm][fn] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_q[d][fm][apl], b[bs][fn][bpl], acc[fm][fn], 0, 0, 0);
+            }
         __builtin_amdgcn_sched_barrier(0);
     }
     // the four partial sums meet in wave 0
     if (w > 0) {
 #pragma unroll
-        for (int fm = 0; fm < FM; fm++) *reinterpret_cast<f32x4_t*>(lds + red_off + ((w - 1) * FM + fm) * 1024 + lane * 16) = acc[fm];
+        for (int fm = 0; fm < FM; fm++)
+#pragma unroll
+            for (int fn = 0; fn < FN; fn++)
+                *reinterpret_cast<f32x4_t*>(lds + red_off + (((w - 1) * FM + fm) * FN + fn) * 1024 + lane * 16) = acc[fm][fn];
     }
     lds_barrier();
     if (w > 0) return;
@@ -1095,13 +1114,16 @@ __global__ __launch_bounds__(512) void conv_kr16_kernel(const ConvP16Params p) {
         const float* sb = reinterpret_cast<const float*>(lds + sb_off);
         store_t* out = reinterpret_cast<store_t*>(p.out);
         const store_t* res = reinterpret_cast<const store_t*>(p.res);
-        const int py = tyi * G::TH + mq / G::TW, px = txi * G::TW + mq % G::TW;
-        const bool okp = py < p.npos_y && px < p.npos_x;
+#pragma unroll
+        for (int fn = 0; fn < FN; fn++)
 #pragma unroll
         for (int fm = 0; fm < FM; fm++) {
-            f32x4_t v = acc[fm];
+            const int m = fn * 16 + mq;
+            const int py = tyi * G::TH + m / G::TW, px = txi * G::TW + m % G::TW;
+            const bool okp = py < p.npos_y && px < p.npos_x;
+            f32x4_t v = acc[fm][fn];
 #pragma unroll
-            for (int o = 0; o < 3; o++) v += *reinterpret_cast<const f32x4_t*>(lds + red_off + (o * FM + fm) * 1024 + lane * 16);
+            for (int o = 0; o < 3; o++) v += *reinterpret_cast<const f32x4_t*>(lds + red_off + ((o * FM + fm) * FN + fn) * 1024 + lane * 16);
             const f32x4_t sc = *reinterpret_cast<const f32x4_t*>(sb + fm * 16 + kq * 4);
             const f32x4_t bi = *reinterpret_cast<const f32x4_t*>(sb + 16 * FM + fm * 16 + kq * 4);
             const int ch = cb * 16 * FM + fm * 16 + kq * 4;
@@ -1183,19 +1205,22 @@ template <int K, int TH, int TW>
 constexpr C4Entry c4entry() { return C4Entry{K, TH, TW, conv_p16c4_kernel<K, TH, TW>, (size_t)GeoC4<K, TH, TW>::BUF, GeoC4<K, TH, TW>::NS}; }
 const C4Entry kC4Entries[] = {c4entry<9, 8, 8>(), c4entry<9, 4, 8>(), c4entry<9, 8, 4>()};
 struct KREntry {
-    int taps, cpw, fm;
+    int taps, cpw, fm, nfrag, th, tw;
     p16_fn fn;
     size_t lds;
 };
-template <int NTAPS, int CPW, int FM>
+template <int NTAPS, int CPW, int FM, int FN = 1>
 constexpr KREntry krentry() {
-    using G = GeoR<NTAPS, CPW>;
-    return KREntry{NTAPS, CPW, FM, conv_kr16_kernel<NTAPS, CPW, FM>, (size_t)(G::RED_OFF + 3 * FM * 1024 + 2 * 16 * FM * 4)};
+    using G = GeoR<NTAPS, CPW, FN>;
+    return KREntry{NTAPS, CPW, FM, FN, G::TH, G::TW, conv_kr16_kernel<NTAPS, CPW, FM, FN>, (size_t)(G::RED_OFF + 3 * FM * FN * 1024 + 2 * 16 * FM * 4)};
 }
 const KREntry kKREntries[] = {
     krentry<1, 1, 1>(), krentry<1, 2, 1>(), krentry<1, 3, 1>(), krentry<1, 4, 1>(), krentry<1, 5, 1>(), krentry<1, 8, 1>(), krentry<1, 16, 1>(),
     krentry<1, 1, 2>(), krentry<1, 2, 2>(), krentry<1, 3, 2>(), krentry<1, 4, 2>(), krentry<1, 5, 2>(), krentry<1, 8, 2>(), krentry<1, 16, 2>(),
     krentry<9, 1, 1>(), krentry<9, 2, 1>(), krentry<9, 4, 1>(), krentry<9, 1, 2>(), krentry<9, 2, 2>(), krentry<9, 4, 2>(),
+    // larger tiles for layers with more positions and a short reduction
+    krentry<1, 1, 1, 2>(), krentry<1, 1, 2, 2>(), krentry<1, 2, 1, 2>(), krentry<1, 2, 2, 2>(), krentry<9, 1, 1, 2>(), krentry<9, 1, 2, 2>(),
+    krentry<1, 1, 1, 4>(), krentry<1, 1, 2, 4>(), krentry<1, 2, 1, 4>(), krentry<1, 2, 2, 4>(), krentry<9, 1, 1, 4>(), krentry<9, 1, 2, 4>(),
 };
 }  // namespace
 
@@ -1236,8 +1261,9 @@ void conv_p16c4_tile(int index, int* k, int* th, int* tw, int* steps) {
     *k = kC4Entries[index].k; *th = kC4Entries[index].th; *tw = kC4Entries[index].tw; *steps = kC4Entries[index].steps;
 }
 int conv_kr16_variant_count() { return (int)(sizeof(kKREntries) / sizeof(kKREntries[0])); }
-void conv_kr16_variant(int index, int* taps, int* chunks, int* fm) {
+void conv_kr16_variant(int index, int* taps, int* chunks, int* fm, int* th, int* tw) {
     *taps = kKREntries[index].taps; *chunks = 4 * kKREntries[index].cpw; *fm = kKREntries[index].fm;
+    *th = kKREntries[index].th; *tw = kKREntries[index].tw;
 }
 bool conv_p16c4_supported(int k, int stride, int dil, int in_cp, int cout, int out_cp, bool f16) {
     (void)f16;
@@ -1247,7 +1273,7 @@ bool conv_p16c4_supported(int k, int stride, int dil, int in_cp, int cout, int o
 
 static const KREntry* find_krentry(const ConvP16Params& p, int k) {
     for (const KREntry& c : kKREntries)
-        if (c.taps == k * k && c.cpw * 4 == p.cin_chunks && c.fm == p.wm) return &c;
+        if (c.taps == k * k && c.cpw * 4 == p.cin_chunks && c.fm == p.wm && c.th == p.tile_h && c.tw == p.tile_w) return &c;
     return nullptr;
 }
 size_t P16_NAME(conv_kr16_lds_bytes)(const ConvP16Params& p, int k) {
@@ -1257,7 +1283,7 @@ size_t P16_NAME(conv_kr16_lds_bytes)(const ConvP16Params& p, int k) {
     const KREntry* e = find_krentry(p, k);
     return e ? e->lds : 0;
 }
-// The K-resident form: k = 1 (any stride) or 3 (stride 1); tiles of 4x4 positions, blocks of 16*p.wm output channels (p.wm = 1 or 2),
+// The K-resident form: k = 1 (any stride) or 3 (stride 1); tiles of tile_h x tile_w = 4x4 (4x8, 8x8 for short reductions) positions, blocks of 16*p.wm output channels (p.wm = 1 or 2),
 // p.cin_chunks = 4, 8, 12, 16, 20, 32 or 64 (3x3: 4, 8 or 16), channels behind in_cp reading as zero; in_y0/in_x0 = input padding - (k-1)/2; one workgroup per tile and block
 int P16_NAME(launch_conv_kr16)(const ConvP16Params& p, int k, hipStream_t s) {
 #if !FYN_P16_HALF
@@ -1266,8 +1292,7 @@ int P16_NAME(launch_conv_kr16)(const ConvP16Params& p, int k, hipStream_t s) {
     const KREntry* e = find_krentry(p, k);
     if (!e) return -1;
     if (p.in_cp > p.cin_chunks * KC || p.in_cp % 8 != 0 || p.in_cp < 8 || p.cout_blocks < 1 || p.mfrags != p.cout_blocks * e->fm || p.stride < 1 || (k != 1 && p.stride != 1) ||
-        p.tile_h != 4 || p.tile_w != 4 ||
-        p.tiles_x * 4 < p.npos_x || p.tiles_y * 4 < p.npos_y || p.out_cp < p.cout_blocks * 16 * e->fm || (p.out_cp * ESZ) % 16 != 0 ||
+        p.tiles_x * e->tw < p.npos_x || p.tiles_y * e->th < p.npos_y || p.out_cp < p.cout_blocks * 16 * e->fm || (p.out_cp * ESZ) % 16 != 0 ||
         (p.res && (p.res_cp < p.cout_blocks * 16 * e->fm || (p.res_cp * ESZ) % 16 != 0)) || p.nreset < 0 || p.nreset > 4 || (p.f16 != 0) != HSTORE ||
         p.tiles_x < 1 || p.tiles_y < 1 || (long long)p.tiles_x * p.tiles_y * p.cout_blocks > 65535)
         return -5;

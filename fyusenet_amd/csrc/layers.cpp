@@ -1207,21 +1207,24 @@ class ConvLayer : public Layer {
         q.res_relu = res_relu; q.res_scale = res_scale;
         q.cin_chunks = (in_v.cp + 127) / 128 * 4;   // (four waves share the chunks: rounded up, the channels behind the pitch read as zero)
         q.f16 = out_v.f16 ? 1 : 0;
-        q.tile_h = q.tile_w = 4;
-        q.tiles_x = (ow + 3) / 4; q.tiles_y = (oh + 3) / 4;
-        q.rcp_tiles_x = 1.0f / (float)q.tiles_x;
-        q.pos_groups = q.tiles_x * q.tiles_y;
         q.scale = scale_dev; q.bias = bias_dev;
         q.acc_mul = 1.f;
         q.act = act();
-        int want_fm = 0;   // FYNHIP_KR16_FM (tests): fragments per block of output channels
-        if (const char* e = getenv("FYNHIP_KR16_FM")) want_fm = atoi(e);
+        int want_fm = 0, want_th = 0, want_tw = 0;   // FYNHIP_KR16_FM=fragments per block of output channels[,tile h,tile w] (tests)
+        if (const char* e = getenv("FYNHIP_KR16_FM")) sscanf(e, "%d,%d,%d", &want_fm, &want_th, &want_tw);
         std::vector<ConvP16Params> cands;
         for (int i = 0; i < conv_kr16_variant_count(); i++) {
-            int taps, chunks, fm;
-            conv_kr16_variant(i, &taps, &chunks, &fm);
+            int taps, chunks, fm, th, tw;
+            conv_kr16_variant(i, &taps, &chunks, &fm, &th, &tw);
             if (taps != k * k || chunks != q.cin_chunks || oc % (16 * fm) != 0 || (want_fm && fm != want_fm)) continue;
+            if (want_th ? (th != want_th || tw != want_tw) : (want_fm && th * tw != 16)) continue;
+            // (larger tiles are for layers that would need several rounds of 16-position workgroups)
+            if (th * tw > 16 && !want_th && ((oh + 3) / 4) * ((ow + 3) / 4) * (oc / (16 * fm)) <= 512) continue;
             ConvP16Params c = q;
+            c.tile_h = th; c.tile_w = tw;
+            c.tiles_x = (ow + tw - 1) / tw; c.tiles_y = (oh + th - 1) / th;
+            c.rcp_tiles_x = 1.0f / (float)c.tiles_x;
+            c.pos_groups = c.tiles_x * c.tiles_y;
             c.wm = fm;
             c.cout_blocks = oc / (16 * fm);
             c.mfrags = oc / 16;
@@ -1245,7 +1248,7 @@ class ConvLayer : public Layer {
             pick = -1;
             if (cached[0] || always)
                 for (size_t i = 0; i < cands.size(); i++)
-                    if (cands[i].wm == cached[1]) pick = (int)i;
+                    if (cands[i].wm == cached[1] && cands[i].tile_h * 100 + cands[i].tile_w == cached[2]) pick = (int)i;
             if (always && pick < 0) pick = 0;
         } else if (!(at && at[0] == '0')) {
             float best = 1e30f, t_other = 1e30f;
@@ -1264,10 +1267,11 @@ class ConvLayer : public Layer {
                     t_other = std::min(t_other, time_launch(net, launch, 10));
             }
             if (getenv("FYNHIP_TUNE_VERBOSE"))
-                fprintf(stderr, "[tune] %dx%d on %d channels, %dx%d positions: K-resident form (%d-channel blocks) %.1f us, %s %.1f us\n", k, k,
-                        d.in_channels, oh, ow, 16 * cands[pick].wm, best * 1e3f, had_p16 ? "16-position 3x3 form" : "general kernel", t_other * 1e3f);
+                fprintf(stderr, "[tune] %dx%d on %d channels, %dx%d positions: K-resident form (%d-channel blocks, %dx%d tiles) %.1f us, %s %.1f us\n", k, k,
+                        d.in_channels, oh, ow, 16 * cands[pick].wm, cands[pick].tile_h, cands[pick].tile_w, best * 1e3f,
+                        had_p16 ? "16-position 3x3 form" : "general kernel", t_other * 1e3f);
             const bool win = best < t_other;
-            if (!want_fm) tune_cache_store_triple(key, win ? 1 : 0, cands[pick].wm, 0);
+            if (!want_fm) tune_cache_store_triple(key, win ? 1 : 0, cands[pick].wm, cands[pick].tile_h * 100 + cands[pick].tile_w);
             if (!win && !always) pick = -1;
         }
         if (pick >= 0) {
@@ -1683,8 +1687,8 @@ class ConvLayer : public Layer {
         }
         if (p16 && kr16) {
             char buf[220];
-            snprintf(buf, sizeof(buf), "conv_kr16 %s tile=%dx16(cout x pos) K-resident, 4 waves split %d chunks, blocks=%d lds=%zu steps=%d", pp.f16 ? "f16" : "f16x2-split",
-                     16 * pp.wm, pp.cin_chunks, pp.pos_groups * pp.cout_blocks, conv_kr16_lds_bytes(pp, k), pp.cin_chunks / 4 * k * k);
+            snprintf(buf, sizeof(buf), "conv_kr16 %s tile=%dx%d(cout x pos) K-resident, 4 waves split %d chunks, blocks=%d lds=%zu steps=%d", pp.f16 ? "f16" : "f16x2-split",
+                     16 * pp.wm, pp.tile_h * pp.tile_w, pp.cin_chunks, pp.pos_groups * pp.cout_blocks, conv_kr16_lds_bytes(pp, k), pp.cin_chunks / 4 * k * k);
             return mode + buf;
         }
         if (p16 && h16) {

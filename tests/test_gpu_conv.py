@@ -401,13 +401,19 @@ KR16_CASES = [
     (3, 64, 64, 12, 12, 1, {"bn": True, "residual": (A.RELU, True)}),
     (1, 2048, 64, 7, 7, 1, {"bn": True}),                                       # 64 chunks: unpadded pixel pitch in LDS
     (1, 2048, 32, 5, 9, 2, {}),
+    # larger tiles (fragments per block, tile h, tile w)
+    (1, 64, 256, 56, 56, "2,8,8", {"bn": True}),
+    (1, 256, 64, 30, 44, "1,4,8", {"residual": (A.RELU, True)}),
+    (3, 64, 64, 29, 35, "2,8,8", {"bn": True, "residual": (A.NONE, False)}),
+    (3, 96, 48, 20, 12, "1,4,8", {"pad_out": 1}),
+    (1, 24, 144, 56, 56, "1,8,8", {}),
 ]
 
 
 @pytest.mark.parametrize("storage", [fa.STORAGE_F32, fa.STORAGE_F16], ids=["f32", "f16"])
 @pytest.mark.parametrize("shallow", [False, True], ids=["deep", "shallow_edge_clamp"])
 @pytest.mark.parametrize("act", [A.RELU, A.LEAKY_RELU], ids=["relu", "leaky"])
-@pytest.mark.parametrize("case", KR16_CASES, ids=lambda c: "k%d_%dx%dx%d_to%d_fm%d" % (c[0], c[1], c[3], c[4], c[2], c[5]))
+@pytest.mark.parametrize("case", KR16_CASES, ids=lambda c: "k%d_%dx%dx%d_to%d_fm%s" % (c[0], c[1], c[3], c[4], c[2], str(c[5]).replace(",", "x")))
 def test_reduction_resident_form(case, act, shallow, storage, monkeypatch):
     """1x1 / 3x3 convolutions on few positions and many input channels with a tile's whole reduction resident in LDS and
     the four MFMA waves of a workgroup splitting the chunks."""
@@ -433,7 +439,11 @@ def test_reduction_resident_form(case, act, shallow, storage, monkeypatch):
     ref = oracle_single(b, storage, inputs, wts)
     err = rel_l2(got, ref)
     print("  ", info, "rel_l2=%.3e" % err, flush=True)
-    assert "conv_kr16" in info and "tile=%dx16" % (16 * fm) in info
+    if isinstance(fm, str):
+        f, th, tw = (int(v) for v in fm.split(","))
+        assert "conv_kr16" in info and "tile=%dx%d" % (16 * f, th * tw) in info
+    else:
+        assert "conv_kr16" in info and "tile=%dx16" % (16 * fm) in info
     assert err <= TOL[storage], info
 
 
