@@ -1127,9 +1127,11 @@ __global__ __launch_bounds__(512) void conv_kr16_kernel(const ConvP16Params p) {
             const f32x4_t sc = *reinterpret_cast<const f32x4_t*>(sb + fm * 16 + kq * 4);
             const f32x4_t bi = *reinterpret_cast<const f32x4_t*>(sb + 16 * FM + fm * 16 + kq * 4);
             const int ch = cb * 16 * FM + fm * 16 + kq * 4;
+            // (the last block of output channels may reach beyond the tensor's channel pitch: those rows are not stored)
+            const bool okc = okp && ch + 4 <= p.out_cp;
 #pragma unroll
             for (int e = 0; e < 4; e++) v[e] = v[e] * (sc[e] * acc_mul) + bi[e];
-            if (res && okp) {
+            if (res && okc) {
                 const store_t* rp = res + ((size_t)(p.res_off_y + py) * p.res_wp + p.res_off_x + px) * p.res_cp + ch;
                 f32x4_t rv;
                 if constexpr (HSTORE) {
@@ -1151,11 +1153,11 @@ __global__ __launch_bounds__(512) void conv_kr16_kernel(const ConvP16Params p) {
                 half4_t hv;
 #pragma unroll
                 for (int e = 0; e < 4; e++) hv[e] = (_Float16)v[e];
-                if (okp) *reinterpret_cast<half4_t*>(op) = hv;
+                if (okc) *reinterpret_cast<half4_t*>(op) = hv;
             } else {
 #pragma unroll
-                for (int e = 0; e < 4; e++) vmax = fmaxf(vmax, okp ? fabsf(v[e]) : 0.f);
-                if (okp) *reinterpret_cast<f32x4_t*>(op) = v;
+                for (int e = 0; e < 4; e++) vmax = fmaxf(vmax, okc ? fabsf(v[e]) : 0.f);
+                if (okc) *reinterpret_cast<f32x4_t*>(op) = v;
             }
         }
     }
@@ -1292,8 +1294,7 @@ int P16_NAME(launch_conv_kr16)(const ConvP16Params& p, int k, hipStream_t s) {
     const KREntry* e = find_krentry(p, k);
     if (!e) return -1;
     if (p.in_cp > p.cin_chunks * KC || p.in_cp % 8 != 0 || p.in_cp < 8 || p.cout_blocks < 1 || p.mfrags != p.cout_blocks * e->fm || p.stride < 1 || (k != 1 && p.stride != 1) ||
-        p.tiles_x * e->tw < p.npos_x || p.tiles_y * e->th < p.npos_y || p.out_cp < p.cout_blocks * 16 * e->fm || (p.out_cp * ESZ) % 16 != 0 ||
-        (p.res && (p.res_cp < p.cout_blocks * 16 * e->fm || (p.res_cp * ESZ) % 16 != 0)) || p.nreset < 0 || p.nreset > 4 || (p.f16 != 0) != HSTORE ||
+        p.tiles_x * e->tw < p.npos_x || p.tiles_y * e->th < p.npos_y || p.out_cp % 4 != 0 || p.out_cp < 4 || (p.res && p.res_cp < p.out_cp) || p.nreset < 0 || p.nreset > 4 || (p.f16 != 0) != HSTORE ||
         p.tiles_x < 1 || p.tiles_y < 1 || (long long)p.tiles_x * p.tiles_y * p.cout_blocks > 65535)
         return -5;
     if (e->lds > 160 * 1024) return -2;

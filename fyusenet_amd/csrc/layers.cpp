@@ -1216,25 +1216,26 @@ class ConvLayer : public Layer {
         for (int i = 0; i < conv_kr16_variant_count(); i++) {
             int taps, chunks, fm, th, tw;
             conv_kr16_variant(i, &taps, &chunks, &fm, &th, &tw);
-            if (taps != k * k || chunks != q.cin_chunks || oc % (16 * fm) != 0 || (want_fm && fm != want_fm)) continue;
+            if (taps != k * k || chunks != q.cin_chunks || (want_fm && fm != want_fm)) continue;
+            if (fm == 2 && oc % 32 != 0 && oc % 32 <= 16) continue;   // (the last block would be half empty: the 16-channel blocks do)
             if (want_th ? (th != want_th || tw != want_tw) : (want_fm && th * tw != 16)) continue;
             // (larger tiles are for layers that would need several rounds of 16-position workgroups)
-            if (th * tw > 16 && !want_th && ((oh + 3) / 4) * ((ow + 3) / 4) * (oc / (16 * fm)) <= 512) continue;
+            if (th * tw > 16 && !want_th && ((oh + 3) / 4) * ((ow + 3) / 4) * ((oc + 16 * fm - 1) / (16 * fm)) <= 512) continue;
             ConvP16Params c = q;
             c.tile_h = th; c.tile_w = tw;
             c.tiles_x = (ow + tw - 1) / tw; c.tiles_y = (oh + th - 1) / th;
             c.rcp_tiles_x = 1.0f / (float)c.tiles_x;
             c.pos_groups = c.tiles_x * c.tiles_y;
             c.wm = fm;
-            c.cout_blocks = oc / (16 * fm);
-            c.mfrags = oc / 16;
+            c.cout_blocks = (oc + 16 * fm - 1) / (16 * fm);   // (the last block may be partly empty: zero weights, rows beyond the pitch not stored)
+            c.mfrags = c.cout_blocks * fm;
             const size_t lds = conv_kr16_lds_bytes(c, k);
             if (lds == 0 || lds > 160 * 1024 || (long long)c.pos_groups * c.cout_blocks > 65535) continue;
             cands.push_back(c);
         }
         if (cands.empty()) return;
-        // (the same size for every candidate: cout blocks x 4 waves x steps x fragments x planes)
-        const size_t halves = (size_t)(oc / 16) * 4 * (q.cin_chunks / 4) * k * k * (q.f16 ? 1 : 2) * 64 * 8;
+        // (large enough for every candidate: cout blocks x 4 waves x steps x fragments x planes)
+        const size_t halves = (size_t)((oc + 31) / 32 * 2) * 4 * (q.cin_chunks / 4) * k * k * (q.f16 ? 1 : 2) * 64 * 8;
         void* const kr_wpack = net->dev_alloc(halves * 2, true);
         for (ConvP16Params& c : cands) c.wpack = kr_wpack;
         const bool had_p16 = p16;   // the 3x3 16-position form was chosen over the general kernel: this form has to beat it instead
@@ -1580,7 +1581,7 @@ class ConvLayer : public Layer {
                 setup_c4(in_v, out_v);
             // few positions, many input channels: the whole reduction of a 4x4 tile resident in LDS instead of K-split launches
             if ((!p16 || (!h16 && !c4)) && !frac_shift && same_storage && (k == 1 || (k == 3 && stride == 1)) && dil == 1 && in_v.cp % 8 == 0 &&
-                d.in_channels == in_v.cp && in_v.cp >= 16 && oc % 16 == 0 && out_v.cp >= oc && oh * ow <= 4096 && (!res_v || (res_v->cp >= oc && res_v->cp % 8 == 0)) &&
+                d.in_channels == in_v.cp && in_v.cp >= 16 && oc % 4 == 0 && oc >= 8 && out_v.cp >= oc && oh * ow <= 4096 && (!res_v || (res_v->cp >= out_v.cp && res_v->cp % 8 == 0)) &&
                 !getenv("FYNHIP_NO_P16_CONV") && !getenv("FYNHIP_NO_KR16_CONV") && !getenv("FYNHIP_FORCE_P16_CONV") &&
                 // (a test that forces a variant of the general kernel wants the general kernel)
                 !getenv("FYNHIP_FORCE_KSPLIT") && !getenv("FYNHIP_CONV_TILE") && !getenv("FYNHIP_CONV_KC") && !getenv("FYNHIP_CONV_KC_MAX") && !getenv("FYNHIP_CONV_PD"))

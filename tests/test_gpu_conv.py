@@ -401,6 +401,11 @@ KR16_CASES = [
     (3, 64, 64, 12, 12, 1, {"bn": True, "residual": (A.RELU, True)}),
     (1, 2048, 64, 7, 7, 1, {"bn": True}),                                       # 64 chunks: unpadded pixel pitch in LDS
     (1, 2048, 32, 5, 9, 2, {}),
+    # output channel counts that are no multiple of the block: the last block is partly empty
+    (1, 96, 24, 20, 20, 1, {"bn": True}),
+    (1, 64, 20, 8, 8, 1, {"residual": (A.RELU, True)}),                         # 20 channels in a pitch of 24
+    (1, 128, 56, 7, 7, 2, {"bn": True, "residual": (A.NONE, False)}),
+    (3, 128, 40, 10, 9, 1, {}),
     # larger tiles (fragments per block, tile h, tile w)
     (1, 64, 256, 56, 56, "2,8,8", {"bn": True}),
     (1, 256, 64, 30, 44, "1,4,8", {"residual": (A.RELU, True)}),
