@@ -924,12 +924,14 @@ __global__ __launch_bounds__(512) void conv_p16c4_kernel(const ConvP16Params p) 
 // and add their accumulators through LDS; wave 0 runs the epilogue.  Small tiles make many workgroups (13 tiles x 16
 // blocks of 16 channels for 1024 -> 256 at 14x14), so the layer's activations and weights are pulled through many CUs.
 // Weights: [cout block][wave][step][fragment][plane][lane][8 halves], the wave's steps being (chunk wave + 4*i, tap).
-template <int NTAPS, int CPW, int FN_ = 1>
+template <int NTAPS, int CPW, int FN_ = 1, int S_ = 1>
 struct GeoR {
     static constexpr int FN = FN_;                      // position fragments per tile: 4x4, 4x8 or 8x8 positions
+    static constexpr int S = S_;                        // stride of a 3x3 layer (a 1x1 layer's stride is a launch parameter: it only thins the pixels fetched)
     static constexpr int TH = (FN == 4) ? 8 : 4, TW = (FN == 1) ? 4 : 8, KH = (NTAPS == 9) ? 2 : 0;
     static_assert(FN == 1 || FN == 2 || FN == 4, "tiles of 16, 32 or 64 positions");
-    static constexpr int HW = TW + KH, HH = TH + KH;
+    static_assert(S == 1 || (S == 2 && NTAPS == 9), "stride 2 for 3x3");
+    static constexpr int HW = S * (TW - 1) + 1 + KH, HH = S * (TH - 1) + 1 + KH;
     static constexpr int NCH = 4 * CPW;                 // chunks of the layer
     // (64 chunks -- 2048 input channels -- fit the LDS only without the padding that keeps the fragment reads free of
     // bank conflicts; the reads are a small part of this kernel)
@@ -947,9 +949,9 @@ struct GeoR {
     static_assert(NTAPS == 1 || NTAPS == 9, "1x1 or 3x3");
 };
 
-template <int NTAPS, int CPW, int FM, int FN>
+template <int NTAPS, int CPW, int FM, int FN, int S>
 __global__ __launch_bounds__(512) void conv_kr16_kernel(const ConvP16Params p) {
-    using G = GeoR<NTAPS, CPW, FN>;
+    using G = GeoR<NTAPS, CPW, FN, S>;
     constexpr int RPD = G::RPD, BD = G::BD, STEPS = G::STEPS;
     extern __shared__ __align__(16) unsigned char lds[];
     __shared__ unsigned range_box[2];
@@ -974,8 +976,9 @@ __global__ __launch_bounds__(512) void conv_kr16_kernel(const ConvP16Params p) {
         int l_off[G::NB];
         bool ok[G::NB];
         // (a 1x1 layer may step over the input: position (y, x) reads pixel (y, x) * stride)
-        const int st = NTAPS == 1 ? p.stride : 1;
-        const int y0 = tyi * G::TH * st + p.in_y0, x0 = txi * G::TW * st + p.in_x0;
+        // (a 3x3 layer with stride 2 stages every pixel under its tile: position (y, x) reads the window at (2y, 2x))
+        const int st = NTAPS == 1 ? p.stride : 1, org = NTAPS == 1 ? p.stride : S;
+        const int y0 = tyi * G::TH * org + p.in_y0, x0 = txi * G::TW * org + p.in_x0;
 #pragma unroll
         for (int i = 0; i < G::NB; i++) {
             const int idx = stid + i * 256;
@@ -1037,7 +1040,7 @@ __global__ __launch_bounds__(512) void conv_kr16_kernel(const ConvP16Params p) {
 #pragma unroll
     for (int fn = 0; fn < FN; fn++) {
         const int m = fn * 16 + mq;
-        bbase[fn] = (m / G::TW) * G::ROW_PITCH + (m % G::TW) * G::PIT + kq * 16 + w * G::BUFC;
+        bbase[fn] = (m / G::TW) * S * G::ROW_PITCH + (m % G::TW) * S * G::PIT + kq * 16 + w * G::BUFC;
     }
     constexpr unsigned wstep = FM * NPL * 1024;
     const unsigned char* wbase = reinterpret_cast<const unsigned char*>(p.wpack) + (size_t)((cb * 4 + w) * STEPS) * wstep + lane * 16;
@@ -1207,14 +1210,14 @@ template <int K, int TH, int TW>
 constexpr C4Entry c4entry() { return C4Entry{K, TH, TW, conv_p16c4_kernel<K, TH, TW>, (size_t)GeoC4<K, TH, TW>::BUF, GeoC4<K, TH, TW>::NS}; }
 const C4Entry kC4Entries[] = {c4entry<9, 8, 8>(), c4entry<9, 4, 8>(), c4entry<9, 8, 4>()};
 struct KREntry {
-    int taps, cpw, fm, nfrag, th, tw;
+    int taps, cpw, fm, nfrag, th, tw, stride;
     p16_fn fn;
     size_t lds;
 };
-template <int NTAPS, int CPW, int FM, int FN = 1>
+template <int NTAPS, int CPW, int FM, int FN = 1, int S = 1>
 constexpr KREntry krentry() {
-    using G = GeoR<NTAPS, CPW, FN>;
-    return KREntry{NTAPS, CPW, FM, FN, G::TH, G::TW, conv_kr16_kernel<NTAPS, CPW, FM, FN>, (size_t)(G::RED_OFF + 3 * FM * FN * 1024 + 2 * 16 * FM * 4)};
+    using G = GeoR<NTAPS, CPW, FN, S>;
+    return KREntry{NTAPS, CPW, FM, FN, G::TH, G::TW, S, conv_kr16_kernel<NTAPS, CPW, FM, FN, S>, (size_t)(G::RED_OFF + 3 * FM * FN * 1024 + 2 * 16 * FM * 4)};
 }
 const KREntry kKREntries[] = {
     krentry<1, 1, 1>(), krentry<1, 2, 1>(), krentry<1, 3, 1>(), krentry<1, 4, 1>(), krentry<1, 5, 1>(), krentry<1, 8, 1>(), krentry<1, 16, 1>(),
@@ -1223,6 +1226,8 @@ const KREntry kKREntries[] = {
     // larger tiles for layers with more positions and a short reduction
     krentry<1, 1, 1, 2>(), krentry<1, 1, 2, 2>(), krentry<1, 2, 1, 2>(), krentry<1, 2, 2, 2>(), krentry<9, 1, 1, 2>(), krentry<9, 1, 2, 2>(),
     krentry<1, 1, 1, 4>(), krentry<1, 1, 2, 4>(), krentry<1, 2, 1, 4>(), krentry<1, 2, 2, 4>(), krentry<9, 1, 1, 4>(), krentry<9, 1, 2, 4>(),
+    // 3x3 with stride 2 (a 9x9-pixel window per chunk under a tile of 4x4 positions)
+    krentry<9, 1, 1, 1, 2>(), krentry<9, 1, 2, 1, 2>(), krentry<9, 2, 1, 1, 2>(), krentry<9, 2, 2, 1, 2>(), krentry<9, 4, 1, 1, 2>(), krentry<9, 4, 2, 1, 2>(),
 };
 }  // namespace
 
@@ -1263,9 +1268,9 @@ void conv_p16c4_tile(int index, int* k, int* th, int* tw, int* steps) {
     *k = kC4Entries[index].k; *th = kC4Entries[index].th; *tw = kC4Entries[index].tw; *steps = kC4Entries[index].steps;
 }
 int conv_kr16_variant_count() { return (int)(sizeof(kKREntries) / sizeof(kKREntries[0])); }
-void conv_kr16_variant(int index, int* taps, int* chunks, int* fm, int* th, int* tw) {
+void conv_kr16_variant(int index, int* taps, int* chunks, int* fm, int* th, int* tw, int* stride) {
     *taps = kKREntries[index].taps; *chunks = 4 * kKREntries[index].cpw; *fm = kKREntries[index].fm;
-    *th = kKREntries[index].th; *tw = kKREntries[index].tw;
+    *th = kKREntries[index].th; *tw = kKREntries[index].tw; *stride = kKREntries[index].stride;
 }
 bool conv_p16c4_supported(int k, int stride, int dil, int in_cp, int cout, int out_cp, bool f16) {
     (void)f16;
@@ -1275,7 +1280,7 @@ bool conv_p16c4_supported(int k, int stride, int dil, int in_cp, int cout, int o
 
 static const KREntry* find_krentry(const ConvP16Params& p, int k) {
     for (const KREntry& c : kKREntries)
-        if (c.taps == k * k && c.cpw * 4 == p.cin_chunks && c.fm == p.wm && c.th == p.tile_h && c.tw == p.tile_w) return &c;
+        if (c.taps == k * k && c.cpw * 4 == p.cin_chunks && c.fm == p.wm && c.th == p.tile_h && c.tw == p.tile_w && c.stride == (k == 1 ? 1 : p.stride)) return &c;
     return nullptr;
 }
 size_t P16_NAME(conv_kr16_lds_bytes)(const ConvP16Params& p, int k) {
@@ -1285,7 +1290,7 @@ size_t P16_NAME(conv_kr16_lds_bytes)(const ConvP16Params& p, int k) {
     const KREntry* e = find_krentry(p, k);
     return e ? e->lds : 0;
 }
-// The K-resident form: k = 1 (any stride) or 3 (stride 1); tiles of tile_h x tile_w = 4x4 (4x8, 8x8 for short reductions) positions, blocks of 16*p.wm output channels (p.wm = 1 or 2),
+// The K-resident form: k = 1 (any stride) or 3 (stride 1, or 2 with 4x4 tiles); tiles of tile_h x tile_w = 4x4 (4x8, 8x8 for short reductions) positions, blocks of 16*p.wm output channels (p.wm = 1 or 2),
 // p.cin_chunks = 4, 8, 12, 16, 20, 32 or 64 (3x3: 4, 8 or 16), channels behind in_cp reading as zero; in_y0/in_x0 = input padding - (k-1)/2; one workgroup per tile and block
 int P16_NAME(launch_conv_kr16)(const ConvP16Params& p, int k, hipStream_t s) {
 #if !FYN_P16_HALF
@@ -1293,7 +1298,7 @@ int P16_NAME(launch_conv_kr16)(const ConvP16Params& p, int k, hipStream_t s) {
 #endif
     const KREntry* e = find_krentry(p, k);
     if (!e) return -1;
-    if (p.in_cp > p.cin_chunks * KC || p.in_cp % 8 != 0 || p.in_cp < 8 || p.cout_blocks < 1 || p.mfrags != p.cout_blocks * e->fm || p.stride < 1 || (k != 1 && p.stride != 1) ||
+    if (p.in_cp > p.cin_chunks * KC || p.in_cp % 8 != 0 || p.in_cp < 8 || p.cout_blocks < 1 || p.mfrags != p.cout_blocks * e->fm || p.stride < 1 ||
         p.tiles_x * e->tw < p.npos_x || p.tiles_y * e->th < p.npos_y || p.out_cp % 4 != 0 || p.out_cp < 4 || (p.res && p.res_cp < p.out_cp) || p.nreset < 0 || p.nreset > 4 || (p.f16 != 0) != HSTORE ||
         p.tiles_x < 1 || p.tiles_y < 1 || (long long)p.tiles_x * p.tiles_y * p.cout_blocks > 65535)
         return -5;

@@ -227,7 +227,7 @@ int launch_conv_p16c4(const ConvP16Params& p, int k, hipStream_t s);
 // positions, blocks of 16*wm output channels, the whole reduction of a tile in LDS; wpack: [cout block][wave 0..3][step]
 // [fragment][plane][lane][8 halves], a wave's steps being (chunk wave + 4*i, tap)
 int conv_kr16_variant_count();
-void conv_kr16_variant(int index, int* taps, int* chunks, int* fm, int* th, int* tw);   // compiled combinations: kernel taps, 32-channel chunks, fragments per block, tile
+void conv_kr16_variant(int index, int* taps, int* chunks, int* fm, int* th, int* tw, int* stride);   // compiled combinations: kernel taps, 32-channel chunks, fragments per block, tile
 size_t conv_kr16_lds_bytes(const ConvP16Params& p, int k);
 int launch_conv_kr16(const ConvP16Params& p, int k, hipStream_t s);
 // the K x K convolution (K = 3 or 9, stride 1) between fp16 tensors on the same parameters (conv_h16.hip): 128 output

@@ -1198,7 +1198,7 @@ class ConvLayer : public Layer {
         ConvP16Params q{};
         q.in = in_v.ptr; q.out = out_v.ptr; q.res = res_v ? res_v->ptr : nullptr;
         q.in_hp = in_v.hp(); q.in_wp = in_v.wp(); q.in_cp = in_v.cp;
-        q.stride = stride;   // (k = 1 only: position (y, x) reads pixel (y, x) * stride)
+        q.stride = stride;   // (k = 1: position (y, x) reads pixel (y, x) * stride; k = 3: the kernel variant's stride)
         q.in_y0 = q.in_x0 = in_v.pad - (k - 1) / 2;
         q.in_clamp = clamp ? 1 : 0;
         q.npos_y = oh; q.npos_x = ow;
@@ -1214,9 +1214,9 @@ class ConvLayer : public Layer {
         if (const char* e = getenv("FYNHIP_KR16_FM")) sscanf(e, "%d,%d,%d", &want_fm, &want_th, &want_tw);
         std::vector<ConvP16Params> cands;
         for (int i = 0; i < conv_kr16_variant_count(); i++) {
-            int taps, chunks, fm, th, tw;
-            conv_kr16_variant(i, &taps, &chunks, &fm, &th, &tw);
-            if (taps != k * k || chunks != q.cin_chunks || (want_fm && fm != want_fm)) continue;
+            int taps, chunks, fm, th, tw, vstride;
+            conv_kr16_variant(i, &taps, &chunks, &fm, &th, &tw, &vstride);
+            if (taps != k * k || chunks != q.cin_chunks || (want_fm && fm != want_fm) || (k != 1 && vstride != stride)) continue;
             if (fm == 2 && oc % 32 != 0 && oc % 32 <= 16) continue;   // (the last block would be half empty: the 16-channel blocks do)
             if (want_th ? (th != want_th || tw != want_tw) : (want_fm && th * tw != 16)) continue;
             // (larger tiles are for layers that would need several rounds of 16-position workgroups)
@@ -1580,7 +1580,7 @@ class ConvLayer : public Layer {
                 !getenv("FYNHIP_NO_P16_CONV"))
                 setup_c4(in_v, out_v);
             // few positions, many input channels: the whole reduction of a 4x4 tile resident in LDS instead of K-split launches
-            if ((!p16 || (!h16 && !c4)) && !frac_shift && same_storage && (k == 1 || (k == 3 && stride == 1)) && dil == 1 && in_v.cp % 8 == 0 &&
+            if ((!p16 || (!h16 && !c4)) && !frac_shift && same_storage && (k == 1 || (k == 3 && (stride == 1 || stride == 2))) && dil == 1 && in_v.cp % 8 == 0 &&
                 d.in_channels == in_v.cp && in_v.cp >= 16 && oc % 4 == 0 && oc >= 8 && out_v.cp >= oc && oh * ow <= 4096 && (!res_v || (res_v->cp >= out_v.cp && res_v->cp % 8 == 0)) &&
                 !getenv("FYNHIP_NO_P16_CONV") && !getenv("FYNHIP_NO_KR16_CONV") && !getenv("FYNHIP_FORCE_P16_CONV") &&
                 // (a test that forces a variant of the general kernel wants the general kernel)

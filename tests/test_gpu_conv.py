@@ -412,13 +412,19 @@ KR16_CASES = [
     (3, 64, 64, 29, 35, "2,8,8", {"bn": True, "residual": (A.NONE, False)}),
     (3, 96, 48, 20, 12, "1,4,8", {"pad_out": 1}),
     (1, 24, 144, 56, 56, "1,8,8", {}),
+    # 3x3 with stride 2: a window of 9x9 pixels per chunk under a tile of 4x4 positions
+    (3, 128, 128, 56, 56, 1, {"stride": 2, "bn": True}),                        # the first 3x3 layer of ResNet's stage 2
+    (3, 256, 64, 28, 28, 2, {"stride": 2}),
+    (3, 256, 48, 13, 15, 1, {"stride": 2, "bn": True, "residual": (A.RELU, True)}),   # odd input size
+    (3, 64, 32, 10, 22, 2, {"stride": 2, "pad_out": 1}),
+    (3, 512, 32, 14, 14, 2, {"stride": 2}),                                     # 16 chunks (fp16 storage only: LDS)
 ]
 
 
 @pytest.mark.parametrize("storage", [fa.STORAGE_F32, fa.STORAGE_F16], ids=["f32", "f16"])
 @pytest.mark.parametrize("shallow", [False, True], ids=["deep", "shallow_edge_clamp"])
 @pytest.mark.parametrize("act", [A.RELU, A.LEAKY_RELU], ids=["relu", "leaky"])
-@pytest.mark.parametrize("case", KR16_CASES, ids=lambda c: "k%d_%dx%dx%d_to%d_fm%s" % (c[0], c[1], c[3], c[4], c[2], str(c[5]).replace(",", "x")))
+@pytest.mark.parametrize("case", KR16_CASES, ids=lambda c: "k%d_%dx%dx%d_to%d_fm%s%s" % (c[0], c[1], c[3], c[4], c[2], str(c[5]).replace(",", "x"), "_s2" if c[6].get("stride") == 2 else ""))
 def test_reduction_resident_form(case, act, shallow, storage, monkeypatch):
     """1x1 / 3x3 convolutions on few positions and many input channels with a tile's whole reduction resident in LDS and
     the four MFMA waves of a workgroup splitting the chunks."""
@@ -427,6 +433,8 @@ def test_reduction_resident_form(case, act, shallow, storage, monkeypatch):
         pytest.skip("the shallow variant is run on the plain 3x3 cases")
     if act is A.LEAKY_RELU and (cin > 512 or "pad_out" in kw):
         pytest.skip("activations are varied on some of the cases")
+    if k == 3 and kw.get("stride", 1) == 2 and cin > 256 and storage == fa.STORAGE_F32:
+        pytest.skip("the stride-2 windows of 16 chunks in two planes are more than a CU's LDS")
     monkeypatch.setenv("FYNHIP_FORCE_KR16_CONV", "1")
     monkeypatch.setenv("FYNHIP_KR16_FM", str(fm))
     if shallow:
