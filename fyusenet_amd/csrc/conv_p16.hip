@@ -949,9 +949,14 @@ struct GeoR {
     static_assert(NTAPS == 1 || NTAPS == 9, "1x1 or 3x3");
 };
 
-template <int NTAPS, int CPW, int FM, int FN, int S>
+// DWS = 1 or 2: the input of a 1x1 layer is not read from memory but computed by the staging waves: it is the output of
+// a depthwise 3x3 layer with step DWS (weights fp32, folded scale and bias, the arithmetic and the rounding to the
+// storage type of the depthwise kernel in layers_direct.hip), whose tensor then never exists.  A staging item is a pair
+// of horizontally neighbouring positions and 8 channels: 3 x (DWS + 3) texels of the depthwise layer's input.
+template <int NTAPS, int CPW, int FM, int FN, int S, int DWS = 0>
 __global__ __launch_bounds__(512) void conv_kr16_kernel(const ConvP16Params p) {
     using G = GeoR<NTAPS, CPW, FN, S>;
+    static_assert(DWS == 0 || (NTAPS == 1 && FN == 1 && S == 1 && DWS <= 2), "a fused depthwise layer: 1x1, tiles of 4x4 positions");
     constexpr int RPD = G::RPD, BD = G::BD, STEPS = G::STEPS;
     extern __shared__ __align__(16) unsigned char lds[];
     __shared__ unsigned range_box[2];
@@ -972,6 +977,126 @@ __global__ __launch_bounds__(512) void conv_kr16_kernel(const ConvP16Params p) {
         const store_t* in = reinterpret_cast<const store_t*>(p.in);
         struct RawF { float4 a, b; };
         typedef typename std::conditional<HSTORE, half8_t, RawF>::type raw_t;
+        if constexpr (DWS > 0) {
+            constexpr int WINW = DWS + 3;
+            constexpr int TOTAL = G::NCH * 32, NB = (TOTAL + 255) / 256;
+            constexpr int IPP_MAX = (HSTORE && !(DWS == 2 && NB > 1)) ? 2 : 1;   // items whose texels are in flight together (registers)
+            constexpr int IPP = NB < IPP_MAX ? NB : IPP_MAX;
+            const store_t* din = reinterpret_cast<const store_t*>(p.dw_in);
+            float in_scale = 1.f, inv_unused;
+            if (p.in_amax) in_scale = range_scale(range_after_act(range_reduce(range_bits), p.act), &inv_unused);
+            if (stid < 16 * FM) {
+                reinterpret_cast<float*>(lds + sb_off)[stid] = p.scale[cb * 16 * FM + stid];
+                reinterpret_cast<float*>(lds + sb_off)[16 * FM + stid] = p.bias[cb * 16 * FM + stid];
+            }
+            // (a clamp that is exact on halves is applied to the packed halves, as in the depthwise kernel)
+            const _Float16 hlo = (_Float16)p.dw_act.lo, hhi = (_Float16)p.dw_act.hi;
+            const bool packed_act = HSTORE && p.dw_act.leak == 0.f && (float)hlo == p.dw_act.lo && (float)hhi == p.dw_act.hi;
+#pragma unroll
+            for (int i0 = 0; i0 < NB; i0 += IPP) {
+                raw_t raw[IPP][3][WINW];
+                unsigned okm[IPP];
+#pragma unroll
+                for (int ii = 0; ii < IPP; ii++) {
+                    if (i0 + ii >= NB) continue;
+                    const int idx = stid + (i0 + ii) * 256;
+                    const int chunk = idx >> 5, pair = (idx >> 2) & 7, g = idx & 3;
+                    const int oy = tyi * 4 + (pair >> 1), ox = txi * 4 + (pair & 1) * 2;
+                    const int ch = chunk * KC + g * 8;
+                    const bool chan_ok = idx < TOTAL && ch < p.dw_cp;
+                    okm[ii] = 0u;
+#pragma unroll
+                    for (int r = 0; r < 3; r++)
+#pragma unroll
+                        for (int c = 0; c < WINW; c++) {
+                            const int iy = oy * DWS + r + p.dw_y0, ix = ox * DWS + c + p.dw_x0;
+                            const bool ok = chan_ok && (unsigned)iy < (unsigned)p.dw_hp && (unsigned)ix < (unsigned)p.dw_wp;
+                            okm[ii] |= ok ? 1u << (r * WINW + c) : 0u;
+                            const store_t* src = din + (ok ? (iy * p.dw_wp + ix) * p.dw_cp + ch : 0);
+                            if constexpr (HSTORE) {
+                                raw[ii][r][c] = *reinterpret_cast<const half8_t*>(src);
+                            } else {
+                                raw[ii][r][c].a = *reinterpret_cast<const float4*>(src);
+                                raw[ii][r][c].b = *reinterpret_cast<const float4*>(src + 4);
+                            }
+                        }
+                }
+#pragma unroll
+                for (int ii = 0; ii < IPP; ii++) {
+                    if (i0 + ii >= NB) continue;
+                    const int idx = stid + (i0 + ii) * 256;
+                    if (idx >= TOTAL) continue;
+                    const int chunk = idx >> 5, pair = (idx >> 2) & 7, g = idx & 3;
+                    const int ch = chunk * KC + g * 8;
+                    const bool chan_ok = ch < p.dw_cp;
+                    const int wch = chan_ok ? ch : 0;
+                    float acc[2][8];
+#pragma unroll
+                    for (int j = 0; j < 2; j++)
+#pragma unroll
+                        for (int e = 0; e < 8; e++) acc[j][e] = 0.f;
+#pragma unroll
+                    for (int r = 0; r < 3; r++) {
+                        // (a texel outside the stored frame is a zero that the activation is applied to, as in the depthwise kernel)
+                        float row[WINW][8];
+#pragma unroll
+                        for (int c = 0; c < WINW; c++) {
+                            const bool ok = (okm[ii] >> (r * WINW + c)) & 1u;
+                            float x[8];
+                            if constexpr (HSTORE) {
+                                if (packed_act) {
+                                    half8_t h = ok ? raw[ii][r][c] : (half8_t)((_Float16)0.f);
+                                    h = __builtin_elementwise_min(__builtin_elementwise_max(h, (half8_t)hlo), (half8_t)hhi);
+#pragma unroll
+                                    for (int e = 0; e < 8; e++) row[c][e] = (float)h[e];
+                                    continue;
+                                }
+#pragma unroll
+                                for (int e = 0; e < 8; e++) x[e] = (float)raw[ii][r][c][e];
+                            } else {
+                                const float4 a = raw[ii][r][c].a, b = raw[ii][r][c].b;
+                                x[0] = a.x; x[1] = a.y; x[2] = a.z; x[3] = a.w; x[4] = b.x; x[5] = b.y; x[6] = b.z; x[7] = b.w;
+                            }
+#pragma unroll
+                            for (int e = 0; e < 8; e++) row[c][e] = act_p16(ok ? x[e] : 0.f, p.dw_act);
+                        }
+#pragma unroll
+                        for (int kx = 0; kx < 3; kx++) {
+                            // (the weights come through the L1: staging them in LDS first cost a barrier and measured slower)
+                            const float* wp = p.dw_w + (r * 3 + kx) * p.dw_cp + wch;
+                            const float4 w0 = *reinterpret_cast<const float4*>(wp), w1 = *reinterpret_cast<const float4*>(wp + 4);
+                            const float w[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
+#pragma unroll
+                            for (int j = 0; j < 2; j++)
+#pragma unroll
+                                for (int e = 0; e < 8; e++) acc[j][e] = fmaf(row[j * DWS + kx][e], w[e], acc[j][e]);
+                        }
+                    }
+                    const float4 s0 = *reinterpret_cast<const float4*>(p.dw_scale + wch), s1 = *reinterpret_cast<const float4*>(p.dw_scale + wch + 4);
+                    const float4 b0 = *reinterpret_cast<const float4*>(p.dw_bias + wch), b1 = *reinterpret_cast<const float4*>(p.dw_bias + wch + 4);
+                    const float sc[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
+                    const float bi[8] = {b0.x, b0.y, b0.z, b0.w, b1.x, b1.y, b1.z, b1.w};
+                    const int lo0 = chunk * G::BUFC + (pair >> 1) * G::ROW_PITCH + (pair & 1) * 2 * G::PIT + g * 16;
+#pragma unroll
+                    for (int j = 0; j < 2; j++) {
+                        half8_t hi, lo;
+#pragma unroll
+                        for (int e = 0; e < 8; e++) {
+                            float o = acc[j][e] * sc[e] + bi[e];
+                            if constexpr (HSTORE) o = (float)(_Float16)o;   // (what the depthwise layer would have stored)
+                            const float v = chan_ok ? act_p16(o, p.act) * in_scale : 0.f;
+                            hi[e] = (_Float16)v;
+                            lo[e] = (_Float16)(v - (float)hi[e]);
+                        }
+                        *reinterpret_cast<half8_t*>(lds + lo0 + j * G::PIT) = hi;
+                        if constexpr (!HSTORE) *reinterpret_cast<half8_t*>(lds + G::PLANE + lo0 + j * G::PIT) = lo;
+                    }
+                }
+            }
+            lds_barrier();   // the tile is staged
+            lds_barrier();   // the MFMA waves have left their accumulators for wave 0
+            return;
+        }
         raw_t raw[G::NB];
         int l_off[G::NB];
         bool ok[G::NB];
@@ -1210,14 +1335,14 @@ template <int K, int TH, int TW>
 constexpr C4Entry c4entry() { return C4Entry{K, TH, TW, conv_p16c4_kernel<K, TH, TW>, (size_t)GeoC4<K, TH, TW>::BUF, GeoC4<K, TH, TW>::NS}; }
 const C4Entry kC4Entries[] = {c4entry<9, 8, 8>(), c4entry<9, 4, 8>(), c4entry<9, 8, 4>()};
 struct KREntry {
-    int taps, cpw, fm, nfrag, th, tw, stride;
+    int taps, cpw, fm, nfrag, th, tw, stride, dws;
     p16_fn fn;
     size_t lds;
 };
-template <int NTAPS, int CPW, int FM, int FN = 1, int S = 1>
+template <int NTAPS, int CPW, int FM, int FN = 1, int S = 1, int DWS = 0>
 constexpr KREntry krentry() {
     using G = GeoR<NTAPS, CPW, FN, S>;
-    return KREntry{NTAPS, CPW, FM, FN, G::TH, G::TW, S, conv_kr16_kernel<NTAPS, CPW, FM, FN, S>, (size_t)(G::RED_OFF + 3 * FM * FN * 1024 + 2 * 16 * FM * 4)};
+    return KREntry{NTAPS, CPW, FM, FN, G::TH, G::TW, S, DWS, conv_kr16_kernel<NTAPS, CPW, FM, FN, S, DWS>, (size_t)(G::RED_OFF + 3 * FM * FN * 1024 + 2 * 16 * FM * 4)};
 }
 const KREntry kKREntries[] = {
     krentry<1, 1, 1>(), krentry<1, 2, 1>(), krentry<1, 3, 1>(), krentry<1, 4, 1>(), krentry<1, 5, 1>(), krentry<1, 8, 1>(), krentry<1, 16, 1>(),
@@ -1229,6 +1354,10 @@ const KREntry kKREntries[] = {
     // 3x3 with stride 2 (a 9x9-pixel window per chunk under a tile of 4x4 positions)
     krentry<9, 1, 1, 1, 2>(), krentry<9, 1, 2, 1, 2>(), krentry<9, 2, 1, 1, 2>(), krentry<9, 2, 2, 1, 2>(), krentry<9, 4, 1, 1, 2>(), krentry<9, 4, 2, 1, 2>(),
 };
+// 1x1 with a depthwise 3x3 layer (step 1 or 2) computed in the staging
+#define FYN_KR_DW(CPW) krentry<1, CPW, 1, 1, 1, 1>(), krentry<1, CPW, 2, 1, 1, 1>(), krentry<1, CPW, 1, 1, 1, 2>(), krentry<1, CPW, 2, 1, 1, 2>()
+const KREntry kKRDwEntries[] = {FYN_KR_DW(1), FYN_KR_DW(2), FYN_KR_DW(3), FYN_KR_DW(4)};   // (up to 512 channels: beyond, two launches are faster)
+#undef FYN_KR_DW
 }  // namespace
 
 // Host entry points.  The fp32 unit holds the public ones and hands launches on fp16 tensors (p.f16) to the other
@@ -1279,6 +1408,11 @@ bool conv_p16c4_supported(int k, int stride, int dil, int in_cp, int cout, int o
 #endif
 
 static const KREntry* find_krentry(const ConvP16Params& p, int k) {
+    if (p.dw_in) {
+        for (const KREntry& c : kKRDwEntries)
+            if (k == 1 && c.cpw * 4 == p.cin_chunks && c.fm == p.wm && c.th == p.tile_h && c.tw == p.tile_w && c.dws == p.dw_stride) return &c;
+        return nullptr;
+    }
     for (const KREntry& c : kKREntries)
         if (c.taps == k * k && c.cpw * 4 == p.cin_chunks && c.fm == p.wm && c.th == p.tile_h && c.tw == p.tile_w && c.stride == (k == 1 ? 1 : p.stride)) return &c;
     return nullptr;
@@ -1302,6 +1436,8 @@ int P16_NAME(launch_conv_kr16)(const ConvP16Params& p, int k, hipStream_t s) {
         p.tiles_x * e->tw < p.npos_x || p.tiles_y * e->th < p.npos_y || p.out_cp % 4 != 0 || p.out_cp < 4 || (p.res && p.res_cp < p.out_cp) || p.nreset < 0 || p.nreset > 4 || (p.f16 != 0) != HSTORE ||
         p.tiles_x < 1 || p.tiles_y < 1 || (long long)p.tiles_x * p.tiles_y * p.cout_blocks > 65535)
         return -5;
+    // (a fused depthwise layer: its tensor has the pointwise layer's channels, in whole groups of 8, and the 1x1 layer does not step)
+    if (p.dw_in && (!p.dw_w || !p.dw_scale || !p.dw_bias || p.dw_cp != p.in_cp || p.stride != 1 || p.in_clamp || p.dw_hp < 1 || p.dw_wp < 1)) return -5;
     if (e->lds > 160 * 1024) return -2;
     if (ensure_lds(reinterpret_cast<const void*>(e->fn), e->lds) != 0) return -2;
     hipLaunchKernelGGL(e->fn, dim3(p.tiles_x * p.tiles_y * p.cout_blocks), dim3(512), e->lds, s, p);

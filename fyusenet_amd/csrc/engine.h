@@ -125,6 +125,9 @@ class Net {
     bool is_setup = false;
     bool timings = false;
     bool reuse_buffers = true;
+    // Layers fused into their neighbour's launch (fuse_depthwise_layers) run that way only in passes that neither time
+    // nor dump single layers, and only in networks whose intermediate tensors may share buffers.
+    bool fusion_on() const { return reuse_buffers && !timings && dump_dir.empty(); }
     std::string dump_dir;
     hipStream_t stream = nullptr;
     std::map<int, std::unique_ptr<Layer>> layers;  // ascending number = execution order
@@ -174,6 +177,7 @@ class Net {
 };
 
 Layer* create_layer(Net* net, const fyn_layer_desc& d);
+void fuse_depthwise_layers(Net* net);   // after every layer's setup(): depthwise 3x3 layers that their 1x1 reader can compute itself
 Layer* create_custom_layer(Net* net, const fyn_layer_desc& d, const fyn_custom_layer& impl);
 
 }  // namespace fynhip

@@ -199,6 +199,15 @@ struct ConvP16Params {
     long long* trace;     // timing-study builds only: 32 timestamps per workgroup and role
 #endif
     Act act;
+    // A depthwise 3x3 layer computed inside the staging of a 1x1 launch of the K-resident form (dw_in null: none): the
+    // layer's input tensor, its weights [9][dw_cp] and folded scale / bias [dw_cp], the stored coordinate of tap (0,0)
+    // of output position (0,0), its step and the activation applied to its input.  `in` is not read then.
+    const void* dw_in;
+    const float* dw_w;
+    const float* dw_scale;
+    const float* dw_bias;
+    int dw_hp, dw_wp, dw_cp, dw_y0, dw_x0, dw_stride;
+    Act dw_act;
 };
 // Output channel held by row `row` (0..15) of packed weight fragment `mf` when a wave holds groups of `fm` fragments: the
 // rows a lane ends up with (four consecutive ones of every fragment) are 4*fm consecutive channels.

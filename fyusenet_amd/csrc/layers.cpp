@@ -1659,6 +1659,10 @@ class ConvLayer : public Layer {
             if (launch_conv_rows(rp, tout().v.f16 != 0, s) != 0) fail(FYN_ERR_DEVICE, "layer %s: convolution launch failed", d.name);
             return;
         }
+        if (p16 && kr16 && dw_fused && net->fusion_on()) {
+            if (launch_conv_kr16(with_depthwise(), k, s) != 0) fail(FYN_ERR_DEVICE, "layer %s: convolution launch failed", d.name);
+            return;
+        }
         if (p16) {
             if ((c4 ? launch_conv_p16c4(pp, k, s) : (kr16 ? launch_conv_kr16(pp, k, s) : (h16 ? launch_conv_h16(pp, k, s) : launch_conv_p16(pp, s)))) != 0 ||
                 (h16 && h16_two && launch_conv_h16(pp2, k, s) != 0))
@@ -1690,6 +1694,7 @@ class ConvLayer : public Layer {
             char buf[220];
             snprintf(buf, sizeof(buf), "conv_kr16 %s tile=%dx%d(cout x pos) K-resident, 4 waves split %d chunks, blocks=%d lds=%zu steps=%d", pp.f16 ? "f16" : "f16x2-split",
                      16 * pp.wm, pp.tile_h * pp.tile_w, pp.cin_chunks, pp.pos_groups * pp.cout_blocks, conv_kr16_lds_bytes(pp, k), pp.cin_chunks / 4 * k * k);
+            if (dw_fused) return mode + buf + "; the depthwise 3x3 layer " + std::to_string(dw_layer_no) + " in front of it is computed by the staging waves";
             return mode + buf;
         }
         if (p16 && h16) {
@@ -1729,6 +1734,21 @@ class ConvLayer : public Layer {
     int c4_steps = 0;
     bool h16 = false;             // ... its fp16-storage form for wide layers (conv_h16.hip)
     bool kr16 = false;            // ... the K-resident form for layers with few positions (conv_p16.hip, conv_kr16_kernel)
+    // A depthwise 3x3 layer whose only reader is this 1x1 layer in the K-resident form can be computed inside this
+    // layer's staging (fuse_depthwise_layers below): the fields of ConvP16Params that describe it
+    bool dw_fused = false;
+    int dw_layer_no = -1;
+    ConvP16Params dw_fields{};
+    ConvP16Params with_depthwise() const {
+        ConvP16Params q = pp;
+        q.dw_in = dw_fields.dw_in; q.dw_w = dw_fields.dw_w; q.dw_scale = dw_fields.dw_scale; q.dw_bias = dw_fields.dw_bias;
+        q.dw_hp = dw_fields.dw_hp; q.dw_wp = dw_fields.dw_wp; q.dw_cp = dw_fields.dw_cp;
+        q.dw_y0 = dw_fields.dw_y0; q.dw_x0 = dw_fields.dw_x0; q.dw_stride = dw_fields.dw_stride; q.dw_act = dw_fields.dw_act;
+        return q;
+    }
+    bool takes_depthwise() const {
+        return p16 && kr16 && k == 1 && stride == 1 && pp.tile_h == 4 && pp.tile_w == 4 && !clamp && !pp.in_amax && !pp.in_clamp;
+    }
     bool h16_two = false;         // ...... as two launches on two bands of rows (pp, pp2)
     ConvP16Params pp{}, pp2{};
     void* p16_wpack_dev = nullptr;
@@ -1791,15 +1811,78 @@ class DwConvLayer : public Layer {
     }
     void forward(hipStream_t s) override {
         if (!have_weights) fail(FYN_ERR_STATE, "layer %s (%d): forward() without weights", d.name, d.number);
+        if (fused_into >= 0 && net->fusion_on()) return;   // computed inside the pointwise layer behind it
         launch_dwconv3x3(p, s);
     }
-    std::string info() const override { return "dwconv3x3"; }
+    std::string info() const override {
+        return fused_into >= 0 ? "dwconv3x3 (computed inside layer " + std::to_string(fused_into) + ", whose staging waves run it; no launch, no tensor)" : "dwconv3x3";
+    }
+    int fused_into = -1;
     int dil, stride;
     bool have_weights = false;
     std::vector<float> block;
     DwConvParams p{};
     float *w_dev = nullptr, *scale_dev = nullptr, *bias_dev = nullptr;
 };
+
+// Depthwise 3x3 -> pointwise 1x1 (the second half of an inverted-residual block) as one launch.  Where the pointwise
+// layer runs the K-resident form on 4x4 tiles and is the depthwise layer's only reader, its staging waves can compute
+// the depthwise layer for the tile instead of fetching that layer's output (conv_kr16_kernel, DWS): every workgroup of
+// a tile -- one per block of 16 or 32 output channels -- repeats the depthwise arithmetic for its tile, which costs
+// less than a launch as long as the blocks are few.  Both ways are timed; the depthwise layer's tensor is not written
+// when the fused way is taken, so the fusion is tied to buffer reuse (a caller who switches reuse off wants every
+// layer's tensor) and is left out of passes that time or dump single layers.
+void fuse_depthwise_layers(Net* net) {
+    if (getenv("FYNHIP_NO_DW_FUSION") || !net->reuse_buffers) return;
+    std::map<int, int> readers;
+    for (auto& kv : net->layers)
+        for (int t : kv.second->in)
+            if (t >= 0) readers[t]++;
+    for (auto& kv : net->layers) {
+        ConvLayer* pw = dynamic_cast<ConvLayer*>(kv.second.get());
+        if (!pw || !pw->takes_depthwise()) continue;
+        const Tensor& t = net->tensors[pw->in[0]];
+        if (t.producer < 0 || t.locked || readers[pw->in[0]] != 1) continue;
+        DwConvLayer* dw = dynamic_cast<DwConvLayer*>(net->layer(t.producer));
+        if (!dw || dw->dil != 1 || (dw->stride != 1 && dw->stride != 2) || dw->p.res.ptr || dw->p.in.cp % 8 != 0 || dw->p.in.cp != dw->p.out.cp ||
+            dw->p.in.f16 != dw->p.out.f16 || dw->p.out.f16 != pw->pp.f16 || dw->p.out.cp != pw->pp.in_cp)
+            continue;
+        ConvP16Params& f = pw->dw_fields;
+        f.dw_in = dw->p.in.ptr; f.dw_w = dw->w_dev; f.dw_scale = dw->scale_dev; f.dw_bias = dw->bias_dev;
+        f.dw_hp = dw->p.in.hp(); f.dw_wp = dw->p.in.wp(); f.dw_cp = dw->p.in.cp;
+        f.dw_y0 = f.dw_x0 = dw->p.in.pad - 1;
+        f.dw_stride = dw->stride; f.dw_act = dw->p.act;
+        const ConvP16Params q = pw->with_depthwise();
+        if (conv_kr16_lds_bytes(q, 1) == 0 || conv_kr16_lds_bytes(q, 1) > 160 * 1024) continue;
+        bool pick = true;
+        char key[200];
+        snprintf(key, sizeof(key), "dwpw:%d:%dx%dx%d:s%d:to%d:fm%d", q.f16, dw->p.in.cp, dw->p.in.h, dw->p.in.w, dw->stride, pw->oc, q.wm);
+        const char* at = getenv("FYNHIP_AUTOTUNE");
+        if (getenv("FYNHIP_FORCE_DW_FUSION")) {
+        } else if (tune_cache_flag(key, &pick)) {
+        } else if (!(at && at[0] == '0')) {
+            float t_fused = 1e30f, t_two = 1e30f;
+            for (int rep = 0; rep < 3; rep++) {
+                t_fused = std::min(t_fused, time_calls(net, [&]() {
+                    if (launch_conv_kr16(q, 1, net->stream) != 0) fail(FYN_ERR_DEVICE, "K-resident convolution with a depthwise layer in its staging: launch failed while tuning");
+                }, 10));
+                t_two = std::min(t_two, time_calls(net, [&]() {
+                    launch_dwconv3x3(dw->p, net->stream);
+                    if (launch_conv_kr16(pw->pp, 1, net->stream) != 0) fail(FYN_ERR_DEVICE, "K-resident convolution launch failed while tuning");
+                }, 10));
+            }
+            if (getenv("FYNHIP_TUNE_VERBOSE"))
+                fprintf(stderr, "[tune] depthwise 3x3 (step %d) on %d channels at %dx%d + 1x1 to %d: one launch %.1f us, two %.1f us\n", dw->stride, dw->p.in.cp,
+                        dw->p.in.h, dw->p.in.w, pw->oc, t_fused * 1e3f, t_two * 1e3f);
+            pick = t_fused < t_two;
+            tune_cache_store_flag(key, pick);
+        }
+        if (!pick) continue;
+        pw->dw_fused = true;
+        pw->dw_layer_no = dw->d.number;
+        dw->fused_into = pw->d.number;
+    }
+}
 
 // =============================================================================================
 // Transposed convolution, stride 2, K in {2,3}: one MFMA sub-convolution per output parity

@@ -1,0 +1,172 @@
+"""A depthwise 3x3 layer computed inside the staging of the 1x1 layer behind it (the second half of an inverted-residual
+block as one launch): parity against the oracle, equality with the two-launch form, and the conditions under which the
+engine leaves the two layers apart.  Tolerances: rel-L2 <= 1e-4 (fp32 storage), <= 2e-3 (fp16 storage)."""
+import numpy as np
+import pytest
+
+import fyusenet_amd as fa
+from fyusenet_amd import networks, prng
+from fyusenet_amd.builders import ActType, UpDownLayerBuilder
+from oracle import oracle as O
+from util import rel_l2
+
+pytestmark = pytest.mark.gpu
+TOL = {fa.STORAGE_F32: 1e-4, fa.STORAGE_F16: 2e-3}
+
+
+class Block(networks._StreamNet):
+    """upload -> 1x1 expand -> depthwise 3x3 (step 1 or 2, clip on fetch) -> 1x1 project (clip on fetch, optional residual
+    from the block's input) -> download."""
+    config_id = 4
+
+    def __init__(self, storage, cin, exp, cout, h, w, stride, residual, side_reader=False):
+        super().__init__(storage)
+        self.cin, self.exp, self.cout, self.h, self.w, self.stride, self.residual, self.side_reader = cin, exp, cout, h, w, stride, residual, side_reader
+
+    def define(self):
+        C, c6 = ActType.CLIP, (0.0, 6.0)
+        self._add(UpDownLayerBuilder(UpDownLayerBuilder.UPLOAD, "upload").number(0).shape(self.cin, self.h, self.w, self.cin))
+        self.conv(1, "expand", 1, self.cin, self.exp, self.h, self.w, 0, pad_out=1)
+        self.conv(2, "dw", 3, self.exp, self.exp, self.h, self.w, 1, stride=self.stride, act=C, clip=c6, groups=self.exp)
+        ho, wo = self.h // self.stride, self.w // self.stride
+        self.conv(3, "project", 1, self.exp, self.cout, ho, wo, 2, act=C, clip=c6, residual=0 if self.residual else None)
+        last = 3
+        if self.side_reader:   # a second reader of the depthwise layer's tensor
+            self.conv(4, "side", 1, self.exp, 16, ho, wo, 2, act=C, clip=c6)
+            last = 4
+        self._add(UpDownLayerBuilder(UpDownLayerBuilder.DOWNLOAD, "download").number(last + 1).shape(self.cout, ho, wo, self.cout).deep())
+        self._edges.append((3, last + 1, 0))
+        self.output_layer = last + 1
+
+    def makeInput(self):
+        return prng.uniform(977 + self.cin + self.h, (self.cin, self.h, self.w), -1.0, 1.0)
+
+    def setInput(self, x):
+        self.layers[0].setInput(x, 0)
+
+    input_key = (0, 0)
+
+
+def run(net, reuse=True):
+    net.setup(reuseBuffers=reuse)
+    x = net.makeInput()
+    net.setInput(x)
+    net.forward()
+    net.finish()
+    out = net.getOutput(net.output_layer)
+    infos = {lyr.name: lyr.kernelInfo() for lyr in net.layers}
+    return x, out, infos
+
+
+def assert_same_as_two_launches(fused, two, storage):
+    """fp32 storage: the same bits (same arithmetic in the same order).  fp16 storage: the depthwise layer's value is
+    rounded to fp16 on its way to the 1x1 layer in both forms, but the compiler may fold that rounding into the
+    multiply-add in front of it in one kernel and not in the other (one rounding instead of two): a few values per
+    thousand differ in their last bit, and a few outputs with them."""
+    if storage == fa.STORAGE_F32:
+        assert np.array_equal(fused, two)
+        return
+    d = np.abs(fused.astype(np.float64) - two.astype(np.float64))
+    assert (d > 0).mean() <= 0.02, "differing outputs: %d of %d" % ((d > 0).sum(), d.size)
+    assert d.max() <= 2.0 ** -9 * np.abs(two).max()
+
+
+CASES = [
+    # (cin, expanded channels, cout, h, w, step, residual)
+    (16, 96, 24, 28, 28, 1, False),      # one chunk per wave (96 channels padded to 128)
+    (24, 144, 24, 20, 24, 1, True),      # two chunks per wave, residual add in the pointwise epilogue
+    (32, 192, 64, 14, 14, 2, False),     # step 2
+    (64, 384, 96, 14, 14, 1, False),     # three chunks per wave, three blocks of 32 output channels
+    (64, 384, 64, 14, 14, 2, False),     # three chunks per wave, step 2: texels in two rounds
+    (80, 480, 112, 7, 7, 1, False),      # 15 chunks in use of 16
+    (32, 32, 16, 26, 22, 1, False),      # a single chunk in use, ragged tiles
+    (24, 144, 40, 13, 11, 2, False),     # odd input size with step 2, 40 output channels (last block partly empty)
+]
+
+
+@pytest.mark.parametrize("storage", [fa.STORAGE_F32, fa.STORAGE_F16], ids=["f32", "f16"])
+@pytest.mark.parametrize("case", CASES, ids=lambda c: "%dto%dto%d_%dx%d_s%d%s" % (c[0], c[1], c[2], c[3], c[4], c[5], "_res" if c[6] else ""))
+def test_depthwise_inside_pointwise_staging(case, storage, monkeypatch):
+    cin, exp, cout, h, w, stride, residual = case
+    monkeypatch.setenv("FYNHIP_FORCE_KR16_CONV", "1")
+    monkeypatch.setenv("FYNHIP_FORCE_DW_FUSION", "1")
+    net = Block(storage, cin, exp, cout, h, w, stride, residual)
+    x, got, infos = run(net)
+    desc = net.describe()
+    net.cleanup()
+    print("  ", infos["dw"], "|", infos["project"], flush=True)
+    assert "computed inside layer 3" in infos["dw"] and "depthwise 3x3 layer 2" in infos["project"]
+    ref = O.run_network(desc, {net.input_key: x})[net.output_layer]
+    err = rel_l2(got, ref)
+    print("   rel_l2=%.3e" % err, flush=True)
+    assert err <= TOL[storage]
+    monkeypatch.setenv("FYNHIP_NO_DW_FUSION", "1")
+    twin = Block(storage, cin, exp, cout, h, w, stride, residual)
+    _, two, infos2 = run(twin)
+    twin.cleanup()
+    assert infos2["dw"] == "dwconv3x3"
+    assert_same_as_two_launches(got, two, storage)
+
+
+def test_layers_stay_apart_when_the_tensor_is_needed(monkeypatch):
+    """No fusion when the depthwise layer's tensor has a second reader, or when the caller keeps every layer's tensor
+    (buffer reuse off); per-layer timing runs the layers apart and leaves the results unchanged."""
+    monkeypatch.setenv("FYNHIP_FORCE_KR16_CONV", "1")
+    monkeypatch.setenv("FYNHIP_FORCE_DW_FUSION", "1")
+    net = Block(fa.STORAGE_F16, 16, 96, 24, 28, 28, 1, False, side_reader=True)
+    _, _, infos = run(net)
+    net.cleanup()
+    assert infos["dw"] == "dwconv3x3"
+    net = Block(fa.STORAGE_F16, 96, 576, 160, 14, 14, 1, False)   # (more than 512 channels: no fused variant)
+    _, _, infos = run(net)
+    net.cleanup()
+    assert infos["dw"] == "dwconv3x3"
+    net = Block(fa.STORAGE_F16, 16, 96, 24, 28, 28, 1, False)
+    _, _, infos = run(net, reuse=False)
+    dw_out = net.layers[2].copyResult()
+    net.cleanup()
+    assert infos["dw"] == "dwconv3x3" and np.abs(dw_out).max() > 0
+    net = Block(fa.STORAGE_F16, 16, 96, 24, 28, 28, 1, False)
+    _, fused, infos = run(net)
+    assert "computed inside" in infos["dw"]
+    net.enableTimings(True)
+    net.forward()
+    net.finish()
+    apart = net.getOutput(net.output_layer)
+    net.enableTimings(False)
+    net.forward()
+    net.finish()
+    again = net.getOutput(net.output_layer)
+    net.cleanup()
+    assert np.array_equal(fused, apart) and np.array_equal(fused, again)
+
+
+@pytest.mark.parametrize("storage", [fa.STORAGE_F32, fa.STORAGE_F16], ids=["f32", "f16"])
+def test_config4_mobilenetv2_with_fused_blocks(storage, monkeypatch):
+    """The whole MobileNetV2-style graph with every eligible depthwise layer fused, eager and as a replayed graph,
+    against the same graph with the layers apart (bit-identical in fp32 storage) and against the oracle's free-running chain."""
+    monkeypatch.setenv("FYNHIP_FORCE_DW_FUSION", "1")
+    net = networks.MobileNetV2(storage)
+    x, got, infos = run(net)
+    net.useGraph(True)
+    net.forward()
+    net.finish()
+    net.forward()
+    net.finish()
+    replay = net.getOutput(net.output_layer)
+    desc = net.describe()
+    net.cleanup()
+    fused = [n for n, i in infos.items() if "computed inside" in i]
+    print("   fused:", len(fused), fused, flush=True)
+    assert len(fused) >= 8
+    assert np.array_equal(got, replay)
+    monkeypatch.setenv("FYNHIP_NO_DW_FUSION", "1")
+    twin = networks.MobileNetV2(storage)
+    _, two, _ = run(twin)
+    twin.cleanup()
+    if storage == fa.STORAGE_F32:
+        assert np.array_equal(got, two)
+    else:   # (last-bit differences of single values grow along the 52 layers of an untrained fp16 chain)
+        assert rel_l2(got, two) <= 5e-2
+    ref = O.run_network(desc, {net.input_key: x})[net.output_layer]
+    assert rel_l2(got, ref) <= (1e-4 if storage == fa.STORAGE_F32 else 5e-2)
