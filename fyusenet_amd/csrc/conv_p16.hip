@@ -1188,6 +1188,26 @@ __global__ __launch_bounds__(512) void conv_kr16_kernel(const ConvP16Params p) {
     float inv_in_scale = 1.f;
     if (p.in_amax) (void)range_scale(range_after_act(range_reduce(range_bits), p.act), &inv_in_scale);
     const float acc_mul = p.acc_mul * inv_in_scale;
+    // The residual values of the epilogue (wave 0) are requested here, so that their memory round trip passes under the
+    // staging and the step stream instead of behind them (small tiles: the registers are there).
+    constexpr bool RES_EARLY = FM * FN <= 4;
+    typedef typename std::conditional<HSTORE, half4_t, f32x4_t>::type res_t;
+    res_t res_early[RES_EARLY ? FM : 1][RES_EARLY ? FN : 1];
+    if constexpr (RES_EARLY) {
+        if (w == 0 && p.res) {
+            const store_t* res = reinterpret_cast<const store_t*>(p.res);
+#pragma unroll
+            for (int fn = 0; fn < FN; fn++)
+#pragma unroll
+                for (int fm = 0; fm < FM; fm++) {
+                    const int m = fn * 16 + mq;
+                    const int py = tyi * G::TH + m / G::TW, px = txi * G::TW + m % G::TW;
+                    const int ch = cb * 16 * FM + fm * 16 + kq * 4;
+                    const bool okc = py < p.npos_y && px < p.npos_x && ch + 4 <= p.out_cp;
+                    res_early[fm][fn] = *reinterpret_cast<const res_t*>(res + (okc ? ((size_t)(p.res_off_y + py) * p.res_wp + p.res_off_x + px) * p.res_cp + ch : 0));
+                }
+        }
+    }
 
     lds_barrier();   // the tile is staged
     // B fragment of step s: chunk w + 4*(s / NTAPS), tap s % NTAPS
@@ -1260,9 +1280,12 @@ __global__ __launch_bounds__(512) void conv_kr16_kernel(const ConvP16Params p) {
 #pragma unroll
             for (int e = 0; e < 4; e++) v[e] = v[e] * (sc[e] * acc_mul) + bi[e];
             if (res && okc) {
-                const store_t* rp = res + ((size_t)(p.res_off_y + py) * p.res_wp + p.res_off_x + px) * p.res_cp + ch;
+                [[maybe_unused]] const store_t* rp = res + ((size_t)(p.res_off_y + py) * p.res_wp + p.res_off_x + px) * p.res_cp + ch;
                 f32x4_t rv;
-                if constexpr (HSTORE) {
+                if constexpr (RES_EARLY) {
+#pragma unroll
+                    for (int e = 0; e < 4; e++) rv[e] = (float)res_early[fm][fn][e];
+                } else if constexpr (HSTORE) {
                     const half4_t rh = *reinterpret_cast<const half4_t*>(rp);
 #pragma unroll
                     for (int e = 0; e < 4; e++) rv[e] = (float)rh[e];
