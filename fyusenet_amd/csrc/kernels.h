@@ -235,6 +235,9 @@ int launch_conv_p16c4(const ConvP16Params& p, int k, hipStream_t s);
 // the K-resident form for layers with few positions (k = 1 or 3, stride 1) on the same parameters: tiles of 4x4
 // positions, blocks of 16*wm output channels, the whole reduction of a tile in LDS; wpack: [cout block][wave 0..3][step]
 // [fragment][plane][lane][8 halves], a wave's steps being (chunk wave + 4*i, tap)
+// 1x1 convolution without LDS for many positions and at most 256 input channels (conv_d16.hip), on the same parameters
+bool conv_d16_supported(int k, int dil, int in_cp, int chunks, int cout, int out_cp);
+int launch_conv_d16(const ConvP16Params& p, hipStream_t s);
 int conv_kr16_variant_count();
 void conv_kr16_variant(int index, int* taps, int* chunks, int* fm, int* th, int* tw, int* stride);   // compiled combinations: kernel taps, 32-channel chunks, fragments per block, tile
 size_t conv_kr16_lds_bytes(const ConvP16Params& p, int k);

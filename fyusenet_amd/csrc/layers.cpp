@@ -1284,6 +1284,98 @@ class ConvLayer : public Layer {
             net->dev_free(kr_wpack);
         }
     }
+    // The LDS-free 1x1 form (conv_d16.hip) against what has been chosen so far (the general kernel or the K-resident form).
+    void setup_d16(const TView& in_v, const TView& out_v, const TView* res_v, int res_relu, int res_scale) {
+        ConvP16Params q{};
+        q.in = in_v.ptr; q.out = out_v.ptr; q.res = res_v ? res_v->ptr : nullptr;
+        q.in_hp = in_v.hp(); q.in_wp = in_v.wp(); q.in_cp = in_v.cp;
+        q.stride = stride;
+        q.in_y0 = q.in_x0 = in_v.pad;
+        q.npos_y = oh; q.npos_x = ow;
+        q.out_wp = out_v.wp(); q.out_cp = out_v.cp; q.out_off_y = q.out_off_x = out_v.pad;
+        if (res_v) { q.res_wp = res_v->wp(); q.res_cp = res_v->cp; q.res_off_y = q.res_off_x = res_v->pad; }
+        q.res_relu = res_relu; q.res_scale = res_scale;
+        q.cin_chunks = (in_v.cp + 31) / 32;
+        q.mfrags = (oc + 15) / 16;
+        q.f16 = out_v.f16 ? 1 : 0;
+        q.scale = scale_dev; q.bias = bias_dev;
+        q.acc_mul = 1.f;
+        q.act = act();
+        const size_t halves = (size_t)q.mfrags * q.cin_chunks * (q.f16 ? 1 : 2) * 64 * 8;
+        void* const wp = net->dev_alloc(halves * 2, true);
+        q.wpack = wp;
+        q.cout_blocks = 1;   // workgroups per 16 positions (they share the fragments of output channels): 1, 2 or 4, timed
+        if (const char* e = getenv("FYNHIP_D16_BLOCKS")) q.cout_blocks = std::max(1, std::min(4, atoi(e)));
+        const bool always = getenv("FYNHIP_FORCE_D16_CONV") != nullptr;
+        const char* at = getenv("FYNHIP_AUTOTUNE");
+        bool pick = true;
+        char key[160];
+        snprintf(key, sizeof(key), "d16:%dx%d:%dx%d:s%d:r%d:h%d:kr%d", d.in_channels, oc, oh, ow, stride, res_v ? 1 : 0, q.f16, kr16 ? 1 : 0);
+        int cached[3] = {0, 0, 0};
+        if (getenv("FYNHIP_D16_BLOCKS")) {
+            pick = always;
+        } else if (tune_cache_triple(key, cached)) {
+            pick = cached[0] != 0 || always;
+            q.cout_blocks = std::max(1, cached[1]);
+        } else if (!(at && at[0] == '0')) {
+            float t_new = 1e30f, t_other = 1e30f;
+            int best_blocks = 1;
+            for (int rep = 0; rep < 3; rep++) {
+                for (int blocks = 1; blocks <= 4 && 4 * blocks <= std::max(4, q.mfrags); blocks *= 2) {
+                    ConvP16Params c = q;
+                    c.cout_blocks = blocks;
+                    const float t = time_calls(net, [&]() {
+                        if (launch_conv_d16(c, net->stream) != 0) fail(FYN_ERR_DEVICE, "LDS-free 1x1 convolution launch failed while tuning");
+                    }, 10);
+                    if (t < t_new) { t_new = t; best_blocks = blocks; }
+                }
+                if (kr16)
+                    t_other = std::min(t_other, time_calls(net, [&]() {
+                        if (launch_conv_kr16(pp, k, net->stream) != 0) fail(FYN_ERR_DEVICE, "K-resident convolution launch failed while tuning");
+                    }, 10));
+                else
+                    t_other = std::min(t_other, time_launch(net, launch, 10));
+            }
+            if (getenv("FYNHIP_TUNE_VERBOSE"))
+                fprintf(stderr, "[tune] 1x1 on %d channels, %dx%d positions, to %d: LDS-free form (%d workgroups per 16 positions) %.1f us, %s %.1f us\n", d.in_channels, oh, ow,
+                        oc, best_blocks, t_new * 1e3f, kr16 ? "K-resident form" : "general kernel", t_other * 1e3f);
+            pick = t_new < t_other || always;
+            q.cout_blocks = best_blocks;
+            tune_cache_store_triple(key, t_new < t_other ? 1 : 0, best_blocks, 0);
+        }
+        if (pick) {
+            if (p16) net->dev_free(p16_wpack_dev);
+            p16_wpack_dev = wp;
+            p16 = true; kr16 = false; d16 = true;
+            pp = q;
+        } else {
+            net->dev_free(wp);
+        }
+    }
+    // weights of that form: [cout fragment][chunk][plane][lane][8 halves]
+    void pack_d16(const float* w, float wmul) {
+        const int cin = d.in_channels, npl = pp.f16 ? 1 : 2;
+        std::vector<uint16_t> pack((size_t)pp.mfrags * pp.cin_chunks * npl * 64 * 8, 0);
+        for (int mf = 0; mf < pp.mfrags; mf++)
+            for (int c = 0; c < pp.cin_chunks; c++) {
+                uint16_t* base = pack.data() + ((size_t)(mf * pp.cin_chunks + c) * npl) * 64 * 8;
+                for (int lane = 0; lane < 64; lane++) {
+                    const int o = mf * 16 + (lane & 15);
+                    if (o >= oc) continue;
+                    for (int j = 0; j < 8; j++) {
+                        const int ci = c * 32 + 8 * (lane >> 4) + j;
+                        if (ci >= cin) continue;
+                        const float v = w[(size_t)o * cin + ci] * wmul;
+                        const uint16_t hi = f2h_bits(v);
+                        base[(size_t)lane * 8 + j] = hi;
+                        if (npl == 2) base[(size_t)(64 + lane) * 8 + j] = f2h_bits(v - h2f(hi));
+                    }
+                }
+            }
+        FYN_HIP(hipStreamSynchronize(net->stream));
+        FYN_HIP(hipMemcpyAsync(p16_wpack_dev, pack.data(), pack.size() * 2, hipMemcpyHostToDevice, net->stream));
+        FYN_HIP(hipStreamSynchronize(net->stream));
+    }
     // weights of that form: [cout block][wave][step][fragment][plane][lane][8 halves]; step s of wave w = (chunk w + 4*(s / taps), tap s % taps)
     void pack_kr16(const float* w, float wmul) {
         const int cin = d.in_channels, taps = k * k, fm_n = pp.wm, npl = pp.f16 ? 1 : 2;
@@ -1586,6 +1678,12 @@ class ConvLayer : public Layer {
                 // (a test that forces a variant of the general kernel wants the general kernel)
                 !getenv("FYNHIP_FORCE_KSPLIT") && !getenv("FYNHIP_CONV_TILE") && !getenv("FYNHIP_CONV_KC") && !getenv("FYNHIP_CONV_KC_MAX") && !getenv("FYNHIP_CONV_PD"))
                 setup_kr16(in_v, out_v, res_v, res_relu, res_scale);
+            // many positions, few input channels, 1x1: fragments straight from the tensor, no LDS
+            if ((!p16 || kr16) && !frac_shift && same_storage && d.in_channels == in_v.cp && oc % 4 == 0 && oc >= 8 && oh * ow >= 256 &&
+                conv_d16_supported(k, dil, in_v.cp, (in_v.cp + 31) / 32, oc, out_v.cp) && (!res_v || (res_v->cp >= out_v.cp && res_v->cp % 8 == 0)) &&
+                !getenv("FYNHIP_NO_P16_CONV") && !getenv("FYNHIP_NO_D16_CONV") && !getenv("FYNHIP_FORCE_P16_CONV") && !getenv("FYNHIP_FORCE_KR16_CONV") &&
+                !getenv("FYNHIP_FORCE_KSPLIT") && !getenv("FYNHIP_CONV_TILE") && !getenv("FYNHIP_CONV_KC") && !getenv("FYNHIP_CONV_KC_MAX") && !getenv("FYNHIP_CONV_PD"))
+                setup_d16(in_v, out_v, res_v, res_relu, res_scale);
         }
         if (direct) {
             scale_dev = static_cast<float*>(net->dev_alloc(padded * sizeof(float)));
@@ -1617,6 +1715,7 @@ class ConvLayer : public Layer {
             const float wmul = weight_prescale(w, (size_t)oc * k * k * d.in_channels);
             pp.acc_mul = pp2.acc_mul = 1.0f / wmul;
             if (c4) pack_c4(w, wmul);
+            else if (d16) pack_d16(w, wmul);
             else if (kr16) pack_kr16(w, wmul);
             else if (h16) pack_h16(w, wmul);
             else pack_p16(w, wmul);
@@ -1664,7 +1763,7 @@ class ConvLayer : public Layer {
             return;
         }
         if (p16) {
-            if ((c4 ? launch_conv_p16c4(pp, k, s) : (kr16 ? launch_conv_kr16(pp, k, s) : (h16 ? launch_conv_h16(pp, k, s) : launch_conv_p16(pp, s)))) != 0 ||
+            if ((c4 ? launch_conv_p16c4(pp, k, s) : (d16 ? launch_conv_d16(pp, s) : (kr16 ? launch_conv_kr16(pp, k, s) : (h16 ? launch_conv_h16(pp, k, s) : launch_conv_p16(pp, s))))) != 0 ||
                 (h16 && h16_two && launch_conv_h16(pp2, k, s) != 0))
                 fail(FYN_ERR_DEVICE, "layer %s: convolution launch failed", d.name);
             return;
@@ -1688,6 +1787,12 @@ class ConvLayer : public Layer {
             snprintf(buf, sizeof(buf), "conv_p16c4 %s (tap pairs of a 4-channel pixel) tile=32x%d(cout x pos) th=%d tw=%d blocks=%d tiles=%d lds=%zu steps=%d",
                      pp.f16 ? "f16" : "f16x2-split", pp.tile_h * pp.tile_w * 4, pp.tile_h, pp.tile_w, pp.pos_groups * pp.cout_blocks, pp.tiles_x * pp.tiles_y * pp.cout_blocks,
                      conv_p16c4_lds_bytes(pp, k), c4_steps);
+            return mode + buf;
+        }
+        if (p16 && d16) {
+            char buf[220];
+            snprintf(buf, sizeof(buf), "conv_d16 %s 1x1 without LDS: %d workgroup(s) of 4 waves per 16 positions, %d chunks in registers, %d fragments of 16 output channels, blocks=%d",
+                     pp.f16 ? "f16" : "f16x2-split", pp.cout_blocks, pp.cin_chunks, pp.mfrags, (pp.npos_y * pp.npos_x + 15) / 16 * pp.cout_blocks);
             return mode + buf;
         }
         if (p16 && kr16) {
@@ -1734,6 +1839,7 @@ class ConvLayer : public Layer {
     int c4_steps = 0;
     bool h16 = false;             // ... its fp16-storage form for wide layers (conv_h16.hip)
     bool kr16 = false;            // ... the K-resident form for layers with few positions (conv_p16.hip, conv_kr16_kernel)
+    bool d16 = false;             // ... the LDS-free 1x1 form for many positions and few input channels (conv_d16.hip)
     // A depthwise 3x3 layer whose only reader is this 1x1 layer in the K-resident form can be computed inside this
     // layer's staging (fuse_depthwise_layers below): the fields of ConvP16Params that describe it
     bool dw_fused = false;

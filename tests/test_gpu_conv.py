@@ -460,6 +460,58 @@ def test_reduction_resident_form(case, act, shallow, storage, monkeypatch):
     assert err <= TOL[storage], info
 
 
+D16_CASES = [
+    # (cin, cout, h, w, kw)
+    (16, 96, 112, 112, {"bn": True}),                                            # an expand layer at the largest resolution
+    (32, 16, 56, 60, {"residual": (A.NONE, False)}),
+    (24, 144, 28, 31, {"bn": True, "pad_out": 1}),                               # 24 channels in a chunk of 32; positions no multiple of 16
+    (96, 24, 37, 29, {"bn": True, "residual": (A.RELU, True)}),                  # three chunks, 24 output channels (second fragment half empty)
+    (144, 40, 20, 20, {}),                                                       # five chunks
+    (192, 64, 37, 45, {"stride": 2, "bn": True}),                                # six chunks, step 2 on an odd-sized input
+    (64, 256, 56, 56, {"bn": True, "residual": (A.NONE, False)}),                # ResNet stage 1: 16 fragments, four per wave
+    (256, 64, 40, 40, {"stride": 2}),                                            # eight chunks
+    (8, 12, 40, 40, {}),                                                         # a quarter of a chunk, 12 output channels
+    (32, 320, 24, 24, {"bn": True}),                                             # 20 fragments: five per wave, one ahead of their use
+    # the fragments of output channels dealt to two or four workgroups per 16 positions
+    (64, 256, 28, 28, {"bn": True, "residual": (A.RELU, True), "blocks": 2}),
+    (32, 320, 24, 24, {"blocks": 4}),
+    (96, 24, 30, 30, {"blocks": 2}),                                             # more waves than fragments
+]
+
+
+@pytest.mark.parametrize("storage", [fa.STORAGE_F32, fa.STORAGE_F16], ids=["f32", "f16"])
+@pytest.mark.parametrize("variant", ["relu", "leaky", "shallow"])
+@pytest.mark.parametrize("case", D16_CASES, ids=lambda c: "%dx%dx%d_to%d%s%s" % (c[0], c[2], c[3], c[1], "_s2" if c[4].get("stride") == 2 else "", "_b%d" % c[4]["blocks"] if "blocks" in c[4] else ""))
+def test_pointwise_without_lds(case, variant, storage, monkeypatch):
+    """1x1 convolutions on many positions whose B fragments come straight from the tensor: a workgroup of four waves per
+    16 positions, the waves sharing the fragments of output channels."""
+    cin, cout, h, w, kw = case
+    if variant != "relu" and ("residual" in kw or "pad_out" in kw or "blocks" in kw or cin > 100):
+        pytest.skip("activation and the shallow variant are varied on the plain cases")
+    monkeypatch.setenv("FYNHIP_FORCE_D16_CONV", "1")
+    kw = dict(kw)
+    stride = kw.pop("stride", 1)
+    blocks = kw.pop("blocks", None)
+    if blocks:
+        monkeypatch.setenv("FYNHIP_D16_BLOCKS", str(blocks))
+    if variant == "shallow":
+        kw.update(deep=False, pad_in=0)
+    act = A.LEAKY_RELU if variant == "leaky" else A.RELU
+    if variant == "leaky":
+        kw["leak"] = 0.1
+    b = conv_builder(1, cout, h, w, cin, stride, 1, act, **kw)
+    wts = conv_block(5000 + cin + cout, cout, 1, cin, bn=kw.get("bn", False))
+    inputs = [prng.uniform(43 * cin + h, (cin, h, w), -1, 1)]
+    if "residual" in kw:
+        inputs.append(prng.uniform(71, (cout, h // stride, w // stride), -1, 1))
+    got, info = run_single(b, storage, inputs, wts)
+    ref = oracle_single(b, storage, inputs, wts)
+    err = rel_l2(got, ref)
+    print("  ", info, "rel_l2=%.3e" % err, flush=True)
+    assert "conv_d16" in info and (not blocks or "%d workgroup(s)" % blocks in info)
+    assert err <= TOL[storage], info
+
+
 ALL_TILES = ["2,2,2,2", "2,2,1,4", "2,1,2,2", "2,1,1,4", "1,2,1,4", "1,1,1,4", "1,1,4,1", "1,1,2,2", "1,2,4,1", "1,3,4,1", "1,4,4,1",
              "1,2,2,2", "1,4,2,2", "1,3,2,2", "1,4,1,4", "1,3,1,4", "1,1,1,1", "1,1,2,1", "1,1,1,2"]
 
