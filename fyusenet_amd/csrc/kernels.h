@@ -202,6 +202,7 @@ struct ConvP16Params {
     // A depthwise 3x3 layer computed inside the staging of a 1x1 launch of the K-resident form (dw_in null: none): the
     // layer's input tensor, its weights [9][dw_cp] and folded scale / bias [dw_cp], the stored coordinate of tap (0,0)
     // of output position (0,0), its step and the activation applied to its input.  `in` is not read then.
+    // (launch_conv_e16dw uses the same fields for a depthwise layer BEHIND a 1x1 layer, with its own meaning of dw_hp / dw_wp.)
     const void* dw_in;
     const float* dw_w;
     const float* dw_scale;
@@ -238,6 +239,9 @@ int launch_conv_p16c4(const ConvP16Params& p, int k, hipStream_t s);
 // 1x1 convolution without LDS for many positions and at most 256 input channels (conv_d16.hip), on the same parameters
 bool conv_d16_supported(int k, int dil, int in_cp, int chunks, int cout, int out_cp);
 int launch_conv_d16(const ConvP16Params& p, hipStream_t s);
+// a 1x1 layer and the depthwise 3x3 layer behind it as one launch (conv_d16.hip: conv_e16dw_kernel)
+bool conv_e16dw_supported(int in_cp, int chunks, int dw_stride);
+int launch_conv_e16dw(const ConvP16Params& p, hipStream_t s);
 int conv_kr16_variant_count();
 void conv_kr16_variant(int index, int* taps, int* chunks, int* fm, int* th, int* tw, int* stride);   // compiled combinations: kernel taps, 32-channel chunks, fragments per block, tile
 size_t conv_kr16_lds_bytes(const ConvP16Params& p, int k);

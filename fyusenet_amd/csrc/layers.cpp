@@ -1353,12 +1353,13 @@ class ConvLayer : public Layer {
         }
     }
     // weights of that form: [cout fragment][chunk][plane][lane][8 halves]
-    void pack_d16(const float* w, float wmul) {
-        const int cin = d.in_channels, npl = pp.f16 ? 1 : 2;
-        std::vector<uint16_t> pack((size_t)pp.mfrags * pp.cin_chunks * npl * 64 * 8, 0);
-        for (int mf = 0; mf < pp.mfrags; mf++)
-            for (int c = 0; c < pp.cin_chunks; c++) {
-                uint16_t* base = pack.data() + ((size_t)(mf * pp.cin_chunks + c) * npl) * 64 * 8;
+    void pack_d16(const float* w, float wmul) { pack_frag16(pp, p16_wpack_dev, w, wmul); }
+    void pack_frag16(const ConvP16Params& q, void* dev, const float* w, float wmul) {
+        const int cin = d.in_channels, npl = q.f16 ? 1 : 2;
+        std::vector<uint16_t> pack((size_t)q.mfrags * q.cin_chunks * npl * 64 * 8, 0);
+        for (int mf = 0; mf < q.mfrags; mf++)
+            for (int c = 0; c < q.cin_chunks; c++) {
+                uint16_t* base = pack.data() + ((size_t)(mf * q.cin_chunks + c) * npl) * 64 * 8;
                 for (int lane = 0; lane < 64; lane++) {
                     const int o = mf * 16 + (lane & 15);
                     if (o >= oc) continue;
@@ -1373,7 +1374,7 @@ class ConvLayer : public Layer {
                 }
             }
         FYN_HIP(hipStreamSynchronize(net->stream));
-        FYN_HIP(hipMemcpyAsync(p16_wpack_dev, pack.data(), pack.size() * 2, hipMemcpyHostToDevice, net->stream));
+        FYN_HIP(hipMemcpyAsync(dev, pack.data(), pack.size() * 2, hipMemcpyHostToDevice, net->stream));
         FYN_HIP(hipStreamSynchronize(net->stream));
     }
     // weights of that form: [cout block][wave][step][fragment][plane][lane][8 halves]; step s of wave w = (chunk w + 4*(s / taps), tap s % taps)
@@ -1750,10 +1751,32 @@ class ConvLayer : public Layer {
             launch.red.acc_mul = 1.0f / wmul;
             pack_mfma_weights(net, launch, w, k, wmul);
         }
+        if (edw_fused) pack_edw();
         have_weights = true;
+    }
+    // the weights once more, in the layout of the launch that also runs the depthwise layer behind this one
+    void pack_edw() {
+        if (block.empty()) return;
+        const float* w = block.data() + oc;
+        const float wmul = weight_prescale(w, (size_t)oc * k * k * d.in_channels);
+        edw.acc_mul = 1.0f / wmul;
+        pack_frag16(edw, edw_wpack_dev, w, wmul);
     }
     void forward(hipStream_t s) override {
         if (!have_weights) fail(FYN_ERR_STATE, "layer %s (%d): forward() without weights", d.name, d.number);
+        if (edw_fused && net->fusion_on()) {
+            ConvP16Params q = edw;   // (value-range words as the layer's own launch carries them)
+            q.in_amax = tin(0).amax;
+            const int n = rows ? rp.nreset : (p16 ? pp.nreset : launch.p.nreset);
+            unsigned* const* r = rows ? rp.reset : (p16 ? pp.reset : launch.p.reset);
+            q.nreset = n;
+            for (int i = 0; i < n; i++) q.reset[i] = r[i];
+            if (launch_conv_e16dw(q, s) != 0) fail(FYN_ERR_DEVICE, "layer %s: convolution launch failed", d.name);
+            return;
+        }
+        run(s);
+    }
+    void run(hipStream_t s) {
         if (rows) {
             if (launch_conv_rows(rp, tout().v.f16 != 0, s) != 0) fail(FYN_ERR_DEVICE, "layer %s: convolution launch failed", d.name);
             return;
@@ -1774,6 +1797,13 @@ class ConvLayer : public Layer {
         if (wide && !fused) launch_shift_reduce(sr, s);
     }
     std::string info() const override {
+        if (edw_fused)
+            return "conv_e16dw " + std::string(edw.f16 ? "f16" : "f16x2-split") + " 1x1 and the depthwise 3x3 layer " + std::to_string(edw_dw_no) +
+                   " behind it in one launch: a workgroup per 4x4 output positions and 64 expanded channels, blocks=" +
+                   std::to_string(edw.tiles_x * edw.tiles_y * ((edw.dw_cp + 63) / 64)) + "; apart: " + own_info();
+        return own_info();
+    }
+    std::string own_info() const {
         const std::string mode = frac_shift ? "(fractional step 1/" + std::to_string(1 << (frac_shift - 1)) + ") " : (clamp ? "(edge-clamp) " : "");
         if (direct) return "conv_direct" + mode;
         if (rows) {
@@ -1842,6 +1872,12 @@ class ConvLayer : public Layer {
     bool d16 = false;             // ... the LDS-free 1x1 form for many positions and few input channels (conv_d16.hip)
     // A depthwise 3x3 layer whose only reader is this 1x1 layer in the K-resident form can be computed inside this
     // layer's staging (fuse_depthwise_layers below): the fields of ConvP16Params that describe it
+    // ... or, where this is a 1x1 layer and the depthwise layer its only reader, both run as one launch of
+    // conv_e16dw_kernel (conv_d16.hip), with the weights packed once more in that kernel's layout
+    bool edw_fused = false;
+    int edw_dw_no = -1;
+    ConvP16Params edw{};
+    void* edw_wpack_dev = nullptr;
     bool dw_fused = false;
     int dw_layer_no = -1;
     ConvP16Params dw_fields{};
@@ -1921,7 +1957,7 @@ class DwConvLayer : public Layer {
         launch_dwconv3x3(p, s);
     }
     std::string info() const override {
-        return fused_into >= 0 ? "dwconv3x3 (computed inside layer " + std::to_string(fused_into) + ", whose staging waves run it; no launch, no tensor)" : "dwconv3x3";
+        return fused_into >= 0 ? "dwconv3x3 (runs inside the launch of layer " + std::to_string(fused_into) + "; no launch of its own)" : "dwconv3x3";
     }
     int fused_into = -1;
     int dil, stride;
@@ -1944,12 +1980,81 @@ void fuse_depthwise_layers(Net* net) {
     for (auto& kv : net->layers)
         for (int t : kv.second->in)
             if (t >= 0) readers[t]++;
+    const char* at = getenv("FYNHIP_AUTOTUNE");
+    // First the other half of the block: a 1x1 layer (expand) whose only reader is the depthwise layer.  Every expanded
+    // channel depends on the 1x1 layer's input only, so a workgroup can compute the window of the expanded tensor that
+    // its tile of the depthwise layer needs (conv_e16dw_kernel); the expanded tensor is then never written.
+    for (auto& kv : net->layers) {
+        if (getenv("FYNHIP_NO_EDW_FUSION")) break;
+        DwConvLayer* dw = dynamic_cast<DwConvLayer*>(kv.second.get());
+        if (!dw || dw->dil != 1 || (dw->stride != 1 && dw->stride != 2) || dw->p.res.ptr || dw->p.in.cp % 8 != 0 || dw->p.in.cp != dw->p.out.cp || dw->p.in.f16 != dw->p.out.f16)
+            continue;
+        const Tensor& t = net->tensors[dw->in[0]];
+        if (t.producer < 0 || t.locked || readers[dw->in[0]] != 1) continue;
+        ConvLayer* ex = dynamic_cast<ConvLayer*>(net->layer(t.producer));
+        if (!ex || ex->k != 1 || ex->stride != 1 || ex->dil != 1 || ex->clamp || ex->frac_shift || ex->direct || (ex->d.flags & FYN_FLAG_RESIDUAL_INPUT)) continue;
+        const TView& in_v = ex->tin(0).v;
+        if (in_v.f16 != dw->p.out.f16 || ex->d.in_channels != in_v.cp || ex->tout().v.cp != dw->p.in.cp || ex->oc % 4 != 0 ||
+            !conv_e16dw_supported(in_v.cp, (in_v.cp + 31) / 32, dw->stride))
+            continue;
+        ConvP16Params q{};
+        q.in = in_v.ptr; q.in_hp = in_v.hp(); q.in_wp = in_v.wp(); q.in_cp = in_v.cp;
+        q.stride = 1; q.in_y0 = q.in_x0 = in_v.pad;
+        q.cin_chunks = (in_v.cp + 31) / 32;
+        q.mfrags = (ex->oc + 15) / 16;
+        q.f16 = in_v.f16 ? 1 : 0;
+        q.scale = ex->scale_dev; q.bias = ex->bias_dev;
+        q.acc_mul = 1.f;
+        q.act = ex->act();
+        q.dw_hp = ex->oh; q.dw_wp = ex->ow;
+        q.out = dw->p.out.ptr; q.out_wp = dw->p.out.wp(); q.out_cp = dw->p.out.cp; q.out_off_y = q.out_off_x = dw->p.out.pad;
+        q.npos_y = dw->p.out.h; q.npos_x = dw->p.out.w;
+        q.tiles_x = (q.npos_x + 3) / 4; q.tiles_y = (q.npos_y + 3) / 4;
+        q.dw_w = dw->w_dev; q.dw_scale = dw->scale_dev; q.dw_bias = dw->bias_dev;
+        q.dw_cp = dw->p.in.cp; q.dw_stride = dw->stride; q.dw_act = dw->p.act;
+        const size_t halves = (size_t)q.mfrags * q.cin_chunks * (q.f16 ? 1 : 2) * 64 * 8;
+        void* const wp = net->dev_alloc(halves * 2, true);
+        q.wpack = wp;
+        bool pick = true;
+        char key[200];
+        snprintf(key, sizeof(key), "edw:%d:%dto%d:%dx%d:s%d", q.f16, in_v.cp, ex->oc, ex->oh, ex->ow, dw->stride);
+        if (getenv("FYNHIP_FORCE_DW_FUSION")) {
+        } else if (tune_cache_flag(key, &pick)) {
+        } else if (!(at && at[0] == '0')) {
+            float t_fused = 1e30f, t_two = 1e30f;
+            for (int rep = 0; rep < 3; rep++) {
+                t_fused = std::min(t_fused, time_calls(net, [&]() {
+                    if (launch_conv_e16dw(q, net->stream) != 0) fail(FYN_ERR_DEVICE, "1x1 + depthwise convolution launch failed while tuning");
+                }, 10));
+                t_two = std::min(t_two, time_calls(net, [&]() {
+                    ex->run(net->stream);
+                    launch_dwconv3x3(dw->p, net->stream);
+                }, 10));
+            }
+            if (getenv("FYNHIP_TUNE_VERBOSE"))
+                fprintf(stderr, "[tune] 1x1 %d to %d at %dx%d + depthwise 3x3 (step %d): one launch %.1f us, two %.1f us\n", in_v.cp, ex->oc, ex->oh, ex->ow, dw->stride,
+                        t_fused * 1e3f, t_two * 1e3f);
+            pick = t_fused < t_two;
+            tune_cache_store_flag(key, pick);
+        }
+        if (!pick) {
+            net->dev_free(wp);
+            continue;
+        }
+        ex->edw = q;
+        ex->edw_wpack_dev = wp;
+        ex->edw_fused = true;
+        ex->edw_dw_no = dw->d.number;
+        dw->fused_into = ex->d.number;
+        ex->pack_edw();
+    }
     for (auto& kv : net->layers) {
         ConvLayer* pw = dynamic_cast<ConvLayer*>(kv.second.get());
         if (!pw || !pw->takes_depthwise()) continue;
         const Tensor& t = net->tensors[pw->in[0]];
         if (t.producer < 0 || t.locked || readers[pw->in[0]] != 1) continue;
         DwConvLayer* dw = dynamic_cast<DwConvLayer*>(net->layer(t.producer));
+        if (dw && dw->fused_into >= 0) continue;   // (already part of the 1x1 layer in front of it)
         if (!dw || dw->dil != 1 || (dw->stride != 1 && dw->stride != 2) || dw->p.res.ptr || dw->p.in.cp % 8 != 0 || dw->p.in.cp != dw->p.out.cp ||
             dw->p.in.f16 != dw->p.out.f16 || dw->p.out.f16 != pw->pp.f16 || dw->p.out.cp != pw->pp.in_cp)
             continue;
@@ -1963,7 +2068,6 @@ void fuse_depthwise_layers(Net* net) {
         bool pick = true;
         char key[200];
         snprintf(key, sizeof(key), "dwpw:%d:%dx%dx%d:s%d:to%d:fm%d", q.f16, dw->p.in.cp, dw->p.in.h, dw->p.in.w, dw->stride, pw->oc, q.wm);
-        const char* at = getenv("FYNHIP_AUTOTUNE");
         if (getenv("FYNHIP_FORCE_DW_FUSION")) {
         } else if (tune_cache_flag(key, &pick)) {
         } else if (!(at && at[0] == '0')) {

@@ -1,6 +1,8 @@
-"""A depthwise 3x3 layer computed inside the staging of the 1x1 layer behind it (the second half of an inverted-residual
-block as one launch): parity against the oracle, equality with the two-launch form, and the conditions under which the
-engine leaves the two layers apart.  Tolerances: rel-L2 <= 1e-4 (fp32 storage), <= 2e-3 (fp16 storage)."""
+"""A depthwise 3x3 layer that runs inside the launch of a neighbour: of the 1x1 layer in front of it (the first half of
+an inverted-residual block as one launch; the expanded tensor is never written) or, in the staging, of the 1x1 layer
+behind it (the second half; the depthwise layer's tensor is never written).  Parity against the oracle, equality with
+the two-launch form, and the conditions under which the engine leaves the layers apart.  Tolerances: rel-L2 <= 1e-4
+(fp32 storage), <= 2e-3 (fp16 storage)."""
 import numpy as np
 import pytest
 
@@ -19,9 +21,10 @@ class Block(networks._StreamNet):
     from the block's input) -> download."""
     config_id = 4
 
-    def __init__(self, storage, cin, exp, cout, h, w, stride, residual, side_reader=False):
+    def __init__(self, storage, cin, exp, cout, h, w, stride, residual, side_reader=False, expand_side_reader=False):
         super().__init__(storage)
         self.cin, self.exp, self.cout, self.h, self.w, self.stride, self.residual, self.side_reader = cin, exp, cout, h, w, stride, residual, side_reader
+        self.expand_side_reader = expand_side_reader
 
     def define(self):
         C, c6 = ActType.CLIP, (0.0, 6.0)
@@ -33,6 +36,9 @@ class Block(networks._StreamNet):
         last = 3
         if self.side_reader:   # a second reader of the depthwise layer's tensor
             self.conv(4, "side", 1, self.exp, 16, ho, wo, 2, act=C, clip=c6)
+            last = 4
+        if self.expand_side_reader:   # a second reader of the expanded tensor (which has a halo of 1)
+            self.conv(4, "side", 3, self.exp, 16, self.h, self.w, 1, act=C, clip=c6)
             last = 4
         self._add(UpDownLayerBuilder(UpDownLayerBuilder.DOWNLOAD, "download").number(last + 1).shape(self.cout, ho, wo, self.cout).deep())
         self._edges.append((3, last + 1, 0))
@@ -84,18 +90,50 @@ CASES = [
 ]
 
 
+FRONT_CASES = CASES + [
+    (160, 960, 320, 7, 7, 1, False),     # five chunks of input channels, 15 blocks of expanded channels
+    (96, 576, 160, 14, 14, 2, False),
+    (16, 96, 24, 112, 112, 2, False),    # the largest resolution of the stack
+]
+
+
+@pytest.mark.parametrize("storage", [fa.STORAGE_F32, fa.STORAGE_F16], ids=["f32", "f16"])
+@pytest.mark.parametrize("case", FRONT_CASES, ids=lambda c: "%dto%dto%d_%dx%d_s%d%s" % (c[0], c[1], c[2], c[3], c[4], c[5], "_res" if c[6] else ""))
+def test_depthwise_inside_the_launch_of_the_expand_layer(case, storage, monkeypatch):
+    cin, exp, cout, h, w, stride, residual = case
+    monkeypatch.setenv("FYNHIP_FORCE_DW_FUSION", "1")
+    net = Block(storage, cin, exp, cout, h, w, stride, residual)
+    x, got, infos = run(net)
+    desc = net.describe()
+    net.cleanup()
+    print("  ", infos["dw"], "|", infos["expand"][:120], flush=True)
+    assert "launch of layer 1" in infos["dw"] and "conv_e16dw" in infos["expand"] and "depthwise 3x3 layer 2" in infos["expand"]
+    ref = O.run_network(desc, {net.input_key: x})[net.output_layer]
+    err = rel_l2(got, ref)
+    print("   rel_l2=%.3e" % err, flush=True)
+    assert err <= TOL[storage]
+    monkeypatch.setenv("FYNHIP_NO_DW_FUSION", "1")
+    twin = Block(storage, cin, exp, cout, h, w, stride, residual)
+    _, two, infos2 = run(twin)
+    twin.cleanup()
+    assert infos2["dw"] == "dwconv3x3"
+    # (the 1x1 layer on its own may run a kernel that sums the reduction in another order: no bit-equality here)
+    assert rel_l2(got, two) <= (2e-6 if storage == fa.STORAGE_F32 else 1e-3)
+
+
 @pytest.mark.parametrize("storage", [fa.STORAGE_F32, fa.STORAGE_F16], ids=["f32", "f16"])
 @pytest.mark.parametrize("case", CASES, ids=lambda c: "%dto%dto%d_%dx%d_s%d%s" % (c[0], c[1], c[2], c[3], c[4], c[5], "_res" if c[6] else ""))
 def test_depthwise_inside_pointwise_staging(case, storage, monkeypatch):
     cin, exp, cout, h, w, stride, residual = case
     monkeypatch.setenv("FYNHIP_FORCE_KR16_CONV", "1")
     monkeypatch.setenv("FYNHIP_FORCE_DW_FUSION", "1")
+    monkeypatch.setenv("FYNHIP_NO_EDW_FUSION", "1")
     net = Block(storage, cin, exp, cout, h, w, stride, residual)
     x, got, infos = run(net)
     desc = net.describe()
     net.cleanup()
     print("  ", infos["dw"], "|", infos["project"], flush=True)
-    assert "computed inside layer 3" in infos["dw"] and "depthwise 3x3 layer 2" in infos["project"]
+    assert "launch of layer 3" in infos["dw"] and "depthwise 3x3 layer 2" in infos["project"]
     ref = O.run_network(desc, {net.input_key: x})[net.output_layer]
     err = rel_l2(got, ref)
     print("   rel_l2=%.3e" % err, flush=True)
@@ -109,42 +147,59 @@ def test_depthwise_inside_pointwise_staging(case, storage, monkeypatch):
 
 
 def test_layers_stay_apart_when_the_tensor_is_needed(monkeypatch):
-    """No fusion when the depthwise layer's tensor has a second reader, or when the caller keeps every layer's tensor
-    (buffer reuse off); per-layer timing runs the layers apart and leaves the results unchanged."""
+    """No fusion when the tensor between the two layers has a second reader, or when the caller keeps every layer's
+    tensor (buffer reuse off); per-layer timing runs the layers apart and leaves the results unchanged."""
     monkeypatch.setenv("FYNHIP_FORCE_KR16_CONV", "1")
     monkeypatch.setenv("FYNHIP_FORCE_DW_FUSION", "1")
+    # a second reader of the depthwise layer's tensor: the 1x1 layer behind it must fetch it; the layer in front may still run it
+    net = Block(fa.STORAGE_F16, 16, 96, 24, 28, 28, 1, False, side_reader=True)
+    _, _, infos = run(net)
+    net.cleanup()
+    assert "launch of layer 1" in infos["dw"]
+    monkeypatch.setenv("FYNHIP_NO_EDW_FUSION", "1")
     net = Block(fa.STORAGE_F16, 16, 96, 24, 28, 28, 1, False, side_reader=True)
     _, _, infos = run(net)
     net.cleanup()
     assert infos["dw"] == "dwconv3x3"
-    net = Block(fa.STORAGE_F16, 96, 576, 160, 14, 14, 1, False)   # (more than 512 channels: no fused variant)
+    net = Block(fa.STORAGE_F16, 96, 576, 160, 14, 14, 1, False)   # (more than 512 channels: no variant of the staging form)
     _, _, infos = run(net)
     net.cleanup()
     assert infos["dw"] == "dwconv3x3"
+    monkeypatch.delenv("FYNHIP_NO_EDW_FUSION")
+    # a second reader of the expanded tensor
+    net = Block(fa.STORAGE_F16, 16, 96, 24, 28, 28, 1, False, expand_side_reader=True)
+    _, _, infos = run(net)
+    net.cleanup()
+    assert "conv_e16dw" not in infos["expand"] and "launch of layer 3" in infos["dw"]
     net = Block(fa.STORAGE_F16, 16, 96, 24, 28, 28, 1, False)
     _, _, infos = run(net, reuse=False)
     dw_out = net.layers[2].copyResult()
+    ex_out = net.layers[1].copyResult()
     net.cleanup()
-    assert infos["dw"] == "dwconv3x3" and np.abs(dw_out).max() > 0
-    net = Block(fa.STORAGE_F16, 16, 96, 24, 28, 28, 1, False)
-    _, fused, infos = run(net)
-    assert "computed inside" in infos["dw"]
-    net.enableTimings(True)
-    net.forward()
-    net.finish()
-    apart = net.getOutput(net.output_layer)
-    net.enableTimings(False)
-    net.forward()
-    net.finish()
-    again = net.getOutput(net.output_layer)
-    net.cleanup()
-    assert np.array_equal(fused, apart) and np.array_equal(fused, again)
+    assert infos["dw"] == "dwconv3x3" and np.abs(dw_out).max() > 0 and np.abs(ex_out).max() > 0
+    for no_edw in (False, True):
+        if no_edw:
+            monkeypatch.setenv("FYNHIP_NO_EDW_FUSION", "1")
+        net = Block(fa.STORAGE_F16, 16, 96, 24, 28, 28, 1, False)
+        _, fused, infos = run(net)
+        assert "inside the launch" in infos["dw"]
+        net.enableTimings(True)
+        net.forward()
+        net.finish()
+        apart = net.getOutput(net.output_layer)
+        net.enableTimings(False)
+        net.forward()
+        net.finish()
+        again = net.getOutput(net.output_layer)
+        net.cleanup()
+        assert rel_l2(fused, apart) <= 1e-3
+        assert np.array_equal(fused, again)
 
 
 @pytest.mark.parametrize("storage", [fa.STORAGE_F32, fa.STORAGE_F16], ids=["f32", "f16"])
 def test_config4_mobilenetv2_with_fused_blocks(storage, monkeypatch):
     """The whole MobileNetV2-style graph with every eligible depthwise layer fused, eager and as a replayed graph,
-    against the same graph with the layers apart (bit-identical in fp32 storage) and against the oracle's free-running chain."""
+    against the same graph with the layers apart and against the oracle's free-running chain."""
     monkeypatch.setenv("FYNHIP_FORCE_DW_FUSION", "1")
     net = networks.MobileNetV2(storage)
     x, got, infos = run(net)
@@ -156,7 +211,7 @@ def test_config4_mobilenetv2_with_fused_blocks(storage, monkeypatch):
     replay = net.getOutput(net.output_layer)
     desc = net.describe()
     net.cleanup()
-    fused = [n for n, i in infos.items() if "computed inside" in i]
+    fused = [n for n, i in infos.items() if "inside the launch" in i]
     print("   fused:", len(fused), fused, flush=True)
     assert len(fused) >= 8
     assert np.array_equal(got, replay)
@@ -164,9 +219,7 @@ def test_config4_mobilenetv2_with_fused_blocks(storage, monkeypatch):
     twin = networks.MobileNetV2(storage)
     _, two, _ = run(twin)
     twin.cleanup()
-    if storage == fa.STORAGE_F32:
-        assert np.array_equal(got, two)
-    else:   # (last-bit differences of single values grow along the 52 layers of an untrained fp16 chain)
-        assert rel_l2(got, two) <= 5e-2
+    # (last-bit differences of single values grow along the 52 layers of an untrained chain, fp16 storage most of all)
+    assert rel_l2(got, two) <= (1e-4 if storage == fa.STORAGE_F32 else 5e-2)
     ref = O.run_network(desc, {net.input_key: x})[net.output_layer]
     assert rel_l2(got, ref) <= (1e-4 if storage == fa.STORAGE_F32 else 5e-2)
