@@ -58,7 +58,7 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--dir", required=True)
     ap.add_argument("--name", required=True)
-    ap.add_argument("--kernel", default="conv_mfma|conv_p16|conv_kr16|conv_h16|conv_rows|conv3x3|dwconv|gemv|pool|reduce")
+    ap.add_argument("--kernel", default="conv_mfma|conv_p16|conv_kr16|conv_d16|conv_e16dw|conv_h16|conv_rows|conv3x3|dwconv|gemv|pool|reduce")
     ap.add_argument("--bench-json")
     ap.add_argument("--kind", default="plain")
     ap.add_argument("--traffic-out")
