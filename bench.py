@@ -204,6 +204,8 @@ def conv_work(b):
 
 def launches_of(info):
     """Kernel launches a layer's forward() makes, from its kernel description."""
+    if "runs inside the launch of layer" in info:   # (a depthwise layer that a neighbouring 1x1 layer's launch computes)
+        return 0
     n = 1
     if "+shift_reduce" in info:
         n += 1

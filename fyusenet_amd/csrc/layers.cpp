@@ -2034,7 +2034,9 @@ void fuse_depthwise_layers(Net* net) {
             if (getenv("FYNHIP_TUNE_VERBOSE"))
                 fprintf(stderr, "[tune] 1x1 %d to %d at %dx%d + depthwise 3x3 (step %d): one launch %.1f us, two %.1f us\n", in_v.cp, ex->oc, ex->oh, ex->ow, dw->stride,
                         t_fused * 1e3f, t_two * 1e3f);
-            pick = t_fused < t_two;
+            // (a near tie goes to the single launch: it leaves the expanded tensor unwritten, which a timing loop that
+            // finds everything in the caches does not reward)
+            pick = t_fused < t_two * 1.05f;
             tune_cache_store_flag(key, pick);
         }
         if (!pick) {
