@@ -28,7 +28,10 @@ namespace fynhip {
 namespace {
 typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
 
-template <bool HS, int NCHK, int FW>
+// DWS = 1 or 2: the layer's input is the output of a depthwise 3x3 layer with step DWS that is not read from memory but
+// computed by every wave for its positions (nine texels of the depthwise layer's input per lane and chunk instead of
+// one of its output; that layer's own arithmetic and rounding), as in conv_kr16_kernel's staging.
+template <bool HS, int NCHK, int FW, int DWS = 0>
 __global__ __launch_bounds__(256) void conv_d16_kernel(const ConvP16Params p) {
     constexpr int NPL = HS ? 1 : 2, NPASS = HS ? 1 : 3;
     typedef typename std::conditional<HS, _Float16, float>::type store_t;
@@ -38,25 +41,51 @@ __global__ __launch_bounds__(256) void conv_d16_kernel(const ConvP16Params p) {
     const int mq = lane & 15, kq = lane >> 4;
     const unsigned range_bits = p.in_amax ? range_load(p.in_amax) : 0u;
     // this lane's position (positions beyond the last one repeat it and are not stored)
+    // p.wm = 4: the layer has no more fragments of output channels than grid rows, and the four waves of a workgroup take
+    // four tiles of 16 positions instead of sharing the fragments of one (p.wm = 1)
+    const int wfr = p.wm == 4 ? 0 : w, fpw = p.wm == 4 ? 1 : 4;   // this wave's first fragment inside the workgroup; fragments per workgroup and round
     const int npos = p.npos_y * p.npos_x;
-    const int pos = blockIdx.x * 16 + mq;
+    const int pos = (p.wm == 4 ? blockIdx.x * 4 + w : blockIdx.x) * 16 + mq;
     const bool okp = pos < npos;
     const int pc = okp ? pos : npos - 1;
     const int py = pc / p.npos_x, px = pc - py * p.npos_x;
-    const store_t* in = reinterpret_cast<const store_t*>(p.in) + ((size_t)(py * p.stride + p.in_y0) * p.in_wp + px * p.stride + p.in_x0) * p.in_cp + kq * 8;
     struct RawF { float4 a, b; };
     typedef typename std::conditional<HS, half8_t, RawF>::type raw_t;
-    raw_t raw[NCHK];
+    constexpr int NT = DWS > 0 ? 9 : 1;   // texels per lane and chunk
+    raw_t raw[NCHK][NT];
+    unsigned okm = 0u;                    // (depthwise input) taps inside the stored frame
+    if constexpr (DWS > 0) {
+        const store_t* din = reinterpret_cast<const store_t*>(p.dw_in);
 #pragma unroll
-    for (int c = 0; c < NCHK; c++) {
-        // (channels behind the tensor's pitch -- the pitch is a multiple of 8, not of 32 -- read as zero)
-        const bool okc = c * KC + kq * 8 < p.in_cp;
-        const store_t* src = okc ? in + c * KC : reinterpret_cast<const store_t*>(p.in);
-        if constexpr (HS) {
-            raw[c] = *reinterpret_cast<const half8_t*>(src);
-        } else {
-            raw[c].a = *reinterpret_cast<const float4*>(src);
-            raw[c].b = *reinterpret_cast<const float4*>(src + 4);
+        for (int t = 0; t < 9; t++) {
+            const int iy = py * DWS + t / 3 + p.dw_y0, ix = px * DWS + t % 3 + p.dw_x0;
+            const bool ok = (unsigned)iy < (unsigned)p.dw_hp && (unsigned)ix < (unsigned)p.dw_wp;
+            okm |= ok ? 1u << t : 0u;
+            const store_t* tap = din + (ok ? ((size_t)iy * p.dw_wp + ix) * p.dw_cp : 0) + kq * 8;
+#pragma unroll
+            for (int c = 0; c < NCHK; c++) {
+                const store_t* src = (c * KC + kq * 8 < p.in_cp) ? tap + c * KC : din;
+                if constexpr (HS) {
+                    raw[c][t] = *reinterpret_cast<const half8_t*>(src);
+                } else {
+                    raw[c][t].a = *reinterpret_cast<const float4*>(src);
+                    raw[c][t].b = *reinterpret_cast<const float4*>(src + 4);
+                }
+            }
+        }
+    } else {
+        const store_t* in = reinterpret_cast<const store_t*>(p.in) + ((size_t)(py * p.stride + p.in_y0) * p.in_wp + px * p.stride + p.in_x0) * p.in_cp + kq * 8;
+#pragma unroll
+        for (int c = 0; c < NCHK; c++) {
+            // (channels behind the tensor's pitch -- the pitch is a multiple of 8, not of 32 -- read as zero)
+            const bool okc = c * KC + kq * 8 < p.in_cp;
+            const store_t* src = okc ? in + c * KC : reinterpret_cast<const store_t*>(p.in);
+            if constexpr (HS) {
+                raw[c][0] = *reinterpret_cast<const half8_t*>(src);
+            } else {
+                raw[c][0].a = *reinterpret_cast<const float4*>(src);
+                raw[c][0].b = *reinterpret_cast<const float4*>(src + 4);
+            }
         }
     }
     const unsigned char* wbase = reinterpret_cast<const unsigned char*>(p.wpack) + lane * 16;
@@ -84,7 +113,7 @@ __global__ __launch_bounds__(256) void conv_d16_kernel(const ConvP16Params p) {
     // (scale and bias hold 16*mfrags values or more)
     auto sb_load = [&](const float* base, int frag) { return frag < p.mfrags ? *reinterpret_cast<const f32x4_t*>(base + frag * 16 + kq * 4) : (f32x4_t)(0.f); };
     // (the fragments of output channels may be dealt to p.cout_blocks workgroups per tile: grid rows)
-    const int f0 = blockIdx.y * 4 + w, fstep = 4 * p.cout_blocks;
+    const int f0 = blockIdx.y * fpw + wfr, fstep = fpw * p.cout_blocks;
     constexpr int NF = FW > 0 ? FW : 1;
     half8_t a_q[NF][NCHK][NPL];
     res_t r_q[NF];
@@ -100,15 +129,47 @@ __global__ __launch_bounds__(256) void conv_d16_kernel(const ConvP16Params p) {
     float in_scale = 1.f, inv_in_scale = 1.f;
     if (p.in_amax) in_scale = range_scale(range_after_act(range_reduce(range_bits), p.act), &inv_in_scale);
     const float acc_mul = p.acc_mul * inv_in_scale;
+    auto texel = [&](const raw_t& rw, float (&x)[8]) {
+        if constexpr (HS) {
+#pragma unroll
+            for (int e = 0; e < 8; e++) x[e] = (float)rw[e];
+        } else {
+            x[0] = rw.a.x; x[1] = rw.a.y; x[2] = rw.a.z; x[3] = rw.a.w; x[4] = rw.b.x; x[5] = rw.b.y; x[6] = rw.b.z; x[7] = rw.b.w;
+        }
+    };
     half8_t b[NCHK][NPL];
 #pragma unroll
     for (int c = 0; c < NCHK; c++) {
         const bool okc = c * KC + kq * 8 < p.in_cp;
+        float r[8];   // the layer's input values of this lane: from the tensor, or the depthwise layer's results
+        if constexpr (DWS > 0) {
+            const int ch = okc ? c * KC + kq * 8 : 0;
+#pragma unroll
+            for (int e = 0; e < 8; e++) r[e] = 0.f;
+#pragma unroll
+            for (int t = 0; t < 9; t++) {   // (ky outer, kx inner, fused multiply-add: the depthwise kernel's order)
+                float x[8];
+                texel(raw[c][t], x);
+                const float4 w0 = *reinterpret_cast<const float4*>(p.dw_w + t * p.dw_cp + ch), w1 = *reinterpret_cast<const float4*>(p.dw_w + t * p.dw_cp + ch + 4);
+                const float wv[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
+#pragma unroll
+                for (int e = 0; e < 8; e++) r[e] = fmaf(act_p16(((okm >> t) & 1u) ? x[e] : 0.f, p.dw_act), wv[e], r[e]);
+            }
+            const float4 s0 = *reinterpret_cast<const float4*>(p.dw_scale + ch), s1 = *reinterpret_cast<const float4*>(p.dw_scale + ch + 4);
+            const float4 b0 = *reinterpret_cast<const float4*>(p.dw_bias + ch), b1 = *reinterpret_cast<const float4*>(p.dw_bias + ch + 4);
+            const float sv[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w}, bv[8] = {b0.x, b0.y, b0.z, b0.w, b1.x, b1.y, b1.z, b1.w};
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                r[e] = r[e] * sv[e] + bv[e];
+                if constexpr (HS) r[e] = (float)(_Float16)r[e];   // (what the depthwise layer would have stored)
+            }
+        } else {
+            texel(raw[c][0], r);
+        }
         if constexpr (HS) {
 #pragma unroll
-            for (int e = 0; e < 8; e++) b[c][0][e] = okc ? (_Float16)act_p16((float)raw[c][e], p.act) : (_Float16)0.f;
+            for (int e = 0; e < 8; e++) b[c][0][e] = okc ? (_Float16)act_p16(r[e], p.act) : (_Float16)0.f;
         } else {
-            const float r[8] = {raw[c].a.x, raw[c].a.y, raw[c].a.z, raw[c].a.w, raw[c].b.x, raw[c].b.y, raw[c].b.z, raw[c].b.w};
 #pragma unroll
             for (int e = 0; e < 8; e++) {
                 const float v = okc ? act_p16(r[e], p.act) * in_scale : 0.f;
@@ -180,8 +241,9 @@ typedef void (*d16_fn)(const ConvP16Params);
 // fragments of 16 output channels per wave whose weights are all requested up front: as many as the layer has when they
 // fit 64 registers, else 0 (one fragment ahead)
 template <bool HS>
-int d16_fw(int chunks, int mfrags, int cout_blocks) {
-    const int fw = (mfrags + 4 * cout_blocks - 1) / (4 * cout_blocks);
+int d16_fw(int chunks, int mfrags, int cout_blocks, int wm) {
+    const int per_round = (wm == 4 ? 1 : 4) * cout_blocks;
+    const int fw = (mfrags + per_round - 1) / per_round;
     return (fw <= 4 && chunks * (HS ? 1 : 2) * fw <= 16) ? fw : 0;
 }
 template <bool HS, int NCHK>
@@ -196,8 +258,8 @@ d16_fn pick_d16_fw(int fw) {
     }
 }
 template <bool HS>
-d16_fn pick_d16(int chunks, int mfrags, int cout_blocks) {
-    const int fw = d16_fw<HS>(chunks, mfrags, cout_blocks);
+d16_fn pick_d16(int chunks, int mfrags, int cout_blocks, int wm) {
+    const int fw = d16_fw<HS>(chunks, mfrags, cout_blocks, wm);
     switch (chunks) {
         case 1: return pick_d16_fw<HS, 1>(fw);
         case 2: return pick_d16_fw<HS, 2>(fw);
@@ -360,26 +422,46 @@ d16_fn pick_e16dw(int chunks) {
         default: return nullptr;
     }
 }
+// with a depthwise layer in front: up to 96 channels, one fragment per wave up front or one ahead
+template <bool HS, int DWS>
+d16_fn pick_d16_dw(int chunks, bool one) {
+    switch (chunks) {
+        case 1: return one ? conv_d16_kernel<HS, 1, 1, DWS> : conv_d16_kernel<HS, 1, 0, DWS>;
+        case 2: return one ? conv_d16_kernel<HS, 2, 1, DWS> : conv_d16_kernel<HS, 2, 0, DWS>;
+        case 3: return one ? conv_d16_kernel<HS, 3, 1, DWS> : conv_d16_kernel<HS, 3, 0, DWS>;
+        default: return nullptr;
+    }
+}
 }  // namespace
 
+bool conv_d16_dw_supported(int chunks, int dw_stride) { return chunks >= 1 && chunks <= 3 && (dw_stride == 1 || dw_stride == 2); }
+
 bool conv_d16_supported(int k, int dil, int in_cp, int chunks, int cout, int out_cp) {
-    return k == 1 && dil == 1 && in_cp % 8 == 0 && in_cp >= 8 && pick_d16<true>(chunks, 1, 1) != nullptr && in_cp <= chunks * KC && cout >= 4 && out_cp % 4 == 0 && out_cp >= cout;
+    return k == 1 && dil == 1 && in_cp % 8 == 0 && in_cp >= 8 && pick_d16<true>(chunks, 1, 1, 1) != nullptr && in_cp <= chunks * KC && cout >= 4 && out_cp % 4 == 0 && out_cp >= cout;
 }
 
 // p.cin_chunks = 32-channel chunks (1..6, 8; channels behind in_cp read as zero), p.mfrags = fragments of 16 output
 // channels (scale and bias hold 16*mfrags values; rows beyond out_cp are not stored), in_y0/in_x0 = input padding,
 // p.stride = pixel step per position; p.cout_blocks (1 or more) workgroups of 256 threads per 16 positions, which
-// share the fragments of output channels
+// share the fragments of output channels, or (p.wm = 4 instead of 1) one wave per 16 positions and grid row
 int launch_conv_d16(const ConvP16Params& p, hipStream_t s) {
-    if (p.cout_blocks < 1 || p.cout_blocks > 64) return -5;
-    const d16_fn fn = p.f16 ? pick_d16<true>(p.cin_chunks, p.mfrags, p.cout_blocks) : pick_d16<false>(p.cin_chunks, p.mfrags, p.cout_blocks);
+    if (p.cout_blocks < 1 || p.cout_blocks > 64 || (p.wm != 1 && p.wm != 4)) return -5;
+    d16_fn fn = p.f16 ? pick_d16<true>(p.cin_chunks, p.mfrags, p.cout_blocks, p.wm) : pick_d16<false>(p.cin_chunks, p.mfrags, p.cout_blocks, p.wm);
+    if (p.dw_in) {
+        // (the depthwise layer's tensor has the 1x1 layer's channels; the 1x1 layer does not step)
+        if (!conv_d16_dw_supported(p.cin_chunks, p.dw_stride) || !p.dw_w || !p.dw_scale || !p.dw_bias || p.dw_cp != p.in_cp || p.stride != 1 || p.dw_hp < 1 || p.dw_wp < 1) return -5;
+        const bool one = p.mfrags <= (p.wm == 4 ? 1 : 4) * p.cout_blocks;
+        fn = p.f16 ? (p.dw_stride == 1 ? pick_d16_dw<true, 1>(p.cin_chunks, one) : pick_d16_dw<true, 2>(p.cin_chunks, one))
+                   : (p.dw_stride == 1 ? pick_d16_dw<false, 1>(p.cin_chunks, one) : pick_d16_dw<false, 2>(p.cin_chunks, one));
+    }
     const long long npos = (long long)p.npos_y * p.npos_x;
     if (!fn) return -1;
     if (p.in_cp > p.cin_chunks * KC || p.in_cp % 8 != 0 || p.in_cp < 8 || p.mfrags < 1 || p.stride < 1 || npos < 1 || npos > (1ll << 30) || p.out_cp % 4 != 0 || p.out_cp < 4 ||
-        (p.res && (p.res_cp < p.out_cp || p.res_cp % 4 != 0)) || p.nreset < 0 || p.nreset > 4 || p.in_clamp || p.dw_in ||
+        (p.res && (p.res_cp < p.out_cp || p.res_cp % 4 != 0)) || p.nreset < 0 || p.nreset > 4 || p.in_clamp ||
         (long long)((p.npos_y - 1) * p.stride + p.in_y0) >= p.in_hp || (long long)((p.npos_x - 1) * p.stride + p.in_x0) >= p.in_wp || p.in_y0 < 0 || p.in_x0 < 0)
         return -5;
-    hipLaunchKernelGGL(fn, dim3((unsigned)((npos + 15) / 16), (unsigned)p.cout_blocks), dim3(256), 0, s, p);
+    const long long per_wg = 16 * p.wm;
+    hipLaunchKernelGGL(fn, dim3((unsigned)((npos + per_wg - 1) / per_wg), (unsigned)p.cout_blocks), dim3(256), 0, s, p);
     return hipGetLastError() == hipSuccess ? 0 : -3;
 }
 

@@ -1304,8 +1304,9 @@ class ConvLayer : public Layer {
         const size_t halves = (size_t)q.mfrags * q.cin_chunks * (q.f16 ? 1 : 2) * 64 * 8;
         void* const wp = net->dev_alloc(halves * 2, true);
         q.wpack = wp;
+        q.wm = 1;
         q.cout_blocks = 1;   // workgroups per 16 positions (they share the fragments of output channels): 1, 2 or 4, timed
-        if (const char* e = getenv("FYNHIP_D16_BLOCKS")) q.cout_blocks = std::max(1, std::min(4, atoi(e)));
+        if (const char* e = getenv("FYNHIP_D16_BLOCKS")) q.cout_blocks = std::max(-4, std::min(4, atoi(e))) ? std::max(-4, std::min(4, atoi(e))) : 1;   // (negative: a wave per 16 positions)
         const bool always = getenv("FYNHIP_FORCE_D16_CONV") != nullptr;
         const char* at = getenv("FYNHIP_AUTOTUNE");
         bool pick = true;
@@ -1316,7 +1317,7 @@ class ConvLayer : public Layer {
             pick = always;
         } else if (tune_cache_triple(key, cached)) {
             pick = cached[0] != 0 || always;
-            q.cout_blocks = std::max(1, cached[1]);
+            q.cout_blocks = cached[1] ? cached[1] : 1;
         } else if (!(at && at[0] == '0')) {
             float t_new = 1e30f, t_other = 1e30f;
             int best_blocks = 1;
@@ -1329,6 +1330,14 @@ class ConvLayer : public Layer {
                     }, 10);
                     if (t < t_new) { t_new = t; best_blocks = blocks; }
                 }
+                if (q.mfrags <= 4) {   // few fragments: a wave per 16 positions and fragment instead (noted as a negative count)
+                    ConvP16Params c = q;
+                    c.wm = 4; c.cout_blocks = q.mfrags;
+                    const float t = time_calls(net, [&]() {
+                        if (launch_conv_d16(c, net->stream) != 0) fail(FYN_ERR_DEVICE, "LDS-free 1x1 convolution launch failed while tuning");
+                    }, 10);
+                    if (t < t_new) { t_new = t; best_blocks = -q.mfrags; }
+                }
                 if (kr16)
                     t_other = std::min(t_other, time_calls(net, [&]() {
                         if (launch_conv_kr16(pp, k, net->stream) != 0) fail(FYN_ERR_DEVICE, "K-resident convolution launch failed while tuning");
@@ -1337,12 +1346,13 @@ class ConvLayer : public Layer {
                     t_other = std::min(t_other, time_launch(net, launch, 10));
             }
             if (getenv("FYNHIP_TUNE_VERBOSE"))
-                fprintf(stderr, "[tune] 1x1 on %d channels, %dx%d positions, to %d: LDS-free form (%d workgroups per 16 positions) %.1f us, %s %.1f us\n", d.in_channels, oh, ow,
-                        oc, best_blocks, t_new * 1e3f, kr16 ? "K-resident form" : "general kernel", t_other * 1e3f);
+                fprintf(stderr, "[tune] 1x1 on %d channels, %dx%d positions, to %d: LDS-free form (%d %s per 16 positions) %.1f us, %s %.1f us\n", d.in_channels, oh, ow,
+                        oc, best_blocks < 0 ? 1 : best_blocks, best_blocks < 0 ? "wave per fragment" : "workgroup(s)", t_new * 1e3f, kr16 ? "K-resident form" : "general kernel", t_other * 1e3f);
             pick = t_new < t_other || always;
             q.cout_blocks = best_blocks;
             tune_cache_store_triple(key, t_new < t_other ? 1 : 0, best_blocks, 0);
         }
+        if (q.cout_blocks < 0) { q.wm = 4; q.cout_blocks = -q.cout_blocks; }
         if (pick) {
             if (p16) net->dev_free(p16_wpack_dev);
             p16_wpack_dev = wp;
@@ -1781,8 +1791,8 @@ class ConvLayer : public Layer {
             if (launch_conv_rows(rp, tout().v.f16 != 0, s) != 0) fail(FYN_ERR_DEVICE, "layer %s: convolution launch failed", d.name);
             return;
         }
-        if (p16 && kr16 && dw_fused && net->fusion_on()) {
-            if (launch_conv_kr16(with_depthwise(), k, s) != 0) fail(FYN_ERR_DEVICE, "layer %s: convolution launch failed", d.name);
+        if (p16 && (kr16 || d16) && dw_fused && net->fusion_on()) {
+            if ((d16 ? launch_conv_d16(with_depthwise(), s) : launch_conv_kr16(with_depthwise(), k, s)) != 0) fail(FYN_ERR_DEVICE, "layer %s: convolution launch failed", d.name);
             return;
         }
         if (p16) {
@@ -1821,8 +1831,10 @@ class ConvLayer : public Layer {
         }
         if (p16 && d16) {
             char buf[220];
-            snprintf(buf, sizeof(buf), "conv_d16 %s 1x1 without LDS: %d workgroup(s) of 4 waves per 16 positions, %d chunks in registers, %d fragments of 16 output channels, blocks=%d",
-                     pp.f16 ? "f16" : "f16x2-split", pp.cout_blocks, pp.cin_chunks, pp.mfrags, (pp.npos_y * pp.npos_x + 15) / 16 * pp.cout_blocks);
+            snprintf(buf, sizeof(buf), "conv_d16 %s 1x1 without LDS: %s, %d chunks in registers, %d fragments of 16 output channels, blocks=%d",
+                     pp.f16 ? "f16" : "f16x2-split", (pp.wm == 4 ? "a wave per 16 positions and fragment" : (std::to_string(pp.cout_blocks) + " workgroup(s) of 4 waves per 16 positions").c_str()),
+                     pp.cin_chunks, pp.mfrags, (pp.npos_y * pp.npos_x + 16 * pp.wm - 1) / (16 * pp.wm) * pp.cout_blocks);
+            if (dw_fused) return mode + buf + "; the depthwise 3x3 layer " + std::to_string(dw_layer_no) + " in front of it is computed by the waves themselves";
             return mode + buf;
         }
         if (p16 && kr16) {
@@ -1889,8 +1901,10 @@ class ConvLayer : public Layer {
         return q;
     }
     bool takes_depthwise() const {
-        return p16 && kr16 && k == 1 && stride == 1 && pp.tile_h == 4 && pp.tile_w == 4 && !clamp && !pp.in_amax && !pp.in_clamp;
+        return p16 && ((kr16 && pp.tile_h == 4 && pp.tile_w == 4) || d16) && k == 1 && stride == 1 && !clamp && !pp.in_amax && !pp.in_clamp;
     }
+    int launch_with_depthwise(const ConvP16Params& q, hipStream_t s) const { return d16 ? launch_conv_d16(q, s) : launch_conv_kr16(q, 1, s); }
+    int launch_own(hipStream_t s) const { return d16 ? launch_conv_d16(pp, s) : launch_conv_kr16(pp, 1, s); }
     bool h16_two = false;         // ...... as two launches on two bands of rows (pp, pp2)
     ConvP16Params pp{}, pp2{};
     void* p16_wpack_dev = nullptr;
@@ -2066,21 +2080,21 @@ void fuse_depthwise_layers(Net* net) {
         f.dw_y0 = f.dw_x0 = dw->p.in.pad - 1;
         f.dw_stride = dw->stride; f.dw_act = dw->p.act;
         const ConvP16Params q = pw->with_depthwise();
-        if (conv_kr16_lds_bytes(q, 1) == 0 || conv_kr16_lds_bytes(q, 1) > 160 * 1024) continue;
+        if (pw->d16 ? !conv_d16_dw_supported(q.cin_chunks, q.dw_stride) : (conv_kr16_lds_bytes(q, 1) == 0 || conv_kr16_lds_bytes(q, 1) > 160 * 1024)) continue;
         bool pick = true;
         char key[200];
-        snprintf(key, sizeof(key), "dwpw:%d:%dx%dx%d:s%d:to%d:fm%d", q.f16, dw->p.in.cp, dw->p.in.h, dw->p.in.w, dw->stride, pw->oc, q.wm);
+        snprintf(key, sizeof(key), "dwpw:%d:%dx%dx%d:s%d:to%d:fm%d:d%d", q.f16, dw->p.in.cp, dw->p.in.h, dw->p.in.w, dw->stride, pw->oc, q.wm, pw->d16 ? 1 : 0);
         if (getenv("FYNHIP_FORCE_DW_FUSION")) {
         } else if (tune_cache_flag(key, &pick)) {
         } else if (!(at && at[0] == '0')) {
             float t_fused = 1e30f, t_two = 1e30f;
             for (int rep = 0; rep < 3; rep++) {
                 t_fused = std::min(t_fused, time_calls(net, [&]() {
-                    if (launch_conv_kr16(q, 1, net->stream) != 0) fail(FYN_ERR_DEVICE, "K-resident convolution with a depthwise layer in its staging: launch failed while tuning");
+                    if (pw->launch_with_depthwise(q, net->stream) != 0) fail(FYN_ERR_DEVICE, "1x1 convolution with a depthwise layer in front: launch failed while tuning");
                 }, 10));
                 t_two = std::min(t_two, time_calls(net, [&]() {
                     launch_dwconv3x3(dw->p, net->stream);
-                    if (launch_conv_kr16(pw->pp, 1, net->stream) != 0) fail(FYN_ERR_DEVICE, "K-resident convolution launch failed while tuning");
+                    if (pw->launch_own(net->stream) != 0) fail(FYN_ERR_DEVICE, "1x1 convolution launch failed while tuning");
                 }, 10));
             }
             if (getenv("FYNHIP_TUNE_VERBOSE"))

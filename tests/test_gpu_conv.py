@@ -476,12 +476,16 @@ D16_CASES = [
     (64, 256, 28, 28, {"bn": True, "residual": (A.RELU, True), "blocks": 2}),
     (32, 320, 24, 24, {"blocks": 4}),
     (96, 24, 30, 30, {"blocks": 2}),                                             # more waves than fragments
+    # a wave per 16 positions and fragment (layers with up to four fragments of output channels)
+    (32, 16, 56, 60, {"residual": (A.NONE, False), "blocks": -1}),
+    (96, 24, 37, 29, {"bn": True, "blocks": -2}),
+    (144, 40, 20, 20, {"blocks": -3}),
 ]
 
 
 @pytest.mark.parametrize("storage", [fa.STORAGE_F32, fa.STORAGE_F16], ids=["f32", "f16"])
 @pytest.mark.parametrize("variant", ["relu", "leaky", "shallow"])
-@pytest.mark.parametrize("case", D16_CASES, ids=lambda c: "%dx%dx%d_to%d%s%s" % (c[0], c[2], c[3], c[1], "_s2" if c[4].get("stride") == 2 else "", "_b%d" % c[4]["blocks"] if "blocks" in c[4] else ""))
+@pytest.mark.parametrize("case", D16_CASES, ids=lambda c: "%dx%dx%d_to%d%s%s" % (c[0], c[2], c[3], c[1], "_s2" if c[4].get("stride") == 2 else "", ("_b%d" % c[4]["blocks"]).replace("-", "w") if "blocks" in c[4] else ""))
 def test_pointwise_without_lds(case, variant, storage, monkeypatch):
     """1x1 convolutions on many positions whose B fragments come straight from the tensor: a workgroup of four waves per
     16 positions, the waves sharing the fragments of output channels."""
@@ -508,7 +512,7 @@ def test_pointwise_without_lds(case, variant, storage, monkeypatch):
     ref = oracle_single(b, storage, inputs, wts)
     err = rel_l2(got, ref)
     print("  ", info, "rel_l2=%.3e" % err, flush=True)
-    assert "conv_d16" in info and (not blocks or "%d workgroup(s)" % blocks in info)
+    assert "conv_d16" in info and (not blocks or ("%d workgroup(s)" % blocks if blocks > 0 else "a wave per 16 positions") in info)
     assert err <= TOL[storage], info
 
 

@@ -146,6 +146,41 @@ def test_depthwise_inside_pointwise_staging(case, storage, monkeypatch):
     assert_same_as_two_launches(got, two, storage)
 
 
+D16_CASES = [
+    (16, 32, 16, 40, 40, 1, False),      # one chunk, one fragment of output channels
+    (16, 96, 24, 36, 36, 2, False),      # three chunks, step 2
+    (24, 48, 24, 30, 34, 1, True),       # a chunk and a half, residual add
+    (32, 64, 80, 20, 20, 1, False),      # five fragments: more than one per wave, one ahead of their use
+]
+
+
+@pytest.mark.parametrize("storage", [fa.STORAGE_F32, fa.STORAGE_F16], ids=["f32", "f16"])
+@pytest.mark.parametrize("case", D16_CASES, ids=lambda c: "%dto%dto%d_%dx%d_s%d%s" % (c[0], c[1], c[2], c[3], c[4], c[5], "_res" if c[6] else ""))
+def test_depthwise_inside_the_lds_free_pointwise_kernel(case, storage, monkeypatch):
+    """The same second half of the block where the 1x1 layer runs the LDS-free kernel (many positions, up to 96
+    channels): every wave computes the depthwise layer for its positions."""
+    cin, exp, cout, h, w, stride, residual = case
+    monkeypatch.setenv("FYNHIP_FORCE_D16_CONV", "1")
+    monkeypatch.setenv("FYNHIP_FORCE_DW_FUSION", "1")
+    monkeypatch.setenv("FYNHIP_NO_EDW_FUSION", "1")
+    net = Block(storage, cin, exp, cout, h, w, stride, residual)
+    x, got, infos = run(net)
+    desc = net.describe()
+    net.cleanup()
+    print("  ", infos["dw"], "|", infos["project"], flush=True)
+    assert "launch of layer 3" in infos["dw"] and "conv_d16" in infos["project"] and "depthwise 3x3 layer 2" in infos["project"]
+    ref = O.run_network(desc, {net.input_key: x})[net.output_layer]
+    err = rel_l2(got, ref)
+    print("   rel_l2=%.3e" % err, flush=True)
+    assert err <= TOL[storage]
+    monkeypatch.setenv("FYNHIP_NO_DW_FUSION", "1")
+    twin = Block(storage, cin, exp, cout, h, w, stride, residual)
+    _, two, infos2 = run(twin)
+    twin.cleanup()
+    assert infos2["dw"] == "dwconv3x3"
+    assert_same_as_two_launches(got, two, storage)
+
+
 def test_layers_stay_apart_when_the_tensor_is_needed(monkeypatch):
     """No fusion when the tensor between the two layers has a second reader, or when the caller keeps every layer's
     tensor (buffer reuse off); per-layer timing runs the layers apart and leaves the results unchanged."""
