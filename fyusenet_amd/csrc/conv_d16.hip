@@ -31,8 +31,14 @@ typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
 // DWS = 1 or 2: the layer's input is the output of a depthwise 3x3 layer with step DWS that is not read from memory but
 // computed by every wave for its positions (nine texels of the depthwise layer's input per lane and chunk instead of
 // one of its output; that layer's own arithmetic and rounding), as in conv_kr16_kernel's staging.
-template <bool HS, int NCHK, int FW, int DWS = 0>
+// KS = 3, 5 or 7: not a 1x1 layer but a KS x KS convolution on an input of at most four channels (a classification
+// net's first layer; reference: gpu/deep/deepconvlayerNxN.cpp:129-211): a stored pixel is four channels, a lane's eight
+// values of a k32 step are two taps in row-major order (tap 8*step + 2*(lane/16) + {0, 1}), gathered from the image
+// with two loads; taps beyond the kernel and pixels outside the stored frame are zeros.  p.stride = step, in_y0 /
+// in_x0 = stored coordinate of tap (0,0) of position (0,0) (may be negative), p.tile_h = KS.
+template <bool HS, int NCHK, int FW, int DWS = 0, int KS = 0>
 __global__ __launch_bounds__(256) void conv_d16_kernel(const ConvP16Params p) {
+    static_assert(KS == 0 || (DWS == 0 && NCHK == (KS * KS + 7) / 8), "a small-input convolution: steps of eight taps");
     constexpr int NPL = HS ? 1 : 2, NPASS = HS ? 1 : 3;
     typedef typename std::conditional<HS, _Float16, float>::type store_t;
     if (blockIdx.x == 0 && blockIdx.y == 0) range_clear(p.reset[0], p.reset[1], p.reset[2], p.reset[3], p.nreset);
@@ -71,6 +77,31 @@ __global__ __launch_bounds__(256) void conv_d16_kernel(const ConvP16Params p) {
                     raw[c][t].a = *reinterpret_cast<const float4*>(src);
                     raw[c][t].b = *reinterpret_cast<const float4*>(src + 4);
                 }
+            }
+        }
+    } else if constexpr (KS > 0) {
+        const store_t* in = reinterpret_cast<const store_t*>(p.in);
+        typedef typename std::conditional<HS, half4_t, float4>::type pix_t;
+#pragma unroll
+        for (int c = 0; c < NCHK; c++) {
+            pix_t pix[2];
+#pragma unroll
+            for (int h = 0; h < 2; h++) {
+                const int t = c * 8 + 2 * kq + h;
+                const int ty = t / KS, tx = t - ty * KS;
+                const int iy = py * p.stride + ty + p.in_y0, ix = px * p.stride + tx + p.in_x0;
+                const bool ok = t < KS * KS && (unsigned)iy < (unsigned)p.in_hp && (unsigned)ix < (unsigned)p.in_wp;
+                pix[h] = *reinterpret_cast<const pix_t*>(in + (ok ? ((size_t)iy * p.in_wp + ix) * 4 : 0));
+                if (!ok) {
+                    if constexpr (HS) pix[h] = (half4_t)((_Float16)0.f);
+                    else pix[h] = make_float4(0.f, 0.f, 0.f, 0.f);
+                }
+            }
+            if constexpr (HS) {
+                raw[c][0] = half8_t{pix[0][0], pix[0][1], pix[0][2], pix[0][3], pix[1][0], pix[1][1], pix[1][2], pix[1][3]};
+            } else {
+                raw[c][0].a = pix[0];
+                raw[c][0].b = pix[1];
             }
         }
     } else {
@@ -140,7 +171,7 @@ __global__ __launch_bounds__(256) void conv_d16_kernel(const ConvP16Params p) {
     half8_t b[NCHK][NPL];
 #pragma unroll
     for (int c = 0; c < NCHK; c++) {
-        const bool okc = c * KC + kq * 8 < p.in_cp;
+        const bool okc = KS > 0 || c * KC + kq * 8 < p.in_cp;
         float r[8];   // the layer's input values of this lane: from the tensor, or the depthwise layer's results
         if constexpr (DWS > 0) {
             const int ch = okc ? c * KC + kq * 8 : 0;
@@ -432,7 +463,21 @@ d16_fn pick_d16_dw(int chunks, bool one) {
         default: return nullptr;
     }
 }
+// a K x K convolution on at most four input channels: one fragment per wave and round
+template <bool HS>
+d16_fn pick_d16_ks(int ks) {
+    switch (ks) {
+        case 3: return conv_d16_kernel<HS, 2, 1, 0, 3>;
+        case 5: return conv_d16_kernel<HS, 4, 1, 0, 5>;
+        case 7: return conv_d16_kernel<HS, 7, 1, 0, 7>;
+        default: return nullptr;
+    }
+}
 }  // namespace
+
+bool conv_d16_small_supported(int k, int dil, int in_cp, int cout, int out_cp) {
+    return (k == 3 || k == 5 || k == 7) && dil == 1 && in_cp == 4 && cout >= 4 && out_cp % 4 == 0 && out_cp >= cout;
+}
 
 bool conv_d16_dw_supported(int chunks, int dw_stride) { return chunks >= 1 && chunks <= 3 && (dw_stride == 1 || dw_stride == 2); }
 
@@ -447,6 +492,12 @@ bool conv_d16_supported(int k, int dil, int in_cp, int chunks, int cout, int out
 int launch_conv_d16(const ConvP16Params& p, hipStream_t s) {
     if (p.cout_blocks < 1 || p.cout_blocks > 64 || (p.wm != 1 && p.wm != 4)) return -5;
     d16_fn fn = p.f16 ? pick_d16<true>(p.cin_chunks, p.mfrags, p.cout_blocks, p.wm) : pick_d16<false>(p.cin_chunks, p.mfrags, p.cout_blocks, p.wm);
+    const int ks = p.tile_h;   // 0: a 1x1 layer
+    if (ks) {
+        // (p.cin_chunks = steps of eight taps; every wave has at most one fragment per round)
+        if (p.dw_in || p.in_cp != 4 || p.cin_chunks != (ks * ks + 7) / 8 || p.mfrags > (p.wm == 4 ? 1 : 4) * p.cout_blocks) return -5;
+        fn = p.f16 ? pick_d16_ks<true>(ks) : pick_d16_ks<false>(ks);
+    }
     if (p.dw_in) {
         // (the depthwise layer's tensor has the 1x1 layer's channels; the 1x1 layer does not step)
         if (!conv_d16_dw_supported(p.cin_chunks, p.dw_stride) || !p.dw_w || !p.dw_scale || !p.dw_bias || p.dw_cp != p.in_cp || p.stride != 1 || p.dw_hp < 1 || p.dw_wp < 1) return -5;
@@ -456,9 +507,9 @@ int launch_conv_d16(const ConvP16Params& p, hipStream_t s) {
     }
     const long long npos = (long long)p.npos_y * p.npos_x;
     if (!fn) return -1;
-    if (p.in_cp > p.cin_chunks * KC || p.in_cp % 8 != 0 || p.in_cp < 8 || p.mfrags < 1 || p.stride < 1 || npos < 1 || npos > (1ll << 30) || p.out_cp % 4 != 0 || p.out_cp < 4 ||
+    if ((!ks && (p.in_cp > p.cin_chunks * KC || p.in_cp % 8 != 0 || p.in_cp < 8)) || p.mfrags < 1 || p.stride < 1 || npos < 1 || npos > (1ll << 30) || p.out_cp % 4 != 0 || p.out_cp < 4 ||
         (p.res && (p.res_cp < p.out_cp || p.res_cp % 4 != 0)) || p.nreset < 0 || p.nreset > 4 || p.in_clamp ||
-        (long long)((p.npos_y - 1) * p.stride + p.in_y0) >= p.in_hp || (long long)((p.npos_x - 1) * p.stride + p.in_x0) >= p.in_wp || p.in_y0 < 0 || p.in_x0 < 0)
+        (!ks && ((long long)((p.npos_y - 1) * p.stride + p.in_y0) >= p.in_hp || (long long)((p.npos_x - 1) * p.stride + p.in_x0) >= p.in_wp || p.in_y0 < 0 || p.in_x0 < 0)))
         return -5;
     const long long per_wg = 16 * p.wm;
     hipLaunchKernelGGL(fn, dim3((unsigned)((npos + per_wg - 1) / per_wg), (unsigned)p.cout_blocks), dim3(256), 0, s, p);

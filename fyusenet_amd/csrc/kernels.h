@@ -240,6 +240,8 @@ int launch_conv_p16c4(const ConvP16Params& p, int k, hipStream_t s);
 bool conv_d16_supported(int k, int dil, int in_cp, int chunks, int cout, int out_cp);
 int launch_conv_d16(const ConvP16Params& p, hipStream_t s);   // (p.dw_in set: with a depthwise 3x3 layer in front computed by the waves, conv_d16_dw_supported)
 bool conv_d16_dw_supported(int chunks, int dw_stride);
+// (p.tile_h = 3, 5 or 7: a K x K convolution on an input of at most four channels instead, cin_chunks = steps of eight taps)
+bool conv_d16_small_supported(int k, int dil, int in_cp, int cout, int out_cp);
 // a 1x1 layer and the depthwise 3x3 layer behind it as one launch (conv_d16.hip: conv_e16dw_kernel)
 bool conv_e16dw_supported(int in_cp, int chunks, int dw_stride);
 int launch_conv_e16dw(const ConvP16Params& p, hipStream_t s);

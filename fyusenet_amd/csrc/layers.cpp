@@ -1290,12 +1290,14 @@ class ConvLayer : public Layer {
         q.in = in_v.ptr; q.out = out_v.ptr; q.res = res_v ? res_v->ptr : nullptr;
         q.in_hp = in_v.hp(); q.in_wp = in_v.wp(); q.in_cp = in_v.cp;
         q.stride = stride;
-        q.in_y0 = q.in_x0 = in_v.pad;
+        const int ks = k == 1 ? 0 : k;   // a K x K convolution on an input of at most four channels: steps of eight taps
+        q.tile_h = ks;
+        q.in_y0 = q.in_x0 = in_v.pad - (k - 1) / 2;
         q.npos_y = oh; q.npos_x = ow;
         q.out_wp = out_v.wp(); q.out_cp = out_v.cp; q.out_off_y = q.out_off_x = out_v.pad;
         if (res_v) { q.res_wp = res_v->wp(); q.res_cp = res_v->cp; q.res_off_y = q.res_off_x = res_v->pad; }
         q.res_relu = res_relu; q.res_scale = res_scale;
-        q.cin_chunks = (in_v.cp + 31) / 32;
+        q.cin_chunks = ks ? (ks * ks + 7) / 8 : (in_v.cp + 31) / 32;
         q.mfrags = (oc + 15) / 16;
         q.f16 = out_v.f16 ? 1 : 0;
         q.scale = scale_dev; q.bias = bias_dev;
@@ -1306,12 +1308,15 @@ class ConvLayer : public Layer {
         q.wpack = wp;
         q.wm = 1;
         q.cout_blocks = 1;   // workgroups per 16 positions (they share the fragments of output channels): 1, 2 or 4, timed
+        const int min_blocks = ks ? (q.mfrags + 3) / 4 : 1;   // (the K x K form: one fragment per wave)
+        if (ks && min_blocks > 4) { net->dev_free(wp); return; }
+        q.cout_blocks = min_blocks;
         if (const char* e = getenv("FYNHIP_D16_BLOCKS")) q.cout_blocks = std::max(-4, std::min(4, atoi(e))) ? std::max(-4, std::min(4, atoi(e))) : 1;   // (negative: a wave per 16 positions)
         const bool always = getenv("FYNHIP_FORCE_D16_CONV") != nullptr;
         const char* at = getenv("FYNHIP_AUTOTUNE");
         bool pick = true;
         char key[160];
-        snprintf(key, sizeof(key), "d16:%dx%d:%dx%d:s%d:r%d:h%d:kr%d", d.in_channels, oc, oh, ow, stride, res_v ? 1 : 0, q.f16, kr16 ? 1 : 0);
+        snprintf(key, sizeof(key), "d16:k%d:%dx%d:%dx%d:s%d:r%d:h%d:kr%d", k, d.in_channels, oc, oh, ow, stride, res_v ? 1 : 0, q.f16, kr16 ? 1 : 0);
         int cached[3] = {0, 0, 0};
         if (getenv("FYNHIP_D16_BLOCKS")) {
             pick = always;
@@ -1322,7 +1327,7 @@ class ConvLayer : public Layer {
             float t_new = 1e30f, t_other = 1e30f;
             int best_blocks = 1;
             for (int rep = 0; rep < 3; rep++) {
-                for (int blocks = 1; blocks <= 4 && 4 * blocks <= std::max(4, q.mfrags); blocks *= 2) {
+                for (int blocks = min_blocks; blocks <= 4 && 4 * blocks <= std::max(4 * min_blocks, q.mfrags); blocks *= 2) {
                     ConvP16Params c = q;
                     c.cout_blocks = blocks;
                     const float t = time_calls(net, [&]() {
@@ -1346,7 +1351,7 @@ class ConvLayer : public Layer {
                     t_other = std::min(t_other, time_launch(net, launch, 10));
             }
             if (getenv("FYNHIP_TUNE_VERBOSE"))
-                fprintf(stderr, "[tune] 1x1 on %d channels, %dx%d positions, to %d: LDS-free form (%d %s per 16 positions) %.1f us, %s %.1f us\n", d.in_channels, oh, ow,
+                fprintf(stderr, "[tune] %dx%d on %d channels, %dx%d positions, to %d: LDS-free form (%d %s per 16 positions) %.1f us, %s %.1f us\n", k, k, d.in_channels, oh, ow,
                         oc, best_blocks < 0 ? 1 : best_blocks, best_blocks < 0 ? "wave per fragment" : "workgroup(s)", t_new * 1e3f, kr16 ? "K-resident form" : "general kernel", t_other * 1e3f);
             pick = t_new < t_other || always;
             q.cout_blocks = best_blocks;
@@ -1363,7 +1368,35 @@ class ConvLayer : public Layer {
         }
     }
     // weights of that form: [cout fragment][chunk][plane][lane][8 halves]
-    void pack_d16(const float* w, float wmul) { pack_frag16(pp, p16_wpack_dev, w, wmul); }
+    void pack_d16(const float* w, float wmul) {
+        if (pp.tile_h) pack_taps16(w, wmul);
+        else pack_frag16(pp, p16_wpack_dev, w, wmul);
+    }
+    // the K x K form on four-channel pixels: [cout fragment][step][plane][lane][8 halves], a lane's eight values being
+    // the four channels of taps 8*step + 2*(lane/16) and the next one, in row-major order
+    void pack_taps16(const float* w, float wmul) {
+        const int cin = d.in_channels, npl = pp.f16 ? 1 : 2;
+        std::vector<uint16_t> pack((size_t)pp.mfrags * pp.cin_chunks * npl * 64 * 8, 0);
+        for (int mf = 0; mf < pp.mfrags; mf++)
+            for (int c = 0; c < pp.cin_chunks; c++) {
+                uint16_t* base = pack.data() + ((size_t)(mf * pp.cin_chunks + c) * npl) * 64 * 8;
+                for (int lane = 0; lane < 64; lane++) {
+                    const int o = mf * 16 + (lane & 15);
+                    if (o >= oc) continue;
+                    for (int j = 0; j < 8; j++) {
+                        const int tap = c * 8 + 2 * (lane >> 4) + j / 4, ci = j % 4;
+                        if (tap >= k * k || ci >= cin) continue;
+                        const float v = w[((size_t)o * k * k + tap) * cin + ci] * wmul;
+                        const uint16_t hi = f2h_bits(v);
+                        base[(size_t)lane * 8 + j] = hi;
+                        if (npl == 2) base[(size_t)(64 + lane) * 8 + j] = f2h_bits(v - h2f(hi));
+                    }
+                }
+            }
+        FYN_HIP(hipStreamSynchronize(net->stream));
+        FYN_HIP(hipMemcpyAsync(p16_wpack_dev, pack.data(), pack.size() * 2, hipMemcpyHostToDevice, net->stream));
+        FYN_HIP(hipStreamSynchronize(net->stream));
+    }
     void pack_frag16(const ConvP16Params& q, void* dev, const float* w, float wmul) {
         const int cin = d.in_channels, npl = q.f16 ? 1 : 2;
         std::vector<uint16_t> pack((size_t)q.mfrags * q.cin_chunks * npl * 64 * 8, 0);
@@ -1695,6 +1728,11 @@ class ConvLayer : public Layer {
                 !getenv("FYNHIP_NO_P16_CONV") && !getenv("FYNHIP_NO_D16_CONV") && !getenv("FYNHIP_FORCE_P16_CONV") && !getenv("FYNHIP_FORCE_KR16_CONV") &&
                 !getenv("FYNHIP_FORCE_KSPLIT") && !getenv("FYNHIP_CONV_TILE") && !getenv("FYNHIP_CONV_KC") && !getenv("FYNHIP_CONV_KC_MAX") && !getenv("FYNHIP_CONV_PD"))
                 setup_d16(in_v, out_v, res_v, res_relu, res_scale);
+            // the same kernel's K x K form for a first layer on at most four channels (3x3, 5x5, 7x7)
+            if (!p16 && !frac_shift && !clamp && same_storage && oc % 4 == 0 && oc >= 8 && oh * ow >= 256 && conv_d16_small_supported(k, dil, in_v.cp, oc, out_v.cp) &&
+                (!res_v || (res_v->cp >= out_v.cp && res_v->cp % 8 == 0)) && !getenv("FYNHIP_NO_P16_CONV") && !getenv("FYNHIP_NO_D16_CONV") && !getenv("FYNHIP_FORCE_P16_CONV") &&
+                !getenv("FYNHIP_FORCE_KSPLIT") && !getenv("FYNHIP_CONV_TILE") && !getenv("FYNHIP_CONV_KC") && !getenv("FYNHIP_CONV_KC_MAX") && !getenv("FYNHIP_CONV_PD"))
+                setup_d16(in_v, out_v, res_v, res_relu, res_scale);
         }
         if (direct) {
             scale_dev = static_cast<float*>(net->dev_alloc(padded * sizeof(float)));
@@ -1830,9 +1868,9 @@ class ConvLayer : public Layer {
             return mode + buf;
         }
         if (p16 && d16) {
-            char buf[220];
-            snprintf(buf, sizeof(buf), "conv_d16 %s 1x1 without LDS: %s, %d chunks in registers, %d fragments of 16 output channels, blocks=%d",
-                     pp.f16 ? "f16" : "f16x2-split", (pp.wm == 4 ? "a wave per 16 positions and fragment" : (std::to_string(pp.cout_blocks) + " workgroup(s) of 4 waves per 16 positions").c_str()),
+            char buf[360];
+            snprintf(buf, sizeof(buf), "conv_d16 %s %s without LDS: %s, %d chunks in registers, %d fragments of 16 output channels, blocks=%d",
+                     pp.f16 ? "f16" : "f16x2-split", (pp.tile_h ? "KxK on four-channel pixels (steps of eight taps)" : "1x1"), (pp.wm == 4 ? "a wave per 16 positions and fragment" : (std::to_string(pp.cout_blocks) + " workgroup(s) of 4 waves per 16 positions").c_str()),
                      pp.cin_chunks, pp.mfrags, (pp.npos_y * pp.npos_x + 16 * pp.wm - 1) / (16 * pp.wm) * pp.cout_blocks);
             if (dw_fused) return mode + buf + "; the depthwise 3x3 layer " + std::to_string(dw_layer_no) + " in front of it is computed by the waves themselves";
             return mode + buf;

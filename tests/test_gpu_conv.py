@@ -516,6 +516,44 @@ def test_pointwise_without_lds(case, variant, storage, monkeypatch):
     assert err <= TOL[storage], info
 
 
+SMALL_INPUT_CASES = [
+    # (k, cin, cout, h, w, stride, kw)
+    (3, 3, 32, 224, 224, 2, {"bn": True}),                      # the first layer of the MobileNetV2-style stack
+    (7, 3, 64, 64, 72, 2, {"bn": True}),                        # a ResNet stem, reduced
+    (5, 4, 24, 40, 36, 1, {"pad_out": 1}),                      # four channels, 24 output channels
+    (3, 1, 16, 33, 47, 1, {"residual": (A.RELU, True)}),        # one channel, odd size, residual
+    (7, 2, 40, 50, 50, 1, {"bn": True, "blocks": -3}),          # a wave per 16 positions and fragment
+    (3, 3, 96, 40, 40, 2, {"blocks": 2}),                       # six fragments on two workgroups per tile
+]
+
+
+@pytest.mark.parametrize("storage", [fa.STORAGE_F32, fa.STORAGE_F16], ids=["f32", "f16"])
+@pytest.mark.parametrize("act", [A.NONE, A.LEAKY_RELU], ids=["linear", "leaky"])
+@pytest.mark.parametrize("case", SMALL_INPUT_CASES, ids=lambda c: "k%d_%dx%dx%d_to%d_s%d" % (c[0], c[1], c[3], c[4], c[2], c[5]))
+def test_small_input_convolution_without_lds(case, act, storage, monkeypatch):
+    """K x K convolutions (3, 5, 7) on at most four input channels whose B fragments are gathered from the image, two
+    taps of four channels per lane and step."""
+    k, cin, cout, h, w, stride, kw = case
+    monkeypatch.setenv("FYNHIP_FORCE_D16_CONV", "1")
+    kw = dict(kw)
+    blocks = kw.pop("blocks", None)
+    if blocks:
+        monkeypatch.setenv("FYNHIP_D16_BLOCKS", str(blocks))
+    if act is A.LEAKY_RELU:
+        kw["leak"] = 0.1
+    b = conv_builder(k, cout, h, w, cin, stride, 1, act, **kw)
+    wts = conv_block(6000 + k * cin + cout, cout, k, cin, bn=kw.get("bn", False))
+    inputs = [prng.uniform(47 * cin + h, (cin, h, w), -1, 1)]
+    if "residual" in kw:
+        inputs.append(prng.uniform(73, (cout, h // stride, w // stride), -1, 1))
+    got, info = run_single(b, storage, inputs, wts)
+    ref = oracle_single(b, storage, inputs, wts)
+    err = rel_l2(got, ref)
+    print("  ", info, "rel_l2=%.3e" % err, flush=True)
+    assert "conv_d16" in info and "KxK" in info
+    assert err <= TOL[storage], info
+
+
 ALL_TILES = ["2,2,2,2", "2,2,1,4", "2,1,2,2", "2,1,1,4", "1,2,1,4", "1,1,1,4", "1,1,4,1", "1,1,2,2", "1,2,4,1", "1,3,4,1", "1,4,4,1",
              "1,2,2,2", "1,4,2,2", "1,3,2,2", "1,4,1,4", "1,3,1,4", "1,1,1,1", "1,1,2,1", "1,1,1,2"]
 
