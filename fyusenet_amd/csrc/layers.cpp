@@ -1705,7 +1705,9 @@ class ConvLayer : public Layer {
             // the 16-position-fragment forms, each against the tuned launch of the general kernel: for wide fp16 layers the
             // one with 64-channel wave tiles first, then the 3x3 form, then the small-input form
             const bool same_storage = in_v.f16 == out_v.f16 && (!res_v || res_v->f16 == out_v.f16);
-            const bool only_kr = getenv("FYNHIP_FORCE_KR16_CONV") != nullptr;   // (tests: the K-resident form or nothing)
+            // (tests: the K-resident form or nothing; a forced variant of the general kernel means the general kernel)
+            const bool only_kr = getenv("FYNHIP_FORCE_KR16_CONV") || getenv("FYNHIP_FORCE_KSPLIT") || getenv("FYNHIP_CONV_TILE") || getenv("FYNHIP_CONV_KC") ||
+                                 getenv("FYNHIP_CONV_KC_MAX") || getenv("FYNHIP_CONV_PD");
             if (!only_kr && !frac_shift && same_storage && conv_h16_supported(k, stride, dil, in_v.cp, oc, out_v.cp, out_v.f16 != 0) && d.in_channels == in_v.cp &&
                 (!res_v || res_v->cp >= oc) && !getenv("FYNHIP_NO_P16_CONV") && !getenv("FYNHIP_NO_H16_CONV"))
                 setup_h16(in_v, out_v, res_v, res_relu, res_scale);

@@ -820,6 +820,8 @@ def test_tuning_choices_are_remembered_across_processes(tmp_path):
     import os
     import subprocess
     import sys
+    if os.environ.get("FYNHIP_AUTOTUNE", "").startswith("0"):
+        pytest.skip("nothing is measured with FYNHIP_AUTOTUNE=0")
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     cache = tmp_path / "tune.txt"
     env = dict(os.environ, FYNHIP_TUNE_CACHE=str(cache))
