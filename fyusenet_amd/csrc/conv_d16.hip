@@ -28,6 +28,17 @@ namespace fynhip {
 namespace {
 typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
 
+// An activation that is exact on halves -- none, or a clamp without leak whose bounds are fp16 values -- is applied to
+// the packed halves (two values per instruction, no conversions): act_half_exact says whether, act_half applies it.
+__device__ __forceinline__ bool act_half_exact(const Act& a, _Float16& lo, _Float16& hi) {
+    lo = (_Float16)fmaxf(a.lo, -65504.f);
+    hi = (_Float16)fminf(a.hi, 65504.f);
+    return a.leak == 0.f && (a.lo < -65504.f || (float)lo == a.lo) && (a.hi > 65504.f || (float)hi == a.hi);
+}
+__device__ __forceinline__ half8_t act_half(half8_t v, _Float16 lo, _Float16 hi) {
+    return __builtin_elementwise_min(__builtin_elementwise_max(v, (half8_t)lo), (half8_t)hi);
+}
+
 // DWS = 1 or 2: the layer's input is the output of a depthwise 3x3 layer with step DWS that is not read from memory but
 // computed by every wave for its positions (nine texels of the depthwise layer's input per lane and chunk instead of
 // one of its output; that layer's own arithmetic and rounding), as in conv_kr16_kernel's staging.
@@ -168,7 +179,11 @@ __global__ __launch_bounds__(256) void conv_d16_kernel(const ConvP16Params p) {
             x[0] = rw.a.x; x[1] = rw.a.y; x[2] = rw.a.z; x[3] = rw.a.w; x[4] = rw.b.x; x[5] = rw.b.y; x[6] = rw.b.z; x[7] = rw.b.w;
         }
     };
+    _Float16 act_lo, act_hi;
+    const bool half_act = HS && act_half_exact(p.act, act_lo, act_hi);
     half8_t b[NCHK][NPL];
+    auto convert = [&](auto kind_) {
+    constexpr int KIND = decltype(kind_)::value;   // (the activation's kind, chosen once per wave: act_kind)
 #pragma unroll
     for (int c = 0; c < NCHK; c++) {
         const bool okc = KS > 0 || c * KC + kq * 8 < p.in_cp;
@@ -198,17 +213,20 @@ __global__ __launch_bounds__(256) void conv_d16_kernel(const ConvP16Params p) {
             texel(raw[c][0], r);
         }
         if constexpr (HS) {
+            if (DWS == 0 && half_act) {
+                b[c][0] = okc ? act_half(raw[c][0], act_lo, act_hi) : (half8_t)((_Float16)0.f);
+            } else {
 #pragma unroll
-            for (int e = 0; e < 8; e++) b[c][0][e] = okc ? (_Float16)act_p16(r[e], p.act) : (_Float16)0.f;
-        } else {
-#pragma unroll
-            for (int e = 0; e < 8; e++) {
-                const float v = okc ? act_p16(r[e], p.act) * in_scale : 0.f;
-                b[c][0][e] = (_Float16)v;
-                b[c][NPL - 1][e] = (_Float16)(v - (float)b[c][0][e]);
+                for (int e = 0; e < 8; e++) b[c][0][e] = okc ? (_Float16)act_p16(r[e], p.act) : (_Float16)0.f;
             }
+        } else {
+            split8<KIND>(r, okc, p.act, in_scale, b[c][0], b[c][NPL - 1]);
         }
     }
+    };
+    if (HS || p.act.kind == ACT_LEAKY || p.act.kind == ACT_CLIP) convert(std::integral_constant<int, ACT_LEAKY>());
+    else if (p.act.kind == ACT_RELU) convert(std::integral_constant<int, ACT_RELU>());
+    else convert(std::integral_constant<int, ACT_NONE>());
     store_t* out = reinterpret_cast<store_t*>(p.out);
     float vmax = 0.f;
     auto fragment = [&](int f, const half8_t (&a)[NCHK][NPL], const res_t& rcur, const f32x4_t& sc, const f32x4_t& bi) {
@@ -377,6 +395,10 @@ __global__ __launch_bounds__(256) void conv_e16dw_kernel(const ConvP16Params p) 
     float in_scale = 1.f, inv_in_scale = 1.f;
     if (p.in_amax) in_scale = range_scale(range_after_act(range_reduce(range_bits), p.act), &inv_in_scale);
     const float acc_mul = p.acc_mul * inv_in_scale;
+    _Float16 act_lo, act_hi;
+    const bool half_act = HS && act_half_exact(p.act, act_lo, act_hi);
+    auto window = [&](auto kind_) {
+    constexpr int KIND = decltype(kind_)::value;   // (the 1x1 layer's activation kind, chosen once per wave: act_kind)
 #pragma unroll
     for (int pf = 0; pf < NPF; pf++) {
         f32x4_t acc = (f32x4_t)(0.f);
@@ -385,16 +407,15 @@ __global__ __launch_bounds__(256) void conv_e16dw_kernel(const ConvP16Params p) 
             const bool okc = c * KC + kq * 8 < p.in_cp;
             half8_t b[NPL];
             if constexpr (HS) {
+                if (half_act) {
+                    b[0] = okc ? act_half(raw[pf][c], act_lo, act_hi) : (half8_t)((_Float16)0.f);
+                } else {
 #pragma unroll
-                for (int e = 0; e < 8; e++) b[0][e] = okc ? (_Float16)act_p16((float)raw[pf][c][e], p.act) : (_Float16)0.f;
+                    for (int e = 0; e < 8; e++) b[0][e] = okc ? (_Float16)act_p16((float)raw[pf][c][e], p.act) : (_Float16)0.f;
+                }
             } else {
                 const float r[8] = {raw[pf][c].a.x, raw[pf][c].a.y, raw[pf][c].a.z, raw[pf][c].a.w, raw[pf][c].b.x, raw[pf][c].b.y, raw[pf][c].b.z, raw[pf][c].b.w};
-#pragma unroll
-                for (int e = 0; e < 8; e++) {
-                    const float v = okc ? act_p16(r[e], p.act) * in_scale : 0.f;
-                    b[0][e] = (_Float16)v;
-                    b[NPL - 1][e] = (_Float16)(v - (float)b[0][e]);
-                }
+                split8<KIND>(r, okc, p.act, in_scale, b[0], b[NPL - 1]);
             }
 #pragma unroll
             for (int i = 0; i < NPASS; i++) {
@@ -413,6 +434,10 @@ __global__ __launch_bounds__(256) void conv_e16dw_kernel(const ConvP16Params p) 
         }
         if (wp_ < NWIN) *reinterpret_cast<f32x4_t*>(&win[wp_][w * 16 + kq * 4]) = v;
     }
+    };
+    if (HS || p.act.kind == ACT_LEAKY || p.act.kind == ACT_CLIP) window(std::integral_constant<int, ACT_LEAKY>());
+    else if (p.act.kind == ACT_RELU) window(std::integral_constant<int, ACT_RELU>());
+    else window(std::integral_constant<int, ACT_NONE>());
     __syncthreads();
     // ---- depthwise 3x3 on the window: one position, four channels per thread (ky outer, kx inner, fused multiply-add) ----
     const int py = dpos >> 2, px = dpos & 3;

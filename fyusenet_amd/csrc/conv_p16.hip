@@ -1132,26 +1132,40 @@ __global__ __launch_bounds__(512) void conv_kr16_kernel(const ConvP16Params p) {
             reinterpret_cast<float*>(lds + sb_off)[stid] = p.scale[cb * 16 * FM + stid];
             reinterpret_cast<float*>(lds + sb_off)[16 * FM + stid] = p.bias[cb * 16 * FM + stid];
         }
+        // (fp16 tensors: no activation, or a clamp without leak whose bounds are fp16 values, is applied to the packed
+        // halves -- two values per instruction, no conversions)
+        const _Float16 hlo = (_Float16)fmaxf(p.act.lo, -65504.f), hhi = (_Float16)fminf(p.act.hi, 65504.f);
+        const bool half_act = HSTORE && p.act.leak == 0.f && (p.act.lo < -65504.f || (float)hlo == p.act.lo) && (p.act.hi > 65504.f || (float)hhi == p.act.hi);
 #pragma unroll
         for (int i = 0; i < G::NB; i++) {
             if (l_off[i] < 0) continue;
             if constexpr (HSTORE) {
                 half8_t v;
+                if (half_act) {
+                    v = ok[i] ? __builtin_elementwise_min(__builtin_elementwise_max(raw[i], (half8_t)hlo), (half8_t)hhi) : (half8_t)((_Float16)0.f);
+                } else {
 #pragma unroll
-                for (int e = 0; e < 8; e++) v[e] = ok[i] ? (_Float16)act_p16((float)raw[i][e], p.act) : (_Float16)0.f;
-                *reinterpret_cast<half8_t*>(lds + l_off[i]) = v;
-            } else {
-                const float r[8] = {raw[i].a.x, raw[i].a.y, raw[i].a.z, raw[i].a.w, raw[i].b.x, raw[i].b.y, raw[i].b.z, raw[i].b.w};
-                half8_t hi, lo;
-#pragma unroll
-                for (int e = 0; e < 8; e++) {
-                    const float v = ok[i] ? act_p16(r[e], p.act) * in_scale : 0.f;
-                    hi[e] = (_Float16)v;
-                    lo[e] = (_Float16)(v - (float)hi[e]);
+                    for (int e = 0; e < 8; e++) v[e] = ok[i] ? (_Float16)act_p16((float)raw[i][e], p.act) : (_Float16)0.f;
                 }
-                *reinterpret_cast<half8_t*>(lds + l_off[i]) = hi;
-                *reinterpret_cast<half8_t*>(lds + G::PLANE + l_off[i]) = lo;
+                *reinterpret_cast<half8_t*>(lds + l_off[i]) = v;
             }
+        }
+        if constexpr (!HSTORE) {
+            auto split_all = [&](auto kind_) {
+                constexpr int KIND = decltype(kind_)::value;
+#pragma unroll
+                for (int i = 0; i < G::NB; i++) {
+                    if (l_off[i] < 0) continue;
+                    const float r[8] = {raw[i].a.x, raw[i].a.y, raw[i].a.z, raw[i].a.w, raw[i].b.x, raw[i].b.y, raw[i].b.z, raw[i].b.w};
+                    half8_t hi, lo;
+                    split8<KIND>(r, ok[i], p.act, in_scale, hi, lo);
+                    *reinterpret_cast<half8_t*>(lds + l_off[i]) = hi;
+                    *reinterpret_cast<half8_t*>(lds + G::PLANE + l_off[i]) = lo;
+                }
+            };
+            if (p.act.kind == ACT_NONE) split_all(std::integral_constant<int, ACT_NONE>());
+            else if (p.act.kind == ACT_RELU) split_all(std::integral_constant<int, ACT_RELU>());
+            else split_all(std::integral_constant<int, ACT_LEAKY>());
         }
         lds_barrier();   // the tile is staged
         lds_barrier();   // the MFMA waves have left their accumulators for wave 0

@@ -14,6 +14,54 @@ typedef float f32x4_t __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 __device__ __forceinline__ float act_p16(float x, const Act& a) { return __builtin_amdgcn_fmed3f(x, a.lo, a.hi) + a.leak * fminf(x, 0.f); }
+// The same with the kind known (a wave-uniform choice made outside the loop over a lane's values): nothing for ACT_NONE,
+// one instruction for ACT_RELU, the general three otherwise.  Where a wave runs alone on its SIMD every vector
+// instruction costs four cycles, and a staging thread converts dozens of values.
+template <int KIND>
+__device__ __forceinline__ float act_kind(float x, const Act& a) {
+    if constexpr (KIND == ACT_NONE) return x;
+    else if constexpr (KIND == ACT_RELU) return fmaxf(x, 0.f);
+    else return act_p16(x, a);
+}
+
+// The fp16 hi/lo split of eight fp32 values of a staging item, scaled by the power of two s: hi = f16(s*x),
+// lo = f16(s*x - hi), as packed halves.  Four instructions per pair of values: the mixed-precision multiply-adds take
+// the fp32 value, the scale and (for lo) the half just written as their operands and round once, which is what the
+// plain expression gives as well (s*x is exact); the compiler's own selection for that expression computes hi twice
+// and needs eleven instructions per pair.  `ok` false: zeros.  KIND as for act_kind; ACT_NONE and ACT_RELU are clamps
+// to +-3e38 and [0, 3e38] (one instruction, and the bounds collapse to 0 for an item outside the tensor).
+__device__ __forceinline__ void split_pair(float x0, float x1, float s, unsigned& H, unsigned& L) {
+    asm volatile(
+        "v_fma_mixlo_f16 %0, %2, %3, 0\n\t"
+        "v_fma_mixhi_f16 %0, %2, %4, 0\n\t"
+        "v_fma_mixlo_f16 %1, %2, %3, -%0 op_sel_hi:[0,0,1]\n\t"
+        "v_fma_mixhi_f16 %1, %2, %4, -%0 op_sel:[0,0,1] op_sel_hi:[0,0,1]"
+        : "=&v"(H), "=&v"(L)
+        : "v"(s), "v"(x0), "v"(x1));
+}
+template <int KIND>
+__device__ __forceinline__ void split8(const float (&r)[8], bool ok, const Act& a, float s, half8_t& hi, half8_t& lo) {
+    typedef unsigned u32x4_t __attribute__((ext_vector_type(4)));
+    float x[8];
+    if constexpr (KIND == ACT_NONE || KIND == ACT_RELU) {
+        const float top = ok ? 3.0e38f : 0.f, bottom = (KIND == ACT_RELU || !ok) ? 0.f : -3.0e38f;
+#pragma unroll
+        for (int e = 0; e < 8; e++) x[e] = __builtin_amdgcn_fmed3f(r[e], bottom, top);
+    } else {
+#pragma unroll
+        for (int e = 0; e < 8; e++) x[e] = ok ? act_p16(r[e], a) : 0.f;
+    }
+    u32x4_t H, L;
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+        unsigned h, l;
+        split_pair(x[2 * e], x[2 * e + 1], s, h, l);
+        H[e] = h;
+        L[e] = l;
+    }
+    hi = __builtin_bit_cast(half8_t, H);
+    lo = __builtin_bit_cast(half8_t, L);
+}
 
 constexpr int KC = 32;        // input channels per chunk
 constexpr int PITCH = KC * 2 + 16;   // bytes per staged pixel and plane: 8 neighbouring lanes' 16-byte reads cover all banks
