@@ -1104,6 +1104,38 @@ __global__ __launch_bounds__(512) void conv_kr16_kernel(const ConvP16Params p) {
         // (a 3x3 layer with stride 2 stages every pixel under its tile: position (y, x) reads the window at (2y, 2x))
         const int st = NTAPS == 1 ? p.stride : 1, org = NTAPS == 1 ? p.stride : S;
         const int y0 = tyi * G::TH * org + p.in_y0, x0 = txi * G::TW * org + p.in_x0;
+        if constexpr (256 % G::NITEMS == 0) {
+            // A chunk's items divide the 256 staging threads (1x1 layers): a thread keeps its pixel and its 8 channels
+            // of the chunk for all its items and only the chunk advances, by CPI per item -- the pixel's arithmetic is
+            // done once, not once per item (a thread has up to 16 items, and nothing is requested before it is through).
+            constexpr int CPI = 256 / G::NITEMS;
+            const int chunk0 = stid / G::NITEMS, rem = stid - chunk0 * G::NITEMS;
+            const int pix = rem >> 2, g = rem & 3;
+            const int py = pix / G::HW, px = pix - py * G::HW;
+            int gy = y0 + py * st, gx = x0 + px * st;
+            if (p.in_clamp) {
+                gy = min(max(gy, 0), p.in_hp - 1);
+                gx = min(max(gx, 0), p.in_wp - 1);
+            }
+            const bool inb = (unsigned)gy < (unsigned)p.in_hp && (unsigned)gx < (unsigned)p.in_wp;
+            const int l0 = chunk0 * G::BUFC + py * G::ROW_PITCH + px * G::PIT + g * 16;
+            const int c0 = chunk0 * KC + g * 8;
+            const store_t* src0 = in + (inb ? (gy * p.in_wp + gx) * p.in_cp : 0) + c0;
+#pragma unroll
+            for (int i = 0; i < G::NB; i++) {
+                const bool in_tile = chunk0 + i * CPI < G::NCH;
+                l_off[i] = in_tile ? l0 + i * CPI * G::BUFC : -1;
+                // (channels behind the tensor's pitch -- the chunk count is rounded up to four per wave -- read as zero)
+                ok[i] = in_tile && inb && c0 + i * CPI * KC < p.in_cp;
+                const store_t* src = ok[i] ? src0 + i * CPI * KC : in;
+                if constexpr (HSTORE) {
+                    raw[i] = *reinterpret_cast<const half8_t*>(src);
+                } else {
+                    raw[i].a = *reinterpret_cast<const float4*>(src);
+                    raw[i].b = *reinterpret_cast<const float4*>(src + 4);
+                }
+            }
+        } else {
 #pragma unroll
         for (int i = 0; i < G::NB; i++) {
             const int idx = stid + i * 256;
@@ -1125,6 +1157,7 @@ __global__ __launch_bounds__(512) void conv_kr16_kernel(const ConvP16Params p) {
                 raw[i].a = *reinterpret_cast<const float4*>(src);
                 raw[i].b = *reinterpret_cast<const float4*>(src + 4);
             }
+        }
         }
         float in_scale = 1.f, inv_unused;
         if (p.in_amax) in_scale = range_scale(range_after_act(range_reduce(range_bits), p.act), &inv_unused);
