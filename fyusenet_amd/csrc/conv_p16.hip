@@ -188,30 +188,37 @@ __device__ __forceinline__ void p16_stager(const ConvP16Params& p, unsigned char
             }
         }
     };
+    const int act_kind_ = p.act.kind;
     auto store = [&](auto set_, unsigned char* buf) {
         constexpr int SET = decltype(set_)::value;
+        if constexpr (HSTORE) {
 #pragma unroll
-        for (int i = 0; i < G::NB; i++) {
-            if (l_off[i] < 0) continue;
-            const bool ok = g_off[SET][i] >= 0;
-            if constexpr (HSTORE) {
+            for (int i = 0; i < G::NB; i++) {
+                if (l_off[i] < 0) continue;
+                const bool ok = g_off[SET][i] >= 0;
                 half8_t v;
 #pragma unroll
                 for (int e = 0; e < 8; e++) v[e] = ok ? (_Float16)act_p16((float)raw[SET][i][e], p.act) : (_Float16)0.f;
                 *reinterpret_cast<half8_t*>(buf + l_off[i]) = v;
-            } else {
-                const float4 r0 = raw[SET][i].a, r1 = raw[SET][i].b;
-                const float r[8] = {r0.x, r0.y, r0.z, r0.w, r1.x, r1.y, r1.z, r1.w};
-                half8_t hi, lo;
-#pragma unroll
-                for (int e = 0; e < 8; e++) {
-                    const float v = ok ? act_p16(r[e], p.act) * in_scale : 0.f;
-                    hi[e] = (_Float16)v;
-                    lo[e] = (_Float16)(v - (float)hi[e]);
-                }
-                *reinterpret_cast<half8_t*>(buf + l_off[i]) = hi;
-                *reinterpret_cast<half8_t*>(buf + G::PLANE + l_off[i]) = lo;
             }
+        } else {
+            // (the activation's kind chosen once per call, the hi/lo split in four instructions per pair: split8)
+            auto split_all = [&](auto kind_) {
+                constexpr int KIND = decltype(kind_)::value;
+#pragma unroll
+                for (int i = 0; i < G::NB; i++) {
+                    if (l_off[i] < 0) continue;
+                    const float4 r0 = raw[SET][i].a, r1 = raw[SET][i].b;
+                    const float r[8] = {r0.x, r0.y, r0.z, r0.w, r1.x, r1.y, r1.z, r1.w};
+                    half8_t hi, lo;
+                    split8<KIND>(r, g_off[SET][i] >= 0, p.act, in_scale, hi, lo);
+                    *reinterpret_cast<half8_t*>(buf + l_off[i]) = hi;
+                    *reinterpret_cast<half8_t*>(buf + G::PLANE + l_off[i]) = lo;
+                }
+            };
+            if (act_kind_ == ACT_RELU) split_all(std::integral_constant<int, ACT_RELU>());
+            else if (act_kind_ == ACT_NONE) split_all(std::integral_constant<int, ACT_NONE>());
+            else split_all(std::integral_constant<int, ACT_LEAKY>());
         }
     };
     auto residual_in = [&](int tile) {   // the residual tile of a tile: [position][CPB channels] as stored, in 16-byte pieces
