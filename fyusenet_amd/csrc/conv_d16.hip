@@ -467,14 +467,135 @@ __global__ __launch_bounds__(256) void conv_e16dw_kernel(const ConvP16Params p) 
     }
 }
 
+
+// The same with a workgroup per 16 expanded channels (p.wm = 2; grid rows = fragments): for layers with few tiles, where
+// blocks of 64 channels leave most of the chip idle and every wave with a long chain of fragments.  All four waves work
+// on the one fragment of channels and deal the window's position fragments among themselves (wave w takes w, w + 4);
+// behind the barrier a thread computes one channel of one output position.
+template <bool HS, int NCHK, int DWS>
+__global__ __launch_bounds__(256) void conv_e16dw_narrow_kernel(const ConvP16Params p) {
+    constexpr int NPL = HS ? 1 : 2, NPASS = HS ? 1 : 3;
+    constexpr int WIN = 3 * DWS + 3, NWIN = WIN * WIN, NPF = (NWIN + 15) / 16, PFW = (NPF + 3) / 4;
+    typedef typename std::conditional<HS, _Float16, float>::type store_t;
+    __shared__ __align__(16) float win[NWIN][20];   // (20: the sixteen positions of a fragment write distinct banks)
+    if (blockIdx.x == 0 && blockIdx.y == 0) range_clear(p.reset[0], p.reset[1], p.reset[2], p.reset[3], p.nreset);
+    const int lane = threadIdx.x & 63;
+    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int mq = lane & 15, kq = lane >> 4;
+    const unsigned range_bits = p.in_amax ? range_load(p.in_amax) : 0u;
+    const int tyi = blockIdx.x / p.tiles_x, txi = blockIdx.x - tyi * p.tiles_x;
+    const int ey0 = tyi * 4 * DWS - 1, ex0 = txi * 4 * DWS - 1;
+    const int mf = blockIdx.y;
+    // depthwise phase operands (requested first: they are used last)
+    const int t = threadIdx.x;
+    const int dpos = t >> 4, dch = mf * 16 + (t & 15);
+    const bool dch_ok = dch < p.dw_cp;
+    float dww[9];
+#pragma unroll
+    for (int i = 0; i < 9; i++) dww[i] = p.dw_w[i * p.dw_cp + (dch_ok ? dch : 0)];
+    const float dsc = p.dw_scale[dch_ok ? dch : 0], dbi = p.dw_bias[dch_ok ? dch : 0];
+    // this wave's position fragments of the window
+    struct RawF { float4 a, b; };
+    typedef typename std::conditional<HS, half8_t, RawF>::type raw_t;
+    raw_t raw[PFW][NCHK];
+    bool inside[PFW];
+#pragma unroll
+    for (int j = 0; j < PFW; j++) {
+        const int pf = w + 4 * j;
+        const int wp_ = min(pf * 16 + mq, NWIN - 1);
+        const int ey = ey0 + wp_ / WIN, ex = ex0 + wp_ % WIN;
+        inside[j] = (unsigned)ey < (unsigned)p.dw_hp && (unsigned)ex < (unsigned)p.dw_wp;
+        const int cy = min(max(ey, 0), p.dw_hp - 1), cx = min(max(ex, 0), p.dw_wp - 1);
+        const store_t* in = reinterpret_cast<const store_t*>(p.in) + ((size_t)(cy + p.in_y0) * p.in_wp + cx + p.in_x0) * p.in_cp + kq * 8;
+#pragma unroll
+        for (int c = 0; c < NCHK; c++) {
+            const bool okc = c * KC + kq * 8 < p.in_cp;
+            const store_t* src = okc ? in + c * KC : reinterpret_cast<const store_t*>(p.in);
+            if constexpr (HS) {
+                raw[j][c] = *reinterpret_cast<const half8_t*>(src);
+            } else {
+                raw[j][c].a = *reinterpret_cast<const float4*>(src);
+                raw[j][c].b = *reinterpret_cast<const float4*>(src + 4);
+            }
+        }
+    }
+    half8_t a[NCHK][NPL];
+    const unsigned char* wbase = reinterpret_cast<const unsigned char*>(p.wpack) + (size_t)mf * (NCHK * NPL * 1024) + lane * 16;
+#pragma unroll
+    for (int c = 0; c < NCHK; c++)
+#pragma unroll
+        for (int pl = 0; pl < NPL; pl++) a[c][pl] = *reinterpret_cast<const half8_t*>(wbase + (c * NPL + pl) * 1024);
+    const f32x4_t sc = *reinterpret_cast<const f32x4_t*>(p.scale + mf * 16 + kq * 4);
+    const f32x4_t bi = *reinterpret_cast<const f32x4_t*>(p.bias + mf * 16 + kq * 4);
+    float in_scale = 1.f, inv_in_scale = 1.f;
+    if (p.in_amax) in_scale = range_scale(range_after_act(range_reduce(range_bits), p.act), &inv_in_scale);
+    const float acc_mul = p.acc_mul * inv_in_scale;
+    _Float16 act_lo, act_hi;
+    const bool half_act = HS && act_half_exact(p.act, act_lo, act_hi);
+    auto window = [&](auto kind_) {
+    constexpr int KIND = decltype(kind_)::value;
+#pragma unroll
+    for (int j = 0; j < PFW; j++) {
+        const int pf = w + 4 * j;
+        if (pf >= NPF) continue;
+        f32x4_t acc = (f32x4_t)(0.f);
+#pragma unroll
+        for (int c = 0; c < NCHK; c++) {
+            const bool okc = c * KC + kq * 8 < p.in_cp;
+            half8_t b[NPL];
+            if constexpr (HS) {
+                if (half_act) {
+                    b[0] = okc ? act_half(raw[j][c], act_lo, act_hi) : (half8_t)((_Float16)0.f);
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 8; e++) b[0][e] = okc ? (_Float16)act_p16((float)raw[j][c][e], p.act) : (_Float16)0.f;
+                }
+            } else {
+                const float r[8] = {raw[j][c].a.x, raw[j][c].a.y, raw[j][c].a.z, raw[j][c].a.w, raw[j][c].b.x, raw[j][c].b.y, raw[j][c].b.z, raw[j][c].b.w};
+                split8<KIND>(r, okc, p.act, in_scale, b[0], b[NPL - 1]);
+            }
+#pragma unroll
+            for (int i = 0; i < NPASS; i++) {
+                const int apl = (i == 1) ? 1 : 0, bpl = (i == 2) ? 1 : 0;
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[c][apl], b[bpl], acc, 0, 0, 0);
+            }
+        }
+        const int wp_ = pf * 16 + mq;
+        f32x4_t v;
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            float x = acc[e] * (sc[e] * acc_mul) + bi[e];
+            if constexpr (HS) x = (float)(_Float16)x;
+            v[e] = act_p16(inside[j] ? x : 0.f, p.dw_act);
+        }
+        if (wp_ < NWIN) *reinterpret_cast<f32x4_t*>(&win[wp_][kq * 4]) = v;
+    }
+    };
+    if (HS || p.act.kind == ACT_LEAKY || p.act.kind == ACT_CLIP) window(std::integral_constant<int, ACT_LEAKY>());
+    else if (p.act.kind == ACT_RELU) window(std::integral_constant<int, ACT_RELU>());
+    else window(std::integral_constant<int, ACT_NONE>());
+    __syncthreads();
+    const int py = dpos >> 2, px = dpos & 3;
+    float dacc = 0.f;
+#pragma unroll
+    for (int ky = 0; ky < 3; ky++)
+#pragma unroll
+        for (int kx = 0; kx < 3; kx++) dacc = fmaf(win[(py * DWS + ky) * WIN + px * DWS + kx][t & 15], dww[ky * 3 + kx], dacc);
+    const int oy = tyi * 4 + py, ox = txi * 4 + px;
+    if (oy < p.npos_y && ox < p.npos_x && dch_ok) {
+        store_t* out = reinterpret_cast<store_t*>(p.out) + ((size_t)(p.out_off_y + oy) * p.out_wp + p.out_off_x + ox) * p.out_cp + dch;
+        *out = (store_t)(dacc * dsc + dbi);
+    }
+}
+
 template <bool HS, int DWS>
-d16_fn pick_e16dw(int chunks) {
+d16_fn pick_e16dw(int chunks, bool narrow) {
     switch (chunks) {
-        case 1: return conv_e16dw_kernel<HS, 1, DWS>;
-        case 2: return conv_e16dw_kernel<HS, 2, DWS>;
-        case 3: return conv_e16dw_kernel<HS, 3, DWS>;
-        case 4: return conv_e16dw_kernel<HS, 4, DWS>;
-        case 5: return conv_e16dw_kernel<HS, 5, DWS>;
+        case 1: return narrow ? conv_e16dw_narrow_kernel<HS, 1, DWS> : conv_e16dw_kernel<HS, 1, DWS>;
+        case 2: return narrow ? conv_e16dw_narrow_kernel<HS, 2, DWS> : conv_e16dw_kernel<HS, 2, DWS>;
+        case 3: return narrow ? conv_e16dw_narrow_kernel<HS, 3, DWS> : conv_e16dw_kernel<HS, 3, DWS>;
+        case 4: return narrow ? conv_e16dw_narrow_kernel<HS, 4, DWS> : conv_e16dw_kernel<HS, 4, DWS>;
+        case 5: return narrow ? conv_e16dw_narrow_kernel<HS, 5, DWS> : conv_e16dw_kernel<HS, 5, DWS>;
         default: return nullptr;
     }
 }
@@ -547,18 +668,20 @@ bool conv_e16dw_supported(int in_cp, int chunks, int dw_stride) {
 
 // The 1x1 layer's parameters as for launch_conv_d16 (stride 1, no residual; wpack in that layout), dw_hp x dw_wp its
 // output size, out* / npos_* the depthwise layer's tensor, tiles_x x tiles_y tiles of 4x4 of its positions, dw_*
-// its weights [9][dw_cp], scale, bias, step and activation; dw_cp = out_cp = channels of both layers (multiple of 8)
+// its weights [9][dw_cp], scale, bias, step and activation; dw_cp = out_cp = channels of both layers (multiple of 8);
+// p.wm = 2: a workgroup per 16 expanded channels instead of 64
 int launch_conv_e16dw(const ConvP16Params& p, hipStream_t s) {
     if (!conv_e16dw_supported(p.in_cp, p.cin_chunks, p.dw_stride)) return -1;
-    const d16_fn fn = p.f16 ? (p.dw_stride == 1 ? pick_e16dw<true, 1>(p.cin_chunks) : pick_e16dw<true, 2>(p.cin_chunks))
-                            : (p.dw_stride == 1 ? pick_e16dw<false, 1>(p.cin_chunks) : pick_e16dw<false, 2>(p.cin_chunks));
+    const bool narrow = p.wm == 2;   // a workgroup per 16 expanded channels instead of 64
+    const d16_fn fn = p.f16 ? (p.dw_stride == 1 ? pick_e16dw<true, 1>(p.cin_chunks, narrow) : pick_e16dw<true, 2>(p.cin_chunks, narrow))
+                            : (p.dw_stride == 1 ? pick_e16dw<false, 1>(p.cin_chunks, narrow) : pick_e16dw<false, 2>(p.cin_chunks, narrow));
     if (!fn) return -1;
     if (p.mfrags < 1 || p.stride != 1 || p.res || p.in_clamp || !p.dw_w || !p.dw_scale || !p.dw_bias || p.dw_cp % 8 != 0 || p.dw_cp != p.out_cp || p.dw_cp > 16 * p.mfrags + 15 ||
         p.dw_hp < 1 || p.dw_wp < 1 || p.dw_hp - 1 + p.in_y0 >= p.in_hp || p.dw_wp - 1 + p.in_x0 >= p.in_wp || p.in_y0 < 0 || p.in_x0 < 0 || p.npos_y < 1 || p.npos_x < 1 ||
         p.tiles_x * 4 < p.npos_x || p.tiles_y * 4 < p.npos_y || (p.npos_y - 1) * p.dw_stride >= p.dw_hp + 1 || (p.npos_x - 1) * p.dw_stride >= p.dw_wp + 1 ||
         (long long)p.tiles_x * p.tiles_y > (1ll << 30) || p.nreset < 0 || p.nreset > 4)
         return -5;
-    hipLaunchKernelGGL(fn, dim3((unsigned)(p.tiles_x * p.tiles_y), (unsigned)((p.dw_cp + 63) / 64)), dim3(256), 0, s, p);
+    hipLaunchKernelGGL(fn, dim3((unsigned)(p.tiles_x * p.tiles_y), (unsigned)(narrow ? p.mfrags : (p.dw_cp + 63) / 64)), dim3(256), 0, s, p);
     return hipGetLastError() == hipSuccess ? 0 : -3;
 }
 

@@ -1849,8 +1849,8 @@ class ConvLayer : public Layer {
     std::string info() const override {
         if (edw_fused)
             return "conv_e16dw " + std::string(edw.f16 ? "f16" : "f16x2-split") + " 1x1 and the depthwise 3x3 layer " + std::to_string(edw_dw_no) +
-                   " behind it in one launch: a workgroup per 4x4 output positions and 64 expanded channels, blocks=" +
-                   std::to_string(edw.tiles_x * edw.tiles_y * ((edw.dw_cp + 63) / 64)) + "; apart: " + own_info();
+                   " behind it in one launch: a workgroup per 4x4 output positions and " + (edw.wm == 2 ? "16" : "64") + " expanded channels, blocks=" +
+                   std::to_string(edw.tiles_x * edw.tiles_y * (edw.wm == 2 ? edw.mfrags : (edw.dw_cp + 63) / 64)) + "; apart: " + own_info();
         return own_info();
     }
     std::string own_info() const {
@@ -2072,26 +2072,39 @@ void fuse_depthwise_layers(Net* net) {
         bool pick = true;
         char key[200];
         snprintf(key, sizeof(key), "edw:%d:%dto%d:%dx%d:s%d", q.f16, in_v.cp, ex->oc, ex->oh, ex->ow, dw->stride);
-        if (getenv("FYNHIP_FORCE_DW_FUSION")) {
-        } else if (tune_cache_flag(key, &pick)) {
+        // (q.wm = 2: a workgroup per 16 expanded channels instead of 64, for layers with few tiles; by rule when nothing is timed)
+        q.wm = (q.tiles_x * q.tiles_y * ((q.dw_cp + 63) / 64) < 128) ? 2 : 0;
+        if (const char* e = getenv("FYNHIP_EDW_NARROW")) q.wm = atoi(e) ? 2 : 0;
+        int cached[3] = {0, 0, 0};
+        if (getenv("FYNHIP_FORCE_DW_FUSION") || getenv("FYNHIP_EDW_NARROW")) {
+        } else if (tune_cache_triple(key, cached)) {
+            pick = cached[0] != 0;
+            q.wm = cached[1];
         } else if (!(at && at[0] == '0')) {
             float t_fused = 1e30f, t_two = 1e30f;
+            int best_wm = 0;
             for (int rep = 0; rep < 3; rep++) {
-                t_fused = std::min(t_fused, time_calls(net, [&]() {
-                    if (launch_conv_e16dw(q, net->stream) != 0) fail(FYN_ERR_DEVICE, "1x1 + depthwise convolution launch failed while tuning");
-                }, 10));
+                for (int wm : {0, 2}) {
+                    ConvP16Params c = q;
+                    c.wm = wm;
+                    const float t = time_calls(net, [&]() {
+                        if (launch_conv_e16dw(c, net->stream) != 0) fail(FYN_ERR_DEVICE, "1x1 + depthwise convolution launch failed while tuning");
+                    }, 10);
+                    if (t < t_fused) { t_fused = t; best_wm = wm; }
+                }
                 t_two = std::min(t_two, time_calls(net, [&]() {
                     ex->run(net->stream);
                     launch_dwconv3x3(dw->p, net->stream);
                 }, 10));
             }
             if (getenv("FYNHIP_TUNE_VERBOSE"))
-                fprintf(stderr, "[tune] 1x1 %d to %d at %dx%d + depthwise 3x3 (step %d): one launch %.1f us, two %.1f us\n", in_v.cp, ex->oc, ex->oh, ex->ow, dw->stride,
-                        t_fused * 1e3f, t_two * 1e3f);
+                fprintf(stderr, "[tune] 1x1 %d to %d at %dx%d + depthwise 3x3 (step %d): one launch (blocks of %d channels) %.1f us, two %.1f us\n", in_v.cp, ex->oc, ex->oh,
+                        ex->ow, dw->stride, best_wm == 2 ? 16 : 64, t_fused * 1e3f, t_two * 1e3f);
             // (a near tie goes to the single launch: it leaves the expanded tensor unwritten, which a timing loop that
             // finds everything in the caches does not reward)
             pick = t_fused < t_two * 1.05f;
-            tune_cache_store_flag(key, pick);
+            q.wm = best_wm;
+            tune_cache_store_triple(key, pick ? 1 : 0, best_wm, 0);
         }
         if (!pick) {
             net->dev_free(wp);

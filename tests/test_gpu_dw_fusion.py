@@ -99,15 +99,20 @@ FRONT_CASES = CASES + [
 
 @pytest.mark.parametrize("storage", [fa.STORAGE_F32, fa.STORAGE_F16], ids=["f32", "f16"])
 @pytest.mark.parametrize("case", FRONT_CASES, ids=lambda c: "%dto%dto%d_%dx%d_s%d%s" % (c[0], c[1], c[2], c[3], c[4], c[5], "_res" if c[6] else ""))
-def test_depthwise_inside_the_launch_of_the_expand_layer(case, storage, monkeypatch):
+@pytest.mark.parametrize("narrow", [0, 1], ids=["blocks64", "blocks16"])
+def test_depthwise_inside_the_launch_of_the_expand_layer(case, storage, narrow, monkeypatch):
     cin, exp, cout, h, w, stride, residual = case
+    if narrow and h * w > 60 * 60:
+        pytest.skip("the 16-channel blocks are for layers with few tiles")
     monkeypatch.setenv("FYNHIP_FORCE_DW_FUSION", "1")
+    monkeypatch.setenv("FYNHIP_EDW_NARROW", str(narrow))
     net = Block(storage, cin, exp, cout, h, w, stride, residual)
     x, got, infos = run(net)
     desc = net.describe()
     net.cleanup()
     print("  ", infos["dw"], "|", infos["expand"][:120], flush=True)
     assert "launch of layer 1" in infos["dw"] and "conv_e16dw" in infos["expand"] and "depthwise 3x3 layer 2" in infos["expand"]
+    assert ("and 16 expanded channels" if narrow else "and 64 expanded channels") in infos["expand"]
     ref = O.run_network(desc, {net.input_key: x})[net.output_layer]
     err = rel_l2(got, ref)
     print("   rel_l2=%.3e" % err, flush=True)
