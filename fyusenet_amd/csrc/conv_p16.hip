@@ -960,6 +960,9 @@ struct GeoR {
 // a depthwise 3x3 layer with step DWS (weights fp32, folded scale and bias, the arithmetic and the rounding to the
 // storage type of the depthwise kernel in layers_direct.hip), whose tensor then never exists.  A staging item is a pair
 // of horizontally neighbouring positions and 8 channels: 3 x (DWS + 3) texels of the depthwise layer's input.
+#ifndef FYN_KR_STAGE_WAVES
+#define FYN_KR_STAGE_WAVES 8
+#endif
 template <int NTAPS, int CPW, int FM, int FN, int S, int DWS = 0>
 __global__ __launch_bounds__(512) void conv_kr16_kernel(const ConvP16Params p) {
     using G = GeoR<NTAPS, CPW, FN, S>;
@@ -978,12 +981,119 @@ __global__ __launch_bounds__(512) void conv_kr16_kernel(const ConvP16Params p) {
     const unsigned range_bits = p.in_amax ? range_load(p.in_amax) : 0u;
     constexpr int red_off = G::RED_OFF;
     constexpr int sb_off = red_off + 3 * FM * FN * 1024;
+    // Staging waves: the four that only stage, and -- without a depthwise layer in front -- the four MFMA waves too,
+    // after they have requested their weights: conversion and address arithmetic of the tile split eight ways.
+    constexpr int SW = DWS > 0 ? 4 : FYN_KR_STAGE_WAVES, NTH = SW * 64;
+
+    // The tile's staging: every thread of the SW staging waves takes the items stid, stid + NTH, ...
+    struct RawF { float4 a, b; };
+    typedef typename std::conditional<HSTORE, half8_t, RawF>::type raw_t;
+    auto stage_tile = [&](const int stid) {
+        constexpr int NB = (G::TOTAL + NTH - 1) / NTH;
+        const store_t* in = reinterpret_cast<const store_t*>(p.in);
+        raw_t raw[NB];
+        int l_off[NB];
+        bool ok[NB];
+        // (a 1x1 layer may step over the input: position (y, x) reads pixel (y, x) * stride)
+        // (a 3x3 layer with stride 2 stages every pixel under its tile: position (y, x) reads the window at (2y, 2x))
+        const int st = NTAPS == 1 ? p.stride : 1, org = NTAPS == 1 ? p.stride : S;
+        const int y0 = tyi * G::TH * org + p.in_y0, x0 = txi * G::TW * org + p.in_x0;
+        if constexpr (NTH % G::NITEMS == 0) {
+            // A chunk's items divide the staging threads (1x1 layers): a thread keeps its pixel and its 8 channels
+            // of the chunk for all its items and only the chunk advances, by CPI per item -- the pixel's arithmetic is
+            // done once, not once per item (a thread has up to 16 items, and nothing is requested before it is through).
+            constexpr int CPI = NTH / G::NITEMS;
+            const int chunk0 = stid / G::NITEMS, rem = stid - chunk0 * G::NITEMS;
+            const int pix = rem >> 2, g = rem & 3;
+            const int py = pix / G::HW, px = pix - py * G::HW;
+            int gy = y0 + py * st, gx = x0 + px * st;
+            if (p.in_clamp) {
+                gy = min(max(gy, 0), p.in_hp - 1);
+                gx = min(max(gx, 0), p.in_wp - 1);
+            }
+            const bool inb = (unsigned)gy < (unsigned)p.in_hp && (unsigned)gx < (unsigned)p.in_wp;
+            const int l0 = chunk0 * G::BUFC + py * G::ROW_PITCH + px * G::PIT + g * 16;
+            const int c0 = chunk0 * KC + g * 8;
+            const store_t* src0 = in + (inb ? (gy * p.in_wp + gx) * p.in_cp : 0) + c0;
+#pragma unroll
+            for (int i = 0; i < NB; i++) {
+                const bool in_tile = chunk0 + i * CPI < G::NCH;
+                l_off[i] = in_tile ? l0 + i * CPI * G::BUFC : -1;
+                // (channels behind the tensor's pitch -- the chunk count is rounded up to four per wave -- read as zero)
+                ok[i] = in_tile && inb && c0 + i * CPI * KC < p.in_cp;
+                const store_t* src = ok[i] ? src0 + i * CPI * KC : in;
+                if constexpr (HSTORE) {
+                    raw[i] = *reinterpret_cast<const half8_t*>(src);
+                } else {
+                    raw[i].a = *reinterpret_cast<const float4*>(src);
+                    raw[i].b = *reinterpret_cast<const float4*>(src + 4);
+                }
+            }
+        } else {
+#pragma unroll
+        for (int i = 0; i < NB; i++) {
+            const int idx = stid + i * NTH;
+            const int chunk = idx / G::NITEMS, rem = idx - chunk * G::NITEMS;
+            const int pix = rem >> 2, g = rem & 3;
+            const int py = pix / G::HW, px = pix - py * G::HW;
+            l_off[i] = idx < G::TOTAL ? chunk * G::BUFC + py * G::ROW_PITCH + px * G::PIT + g * 16 : -1;
+            int gy = y0 + py * st, gx = x0 + px * st;
+            if (p.in_clamp) {
+                gy = min(max(gy, 0), p.in_hp - 1);
+                gx = min(max(gx, 0), p.in_wp - 1);
+            }
+            // (channels behind the tensor's pitch -- the chunk count is rounded up to four per wave -- read as zero)
+            ok[i] = idx < G::TOTAL && (unsigned)gy < (unsigned)p.in_hp && (unsigned)gx < (unsigned)p.in_wp && chunk * KC + g * 8 < p.in_cp;
+            const store_t* src = in + (ok[i] ? (gy * p.in_wp + gx) * p.in_cp + chunk * KC + g * 8 : 0);
+            if constexpr (HSTORE) {
+                raw[i] = *reinterpret_cast<const half8_t*>(src);
+            } else {
+                raw[i].a = *reinterpret_cast<const float4*>(src);
+                raw[i].b = *reinterpret_cast<const float4*>(src + 4);
+            }
+        }
+        }
+        float in_scale = 1.f, inv_unused;
+        if (p.in_amax) in_scale = range_scale(range_after_act(range_reduce(range_bits), p.act), &inv_unused);
+        // (fp16 tensors: no activation, or a clamp without leak whose bounds are fp16 values, is applied to the packed
+        // halves -- two values per instruction, no conversions)
+        const _Float16 hlo = (_Float16)fmaxf(p.act.lo, -65504.f), hhi = (_Float16)fminf(p.act.hi, 65504.f);
+        const bool half_act = HSTORE && p.act.leak == 0.f && (p.act.lo < -65504.f || (float)hlo == p.act.lo) && (p.act.hi > 65504.f || (float)hhi == p.act.hi);
+#pragma unroll
+        for (int i = 0; i < NB; i++) {
+            if (l_off[i] < 0) continue;
+            if constexpr (HSTORE) {
+                half8_t v;
+                if (half_act) {
+                    v = ok[i] ? __builtin_elementwise_min(__builtin_elementwise_max(raw[i], (half8_t)hlo), (half8_t)hhi) : (half8_t)((_Float16)0.f);
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 8; e++) v[e] = ok[i] ? (_Float16)act_p16((float)raw[i][e], p.act) : (_Float16)0.f;
+                }
+                *reinterpret_cast<half8_t*>(lds + l_off[i]) = v;
+            }
+        }
+        if constexpr (!HSTORE) {
+            auto split_all = [&](auto kind_) {
+                constexpr int KIND = decltype(kind_)::value;
+#pragma unroll
+                for (int i = 0; i < NB; i++) {
+                    if (l_off[i] < 0) continue;
+                    const float r[8] = {raw[i].a.x, raw[i].a.y, raw[i].a.z, raw[i].a.w, raw[i].b.x, raw[i].b.y, raw[i].b.z, raw[i].b.w};
+                    half8_t hi, lo;
+                    split8<KIND>(r, ok[i], p.act, in_scale, hi, lo);
+                    *reinterpret_cast<half8_t*>(lds + l_off[i]) = hi;
+                    *reinterpret_cast<half8_t*>(lds + G::PLANE + l_off[i]) = lo;
+                }
+            };
+            if (p.act.kind == ACT_NONE) split_all(std::integral_constant<int, ACT_NONE>());
+            else if (p.act.kind == ACT_RELU) split_all(std::integral_constant<int, ACT_RELU>());
+            else split_all(std::integral_constant<int, ACT_LEAKY>());
+        }
+    };
 
     if (wave < 4) {   // ------------------------------------------------------------ staging waves
         const int stid = tid & 255;
-        const store_t* in = reinterpret_cast<const store_t*>(p.in);
-        struct RawF { float4 a, b; };
-        typedef typename std::conditional<HSTORE, half8_t, RawF>::type raw_t;
         if constexpr (DWS > 0) {
             constexpr int WINW = DWS + 3;
             constexpr int TOTAL = G::NCH * 32, NB = (TOTAL + 255) / 256;
@@ -1104,108 +1214,10 @@ __global__ __launch_bounds__(512) void conv_kr16_kernel(const ConvP16Params p) {
             lds_barrier();   // the MFMA waves have left their accumulators for wave 0
             return;
         }
-        raw_t raw[G::NB];
-        int l_off[G::NB];
-        bool ok[G::NB];
-        // (a 1x1 layer may step over the input: position (y, x) reads pixel (y, x) * stride)
-        // (a 3x3 layer with stride 2 stages every pixel under its tile: position (y, x) reads the window at (2y, 2x))
-        const int st = NTAPS == 1 ? p.stride : 1, org = NTAPS == 1 ? p.stride : S;
-        const int y0 = tyi * G::TH * org + p.in_y0, x0 = txi * G::TW * org + p.in_x0;
-        if constexpr (256 % G::NITEMS == 0) {
-            // A chunk's items divide the 256 staging threads (1x1 layers): a thread keeps its pixel and its 8 channels
-            // of the chunk for all its items and only the chunk advances, by CPI per item -- the pixel's arithmetic is
-            // done once, not once per item (a thread has up to 16 items, and nothing is requested before it is through).
-            constexpr int CPI = 256 / G::NITEMS;
-            const int chunk0 = stid / G::NITEMS, rem = stid - chunk0 * G::NITEMS;
-            const int pix = rem >> 2, g = rem & 3;
-            const int py = pix / G::HW, px = pix - py * G::HW;
-            int gy = y0 + py * st, gx = x0 + px * st;
-            if (p.in_clamp) {
-                gy = min(max(gy, 0), p.in_hp - 1);
-                gx = min(max(gx, 0), p.in_wp - 1);
-            }
-            const bool inb = (unsigned)gy < (unsigned)p.in_hp && (unsigned)gx < (unsigned)p.in_wp;
-            const int l0 = chunk0 * G::BUFC + py * G::ROW_PITCH + px * G::PIT + g * 16;
-            const int c0 = chunk0 * KC + g * 8;
-            const store_t* src0 = in + (inb ? (gy * p.in_wp + gx) * p.in_cp : 0) + c0;
-#pragma unroll
-            for (int i = 0; i < G::NB; i++) {
-                const bool in_tile = chunk0 + i * CPI < G::NCH;
-                l_off[i] = in_tile ? l0 + i * CPI * G::BUFC : -1;
-                // (channels behind the tensor's pitch -- the chunk count is rounded up to four per wave -- read as zero)
-                ok[i] = in_tile && inb && c0 + i * CPI * KC < p.in_cp;
-                const store_t* src = ok[i] ? src0 + i * CPI * KC : in;
-                if constexpr (HSTORE) {
-                    raw[i] = *reinterpret_cast<const half8_t*>(src);
-                } else {
-                    raw[i].a = *reinterpret_cast<const float4*>(src);
-                    raw[i].b = *reinterpret_cast<const float4*>(src + 4);
-                }
-            }
-        } else {
-#pragma unroll
-        for (int i = 0; i < G::NB; i++) {
-            const int idx = stid + i * 256;
-            const int chunk = idx / G::NITEMS, rem = idx - chunk * G::NITEMS;
-            const int pix = rem >> 2, g = rem & 3;
-            const int py = pix / G::HW, px = pix - py * G::HW;
-            l_off[i] = idx < G::TOTAL ? chunk * G::BUFC + py * G::ROW_PITCH + px * G::PIT + g * 16 : -1;
-            int gy = y0 + py * st, gx = x0 + px * st;
-            if (p.in_clamp) {
-                gy = min(max(gy, 0), p.in_hp - 1);
-                gx = min(max(gx, 0), p.in_wp - 1);
-            }
-            // (channels behind the tensor's pitch -- the chunk count is rounded up to four per wave -- read as zero)
-            ok[i] = idx < G::TOTAL && (unsigned)gy < (unsigned)p.in_hp && (unsigned)gx < (unsigned)p.in_wp && chunk * KC + g * 8 < p.in_cp;
-            const store_t* src = in + (ok[i] ? (gy * p.in_wp + gx) * p.in_cp + chunk * KC + g * 8 : 0);
-            if constexpr (HSTORE) {
-                raw[i] = *reinterpret_cast<const half8_t*>(src);
-            } else {
-                raw[i].a = *reinterpret_cast<const float4*>(src);
-                raw[i].b = *reinterpret_cast<const float4*>(src + 4);
-            }
-        }
-        }
-        float in_scale = 1.f, inv_unused;
-        if (p.in_amax) in_scale = range_scale(range_after_act(range_reduce(range_bits), p.act), &inv_unused);
+        stage_tile(SW == 8 ? tid : stid);
         if (stid < 16 * FM) {
             reinterpret_cast<float*>(lds + sb_off)[stid] = p.scale[cb * 16 * FM + stid];
             reinterpret_cast<float*>(lds + sb_off)[16 * FM + stid] = p.bias[cb * 16 * FM + stid];
-        }
-        // (fp16 tensors: no activation, or a clamp without leak whose bounds are fp16 values, is applied to the packed
-        // halves -- two values per instruction, no conversions)
-        const _Float16 hlo = (_Float16)fmaxf(p.act.lo, -65504.f), hhi = (_Float16)fminf(p.act.hi, 65504.f);
-        const bool half_act = HSTORE && p.act.leak == 0.f && (p.act.lo < -65504.f || (float)hlo == p.act.lo) && (p.act.hi > 65504.f || (float)hhi == p.act.hi);
-#pragma unroll
-        for (int i = 0; i < G::NB; i++) {
-            if (l_off[i] < 0) continue;
-            if constexpr (HSTORE) {
-                half8_t v;
-                if (half_act) {
-                    v = ok[i] ? __builtin_elementwise_min(__builtin_elementwise_max(raw[i], (half8_t)hlo), (half8_t)hhi) : (half8_t)((_Float16)0.f);
-                } else {
-#pragma unroll
-                    for (int e = 0; e < 8; e++) v[e] = ok[i] ? (_Float16)act_p16((float)raw[i][e], p.act) : (_Float16)0.f;
-                }
-                *reinterpret_cast<half8_t*>(lds + l_off[i]) = v;
-            }
-        }
-        if constexpr (!HSTORE) {
-            auto split_all = [&](auto kind_) {
-                constexpr int KIND = decltype(kind_)::value;
-#pragma unroll
-                for (int i = 0; i < G::NB; i++) {
-                    if (l_off[i] < 0) continue;
-                    const float r[8] = {raw[i].a.x, raw[i].a.y, raw[i].a.z, raw[i].a.w, raw[i].b.x, raw[i].b.y, raw[i].b.z, raw[i].b.w};
-                    half8_t hi, lo;
-                    split8<KIND>(r, ok[i], p.act, in_scale, hi, lo);
-                    *reinterpret_cast<half8_t*>(lds + l_off[i]) = hi;
-                    *reinterpret_cast<half8_t*>(lds + G::PLANE + l_off[i]) = lo;
-                }
-            };
-            if (p.act.kind == ACT_NONE) split_all(std::integral_constant<int, ACT_NONE>());
-            else if (p.act.kind == ACT_RELU) split_all(std::integral_constant<int, ACT_RELU>());
-            else split_all(std::integral_constant<int, ACT_LEAKY>());
         }
         lds_barrier();   // the tile is staged
         lds_barrier();   // the MFMA waves have left their accumulators for wave 0
@@ -1263,6 +1275,7 @@ __global__ __launch_bounds__(512) void conv_kr16_kernel(const ConvP16Params p) {
         }
     }
 
+    if constexpr (SW == 8) stage_tile(tid);
     lds_barrier();   // the tile is staged
     // B fragment of step s: chunk w + 4*(s / NTAPS), tap s % NTAPS
     auto b_off = [&](int s) { return (s / NTAPS) * 4 * G::BUFC + G::tap_off(s % NTAPS); };
