@@ -963,10 +963,14 @@ struct GeoR {
 #ifndef FYN_KR_STAGE_WAVES
 #define FYN_KR_STAGE_WAVES 8
 #endif
-template <int NTAPS, int CPW, int FM, int FN, int S, int DWS = 0>
+template <int NTAPS, int CPW, int FM, int FN, int S, int DWS = 0, int R = 1>
 __global__ __launch_bounds__(512) void conv_kr16_kernel(const ConvP16Params p) {
+    // R > 1: the reduction passes through the LDS in R rounds of 4 * CPW chunks each (layers whose whole reduction does
+    // not fit: 3x3 with stride 2 on 512 channels needs 166 KB).  The staging waves request round r + 1 while the MFMA
+    // waves work on round r and write it once those are through.
     using G = GeoR<NTAPS, CPW, FN, S>;
     static_assert(DWS == 0 || (NTAPS == 1 && FN == 1 && S == 1 && DWS <= 2), "a fused depthwise layer: 1x1, tiles of 4x4 positions");
+    static_assert(R >= 1 && (R == 1 || DWS == 0), "rounds: without a depthwise layer in the staging");
     constexpr int RPD = G::RPD, BD = G::BD, STEPS = G::STEPS;
     extern __shared__ __align__(16) unsigned char lds[];
     __shared__ unsigned range_box[2];
@@ -983,12 +987,13 @@ __global__ __launch_bounds__(512) void conv_kr16_kernel(const ConvP16Params p) {
     constexpr int sb_off = red_off + 3 * FM * FN * 1024;
     // Staging waves: the four that only stage, and -- without a depthwise layer in front -- the four MFMA waves too,
     // after they have requested their weights: conversion and address arithmetic of the tile split eight ways.
-    constexpr int SW = DWS > 0 ? 4 : FYN_KR_STAGE_WAVES, NTH = SW * 64;
+    constexpr int SW = (DWS > 0 || R > 1) ? 4 : FYN_KR_STAGE_WAVES, NTH = SW * 64;
 
     // The tile's staging: every thread of the SW staging waves takes the items stid, stid + NTH, ...
     struct RawF { float4 a, b; };
     typedef typename std::conditional<HSTORE, half8_t, RawF>::type raw_t;
-    auto stage_tile = [&](const int stid) {
+    auto stage_tile = [&](const int stid, const int round, const bool wait) {
+        const int ch_r = round * G::NCH * KC;   // the round's first channel
         constexpr int NB = (G::TOTAL + NTH - 1) / NTH;
         const store_t* in = reinterpret_cast<const store_t*>(p.in);
         raw_t raw[NB];
@@ -1013,7 +1018,7 @@ __global__ __launch_bounds__(512) void conv_kr16_kernel(const ConvP16Params p) {
             }
             const bool inb = (unsigned)gy < (unsigned)p.in_hp && (unsigned)gx < (unsigned)p.in_wp;
             const int l0 = chunk0 * G::BUFC + py * G::ROW_PITCH + px * G::PIT + g * 16;
-            const int c0 = chunk0 * KC + g * 8;
+            const int c0 = ch_r + chunk0 * KC + g * 8;
             const store_t* src0 = in + (inb ? (gy * p.in_wp + gx) * p.in_cp : 0) + c0;
 #pragma unroll
             for (int i = 0; i < NB; i++) {
@@ -1043,8 +1048,8 @@ __global__ __launch_bounds__(512) void conv_kr16_kernel(const ConvP16Params p) {
                 gx = min(max(gx, 0), p.in_wp - 1);
             }
             // (channels behind the tensor's pitch -- the chunk count is rounded up to four per wave -- read as zero)
-            ok[i] = idx < G::TOTAL && (unsigned)gy < (unsigned)p.in_hp && (unsigned)gx < (unsigned)p.in_wp && chunk * KC + g * 8 < p.in_cp;
-            const store_t* src = in + (ok[i] ? (gy * p.in_wp + gx) * p.in_cp + chunk * KC + g * 8 : 0);
+            ok[i] = idx < G::TOTAL && (unsigned)gy < (unsigned)p.in_hp && (unsigned)gx < (unsigned)p.in_wp && ch_r + chunk * KC + g * 8 < p.in_cp;
+            const store_t* src = in + (ok[i] ? (gy * p.in_wp + gx) * p.in_cp + ch_r + chunk * KC + g * 8 : 0);
             if constexpr (HSTORE) {
                 raw[i] = *reinterpret_cast<const half8_t*>(src);
             } else {
@@ -1059,6 +1064,7 @@ __global__ __launch_bounds__(512) void conv_kr16_kernel(const ConvP16Params p) {
         // halves -- two values per instruction, no conversions)
         const _Float16 hlo = (_Float16)fmaxf(p.act.lo, -65504.f), hhi = (_Float16)fminf(p.act.hi, 65504.f);
         const bool half_act = HSTORE && p.act.leak == 0.f && (p.act.lo < -65504.f || (float)hlo == p.act.lo) && (p.act.hi > 65504.f || (float)hhi == p.act.hi);
+        if (wait) lds_barrier();   // the MFMA waves are through with the round before: its place in the LDS is free
 #pragma unroll
         for (int i = 0; i < NB; i++) {
             if (l_off[i] < 0) continue;
@@ -1214,12 +1220,15 @@ __global__ __launch_bounds__(512) void conv_kr16_kernel(const ConvP16Params p) {
             lds_barrier();   // the MFMA waves have left their accumulators for wave 0
             return;
         }
-        stage_tile(SW == 8 ? tid : stid);
         if (stid < 16 * FM) {
             reinterpret_cast<float*>(lds + sb_off)[stid] = p.scale[cb * 16 * FM + stid];
             reinterpret_cast<float*>(lds + sb_off)[16 * FM + stid] = p.bias[cb * 16 * FM + stid];
         }
-        lds_barrier();   // the tile is staged
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            stage_tile(SW == 8 ? tid : stid, r, r > 0);
+            lds_barrier();   // the round is staged
+        }
         lds_barrier();   // the MFMA waves have left their accumulators for wave 0
         return;
     }
@@ -1234,18 +1243,21 @@ __global__ __launch_bounds__(512) void conv_kr16_kernel(const ConvP16Params p) {
         bbase[fn] = (m / G::TW) * S * G::ROW_PITCH + (m % G::TW) * S * G::PIT + kq * 16 + w * G::BUFC;
     }
     constexpr unsigned wstep = FM * NPL * 1024;
-    const unsigned char* wbase = reinterpret_cast<const unsigned char*>(p.wpack) + (size_t)((cb * 4 + w) * STEPS) * wstep + lane * 16;
+    const unsigned char* wbase = reinterpret_cast<const unsigned char*>(p.wpack) + (size_t)((cb * 4 + w) * R * STEPS) * wstep + lane * 16;
     half8_t a_q[RPD][FM][NPL];
+    auto ring_fill = [&](const unsigned char* wb) {   // the weights of a round's first RPD - 1 steps
 #pragma unroll
-    for (int d = 0; d < RPD - 1; d++)
+        for (int d = 0; d < RPD - 1; d++)
+#pragma unroll
+            for (int fm = 0; fm < FM; fm++)
+#pragma unroll
+                for (int pl = 0; pl < NPL; pl++) a_q[d][fm][pl] = *reinterpret_cast<const half8_t*>(wb + (size_t)d * wstep + (fm * NPL + pl) * 1024);
 #pragma unroll
         for (int fm = 0; fm < FM; fm++)
 #pragma unroll
-            for (int pl = 0; pl < NPL; pl++) a_q[d][fm][pl] = *reinterpret_cast<const half8_t*>(wbase + (size_t)d * wstep + (fm * NPL + pl) * 1024);
-#pragma unroll
-    for (int fm = 0; fm < FM; fm++)
-#pragma unroll
-        for (int pl = 0; pl < NPL; pl++) a_q[RPD - 1][fm][pl] = a_q[0][fm][pl];   // (defined; replaced during the first step)
+            for (int pl = 0; pl < NPL; pl++) a_q[RPD - 1][fm][pl] = a_q[0][fm][pl];   // (defined; replaced during the first step)
+    };
+    ring_fill(wbase);
     f32x4_t acc[FM][FN];
 #pragma unroll
     for (int fm = 0; fm < FM; fm++)
@@ -1275,44 +1287,52 @@ __global__ __launch_bounds__(512) void conv_kr16_kernel(const ConvP16Params p) {
         }
     }
 
-    if constexpr (SW == 8) stage_tile(tid);
-    lds_barrier();   // the tile is staged
-    // B fragment of step s: chunk w + 4*(s / NTAPS), tap s % NTAPS
-    auto b_off = [&](int s) { return (s / NTAPS) * 4 * G::BUFC + G::tap_off(s % NTAPS); };
-    half8_t b[BD][FN][NPL];
+    if constexpr (SW == 8) stage_tile(tid, 0, false);
 #pragma unroll
-    for (int s = 0; s < BD - 1; s++)
+    for (int r = 0; r < R; r++) {
+        const unsigned char* wb = wbase + (size_t)r * STEPS * wstep;
+        lds_barrier();   // the round is staged
+        // B fragment of step s: chunk w + 4*(s / NTAPS), tap s % NTAPS
+        auto b_off = [&](int s) { return (s / NTAPS) * 4 * G::BUFC + G::tap_off(s % NTAPS); };
+        half8_t b[BD][FN][NPL];
 #pragma unroll
-        for (int fn = 0; fn < FN; fn++)
-#pragma unroll
-            for (int pl = 0; pl < NPL; pl++) b[s][fn][pl] = *reinterpret_cast<const half8_t*>(lds + bbase[fn] + b_off(s) + pl * G::PLANE);
-#pragma unroll
-    for (int s = 0; s < STEPS; s++) {
-        const int d = s % RPD, dload = (s + RPD - 1) % RPD, bs = s % BD, bload = (s + BD - 1) % BD;
-        // the weights of step s + RPD - 1 and the fragment of step s + BD - 1 go into the slots the previous step left
-        if (s + RPD - 1 < STEPS) {
-#pragma unroll
-            for (int fm = 0; fm < FM; fm++)
-#pragma unroll
-                for (int pl = 0; pl < NPL; pl++)
-                    a_q[dload][fm][pl] = *reinterpret_cast<const half8_t*>(wbase + (size_t)(s + RPD - 1) * wstep + (fm * NPL + pl) * 1024);
-        }
-        if (s + BD - 1 < STEPS) {
+        for (int s = 0; s < BD - 1; s++)
 #pragma unroll
             for (int fn = 0; fn < FN; fn++)
 #pragma unroll
-                for (int pl = 0; pl < NPL; pl++)
-                    b[bload][fn][pl] = *reinterpret_cast<const half8_t*>(lds + bbase[fn] + b_off(s + BD - 1) + pl * G::PLANE);
-        }
+                for (int pl = 0; pl < NPL; pl++) b[s][fn][pl] = *reinterpret_cast<const half8_t*>(lds + bbase[fn] + b_off(s) + pl * G::PLANE);
 #pragma unroll
-        for (int fn = 0; fn < FN; fn++)
+        for (int s = 0; s < STEPS; s++) {
+            const int d = s % RPD, dload = (s + RPD - 1) % RPD, bs = s % BD, bload = (s + BD - 1) % BD;
+            // the weights of step s + RPD - 1 and the fragment of step s + BD - 1 go into the slots the previous step left
+            if (s + RPD - 1 < STEPS) {
 #pragma unroll
-            for (int i = 0; i < NPASS * FM; i++) {
-                const int kind = i / FM, fm = i % FM;
-                const int apl = (kind == 1) ? 1 : 0, bpl = (kind == 2) ? 1 : 0;
-                acc[fm][fn] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_q[d][fm][apl], b[bs][fn][bpl], acc[fm][fn], 0, 0, 0);
+                for (int fm = 0; fm < FM; fm++)
+#pragma unroll
+                    for (int pl = 0; pl < NPL; pl++)
+                        a_q[dload][fm][pl] = *reinterpret_cast<const half8_t*>(wb + (size_t)(s + RPD - 1) * wstep + (fm * NPL + pl) * 1024);
             }
-        __builtin_amdgcn_sched_barrier(0);
+            if (s + BD - 1 < STEPS) {
+#pragma unroll
+                for (int fn = 0; fn < FN; fn++)
+#pragma unroll
+                    for (int pl = 0; pl < NPL; pl++)
+                        b[bload][fn][pl] = *reinterpret_cast<const half8_t*>(lds + bbase[fn] + b_off(s + BD - 1) + pl * G::PLANE);
+            }
+#pragma unroll
+            for (int fn = 0; fn < FN; fn++)
+#pragma unroll
+                for (int i = 0; i < NPASS * FM; i++) {
+                    const int kind = i / FM, fm = i % FM;
+                    const int apl = (kind == 1) ? 1 : 0, bpl = (kind == 2) ? 1 : 0;
+                    acc[fm][fn] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_q[d][fm][apl], b[bs][fn][bpl], acc[fm][fn], 0, 0, 0);
+                }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        if (r + 1 < R) {
+            ring_fill(wb + (size_t)STEPS * wstep);
+            lds_barrier();   // every MFMA wave is through with the round: the staging waves may write the next
+        }
     }
     // the four partial sums meet in wave 0
     if (w > 0) {
@@ -1425,14 +1445,14 @@ template <int K, int TH, int TW>
 constexpr C4Entry c4entry() { return C4Entry{K, TH, TW, conv_p16c4_kernel<K, TH, TW>, (size_t)GeoC4<K, TH, TW>::BUF, GeoC4<K, TH, TW>::NS}; }
 const C4Entry kC4Entries[] = {c4entry<9, 8, 8>(), c4entry<9, 4, 8>(), c4entry<9, 8, 4>()};
 struct KREntry {
-    int taps, cpw, fm, nfrag, th, tw, stride, dws;
+    int taps, cpw, fm, nfrag, th, tw, stride, dws, rounds;   // (cpw: chunks per wave and round)
     p16_fn fn;
     size_t lds;
 };
-template <int NTAPS, int CPW, int FM, int FN = 1, int S = 1, int DWS = 0>
+template <int NTAPS, int CPW, int FM, int FN = 1, int S = 1, int DWS = 0, int R = 1>
 constexpr KREntry krentry() {
     using G = GeoR<NTAPS, CPW, FN, S>;
-    return KREntry{NTAPS, CPW, FM, FN, G::TH, G::TW, S, DWS, conv_kr16_kernel<NTAPS, CPW, FM, FN, S, DWS>, (size_t)(G::RED_OFF + 3 * FM * FN * 1024 + 2 * 16 * FM * 4)};
+    return KREntry{NTAPS, CPW, FM, FN, G::TH, G::TW, S, DWS, R, conv_kr16_kernel<NTAPS, CPW, FM, FN, S, DWS, R>, (size_t)(G::RED_OFF + 3 * FM * FN * 1024 + 2 * 16 * FM * 4)};
 }
 const KREntry kKREntries[] = {
     krentry<1, 1, 1>(), krentry<1, 2, 1>(), krentry<1, 3, 1>(), krentry<1, 4, 1>(), krentry<1, 5, 1>(), krentry<1, 8, 1>(), krentry<1, 16, 1>(),
@@ -1443,6 +1463,10 @@ const KREntry kKREntries[] = {
     krentry<1, 1, 1, 4>(), krentry<1, 1, 2, 4>(), krentry<1, 2, 1, 4>(), krentry<1, 2, 2, 4>(), krentry<9, 1, 1, 4>(), krentry<9, 1, 2, 4>(),
     // 3x3 with stride 2 (a 9x9-pixel window per chunk under a tile of 4x4 positions)
     krentry<9, 1, 1, 1, 2>(), krentry<9, 1, 2, 1, 2>(), krentry<9, 2, 1, 1, 2>(), krentry<9, 2, 2, 1, 2>(), krentry<9, 4, 1, 1, 2>(), krentry<9, 4, 2, 1, 2>(),
+    // reductions that pass through the LDS in two rounds (taken where the one-round entry above is more than a CU's LDS):
+    // 3x3 with stride 2 on 512 channels in fp32, 3x3 on 1024 channels, 1x1 on 4096
+    krentry<9, 2, 1, 1, 2, 0, 2>(), krentry<9, 2, 2, 1, 2, 0, 2>(), krentry<9, 4, 1, 1, 1, 0, 2>(), krentry<9, 4, 2, 1, 1, 0, 2>(),
+    krentry<1, 16, 1, 1, 1, 0, 2>(), krentry<1, 16, 2, 1, 1, 0, 2>(),
 };
 // 1x1 with a depthwise 3x3 layer (step 1 or 2) computed in the staging
 #define FYN_KR_DW(CPW) krentry<1, CPW, 1, 1, 1, 1>(), krentry<1, CPW, 2, 1, 1, 1>(), krentry<1, CPW, 1, 1, 1, 2>(), krentry<1, CPW, 2, 1, 1, 2>()
@@ -1488,7 +1512,7 @@ void conv_p16c4_tile(int index, int* k, int* th, int* tw, int* steps) {
 }
 int conv_kr16_variant_count() { return (int)(sizeof(kKREntries) / sizeof(kKREntries[0])); }
 void conv_kr16_variant(int index, int* taps, int* chunks, int* fm, int* th, int* tw, int* stride) {
-    *taps = kKREntries[index].taps; *chunks = 4 * kKREntries[index].cpw; *fm = kKREntries[index].fm;
+    *taps = kKREntries[index].taps; *chunks = 4 * kKREntries[index].cpw * kKREntries[index].rounds; *fm = kKREntries[index].fm;
     *th = kKREntries[index].th; *tw = kKREntries[index].tw; *stride = kKREntries[index].stride;
 }
 bool conv_p16c4_supported(int k, int stride, int dil, int in_cp, int cout, int out_cp, bool f16) {
@@ -1504,7 +1528,9 @@ static const KREntry* find_krentry(const ConvP16Params& p, int k) {
         return nullptr;
     }
     for (const KREntry& c : kKREntries)
-        if (c.taps == k * k && c.cpw * 4 == p.cin_chunks && c.fm == p.wm && c.th == p.tile_h && c.tw == p.tile_w && c.stride == (k == 1 ? 1 : p.stride)) return &c;
+        if (c.taps == k * k && c.cpw * 4 * c.rounds == p.cin_chunks && c.fm == p.wm && c.th == p.tile_h && c.tw == p.tile_w && c.stride == (k == 1 ? 1 : p.stride) &&
+            c.lds <= 160 * 1024)
+            return &c;
     return nullptr;
 }
 size_t P16_NAME(conv_kr16_lds_bytes)(const ConvP16Params& p, int k) {
@@ -1515,7 +1541,7 @@ size_t P16_NAME(conv_kr16_lds_bytes)(const ConvP16Params& p, int k) {
     return e ? e->lds : 0;
 }
 // The K-resident form: k = 1 (any stride) or 3 (stride 1, or 2 with 4x4 tiles); tiles of tile_h x tile_w = 4x4 (4x8, 8x8 for short reductions) positions, blocks of 16*p.wm output channels (p.wm = 1 or 2),
-// p.cin_chunks = 4, 8, 12, 16, 20, 32 or 64 (3x3: 4, 8 or 16), channels behind in_cp reading as zero; in_y0/in_x0 = input padding - (k-1)/2; one workgroup per tile and block
+// p.cin_chunks = 4, 8, 12, 16, 20, 32, 64 or 128 (3x3: 4, 8, 16 or 32; with stride 2: 4, 8 or 16), channels behind in_cp reading as zero; in_y0/in_x0 = input padding - (k-1)/2; one workgroup per tile and block
 int P16_NAME(launch_conv_kr16)(const ConvP16Params& p, int k, hipStream_t s) {
 #if !FYN_P16_HALF
     if (p.f16) return launch_conv_kr16_half(p, k, s);

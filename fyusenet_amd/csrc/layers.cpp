@@ -1231,7 +1231,9 @@ class ConvLayer : public Layer {
             c.mfrags = c.cout_blocks * fm;
             const size_t lds = conv_kr16_lds_bytes(c, k);
             if (lds == 0 || lds > 160 * 1024 || (long long)c.pos_groups * c.cout_blocks > 65535) continue;
-            cands.push_back(c);
+            bool listed = false;   // (a one-round and a two-round variant of the same shape are one launch: the first that fits the LDS)
+            for (const ConvP16Params& o : cands) listed = listed || (o.wm == c.wm && o.tile_h == c.tile_h && o.tile_w == c.tile_w);
+            if (!listed) cands.push_back(c);
         }
         if (cands.empty()) return;
         // (large enough for every candidate: cout blocks x 4 waves x steps x fragments x planes)

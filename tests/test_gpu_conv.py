@@ -417,7 +417,13 @@ KR16_CASES = [
     (3, 256, 64, 28, 28, 2, {"stride": 2}),
     (3, 256, 48, 13, 15, 1, {"stride": 2, "bn": True, "residual": (A.RELU, True)}),   # odd input size
     (3, 64, 32, 10, 22, 2, {"stride": 2, "pad_out": 1}),
-    (3, 512, 32, 14, 14, 2, {"stride": 2}),                                     # 16 chunks (fp16 storage only: LDS)
+    (3, 512, 32, 14, 14, 2, {"stride": 2}),                                     # 16 chunks: in fp32 in two rounds through the LDS
+    (3, 512, 64, 15, 13, 1, {"stride": 2, "bn": True, "residual": (A.RELU, True)}),
+    # reductions in two rounds through the LDS
+    (3, 1024, 32, 7, 7, 1, {"bn": True}),
+    (3, 1024, 64, 6, 9, 2, {"residual": (A.NONE, False)}),
+    (1, 4096, 32, 5, 6, 2, {"bn": True}),
+    (1, 4096, 48, 7, 7, 1, {"residual": (A.RELU, True)}),
 ]
 
 
@@ -433,8 +439,6 @@ def test_reduction_resident_form(case, act, shallow, storage, monkeypatch):
         pytest.skip("the shallow variant is run on the plain 3x3 cases")
     if act is A.LEAKY_RELU and (cin > 512 or "pad_out" in kw):
         pytest.skip("activations are varied on some of the cases")
-    if k == 3 and kw.get("stride", 1) == 2 and cin > 256 and storage == fa.STORAGE_F32:
-        pytest.skip("the stride-2 windows of 16 chunks in two planes are more than a CU's LDS")
     monkeypatch.setenv("FYNHIP_FORCE_KR16_CONV", "1")
     monkeypatch.setenv("FYNHIP_KR16_FM", str(fm))
     if shallow:
