@@ -182,6 +182,7 @@ __global__ __launch_bounds__(256) void conv_d16_kernel(const ConvP16Params p) {
     _Float16 act_lo, act_hi;
     const bool half_act = HS && act_half_exact(p.act, act_lo, act_hi);
     half8_t b[NCHK][NPL];
+    const bool affine = DWS == 0 && KS == 0 && p.in_mul != nullptr;
     auto convert = [&](auto kind_) {
     constexpr int KIND = decltype(kind_)::value;   // (the activation's kind, chosen once per wave: act_kind)
 #pragma unroll
@@ -211,9 +212,22 @@ __global__ __launch_bounds__(256) void conv_d16_kernel(const ConvP16Params p) {
             }
         } else {
             texel(raw[c][0], r);
+            if constexpr (KS == 0) {
+                if (affine) {   // a batch-norm layer in front, applied here: x * in_mul[channel] + in_add[channel]
+                    const int ch = okc ? c * KC + kq * 8 : 0;
+                    const float4 m0 = *reinterpret_cast<const float4*>(p.in_mul + ch), m1 = *reinterpret_cast<const float4*>(p.in_mul + ch + 4);
+                    const float4 a0 = *reinterpret_cast<const float4*>(p.in_add + ch), a1 = *reinterpret_cast<const float4*>(p.in_add + ch + 4);
+                    const float mv[8] = {m0.x, m0.y, m0.z, m0.w, m1.x, m1.y, m1.z, m1.w}, av[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
+#pragma unroll
+                    for (int e = 0; e < 8; e++) {
+                        r[e] = r[e] * mv[e] + av[e];
+                        if constexpr (HS) r[e] = (float)(_Float16)r[e];   // (what the batch-norm layer would have stored)
+                    }
+                }
+            }
         }
         if constexpr (HS) {
-            if (DWS == 0 && half_act) {
+            if (DWS == 0 && half_act && !affine) {
                 b[c][0] = okc ? act_half(raw[c][0], act_lo, act_hi) : (half8_t)((_Float16)0.f);
             } else {
 #pragma unroll
@@ -651,6 +665,8 @@ int launch_conv_d16(const ConvP16Params& p, hipStream_t s) {
         fn = p.f16 ? (p.dw_stride == 1 ? pick_d16_dw<true, 1>(p.cin_chunks, one) : pick_d16_dw<true, 2>(p.cin_chunks, one))
                    : (p.dw_stride == 1 ? pick_d16_dw<false, 1>(p.cin_chunks, one) : pick_d16_dw<false, 2>(p.cin_chunks, one));
     }
+    // (a batch-norm layer applied on fetch: plain 1x1 launches only, both arrays or none)
+    if ((p.in_mul != nullptr) != (p.in_add != nullptr) || (p.in_mul && (ks || p.dw_in))) return -5;
     const long long npos = (long long)p.npos_y * p.npos_x;
     if (!fn) return -1;
     if ((!ks && (p.in_cp > p.cin_chunks * KC || p.in_cp % 8 != 0 || p.in_cp < 8)) || p.mfrags < 1 || p.stride < 1 || npos < 1 || npos > (1ll << 30) || p.out_cp % 4 != 0 || p.out_cp < 4 ||

@@ -998,6 +998,7 @@ __global__ __launch_bounds__(512) void conv_kr16_kernel(const ConvP16Params p) {
         const store_t* in = reinterpret_cast<const store_t*>(p.in);
         raw_t raw[NB];
         int l_off[NB];
+        int ch_of[NB];   // the item's first channel
         bool ok[NB];
         // (a 1x1 layer may step over the input: position (y, x) reads pixel (y, x) * stride)
         // (a 3x3 layer with stride 2 stages every pixel under its tile: position (y, x) reads the window at (2y, 2x))
@@ -1026,6 +1027,7 @@ __global__ __launch_bounds__(512) void conv_kr16_kernel(const ConvP16Params p) {
                 l_off[i] = in_tile ? l0 + i * CPI * G::BUFC : -1;
                 // (channels behind the tensor's pitch -- the chunk count is rounded up to four per wave -- read as zero)
                 ok[i] = in_tile && inb && c0 + i * CPI * KC < p.in_cp;
+                ch_of[i] = c0 + i * CPI * KC;
                 const store_t* src = ok[i] ? src0 + i * CPI * KC : in;
                 if constexpr (HSTORE) {
                     raw[i] = *reinterpret_cast<const half8_t*>(src);
@@ -1049,6 +1051,7 @@ __global__ __launch_bounds__(512) void conv_kr16_kernel(const ConvP16Params p) {
             }
             // (channels behind the tensor's pitch -- the chunk count is rounded up to four per wave -- read as zero)
             ok[i] = idx < G::TOTAL && (unsigned)gy < (unsigned)p.in_hp && (unsigned)gx < (unsigned)p.in_wp && ch_r + chunk * KC + g * 8 < p.in_cp;
+            ch_of[i] = ch_r + chunk * KC + g * 8;
             const store_t* src = in + (ok[i] ? (gy * p.in_wp + gx) * p.in_cp + ch_r + chunk * KC + g * 8 : 0);
             if constexpr (HSTORE) {
                 raw[i] = *reinterpret_cast<const half8_t*>(src);
@@ -1064,17 +1067,36 @@ __global__ __launch_bounds__(512) void conv_kr16_kernel(const ConvP16Params p) {
         // halves -- two values per instruction, no conversions)
         const _Float16 hlo = (_Float16)fmaxf(p.act.lo, -65504.f), hhi = (_Float16)fminf(p.act.hi, 65504.f);
         const bool half_act = HSTORE && p.act.leak == 0.f && (p.act.lo < -65504.f || (float)hlo == p.act.lo) && (p.act.hi > 65504.f || (float)hhi == p.act.hi);
+        // a batch-norm layer in front: x * in_mul[c] + in_add[c] on the item's eight channels (the arrays come through the L1)
+        const bool affine = p.in_mul != nullptr;
+        auto affine8 = [&](float (&x)[8], const int i) {
+            const int c = ok[i] ? ch_of[i] : 0;
+            const float4 m0 = *reinterpret_cast<const float4*>(p.in_mul + c), m1 = *reinterpret_cast<const float4*>(p.in_mul + c + 4);
+            const float4 a0 = *reinterpret_cast<const float4*>(p.in_add + c), a1 = *reinterpret_cast<const float4*>(p.in_add + c + 4);
+            const float m[8] = {m0.x, m0.y, m0.z, m0.w, m1.x, m1.y, m1.z, m1.w}, a[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
+#pragma unroll
+            for (int e = 0; e < 8; e++) x[e] = x[e] * m[e] + a[e];
+        };
         if (wait) lds_barrier();   // the MFMA waves are through with the round before: its place in the LDS is free
 #pragma unroll
         for (int i = 0; i < NB; i++) {
             if (l_off[i] < 0) continue;
             if constexpr (HSTORE) {
+                half8_t rv = raw[i];
+                if (affine) {
+                    float x[8];
+#pragma unroll
+                    for (int e = 0; e < 8; e++) x[e] = (float)rv[e];
+                    affine8(x, i);
+#pragma unroll
+                    for (int e = 0; e < 8; e++) rv[e] = (_Float16)x[e];   // (what the batch-norm layer would have stored)
+                }
                 half8_t v;
                 if (half_act) {
-                    v = ok[i] ? __builtin_elementwise_min(__builtin_elementwise_max(raw[i], (half8_t)hlo), (half8_t)hhi) : (half8_t)((_Float16)0.f);
+                    v = ok[i] ? __builtin_elementwise_min(__builtin_elementwise_max(rv, (half8_t)hlo), (half8_t)hhi) : (half8_t)((_Float16)0.f);
                 } else {
 #pragma unroll
-                    for (int e = 0; e < 8; e++) v[e] = ok[i] ? (_Float16)act_p16((float)raw[i][e], p.act) : (_Float16)0.f;
+                    for (int e = 0; e < 8; e++) v[e] = ok[i] ? (_Float16)act_p16((float)rv[e], p.act) : (_Float16)0.f;
                 }
                 *reinterpret_cast<half8_t*>(lds + l_off[i]) = v;
             }
@@ -1085,7 +1107,8 @@ __global__ __launch_bounds__(512) void conv_kr16_kernel(const ConvP16Params p) {
 #pragma unroll
                 for (int i = 0; i < NB; i++) {
                     if (l_off[i] < 0) continue;
-                    const float r[8] = {raw[i].a.x, raw[i].a.y, raw[i].a.z, raw[i].a.w, raw[i].b.x, raw[i].b.y, raw[i].b.z, raw[i].b.w};
+                    float r[8] = {raw[i].a.x, raw[i].a.y, raw[i].a.z, raw[i].a.w, raw[i].b.x, raw[i].b.y, raw[i].b.z, raw[i].b.w};
+                    if (affine) affine8(r, i);
                     half8_t hi, lo;
                     split8<KIND>(r, ok[i], p.act, in_scale, hi, lo);
                     *reinterpret_cast<half8_t*>(lds + l_off[i]) = hi;
@@ -1554,6 +1577,8 @@ int P16_NAME(launch_conv_kr16)(const ConvP16Params& p, int k, hipStream_t s) {
         return -5;
     // (a fused depthwise layer: its tensor has the pointwise layer's channels, in whole groups of 8, and the 1x1 layer does not step)
     if (p.dw_in && (!p.dw_w || !p.dw_scale || !p.dw_bias || p.dw_cp != p.in_cp || p.stride != 1 || p.in_clamp || p.dw_hp < 1 || p.dw_wp < 1)) return -5;
+    // (a batch-norm layer applied while staging: not beside a depthwise layer, and both arrays or none)
+    if ((p.in_mul != nullptr) != (p.in_add != nullptr) || (p.in_mul && p.dw_in)) return -5;
     if (e->lds > 160 * 1024) return -2;
     if (ensure_lds(reinterpret_cast<const void*>(e->fn), e->lds) != 0) return -2;
     hipLaunchKernelGGL(e->fn, dim3(p.tiles_x * p.tiles_y * p.cout_blocks), dim3(512), e->lds, s, p);

@@ -368,6 +368,7 @@ void Net::setup() {
         kv.second->set_up = true;
     }
     fuse_depthwise_layers(this);
+    fuse_batchnorm_layers(this);
     assign_range_resets();
     poison_lds_ = getenv("FYNHIP_POISON_LDS") != nullptr;
     FYN_HIP(hipStreamSynchronize(stream));

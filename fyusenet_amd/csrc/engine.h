@@ -177,6 +177,7 @@ class Net {
 };
 
 Layer* create_layer(Net* net, const fyn_layer_desc& d);
+void fuse_batchnorm_layers(Net* net);   // after every layer's setup(): batch-norm layers that their readers (K-resident convolutions) can apply while staging
 void fuse_depthwise_layers(Net* net);   // after every layer's setup(): depthwise 3x3 layers that their 1x1 reader can compute itself
 Layer* create_custom_layer(Net* net, const fyn_layer_desc& d, const fyn_custom_layer& impl);
 

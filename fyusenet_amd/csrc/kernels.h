@@ -209,6 +209,11 @@ struct ConvP16Params {
     const float* dw_bias;
     int dw_hp, dw_wp, dw_cp, dw_y0, dw_x0, dw_stride;
     Act dw_act;
+    // A batch-norm layer in front of the convolution applied while staging (launch_conv_kr16, and launch_conv_d16 on 1x1
+    // layers, without a depthwise layer; null: none): x * in_mul[channel] + in_add[channel] before the activation, `in` being the batch-norm layer's input;
+    // arrays of at least in_cp floats.  fp16 tensors: rounded to fp16 as the layer would have stored it.
+    const float* in_mul;
+    const float* in_add;
 };
 // Output channel held by row `row` (0..15) of packed weight fragment `mf` when a wave holds groups of `fm` fragments: the
 // rows a lane ends up with (four consecutive ones of every fragment) are 4*fm consecutive channels.

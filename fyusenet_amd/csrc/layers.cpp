@@ -1837,6 +1837,10 @@ class ConvLayer : public Layer {
             if ((d16 ? launch_conv_d16(with_depthwise(), s) : launch_conv_kr16(with_depthwise(), k, s)) != 0) fail(FYN_ERR_DEVICE, "layer %s: convolution launch failed", d.name);
             return;
         }
+        if (p16 && (kr16 || d16) && bn_fused && net->fusion_on()) {
+            if ((d16 ? launch_conv_d16(with_batchnorm(), s) : launch_conv_kr16(with_batchnorm(), k, s)) != 0) fail(FYN_ERR_DEVICE, "layer %s: convolution launch failed", d.name);
+            return;
+        }
         if (p16) {
             if ((c4 ? launch_conv_p16c4(pp, k, s) : (d16 ? launch_conv_d16(pp, s) : (kr16 ? launch_conv_kr16(pp, k, s) : (h16 ? launch_conv_h16(pp, k, s) : launch_conv_p16(pp, s))))) != 0 ||
                 (h16 && h16_two && launch_conv_h16(pp2, k, s) != 0))
@@ -1877,6 +1881,7 @@ class ConvLayer : public Layer {
                      pp.f16 ? "f16" : "f16x2-split", (pp.tile_h ? "KxK on four-channel pixels (steps of eight taps)" : "1x1"), (pp.wm == 4 ? "a wave per 16 positions and fragment" : (std::to_string(pp.cout_blocks) + " workgroup(s) of 4 waves per 16 positions").c_str()),
                      pp.cin_chunks, pp.mfrags, (pp.npos_y * pp.npos_x + 16 * pp.wm - 1) / (16 * pp.wm) * pp.cout_blocks);
             if (dw_fused) return mode + buf + "; the depthwise 3x3 layer " + std::to_string(dw_layer_no) + " in front of it is computed by the waves themselves";
+            if (bn_fused) return mode + buf + "; the batch-norm layer " + std::to_string(bn_layer_no) + " in front of it is applied on fetch";
             return mode + buf;
         }
         if (p16 && kr16) {
@@ -1884,6 +1889,7 @@ class ConvLayer : public Layer {
             snprintf(buf, sizeof(buf), "conv_kr16 %s tile=%dx%d(cout x pos) K-resident, 4 waves split %d chunks, blocks=%d lds=%zu steps=%d", pp.f16 ? "f16" : "f16x2-split",
                      16 * pp.wm, pp.tile_h * pp.tile_w, pp.cin_chunks, pp.pos_groups * pp.cout_blocks, conv_kr16_lds_bytes(pp, k), pp.cin_chunks / 4 * k * k);
             if (dw_fused) return mode + buf + "; the depthwise 3x3 layer " + std::to_string(dw_layer_no) + " in front of it is computed by the staging waves";
+            if (bn_fused) return mode + buf + "; the batch-norm layer " + std::to_string(bn_layer_no) + " in front of it is applied while staging";
             return mode + buf;
         }
         if (p16 && h16) {
@@ -1942,6 +1948,19 @@ class ConvLayer : public Layer {
         q.dw_y0 = dw_fields.dw_y0; q.dw_x0 = dw_fields.dw_x0; q.dw_stride = dw_fields.dw_stride; q.dw_act = dw_fields.dw_act;
         return q;
     }
+    // A batch-norm layer in front of this layer applied while the K-resident form stages its tile or the LDS-free 1x1
+    // form fetches its fragments (fuse_batchnorm_layers below): the layer's input tensor -- same geometry as its output -- and its scale / bias arrays.
+    bool bn_fused = false;
+    int bn_layer_no = -1;
+    const void* bn_in = nullptr;
+    const float *bn_mul = nullptr, *bn_add = nullptr;
+    ConvP16Params with_batchnorm() const {
+        ConvP16Params q = pp;
+        q.in = bn_in; q.in_mul = bn_mul; q.in_add = bn_add;
+        q.in_amax = nullptr;   // (the batch-norm layer keeps no value-range word: its readers stage unscaled either way)
+        return q;
+    }
+    bool takes_batchnorm() const { return p16 && (kr16 || (d16 && k == 1)) && !dw_fused && !edw_fused && !pp.in_amax; }
     bool takes_depthwise() const {
         return p16 && ((kr16 && pp.tile_h == 4 && pp.tile_w == 4) || d16) && k == 1 && stride == 1 && !clamp && !pp.in_amax && !pp.in_clamp;
     }
@@ -2050,6 +2069,8 @@ void fuse_depthwise_layers(Net* net) {
         ConvLayer* ex = dynamic_cast<ConvLayer*>(net->layer(t.producer));
         if (!ex || ex->k != 1 || ex->stride != 1 || ex->dil != 1 || ex->clamp || ex->frac_shift || ex->direct || (ex->d.flags & FYN_FLAG_RESIDUAL_INPUT)) continue;
         const TView& in_v = ex->tin(0).v;
+        // (the launch reads the 1x1 layer's input while it writes the depthwise layer's output: not in one buffer)
+        if (net->tensors[dw->out].buffer == net->tensors[ex->in[0]].buffer) continue;
         if (in_v.f16 != dw->p.out.f16 || ex->d.in_channels != in_v.cp || ex->tout().v.cp != dw->p.in.cp || ex->oc % 4 != 0 ||
             !conv_e16dw_supported(in_v.cp, (in_v.cp + 31) / 32, dw->stride))
             continue;
@@ -2129,6 +2150,8 @@ void fuse_depthwise_layers(Net* net) {
         if (!dw || dw->dil != 1 || (dw->stride != 1 && dw->stride != 2) || dw->p.res.ptr || dw->p.in.cp % 8 != 0 || dw->p.in.cp != dw->p.out.cp ||
             dw->p.in.f16 != dw->p.out.f16 || dw->p.out.f16 != pw->pp.f16 || dw->p.out.cp != pw->pp.in_cp)
             continue;
+        // (the launch reads the depthwise layer's input while it writes the 1x1 layer's output: not in one buffer)
+        if (net->tensors[pw->out].buffer == net->tensors[dw->in[0]].buffer) continue;
         ConvP16Params& f = pw->dw_fields;
         f.dw_in = dw->p.in.ptr; f.dw_w = dw->w_dev; f.dw_scale = dw->scale_dev; f.dw_bias = dw->bias_dev;
         f.dw_hp = dw->p.in.hp(); f.dw_wp = dw->p.in.wp(); f.dw_cp = dw->p.in.cp;
@@ -2546,14 +2569,61 @@ class BatchNormLayer : public Layer {
     }
     void forward(hipStream_t s) override {
         if (!have_weights) fail(FYN_ERR_STATE, "layer %s (%d): forward() without scale/bias", d.name, d.number);
+        if (fused_into >= 0 && net->fusion_on()) return;   // applied by the convolution layers that read it
         launch_batchnorm(p, s);
     }
-    std::string info() const override { return "batchnorm"; }
+    std::string info() const override {
+        return fused_into >= 0 ? "batchnorm (runs inside the launch of layer " + std::to_string(fused_into) + "; no launch of its own)" : "batchnorm";
+    }
+    int fused_into = -1;
     bool have_weights = false;
     std::vector<float> block;
     BnParams p{};
     float *scale_dev = nullptr, *bias_dev = nullptr;
 };
+
+// Batch-norm layers whose readers can apply them: a plain x * scale + bias (no activation, no residual input) between
+// tensors of one geometry without a halo, read only by convolution layers on the K-resident or the LDS-free 1x1 form, as
+// their data input.  Each reader then fetches from the batch-norm layer's input and applies scale and bias per channel
+// before its own activation; the layer's output is never written and its launch is gone (the reference's ResNet-50 sample graph has one such layer in
+// front of most blocks).  The input tensor must still hold its values when the last reader runs: no tensor produced
+// between the batch-norm layer and that reader may live in the same buffer.
+void fuse_batchnorm_layers(Net* net) {
+    if (getenv("FYNHIP_NO_BN_FUSION") || !net->reuse_buffers) return;
+    for (auto& kv : net->layers) {
+        BatchNormLayer* bn = dynamic_cast<BatchNormLayer*>(kv.second.get());
+        if (!bn || bn->p.res.ptr || bn->p.act.kind != ACT_NONE) continue;
+        Tensor& x = net->tensors[bn->in[0]];
+        const Tensor& y = net->tensors[bn->out];
+        // (no halo: around the layer's output it holds zeros, which scale and bias applied to the input's halo would not give)
+        if (y.locked || x.v.pad != 0 || y.v.pad != 0 || x.v.h != y.v.h || x.v.w != y.v.w || x.v.cp != y.v.cp || x.v.f16 != y.v.f16 || x.v.c != y.v.c) continue;
+        std::vector<ConvLayer*> readers;
+        bool all = true;
+        int last = -1;
+        for (auto& kr : net->layers) {
+            Layer* l = kr.second.get();
+            for (size_t port = 0; port < l->in.size(); port++) {
+                if (l->in[port] != bn->out) continue;
+                ConvLayer* c = dynamic_cast<ConvLayer*>(l);
+                if (!c || port != 0 || !c->takes_batchnorm() || c->d.number <= bn->d.number) { all = false; continue; }
+                readers.push_back(c);
+                last = std::max(last, c->d.number);
+            }
+        }
+        if (!all || readers.empty()) continue;
+        bool live = true;
+        for (const Tensor& o : net->tensors)
+            if (&o != &x && o.buffer == x.buffer && o.producer > bn->d.number && o.producer <= last) live = false;
+        if (!live) continue;
+        for (ConvLayer* c : readers) {
+            c->bn_fused = true;
+            c->bn_layer_no = bn->d.number;
+            c->bn_in = x.v.ptr; c->bn_mul = bn->scale_dev; c->bn_add = bn->bias_dev;
+        }
+        bn->fused_into = readers.front()->d.number;
+        x.last_reader = std::max(x.last_reader, last);   // (its value-range word is cleared behind its last reader)
+    }
+}
 
 class AddSubLayer : public Layer {
   public:
