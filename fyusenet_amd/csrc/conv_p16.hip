@@ -982,7 +982,10 @@ __global__ __launch_bounds__(512) void conv_kr16_kernel(const ConvP16Params p) {
     const int tile = blockIdx.x / p.cout_blocks;
     const int tyi = tile / p.tiles_x, txi = tile - tyi * p.tiles_x;
     if (tid < 2) range_box[tid] = 0u;
-    const unsigned range_bits = p.in_amax ? range_load(p.in_amax) : 0u;
+    // (two source tensors: the larger of their value ranges scales both, or nothing is scaled when one keeps no word)
+    const bool ranged = p.in_amax && (!p.in2 || p.in2_amax);
+    unsigned range_bits = ranged ? range_load(p.in_amax) : 0u;
+    if (ranged && p.in2) range_bits = max(range_bits, range_load(p.in2_amax));
     constexpr int red_off = G::RED_OFF;
     constexpr int sb_off = red_off + 3 * FM * FN * 1024;
     // Staging waves: the four that only stage, and -- without a depthwise layer in front -- the four MFMA waves too,
@@ -1021,6 +1024,18 @@ __global__ __launch_bounds__(512) void conv_kr16_kernel(const ConvP16Params p) {
             const int l0 = chunk0 * G::BUFC + py * G::ROW_PITCH + px * G::PIT + g * 16;
             const int c0 = ch_r + chunk0 * KC + g * 8;
             const store_t* src0 = in + (inb ? (gy * p.in_wp + gx) * p.in_cp : 0) + c0;
+            // the second source tensor (1x1 layers): the same pixel of the tile at that tensor's own step, origin and pitch
+            [[maybe_unused]] bool inb2 = false;
+            [[maybe_unused]] const store_t* src2 = in;
+            [[maybe_unused]] int c2 = 0;
+            if constexpr (NTAPS == 1 && R == 1) {
+                if (p.in2) {
+                    const int gy2 = (tyi * G::TH + py) * p.in2_stride + p.in2_y0, gx2 = (txi * G::TW + px) * p.in2_stride + p.in2_x0;
+                    inb2 = (unsigned)gy2 < (unsigned)p.in2_hp && (unsigned)gx2 < (unsigned)p.in2_wp;
+                    c2 = (chunk0 - p.in2_chunk0) * KC + g * 8;   // (negative for the chunks of the first tensor)
+                    src2 = reinterpret_cast<const store_t*>(p.in2) + (inb2 ? (gy2 * p.in2_wp + gx2) * p.in2_cp : 0) + c2;
+                }
+            }
 #pragma unroll
             for (int i = 0; i < NB; i++) {
                 const bool in_tile = chunk0 + i * CPI < G::NCH;
@@ -1029,6 +1044,12 @@ __global__ __launch_bounds__(512) void conv_kr16_kernel(const ConvP16Params p) {
                 ok[i] = in_tile && inb && c0 + i * CPI * KC < p.in_cp;
                 ch_of[i] = c0 + i * CPI * KC;
                 const store_t* src = ok[i] ? src0 + i * CPI * KC : in;
+                if constexpr (NTAPS == 1 && R == 1) {
+                    if (p.in2 && chunk0 + i * CPI >= p.in2_chunk0) {
+                        ok[i] = in_tile && inb2 && c2 + i * CPI * KC < p.in2_cp;
+                        src = ok[i] ? src2 + i * CPI * KC : in;
+                    }
+                }
                 if constexpr (HSTORE) {
                     raw[i] = *reinterpret_cast<const half8_t*>(src);
                 } else {
@@ -1062,7 +1083,7 @@ __global__ __launch_bounds__(512) void conv_kr16_kernel(const ConvP16Params p) {
         }
         }
         float in_scale = 1.f, inv_unused;
-        if (p.in_amax) in_scale = range_scale(range_after_act(range_reduce(range_bits), p.act), &inv_unused);
+        if (ranged) in_scale = range_scale(range_after_act(range_reduce(range_bits), p.act), &inv_unused);
         // (fp16 tensors: no activation, or a clamp without leak whose bounds are fp16 values, is applied to the packed
         // halves -- two values per instruction, no conversions)
         const _Float16 hlo = (_Float16)fmaxf(p.act.lo, -65504.f), hhi = (_Float16)fminf(p.act.hi, 65504.f);
@@ -1287,7 +1308,7 @@ __global__ __launch_bounds__(512) void conv_kr16_kernel(const ConvP16Params p) {
 #pragma unroll
         for (int fn = 0; fn < FN; fn++) acc[fm][fn] = (f32x4_t)(0.f);
     float inv_in_scale = 1.f;
-    if (p.in_amax) (void)range_scale(range_after_act(range_reduce(range_bits), p.act), &inv_in_scale);
+    if (ranged) (void)range_scale(range_after_act(range_reduce(range_bits), p.act), &inv_in_scale);
     const float acc_mul = p.acc_mul * inv_in_scale;
     // The residual values of the epilogue (wave 0) are requested here, so that their memory round trip passes under the
     // staging and the step stream instead of behind them (small tiles: the registers are there).
@@ -1579,6 +1600,10 @@ int P16_NAME(launch_conv_kr16)(const ConvP16Params& p, int k, hipStream_t s) {
     if (p.dw_in && (!p.dw_w || !p.dw_scale || !p.dw_bias || p.dw_cp != p.in_cp || p.stride != 1 || p.in_clamp || p.dw_hp < 1 || p.dw_wp < 1)) return -5;
     // (a batch-norm layer applied while staging: not beside a depthwise layer, and both arrays or none)
     if ((p.in_mul != nullptr) != (p.in_add != nullptr) || (p.in_mul && p.dw_in)) return -5;
+    // (a second source tensor: 1x1 in one round, the first tensor's channels end where the second's chunks begin)
+    if (p.in2 && (k != 1 || e->rounds != 1 || p.dw_in || p.in_mul || p.in_clamp || p.in2_chunk0 < 1 || p.in2_chunk0 >= p.cin_chunks || p.in_cp > p.in2_chunk0 * KC ||
+                  p.in2_cp % 8 != 0 || p.in2_cp < 8 || p.in2_cp > (p.cin_chunks - p.in2_chunk0) * KC || p.in2_stride < 1 || p.in2_hp < 1 || p.in2_wp < 1 || p.in2_y0 < 0 || p.in2_x0 < 0))
+        return -5;
     if (e->lds > 160 * 1024) return -2;
     if (ensure_lds(reinterpret_cast<const void*>(e->fn), e->lds) != 0) return -2;
     hipLaunchKernelGGL(e->fn, dim3(p.tiles_x * p.tiles_y * p.cout_blocks), dim3(512), e->lds, s, p);

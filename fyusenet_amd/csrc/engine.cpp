@@ -315,6 +315,7 @@ void Net::setup() {
             tensors[l->out].locked = true;
         }
     }
+    keep_projection_inputs(this);
     // 2. device buffers.  Liveness rule of BufferManager::findTexture (base/buffermanager.cpp:512-525)
     //    restated for in-order stream execution: a buffer can take layer N's output when every reader of
     //    its current tenant has a number < N; only buffers of identical geometry are shared so that the
@@ -368,6 +369,7 @@ void Net::setup() {
         kv.second->set_up = true;
     }
     fuse_depthwise_layers(this);
+    fuse_projection_layers(this);
     fuse_batchnorm_layers(this);
     assign_range_resets();
     poison_lds_ = getenv("FYNHIP_POISON_LDS") != nullptr;

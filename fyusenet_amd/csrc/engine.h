@@ -178,6 +178,8 @@ class Net {
 
 Layer* create_layer(Net* net, const fyn_layer_desc& d);
 void fuse_batchnorm_layers(Net* net);   // after every layer's setup(): batch-norm layers that their readers (K-resident convolutions) can apply while staging
+void keep_projection_inputs(Net* net);    // before buffers are assigned: inputs of such projections live until the layer that may compute them has run
+void fuse_projection_layers(Net* net);   // after every layer's setup(): 1x1 shortcut projections that the 1x1 layer adding them can compute in its own launch
 void fuse_depthwise_layers(Net* net);   // after every layer's setup(): depthwise 3x3 layers that their 1x1 reader can compute itself
 Layer* create_custom_layer(Net* net, const fyn_layer_desc& d, const fyn_custom_layer& impl);
 

@@ -214,6 +214,13 @@ struct ConvP16Params {
     // arrays of at least in_cp floats.  fp16 tensors: rounded to fp16 as the layer would have stored it.
     const float* in_mul;
     const float* in_add;
+    // A reduction over two tensors (launch_conv_kr16, 1x1, one round, no depthwise or batch-norm layer in front; in2
+    // null: none): chunks from in2_chunk0 on read in2 -- its own pitch, step and origin, the same activation -- at the
+    // position's pixel (y, x) * in2_stride + (in2_y0, in2_x0).  A 1x1 layer and the 1x1 projection whose result it
+    // adds run as one launch this way.  in2_amax: that tensor's value-range word (both or none are used).
+    const void* in2;
+    int in2_hp, in2_wp, in2_cp, in2_y0, in2_x0, in2_stride, in2_chunk0;
+    const unsigned* in2_amax;
 };
 // Output channel held by row `row` (0..15) of packed weight fragment `mf` when a wave holds groups of `fm` fragments: the
 // rows a lane ends up with (four consecutive ones of every fragment) are 4*fm consecutive channels.

@@ -870,7 +870,7 @@ class ConvLayer : public Layer {
         pp.out_amax = out_w;
     }
     bool add_range_reset(unsigned* w) override {
-        if (direct || !set_up) return false;
+        if (direct || !set_up || pj_into >= 0) return false;   // (a projection computed by its reader has no launch to clear words in)
         int& n = rows ? rp.nreset : (p16 ? pp.nreset : launch.p.nreset);
         if (n >= 4) return false;
         (rows ? rp.reset : (p16 ? pp.reset : launch.p.reset))[n++] = w;
@@ -1805,6 +1805,8 @@ class ConvLayer : public Layer {
         }
         if (edw_fused) pack_edw();
         have_weights = true;
+        if (pj_fused) pack_two_sources();
+        if (pj_into >= 0) static_cast<ConvLayer*>(net->layer(pj_into))->pack_two_sources();
     }
     // the weights once more, in the layout of the launch that also runs the depthwise layer behind this one
     void pack_edw() {
@@ -1816,6 +1818,19 @@ class ConvLayer : public Layer {
     }
     void forward(hipStream_t s) override {
         if (!have_weights) fail(FYN_ERR_STATE, "layer %s (%d): forward() without weights", d.name, d.number);
+        if (pj_into >= 0 && net->fusion_on()) return;   // computed by the layer that adds it
+        if (pj_fused && net->fusion_on()) {
+            ConvP16Params q = pj;   // (value-range words as the layer's own launch carries them)
+            q.in_amax = tin(0).amax;
+            q.in2_amax = net->layer(pj_layer_no)->tin(0).amax;
+            q.out_amax = tout().amax;
+            const int n = rows ? rp.nreset : (p16 ? pp.nreset : launch.p.nreset);
+            unsigned* const* r = rows ? rp.reset : (p16 ? pp.reset : launch.p.reset);
+            q.nreset = n;
+            for (int i = 0; i < n; i++) q.reset[i] = r[i];
+            if (launch_conv_kr16(q, 1, s) != 0) fail(FYN_ERR_DEVICE, "layer %s: convolution launch failed", d.name);
+            return;
+        }
         if (edw_fused && net->fusion_on()) {
             ConvP16Params q = edw;   // (value-range words as the layer's own launch carries them)
             q.in_amax = tin(0).amax;
@@ -1853,6 +1868,13 @@ class ConvLayer : public Layer {
         if (wide && !fused) launch_shift_reduce(sr, s);
     }
     std::string info() const override {
+        if (pj_into >= 0) return "conv 1x1 projection (runs inside the launch of layer " + std::to_string(pj_into) + "; no launch of its own); apart: " + own_info();
+        if (pj_fused) {
+            char buf[300];
+            snprintf(buf, sizeof(buf), "conv_kr16 %s tile=%dx16(cout x pos) K-resident over two tensors, 4 waves split %d chunks (%d of them of the 1x1 projection %d, whose result the layer adds), blocks=%d lds=%zu; apart: ",
+                     pj.f16 ? "f16" : "f16x2-split", 16 * pj.wm, pj.cin_chunks, pj.cin_chunks - pj.in2_chunk0, pj_layer_no, pj.pos_groups * pj.cout_blocks, conv_kr16_lds_bytes(pj, 1));
+            return buf + own_info();
+        }
         if (edw_fused)
             return "conv_e16dw " + std::string(edw.f16 ? "f16" : "f16x2-split") + " 1x1 and the depthwise 3x3 layer " + std::to_string(edw_dw_no) +
                    " behind it in one launch: a workgroup per 4x4 output positions and " + (edw.wm == 2 ? "16" : "64") + " expanded channels, blocks=" +
@@ -1960,7 +1982,68 @@ class ConvLayer : public Layer {
         q.in_amax = nullptr;   // (the batch-norm layer keeps no value-range word: its readers stage unscaled either way)
         return q;
     }
-    bool takes_batchnorm() const { return p16 && (kr16 || (d16 && k == 1)) && !dw_fused && !edw_fused && !pp.in_amax; }
+    bool takes_batchnorm() const { return p16 && (kr16 || (d16 && k == 1)) && !dw_fused && !edw_fused && !pj_fused && pj_into < 0 && !pp.in_amax; }
+    // A 1x1 projection whose result this 1x1 layer adds (its residual input) computed in the layer's own launch, as one
+    // reduction over two tensors (fuse_projection_layers below): the rows of both weight matrices carry their layers'
+    // folded scales, the bias is the sum of both, and the projection's tensor is never written.
+    bool pj_fused = false;
+    int pj_layer_no = -1;   // the projection this layer computes
+    int pj_into = -1;       // on the projection: the layer that computes it
+    ConvP16Params pj{};
+    void* pj_wpack_dev = nullptr;
+    float *pj_scale_dev = nullptr, *pj_bias_dev = nullptr;
+    void pack_two_sources() {
+        ConvLayer* P = static_cast<ConvLayer*>(net->layer(pj_layer_no));
+        if (block.empty() || P->block.empty()) return;
+        const int c1 = d.in_channels, c2 = P->d.in_channels, n1 = pj.in2_chunk0, fm_n = pj.wm, npl = pj.f16 ? 1 : 2, steps = pj.cin_chunks / 4;
+        const float *b1 = block.data(), *w1 = b1 + oc, *bn1 = w1 + (size_t)oc * c1;
+        const float *b2 = P->block.data(), *w2 = b2 + oc, *bn2 = w2 + (size_t)oc * c2;
+        std::vector<float> s1, o1, s2, o2;
+        fold_bn(b1, bn1, oc, (d.flags & FYN_FLAG_POST_BATCHNORM) != 0, oc, s1, o1);
+        fold_bn(b2, bn2, oc, (P->d.flags & FYN_FLAG_POST_BATCHNORM) != 0, oc, s2, o2);
+        // (batch-norm on the residual: the layer's scale multiplies what it adds, convlayerbase's residual variant)
+        const bool rs = (d.flags & FYN_FLAG_BATCHNORM_ON_RESIDUAL) && (d.flags & FYN_FLAG_POST_BATCHNORM);
+        std::vector<float> wa((size_t)oc * c1), wb((size_t)oc * c2), ones(padded, 0.f), bias(padded, 0.f);
+        float mx = 0.f;
+        for (int o = 0; o < oc; o++) {
+            const float r2 = rs ? s1[o] * s2[o] : s2[o];
+            for (int i = 0; i < c1; i++) mx = std::max(mx, std::fabs(wa[(size_t)o * c1 + i] = w1[(size_t)o * c1 + i] * s1[o]));
+            for (int i = 0; i < c2; i++) mx = std::max(mx, std::fabs(wb[(size_t)o * c2 + i] = w2[(size_t)o * c2 + i] * r2));
+            ones[o] = 1.f;
+            bias[o] = o1[o] + (rs ? s1[o] * o2[o] : o2[o]);
+        }
+        const float wmul = weight_prescale(&mx, 1);
+        pj.acc_mul = 1.0f / wmul;
+        std::vector<uint16_t> pack((size_t)pj.cout_blocks * 4 * steps * fm_n * npl * 64 * 8, 0);
+        for (int cb = 0; cb < pj.cout_blocks; cb++)
+            for (int wv = 0; wv < 4; wv++)
+                for (int st = 0; st < steps; st++) {
+                    const int chunk = wv + 4 * st;
+                    const bool second = chunk >= n1;
+                    const float* src = second ? wb.data() : wa.data();
+                    const int cn = second ? c2 : c1, cbase = (second ? chunk - n1 : chunk) * 32;
+                    for (int fm = 0; fm < fm_n; fm++) {
+                        uint16_t* base = pack.data() + ((((size_t)(cb * 4 + wv) * steps + st) * fm_n + fm) * npl) * 64 * 8;
+                        for (int lane = 0; lane < 64; lane++) {
+                            const int o = (cb * fm_n + fm) * 16 + (lane & 15);
+                            if (o >= oc) continue;
+                            for (int j = 0; j < 8; j++) {
+                                const int ci = cbase + 8 * (lane >> 4) + j;
+                                if (ci >= cn) continue;
+                                const float v = src[(size_t)o * cn + ci] * wmul;
+                                const uint16_t hi = f2h_bits(v);
+                                base[(size_t)lane * 8 + j] = hi;
+                                if (npl == 2) base[(size_t)(64 + lane) * 8 + j] = f2h_bits(v - h2f(hi));
+                            }
+                        }
+                    }
+                }
+        reupload(net, pj_scale_dev, ones);
+        reupload(net, pj_bias_dev, bias);
+        FYN_HIP(hipStreamSynchronize(net->stream));
+        FYN_HIP(hipMemcpyAsync(pj_wpack_dev, pack.data(), pack.size() * 2, hipMemcpyHostToDevice, net->stream));
+        FYN_HIP(hipStreamSynchronize(net->stream));
+    }
     bool takes_depthwise() const {
         return p16 && ((kr16 && pp.tile_h == 4 && pp.tile_w == 4) || d16) && k == 1 && stride == 1 && !clamp && !pp.in_amax && !pp.in_clamp;
     }
@@ -2185,6 +2268,151 @@ void fuse_depthwise_layers(Net* net) {
         pw->dw_fused = true;
         pw->dw_layer_no = dw->d.number;
         dw->fused_into = pw->d.number;
+    }
+}
+
+// The projection that layer `c` could compute itself (fuse_projection_layers below), by the graph alone: `c` a 1x1 layer
+// without step that adds, unactivated, the result of a 1x1 layer nothing else reads.
+static ConvLayer* projection_of(Net* net, ConvLayer* c) {
+    if (!c || c->k != 1 || c->stride != 1 || c->dil != 1 || c->clamp || c->frac_shift || c->direct || !(c->d.flags & FYN_FLAG_RESIDUAL_INPUT) ||
+        (c->d.flags & FYN_FLAG_RELU_ON_RESIDUAL) || c->in.size() < 2 || c->in[1] < 0 || c->in[0] == c->in[1])
+        return nullptr;
+    const Tensor& rt = net->tensors[c->in[1]];
+    if (rt.producer < 0 || rt.locked) return nullptr;
+    int readers = 0;
+    for (auto& kv : net->layers)
+        for (int t : kv.second->in) readers += t == c->in[1];
+    if (readers != 1) return nullptr;
+    ConvLayer* pr = dynamic_cast<ConvLayer*>(net->layer(rt.producer));
+    if (!pr || pr->k != 1 || pr->dil != 1 || pr->clamp || pr->frac_shift || pr->direct || (pr->d.flags & FYN_FLAG_RESIDUAL_INPUT) || pr->oc != c->oc ||
+        pr->d.number >= c->d.number || pr->in.empty() || pr->in[0] < 0)
+        return nullptr;
+    return pr;
+}
+// Before buffers are assigned: the input of such a projection stays whole until the layer that may compute it has run
+// (a few more buffers in networks with such pairs, whether the pair is joined in the end or not).
+void keep_projection_inputs(Net* net) {
+    if (getenv("FYNHIP_NO_PROJECTION_FUSION") || !net->reuse_buffers) return;
+    for (auto& kv : net->layers) {
+        ConvLayer* c = dynamic_cast<ConvLayer*>(kv.second.get());
+        ConvLayer* pr = projection_of(net, c);
+        if (!pr) continue;
+        Tensor& x2 = net->tensors[pr->in[0]];
+        x2.last_reader = std::max(x2.last_reader, c->d.number);
+    }
+}
+// A 1x1 projection (a residual block's shortcut convolution) whose only reader adds it to its own 1x1 convolution: both
+// are sums over channels at the same output position, so they run as ONE reduction over two tensors on the K-resident
+// form -- the projection's chunks behind the layer's own, each weight row carrying its layer's folded scale -- and the
+// projection's tensor is never written.  Conditions: both 1x1 without dilation on tensors of one storage type, the same
+// activation on fetch, no activation on the residual, the projection's input still whole when the reader runs, and a
+// compiled variant for the joint chunk count; timed against the two launches.
+void fuse_projection_layers(Net* net) {
+    if (getenv("FYNHIP_NO_PROJECTION_FUSION") || getenv("FYNHIP_NO_P16_CONV") || getenv("FYNHIP_NO_KR16_CONV") || !net->reuse_buffers) return;
+    const char* at = getenv("FYNHIP_AUTOTUNE");
+    for (auto& kv : net->layers) {
+        ConvLayer* c = dynamic_cast<ConvLayer*>(kv.second.get());
+        ConvLayer* pr = projection_of(net, c);
+        if (!pr || c->dw_fused || c->edw_fused || c->bn_fused || pr->dw_fused || pr->edw_fused || pr->bn_fused || pr->pj_fused || pr->pj_into >= 0) continue;
+        const Tensor& rt = net->tensors[c->in[1]];
+        const Act a1 = c->act(), a2 = pr->act();
+        if (a1.kind != a2.kind || a1.lo != a2.lo || a1.hi != a2.hi || a1.leak != a2.leak) continue;
+        const TView& v1 = c->tin(0).v;
+        const TView& v2 = pr->tin(0).v;
+        const TView& ov = c->tout().v;
+        Tensor& x2 = net->tensors[pr->in[0]];
+        if (v1.f16 != ov.f16 || v2.f16 != ov.f16 || rt.v.f16 != ov.f16 || c->d.in_channels != v1.cp || pr->d.in_channels != v2.cp || v1.cp % 8 != 0 || v2.cp % 8 != 0 ||
+            v1.cp < 8 || v2.cp < 8 || c->oc % 4 != 0 || c->oc < 8 || ov.cp < c->oc || c->oh * c->ow > 4096)
+            continue;
+        bool live = true;   // (the projection's input must still hold its values when the reader runs)
+        for (const Tensor& o : net->tensors)
+            if (&o != &x2 && o.buffer == x2.buffer && o.producer > pr->d.number && o.producer <= c->d.number) live = false;
+        if (!live) continue;
+        const int n1 = (v1.cp + 31) / 32, n2 = (v2.cp + 31) / 32;
+        ConvP16Params q{};
+        q.in = v1.ptr; q.out = ov.ptr;
+        q.in_hp = v1.hp(); q.in_wp = v1.wp(); q.in_cp = v1.cp;
+        q.stride = 1; q.in_y0 = q.in_x0 = v1.pad;
+        q.in2 = v2.ptr; q.in2_hp = v2.hp(); q.in2_wp = v2.wp(); q.in2_cp = v2.cp;
+        q.in2_stride = pr->stride; q.in2_y0 = q.in2_x0 = v2.pad; q.in2_chunk0 = n1;
+        q.npos_y = c->oh; q.npos_x = c->ow;
+        q.out_wp = ov.wp(); q.out_cp = ov.cp; q.out_off_y = q.out_off_x = ov.pad;
+        q.f16 = ov.f16 ? 1 : 0;
+        q.acc_mul = 1.f;
+        q.act = a1;
+        q.tile_h = q.tile_w = 4;
+        q.tiles_x = (c->ow + 3) / 4; q.tiles_y = (c->oh + 3) / 4;
+        q.rcp_tiles_x = 1.0f / (float)q.tiles_x;
+        q.pos_groups = q.tiles_x * q.tiles_y;
+        // (the last pixel either tensor is read at lies inside it)
+        if ((c->oh - 1) * pr->stride + v2.pad >= v2.hp() || (c->ow - 1) * pr->stride + v2.pad >= v2.wp()) continue;
+        // the joint chunk count, rounded up to the next one a variant is compiled for (the chunks behind both tensors read as zero)
+        int chunks = 0;
+        for (int n = (n1 + n2 + 3) / 4 * 4; n <= 64 && !chunks; n += 4) {
+            ConvP16Params t = q;
+            t.cin_chunks = n; t.wm = 1; t.cout_blocks = (c->oc + 15) / 16; t.mfrags = t.cout_blocks;
+            if (conv_kr16_lds_bytes(t, 1) != 0) chunks = n;
+        }
+        if (!chunks) continue;
+        q.cin_chunks = chunks;
+        std::vector<ConvP16Params> cands;
+        for (int fm : {1, 2}) {
+            if (fm == 2 && c->oc % 32 != 0 && c->oc % 32 <= 16) continue;
+            ConvP16Params t = q;
+            t.wm = fm;
+            t.cout_blocks = (c->oc + 16 * fm - 1) / (16 * fm);
+            t.mfrags = t.cout_blocks * fm;
+            const size_t lds = conv_kr16_lds_bytes(t, 1);
+            if (lds == 0 || lds > 160 * 1024 || (long long)t.pos_groups * t.cout_blocks > 65535) continue;
+            cands.push_back(t);
+        }
+        if (cands.empty()) continue;
+        const size_t halves = (size_t)((c->oc + 31) / 32 * 2) * 4 * (chunks / 4) * (q.f16 ? 1 : 2) * 64 * 8;
+        void* const wp = net->dev_alloc(halves * 2, true);
+        float* const sc = static_cast<float*>(net->dev_alloc(c->padded * sizeof(float), true));
+        float* const bi = static_cast<float*>(net->dev_alloc(c->padded * sizeof(float), true));
+        for (ConvP16Params& t : cands) { t.wpack = wp; t.scale = sc; t.bias = bi; }
+        int pick = 0;
+        bool win = true;
+        char key[200];
+        snprintf(key, sizeof(key), "pj:%d:%dand%dto%d:%dx%d:s%d", q.f16, v1.cp, v2.cp, c->oc, c->oh, c->ow, pr->stride);
+        int cached[3] = {0, 0, 0};
+        if (getenv("FYNHIP_FORCE_PROJECTION_FUSION")) {
+        } else if (tune_cache_triple(key, cached)) {
+            win = cached[0] != 0;
+            for (size_t i = 0; i < cands.size(); i++)
+                if (cands[i].wm == cached[1]) pick = (int)i;
+        } else if (!(at && at[0] == '0')) {
+            float t_fused = 1e30f, t_two = 1e30f;
+            for (int rep = 0; rep < 3; rep++) {
+                for (size_t i = 0; i < cands.size(); i++) {
+                    const float t = time_calls(net, [&]() {
+                        if (launch_conv_kr16(cands[i], 1, net->stream) != 0) fail(FYN_ERR_DEVICE, "1x1 convolution over two tensors: launch failed while tuning");
+                    }, 10);
+                    if (t < t_fused) { t_fused = t; pick = (int)i; }
+                }
+                t_two = std::min(t_two, time_calls(net, [&]() {
+                    pr->run(net->stream);
+                    c->run(net->stream);
+                }, 10));
+            }
+            if (getenv("FYNHIP_TUNE_VERBOSE"))
+                fprintf(stderr, "[tune] 1x1 on %d channels + 1x1 projection on %d (step %d) to %d at %dx%d: one launch %.1f us, two %.1f us\n", v1.cp, v2.cp, pr->stride, c->oc,
+                        c->oh, c->ow, t_fused * 1e3f, t_two * 1e3f);
+            win = t_fused < t_two;
+            tune_cache_store_triple(key, win ? 1 : 0, cands[pick].wm, 0);
+        }
+        if (!win) {
+            net->dev_free(wp); net->dev_free(sc); net->dev_free(bi);
+            continue;
+        }
+        c->pj = cands[pick];
+        c->pj_wpack_dev = wp; c->pj_scale_dev = sc; c->pj_bias_dev = bi;
+        c->pj_fused = true;
+        c->pj_layer_no = pr->d.number;
+        pr->pj_into = c->d.number;
+        x2.last_reader = std::max(x2.last_reader, c->d.number);   // (its value-range word is cleared behind its last reader)
+        c->pack_two_sources();
     }
 }
 

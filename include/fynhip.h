@@ -249,8 +249,9 @@ int fyn_net_enable_intermediate_output(fyn_net* net, const char* dir);
  * BufferManager::findTexture, base/buffermanager.cpp:512-525).  On by default; switch off before
  * fyn_net_setup to keep every intermediate tensor readable with fyn_layer_copy_result after forward.
  * With sharing on, an intermediate tensor may also never be written: a depthwise 3x3 layer and a 1x1
- * convolution next to it can run as one launch when nothing else reads the tensor between them, and a
- * plain batch-norm layer is applied on fetch by the convolutions that read it. */
+ * convolution next to it can run as one launch when nothing else reads the tensor between them, a
+ * plain batch-norm layer is applied on fetch by the convolutions that read it, and a 1x1 shortcut
+ * projection is computed by the 1x1 layer that adds it. */
 int fyn_net_set_buffer_reuse(fyn_net* net, int enable);
 
 /* Replays forward() from a captured hipGraph (launch-latency removal; no reference counterpart). */
