@@ -1499,14 +1499,17 @@ constexpr KREntry krentry() {
     return KREntry{NTAPS, CPW, FM, FN, G::TH, G::TW, S, DWS, R, conv_kr16_kernel<NTAPS, CPW, FM, FN, S, DWS, R>, (size_t)(G::RED_OFF + 3 * FM * FN * 1024 + 2 * 16 * FM * 4)};
 }
 const KREntry kKREntries[] = {
-    krentry<1, 1, 1>(), krentry<1, 2, 1>(), krentry<1, 3, 1>(), krentry<1, 4, 1>(), krentry<1, 5, 1>(), krentry<1, 8, 1>(), krentry<1, 16, 1>(),
-    krentry<1, 1, 2>(), krentry<1, 2, 2>(), krentry<1, 3, 2>(), krentry<1, 4, 2>(), krentry<1, 5, 2>(), krentry<1, 8, 2>(), krentry<1, 16, 2>(),
+    krentry<1, 1, 1>(), krentry<1, 2, 1>(), krentry<1, 3, 1>(), krentry<1, 4, 1>(), krentry<1, 5, 1>(), krentry<1, 6, 1>(), krentry<1, 8, 1>(), krentry<1, 12, 1>(), krentry<1, 16, 1>(),
+    krentry<1, 1, 2>(), krentry<1, 2, 2>(), krentry<1, 3, 2>(), krentry<1, 4, 2>(), krentry<1, 5, 2>(), krentry<1, 6, 2>(), krentry<1, 8, 2>(), krentry<1, 12, 2>(), krentry<1, 16, 2>(),
     krentry<9, 1, 1>(), krentry<9, 2, 1>(), krentry<9, 4, 1>(), krentry<9, 1, 2>(), krentry<9, 2, 2>(), krentry<9, 4, 2>(),
     // larger tiles for layers with more positions and a short reduction
     krentry<1, 1, 1, 2>(), krentry<1, 1, 2, 2>(), krentry<1, 2, 1, 2>(), krentry<1, 2, 2, 2>(), krentry<9, 1, 1, 2>(), krentry<9, 1, 2, 2>(),
     krentry<1, 1, 1, 4>(), krentry<1, 1, 2, 4>(), krentry<1, 2, 1, 4>(), krentry<1, 2, 2, 4>(), krentry<9, 1, 1, 4>(), krentry<9, 1, 2, 4>(),
     // 3x3 with stride 2 (a 9x9-pixel window per chunk under a tile of 4x4 positions)
-    krentry<9, 1, 1, 1, 2>(), krentry<9, 1, 2, 1, 2>(), krentry<9, 2, 1, 1, 2>(), krentry<9, 2, 2, 1, 2>(), krentry<9, 4, 1, 1, 2>(), krentry<9, 4, 2, 1, 2>(),
+    krentry<9, 1, 1, 1, 2>(), krentry<9, 1, 2, 1, 2>(), krentry<9, 2, 1, 1, 2>(), krentry<9, 2, 2, 1, 2>(),
+#if FYN_P16_HALF   // (16 chunks in one round: 83 KB of fp16, 166 KB in two fp32 planes -- that unit takes the two-round variant below)
+    krentry<9, 4, 1, 1, 2>(), krentry<9, 4, 2, 1, 2>(),
+#endif
     // reductions that pass through the LDS in two rounds (taken where the one-round entry above is more than a CU's LDS):
     // 3x3 with stride 2 on 512 channels in fp32, 3x3 on 1024 channels, 1x1 on 4096
     krentry<9, 2, 1, 1, 2, 0, 2>(), krentry<9, 2, 2, 1, 2, 0, 2>(), krentry<9, 4, 1, 1, 1, 0, 2>(), krentry<9, 4, 2, 1, 1, 0, 2>(),
@@ -1585,7 +1588,7 @@ size_t P16_NAME(conv_kr16_lds_bytes)(const ConvP16Params& p, int k) {
     return e ? e->lds : 0;
 }
 // The K-resident form: k = 1 (any stride) or 3 (stride 1, or 2 with 4x4 tiles); tiles of tile_h x tile_w = 4x4 (4x8, 8x8 for short reductions) positions, blocks of 16*p.wm output channels (p.wm = 1 or 2),
-// p.cin_chunks = 4, 8, 12, 16, 20, 32, 64 or 128 (3x3: 4, 8, 16 or 32; with stride 2: 4, 8 or 16), channels behind in_cp reading as zero; in_y0/in_x0 = input padding - (k-1)/2; one workgroup per tile and block
+// p.cin_chunks = 4, 8, 12, 16, 20, 24, 32, 48, 64 or 128 (3x3: 4, 8, 16 or 32; with stride 2: 4, 8 or 16), channels behind in_cp reading as zero; in_y0/in_x0 = input padding - (k-1)/2; one workgroup per tile and block
 int P16_NAME(launch_conv_kr16)(const ConvP16Params& p, int k, hipStream_t s) {
 #if !FYN_P16_HALF
     if (p.f16) return launch_conv_kr16_half(p, k, s);
