@@ -20,8 +20,9 @@ class Bottleneck(networks._StreamNet):
     download: the first block of a ResNet stage (samples/samplenetworks/resnet50.cpp:260-275)."""
     config_id = 3
 
-    def __init__(self, storage, cin, mid, cout, h, w, stride, res_act=ActType.NONE, second_reader=False):
+    def __init__(self, storage, cin, mid, cout, h, w, stride, res_act=ActType.NONE, second_reader=False, res_bn=False):
         super().__init__(storage)
+        self.res_bn = res_bn
         self.cin, self.mid, self.cout, self.h, self.w, self.stride = cin, mid, cout, h, w, stride
         self.res_act, self.second_reader = res_act, second_reader
 
@@ -34,6 +35,8 @@ class Bottleneck(networks._StreamNet):
         self.conv(3, "reduce", 1, self.cin, self.mid, self.h, self.w, 1, act=R, pad_out=1)
         self.conv(4, "spatial", 3, self.mid, self.mid, self.h, self.w, 3, stride=self.stride, act=R)
         self.conv(5, "expand", 1, self.mid, self.cout, ho, wo, 4, act=R, residual=2, res_act=self.res_act)
+        if self.res_bn:   # the layer's batch-norm scale multiplies what it adds as well (ConvLayerBuilder::residual(act, true))
+            self._builders[-1].residual(self.res_act, True)
         last = 5
         if self.second_reader:   # something else reads the projection's tensor
             self.conv(6, "side", 1, self.cout, 32, ho, wo, 2, act=R)
@@ -66,19 +69,22 @@ CASES = [
     # (cin, mid, cout, h, w, step)
     (64, 64, 256, 28, 28, 1),        # stage 1 of ResNet-50 (smaller): 2 + 2 chunks
     (256, 128, 512, 28, 28, 2),      # stage 2: the projection reads every other pixel; 4 + 8 chunks
-    (512, 256, 1024, 14, 14, 2),     # stage 3: 8 + 16 chunks rounded up to 32
-    (1024, 512, 2048, 14, 14, 2),    # stage 4: 16 + 32 chunks rounded up to 64
-    (96, 48, 80, 13, 11, 1),         # channel counts that are no multiples of 32 or of the block, ragged tiles
+    (512, 256, 1024, 14, 14, 2),     # stage 3: 8 + 16 chunks
+    (1024, 512, 2048, 14, 14, 2),    # stage 4: 16 + 32 chunks
+    (96, 48, 80, 13, 11, 1),         # channel counts that are no multiples of 32 or of the block, ragged tiles; 2 + 3 chunks rounded up to 8
     (40, 24, 72, 9, 15, 2),          # odd sizes with step 2
 ]
 
 
 @pytest.mark.parametrize("storage", [fa.STORAGE_F32, fa.STORAGE_F16], ids=["f32", "f16"])
+@pytest.mark.parametrize("res_bn", [False, True], ids=["plain", "bn_on_residual"])
 @pytest.mark.parametrize("case", CASES, ids=lambda c: "%d_%d_%d_%dx%d_s%d" % c)
-def test_projection_inside_the_layer_that_adds_it(case, storage, monkeypatch):
+def test_projection_inside_the_layer_that_adds_it(case, res_bn, storage, monkeypatch):
     cin, mid, cout, h, w, stride = case
+    if res_bn and cin > 256:
+        pytest.skip("the residual's batch-norm is varied on the smaller cases")
     monkeypatch.setenv("FYNHIP_FORCE_PROJECTION_FUSION", "1")
-    net = Bottleneck(storage, cin, mid, cout, h, w, stride)
+    net = Bottleneck(storage, cin, mid, cout, h, w, stride, res_bn=res_bn)
     x, got, infos = run(net)
     desc = net.describe()
     net.cleanup()
@@ -90,7 +96,7 @@ def test_projection_inside_the_layer_that_adds_it(case, storage, monkeypatch):
     assert err <= TOL[storage]
     monkeypatch.delenv("FYNHIP_FORCE_PROJECTION_FUSION")
     monkeypatch.setenv("FYNHIP_NO_PROJECTION_FUSION", "1")
-    twin = Bottleneck(storage, cin, mid, cout, h, w, stride)
+    twin = Bottleneck(storage, cin, mid, cout, h, w, stride, res_bn=res_bn)
     _, two, infos2 = run(twin)
     twin.cleanup()
     assert "no launch of its own" not in infos2["projection"]
