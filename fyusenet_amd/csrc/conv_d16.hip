@@ -182,9 +182,13 @@ __global__ __launch_bounds__(256) void conv_d16_kernel(const ConvP16Params p) {
     _Float16 act_lo, act_hi;
     const bool half_act = HS && act_half_exact(p.act, act_lo, act_hi);
     half8_t b[NCHK][NPL];
-    const bool affine = DWS == 0 && KS == 0 && p.in_mul != nullptr;
-    auto convert = [&](auto kind_) {
-    constexpr int KIND = decltype(kind_)::value;   // (the activation's kind, chosen once per wave: act_kind)
+#ifndef FYN_AFFINE_ON
+#define FYN_AFFINE_ON 1
+#endif
+    const bool affine = FYN_AFFINE_ON && DWS == 0 && KS == 0 && p.in_mul != nullptr;
+    auto convert = [&](auto kind_, auto aff_) {
+    constexpr int KIND = decltype(kind_)::value;
+    constexpr bool AFF = decltype(aff_)::value;   // (with the batch-norm layer in front: chosen once per wave, like the kind)   // (the activation's kind, chosen once per wave: act_kind)
 #pragma unroll
     for (int c = 0; c < NCHK; c++) {
         const bool okc = KS > 0 || c * KC + kq * 8 < p.in_cp;
@@ -213,7 +217,7 @@ __global__ __launch_bounds__(256) void conv_d16_kernel(const ConvP16Params p) {
         } else {
             texel(raw[c][0], r);
             if constexpr (KS == 0) {
-                if (affine) {   // a batch-norm layer in front, applied here: x * in_mul[channel] + in_add[channel]
+                if constexpr (AFF) {   // a batch-norm layer in front, applied here: x * in_mul[channel] + in_add[channel]
                     const int ch = okc ? c * KC + kq * 8 : 0;
                     const float4 m0 = *reinterpret_cast<const float4*>(p.in_mul + ch), m1 = *reinterpret_cast<const float4*>(p.in_mul + ch + 4);
                     const float4 a0 = *reinterpret_cast<const float4*>(p.in_add + ch), a1 = *reinterpret_cast<const float4*>(p.in_add + ch + 4);
@@ -227,7 +231,7 @@ __global__ __launch_bounds__(256) void conv_d16_kernel(const ConvP16Params p) {
             }
         }
         if constexpr (HS) {
-            if (DWS == 0 && half_act && !affine) {
+            if (DWS == 0 && half_act && !AFF) {
                 b[c][0] = okc ? act_half(raw[c][0], act_lo, act_hi) : (half8_t)((_Float16)0.f);
             } else {
 #pragma unroll
@@ -238,9 +242,13 @@ __global__ __launch_bounds__(256) void conv_d16_kernel(const ConvP16Params p) {
         }
     }
     };
-    if (HS || p.act.kind == ACT_LEAKY || p.act.kind == ACT_CLIP) convert(std::integral_constant<int, ACT_LEAKY>());
-    else if (p.act.kind == ACT_RELU) convert(std::integral_constant<int, ACT_RELU>());
-    else convert(std::integral_constant<int, ACT_NONE>());
+    if (affine) {
+        if (HS || p.act.kind == ACT_LEAKY || p.act.kind == ACT_CLIP) convert(std::integral_constant<int, ACT_LEAKY>(), std::true_type());
+        else if (p.act.kind == ACT_RELU) convert(std::integral_constant<int, ACT_RELU>(), std::true_type());
+        else convert(std::integral_constant<int, ACT_NONE>(), std::true_type());
+    } else if (HS || p.act.kind == ACT_LEAKY || p.act.kind == ACT_CLIP) convert(std::integral_constant<int, ACT_LEAKY>(), std::false_type());
+    else if (p.act.kind == ACT_RELU) convert(std::integral_constant<int, ACT_RELU>(), std::false_type());
+    else convert(std::integral_constant<int, ACT_NONE>(), std::false_type());
     store_t* out = reinterpret_cast<store_t*>(p.out);
     float vmax = 0.f;
     auto fragment = [&](int f, const half8_t (&a)[NCHK][NPL], const res_t& rcur, const f32x4_t& sc, const f32x4_t& bi) {

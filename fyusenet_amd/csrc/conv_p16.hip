@@ -963,8 +963,11 @@ struct GeoR {
 #ifndef FYN_KR_STAGE_WAVES
 #define FYN_KR_STAGE_WAVES 8
 #endif
-template <int NTAPS, int CPW, int FM, int FN, int S, int DWS = 0, int R = 1>
+template <int NTAPS, int CPW, int FM, int FN, int S, int DWS = 0, int R = 1, int SRC = 0>
 __global__ __launch_bounds__(512) void conv_kr16_kernel(const ConvP16Params p) {
+    // SRC: 0 = the plain layer; 1 = a batch-norm layer in front applied while staging (p.in_mul, p.in_add); 2 = a reduction
+    // over two tensors (p.in2...).  Kernels of their own, so that the plain one carries none of their instructions.
+    static_assert(SRC == 0 || (NTAPS == 1 && FN == 1 && S == 1 && DWS == 0 && R == 1), "batch-norm in front / two tensors: 1x1, tiles of 4x4 positions, one round");
     // R > 1: the reduction passes through the LDS in R rounds of 4 * CPW chunks each (layers whose whole reduction does
     // not fit: 3x3 with stride 2 on 512 channels needs 166 KB).  The staging waves request round r + 1 while the MFMA
     // waves work on round r and write it once those are through.
@@ -983,9 +986,11 @@ __global__ __launch_bounds__(512) void conv_kr16_kernel(const ConvP16Params p) {
     const int tyi = tile / p.tiles_x, txi = tile - tyi * p.tiles_x;
     if (tid < 2) range_box[tid] = 0u;
     // (two source tensors: the larger of their value ranges scales both, or nothing is scaled when one keeps no word)
-    const bool ranged = p.in_amax && (!p.in2 || p.in2_amax);
-    unsigned range_bits = ranged ? range_load(p.in_amax) : 0u;
-    if (ranged && p.in2) range_bits = max(range_bits, range_load(p.in2_amax));
+    const bool ranged = p.in_amax && (SRC != 2 || p.in2_amax);
+    // (both loads are issued here and met where the scale is computed: nothing waits for them in between)
+    const unsigned range_bits1 = ranged ? range_load(p.in_amax) : 0u;
+    const unsigned range_bits2 = (SRC == 2 && ranged) ? range_load(p.in2_amax) : 0u;
+    auto range_word = [&]() { return max(range_bits1, range_bits2); };
     constexpr int red_off = G::RED_OFF;
     constexpr int sb_off = red_off + 3 * FM * FN * 1024;
     // Staging waves: the four that only stage, and -- without a depthwise layer in front -- the four MFMA waves too,
@@ -1028,8 +1033,8 @@ __global__ __launch_bounds__(512) void conv_kr16_kernel(const ConvP16Params p) {
             [[maybe_unused]] bool inb2 = false;
             [[maybe_unused]] const store_t* src2 = in;
             [[maybe_unused]] int c2 = 0;
-            if constexpr (NTAPS == 1 && R == 1) {
-                if (p.in2) {
+            if constexpr (SRC == 2) {
+                {
                     const int gy2 = (tyi * G::TH + py) * p.in2_stride + p.in2_y0, gx2 = (txi * G::TW + px) * p.in2_stride + p.in2_x0;
                     inb2 = (unsigned)gy2 < (unsigned)p.in2_hp && (unsigned)gx2 < (unsigned)p.in2_wp;
                     c2 = (chunk0 - p.in2_chunk0) * KC + g * 8;   // (negative for the chunks of the first tensor)
@@ -1044,8 +1049,8 @@ __global__ __launch_bounds__(512) void conv_kr16_kernel(const ConvP16Params p) {
                 ok[i] = in_tile && inb && c0 + i * CPI * KC < p.in_cp;
                 ch_of[i] = c0 + i * CPI * KC;
                 const store_t* src = ok[i] ? src0 + i * CPI * KC : in;
-                if constexpr (NTAPS == 1 && R == 1) {
-                    if (p.in2 && chunk0 + i * CPI >= p.in2_chunk0) {
+                if constexpr (SRC == 2) {
+                    if (chunk0 + i * CPI >= p.in2_chunk0) {
                         ok[i] = in_tile && inb2 && c2 + i * CPI * KC < p.in2_cp;
                         src = ok[i] ? src2 + i * CPI * KC : in;
                     }
@@ -1083,13 +1088,12 @@ __global__ __launch_bounds__(512) void conv_kr16_kernel(const ConvP16Params p) {
         }
         }
         float in_scale = 1.f, inv_unused;
-        if (ranged) in_scale = range_scale(range_after_act(range_reduce(range_bits), p.act), &inv_unused);
+        if (ranged) in_scale = range_scale(range_after_act(range_reduce(range_word()), p.act), &inv_unused);
         // (fp16 tensors: no activation, or a clamp without leak whose bounds are fp16 values, is applied to the packed
         // halves -- two values per instruction, no conversions)
         const _Float16 hlo = (_Float16)fmaxf(p.act.lo, -65504.f), hhi = (_Float16)fminf(p.act.hi, 65504.f);
         const bool half_act = HSTORE && p.act.leak == 0.f && (p.act.lo < -65504.f || (float)hlo == p.act.lo) && (p.act.hi > 65504.f || (float)hhi == p.act.hi);
         // a batch-norm layer in front: x * in_mul[c] + in_add[c] on the item's eight channels (the arrays come through the L1)
-        const bool affine = p.in_mul != nullptr;
         auto affine8 = [&](float (&x)[8], const int i) {
             const int c = ok[i] ? ch_of[i] : 0;
             const float4 m0 = *reinterpret_cast<const float4*>(p.in_mul + c), m1 = *reinterpret_cast<const float4*>(p.in_mul + c + 4);
@@ -1099,12 +1103,15 @@ __global__ __launch_bounds__(512) void conv_kr16_kernel(const ConvP16Params p) {
             for (int e = 0; e < 8; e++) x[e] = x[e] * m[e] + a[e];
         };
         if (wait) lds_barrier();   // the MFMA waves are through with the round before: its place in the LDS is free
+        // (with or without the batch-norm layer: chosen once, outside the loops over the items)
+        [[maybe_unused]] auto store_halves = [&](auto aff_) {
+        constexpr bool AFF = decltype(aff_)::value;
 #pragma unroll
         for (int i = 0; i < NB; i++) {
             if (l_off[i] < 0) continue;
             if constexpr (HSTORE) {
                 half8_t rv = raw[i];
-                if (affine) {
+                if constexpr (AFF) {
                     float x[8];
 #pragma unroll
                     for (int e = 0; e < 8; e++) x[e] = (float)rv[e];
@@ -1122,23 +1129,27 @@ __global__ __launch_bounds__(512) void conv_kr16_kernel(const ConvP16Params p) {
                 *reinterpret_cast<half8_t*>(lds + l_off[i]) = v;
             }
         }
+        };
+        if constexpr (HSTORE) store_halves(std::integral_constant<bool, SRC == 1>());
         if constexpr (!HSTORE) {
-            auto split_all = [&](auto kind_) {
+            auto split_all = [&](auto kind_, auto aff_) {
                 constexpr int KIND = decltype(kind_)::value;
+                constexpr bool AFF = decltype(aff_)::value;
 #pragma unroll
                 for (int i = 0; i < NB; i++) {
                     if (l_off[i] < 0) continue;
                     float r[8] = {raw[i].a.x, raw[i].a.y, raw[i].a.z, raw[i].a.w, raw[i].b.x, raw[i].b.y, raw[i].b.z, raw[i].b.w};
-                    if (affine) affine8(r, i);
+                    if constexpr (AFF) affine8(r, i);
                     half8_t hi, lo;
                     split8<KIND>(r, ok[i], p.act, in_scale, hi, lo);
                     *reinterpret_cast<half8_t*>(lds + l_off[i]) = hi;
                     *reinterpret_cast<half8_t*>(lds + G::PLANE + l_off[i]) = lo;
                 }
             };
-            if (p.act.kind == ACT_NONE) split_all(std::integral_constant<int, ACT_NONE>());
-            else if (p.act.kind == ACT_RELU) split_all(std::integral_constant<int, ACT_RELU>());
-            else split_all(std::integral_constant<int, ACT_LEAKY>());
+            constexpr std::integral_constant<bool, SRC == 1> aff;
+            if (p.act.kind == ACT_NONE) split_all(std::integral_constant<int, ACT_NONE>(), aff);
+            else if (p.act.kind == ACT_RELU) split_all(std::integral_constant<int, ACT_RELU>(), aff);
+            else split_all(std::integral_constant<int, ACT_LEAKY>(), aff);
         }
     };
 
@@ -1151,7 +1162,7 @@ __global__ __launch_bounds__(512) void conv_kr16_kernel(const ConvP16Params p) {
             constexpr int IPP = NB < IPP_MAX ? NB : IPP_MAX;
             const store_t* din = reinterpret_cast<const store_t*>(p.dw_in);
             float in_scale = 1.f, inv_unused;
-            if (p.in_amax) in_scale = range_scale(range_after_act(range_reduce(range_bits), p.act), &inv_unused);
+            if (p.in_amax) in_scale = range_scale(range_after_act(range_reduce(range_word()), p.act), &inv_unused);
             if (stid < 16 * FM) {
                 reinterpret_cast<float*>(lds + sb_off)[stid] = p.scale[cb * 16 * FM + stid];
                 reinterpret_cast<float*>(lds + sb_off)[16 * FM + stid] = p.bias[cb * 16 * FM + stid];
@@ -1308,7 +1319,7 @@ __global__ __launch_bounds__(512) void conv_kr16_kernel(const ConvP16Params p) {
 #pragma unroll
         for (int fn = 0; fn < FN; fn++) acc[fm][fn] = (f32x4_t)(0.f);
     float inv_in_scale = 1.f;
-    if (ranged) (void)range_scale(range_after_act(range_reduce(range_bits), p.act), &inv_in_scale);
+    if (ranged) (void)range_scale(range_after_act(range_reduce(range_word()), p.act), &inv_in_scale);
     const float acc_mul = p.acc_mul * inv_in_scale;
     // The residual values of the epilogue (wave 0) are requested here, so that their memory round trip passes under the
     // staging and the step stream instead of behind them (small tiles: the registers are there).
@@ -1489,14 +1500,14 @@ template <int K, int TH, int TW>
 constexpr C4Entry c4entry() { return C4Entry{K, TH, TW, conv_p16c4_kernel<K, TH, TW>, (size_t)GeoC4<K, TH, TW>::BUF, GeoC4<K, TH, TW>::NS}; }
 const C4Entry kC4Entries[] = {c4entry<9, 8, 8>(), c4entry<9, 4, 8>(), c4entry<9, 8, 4>()};
 struct KREntry {
-    int taps, cpw, fm, nfrag, th, tw, stride, dws, rounds;   // (cpw: chunks per wave and round)
+    int taps, cpw, fm, nfrag, th, tw, stride, dws, rounds, src;   // (cpw: chunks per wave and round)
     p16_fn fn;
     size_t lds;
 };
-template <int NTAPS, int CPW, int FM, int FN = 1, int S = 1, int DWS = 0, int R = 1>
+template <int NTAPS, int CPW, int FM, int FN = 1, int S = 1, int DWS = 0, int R = 1, int SRC = 0>
 constexpr KREntry krentry() {
     using G = GeoR<NTAPS, CPW, FN, S>;
-    return KREntry{NTAPS, CPW, FM, FN, G::TH, G::TW, S, DWS, R, conv_kr16_kernel<NTAPS, CPW, FM, FN, S, DWS, R>, (size_t)(G::RED_OFF + 3 * FM * FN * 1024 + 2 * 16 * FM * 4)};
+    return KREntry{NTAPS, CPW, FM, FN, G::TH, G::TW, S, DWS, R, SRC, conv_kr16_kernel<NTAPS, CPW, FM, FN, S, DWS, R, SRC>, (size_t)(G::RED_OFF + 3 * FM * FN * 1024 + 2 * 16 * FM * 4)};
 }
 const KREntry kKREntries[] = {
     krentry<1, 1, 1>(), krentry<1, 2, 1>(), krentry<1, 3, 1>(), krentry<1, 4, 1>(), krentry<1, 5, 1>(), krentry<1, 6, 1>(), krentry<1, 8, 1>(), krentry<1, 12, 1>(), krentry<1, 16, 1>(),
@@ -1519,6 +1530,10 @@ const KREntry kKREntries[] = {
 #define FYN_KR_DW(CPW) krentry<1, CPW, 1, 1, 1, 1>(), krentry<1, CPW, 2, 1, 1, 1>(), krentry<1, CPW, 1, 1, 1, 2>(), krentry<1, CPW, 2, 1, 1, 2>()
 const KREntry kKRDwEntries[] = {FYN_KR_DW(1), FYN_KR_DW(2), FYN_KR_DW(3), FYN_KR_DW(4)};   // (up to 512 channels: beyond, two launches are faster)
 #undef FYN_KR_DW
+// 1x1 on 4x4 tiles with a batch-norm layer applied while staging (1) or over two tensors (2)
+#define FYN_KR_SRC(CPW) krentry<1, CPW, 1, 1, 1, 0, 1, 1>(), krentry<1, CPW, 2, 1, 1, 0, 1, 1>(), krentry<1, CPW, 1, 1, 1, 0, 1, 2>(), krentry<1, CPW, 2, 1, 1, 0, 1, 2>()
+const KREntry kKRSrcEntries[] = {FYN_KR_SRC(1), FYN_KR_SRC(2), FYN_KR_SRC(3), FYN_KR_SRC(4), FYN_KR_SRC(5), FYN_KR_SRC(6), FYN_KR_SRC(8), FYN_KR_SRC(12), FYN_KR_SRC(16)};
+#undef FYN_KR_SRC
 }  // namespace
 
 // Host entry points.  The fp32 unit holds the public ones and hands launches on fp16 tensors (p.f16) to the other
@@ -1574,6 +1589,12 @@ static const KREntry* find_krentry(const ConvP16Params& p, int k) {
             if (k == 1 && c.cpw * 4 == p.cin_chunks && c.fm == p.wm && c.th == p.tile_h && c.tw == p.tile_w && c.dws == p.dw_stride) return &c;
         return nullptr;
     }
+    if (p.in_mul || p.in2) {
+        const int src = p.in_mul ? 1 : 2;
+        for (const KREntry& c : kKRSrcEntries)
+            if (k == 1 && c.cpw * 4 == p.cin_chunks && c.fm == p.wm && c.th == p.tile_h && c.tw == p.tile_w && c.src == src && c.lds <= 160 * 1024) return &c;
+        return nullptr;
+    }
     for (const KREntry& c : kKREntries)
         if (c.taps == k * k && c.cpw * 4 * c.rounds == p.cin_chunks && c.fm == p.wm && c.th == p.tile_h && c.tw == p.tile_w && c.stride == (k == 1 ? 1 : p.stride) &&
             c.lds <= 160 * 1024)
@@ -1602,7 +1623,7 @@ int P16_NAME(launch_conv_kr16)(const ConvP16Params& p, int k, hipStream_t s) {
     // (a fused depthwise layer: its tensor has the pointwise layer's channels, in whole groups of 8, and the 1x1 layer does not step)
     if (p.dw_in && (!p.dw_w || !p.dw_scale || !p.dw_bias || p.dw_cp != p.in_cp || p.stride != 1 || p.in_clamp || p.dw_hp < 1 || p.dw_wp < 1)) return -5;
     // (a batch-norm layer applied while staging: not beside a depthwise layer, and both arrays or none)
-    if ((p.in_mul != nullptr) != (p.in_add != nullptr) || (p.in_mul && p.dw_in)) return -5;
+    if ((p.in_mul != nullptr) != (p.in_add != nullptr) || (p.in_mul && (p.dw_in || p.in2))) return -5;
     // (a second source tensor: 1x1 in one round, the first tensor's channels end where the second's chunks begin)
     if (p.in2 && (k != 1 || e->rounds != 1 || p.dw_in || p.in_mul || p.in_clamp || p.in2_chunk0 < 1 || p.in2_chunk0 >= p.cin_chunks || p.in_cp > p.in2_chunk0 * KC ||
                   p.in2_cp % 8 != 0 || p.in2_cp < 8 || p.in2_cp > (p.cin_chunks - p.in2_chunk0) * KC || p.in2_stride < 1 || p.in2_hp < 1 || p.in2_wp < 1 || p.in2_y0 < 0 || p.in2_x0 < 0))

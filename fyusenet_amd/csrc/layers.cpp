@@ -1982,7 +1982,14 @@ class ConvLayer : public Layer {
         q.in_amax = nullptr;   // (the batch-norm layer keeps no value-range word: its readers stage unscaled either way)
         return q;
     }
-    bool takes_batchnorm() const { return p16 && (kr16 || (d16 && k == 1)) && !dw_fused && !edw_fused && !pj_fused && pj_into < 0 && !pp.in_amax; }
+    bool takes_batchnorm() const {
+        if (!p16 || dw_fused || edw_fused || pj_fused || pj_into >= 0 || pp.in_amax) return false;
+        if (d16) return k == 1;
+        if (!kr16) return false;
+        ConvP16Params t = pp;   // (a variant of the K-resident form that applies the layer: 1x1 on 4x4 tiles)
+        t.in_mul = t.in_add = scale_dev;
+        return conv_kr16_lds_bytes(t, k) != 0;
+    }
     // A 1x1 projection whose result this 1x1 layer adds (its residual input) computed in the layer's own launch, as one
     // reduction over two tensors (fuse_projection_layers below): the rows of both weight matrices carry their layers'
     // folded scales, the bias is the sum of both, and the projection's tensor is never written.
