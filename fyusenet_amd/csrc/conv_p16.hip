@@ -977,13 +977,13 @@ __global__ __launch_bounds__(512) void conv_kr16_kernel(const ConvP16Params p) {
     constexpr int RPD = G::RPD, BD = G::BD, STEPS = G::STEPS;
     extern __shared__ __align__(16) unsigned char lds[];
     __shared__ unsigned range_box[2];
-    if (blockIdx.x == 0) range_clear(p.reset[0], p.reset[1], p.reset[2], p.reset[3], p.nreset);
+    if ((blockIdx.x | blockIdx.y | blockIdx.z) == 0) range_clear(p.reset[0], p.reset[1], p.reset[2], p.reset[3], p.nreset);
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int cb = blockIdx.x % p.cout_blocks;
-    const int tile = blockIdx.x / p.cout_blocks;
-    const int tyi = tile / p.tiles_x, txi = tile - tyi * p.tiles_x;
+    // (a grid of output-channel blocks x tile columns x tile rows: no division stands between the kernel's start and its
+    // first request; consecutive workgroups are the channel blocks of one tile)
+    const int cb = blockIdx.x, txi = blockIdx.y, tyi = blockIdx.z;
     if (tid < 2) range_box[tid] = 0u;
     // (two source tensors: the larger of their value ranges scales both, or nothing is scaled when one keeps no word)
     const bool ranged = p.in_amax && (SRC != 2 || p.in2_amax);
@@ -1618,7 +1618,7 @@ int P16_NAME(launch_conv_kr16)(const ConvP16Params& p, int k, hipStream_t s) {
     if (!e) return -1;
     if (p.in_cp > p.cin_chunks * KC || p.in_cp % 8 != 0 || p.in_cp < 8 || p.cout_blocks < 1 || p.mfrags != p.cout_blocks * e->fm || p.stride < 1 ||
         p.tiles_x * e->tw < p.npos_x || p.tiles_y * e->th < p.npos_y || p.out_cp % 4 != 0 || p.out_cp < 4 || (p.res && p.res_cp < p.out_cp) || p.nreset < 0 || p.nreset > 4 || (p.f16 != 0) != HSTORE ||
-        p.tiles_x < 1 || p.tiles_y < 1 || (long long)p.tiles_x * p.tiles_y * p.cout_blocks > 65535)
+        p.tiles_x < 1 || p.tiles_y < 1 || p.tiles_x > 65535 || p.tiles_y > 65535 || (long long)p.tiles_x * p.tiles_y * p.cout_blocks > 65535)
         return -5;
     // (a fused depthwise layer: its tensor has the pointwise layer's channels, in whole groups of 8, and the 1x1 layer does not step)
     if (p.dw_in && (!p.dw_w || !p.dw_scale || !p.dw_bias || p.dw_cp != p.in_cp || p.stride != 1 || p.in_clamp || p.dw_hp < 1 || p.dw_wp < 1)) return -5;
@@ -1630,7 +1630,7 @@ int P16_NAME(launch_conv_kr16)(const ConvP16Params& p, int k, hipStream_t s) {
         return -5;
     if (e->lds > 160 * 1024) return -2;
     if (ensure_lds(reinterpret_cast<const void*>(e->fn), e->lds) != 0) return -2;
-    hipLaunchKernelGGL(e->fn, dim3(p.tiles_x * p.tiles_y * p.cout_blocks), dim3(512), e->lds, s, p);
+    hipLaunchKernelGGL(e->fn, dim3(p.cout_blocks, p.tiles_x, p.tiles_y), dim3(512), e->lds, s, p);
     return hipGetLastError() == hipSuccess ? 0 : -3;
 }
 
