@@ -65,7 +65,18 @@ __global__ __launch_bounds__(256) void conv_d16_kernel(const ConvP16Params p) {
     const int pos = (p.wm == 4 ? blockIdx.x * 4 + w : blockIdx.x) * 16 + mq;
     const bool okp = pos < npos;
     const int pc = okp ? pos : npos - 1;
-    const int py = pc / p.npos_x, px = pc - py * p.npos_x;
+    // (row and column without an integer division in front of the first request: the reciprocal of the row length comes
+    // with the launch, one step of correction makes the quotient exact; beyond 2^22 positions the division is used)
+    int py, px;
+    if (npos <= (1 << 22)) {
+        py = (int)(((float)pc + 0.5f) * p.rcp_tiles_x);
+        px = pc - py * p.npos_x;
+        if (px < 0) { py--; px += p.npos_x; }
+        else if (px >= p.npos_x) { py++; px -= p.npos_x; }
+    } else {
+        py = pc / p.npos_x;
+        px = pc - py * p.npos_x;
+    }
     struct RawF { float4 a, b; };
     typedef typename std::conditional<HS, half8_t, RawF>::type raw_t;
     constexpr int NT = DWS > 0 ? 9 : 1;   // texels per lane and chunk
@@ -362,17 +373,17 @@ __global__ __launch_bounds__(256) void conv_e16dw_kernel(const ConvP16Params p) 
     constexpr int WIN = 3 * DWS + 3, NWIN = WIN * WIN, NPF = (NWIN + 15) / 16;
     typedef typename std::conditional<HS, _Float16, float>::type store_t;
     __shared__ __align__(16) float win[NWIN][68];   // (68: the sixteen positions of a fragment write distinct banks)
-    if (blockIdx.x == 0 && blockIdx.y == 0) range_clear(p.reset[0], p.reset[1], p.reset[2], p.reset[3], p.nreset);
+    if ((blockIdx.x | blockIdx.y | blockIdx.z) == 0) range_clear(p.reset[0], p.reset[1], p.reset[2], p.reset[3], p.nreset);
     const int lane = threadIdx.x & 63;
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int mq = lane & 15, kq = lane >> 4;
     const unsigned range_bits = p.in_amax ? range_load(p.in_amax) : 0u;
-    const int tyi = blockIdx.x / p.tiles_x, txi = blockIdx.x - tyi * p.tiles_x;
+    const int txi = blockIdx.x, tyi = blockIdx.y;   // (a grid of tile columns x tile rows x channel blocks: no division in front of the first request)
     const int ey0 = tyi * 4 * DWS - 1, ex0 = txi * 4 * DWS - 1;   // the window's first position in the expanded tensor
     // ---- depthwise phase operands (requested first: they are used last) ----
     const int t = threadIdx.x;
     const int dpos = t >> 4, dc = (t & 15) * 4;                   // output position of the tile, first of four channels of the block
-    const int dch = blockIdx.y * 64 + dc;
+    const int dch = blockIdx.z * 64 + dc;
     const bool dch_ok = dch + 4 <= p.dw_cp;
     f32x4_t dww[9], dsc, dbi;
 #pragma unroll
@@ -404,7 +415,7 @@ __global__ __launch_bounds__(256) void conv_e16dw_kernel(const ConvP16Params p) 
         }
     }
     // ---- this wave's fragment of expanded channels: weights, scale, bias ----
-    const int mf = blockIdx.y * 4 + w;
+    const int mf = blockIdx.z * 4 + w;
     const bool mf_ok = mf < p.mfrags;
     half8_t a[NCHK][NPL];
     const unsigned char* wbase = reinterpret_cast<const unsigned char*>(p.wpack) + (size_t)(mf_ok ? mf : 0) * (NCHK * NPL * 1024) + lane * 16;
@@ -500,14 +511,14 @@ __global__ __launch_bounds__(256) void conv_e16dw_narrow_kernel(const ConvP16Par
     constexpr int WIN = 3 * DWS + 3, NWIN = WIN * WIN, NPF = (NWIN + 15) / 16, PFW = (NPF + 3) / 4;
     typedef typename std::conditional<HS, _Float16, float>::type store_t;
     __shared__ __align__(16) float win[NWIN][20];   // (20: the sixteen positions of a fragment write distinct banks)
-    if (blockIdx.x == 0 && blockIdx.y == 0) range_clear(p.reset[0], p.reset[1], p.reset[2], p.reset[3], p.nreset);
+    if ((blockIdx.x | blockIdx.y | blockIdx.z) == 0) range_clear(p.reset[0], p.reset[1], p.reset[2], p.reset[3], p.nreset);
     const int lane = threadIdx.x & 63;
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int mq = lane & 15, kq = lane >> 4;
     const unsigned range_bits = p.in_amax ? range_load(p.in_amax) : 0u;
-    const int tyi = blockIdx.x / p.tiles_x, txi = blockIdx.x - tyi * p.tiles_x;
+    const int txi = blockIdx.x, tyi = blockIdx.y;   // (a grid of tile columns x tile rows x channel blocks: no division in front of the first request)
     const int ey0 = tyi * 4 * DWS - 1, ex0 = txi * 4 * DWS - 1;
-    const int mf = blockIdx.y;
+    const int mf = blockIdx.z;
     // depthwise phase operands (requested first: they are used last)
     const int t = threadIdx.x;
     const int dpos = t >> 4, dch = mf * 16 + (t & 15);
@@ -682,7 +693,9 @@ int launch_conv_d16(const ConvP16Params& p, hipStream_t s) {
         (!ks && ((long long)((p.npos_y - 1) * p.stride + p.in_y0) >= p.in_hp || (long long)((p.npos_x - 1) * p.stride + p.in_x0) >= p.in_wp || p.in_y0 < 0 || p.in_x0 < 0)))
         return -5;
     const long long per_wg = 16 * p.wm;
-    hipLaunchKernelGGL(fn, dim3((unsigned)((npos + per_wg - 1) / per_wg), (unsigned)p.cout_blocks), dim3(256), 0, s, p);
+    ConvP16Params q = p;
+    q.rcp_tiles_x = 1.0f / (float)p.npos_x;   // (this kernel's use of the field: the reciprocal of a row of positions)
+    hipLaunchKernelGGL(fn, dim3((unsigned)((npos + per_wg - 1) / per_wg), (unsigned)p.cout_blocks), dim3(256), 0, s, q);
     return hipGetLastError() == hipSuccess ? 0 : -3;
 }
 
@@ -703,9 +716,9 @@ int launch_conv_e16dw(const ConvP16Params& p, hipStream_t s) {
     if (p.mfrags < 1 || p.stride != 1 || p.res || p.in_clamp || !p.dw_w || !p.dw_scale || !p.dw_bias || p.dw_cp % 8 != 0 || p.dw_cp != p.out_cp || p.dw_cp > 16 * p.mfrags + 15 ||
         p.dw_hp < 1 || p.dw_wp < 1 || p.dw_hp - 1 + p.in_y0 >= p.in_hp || p.dw_wp - 1 + p.in_x0 >= p.in_wp || p.in_y0 < 0 || p.in_x0 < 0 || p.npos_y < 1 || p.npos_x < 1 ||
         p.tiles_x * 4 < p.npos_x || p.tiles_y * 4 < p.npos_y || (p.npos_y - 1) * p.dw_stride >= p.dw_hp + 1 || (p.npos_x - 1) * p.dw_stride >= p.dw_wp + 1 ||
-        (long long)p.tiles_x * p.tiles_y > (1ll << 30) || p.nreset < 0 || p.nreset > 4)
+        (long long)p.tiles_x * p.tiles_y > (1ll << 30) || p.tiles_y > 65535 || p.mfrags > 65535 || p.nreset < 0 || p.nreset > 4)
         return -5;
-    hipLaunchKernelGGL(fn, dim3((unsigned)(p.tiles_x * p.tiles_y), (unsigned)(narrow ? p.mfrags : (p.dw_cp + 63) / 64)), dim3(256), 0, s, p);
+    hipLaunchKernelGGL(fn, dim3((unsigned)p.tiles_x, (unsigned)p.tiles_y, (unsigned)(narrow ? p.mfrags : (p.dw_cp + 63) / 64)), dim3(256), 0, s, p);
     return hipGetLastError() == hipSuccess ? 0 : -3;
 }
 
