@@ -268,7 +268,8 @@ def roofline_records(net, storage_bytes, iters=20):
         flops, nbytes, passes = layer_work(b, storage_bytes)
         info = lyr.kernelInfo()
         res = bool(int(b.getFlags()) & 1)
-        key = (t, getattr(b, "kernel_", 0), b.inputChannels_, b.outputChannels_, b.height_, b.width_, tuple(b.downsample_), res)
+        # (layers of one shape that run different kernels -- one of them carries a shortcut projection, say -- are rows of their own)
+        key = (t, getattr(b, "kernel_", 0), b.inputChannels_, b.outputChannels_, b.height_, b.width_, tuple(b.downsample_), res, info)
         g = groups.setdefault(key, {"ms": 0.0, "n": 0, "layer": lyr, "flops": flops, "bytes": nbytes, "passes": passes, "info": info,
                                     "launches": launches_of(info), "res": res})
         g["ms"] += ms
