@@ -60,15 +60,21 @@ def make_net(workload):
         kind = workload[3:]
         if kind not in BandwidthNet.KINDS:
             raise SystemExit("unknown workload %s (bw-%s)" % (workload, "|bw-".join(BandwidthNet.KINDS)))
-        return BandwidthNet(kind), "%s 128x1024x1024 fp16 GB/s" % kind, "GB/s", "fp16 storage"
+        return BandwidthNet(kind), "%s %s fp16 GB/s" % (kind, BandwidthNet.size_text(kind)), "GB/s", "fp16 storage"
     raise SystemExit("unknown workload %s" % workload)
 
 
 class BandwidthNet(fa.NeuralNetwork):
-    """One layer of a bandwidth-bound class on a 128 x 1024 x 1024 fp16 tensor (268 MB), inputs fed from the host."""
-    KINDS = ("dwconv", "maxpool", "avgpool", "batchnorm", "add", "concat", "scale", "sigmoid")
+    """One layer of a bandwidth-bound class on a 128 x 1024 x 1024 fp16 tensor (268 MB), inputs fed from the host; the
+    fully connected layer (gemv) multiplies a vector of 8192 by an 8192 x 8192 fp16 matrix (134 MB of weights)."""
+    KINDS = ("dwconv", "maxpool", "avgpool", "globalpool", "batchnorm", "add", "concat", "argmax", "gemv", "scale", "sigmoid")
     C, S = 128, 1024
+    GEMV_N = 8192
     output_layer = 1
+
+    @classmethod
+    def size_text(cls, kind):
+        return "%dx%d" % (cls.GEMV_N, cls.GEMV_N) if kind == "gemv" else "%dx%dx%d" % (cls.C, cls.S, cls.S)
 
     def __init__(self, kind):
         super().__init__(fa.STORAGE_F16)
@@ -82,6 +88,12 @@ class BandwidthNet(fa.NeuralNetwork):
         elif k in ("maxpool", "avgpool"):
             op = fa.PoolLayerBuilder.POOL_MAX if k == "maxpool" else fa.PoolLayerBuilder.POOL_AVG
             b = fa.PoolLayerBuilder(op, k).shape(C, S, S, C).poolSize(2).downsample(2)
+        elif k == "globalpool":
+            b = fa.PoolLayerBuilder(fa.PoolLayerBuilder.POOL_AVG, k).shape(C, S, S, C).prefixAct(fa.ActType.RELU).global_pool()
+        elif k == "argmax":
+            b = fa.ArgMaxLayerBuilder(k).shape(2, S, S, C)
+        elif k == "gemv":
+            b = fa.GPULayerBuilder(k).type(fa.LayerType.GEMM).shape(self.GEMV_N, 1, 1, self.GEMV_N)
         elif k == "batchnorm":
             b = fa.GPULayerBuilder(k).type(fa.LayerType.BATCHNORM).shape(C, S, S, C).prefixAct(fa.ActType.RELU)
         elif k == "add":
@@ -107,6 +119,9 @@ class BandwidthNet(fa.NeuralNetwork):
             layers[1].loadWeightsAndBiases(np.concatenate([np.zeros(C, np.float32), np.full(9 * C, 1.0 / 9.0, np.float32)]), 0)
         elif self.kind == "batchnorm":
             layers[1].loadScaleAndBias(np.concatenate([np.full(C, 0.5, np.float32), np.zeros(C, np.float32)]), 0)
+        elif self.kind == "gemv":
+            n = self.GEMV_N
+            layers[1].loadWeightsAndBiases(np.concatenate([np.zeros(n, np.float32), np.full(n * n, 1.0 / n, np.float32)]), 0)
 
     def ports(self):
         C, S = self.C, self.S
@@ -116,6 +131,8 @@ class BandwidthNet(fa.NeuralNetwork):
             return [(C // 2, S, S)] * 2
         if self.kind == "scale":
             return [(C, S // 2, S // 2)]
+        if self.kind == "gemv":
+            return [(self.GEMV_N, 1, 1)]
         return [(C, S, S)]
 
     def makeInput(self):
@@ -129,6 +146,8 @@ class BandwidthNet(fa.NeuralNetwork):
         """Bytes one launch has to move: every input element once, every output element once (fp16)."""
         n_in = sum(c * h * w for c, h, w in self.ports())
         oc, oh, ow = self.layers[1].outputShape()[:3]
+        if self.kind == "gemv":   # the weight matrix and the bias, once
+            n_in += self.GEMV_N * self.GEMV_N + self.GEMV_N
         return 2 * (n_in + oc * oh * ow)
 
 
@@ -388,12 +407,13 @@ def cpu_baseline(net, x, unit, total_flops):
     threads = min(os.cpu_count() or 1, 16)
     O.set_threads(threads)
     rec = {"unit": unit, "cores": threads, "kind": "port"}
+    double_note = "; the oracle accumulates in double, the reference's unit-test function paddedConvolution in float (somewhat faster)"
     if total_flops <= 100e9:
         t0 = time.perf_counter()
         O.run_network(net.describe(), {net.input_key: x})
         dt = time.perf_counter() - t0
         cpu_ms = dt * 1e3
-        rec["sample"] = "one whole step (%.1f GFLOP) through the oracle, %.1f s on %d threads" % (total_flops / 1e9, dt, threads)
+        rec["sample"] = "one whole step (%.1f GFLOP) through the oracle, %.1f s on %d threads" % (total_flops / 1e9, dt, threads) + double_note
     else:
         convs = [l for l in net.layers if int(l.builder.type_) == int(fa.LayerType.CONVOLUTION2D) and getattr(l.builder, "groupSize_", 1) == 1]
         lyr = min(convs, key=lambda l: abs(conv_work(l.builder)[0] - 20e9))   # a layer of about 20 GFLOP: 10-30 s of CPU work
@@ -406,7 +426,7 @@ def cpu_baseline(net, x, unit, total_flops):
         O.run_layer(b, lyr.weights, ins)
         dt = time.perf_counter() - t0
         cpu_ms = dt * 1e3 * total_flops / flops
-        rec["sample"] = "layer %s at full size (%.2f GFLOP, %.2f s on %d threads), scaled by the step's %.1f GFLOP" % (lyr.name, flops / 1e9, dt, threads, total_flops / 1e9)
+        rec["sample"] = "layer %s at full size (%.2f GFLOP, %.2f s on %d threads), scaled by the step's %.1f GFLOP" % (lyr.name, flops / 1e9, dt, threads, total_flops / 1e9) + double_note
     rec["value"] = cpu_ms if unit == "ms/frame" else (cpu_ms * 1e3 if unit == "us" else 1e3 / cpu_ms)
     # BASELINE config 1 on ONE core, in full: 3x3 64->64 at 256x256, ReLU on fetch (4.83 GFLOP)
     O.set_threads(1)
@@ -468,6 +488,30 @@ def measure(workload, steps, warmup, want_roofline=True):
     return net, x, rec, total_flops
 
 
+def summary_line(rec):
+    """One line per workload for the end of stderr: value, unit, the dominant kernel with its fraction of the bound,
+    the sum of kernel times against the sum of bounds, launches."""
+    roof, whole = rec.get("roofline", {}), rec.get("network_roofline", {})
+    kern = (roof.get("kernel") or "").split(" ")[0]
+    return "SUMMARY %-52s %10.4f %-8s | dominant %s (%s) x%d %.2f us, %s-bound frac %.3f | kernels %.1f us / bounds %.1f us = %.2f, %d launches" % (
+        rec["metric"], rec["value"], rec["unit"], roof.get("layer", "-"), kern, roof.get("launches_per_step", 0), roof.get("avg_launch_us", 0.0),
+        roof.get("bound", "-"), roof.get("frac", 0.0), whole.get("sum_kernel_us", 0.0), whole.get("sum_bound_us", 0.0), whole.get("frac_of_bound", 0.0),
+        whole.get("launches_per_step", 0))
+
+
+def bandwidth_block(steps, warmup):
+    """Achieved HBM rate of every bandwidth-bound layer class on a tensor far beyond the caches (128 x 1024 x 1024 fp16;
+    the fully connected layer on an 8192 x 8192 fp16 matrix): algorithmic bytes / average launch time, against 8 TB/s."""
+    block = {}
+    for kind in BandwidthNet.KINDS:
+        n, _x, r, _f = measure("bw-" + kind, steps, warmup)
+        n.cleanup()
+        roof = r["roofline"]
+        block[kind] = {"GB_per_s": roof["achieved"], "frac": roof["frac"], "avg_launch_us": roof["avg_launch_us"],
+                       "algorithmic_bytes_per_launch": roof["algorithmic_bytes_per_launch"], "size": BandwidthNet.size_text(kind)}
+    return block
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -519,6 +563,7 @@ def main():
         out["frame_pool"] = frame_pool_rate_in_child(args.workload, max(8 * args.steps, 400))
         log("frame pool: %s" % out["frame_pool"])
 
+    lines = [summary_line(rec)]
     if not args.no_also and args.workload == "stylenet":
         # the other BASELINE configurations and the reference's own sample graphs, each with its own roofline record
         also = {}
@@ -533,7 +578,14 @@ def main():
             if wl == "resnet50" and not args.no_pool:
                 entry["frame_pool"] = frame_pool_rate_in_child(wl, 800)
             also[r2["metric"]] = entry
+            lines.append(summary_line(r2))
+        also["bandwidth"] = bandwidth_block(min(max(args.steps // 4, 10), 25), min(args.warmup, 3))
+        for kind, b in also["bandwidth"].items():
+            lines.append("SUMMARY bandwidth class %-10s %-14s fp16 %8.0f GB/s = %.3f of 8 TB/s (%.1f us per launch)" % (kind, b["size"], b["GB_per_s"], b["frac"], b["avg_launch_us"]))
         out["also"] = also
+    # the figures the metric names, once more at the very end of stderr (a record keeps the tail of it)
+    for ln in lines:
+        log(ln)
     print(json.dumps(out), flush=True)
 
 

@@ -128,6 +128,7 @@ SYMBOLS = {
     "fyn_net_async_wait": (ctypes.c_int, [_P, ctypes.c_uint64]),
     "fyn_net_async_end": (ctypes.c_int, [_P]),
     "fyn_layer_kernel_info": (ctypes.c_int, [_P, ctypes.c_int, ctypes.c_char_p, ctypes.c_size_t]),
+    "fyn_net_device_allocations": (ctypes.c_int, [_P, ctypes.POINTER(ctypes.c_size_t), ctypes.POINTER(ctypes.c_size_t)]),
 }
 
 _lib = None

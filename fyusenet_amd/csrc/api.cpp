@@ -284,6 +284,13 @@ int fyn_net_async_end(fyn_net* net) {
     FYN_API_END
 }
 
+int fyn_net_device_allocations(fyn_net* net, size_t* calls, size_t* bytes) {
+    FYN_API_BEGIN
+    if (calls) *calls = N(net)->alloc_calls_;
+    if (bytes) *bytes = N(net)->alloc_bytes_;
+    FYN_API_END
+}
+
 int fyn_layer_kernel_info(fyn_net* net, int layer, char* buf, size_t buflen) {
     FYN_API_BEGIN
     if (!buf || buflen == 0) fynhip::fail(FYN_ERR_INVALID, "null buffer");

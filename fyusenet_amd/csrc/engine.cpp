@@ -182,6 +182,8 @@ void* Net::dev_alloc(size_t bytes, bool zero) {
     if (bytes == 0) bytes = 16;
     FYN_HIP(hipMalloc(&p, bytes));
     allocs_.push_back(p);
+    alloc_calls_++;
+    alloc_bytes_ += bytes;
     if (zero) {
         launch_fill_zero(p, bytes, stream);
         FYN_HIP(hipGetLastError());

@@ -163,6 +163,10 @@ class Net {
     void collect_timings();
     void dump_layer(Layer* l);
     std::vector<void*> allocs_;
+  public:
+    // device allocations made for this network since it was created (calls of hipMalloc, bytes asked for)
+    size_t alloc_calls_ = 0, alloc_bytes_ = 0;
+  private:
     float* staging_ = nullptr;
     size_t staging_floats_ = 0;
     float* static_scratch_ = nullptr;   // this device's address of the fixed staging area

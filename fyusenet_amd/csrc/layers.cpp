@@ -1818,8 +1818,8 @@ class ConvLayer : public Layer {
     }
     void forward(hipStream_t s) override {
         if (!have_weights) fail(FYN_ERR_STATE, "layer %s (%d): forward() without weights", d.name, d.number);
-        if (pj_into >= 0 && net->fusion_on()) return;   // computed by the layer that adds it
-        if (pj_fused && net->fusion_on()) {
+        if (pj_into >= 0 && net->fusion_on() && static_cast<ConvLayer*>(net->layer(pj_into))->pj_spread_ok) return;   // computed by the layer that adds it
+        if (pj_fused && pj_spread_ok && net->fusion_on()) {
             ConvP16Params q = pj;   // (value-range words as the layer's own launch carries them)
             q.in_amax = tin(0).amax;
             q.in2_amax = net->layer(pj_layer_no)->tin(0).amax;
@@ -1868,8 +1868,9 @@ class ConvLayer : public Layer {
         if (wide && !fused) launch_shift_reduce(sr, s);
     }
     std::string info() const override {
-        if (pj_into >= 0) return "conv 1x1 projection (runs inside the launch of layer " + std::to_string(pj_into) + "; no launch of its own); apart: " + own_info();
-        if (pj_fused) {
+        if (pj_into >= 0 && static_cast<ConvLayer*>(net->layer(pj_into))->pj_spread_ok)
+            return "conv 1x1 projection (runs inside the launch of layer " + std::to_string(pj_into) + "; no launch of its own); apart: " + own_info();
+        if (pj_fused && pj_spread_ok) {
             char buf[300];
             snprintf(buf, sizeof(buf), "conv_kr16 %s tile=%dx16(cout x pos) K-resident over two tensors, 4 waves split %d chunks (%d of them of the 1x1 projection %d, whose result the layer adds), blocks=%d lds=%zu; apart: ",
                      pj.f16 ? "f16" : "f16x2-split", 16 * pj.wm, pj.cin_chunks, pj.cin_chunks - pj.in2_chunk0, pj_layer_no, pj.pos_groups * pj.cout_blocks, conv_kr16_lds_bytes(pj, 1));
@@ -1994,6 +1995,7 @@ class ConvLayer : public Layer {
     // reduction over two tensors (fuse_projection_layers below): the rows of both weight matrices carry their layers'
     // folded scales, the bias is the sum of both, and the projection's tensor is never written.
     bool pj_fused = false;
+    bool pj_spread_ok = true;   // set with the weights (pack_two_sources): false keeps the two launches
     int pj_layer_no = -1;   // the projection this layer computes
     int pj_into = -1;       // on the projection: the layer that computes it
     ConvP16Params pj{};
@@ -2011,14 +2013,21 @@ class ConvLayer : public Layer {
         // (batch-norm on the residual: the layer's scale multiplies what it adds, convlayerbase's residual variant)
         const bool rs = (d.flags & FYN_FLAG_BATCHNORM_ON_RESIDUAL) && (d.flags & FYN_FLAG_POST_BATCHNORM);
         std::vector<float> wa((size_t)oc * c1), wb((size_t)oc * c2), ones(padded, 0.f), bias(padded, 0.f);
-        float mx = 0.f;
+        float mx = 0.f, row_lo = 0.f;
         for (int o = 0; o < oc; o++) {
             const float r2 = rs ? s1[o] * s2[o] : s2[o];
-            for (int i = 0; i < c1; i++) mx = std::max(mx, std::fabs(wa[(size_t)o * c1 + i] = w1[(size_t)o * c1 + i] * s1[o]));
-            for (int i = 0; i < c2; i++) mx = std::max(mx, std::fabs(wb[(size_t)o * c2 + i] = w2[(size_t)o * c2 + i] * r2));
+            float row = 0.f;
+            for (int i = 0; i < c1; i++) row = std::max(row, std::fabs(wa[(size_t)o * c1 + i] = w1[(size_t)o * c1 + i] * s1[o]));
+            for (int i = 0; i < c2; i++) row = std::max(row, std::fabs(wb[(size_t)o * c2 + i] = w2[(size_t)o * c2 + i] * r2));
+            mx = std::max(mx, row);
+            if (row > 0.f) row_lo = row_lo == 0.f ? row : std::min(row_lo, row);
             ones[o] = 1.f;
             bias[o] = o1[o] + (rs ? s1[o] * o2[o] : o2[o]);
         }
+        // The folded scales ride on the weights and one power of two brings the largest of them to the top of fp16's
+        // range: a row 2^16 times smaller than the largest still keeps 20 bits (11 in a single fp16 plane); beyond that
+        // spread the pair runs as two launches, where each layer's scale multiplies its fp32 sum.
+        pj_spread_ok = !(row_lo > 0.f) || mx <= row_lo * 65536.f;
         const float wmul = weight_prescale(&mx, 1);
         pj.acc_mul = 1.0f / wmul;
         std::vector<uint16_t> pack((size_t)pj.cout_blocks * 4 * steps * fm_n * npl * 64 * 8, 0);
@@ -2052,7 +2061,8 @@ class ConvLayer : public Layer {
         FYN_HIP(hipStreamSynchronize(net->stream));
     }
     bool takes_depthwise() const {
-        return p16 && ((kr16 && pp.tile_h == 4 && pp.tile_w == 4) || d16) && k == 1 && stride == 1 && !clamp && !pp.in_amax && !pp.in_clamp;
+        // (not a layer that already runs the depthwise layer behind it: one launch cannot do both)
+        return p16 && !edw_fused && ((kr16 && pp.tile_h == 4 && pp.tile_w == 4) || d16) && k == 1 && stride == 1 && !clamp && !pp.in_amax && !pp.in_clamp;
     }
     int launch_with_depthwise(const ConvP16Params& q, hipStream_t s) const { return d16 ? launch_conv_d16(q, s) : launch_conv_kr16(q, 1, s); }
     int launch_own(hipStream_t s) const { return d16 ? launch_conv_d16(pp, s) : launch_conv_kr16(pp, 1, s); }
@@ -2159,8 +2169,15 @@ void fuse_depthwise_layers(Net* net) {
         ConvLayer* ex = dynamic_cast<ConvLayer*>(net->layer(t.producer));
         if (!ex || ex->k != 1 || ex->stride != 1 || ex->dil != 1 || ex->clamp || ex->frac_shift || ex->direct || (ex->d.flags & FYN_FLAG_RESIDUAL_INPUT)) continue;
         const TView& in_v = ex->tin(0).v;
-        // (the launch reads the 1x1 layer's input while it writes the depthwise layer's output: not in one buffer)
-        if (net->tensors[dw->out].buffer == net->tensors[ex->in[0]].buffer) continue;
+        // The launch writes the depthwise layer's output in the 1x1 layer's place in the order, i.e. earlier than the
+        // buffer was handed over for: every other tenant of that buffer must be through by then -- neither read at or
+        // behind the 1x1 layer (its own input included: the launch reads it while it writes) nor produced between the two.
+        bool early_ok = true;
+        for (const Tensor& o : net->tensors)
+            if (&o != &net->tensors[dw->out] && o.buffer == net->tensors[dw->out].buffer && o.producer < dw->d.number &&
+                std::max(o.last_reader, o.producer) >= ex->d.number)
+                early_ok = false;
+        if (!early_ok) continue;
         if (in_v.f16 != dw->p.out.f16 || ex->d.in_channels != in_v.cp || ex->tout().v.cp != dw->p.in.cp || ex->oc % 4 != 0 ||
             !conv_e16dw_supported(in_v.cp, (in_v.cp + 31) / 32, dw->stride))
             continue;
@@ -2240,8 +2257,15 @@ void fuse_depthwise_layers(Net* net) {
         if (!dw || dw->dil != 1 || (dw->stride != 1 && dw->stride != 2) || dw->p.res.ptr || dw->p.in.cp % 8 != 0 || dw->p.in.cp != dw->p.out.cp ||
             dw->p.in.f16 != dw->p.out.f16 || dw->p.out.f16 != pw->pp.f16 || dw->p.out.cp != pw->pp.in_cp)
             continue;
-        // (the launch reads the depthwise layer's input while it writes the 1x1 layer's output: not in one buffer)
-        if (net->tensors[pw->out].buffer == net->tensors[dw->in[0]].buffer) continue;
+        // The launch reads the depthwise layer's input in the 1x1 layer's place in the order, i.e. later than the buffer
+        // was kept for: no tensor produced behind the depthwise layer up to and including the 1x1 layer (whose output
+        // the launch writes while it reads) may live in that buffer.
+        bool late_ok = true;
+        for (const Tensor& o : net->tensors)
+            if (&o != &net->tensors[dw->in[0]] && o.buffer == net->tensors[dw->in[0]].buffer && o.producer > dw->d.number &&
+                o.producer <= pw->d.number)
+                late_ok = false;
+        if (!late_ok) continue;
         ConvP16Params& f = pw->dw_fields;
         f.dw_in = dw->p.in.ptr; f.dw_w = dw->w_dev; f.dw_scale = dw->scale_dev; f.dw_bias = dw->bias_dev;
         f.dw_hp = dw->p.in.hp(); f.dw_wp = dw->p.in.wp(); f.dw_cp = dw->p.in.cp;

@@ -282,6 +282,10 @@ int fyn_net_async_wait(fyn_net* net, uint64_t ticket);
 /* Floats per frame that submit reads from `in` and writes to `out` (between begin and end). */
 int fyn_net_async_sizes(fyn_net* net, size_t* in_floats, size_t* out_floats);
 int fyn_net_async_end(fyn_net* net);
+/* Device allocations this network has made since fyn_net_create: number of hipMalloc calls and the bytes asked for
+ * (both only ever grow).  A diagnostic without a counterpart in the reference, whose textures belong to the GL driver;
+ * it lets a caller check that a call sequence of its serving loop allocates nothing. */
+int fyn_net_device_allocations(fyn_net* net, size_t* calls, size_t* bytes);
 /* Text description of the kernel variant chosen for a layer (for profiles / reports). */
 int fyn_layer_kernel_info(fyn_net* net, int layer, char* buf, size_t buflen);
 

@@ -466,7 +466,7 @@ def port_channels(b, port):
     return b.outputChannels_ if port == 1 else None       # residual input
 
 
-def run_network(desc, inputs, fp16_storage=None, forced=None):
+def run_network(desc, inputs, fp16_storage=None, forced=None, known=None, only=None):
     """Executes a network description on the CPU.
 
     desc: NeuralNetwork.describe(); inputs: {(layer_number, port): CHW array} for upload layers
@@ -474,15 +474,19 @@ def run_network(desc, inputs, fp16_storage=None, forced=None):
     fp16_storage: emulate fp16 tensors/weights (default: desc['storage'] == 1).
     forced: optional {layer_number: CHW array}; when given, every layer reads these tensors instead of
     the oracle's own upstream results (per-layer check on identical inputs).
+    known / only: evaluate a part of the graph: `only` is the set of layer numbers to run, `known` holds the tensors
+    that this part reads from layers outside it ({layer_number: CHW array}).
     """
     f16 = (desc.get("storage", 0) == 1) if fp16_storage is None else fp16_storage
     rnd = round_fp16 if f16 else (lambda a: np.asarray(a, dtype=np.float32))
     feeds = {}
     for (src, dst, port) in desc["connections"]:
         feeds[(dst, port)] = src
-    outs = {}
+    outs = dict(known) if known else {}
     for entry in sorted(desc["layers"], key=lambda e: e["number"]):
         b, no, w = entry["builder"], entry["number"], entry["weights"]
+        if only is not None and no not in only:
+            continue
         ins = []
         for port in range(num_ports(b)):
             if (no, port) in feeds:

@@ -7,11 +7,15 @@ import pytest
 
 import fyusenet_amd as fa
 from fyusenet_amd import prng
-from util import conv_block, oracle_single, rel_l2, run_single
+from util import combos, conv_block, oracle_single, rel_l2, run_single
 
 pytestmark = pytest.mark.gpu
 TOL = {fa.STORAGE_F32: 1e-4, fa.STORAGE_F16: 2e-3}
 A = fa.ActType
+# axes of the generated combinations: (values, id function)
+STORAGE_AXIS = ([fa.STORAGE_F32, fa.STORAGE_F16], lambda s: "f32" if s == fa.STORAGE_F32 else "f16")
+SHALLOW_AXIS = ([False, True], lambda sh: "shallow_edge_clamp" if sh else "deep")
+ACT3_AXIS = ([A.RELU, A.LEAKY_RELU, A.NONE], lambda a: {A.RELU: "relu", A.LEAKY_RELU: "leaky", A.NONE: "none"}[a])
 
 
 def conv_builder(k, cout, h, w, cin, stride=1, dil=1, act=A.NONE, deep=True, pad_in=None, pad_out=0, bn=False, residual=None,
@@ -225,14 +229,13 @@ ROWS_CASES = WIDE_CASES[:3] + [
 ]
 
 
-@pytest.mark.parametrize("storage", [fa.STORAGE_F32, fa.STORAGE_F16], ids=["f32", "f16"])
-@pytest.mark.parametrize("shallow", [False, True], ids=["deep", "shallow_edge_clamp"])
-@pytest.mark.parametrize("case", ROWS_CASES, ids=lambda c: "k%d_%dx%dx%d_to%d" % (c[0], c[4], c[2], c[3], c[1]))
+@pytest.mark.parametrize(*combos(
+    # (the shallow variant is run on the plain cases)
+    lambda case, shallow, storage: not (shallow and ("residual" in case[5] or "pad_out" in case[5])),
+    case=(ROWS_CASES, lambda c: "k%d_%dx%dx%d_to%d" % (c[0], c[4], c[2], c[3], c[1])), shallow=SHALLOW_AXIS, storage=STORAGE_AXIS))
 def test_wide_kernel_row_rolling_form(case, shallow, storage, monkeypatch):
     """The folded-kx convolution with the input rows rolled through an LDS ring and the weights held in registers."""
     k, cout, h, w, cin, kw = case
-    if shallow and ("residual" in kw or "pad_out" in kw):
-        pytest.skip("the shallow variant is run on the plain cases")
     monkeypatch.setenv("FYNHIP_FORCE_ROWS_WIDE_CONV", "1")
     if shallow:   # unpadded shallow input: the sampler repeats the edge
         kw = dict(kw, deep=False, pad_in=0)
@@ -277,20 +280,21 @@ P16_CASES = [
 ]
 
 
-@pytest.mark.parametrize("storage", [fa.STORAGE_F32, fa.STORAGE_F16], ids=["f32", "f16"])
-@pytest.mark.parametrize("shallow", [False, True], ids=["deep", "shallow_edge_clamp"])
-@pytest.mark.parametrize("act", [A.RELU, A.LEAKY_RELU, A.NONE], ids=["relu", "leaky", "none"])
-@pytest.mark.parametrize("case", P16_CASES, ids=lambda c: "%dx%dx%d_to%d_s%d_%s" % (c[0], c[2], c[3], c[1], c[4], (c[5] or "auto").replace(",", "x")))
+def _p16_runs(case, act, shallow, storage):
+    cin, cout, h, w, stride, tile, kw = case
+    if shallow and ("residual" in kw or "pad_out" in kw):
+        return False   # the shallow variant is run on the plain cases
+    if act is not A.RELU and ("pad_out" in kw or tile in ("4,4,4", "8,6,4", "8,8,4", "8,4,2", "4,8,2") or h > 60):
+        return False   # activations are varied on some of the cases
+    return not (storage == fa.STORAGE_F16 and (act is A.NONE or (shallow and h > 30)))   # fp16 storage on some of the combinations
+
+
+@pytest.mark.parametrize(*combos(_p16_runs, case=(P16_CASES, lambda c: "%dx%dx%d_to%d_s%d_%s" % (c[0], c[2], c[3], c[1], c[4], (c[5] or "auto").replace(",", "x"))),
+                                 act=ACT3_AXIS, shallow=SHALLOW_AXIS, storage=STORAGE_AXIS))
 def test_sixteen_position_fragment_form(case, act, shallow, storage, monkeypatch):
     """The 3x3 convolution on 16-position fragments: every compiled tile, ragged edges, the residual tile through LDS;
     fp32 storage (operand split, value ranges on both sides) and fp16 storage (one plane, one pass)."""
     cin, cout, h, w, stride, tile, kw = case
-    if shallow and ("residual" in kw or "pad_out" in kw):
-        pytest.skip("the shallow variant is run on the plain cases")
-    if act is not A.RELU and ("pad_out" in kw or tile in ("4,4,4", "8,6,4", "8,8,4", "8,4,2", "4,8,2") or h > 60):
-        pytest.skip("activations are varied on some of the cases")
-    if storage == fa.STORAGE_F16 and (act is A.NONE or (shallow and h > 30)):
-        pytest.skip("fp16 storage is run on some of the combinations")
     if storage == fa.STORAGE_F16:
         monkeypatch.setenv("FYNHIP_NO_H16_CONV", "1")   # (the form with 64-channel wave tiles has its own test)
     monkeypatch.setenv("FYNHIP_FORCE_P16_CONV", "1")
@@ -336,17 +340,19 @@ H16_CASES = [
 ]
 
 
-@pytest.mark.parametrize("shallow", [False, True], ids=["deep", "shallow_edge_clamp"])
-@pytest.mark.parametrize("act", [A.RELU, A.LEAKY_RELU, A.NONE], ids=["relu", "leaky", "none"])
-@pytest.mark.parametrize("case", H16_CASES, ids=lambda c: "k%d_%dx%dx%d_to%d_%s" % (c[0], c[1], c[3], c[4], c[2], (c[5] or "auto").replace(",", "x").replace(";", "_")))
+def _h16_runs(case, act, shallow):
+    k, cin, cout, h, w, tile, kw = case
+    if shallow and ("residual" in kw or "pad_out" in kw or h > 100):
+        return False   # the shallow variant is run on the plain cases
+    return not (act is not A.RELU and ("pad_out" in kw or h > 100 or cout > 128))   # activations are varied on some of the cases
+
+
+@pytest.mark.parametrize(*combos(_h16_runs, case=(H16_CASES, lambda c: "k%d_%dx%dx%d_to%d_%s" % (c[0], c[1], c[3], c[4], c[2], (c[5] or "auto").replace(",", "x").replace(";", "_"))),
+                                 act=ACT3_AXIS, shallow=SHALLOW_AXIS))
 def test_fp16_sixteen_position_fragment_form(case, act, shallow, monkeypatch):
     """The 3x3 / 9x9 convolution between wide fp16 tensors on 16-position fragments: every compiled tile, ragged edges,
     tile walking, the residual tile through LDS."""
     k, cin, cout, h, w, tile, kw = case
-    if shallow and ("residual" in kw or "pad_out" in kw or h > 100):
-        pytest.skip("the shallow variant is run on the plain cases")
-    if act is not A.RELU and ("pad_out" in kw or h > 100 or cout > 128):
-        pytest.skip("activations are varied on some of the cases")
     monkeypatch.setenv("FYNHIP_FORCE_P16_CONV", "1")
     split = None
     if tile and ";" in tile:
@@ -427,18 +433,19 @@ KR16_CASES = [
 ]
 
 
-@pytest.mark.parametrize("storage", [fa.STORAGE_F32, fa.STORAGE_F16], ids=["f32", "f16"])
-@pytest.mark.parametrize("shallow", [False, True], ids=["deep", "shallow_edge_clamp"])
-@pytest.mark.parametrize("act", [A.RELU, A.LEAKY_RELU], ids=["relu", "leaky"])
-@pytest.mark.parametrize("case", KR16_CASES, ids=lambda c: "k%d_%dx%dx%d_to%d_fm%s%s" % (c[0], c[1], c[3], c[4], c[2], str(c[5]).replace(",", "x"), "_s2" if c[6].get("stride") == 2 else ""))
+def _kr16_runs(case, act, shallow, storage):
+    k, cin, cout, h, w, fm, kw = case
+    if shallow and (k == 1 or "residual" in kw or "pad_out" in kw):
+        return False   # the shallow variant is run on the plain 3x3 cases
+    return not (act is A.LEAKY_RELU and (cin > 512 or "pad_out" in kw))   # activations are varied on some of the cases
+
+
+@pytest.mark.parametrize(*combos(_kr16_runs, case=(KR16_CASES, lambda c: "k%d_%dx%dx%d_to%d_fm%s%s" % (c[0], c[1], c[3], c[4], c[2], str(c[5]).replace(",", "x"), "_s2" if c[6].get("stride") == 2 else "")),
+                                 act=([A.RELU, A.LEAKY_RELU], lambda a: "relu" if a is A.RELU else "leaky"), shallow=SHALLOW_AXIS, storage=STORAGE_AXIS))
 def test_reduction_resident_form(case, act, shallow, storage, monkeypatch):
     """1x1 / 3x3 convolutions on few positions and many input channels with a tile's whole reduction resident in LDS and
     the four MFMA waves of a workgroup splitting the chunks."""
     k, cin, cout, h, w, fm, kw = case
-    if shallow and (k == 1 or "residual" in kw or "pad_out" in kw):
-        pytest.skip("the shallow variant is run on the plain 3x3 cases")
-    if act is A.LEAKY_RELU and (cin > 512 or "pad_out" in kw):
-        pytest.skip("activations are varied on some of the cases")
     monkeypatch.setenv("FYNHIP_FORCE_KR16_CONV", "1")
     monkeypatch.setenv("FYNHIP_KR16_FM", str(fm))
     if shallow:
@@ -487,15 +494,15 @@ D16_CASES = [
 ]
 
 
-@pytest.mark.parametrize("storage", [fa.STORAGE_F32, fa.STORAGE_F16], ids=["f32", "f16"])
-@pytest.mark.parametrize("variant", ["relu", "leaky", "shallow"])
-@pytest.mark.parametrize("case", D16_CASES, ids=lambda c: "%dx%dx%d_to%d%s%s" % (c[0], c[2], c[3], c[1], "_s2" if c[4].get("stride") == 2 else "", ("_b%d" % c[4]["blocks"]).replace("-", "w") if "blocks" in c[4] else ""))
+@pytest.mark.parametrize(*combos(
+    # (activation and the shallow variant are varied on the plain cases)
+    lambda case, variant, storage: variant == "relu" or not ("residual" in case[4] or "pad_out" in case[4] or "blocks" in case[4] or case[0] > 100),
+    case=(D16_CASES, lambda c: "%dx%dx%d_to%d%s%s" % (c[0], c[2], c[3], c[1], "_s2" if c[4].get("stride") == 2 else "", ("_b%d" % c[4]["blocks"]).replace("-", "w") if "blocks" in c[4] else "")),
+    variant=(["relu", "leaky", "shallow"], str), storage=STORAGE_AXIS))
 def test_pointwise_without_lds(case, variant, storage, monkeypatch):
     """1x1 convolutions on many positions whose B fragments come straight from the tensor: a workgroup of four waves per
     16 positions, the waves sharing the fragments of output channels."""
     cin, cout, h, w, kw = case
-    if variant != "relu" and ("residual" in kw or "pad_out" in kw or "blocks" in kw or cin > 100):
-        pytest.skip("activation and the shallow variant are varied on the plain cases")
     monkeypatch.setenv("FYNHIP_FORCE_D16_CONV", "1")
     kw = dict(kw)
     stride = kw.pop("stride", 1)
@@ -562,6 +569,13 @@ ALL_TILES = ["2,2,2,2", "2,2,1,4", "2,1,2,2", "2,1,1,4", "1,2,1,4", "1,1,1,4", "
              "1,2,2,2", "1,4,2,2", "1,3,2,2", "1,4,1,4", "1,3,1,4", "1,1,1,1", "1,1,2,1", "1,1,1,2"]
 
 
+# Combinations for which the engine has no such tile and says so: the halo tile of the widest shape (32 x 512 positions)
+# in two fp32 operand planes is more than a CU's LDS (for the 5x5 kernel with step 2 also the next narrower), and the
+# tiles whose waves split the reduction exist for chunks of 32 channels and more.
+NO_SUCH_TILE = {(kk, "1,4,1,4", fa.STORAGE_F32) for kk in (3, 1, 5)} | {(5, "1,3,1,4", fa.STORAGE_F32)} | \
+               {(5, t, st) for t in ("1,1,1,1", "1,1,2,1", "1,1,1,2") for st in (fa.STORAGE_F32, fa.STORAGE_F16)}
+
+
 @pytest.mark.parametrize("storage", [fa.STORAGE_F32, fa.STORAGE_F16], ids=["f32", "f16"])
 @pytest.mark.parametrize("tile", ALL_TILES)
 @pytest.mark.parametrize("k,cin,cout,h,w,stride,kw", [
@@ -578,12 +592,11 @@ def test_every_tile_shape(k, cin, cout, h, w, stride, kw, tile, storage, monkeyp
     inputs = [prng.uniform(15 * k + cin, (cin, h, w), -1, 1)]
     if "residual" in kw:
         inputs.append(prng.uniform(27, (cout, h // stride, w // stride), -1, 1))
-    try:
-        got, info = run_single(b, storage, inputs, wts)
-    except fa.FynException as e:
-        if "no MFMA tile configuration fits" in str(e):     # e.g. the K-split tiles exist for chunks of 32+ channels only
-            pytest.skip("tile %s does not exist for this layer" % tile)
-        raise
+    if (k, tile, storage) in NO_SUCH_TILE:
+        with pytest.raises(fa.FynException, match="no MFMA tile configuration fits"):
+            run_single(b, storage, inputs, wts)
+        return
+    got, info = run_single(b, storage, inputs, wts)
     fm, fn, wm, wn = (int(v) for v in tile.split(","))
     assert "tile=%dx%d" % (32 * fm * wm, 32 * fn * wn) in info and "waves=%dx%d" % (wm, wn) in info
     err = rel_l2(got, oracle_single(b, storage, inputs, wts))
@@ -658,14 +671,13 @@ C4_CASES = [
 ]
 
 
-@pytest.mark.parametrize("storage", [fa.STORAGE_F32, fa.STORAGE_F16], ids=["f32", "f16"])
-@pytest.mark.parametrize("shallow", [False, True], ids=["deep", "shallow_edge_clamp"])
-@pytest.mark.parametrize("case", C4_CASES, ids=lambda c: "%dx%dx%d_to%d_%s" % (c[0], c[2], c[3], c[1], (c[4] or "auto").replace(",", "x")))
+@pytest.mark.parametrize(*combos(
+    # (the shallow variant is run on the plain cases)
+    lambda case, shallow, storage: not (shallow and ("pad_out" in case[5] or case[2] > 60)),
+    case=(C4_CASES, lambda c: "%dx%dx%d_to%d_%s" % (c[0], c[2], c[3], c[1], (c[4] or "auto").replace(",", "x"))), shallow=SHALLOW_AXIS, storage=STORAGE_AXIS))
 def test_small_input_sixteen_position_fragment_form(case, shallow, storage, monkeypatch):
     """The 9x9 convolution on at most four input channels with two taps of a 4-channel pixel per lane and step."""
     cin, cout, h, w, tile, kw = case
-    if shallow and ("pad_out" in kw or h > 60):
-        pytest.skip("the shallow variant is run on the plain cases")
     monkeypatch.setenv("FYNHIP_FORCE_P16_CONV", "1")
     if tile:
         monkeypatch.setenv("FYNHIP_P16_TILE", tile)
@@ -700,15 +712,15 @@ TP16_CASES = [
 ]
 
 
-@pytest.mark.parametrize("storage", [fa.STORAGE_F32, fa.STORAGE_F16], ids=["f32", "f16"])
-@pytest.mark.parametrize("act", [A.RELU, A.NONE], ids=["relu", "none"])
-@pytest.mark.parametrize("case", TP16_CASES, ids=lambda c: "%dx%dx%d_to%d_%s" % (c[0], c[2], c[3], c[1], (c[4] or "auto").replace(",", "x")))
+@pytest.mark.parametrize(*combos(
+    # (the activation is varied on the small cases)
+    lambda case, act, storage: not (act is A.NONE and (case[4] is None or case[2] > 60 or storage == fa.STORAGE_F16)),
+    case=(TP16_CASES, lambda c: "%dx%dx%d_to%d_%s" % (c[0], c[2], c[3], c[1], (c[4] or "auto").replace(",", "x"))),
+    act=([A.RELU, A.NONE], lambda a: "relu" if a is A.RELU else "none"), storage=STORAGE_AXIS))
 def test_transconv_sixteen_position_fragment_form(case, act, storage, monkeypatch):
     """The doubling transposed 3x3 convolution on 16-position fragments: all four output parities from one staged input
     tile; fp32 and fp16 storage."""
     cin, cout, h, w, tile, bn = case
-    if act is A.NONE and (tile is None or h > 60 or storage == fa.STORAGE_F16):
-        pytest.skip("the activation is varied on the small cases")
     monkeypatch.setenv("FYNHIP_FORCE_P16_CONV", "1")
     if tile:
         monkeypatch.setenv("FYNHIP_P16_TILE", tile)

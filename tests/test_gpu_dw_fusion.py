@@ -10,7 +10,7 @@ import fyusenet_amd as fa
 from fyusenet_amd import networks, prng
 from fyusenet_amd.builders import ActType, UpDownLayerBuilder
 from oracle import oracle as O
-from util import rel_l2
+from util import combos, rel_l2
 
 pytestmark = pytest.mark.gpu
 TOL = {fa.STORAGE_F32: 1e-4, fa.STORAGE_F16: 2e-3}
@@ -97,13 +97,14 @@ FRONT_CASES = CASES + [
 ]
 
 
-@pytest.mark.parametrize("storage", [fa.STORAGE_F32, fa.STORAGE_F16], ids=["f32", "f16"])
-@pytest.mark.parametrize("case", FRONT_CASES, ids=lambda c: "%dto%dto%d_%dx%d_s%d%s" % (c[0], c[1], c[2], c[3], c[4], c[5], "_res" if c[6] else ""))
-@pytest.mark.parametrize("narrow", [0, 1], ids=["blocks64", "blocks16"])
-def test_depthwise_inside_the_launch_of_the_expand_layer(case, storage, narrow, monkeypatch):
+@pytest.mark.parametrize(*combos(
+    # (the 16-channel blocks are for layers with few tiles)
+    lambda narrow, case, storage: not (narrow and case[3] * case[4] > 60 * 60),
+    narrow=([0, 1], lambda n: "blocks16" if n else "blocks64"),
+    case=(FRONT_CASES, lambda c: "%dto%dto%d_%dx%d_s%d%s" % (c[0], c[1], c[2], c[3], c[4], c[5], "_res" if c[6] else "")),
+    storage=([fa.STORAGE_F32, fa.STORAGE_F16], lambda st: "f32" if st == fa.STORAGE_F32 else "f16")))
+def test_depthwise_inside_the_launch_of_the_expand_layer(narrow, case, storage, monkeypatch):
     cin, exp, cout, h, w, stride, residual = case
-    if narrow and h * w > 60 * 60:
-        pytest.skip("the 16-channel blocks are for layers with few tiles")
     monkeypatch.setenv("FYNHIP_FORCE_DW_FUSION", "1")
     monkeypatch.setenv("FYNHIP_EDW_NARROW", str(narrow))
     net = Block(storage, cin, exp, cout, h, w, stride, residual)
@@ -234,6 +235,169 @@ def test_layers_stay_apart_when_the_tensor_is_needed(monkeypatch):
         net.cleanup()
         assert rel_l2(fused, apart) <= 1e-3
         assert np.array_equal(fused, again)
+
+
+class Chain(networks._StreamNet):
+    """upload -> depthwise 3x3 -> 1x1 -> depthwise 3x3 -> 1x1 -> download (the MobileNetV1 pattern): the middle 1x1
+    layer has a depthwise layer on either side and can run only one of them inside its launch."""
+    config_id = 4
+
+    def __init__(self, storage, c, e, cout, h, w):
+        super().__init__(storage)
+        self.c, self.e, self.cout, self.h, self.w = c, e, cout, h, w
+
+    def define(self):
+        C, c6 = ActType.CLIP, (0.0, 6.0)
+        self._add(UpDownLayerBuilder(UpDownLayerBuilder.UPLOAD, "upload").number(0).shape(self.c, self.h, self.w, self.c).outputPadding(1))
+        self.conv(1, "dw1", 3, self.c, self.c, self.h, self.w, 0, groups=self.c)
+        self.conv(2, "pw1", 1, self.c, self.e, self.h, self.w, 1, act=C, clip=c6, pad_out=1)
+        self.conv(3, "dw2", 3, self.e, self.e, self.h, self.w, 2, act=C, clip=c6, groups=self.e)
+        self.conv(4, "pw2", 1, self.e, self.cout, self.h, self.w, 3, act=C, clip=c6)
+        self._add(UpDownLayerBuilder(UpDownLayerBuilder.DOWNLOAD, "download").number(5).shape(self.cout, self.h, self.w, self.cout).deep())
+        self._edges.append((4, 5, 0))
+        self.output_layer = 5
+
+    def makeInput(self):
+        return prng.uniform(4211 + self.c + self.h, (self.c, self.h, self.w), -1.0, 1.0)
+
+    def setInput(self, x):
+        self.layers[0].setInput(x, 0)
+
+    input_key = (0, 0)
+
+
+@pytest.mark.parametrize("storage", [fa.STORAGE_F32, fa.STORAGE_F16], ids=["f32", "f16"])
+@pytest.mark.parametrize("form", ["kr16", "d16"])
+def test_pointwise_layer_between_two_depthwise_layers_takes_one(storage, form, monkeypatch):
+    """The 1x1 layer in the middle is a candidate for both passes (the depthwise layer behind it as one launch, the one
+    in front of it inside its staging); it may take one, and every depthwise layer is computed exactly once."""
+    monkeypatch.setenv("FYNHIP_FORCE_KR16_CONV" if form == "kr16" else "FYNHIP_FORCE_D16_CONV", "1")
+    monkeypatch.setenv("FYNHIP_FORCE_DW_FUSION", "1")
+    net = Chain(storage, 32, 64, 48, 28, 28)
+    x, got, infos = run(net)
+    desc = net.describe()
+    net.cleanup()
+    print("  ", {k: v[:90] for k, v in infos.items() if k != "upload"}, flush=True)
+    assert "conv_e16dw" in infos["pw1"] and "launch of layer 2" in infos["dw2"]
+    assert infos["dw1"] == "dwconv3x3", "the layer that already runs the depthwise layer behind it must fetch the one in front of it"
+    ref = O.run_network(desc, {net.input_key: x})[net.output_layer]
+    err = rel_l2(got, ref)
+    print("   rel_l2=%.3e" % err, flush=True)
+    assert err <= TOL[storage]
+
+
+class Interleaved(networks._StreamNet):
+    """Two graphs in which a layer numbered between the fused pair lives in the buffer that the fused launch would read
+    late or write early.
+    kind "late" (depthwise -> 1x1): 1 a (1x1, halo) -> 2 dw -> 4 pw, and 3 mid (1x1 from the upload, same geometry as a's
+        tensor, which is free behind layer 2): a launch of layer 4 that computes layer 2 itself would read a's buffer
+        after layer 3 has overwritten it.
+    kind "early" (1x1 -> depthwise): 1 pre -> 3 side, 2 expand -> 4 dw -> 5 project; the depthwise layer's output takes
+        pre's buffer (free behind layer 3): a launch of layer 2 that also runs layer 4 would write into it before layer
+        3 has read it."""
+    config_id = 4
+
+    def __init__(self, storage, kind, c=32, h=20, w=24):
+        super().__init__(storage)
+        self.kind, self.c, self.h, self.w = kind, c, h, w
+
+    def define(self):
+        C, c6 = ActType.CLIP, (0.0, 6.0)
+        c, h, w = self.c, self.h, self.w
+        self._add(UpDownLayerBuilder(UpDownLayerBuilder.UPLOAD, "upload").number(0).shape(c, h, w, c))
+        if self.kind == "late":
+            self.conv(1, "a", 1, c, c, h, w, 0, pad_out=1)
+            self.conv(2, "dw", 3, c, c, h, w, 1, act=C, clip=c6, groups=c)
+            self.conv(3, "mid", 1, c, c, h, w, 0, pad_out=1)
+            self.conv(4, "pw", 1, c, 48, h, w, 2, act=C, clip=c6)
+            self.conv(5, "tail", 3, c, 16, h, w, 3, act=C, clip=c6)
+            self.outputs = (4, 5)
+        else:
+            self.conv(1, "pre", 1, c, c, h, w, 0)
+            self.conv(2, "expand", 1, c, c, h, w, 0, pad_out=1)
+            self.conv(3, "side", 1, c, 16, h, w, 1, act=C, clip=c6)
+            self.conv(4, "dw", 3, c, c, h, w, 2, act=C, clip=c6, groups=c)
+            self.conv(5, "project", 1, c, 48, h, w, 4, act=C, clip=c6)
+            self.outputs = (3, 5)
+
+    def makeInput(self):
+        return prng.uniform(5003 + self.c + self.h, (self.c, self.h, self.w), -1.0, 1.0)
+
+    def setInput(self, x):
+        self.layers[0].setInput(x, 0)
+
+    input_key = (0, 0)
+
+
+@pytest.mark.parametrize("storage", [fa.STORAGE_F32, fa.STORAGE_F16], ids=["f32", "f16"])
+@pytest.mark.parametrize("kind", ["late", "early"])
+def test_no_fusion_across_a_layer_that_reuses_the_buffer(kind, storage, monkeypatch):
+    monkeypatch.setenv("FYNHIP_FORCE_KR16_CONV", "1")
+    monkeypatch.setenv("FYNHIP_FORCE_DW_FUSION", "1")
+    if kind == "late":
+        monkeypatch.setenv("FYNHIP_NO_EDW_FUSION", "1")
+    net = Interleaved(storage, kind)
+    net.setup(reuseBuffers=True)
+    x = net.makeInput()
+    net.setInput(x)
+    net.forward()
+    net.finish()
+    got = {no: net.layers[no].copyResult() for no in net.outputs}
+    infos = {lyr.name: lyr.kernelInfo() for lyr in net.layers}
+    desc = net.describe()
+    net.cleanup()
+    print("  ", {k: v[:80] for k, v in infos.items() if k != "upload"}, flush=True)
+    if kind == "late":
+        assert infos["dw"] == "dwconv3x3"
+    else:
+        assert "conv_e16dw" not in infos["expand"]
+    ref = O.run_network(desc, {net.input_key: x})
+    for no in net.outputs:
+        err = rel_l2(got[no], ref[no])
+        print("   layer %d rel_l2=%.3e" % (no, err), flush=True)
+        assert err <= TOL[storage]
+
+
+class TappedMobileNetV2(networks.MobileNetV2):
+    """BASELINE's MobileNetV2-style graph with a download layer on the stem's and on every block's output: those tensors
+    keep their buffers, so they can be read after a pass in which buffers are shared and the layers inside the blocks
+    run fused (the taps are further readers of tensors between blocks, not of the tensors that the fusions remove)."""
+
+    def define(self):
+        super().define()
+        taps = [b for b in self._builders if b.name_ == "stem" or b.name_.endswith("_project")]
+        for i, b in enumerate(taps):
+            c, h, w = b.outputChannels_, b.height_ // b.downsample_[1], b.width_ // b.downsample_[0]
+            self._add(UpDownLayerBuilder(UpDownLayerBuilder.DOWNLOAD, "tap_" + b.name_).number(1000 + i).shape(c, h, w, c).inputPadding(b.outputPadding_).deep())
+            self._edges.append((b.number_, 1000 + i, 0))
+
+
+@pytest.mark.parametrize("storage", [fa.STORAGE_F32, fa.STORAGE_F16], ids=["f32", "f16"])
+def test_config4_fused_blocks_one_by_one_on_the_engines_own_inputs(storage, monkeypatch):
+    """Every inverted-residual block of the fused stack against the oracle evaluated on the engine's own block input
+    (and residual): the per-layer bound (1e-4 / 2e-3) on each block, in the storage type the benchmark runs, instead of
+    only the end-to-end bound of two free-running fp16 chains."""
+    monkeypatch.setenv("FYNHIP_FORCE_DW_FUSION", "1")
+    net = TappedMobileNetV2(storage)
+    x, got, infos = run(net)
+    desc = net.describe()
+    number = {lyr.name: lyr.number for lyr in net.layers}
+    fused = [n for n, i in infos.items() if "inside the launch" in i]
+    assert len(fused) >= 8
+    prev = number["stem"]
+    tensors = {prev: net.layers[prev].copyResult()}
+    worst = 0.0
+    for i in range(len(networks.MobileNetV2.BLOCKS)):
+        part = [number[n] for n in ("b%d_expand" % i, "b%d_dw" % i, "b%d_project" % i) if n in number]
+        out_no = number["b%d_project" % i]
+        tensors[out_no] = net.layers[out_no].copyResult()
+        ref = O.run_network(desc, {}, known={prev: tensors[prev]}, only=set(part))[out_no]
+        err = rel_l2(tensors[out_no], ref)
+        worst = max(worst, err)
+        print("   block %2d (%s) rel_l2=%.3e" % (i, "fused" if "b%d_dw" % i in fused else "apart", err), flush=True)
+        assert err <= TOL[storage], "block %d" % i
+        prev = out_no
+    net.cleanup()
 
 
 @pytest.mark.parametrize("storage", [fa.STORAGE_F32, fa.STORAGE_F16], ids=["f32", "f16"])

@@ -91,6 +91,78 @@ def test_config4_mobilenetv2_full_size(storage):
     net.cleanup()
 
 
+def _inference_output(net, graph=False):
+    net.setup(reuseBuffers=True)
+    x = net.makeInput()
+    net.setInput(x)
+    if graph:
+        net.useGraph(True)
+    net.forward()
+    net.finish()
+    out = net.getOutput(net.output_layer)
+    infos = {lyr.name: lyr.kernelInfo() for lyr in net.layers}
+    return x, out, infos
+
+
+INFERENCE_NETS = {
+    "config1": lambda st: networks.SingleConvNet(st),
+    "config2_reduced": lambda st: networks.StyleNet(st, width=128, height=156, res_kernel=3),
+    "config3": lambda st: networks.ResNet50(st),
+    "config4": lambda st: networks.MobileNetV2(st),
+    "config5_reduced": lambda st: networks.StyleNet(st, width=96, height=64, res_kernel=9),
+}
+
+
+@STORAGES
+@pytest.mark.parametrize("name", list(INFERENCE_NETS))
+def test_configs_in_the_inference_setting(name, storage):
+    """Every BASELINE configuration the way bench.py times it: buffers shared between tensors, layers that can run
+    inside a neighbour's launch doing so (by the engine's own choice), the captured graph replayed.  Only the network's
+    output is readable in this setting; it is held to the oracle's (fp32 storage: 1e-4; fp16 storage: the end-to-end
+    bound explained above) and must not change between eager launches and the replayed graph."""
+    net = INFERENCE_NETS[name](storage)
+    x, got, infos = _inference_output(net)
+    net.useGraph(True)
+    for _ in range(2):
+        net.forward()
+        net.finish()
+    replay = net.getOutput(net.output_layer)
+    hidden = [n for n, i in infos.items() if "no launch of its own" in i]
+    print("   layers without a launch of their own:", len(hidden), hidden[:8], flush=True)
+    ref = O.run_network(net.describe(), {net.input_key: x})
+    err = rel_l2(got, ref[net.output_layer])
+    print("   %s storage=%d rel_l2=%.3e" % (name, storage, err), flush=True)
+    assert np.array_equal(got, replay)
+    assert err <= (TOL[storage] if storage == fa.STORAGE_F32 else F16_END_TO_END)
+    if name == "config3":
+        idx, val = net.getArgMax(net.argmax_layer)
+        assert idx[0, 0] == int(np.argmax(got.ravel()))
+        if storage == fa.STORAGE_F32:
+            assert idx[0, 0] == int(ref[net.argmax_layer][0, 0, 0])
+    net.cleanup()
+
+
+@pytest.mark.parametrize("switch", ["FYNHIP_FORCE_PROJECTION_FUSION", "FYNHIP_AUTOTUNE"])
+def test_config3_resnet50_inference_setting_with_forced_choices(switch, monkeypatch):
+    """BASELINE's ResNet-50, buffers shared, (a) with every shortcut projection computed by the layer that adds it
+    whatever the timing says, (b) with every choice between kernel forms taken by rule instead of by timing: logits
+    within 1e-4 of the oracle's, the same class."""
+    monkeypatch.setenv(switch, "1" if switch != "FYNHIP_AUTOTUNE" else "0")
+    net = networks.ResNet50(fa.STORAGE_F32)
+    x, got, infos = _inference_output(net)
+    joined = [n for n, i in infos.items() if "no launch of its own" in i]
+    print("   layers without a launch of their own:", joined, flush=True)
+    if switch == "FYNHIP_FORCE_PROJECTION_FUSION":
+        assert len([n for n in joined if n.endswith("_proj")]) == 4
+    ref = O.run_network(net.describe(), {net.input_key: x})
+    err = rel_l2(got, ref[net.logits_layer])
+    print("   rel_l2=%.3e" % err, flush=True)
+    assert err <= 1e-4
+    idx, _ = net.getArgMax(net.argmax_layer)
+    assert idx[0, 0] == int(ref[net.argmax_layer][0, 0, 0])
+    net.cleanup()
+
+
 def test_config2_full_size_properties():
     """512x624 fp32: buffer sharing, HIP-graph replay and repetition must not change a single bit."""
     outs = []

@@ -9,7 +9,7 @@ import fyusenet_amd as fa
 from fyusenet_amd import networks, prng
 from fyusenet_amd.builders import ActType, UpDownLayerBuilder
 from oracle import oracle as O
-from util import rel_l2
+from util import combos, rel_l2
 
 pytestmark = pytest.mark.gpu
 TOL = {fa.STORAGE_F32: 1e-4, fa.STORAGE_F16: 2e-3}
@@ -20,9 +20,10 @@ class Bottleneck(networks._StreamNet):
     download: the first block of a ResNet stage (samples/samplenetworks/resnet50.cpp:260-275)."""
     config_id = 3
 
-    def __init__(self, storage, cin, mid, cout, h, w, stride, res_act=ActType.NONE, second_reader=False, res_bn=False):
+    def __init__(self, storage, cin, mid, cout, h, w, stride, res_act=ActType.NONE, second_reader=False, res_bn=False, scale_decades=0):
         super().__init__(storage)
         self.res_bn = res_bn
+        self.scale_decades = scale_decades
         self.cin, self.mid, self.cout, self.h, self.w, self.stride = cin, mid, cout, h, w, stride
         self.res_act, self.second_reader = res_act, second_reader
 
@@ -37,6 +38,10 @@ class Bottleneck(networks._StreamNet):
         self.conv(5, "expand", 1, self.mid, self.cout, ho, wo, 4, act=R, residual=2, res_act=self.res_act)
         if self.res_bn:   # the layer's batch-norm scale multiplies what it adds as well (ConvLayerBuilder::residual(act, true))
             self._builders[-1].residual(self.res_act, True)
+        if self.scale_decades:   # batch-norm scales of the projection and of the adding layer log-uniform over so many decades
+            for idx, (no, gen) in enumerate(self._blocks):
+                if no in (2, 5):
+                    self._blocks[idx] = (no, lambda g=gen, n=no: self._spread(g(), n))
         last = 5
         if self.second_reader:   # something else reads the projection's tensor
             self.conv(6, "side", 1, self.cout, 32, ho, wo, 2, act=R)
@@ -44,6 +49,11 @@ class Bottleneck(networks._StreamNet):
         self._add(UpDownLayerBuilder(UpDownLayerBuilder.DOWNLOAD, "download").number(last + 1).shape(self.cout, ho, wo, self.cout).deep())
         self._edges.append((5, last + 1, 0))
         self.output_layer = last + 1
+
+    def _spread(self, blk, no):
+        # (downwards from 1, so that fp16 tensors hold the results)
+        blk[-2 * self.cout:-self.cout] = (10.0 ** prng.uniform(8101 + no, (self.cout,), -float(self.scale_decades), 0.0)).astype(np.float32)
+        return blk
 
     def makeInput(self):
         return prng.uniform(1709 + self.cin + self.h, (self.cin, self.h, self.w), -1.0, 1.0)
@@ -76,13 +86,13 @@ CASES = [
 ]
 
 
-@pytest.mark.parametrize("storage", [fa.STORAGE_F32, fa.STORAGE_F16], ids=["f32", "f16"])
-@pytest.mark.parametrize("res_bn", [False, True], ids=["plain", "bn_on_residual"])
-@pytest.mark.parametrize("case", CASES, ids=lambda c: "%d_%d_%d_%dx%d_s%d" % c)
+@pytest.mark.parametrize(*combos(
+    # (the residual's batch-norm is varied on the smaller cases)
+    lambda case, res_bn, storage: not (res_bn and case[0] > 256),
+    case=(CASES, lambda c: "%d_%d_%d_%dx%d_s%d" % c), res_bn=([False, True], lambda r: "bn_on_residual" if r else "plain"),
+    storage=([fa.STORAGE_F32, fa.STORAGE_F16], lambda st: "f32" if st == fa.STORAGE_F32 else "f16")))
 def test_projection_inside_the_layer_that_adds_it(case, res_bn, storage, monkeypatch):
     cin, mid, cout, h, w, stride = case
-    if res_bn and cin > 256:
-        pytest.skip("the residual's batch-norm is varied on the smaller cases")
     monkeypatch.setenv("FYNHIP_FORCE_PROJECTION_FUSION", "1")
     net = Bottleneck(storage, cin, mid, cout, h, w, stride, res_bn=res_bn)
     x, got, infos = run(net)
@@ -118,3 +128,25 @@ def test_projection_keeps_its_launch_when_it_has_to(why, monkeypatch):
     assert "no launch of its own" not in infos["projection"] and "two tensors" not in infos["expand"]
     ref = O.run_network(desc, {net.input_key: x})[net.output_layer]
     assert rel_l2(got, ref) <= TOL[fa.STORAGE_F32]
+
+
+@pytest.mark.parametrize("storage", [fa.STORAGE_F32, fa.STORAGE_F16], ids=["f32", "f16"])
+@pytest.mark.parametrize("decades", [4, 8])
+def test_projection_with_scales_of_very_different_magnitude(decades, storage, monkeypatch):
+    """The one launch carries both layers' batch-norm scales on its weight rows, under one common power of two.  Scales
+    spread over four decades keep the bound; over eight decades (beyond the 2^16 between rows that the packing allows)
+    the pair runs as two launches, each layer's scale on its fp32 sum, and keeps it as well."""
+    monkeypatch.setenv("FYNHIP_FORCE_PROJECTION_FUSION", "1")
+    net = Bottleneck(storage, 64, 64, 256, 28, 28, 1, scale_decades=decades)
+    x, got, infos = run(net)
+    desc = net.describe()
+    net.cleanup()
+    print("  ", infos["projection"][:100], "|", infos["expand"][:120], flush=True)
+    if decades <= 4:
+        assert "launch of layer 5" in infos["projection"] and "over two tensors" in infos["expand"]
+    else:
+        assert "no launch of its own" not in infos["projection"] and "two tensors" not in infos["expand"]
+    ref = O.run_network(desc, {net.input_key: x})[net.output_layer]
+    err = rel_l2(got, ref)
+    print("   rel_l2=%.3e" % err, flush=True)
+    assert err <= TOL[storage]

@@ -163,11 +163,9 @@ def _builder(i, s, pad_out, specs=None, pads=None):
 
 
 @pytest.mark.parametrize("storage", [fa.STORAGE_F32, fa.STORAGE_F16], ids=["f32", "f16"])
-@pytest.mark.parametrize("seed", range(40))
+@pytest.mark.parametrize("seed", [sd for sd in range(40) if _random_chain(sd)[1]])   # (seeds whose chain has a layer)
 def test_random_chain(seed, storage):
     shape0, specs, last_pad = _random_chain(seed)
-    if not specs:
-        pytest.skip("empty chain")
     built = []
     pads = [specs[i + 1]["pad_in"] if i + 1 < len(specs) else last_pad for i in range(len(specs))]   # output padding per layer
     for i, s in enumerate(specs):

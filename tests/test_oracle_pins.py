@@ -213,6 +213,23 @@ def test_deep_tiling_and_layout_round_trips():
     assert np.array_equal(O.shallow_to_chw(O.chw_to_shallow(x[:3], 4), 3), x[:3])
 
 
+def test_shallow_layout_is_the_pixel_major_transposition():
+    # GPU_SHALLOW host buffers are pixel-major with 3 or 4 components per pixel (RGB triplets in, RGBA out:
+    # cpu/cpubuffer.cpp:121-158 walks them as src[(y*width + x)*packing + c]); channels beyond the tensor's read as zero.
+    for c, pc in ((3, 3), (3, 4), (4, 4), (1, 4), (2, 3)):
+        x = prng.uniform(19 + c + pc, (c, 5, 7), -1, 1)
+        hwc = O.chw_to_shallow(x, pc)
+        assert hwc.shape == (5, 7, pc)
+        assert np.array_equal(hwc[..., :c], x.transpose(1, 2, 0))
+        assert not hwc[..., c:].any()
+        back = O.shallow_to_chw(np.ascontiguousarray(hwc), c)
+        assert np.array_equal(back, x)
+        # a pixel-major array of our own making, read back channel by channel (a converter that walked rows or
+        # components in another order would return something else)
+        own = prng.uniform(31 + c + pc, (5, 7, pc), -1, 1)
+        assert np.array_equal(O.shallow_to_chw(own, c), own[..., :c].transpose(2, 0, 1))
+
+
 # ---- leaky ReLU, batch-norm layer with residual, GPU_DEEP layout ----------------------------------
 @pytest.mark.parametrize("leak", [0.1, 0.25, 1.5])
 def test_leaky_relu_on_fetch(leak):

@@ -1,6 +1,6 @@
 """fyn_layer_copy_result_noalloc (read-back through the library's fixed device array, no allocation) against
 fyn_layer_copy_result, bit for bit, through the C ABI: two calls in a row, the second on a smaller tensor, then the
-size limit."""
+size limit; and that a call leaves the GPU's free memory where it was."""
 import ctypes
 
 import numpy as np
@@ -62,4 +62,46 @@ def test_no_alloc_read_back_refuses_what_does_not_fit():
     # the allocating entry point still serves it
     capi.check(capi.lib().fyn_layer_copy_result(net._h, 1, capi.fptr(out), 0))
     assert out.any()
+    net.cleanup()
+
+
+def _allocations(net):
+    from fyusenet_amd import capi
+    calls, nbytes = ctypes.c_size_t(0), ctypes.c_size_t(0)
+    capi.check(capi.lib().fyn_net_device_allocations(net._h, ctypes.byref(calls), ctypes.byref(nbytes)))
+    return calls.value, nbytes.value
+
+
+def _free_device_bytes():
+    hip = ctypes.CDLL("libamdhip64.so")
+    free, total = ctypes.c_size_t(0), ctypes.c_size_t(0)
+    assert hip.hipMemGetInfo(ctypes.byref(free), ctypes.byref(total)) == 0
+    return free.value
+
+
+@pytest.mark.gpu
+def test_no_alloc_read_back_allocates_nothing():
+    """What the entry point exists for: on a network whose growable staging area has never been sized, reading back a
+    1.6 M-float tensor through it makes no device allocation (the engine's own count of its hipMalloc calls, and the
+    GPU's free memory as the runtime reports it), while the allocating entry point, called afterwards on the same
+    tensor, makes one of at least the tensor's size."""
+    from fyusenet_amd import capi, networks
+    net = networks.StyleNet(0, width=256, height=192)   # (the input, 3 channels, sizes the staging area for 147 K floats only)
+    net.setup(reuseBuffers=False)
+    net.setInput(net.makeInput())
+    net.forward()
+    net.finish()
+    out = np.zeros((32, 192, 256), np.float32)   # the first layer's result: 1.6 M floats
+    calls0, bytes0 = _allocations(net)
+    free0 = _free_device_bytes()
+    for _ in range(2):
+        capi.check(capi.lib().fyn_layer_copy_result_noalloc(net._h, 1, capi.fptr(out), 0))
+    assert _allocations(net) == (calls0, bytes0)
+    assert _free_device_bytes() == free0
+    assert out.any()
+    want = np.zeros_like(out)
+    capi.check(capi.lib().fyn_layer_copy_result(net._h, 1, capi.fptr(want), 0))
+    calls1, bytes1 = _allocations(net)
+    assert calls1 == calls0 + 1 and bytes1 - bytes0 >= out.nbytes   # (the count sees the staging area being sized)
+    assert np.array_equal(out, want)
     net.cleanup()

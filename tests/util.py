@@ -1,7 +1,22 @@
 """Shared helpers of the test-suite."""
+import itertools
+
 import numpy as np
+import pytest
 
 from fyusenet_amd import prng
+
+
+def combos(runs, **axes):
+    """Arguments for pytest.mark.parametrize: the combinations of the named axes that runs(**combination) accepts, so
+    that a test is generated only where it has something to run (instead of being generated and skipped).
+    axes: name=(values, id function)."""
+    names = list(axes)
+    out = []
+    for vals in itertools.product(*[axes[n][0] for n in names]):
+        if runs(**dict(zip(names, vals))):
+            out.append(pytest.param(*vals, id="-".join(axes[n][1](v) for n, v in zip(names, vals))))
+    return ",".join(names), out
 
 
 def rel_l2(a, b):
