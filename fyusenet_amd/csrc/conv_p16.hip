@@ -54,6 +54,11 @@ constexpr int PD = 6;         // depth of the weight-fragment ring (steps)
 constexpr bool HSTORE = FYN_P16_HALF != 0;   // fp16 tensors
 constexpr int NPL = HSTORE ? 1 : 2;          // staged planes (hi, lo)
 constexpr int NPASS = HSTORE ? 1 : 3;        // MFMAs per fragment pair (hi*hi, lo*hi, hi*lo)
+// fp32 tensors, weight planes per fragment (launch_conv_p16, launch_tconv_p16): fp16 hi, fp16 lo, and the fp8 operands of
+// the correction terms, [8 x fp8(hi / 32) | 8 x fp8(lo * 64)] per lane; a kernel reads plane 0 and one of the other two
+constexpr int NPLW = HSTORE ? 1 : 3;
+typedef int i32x8_t __attribute__((ext_vector_type(8)));
+typedef int i32x4_t __attribute__((ext_vector_type(4)));
 constexpr int ESZ = HSTORE ? 2 : 4;          // bytes per stored element
 typedef std::conditional<HSTORE, _Float16, float>::type store_t;
 // Output channel, inside a wave's 32, of accumulator element e of channel fragment fm in the lanes kq = lane / 16:
@@ -128,7 +133,74 @@ __device__ __forceinline__ void p16_stage(f32x4_t (&acc)[2][G::FN], half8_t (&a_
 #pragma unroll
             for (int j = 0; j < NW; j++)   // the weight fragments of a step, spread over its slots
                 if (i == ((j * NS) / NW + 1 < NS ? (j * NS) / NW + 1 : NS - 1))
-                    a_q[dprev][j % 2][j / 2] = *reinterpret_cast<const half8_t*>(w_ + ((j % 2) * NPL + j / 2) * 1024 + wlane);
+                    a_q[dprev][j % 2][j / 2] = *reinterpret_cast<const half8_t*>(w_ + ((j % 2) * NPLW + j / 2) * 1024 + wlane);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+}
+
+// The same stage with the two correction terms of the operand split (lo*hi and hi*lo, 2^-11 of the result) as fp8
+// matrix instructions, v_mfma_f32_16x16x128_f8f6f4: 128 products per lane row and instruction at twice the fp16 rate.
+// The second staged plane then holds, per pixel and eight channels, [8 x fp8(32 lo) | 8 x fp8(hi / 64)], the third
+// weight plane [8 x fp8(hi / 32) | 8 x fp8(64 lo)]: element by element the products are lo*hi and hi*lo with the scales
+// cancelling, so all passes add into one accumulator.  One instruction takes the sixteen bytes of two consecutive steps
+// (two taps) on either side; steps are paired along the whole tile (s = 9 * chunk + tap even with s + 1), which needs an
+// even number of chunks.  Per step: ten fp16 MFMAs (hi*hi), and in every second step ten fp8 ones in front of them --
+// 304 matrix-pipe cycles per fragment pair and chunk instead of 432.  The correction terms keep four significant bits
+// for operands down to 2^-14 of the largest a tensor holds, which needs the tensor's value range (range.h): the kernel
+// runs on inputs that carry a range word; measured against the fp64 oracle: rel-L2 1e-5 (three fp16 passes: 3e-7).
+// Registers: a0 = ring of the fp16 hi weights, a2 = ring of the fp8 weights in pairs of steps, b0 = fp16 hi fragments,
+// b1 = the fp8 fragments of a pair of steps.  The refills follow the uses in program order: a fragment's registers for
+// the next step after its own MFMAs, the ring slot of step s-1 (whose fp8 half this step's fp8 block may still read)
+// behind that block.
+template <class G, int PH>
+__device__ __forceinline__ void p16_stage_c8(f32x4_t (&acc)[2][G::FN], half8_t (&a0)[PD][2], i32x8_t (&a2)[PD / 2][2], half8_t (&b0)[G::FN],
+                                             i32x8_t (&b1)[G::FN], const int (&bbase)[2][G::FN], const unsigned char* lds,
+                                             const unsigned char*& wnext, const unsigned char* wbase, const unsigned char* wend, unsigned wstep,
+                                             unsigned wlane) {
+    constexpr int FN = G::FN;
+    static_assert(PD % 2 == 0 && (2 * NT) % PD == 0, "pairs of steps keep their ring slots over two stages");
+#pragma unroll
+    for (int t = 0; t < NT; t++) {
+        const int s = PH * NT + t, d = s % PD, dprev = (d + PD - 1) % PD;
+        const bool pair = (s & 1) != 0;                    // the second step of a pair: the fp8 block runs
+        const int nbuf = (t + 1 == NT) ? 1 - PH : PH, noff = G::tap_off((t + 1) % NT);
+        const unsigned char* w_ = wnext;
+        wnext += wstep;
+        if (wnext == wend) wnext = wbase;
+        if (pair) {
+#pragma unroll
+            for (int i = 0; i < 2 * FN; i++) {
+                const int fn = i / 2, fm = i % 2;
+                acc[fm][fn] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a2[d / 2][fm], b1[fn], acc[fm][fn], 0, 0, 0, 0, 0, 0);
+                if (t == NT - 1 && i == 0) lds_barrier();
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < 2 * FN; i++) {
+            const int fn = i / 2, fm = i % 2;
+            acc[fm][fn] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0[d][fm], b0[fn], acc[fm][fn], 0, 0, 0);
+            if (!pair && t == NT - 1 && i == 0) lds_barrier();
+            if (fm == 1) {   // the fragment's MFMAs of this step are issued: its operands of the next step
+                b0[fn] = *reinterpret_cast<const half8_t*>(lds + bbase[nbuf][fn] + noff);
+                const i32x4_t v = *reinterpret_cast<const i32x4_t*>(lds + bbase[nbuf][fn] + noff + G::PLANE);
+                if (((s + 1) & 1) == 0) { b1[fn][0] = v[0]; b1[fn][1] = v[1]; b1[fn][2] = v[2]; b1[fn][3] = v[3]; }
+                else { b1[fn][4] = v[0]; b1[fn][5] = v[1]; b1[fn][6] = v[2]; b1[fn][7] = v[3]; }
+            }
+            // the weights of step s + PD - 1 into the slot of step s - 1: four loads, spread over the step's slots
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                if ((j * 2 * FN) / 4 != i) continue;
+                const int wfm = j & 1;
+                if (j < 2) {
+                    a0[dprev][wfm] = *reinterpret_cast<const half8_t*>(w_ + (wfm * NPLW) * 1024 + wlane);
+                } else {
+                    const i32x4_t v = *reinterpret_cast<const i32x4_t*>(w_ + (wfm * NPLW + 2) * 1024 + wlane);
+                    if ((dprev & 1) == 0) { a2[dprev / 2][wfm][0] = v[0]; a2[dprev / 2][wfm][1] = v[1]; a2[dprev / 2][wfm][2] = v[2]; a2[dprev / 2][wfm][3] = v[3]; }
+                    else { a2[dprev / 2][wfm][4] = v[0]; a2[dprev / 2][wfm][5] = v[1]; a2[dprev / 2][wfm][6] = v[2]; a2[dprev / 2][wfm][7] = v[3]; }
+                }
+            }
             __builtin_amdgcn_sched_barrier(0);
         }
     }
@@ -138,7 +210,8 @@ __device__ __forceinline__ void p16_stage(f32x4_t (&acc)[2][G::FN], half8_t (&a_
 // loads, activation, hi/lo conversion, LDS writes -- one stage ahead of the MFMA waves, across tile boundaries; scale and
 // bias at the start and, during a tile's last chunk, its residual tile.  One barrier per stage, after the one that hands
 // over the first.
-template <class G>
+// (C8: the second plane in the fp8 form, see p16_stage_c8)
+template <class G, bool C8 = false>
 __device__ __forceinline__ void p16_stager(const ConvP16Params& p, unsigned char* lds, int stid, int cb, int group, int ntiles,
                                            int nchunks, unsigned range_bits) {
     constexpr int CPB = G::CPB;
@@ -213,7 +286,7 @@ __device__ __forceinline__ void p16_stager(const ConvP16Params& p, unsigned char
                     half8_t hi, lo;
                     split8<KIND>(r, g_off[SET][i] >= 0, p.act, in_scale, hi, lo);
                     *reinterpret_cast<half8_t*>(buf + l_off[i]) = hi;
-                    *reinterpret_cast<half8_t*>(buf + G::PLANE + l_off[i]) = lo;
+                    *reinterpret_cast<half8_t*>(buf + G::PLANE + l_off[i]) = C8 ? c8_plane(hi, lo) : lo;
                 }
             };
             if (act_kind_ == ACT_RELU) split_all(std::integral_constant<int, ACT_RELU>());
@@ -285,7 +358,8 @@ __device__ __forceinline__ void p16_stager(const ConvP16Params& p, unsigned char
 // group, group + pos_groups, ... (one tile each when the layer has no more tiles than the chip has CUs).  The staging
 // waves run one stage ahead of the MFMA waves, across tile boundaries, so that from the second tile on a tile's fetch
 // and the previous tile's stores overlap with MFMA work.
-template <int TH, int TW, int S, int WM>
+// C8 (fp32 tensors, an even number of chunks, an input with a range word): the correction terms as fp8 MFMAs (p16_stage_c8)
+template <int TH, int TW, int S, int WM, bool C8 = false>
 __global__ __launch_bounds__(512) void conv_p16_kernel(const ConvP16Params p) {
     using G = Geo<TH, TW, S, WM>;
     constexpr int FN = G::FN, CPB = G::CPB;
@@ -314,7 +388,7 @@ __global__ __launch_bounds__(512) void conv_p16_kernel(const ConvP16Params p) {
     constexpr int res_off = sb_off + 2 * CPB * 4;
 
     if (wave < 4) {   // the first four waves stage: they start first
-        p16_stager<G>(p, lds, tid & 255, cb, group, ntiles, nchunks, range_bits);
+        p16_stager<G, C8>(p, lds, tid & 255, cb, group, ntiles, nchunks, range_bits);
         return;
     }
 
@@ -332,17 +406,31 @@ __global__ __launch_bounds__(512) void conv_p16_kernel(const ConvP16Params p) {
         bbase[1][fn] = bbase[0][fn] + G::BUF;
     }
     // A fragments: [(chunk*9 + tap)][cout fragment of 16][plane][lane] x 8 halves
-    const unsigned wstep = (unsigned)p.mfrags * NPL * 1024;
-    const unsigned char* wbase = reinterpret_cast<const unsigned char*>(p.wpack) + (size_t)((cb * 2 * WM + mw * 2) * NPL) * 1024;   // (uniform: the loads take it as their scalar base)
+    const unsigned wstep = (unsigned)p.mfrags * NPLW * 1024;
+    const unsigned char* wbase = reinterpret_cast<const unsigned char*>(p.wpack) + (size_t)((cb * 2 * WM + mw * 2) * NPLW) * 1024;   // (uniform: the loads take it as their scalar base)
     const unsigned wlane = lane * 16;
     const unsigned char* wend = wbase + (size_t)nchunks * NT * wstep;
-    half8_t a_q[PD][2][NPL];
+    half8_t a_q[C8 ? 1 : PD][2][NPL];   // exact form: hi and lo weights of a step
+    half8_t a0[C8 ? PD : 1][2];         // fp8 form: hi weights of a step ...
+    i32x8_t a2[C8 ? PD / 2 : 1][2];     // ... and the fp8 weights of a pair of steps
+    if constexpr (C8) {
 #pragma unroll
-    for (int d = 0; d < PD; d++)
+        for (int d = 0; d < PD; d++)
 #pragma unroll
-        for (int fm = 0; fm < 2; fm++)
+            for (int fm = 0; fm < 2; fm++) {
+                a0[d][fm] = *reinterpret_cast<const half8_t*>(wbase + (size_t)d * wstep + (fm * NPLW) * 1024 + wlane);
+                const i32x4_t v = *reinterpret_cast<const i32x4_t*>(wbase + (size_t)d * wstep + (fm * NPLW + 2) * 1024 + wlane);
 #pragma unroll
-            for (int pl = 0; pl < NPL; pl++) a_q[d][fm][pl] = *reinterpret_cast<const half8_t*>(wbase + (size_t)d * wstep + (fm * NPL + pl) * 1024 + wlane);
+                for (int e = 0; e < 4; e++) a2[d / 2][fm][(d & 1) * 4 + e] = v[e];
+            }
+    } else {
+#pragma unroll
+        for (int d = 0; d < PD; d++)
+#pragma unroll
+            for (int fm = 0; fm < 2; fm++)
+#pragma unroll
+                for (int pl = 0; pl < NPL; pl++) a_q[d][fm][pl] = *reinterpret_cast<const half8_t*>(wbase + (size_t)d * wstep + (fm * NPLW + pl) * 1024 + wlane);
+    }
     f32x4_t acc[2][FN];
     auto zero_acc = [&]() {
 #pragma unroll
@@ -419,14 +507,44 @@ __global__ __launch_bounds__(512) void conv_p16_kernel(const ConvP16Params p) {
     FYN_PTRACE(1);
     lds_barrier();   // the first stage is staged
     FYN_PTRACE(2);
-    half8_t b[FN][NPL];
+    half8_t b[C8 ? 1 : FN][NPL];
+    half8_t b0[C8 ? FN : 1];
+    i32x8_t b1[C8 ? FN : 1];
+    if constexpr (C8) {
 #pragma unroll
-    for (int fn = 0; fn < FN; fn++)
+        for (int fn = 0; fn < FN; fn++) {
+            b0[fn] = *reinterpret_cast<const half8_t*>(lds + bbase[0][fn]);
+            const i32x4_t v = *reinterpret_cast<const i32x4_t*>(lds + bbase[0][fn] + G::PLANE);
 #pragma unroll
-        for (int pl = 0; pl < NPL; pl++) b[fn][pl] = *reinterpret_cast<const half8_t*>(lds + bbase[0][fn] + pl * G::PLANE);
+            for (int e = 0; e < 4; e++) { b1[fn][e] = v[e]; b1[fn][4 + e] = 0; }
+        }
+    } else {
+#pragma unroll
+        for (int fn = 0; fn < FN; fn++)
+#pragma unroll
+            for (int pl = 0; pl < NPL; pl++) b[fn][pl] = *reinterpret_cast<const half8_t*>(lds + bbase[0][fn] + pl * G::PLANE);
+    }
 
     const unsigned char* wnext = wbase + (size_t)((PD - 1) % (nchunks * NT)) * wstep;
     int tile = group, c = 0;
+    if constexpr (C8) {
+        // (an even number of chunks: a tile is whole pairs of stages)
+        for (;;) {
+            p16_stage_c8<G, 0>(acc, a0, a2, b0, b1, bbase, lds, wnext, wbase, wend, wstep, wlane);
+            FYN_PTRACE(3 + (c < 12 ? c : 12));
+            p16_stage_c8<G, 1>(acc, a0, a2, b0, b1, bbase, lds, wnext, wbase, wend, wstep, wlane);
+            FYN_PTRACE(4 + (c < 11 ? c : 11));
+            c += 2;
+            if (c == nchunks) {
+                FYN_PTRACE(29);
+                finish_tile(tile);
+                FYN_PTRACE(30);
+                c = 0; tile += p.pos_groups;
+                if (tile >= ntiles) break;
+                zero_acc();
+            }
+        }
+    } else {
     for (;;) {
         p16_stage<G, 0>(acc, a_q, b, bbase, lds, wnext, wbase, wend, wstep, wlane);
         FYN_PTRACE(3 + (c < 12 ? c : 12));
@@ -448,6 +566,7 @@ __global__ __launch_bounds__(512) void conv_p16_kernel(const ConvP16Params p) {
             if (tile >= ntiles) break;
             zero_acc();
         }
+    }
     }
     if (p.out_amax) range_publish_waves(p.out_amax, vmax, range_box, 4);
     FYN_PTRACE(31);
@@ -500,7 +619,7 @@ __device__ __forceinline__ void tp16_stage(f32x4_t (&acc)[4][2][G::FN], half8_t 
 #pragma unroll
             for (int j = 0; j < NW; j++)   // the weight fragments of a step, spread over its slots
                 if (i == ((j * NS) / NW + 1 < NS ? (j * NS) / NW + 1 : NS - 1))
-                    a_q[dprev][j % 2][j / 2] = *reinterpret_cast<const half8_t*>(w_ + ((j % 2) * NPL + j / 2) * 1024 + wlane);
+                    a_q[dprev][j % 2][j / 2] = *reinterpret_cast<const half8_t*>(w_ + ((j % 2) * NPLW + j / 2) * 1024 + wlane);
             __builtin_amdgcn_sched_barrier(0);
         }
     }
@@ -546,8 +665,8 @@ __global__ __launch_bounds__(512) void tconv_p16_kernel(const ConvP16Params p) {
         bbase[0][fn] = ty * G::ROW_PITCH + (wn * TW + tx) * PITCH + kq * 16;
         bbase[1][fn] = bbase[0][fn] + G::BUF;
     }
-    const unsigned wstep = (unsigned)p.mfrags * NPL * 1024;
-    const unsigned char* wbase = reinterpret_cast<const unsigned char*>(p.wpack) + (size_t)((cb * 2 * WM + mw * 2) * NPL) * 1024;   // (uniform: the loads take it as their scalar base)
+    const unsigned wstep = (unsigned)p.mfrags * NPLW * 1024;
+    const unsigned char* wbase = reinterpret_cast<const unsigned char*>(p.wpack) + (size_t)((cb * 2 * WM + mw * 2) * NPLW) * 1024;   // (uniform: the loads take it as their scalar base)
     const unsigned wlane = lane * 16;
     const unsigned char* wend = wbase + (size_t)nchunks * NT * wstep;
     half8_t a_q[PDT][2][NPL];
@@ -556,7 +675,7 @@ __global__ __launch_bounds__(512) void tconv_p16_kernel(const ConvP16Params p) {
 #pragma unroll
         for (int fm = 0; fm < 2; fm++)
 #pragma unroll
-            for (int pl = 0; pl < NPL; pl++) a_q[d][fm][pl] = *reinterpret_cast<const half8_t*>(wbase + (size_t)d * wstep + (fm * NPL + pl) * 1024 + wlane);
+            for (int pl = 0; pl < NPL; pl++) a_q[d][fm][pl] = *reinterpret_cast<const half8_t*>(wbase + (size_t)d * wstep + (fm * NPLW + pl) * 1024 + wlane);
     f32x4_t acc[4][2][FN];
     auto zero_acc = [&]() {
 #pragma unroll
@@ -1462,11 +1581,14 @@ struct P16Entry {
     int th, tw, stride, wm;
     p16_fn fn;
     size_t buf, res_bytes;   // one staging buffer; the residual tile
+    p16_fn fn_c8;            // fp32 tensors: the form with the correction terms as fp8 MFMAs
 };
 template <int TH, int TW, int S, int WM>
 constexpr P16Entry entry() {
     using G = Geo<TH, TW, S, WM>;
-    return P16Entry{TH, TW, S, WM, conv_p16_kernel<TH, TW, S, WM>, (size_t)G::BUF, (size_t)TH * G::TWG * G::RES_PITCH};
+    P16Entry e{TH, TW, S, WM, conv_p16_kernel<TH, TW, S, WM>, (size_t)G::BUF, (size_t)TH * G::TWG * G::RES_PITCH, nullptr};
+    if constexpr (!HSTORE) e.fn_c8 = conv_p16_kernel<TH, TW, S, WM, true>;
+    return e;
 }
 const P16Entry kEntries[] = {
     entry<8, 10, 1, 4>(), entry<10, 8, 1, 4>(), entry<8, 8, 1, 4>(), entry<8, 6, 1, 4>(), entry<4, 8, 1, 4>(), entry<4, 4, 1, 4>(),
@@ -1583,6 +1705,28 @@ bool conv_p16c4_supported(int k, int stride, int dil, int in_cp, int cout, int o
 }
 #endif
 
+#if !FYN_P16_HALF
+// Third weight plane of the 16-position forms on fp32 tensors: src holds, per fragment and lane, sixteen floats -- the
+// eight hi parts divided by 32, then the eight lo parts times 64 -- which become the sixteen fp8 values of the lane in
+// plane 2 of the fragment (three planes of 1 KB each).  Converted on the device, so that the format is the one the
+// matrix instruction reads.
+__global__ __launch_bounds__(256) void pack_fp8_plane_kernel(const float* __restrict__ src, unsigned char* __restrict__ wpack, size_t n4) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;   // four values each
+    if (i >= n4) return;
+    const float4 v = reinterpret_cast<const float4*>(src)[i];
+    int w = __builtin_amdgcn_cvt_pk_fp8_f32(v.x, v.y, 0, false);
+    w = __builtin_amdgcn_cvt_pk_fp8_f32(v.z, v.w, w, true);
+    const size_t lane16 = i >> 2, frag = lane16 >> 6;   // sixteen values per lane, 64 lanes per fragment
+    *reinterpret_cast<int*>(wpack + frag * 3072 + 2048 + (lane16 & 63) * 16 + (i & 3) * 4) = w;
+}
+int launch_pack_fp8_plane(const float* src, void* wpack, size_t frags, hipStream_t s) {
+    const size_t n4 = frags * 64 * 4;
+    if (n4 == 0) return 0;
+    hipLaunchKernelGGL(pack_fp8_plane_kernel, dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, s, src, static_cast<unsigned char*>(wpack), n4);
+    return hipGetLastError() == hipSuccess ? 0 : -3;
+}
+#endif
+
 static const KREntry* find_krentry(const ConvP16Params& p, int k) {
     if (p.dw_in) {
         for (const KREntry& c : kKRDwEntries)
@@ -1634,6 +1778,13 @@ int P16_NAME(launch_conv_kr16)(const ConvP16Params& p, int k, hipStream_t s) {
     return hipGetLastError() == hipSuccess ? 0 : -3;
 }
 
+// The correction terms run as fp8 MFMAs where the input carries a value-range word (fp32 tensors) and the chunks pair up;
+// FYNHIP_EXACT_SPLIT=1 keeps the three fp16 passes everywhere.
+static bool p16_uses_fp8(const ConvP16Params& p) {
+    static const bool exact = getenv("FYNHIP_EXACT_SPLIT") != nullptr;
+    return !HSTORE && !exact && p.in_amax != nullptr && p.cin_chunks % 2 == 0;
+}
+
 static const P16Entry* find_entry(const ConvP16Params& p) {
     for (const P16Entry& c : kEntries)
         if (c.th == p.tile_h && c.tw == p.tile_w && c.stride == p.stride && c.wm == p.wm) return &c;
@@ -1665,7 +1816,8 @@ int P16_NAME(launch_conv_p16)(const ConvP16Params& p, hipStream_t s) {
         return -5;
     const size_t lds_bytes = entry_lds(*e, p.res != nullptr);
     if (lds_bytes > 160 * 1024) return -2;
-    if (ensure_lds(reinterpret_cast<const void*>(e->fn), lds_bytes) != 0) return -2;
+    const p16_fn fn = p16_uses_fp8(p) ? e->fn_c8 : e->fn;
+    if (ensure_lds(reinterpret_cast<const void*>(fn), lds_bytes) != 0) return -2;
 #ifdef FYN_P16_TRACE
     {
         static long long* dev = nullptr;
@@ -1674,7 +1826,7 @@ int P16_NAME(launch_conv_p16)(const ConvP16Params& p, hipStream_t s) {
         ConvP16Params q = p;
         q.trace = dev;
         if (const char* e = getenv("FYNHIP_P16_CHUNKS")) q.cin_chunks = atoi(e);   // (timing study: fewer chunks, wrong results)
-        hipLaunchKernelGGL(e->fn, dim3(p.pos_groups * p.cout_blocks), dim3(512), lds_bytes, s, q);
+        hipLaunchKernelGGL(fn, dim3(p.pos_groups * p.cout_blocks), dim3(512), lds_bytes, s, q);
         hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
         (void)hipStreamIsCapturing(s, &cap);
         const char* path = cap == hipStreamCaptureStatusNone ? getenv("FYNHIP_TRACE_DUMP") : nullptr;
@@ -1687,7 +1839,7 @@ int P16_NAME(launch_conv_p16)(const ConvP16Params& p, hipStream_t s) {
         return hipGetLastError() == hipSuccess ? 0 : -3;
     }
 #endif
-    hipLaunchKernelGGL(e->fn, dim3(p.pos_groups * p.cout_blocks), dim3(512), lds_bytes, s, p);
+    hipLaunchKernelGGL(fn, dim3(p.pos_groups * p.cout_blocks), dim3(512), lds_bytes, s, p);
     return hipGetLastError() == hipSuccess ? 0 : -3;
 }
 

@@ -171,7 +171,7 @@ struct ConvP16Params {
     const void* in;
     void* out;
     const void* res;      // residual tensor or nullptr
-    const void* wpack;    // [(chunk*9 + ky*3 + kx)][cout fragment of 16][plane hi, lo][lane 0..63][8 halves]: output channel
+    const void* wpack;    // [(chunk*9 + ky*3 + kx)][cout fragment of 16][plane hi, lo (launch_conv_p16, launch_tconv_p16 on fp32 tensors: a third, see launch_pack_fp8_plane)][lane 0..63][8 halves]: output channel
                           // 16*fragment + lane%16, input channel 32*chunk + 8*(lane/16) + j; 6 steps of zeros behind the last
     const float* scale;   // [cout_blocks*32*wm]
     const float* bias;    // [cout_blocks*32*wm]
@@ -229,6 +229,9 @@ bool conv_p16_supported(int k, int stride, int dil, int in_cp, int cout, int out
 int conv_p16_tile_count();
 void conv_p16_tile(int index, int* th, int* tw, int* stride, int* wm);
 size_t conv_p16_lds_bytes(const ConvP16Params& p);   // 0: no such compiled combination
+// fp32 tensors: wpack of launch_conv_p16 / launch_tconv_p16 has three planes per fragment (fp16 hi, fp16 lo, and
+// [8 x fp8(hi / 32) | 8 x fp8(64 lo)] per lane); this fills the third from src = [fragment][lane][those sixteen floats]
+int launch_pack_fp8_plane(const float* src, void* wpack, size_t frags, hipStream_t s);
 int launch_conv_p16(const ConvP16Params& p, hipStream_t s);
 // the transposed 3x3 convolution that doubles the image size, on the same parameters: positions (npos_y x npos_x,
 // tiles) are input pixels, out_off_* the stored coordinate of output pixel (0, 0), wpack holds the nine taps of a chunk

@@ -759,6 +759,27 @@ static float weight_prescale(const float* w, size_t n) {
     return std::ldexp(1.f, 12 - e);
 }
 
+// The planes behind the first of a packed fragment of the 16-position forms on fp32 tensors (three planes of 64 lanes x 8
+// halves): plane 1 takes the fp16 lo part of weight j of a lane; c8 takes the sources of plane 2, the fp8 operands of
+// the correction terms: hi / 32 in its first eight places, lo * 64 in the other eight (the staged activations carry the
+// inverse factors, conv_p16.hip).
+static void p16_lo_planes(uint16_t* frag_base, float* c8_lane, int lane, int j, float v, uint16_t hi) {
+    const float lo = v - h2f(hi);
+    frag_base[(size_t)(64 + lane) * 8 + j] = f2h_bits(lo);
+    c8_lane[j] = h2f(hi) * (1.0f / 32.0f);
+    c8_lane[8 + j] = lo * 64.0f;
+}
+static void upload_p16_pack(Net* net, void* dev, const std::vector<uint16_t>& pack, const std::vector<float>& c8, size_t frags) {
+    FYN_HIP(hipStreamSynchronize(net->stream));
+    FYN_HIP(hipMemcpyAsync(dev, pack.data(), pack.size() * 2, hipMemcpyHostToDevice, net->stream));
+    if (!c8.empty()) {
+        float* src = upload(net, c8);
+        if (launch_pack_fp8_plane(src, dev, frags, net->stream) != 0) fail(FYN_ERR_DEVICE, "packing the fp8 weight plane failed");
+        net->dev_free(src);   // (waits for the stream)
+    }
+    FYN_HIP(hipStreamSynchronize(net->stream));
+}
+
 static std::string mfma_info(const MfmaLaunch& L) {
     char buf[256];
     snprintf(buf, sizeof(buf), "conv_mfma %s tile=%dx%d(cout x pos) waves=%dx%d kc=%d th=%d tw=%d blocks=%d lds=%zu steps=%d chunks=%d ksplit=%d",
@@ -896,6 +917,7 @@ class ConvLayer : public Layer {
         q.scale = scale_dev; q.bias = bias_dev;
         q.acc_mul = 1.f;
         q.act = act();
+        q.in_amax = tin(0).amax;   // (the candidates are timed in the form the frame will run: fp8 correction terms where the input has a range word)
         int want_h = 0, want_w = 0, want_wm = 0;   // FYNHIP_P16_TILE=h,w[,wm] (tests): that combination
         if (const char* e = getenv("FYNHIP_P16_TILE")) sscanf(e, "%d,%d,%d", &want_h, &want_w, &want_wm);
         struct Cand { double cost; ConvP16Params q; };
@@ -923,7 +945,7 @@ class ConvLayer : public Layer {
         if (cands.empty()) return;
         std::sort(cands.begin(), cands.end(), [](const Cand& a, const Cand& b) { return a.cost < b.cost; });
         if (cands.size() > 3) cands.resize(3);
-        const size_t halves = ((size_t)q.cin_chunks * 9 + 8) * q.mfrags * (q.f16 ? 1 : 2) * 64 * 8;
+        const size_t halves = ((size_t)q.cin_chunks * 9 + 8) * q.mfrags * (q.f16 ? 1 : 3) * 64 * 8;
         p16_wpack_dev = net->dev_alloc(halves * 2, true);
         for (Cand& c : cands) c.q.wpack = p16_wpack_dev;
         const bool always = getenv("FYNHIP_FORCE_P16_CONV") != nullptr;
@@ -1480,12 +1502,15 @@ class ConvLayer : public Layer {
     // weights of that form: [(chunk*9 + tap)][cout fragment of 16][plane][lane][8 halves], zero steps behind the last
     void pack_p16(const float* w, float wmul) {
         const int cin = d.in_channels;
-        const int npl = pp.f16 ? 1 : 2;
-        std::vector<uint16_t> pack(((size_t)pp.cin_chunks * 9 + 8) * pp.mfrags * npl * 64 * 8, 0);
+        const int npl = pp.f16 ? 1 : 3;   // fp32 tensors: hi, lo, and the fp8 operands of the correction terms
+        const size_t frags = ((size_t)pp.cin_chunks * 9 + 8) * pp.mfrags;
+        std::vector<uint16_t> pack(frags * npl * 64 * 8, 0);
+        std::vector<float> c8(npl == 3 ? frags * 64 * 16 : 0, 0.f);
         for (int chunk = 0; chunk < pp.cin_chunks; chunk++)
             for (int tap = 0; tap < 9; tap++)
                 for (int mf = 0; mf < pp.mfrags; mf++) {
-                    uint16_t* base = pack.data() + (((size_t)(chunk * 9 + tap) * pp.mfrags + mf) * npl) * 64 * 8;
+                    const size_t frag = (size_t)(chunk * 9 + tap) * pp.mfrags + mf;
+                    uint16_t* base = pack.data() + frag * npl * 64 * 8;
                     for (int lane = 0; lane < 64; lane++) {
                         const int o = p16_row_channel(mf, lane & 15, pp.f16 ? 2 : 1);
                         if (o >= oc) continue;
@@ -1495,13 +1520,11 @@ class ConvLayer : public Layer {
                             const float v = w[(((size_t)o * 3 + tap / 3) * 3 + tap % 3) * cin + ci] * wmul;
                             const uint16_t hi = f2h_bits(v);
                             base[(size_t)lane * 8 + j] = hi;
-                            if (npl == 2) base[(size_t)(64 + lane) * 8 + j] = f2h_bits(v - h2f(hi));
+                            if (npl == 3) p16_lo_planes(base, c8.data() + (frag * 64 + lane) * 16, lane, j, v, hi);
                         }
                     }
                 }
-        FYN_HIP(hipStreamSynchronize(net->stream));
-        FYN_HIP(hipMemcpyAsync(p16_wpack_dev, pack.data(), pack.size() * 2, hipMemcpyHostToDevice, net->stream));
-        FYN_HIP(hipStreamSynchronize(net->stream));
+        upload_p16_pack(net, p16_wpack_dev, pack, c8, frags);
     }
     void setup_rows_wide(const TView& in_v, const TView& out_v, const TView* res_v, int res_relu, int res_scale) {
         const int r = (k - 1) / 2;
@@ -2520,6 +2543,7 @@ class TransConvLayer : public Layer {
         q.scale = scale_dev; q.bias = bias_dev;
         q.acc_mul = 1.f;
         q.act = act();
+        q.in_amax = tin(0).amax;   // (timed in the form the frame will run)
         int want_h = 0, want_w = 0, want_wm = 0;   // FYNHIP_P16_TILE=h,w[,wm] (tests): that combination
         if (const char* e = getenv("FYNHIP_P16_TILE")) sscanf(e, "%d,%d,%d", &want_h, &want_w, &want_wm);
         std::vector<ConvP16Params> cands;
@@ -2540,7 +2564,7 @@ class TransConvLayer : public Layer {
             cands.push_back(c);
         }
         if (cands.empty()) return;
-        const size_t halves = ((size_t)q.cin_chunks * 9 + 8) * q.mfrags * (q.f16 ? 1 : 2) * 64 * 8;
+        const size_t halves = ((size_t)q.cin_chunks * 9 + 8) * q.mfrags * (q.f16 ? 1 : 3) * 64 * 8;
         p16_wpack_dev = net->dev_alloc(halves * 2, true);
         for (ConvP16Params& c : cands) c.wpack = p16_wpack_dev;
         const bool always = getenv("FYNHIP_FORCE_P16_CONV") != nullptr;
@@ -2584,14 +2608,17 @@ class TransConvLayer : public Layer {
     // weights of that form: [(chunk*9 + step)][cout fragment of 16][plane][lane][8 halves], steps in the kernel's tap order
     void pack_p16(const float* w, float wmul) {
         const int cin = d.in_channels;
-        const int npl = pp.f16 ? 1 : 2;
-        std::vector<uint16_t> pack(((size_t)pp.cin_chunks * 9 + 8) * pp.mfrags * npl * 64 * 8, 0);
+        const int npl = pp.f16 ? 1 : 3;   // fp32 tensors: hi, lo, and the fp8 operands of the correction terms
+        const size_t frags = ((size_t)pp.cin_chunks * 9 + 8) * pp.mfrags;
+        std::vector<uint16_t> pack(frags * npl * 64 * 8, 0);
+        std::vector<float> c8(npl == 3 ? frags * 64 * 16 : 0, 0.f);
         for (int chunk = 0; chunk < pp.cin_chunks; chunk++)
             for (int t = 0; t < 9; t++) {
                 int ky, kx;
                 tconv_p16_tap(t, &ky, &kx);
                 for (int mf = 0; mf < pp.mfrags; mf++) {
-                    uint16_t* base = pack.data() + (((size_t)(chunk * 9 + t) * pp.mfrags + mf) * npl) * 64 * 8;
+                    const size_t frag = (size_t)(chunk * 9 + t) * pp.mfrags + mf;
+                    uint16_t* base = pack.data() + frag * npl * 64 * 8;
                     for (int lane = 0; lane < 64; lane++) {
                         const int o = p16_row_channel(mf, lane & 15, pp.f16 ? 2 : 1);
                         if (o >= oc) continue;
@@ -2601,14 +2628,12 @@ class TransConvLayer : public Layer {
                             const float v = w[(((size_t)o * 3 + ky) * 3 + kx) * cin + ci] * wmul;
                             const uint16_t hi = f2h_bits(v);
                             base[(size_t)lane * 8 + j] = hi;
-                            if (npl == 2) base[(size_t)(64 + lane) * 8 + j] = f2h_bits(v - h2f(hi));
+                            if (npl == 3) p16_lo_planes(base, c8.data() + (frag * 64 + lane) * 16, lane, j, v, hi);
                         }
                     }
                 }
             }
-        FYN_HIP(hipStreamSynchronize(net->stream));
-        FYN_HIP(hipMemcpyAsync(p16_wpack_dev, pack.data(), pack.size() * 2, hipMemcpyHostToDevice, net->stream));
-        FYN_HIP(hipStreamSynchronize(net->stream));
+        upload_p16_pack(net, p16_wpack_dev, pack, c8, frags);
     }
     // value ranges (range.h): every parity reads the input's word and raises the output's; the first one clears
     bool tracks_range() const override { return true; }

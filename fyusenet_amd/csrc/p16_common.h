@@ -63,6 +63,24 @@ __device__ __forceinline__ void split8(const float (&r)[8], bool ok, const Act& 
     lo = __builtin_bit_cast(half8_t, L);
 }
 
+// The second staged plane of the fp8 form of the correction terms, from the split halves of eight values:
+// [8 x fp8(32 lo) | 8 x fp8(hi / 64)] (e4m3, round to nearest even).  With hi below 2^14 and lo below 2^3 (the value
+// range's scale) both stay inside fp8's range, and values down to 2^-14 of the largest keep their four bits.
+__device__ __forceinline__ half8_t c8_plane(const half8_t& hi, const half8_t& lo) {
+    typedef unsigned u32x4_t __attribute__((ext_vector_type(4)));
+    u32x4_t w;
+#pragma unroll
+    for (int q = 0; q < 2; q++) {
+        int v = __builtin_amdgcn_cvt_pk_fp8_f32((float)lo[4 * q] * 32.f, (float)lo[4 * q + 1] * 32.f, 0, false);
+        v = __builtin_amdgcn_cvt_pk_fp8_f32((float)lo[4 * q + 2] * 32.f, (float)lo[4 * q + 3] * 32.f, v, true);
+        w[q] = (unsigned)v;
+        int u = __builtin_amdgcn_cvt_pk_fp8_f32((float)hi[4 * q] * 0.015625f, (float)hi[4 * q + 1] * 0.015625f, 0, false);
+        u = __builtin_amdgcn_cvt_pk_fp8_f32((float)hi[4 * q + 2] * 0.015625f, (float)hi[4 * q + 3] * 0.015625f, u, true);
+        w[2 + q] = (unsigned)u;
+    }
+    return __builtin_bit_cast(half8_t, w);
+}
+
 constexpr int KC = 32;        // input channels per chunk
 constexpr int PITCH = KC * 2 + 16;   // bytes per staged pixel and plane: 8 neighbouring lanes' 16-byte reads cover all banks
 
