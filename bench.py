@@ -226,7 +226,7 @@ def launches_of(info):
     if "runs inside the launch of layer" in info:   # (a depthwise layer that a neighbouring 1x1 layer's launch computes)
         return 0
     n = 1
-    if "+shift_reduce" in info:
+    if "+shift_reduce" in info or "then a second launch" in info:
         n += 1
     if "ksplit=" in info and int(info.split("ksplit=")[1].split()[0]) > 1:
         n += 1

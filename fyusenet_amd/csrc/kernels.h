@@ -312,7 +312,9 @@ struct PoolParams {
     Act act;
 };
 void launch_pool(const PoolParams& p, hipStream_t s);
-void launch_global_pool(const TView& in, const TView& out, int is_max, const Act& act, hipStream_t s);
+// partial / splits: for large images, splits x in.cp floats of scratch memory; the pixels are then dealt to `splits`
+// workgroups per run of channel groups and a second launch pools their results (null / 1: one launch)
+void launch_global_pool(const TView& in, const TView& out, int is_max, const Act& act, hipStream_t s, float* partial = nullptr, int splits = 1);
 
 struct BnParams {
     TView in, out, res;

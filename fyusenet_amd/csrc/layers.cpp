@@ -2803,12 +2803,23 @@ class PoolLayer : public Layer {
         //   max: window begins input_padding before the stride origin (deepmaxpool.frag:15-45) -> 0
         //   avg: P=3 window [-1,1], otherwise [0,P) from the origin (deepavgpool.frag:17-44)
         p.off = is_max ? 0 : p.in.pad + (pool == 3 ? -1 : 0);
+        // a large image is pooled by many workgroups per run of channel groups (about 2048 pixels each) and a second launch
+        const long long npix = (long long)p.in.h * p.in.w;
+        if (global && npix >= 16384) {
+            splits = (int)std::min<long long>(1024, (npix + 2047) / 2048);
+            partial_dev = static_cast<float*>(net->dev_alloc((size_t)splits * p.in.cp * sizeof(float)));
+        }
     }
     void forward(hipStream_t s) override {
-        if (global) launch_global_pool(tin(0).v, tout().v, is_max, act(), s);
+        if (global) launch_global_pool(tin(0).v, tout().v, is_max, act(), s, partial_dev, splits);
         else launch_pool(p, s);
     }
-    std::string info() const override { return global ? "global_pool" : "pool"; }
+    std::string info() const override {
+        if (!global) return "pool";
+        return splits > 1 ? "global_pool (pixels dealt to " + std::to_string(splits) + " workgroups per run of channel groups, then a second launch)" : "global_pool";
+    }
+    int splits = 1;
+    float* partial_dev = nullptr;
     bool is_max, global;
     int pool = 1, stride = 1;
     PoolParams p{};

@@ -493,9 +493,12 @@ void launch_pool(const PoolParams& p, hipStream_t s) {
 //                  shaders/deep/deepglobavgpool.frag:15-24).  One block per run of up to 64
 // channel groups; the block's threads split the pixels, partial results meet in LDS.
 // ---------------------------------------------------------------------------------------------
-template <typename T>
+// Large images: the pixels are dealt to gridDim.y workgroups per run of channel groups, each of which leaves its
+// sum (maximum) in row blockIdx.y of a small fp32 tensor (`out`, `mul` = 1), and a second launch of the same kernel
+// pools that tensor (`mul` = 1 / pixels of the image).  TOut: the element type of `out`.
+template <typename T, typename TOut>
 __global__ __launch_bounds__(256) void global_pool_kernel(const TView in, const TView out, int is_max, const Act act,
-                                                          int cgb_log2) {
+                                                          int cgb_log2, float mul) {
     __shared__ float4 red[256];
     const int cgs = in.cp >> 2;
     const int cgb = 1 << cgb_log2;             // channel groups handled by this block
@@ -503,23 +506,35 @@ __global__ __launch_bounds__(256) void global_pool_kernel(const TView in, const 
     const int lg = threadIdx.x & (cgb - 1);
     const int part = threadIdx.x >> cgb_log2;
     const int g = blockIdx.x * cgb + lg;
-    const int npix = in.h * in.w;
+    const int total = in.h * in.w;
+    const int share = (total + gridDim.y - 1) / gridDim.y;
+    const int pbeg = blockIdx.y * share;
+    const int npix = min(total, pbeg + share);   // (end of this workgroup's pixels)
     const T* src = reinterpret_cast<const T*>(in.ptr);
     float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
     bool first = true;
     if (g < cgs) {
-        // four pixels per trip: their loads are issued together, then folded in pixel order
-        for (int pix0 = part; pix0 < npix; pix0 += 4 * parts) {
-            float4 v4[4];
+        // eight pixels per trip: their loads are issued together, then folded in pixel order (a tensor without a halo
+        // is one run of pixels: no row arithmetic)
+        constexpr int NJ = 8;
+        const bool flat = in.pad == 0;
+        for (int pix0 = pbeg + part; pix0 < npix; pix0 += NJ * parts) {
+            float4 v4[NJ];
 #pragma unroll
-            for (int j = 0; j < 4; j++) {
+            for (int j = 0; j < NJ; j++) {
                 const int pix = pix0 + j * parts;
                 const int pc = pix < npix ? pix : pix0;
-                const int y = pc / in.w, x = pc - y * in.w;
-                v4[j] = ld4<T>(src + tv_off(in, y, x) + g * 4);
+                size_t off;
+                if (flat) {
+                    off = (size_t)pc * in.cp;
+                } else {
+                    const int y = pc / in.w, x = pc - y * in.w;
+                    off = tv_off(in, y, x);
+                }
+                v4[j] = ld4<T>(src + off + g * 4);
             }
 #pragma unroll
-            for (int j = 0; j < 4; j++) {
+            for (int j = 0; j < NJ; j++) {
                 if (pix0 + j * parts >= npix) break;
                 const float4 v = act4(v4[j], act);
                 if (is_max) {
@@ -544,20 +559,32 @@ __global__ __launch_bounds__(256) void global_pool_kernel(const TView in, const 
     }
     if (part == 0 && g < cgs) {
         float4 r = red[threadIdx.x];
-        if (!is_max) {
-            const float inv = 1.0f / (float)npix;
-            r = make_float4(r.x * inv, r.y * inv, r.z * inv, r.w * inv);
-        }
-        st4<T>(reinterpret_cast<T*>(out.ptr) + tv_off(out, 0, 0) + g * 4, r);
+        if (!is_max) r = make_float4(r.x * mul, r.y * mul, r.z * mul, r.w * mul);
+        st4<TOut>(reinterpret_cast<TOut*>(out.ptr) + tv_off(out, 0, blockIdx.y) + g * 4, r);
     }
 }
-void launch_global_pool(const TView& in, const TView& out, int is_max, const Act& act, hipStream_t s) {
+// splits > 1: `partial` holds splits x in.cp floats (the pixels are dealt to that many workgroups per run of channel groups)
+void launch_global_pool(const TView& in, const TView& out, int is_max, const Act& act, hipStream_t s, float* partial, int splits) {
     const int cgs = in.cp >> 2;
     // few channel groups per workgroup: more workgroups, and more threads sharing the pixels of a group
     int l2 = 0;
     while ((1 << l2) < cgs && l2 < 4) l2++;
     const int cgb = 1 << l2;
-    FYN_DISPATCH_T(in.f16, global_pool_kernel, dim3((cgs + cgb - 1) / cgb), dim3(256), s, in, out, is_max, act, l2);
+    const dim3 grid((cgs + cgb - 1) / cgb);
+    const float inv = 1.0f / (float)(in.h * in.w);
+    if (partial && splits > 1) {
+        TView pv{};
+        pv.ptr = partial; pv.h = 1; pv.w = splits; pv.pad = 0; pv.c = in.c; pv.cp = in.cp; pv.f16 = 0;
+        Act none{};
+        none.kind = ACT_NONE;
+        if (in.f16) hipLaunchKernelGGL((global_pool_kernel<_Float16, float>), dim3(grid.x, splits), dim3(256), 0, s, in, pv, is_max, act, l2, 1.0f);
+        else hipLaunchKernelGGL((global_pool_kernel<float, float>), dim3(grid.x, splits), dim3(256), 0, s, in, pv, is_max, act, l2, 1.0f);
+        if (out.f16) hipLaunchKernelGGL((global_pool_kernel<float, _Float16>), grid, dim3(256), 0, s, pv, out, is_max, none, l2, inv);
+        else hipLaunchKernelGGL((global_pool_kernel<float, float>), grid, dim3(256), 0, s, pv, out, is_max, none, l2, inv);
+        return;
+    }
+    if (in.f16) hipLaunchKernelGGL((global_pool_kernel<_Float16, _Float16>), grid, dim3(256), 0, s, in, out, is_max, act, l2, inv);
+    else hipLaunchKernelGGL((global_pool_kernel<float, float>), grid, dim3(256), 0, s, in, out, is_max, act, l2, inv);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -712,7 +739,60 @@ __global__ __launch_bounds__(256) void func_kernel(const FuncParams p) {
     }
     stv<T, V>(reinterpret_cast<T*>(p.out.ptr) + tv_off(p.out, y, x) + c, v);
 }
+// Scaling up by two (nearest): a thread owns a block of 2 x 2 output pixels and V channels.  The four source texels
+// come from the same rule as above; where they coincide -- everywhere but at most at the frame's edges, by the
+// offsets -- the texel is fetched and converted once and stored four times, instead of four threads fetching it.
+template <typename T, int V>
+__global__ __launch_bounds__(256) void func_up2_kernel(const FuncParams p) {
+    const int cg = p.out.cp / V;
+    const int bw = (p.out.w + 1) >> 1, bh = (p.out.h + 1) >> 1;
+    const size_t n = (size_t)bh * bw * cg;
+    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= n) return;
+    const int g = (int)(idx % cg);
+    const size_t blk = idx / cg;
+    const int x0 = 2 * (int)(blk % bw), y0 = 2 * (int)(blk / bw);
+    const int c = g * V;
+    int sy[2], sx[2];
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        sy[i] = floordiv_pos((2 * (y0 + i) + 1) * p.dy - p.oy, 2 * p.uy);
+        sx[i] = floordiv_pos((2 * (x0 + i) + 1) * p.dx - p.ox, 2 * p.ux);
+    }
+    FV<V> v[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            if (i == 1 && sy[1] == sy[0]) { v[1][j] = v[0][j]; continue; }
+            if (j == 1 && sx[1] == sx[0]) { v[i][1] = v[i][0]; continue; }
+            FV<V> t = zerov<V>();
+            if (c < p.in.cp) t = fetch_clamped_v<T, V>(p.in, sy[i] + p.in.pad, sx[j] + p.in.pad, c);
+            t = actv<V>(t, p.act);
+            if (p.fn != FFN_COPY) {
+#pragma unroll
+                for (int e = 0; e < V; e++) t.v[e] = func1(t.v[e], p.fn, p.op, p.operand);
+            }
+            if (c + V > p.out.c) {
+#pragma unroll
+                for (int e = 0; e < V; e++)
+                    if (c + e >= p.out.c) t.v[e] = 0.f;
+            }
+            v[i][j] = t;
+        }
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+            if (y0 + i < p.out.h && x0 + j < p.out.w) stv<T, V>(reinterpret_cast<T*>(p.out.ptr) + tv_off(p.out, y0 + i, x0 + j) + c, v[i][j]);
+}
 void launch_func(const FuncParams& p, hipStream_t s) {
+    if (p.map == FMAP_SCALE && p.ux == 2 && p.uy == 2 && p.dx == 1 && p.dy == 1 && p.fn != FFN_BGR) {
+        const bool wide2 = (p.in.cp % 8 == 0) && (p.out.cp % 8 == 0);
+        const size_t n2 = (size_t)((p.out.h + 1) / 2) * ((p.out.w + 1) / 2) * (p.out.cp / ((p.out.f16 && wide2) ? 8 : 4));
+        FYN_DISPATCH_TV(p.out.f16, wide2, func_up2_kernel, grid1d(n2, 256), dim3(256), s, p);
+        return;
+    }
     const bool wide = p.map != FMAP_IMGEXTRACT && (p.in.cp % 8 == 0) && (p.out.cp % 8 == 0);
     const size_t n = (size_t)p.out.h * p.out.w * (p.out.cp / ((p.out.f16 && wide) ? 8 : 4));
     FYN_DISPATCH_TV(p.out.f16, wide, func_kernel, grid1d(n, 256), dim3(256), s, p);
@@ -856,67 +936,122 @@ void launch_concat_part(const TView& in, const TView& out, int c_off, const Act&
 // DeepArgMaxLayer::forward, gpu/deep/deepargmaxlayer.cpp:113-152).  L lanes cooperate on one pixel and
 // merge with cross-lane shuffles (DPP / ds_swizzle on gfx950).
 // ---------------------------------------------------------------------------------------------
-template <typename T>
+// One (value, index) pair per lane; the better of two: larger value, lower index among equals.
+__device__ __forceinline__ void argmax_merge(float& best, int& bidx, float ob, int oi) {
+    if (ob > best || (ob == best && oi < bidx)) {
+        best = ob;
+        bidx = oi;
+    }
+}
+// The pair of the lane that the data-parallel path CTRL pairs this lane with (quad permutations and the mirrors of a row
+// of 16 lanes: after xor 1, xor 2, half-row mirror and row mirror every lane of a row holds the row's result).
+template <int CTRL>
+__device__ __forceinline__ void argmax_dpp_step(float& best, int& bidx) {
+    const float ob = __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(best), CTRL, 0xf, 0xf, false));
+    const int oi = __builtin_amdgcn_update_dpp(0, bidx, CTRL, 0xf, 0xf, false);
+    argmax_merge(best, bidx, ob, oi);
+}
+// V channels per load (16 bytes of an fp16 tensor, 4 channels otherwise), L = 2^l_log2 lanes per pixel, R pixels per
+// lane group with all their loads in flight before the first comparison.
+template <typename T, int V, int R>
 __global__ __launch_bounds__(256) void argmax_kernel(const TView in, const TView out, int32_t* idx_out, const Act act,
                                                      int l_log2) {
     const int L = 1 << l_log2;
     const int lane = threadIdx.x & 63;
     const int sub = lane & (L - 1);
-    const int ppw = 64 >> l_log2;  // pixels per wave
+    const int ppw = 64 >> l_log2;  // lane groups per wave
     const size_t wave = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-    const size_t pix = wave * ppw + (lane >> l_log2);
+    const size_t pix0 = (wave * ppw + (lane >> l_log2)) * R;
     const size_t npix = (size_t)in.h * in.w;
-    const bool valid = pix < npix;
-    const int x = valid ? (int)(pix % in.w) : 0, y = valid ? (int)(pix / in.w) : 0;
-    const T* src = reinterpret_cast<const T*>(in.ptr) + tv_off(in, y, x);
-    float best = -INFINITY;
-    int bidx = 0x7fffffff;
-    const int cgs = (in.c + 3) >> 2;
-    if (valid) {
-        // four channel groups per trip: loads first, then the scan in channel order
-        for (int g0 = sub; g0 < cgs; g0 += 4 * L) {
-            float4 v4[4];
+    const int cgs = (in.c + V - 1) / V;   // (channels beyond in.c inside the last group are masked below; the pitch covers them)
+    const T* src[R];
+    bool valid[R];
+    float best[R];
+    int bidx[R];
 #pragma unroll
-            for (int j = 0; j < 4; j++) v4[j] = ld4<T>(src + (g0 + j * L < cgs ? g0 + j * L : g0) * 4);
+    for (int r = 0; r < R; r++) {
+        valid[r] = pix0 + r < npix;
+        const size_t pix = valid[r] ? pix0 + r : 0;
+        // (a tensor without a halo is one run of pixels: no row arithmetic)
+        src[r] = reinterpret_cast<const T*>(in.ptr) + (in.pad == 0 ? pix * in.cp : tv_off(in, (int)(pix / in.w), (int)(pix % in.w)));
+        best[r] = -INFINITY;
+        bidx[r] = 0x7fffffff;
+    }
+    for (int g0 = sub; g0 < cgs; g0 += 2 * L) {   // two groups of every pixel per trip: loads first, then the scan in channel order
+        FV<V> v[R][2];
 #pragma unroll
-            for (int j = 0; j < 4; j++) {
+        for (int r = 0; r < R; r++)
+#pragma unroll
+            for (int j = 0; j < 2; j++) v[r][j] = ldv<T, V>(src[r] + (g0 + j * L < cgs ? g0 + j * L : g0) * V);
+#pragma unroll
+        for (int r = 0; r < R; r++)
+#pragma unroll
+            for (int j = 0; j < 2; j++) {
                 const int g = g0 + j * L;
                 if (g >= cgs) break;
-                const float4 v = act4(v4[j], act);
-                const float vv[4] = {v.x, v.y, v.z, v.w};
+                const FV<V> a = actv<V>(v[r][j], act);
+                // (a lane meets its channels in rising order: a later equal value never replaces the first)
+                if (g * V + V <= in.c) {
 #pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    const int c = g * 4 + i;
-                    if (c < in.c && (vv[i] > best || (vv[i] == best && c < bidx))) {
-                        best = vv[i];
-                        bidx = c;
+                    for (int i = 0; i < V; i++) {
+                        const bool up = a.v[i] > best[r];
+                        best[r] = up ? a.v[i] : best[r];
+                        bidx[r] = up ? g * V + i : bidx[r];
+                    }
+                } else {
+#pragma unroll
+                    for (int i = 0; i < V; i++) {
+                        const int c = g * V + i;
+                        if (c < in.c && a.v[i] > best[r]) {
+                            best[r] = a.v[i];
+                            bidx[r] = c;
+                        }
                     }
                 }
             }
-        }
     }
-    for (int o = L >> 1; o > 0; o >>= 1) {
-        const float ob = __shfl_xor(best, o, 64);
-        const int oi = __shfl_xor(bidx, o, 64);
-        if (ob > best || (ob == best && oi < bidx)) {
-            best = ob;
-            bidx = oi;
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        if (L >= 2) argmax_dpp_step<0xB1>(best[r], bidx[r]);    // quad_perm [1,0,3,2]
+        if (L >= 4) argmax_dpp_step<0x4E>(best[r], bidx[r]);    // quad_perm [2,3,0,1]
+        if (L >= 8) argmax_dpp_step<0x141>(best[r], bidx[r]);   // row_half_mirror
+        if (L >= 16) argmax_dpp_step<0x140>(best[r], bidx[r]);  // row_mirror
+        if (L >= 32) {   // across rows of 16: swizzle inside a half wave (xor 16), then across the halves
+            const float ob = __int_as_float(__builtin_amdgcn_ds_swizzle(__float_as_int(best[r]), 0x401f));
+            const int oi = __builtin_amdgcn_ds_swizzle(bidx[r], 0x401f);
+            argmax_merge(best[r], bidx[r], ob, oi);
         }
-    }
-    if (valid && sub == 0) {
-        T* dst = reinterpret_cast<T*>(out.ptr) + tv_off(out, y, x);
-        st4<T>(dst, make_float4((float)bidx, best, 0.f, 0.f));
-        if (idx_out) idx_out[pix] = bidx;
+        if (L >= 64) argmax_merge(best[r], bidx[r], __shfl_xor(best[r], 32, 64), __shfl_xor(bidx[r], 32, 64));
+        if (valid[r] && sub == 0) {
+            const size_t pix = pix0 + r;
+            T* dst = reinterpret_cast<T*>(out.ptr) + (out.pad == 0 ? pix * out.cp : tv_off(out, (int)(pix / in.w), (int)(pix % in.w)));
+            st4<T>(dst, make_float4((float)bidx[r], best[r], 0.f, 0.f));
+            if (idx_out) idx_out[pix] = bidx[r];
+        }
     }
 }
 void launch_argmax(const TView& in, const TView& out, int32_t* idx_out, const Act& act, hipStream_t s) {
-    const int cgs = (in.c + 3) >> 2;
+    const bool wide = in.f16 && in.cp % 8 == 0;
+    const int v = wide ? 8 : 4;
+    const int cgs = (in.c + v - 1) / v;
     int l2 = 0;
     while ((1 << l2) < cgs && l2 < 6) l2++;
     const size_t npix = (size_t)in.h * in.w;
     const size_t ppw = 64 >> l2;
-    const size_t waves = (npix + ppw - 1) / ppw;
-    FYN_DISPATCH_T(in.f16, argmax_kernel, dim3((unsigned)((waves + 3) / 4)), dim3(256), s, in, out, idx_out, act, l2);
+    // four pixels per lane group where that still leaves every SIMD of the chip a few waves
+    const bool many = npix / (ppw * 4) >= 4096;
+    const size_t waves = (npix + ppw * (many ? 4 : 1) - 1) / (ppw * (many ? 4 : 1));
+    const dim3 grid((unsigned)((waves + 3) / 4)), block(256);
+    if (wide) {
+        if (many) hipLaunchKernelGGL((argmax_kernel<_Float16, 8, 4>), grid, block, 0, s, in, out, idx_out, act, l2);
+        else hipLaunchKernelGGL((argmax_kernel<_Float16, 8, 1>), grid, block, 0, s, in, out, idx_out, act, l2);
+    } else if (in.f16) {
+        if (many) hipLaunchKernelGGL((argmax_kernel<_Float16, 4, 4>), grid, block, 0, s, in, out, idx_out, act, l2);
+        else hipLaunchKernelGGL((argmax_kernel<_Float16, 4, 1>), grid, block, 0, s, in, out, idx_out, act, l2);
+    } else {
+        if (many) hipLaunchKernelGGL((argmax_kernel<float, 4, 4>), grid, block, 0, s, in, out, idx_out, act, l2);
+        else hipLaunchKernelGGL((argmax_kernel<float, 4, 1>), grid, block, 0, s, in, out, idx_out, act, l2);
+    }
 }
 
 // ---------------------------------------------------------------------------------------------

@@ -59,7 +59,9 @@ def test_pool_parity(op, pool, stride, pad, c, h, w, act, storage):
 
 
 @STORAGES
-@pytest.mark.parametrize("op,c,h,w", [("avg", 1, 1, 1), ("max", 3, 1, 5), ("avg", 9, 2, 2), ("avg", 2048, 7, 7), ("max", 4, 200, 200), ("avg", 4, 200, 200), ("avg", 23, 13, 9), ("max", 80, 16, 16)])
+@pytest.mark.parametrize("op,c,h,w", [("avg", 1, 1, 1), ("max", 3, 1, 5), ("avg", 9, 2, 2), ("avg", 2048, 7, 7), ("max", 4, 200, 200), ("avg", 4, 200, 200), ("avg", 23, 13, 9), ("max", 80, 16, 16),
+                                        # images of 16384 pixels and more: the pixels are dealt to many workgroups, a second launch pools their results
+                                        ("avg", 23, 160, 130), ("max", 12, 300, 200), ("avg", 128, 200, 200), ("max", 4, 128, 128)])
 def test_global_pool_parity(op, c, h, w, storage):
     kind = fa.PoolLayerBuilder.POOL_MAX if op == "max" else fa.PoolLayerBuilder.POOL_AVG
     b = fa.PoolLayerBuilder(kind, "gpool").number(1).shape(c, h, w, c).prefixAct(A.RELU).deep().global_pool()
@@ -122,7 +124,8 @@ def test_concat_bit_exact(chans, relu, storage):
 
 
 @STORAGES
-@pytest.mark.parametrize("c,h,w", [(1, 1, 1), (2, 3, 1), (5, 1, 7), (1000, 1, 1), (64, 128, 256), (128, 40, 40), (21, 33, 17), (2048, 3, 5)])  # misctests.cpp:269-275 shapes
+@pytest.mark.parametrize("c,h,w", [(1, 1, 1), (2, 3, 1), (5, 1, 7), (1000, 1, 1), (64, 128, 256), (128, 40, 40), (21, 33, 17), (2048, 3, 5),
+                                   (128, 259, 257), (12, 725, 724)])  # misctests.cpp:269-275 shapes; the last two: four pixels per lane group, ragged end
 def test_argmax_indices_exact(c, h, w, storage):
     b = fa.ArgMaxLayerBuilder("argmax").number(1).shape(2, h, w, c).deep()
     x = prng.normal(90, (c, h, w))
