@@ -168,12 +168,42 @@ __device__ __forceinline__ void p16_stage_c8(f32x4_t (&acc)[2][G::FN], half8_t (
         const unsigned char* w_ = wnext;
         wnext += wstep;
         if (wnext == wend) wnext = wbase;
+        // the loads of the step: weights of step s + PD - 1 into the ring slot of step s - 1 (a0: two fragments, a2: two
+        // halves of fragments), and every position fragment's operands of step s + 1
+        auto load_a0 = [&](int wfm) { a0[dprev][wfm] = *reinterpret_cast<const half8_t*>(w_ + (wfm * NPLW) * 1024 + wlane); };
+        auto load_a2 = [&](int wfm) {
+            const i32x4_t v = *reinterpret_cast<const i32x4_t*>(w_ + (wfm * NPLW + 2) * 1024 + wlane);
+            if ((dprev & 1) == 0) { a2[dprev / 2][wfm][0] = v[0]; a2[dprev / 2][wfm][1] = v[1]; a2[dprev / 2][wfm][2] = v[2]; a2[dprev / 2][wfm][3] = v[3]; }
+            else { a2[dprev / 2][wfm][4] = v[0]; a2[dprev / 2][wfm][5] = v[1]; a2[dprev / 2][wfm][6] = v[2]; a2[dprev / 2][wfm][7] = v[3]; }
+        };
+        auto load_b0 = [&](int fn) { b0[fn] = *reinterpret_cast<const half8_t*>(lds + bbase[nbuf][fn] + noff); };
+        auto load_b1 = [&](int fn) {
+            const i32x4_t v = *reinterpret_cast<const i32x4_t*>(lds + bbase[nbuf][fn] + noff + G::PLANE);
+            if (((s + 1) & 1) == 0) { b1[fn][0] = v[0]; b1[fn][1] = v[1]; b1[fn][2] = v[2]; b1[fn][3] = v[3]; }
+            else { b1[fn][4] = v[0]; b1[fn][5] = v[1]; b1[fn][6] = v[2]; b1[fn][7] = v[3]; }
+        };
+        // (a pair step also fetches the second half of the NEXT pair, two steps ahead -- that half is free once the
+        // step's fp8 block has run --, which leaves the short step between two pair steps with five LDS reads instead
+        // of ten; not across the end of a stage, where the other buffer is handed over in the last step only)
+        const bool ahead2 = pair && t + 2 < NT;
+        const bool have_b1 = !pair && t > 0 && (((s - 1) & 1) != 0) && (t - 1) + 2 < NT;   // step s - 1 fetched this step's share
+        auto load_b1_ahead = [&](int fn) {
+            const i32x4_t v = *reinterpret_cast<const i32x4_t*>(lds + bbase[PH][fn] + G::tap_off(t + 2) + G::PLANE);
+            b1[fn][4] = v[0]; b1[fn][5] = v[1]; b1[fn][6] = v[2]; b1[fn][7] = v[3];
+        };
         if (pair) {
+            // fp8 block: a fragment's fp8 operands of the next step (the half that this block has just read) behind its
+            // two MFMAs, the fp16 weights in the first slots; the barrier of a stage's last step ahead of every read
+            // of the other buffer
 #pragma unroll
             for (int i = 0; i < 2 * FN; i++) {
                 const int fn = i / 2, fm = i % 2;
                 acc[fm][fn] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a2[d / 2][fm], b1[fn], acc[fm][fn], 0, 0, 0, 0, 0, 0);
                 if (t == NT - 1 && i == 0) lds_barrier();
+                if (fm == 1) load_b1(fn);
+#pragma unroll
+                for (int j = 0; j < 2; j++)
+                    if ((j * 2 * FN) / 2 == i) load_a0(j);
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
@@ -183,23 +213,18 @@ __device__ __forceinline__ void p16_stage_c8(f32x4_t (&acc)[2][G::FN], half8_t (
             acc[fm][fn] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0[d][fm], b0[fn], acc[fm][fn], 0, 0, 0);
             if (!pair && t == NT - 1 && i == 0) lds_barrier();
             if (fm == 1) {   // the fragment's MFMAs of this step are issued: its operands of the next step
-                b0[fn] = *reinterpret_cast<const half8_t*>(lds + bbase[nbuf][fn] + noff);
-                const i32x4_t v = *reinterpret_cast<const i32x4_t*>(lds + bbase[nbuf][fn] + noff + G::PLANE);
-                if (((s + 1) & 1) == 0) { b1[fn][0] = v[0]; b1[fn][1] = v[1]; b1[fn][2] = v[2]; b1[fn][3] = v[3]; }
-                else { b1[fn][4] = v[0]; b1[fn][5] = v[1]; b1[fn][6] = v[2]; b1[fn][7] = v[3]; }
+                load_b0(fn);
+                if (!pair && !have_b1) load_b1(fn);
+                if (ahead2) load_b1_ahead(fn);
             }
-            // the weights of step s + PD - 1 into the slot of step s - 1: four loads, spread over the step's slots
+            if (pair) {
 #pragma unroll
-            for (int j = 0; j < 4; j++) {
-                if ((j * 2 * FN) / 4 != i) continue;
-                const int wfm = j & 1;
-                if (j < 2) {
-                    a0[dprev][wfm] = *reinterpret_cast<const half8_t*>(w_ + (wfm * NPLW) * 1024 + wlane);
-                } else {
-                    const i32x4_t v = *reinterpret_cast<const i32x4_t*>(w_ + (wfm * NPLW + 2) * 1024 + wlane);
-                    if ((dprev & 1) == 0) { a2[dprev / 2][wfm][0] = v[0]; a2[dprev / 2][wfm][1] = v[1]; a2[dprev / 2][wfm][2] = v[2]; a2[dprev / 2][wfm][3] = v[3]; }
-                    else { a2[dprev / 2][wfm][4] = v[0]; a2[dprev / 2][wfm][5] = v[1]; a2[dprev / 2][wfm][6] = v[2]; a2[dprev / 2][wfm][7] = v[3]; }
-                }
+                for (int j = 0; j < 2; j++)
+                    if ((j * 2 * FN) / 2 == i) load_a2(j);
+            } else {
+#pragma unroll
+                for (int j = 0; j < 4; j++)
+                    if ((j * 2 * FN) / 4 == i) { if (j < 2) load_a0(j); else load_a2(j - 2); }
             }
             __builtin_amdgcn_sched_barrier(0);
         }
