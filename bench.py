@@ -35,7 +35,7 @@ def log(*a):
 
 def make_net(workload):
     if workload == "stylenet":
-        return networks.StyleNet(fa.STORAGE_F32, 512, 624, 3), "stylenet 512x624 ms/frame", "ms/frame", "fp32 storage, fp16x2-split MFMA, fp32 accumulate"
+        return networks.StyleNet(fa.STORAGE_F32, 512, 624, 3), "stylenet 512x624 ms/frame", "ms/frame", "fp32 storage; fp16 MFMA on the split operands' high parts + fp8 MFMA correction terms (three fp16 passes where chunks do not pair), fp32 accumulate; 1e-5 rel-L2 against the fp64 oracle"
     if workload == "stylenet9x9":
         return networks.StyleNet(fa.STORAGE_F16, 1524, 1856, 9), "stylenet9x9 1524x1856 ms/frame", "ms/frame", "fp16 storage, fp16 MFMA, fp32 accumulate"
     if workload == "resnet50":
@@ -286,6 +286,8 @@ def roofline_records(net, storage_bytes, iters=20):
         ms = lyr.timeKernel(iters)                # launches back to back in one hipGraph (dispatch gaps included)
         flops, nbytes, passes = layer_work(b, storage_bytes)
         info = lyr.kernelInfo()
+        if passes == 3 and "f16+fp8-split" in info:
+            passes = 2   # one fp16 pass and two correction passes at the fp8 rate (twice the fp16 rate) = two fp16 passes' worth of matrix-pipe time
         res = bool(int(b.getFlags()) & 1)
         # (layers of one shape that run different kernels -- one of them carries a shortcut projection, say -- are rows of their own)
         key = (t, getattr(b, "kernel_", 0), b.inputChannels_, b.outputChannels_, b.height_, b.width_, tuple(b.downsample_), res, info)

@@ -187,6 +187,7 @@ struct ConvP16Params {
     float rcp_tiles_x;    // 1.0f / tiles_x
     int pos_groups;       // workgroups per block of output channels; workgroup g walks tiles g, g + pos_groups, ...
     int cin_chunks;
+    int exact_split;      // launch_conv_p16 on fp32 tensors: three fp16 passes even where the fp8 form of the correction terms would run
     int mfrags;           // cout fragments (16 each) in wpack
     int cout_blocks;      // workgroups along cout (32*wm channels each)
     int f16;              // tensors hold fp16 (wpack then has one plane, and there are no value-range words)
@@ -233,6 +234,7 @@ size_t conv_p16_lds_bytes(const ConvP16Params& p);   // 0: no such compiled comb
 // [8 x fp8(hi / 32) | 8 x fp8(64 lo)] per lane); this fills the third from src = [fragment][lane][those sixteen floats]
 int launch_pack_fp8_plane(const float* src, void* wpack, size_t frags, hipStream_t s);
 int launch_conv_p16(const ConvP16Params& p, hipStream_t s);
+bool conv_p16_uses_fp8(const ConvP16Params& p);   // whether launch_conv_p16 runs the form with the correction terms as fp8 MFMAs
 // the transposed 3x3 convolution that doubles the image size, on the same parameters: positions (npos_y x npos_x,
 // tiles) are input pixels, out_off_* the stored coordinate of output pixel (0, 0), wpack holds the nine taps of a chunk
 // in the order of their input shift (conv_p16.hip: TT_KY / TT_KX)
