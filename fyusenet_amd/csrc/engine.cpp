@@ -148,7 +148,23 @@ float* static_scratch(int device) {
 // ---------------------------------------------------------------------------------------------
 // Net
 // ---------------------------------------------------------------------------------------------
+extern "C" char** environ;
+
+void Switches::read() {
+    v_.clear();
+    for (char** e = environ; e && *e; e++) {
+        if (strncmp(*e, "FYNHIP_", 7) != 0) continue;
+        const char* eq = strchr(*e, '=');
+        if (eq) v_[std::string(*e, eq - *e)] = std::string(eq + 1);
+    }
+}
+const char* Switches::get(const char* name) const {
+    auto it = v_.find(name);
+    return it == v_.end() ? nullptr : it->second.c_str();
+}
+
 Net::Net(int dev, int stor) : device(dev), storage(stor) {
+    sw.read();
     if (stor != FYN_STORAGE_F32 && stor != FYN_STORAGE_F16) fail(FYN_ERR_INVALID, "unknown storage type %d", stor);
     int count = 0;
     FYN_HIP(hipGetDeviceCount(&count));
@@ -374,7 +390,7 @@ void Net::setup() {
     fuse_projection_layers(this);
     fuse_batchnorm_layers(this);
     assign_range_resets();
-    poison_lds_ = getenv("FYNHIP_POISON_LDS") != nullptr;
+    poison_lds_ = sw.get("FYNHIP_POISON_LDS") != nullptr;
     FYN_HIP(hipStreamSynchronize(stream));
     is_setup = true;
 }
@@ -383,7 +399,7 @@ void Net::setup() {
 // tensors fed from the host (set_input and the frame pipeline clear and raise the word themselves) and the outputs of
 // layers whose kernels do (tracks_range()).
 void Net::assign_range_words() {
-    if (f16() || getenv("FYNHIP_NO_RANGE_TRACKING") || getenv("FYNHIP_FORCE_DIRECT_CONV") || tensors.empty()) return;
+    if (f16() || sw.get("FYNHIP_NO_RANGE_TRACKING") || sw.get("FYNHIP_FORCE_DIRECT_CONV") || tensors.empty()) return;
     amax_dev_ = static_cast<unsigned*>(dev_alloc(tensors.size() * RANGE_WORDS * sizeof(unsigned), true));
     for (size_t i = 0; i < tensors.size(); i++) {
         Tensor& t = tensors[i];

@@ -53,6 +53,17 @@ struct DevBuffer {
 
 class Net;
 
+// The FYNHIP_* environment switches (tests, experiments, tuning cache), read once when a network is created: nothing on
+// a launch path, and nothing during a later setup or weight load, looks at the environment again.
+class Switches {
+  public:
+    void read();                               // every variable of the environment whose name begins with FYNHIP_
+    const char* get(const char* name) const;   // the value, or nullptr when the variable was not set (like getenv)
+    bool on(const char* name) const { return get(name) != nullptr; }
+  private:
+    std::map<std::string, std::string> v_;
+};
+
 class Layer {
   public:
     Layer(Net* net, const fyn_layer_desc& d);
@@ -90,6 +101,7 @@ class Layer {
 class Net {
   public:
     Net(int device, int storage);
+    Switches sw;
     ~Net();
     void add_layer(const fyn_layer_desc& d);
     void add_custom_layer(const fyn_layer_desc& d, const fyn_custom_layer& impl);

@@ -302,6 +302,7 @@ struct DwConvParams {
     const float* bias;
     int dil, stride;
     int res_relu, res_scale;
+    int no_strips;       // keep to the one-row kernels (a test switch)
     Act act;
 };
 void launch_dwconv3x3(const DwConvParams& p, hipStream_t s);

@@ -116,9 +116,9 @@ struct TileChoice {
 };
 
 // All tile configurations that fit (possibly none), best heuristic score first.
-static std::vector<TileChoice> enumerate_tiles(int cout, const SubConv& sc, int pitch, int npl, int slack, int nbuf) {
+static std::vector<TileChoice> enumerate_tiles(Net* net, int cout, const SubConv& sc, int pitch, int npl, int slack, int nbuf) {
     std::vector<TileChoice> all;
-    const char* force = getenv("FYNHIP_CONV_TILE");  // "fm,fn,wm,wn" for experiments
+    const char* force = net->sw.get("FYNHIP_CONV_TILE");  // "fm,fn,wm,wn" for experiments
     int ff[4] = {0, 0, 0, 0};
     if (force) sscanf(force, "%d,%d,%d,%d", &ff[0], &ff[1], &ff[2], &ff[3]);
     for (int ti = 0; ti < conv_mfma_tile_count(); ti++) {
@@ -150,7 +150,7 @@ static std::vector<TileChoice> enumerate_tiles(int cout, const SubConv& sc, int 
         const int cpb = wm * fm * 32;
         const int cblocks = (cout + cpb - 1) / cpb;
         const int halo_w = (tw - 1) * sc.in_stride + sc.span_x, halo_h = (th - 1) * sc.in_stride + sc.span_y;
-        const char* rp = getenv("FYNHIP_ROWPAD");
+        const char* rp = net->sw.get("FYNHIP_ROWPAD");
         const int rowpad = rp ? atoi(rp) : 0;
         const size_t lds = 1024 + (size_t)nbuf * npl * ((size_t)halo_h * (halo_w * pitch + rowpad) + slack);
         if (lds > 150 * 1024) continue;
@@ -166,9 +166,9 @@ static std::vector<TileChoice> enumerate_tiles(int cout, const SubConv& sc, int 
 }
 
 // kc_force > 0 selects the chunk width, 0 the default for the geometry.
-static void conv_geometry(const TView& in, bool split, int ntaps, int kc_force, int& kc, int& pitch, int& slack, int& npl) {
+static void conv_geometry(Net* net, const TView& in, bool split, int ntaps, int kc_force, int& kc, int& pitch, int& slack, int& npl) {
     // input channels staged per chunk: kernels with few taps take wide chunks (fewer barriers per output)
-    const char* kmax = getenv("FYNHIP_CONV_KC_MAX");
+    const char* kmax = net->sw.get("FYNHIP_CONV_KC_MAX");
     const int cap = kmax ? atoi(kmax) : 128;
     if (in.cp == 4) kc = 4;
     else if (in.cp <= 16) kc = 16;
@@ -192,7 +192,7 @@ static MfmaLaunch plan_mfma(Net* net, const SubConv& sc, const TView& in, const 
     L.cout = cout;
     const bool split = !net->f16();
     int kc, pitch, slack, npl;
-    conv_geometry(in, split, (int)sc.taps.size(), tc.kc, kc, pitch, slack, npl);
+    conv_geometry(net, in, split, (int)sc.taps.size(), tc.kc, kc, pitch, slack, npl);
     const int tw = 1 << tc.twl;
     ConvMfmaParams& p = L.p;
     p.in = in.ptr;
@@ -279,12 +279,12 @@ static MfmaLaunch plan_mfma(Net* net, const SubConv& sc, const TView& in, const 
         int pd = 2;
         if (kc == 32) pd = (raw % 6 == 0) ? 6 : ((raw % 4 == 0) ? 4 : 2);
         if (kc >= 64) pd = 4;
-        if (const char* e = getenv("FYNHIP_CONV_PD")) pd = atoi(e);
+        if (const char* e = net->sw.get("FYNHIP_CONV_PD")) pd = atoi(e);
         if (force_pd > 0 && kc <= 32) pd = force_pd;
         const bool ksplit_tile = tc.wm * tc.wn < 4;      // waves split the steps of a chunk: smallest step group
         if (ksplit_tile) pd = kc > 128 ? 4 : 2;
         L.var.pd = pd;
-        L.var.unr = (pd == 6 && raw % 18 == 0 && force_pd == 0 && !getenv("FYNHIP_CONV_NO_FULL_UNROLL")) ? 18 : pd;
+        L.var.unr = (pd == 6 && raw % 18 == 0 && force_pd == 0 && !net->sw.get("FYNHIP_CONV_NO_FULL_UNROLL")) ? 18 : pd;
         if (kc == 128 && !ksplit_tile) L.var.unr = 8;
         if (!conv_mfma_variant_exists(L.var)) fail(FYN_ERR_UNSUPPORTED, "MFMA convolution variant not compiled");
     }
@@ -377,12 +377,12 @@ static float time_launch(Net* net, const MfmaLaunch& L, int iters) {
 
 // ---- optional on-disk memory of tuning results (text: "<key> fm fn wm wn kc ksplit tile_w_log2" per line) ----
 static std::mutex g_tune_mu;   // guards the map and the file: networks may be set up from several threads
-static std::map<std::string, std::array<int, 7>>& tune_cache() {
+static std::map<std::string, std::array<int, 7>>& tune_cache(Net* net) {
     static std::map<std::string, std::array<int, 7>> cache;
     static bool loaded = false;
     if (!loaded) {
         loaded = true;
-        const char* path = getenv("FYNHIP_TUNE_CACHE");
+        const char* path = net->sw.get("FYNHIP_TUNE_CACHE");
         FILE* f = path ? fopen(path, "r") : nullptr;
         if (f) {
             char k[160];
@@ -395,17 +395,17 @@ static std::map<std::string, std::array<int, 7>>& tune_cache() {
 }
 
 // switches that pin part of the choice are for experiments: choices are neither remembered nor recalled then
-static bool tune_cache_bypassed() {
+static bool tune_cache_bypassed(Net* net) {
     for (const char* e : {"FYNHIP_FORCE_KSPLIT", "FYNHIP_CONV_TILE", "FYNHIP_CONV_KC_MAX", "FYNHIP_CONV_KC", "FYNHIP_CONV_PD"})
-        if (getenv(e)) return true;
+        if (net->sw.get(e)) return true;
     return false;
 }
 
-static const TileChoice* tune_cache_lookup(const char* key, const std::vector<TileChoice>& cands, int* ksplit) {
-    if (tune_cache_bypassed()) return nullptr;
+static const TileChoice* tune_cache_lookup(Net* net, const char* key, const std::vector<TileChoice>& cands, int* ksplit) {
+    if (tune_cache_bypassed(net)) return nullptr;
     std::lock_guard<std::mutex> lk(g_tune_mu);
-    auto it = tune_cache().find(key);
-    if (it == tune_cache().end()) return nullptr;
+    auto it = tune_cache(net).find(key);
+    if (it == tune_cache(net).end()) return nullptr;
     for (const TileChoice& c : cands)
         if (c.fm == it->second[0] && c.fn == it->second[1] && c.wm == it->second[2] && c.wn == it->second[3] && c.kc == it->second[4] &&
             c.twl == it->second[6]) {
@@ -415,11 +415,11 @@ static const TileChoice* tune_cache_lookup(const char* key, const std::vector<Ti
     return nullptr;
 }
 
-static void tune_cache_store(const char* key, const ConvVariant& v, int ksplit, int twl) {
-    if (tune_cache_bypassed()) return;
+static void tune_cache_store(Net* net, const char* key, const ConvVariant& v, int ksplit, int twl) {
+    if (tune_cache_bypassed(net)) return;
     std::lock_guard<std::mutex> lk(g_tune_mu);
-    tune_cache()[key] = {v.fm, v.fn, v.wm, v.wn, v.kc, ksplit, twl};   // same geometry later in this process: same choice
-    const char* path = getenv("FYNHIP_TUNE_CACHE");
+    tune_cache(net)[key] = {v.fm, v.fn, v.wm, v.wn, v.kc, ksplit, twl};   // same geometry later in this process: same choice
+    const char* path = net->sw.get("FYNHIP_TUNE_CACHE");
     if (!path) return;
     FILE* f = fopen(path, "a");
     if (!f) return;
@@ -428,32 +428,32 @@ static void tune_cache_store(const char* key, const ConvVariant& v, int ksplit, 
 }
 
 // a measured yes/no choice under a key of its own (same file, the first number is the flag)
-static bool tune_cache_flag(const char* key, bool* flag) {
-    if (tune_cache_bypassed()) return false;
+static bool tune_cache_flag(Net* net, const char* key, bool* flag) {
+    if (tune_cache_bypassed(net)) return false;
     std::lock_guard<std::mutex> lk(g_tune_mu);
-    auto it = tune_cache().find(key);
-    if (it == tune_cache().end()) return false;
+    auto it = tune_cache(net).find(key);
+    if (it == tune_cache(net).end()) return false;
     *flag = it->second[0] != 0;
     return true;
 }
-static void tune_cache_store_flag(const char* key, bool flag) {
+static void tune_cache_store_flag(Net* net, const char* key, bool flag) {
     ConvVariant v{};
     v.fm = flag ? 1 : 0;
-    tune_cache_store(key, v, 0, 0);
+    tune_cache_store(net, key, v, 0, 0);
 }
 // three numbers under a key of their own (same file)
-static bool tune_cache_triple(const char* key, int (&out)[3]) {
-    if (tune_cache_bypassed()) return false;
+static bool tune_cache_triple(Net* net, const char* key, int (&out)[3]) {
+    if (tune_cache_bypassed(net)) return false;
     std::lock_guard<std::mutex> lk(g_tune_mu);
-    auto it = tune_cache().find(key);
-    if (it == tune_cache().end()) return false;
+    auto it = tune_cache(net).find(key);
+    if (it == tune_cache(net).end()) return false;
     out[0] = it->second[0]; out[1] = it->second[1]; out[2] = it->second[2];
     return true;
 }
-static void tune_cache_store_triple(const char* key, int a, int b, int c) {
+static void tune_cache_store_triple(Net* net, const char* key, int a, int b, int c) {
     ConvVariant v{};
     v.fm = a; v.fn = b; v.wm = c;
-    tune_cache_store(key, v, 0, 0);
+    tune_cache_store(net, key, v, 0, 0);
 }
 
 // Picks the tile configuration of one (sub-)convolution: by measurement on the layer's own tensors (default), or by
@@ -468,24 +468,24 @@ static MfmaLaunch tune_mfma(Net* net, const SubConv& sc, const TView& in, const 
     std::vector<TileChoice> cands;
     {
         int kc0, pitch, slack, npl;
-        conv_geometry(in, !net->f16(), (int)sc.taps.size(), 0, kc0, pitch, slack, npl);
+        conv_geometry(net, in, !net->f16(), (int)sc.taps.size(), 0, kc0, pitch, slack, npl);
         std::vector<int> kcs{kc0};
         if (kc0 > 32) kcs.push_back(32);
         // one-tap layers with many input channels: also chunks of 256 to 1024 channels (K-split tiles only)
-        if (sc.taps.size() == 1 && !getenv("FYNHIP_CONV_KC_MAX"))
+        if (sc.taps.size() == 1 && !net->sw.get("FYNHIP_CONV_KC_MAX"))
             for (int big : {256, 512, 1024})
                 if (in.cp >= big) kcs.push_back(big);
-        if (const char* fk = getenv("FYNHIP_CONV_KC")) {   // testing: this chunk width first, the others only if it fits no tile
+        if (const char* fk = net->sw.get("FYNHIP_CONV_KC")) {   // testing: this chunk width first, the others only if it fits no tile
             const int f = atoi(fk);
             const bool known = f == 32 || f == 64 || f == 128 || ((f == 256 || f == 512 || f == 1024) && sc.taps.size() == 1);
             if (known && in.cp >= 32) kcs.insert(kcs.begin(), f);
         }
         for (int kco : kcs) {
-            if (getenv("FYNHIP_CONV_KC") && kco != kcs[0] && !cands.empty()) break;
+            if (net->sw.get("FYNHIP_CONV_KC") && kco != kcs[0] && !cands.empty()) break;
             int kc;
-            conv_geometry(in, !net->f16(), (int)sc.taps.size(), kco, kc, pitch, slack, npl);
+            conv_geometry(net, in, !net->f16(), (int)sc.taps.size(), kco, kc, pitch, slack, npl);
             const int chunks = (kc == 4) ? 1 : (in.cp + kc - 1) / kc;
-            std::vector<TileChoice> c = enumerate_tiles(cout, sc, pitch, npl, slack, chunks > 1 ? 2 : 1);
+            std::vector<TileChoice> c = enumerate_tiles(net, cout, sc, pitch, npl, slack, chunks > 1 ? 2 : 1);
             for (TileChoice& tc : c) {
                 tc.kc = kc;
                 if (kco != kc0) tc.score *= 0.9;
@@ -502,7 +502,7 @@ static MfmaLaunch tune_mfma(Net* net, const SubConv& sc, const TView& in, const 
         std::stable_sort(cands.begin(), cands.end(), [](const TileChoice& x, const TileChoice& y) { return x.score > y.score; });
     }
     if (cands.empty()) fail(FYN_ERR_UNSUPPORTED, "no MFMA tile configuration fits this convolution");
-    const char* at = getenv("FYNHIP_AUTOTUNE");
+    const char* at = net->sw.get("FYNHIP_AUTOTUNE");
     const bool tune = !(at && at[0] == '0') && cands.size() > 1;
     // FYNHIP_TUNE_CACHE=<file>: measured choices are remembered per problem geometry, so that later
     // processes (e.g. under a profiler, where timing is distorted) pick the same kernels
@@ -511,7 +511,7 @@ static MfmaLaunch tune_mfma(Net* net, const SubConv& sc, const TView& in, const 
              sc.in_stride, sc.taps.size(), sc.span_y, sc.span_x, sc.out_step, res ? 1 : 0, in.cp, sc.clamp, sc.in_shift, sc.in_sub, sc.fuse_k);
     if (tune) {
         int ks = 1;
-        const TileChoice* hit = tune_cache_lookup(key, cands, &ks);
+        const TileChoice* hit = tune_cache_lookup(net, key, cands, &ks);
         if (hit) {
             MfmaLaunch L = plan_mfma(net, sc, in, out, res, cin, cout, act, res_relu, res_scale, *hit, scale, bias);
             // a remembered split factor is held to what this layer allows, like a forced one
@@ -522,14 +522,14 @@ static MfmaLaunch tune_mfma(Net* net, const SubConv& sc, const TView& in, const 
         }
     }
     MfmaLaunch best = plan_mfma(net, sc, in, out, res, cin, cout, act, res_relu, res_scale, cands[0], scale, bias);
-    if (const char* fk = getenv("FYNHIP_FORCE_KSPLIT")) {   // testing: fixed split-K factor (clamped to what the layer allows)
+    if (const char* fk = net->sw.get("FYNHIP_FORCE_KSPLIT")) {   // testing: fixed split-K factor (clamped to what the layer allows)
         int ks = sc.fuse_k ? 1 : atoi(fk);   // (the fused shift-sum needs the whole reduction in one workgroup)
         while (ks > 1 && (ks - 1) * ((best.p.cin_chunks + ks - 1) / ks) >= best.p.cin_chunks) ks--;
         set_ksplit(net, best, ks);
         return best;
     }
     if (!tune) return best;
-    const bool verbose = getenv("FYNHIP_TUNE_VERBOSE") != nullptr;
+    const bool verbose = net->sw.get("FYNHIP_TUNE_VERBOSE") != nullptr;
     float best_ms = std::min(time_launch(net, best, 4), time_launch(net, best, 4));
     if (verbose) fprintf(stderr, "[tune] %s -> %.1f us\n", mfma_info(best).c_str(), best_ms * 1e3f);
     std::vector<std::pair<float, MfmaLaunch>> timed;
@@ -590,7 +590,7 @@ static MfmaLaunch tune_mfma(Net* net, const SubConv& sc, const TView& in, const 
             }
         }
     }
-    tune_cache_store(key, best.var, best.p.ksplit, best.p.tile_w_log2);
+    tune_cache_store(net, key, best.var, best.p.ksplit, best.p.tile_w_log2);
     // the losing candidates' device buffers (step tables, weight buffers of their own, split-K partial sums) go back
     {
         std::vector<void*> drop;
@@ -659,14 +659,14 @@ static MfmaGroup tune_mfma_group(Net* net, const std::vector<SubConv>& scs, cons
     std::vector<TileChoice> cands;
     {
         int kc0, pitch, slack, npl;
-        conv_geometry(in, !net->f16(), (int)scs[big].taps.size(), 0, kc0, pitch, slack, npl);
+        conv_geometry(net, in, !net->f16(), (int)scs[big].taps.size(), 0, kc0, pitch, slack, npl);
         std::vector<int> kcs{kc0};
         if (kc0 > 32) kcs.push_back(32);
         for (int kco : kcs) {
             int kc;
-            conv_geometry(in, !net->f16(), (int)scs[big].taps.size(), kco, kc, pitch, slack, npl);
+            conv_geometry(net, in, !net->f16(), (int)scs[big].taps.size(), kco, kc, pitch, slack, npl);
             const int chunks = (kc == 4) ? 1 : (in.cp + kc - 1) / kc;
-            std::vector<TileChoice> c = enumerate_tiles(cout, scs[big], pitch, npl, slack, chunks > 1 ? 2 : 1);
+            std::vector<TileChoice> c = enumerate_tiles(net, cout, scs[big], pitch, npl, slack, chunks > 1 ? 2 : 1);
             for (TileChoice& tc : c) {
                 tc.kc = kc;
                 if (tc.wm * tc.wn < 4) continue;   // no merged entry point for tiles whose waves split K
@@ -683,19 +683,19 @@ static MfmaGroup tune_mfma_group(Net* net, const std::vector<SubConv>& scs, cons
         g.sync();
         return g;
     };
-    const char* at = getenv("FYNHIP_AUTOTUNE");
+    const char* at = net->sw.get("FYNHIP_AUTOTUNE");
     const bool tune = !(at && at[0] == '0') && cands.size() > 1;
     char key[160];
     snprintf(key, sizeof(key), "g%zu:%d%d:%dx%d:%dx%d:t%zu:o%d:cp%d", scs.size(), in.f16, out.f16, cin, cout, scs[big].npos_y, scs[big].npos_x,
              scs[big].taps.size(), scs[big].out_step, in.cp);
     if (tune) {
         int ks = 1;
-        const TileChoice* hit = tune_cache_lookup(key, cands, &ks);
+        const TileChoice* hit = tune_cache_lookup(net, key, cands, &ks);
         if (hit) return plan_all(*hit, nullptr);
     }
     MfmaGroup best = plan_all(cands[0], nullptr);
     if (!tune) return best;
-    const bool verbose = getenv("FYNHIP_TUNE_VERBOSE") != nullptr;
+    const bool verbose = net->sw.get("FYNHIP_TUNE_VERBOSE") != nullptr;
     float best_ms = std::min(time_group(net, best, 4), time_group(net, best, 4));
     if (verbose) fprintf(stderr, "[tune] group of %zu: %s -> %.1f us\n", scs.size(), mfma_info(best.subs[0]).c_str(), best_ms * 1e3f);
     for (size_t i = 1; i < cands.size(); i++) {
@@ -707,7 +707,7 @@ static MfmaGroup tune_mfma_group(Net* net, const std::vector<SubConv>& scs, cons
             best = g;
         }
     }
-    tune_cache_store(key, best.var, 1, best.subs[0].p.tile_w_log2);
+    tune_cache_store(net, key, best.var, 1, best.subs[0].p.tile_w_log2);
     return best;
 }
 
@@ -824,17 +824,17 @@ class ConvLayer : public Layer {
             oh = d.height * inv / stride;
             ow = d.width * inv / stride;
             clamp = true;
-            direct = getenv("FYNHIP_FORCE_DIRECT_CONV") != nullptr;
-            wide = !direct && oc <= 4 && oc * k <= 32 && stride == 1 && d.in_channels > 4 && getenv("FYNHIP_NO_WIDE_CONV") == nullptr;
+            direct = net->sw.get("FYNHIP_FORCE_DIRECT_CONV") != nullptr;
+            wide = !direct && oc <= 4 && oc * k <= 32 && stride == 1 && d.in_channels > 4 && net->sw.get("FYNHIP_NO_WIDE_CONV") == nullptr;
             return;
         }
         // shallow, unpadded input: the sampler clamps to the edge (gpu/gpulayerbase.h:80-90)
         clamp = !(d.flags & FYN_FLAG_DEEP) && d.input_padding < r * dil && k > 1;
-        direct = getenv("FYNHIP_FORCE_DIRECT_CONV") != nullptr;   // (testing: the plain fp32 kernel instead of the MFMA path)
+        direct = net->sw.get("FYNHIP_FORCE_DIRECT_CONV") != nullptr;   // (testing: the plain fp32 kernel instead of the MFMA path)
         // few output channels under a wide kernel: fold the kx taps into the GEMM's M dimension
         // (cout*K virtual channels, K taps) and reduce the K shifted partial sums in a second pass
         wide = !direct && oc <= 4 && oc * k <= 32 && k >= 3 && stride == 1 && dil == 1 && d.in_channels > 4 &&
-               getenv("FYNHIP_NO_WIDE_CONV") == nullptr;
+               net->sw.get("FYNHIP_NO_WIDE_CONV") == nullptr;
     }
     // the sub-convolution of the folded form: K vertical taps over the columns of q
     SubConv wide_subconv() {
@@ -918,9 +918,9 @@ class ConvLayer : public Layer {
         q.acc_mul = 1.f;
         q.act = act();
         q.in_amax = tin(0).amax;   // (the candidates are timed in the form the frame will run: fp8 correction terms where the input has a range word)
-        q.exact_split = getenv("FYNHIP_EXACT_SPLIT") ? 1 : 0;
+        q.exact_split = net->sw.get("FYNHIP_EXACT_SPLIT") ? 1 : 0;
         int want_h = 0, want_w = 0, want_wm = 0;   // FYNHIP_P16_TILE=h,w[,wm] (tests): that combination
-        if (const char* e = getenv("FYNHIP_P16_TILE")) sscanf(e, "%d,%d,%d", &want_h, &want_w, &want_wm);
+        if (const char* e = net->sw.get("FYNHIP_P16_TILE")) sscanf(e, "%d,%d,%d", &want_h, &want_w, &want_wm);
         struct Cand { double cost; ConvP16Params q; };
         std::vector<Cand> cands;
         for (int i = 0; i < conv_p16_tile_count(); i++) {
@@ -949,15 +949,15 @@ class ConvLayer : public Layer {
         const size_t halves = ((size_t)q.cin_chunks * 9 + 8) * q.mfrags * (q.f16 ? 1 : 3) * 64 * 8;
         p16_wpack_dev = net->dev_alloc(halves * 2, true);
         for (Cand& c : cands) c.q.wpack = p16_wpack_dev;
-        const bool always = getenv("FYNHIP_FORCE_P16_CONV") != nullptr;
-        const char* at = getenv("FYNHIP_AUTOTUNE");
+        const bool always = net->sw.get("FYNHIP_FORCE_P16_CONV") != nullptr;
+        const char* at = net->sw.get("FYNHIP_AUTOTUNE");
         const bool timing = !(at && at[0] == '0');
         int pick = 0;   // index into cands, -1: the general kernel
         char key[160];
         snprintf(key, sizeof(key), "p16:%dx%d:%dx%d:s%d:cp%d:r%d:e%d:h%d", d.in_channels, oc, oh, ow, stride, in_v.cp, res_v ? 1 : 0, clamp ? 1 : 0, q.f16);
         int cached[3] = {0, 0, 0};
         bool have_cached = false;
-        if (!want_h) have_cached = tune_cache_triple(key, cached);   // (the cache keeps: chosen?, tile_h*1000 + tile_w, wm)
+        if (!want_h) have_cached = tune_cache_triple(net, key, cached);   // (the cache keeps: chosen?, tile_h*1000 + tile_w, wm)
         if (have_cached) {
             pick = -1;
             if (cached[0] || always)
@@ -975,11 +975,11 @@ class ConvLayer : public Layer {
                 }
                 t_other = std::min(t_other, time_launch(net, launch, 10));
             }
-            if (getenv("FYNHIP_TUNE_VERBOSE"))
+            if (net->sw.get("FYNHIP_TUNE_VERBOSE"))
                 fprintf(stderr, "[tune] 3x3: 16-position fragments (%dx%d tiles, %d channel groups) %.1f us, general kernel %.1f us\n",
                         cands[pick].q.tile_h, cands[pick].q.tile_w, cands[pick].q.wm, best * 1e3f, t_other * 1e3f);
             const bool win = best < t_other;
-            if (!want_h) tune_cache_store_triple(key, win ? 1 : 0, cands[pick].q.tile_h * 1000 + cands[pick].q.tile_w, cands[pick].q.wm);
+            if (!want_h) tune_cache_store_triple(net, key, win ? 1 : 0, cands[pick].q.tile_h * 1000 + cands[pick].q.tile_w, cands[pick].q.wm);
             if (!win && !always) pick = -1;
         }
         if (pick >= 0) {
@@ -1008,7 +1008,7 @@ class ConvLayer : public Layer {
         q.acc_mul = 1.f;
         q.act = act();
         int want_h = 0, want_w = 0;
-        if (const char* e = getenv("FYNHIP_P16_TILE")) sscanf(e, "%d,%d", &want_h, &want_w);
+        if (const char* e = net->sw.get("FYNHIP_P16_TILE")) sscanf(e, "%d,%d", &want_h, &want_w);
         std::vector<ConvP16Params> cands;
         int steps = 0;
         for (int i = 0; i < conv_p16c4_tile_count(); i++) {
@@ -1030,13 +1030,13 @@ class ConvLayer : public Layer {
         const size_t halves = ((size_t)steps + 8) * q.mfrags * (q.f16 ? 1 : 2) * 64 * 8;
         p16_wpack_dev = net->dev_alloc(halves * 2, true);
         for (ConvP16Params& c : cands) c.wpack = p16_wpack_dev;
-        const bool always = getenv("FYNHIP_FORCE_P16_CONV") != nullptr;
-        const char* at = getenv("FYNHIP_AUTOTUNE");
+        const bool always = net->sw.get("FYNHIP_FORCE_P16_CONV") != nullptr;
+        const char* at = net->sw.get("FYNHIP_AUTOTUNE");
         int pick = 0;
         char key[160];
         snprintf(key, sizeof(key), "c4p16:k%d:%dx%d:%dx%d:e%d:h%d", k, d.in_channels, oc, oh, ow, clamp ? 1 : 0, q.f16);
         int cached[3] = {0, 0, 0};
-        if (!want_h && tune_cache_triple(key, cached)) {
+        if (!want_h && tune_cache_triple(net, key, cached)) {
             pick = -1;
             if (cached[0] || always)
                 for (size_t i = 0; i < cands.size(); i++)
@@ -1053,11 +1053,11 @@ class ConvLayer : public Layer {
                 }
                 t_other = std::min(t_other, time_launch(net, launch, 10));
             }
-            if (getenv("FYNHIP_TUNE_VERBOSE"))
+            if (net->sw.get("FYNHIP_TUNE_VERBOSE"))
                 fprintf(stderr, "[tune] %dx%d on %d channels: 16-position fragments (%dx%d tiles) %.1f us, general kernel %.1f us\n", k, k, d.in_channels,
                         cands[pick].tile_h, cands[pick].tile_w, best * 1e3f, t_other * 1e3f);
             const bool win = best < t_other;
-            if (!want_h) tune_cache_store_triple(key, win ? 1 : 0, cands[pick].tile_h * 1000 + cands[pick].tile_w, 1);
+            if (!want_h) tune_cache_store_triple(net, key, win ? 1 : 0, cands[pick].tile_h * 1000 + cands[pick].tile_w, 1);
             if (!win && !always) pick = -1;
         }
         if (pick >= 0) {
@@ -1091,8 +1091,8 @@ class ConvLayer : public Layer {
         q.acc_mul = 1.f;
         q.act = act();
         int want_h = 0, want_w = 0, want_rows1 = 0, want_h2 = 0;   // FYNHIP_P16_TILE=h,w and FYNHIP_H16_SPLIT=rows of the first band,h of the second (tests)
-        if (const char* e = getenv("FYNHIP_P16_TILE")) sscanf(e, "%d,%d", &want_h, &want_w);
-        if (const char* e = getenv("FYNHIP_H16_SPLIT")) sscanf(e, "%d,%d", &want_rows1, &want_h2);
+        if (const char* e = net->sw.get("FYNHIP_P16_TILE")) sscanf(e, "%d,%d", &want_h, &want_w);
+        if (const char* e = net->sw.get("FYNHIP_H16_SPLIT")) sscanf(e, "%d,%d", &want_rows1, &want_h2);
         // a band of `rows` output rows from row `row0` on, in tiles of th x tw; cost in MFMA cycles per wave (0: cannot be built)
         auto band = [&](int th, int tw, int row0, int rows, ConvP16Params* c, double* cost) {
             *c = q;
@@ -1153,8 +1153,8 @@ class ConvLayer : public Layer {
                 fail(FYN_ERR_DEVICE, "fp16 16-position convolution launch failed while tuning");
         };
         const bool forced = want_h || want_rows1;
-        const bool always = getenv("FYNHIP_FORCE_P16_CONV") != nullptr;
-        const char* at = getenv("FYNHIP_AUTOTUNE");
+        const bool always = net->sw.get("FYNHIP_FORCE_P16_CONV") != nullptr;
+        const char* at = net->sw.get("FYNHIP_AUTOTUNE");
         int pick = 0;
         char key[160];
         snprintf(key, sizeof(key), "h16:k%d:%dx%d:%dx%d:cp%d:r%d:e%d", k, d.in_channels, oc, oh, ow, in_v.cp, res_v ? 1 : 0, clamp ? 1 : 0);
@@ -1162,7 +1162,7 @@ class ConvLayer : public Layer {
         auto code1 = [](const Cand& c) { return c.a.tile_h * 1000 + c.a.tile_w; };
         auto code2 = [](const Cand& c) { return c.two ? c.a.npos_y * 1000 + c.b.tile_h : 0; };
         int cached[3] = {0, 0, 0};
-        if (!forced && tune_cache_triple(key, cached)) {
+        if (!forced && tune_cache_triple(net, key, cached)) {
             pick = -1;
             if (cached[0] || always)
                 for (size_t i = 0; i < cands.size(); i++)
@@ -1177,11 +1177,11 @@ class ConvLayer : public Layer {
                 }
                 t_other = std::min(t_other, time_launch(net, launch, 5));
             }
-            if (getenv("FYNHIP_TUNE_VERBOSE"))
+            if (net->sw.get("FYNHIP_TUNE_VERBOSE"))
                 fprintf(stderr, "[tune] %dx%d fp16: 16-position fragments (%dx%d tiles%s) %.1f us, general kernel %.1f us\n", k, k,
                         cands[pick].a.tile_h, cands[pick].a.tile_w, cands[pick].two ? ", two bands" : "", best * 1e3f, t_other * 1e3f);
             const bool win = best < t_other;
-            if (!forced) tune_cache_store_triple(key, win ? 1 : 0, code1(cands[pick]), code2(cands[pick]));
+            if (!forced) tune_cache_store_triple(net, key, win ? 1 : 0, code1(cands[pick]), code2(cands[pick]));
             if (!win && !always) pick = -1;
         }
         if (pick >= 0) {
@@ -1234,7 +1234,7 @@ class ConvLayer : public Layer {
         q.acc_mul = 1.f;
         q.act = act();
         int want_fm = 0, want_th = 0, want_tw = 0;   // FYNHIP_KR16_FM=fragments per block of output channels[,tile h,tile w] (tests)
-        if (const char* e = getenv("FYNHIP_KR16_FM")) sscanf(e, "%d,%d,%d", &want_fm, &want_th, &want_tw);
+        if (const char* e = net->sw.get("FYNHIP_KR16_FM")) sscanf(e, "%d,%d,%d", &want_fm, &want_th, &want_tw);
         std::vector<ConvP16Params> cands;
         for (int i = 0; i < conv_kr16_variant_count(); i++) {
             int taps, chunks, fm, th, tw, vstride;
@@ -1264,13 +1264,13 @@ class ConvLayer : public Layer {
         void* const kr_wpack = net->dev_alloc(halves * 2, true);
         for (ConvP16Params& c : cands) c.wpack = kr_wpack;
         const bool had_p16 = p16;   // the 3x3 16-position form was chosen over the general kernel: this form has to beat it instead
-        const bool always = getenv("FYNHIP_FORCE_KR16_CONV") != nullptr;
-        const char* at = getenv("FYNHIP_AUTOTUNE");
+        const bool always = net->sw.get("FYNHIP_FORCE_KR16_CONV") != nullptr;
+        const char* at = net->sw.get("FYNHIP_AUTOTUNE");
         int pick = 0;
         char key[160];
         snprintf(key, sizeof(key), "kr16:k%d:%dx%d:%dx%d:s%d:r%d:e%d:h%d:p%d", k, d.in_channels, oc, oh, ow, stride, res_v ? 1 : 0, clamp ? 1 : 0, q.f16, had_p16 ? 1 : 0);
         int cached[3] = {0, 0, 0};
-        if (!want_fm && tune_cache_triple(key, cached)) {
+        if (!want_fm && tune_cache_triple(net, key, cached)) {
             pick = -1;
             if (cached[0] || always)
                 for (size_t i = 0; i < cands.size(); i++)
@@ -1292,12 +1292,12 @@ class ConvLayer : public Layer {
                 else
                     t_other = std::min(t_other, time_launch(net, launch, 10));
             }
-            if (getenv("FYNHIP_TUNE_VERBOSE"))
+            if (net->sw.get("FYNHIP_TUNE_VERBOSE"))
                 fprintf(stderr, "[tune] %dx%d on %d channels, %dx%d positions: K-resident form (%d-channel blocks, %dx%d tiles) %.1f us, %s %.1f us\n", k, k,
                         d.in_channels, oh, ow, 16 * cands[pick].wm, cands[pick].tile_h, cands[pick].tile_w, best * 1e3f,
                         had_p16 ? "16-position 3x3 form" : "general kernel", t_other * 1e3f);
             const bool win = best < t_other;
-            if (!want_fm) tune_cache_store_triple(key, win ? 1 : 0, cands[pick].wm, cands[pick].tile_h * 100 + cands[pick].tile_w);
+            if (!want_fm) tune_cache_store_triple(net, key, win ? 1 : 0, cands[pick].wm, cands[pick].tile_h * 100 + cands[pick].tile_w);
             if (!win && !always) pick = -1;
         }
         if (pick >= 0) {
@@ -1336,16 +1336,16 @@ class ConvLayer : public Layer {
         const int min_blocks = ks ? (q.mfrags + 3) / 4 : 1;   // (the K x K form: one fragment per wave)
         if (ks && min_blocks > 4) { net->dev_free(wp); return; }
         q.cout_blocks = min_blocks;
-        if (const char* e = getenv("FYNHIP_D16_BLOCKS")) q.cout_blocks = std::max(-4, std::min(4, atoi(e))) ? std::max(-4, std::min(4, atoi(e))) : 1;   // (negative: a wave per 16 positions)
-        const bool always = getenv("FYNHIP_FORCE_D16_CONV") != nullptr;
-        const char* at = getenv("FYNHIP_AUTOTUNE");
+        if (const char* e = net->sw.get("FYNHIP_D16_BLOCKS")) q.cout_blocks = std::max(-4, std::min(4, atoi(e))) ? std::max(-4, std::min(4, atoi(e))) : 1;   // (negative: a wave per 16 positions)
+        const bool always = net->sw.get("FYNHIP_FORCE_D16_CONV") != nullptr;
+        const char* at = net->sw.get("FYNHIP_AUTOTUNE");
         bool pick = true;
         char key[160];
         snprintf(key, sizeof(key), "d16:k%d:%dx%d:%dx%d:s%d:r%d:h%d:kr%d", k, d.in_channels, oc, oh, ow, stride, res_v ? 1 : 0, q.f16, kr16 ? 1 : 0);
         int cached[3] = {0, 0, 0};
-        if (getenv("FYNHIP_D16_BLOCKS")) {
+        if (net->sw.get("FYNHIP_D16_BLOCKS")) {
             pick = always;
-        } else if (tune_cache_triple(key, cached)) {
+        } else if (tune_cache_triple(net, key, cached)) {
             pick = cached[0] != 0 || always;
             q.cout_blocks = cached[1] ? cached[1] : 1;
         } else if (!(at && at[0] == '0')) {
@@ -1375,12 +1375,12 @@ class ConvLayer : public Layer {
                 else
                     t_other = std::min(t_other, time_launch(net, launch, 10));
             }
-            if (getenv("FYNHIP_TUNE_VERBOSE"))
+            if (net->sw.get("FYNHIP_TUNE_VERBOSE"))
                 fprintf(stderr, "[tune] %dx%d on %d channels, %dx%d positions, to %d: LDS-free form (%d %s per 16 positions) %.1f us, %s %.1f us\n", k, k, d.in_channels, oh, ow,
                         oc, best_blocks < 0 ? 1 : best_blocks, best_blocks < 0 ? "wave per fragment" : "workgroup(s)", t_new * 1e3f, kr16 ? "K-resident form" : "general kernel", t_other * 1e3f);
             pick = t_new < t_other || always;
             q.cout_blocks = best_blocks;
-            tune_cache_store_triple(key, t_new < t_other ? 1 : 0, best_blocks, 0);
+            tune_cache_store_triple(net, key, t_new < t_other ? 1 : 0, best_blocks, 0);
         }
         if (q.cout_blocks < 0) { q.wm = 4; q.cout_blocks = -q.cout_blocks; }
         if (pick) {
@@ -1552,13 +1552,13 @@ class ConvLayer : public Layer {
         if (conv_rows_lds_bytes(q, out_v.f16 != 0) > 160 * 1024) return;
         const size_t halves = (size_t)k * q.cs * (out_v.f16 ? 1 : 2) * 64 * 8;
         q.wpack = rows_wpack_dev = net->dev_alloc(halves * 2, true);
-        const bool always = getenv("FYNHIP_FORCE_ROWS_WIDE_CONV") != nullptr;
-        const char* at = getenv("FYNHIP_AUTOTUNE");
+        const bool always = net->sw.get("FYNHIP_FORCE_ROWS_WIDE_CONV") != nullptr;
+        const char* at = net->sw.get("FYNHIP_AUTOTUNE");
         bool pick = true;
         char key[160];
         snprintf(key, sizeof(key), "rows:%d:%dx%d:%dx%d:k%d:cp%d:r%d:e%d", out_v.f16, d.in_channels, oc, oh, ow, k, in_v.cp, res_v ? 1 : 0, clamp ? 1 : 0);
         if (always) {
-        } else if (tune_cache_flag(key, &pick)) {
+        } else if (tune_cache_flag(net, key, &pick)) {
         } else if (!(at && at[0] == '0')) {
             float t_rows = 1e30f, t_other = 1e30f;
             for (int rep = 0; rep < 3; rep++) {
@@ -1570,9 +1570,9 @@ class ConvLayer : public Layer {
                     if (!fused) launch_shift_reduce(sr, net->stream);
                 }, 10));
             }
-            if (getenv("FYNHIP_TUNE_VERBOSE")) fprintf(stderr, "[tune] folded kx taps: row-rolling %.1f us, %s %.1f us\n", t_rows * 1e3f, fused ? "one launch" : "two passes", t_other * 1e3f);
+            if (net->sw.get("FYNHIP_TUNE_VERBOSE")) fprintf(stderr, "[tune] folded kx taps: row-rolling %.1f us, %s %.1f us\n", t_rows * 1e3f, fused ? "one launch" : "two passes", t_other * 1e3f);
             pick = t_rows < t_other;
-            tune_cache_store_flag(key, pick);
+            tune_cache_store_flag(net, key, pick);
         }
         if (pick) {
             rows = true;
@@ -1641,7 +1641,7 @@ class ConvLayer : public Layer {
             // q[y][x'][o*K+kx], x' in [0, W+K-1) <-> input column x'-r; out[y][x][o] = sum_kx q[y][x+kx][o*K+kx].
             // One launch when a tile as wide as two kernels fits (q stays in the workgroup's LDS), else q goes through
             // memory and a second pass sums it.
-            const bool never = getenv("FYNHIP_NO_FUSED_WIDE_CONV") != nullptr, always = getenv("FYNHIP_FORCE_FUSED_WIDE_CONV") != nullptr;
+            const bool never = net->sw.get("FYNHIP_NO_FUSED_WIDE_CONV") != nullptr, always = net->sw.get("FYNHIP_FORCE_FUSED_WIDE_CONV") != nullptr;
             MfmaLaunch one;
             bool have_one = false;
             if (!never) {
@@ -1667,12 +1667,12 @@ class ConvLayer : public Layer {
                 if (have_one) {
                     // The one-launch form needs halo rows and columns, i.e. large tiles and few workgroups per CU; which
                     // form is faster depends on the image size and the storage type, so both are timed.
-                    const char* at = getenv("FYNHIP_AUTOTUNE");
+                    const char* at = net->sw.get("FYNHIP_AUTOTUNE");
                     bool pick = out_v.f16 != 0;
                     char key[160];
                     snprintf(key, sizeof(key), "folded:%d:%dx%d:%dx%d:k%d:cp%d:r%d:e%d%d", out_v.f16, d.in_channels, oc, oh, ow, k, in_v.cp,
                              res_v ? 1 : 0, clamp ? 1 : 0, frac_shift);
-                    if (tune_cache_flag(key, &pick)) {
+                    if (tune_cache_flag(net, key, &pick)) {
                     } else if (!(at && at[0] == '0')) {
                         float t1 = 1e30f, t2 = 1e30f;
                         for (int rep = 0; rep < 3; rep++) {
@@ -1682,9 +1682,9 @@ class ConvLayer : public Layer {
                                 launch_shift_reduce(sr, net->stream);
                             }, 10));
                         }
-                        if (getenv("FYNHIP_TUNE_VERBOSE")) fprintf(stderr, "[tune] folded kx taps: one launch %.1f us, two passes %.1f us\n", t1 * 1e3f, t2 * 1e3f);
+                        if (net->sw.get("FYNHIP_TUNE_VERBOSE")) fprintf(stderr, "[tune] folded kx taps: one launch %.1f us, two passes %.1f us\n", t1 * 1e3f, t2 * 1e3f);
                         pick = t1 < t2;
-                        tune_cache_store_flag(key, pick);
+                        tune_cache_store_flag(net, key, pick);
                     }
                     if (pick) {
                         fused = true;
@@ -1696,7 +1696,7 @@ class ConvLayer : public Layer {
             }
             // Third form: a workgroup walks down a strip of the image with the input rows in an LDS ring and the weights
             // in registers (conv_rows.hip); every input row is fetched once per strip and q never leaves the wave.
-            if (!frac_shift && conv_rows_supported(k, in_v.cp, oc, out_v.f16 != 0) && out_v.cp == 4 && !getenv("FYNHIP_NO_ROWS_WIDE_CONV"))
+            if (!frac_shift && conv_rows_supported(k, in_v.cp, oc, out_v.f16 != 0) && out_v.cp == 4 && !net->sw.get("FYNHIP_NO_ROWS_WIDE_CONV"))
                 setup_rows_wide(in_v, out_v, res_v, res_relu, res_scale);
         } else {
             SubConv sc;
@@ -1714,7 +1714,7 @@ class ConvLayer : public Layer {
                 sc.in_x0 = (in_v.pad << sc.in_shift) + ((k == 3) ? -2 : -r);
             }
             sc.in_stride = stride;
-            if (k == 1 && stride > 1 && !frac_shift && !getenv("FYNHIP_NO_SUBSAMPLED_STAGING")) {
+            if (k == 1 && stride > 1 && !frac_shift && !net->sw.get("FYNHIP_NO_SUBSAMPLED_STAGING")) {
                 // strided pointwise layer: stage the pixels it reads and nothing between them
                 sc.in_sub = stride;
                 sc.in_stride = 1;
@@ -1732,34 +1732,34 @@ class ConvLayer : public Layer {
             // one with 64-channel wave tiles first, then the 3x3 form, then the small-input form
             const bool same_storage = in_v.f16 == out_v.f16 && (!res_v || res_v->f16 == out_v.f16);
             // (tests: the K-resident form or nothing; a forced variant of the general kernel means the general kernel)
-            const bool only_kr = getenv("FYNHIP_FORCE_KR16_CONV") || getenv("FYNHIP_FORCE_KSPLIT") || getenv("FYNHIP_CONV_TILE") || getenv("FYNHIP_CONV_KC") ||
-                                 getenv("FYNHIP_CONV_KC_MAX") || getenv("FYNHIP_CONV_PD");
+            const bool only_kr = net->sw.get("FYNHIP_FORCE_KR16_CONV") || net->sw.get("FYNHIP_FORCE_KSPLIT") || net->sw.get("FYNHIP_CONV_TILE") || net->sw.get("FYNHIP_CONV_KC") ||
+                                 net->sw.get("FYNHIP_CONV_KC_MAX") || net->sw.get("FYNHIP_CONV_PD");
             if (!only_kr && !frac_shift && same_storage && conv_h16_supported(k, stride, dil, in_v.cp, oc, out_v.cp, out_v.f16 != 0) && d.in_channels == in_v.cp &&
-                (!res_v || res_v->cp >= oc) && !getenv("FYNHIP_NO_P16_CONV") && !getenv("FYNHIP_NO_H16_CONV"))
+                (!res_v || res_v->cp >= oc) && !net->sw.get("FYNHIP_NO_P16_CONV") && !net->sw.get("FYNHIP_NO_H16_CONV"))
                 setup_h16(in_v, out_v, res_v, res_relu, res_scale);
             if (!only_kr && !p16 && !frac_shift && same_storage && !sc.in_sub && conv_p16_supported(k, stride, dil, in_v.cp, oc, out_v.cp, out_v.f16 != 0) &&
-                d.in_channels == in_v.cp && (!res_v || (res_v->cp >= oc && res_v->cp % 8 == 0)) && !getenv("FYNHIP_NO_P16_CONV"))
+                d.in_channels == in_v.cp && (!res_v || (res_v->cp >= oc && res_v->cp % 8 == 0)) && !net->sw.get("FYNHIP_NO_P16_CONV"))
                 setup_p16(in_v, out_v, res_v, res_relu, res_scale);
             if (!only_kr && !p16 && !frac_shift && same_storage && !res_v && conv_p16c4_supported(k, stride, dil, in_v.cp, oc, out_v.cp, out_v.f16 != 0) &&
-                !getenv("FYNHIP_NO_P16_CONV"))
+                !net->sw.get("FYNHIP_NO_P16_CONV"))
                 setup_c4(in_v, out_v);
             // few positions, many input channels: the whole reduction of a 4x4 tile resident in LDS instead of K-split launches
             if ((!p16 || (!h16 && !c4)) && !frac_shift && same_storage && (k == 1 || (k == 3 && (stride == 1 || stride == 2))) && dil == 1 && in_v.cp % 8 == 0 &&
                 d.in_channels == in_v.cp && in_v.cp >= 16 && oc % 4 == 0 && oc >= 8 && out_v.cp >= oc && oh * ow <= 4096 && (!res_v || (res_v->cp >= out_v.cp && res_v->cp % 8 == 0)) &&
-                !getenv("FYNHIP_NO_P16_CONV") && !getenv("FYNHIP_NO_KR16_CONV") && !getenv("FYNHIP_FORCE_P16_CONV") &&
+                !net->sw.get("FYNHIP_NO_P16_CONV") && !net->sw.get("FYNHIP_NO_KR16_CONV") && !net->sw.get("FYNHIP_FORCE_P16_CONV") &&
                 // (a test that forces a variant of the general kernel wants the general kernel)
-                !getenv("FYNHIP_FORCE_KSPLIT") && !getenv("FYNHIP_CONV_TILE") && !getenv("FYNHIP_CONV_KC") && !getenv("FYNHIP_CONV_KC_MAX") && !getenv("FYNHIP_CONV_PD"))
+                !net->sw.get("FYNHIP_FORCE_KSPLIT") && !net->sw.get("FYNHIP_CONV_TILE") && !net->sw.get("FYNHIP_CONV_KC") && !net->sw.get("FYNHIP_CONV_KC_MAX") && !net->sw.get("FYNHIP_CONV_PD"))
                 setup_kr16(in_v, out_v, res_v, res_relu, res_scale);
             // many positions, few input channels, 1x1: fragments straight from the tensor, no LDS
             if ((!p16 || kr16) && !frac_shift && same_storage && d.in_channels == in_v.cp && oc % 4 == 0 && oc >= 8 && oh * ow >= 256 &&
                 conv_d16_supported(k, dil, in_v.cp, (in_v.cp + 31) / 32, oc, out_v.cp) && (!res_v || (res_v->cp >= out_v.cp && res_v->cp % 8 == 0)) &&
-                !getenv("FYNHIP_NO_P16_CONV") && !getenv("FYNHIP_NO_D16_CONV") && !getenv("FYNHIP_FORCE_P16_CONV") && !getenv("FYNHIP_FORCE_KR16_CONV") &&
-                !getenv("FYNHIP_FORCE_KSPLIT") && !getenv("FYNHIP_CONV_TILE") && !getenv("FYNHIP_CONV_KC") && !getenv("FYNHIP_CONV_KC_MAX") && !getenv("FYNHIP_CONV_PD"))
+                !net->sw.get("FYNHIP_NO_P16_CONV") && !net->sw.get("FYNHIP_NO_D16_CONV") && !net->sw.get("FYNHIP_FORCE_P16_CONV") && !net->sw.get("FYNHIP_FORCE_KR16_CONV") &&
+                !net->sw.get("FYNHIP_FORCE_KSPLIT") && !net->sw.get("FYNHIP_CONV_TILE") && !net->sw.get("FYNHIP_CONV_KC") && !net->sw.get("FYNHIP_CONV_KC_MAX") && !net->sw.get("FYNHIP_CONV_PD"))
                 setup_d16(in_v, out_v, res_v, res_relu, res_scale);
             // the same kernel's K x K form for a first layer on at most four channels (3x3, 5x5, 7x7)
             if (!p16 && !frac_shift && !clamp && same_storage && oc % 4 == 0 && oc >= 8 && oh * ow >= 256 && conv_d16_small_supported(k, dil, in_v.cp, oc, out_v.cp) &&
-                (!res_v || (res_v->cp >= out_v.cp && res_v->cp % 8 == 0)) && !getenv("FYNHIP_NO_P16_CONV") && !getenv("FYNHIP_NO_D16_CONV") && !getenv("FYNHIP_FORCE_P16_CONV") &&
-                !getenv("FYNHIP_FORCE_KSPLIT") && !getenv("FYNHIP_CONV_TILE") && !getenv("FYNHIP_CONV_KC") && !getenv("FYNHIP_CONV_KC_MAX") && !getenv("FYNHIP_CONV_PD"))
+                (!res_v || (res_v->cp >= out_v.cp && res_v->cp % 8 == 0)) && !net->sw.get("FYNHIP_NO_P16_CONV") && !net->sw.get("FYNHIP_NO_D16_CONV") && !net->sw.get("FYNHIP_FORCE_P16_CONV") &&
+                !net->sw.get("FYNHIP_FORCE_KSPLIT") && !net->sw.get("FYNHIP_CONV_TILE") && !net->sw.get("FYNHIP_CONV_KC") && !net->sw.get("FYNHIP_CONV_KC_MAX") && !net->sw.get("FYNHIP_CONV_PD"))
                 setup_d16(in_v, out_v, res_v, res_relu, res_scale);
         }
         if (direct) {
@@ -2127,6 +2127,7 @@ class DwConvLayer : public Layer {
         p.dil = dil; p.stride = stride;
         p.res_relu = (d.flags & FYN_FLAG_RELU_ON_RESIDUAL) ? 1 : 0;
         p.res_scale = ((d.flags & FYN_FLAG_BATCHNORM_ON_RESIDUAL) && (d.flags & FYN_FLAG_POST_BATCHNORM)) ? 1 : 0;
+        p.no_strips = net->sw.on("FYNHIP_NO_DW_STRIPS") ? 1 : 0;
         p.act = act();
         const int cp = p.out.cp;
         w_dev = static_cast<float*>(net->dev_alloc(9 * (size_t)cp * sizeof(float)));
@@ -2174,17 +2175,17 @@ class DwConvLayer : public Layer {
 // when the fused way is taken, so the fusion is tied to buffer reuse (a caller who switches reuse off wants every
 // layer's tensor) and is left out of passes that time or dump single layers.
 void fuse_depthwise_layers(Net* net) {
-    if (getenv("FYNHIP_NO_DW_FUSION") || !net->reuse_buffers) return;
+    if (net->sw.get("FYNHIP_NO_DW_FUSION") || !net->reuse_buffers) return;
     std::map<int, int> readers;
     for (auto& kv : net->layers)
         for (int t : kv.second->in)
             if (t >= 0) readers[t]++;
-    const char* at = getenv("FYNHIP_AUTOTUNE");
+    const char* at = net->sw.get("FYNHIP_AUTOTUNE");
     // First the other half of the block: a 1x1 layer (expand) whose only reader is the depthwise layer.  Every expanded
     // channel depends on the 1x1 layer's input only, so a workgroup can compute the window of the expanded tensor that
     // its tile of the depthwise layer needs (conv_e16dw_kernel); the expanded tensor is then never written.
     for (auto& kv : net->layers) {
-        if (getenv("FYNHIP_NO_EDW_FUSION")) break;
+        if (net->sw.get("FYNHIP_NO_EDW_FUSION")) break;
         DwConvLayer* dw = dynamic_cast<DwConvLayer*>(kv.second.get());
         if (!dw || dw->dil != 1 || (dw->stride != 1 && dw->stride != 2) || dw->p.res.ptr || dw->p.in.cp % 8 != 0 || dw->p.in.cp != dw->p.out.cp || dw->p.in.f16 != dw->p.out.f16)
             continue;
@@ -2228,10 +2229,10 @@ void fuse_depthwise_layers(Net* net) {
         snprintf(key, sizeof(key), "edw:%d:%dto%d:%dx%d:s%d", q.f16, in_v.cp, ex->oc, ex->oh, ex->ow, dw->stride);
         // (q.wm = 2: a workgroup per 16 expanded channels instead of 64, for layers with few tiles; by rule when nothing is timed)
         q.wm = (q.tiles_x * q.tiles_y * ((q.dw_cp + 63) / 64) < 128) ? 2 : 0;
-        if (const char* e = getenv("FYNHIP_EDW_NARROW")) q.wm = atoi(e) ? 2 : 0;
+        if (const char* e = net->sw.get("FYNHIP_EDW_NARROW")) q.wm = atoi(e) ? 2 : 0;
         int cached[3] = {0, 0, 0};
-        if (getenv("FYNHIP_FORCE_DW_FUSION") || getenv("FYNHIP_EDW_NARROW")) {
-        } else if (tune_cache_triple(key, cached)) {
+        if (net->sw.get("FYNHIP_FORCE_DW_FUSION") || net->sw.get("FYNHIP_EDW_NARROW")) {
+        } else if (tune_cache_triple(net, key, cached)) {
             pick = cached[0] != 0;
             q.wm = cached[1];
         } else if (!(at && at[0] == '0')) {
@@ -2251,14 +2252,14 @@ void fuse_depthwise_layers(Net* net) {
                     launch_dwconv3x3(dw->p, net->stream);
                 }, 10));
             }
-            if (getenv("FYNHIP_TUNE_VERBOSE"))
+            if (net->sw.get("FYNHIP_TUNE_VERBOSE"))
                 fprintf(stderr, "[tune] 1x1 %d to %d at %dx%d + depthwise 3x3 (step %d): one launch (blocks of %d channels) %.1f us, two %.1f us\n", in_v.cp, ex->oc, ex->oh,
                         ex->ow, dw->stride, best_wm == 2 ? 16 : 64, t_fused * 1e3f, t_two * 1e3f);
             // (a near tie goes to the single launch: it leaves the expanded tensor unwritten, which a timing loop that
             // finds everything in the caches does not reward)
             pick = t_fused < t_two * 1.05f;
             q.wm = best_wm;
-            tune_cache_store_triple(key, pick ? 1 : 0, best_wm, 0);
+            tune_cache_store_triple(net, key, pick ? 1 : 0, best_wm, 0);
         }
         if (!pick) {
             net->dev_free(wp);
@@ -2300,8 +2301,8 @@ void fuse_depthwise_layers(Net* net) {
         bool pick = true;
         char key[200];
         snprintf(key, sizeof(key), "dwpw:%d:%dx%dx%d:s%d:to%d:fm%d:d%d", q.f16, dw->p.in.cp, dw->p.in.h, dw->p.in.w, dw->stride, pw->oc, q.wm, pw->d16 ? 1 : 0);
-        if (getenv("FYNHIP_FORCE_DW_FUSION")) {
-        } else if (tune_cache_flag(key, &pick)) {
+        if (net->sw.get("FYNHIP_FORCE_DW_FUSION")) {
+        } else if (tune_cache_flag(net, key, &pick)) {
         } else if (!(at && at[0] == '0')) {
             float t_fused = 1e30f, t_two = 1e30f;
             for (int rep = 0; rep < 3; rep++) {
@@ -2313,11 +2314,11 @@ void fuse_depthwise_layers(Net* net) {
                     if (pw->launch_own(net->stream) != 0) fail(FYN_ERR_DEVICE, "1x1 convolution launch failed while tuning");
                 }, 10));
             }
-            if (getenv("FYNHIP_TUNE_VERBOSE"))
+            if (net->sw.get("FYNHIP_TUNE_VERBOSE"))
                 fprintf(stderr, "[tune] depthwise 3x3 (step %d) on %d channels at %dx%d + 1x1 to %d: one launch %.1f us, two %.1f us\n", dw->stride, dw->p.in.cp,
                         dw->p.in.h, dw->p.in.w, pw->oc, t_fused * 1e3f, t_two * 1e3f);
             pick = t_fused < t_two;
-            tune_cache_store_flag(key, pick);
+            tune_cache_store_flag(net, key, pick);
         }
         if (!pick) continue;
         pw->dw_fused = true;
@@ -2347,7 +2348,7 @@ static ConvLayer* projection_of(Net* net, ConvLayer* c) {
 // Before buffers are assigned: the input of such a projection stays whole until the layer that may compute it has run
 // (a few more buffers in networks with such pairs, whether the pair is joined in the end or not).
 void keep_projection_inputs(Net* net) {
-    if (getenv("FYNHIP_NO_PROJECTION_FUSION") || !net->reuse_buffers) return;
+    if (net->sw.get("FYNHIP_NO_PROJECTION_FUSION") || !net->reuse_buffers) return;
     for (auto& kv : net->layers) {
         ConvLayer* c = dynamic_cast<ConvLayer*>(kv.second.get());
         ConvLayer* pr = projection_of(net, c);
@@ -2363,8 +2364,8 @@ void keep_projection_inputs(Net* net) {
 // activation on fetch, no activation on the residual, the projection's input still whole when the reader runs, and a
 // compiled variant for the joint chunk count; timed against the two launches.
 void fuse_projection_layers(Net* net) {
-    if (getenv("FYNHIP_NO_PROJECTION_FUSION") || getenv("FYNHIP_NO_P16_CONV") || getenv("FYNHIP_NO_KR16_CONV") || !net->reuse_buffers) return;
-    const char* at = getenv("FYNHIP_AUTOTUNE");
+    if (net->sw.get("FYNHIP_NO_PROJECTION_FUSION") || net->sw.get("FYNHIP_NO_P16_CONV") || net->sw.get("FYNHIP_NO_KR16_CONV") || !net->reuse_buffers) return;
+    const char* at = net->sw.get("FYNHIP_AUTOTUNE");
     for (auto& kv : net->layers) {
         ConvLayer* c = dynamic_cast<ConvLayer*>(kv.second.get());
         ConvLayer* pr = projection_of(net, c);
@@ -2432,8 +2433,8 @@ void fuse_projection_layers(Net* net) {
         char key[200];
         snprintf(key, sizeof(key), "pj:%d:%dand%dto%d:%dx%d:s%d", q.f16, v1.cp, v2.cp, c->oc, c->oh, c->ow, pr->stride);
         int cached[3] = {0, 0, 0};
-        if (getenv("FYNHIP_FORCE_PROJECTION_FUSION")) {
-        } else if (tune_cache_triple(key, cached)) {
+        if (net->sw.get("FYNHIP_FORCE_PROJECTION_FUSION")) {
+        } else if (tune_cache_triple(net, key, cached)) {
             win = cached[0] != 0;
             for (size_t i = 0; i < cands.size(); i++)
                 if (cands[i].wm == cached[1]) pick = (int)i;
@@ -2451,11 +2452,11 @@ void fuse_projection_layers(Net* net) {
                     c->run(net->stream);
                 }, 10));
             }
-            if (getenv("FYNHIP_TUNE_VERBOSE"))
+            if (net->sw.get("FYNHIP_TUNE_VERBOSE"))
                 fprintf(stderr, "[tune] 1x1 on %d channels + 1x1 projection on %d (step %d) to %d at %dx%d: one launch %.1f us, two %.1f us\n", v1.cp, v2.cp, pr->stride, c->oc,
                         c->oh, c->ow, t_fused * 1e3f, t_two * 1e3f);
             win = t_fused < t_two;
-            tune_cache_store_triple(key, win ? 1 : 0, cands[pick].wm, 0);
+            tune_cache_store_triple(net, key, win ? 1 : 0, cands[pick].wm, 0);
         }
         if (!win) {
             net->dev_free(wp); net->dev_free(sc); net->dev_free(bi);
@@ -2522,7 +2523,7 @@ class TransConvLayer : public Layer {
             }
         group = tune_mfma_group(net, subconvs, in_v, out_v, d.in_channels, oc, act(), scale_dev, bias_dev);
         if (tconv_p16_supported(k, crop, in_v.cp, in_v.pad, oc, out_v.cp, out_v.f16 != 0) && in_v.f16 == out_v.f16 && d.in_channels == in_v.cp &&
-            !getenv("FYNHIP_NO_P16_CONV"))
+            !net->sw.get("FYNHIP_NO_P16_CONV"))
             setup_p16(in_v, out_v);
         set_up = true;
         setup_ranges();
@@ -2546,7 +2547,7 @@ class TransConvLayer : public Layer {
         q.act = act();
         q.in_amax = tin(0).amax;   // (timed in the form the frame will run)
         int want_h = 0, want_w = 0, want_wm = 0;   // FYNHIP_P16_TILE=h,w[,wm] (tests): that combination
-        if (const char* e = getenv("FYNHIP_P16_TILE")) sscanf(e, "%d,%d,%d", &want_h, &want_w, &want_wm);
+        if (const char* e = net->sw.get("FYNHIP_P16_TILE")) sscanf(e, "%d,%d,%d", &want_h, &want_w, &want_wm);
         std::vector<ConvP16Params> cands;
         for (int i = 0; i < tconv_p16_tile_count(); i++) {
             int th, tw, wm;
@@ -2568,13 +2569,13 @@ class TransConvLayer : public Layer {
         const size_t halves = ((size_t)q.cin_chunks * 9 + 8) * q.mfrags * (q.f16 ? 1 : 3) * 64 * 8;
         p16_wpack_dev = net->dev_alloc(halves * 2, true);
         for (ConvP16Params& c : cands) c.wpack = p16_wpack_dev;
-        const bool always = getenv("FYNHIP_FORCE_P16_CONV") != nullptr;
-        const char* at = getenv("FYNHIP_AUTOTUNE");
+        const bool always = net->sw.get("FYNHIP_FORCE_P16_CONV") != nullptr;
+        const char* at = net->sw.get("FYNHIP_AUTOTUNE");
         int pick = 0;
         char key[160];
         snprintf(key, sizeof(key), "tp16:%dx%d:%dx%d:cp%d:h%d", d.in_channels, oc, d.height, d.width, in_v.cp, q.f16);
         int cached[3] = {0, 0, 0};
-        if (!want_h && tune_cache_triple(key, cached)) {
+        if (!want_h && tune_cache_triple(net, key, cached)) {
             pick = -1;
             if (cached[0] || always)
                 for (size_t i = 0; i < cands.size(); i++)
@@ -2591,11 +2592,11 @@ class TransConvLayer : public Layer {
                 }
                 t_other = std::min(t_other, time_group(net, group, 10));
             }
-            if (getenv("FYNHIP_TUNE_VERBOSE"))
+            if (net->sw.get("FYNHIP_TUNE_VERBOSE"))
                 fprintf(stderr, "[tune] transposed 3x3: 16-position fragments (%dx%d tiles, %d channel groups) %.1f us, general kernel %.1f us\n",
                         cands[pick].tile_h, cands[pick].tile_w, cands[pick].wm, best * 1e3f, t_other * 1e3f);
             const bool win = best < t_other;
-            if (!want_h) tune_cache_store_triple(key, win ? 1 : 0, cands[pick].tile_h * 1000 + cands[pick].tile_w, cands[pick].wm);
+            if (!want_h) tune_cache_store_triple(net, key, win ? 1 : 0, cands[pick].tile_h * 1000 + cands[pick].tile_w, cands[pick].wm);
             if (!win && !always) pick = -1;
         }
         if (pick >= 0) {
@@ -2885,7 +2886,7 @@ class BatchNormLayer : public Layer {
 // front of most blocks).  The input tensor must still hold its values when the last reader runs: no tensor produced
 // between the batch-norm layer and that reader may live in the same buffer.
 void fuse_batchnorm_layers(Net* net) {
-    if (getenv("FYNHIP_NO_BN_FUSION") || !net->reuse_buffers) return;
+    if (net->sw.get("FYNHIP_NO_BN_FUSION") || !net->reuse_buffers) return;
     for (auto& kv : net->layers) {
         BatchNormLayer* bn = dynamic_cast<BatchNormLayer*>(kv.second.get());
         if (!bn || bn->p.res.ptr || bn->p.act.kind != ACT_NONE) continue;

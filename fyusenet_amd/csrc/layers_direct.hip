@@ -394,7 +394,7 @@ static void launch_dw_row(const DwConvParams& p, hipStream_t s) {
 // strips of `rows` output rows per thread, when the image is tall enough to leave the chip enough threads
 template <typename T, int V>
 static bool launch_dw_col(const DwConvParams& p, hipStream_t s) {
-    if (getenv("FYNHIP_NO_DW_STRIPS")) return false;
+    if (p.no_strips) return false;
     const size_t per_row = (size_t)((p.out.w + 3) / 4) * (p.out.cp / V);
     int rows = 16;
     while (rows > 2 && per_row * ((p.out.h + rows - 1) / rows) < 256 * 256 * 2) rows /= 2;   // at least two waves per SIMD of work
