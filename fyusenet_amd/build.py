@@ -7,7 +7,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.environ.get("FYNHIP_BUILD_LIB", os.path.join(HERE, "libfynhip.so"))  # experimental builds go elsewhere
 CONV_PARTS = 8  # conv_mfma.hip is compiled this many times, each time with a slice of the tile table
-SOURCES = ["layers_direct.hip", "conv_rows.hip", "conv_h16.hip", "conv_d16.hip", "engine.cpp", "layers.cpp", "api.cpp"]
+SOURCES = ["layers_direct.hip", "conv_rows.hip", "conv_h16.hip", "conv_d16.hip", "engine.cpp", "conv_plan.cpp", "fusion.cpp", "layers.cpp", "api.cpp"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 EXTRA = os.environ.get("FYNHIP_EXTRA_FLAGS", "").split()  # e.g. -D switches of experimental builds
 FLAGS = [

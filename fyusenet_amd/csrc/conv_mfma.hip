@@ -33,12 +33,6 @@
 #include "kernels.h"
 #include "range.h"
 
-// Timing-study builds (-DFYN_CONV_TRACE): wave 0 of every workgroup records the shader clock at phase boundaries.
-#ifdef FYN_CONV_TRACE
-#define FYN_TRACE(slot) do { if (tid == 0 && (slot) < 16) p.trace[((size_t)blockIdx.y * gridDim.x + blockIdx.x) * 16 + (slot)] = clock64(); } while (0)
-#else
-#define FYN_TRACE(slot) do { } while (0)
-#endif
 
 namespace fynhip {
 
@@ -232,7 +226,6 @@ __device__ __forceinline__ void conv_mfma_body(const ConvMfmaParams& p, unsigned
         const int per = nblk >> 3;
         if (bid < (per << 3)) bid = (bid & 7) * per + (bid >> 3);
     }
-    FYN_TRACE(0);
     // value ranges (range.h): read the input tensor's record (the records in this launch's care are cleared by the
     // kernel entry points)
     float in_scale = 1.f, inv_in_scale = 1.f;   // (set once the first tile's loads are on their way)
@@ -412,7 +405,6 @@ __device__ __forceinline__ void conv_mfma_body(const ConvMfmaParams& p, unsigned
         stage_rest(chunk0, sbase);
     }
     __syncthreads();
-    FYN_TRACE(1);
 
     // ---- main loop: channel chunks, each nsteps k16 steps in groups of PD.  B fragments of step t+1 are
     //      read from LDS while the MFMAs of step t run; the next chunk's tile is fetched from HBM/L2 at the
@@ -491,7 +483,6 @@ __device__ __forceinline__ void conv_mfma_body(const ConvMfmaParams& p, unsigned
                     for (int pl = 0; pl < NPL; pl++) b_buf[0][fn][pl] = load_b_frag<KC>(cur + pl * p.plane + boff[fn], ao);
                 for (int t0 = 0; t0 < nsub; t0 += UNR) run_group(t0);
             }
-            FYN_TRACE(2 + 2 * (chunk - chunk0));
             if (more_chunks) {
                 unsigned char* nxt = sbase + ((chunk - chunk0 + 1) & 1) * bufsz;
                 if (!SPEC) {
@@ -500,7 +491,6 @@ __device__ __forceinline__ void conv_mfma_body(const ConvMfmaParams& p, unsigned
                 }
                 __syncthreads();  // everyone is done reading `cur` and writing `nxt`
                 cur = nxt;
-                FYN_TRACE(3 + 2 * (chunk - chunk0));
             }
         }
     }
@@ -594,7 +584,6 @@ __device__ __forceinline__ void conv_mfma_body(const ConvMfmaParams& p, unsigned
         }
     }
     if (!consumer) return;
-    FYN_TRACE(14);
     const float* tr0 = reinterpret_cast<const float*>(lds) + ((wave & 3) % (WM * WN)) * (FN * 32 * ROWF);   // K group 0's area of this sub-tile
     constexpr int TRK = WM * WN * FN * 32 * ROWF;     // floats between the areas of consecutive K groups
     auto row_from_lds = [&](int fn, int it) {
@@ -664,9 +653,7 @@ __device__ __forceinline__ void conv_mfma_body(const ConvMfmaParams& p, unsigned
                 for (int i = 0; i < 4; i++) rres[fn][it][i] = r[i];
             }
         }
-    FYN_TRACE(9);
     if constexpr (WK == 1) acc_to_lds();
-    FYN_TRACE(10);
     f32x4_t a4[FN][ITW];
 #pragma unroll
     for (int fn = 0; fn < FN; fn++)
@@ -691,7 +678,6 @@ __device__ __forceinline__ void conv_mfma_body(const ConvMfmaParams& p, unsigned
     for (int fn = 0; fn < FN; fn++)
 #pragma unroll
         for (int it = 0; it < ITW; it++) asm volatile("" : "+v"(a4[fn][it]));
-    FYN_TRACE(11);
     if (SPLIT && p.out_amax) {
         float vmax = 0.f;
 #pragma unroll
@@ -716,7 +702,6 @@ __device__ __forceinline__ void conv_mfma_body(const ConvMfmaParams& p, unsigned
                 *reinterpret_cast<half4_t*>(reinterpret_cast<_Float16*>(out) + obase[fn][it]) = hv;
             }
         }
-    FYN_TRACE(15);
 }
 
 // Entry points: one convolution per launch (parameters by value), or up to four sub-convolutions of one layer
@@ -945,23 +930,6 @@ int ensure_lds(const void* fn, size_t lds_bytes) {
     return 0;
 }
 
-#ifdef FYN_CONV_TRACE
-static long long* trace_buffer() {
-    static long long* dev = nullptr;
-    if (!dev && hipMalloc(&dev, sizeof(long long) * 16 * 65536) != hipSuccess) return nullptr;
-    return dev;
-}
-static void trace_dump(hipStream_t s, long long* dev, size_t blocks) {
-    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
-    (void)hipStreamIsCapturing(s, &cap);
-    const char* path = cap == hipStreamCaptureStatusNone ? getenv("FYNHIP_TRACE_DUMP") : nullptr;
-    if (!path) return;
-    std::vector<long long> h(blocks * 16);
-    if (hipStreamSynchronize(s) == hipSuccess && hipMemcpy(h.data(), dev, h.size() * 8, hipMemcpyDeviceToHost) == hipSuccess) {
-        if (FILE* f = fopen(path, "wb")) { fwrite(h.data(), 8, h.size(), f); fclose(f); }
-    }
-}
-#endif
 
 int launch_conv_mfma(const ConvVariant& v, const ConvMfmaParams& p_in, size_t lds_bytes, hipStream_t s) {
     conv_kernel_fn fn = pick_kernel(v).single;
@@ -970,15 +938,7 @@ int launch_conv_mfma(const ConvVariant& v, const ConvMfmaParams& p_in, size_t ld
     if (int rc = ensure_lds(reinterpret_cast<const void*>(fn), lds_bytes)) return rc;
     const int blocks = blocks_of(p_in);
     const dim3 threads(v.fm * v.fn >= 2 ? 512 : 256);
-#ifdef FYN_CONV_TRACE
-    ConvMfmaParams p = p_in;
-    p.trace = trace_buffer();
-    if (!p.trace || blocks > 65536) return -6;
-    hipLaunchKernelGGL(fn, dim3(blocks), threads, lds_bytes, s, p);
-    trace_dump(s, p.trace, blocks);
-#else
     hipLaunchKernelGGL(fn, dim3(blocks), threads, lds_bytes, s, p_in);
-#endif
     return hipGetLastError() == hipSuccess ? 0 : -3;
 }
 
@@ -994,16 +954,7 @@ int launch_conv_mfma_multi(const ConvVariant& v, const ConvMfmaMulti& m_in, size
     }
     if (int rc = ensure_lds(reinterpret_cast<const void*>(fn), lds_bytes)) return rc;
     const dim3 threads(v.fm * v.fn >= 2 ? 512 : 256);
-#ifdef FYN_CONV_TRACE
-    ConvMfmaMulti m = m_in;
-    long long* tb = trace_buffer();
-    if (!tb || (size_t)blocks * m.nsub > 65536) return -6;
-    for (int i = 0; i < m.nsub; i++) m.sub[i].trace = tb;
-    hipLaunchKernelGGL(fn, dim3(blocks, m.nsub), threads, lds_bytes, s, m);
-    trace_dump(s, tb, (size_t)blocks * m.nsub);
-#else
     hipLaunchKernelGGL(fn, dim3(blocks, m_in.nsub), threads, lds_bytes, s, m_in);
-#endif
     return hipGetLastError() == hipSuccess ? 0 : -3;
 }
 #endif  // FYN_CONV_PART == 0

@@ -30,15 +30,6 @@
 #include "p16_common.h"
 #include "range.h"
 
-// Timing-study builds (-DFYN_P16_TRACE): wave 0 and wave 4 of every workgroup record the shader clock at phase boundaries.
-#ifdef FYN_P16_TRACE
-#include <cstdio>
-#include <cstdlib>
-#include <vector>
-#define FYN_PTRACE(slot) do { if (lane == 0 && (wave & 3) == 0 && (slot) < 32) p.trace[((size_t)blockIdx.x * 2 + 1 - (wave >> 2)) * 32 + (slot)] = clock64(); } while (0)
-#else
-#define FYN_PTRACE(slot) do { } while (0)
-#endif
 
 namespace fynhip {
 
@@ -418,7 +409,6 @@ __global__ __launch_bounds__(512) void conv_p16_kernel(const ConvP16Params p) {
     }
 
     // ---------------------------------------------------------------------- MFMA waves
-    FYN_PTRACE(0);
     const int mq = lane & 15, kq = lane >> 4;
     const int mw = (wave - 4) % WM;   // this wave's 32 output channels of the workgroup's CPB
     const int wn = (wave - 4) / WM;   // ... and its tile of positions
@@ -529,9 +519,7 @@ __global__ __launch_bounds__(512) void conv_p16_kernel(const ConvP16Params p) {
         }
     };
 
-    FYN_PTRACE(1);
     lds_barrier();   // the first stage is staged
-    FYN_PTRACE(2);
     half8_t b[C8 ? 1 : FN][NPL];
     half8_t b0[C8 ? FN : 1];
     i32x8_t b1[C8 ? FN : 1];
@@ -556,14 +544,10 @@ __global__ __launch_bounds__(512) void conv_p16_kernel(const ConvP16Params p) {
         // (an even number of chunks: a tile is whole pairs of stages)
         for (;;) {
             p16_stage_c8<G, 0>(acc, a0, a2, b0, b1, bbase, lds, wnext, wbase, wend, wstep, wlane);
-            FYN_PTRACE(3 + (c < 12 ? c : 12));
             p16_stage_c8<G, 1>(acc, a0, a2, b0, b1, bbase, lds, wnext, wbase, wend, wstep, wlane);
-            FYN_PTRACE(4 + (c < 11 ? c : 11));
             c += 2;
             if (c == nchunks) {
-                FYN_PTRACE(29);
                 finish_tile(tile);
-                FYN_PTRACE(30);
                 c = 0; tile += p.pos_groups;
                 if (tile >= ntiles) break;
                 zero_acc();
@@ -572,21 +556,15 @@ __global__ __launch_bounds__(512) void conv_p16_kernel(const ConvP16Params p) {
     } else {
     for (;;) {
         p16_stage<G, 0>(acc, a_q, b, bbase, lds, wnext, wbase, wend, wstep, wlane);
-        FYN_PTRACE(3 + (c < 12 ? c : 12));
         if (++c == nchunks) {
-            FYN_PTRACE(29);
             finish_tile(tile);
-            FYN_PTRACE(30);
             c = 0; tile += p.pos_groups;
             if (tile >= ntiles) break;
             zero_acc();
         }
         p16_stage<G, 1>(acc, a_q, b, bbase, lds, wnext, wbase, wend, wstep, wlane);
-        FYN_PTRACE(3 + (c < 12 ? c : 12));
         if (++c == nchunks) {
-            FYN_PTRACE(29);
             finish_tile(tile);
-            FYN_PTRACE(30);
             c = 0; tile += p.pos_groups;
             if (tile >= ntiles) break;
             zero_acc();
@@ -594,7 +572,6 @@ __global__ __launch_bounds__(512) void conv_p16_kernel(const ConvP16Params p) {
     }
     }
     if (p.out_amax) range_publish_waves(p.out_amax, vmax, range_box, 4);
-    FYN_PTRACE(31);
 }
 
 // ---------------------------------------------------------------------------------------------------------------
@@ -1845,27 +1822,6 @@ int P16_NAME(launch_conv_p16)(const ConvP16Params& p, hipStream_t s) {
     if (lds_bytes > 160 * 1024) return -2;
     const p16_fn fn = p16_uses_fp8(p) ? e->fn_c8 : e->fn;
     if (ensure_lds(reinterpret_cast<const void*>(fn), lds_bytes) != 0) return -2;
-#ifdef FYN_P16_TRACE
-    {
-        static long long* dev = nullptr;
-        const size_t n = (size_t)p.pos_groups * p.cout_blocks * 64;
-        if (!dev && hipMalloc(&dev, sizeof(long long) * 65536 * 64) != hipSuccess) return -6;
-        ConvP16Params q = p;
-        q.trace = dev;
-        if (const char* e = getenv("FYNHIP_P16_CHUNKS")) q.cin_chunks = atoi(e);   // (timing study: fewer chunks, wrong results)
-        hipLaunchKernelGGL(fn, dim3(p.pos_groups * p.cout_blocks), dim3(512), lds_bytes, s, q);
-        hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
-        (void)hipStreamIsCapturing(s, &cap);
-        const char* path = cap == hipStreamCaptureStatusNone ? getenv("FYNHIP_TRACE_DUMP") : nullptr;
-        if (path) {
-            std::vector<long long> h(n);
-            if (hipStreamSynchronize(s) == hipSuccess && hipMemcpy(h.data(), dev, n * 8, hipMemcpyDeviceToHost) == hipSuccess) {
-                if (FILE* f = fopen(path, "wb")) { fwrite(h.data(), 8, n, f); fclose(f); }
-            }
-        }
-        return hipGetLastError() == hipSuccess ? 0 : -3;
-    }
-#endif
     hipLaunchKernelGGL(fn, dim3(p.pos_groups * p.cout_blocks), dim3(512), lds_bytes, s, p);
     return hipGetLastError() == hipSuccess ? 0 : -3;
 }

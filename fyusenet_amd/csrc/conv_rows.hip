@@ -19,15 +19,6 @@
 #include "kernels.h"
 #include "range.h"
 
-// Timing-study builds (-DFYN_ROWS_TRACE): wave 0 and wave 4 of every workgroup record the shader clock at phase boundaries.
-#ifdef FYN_ROWS_TRACE
-#include <cstdio>
-#include <cstdlib>
-#include <vector>
-#define FYN_RTRACE(slot) do { if (lane == 0 && (wave & 3) == 0 && (slot) < 32) p.trace[((size_t)blockIdx.x * 2 + (wave >> 2)) * 32 + (slot)] = clock64(); } while (0)
-#else
-#define FYN_RTRACE(slot) do { } while (0)
-#endif
 
 namespace fynhip {
 
@@ -160,7 +151,6 @@ __global__ __launch_bounds__(512) void conv_rows_kernel(const ConvRowsParams p) 
     const int nbatches = (rows_total + 3) >> 2;
     auto rows_of = [&](int b) { return min(4, rows_total - 4 * b); };
     Batch nxt;   // the batch in flight (staging waves)
-    FYN_RTRACE(0);
     if (!mfma_wave) {
         // all loads of the first rounds' rows are issued before the first conversion
         Batch first[NB0];
@@ -182,9 +172,7 @@ __global__ __launch_bounds__(512) void conv_rows_kernel(const ConvRowsParams p) 
 #pragma unroll
             for (int pl = 0; pl < NPL; pl++) a_reg[t][pl] = w[(t * NPL + pl) * 64 + lane];
     }
-    FYN_RTRACE(1);
     lds_barrier();
-    FYN_RTRACE(2);
 
     // per-lane byte offsets of the B fragments inside a ring row: column fn*32 + lane%32, chunk 2*sub + lane/32
     int boff[CS][FN];
@@ -209,12 +197,9 @@ __global__ __launch_bounds__(512) void conv_rows_kernel(const ConvRowsParams p) 
         for (int g = 0; g < nrounds; g++) {
             // write batch NB0 + g (fetched a round ago; no round up to g reads its ring slots), fetch the next one
             store(nxt);
-            FYN_RTRACE(3 + 3 * g);
             const int b = NB0 + g + 1;
             fetch(nxt, 4 * b, b < nbatches ? rows_of(b) : 0);
-            FYN_RTRACE(4 + 3 * g);
             lds_barrier();
-            FYN_RTRACE(5 + 3 * g);
         }
         return;
     }
@@ -259,7 +244,6 @@ __global__ __launch_bounds__(512) void conv_rows_kernel(const ConvRowsParams p) 
                         __builtin_amdgcn_sched_barrier(0);
                     }
                 }
-                FYN_RTRACE(3 + 3 * g);
                 // accumulators -> this wave's area [column][virtual channel]: a lane holds column lane%32 of each
                 // fragment and rows 8*(r/4) + 4*(lane/32) + r%4
 #pragma unroll
@@ -324,9 +308,7 @@ __global__ __launch_bounds__(512) void conv_rows_kernel(const ConvRowsParams p) 
                 }
             }
         }
-        FYN_RTRACE(4 + 3 * g);
         lds_barrier();   // the round's rows are consumed, the next round's rows are in the ring
-        FYN_RTRACE(5 + 3 * g);
     }
     if (SPLIT && p.out_amax) range_publish_waves(p.out_amax, vmax, range_box, 4);
 }
@@ -366,26 +348,6 @@ int launch_conv_rows(const ConvRowsParams& p, bool f16, hipStream_t s) {
     const size_t lds_bytes = conv_rows_lds_bytes(p, f16);
     if (lds_bytes > 160 * 1024) return -2;
     if (ensure_lds(reinterpret_cast<const void*>(fn), lds_bytes) != 0) return -2;
-#ifdef FYN_ROWS_TRACE
-    {
-        static long long* dev = nullptr;
-        const size_t n = (size_t)p.strips * p.row_blocks * 64;
-        if (!dev && hipMalloc(&dev, sizeof(long long) * 65536 * 64) != hipSuccess) return -6;
-        ConvRowsParams q = p;
-        q.trace = dev;
-        hipLaunchKernelGGL(fn, dim3(p.strips * p.row_blocks), dim3(512), lds_bytes, s, q);
-        hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
-        (void)hipStreamIsCapturing(s, &cap);
-        const char* path = cap == hipStreamCaptureStatusNone ? getenv("FYNHIP_TRACE_DUMP") : nullptr;
-        if (path) {
-            std::vector<long long> h(n);
-            if (hipStreamSynchronize(s) == hipSuccess && hipMemcpy(h.data(), dev, n * 8, hipMemcpyDeviceToHost) == hipSuccess) {
-                if (FILE* f = fopen(path, "wb")) { fwrite(h.data(), 8, n, f); fclose(f); }
-            }
-        }
-        return hipGetLastError() == hipSuccess ? 0 : -3;
-    }
-#endif
     hipLaunchKernelGGL(fn, dim3(p.strips * p.row_blocks), dim3(512), lds_bytes, s, p);
     return hipGetLastError() == hipSuccess ? 0 : -3;
 }

@@ -94,9 +94,6 @@ struct ConvMfmaParams {
     unsigned* out_amax;
     unsigned* reset[4];
     int nreset;
-#ifdef FYN_CONV_TRACE
-    long long* trace;    // timing-study builds only: 16 timestamps per workgroup
-#endif
     Act act;
 };
 
@@ -154,9 +151,6 @@ struct ConvRowsParams {
     unsigned* out_amax;
     unsigned* reset[4];
     int nreset;
-#ifdef FYN_ROWS_TRACE
-    long long* trace;     // timing-study builds only: 32 timestamps per workgroup and role
-#endif
     Act act;
 };
 int ensure_lds(const void* fn, size_t lds_bytes);   // 0, or -2 when the device refuses the size (conv_mfma.hip)
@@ -196,9 +190,6 @@ struct ConvP16Params {
     unsigned* out_amax;
     unsigned* reset[4];
     int nreset;
-#ifdef FYN_P16_TRACE
-    long long* trace;     // timing-study builds only: 32 timestamps per workgroup and role
-#endif
     Act act;
     // A depthwise 3x3 layer computed inside the staging of a 1x1 launch of the K-resident form (dw_in null: none): the
     // layer's input tensor, its weights [9][dw_cp] and folded scale / bias [dw_cp], the stored coordinate of tap (0,0)
