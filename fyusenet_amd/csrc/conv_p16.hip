@@ -778,7 +778,14 @@ struct GeoC4 {
     static constexpr int NS = ((NPAIR + 3) / 4 + 2) / 3 * 3;          // steps per stage (two stages are whole turns of the weight ring)
     static constexpr int PIX = 8;                                     // bytes per staged pixel and plane
     static constexpr int ROW_PITCH = (HW * PIX + 15) / 16 * 16 + 16;
-    static constexpr int PLANE = HH * ROW_PITCH;
+    // A plane is staged twice, the second copy eight bytes further on: the two pixels of a tap pair are then 16 aligned
+    // bytes in one of the copies whatever the parity of the pair's first pixel, and a B fragment is one 16-byte LDS read
+    // (with 8-byte reads the four tap pairs of a step meet in the same banks and the reads, not the MFMAs, set the pace:
+    // 59 % MFMA issue inside the step loop).  The copies lie 64 bytes apart modulo the 128 of the banks: of eight
+    // neighbouring positions the even ones read the first copy and the odd ones the second, all banks once.
+    static constexpr int COPY = HH * ROW_PITCH;
+    static constexpr int COPY2 = (COPY + 127) / 128 * 128 + 48;        // offset of the second copy (its pixel x at COPY2 + 8 + 8 x)
+    static constexpr int PLANE = COPY2 + COPY + 16;
     static constexpr int BUF = NPL * PLANE;
     static constexpr int NPOS = TH * TW, FN = NPOS / 16;
     static constexpr int NITEMS = HH * HW;                            // staging items: pixels
@@ -833,6 +840,7 @@ __device__ __forceinline__ void c4_stager(const ConvP16Params& p, unsigned char*
 #pragma unroll
                 for (int e = 0; e < 4; e++) v[e] = ok ? (_Float16)act_p16((float)raw[SET][i][e], p.act) : (_Float16)0.f;
                 *reinterpret_cast<half4_t*>(buf + l_off[i]) = v;
+                *reinterpret_cast<half4_t*>(buf + G::COPY2 + 8 + l_off[i]) = v;
             } else {
                 const float r[4] = {raw[SET][i].x, raw[SET][i].y, raw[SET][i].z, raw[SET][i].w};
                 half4_t hi, lo;
@@ -843,7 +851,9 @@ __device__ __forceinline__ void c4_stager(const ConvP16Params& p, unsigned char*
                     lo[e] = (_Float16)(v - (float)hi[e]);
                 }
                 *reinterpret_cast<half4_t*>(buf + l_off[i]) = hi;
+                *reinterpret_cast<half4_t*>(buf + G::COPY2 + 8 + l_off[i]) = hi;
                 *reinterpret_cast<half4_t*>(buf + G::PLANE + l_off[i]) = lo;
+                *reinterpret_cast<half4_t*>(buf + G::PLANE + G::COPY2 + 8 + l_off[i]) = lo;
             }
         }
     };
@@ -896,11 +906,7 @@ __device__ __forceinline__ void c4_stage(f32x4_t (&acc)[2][G::FN], half8_t (&a_q
             if (r == SL - 1) {
                 const unsigned char* src = lds + nbuf * G::BUF + bbase[fn] + off[ns];
 #pragma unroll
-                for (int pl = 0; pl < NPL; pl++) {
-                    const half4_t t0 = *reinterpret_cast<const half4_t*>(src + pl * G::PLANE);
-                    const half4_t t1 = *reinterpret_cast<const half4_t*>(src + pl * G::PLANE + G::PIX);
-                    b[fn][pl] = half8_t{t0[0], t0[1], t0[2], t0[3], t1[0], t1[1], t1[2], t1[3]};
-                }
+                for (int pl = 0; pl < NPL; pl++) b[fn][pl] = *reinterpret_cast<const half8_t*>(src + pl * G::PLANE);
             }
 #pragma unroll
             for (int j = 0; j < NW; j++)
@@ -944,7 +950,8 @@ __global__ __launch_bounds__(512) void conv_p16c4_kernel(const ConvP16Params p) 
     for (int fn = 0; fn < FN; fn++) {
         const int m = fn * 16 + mq;
         const int ty = m / TW, tx = m - ty * TW;
-        bbase[fn] = ty * G::ROW_PITCH + (wn * TW + tx) * G::PIX;
+        const int x = wn * TW + tx;   // (a tap pair starts an even number of pixels from its position: the position's parity picks the copy)
+        bbase[fn] = ty * G::ROW_PITCH + x * G::PIX + ((x & 1) ? G::COPY2 + 8 : 0);
     }
     int off[NS];   // LDS offset of this lane's tap pair in each step (pairs beyond the kernel: pair 0, their weights are zero)
 #pragma unroll
@@ -1019,12 +1026,7 @@ __global__ __launch_bounds__(512) void conv_p16c4_kernel(const ConvP16Params p) 
 #pragma unroll
     for (int fn = 0; fn < FN; fn++)
 #pragma unroll
-        for (int pl = 0; pl < NPL; pl++) {
-            const unsigned char* src = lds + bbase[fn] + off[0] + pl * G::PLANE;
-            const half4_t t0 = *reinterpret_cast<const half4_t*>(src);
-            const half4_t t1 = *reinterpret_cast<const half4_t*>(src + G::PIX);
-            b[fn][pl] = half8_t{t0[0], t0[1], t0[2], t0[3], t1[0], t1[1], t1[2], t1[3]};
-        }
+        for (int pl = 0; pl < NPL; pl++) b[fn][pl] = *reinterpret_cast<const half8_t*>(lds + bbase[fn] + off[0] + pl * G::PLANE);
     const unsigned char* wnext = wbase + (size_t)(PD - 1) * wstep;
     int tile = group;
     for (;;) {
