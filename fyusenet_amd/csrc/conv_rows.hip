@@ -53,6 +53,13 @@ __device__ __forceinline__ void load8<_Float16>(const _Float16* src, float* v) {
     for (int i = 0; i < 8; i++) v[i] = (float)a[i];
 }
 
+// Staging items in flight in a thread's registers: 8 channels of one column each, and where they go in the ring.
+template <int N>
+struct RowBatch {
+    float v[N][8];
+    int dst[N];
+};
+
 // CS: k16 steps per input row (input channels padded to 16*CS); a column of the ring holds 2*CS chunks of 8 halves.
 // The chunk order inside a column is permuted with the column index so that the 16-byte reads of 8 neighbouring lanes
 // cover all 32 banks.
@@ -102,15 +109,13 @@ __global__ __launch_bounds__(512) void conv_rows_kernel(const ConvRowsParams p) 
     const int stid = tid & 255;
     // Four rows at a time: ITEMS items per row dealt to the 256 staging threads.  fetch() issues the loads of a batch
     // into registers, store() converts and writes them into the ring; a batch is fetched one round before it is stored.
+    // (The rows of the first round are dealt to all 512 threads: the MFMA waves have nothing else to do until they are in.)
     constexpr int PER = (4 * ITEMS + 255) / 256;   // items per thread and batch
-    struct Batch {
-        float v[PER][8];
-        int dst[PER];
-    };
-    auto fetch = [&](Batch& bt, int j_first, int nrows) {
+    auto fetch = [&](auto& bt, int j_first, int nrows, int t, int nthreads) {
+        constexpr int N = sizeof(bt.dst) / sizeof(int);
 #pragma unroll
-        for (int i = 0; i < PER; i++) {
-            const int idx = i * 256 + stid;
+        for (int i = 0; i < N; i++) {
+            const int idx = i * nthreads + t;
             bt.dst[i] = -1;
 #pragma unroll
             for (int e = 0; e < 8; e++) bt.v[i][e] = 0.f;
@@ -129,9 +134,10 @@ __global__ __launch_bounds__(512) void conv_rows_kernel(const ConvRowsParams p) 
             }
         }
     };
-    auto store = [&](const Batch& bt) {
+    auto store = [&](const auto& bt) {
+        constexpr int N = sizeof(bt.dst) / sizeof(int);
 #pragma unroll
-        for (int i = 0; i < PER; i++) {
+        for (int i = 0; i < N; i++) {
             if (bt.dst[i] < 0) continue;
             half8_t hi, lo;
 #pragma unroll
@@ -150,20 +156,19 @@ __global__ __launch_bounds__(512) void conv_rows_kernel(const ConvRowsParams p) 
     constexpr int NB0 = (K + 2) / 4 + 1;      // batches in the ring before the first round
     const int nbatches = (rows_total + 3) >> 2;
     auto rows_of = [&](int b) { return min(4, rows_total - 4 * b); };
-    Batch nxt;   // the batch in flight (staging waves)
-    if (!mfma_wave) {
-        // all loads of the first rounds' rows are issued before the first conversion
-        Batch first[NB0];
-#pragma unroll
-        for (int b = 0; b < NB0; b++) fetch(first[b], 4 * b, b < nbatches ? rows_of(b) : 0);
-#pragma unroll
-        for (int b = 0; b < NB0; b++) store(first[b]);
-        // (the batch of the second round is requested once the first round's rows are in: every workgroup of the
-        // launch is in this phase at the same time, and it is bound by memory bandwidth)
-        fetch(nxt, 4 * NB0, NB0 < nbatches ? rows_of(NB0) : 0);
+    RowBatch<PER> nxt;   // the batch in flight (staging waves)
+    {
+        // the first round's rows, all threads: every load is issued before the first conversion
+        constexpr int PER0 = (NB0 * 4 * ITEMS + 511) / 512;
+        RowBatch<PER0> first;
+        fetch(first, 0, min(4 * NB0, rows_total), tid, 512);
+        store(first);
     }
-    // ---- weights: one fragment per step and plane, in registers from here on (loaded while the staging waves fill
-    //      the ring; placed behind their code so that the two never hold registers at the same point) ----
+    // (the batch of the second round is requested once the first round's rows are in: every workgroup of the
+    // launch is in this phase at the same time, and it is bound by memory bandwidth)
+    if (!mfma_wave) fetch(nxt, 4 * NB0, NB0 < nbatches ? rows_of(NB0) : 0, stid, 256);
+    // ---- weights: one fragment per step and plane, in registers from here on (placed behind the staging code so that
+    //      the two never hold registers at the same point) ----
     half8_t a_reg[NSTEPS][NPL];
     if (mfma_wave) {
         const half8_t* w = reinterpret_cast<const half8_t*>(p.wpack);
@@ -198,7 +203,7 @@ __global__ __launch_bounds__(512) void conv_rows_kernel(const ConvRowsParams p) 
             // write batch NB0 + g (fetched a round ago; no round up to g reads its ring slots), fetch the next one
             store(nxt);
             const int b = NB0 + g + 1;
-            fetch(nxt, 4 * b, b < nbatches ? rows_of(b) : 0);
+            fetch(nxt, 4 * b, b < nbatches ? rows_of(b) : 0, stid, 256);
             lds_barrier();
         }
         return;
