@@ -3,7 +3,7 @@
 //   LayerFactory / GPULayerFactoryBackend   -> Net::add_layer          (base/layerfactory.cpp, gpu/gpulayerfactory.cpp)
 //   BufferManager                           -> Net::connect / assign_buffers (base/buffermanager.cpp)
 //   NeuralNetwork / Engine (sync branch)    -> Net::setup / forward / finish (base/neuralnetwork.cpp, base/engine.cpp)
-//   GPULayerBase subclasses                 -> Layer subclasses in layers.cpp
+//   GPULayerBase subclasses                 -> Layer subclasses in layer_classes.h and layers.cpp
 #pragma once
 #include <hip/hip_runtime.h>
 
