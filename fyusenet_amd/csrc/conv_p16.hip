@@ -267,7 +267,8 @@ __device__ __forceinline__ void p16_stager(const ConvP16Params& p, unsigned char
                 gy = min(max(gy, 0), p.in_hp - 1);
                 gx = min(max(gx, 0), p.in_wp - 1);
             }
-            g_off[SET][i] = ((unsigned)gy < (unsigned)p.in_hp && (unsigned)gx < (unsigned)p.in_wp) ? (gy * p.in_wp + gx) * p.in_cp + g8 + chunk * KC : -1;
+            // (the last chunk of a tensor whose channel pitch is not a multiple of 32: the groups of 8 behind the pitch are zeros)
+            g_off[SET][i] = ((unsigned)gy < (unsigned)p.in_hp && (unsigned)gx < (unsigned)p.in_wp && g8 + chunk * KC < p.in_cp) ? (gy * p.in_wp + gx) * p.in_cp + g8 + chunk * KC : -1;
             const store_t* src = in + (g_off[SET][i] >= 0 ? g_off[SET][i] : 0);
             if constexpr (HSTORE) {
                 raw[SET][i] = *reinterpret_cast<const half8_t*>(src);
@@ -320,7 +321,7 @@ __device__ __forceinline__ void p16_stager(const ConvP16Params& p, unsigned char
             const int m = idx / G::RPP, piece = idx % G::RPP;
             const int ty = m / G::TWG, tx = m - ty * G::TWG;
             const int py = tyi * G::TH + ty, px = txi * G::TWG + tx;
-            const bool ok = idx < G::RPIECES && py < p.npos_y && px < p.npos_x;
+            const bool ok = idx < G::RPIECES && py < p.npos_y && px < p.npos_x && cb * CPB + piece * (16 / ESZ) < p.res_cp;
             rv[i] = *reinterpret_cast<const f32x4_t*>(res + (ok ? ((size_t)(p.res_off_y + py) * p.res_wp + p.res_off_x + px) * p.res_cp + cb * CPB + piece * (16 / ESZ) : 0));
         }
 #pragma unroll
@@ -344,9 +345,10 @@ __device__ __forceinline__ void p16_stager(const ConvP16Params& p, unsigned char
     int t2 = t1, c2 = c1;             // stage n+2
     bool have2 = have1 && advance(t2, c2);
     if (p.in_amax) in_scale = range_scale(range_after_act(range_reduce(range_bits), p.act), &inv_unused);
-    if (stid < CPB) {
-        reinterpret_cast<float*>(lds + sb_off)[stid] = p.scale[cb * CPB + stid];
-        reinterpret_cast<float*>(lds + sb_off)[CPB + stid] = p.bias[cb * CPB + stid];
+    if (stid < CPB) {   // (scale and bias have one entry per channel of the output tensor's pitch)
+        const bool have = cb * CPB + stid < p.out_cp;
+        reinterpret_cast<float*>(lds + sb_off)[stid] = have ? p.scale[cb * CPB + stid] : 0.f;
+        reinterpret_cast<float*>(lds + sb_off)[CPB + stid] = have ? p.bias[cb * CPB + stid] : 0.f;
     }
     store(Set0(), lds);
     
@@ -482,12 +484,14 @@ __global__ __launch_bounds__(512) void conv_p16_kernel(const ConvP16Params p) {
             const int m = fn * 16 + mq;
             const int ty = m / TW, tx = wn * TW + (m - ty * TW);
             const int py = tyi * TH + ty, px = txi * G::TWG + tx;
-            const bool ok = py < p.npos_y && px < p.npos_x;
+            const bool inside = py < p.npos_y && px < p.npos_x;
             const size_t obase = ((size_t)(p.out_off_y + py) * p.out_wp + p.out_off_x + px) * p.out_cp + cb * CPB + mw * 32 + kq * CHK;
             float fmax_ = 0.f;
             half8_t hv;
 #pragma unroll
             for (int fm = 0; fm < 2; fm++) {
+                // (a block of output channels may reach behind the tensor's channel pitch: those groups are not stored)
+                const bool ok = inside && cb * CPB + mw * 32 + kq * CHK + (HSTORE ? 0 : fm * CHF) < p.out_cp;
                 f32x4_t v;
 #pragma unroll
                 for (int e = 0; e < 4; e++) v[e] = acc[fm][fn][e] * scm[fm][e] + bi[fm][e];
@@ -511,11 +515,11 @@ __global__ __launch_bounds__(512) void conv_p16_kernel(const ConvP16Params p) {
                     if (fm == 1 && ok) *reinterpret_cast<half8_t*>(out + obase) = hv;   // the lane's eight channels in one store
                 } else {
 #pragma unroll
-                    for (int e = 0; e < 4; e++) fmax_ = fmaxf(fmax_, fabsf(v[e]));
+                    for (int e = 0; e < 4; e++) fmax_ = fmaxf(fmax_, ok ? fabsf(v[e]) : 0.f);
                     if (ok) *reinterpret_cast<f32x4_t*>(out + obase + fm * CHF) = v;
                 }
             }
-            vmax = fmaxf(vmax, ok ? fmax_ : 0.f);
+            vmax = fmaxf(vmax, fmax_);
         }
     };
 
@@ -1682,8 +1686,10 @@ void conv_p16_tile(int index, int* th, int* tw, int* stride, int* wm) {
     *th = kEntries[index].th; *tw = kEntries[index].tw; *stride = kEntries[index].stride; *wm = kEntries[index].wm;
 }
 bool conv_p16_supported(int k, int stride, int dil, int in_cp, int cout, int out_cp, bool f16) {
-    (void)f16;   // (both storage types; 16-byte loads and 8- or 16-byte stores hold for any pitch that is a multiple of 32 / 4)
-    return k == 3 && (stride == 1 || stride == 2) && dil == 1 && in_cp % KC == 0 && cout % 64 == 0 && out_cp % 4 == 0 && out_cp >= cout;
+    // (16-byte loads of 8 channels, 16-byte stores of 4 fp32 or 8 fp16 channels; the last chunk and the last block of
+    // output channels may be ragged: what lies behind a pitch is read as zero and not stored)
+    const int og = f16 ? 8 : 4;
+    return k == 3 && (stride == 1 || stride == 2) && dil == 1 && in_cp % 8 == 0 && in_cp >= 16 && cout >= 16 && out_cp % og == 0 && out_cp >= cout;
 }
 int tconv_p16_tile_count() { return (int)(sizeof(kTEntries) / sizeof(kTEntries[0])); }
 void tconv_p16_tile(int index, int* th, int* tw, int* wm) {
@@ -1812,9 +1818,9 @@ int P16_NAME(launch_conv_p16)(const ConvP16Params& p, hipStream_t s) {
     if (!e) return -1;
     const int cpb = 32 * e->wm, twg = (4 / e->wm) * e->tw;
     // what the kernel's indexing assumes
-    if (p.cin_chunks < 1 || p.in_cp != p.cin_chunks * KC || p.cout_blocks < 1 || p.mfrags < p.cout_blocks * 2 * e->wm ||
-        p.tiles_x * twg < p.npos_x || p.tiles_y * p.tile_h < p.npos_y || p.out_cp < p.cout_blocks * cpb || (p.out_cp * ESZ) % 16 != 0 ||
-        (p.res && (p.res_cp < p.cout_blocks * cpb || (p.res_cp * ESZ) % 16 != 0)) || p.nreset < 0 || p.nreset > 4 || p.pos_groups < 1 ||
+    if (p.cin_chunks < 1 || p.in_cp > p.cin_chunks * KC || p.in_cp <= (p.cin_chunks - 1) * KC || p.in_cp % 8 != 0 || p.cout_blocks < 1 || p.mfrags < p.cout_blocks * 2 * e->wm ||
+        p.tiles_x * twg < p.npos_x || p.tiles_y * p.tile_h < p.npos_y || p.out_cp <= (p.cout_blocks - 1) * cpb || (p.out_cp * ESZ) % 16 != 0 ||
+        (p.res && (p.res_cp <= (p.cout_blocks - 1) * cpb || (p.res_cp * ESZ) % 16 != 0)) || p.nreset < 0 || p.nreset > 4 || p.pos_groups < 1 ||
         p.pos_groups > p.tiles_x * p.tiles_y || (p.f16 != 0) != HSTORE ||
         // (a tile's residual tile may not be overwritten while its epilogue reads it: the next one comes a stage later)
         (p.res && p.cin_chunks < 2 && p.pos_groups < p.tiles_x * p.tiles_y) || p.rcp_tiles_x != 1.0f / (float)p.tiles_x ||

@@ -136,8 +136,10 @@ class ConvLayer : public Layer {
         q.out_wp = out_v.wp(); q.out_cp = out_v.cp; q.out_off_y = q.out_off_x = out_v.pad;
         if (res_v) { q.res_wp = res_v->wp(); q.res_cp = res_v->cp; q.res_off_y = q.res_off_x = res_v->pad; }
         q.res_relu = res_relu; q.res_scale = res_scale;
-        q.cin_chunks = in_v.cp / 32;
-        q.mfrags = oc / 16;
+        // (ragged channel counts: the last chunk reads zeros behind the input's pitch, the weights are packed for whole
+        // blocks of 64 output channels, and a block's channels behind the output's pitch are not stored)
+        q.cin_chunks = (in_v.cp + 31) / 32;
+        q.mfrags = (oc + 63) / 64 * 4;
         q.f16 = out_v.f16 ? 1 : 0;
         q.scale = scale_dev; q.bias = bias_dev;
         q.acc_mul = 1.f;
@@ -151,14 +153,14 @@ class ConvLayer : public Layer {
         for (int i = 0; i < conv_p16_tile_count(); i++) {
             int th, tw, st, wm;
             conv_p16_tile(i, &th, &tw, &st, &wm);
-            if (st != stride || oc % (32 * wm) != 0) continue;
+            if (st != stride || (wm == 4 && oc % 128 != 0)) continue;
             if (want_h && (th != want_h || tw != want_w || (want_wm && wm != want_wm))) continue;
             ConvP16Params c = q;
             c.tile_h = th; c.tile_w = tw; c.wm = wm;
             const int twg = (4 / wm) * tw;
             c.tiles_x = (ow + twg - 1) / twg; c.tiles_y = (oh + th - 1) / th;
             c.rcp_tiles_x = 1.0f / (float)c.tiles_x;
-            c.cout_blocks = oc / (32 * wm);
+            c.cout_blocks = (oc + 32 * wm - 1) / (32 * wm);
             // one workgroup per CU: as many tile walkers per block of output channels as the chip has room for
             c.pos_groups = std::max(1, std::min(c.tiles_x * c.tiles_y, 256 / c.cout_blocks));
             if (res_v && c.cin_chunks < 2) c.pos_groups = c.tiles_x * c.tiles_y;   // (residual tile: one stage per tile is too few to walk)

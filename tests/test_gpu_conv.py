@@ -277,6 +277,12 @@ P16_CASES = [
     (32, 192, 21, 50, 1, "8,6,2", {}),
     (64, 64, 90, 100, 1, "4,8,2", {"residual": (A.NONE, False)}),                  # 161 tiles x 1 block
     (64, 64, 256, 256, 1, None, {}),                                               # BASELINE's single-layer case
+    # channel counts that are not whole chunks / blocks: zeros behind the input's pitch, nothing stored behind the output's
+    (40, 40, 21, 26, 1, "8,8,2", {"bn": True, "residual": (A.RELU, True)}),         # the residual layers of the reference's sample style nets, reduced
+    (40, 40, 39, 32, 1, None, {"residual": (A.NONE, False)}),
+    (24, 72, 30, 22, 2, "8,6,2", {"bn": True}),                                    # one ragged chunk; the second block of 64 output channels holds 8
+    (72, 136, 17, 19, 1, "8,8,2", {"residual": (A.NONE, False)}),                  # three chunks, the last with 8 channels; three blocks of output channels
+    (48, 200, 20, 20, 1, "4,8,2", {"pad_out": 1}),
 ]
 
 
@@ -314,7 +320,7 @@ def test_sixteen_position_fragment_form(case, act, shallow, storage, monkeypatch
     err = rel_l2(got, ref)
     print("  ", info, "rel_l2=%.3e" % err, flush=True)
     # (fp32 tensors: the correction terms of the operand split run as fp8 MFMAs where the 32-channel chunks pair up)
-    assert ("conv_p16 f16+fp8-split" if cin % 64 == 0 else "conv_p16 f16x2-split") in info if storage == fa.STORAGE_F32 else "conv_p16 f16 " in info
+    assert ("conv_p16 f16+fp8-split" if ((cin + 31) // 32) % 2 == 0 else "conv_p16 f16x2-split") in info if storage == fa.STORAGE_F32 else "conv_p16 f16 " in info
     if tile:
         th, tw, wm = tile.split(",")
         assert "waves=%sx" % wm in info and "th=%s tw=%s" % (th, tw) in info
