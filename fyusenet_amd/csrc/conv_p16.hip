@@ -1689,7 +1689,7 @@ bool conv_p16_supported(int k, int stride, int dil, int in_cp, int cout, int out
     // (16-byte loads of 8 channels, 16-byte stores of 4 fp32 or 8 fp16 channels; the last chunk and the last block of
     // output channels may be ragged: what lies behind a pitch is read as zero and not stored)
     const int og = f16 ? 8 : 4;
-    return k == 3 && (stride == 1 || stride == 2) && dil == 1 && in_cp % 8 == 0 && in_cp >= 16 && cout >= 16 && out_cp % og == 0 && out_cp >= cout;
+    return k == 3 && (stride == 1 || stride == 2) && dil == 1 && in_cp % 8 == 0 && in_cp >= 16 && cout >= 8 && out_cp % og == 0 && out_cp >= cout;
 }
 int tconv_p16_tile_count() { return (int)(sizeof(kTEntries) / sizeof(kTEntries[0])); }
 void tconv_p16_tile(int index, int* th, int* tw, int* wm) {

@@ -283,6 +283,9 @@ P16_CASES = [
     (24, 72, 30, 22, 2, "8,6,2", {"bn": True}),                                    # one ragged chunk; the second block of 64 output channels holds 8
     (72, 136, 17, 19, 1, "8,8,2", {"residual": (A.NONE, False)}),                  # three chunks, the last with 8 channels; three blocks of output channels
     (48, 200, 20, 20, 1, "4,8,2", {"pad_out": 1}),
+    (20, 40, 38, 44, 2, "8,6,2", {"bn": True}),                                    # fewer channels than the tensors' pitch (conv3 and conv2 of those nets)
+    (12, 20, 50, 36, 2, "4,8,2", {}),
+    (44, 48, 23, 19, 1, "8,8,2", {"residual": (A.RELU, False)}),
 ]
 
 
