@@ -123,14 +123,16 @@ __global__ __launch_bounds__(512) void conv_rows_kernel(const ConvRowsParams p) 
                 const int jr = idx / ITEMS, it = idx - jr * ITEMS;
                 const int col = it / NCH, chunk = it - col * NCH;
                 const int j = j_first + jr;
+                // (coordinates in the frame of repeated pixels, which is the stored frame unless the step is fractional)
                 int gy = p.in_y0 + y_begin + j, gx = p.in_x0 + x0 + col;
+                const int vhp = p.in_hp << p.in_shift, vwp = p.in_wp << p.in_shift;
                 if (p.in_clamp) {
-                    gy = min(max(gy, 0), p.in_hp - 1);
-                    gx = min(max(gx, 0), p.in_wp - 1);
+                    gy = min(max(gy, 0), vhp - 1);
+                    gx = min(max(gx, 0), vwp - 1);
                 }
                 bt.dst[i] = (j & (RING - 1)) * ROWB + ring_off<CS>(col, chunk);
-                if ((unsigned)gy < (unsigned)p.in_hp && (unsigned)gx < (unsigned)p.in_wp && chunk * 8 < p.in_cp)
-                    load8<TIn>(in + ((size_t)gy * p.in_wp + gx) * p.in_cp + chunk * 8, bt.v[i]);
+                if ((unsigned)gy < (unsigned)vhp && (unsigned)gx < (unsigned)vwp && chunk * 8 < p.in_cp)
+                    load8<TIn>(in + ((size_t)(gy >> p.in_shift) * p.in_wp + (gx >> p.in_shift)) * p.in_cp + chunk * 8, bt.v[i]);
             }
         }
     };
@@ -346,7 +348,7 @@ int launch_conv_rows(const ConvRowsParams& p, bool f16, hipStream_t s) {
     rows_fn fn = f16 ? pick_rows<_Float16, _Float16, false, 2>(p.k, p.cs) : pick_rows<float, float, true, 2>(p.k, p.cs);
     if (!fn) return -1;
     // what the kernel's indexing assumes
-    if (p.cout * p.k > 28 || p.out_cp != 4 || p.strips < 1 || p.row_blocks < 1 ||
+    if (p.cout * p.k > 28 || p.out_cp != 4 || p.strips < 1 || p.row_blocks < 1 || p.in_shift < 0 || p.in_shift > 8 ||
         p.rows_per_block < 1 || p.rows_per_block % 4 || p.in_cp > 16 * p.cs || p.in_cp % 8 || p.cout * p.k > 32 ||
         (long long)p.strips * (32 * p.fn - (p.k - 1)) < p.out_w || (long long)p.row_blocks * p.rows_per_block < p.out_h)
         return -5;

@@ -141,6 +141,7 @@ struct ConvRowsParams {
     int in_hp, in_wp, in_cp;   // stored input frame
     int in_y0, in_x0;     // stored row of (output row 0, tap ky 0) and stored column of q column 0 (input padding - radius)
     int in_clamp;         // coordinates outside the stored frame repeat its edge instead of reading 0
+    int in_shift;         // fractional-step convolution: in_y0 / in_x0 and the taps count in the frame whose pixels are repeated 2^in_shift times
     int out_h, out_w;
     int out_wp, out_cp, out_off_y, out_off_x;
     int res_wp, res_cp, res_off_y, res_off_x, res_relu, res_scale;

@@ -761,6 +761,11 @@ class ConvLayer : public Layer {
         q.k = k; q.cs = (in_v.cp + 15) / 16; q.fn = 2;
         q.in_hp = in_v.hp(); q.in_wp = in_v.wp(); q.in_cp = in_v.cp;
         q.in_y0 = in_v.pad - r; q.in_x0 = in_v.pad - r;
+        if (frac_shift) {   // (the frame of repeated pixels, and the 3x3 shader's taps at -2, -1, 0: as in wide_subconv)
+            q.in_shift = frac_shift - 1;
+            q.in_y0 = (in_v.pad << q.in_shift) - r;
+            q.in_x0 = (in_v.pad << q.in_shift) + ((k == 3) ? -2 : -r);
+        }
         q.in_clamp = clamp ? 1 : 0;
         q.out_h = oh; q.out_w = ow;
         q.out_wp = out_v.wp(); q.out_cp = out_v.cp; q.out_off_y = q.out_off_x = out_v.pad;
@@ -783,7 +788,7 @@ class ConvLayer : public Layer {
         const char* at = net->sw.get("FYNHIP_AUTOTUNE");
         bool pick = true;
         char key[160];
-        snprintf(key, sizeof(key), "rows:%d:%dx%d:%dx%d:k%d:cp%d:r%d:e%d", out_v.f16, d.in_channels, oc, oh, ow, k, in_v.cp, res_v ? 1 : 0, clamp ? 1 : 0);
+        snprintf(key, sizeof(key), "rows:%d:%dx%d:%dx%d:k%d:cp%d:r%d:e%d:f%d", out_v.f16, d.in_channels, oc, oh, ow, k, in_v.cp, res_v ? 1 : 0, clamp ? 1 : 0, frac_shift);
         if (always) {
         } else if (tune_cache_flag(net, key, &pick)) {
         } else if (!(at && at[0] == '0')) {
@@ -923,7 +928,7 @@ class ConvLayer : public Layer {
             }
             // Third form: a workgroup walks down a strip of the image with the input rows in an LDS ring and the weights
             // in registers (conv_rows.hip); every input row is fetched once per strip and q never leaves the wave.
-            if (!frac_shift && conv_rows_supported(k, in_v.cp, oc, out_v.f16 != 0) && out_v.cp == 4 && !net->sw.get("FYNHIP_NO_ROWS_WIDE_CONV"))
+            if (conv_rows_supported(k, in_v.cp, oc, out_v.f16 != 0) && out_v.cp == 4 && !net->sw.get("FYNHIP_NO_ROWS_WIDE_CONV"))
                 setup_rows_wide(in_v, out_v, res_v, res_relu, res_scale);
         } else {
             SubConv sc;

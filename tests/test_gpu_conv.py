@@ -802,9 +802,27 @@ def test_fractional_convolution_parity(case, storage, expect="conv_mfma"):
     ref = oracle_single(b, storage, inputs, wts)
     err = rel_l2(got, ref)
     print("  ", info, "rel_l2=%.3e" % err, flush=True)
-    assert "fractional step 1/%d" % inv in info and expect in info
+    # (a layer with at most four output channels may also take the row-rolling form, whichever the engine times faster)
+    assert "fractional step 1/%d" % inv in info and (expect in info or (expect == "conv_mfma" and "conv_rows" in info and cout <= 4))
     assert got.shape == ref.shape == (cout, oh, ow)
     assert err <= TOL[storage], info
+
+
+FRAC_ROWS_CASES = [
+    FRAC_CASES[2], FRAC_CASES[3],                                 # the last layers of the reference's style nets, reduced
+    (9, 12, 3, 70, 41, 0.5, 1, 0, A.RELU, {}),                    # three strips, several row blocks
+    (5, 12, 4, 9, 40, 0.5, 1, 1, A.RELU, {"bn": True, "residual": (A.RELU, True)}),
+    (7, 24, 2, 13, 11, 0.25, 1, 0, A.NONE, {}),                   # two k16 steps per row, pixels repeated four times
+]
+
+
+@pytest.mark.parametrize("storage", [fa.STORAGE_F32, fa.STORAGE_F16], ids=["f32", "f16"])
+@pytest.mark.parametrize("case", FRAC_ROWS_CASES, ids=lambda c: "k%d_%dx%dx%d_to%d_step%g" % (c[0], c[1], c[3], c[4], c[2], c[5]))
+def test_fractional_convolution_row_rolling_form(case, storage, monkeypatch):
+    """The fractional-step convolution onto at most four channels on the row-rolling kernel: the rows it stages are rows
+    of the frame of repeated pixels."""
+    monkeypatch.setenv("FYNHIP_FORCE_ROWS_WIDE_CONV", "1")
+    test_fractional_convolution_parity(case, storage, expect="conv_rows")
 
 
 @pytest.mark.parametrize("case", [FRAC_CASES[1], FRAC_CASES[3], FRAC_CASES[6]], ids=["deconv2", "deconv3_9x9", "k5_bn_residual"])
