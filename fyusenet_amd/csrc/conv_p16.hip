@@ -262,13 +262,15 @@ __device__ __forceinline__ void p16_stager(const ConvP16Params& p, unsigned char
         const int y0 = tyi * G::TH * G::STEP + p.in_y0, x0 = txi * G::TWG * G::STEP + p.in_x0;
 #pragma unroll
         for (int i = 0; i < G::NB; i++) {
+            // (coordinates in the frame of repeated pixels, which is the stored frame unless the step is fractional)
             int gy = y0 + i_y[i], gx = x0 + i_x[i];
+            const int vhp = p.in_hp << p.in_shift, vwp = p.in_wp << p.in_shift;
             if (p.in_clamp && l_off[i] >= 0) {
-                gy = min(max(gy, 0), p.in_hp - 1);
-                gx = min(max(gx, 0), p.in_wp - 1);
+                gy = min(max(gy, 0), vhp - 1);
+                gx = min(max(gx, 0), vwp - 1);
             }
             // (the last chunk of a tensor whose channel pitch is not a multiple of 32: the groups of 8 behind the pitch are zeros)
-            g_off[SET][i] = ((unsigned)gy < (unsigned)p.in_hp && (unsigned)gx < (unsigned)p.in_wp && g8 + chunk * KC < p.in_cp) ? (gy * p.in_wp + gx) * p.in_cp + g8 + chunk * KC : -1;
+            g_off[SET][i] = ((unsigned)gy < (unsigned)vhp && (unsigned)gx < (unsigned)vwp && g8 + chunk * KC < p.in_cp) ? ((gy >> p.in_shift) * p.in_wp + (gx >> p.in_shift)) * p.in_cp + g8 + chunk * KC : -1;
             const store_t* src = in + (g_off[SET][i] >= 0 ? g_off[SET][i] : 0);
             if constexpr (HSTORE) {
                 raw[SET][i] = *reinterpret_cast<const half8_t*>(src);
@@ -1818,7 +1820,7 @@ int P16_NAME(launch_conv_p16)(const ConvP16Params& p, hipStream_t s) {
     if (!e) return -1;
     const int cpb = 32 * e->wm, twg = (4 / e->wm) * e->tw;
     // what the kernel's indexing assumes
-    if (p.cin_chunks < 1 || p.in_cp > p.cin_chunks * KC || p.in_cp <= (p.cin_chunks - 1) * KC || p.in_cp % 8 != 0 || p.cout_blocks < 1 || p.mfrags < p.cout_blocks * 2 * e->wm ||
+    if (p.cin_chunks < 1 || p.in_cp > p.cin_chunks * KC || p.in_cp <= (p.cin_chunks - 1) * KC || p.in_cp % 8 != 0 || p.in_shift < 0 || p.in_shift > 8 || p.cout_blocks < 1 || p.mfrags < p.cout_blocks * 2 * e->wm ||
         p.tiles_x * twg < p.npos_x || p.tiles_y * p.tile_h < p.npos_y || p.out_cp <= (p.cout_blocks - 1) * cpb || (p.out_cp * ESZ) % 16 != 0 ||
         (p.res && (p.res_cp <= (p.cout_blocks - 1) * cpb || (p.res_cp * ESZ) % 16 != 0)) || p.nreset < 0 || p.nreset > 4 || p.pos_groups < 1 ||
         p.pos_groups > p.tiles_x * p.tiles_y || (p.f16 != 0) != HSTORE ||
@@ -1856,7 +1858,7 @@ int P16_NAME(launch_tconv_p16)(const ConvP16Params& p, hipStream_t s) {
     if (!e) return -1;
     const int cpb = 32 * e->wm, twg = (4 / e->wm) * e->tw;
     if (p.cin_chunks < 1 || p.in_cp != p.cin_chunks * KC || p.cout_blocks < 1 || p.mfrags < p.cout_blocks * 2 * e->wm ||
-        p.tiles_x * twg < p.npos_x || p.tiles_y * p.tile_h < p.npos_y || p.out_cp < p.cout_blocks * cpb || (p.out_cp * ESZ) % 16 != 0 || p.res || p.stride != 1 ||
+        p.tiles_x * twg < p.npos_x || p.tiles_y * p.tile_h < p.npos_y || p.out_cp < p.cout_blocks * cpb || (p.out_cp * ESZ) % 16 != 0 || p.res || p.stride != 1 || p.in_shift != 0 ||
         p.nreset < 0 || p.nreset > 4 || p.pos_groups < 1 || p.pos_groups > p.tiles_x * p.tiles_y || (p.f16 != 0) != HSTORE ||
         p.rcp_tiles_x != 1.0f / (float)p.tiles_x || p.tiles_x * p.tiles_y > 4000000)
         return -5;
@@ -1889,7 +1891,7 @@ int P16_NAME(launch_conv_p16c4)(const ConvP16Params& p, int k, hipStream_t s) {
 #endif
     const C4Entry* e = find_c4entry(p, k);
     if (!e) return -1;
-    if (p.in_cp != 4 || p.cin_chunks != 1 || p.cout_blocks < 1 || p.mfrags < p.cout_blocks * 2 || p.wm != 1 || p.stride != 1 || p.res ||
+    if (p.in_cp != 4 || p.cin_chunks != 1 || p.cout_blocks < 1 || p.mfrags < p.cout_blocks * 2 || p.wm != 1 || p.stride != 1 || p.res || p.in_shift != 0 ||
         p.tiles_x * 4 * e->tw < p.npos_x || p.tiles_y * e->th < p.npos_y || p.out_cp < p.cout_blocks * 32 || (p.out_cp * ESZ) % 16 != 0 ||
         p.nreset < 0 || p.nreset > 4 || p.pos_groups < 1 || p.pos_groups > p.tiles_x * p.tiles_y || (p.f16 != 0) != HSTORE ||
         p.rcp_tiles_x != 1.0f / (float)p.tiles_x || p.tiles_x * p.tiles_y > 4000000)

@@ -174,6 +174,7 @@ struct ConvP16Params {
     int stride;           // input step per output position
     int in_y0, in_x0;     // stored coordinate of tap (0,0) of output position (0,0) (input padding - 1)
     int in_clamp;         // coordinates outside the stored frame repeat its edge instead of reading 0
+    int in_shift;         // launch_conv_p16, fractional-step convolution: in_y0 / in_x0, the taps and the stride count in the frame whose pixels are repeated 2^in_shift times
     int npos_y, npos_x;
     int out_wp, out_cp, out_off_y, out_off_x;
     int res_wp, res_cp, res_off_y, res_off_x, res_relu, res_scale;

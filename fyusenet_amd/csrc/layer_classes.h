@@ -131,6 +131,11 @@ class ConvLayer : public Layer {
         q.in_hp = in_v.hp(); q.in_wp = in_v.wp(); q.in_cp = in_v.cp;
         q.stride = stride;
         q.in_y0 = q.in_x0 = in_v.pad - 1;
+        if (frac_shift) {   // (the frame of repeated pixels; the 3x3 shader's columns at -2, -1, 0: as in the general kernel's sub-convolution)
+            q.in_shift = frac_shift - 1;
+            q.in_y0 = (in_v.pad << q.in_shift) - 1;
+            q.in_x0 = (in_v.pad << q.in_shift) - 2;
+        }
         q.in_clamp = clamp ? 1 : 0;
         q.npos_y = oh; q.npos_x = ow;
         q.out_wp = out_v.wp(); q.out_cp = out_v.cp; q.out_off_y = q.out_off_x = out_v.pad;
@@ -181,7 +186,7 @@ class ConvLayer : public Layer {
         const bool timing = !(at && at[0] == '0');
         int pick = 0;   // index into cands, -1: the general kernel
         char key[160];
-        snprintf(key, sizeof(key), "p16:%dx%d:%dx%d:s%d:cp%d:r%d:e%d:h%d", d.in_channels, oc, oh, ow, stride, in_v.cp, res_v ? 1 : 0, clamp ? 1 : 0, q.f16);
+        snprintf(key, sizeof(key), "p16:%dx%d:%dx%d:s%d:cp%d:r%d:e%d:h%d:f%d", d.in_channels, oc, oh, ow, stride, in_v.cp, res_v ? 1 : 0, clamp ? 1 : 0, q.f16, frac_shift);
         int cached[3] = {0, 0, 0};
         bool have_cached = false;
         if (!want_h) have_cached = tune_cache_triple(net, key, cached);   // (the cache keeps: chosen?, tile_h*1000 + tile_w, wm)
@@ -970,7 +975,7 @@ class ConvLayer : public Layer {
                 (!res_v || res_v->cp >= oc) && !net->sw.get("FYNHIP_NO_P16_CONV") && !net->sw.get("FYNHIP_NO_H16_CONV"))
                 setup_h16(in_v, out_v, res_v, res_relu, res_scale);
             // (channels between a layer's count and the tensor's pitch hold zeros and meet zero weights)
-            if (!only_kr && !p16 && !frac_shift && same_storage && !sc.in_sub && conv_p16_supported(k, stride, dil, in_v.cp, oc, out_v.cp, out_v.f16 != 0) &&
+            if (!only_kr && !p16 && same_storage && !sc.in_sub && conv_p16_supported(k, stride, dil, in_v.cp, oc, out_v.cp, out_v.f16 != 0) &&
                 d.in_channels <= in_v.cp && (!res_v || (res_v->cp >= oc && res_v->cp % 8 == 0)) && !net->sw.get("FYNHIP_NO_P16_CONV"))
                 setup_p16(in_v, out_v, res_v, res_relu, res_scale);
             if (!only_kr && !p16 && !frac_shift && same_storage && !res_v && conv_p16c4_supported(k, stride, dil, in_v.cp, oc, out_v.cp, out_v.f16 != 0) &&

@@ -802,8 +802,9 @@ def test_fractional_convolution_parity(case, storage, expect="conv_mfma"):
     ref = oracle_single(b, storage, inputs, wts)
     err = rel_l2(got, ref)
     print("  ", info, "rel_l2=%.3e" % err, flush=True)
-    # (a layer with at most four output channels may also take the row-rolling form, whichever the engine times faster)
-    assert "fractional step 1/%d" % inv in info and (expect in info or (expect == "conv_mfma" and "conv_rows" in info and cout <= 4))
+    # (a layer with at most four output channels may also take the row-rolling form, a 3x3 layer the 16-position-fragment
+    # form, whichever the engine times faster)
+    assert "fractional step 1/%d" % inv in info and (expect in info or (expect == "conv_mfma" and (("conv_rows" in info and cout <= 4) or ("conv_p16" in info and k == 3))))
     assert got.shape == ref.shape == (cout, oh, ow)
     assert err <= TOL[storage], info
 
@@ -823,6 +824,24 @@ def test_fractional_convolution_row_rolling_form(case, storage, monkeypatch):
     of the frame of repeated pixels."""
     monkeypatch.setenv("FYNHIP_FORCE_ROWS_WIDE_CONV", "1")
     test_fractional_convolution_parity(case, storage, expect="conv_rows")
+
+
+FRAC_P16_CASES = [
+    FRAC_CASES[0], FRAC_CASES[1],                                  # deconv1 and deconv2 of the reference's style nets, reduced
+    (3, 40, 20, 37, 45, 0.5, 2, 0, A.RELU, {}),                    # several tiles, ragged on both sides
+    (3, 24, 16, 19, 23, 0.5, 1, 1, A.RELU, {"bn": True, "residual": (A.NONE, False), "pad_out": 1}),   # no down-sampling, padded tensors
+    (3, 64, 64, 9, 12, 0.25, 2, 0, A.NONE, {"bn": True}),          # whole chunks and blocks, pixels repeated four times
+]
+
+
+@pytest.mark.parametrize("storage", [fa.STORAGE_F32, fa.STORAGE_F16], ids=["f32", "f16"])
+@pytest.mark.parametrize("case", FRAC_P16_CASES, ids=lambda c: "k%d_%dx%dx%d_to%d_step%g_s%d" % (c[0], c[1], c[3], c[4], c[2], c[5], c[6]))
+def test_fractional_convolution_sixteen_position_form(case, storage, monkeypatch):
+    """The fractional-step 3x3 convolution on the 16-position-fragment kernel: its staging waves fetch the halo tile of
+    the frame of repeated pixels."""
+    monkeypatch.setenv("FYNHIP_FORCE_P16_CONV", "1")
+    monkeypatch.setenv("FYNHIP_NO_H16_CONV", "1")
+    test_fractional_convolution_parity(case, storage, expect="conv_p16")
 
 
 @pytest.mark.parametrize("case", [FRAC_CASES[1], FRAC_CASES[3], FRAC_CASES[6]], ids=["deconv2", "deconv3_9x9", "k5_bn_residual"])
