@@ -869,9 +869,10 @@ __device__ __forceinline__ void c4_stager(const ConvP16Params& p, unsigned char*
     int t1 = tile + p.pos_groups, t2 = t1 + p.pos_groups;
     fetch(Set0(), tile);
     if (p.in_amax) in_scale = range_scale(range_after_act(range_reduce(range_bits), p.act), &inv_unused);
-    if (stid < 32) {
-        reinterpret_cast<float*>(lds + sb_off)[stid] = p.scale[cb * 32 + stid];
-        reinterpret_cast<float*>(lds + sb_off)[32 + stid] = p.bias[cb * 32 + stid];
+    if (stid < 32) {   // (scale and bias have one entry per channel of the output tensor's pitch)
+        const bool have = cb * 32 + stid < p.out_cp;
+        reinterpret_cast<float*>(lds + sb_off)[stid] = have ? p.scale[cb * 32 + stid] : 0.f;
+        reinterpret_cast<float*>(lds + sb_off)[32 + stid] = have ? p.bias[cb * 32 + stid] : 0.f;
     }
     store(Set0(), lds);
     lds_barrier();
@@ -976,7 +977,7 @@ __global__ __launch_bounds__(512) void conv_p16c4_kernel(const ConvP16Params p) 
 #pragma unroll
         for (int fm = 0; fm < 2; fm++)
 #pragma unroll
-            for (int pl = 0; pl < NPL; pl++) a_q[d][fm][pl] = *reinterpret_cast<const half8_t*>(wbase + (size_t)d * wstep + (fm * NPL + pl) * 1024 + wlane);
+            for (int pl = 0; pl < NPL; pl++) a_q[d][fm][pl] = *reinterpret_cast<const half8_t*>(wbase + (size_t)(d % NS) * wstep + (fm * NPL + pl) * 1024 + wlane);   // (a stage of fewer steps than the ring holds: the next tile's)
     f32x4_t acc[2][FN];
     auto zero_acc = [&]() {
 #pragma unroll
@@ -1004,17 +1005,19 @@ __global__ __launch_bounds__(512) void conv_p16c4_kernel(const ConvP16Params p) 
             const int m = fn * 16 + mq;
             const int ty = m / TW, tx = wn * TW + (m - ty * TW);
             const int py = tyi * TH + ty, px = txi * G::TWG + tx;
-            const bool ok = py < p.npos_y && px < p.npos_x;
+            const bool inside = py < p.npos_y && px < p.npos_x;
             const size_t obase = ((size_t)(p.out_off_y + py) * p.out_wp + p.out_off_x + px) * p.out_cp + cb * 32 + kq * CHK;
             float fmax_ = 0.f;
             half8_t hv;
 #pragma unroll
             for (int fm = 0; fm < 2; fm++) {
+                // (the block of 32 output channels may reach behind the tensor's channel pitch: those groups are not stored)
+                const bool ok = inside && cb * 32 + kq * CHK + (HSTORE ? 0 : fm * CHF) < p.out_cp;
                 f32x4_t v;
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
                     v[e] = acc[fm][fn][e] * scm[fm][e] + bi[fm][e];
-                    if constexpr (!HSTORE) fmax_ = fmaxf(fmax_, fabsf(v[e]));
+                    if constexpr (!HSTORE) fmax_ = fmaxf(fmax_, ok ? fabsf(v[e]) : 0.f);
                 }
                 if constexpr (HSTORE) {
 #pragma unroll
@@ -1024,7 +1027,7 @@ __global__ __launch_bounds__(512) void conv_p16c4_kernel(const ConvP16Params p) 
                     if (ok) *reinterpret_cast<f32x4_t*>(out + obase + fm * CHF) = v;
                 }
             }
-            vmax = fmaxf(vmax, ok ? fmax_ : 0.f);
+            vmax = fmaxf(vmax, fmax_);
         }
     };
     lds_barrier();   // the first stage is staged
@@ -1033,7 +1036,7 @@ __global__ __launch_bounds__(512) void conv_p16c4_kernel(const ConvP16Params p) 
     for (int fn = 0; fn < FN; fn++)
 #pragma unroll
         for (int pl = 0; pl < NPL; pl++) b[fn][pl] = *reinterpret_cast<const half8_t*>(lds + bbase[fn] + off[0] + pl * G::PLANE);
-    const unsigned char* wnext = wbase + (size_t)(PD - 1) * wstep;
+    const unsigned char* wnext = wbase + (size_t)((PD - 1) % NS) * wstep;
     int tile = group;
     for (;;) {
         c4_stage<G, 0>(acc, a_q, b, bbase, off, lds, wnext, wbase, wend, wstep, wlane);
@@ -1630,7 +1633,7 @@ struct C4Entry {
 };
 template <int K, int TH, int TW>
 constexpr C4Entry c4entry() { return C4Entry{K, TH, TW, conv_p16c4_kernel<K, TH, TW>, (size_t)GeoC4<K, TH, TW>::BUF, GeoC4<K, TH, TW>::NS}; }
-const C4Entry kC4Entries[] = {c4entry<9, 8, 8>(), c4entry<9, 4, 8>(), c4entry<9, 8, 4>()};
+const C4Entry kC4Entries[] = {c4entry<9, 8, 8>(), c4entry<9, 4, 8>(), c4entry<9, 8, 4>(), c4entry<3, 8, 8>(), c4entry<3, 4, 8>()};
 struct KREntry {
     int taps, cpw, fm, nfrag, th, tw, stride, dws, rounds, src;   // (cpw: chunks per wave and round)
     p16_fn fn;
@@ -1712,8 +1715,8 @@ void conv_kr16_variant(int index, int* taps, int* chunks, int* fm, int* th, int*
     *th = kKREntries[index].th; *tw = kKREntries[index].tw; *stride = kKREntries[index].stride;
 }
 bool conv_p16c4_supported(int k, int stride, int dil, int in_cp, int cout, int out_cp, bool f16) {
-    (void)f16;
-    return k == 9 && stride == 1 && dil == 1 && in_cp == 4 && cout % 32 == 0 && out_cp % 4 == 0 && out_cp >= cout;
+    // (any number of output channels: the weights are packed for whole blocks of 32, what lies behind the pitch is not stored)
+    return (k == 9 || k == 3) && stride == 1 && dil == 1 && in_cp == 4 && cout >= 8 && out_cp % (f16 ? 8 : 4) == 0 && out_cp >= cout;
 }
 #endif
 
@@ -1892,7 +1895,7 @@ int P16_NAME(launch_conv_p16c4)(const ConvP16Params& p, int k, hipStream_t s) {
     const C4Entry* e = find_c4entry(p, k);
     if (!e) return -1;
     if (p.in_cp != 4 || p.cin_chunks != 1 || p.cout_blocks < 1 || p.mfrags < p.cout_blocks * 2 || p.wm != 1 || p.stride != 1 || p.res || p.in_shift != 0 ||
-        p.tiles_x * 4 * e->tw < p.npos_x || p.tiles_y * e->th < p.npos_y || p.out_cp < p.cout_blocks * 32 || (p.out_cp * ESZ) % 16 != 0 ||
+        p.tiles_x * 4 * e->tw < p.npos_x || p.tiles_y * e->th < p.npos_y || p.out_cp <= (p.cout_blocks - 1) * 32 || (p.out_cp * ESZ) % 16 != 0 ||
         p.nreset < 0 || p.nreset > 4 || p.pos_groups < 1 || p.pos_groups > p.tiles_x * p.tiles_y || (p.f16 != 0) != HSTORE ||
         p.rcp_tiles_x != 1.0f / (float)p.tiles_x || p.tiles_x * p.tiles_y > 4000000)
         return -5;

@@ -233,8 +233,8 @@ class ConvLayer : public Layer {
         q.npos_y = oh; q.npos_x = ow;
         q.out_wp = out_v.wp(); q.out_cp = out_v.cp; q.out_off_y = q.out_off_x = out_v.pad;
         q.cin_chunks = 1;
-        q.mfrags = oc / 16;
-        q.cout_blocks = oc / 32;
+        q.mfrags = (oc + 31) / 32 * 2;
+        q.cout_blocks = (oc + 31) / 32;
         q.f16 = out_v.f16 ? 1 : 0;
         q.scale = scale_dev; q.bias = bias_dev;
         q.acc_mul = 1.f;

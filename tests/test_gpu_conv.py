@@ -687,6 +687,11 @@ C4_CASES = [
     (1, 32, 12, 70, "4,8", {"bn": True}),
     (3, 32, 90, 300, "8,8", {}),                     # 360 tiles: workgroups walk
     (3, 32, 33, 50, None, {"pad_out": 2}),
+    (3, 12, 30, 70, "8,8", {"bn": True}),            # fewer output channels than a block of 32 (the first layer of the reference's sample style nets)
+    (3, 40, 21, 33, "4,8", {}),                      # a second block that holds 8 channels
+    (3, 12, 40, 64, "8,8", {"k": 3}),                # 3x3: a stage of three steps, two turns of it in the weight ring
+    (4, 32, 19, 37, "4,8", {"k": 3, "bn": True}),
+    (3, 24, 50, 41, None, {"k": 3}),
 ]
 
 
@@ -697,13 +702,16 @@ C4_CASES = [
 def test_small_input_sixteen_position_fragment_form(case, shallow, storage, monkeypatch):
     """The 9x9 convolution on at most four input channels with two taps of a 4-channel pixel per lane and step."""
     cin, cout, h, w, tile, kw = case
+    kw = dict(kw)
+    k = kw.pop("k", 9)
     monkeypatch.setenv("FYNHIP_FORCE_P16_CONV", "1")
+    monkeypatch.setenv("FYNHIP_NO_D16_CONV", "1")   # (the LDS-free form for first layers has its own test)
     if tile:
         monkeypatch.setenv("FYNHIP_P16_TILE", tile)
     if shallow:
         kw = dict(kw, deep=False, pad_in=0)
-    b = conv_builder(9, cout, h, w, cin, 1, 1, A.NONE, **kw)
-    wts = conv_block(1200 + cin, cout, 9, cin, bn=kw.get("bn", False))
+    b = conv_builder(k, cout, h, w, cin, 1, 1, A.NONE, **kw)
+    wts = conv_block(1200 + cin, cout, k, cin, bn=kw.get("bn", False))
     x = prng.uniform(61 * cin + w, (cin, h, w), 0, 1)
     got, info = run_single(b, storage, [x], wts)
     ref = oracle_single(b, storage, [x], wts)
