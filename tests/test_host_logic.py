@@ -88,6 +88,14 @@ def test_no_gpu_fails_loudly():
     assert rc == capi.ERR_DEVICE and b"hip" in capi.lib().fyn_last_error().lower()
 
 
+def test_bench_refuses_more_than_one_gpu():
+    """The engine runs on one GPU; bench.py says so instead of pretending to scale."""
+    import subprocess, sys
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert r.returncode != 0 and "one GPU" in (r.stderr + r.stdout)
+    assert not r.stdout.strip().startswith("{")   # (no record is printed)
+
+
 def test_prng_is_stable():
     # golden values pin the generator so that every machine sees the same tensors
     from fyusenet_amd import prng
