@@ -39,24 +39,32 @@ __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(
 
 __device__ __forceinline__ float act1r(float x, const Act& a) { return __builtin_amdgcn_fmed3f(x, a.lo, a.hi) + a.leak * fminf(x, 0.f); }
 
+// Eight channels of a staging item as they come from memory; they are converted when the item is written to the ring,
+// a round after its load was issued (a conversion at the load would wait for it: one memory round trip per item).
 template <typename T>
-__device__ __forceinline__ void load8(const T* src, float* v);
+struct Raw8;
 template <>
-__device__ __forceinline__ void load8<float>(const float* src, float* v) {
-    const float4 a = *reinterpret_cast<const float4*>(src), b = *reinterpret_cast<const float4*>(src + 4);
-    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
-}
+struct Raw8<float> {
+    float4 a, b;
+    __device__ __forceinline__ void zero() { a = b = float4{0.f, 0.f, 0.f, 0.f}; }
+    __device__ __forceinline__ void load(const float* src) { a = *reinterpret_cast<const float4*>(src); b = *reinterpret_cast<const float4*>(src + 4); }
+    __device__ __forceinline__ void get(float* v) const { v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w; }
+};
 template <>
-__device__ __forceinline__ void load8<_Float16>(const _Float16* src, float* v) {
-    const half8_t a = *reinterpret_cast<const half8_t*>(src);
+struct Raw8<_Float16> {
+    half8_t h;
+    __device__ __forceinline__ void zero() { h = (half8_t)((_Float16)0.f); }
+    __device__ __forceinline__ void load(const _Float16* src) { h = *reinterpret_cast<const half8_t*>(src); }
+    __device__ __forceinline__ void get(float* v) const {
 #pragma unroll
-    for (int i = 0; i < 8; i++) v[i] = (float)a[i];
-}
+        for (int i = 0; i < 8; i++) v[i] = (float)h[i];
+    }
+};
 
 // Staging items in flight in a thread's registers: 8 channels of one column each, and where they go in the ring.
-template <int N>
+template <typename T, int N>
 struct RowBatch {
-    float v[N][8];
+    Raw8<T> v[N];
     int dst[N];
 };
 
@@ -117,8 +125,7 @@ __global__ __launch_bounds__(512) void conv_rows_kernel(const ConvRowsParams p) 
         for (int i = 0; i < N; i++) {
             const int idx = i * nthreads + t;
             bt.dst[i] = -1;
-#pragma unroll
-            for (int e = 0; e < 8; e++) bt.v[i][e] = 0.f;
+            bt.v[i].zero();
             if (idx < nrows * ITEMS) {
                 const int jr = idx / ITEMS, it = idx - jr * ITEMS;
                 const int col = it / NCH, chunk = it - col * NCH;
@@ -132,7 +139,7 @@ __global__ __launch_bounds__(512) void conv_rows_kernel(const ConvRowsParams p) 
                 }
                 bt.dst[i] = (j & (RING - 1)) * ROWB + ring_off<CS>(col, chunk);
                 if ((unsigned)gy < (unsigned)vhp && (unsigned)gx < (unsigned)vwp && chunk * 8 < p.in_cp)
-                    load8<TIn>(in + ((size_t)(gy >> p.in_shift) * p.in_wp + (gx >> p.in_shift)) * p.in_cp + chunk * 8, bt.v[i]);
+                    bt.v[i].load(in + ((size_t)(gy >> p.in_shift) * p.in_wp + (gx >> p.in_shift)) * p.in_cp + chunk * 8);
             }
         }
     };
@@ -141,10 +148,12 @@ __global__ __launch_bounds__(512) void conv_rows_kernel(const ConvRowsParams p) 
 #pragma unroll
         for (int i = 0; i < N; i++) {
             if (bt.dst[i] < 0) continue;
+            float r[8];
+            bt.v[i].get(r);
             half8_t hi, lo;
 #pragma unroll
             for (int e = 0; e < 8; e++) {
-                const float a = SPLIT ? act1r(bt.v[i][e], p.act) * in_scale : act1r(bt.v[i][e], p.act);
+                const float a = SPLIT ? act1r(r[e], p.act) * in_scale : act1r(r[e], p.act);
                 hi[e] = (_Float16)a;
                 lo[e] = (_Float16)(a - (float)hi[e]);
             }
@@ -158,11 +167,11 @@ __global__ __launch_bounds__(512) void conv_rows_kernel(const ConvRowsParams p) 
     constexpr int NB0 = (K + 2) / 4 + 1;      // batches in the ring before the first round
     const int nbatches = (rows_total + 3) >> 2;
     auto rows_of = [&](int b) { return min(4, rows_total - 4 * b); };
-    RowBatch<PER> nxt;   // the batch in flight (staging waves)
+    RowBatch<TIn, PER> nxt;   // the batch in flight (staging waves)
     {
         // the first round's rows, all threads: every load is issued before the first conversion
         constexpr int PER0 = (NB0 * 4 * ITEMS + 511) / 512;
-        RowBatch<PER0> first;
+        RowBatch<TIn, PER0> first;
         fetch(first, 0, min(4 * NB0, rows_total), tid, 512);
         store(first);
     }
