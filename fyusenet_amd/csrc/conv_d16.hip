@@ -28,17 +28,6 @@ namespace fynhip {
 namespace {
 typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
 
-// An activation that is exact on halves -- none, or a clamp without leak whose bounds are fp16 values -- is applied to
-// the packed halves (two values per instruction, no conversions): act_half_exact says whether, act_half applies it.
-__device__ __forceinline__ bool act_half_exact(const Act& a, _Float16& lo, _Float16& hi) {
-    lo = (_Float16)fmaxf(a.lo, -65504.f);
-    hi = (_Float16)fminf(a.hi, 65504.f);
-    return a.leak == 0.f && (a.lo < -65504.f || (float)lo == a.lo) && (a.hi > 65504.f || (float)hi == a.hi);
-}
-__device__ __forceinline__ half8_t act_half(half8_t v, _Float16 lo, _Float16 hi) {
-    return __builtin_elementwise_min(__builtin_elementwise_max(v, (half8_t)lo), (half8_t)hi);
-}
-
 // DWS = 1 or 2: the layer's input is the output of a depthwise 3x3 layer with step DWS that is not read from memory but
 // computed by every wave for its positions (nine texels of the depthwise layer's input per lane and chunk instead of
 // one of its output; that layer's own arithmetic and rounding), as in conv_kr16_kernel's staging.

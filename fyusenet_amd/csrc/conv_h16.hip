@@ -137,13 +137,11 @@ __device__ __forceinline__ void h16_stager(const ConvP16Params& p, unsigned char
             if (l_off[i] < 0) continue;
             const bool ok = g_off[i] >= 0;
             half8_t v;
-            if (p.act.kind == ACT_NONE || p.act.kind == ACT_RELU) {
-                // (on the packed halves: one instruction per pair instead of seven per value; the staging waves share their
+            _Float16 hlo, hhi;
+            if (act_half_exact(p.act, hlo, hhi)) {
+                // (on the packed halves: two instructions per item instead of seven per value; the staging waves share their
                 // SIMDs' issue slots with the MFMA waves)
-                typedef unsigned u32x4_t __attribute__((ext_vector_type(4)));
-                v = raw[i];
-                if (p.act.kind == ACT_RELU) v = __builtin_elementwise_max(v, (half8_t)((_Float16)0.f));
-                v = __builtin_bit_cast(half8_t, __builtin_bit_cast(u32x4_t, v) & (u32x4_t)(ok ? 0xffffffffu : 0u));
+                v = ok ? act_half(raw[i], hlo, hhi) : (half8_t)((_Float16)0.f);
             } else {
 #pragma unroll
                 for (int e = 0; e < 8; e++) v[e] = ok ? (_Float16)act_p16((float)raw[i][e], p.act) : (_Float16)0.f;

@@ -284,18 +284,16 @@ __device__ __forceinline__ void p16_stager(const ConvP16Params& p, unsigned char
     auto store = [&](auto set_, unsigned char* buf) {
         constexpr int SET = decltype(set_)::value;
         if constexpr (HSTORE) {
-            // (no activation and ReLU act on the packed halves: one instruction per pair instead of seven per value)
-            typedef unsigned u32x4_t __attribute__((ext_vector_type(4)));
+            // (an activation that is exact on halves acts on the packed halves: two instructions per item instead of seven per value)
+            _Float16 hlo, hhi;
+            const bool half_act = act_half_exact(p.act, hlo, hhi);
 #pragma unroll
             for (int i = 0; i < G::NB; i++) {
                 if (l_off[i] < 0) continue;
                 const bool ok = g_off[SET][i] >= 0;
                 half8_t v;
-                if (act_kind_ == ACT_NONE || act_kind_ == ACT_RELU) {
-                    v = raw[SET][i];
-                    if (act_kind_ == ACT_RELU) v = __builtin_elementwise_max(v, (half8_t)((_Float16)0.f));
-                    const u32x4_t keep = __builtin_bit_cast(u32x4_t, v) & (u32x4_t)(ok ? 0xffffffffu : 0u);
-                    v = __builtin_bit_cast(half8_t, keep);
+                if (half_act) {
+                    v = ok ? act_half(raw[SET][i], hlo, hhi) : (half8_t)((_Float16)0.f);
                 } else {
 #pragma unroll
                     for (int e = 0; e < 8; e++) v[e] = ok ? (_Float16)act_p16((float)raw[SET][i][e], p.act) : (_Float16)0.f;
@@ -852,11 +850,9 @@ __device__ __forceinline__ void c4_stager(const ConvP16Params& p, unsigned char*
             const bool ok = g_off[SET][i] >= 0;
             if constexpr (HSTORE) {
                 half4_t v;
-                if (p.act.kind == ACT_NONE || p.act.kind == ACT_RELU) {   // (on the packed halves, as in p16_stager)
-                    typedef unsigned u32x2_t __attribute__((ext_vector_type(2)));
-                    v = raw[SET][i];
-                    if (p.act.kind == ACT_RELU) v = __builtin_elementwise_max(v, (half4_t)((_Float16)0.f));
-                    v = __builtin_bit_cast(half4_t, __builtin_bit_cast(u32x2_t, v) & (u32x2_t)(ok ? 0xffffffffu : 0u));
+                _Float16 hlo, hhi;
+                if (act_half_exact(p.act, hlo, hhi)) {   // (on the packed halves, as in p16_stager)
+                    v = ok ? act_half4(raw[SET][i], hlo, hhi) : (half4_t)((_Float16)0.f);
                 } else {
 #pragma unroll
                     for (int e = 0; e < 4; e++) v[e] = ok ? (_Float16)act_p16((float)raw[SET][i][e], p.act) : (_Float16)0.f;
@@ -1239,8 +1235,8 @@ __global__ __launch_bounds__(512) void conv_kr16_kernel(const ConvP16Params p) {
         if (ranged) in_scale = range_scale(range_after_act(range_reduce(range_word()), p.act), &inv_unused);
         // (fp16 tensors: no activation, or a clamp without leak whose bounds are fp16 values, is applied to the packed
         // halves -- two values per instruction, no conversions)
-        const _Float16 hlo = (_Float16)fmaxf(p.act.lo, -65504.f), hhi = (_Float16)fminf(p.act.hi, 65504.f);
-        const bool half_act = HSTORE && p.act.leak == 0.f && (p.act.lo < -65504.f || (float)hlo == p.act.lo) && (p.act.hi > 65504.f || (float)hhi == p.act.hi);
+        _Float16 hlo, hhi;
+        const bool half_act = act_half_exact(p.act, hlo, hhi) && HSTORE;
         // a batch-norm layer in front: x * in_mul[c] + in_add[c] on the item's eight channels (the arrays come through the L1)
         auto affine8 = [&](float (&x)[8], const int i) {
             const int c = ok[i] ? ch_of[i] : 0;
@@ -1269,7 +1265,7 @@ __global__ __launch_bounds__(512) void conv_kr16_kernel(const ConvP16Params p) {
                 }
                 half8_t v;
                 if (half_act) {
-                    v = ok[i] ? __builtin_elementwise_min(__builtin_elementwise_max(rv, (half8_t)hlo), (half8_t)hhi) : (half8_t)((_Float16)0.f);
+                    v = ok[i] ? act_half(rv, hlo, hhi) : (half8_t)((_Float16)0.f);
                 } else {
 #pragma unroll
                     for (int e = 0; e < 8; e++) v[e] = ok[i] ? (_Float16)act_p16((float)rv[e], p.act) : (_Float16)0.f;

@@ -14,6 +14,21 @@ typedef float f32x4_t __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 __device__ __forceinline__ float act_p16(float x, const Act& a) { return __builtin_amdgcn_fmed3f(x, a.lo, a.hi) + a.leak * fminf(x, 0.f); }
+// An activation that is exact on halves -- none, or a clamp without leak whose bounds are fp16 values -- is applied to
+// the packed halves (two values per instruction, no conversions): act_half_exact says whether, act_half applies it.
+__device__ __forceinline__ bool act_half_exact(const Act& a, _Float16& lo, _Float16& hi) {
+    lo = (_Float16)fmaxf(a.lo, -65504.f);
+    hi = (_Float16)fminf(a.hi, 65504.f);
+    return a.leak == 0.f && (a.lo < -65504.f || (float)lo == a.lo) && (a.hi > 65504.f || (float)hi == a.hi);
+}
+__device__ __forceinline__ half8_t act_half(half8_t v, _Float16 lo, _Float16 hi) {
+    return __builtin_elementwise_min(__builtin_elementwise_max(v, (half8_t)lo), (half8_t)hi);
+}
+// The same on four halves, and with an item outside the tensor (ok false) reading as zeros.
+typedef _Float16 half4c_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ half4c_t act_half4(half4c_t v, _Float16 lo, _Float16 hi) {
+    return __builtin_elementwise_min(__builtin_elementwise_max(v, (half4c_t)lo), (half4c_t)hi);
+}
 // The same with the kind known (a wave-uniform choice made outside the loop over a lane's values): nothing for ACT_NONE,
 // one instruction for ACT_RELU, the general three otherwise.  Where a wave runs alone on its SIMD every vector
 // instruction costs four cycles, and a staging thread converts dozens of values.
