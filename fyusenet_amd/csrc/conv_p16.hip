@@ -808,7 +808,7 @@ struct GeoC4 {
     static_assert(2 * BUF + PLANE < 65536, "offsets fit the LDS instructions' immediate field");
 };
 
-template <class G>
+template <class G, bool C8>
 __device__ __forceinline__ void c4_stager(const ConvP16Params& p, unsigned char* lds, int stid, int cb, int group, int ntiles, unsigned range_bits) {
     constexpr int sb_off = 2 * G::BUF;
     const store_t* in = reinterpret_cast<const store_t*>(p.in);
@@ -870,8 +870,19 @@ __device__ __forceinline__ void c4_stager(const ConvP16Params& p, unsigned char*
                 }
                 *reinterpret_cast<half4_t*>(buf + l_off[i]) = hi;
                 *reinterpret_cast<half4_t*>(buf + G::COPY2 + 8 + l_off[i]) = hi;
-                *reinterpret_cast<half4_t*>(buf + G::PLANE + l_off[i]) = lo;
-                *reinterpret_cast<half4_t*>(buf + G::PLANE + G::COPY2 + 8 + l_off[i]) = lo;
+                if constexpr (C8) {
+                    // the pixel's fp8 operands of the correction terms: [4 x fp8(32 lo) | 4 x fp8(hi / 64)]
+                    int l8 = __builtin_amdgcn_cvt_pk_fp8_f32((float)lo[0] * 32.f, (float)lo[1] * 32.f, 0, false);
+                    l8 = __builtin_amdgcn_cvt_pk_fp8_f32((float)lo[2] * 32.f, (float)lo[3] * 32.f, l8, true);
+                    int h8 = __builtin_amdgcn_cvt_pk_fp8_f32((float)hi[0] * 0.015625f, (float)hi[1] * 0.015625f, 0, false);
+                    h8 = __builtin_amdgcn_cvt_pk_fp8_f32((float)hi[2] * 0.015625f, (float)hi[3] * 0.015625f, h8, true);
+                    const int2 c8 = int2{l8, h8};
+                    *reinterpret_cast<int2*>(buf + G::PLANE + l_off[i]) = c8;
+                    *reinterpret_cast<int2*>(buf + G::PLANE + G::COPY2 + 8 + l_off[i]) = c8;
+                } else {
+                    *reinterpret_cast<half4_t*>(buf + G::PLANE + l_off[i]) = lo;
+                    *reinterpret_cast<half4_t*>(buf + G::PLANE + G::COPY2 + 8 + l_off[i]) = lo;
+                }
             }
         }
     };
@@ -930,13 +941,79 @@ __device__ __forceinline__ void c4_stage(f32x4_t (&acc)[2][G::FN], half8_t (&a_q
 #pragma unroll
             for (int j = 0; j < NW; j++)
                 if (i == ((j * NSL) / NW + 1 < NSL ? (j * NSL) / NW + 1 : NSL - 1))
-                    a_q[dprev][j % 2][j / 2] = *reinterpret_cast<const half8_t*>(w_ + ((j % 2) * NPL + j / 2) * 1024 + wlane);
+                    a_q[dprev][j % 2][j / 2] = *reinterpret_cast<const half8_t*>(w_ + ((j % 2) * NPLW + j / 2) * 1024 + wlane);
             __builtin_amdgcn_sched_barrier(0);
         }
     }
 }
 
-template <int K, int TH, int TW>
+// The same stage with the correction terms as fp8 matrix instructions (see p16_stage_c8).  The second staged plane holds
+// per pixel [4 x fp8(32 lo) | 4 x fp8(hi / 64)], the third weight plane per tap [4 x fp8(hi / 32) | 4 x fp8(64 lo)]; one
+// v_mfma_f32_16x16x128_f8f6f4 takes the tap pairs of two consecutive steps.  Per pair of steps and fragment pair:
+// four fp16 MFMAs and two fp8 ones, 128 matrix-pipe cycles instead of 192.  The stage has an even number of steps, so
+// its last step is a pair step and the stage's barrier sits behind that step's first fp8 MFMA.
+template <class G, int BUFI>
+__device__ __forceinline__ void c4_stage_c8(f32x4_t (&acc)[2][G::FN], half8_t (&a0)[PD][2], i32x8_t (&a2)[PD / 2][2], half8_t (&b0)[G::FN], i32x8_t (&b1)[G::FN],
+                                            const int (&bbase)[G::FN], const int (&off)[G::NS], const unsigned char* lds, const unsigned char*& wnext,
+                                            const unsigned char* wbase, const unsigned char* wend, unsigned wstep, unsigned wlane) {
+    constexpr int FN = G::FN, NS = G::NS;
+    static_assert(NS % 2 == 0 && PD % 2 == 0, "pairs of steps");
+#pragma unroll
+    for (int dd = 0; dd < NS; dd++) {
+        const int d = (BUFI * NS + dd) % PD, dprev = (d + PD - 1) % PD;
+        const bool pair = (dd & 1) != 0;
+        const int nbuf = (dd + 1 == NS) ? 1 - BUFI : BUFI, ns = (dd + 1) % NS;
+        const unsigned char* w_ = wnext;
+        wnext += wstep;
+        if (wnext == wend) wnext = wbase;
+        // weights of step s + PD - 1 into the ring slot of step s - 1; every position fragment's operands of step s + 1
+        auto load_a0 = [&](int fm) { a0[dprev][fm] = *reinterpret_cast<const half8_t*>(w_ + (fm * NPLW) * 1024 + wlane); };
+        auto load_a2 = [&](int fm) {
+            const i32x4_t v = *reinterpret_cast<const i32x4_t*>(w_ + (fm * NPLW + 2) * 1024 + wlane);
+            if ((dprev & 1) == 0) { a2[dprev / 2][fm][0] = v[0]; a2[dprev / 2][fm][1] = v[1]; a2[dprev / 2][fm][2] = v[2]; a2[dprev / 2][fm][3] = v[3]; }
+            else { a2[dprev / 2][fm][4] = v[0]; a2[dprev / 2][fm][5] = v[1]; a2[dprev / 2][fm][6] = v[2]; a2[dprev / 2][fm][7] = v[3]; }
+        };
+        auto load_b0 = [&](int fn) { b0[fn] = *reinterpret_cast<const half8_t*>(lds + nbuf * G::BUF + bbase[fn] + off[ns]); };
+        auto load_b1 = [&](int fn) {
+            const i32x4_t v = *reinterpret_cast<const i32x4_t*>(lds + nbuf * G::BUF + bbase[fn] + off[ns] + G::PLANE);
+            if (pair) { b1[fn][0] = v[0]; b1[fn][1] = v[1]; b1[fn][2] = v[2]; b1[fn][3] = v[3]; }   // (the next step opens a pair)
+            else { b1[fn][4] = v[0]; b1[fn][5] = v[1]; b1[fn][6] = v[2]; b1[fn][7] = v[3]; }
+        };
+        if (pair) {
+#pragma unroll
+            for (int i = 0; i < 2 * FN; i++) {
+                const int fn = i / 2, fm = i % 2;
+                acc[fm][fn] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a2[d / 2][fm], b1[fn], acc[fm][fn], 0, 0, 0, 0, 0, 0);
+                if (dd == NS - 1 && i == 0) lds_barrier();
+                if (fm == 1) load_b1(fn);
+                if (i == 0) load_a0(0);
+                if (i == FN) load_a0(1);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < 2 * FN; i++) {
+            const int fn = i / 2, fm = i % 2;
+            acc[fm][fn] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0[d][fm], b0[fn], acc[fm][fn], 0, 0, 0);
+            if (fm == 1) {
+                load_b0(fn);
+                if (!pair) load_b1(fn);
+            }
+            if (pair) {
+                if (i == 0) load_a2(0);
+                if (i == FN) load_a2(1);
+            } else {
+                if (i == 0) load_a0(0);
+                if (i == FN / 2) load_a0(1);
+                if (i == FN) load_a2(0);
+                if (i == FN + FN / 2) load_a2(1);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+}
+
+template <int K, int TH, int TW, bool C8>
 __global__ __launch_bounds__(512) void conv_p16c4_kernel(const ConvP16Params p) {
     using G = GeoC4<K, TH, TW>;
     constexpr int FN = G::FN, NS = G::NS;
@@ -959,7 +1036,7 @@ __global__ __launch_bounds__(512) void conv_p16c4_kernel(const ConvP16Params p) 
     const unsigned range_bits = p.in_amax ? range_load(p.in_amax) : 0u;
     constexpr int sb_off = 2 * G::BUF;
     if (wave < 4) {
-        c4_stager<G>(p, lds, tid & 255, cb, group, ntiles, range_bits);
+        c4_stager<G, C8>(p, lds, tid & 255, cb, group, ntiles, range_bits);
         return;
     }
     const int mq = lane & 15, kq = lane >> 4;
@@ -979,17 +1056,29 @@ __global__ __launch_bounds__(512) void conv_p16c4_kernel(const ConvP16Params p) 
         const int row = pi / G::PPR, col = 2 * (pi - row * G::PPR);
         off[st] = pi < G::NPAIR ? row * G::ROW_PITCH + col * G::PIX : 0;
     }
-    const unsigned wstep = (unsigned)p.mfrags * NPL * 1024;
-    const unsigned char* wbase = reinterpret_cast<const unsigned char*>(p.wpack) + (size_t)(cb * 2 * NPL) * 1024;   // (uniform: the loads take it as their scalar base)
+    const unsigned wstep = (unsigned)p.mfrags * NPLW * 1024;
+    const unsigned char* wbase = reinterpret_cast<const unsigned char*>(p.wpack) + (size_t)(cb * 2 * NPLW) * 1024;   // (uniform: the loads take it as their scalar base)
     const unsigned wlane = lane * 16;
     const unsigned char* wend = wbase + (size_t)NS * wstep;
-    half8_t a_q[PD][2][NPL];
+    // weight ring: fp16 planes (hi, lo), or with the fp8 form the hi plane and the fp8 plane in pairs of steps
+    half8_t a_q[PD][2][C8 ? 1 : NPL];
+    half8_t a0[C8 ? PD : 1][2];
+    i32x8_t a2[C8 ? PD / 2 : 1][2];
 #pragma unroll
     for (int d = 0; d < PD; d++)
 #pragma unroll
-        for (int fm = 0; fm < 2; fm++)
+        for (int fm = 0; fm < 2; fm++) {
+            const unsigned char* wf = wbase + (size_t)(d % NS) * wstep + (fm * NPLW) * 1024 + wlane;   // (a stage of fewer steps than the ring holds: the next tile's)
+            if constexpr (C8) {
+                a0[d][fm] = *reinterpret_cast<const half8_t*>(wf);
+                const i32x4_t v = *reinterpret_cast<const i32x4_t*>(wf + 2 * 1024);
 #pragma unroll
-            for (int pl = 0; pl < NPL; pl++) a_q[d][fm][pl] = *reinterpret_cast<const half8_t*>(wbase + (size_t)(d % NS) * wstep + (fm * NPL + pl) * 1024 + wlane);   // (a stage of fewer steps than the ring holds: the next tile's)
+                for (int e = 0; e < 4; e++) a2[d / 2][fm][(d & 1) * 4 + e] = v[e];
+            } else {
+#pragma unroll
+                for (int pl = 0; pl < NPL; pl++) a_q[d][fm][pl] = *reinterpret_cast<const half8_t*>(wf + pl * 1024);
+            }
+        }
     f32x4_t acc[2][FN];
     auto zero_acc = [&]() {
 #pragma unroll
@@ -1043,20 +1132,38 @@ __global__ __launch_bounds__(512) void conv_p16c4_kernel(const ConvP16Params p) 
         }
     };
     lds_barrier();   // the first stage is staged
-    half8_t b[FN][NPL];
+    half8_t b[FN][C8 ? 1 : NPL];
+    i32x8_t b1[C8 ? FN : 1];
 #pragma unroll
-    for (int fn = 0; fn < FN; fn++)
+    for (int fn = 0; fn < FN; fn++) {
+        if constexpr (C8) {
+            b[fn][0] = *reinterpret_cast<const half8_t*>(lds + bbase[fn] + off[0]);
+            const i32x4_t v = *reinterpret_cast<const i32x4_t*>(lds + bbase[fn] + off[0] + G::PLANE);
 #pragma unroll
-        for (int pl = 0; pl < NPL; pl++) b[fn][pl] = *reinterpret_cast<const half8_t*>(lds + bbase[fn] + off[0] + pl * G::PLANE);
+            for (int e = 0; e < 4; e++) b1[fn][e] = v[e];
+        } else {
+#pragma unroll
+            for (int pl = 0; pl < NPL; pl++) b[fn][pl] = *reinterpret_cast<const half8_t*>(lds + bbase[fn] + off[0] + pl * G::PLANE);
+        }
+    }
     const unsigned char* wnext = wbase + (size_t)((PD - 1) % NS) * wstep;
     int tile = group;
+    auto stage = [&](auto bufi) {
+        constexpr int BUFI = decltype(bufi)::value;
+        if constexpr (C8) {
+            half8_t (&b0)[FN] = reinterpret_cast<half8_t (&)[FN]>(b);
+            c4_stage_c8<G, BUFI>(acc, a0, a2, b0, b1, bbase, off, lds, wnext, wbase, wend, wstep, wlane);
+        } else {
+            c4_stage<G, BUFI>(acc, a_q, b, bbase, off, lds, wnext, wbase, wend, wstep, wlane);
+        }
+    };
     for (;;) {
-        c4_stage<G, 0>(acc, a_q, b, bbase, off, lds, wnext, wbase, wend, wstep, wlane);
+        stage(std::integral_constant<int, 0>());
         finish_tile(tile);
         tile += p.pos_groups;
         if (tile >= ntiles) break;
         zero_acc();
-        c4_stage<G, 1>(acc, a_q, b, bbase, off, lds, wnext, wbase, wend, wstep, wlane);
+        stage(std::integral_constant<int, 1>());
         finish_tile(tile);
         tile += p.pos_groups;
         if (tile >= ntiles) break;
@@ -1639,12 +1746,16 @@ const TP16Entry kTEntries[] = {
 };
 struct C4Entry {
     int k, th, tw;
-    p16_fn fn;
+    p16_fn fn, fn8;   // three fp16 passes; fp8 correction terms (fp32 tensors, an even number of steps) or null
     size_t buf;
     int steps;
 };
 template <int K, int TH, int TW>
-constexpr C4Entry c4entry() { return C4Entry{K, TH, TW, conv_p16c4_kernel<K, TH, TW>, (size_t)GeoC4<K, TH, TW>::BUF, GeoC4<K, TH, TW>::NS}; }
+constexpr C4Entry c4entry() {
+    using G = GeoC4<K, TH, TW>;
+    if constexpr (!HSTORE && G::NS % 2 == 0) return C4Entry{K, TH, TW, conv_p16c4_kernel<K, TH, TW, false>, conv_p16c4_kernel<K, TH, TW, true>, (size_t)G::BUF, G::NS};
+    else return C4Entry{K, TH, TW, conv_p16c4_kernel<K, TH, TW, false>, nullptr, (size_t)G::BUF, G::NS};
+}
 const C4Entry kC4Entries[] = {c4entry<9, 8, 8>(), c4entry<9, 4, 8>(), c4entry<9, 8, 4>(), c4entry<3, 8, 8>(), c4entry<3, 4, 8>()};
 struct KREntry {
     int taps, cpw, fm, nfrag, th, tw, stride, dws, rounds, src;   // (cpw: chunks per wave and round)
@@ -1884,6 +1995,10 @@ int P16_NAME(launch_tconv_p16)(const ConvP16Params& p, hipStream_t s) {
     return hipGetLastError() == hipSuccess ? 0 : -3;
 }
 
+// (the fp8 form of the correction terms: as p16_uses_fp8, for the kernels whose stage has an even number of steps)
+static bool c4_uses_fp8(const ConvP16Params& p, const C4Entry* e) {
+    return !HSTORE && !p.f16 && !p.exact_split && p.in_amax != nullptr && e->fn8 != nullptr;
+}
 static const C4Entry* find_c4entry(const ConvP16Params& p, int k) {
     for (const C4Entry& c : kC4Entries)
         if (c.k == k && c.th == p.tile_h && c.tw == p.tile_w) return &c;
@@ -1914,8 +2029,16 @@ int P16_NAME(launch_conv_p16c4)(const ConvP16Params& p, int k, hipStream_t s) {
     const size_t lds_bytes = P16_NAME(conv_p16c4_lds_bytes)(p, k);
     if (lds_bytes > 160 * 1024) return -2;
     if (ensure_lds(reinterpret_cast<const void*>(e->fn), lds_bytes) != 0) return -2;
-    hipLaunchKernelGGL(e->fn, dim3(p.pos_groups * p.cout_blocks), dim3(512), lds_bytes, s, p);
+    const p16_fn fn = c4_uses_fp8(p, e) ? e->fn8 : e->fn;
+    if (fn != e->fn && ensure_lds(reinterpret_cast<const void*>(fn), lds_bytes) != 0) return -2;
+    hipLaunchKernelGGL(fn, dim3(p.pos_groups * p.cout_blocks), dim3(512), lds_bytes, s, p);
     return hipGetLastError() == hipSuccess ? 0 : -3;
 }
+#if !FYN_P16_HALF
+bool conv_p16c4_uses_fp8(const ConvP16Params& p, int k) {
+    const C4Entry* e = find_c4entry(p, k);
+    return e && c4_uses_fp8(p, e);
+}
+#endif
 
 }  // namespace fynhip

@@ -13,30 +13,36 @@
 // is fetched from memory once per strip, by four staging waves, four rows ahead of the four MFMA waves, each of which
 // computes one output row per round (K input rows, K*CS k16-steps).  The weights -- one fragment per step and plane --
 // stay in registers for the whole kernel, so the step loop reads nothing but the ring.
+//
+// fp32 tensors, whose operands are split into fp16 halves: hi*hi runs as fp16 matrix instructions; the two correction
+// terms (lo*hi + hi*lo, 2^-11 of the result) run either as two more fp16 passes over the lo planes or -- 32-channel rows
+// of an input that carries a value range -- as one v_mfma_f32_32x32x64_f8f6f4 per input row and fragment at twice the
+// fp16 rate: the second plane of the ring then holds, per column and eight channels, [8 x fp8(32 lo) | 8 x fp8(hi / 64)]
+// and the third weight plane [8 x fp8(hi / 32) | 8 x fp8(64 lo)], so that byte by byte the products are lo*hi and hi*lo
+// (p16_common.h; rel-L2 against the fp64 oracle 1e-5 instead of 3e-7).
 #include <hip/hip_fp16.h>
 #include <hip/hip_runtime.h>
 
 #include "kernels.h"
+#include "p16_common.h"
 #include "range.h"
 
 
 namespace fynhip {
 
 namespace {
-typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
 typedef float float16_t __attribute__((ext_vector_type(16)));
-typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef int i32x4_t __attribute__((ext_vector_type(4)));
+typedef int i32x8_t __attribute__((ext_vector_type(8)));
 
 constexpr int RING = 16;   // input rows resident per strip: K + 3 in use by a round, 4 being staged (K <= 9)
 // Floats per column of a wave's epilogue area [column][virtual channel]: odd, so that the lanes of a wave (one column
 // each) fall into distinct banks; cout*K <= 28 virtual channels are kept.
 constexpr int ROWS_SCRATCH_PITCH = 29;
 
-// Workgroup barrier that orders LDS traffic only: outstanding global loads (rows fetched two rounds ahead) and global
-// stores (finished output rows) stay in flight across it.  __syncthreads() would wait for them as well.
-__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
-
+// (lds_barrier() orders LDS traffic only: outstanding global loads -- rows fetched two rounds ahead -- and global stores
+// -- finished output rows -- stay in flight across it; __syncthreads() would wait for them as well.)
 __device__ __forceinline__ float act1r(float x, const Act& a) { return __builtin_amdgcn_fmed3f(x, a.lo, a.hi) + a.leak * fminf(x, 0.f); }
 
 // Eight channels of a staging item as they come from memory; they are converted when the item is written to the ring,
@@ -77,10 +83,12 @@ __device__ __forceinline__ int ring_off(int col, int chunk) {
     return col * (NCH * 16) + ((chunk ^ ((col / CPB) & (NCH - 1))) * 16);
 }
 
-template <typename TIn, typename TOut, bool SPLIT, int K, int CS, int FN>
+template <typename TIn, typename TOut, bool SPLIT, bool C8, int K, int CS, int FN>
 __global__ __launch_bounds__(512) void conv_rows_kernel(const ConvRowsParams p) {
     extern __shared__ __align__(16) unsigned char lds[];
+    static_assert(!C8 || (SPLIT && CS == 2), "the fp8 form pairs the two k16 steps of a 32-channel row");
     constexpr int NPL = SPLIT ? 2 : 1;
+    constexpr int NPLW = SPLIT ? 3 : 1;       // planes of a packed weight fragment
     constexpr int WC = 32 * FN;               // q columns per strip
     constexpr int OW = WC - (K - 1);          // output columns per strip
     constexpr int NCH = 2 * CS;
@@ -95,8 +103,17 @@ __global__ __launch_bounds__(512) void conv_rows_kernel(const ConvRowsParams p) 
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const bool mfma_wave = wave < 4;
-    const int strip = blockIdx.x % p.strips;
-    const int rblk = blockIdx.x / p.strips;
+    // Workgroups go to the chip's eight XCDs (one L2 each) in turn: workgroup b runs tile (b % 8) * ceil(tiles / 8) + b / 8,
+    // so that an XCD holds neighbouring strips and row blocks, whose input columns and rows overlap.
+    const int per_xcd = (p.strips * p.row_blocks + 7) >> 3;
+#ifdef FYN_ROWS_PLAIN_MAP
+    const int tile = blockIdx.x;
+#else
+    const int tile = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+#endif
+    if (tile >= p.strips * p.row_blocks) return;
+    const int strip = tile % p.strips;
+    const int rblk = tile / p.strips;
     const int y_begin = rblk * p.rows_per_block;
     const int y_end = min(y_begin + p.rows_per_block, p.out_h);
     const int x0 = strip * OW;                // first q column (= first output column) of the strip
@@ -158,7 +175,7 @@ __global__ __launch_bounds__(512) void conv_rows_kernel(const ConvRowsParams p) 
                 lo[e] = (_Float16)(a - (float)hi[e]);
             }
             *reinterpret_cast<half8_t*>(ring + bt.dst[i]) = hi;
-            if (SPLIT) *reinterpret_cast<half8_t*>(ring + bt.dst[i] + PLANE) = lo;
+            if (SPLIT) *reinterpret_cast<half8_t*>(ring + bt.dst[i] + PLANE) = C8 ? c8_plane(hi, lo) : lo;
         }
     };
 
@@ -180,13 +197,26 @@ __global__ __launch_bounds__(512) void conv_rows_kernel(const ConvRowsParams p) 
     if (!mfma_wave) fetch(nxt, 4 * NB0, NB0 < nbatches ? rows_of(NB0) : 0, stid, 256);
     // ---- weights: one fragment per step and plane, in registers from here on (placed behind the staging code so that
     //      the two never hold registers at the same point) ----
-    half8_t a_reg[NSTEPS][NPL];
+    // (fp8 form: the fp16 hi fragment of every step, and per input row the fp8 operands of channels 16g .. 16g + 15 for
+    // the lanes of half g = lane / 32: the halves 0 and 1 of the third plane of step sub = g)
+    constexpr int NPLA = C8 ? 1 : NPL;
+    half8_t a_reg[NSTEPS][NPLA];
+    i32x8_t a8[C8 ? K : 1];
     if (mfma_wave) {
         const half8_t* w = reinterpret_cast<const half8_t*>(p.wpack);
 #pragma unroll
         for (int t = 0; t < NSTEPS; t++)
 #pragma unroll
-            for (int pl = 0; pl < NPL; pl++) a_reg[t][pl] = w[(t * NPL + pl) * 64 + lane];
+            for (int pl = 0; pl < NPLA; pl++) a_reg[t][pl] = w[(t * NPLW + pl) * 64 + lane];
+        if constexpr (C8) {
+            const i32x4_t* w8 = reinterpret_cast<const i32x4_t*>(p.wpack);
+#pragma unroll
+            for (int ky = 0; ky < K; ky++) {
+                const int frag = ((ky * CS + (lane >> 5)) * NPLW + 2) * 64;
+                const i32x4_t u = w8[frag + (lane & 31)], v = w8[frag + 32 + (lane & 31)];
+                a8[ky] = i32x8_t{u[0], u[1], u[2], u[3], v[0], v[1], v[2], v[3]};
+            }
+        }
     }
     lds_barrier();
 
@@ -196,6 +226,12 @@ __global__ __launch_bounds__(512) void conv_rows_kernel(const ConvRowsParams p) 
     for (int sub = 0; sub < CS; sub++)
 #pragma unroll
         for (int fn = 0; fn < FN; fn++) boff[sub][fn] = ring_off<CS>(fn * 32 + (lane & 31), 2 * sub + (lane >> 5));
+    // fp8 form: the chunks 2g and 2g + 1 of the lane's column in the second plane
+    int coff[2][FN];
+#pragma unroll
+    for (int h = 0; h < 2; h++)
+#pragma unroll
+        for (int fn = 0; fn < FN; fn++) coff[h][fn] = PLANE + ring_off<CS>(fn * 32 + (lane & 31), (2 * (lane >> 5) + h) % NCH);
 
     float sc4[4], bi4[4];
 #pragma unroll
@@ -230,6 +266,43 @@ __global__ __launch_bounds__(512) void conv_rows_kernel(const ConvRowsParams p) 
                 for (int fn = 0; fn < FN; fn++)
 #pragma unroll
                     for (int r = 0; r < 16; r++) acc[fn][r] = 0.f;
+                if constexpr (C8) {
+                    // Per input row: FN fp16 MFMAs on each of its two k16 steps, then FN fp8 MFMAs on the whole row.  Every
+                    // operand buffer is refilled for the next row right behind the MFMA that read it (a memory
+                    // instruction issued behind an MFMA runs in its shadow), a row's worth of MFMAs ahead of its use.
+                    half8_t bh[CS][FN];
+                    i32x8_t bc[FN];
+                    auto row_of = [&](int ky) { return ring + ((yl + ky) & (RING - 1)) * ROWB; };
+                    auto load_h = [&](int ky, int sub, int fn) { bh[sub][fn] = *reinterpret_cast<const half8_t*>(row_of(ky) + boff[sub][fn]); };
+                    auto load_c = [&](int ky, int fn) {
+                        const i32x4_t u = *reinterpret_cast<const i32x4_t*>(row_of(ky) + coff[0][fn]);
+                        const i32x4_t v = *reinterpret_cast<const i32x4_t*>(row_of(ky) + coff[1][fn]);
+                        bc[fn] = i32x8_t{u[0], u[1], u[2], u[3], v[0], v[1], v[2], v[3]};
+                    };
+#pragma unroll
+                    for (int fn = 0; fn < FN; fn++) {
+#pragma unroll
+                        for (int sub = 0; sub < CS; sub++) load_h(0, sub, fn);
+                        load_c(0, fn);
+                    }
+#pragma unroll
+                    for (int ky = 0; ky < K; ky++) {
+#pragma unroll
+                        for (int sub = 0; sub < CS; sub++)
+#pragma unroll
+                            for (int fn = 0; fn < FN; fn++) {
+                                acc[fn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_reg[ky * CS + sub][0], bh[sub][fn], acc[fn], 0, 0, 0);
+                                if (ky + 1 < K) load_h(ky + 1, sub, fn);
+                                __builtin_amdgcn_sched_barrier(0);
+                            }
+#pragma unroll
+                        for (int fn = 0; fn < FN; fn++) {
+                            acc[fn] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a8[ky], bc[fn], acc[fn], 0, 0, 0, 0, 0, 0);
+                            if (ky + 1 < K) load_c(ky + 1, fn);
+                            __builtin_amdgcn_sched_barrier(0);
+                        }
+                    }
+                } else {
                 half8_t b[2][FN][NPL];
                 auto load_b = [&](int t, half8_t (&dst)[FN][NPL]) {
                     const int ky = t / CS, sub = t % CS;
@@ -251,7 +324,7 @@ __global__ __launch_bounds__(512) void conv_rows_kernel(const ConvRowsParams p) 
                     for (int i = 0; i < NMF; i++) {
                         const int kind = i / FN, fn = i % FN;
                         const int apl = (kind == 1) ? 1 : 0, bpl = (kind == 2) ? 1 : 0;
-                        acc[fn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_reg[t][apl], b[t & 1][fn][bpl], acc[fn], 0, 0, 0);
+                        acc[fn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_reg[t][C8 ? 0 : apl], b[t & 1][fn][bpl], acc[fn], 0, 0, 0);
                         if (t + 1 < NSTEPS) {
 #pragma unroll
                             for (int j = i * NDS / NMF; j < (i + 1) * NDS / NMF; j++)
@@ -259,6 +332,7 @@ __global__ __launch_bounds__(512) void conv_rows_kernel(const ConvRowsParams p) 
                         }
                         __builtin_amdgcn_sched_barrier(0);
                     }
+                }
                 }
                 // accumulators -> this wave's area [column][virtual channel]: a lane holds column lane%32 of each
                 // fragment and rows 8*(r/4) + 4*(lane/32) + r%4
@@ -332,14 +406,24 @@ __global__ __launch_bounds__(512) void conv_rows_kernel(const ConvRowsParams p) 
 typedef void (*rows_fn)(const ConvRowsParams);
 
 template <typename TIn, typename TOut, bool SPLIT, int FN>
-rows_fn pick_rows(int k, int cs) {
+rows_fn pick_rows(int k, int cs, bool c8) {
 #define FYN_ROWS(K_, CS_) \
-    if (k == K_ && cs == CS_) return conv_rows_kernel<TIn, TOut, SPLIT, K_, CS_, FN>;
+    if (k == K_ && cs == CS_ && !c8) return conv_rows_kernel<TIn, TOut, SPLIT, false, K_, CS_, FN>;
     FYN_ROWS(3, 1) FYN_ROWS(3, 2) FYN_ROWS(5, 1) FYN_ROWS(5, 2) FYN_ROWS(7, 1) FYN_ROWS(7, 2) FYN_ROWS(9, 1) FYN_ROWS(9, 2)
 #undef FYN_ROWS
+    if constexpr (SPLIT) {
+#define FYN_ROWS8(K_) \
+    if (k == K_ && cs == 2 && c8) return conv_rows_kernel<TIn, TOut, true, true, K_, 2, FN>;
+        FYN_ROWS8(3) FYN_ROWS8(5) FYN_ROWS8(7) FYN_ROWS8(9)
+#undef FYN_ROWS8
+    }
     return nullptr;
 }
 }  // namespace
+
+// fp32 tensors, 32-channel rows, an input with a value range (the fp8 operands need its scale), unless the layer asks
+// for the three fp16 passes.
+bool conv_rows_uses_fp8(const ConvRowsParams& p, bool f16) { return !f16 && p.cs == 2 && p.in_amax != nullptr && !p.exact_split; }
 
 bool conv_rows_supported(int k, int cin_pitch, int cout, bool f16) {
     (void)f16;
@@ -354,7 +438,7 @@ size_t conv_rows_lds_bytes(const ConvRowsParams& p, bool f16) {
 
 int launch_conv_rows(const ConvRowsParams& p, bool f16, hipStream_t s) {
     if (p.fn != 2) return -1;
-    rows_fn fn = f16 ? pick_rows<_Float16, _Float16, false, 2>(p.k, p.cs) : pick_rows<float, float, true, 2>(p.k, p.cs);
+    rows_fn fn = f16 ? pick_rows<_Float16, _Float16, false, 2>(p.k, p.cs, false) : pick_rows<float, float, true, 2>(p.k, p.cs, conv_rows_uses_fp8(p, f16));
     if (!fn) return -1;
     // what the kernel's indexing assumes
     if (p.cout * p.k > 28 || p.out_cp != 4 || p.strips < 1 || p.row_blocks < 1 || p.in_shift < 0 || p.in_shift > 8 ||
@@ -364,7 +448,7 @@ int launch_conv_rows(const ConvRowsParams& p, bool f16, hipStream_t s) {
     const size_t lds_bytes = conv_rows_lds_bytes(p, f16);
     if (lds_bytes > 160 * 1024) return -2;
     if (ensure_lds(reinterpret_cast<const void*>(fn), lds_bytes) != 0) return -2;
-    hipLaunchKernelGGL(fn, dim3(p.strips * p.row_blocks), dim3(512), lds_bytes, s, p);
+    hipLaunchKernelGGL(fn, dim3((p.strips * p.row_blocks + 7) / 8 * 8), dim3(512), lds_bytes, s, p);
     return hipGetLastError() == hipSuccess ? 0 : -3;
 }
 

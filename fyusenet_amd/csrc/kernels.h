@@ -134,7 +134,8 @@ struct ConvRowsParams {
     const void* in;
     void* out;
     const void* res;      // residual tensor or nullptr
-    const void* wpack;    // [k*cs steps][plane][lane 0..63][8 halves]: virtual channel o*k+kx = lane%32, input channel 16*sub + 8*(lane/32) + j
+    const void* wpack;    // [k*cs steps][plane][lane 0..63][8 halves]: virtual channel o*k+kx = lane%32, input channel 16*sub + 8*(lane/32) + j;
+                          // one plane with fp16 tensors, three with fp32 tensors (fp16 hi, fp16 lo, fp8 operands of the correction terms)
     const float* scale;   // [cout]
     const float* bias;    // [cout]
     int k, cs, fn;        // kernel size; k16 steps per input row (input channel pitch <= 16*cs); 32-column fragments per strip
@@ -148,6 +149,7 @@ struct ConvRowsParams {
     int strips, row_blocks, rows_per_block;   // grid = strips * row_blocks workgroups; rows_per_block is a multiple of 4
     int cout;
     float acc_mul;
+    int exact_split;      // fp32 tensors: three fp16 passes even where the fp8 form of the correction terms would run
     const unsigned* in_amax;   // value-range words as in ConvMfmaParams
     unsigned* out_amax;
     unsigned* reset[4];
@@ -158,6 +160,7 @@ int ensure_lds(const void* fn, size_t lds_bytes);   // 0, or -2 when the device 
 bool conv_rows_supported(int k, int cin_pitch, int cout, bool f16);
 size_t conv_rows_lds_bytes(const ConvRowsParams& p, bool f16);
 int launch_conv_rows(const ConvRowsParams& p, bool f16, hipStream_t s);
+bool conv_rows_uses_fp8(const ConvRowsParams& p, bool f16);   // the form launch_conv_rows runs
 
 // 3x3 convolution (stride 1 or 2) with fp32 storage on 16-position fragments (conv_p16.hip).  A workgroup's four MFMA
 // waves are wm groups of 32 output channels x 4/wm tiles of tile_h x tile_w positions side by side (compiled
@@ -228,6 +231,7 @@ size_t conv_p16_lds_bytes(const ConvP16Params& p);   // 0: no such compiled comb
 int launch_pack_fp8_plane(const float* src, void* wpack, size_t frags, hipStream_t s);
 int launch_conv_p16(const ConvP16Params& p, hipStream_t s);
 bool conv_p16_uses_fp8(const ConvP16Params& p);   // whether launch_conv_p16 runs the form with the correction terms as fp8 MFMAs
+bool conv_p16c4_uses_fp8(const ConvP16Params& p, int k);   // the same for launch_conv_p16c4
 // the transposed 3x3 convolution that doubles the image size, on the same parameters: positions (npos_y x npos_x,
 // tiles) are input pixels, out_off_* the stored coordinate of output pixel (0, 0), wpack holds the nine taps of a chunk
 // in the order of their input shift (conv_p16.hip: TT_KY / TT_KX)

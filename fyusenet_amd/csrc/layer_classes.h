@@ -239,6 +239,8 @@ class ConvLayer : public Layer {
         q.scale = scale_dev; q.bias = bias_dev;
         q.acc_mul = 1.f;
         q.act = act();
+        q.in_amax = tin(0).amax;   // (timed in the form the frame will run)
+        q.exact_split = net->sw.get("FYNHIP_EXACT_SPLIT") ? 1 : 0;
         int want_h = 0, want_w = 0;
         if (const char* e = net->sw.get("FYNHIP_P16_TILE")) sscanf(e, "%d,%d", &want_h, &want_w);
         std::vector<ConvP16Params> cands;
@@ -259,7 +261,7 @@ class ConvLayer : public Layer {
         }
         if (cands.empty()) return;
         c4_steps = steps;
-        const size_t halves = ((size_t)steps + 8) * q.mfrags * (q.f16 ? 1 : 2) * 64 * 8;
+        const size_t halves = ((size_t)steps + 8) * q.mfrags * (q.f16 ? 1 : 3) * 64 * 8;
         p16_wpack_dev = net->dev_alloc(halves * 2, true);
         for (ConvP16Params& c : cands) c.wpack = p16_wpack_dev;
         const bool always = net->sw.get("FYNHIP_FORCE_P16_CONV") != nullptr;
@@ -709,8 +711,11 @@ class ConvLayer : public Layer {
     // weights of that form: [step][cout fragment of 16][plane][lane][8 halves]; lane = (channel lane%16, tap pair 4*step + lane/16)
     void pack_c4(const float* w, float wmul) {
         const int cin = d.in_channels, ppr = (k + 1) / 2;
-        const int npl = pp.f16 ? 1 : 2;   // (fp16 tensors: the hi plane only)
-        std::vector<uint16_t> pack(((size_t)c4_steps + 8) * pp.mfrags * npl * 64 * 8, 0);
+        const int npl = pp.f16 ? 1 : 3;   // (fp16 tensors: the hi plane only; fp32: hi, lo, fp8 operands of the correction terms)
+        const size_t frags = ((size_t)c4_steps + 8) * pp.mfrags;
+        std::vector<uint16_t> pack(frags * npl * 64 * 8, 0);
+        // (sources of the third plane, per tap of a lane's pair: four hi parts / 32, then four lo parts * 64)
+        std::vector<float> c8(npl == 3 ? frags * 64 * 16 : 0, 0.f);
         for (int st = 0; st < c4_steps; st++)
             for (int mf = 0; mf < pp.mfrags; mf++) {
                 uint16_t* base = pack.data() + (((size_t)st * pp.mfrags + mf) * npl) * 64 * 8;
@@ -724,13 +729,17 @@ class ConvLayer : public Layer {
                         const float v = w[(((size_t)o * k + ky) * k + kx) * cin + ci] * wmul;
                         const uint16_t hi = f2h_bits(v);
                         base[(size_t)lane * 8 + j] = hi;
-                        if (npl == 2) base[(size_t)(64 + lane) * 8 + j] = f2h_bits(v - h2f(hi));
+                        if (npl == 3) {
+                            const float lo = v - h2f(hi);
+                            base[(size_t)(64 + lane) * 8 + j] = f2h_bits(lo);
+                            float* c8_lane = c8.data() + (((size_t)st * pp.mfrags + mf) * 64 + lane) * 16;
+                            c8_lane[(j / 4) * 8 + j % 4] = h2f(hi) * (1.0f / 32.0f);
+                            c8_lane[(j / 4) * 8 + 4 + j % 4] = lo * 64.0f;
+                        }
                     }
                 }
             }
-        FYN_HIP(hipStreamSynchronize(net->stream));
-        FYN_HIP(hipMemcpyAsync(p16_wpack_dev, pack.data(), pack.size() * 2, hipMemcpyHostToDevice, net->stream));
-        FYN_HIP(hipStreamSynchronize(net->stream));
+        upload_p16_pack(net, p16_wpack_dev, pack, c8, frags);
     }
     // weights of that form: [(chunk*9 + tap)][cout fragment of 16][plane][lane][8 halves], zero steps behind the last
     void pack_p16(const float* w, float wmul) {
@@ -787,7 +796,9 @@ class ConvLayer : public Layer {
         q.acc_mul = 1.f;
         q.act = act();
         if (conv_rows_lds_bytes(q, out_v.f16 != 0) > 160 * 1024) return;
-        const size_t halves = (size_t)k * q.cs * (out_v.f16 ? 1 : 2) * 64 * 8;
+        q.in_amax = tin(0).amax;   // (timed in the form the frame will run: fp8 correction terms where the input has a range word)
+        q.exact_split = net->sw.get("FYNHIP_EXACT_SPLIT") ? 1 : 0;
+        const size_t halves = (size_t)k * q.cs * (out_v.f16 ? 1 : 3) * 64 * 8;
         q.wpack = rows_wpack_dev = net->dev_alloc(halves * 2, true);
         const bool always = net->sw.get("FYNHIP_FORCE_ROWS_WIDE_CONV") != nullptr;
         const char* at = net->sw.get("FYNHIP_AUTOTUNE");
@@ -820,10 +831,13 @@ class ConvLayer : public Layer {
             rows_wpack_dev = nullptr;
         }
     }
-    // weights of the row-rolling form: [step = ky*cs + sub][plane][lane][8 halves]
+    // weights of the row-rolling form: [step = ky*cs + sub][plane][lane][8 halves]; fp32 tensors: fp16 hi, fp16 lo and the
+    // fp8 operands of the correction terms, as in the fragments of the 16-position forms
     void pack_rows(const float* w, float wmul) {
-        const int cin = d.in_channels, npl = tout().v.f16 ? 1 : 2;
-        std::vector<uint16_t> pack((size_t)k * rp.cs * npl * 64 * 8, 0);
+        const int cin = d.in_channels, npl = tout().v.f16 ? 1 : 3;
+        const size_t frags = (size_t)k * rp.cs;
+        std::vector<uint16_t> pack(frags * npl * 64 * 8, 0);
+        std::vector<float> c8(npl == 3 ? frags * 64 * 16 : 0, 0.f);
         for (int ky = 0; ky < k; ky++)
             for (int sub = 0; sub < rp.cs; sub++)
                 for (int lane = 0; lane < 64; lane++) {
@@ -834,14 +848,12 @@ class ConvLayer : public Layer {
                         if (ci >= cin) continue;
                         const float v = w[(((size_t)o * k + ky) * k + kx) * cin + ci] * wmul;
                         const uint16_t hi = f2h_bits(v);
-                        const size_t base = ((size_t)(ky * rp.cs + sub) * npl) * 64 * 8;
+                        const size_t frag = (size_t)(ky * rp.cs + sub), base = frag * npl * 64 * 8;
                         pack[base + (size_t)lane * 8 + j] = hi;
-                        if (npl == 2) pack[base + (size_t)(64 + lane) * 8 + j] = f2h_bits(v - h2f(hi));
+                        if (npl == 3) p16_lo_planes(pack.data() + base, c8.data() + (frag * 64 + lane) * 16, lane, j, v, hi);
                     }
                 }
-        FYN_HIP(hipStreamSynchronize(net->stream));
-        FYN_HIP(hipMemcpyAsync(rows_wpack_dev, pack.data(), pack.size() * 2, hipMemcpyHostToDevice, net->stream));
-        FYN_HIP(hipStreamSynchronize(net->stream));
+        upload_p16_pack(net, rows_wpack_dev, pack, c8, frags);
     }
     size_t weight_floats() const override {
         return (size_t)oc + (size_t)oc * k * k * d.in_channels + ((d.flags & FYN_FLAG_POST_BATCHNORM) ? 2 * (size_t)oc : 0);
@@ -1150,13 +1162,13 @@ class ConvLayer : public Layer {
         if (rows) {
             char buf[200];
             snprintf(buf, sizeof(buf), "conv_rows %s(kx folded into cout, rows rolled through an LDS ring) strips=%d x %d row blocks of %d rows, lds=%zu",
-                     tout().v.f16 ? "f16 " : "f16x2-split ", rp.strips, rp.row_blocks, rp.rows_per_block, conv_rows_lds_bytes(rp, tout().v.f16 != 0));
+                     tout().v.f16 ? "f16 " : (conv_rows_uses_fp8(rp, false) ? "f16+fp8-split " : "f16x2-split "), rp.strips, rp.row_blocks, rp.rows_per_block, conv_rows_lds_bytes(rp, tout().v.f16 != 0));
             return mode + buf;
         }
         if (p16 && c4) {
             char buf[220];
             snprintf(buf, sizeof(buf), "conv_p16c4 %s (tap pairs of a 4-channel pixel) tile=32x%d(cout x pos) th=%d tw=%d blocks=%d tiles=%d lds=%zu steps=%d",
-                     pp.f16 ? "f16" : "f16x2-split", pp.tile_h * pp.tile_w * 4, pp.tile_h, pp.tile_w, pp.pos_groups * pp.cout_blocks, pp.tiles_x * pp.tiles_y * pp.cout_blocks,
+                     pp.f16 ? "f16" : (conv_p16c4_uses_fp8(pp, k) ? "f16+fp8-split" : "f16x2-split"), pp.tile_h * pp.tile_w * 4, pp.tile_h, pp.tile_w, pp.pos_groups * pp.cout_blocks, pp.tiles_x * pp.tiles_y * pp.cout_blocks,
                      conv_p16c4_lds_bytes(pp, k), c4_steps);
             return mode + buf;
         }

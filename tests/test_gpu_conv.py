@@ -248,8 +248,17 @@ def test_wide_kernel_row_rolling_form(case, shallow, storage, monkeypatch):
     ref = oracle_single(b, storage, inputs, wts)
     err = rel_l2(got, ref)
     print("  ", info, "rel_l2=%.3e" % err, flush=True)
-    assert "conv_rows" in info
+    # (fp32 tensors: the correction terms of the operand split run as fp8 MFMAs on 32-channel rows)
+    fp8_form = storage == fa.STORAGE_F32 and cin > 16
+    assert ("conv_rows f16+fp8-split" if fp8_form else ("conv_rows f16x2-split" if storage == fa.STORAGE_F32 else "conv_rows f16 ")) in info
     assert err <= TOL[storage], info
+    if fp8_form and not shallow:
+        monkeypatch.setenv("FYNHIP_EXACT_SPLIT", "1")   # three fp16 passes
+        b2 = conv_builder(k, cout, h, w, cin, 1, 1, A.RELU, **kw)
+        exact, info2 = run_single(b2, storage, inputs, wts)
+        assert "conv_rows f16x2-split" in info2
+        assert rel_l2(exact, ref) <= 2e-6, info2
+        assert rel_l2(got, exact) <= 3e-5
 
 
 P16_CASES = [
@@ -717,10 +726,20 @@ def test_small_input_sixteen_position_fragment_form(case, shallow, storage, monk
     ref = oracle_single(b, storage, [x], wts)
     err = rel_l2(got, ref)
     print("  ", info, "rel_l2=%.3e" % err, flush=True)
-    assert "conv_p16c4 f16x2-split" in info if storage == fa.STORAGE_F32 else "conv_p16c4 f16 " in info
+    # (fp32 tensors: the correction terms of the operand split run as fp8 MFMAs where a stage has an even number of steps)
+    assert ("conv_p16c4 f16+fp8-split" if k == 9 else "conv_p16c4 f16x2-split") in info if storage == fa.STORAGE_F32 else "conv_p16c4 f16 " in info
     if tile:
         assert "th=%s tw=%s" % tuple(tile.split(",")) in info
     assert err <= TOL[storage], info
+    if storage == fa.STORAGE_F32 and k == 9 and not shallow:
+        # the same layer with three fp16 passes: fp32-class agreement with the oracle, and the two forms agree to what
+        # four-bit correction terms leave
+        monkeypatch.setenv("FYNHIP_EXACT_SPLIT", "1")
+        b2 = conv_builder(k, cout, h, w, cin, 1, 1, A.NONE, **kw)
+        exact, info2 = run_single(b2, storage, [x], wts)
+        assert "conv_p16c4 f16x2-split" in info2
+        assert rel_l2(exact, ref) <= 2e-6, info2
+        assert rel_l2(got, exact) <= 3e-5
 
 
 TP16_CASES = [
