@@ -872,11 +872,7 @@ __device__ __forceinline__ void c4_stager(const ConvP16Params& p, unsigned char*
                 *reinterpret_cast<half4_t*>(buf + G::COPY2 + 8 + l_off[i]) = hi;
                 if constexpr (C8) {
                     // the pixel's fp8 operands of the correction terms: [4 x fp8(32 lo) | 4 x fp8(hi / 64)]
-                    int l8 = __builtin_amdgcn_cvt_pk_fp8_f32((float)lo[0] * 32.f, (float)lo[1] * 32.f, 0, false);
-                    l8 = __builtin_amdgcn_cvt_pk_fp8_f32((float)lo[2] * 32.f, (float)lo[3] * 32.f, l8, true);
-                    int h8 = __builtin_amdgcn_cvt_pk_fp8_f32((float)hi[0] * 0.015625f, (float)hi[1] * 0.015625f, 0, false);
-                    h8 = __builtin_amdgcn_cvt_pk_fp8_f32((float)hi[2] * 0.015625f, (float)hi[3] * 0.015625f, h8, true);
-                    const int2 c8 = int2{l8, h8};
+                    const int2 c8 = int2{(int)c8_quad(lo[0], lo[1], lo[2], lo[3], 0.03125f), (int)c8_quad(hi[0], hi[1], hi[2], hi[3], 64.f)};
                     *reinterpret_cast<int2*>(buf + G::PLANE + l_off[i]) = c8;
                     *reinterpret_cast<int2*>(buf + G::PLANE + G::COPY2 + 8 + l_off[i]) = c8;
                 } else {

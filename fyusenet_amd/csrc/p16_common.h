@@ -81,17 +81,22 @@ __device__ __forceinline__ void split8(const float (&r)[8], bool ok, const Act& 
 // The second staged plane of the fp8 form of the correction terms, from the split halves of eight values:
 // [8 x fp8(32 lo) | 8 x fp8(hi / 64)] (e4m3, round to nearest even).  With hi below 2^14 and lo below 2^3 (the value
 // range's scale) both stay inside fp8's range, and values down to 2^-14 of the largest keep their four bits.
+// (v_cvt_scalef32_pk_fp8_f16 converts two halves divided by a power of two: one instruction per pair)
+typedef short c8_short2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 c8_half2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ unsigned c8_quad(_Float16 v0, _Float16 v1, _Float16 v2, _Float16 v3, float divisor) {
+    c8_short2_t w = {0, 0};
+    w = __builtin_amdgcn_cvt_scalef32_pk_fp8_f16(w, c8_half2_t{v0, v1}, divisor, false);
+    w = __builtin_amdgcn_cvt_scalef32_pk_fp8_f16(w, c8_half2_t{v2, v3}, divisor, true);
+    return __builtin_bit_cast(unsigned, w);
+}
 __device__ __forceinline__ half8_t c8_plane(const half8_t& hi, const half8_t& lo) {
     typedef unsigned u32x4_t __attribute__((ext_vector_type(4)));
     u32x4_t w;
 #pragma unroll
     for (int q = 0; q < 2; q++) {
-        int v = __builtin_amdgcn_cvt_pk_fp8_f32((float)lo[4 * q] * 32.f, (float)lo[4 * q + 1] * 32.f, 0, false);
-        v = __builtin_amdgcn_cvt_pk_fp8_f32((float)lo[4 * q + 2] * 32.f, (float)lo[4 * q + 3] * 32.f, v, true);
-        w[q] = (unsigned)v;
-        int u = __builtin_amdgcn_cvt_pk_fp8_f32((float)hi[4 * q] * 0.015625f, (float)hi[4 * q + 1] * 0.015625f, 0, false);
-        u = __builtin_amdgcn_cvt_pk_fp8_f32((float)hi[4 * q + 2] * 0.015625f, (float)hi[4 * q + 3] * 0.015625f, u, true);
-        w[2 + q] = (unsigned)u;
+        w[q] = c8_quad(lo[4 * q], lo[4 * q + 1], lo[4 * q + 2], lo[4 * q + 3], 0.03125f);
+        w[2 + q] = c8_quad(hi[4 * q], hi[4 * q + 1], hi[4 * q + 2], hi[4 * q + 3], 64.f);
     }
     return __builtin_bit_cast(half8_t, w);
 }
