@@ -842,6 +842,7 @@ __device__ __forceinline__ void c4_stager(const ConvP16Params& p, unsigned char*
             raw[SET][i] = *reinterpret_cast<const raw_t*>(in + (g_off[SET][i] >= 0 ? g_off[SET][i] : 0));
         }
     };
+    const bool plain_act = p.act.kind == ACT_NONE;   // (a first layer reads its input as it is)
     auto store = [&](auto set_, unsigned char* buf) {
         constexpr int SET = decltype(set_)::value;
 #pragma unroll
@@ -860,14 +861,15 @@ __device__ __forceinline__ void c4_stager(const ConvP16Params& p, unsigned char*
                 *reinterpret_cast<half4_t*>(buf + l_off[i]) = v;
                 *reinterpret_cast<half4_t*>(buf + G::COPY2 + 8 + l_off[i]) = v;
             } else {
+                // (the hi/lo split of a pair of values in four instructions, as in split8)
                 const float r[4] = {raw[SET][i].x, raw[SET][i].y, raw[SET][i].z, raw[SET][i].w};
-                half4_t hi, lo;
+                float x[4];
 #pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    const float v = ok ? act_p16(r[e], p.act) * in_scale : 0.f;
-                    hi[e] = (_Float16)v;
-                    lo[e] = (_Float16)(v - (float)hi[e]);
-                }
+                for (int e = 0; e < 4; e++) x[e] = ok ? (plain_act ? r[e] : act_p16(r[e], p.act)) : 0.f;
+                unsigned h0, l0, h1, l1;
+                split_pair(x[0], x[1], in_scale, h0, l0);
+                split_pair(x[2], x[3], in_scale, h1, l1);
+                const half4_t hi = __builtin_bit_cast(half4_t, uint2{h0, h1}), lo = __builtin_bit_cast(half4_t, uint2{l0, l1});
                 *reinterpret_cast<half4_t*>(buf + l_off[i]) = hi;
                 *reinterpret_cast<half4_t*>(buf + G::COPY2 + 8 + l_off[i]) = hi;
                 if constexpr (C8) {
@@ -1128,12 +1130,13 @@ __global__ __launch_bounds__(512) void conv_p16c4_kernel(const ConvP16Params p) 
         }
     };
     lds_barrier();   // the first stage is staged
-    half8_t b[FN][C8 ? 1 : NPL];
-    i32x8_t b1[C8 ? FN : 1];
+    half8_t b[C8 ? 1 : FN][NPL];   // exact form: hi and lo fragments of a step
+    half8_t b0[C8 ? FN : 1];       // fp8 form: hi fragments ...
+    i32x8_t b1[C8 ? FN : 1];       // ... and the fp8 fragments of a pair of steps
 #pragma unroll
     for (int fn = 0; fn < FN; fn++) {
         if constexpr (C8) {
-            b[fn][0] = *reinterpret_cast<const half8_t*>(lds + bbase[fn] + off[0]);
+            b0[fn] = *reinterpret_cast<const half8_t*>(lds + bbase[fn] + off[0]);
             const i32x4_t v = *reinterpret_cast<const i32x4_t*>(lds + bbase[fn] + off[0] + G::PLANE);
 #pragma unroll
             for (int e = 0; e < 4; e++) b1[fn][e] = v[e];
@@ -1147,7 +1150,6 @@ __global__ __launch_bounds__(512) void conv_p16c4_kernel(const ConvP16Params p) 
     auto stage = [&](auto bufi) {
         constexpr int BUFI = decltype(bufi)::value;
         if constexpr (C8) {
-            half8_t (&b0)[FN] = reinterpret_cast<half8_t (&)[FN]>(b);
             c4_stage_c8<G, BUFI>(acc, a0, a2, b0, b1, bbase, off, lds, wnext, wbase, wend, wstep, wlane);
         } else {
             c4_stage<G, BUFI>(acc, a_q, b, bbase, off, lds, wnext, wbase, wend, wstep, wlane);
