@@ -123,6 +123,36 @@ __device__ __forceinline__ FV<V> actv(FV<V> r, const Act& a) {
     } while (0)
 
 static inline dim3 grid1d(size_t n, int block) { return dim3((unsigned)((n + block - 1) / block)); }
+// A thread's pixel and channel group in the element-wise kernels.  grid_rows() gives one grid row per tensor row where a
+// row fills at least a workgroup and the height fits the grid's second dimension: the index arithmetic is then one
+// 32-bit division instead of three 64-bit ones, which were most of the instructions of a thread that moves 16 bytes.
+struct PixelIndex {
+    int y, x, g;
+    bool inside;
+};
+__device__ __forceinline__ PixelIndex pixel_index(int h, int w, int cg) {
+    PixelIndex r;
+    if (gridDim.y > 1) {
+        const unsigned i = blockIdx.x * 256u + threadIdx.x;
+        r.inside = i < (unsigned)w * (unsigned)cg;
+        r.y = (int)blockIdx.y;
+        r.x = (int)(i / (unsigned)cg);
+        r.g = (int)(i - (unsigned)r.x * (unsigned)cg);
+    } else {
+        const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+        r.inside = idx < (size_t)h * w * cg;
+        r.g = (int)(idx % cg);
+        const size_t pix = idx / cg;
+        r.x = (int)(pix % w);
+        r.y = (int)(pix / w);
+    }
+    return r;
+}
+static inline dim3 grid_rows(int h, int w, int cg) {
+    const long long row = (long long)w * cg;
+    if (h > 1 && h <= 65535 && row >= 256 && row < (1ll << 31)) return dim3((unsigned)((row + 255) / 256), (unsigned)h);
+    return grid1d((size_t)h * w * cg, 256);
+}
 
 // ---------------------------------------------------------------------------------------------
 // depthwise 3x3  (DeepDepthwiseConvLayer3x3::forward, gpu/deep/deepdwconvlayer3x3.cpp:67-102;
@@ -430,12 +460,9 @@ void launch_dwconv3x3(const DwConvParams& p, hipStream_t s) {
 template <typename T, int V, int P>
 __global__ __launch_bounds__(256) void pool_kernel(const PoolParams p) {
     const int cg = p.out.cp / V;
-    const size_t n = (size_t)p.out.h * p.out.w * cg;
-    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
-    if (idx >= n) return;
-    const int g = (int)(idx % cg);
-    const size_t pix = idx / cg;
-    const int x = (int)(pix % p.out.w), y = (int)(pix / p.out.w);
+    const PixelIndex pi = pixel_index(p.out.h, p.out.w, cg);
+    if (!pi.inside) return;
+    const int g = pi.g, x = pi.x, y = pi.y;
     const int c = g * V;
     const T* in = reinterpret_cast<const T*>(p.in.ptr);
     const int iwp = p.in.wp(), ihp = p.in.hp();
@@ -477,10 +504,10 @@ __global__ __launch_bounds__(256) void pool_kernel(const PoolParams p) {
 template <int P>
 static void launch_pool_p(const PoolParams& p, hipStream_t s) {
     const bool wide = (p.in.cp % 8 == 0) && (p.out.cp % 8 == 0);
-    const size_t n = (size_t)p.out.h * p.out.w * (p.out.cp / ((p.out.f16 && wide) ? 8 : 4));
-    if (p.out.f16 && wide) hipLaunchKernelGGL((pool_kernel<_Float16, 8, P>), grid1d(n, 256), dim3(256), 0, s, p);
-    else if (p.out.f16) hipLaunchKernelGGL((pool_kernel<_Float16, 4, P>), grid1d(n, 256), dim3(256), 0, s, p);
-    else hipLaunchKernelGGL((pool_kernel<float, 4, P>), grid1d(n, 256), dim3(256), 0, s, p);
+    const dim3 grid = grid_rows(p.out.h, p.out.w, p.out.cp / ((p.out.f16 && wide) ? 8 : 4));
+    if (p.out.f16 && wide) hipLaunchKernelGGL((pool_kernel<_Float16, 8, P>), grid, dim3(256), 0, s, p);
+    else if (p.out.f16) hipLaunchKernelGGL((pool_kernel<_Float16, 4, P>), grid, dim3(256), 0, s, p);
+    else hipLaunchKernelGGL((pool_kernel<float, 4, P>), grid, dim3(256), 0, s, p);
 }
 void launch_pool(const PoolParams& p, hipStream_t s) {
     if (p.pool == 2) launch_pool_p<2>(p, s);
@@ -594,12 +621,9 @@ void launch_global_pool(const TView& in, const TView& out, int is_max, const Act
 template <typename T, int V>
 __global__ __launch_bounds__(256) void batchnorm_kernel(const BnParams p) {
     const int cg = p.out.cp / V;
-    const size_t n = (size_t)p.out.h * p.out.w * cg;
-    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
-    if (idx >= n) return;
-    const int g = (int)(idx % cg);
-    const size_t pix = idx / cg;
-    const int x = (int)(pix % p.out.w), y = (int)(pix / p.out.w);
+    const PixelIndex pi = pixel_index(p.out.h, p.out.w, cg);
+    if (!pi.inside) return;
+    const int g = pi.g, x = pi.x, y = pi.y;
     const int c = g * V;
     FV<V> v = actv<V>(ldv<T, V>(reinterpret_cast<const T*>(p.in.ptr) + tv_off(p.in, y, x) + c), p.act);
     const FV<V> sc = ldv<float, V>(p.scale + c), bi = ldv<float, V>(p.bias + c);
@@ -620,8 +644,7 @@ __global__ __launch_bounds__(256) void batchnorm_kernel(const BnParams p) {
 }
 void launch_batchnorm(const BnParams& p, hipStream_t s) {
     const bool wide = (p.in.cp % 8 == 0) && (p.out.cp % 8 == 0) && (!p.res.ptr || p.res.cp % 8 == 0);
-    const size_t n = (size_t)p.out.h * p.out.w * (p.out.cp / ((p.out.f16 && wide) ? 8 : 4));
-    FYN_DISPATCH_TV(p.out.f16, wide, batchnorm_kernel, grid1d(n, 256), dim3(256), s, p);
+    FYN_DISPATCH_TV(p.out.f16, wide, batchnorm_kernel, grid_rows(p.out.h, p.out.w, p.out.cp / ((p.out.f16 && wide) ? 8 : 4)), dim3(256), s, p);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -786,7 +809,44 @@ __global__ __launch_bounds__(256) void func_up2_kernel(const FuncParams p) {
         for (int j = 0; j < 2; j++)
             if (y0 + i < p.out.h && x0 + j < p.out.w) stv<T, V>(reinterpret_cast<T*>(p.out.ptr) + tv_off(p.out, y0 + i, x0 + j) + c, v[i][j]);
 }
+// The same size in and out (the scaling map's steps equal and its offsets inside a texel): output texel (y, x) reads
+// source texel (y, x).  One grid row per image row and 32-bit indices inside it, so that a thread's index arithmetic is
+// a shift or one short division -- in func_kernel it is most of the instructions of a thread that moves 16 bytes in
+// and 16 out, and holds a transcendental function like the sigmoid under the memory's speed.
+template <typename T, int V>
+__global__ __launch_bounds__(256) void func_same_kernel(const FuncParams p, int cg_shift) {
+    const int cg = p.out.cp / V;
+    const unsigned i = blockIdx.x * 256u + threadIdx.x;
+    if (i >= (unsigned)(p.out.w * cg)) return;
+    const int y = blockIdx.y;
+    const int x = cg_shift >= 0 ? (int)(i >> cg_shift) : (int)(i / (unsigned)cg);
+    const int c = ((int)i - x * cg) * V;
+    FV<V> v = zerov<V>();
+    if (c < p.in.cp) v = fetch_clamped_v<T, V>(p.in, y + p.in.pad, x + p.in.pad, c);
+    v = actv<V>(v, p.act);
+    if (p.fn != FFN_COPY) {
+#pragma unroll
+        for (int e = 0; e < V; e++) v.v[e] = func1(v.v[e], p.fn, p.op, p.operand);
+    }
+    if (c + V > p.out.c) {
+#pragma unroll
+        for (int e = 0; e < V; e++)
+            if (c + e >= p.out.c) v.v[e] = 0.f;
+    }
+    stv<T, V>(reinterpret_cast<T*>(p.out.ptr) + tv_off(p.out, y, x) + c, v);
+}
 void launch_func(const FuncParams& p, hipStream_t s) {
+    if (p.map == FMAP_SCALE && p.fn != FFN_BGR && p.dx == p.ux && p.dy == p.uy && p.ox > -p.ux && p.ox <= p.ux && p.oy > -p.uy && p.oy <= p.uy &&
+        p.out.h <= 65535 && (long long)p.out.w * p.out.cp < (1ll << 30)) {
+        const bool wide = (p.in.cp % 8 == 0) && (p.out.cp % 8 == 0);
+        const int cg = p.out.cp / ((p.out.f16 && wide) ? 8 : 4);
+        int shift = -1;
+        for (int b = 0; b < 16; b++)
+            if ((1 << b) == cg) shift = b;
+        const dim3 grid((unsigned)(((size_t)p.out.w * cg + 255) / 256), (unsigned)p.out.h);
+        FYN_DISPATCH_TV(p.out.f16, wide, func_same_kernel, grid, dim3(256), s, p, shift);
+        return;
+    }
     if (p.map == FMAP_SCALE && p.ux == 2 && p.uy == 2 && p.dx == 1 && p.dy == 1 && p.fn != FFN_BGR) {
         const bool wide2 = (p.in.cp % 8 == 0) && (p.out.cp % 8 == 0);
         const size_t n2 = (size_t)((p.out.h + 1) / 2) * ((p.out.w + 1) / 2) * (p.out.cp / ((p.out.f16 && wide2) ? 8 : 4));
@@ -879,12 +939,9 @@ void launch_blur(const TView& in, const TView& out, const float* coef, int r, in
 template <typename T, int V>
 __global__ __launch_bounds__(256) void addsub_kernel(const TView a, const TView b, const TView out, int sub, const Act act) {
     const int cg = out.cp / V;
-    const size_t n = (size_t)out.h * out.w * cg;
-    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
-    if (idx >= n) return;
-    const int g = (int)(idx % cg);
-    const size_t pix = idx / cg;
-    const int x = (int)(pix % out.w), y = (int)(pix / out.w);
+    const PixelIndex pi = pixel_index(out.h, out.w, cg);
+    if (!pi.inside) return;
+    const int g = pi.g, x = pi.x, y = pi.y;
     const int c = g * V;
     const FV<V> u = actv<V>(ldv<T, V>(reinterpret_cast<const T*>(a.ptr) + tv_off(a, y, x) + c), act);
     const FV<V> v = actv<V>(ldv<T, V>(reinterpret_cast<const T*>(b.ptr) + tv_off(b, y, x) + c), act);
@@ -895,8 +952,7 @@ __global__ __launch_bounds__(256) void addsub_kernel(const TView a, const TView 
 }
 void launch_addsub(const TView& a, const TView& b, const TView& out, int sub, const Act& act, hipStream_t s) {
     const bool wide = (a.cp % 8 == 0) && (b.cp % 8 == 0) && (out.cp % 8 == 0);
-    const size_t n = (size_t)out.h * out.w * (out.cp / ((out.f16 && wide) ? 8 : 4));
-    FYN_DISPATCH_TV(out.f16, wide, addsub_kernel, grid1d(n, 256), dim3(256), s, a, b, out, sub, act);
+    FYN_DISPATCH_TV(out.f16, wide, addsub_kernel, grid_rows(out.h, out.w, out.cp / ((out.f16 && wide) ? 8 : 4)), dim3(256), s, a, b, out, sub, act);
 }
 
 // Channel offsets that are not multiples of the vector width (the "component shift" case of deepconcat.frag) are
@@ -904,12 +960,9 @@ void launch_addsub(const TView& a, const TView& b, const TView& out, int sub, co
 template <typename T, int V>
 __global__ __launch_bounds__(256) void concat_kernel(const TView in, const TView out, int c_off, const Act act, int zero_to) {
     const int cg = (in.c + V - 1) / V;
-    const size_t n = (size_t)out.h * out.w * cg;
-    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
-    if (idx >= n) return;
-    const int g = (int)(idx % cg);
-    const size_t pix = idx / cg;
-    const int x = (int)(pix % out.w), y = (int)(pix / out.w);
+    const PixelIndex pi = pixel_index(out.h, out.w, cg);
+    if (!pi.inside) return;
+    const int g = pi.g, x = pi.x, y = pi.y;
     const int c = g * V;
     const T* src = reinterpret_cast<const T*>(in.ptr) + tv_off(in, y, x) + c;
     T* dst = reinterpret_cast<T*>(out.ptr) + tv_off(out, y, x) + c_off + c;
@@ -927,8 +980,7 @@ __global__ __launch_bounds__(256) void concat_kernel(const TView in, const TView
 void launch_concat_part(const TView& in, const TView& out, int c_off, const Act& act, hipStream_t s, bool last) {
     const bool wide = (in.cp % 8 == 0) && (out.cp % 8 == 0);
     const int v = (out.f16 && wide) ? 8 : 4;
-    const size_t n = (size_t)out.h * out.w * ((in.c + v - 1) / v);
-    FYN_DISPATCH_TV(out.f16, wide, concat_kernel, grid1d(n, 256), dim3(256), s, in, out, c_off, act, last ? out.cp : 0);
+    FYN_DISPATCH_TV(out.f16, wide, concat_kernel, grid_rows(out.h, out.w, (in.c + v - 1) / v), dim3(256), s, in, out, c_off, act, last ? out.cp : 0);
 }
 
 // ---------------------------------------------------------------------------------------------
