@@ -99,9 +99,10 @@ def test_batchnorm_parity(c, h, w, res, storage):
 
 @STORAGES
 @pytest.mark.parametrize("sub", [False, True])
-def test_addsub_parity(sub, storage):
-    b = fa.GPULayerBuilder("add").type(fa.LayerType.SUB if sub else fa.LayerType.ADD).number(1).shape(24, 30, 40, 24)
-    xs = [prng.normal(70, (24, 30, 40)), prng.normal(71, (24, 30, 40))]
+@pytest.mark.parametrize("c,h,w", [(24, 30, 40), (20, 5, 333)], ids=["24x30x40", "wide-rows"])   # (rows of 256 items and more take their indices from a 2-D grid)
+def test_addsub_parity(sub, c, h, w, storage):
+    b = fa.GPULayerBuilder("add").type(fa.LayerType.SUB if sub else fa.LayerType.ADD).number(1).shape(c, h, w, c)
+    xs = [prng.normal(70, (c, h, w)), prng.normal(71, (c, h, w))]
     got, _ = run_single(b, storage, xs)
     ref = oracle_single(b, storage, xs)
     assert rel_l2(got, ref) <= TOL[storage]
@@ -109,17 +110,18 @@ def test_addsub_parity(sub, storage):
 
 @STORAGES
 @pytest.mark.parametrize("chans,relu", [([32, 32], False), ([23, 52], False), ([3, 5, 12], True), ([8, 4, 4, 16], False)])
-def test_concat_bit_exact(chans, relu, storage):
+@pytest.mark.parametrize("w,h", [(28, 20), (301, 6)], ids=["28x20", "wide-rows"])   # (rows of 256 items and more take their indices from a 2-D grid)
+def test_concat_bit_exact(chans, relu, w, h, storage):
     b = fa.ConcatLayerBuilder("cat").number(1).deep()
     flags = fa.LayerFlags.PRE_RELU if relu else fa.LayerFlags.NO_LAYER_FLAGS
     for c in chans:
         b.input(c, 0, flags)
-    b.size(28, 20)
+    b.size(w, h)
     b.outputChannels_ = sum(chans)
-    xs = [prng.normal(80 + i, (c, 20, 28)) for i, c in enumerate(chans)]
+    xs = [prng.normal(80 + i, (c, h, w)) for i, c in enumerate(chans)]
     got, _ = run_single(b, storage, xs)
     ref = oracle_single(b, storage, xs)
-    assert got.shape == (sum(chans), 20, 28)
+    assert got.shape == (sum(chans), h, w)
     assert np.array_equal(got, ref)
 
 
