@@ -470,6 +470,8 @@ __global__ __launch_bounds__(512) void conv_p16_kernel(const ConvP16Params p) {
     const float acc_mul = p.acc_mul * inv_in_scale;
     store_t* out = reinterpret_cast<store_t*>(p.out);
     const bool have_res = p.res != nullptr;
+    const bool through = store_through_pays(p.out, p.npos_y, p.npos_x, p.out_cp * ESZ, p.cout_blocks == 1 && !p.plain_stores, hw_block_count());
+    bool drop = through && wave == 4 && hw_block_id() < 8;
     const bool res_scale = p.res_scale != 0;
     const float res_floor = p.res_relu ? 0.f : -__builtin_inff();
     float vmax = 0.f;
@@ -478,6 +480,10 @@ __global__ __launch_bounds__(512) void conv_p16_kernel(const ConvP16Params p) {
     // wave per SIMD pays four cycles per vector instruction, so the arithmetic is kept short (acc_mul is a power of two:
     // folding it into the scale changes no bit) and every fragment is stored as soon as it is finished.
     auto finish_tile = [&](int tile) {
+        if (drop) {   // (ahead of this workgroup's first store: what it has read so far may go as well)
+            drop_clean_l2_lines();
+            drop = false;
+        }
         const int tyi = (int)(((float)tile + 0.5f) * p.rcp_tiles_x), txi = tile - tyi * p.tiles_x;
         const float* sb = reinterpret_cast<const float*>(lds + sb_off);
         f32x4_t rs[2], bi[2], scm[2];
@@ -521,11 +527,11 @@ __global__ __launch_bounds__(512) void conv_p16_kernel(const ConvP16Params p) {
                 if constexpr (HSTORE) {
 #pragma unroll
                     for (int e = 0; e < 4; e++) hv[fm * 4 + e] = (_Float16)v[e];
-                    if (fm == 1 && ok) *reinterpret_cast<half8_t*>(out + obase) = hv;   // the lane's eight channels in one store
+                    if (fm == 1 && ok) store_out(through, reinterpret_cast<half8_t*>(out + obase), hv);   // the lane's eight channels in one store
                 } else {
 #pragma unroll
                     for (int e = 0; e < 4; e++) fmax_ = fmaxf(fmax_, ok ? fabsf(v[e]) : 0.f);
-                    if (ok) *reinterpret_cast<f32x4_t*>(out + obase + fm * CHF) = v;
+                    if (ok) store_out(through, reinterpret_cast<f32x4_t*>(out + obase + fm * CHF), v);
                 }
             }
             vmax = fmaxf(vmax, fmax_);
@@ -705,8 +711,14 @@ __global__ __launch_bounds__(512) void tconv_p16_kernel(const ConvP16Params p) {
     if (p.in_amax) (void)range_scale(range_after_act(range_reduce(range_bits), p.act), &inv_in_scale);
     const float acc_mul = p.acc_mul * inv_in_scale;
     store_t* out = reinterpret_cast<store_t*>(p.out);
+    const bool through = store_through_pays(p.out, 2 * p.npos_y, 2 * p.npos_x, p.out_cp * ESZ, p.cout_blocks == 1 && !p.plain_stores, hw_block_count());
+    bool drop = through && wave == 4 && hw_block_id() < 8;
     float vmax = 0.f;
     auto finish_tile = [&](int tile) {
+        if (drop) {   // (ahead of this workgroup's first store: what it has read so far may go as well)
+            drop_clean_l2_lines();
+            drop = false;
+        }
         const int tyi = (int)(((float)tile + 0.5f) * p.rcp_tiles_x), txi = tile - tyi * p.tiles_x;
         const float* sb = reinterpret_cast<const float*>(lds + sb_off);
         f32x4_t bi[2], scm[2];
@@ -738,9 +750,9 @@ __global__ __launch_bounds__(512) void tconv_p16_kernel(const ConvP16Params p) {
                     if constexpr (HSTORE) {
 #pragma unroll
                         for (int e = 0; e < 4; e++) hv[fm * 4 + e] = (_Float16)v[e];
-                        if (fm == 1 && ok) *reinterpret_cast<half8_t*>(out + o) = hv;
+                        if (fm == 1 && ok) store_out(through, reinterpret_cast<half8_t*>(out + o), hv);
                     } else {
-                        if (ok) *reinterpret_cast<f32x4_t*>(out + o + fm * CHF) = v;
+                        if (ok) store_out(through, reinterpret_cast<f32x4_t*>(out + o + fm * CHF), v);
                     }
                 }
             }
@@ -1089,8 +1101,14 @@ __global__ __launch_bounds__(512) void conv_p16c4_kernel(const ConvP16Params p) 
     if (p.in_amax) (void)range_scale(range_after_act(range_reduce(range_bits), p.act), &inv_in_scale);
     const float acc_mul = p.acc_mul * inv_in_scale;
     store_t* out = reinterpret_cast<store_t*>(p.out);
+    const bool through = store_through_pays(p.out, p.npos_y, p.npos_x, p.out_cp * ESZ, p.cout_blocks == 1 && !p.plain_stores, hw_block_count());
+    bool drop = through && wave == 4 && hw_block_id() < 8;
     float vmax = 0.f;
     auto finish_tile = [&](int tile) {
+        if (drop) {   // (ahead of this workgroup's first store: what it has read so far may go as well)
+            drop_clean_l2_lines();
+            drop = false;
+        }
         const int tyi = (int)(((float)tile + 0.5f) * p.rcp_tiles_x), txi = tile - tyi * p.tiles_x;
         const float* sb = reinterpret_cast<const float*>(lds + sb_off);
         f32x4_t bi[2], scm[2];
@@ -1121,9 +1139,9 @@ __global__ __launch_bounds__(512) void conv_p16c4_kernel(const ConvP16Params p) 
                 if constexpr (HSTORE) {
 #pragma unroll
                     for (int e = 0; e < 4; e++) hv[fm * 4 + e] = (_Float16)v[e];
-                    if (fm == 1 && ok) *reinterpret_cast<half8_t*>(out + obase) = hv;
+                    if (fm == 1 && ok) store_out(through, reinterpret_cast<half8_t*>(out + obase), hv);
                 } else {
-                    if (ok) *reinterpret_cast<f32x4_t*>(out + obase + fm * CHF) = v;
+                    if (ok) store_out(through, reinterpret_cast<f32x4_t*>(out + obase + fm * CHF), v);
                 }
             }
             vmax = fmaxf(vmax, fmax_);

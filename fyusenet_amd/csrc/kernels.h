@@ -17,6 +17,51 @@ struct Act {
     float leak, lo, hi;
 };
 
+// Output stores that are written through the XCD's L2 as they are issued (sc1: visible at device scope) instead of
+// staying dirty there until the write-back at the kernel's end.  A kernel's stores then overlap the work of the
+// workgroups that are still computing, and the next launch does not wait behind the write-back of a whole output
+// tensor (measured: 1.2 to 3.5 us per launch on outputs of 10 to 40 MB).  The line stays cached as with a plain store
+// (no streaming hint: the consumer reads it next).
+//
+// What such a store does not take part in is the bookkeeping that keeps the eight L2s of the chip consistent for plain
+// stores.  Observed: kernels that wrote through pieces of 64 bytes, where two workgroups on two XCDs share a 128-byte
+// line, left later launches reading an old half of such lines now and then (whole networks off by O(1), differently
+// from pass to pass); a buffer_inv sc1 in every wave of every kernel made the results stable again (and the frames
+// 1.7x slower).  A kernel therefore writes through only where (1) every 128-byte line of the output is stored whole by
+// one workgroup (a pixel is whole lines and all its channels come from one workgroup), (2) the launch has at least
+// eight workgroups, and (3) its workgroups 0..7 -- consecutive workgroups are dealt to consecutive XCDs, so these sit
+// on all eight -- drop the clean lines of their L2 once during the launch (the acquire half of device-scope
+// visibility: copies of the buffer's earlier contents that other XCDs may hold; nothing in the kernel reads the
+// output buffer, so none appears after that).  With (1) and (2) alone no stale read was seen either; (3) costs 1 % of
+// the style net's frame and stays.  Everything else stores plainly.  Outputs beyond kStoreThroughMaxBytes do so as
+// well: there the L2's write-back of whole lines serves HBM better than 64-byte pieces (measured on 90 and 180 MB
+// outputs: 10 to 19 % slower written through).
+//
+// (The compiler does not look inside the asm statement: a vector instruction that writes a register of a store of more
+// than eight bytes must be two wait states ahead of it on this part, which the s_nop provides whatever came before.)
+template <class V>
+__device__ __forceinline__ void store_through(V* dst, const V v) {
+    static_assert(sizeof(V) == 16, "store_through: 16-byte values");
+    typedef int wt_i4 __attribute__((ext_vector_type(4)));
+    asm volatile("s_nop 1\n\tglobal_store_dwordx4 %0, %1, off sc1" ::"v"(dst), "v"(__builtin_bit_cast(wt_i4, v)) : "memory");
+}
+template <class V>
+__device__ __forceinline__ void store_out(bool through, V* dst, const V v) {
+    if (through) store_through(dst, v);
+    else *dst = v;
+}
+constexpr size_t kStoreThroughMaxBytes = size_t(64) << 20;
+// the order in which the hardware deals workgroups to the XCDs
+__device__ __forceinline__ unsigned hw_block_id() { return blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z); }
+// `out`: the tensor's allocation; pixel_bytes: channel pitch in bytes; one_block_per_pixel: a pixel's channels all come
+// from one workgroup; nblocks: workgroups of the launch
+__host__ __device__ inline bool store_through_pays(const void* out, int rows, int cols, int pixel_bytes, bool one_block_per_pixel, size_t nblocks) {
+    return one_block_per_pixel && (pixel_bytes & 127) == 0 && (reinterpret_cast<size_t>(out) & 127) == 0 &&
+           (size_t)rows * cols * pixel_bytes <= kStoreThroughMaxBytes && nblocks >= 8;
+}
+__device__ __forceinline__ size_t hw_block_count() { return (size_t)gridDim.x * gridDim.y * gridDim.z; }
+__device__ __forceinline__ void drop_clean_l2_lines() { asm volatile("buffer_inv sc1" ::: "memory"); }
+
 // View of a device tensor as kernels see it.
 struct TView {
     void* ptr;
@@ -187,6 +232,7 @@ struct ConvP16Params {
     int pos_groups;       // workgroups per block of output channels; workgroup g walks tiles g, g + pos_groups, ...
     int cin_chunks;
     int exact_split;      // launch_conv_p16 on fp32 tensors: three fp16 passes even where the fp8 form of the correction terms would run
+    int plain_stores;     // launch_conv_p16, launch_tconv_p16, launch_conv_p16c4: never write the output through (store_through_pays)
     int mfrags;           // cout fragments (16 each) in wpack
     int cout_blocks;      // workgroups along cout (32*wm channels each)
     int f16;              // tensors hold fp16 (wpack then has one plane, and there are no value-range words)
@@ -219,6 +265,12 @@ struct ConvP16Params {
     int in2_hp, in2_wp, in2_cp, in2_y0, in2_x0, in2_stride, in2_chunk0;
     const unsigned* in2_amax;
 };
+// Whether launch_conv_p16 / launch_conv_p16c4 (upsample 1) or launch_tconv_p16 (upsample 2) write their output through
+// (the rule the kernels apply, for kernel descriptions).
+inline bool conv_p16_stores_through(const ConvP16Params& p, int upsample) {
+    return !p.plain_stores && store_through_pays(p.out, upsample * p.npos_y, upsample * p.npos_x, p.out_cp * (p.f16 ? 2 : 4), p.cout_blocks == 1,
+                                                 (size_t)p.pos_groups * p.cout_blocks);
+}
 // Output channel held by row `row` (0..15) of packed weight fragment `mf` when a wave holds groups of `fm` fragments: the
 // rows a lane ends up with (four consecutive ones of every fragment) are 4*fm consecutive channels.
 inline int p16_row_channel(int mf, int row, int fm) { return (mf / fm) * 16 * fm + 4 * fm * (row / 4) + 4 * (mf % fm) + (row % 4); }

@@ -151,6 +151,7 @@ class ConvLayer : public Layer {
         q.act = act();
         q.in_amax = tin(0).amax;   // (the candidates are timed in the form the frame will run: fp8 correction terms where the input has a range word)
         q.exact_split = net->sw.get("FYNHIP_EXACT_SPLIT") ? 1 : 0;
+        q.plain_stores = net->sw.get("FYNHIP_PLAIN_STORES") ? 1 : 0;
         int want_h = 0, want_w = 0, want_wm = 0;   // FYNHIP_P16_TILE=h,w[,wm] (tests): that combination
         if (const char* e = net->sw.get("FYNHIP_P16_TILE")) sscanf(e, "%d,%d,%d", &want_h, &want_w, &want_wm);
         struct Cand { double cost; ConvP16Params q; };
@@ -241,6 +242,7 @@ class ConvLayer : public Layer {
         q.act = act();
         q.in_amax = tin(0).amax;   // (timed in the form the frame will run)
         q.exact_split = net->sw.get("FYNHIP_EXACT_SPLIT") ? 1 : 0;
+        q.plain_stores = net->sw.get("FYNHIP_PLAIN_STORES") ? 1 : 0;
         int want_h = 0, want_w = 0;
         if (const char* e = net->sw.get("FYNHIP_P16_TILE")) sscanf(e, "%d,%d", &want_h, &want_w);
         std::vector<ConvP16Params> cands;
@@ -1170,7 +1172,7 @@ class ConvLayer : public Layer {
             snprintf(buf, sizeof(buf), "conv_p16c4 %s (tap pairs of a 4-channel pixel) tile=32x%d(cout x pos) th=%d tw=%d blocks=%d tiles=%d lds=%zu steps=%d",
                      pp.f16 ? "f16" : (conv_p16c4_uses_fp8(pp, k) ? "f16+fp8-split" : "f16x2-split"), pp.tile_h * pp.tile_w * 4, pp.tile_h, pp.tile_w, pp.pos_groups * pp.cout_blocks, pp.tiles_x * pp.tiles_y * pp.cout_blocks,
                      conv_p16c4_lds_bytes(pp, k), c4_steps);
-            return mode + buf;
+            return mode + buf + (conv_p16_stores_through(pp, 1) ? " stores=through" : "");
         }
         if (p16 && d16) {
             char buf[360];
@@ -1207,7 +1209,7 @@ class ConvLayer : public Layer {
             snprintf(buf, sizeof(buf), "conv_p16 %s tile=%dx%d(cout x pos) waves=%dx%d th=%d tw=%d blocks=%d tiles=%d lds=%zu steps=9 chunks=%d",
                      pp.f16 ? "f16" : (conv_p16_uses_fp8(pp) ? "f16+fp8-split" : "f16x2-split"), 32 * pp.wm, pp.tile_h * pp.tile_w * (4 / pp.wm), pp.wm, 4 / pp.wm, pp.tile_h, pp.tile_w, pp.pos_groups * pp.cout_blocks,
                      pp.tiles_x * pp.tiles_y * pp.cout_blocks, conv_p16_lds_bytes(pp), pp.cin_chunks);
-            return mode + buf;
+            return mode + buf + (conv_p16_stores_through(pp, 1) ? " stores=through" : "");
         }
         if (wide) return mode + (fused ? "wide-kernel(kx folded into cout, summed in the epilogue) " : "wide-kernel(kx folded into cout)+shift_reduce ") + mfma_info(launch);
         return mode + mfma_info(launch);

@@ -89,6 +89,7 @@ class TransConvLayer : public Layer {
         q.acc_mul = 1.f;
         q.act = act();
         q.in_amax = tin(0).amax;   // (timed in the form the frame will run)
+        q.plain_stores = net->sw.get("FYNHIP_PLAIN_STORES") ? 1 : 0;
         int want_h = 0, want_w = 0, want_wm = 0;   // FYNHIP_P16_TILE=h,w[,wm] (tests): that combination
         if (const char* e = net->sw.get("FYNHIP_P16_TILE")) sscanf(e, "%d,%d,%d", &want_h, &want_w, &want_wm);
         std::vector<ConvP16Params> cands;
@@ -238,7 +239,7 @@ class TransConvLayer : public Layer {
             snprintf(buf, sizeof(buf), "transconv, tconv_p16 %s 4 parities per tile, tile=%dx%d(cout x input pos) waves=%dx%d th=%d tw=%d blocks=%d tiles=%d lds=%zu steps=9 chunks=%d", pp.f16 ? "f16" : "f16x2-split",
                      32 * pp.wm, pp.tile_h * pp.tile_w * (4 / pp.wm), pp.wm, 4 / pp.wm, pp.tile_h, pp.tile_w, pp.pos_groups * pp.cout_blocks,
                      pp.tiles_x * pp.tiles_y * pp.cout_blocks, tconv_p16_lds_bytes(pp), pp.cin_chunks);
-            return buf;
+            return std::string(buf) + (conv_p16_stores_through(pp, 2) ? " stores=through" : "");
         }
         return group.subs.empty() ? "transconv" : "transconv, " + std::to_string(group.subs.size()) + " parities in one launch: " + mfma_info(group.subs[0]);
     }
