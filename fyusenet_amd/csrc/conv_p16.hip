@@ -470,7 +470,7 @@ __global__ __launch_bounds__(512) void conv_p16_kernel(const ConvP16Params p) {
     const float acc_mul = p.acc_mul * inv_in_scale;
     store_t* out = reinterpret_cast<store_t*>(p.out);
     const bool have_res = p.res != nullptr;
-    const bool through = store_through_pays(p.out, p.npos_y, p.npos_x, p.out_cp * ESZ, p.cout_blocks == 1 && !p.plain_stores, hw_block_count());
+    const bool through = store_through_pays(p.out, p.npos_y, p.npos_x, p.out_cp * ESZ, (p.cout_blocks == 1 || (CPB * ESZ) % 128 == 0) && !p.plain_stores, hw_block_count());
     bool drop = through && wave == 4 && hw_block_id() < 8;
     const bool res_scale = p.res_scale != 0;
     const float res_floor = p.res_relu ? 0.f : -__builtin_inff();
@@ -711,7 +711,7 @@ __global__ __launch_bounds__(512) void tconv_p16_kernel(const ConvP16Params p) {
     if (p.in_amax) (void)range_scale(range_after_act(range_reduce(range_bits), p.act), &inv_in_scale);
     const float acc_mul = p.acc_mul * inv_in_scale;
     store_t* out = reinterpret_cast<store_t*>(p.out);
-    const bool through = store_through_pays(p.out, 2 * p.npos_y, 2 * p.npos_x, p.out_cp * ESZ, p.cout_blocks == 1 && !p.plain_stores, hw_block_count());
+    const bool through = store_through_pays(p.out, 2 * p.npos_y, 2 * p.npos_x, p.out_cp * ESZ, (p.cout_blocks == 1 || (CPB * ESZ) % 128 == 0) && !p.plain_stores, hw_block_count());
     bool drop = through && wave == 4 && hw_block_id() < 8;
     float vmax = 0.f;
     auto finish_tile = [&](int tile) {
@@ -1101,7 +1101,7 @@ __global__ __launch_bounds__(512) void conv_p16c4_kernel(const ConvP16Params p) 
     if (p.in_amax) (void)range_scale(range_after_act(range_reduce(range_bits), p.act), &inv_in_scale);
     const float acc_mul = p.acc_mul * inv_in_scale;
     store_t* out = reinterpret_cast<store_t*>(p.out);
-    const bool through = store_through_pays(p.out, p.npos_y, p.npos_x, p.out_cp * ESZ, p.cout_blocks == 1 && !p.plain_stores, hw_block_count());
+    const bool through = store_through_pays(p.out, p.npos_y, p.npos_x, p.out_cp * ESZ, (p.cout_blocks == 1 || (32 * ESZ) % 128 == 0) && !p.plain_stores, hw_block_count());
     bool drop = through && wave == 4 && hw_block_id() < 8;
     float vmax = 0.f;
     auto finish_tile = [&](int tile) {

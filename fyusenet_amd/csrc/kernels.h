@@ -28,7 +28,7 @@ struct Act {
 // line, left later launches reading an old half of such lines now and then (whole networks off by O(1), differently
 // from pass to pass); a buffer_inv sc1 in every wave of every kernel made the results stable again (and the frames
 // 1.7x slower).  A kernel therefore writes through only where (1) every 128-byte line of the output is stored whole by
-// one workgroup (a pixel is whole lines and all its channels come from one workgroup), (2) the launch has at least
+// one workgroup (a pixel is whole lines, and so is a workgroup's block of its channels), (2) the launch has at least
 // eight workgroups, and (3) its workgroups 0..7 -- consecutive workgroups are dealt to consecutive XCDs, so these sit
 // on all eight -- drop the clean lines of their L2 once during the launch (the acquire half of device-scope
 // visibility: copies of the buffer's earlier contents that other XCDs may hold; nothing in the kernel reads the
@@ -54,7 +54,7 @@ constexpr size_t kStoreThroughMaxBytes = size_t(64) << 20;
 // the order in which the hardware deals workgroups to the XCDs
 __device__ __forceinline__ unsigned hw_block_id() { return blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z); }
 // `out`: the tensor's allocation; pixel_bytes: channel pitch in bytes; one_block_per_pixel: a pixel's channels all come
-// from one workgroup; nblocks: workgroups of the launch
+// from one workgroup, or from workgroups that each store whole lines of it; nblocks: workgroups of the launch
 __host__ __device__ inline bool store_through_pays(const void* out, int rows, int cols, int pixel_bytes, bool one_block_per_pixel, size_t nblocks) {
     return one_block_per_pixel && (pixel_bytes & 127) == 0 && (reinterpret_cast<size_t>(out) & 127) == 0 &&
            (size_t)rows * cols * pixel_bytes <= kStoreThroughMaxBytes && nblocks >= 8;
@@ -268,7 +268,8 @@ struct ConvP16Params {
 // Whether launch_conv_p16 / launch_conv_p16c4 (upsample 1) or launch_tconv_p16 (upsample 2) write their output through
 // (the rule the kernels apply, for kernel descriptions).
 inline bool conv_p16_stores_through(const ConvP16Params& p, int upsample) {
-    return !p.plain_stores && store_through_pays(p.out, upsample * p.npos_y, upsample * p.npos_x, p.out_cp * (p.f16 ? 2 : 4), p.cout_blocks == 1,
+    const int esz = p.f16 ? 2 : 4;
+    return !p.plain_stores && store_through_pays(p.out, upsample * p.npos_y, upsample * p.npos_x, p.out_cp * esz, p.cout_blocks == 1 || (32 * p.wm * esz) % 128 == 0,
                                                  (size_t)p.pos_groups * p.cout_blocks);
 }
 // Output channel held by row `row` (0..15) of packed weight fragment `mf` when a wave holds groups of `fm` fragments: the
