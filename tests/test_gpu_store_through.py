@@ -29,21 +29,24 @@ def _passes(net, frames, graph):
     return outs, infos
 
 
+@pytest.mark.parametrize("storage", [fa.STORAGE_F32, fa.STORAGE_F16], ids=["f32", "f16"])
 @pytest.mark.parametrize("size", [(128, 96), (256, 192)], ids=["128x96", "256x192"])
 @pytest.mark.parametrize("graph", [False, True], ids=["eager", "graph"])
-def test_written_through_outputs_equal_plain_stores_frame_after_frame(size, graph, monkeypatch):
+def test_written_through_outputs_equal_plain_stores_frame_after_frame(size, graph, storage, monkeypatch):
     w, h = size
     frames = [prng.uniform(4100 + i, (3, h, w), 0.0, 1.0) for i in range(8)]
     frames.insert(4, np.zeros((3, h, w), np.float32))   # (a frame that changes every value)
     monkeypatch.setenv("FYNHIP_FORCE_P16_CONV", "1")
     monkeypatch.delenv("FYNHIP_PLAIN_STORES", raising=False)
-    got, infos = _passes(networks.StyleNet(fa.STORAGE_F32, w, h), frames, graph)
+    got, infos = _passes(networks.StyleNet(storage, w, h), frames, graph)
     through = [n for n, i in infos.items() if "stores=through" in i]
     print("   written through:", through, flush=True)
-    # the residual layers, the stride-2 layers and the transposed ones at least
-    assert len(through) >= 12, infos
+    # fp32 tensors: the residual layers, the first two layers and the transposed ones (conv3's two blocks of 64 channels
+    # are whole lines as well where its tile choice has them); fp16 tensors: the residual layers run another kernel
+    # (conv_h16, plain stores), which leaves the stride-2 layers and the first transposed one
+    assert len(through) >= (12 if storage == fa.STORAGE_F32 else 3), infos
     monkeypatch.setenv("FYNHIP_PLAIN_STORES", "1")
-    want, infos2 = _passes(networks.StyleNet(fa.STORAGE_F32, w, h), frames, graph)
+    want, infos2 = _passes(networks.StyleNet(storage, w, h), frames, graph)
     assert not any("stores=through" in i for i in infos2.values())
     for i, (a, b) in enumerate(zip(got, want)):
         assert np.array_equal(a, b), "pass %d: %d values differ" % (i, int((a != b).sum()))
