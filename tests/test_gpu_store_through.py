@@ -43,8 +43,8 @@ def test_written_through_outputs_equal_plain_stores_frame_after_frame(size, grap
     print("   written through:", through, flush=True)
     # fp32 tensors: the residual layers, the first two layers and the transposed ones (conv3's two blocks of 64 channels
     # are whole lines as well where its tile choice has them); fp16 tensors: the residual layers run another kernel
-    # (conv_h16, plain stores), which leaves the stride-2 layers and the first transposed one
-    assert len(through) >= (12 if storage == fa.STORAGE_F32 else 3), infos
+    # (conv_h16, plain stores), which leaves the stride-2 layers and, with some tile choices, the first transposed one
+    assert len(through) >= (12 if storage == fa.STORAGE_F32 else 2), infos
     monkeypatch.setenv("FYNHIP_PLAIN_STORES", "1")
     want, infos2 = _passes(networks.StyleNet(storage, w, h), frames, graph)
     assert not any("stores=through" in i for i in infos2.values())
