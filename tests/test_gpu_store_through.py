@@ -77,3 +77,22 @@ def test_written_through_single_layers_on_a_dirty_buffer(monkeypatch):
     for i in range(10):
         assert np.array_equal(outs[False][i], outs[True][i]), i
     assert not np.array_equal(outs[False][0], outs[False][1])
+
+
+def test_written_through_outputs_with_several_networks_in_flight(monkeypatch):
+    """Four instances of the style net, each with a frame pipeline of its own streams, run side by side (their kernels
+    share the XCDs and their L2s, and each launch's workgroups 0..7 drop clean lines under the other instances'
+    kernels): every frame equals the plain-store network's synchronous result."""
+    monkeypatch.setenv("FYNHIP_FORCE_P16_CONV", "1")
+    w, h = 256, 192
+    frames = [prng.uniform(6300 + i, (3, h, w), 0.0, 1.0) for i in range(16)]
+    monkeypatch.setenv("FYNHIP_PLAIN_STORES", "1")
+    want, _ = _passes(networks.StyleNet(fa.STORAGE_F32, w, h), frames, False)
+    monkeypatch.delenv("FYNHIP_PLAIN_STORES", raising=False)
+    pool = fa.FramePool(lambda: networks.StyleNet(fa.STORAGE_F32, w, h), instances=4, depth=2)
+    outs = [np.full_like(want[0], np.nan) for _ in frames]
+    tickets = [pool.submit(f, o) for f, o in zip(frames, outs)]
+    pool.wait(tickets[-1])
+    pool.close()
+    for i in range(len(frames)):
+        assert np.array_equal(outs[i], want[i]), i
