@@ -445,6 +445,10 @@ struct GemvParams {
     Act act;
 };
 void launch_gemv(const GemvParams& p, hipStream_t s);
+// The same layer on the matrix cores (16 output rows per workgroup, the reduction split over its four waves): tensors and
+// matrix of one storage type, 32 to 8192 (fp32) or 16384 (fp16) input channels; fp32 weights must lie inside fp16's range (the caller checks).
+bool fc_mfma_supported(const GemvParams& p);
+int launch_fc_mfma(const GemvParams& p, hipStream_t s);
 
 // Layout conversion between the engine layout and CHW fp32 staging buffers.
 // (amax: value-range word of the tensor, raised by what is written, or null; range.h)

@@ -304,14 +304,44 @@ class GemmLayer : public Layer {
                 for (int i = 0; i < cin; i++) wd[(size_t)o * cinp + i] = w[(size_t)o * cin + i];
             reupload(net, static_cast<float*>(w_dev), wd);
         }
+        float wmax = 0.f;
+        for (size_t i = 0; i < (size_t)oc * cin; i++) wmax = std::max(wmax, std::fabs(w[i]));
         have_weights = true;
+        choose(wmax);
+    }
+    // The matrix-core form (fc_mfma_kernel) where it fits -- fp32 weights are split into fp16 halves in registers, so
+    // they must lie inside fp16's range -- and is measured not to be slower than the vector-unit form on this layer
+    // (both stream the matrix once and are bound by that; with one right-hand side the matrix-core form pays for the
+    // operand split and for staging the vector in every workgroup: 8.0 against 3.1 us on 2048 -> 1000 in fp32, 23.7
+    // against 22.4 us on 8192 -> 8192 in fp16; FYNHIP_NO_MFMA_GEMM / FYNHIP_FORCE_MFMA_GEMM pin the choice).
+    void choose(float wmax) {
+        use_mfma = false;
+        if (net->sw.get("FYNHIP_NO_MFMA_GEMM") || !fc_mfma_supported(p) || !(wmax < 3.0e4f)) return;
+        if (net->sw.get("FYNHIP_FORCE_MFMA_GEMM")) { use_mfma = true; return; }
+        const char* at = net->sw.get("FYNHIP_AUTOTUNE");
+        if (at && at[0] == '0') return;   // (unmeasured: the vector-unit form, which wins on every layer measured so far)
+        float t_m = 1e30f, t_v = 1e30f;
+        for (int rep = 0; rep < 3; rep++) {
+            t_m = std::min(t_m, time_calls(net, [&]() {
+                if (launch_fc_mfma(p, net->stream) != 0) fail(FYN_ERR_DEVICE, "layer %s: matrix-core launch failed while tuning", d.name);
+            }, 10));
+            t_v = std::min(t_v, time_calls(net, [&]() { launch_gemv(p, net->stream); }, 10));
+        }
+        use_mfma = t_m <= 1.05f * t_v;
+        if (net->sw.get("FYNHIP_TUNE_VERBOSE")) fprintf(stderr, "[tune] fully connected %s: matrix cores %.2f us, vector units %.2f us\n", d.name, t_m * 1e3f, t_v * 1e3f);
     }
     void forward(hipStream_t s) override {
         if (!have_weights) fail(FYN_ERR_STATE, "layer %s (%d): forward() without weights", d.name, d.number);
-        launch_gemv(p, s);
+        if (use_mfma) {
+            if (launch_fc_mfma(p, s) != 0) fail(FYN_ERR_DEVICE, "layer %s: matrix-core launch failed", d.name);
+        } else {
+            launch_gemv(p, s);
+        }
     }
-    std::string info() const override { return "gemv"; }
-    bool have_weights = false;
+    std::string info() const override {
+        return use_mfma ? (p.out.f16 ? "fc_mfma f16 16 rows per workgroup, 4 waves split the reduction" : "fc_mfma f16x2-split 16 rows per workgroup, 4 waves split the reduction") : "gemv";
+    }
+    bool have_weights = false, use_mfma = false;
     std::vector<float> block;
     GemvParams p{};
     void* w_dev = nullptr;

@@ -1175,6 +1175,172 @@ void launch_gemv(const GemvParams& p, hipStream_t s) {
 }
 
 // ---------------------------------------------------------------------------------------------
+// The same product on the matrix cores (v_mfma_f32_16x16x32_f16, fp32 accumulate).  A workgroup owns 16 output rows;
+// its four waves take a quarter of the reduction each, in steps of 32 input channels: the A operand is the 16 x 32
+// block of weights as it lies in memory (lane = row, eight consecutive channels; fp32 weights are split into fp16 hi
+// and lo halves in registers: nothing is packed beforehand, the matrix is streamed once as in gemv_kernel), the B
+// operand the input vector's 32 values in every one of the 16 columns (staged once per workgroup in LDS as fp16, with
+// fp32 tensors as hi and lo planes scaled by a power of two that puts the largest value at 2^14), so all columns of
+// the result are equal and column 0 is taken.  fp32 tensors: hi*hi + lo*hi + hi*lo, 22 significant bits per operand.
+// The four partial sums meet in LDS in a fixed order.  With one right-hand side 15 of the 16 columns are idle; what
+// the kernel is bound by is the weight stream, like gemv_kernel.
+// ---------------------------------------------------------------------------------------------
+typedef float fc_f32x4 __attribute__((ext_vector_type(4)));
+constexpr int FC_TRIP = 8;   // steps whose weight loads are in flight together (two such sets: one is converted while the next arrives)
+
+template <typename T>
+struct FcRaw;
+template <>
+struct FcRaw<float> { float4 a, b; };
+template <>
+struct FcRaw<_Float16> { half8_t a; };
+
+template <typename T>
+__global__ __launch_bounds__(256) void fc_mfma_kernel(const GemvParams p) {
+    constexpr bool F32 = sizeof(T) == 4;
+    extern __shared__ __align__(16) unsigned char fc_lds[];   // x hi [kpad] halves, then (fp32 tensors) x lo [kpad] halves
+    __shared__ float part[4][16];
+    __shared__ float wmax[4];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int mq = lane & 15, kq = lane >> 4;
+    const int cinp = p.in.cp;
+    const int nsteps = (cinp + 31) >> 5, kpad = nsteps * 32;
+    const int per = (nsteps + 3) >> 2;
+    const int s0 = wave * per, s1 = min(nsteps, s0 + per);
+    const int row0 = blockIdx.x * 16;
+    const int wrow = min(row0 + mq, p.out.cp - 1);   // (the matrix has out.cp rows; fragment rows behind them repeat the last and are not stored)
+    const T* w = reinterpret_cast<const T*>(p.w) + (size_t)wrow * cinp + kq * 8;
+    auto load_trip = [&](FcRaw<T> (&raw)[FC_TRIP], int first) {
+#pragma unroll
+        for (int j = 0; j < FC_TRIP; j++) {
+            const int s = first + j;
+            const bool ok = s < s1 && s * 32 + kq * 8 < cinp;
+            const T* src = w + (ok ? s * 32 : 0);
+            if constexpr (F32) {
+                raw[j].a = *reinterpret_cast<const float4*>(src);
+                raw[j].b = *reinterpret_cast<const float4*>(src + 4);
+                if (!ok) raw[j].a = raw[j].b = float4{0.f, 0.f, 0.f, 0.f};
+            } else {
+                raw[j].a = *reinterpret_cast<const half8_t*>(src);
+                if (!ok) raw[j].a = (half8_t)((_Float16)0.f);
+            }
+        }
+    };
+    FcRaw<T> ra[FC_TRIP], rb[FC_TRIP];
+    load_trip(ra, s0);   // (the weights do not depend on the vector: their first loads go out ahead of its staging)
+
+    // the input vector: activation, scale, fp16 planes
+    const T* x = reinterpret_cast<const T*>(p.in.ptr) + tv_off(p.in, 0, 0);
+    constexpr int XG = 8;   // groups of 8 values per thread: up to 16384 inputs
+    float xv[XG][8];
+    float amax = 0.f;
+#pragma unroll
+    for (int g = 0; g < XG; g++) {
+        const int c = (tid + g * 256) * 8;
+#pragma unroll
+        for (int e = 0; e < 8; e++) xv[g][e] = 0.f;
+        if (c < cinp) {
+            const float4 v0 = act4(ld4<T>(x + c), p.act), v1 = act4(ld4<T>(x + c + 4), p.act);
+            xv[g][0] = v0.x; xv[g][1] = v0.y; xv[g][2] = v0.z; xv[g][3] = v0.w;
+            xv[g][4] = v1.x; xv[g][5] = v1.y; xv[g][6] = v1.z; xv[g][7] = v1.w;
+#pragma unroll
+            for (int e = 0; e < 8; e++) amax = fmaxf(amax, fabsf(xv[g][e]));
+        }
+    }
+    float mul = 1.f, inv = 1.f;
+    if constexpr (F32) {
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o));
+        if (lane == 0) wmax[wave] = amax;
+        __syncthreads();
+        amax = fmaxf(fmaxf(wmax[0], wmax[1]), fmaxf(wmax[2], wmax[3]));
+        // a power of two that takes the largest value to [2^14, 2^15): no overflow in fp16, and the lo halves stay normal
+        int e = (int)((__float_as_uint(amax) >> 23) & 0xffu) - 127;
+        if (amax > 0.f && e > -100 && e < 128) {
+            mul = __uint_as_float((unsigned)(127 + 14 - e) << 23);
+            inv = __uint_as_float((unsigned)(127 - 14 + e) << 23);
+        }
+    }
+#pragma unroll
+    for (int g = 0; g < XG; g++) {
+        const int c = (tid + g * 256) * 8;
+        if (c < kpad) {
+            half8_t hi, lo;
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                const float v = xv[g][e] * mul;
+                hi[e] = (_Float16)v;
+                lo[e] = (_Float16)(v - (float)hi[e]);
+            }
+            *reinterpret_cast<half8_t*>(fc_lds + (size_t)c * 2) = hi;
+            if constexpr (F32) *reinterpret_cast<half8_t*>(fc_lds + (size_t)(kpad + c) * 2) = lo;
+        }
+    }
+    __syncthreads();
+
+    fc_f32x4 acc = (fc_f32x4)(0.f);
+    auto run_trip = [&](const FcRaw<T> (&raw)[FC_TRIP], int first) {
+#pragma unroll
+        for (int j = 0; j < FC_TRIP; j++) {
+            const int s = first + j;
+            if (s >= s1) break;
+            const half8_t bh = *reinterpret_cast<const half8_t*>(fc_lds + (size_t)(s * 32 + kq * 8) * 2);
+            if constexpr (F32) {
+                const half8_t bl = *reinterpret_cast<const half8_t*>(fc_lds + (size_t)(kpad + s * 32 + kq * 8) * 2);
+                const float r[8] = {raw[j].a.x, raw[j].a.y, raw[j].a.z, raw[j].a.w, raw[j].b.x, raw[j].b.y, raw[j].b.z, raw[j].b.w};
+                half8_t ah, al;
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    ah[e] = (_Float16)r[e];
+                    al[e] = (_Float16)(r[e] - (float)ah[e]);
+                }
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(ah, bh, acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(al, bh, acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(ah, bl, acc, 0, 0, 0);
+            } else {
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(raw[j].a, bh, acc, 0, 0, 0);
+            }
+        }
+    };
+    for (int t = s0; t < s1; t += 2 * FC_TRIP) {
+        if (t + FC_TRIP < s1) load_trip(rb, t + FC_TRIP);
+        run_trip(ra, t);
+        if (t + FC_TRIP >= s1) break;
+        if (t + 2 * FC_TRIP < s1) load_trip(ra, t + 2 * FC_TRIP);
+        run_trip(rb, t + FC_TRIP);
+    }
+    // a lane of column 0 holds rows 4 * kq .. 4 * kq + 3
+    if (mq == 0) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) part[wave][kq * 4 + i] = acc[i];
+    }
+    __syncthreads();
+    if (tid < 16) {
+        const int row = row0 + tid;
+        if (row < p.out.cp) {
+            const float sum = ((part[0][tid] + part[1][tid]) + part[2][tid]) + part[3][tid];
+            const float r = (row < p.out.c) ? (sum * inv) * p.scale[row] + p.bias[row] : 0.f;
+            reinterpret_cast<T*>(p.out.ptr)[tv_off(p.out, 0, 0) + row] = (T)r;
+        }
+    }
+}
+// fp16 tensors hold the vector and the matrix in fp16 already; fp32 weights must stay below fp16's range (the caller
+// knows the matrix and checks: fc_mfma_supported says nothing about its values)
+bool fc_mfma_supported(const GemvParams& p) {
+    const int kpad = (p.in.cp + 31) / 32 * 32;
+    return p.in.cp >= 32 && p.in.cp % 8 == 0 && (size_t)kpad * (p.out.f16 ? 2 : 4) <= 32768 && (p.w_f16 != 0) == (p.out.f16 != 0) && p.in.f16 == p.out.f16 && p.out.cp >= 1;
+}
+int launch_fc_mfma(const GemvParams& p, hipStream_t s) {
+    if (!fc_mfma_supported(p)) return -1;
+    const int kpad = (p.in.cp + 31) / 32 * 32;
+    dim3 grid((p.out.cp + 15) / 16), block(256);
+    if (p.out.f16) hipLaunchKernelGGL((fc_mfma_kernel<_Float16>), grid, block, (size_t)kpad * 2, s, p);
+    else hipLaunchKernelGGL((fc_mfma_kernel<float>), grid, block, (size_t)kpad * 4, s, p);
+    return hipGetLastError() == hipSuccess ? 0 : -3;
+}
+
+// ---------------------------------------------------------------------------------------------
 // direct convolution: the engine's second, plain implementation of the convolution family's sampling rules (zero halo,
 // edge clamp of shallow layers, fractional steps), selected by FYNHIP_FORCE_DIRECT_CONV for cross-checks.
 // fp32 FMA, one thread = one output pixel x 4 output channels.

@@ -159,6 +159,37 @@ def test_gemm_parity(cin, cout, bn, storage):
     assert rel_l2(got, ref) <= TOL[storage]
 
 
+_FC_CASES = [(32, 16, False, A.NONE, 1.0), (40, 7, True, A.RELU, 1.0), (1025, 2, False, A.RELU, 1.0), (2048, 1000, False, A.RELU, 1.0),
+             (512, 256, True, A.LEAKY_RELU, 3.0e5), (100, 10, True, A.CLIP, 1.0), (4096, 24, False, A.NONE, 1.0e-7), (8192, 40, False, A.RELU, 1.0)]
+# (fp16 tensors cannot hold the value ranges that the scaled cases are about)
+_FC_PARAMS = [pytest.param(*c, st, id="%dx%d-%s-%g-%s" % (c[0], c[1], c[3].name, c[4], "f32" if st == fa.STORAGE_F32 else "f16"))
+              for c in _FC_CASES for st in (fa.STORAGE_F32, fa.STORAGE_F16) if st == fa.STORAGE_F32 or c[4] == 1.0]
+
+
+@pytest.mark.parametrize("form", ["mfma", "vector"])
+@pytest.mark.parametrize("cin,cout,bn,act,xscale,storage", _FC_PARAMS)
+def test_gemm_parity_of_both_forms(cin, cout, bn, act, xscale, form, storage, monkeypatch):
+    """The fully connected layer on the matrix cores (fc_mfma_kernel) and on the vector units (gemv_kernel), each forced
+    (gpu/deep/deepgemmlayer.cpp:66-236): reductions that are not whole steps of 32, fragments of 16 rows that reach
+    behind the last output, inputs far above fp16's range and far below it (the vector is scaled by a power of two
+    before it is split), all four activations on the fetch."""
+    monkeypatch.setenv("FYNHIP_FORCE_MFMA_GEMM" if form == "mfma" else "FYNHIP_NO_MFMA_GEMM", "1")
+    b = fa.GPULayerBuilder("fc").type(fa.LayerType.GEMM).number(1).shape(cout, 1, 1, cin).prefixAct(act).deep()
+    if act == A.LEAKY_RELU:
+        b.leakyReLU(0.1)
+    if act == A.CLIP:
+        b.clip(-0.5, 1.5)
+    if bn:
+        b.postfixNorm(fa.NormType.BATCHNORM)
+    wts = conv_block(195, cout, 1, cin, bn=bn)
+    x = (prng.normal(196, (cin, 1, 1)) * xscale).astype(np.float32)
+    got, info = run_single(b, storage, [x], wts)
+    ref = oracle_single(b, storage, [x], wts)
+    wide = cin <= (8192 if storage == fa.STORAGE_F32 else 16384)
+    assert info.startswith("fc_mfma" if form == "mfma" and wide else "gemv"), info
+    assert rel_l2(got, ref) <= TOL[storage]
+
+
 def test_gemm_reference_pattern():
     # misctests.cpp:238-265: 512 -> 256, alternating +-1 rows on ones => exactly 0
     cin, cout = 512, 256
