@@ -439,6 +439,7 @@ void launch_splitk_reduce(const SplitKReduceParams& p, hipStream_t s);
 struct GemvParams {
     TView in, out;       // 1x1 spatial
     const void* w;       // [cout][cinp] in storage type (f16) or fp32
+    const void* w_split; // launch_fc_mfma on fp32 tensors: [cout][cinp / 8][8 x fp16 hi | 8 x fp16 lo] of the same matrix (null: none)
     int w_f16;
     const float* scale;
     const float* bias;
@@ -446,7 +447,8 @@ struct GemvParams {
 };
 void launch_gemv(const GemvParams& p, hipStream_t s);
 // The same layer on the matrix cores (16 output rows per workgroup, the reduction split over its four waves): tensors and
-// matrix of one storage type, 32 to 8192 (fp32) or 16384 (fp16) input channels; fp32 weights must lie inside fp16's range (the caller checks).
+// matrix of one storage type, 32 to 8192 (fp32) or 16384 (fp16) input channels; fp32 tensors: the matrix once more as fp16
+// halves (w_split), which asks for weights inside fp16's range (the caller checks).
 bool fc_mfma_supported(const GemvParams& p);
 int launch_fc_mfma(const GemvParams& p, hipStream_t s);
 

@@ -306,14 +306,30 @@ class GemmLayer : public Layer {
         }
         float wmax = 0.f;
         for (size_t i = 0; i < (size_t)oc * cin; i++) wmax = std::max(wmax, std::fabs(w[i]));
+        // the matrix once more for the matrix-core form on fp32 tensors: fp16 hi and lo halves, eight weights at a time
+        p.w_split = nullptr;
+        if (!p.w_f16 && wmax < 3.0e4f && !net->sw.get("FYNHIP_NO_MFMA_GEMM")) {
+            std::vector<uint16_t> ws((size_t)p.out.cp * cinp * 2, 0);
+            for (int o = 0; o < oc; o++)
+                for (int i = 0; i < cin; i++) {
+                    const float v = w[(size_t)o * cin + i];
+                    const uint16_t hb = f2h_bits(v);
+                    const size_t at = ((size_t)o * cinp + (i & ~7)) * 2 + (i & 7);
+                    ws[at] = hb;
+                    ws[at + 8] = f2h_bits(v - h2f(hb));
+                }
+            if (!w_split_dev) w_split_dev = net->dev_alloc(ws.size() * 2);
+            reupload(net, static_cast<uint16_t*>(w_split_dev), ws);
+            p.w_split = w_split_dev;
+        }
         have_weights = true;
         choose(wmax);
     }
     // The matrix-core form (fc_mfma_kernel) where it fits -- fp32 weights are split into fp16 halves in registers, so
-    // they must lie inside fp16's range -- and is measured not to be slower than the vector-unit form on this layer
-    // (both stream the matrix once and are bound by that; with one right-hand side the matrix-core form pays for the
-    // operand split and for staging the vector in every workgroup: 8.0 against 3.1 us on 2048 -> 1000 in fp32, 23.7
-    // against 22.4 us on 8192 -> 8192 in fp16; FYNHIP_NO_MFMA_GEMM / FYNHIP_FORCE_MFMA_GEMM pin the choice).
+    // they must lie inside fp16's range -- and is measured to be faster than the vector-unit form on this layer (both
+    // stream the matrix once and are bound by that; with one right-hand side the matrix-core form pays for staging the
+    // vector in every workgroup and for two barriers: 7.3 against 3.1 us on 2048 -> 1000 in fp32, 23.3 against 22.5 us
+    // on 8192 -> 8192 in fp16; FYNHIP_NO_MFMA_GEMM / FYNHIP_FORCE_MFMA_GEMM pin the choice).
     void choose(float wmax) {
         use_mfma = false;
         if (net->sw.get("FYNHIP_NO_MFMA_GEMM") || !fc_mfma_supported(p) || !(wmax < 3.0e4f)) return;
@@ -327,7 +343,7 @@ class GemmLayer : public Layer {
             }, 10));
             t_v = std::min(t_v, time_calls(net, [&]() { launch_gemv(p, net->stream); }, 10));
         }
-        use_mfma = t_m <= 1.05f * t_v;
+        use_mfma = t_m < t_v;
         if (net->sw.get("FYNHIP_TUNE_VERBOSE")) fprintf(stderr, "[tune] fully connected %s: matrix cores %.2f us, vector units %.2f us\n", d.name, t_m * 1e3f, t_v * 1e3f);
     }
     void forward(hipStream_t s) override {
@@ -339,12 +355,12 @@ class GemmLayer : public Layer {
         }
     }
     std::string info() const override {
-        return use_mfma ? (p.out.f16 ? "fc_mfma f16 16 rows per workgroup, 4 waves split the reduction" : "fc_mfma f16x2-split 16 rows per workgroup, 4 waves split the reduction") : "gemv";
+        return use_mfma ? (p.out.f16 ? "fc_mfma f16, 16 or 4 rows per workgroup, 4 waves split the reduction" : "fc_mfma f16x2-split, 16 or 4 rows per workgroup, 4 waves split the reduction") : "gemv";
     }
     bool have_weights = false, use_mfma = false;
     std::vector<float> block;
     GemvParams p{};
-    void* w_dev = nullptr;
+    void *w_dev = nullptr, *w_split_dev = nullptr;
     float *scale_dev = nullptr, *bias_dev = nullptr;
 };
 

@@ -1177,8 +1177,9 @@ void launch_gemv(const GemvParams& p, hipStream_t s) {
 // ---------------------------------------------------------------------------------------------
 // The same product on the matrix cores (v_mfma_f32_16x16x32_f16, fp32 accumulate).  A workgroup owns 16 output rows;
 // its four waves take a quarter of the reduction each, in steps of 32 input channels: the A operand is the 16 x 32
-// block of weights as it lies in memory (lane = row, eight consecutive channels; fp32 weights are split into fp16 hi
-// and lo halves in registers: nothing is packed beforehand, the matrix is streamed once as in gemv_kernel), the B
+// block of weights (lane = row, eight consecutive channels; fp16 weights as they lie in memory, fp32 weights from a
+// copy packed at weight load as [row][group of 8 channels][8 x fp16 hi | 8 x fp16 lo], the same four bytes per weight,
+// so that the matrix is streamed once as in gemv_kernel and nothing is converted on the way), the B
 // operand the input vector's 32 values in every one of the 16 columns (staged once per workgroup in LDS as fp16, with
 // fp32 tensors as hi and lo planes scaled by a power of two that puts the largest value at 2^14), so all columns of
 // the result are equal and column 0 is taken.  fp32 tensors: hi*hi + lo*hi + hi*lo, 22 significant bits per operand.
@@ -1191,11 +1192,13 @@ constexpr int FC_TRIP = 8;   // steps whose weight loads are in flight together 
 template <typename T>
 struct FcRaw;
 template <>
-struct FcRaw<float> { float4 a, b; };
+struct FcRaw<float> { half8_t a, b; };   // hi and lo halves of eight weights
 template <>
 struct FcRaw<_Float16> { half8_t a; };
 
-template <typename T>
+// R: output rows per workgroup, 16 or -- for matrices of few rows, so that every CU of the chip pulls a share of the
+// stream -- 4 (the fragment's rows then repeat those four; lanes that ask for the same bytes cost no traffic).
+template <typename T, int R>
 __global__ __launch_bounds__(256) void fc_mfma_kernel(const GemvParams p) {
     constexpr bool F32 = sizeof(T) == 4;
     extern __shared__ __align__(16) unsigned char fc_lds[];   // x hi [kpad] halves, then (fp32 tensors) x lo [kpad] halves
@@ -1208,45 +1211,59 @@ __global__ __launch_bounds__(256) void fc_mfma_kernel(const GemvParams p) {
     const int nsteps = (cinp + 31) >> 5, kpad = nsteps * 32;
     const int per = (nsteps + 3) >> 2;
     const int s0 = wave * per, s1 = min(nsteps, s0 + per);
-    const int row0 = blockIdx.x * 16;
-    const int wrow = min(row0 + mq, p.out.cp - 1);   // (the matrix has out.cp rows; fragment rows behind them repeat the last and are not stored)
-    const T* w = reinterpret_cast<const T*>(p.w) + (size_t)wrow * cinp + kq * 8;
+    const int row0 = blockIdx.x * R;
+    const int wrow = min(row0 + (mq & (R - 1)), p.out.cp - 1);   // (the matrix has out.cp rows; fragment rows behind them repeat the last and are not stored)
+    // (fp32 tensors: p.w_split, 16 halves per group of 8 weights)
+    const _Float16* w = F32 ? reinterpret_cast<const _Float16*>(p.w_split) + ((size_t)wrow * cinp + kq * 8) * 2
+                            : reinterpret_cast<const _Float16*>(p.w) + (size_t)wrow * cinp + kq * 8;
     auto load_trip = [&](FcRaw<T> (&raw)[FC_TRIP], int first) {
 #pragma unroll
         for (int j = 0; j < FC_TRIP; j++) {
             const int s = first + j;
             const bool ok = s < s1 && s * 32 + kq * 8 < cinp;
-            const T* src = w + (ok ? s * 32 : 0);
+            const _Float16* src = w + (ok ? s * 32 * (F32 ? 2 : 1) : 0);
+            raw[j].a = *reinterpret_cast<const half8_t*>(src);
+            if (!ok) raw[j].a = (half8_t)((_Float16)0.f);
             if constexpr (F32) {
-                raw[j].a = *reinterpret_cast<const float4*>(src);
-                raw[j].b = *reinterpret_cast<const float4*>(src + 4);
-                if (!ok) raw[j].a = raw[j].b = float4{0.f, 0.f, 0.f, 0.f};
-            } else {
-                raw[j].a = *reinterpret_cast<const half8_t*>(src);
-                if (!ok) raw[j].a = (half8_t)((_Float16)0.f);
+                raw[j].b = *reinterpret_cast<const half8_t*>(src + 8);
+                if (!ok) raw[j].b = (half8_t)((_Float16)0.f);
             }
         }
     };
-    FcRaw<T> ra[FC_TRIP], rb[FC_TRIP];
-    load_trip(ra, s0);   // (the weights do not depend on the vector: their first loads go out ahead of its staging)
-
-    // the input vector: activation, scale, fp16 planes
+    // the input vector's loads first (the counters retire loads in order: waiting for these must not wait for the weights),
+    // unconditional, from a clamped address
     const T* x = reinterpret_cast<const T*>(p.in.ptr) + tv_off(p.in, 0, 0);
     constexpr int XG = 8;   // groups of 8 values per thread: up to 16384 inputs
+    float4 x0[XG], x1[XG];
+#pragma unroll
+    for (int g = 0; g < XG; g++) {
+        const int c = (tid + g * 256) * 8;
+        if (g * 2048 < cinp) {   // (uniform)
+            const int cc = min(c, cinp - 8);
+            x0[g] = ld4<T>(x + cc);
+            x1[g] = ld4<T>(x + cc + 4);
+        } else {
+            x0[g] = x1[g] = float4{0.f, 0.f, 0.f, 0.f};
+        }
+    }
+    FcRaw<T> ra[FC_TRIP], rb[FC_TRIP];
+    // (the weights do not depend on the vector: both sets of loads go out ahead of its staging, so that a reduction of up
+    // to 2048 channels pays the memory's latency once)
+    load_trip(ra, s0);
+    load_trip(rb, s0 + FC_TRIP);
+
+    // the input vector: activation, scale, fp16 planes
     float xv[XG][8];
     float amax = 0.f;
 #pragma unroll
     for (int g = 0; g < XG; g++) {
         const int c = (tid + g * 256) * 8;
+        const bool in = c < cinp;
+        const float4 v0 = act4(x0[g], p.act), v1 = act4(x1[g], p.act);
+        xv[g][0] = in ? v0.x : 0.f; xv[g][1] = in ? v0.y : 0.f; xv[g][2] = in ? v0.z : 0.f; xv[g][3] = in ? v0.w : 0.f;
+        xv[g][4] = in ? v1.x : 0.f; xv[g][5] = in ? v1.y : 0.f; xv[g][6] = in ? v1.z : 0.f; xv[g][7] = in ? v1.w : 0.f;
 #pragma unroll
-        for (int e = 0; e < 8; e++) xv[g][e] = 0.f;
-        if (c < cinp) {
-            const float4 v0 = act4(ld4<T>(x + c), p.act), v1 = act4(ld4<T>(x + c + 4), p.act);
-            xv[g][0] = v0.x; xv[g][1] = v0.y; xv[g][2] = v0.z; xv[g][3] = v0.w;
-            xv[g][4] = v1.x; xv[g][5] = v1.y; xv[g][6] = v1.z; xv[g][7] = v1.w;
-#pragma unroll
-            for (int e = 0; e < 8; e++) amax = fmaxf(amax, fabsf(xv[g][e]));
-        }
+        for (int e = 0; e < 8; e++) amax = fmaxf(amax, fabsf(xv[g][e]));
     }
     float mul = 1.f, inv = 1.f;
     if constexpr (F32) {
@@ -1279,44 +1296,35 @@ __global__ __launch_bounds__(256) void fc_mfma_kernel(const GemvParams p) {
     }
     __syncthreads();
 
-    fc_f32x4 acc = (fc_f32x4)(0.f);
+    fc_f32x4 acc = (fc_f32x4)(0.f), acc1 = (fc_f32x4)(0.f), acc2 = (fc_f32x4)(0.f);   // (one chain per pass: no MFMA waits for the one before it)
     auto run_trip = [&](const FcRaw<T> (&raw)[FC_TRIP], int first) {
 #pragma unroll
         for (int j = 0; j < FC_TRIP; j++) {
             const int s = first + j;
             if (s >= s1) break;
             const half8_t bh = *reinterpret_cast<const half8_t*>(fc_lds + (size_t)(s * 32 + kq * 8) * 2);
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(raw[j].a, bh, acc, 0, 0, 0);
             if constexpr (F32) {
                 const half8_t bl = *reinterpret_cast<const half8_t*>(fc_lds + (size_t)(kpad + s * 32 + kq * 8) * 2);
-                const float r[8] = {raw[j].a.x, raw[j].a.y, raw[j].a.z, raw[j].a.w, raw[j].b.x, raw[j].b.y, raw[j].b.z, raw[j].b.w};
-                half8_t ah, al;
-#pragma unroll
-                for (int e = 0; e < 8; e++) {
-                    ah[e] = (_Float16)r[e];
-                    al[e] = (_Float16)(r[e] - (float)ah[e]);
-                }
-                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(ah, bh, acc, 0, 0, 0);
-                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(al, bh, acc, 0, 0, 0);
-                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(ah, bl, acc, 0, 0, 0);
-            } else {
-                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(raw[j].a, bh, acc, 0, 0, 0);
+                acc1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(raw[j].b, bh, acc1, 0, 0, 0);
+                acc2 = __builtin_amdgcn_mfma_f32_16x16x32_f16(raw[j].a, bl, acc2, 0, 0, 0);
             }
         }
     };
     for (int t = s0; t < s1; t += 2 * FC_TRIP) {
-        if (t + FC_TRIP < s1) load_trip(rb, t + FC_TRIP);
         run_trip(ra, t);
-        if (t + FC_TRIP >= s1) break;
         if (t + 2 * FC_TRIP < s1) load_trip(ra, t + 2 * FC_TRIP);
+        if (t + FC_TRIP >= s1) break;
         run_trip(rb, t + FC_TRIP);
+        if (t + 3 * FC_TRIP < s1) load_trip(rb, t + 3 * FC_TRIP);
     }
     // a lane of column 0 holds rows 4 * kq .. 4 * kq + 3
     if (mq == 0) {
 #pragma unroll
-        for (int i = 0; i < 4; i++) part[wave][kq * 4 + i] = acc[i];
+        for (int i = 0; i < 4; i++) part[wave][kq * 4 + i] = acc[i] + (acc1[i] + acc2[i]);
     }
     __syncthreads();
-    if (tid < 16) {
+    if (tid < R) {
         const int row = row0 + tid;
         if (row < p.out.cp) {
             const float sum = ((part[0][tid] + part[1][tid]) + part[2][tid]) + part[3][tid];
@@ -1329,14 +1337,21 @@ __global__ __launch_bounds__(256) void fc_mfma_kernel(const GemvParams p) {
 // knows the matrix and checks: fc_mfma_supported says nothing about its values)
 bool fc_mfma_supported(const GemvParams& p) {
     const int kpad = (p.in.cp + 31) / 32 * 32;
-    return p.in.cp >= 32 && p.in.cp % 8 == 0 && (size_t)kpad * (p.out.f16 ? 2 : 4) <= 32768 && (p.w_f16 != 0) == (p.out.f16 != 0) && p.in.f16 == p.out.f16 && p.out.cp >= 1;
+    return (p.out.f16 || p.w_split) && p.in.cp >= 32 && p.in.cp % 8 == 0 && (size_t)kpad * (p.out.f16 ? 2 : 4) <= 32768 && (p.w_f16 != 0) == (p.out.f16 != 0) && p.in.f16 == p.out.f16 && p.out.cp >= 1;
 }
 int launch_fc_mfma(const GemvParams& p, hipStream_t s) {
     if (!fc_mfma_supported(p)) return -1;
     const int kpad = (p.in.cp + 31) / 32 * 32;
-    dim3 grid((p.out.cp + 15) / 16), block(256);
-    if (p.out.f16) hipLaunchKernelGGL((fc_mfma_kernel<_Float16>), grid, block, (size_t)kpad * 2, s, p);
-    else hipLaunchKernelGGL((fc_mfma_kernel<float>), grid, block, (size_t)kpad * 4, s, p);
+    const bool few = (p.out.cp + 15) / 16 < 256;
+    dim3 grid(few ? (p.out.cp + 3) / 4 : (p.out.cp + 15) / 16), block(256);
+    const size_t lds = (size_t)kpad * (p.out.f16 ? 2 : 4);
+    if (p.out.f16) {
+        if (few) hipLaunchKernelGGL((fc_mfma_kernel<_Float16, 4>), grid, block, lds, s, p);
+        else hipLaunchKernelGGL((fc_mfma_kernel<_Float16, 16>), grid, block, lds, s, p);
+    } else {
+        if (few) hipLaunchKernelGGL((fc_mfma_kernel<float, 4>), grid, block, lds, s, p);
+        else hipLaunchKernelGGL((fc_mfma_kernel<float, 16>), grid, block, lds, s, p);
+    }
     return hipGetLastError() == hipSuccess ? 0 : -3;
 }
 
